@@ -1,0 +1,243 @@
+/*
+ * nblahip.h - C-ABI of the MI355X (gfx950) normalization kernel layer.
+ *
+ * This is the whole device-facing surface of the backend: plain pointers and
+ * sizes, no C++ types, no exceptions.  The nbla::Function subclasses of the
+ * "hip" backend (BatchNormalizationHip<T>, LayerNormalizationHip<T>,
+ * GroupNormalizationHip<T>, InstanceNormalizationHip<T>) call nothing else.
+ * Each entry point replaces the kernel launches of one reference function
+ * body; the citation names that body under sony/nnabla-ext-cuda.
+ *
+ * Conventions (all entry points):
+ *   - return 0 on success, a negative NBLAHIP_E* code for a bad argument, or a
+ *     positive hipError_t value for a runtime failure; never throw, never
+ *     allocate, never synchronise the host; nblahip_error_string() explains;
+ *   - every pointer is a borrowed device pointer on the current device;
+ *   - `dtype` is the storage type of the activation tensors x, y, dy, dx
+ *     (NBLAHIP_F32 or NBLAHIP_F16).  gamma, beta, their gradients, running
+ *     and batch statistics and the statistic gradients are ALWAYS float32,
+ *     all arithmetic and accumulation is float32;
+ *   - a NULL gamma / beta means no_scale / no_bias (1 and 0); a NULL
+ *     dx / dgamma / dbeta means "not propagated"; NULL dmean / dvar means the
+ *     function had a single output; `accum_*` != 0 adds onto the existing
+ *     gradient instead of overwriting it;
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*; NULL is the
+ *     null stream the reference launches on);
+ *   - `workspace` is caller-owned scratch of at least the matching
+ *     *_workspace_bytes() (256-byte aligned); its contents need not persist
+ *     between calls.  Results are deterministic (no atomics): same inputs,
+ *     same bits.
+ */
+#ifndef NBLAHIP_H_
+#define NBLAHIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NBLAHIP_EXPORT __attribute__((visibility("default")))
+
+enum nblahip_dtype { NBLAHIP_F32 = 0, NBLAHIP_F16 = 1 };
+
+enum nblahip_status {
+  NBLAHIP_OK = 0,
+  NBLAHIP_EINVAL = -1,    /* NULL required pointer, non-positive size, bad enum */
+  NBLAHIP_EWORKSPACE = -2,/* workspace NULL, misaligned or too small */
+  NBLAHIP_ERANGE = -3,    /* tensor has 2^31 or more elements */
+  NBLAHIP_EALIAS = -4     /* output overlaps an input it must not overlap */
+};
+
+/* Human-readable text for a status (negative) or hipError_t (positive). */
+NBLAHIP_EXPORT const char *nblahip_error_string(int code);
+/* ABI version: bumps when a signature changes. */
+NBLAHIP_EXPORT int nblahip_abi_version(void);
+
+/* ------------------------------------------------------------------------
+ * BatchNormalization.  x is viewed as [size0, size1, size2] with size1 = C the
+ * normalised axis (src/nbla/cuda/function/generic/batch_normalization.cu:34-35,
+ * 53-55); size2 == 1 is the channel-last layout.  N = size0*size2.
+ * ---------------------------------------------------------------------- */
+
+/* Replaces forward_impl_global + forward_global_kernel
+ * (batch_normalization.cu:175-199, kernel/batch_normalization.cuh:332-349):
+ *   y = (x - rm[c]) * gamma[c] / sqrt(rv[c] + eps) + beta[c]. */
+NBLAHIP_EXPORT int nblahip_bn_fwd_infer(const void *x, const float *rmean,
+                                        const float *rvar, const float *gamma,
+                                        const float *beta, void *y,
+                                        int64_t size0, int64_t size1,
+                                        int64_t size2, float eps, int dtype,
+                                        void *stream);
+
+NBLAHIP_EXPORT size_t nblahip_bn_workspace_bytes(int64_t size0, int64_t size1,
+                                                 int64_t size2, int dtype);
+
+/* Replaces forward_impl_batch -> forward_batch_parallel_reduction
+ * (batch_normalization.cu:109-172, generic/kernel/batch_normalization.cu:64-111,
+ * kernels cuh:259-325) and the cuDNN ForwardTraining(Ex) call of the cudnn
+ * context (cudnn/function/generic/batch_normalization.cu:171-261):
+ *   batch_mean[c], batch_var[c] (biased) are always written (they are the
+ *   saved statistics backward needs);
+ *   rmean <- d*rmean + (1-d)*mean, rvar <- d*rvar + (1-d)*var*N/(N-1) when the
+ *   pointers are non-NULL (NULL = recompute_impl, no running-stat update);
+ *   y = (x-mean)*gamma/sqrt(var+eps)+beta. */
+NBLAHIP_EXPORT int nblahip_bn_fwd_train(const void *x, const float *gamma,
+                                        const float *beta, void *y,
+                                        float *batch_mean, float *batch_var,
+                                        float *rmean, float *rvar,
+                                        int64_t size0, int64_t size1,
+                                        int64_t size2, float decay_rate,
+                                        float eps, int dtype, void *workspace,
+                                        size_t workspace_bytes, void *stream);
+
+/* Replaces backward_impl_batch (batch_normalization.cu:215-316, kernels
+ * cuh:402-540) and cudnnBatchNormalizationBackward(Ex)
+ * (cudnn/.../batch_normalization.cu:328-457).  mean/var are the statistics the
+ * forward used: the batch statistics when batch_stat != 0, the running ones
+ * otherwise (inference-mode backward: statistics are constants, so
+ * dx = dy*gamma/sqrt(var+eps)).  dmean/dvar (3-output form) only apply to
+ * batch_stat != 0. */
+NBLAHIP_EXPORT int nblahip_bn_bwd(const void *x, const void *dy,
+                                  const float *gamma, const float *mean,
+                                  const float *var, const float *dmean,
+                                  const float *dvar, void *dx, float *dgamma,
+                                  float *dbeta, int accum_dx, int accum_dgamma,
+                                  int accum_dbeta, int64_t size0, int64_t size1,
+                                  int64_t size2, float eps, int batch_stat,
+                                  int dtype, void *workspace,
+                                  size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------
+ * LayerNormalization.  x viewed as [outer, reduce]
+ * (src/nbla/cuda/function/generic/layer_normalization.cu:53-59).
+ * ---------------------------------------------------------------------- */
+
+/* Replaces forward_impl (layer_normalization.cu:77-133): reduce_2d_x<WelfordOp>
+ * + layer_norm_forward_normalization.  mean[outer], var[outer] (biased) are
+ * always written. gamma/beta have `reduce` elements. */
+NBLAHIP_EXPORT int nblahip_ln_fwd(const void *x, const float *gamma,
+                                  const float *beta, void *y, float *mean,
+                                  float *var, int64_t outer, int64_t reduce,
+                                  float eps, int dtype, void *stream);
+
+NBLAHIP_EXPORT size_t nblahip_ln_bwd_workspace_bytes(int64_t outer,
+                                                     int64_t reduce, int dtype);
+
+/* Replaces backward_impl (layer_normalization.cu:136-279): the four launches
+ * reduce_2d_x<LNGradOp>, ..._dx_factor, ..._dx, ..._dbeta_dgamma. */
+NBLAHIP_EXPORT int nblahip_ln_bwd(const void *x, const void *dy,
+                                  const float *gamma, const float *mean,
+                                  const float *var, const float *dmean,
+                                  const float *dvar, void *dx, float *dgamma,
+                                  float *dbeta, int accum_dx, int accum_dgamma,
+                                  int accum_dbeta, int64_t outer,
+                                  int64_t reduce, float eps, int dtype,
+                                  void *workspace, size_t workspace_bytes,
+                                  void *stream);
+
+/* ------------------------------------------------------------------------
+ * GroupNormalization.  x viewed as [batch, channels, spatial] (channel-first),
+ * statistics per (n, group) over (channels/groups)*spatial elements
+ * (src/nbla/cuda/function/generic/group_normalization.cu:57-62).  gamma/beta
+ * have `channels` elements.
+ * ---------------------------------------------------------------------- */
+
+/* Replaces forward_channel_first (group_normalization.cu:112-186): Welford,
+ * normalization_factor and normalization launches.  mean/var: [batch*groups]. */
+NBLAHIP_EXPORT int nblahip_gn_fwd(const void *x, const float *gamma,
+                                  const float *beta, void *y, float *mean,
+                                  float *var, int64_t batch, int64_t channels,
+                                  int64_t spatial, int groups, float eps,
+                                  int dtype, void *stream);
+
+NBLAHIP_EXPORT size_t nblahip_gn_bwd_workspace_bytes(int64_t batch,
+                                                     int64_t channels,
+                                                     int64_t spatial,
+                                                     int groups, int dtype);
+
+/* Replaces backward_channel_first (group_normalization.cu:227-398): the five
+ * launches GNGradOp reduce, gamma_invstd, dx_factor, dx, dbeta_dgamma. */
+NBLAHIP_EXPORT int nblahip_gn_bwd(const void *x, const void *dy,
+                                  const float *gamma, const float *mean,
+                                  const float *var, const float *dmean,
+                                  const float *dvar, void *dx, float *dgamma,
+                                  float *dbeta, int accum_dx, int accum_dgamma,
+                                  int accum_dbeta, int64_t batch,
+                                  int64_t channels, int64_t spatial, int groups,
+                                  float eps, int dtype, void *workspace,
+                                  size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------
+ * InstanceNormalization.  x viewed as [batch, channels, spatial]; statistics
+ * per (n, c) (src/nbla/cuda/function/generic/instance_normalization.cu:53-55).
+ * bc_gamma / bc_beta != 0: the parameter has `channels` elements and is
+ * broadcast over the batch (index row % channels); == 0: it has
+ * batch*channels elements (index row)
+ * (kernel/instance_normalization.cuh:37-38).
+ * ---------------------------------------------------------------------- */
+
+/* Replaces forward_channel_first (instance_normalization.cu:99-174). */
+NBLAHIP_EXPORT int nblahip_in_fwd(const void *x, const float *gamma,
+                                  const float *beta, void *y, float *mean,
+                                  float *var, int64_t batch, int64_t channels,
+                                  int64_t spatial, int bc_gamma, int bc_beta,
+                                  float eps, int dtype, void *stream);
+
+NBLAHIP_EXPORT size_t nblahip_in_bwd_workspace_bytes(int64_t batch,
+                                                     int64_t channels,
+                                                     int64_t spatial,
+                                                     int dtype);
+
+/* Replaces backward_channel_first (instance_normalization.cu:203-465) including
+ * the broadcast-backward sum over the batch (device_sum, :427-464). */
+NBLAHIP_EXPORT int nblahip_in_bwd(const void *x, const void *dy,
+                                  const float *gamma, const float *mean,
+                                  const float *var, const float *dmean,
+                                  const float *dvar, void *dx, float *dgamma,
+                                  float *dbeta, int accum_dx, int accum_dgamma,
+                                  int accum_dbeta, int64_t batch,
+                                  int64_t channels, int64_t spatial,
+                                  int bc_gamma, int bc_beta, float eps,
+                                  int dtype, void *workspace,
+                                  size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------
+ * Runtime shims used by the backend's array class and singleton so that host
+ * C++ never includes a HIP header.  They replace the cudaMalloc / cudaMemcpy /
+ * cudaMemset / dtype-converting copy paths of src/nbla/cuda/memory/
+ * cuda_memory.cpp:51-75 and src/nbla/cuda/array/cuda_array.cpp:211-347, and
+ * cuda_set_device / device synchronisation of src/nbla/cuda/common.cpp:20-32,
+ * src/nbla/cuda/cuda.cpp (Cuda::device_synchronize).
+ * ---------------------------------------------------------------------- */
+NBLAHIP_EXPORT int nblahip_device_count(int *count);
+NBLAHIP_EXPORT int nblahip_set_device(int device);
+NBLAHIP_EXPORT int nblahip_get_device(int *device);
+NBLAHIP_EXPORT int nblahip_device_synchronize(void);
+NBLAHIP_EXPORT int nblahip_stream_synchronize(void *stream);
+/* name (up to name_len-1 chars), compute units, wavefront size, HBM bytes. */
+NBLAHIP_EXPORT int nblahip_device_info(int device, char *name, size_t name_len,
+                                       int *compute_units, int *wave_size,
+                                       size_t *total_mem);
+NBLAHIP_EXPORT int nblahip_malloc(void **ptr, size_t bytes);
+NBLAHIP_EXPORT int nblahip_free(void *ptr);
+NBLAHIP_EXPORT int nblahip_memcpy_h2d(void *dst, const void *src, size_t bytes,
+                                      void *stream);
+NBLAHIP_EXPORT int nblahip_memcpy_d2h(void *dst, const void *src, size_t bytes,
+                                      void *stream);
+NBLAHIP_EXPORT int nblahip_memcpy_d2d(void *dst, const void *src, size_t bytes,
+                                      void *stream);
+NBLAHIP_EXPORT int nblahip_memset(void *dst, int byte, size_t bytes,
+                                  void *stream);
+/* dst[i] = (dst_dtype) src[i] for n elements (float32 <-> float16). */
+NBLAHIP_EXPORT int nblahip_convert(void *dst, int dst_dtype, const void *src,
+                                   int src_dtype, int64_t n, void *stream);
+/* dst[i] = value for n elements of dtype. */
+NBLAHIP_EXPORT int nblahip_fill(void *dst, int dtype, float value, int64_t n,
+                                void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NBLAHIP_H_ */

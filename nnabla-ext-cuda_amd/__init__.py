@@ -1,0 +1,308 @@
+"""ctypes binding of the nblahip C-ABI (include/nblahip.h) for tests, the
+smoke check and the benchmark.
+
+The product is the C/C++ library; this module only hands it device pointers.
+torch supplies device memory and the current stream, nothing else: there is
+no fallback implementation here, and loading fails loudly when the HIP
+library has not been built.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libnblahip.so")
+HOST_LIB_PATH = os.path.join(_HERE, "lib", "libnnabla_hip.so")
+CSRC = os.path.join(_HERE, "csrc")
+
+F32, F16 = 0, 1
+
+_c_void_p = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+_f = ctypes.c_float
+_sz = ctypes.c_size_t
+
+# name -> (restype, argtypes); mirrors include/nblahip.h one to one.
+SIGNATURES = {
+    "nblahip_error_string": (ctypes.c_char_p, [_int]),
+    "nblahip_abi_version": (_int, []),
+    "nblahip_bn_fwd_infer": (_int, [_c_void_p] * 6 + [_i64] * 3 + [_f, _int, _c_void_p]),
+    "nblahip_bn_workspace_bytes": (_sz, [_i64] * 3 + [_int]),
+    "nblahip_bn_fwd_train": (_int, [_c_void_p] * 8 + [_i64] * 3 + [_f, _f, _int, _c_void_p, _sz,
+                                                              _c_void_p]),
+    "nblahip_bn_bwd": (_int, [_c_void_p] * 10 + [_int] * 3 + [_i64] * 3 + [_f, _int, _int,
+                                                                   _c_void_p, _sz, _c_void_p]),
+    "nblahip_ln_fwd": (_int, [_c_void_p] * 6 + [_i64] * 2 + [_f, _int, _c_void_p]),
+    "nblahip_ln_bwd_workspace_bytes": (_sz, [_i64] * 2 + [_int]),
+    "nblahip_ln_bwd": (_int, [_c_void_p] * 10 + [_int] * 3 + [_i64] * 2 + [_f, _int, _c_void_p,
+                                                                   _sz, _c_void_p]),
+    "nblahip_gn_fwd": (_int, [_c_void_p] * 6 + [_i64] * 3 + [_int, _f, _int, _c_void_p]),
+    "nblahip_gn_bwd_workspace_bytes": (_sz, [_i64] * 3 + [_int, _int]),
+    "nblahip_gn_bwd": (_int, [_c_void_p] * 10 + [_int] * 3 + [_i64] * 3 + [_int, _f, _int,
+                                                                   _c_void_p, _sz, _c_void_p]),
+    "nblahip_in_fwd": (_int, [_c_void_p] * 6 + [_i64] * 3 + [_int, _int, _f, _int, _c_void_p]),
+    "nblahip_in_bwd_workspace_bytes": (_sz, [_i64] * 3 + [_int]),
+    "nblahip_in_bwd": (_int, [_c_void_p] * 10 + [_int] * 3 + [_i64] * 3 + [_int, _int, _f, _int,
+                                                                   _c_void_p, _sz, _c_void_p]),
+    "nblahip_device_count": (_int, [ctypes.POINTER(_int)]),
+    "nblahip_set_device": (_int, [_int]),
+    "nblahip_get_device": (_int, [ctypes.POINTER(_int)]),
+    "nblahip_device_synchronize": (_int, []),
+    "nblahip_stream_synchronize": (_int, [_c_void_p]),
+    "nblahip_device_info": (_int, [_int, ctypes.c_char_p, _sz, ctypes.POINTER(_int),
+                                   ctypes.POINTER(_int), ctypes.POINTER(_sz)]),
+    "nblahip_malloc": (_int, [ctypes.POINTER(_c_void_p), _sz]),
+    "nblahip_free": (_int, [_c_void_p]),
+    "nblahip_memcpy_h2d": (_int, [_c_void_p, _c_void_p, _sz, _c_void_p]),
+    "nblahip_memcpy_d2h": (_int, [_c_void_p, _c_void_p, _sz, _c_void_p]),
+    "nblahip_memcpy_d2d": (_int, [_c_void_p, _c_void_p, _sz, _c_void_p]),
+    "nblahip_memset": (_int, [_c_void_p, _int, _sz, _c_void_p]),
+    "nblahip_convert": (_int, [_c_void_p, _int, _c_void_p, _int, _i64, _c_void_p]),
+    "nblahip_fill": (_int, [_c_void_p, _int, _f, _i64, _c_void_p]),
+}
+
+_lib = None
+
+
+class NblaHipError(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__(f"nblahip status {code}: {text}")
+        self.code = code
+
+
+def lib():
+    """The loaded libnblahip.so.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `make -C {CSRC} -j8` "
+                "(or __graft_entry__.build()); there is no fallback path")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(code):
+    if code != 0:
+        raise NblaHipError(code, lib().nblahip_error_string(code).decode())
+
+
+# ---------------------------------------------------------------------------
+# torch-tensor conveniences (device memory + current stream only)
+# ---------------------------------------------------------------------------
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dtype_code(t):
+    import torch
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.float16:
+        return F16
+    raise TypeError(f"unsupported activation dtype {t.dtype}")
+
+
+def _f32(t, name):
+    import torch
+    if t is not None and (t.dtype != torch.float32 or not t.is_contiguous()):
+        raise TypeError(f"{name} must be a contiguous float32 tensor")
+    return t
+
+
+def _workspace(nbytes, device):
+    import torch
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def _bn_sizes(shape, axis):
+    size0 = 1
+    for s in shape[:axis]:
+        size0 *= s
+    size2 = 1
+    for s in shape[axis + 1:]:
+        size2 *= s
+    return size0, shape[axis], size2
+
+
+def bn_forward_global(x, beta, gamma, rmean, rvar, axis=1, eps=1e-5):
+    import torch
+    assert x.is_contiguous()
+    s0, c, s2 = _bn_sizes(x.shape, axis)
+    y = torch.empty_like(x)
+    check(lib().nblahip_bn_fwd_infer(_ptr(x), _ptr(_f32(rmean, "rmean")), _ptr(_f32(rvar, "rvar")),
+                                     _ptr(_f32(gamma, "gamma")), _ptr(_f32(beta, "beta")), _ptr(y),
+                                     s0, c, s2, eps, _dtype_code(x), _stream()))
+    return y
+
+
+def bn_forward_batch(x, beta, gamma, rmean, rvar, axis=1, decay_rate=0.9, eps=1e-5, ws=None):
+    """Returns y, batch_mean, batch_var; rmean/rvar are updated in place."""
+    import torch
+    assert x.is_contiguous()
+    s0, c, s2 = _bn_sizes(x.shape, axis)
+    dt = _dtype_code(x)
+    y = torch.empty_like(x)
+    mean = torch.empty(c, dtype=torch.float32, device=x.device)
+    var = torch.empty(c, dtype=torch.float32, device=x.device)
+    need = lib().nblahip_bn_workspace_bytes(s0, c, s2, dt)
+    ws = ws if ws is not None else _workspace(need, x.device)
+    check(lib().nblahip_bn_fwd_train(_ptr(x), _ptr(_f32(gamma, "gamma")), _ptr(_f32(beta, "beta")),
+                                     _ptr(y), _ptr(mean), _ptr(var), _ptr(_f32(rmean, "rmean")),
+                                     _ptr(_f32(rvar, "rvar")), s0, c, s2, decay_rate, eps, dt,
+                                     _ptr(ws), ws.numel(), _stream()))
+    return y, mean, var
+
+
+def bn_backward(x, dy, gamma, mean, var, axis=1, eps=1e-5, batch_stat=True, dmean=None,
+                dvar=None, dx=None, dgamma=None, dbeta=None, accum=(False, False, False),
+                need=(True, True, True), ws=None):
+    """need = (dx, dgamma, dbeta) propagate_down flags; accum likewise.
+    Returns dx, dgamma, dbeta (None where not needed)."""
+    import torch
+    assert x.is_contiguous() and dy.is_contiguous()
+    s0, c, s2 = _bn_sizes(x.shape, axis)
+    dt = _dtype_code(x)
+    if need[0] and dx is None:
+        dx = torch.empty_like(x)
+    if need[1] and dgamma is None:
+        dgamma = torch.empty(c, dtype=torch.float32, device=x.device)
+    if need[2] and dbeta is None:
+        dbeta = torch.empty(c, dtype=torch.float32, device=x.device)
+    nbytes = lib().nblahip_bn_workspace_bytes(s0, c, s2, dt)
+    ws = ws if ws is not None else _workspace(nbytes, x.device)
+    check(lib().nblahip_bn_bwd(_ptr(x), _ptr(dy), _ptr(_f32(gamma, "gamma")), _ptr(mean), _ptr(var),
+                               _ptr(dmean), _ptr(dvar), _ptr(dx if need[0] else None),
+                               _ptr(dgamma if need[1] else None), _ptr(dbeta if need[2] else None),
+                               int(accum[0]), int(accum[1]), int(accum[2]), s0, c, s2, eps,
+                               int(batch_stat), dt, _ptr(ws), ws.numel(), _stream()))
+    return (dx if need[0] else None, dgamma if need[1] else None, dbeta if need[2] else None)
+
+
+def ln_forward(x, beta, gamma, outer, eps=1e-5):
+    import torch
+    assert x.is_contiguous()
+    reduce = x.numel() // outer if outer else 0
+    y = torch.empty_like(x)
+    mean = torch.empty(outer, dtype=torch.float32, device=x.device)
+    var = torch.empty(outer, dtype=torch.float32, device=x.device)
+    check(lib().nblahip_ln_fwd(_ptr(x), _ptr(_f32(gamma, "gamma")), _ptr(_f32(beta, "beta")),
+                               _ptr(y), _ptr(mean), _ptr(var), outer, reduce, eps, _dtype_code(x),
+                               _stream()))
+    return y, mean, var
+
+
+def ln_backward(x, dy, gamma, mean, var, outer, eps=1e-5, dmean=None, dvar=None, dx=None,
+                dgamma=None, dbeta=None, accum=(False, False, False), need=(True, True, True),
+                ws=None):
+    import torch
+    assert x.is_contiguous() and dy.is_contiguous()
+    reduce = x.numel() // outer if outer else 0
+    dt = _dtype_code(x)
+    if need[0] and dx is None:
+        dx = torch.empty_like(x)
+    if need[1] and dgamma is None:
+        dgamma = torch.empty(reduce, dtype=torch.float32, device=x.device)
+    if need[2] and dbeta is None:
+        dbeta = torch.empty(reduce, dtype=torch.float32, device=x.device)
+    nbytes = lib().nblahip_ln_bwd_workspace_bytes(outer, reduce, dt)
+    ws = ws if ws is not None else _workspace(nbytes, x.device)
+    check(lib().nblahip_ln_bwd(_ptr(x), _ptr(dy), _ptr(_f32(gamma, "gamma")), _ptr(mean), _ptr(var),
+                               _ptr(dmean), _ptr(dvar), _ptr(dx if need[0] else None),
+                               _ptr(dgamma if need[1] else None), _ptr(dbeta if need[2] else None),
+                               int(accum[0]), int(accum[1]), int(accum[2]), outer, reduce, eps, dt,
+                               _ptr(ws), ws.numel(), _stream()))
+    return (dx if need[0] else None, dgamma if need[1] else None, dbeta if need[2] else None)
+
+
+def _ncs(x):
+    n, c = x.shape[0], x.shape[1]
+    sp = 1
+    for s in x.shape[2:]:
+        sp *= s
+    return n, c, sp
+
+
+def gn_forward(x, beta, gamma, num_groups, eps=1e-5):
+    import torch
+    assert x.is_contiguous()
+    n, c, sp = _ncs(x)
+    y = torch.empty_like(x)
+    mean = torch.empty(n * num_groups, dtype=torch.float32, device=x.device)
+    var = torch.empty(n * num_groups, dtype=torch.float32, device=x.device)
+    check(lib().nblahip_gn_fwd(_ptr(x), _ptr(_f32(gamma, "gamma")), _ptr(_f32(beta, "beta")),
+                               _ptr(y), _ptr(mean), _ptr(var), n, c, sp, num_groups, eps,
+                               _dtype_code(x), _stream()))
+    return y, mean, var
+
+
+def gn_backward(x, dy, gamma, mean, var, num_groups, eps=1e-5, dmean=None, dvar=None, dx=None,
+                dgamma=None, dbeta=None, accum=(False, False, False), need=(True, True, True),
+                ws=None):
+    import torch
+    assert x.is_contiguous() and dy.is_contiguous()
+    n, c, sp = _ncs(x)
+    dt = _dtype_code(x)
+    if need[0] and dx is None:
+        dx = torch.empty_like(x)
+    if need[1] and dgamma is None:
+        dgamma = torch.empty(c, dtype=torch.float32, device=x.device)
+    if need[2] and dbeta is None:
+        dbeta = torch.empty(c, dtype=torch.float32, device=x.device)
+    nbytes = lib().nblahip_gn_bwd_workspace_bytes(n, c, sp, num_groups, dt)
+    ws = ws if ws is not None else _workspace(nbytes, x.device)
+    check(lib().nblahip_gn_bwd(_ptr(x), _ptr(dy), _ptr(_f32(gamma, "gamma")), _ptr(mean), _ptr(var),
+                               _ptr(dmean), _ptr(dvar), _ptr(dx if need[0] else None),
+                               _ptr(dgamma if need[1] else None), _ptr(dbeta if need[2] else None),
+                               int(accum[0]), int(accum[1]), int(accum[2]), n, c, sp, num_groups,
+                               eps, dt, _ptr(ws), ws.numel(), _stream()))
+    return (dx if need[0] else None, dgamma if need[1] else None, dbeta if need[2] else None)
+
+
+def in_forward(x, beta, gamma, eps=1e-5, bc_gamma=True, bc_beta=True):
+    import torch
+    assert x.is_contiguous()
+    n, c, sp = _ncs(x)
+    y = torch.empty_like(x)
+    mean = torch.empty(n * c, dtype=torch.float32, device=x.device)
+    var = torch.empty(n * c, dtype=torch.float32, device=x.device)
+    check(lib().nblahip_in_fwd(_ptr(x), _ptr(_f32(gamma, "gamma")), _ptr(_f32(beta, "beta")),
+                               _ptr(y), _ptr(mean), _ptr(var), n, c, sp, int(bc_gamma),
+                               int(bc_beta), eps, _dtype_code(x), _stream()))
+    return y, mean, var
+
+
+def in_backward(x, dy, gamma, mean, var, eps=1e-5, bc_gamma=True, bc_beta=True, dmean=None,
+                dvar=None, dx=None, dgamma=None, dbeta=None, accum=(False, False, False),
+                need=(True, True, True), ws=None):
+    import torch
+    assert x.is_contiguous() and dy.is_contiguous()
+    n, c, sp = _ncs(x)
+    dt = _dtype_code(x)
+    if need[0] and dx is None:
+        dx = torch.empty_like(x)
+    if need[1] and dgamma is None:
+        dgamma = torch.empty(c if bc_gamma else n * c, dtype=torch.float32, device=x.device)
+    if need[2] and dbeta is None:
+        dbeta = torch.empty(c if bc_beta else n * c, dtype=torch.float32, device=x.device)
+    nbytes = lib().nblahip_in_bwd_workspace_bytes(n, c, sp, dt)
+    ws = ws if ws is not None else _workspace(nbytes, x.device)
+    check(lib().nblahip_in_bwd(_ptr(x), _ptr(dy), _ptr(_f32(gamma, "gamma")), _ptr(mean), _ptr(var),
+                               _ptr(dmean), _ptr(dvar), _ptr(dx if need[0] else None),
+                               _ptr(dgamma if need[1] else None), _ptr(dbeta if need[2] else None),
+                               int(accum[0]), int(accum[1]), int(accum[2]), n, c, sp,
+                               int(bc_gamma), int(bc_beta), eps, dt, _ptr(ws), ws.numel(),
+                               _stream()))
+    return (dx if need[0] else None, dgamma if need[1] else None, dbeta if need[2] else None)

@@ -1,0 +1,348 @@
+// C-ABI entry points of the normalization kernels: argument validation and
+// translation into launch-layer problems.  Nothing here allocates, throws or
+// waits for the device.
+#include "launch.hpp"
+
+using namespace nblahip;
+
+namespace {
+
+constexpr int64_t kMaxElems = (1ll << 31) - 1;
+
+bool dtype_ok(int d) { return d == NBLAHIP_F32 || d == NBLAHIP_F16; }
+
+int check_ws(const void *ws, size_t have, size_t need) {
+  if (need == 0) return 0;
+  if (!ws || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0 || have < need) return NBLAHIP_EWORKSPACE;
+  return 0;
+}
+
+// 0: proceed; 1: empty tensor, nothing to do; <0: error.
+int check_dims3(int64_t a, int64_t b, int64_t c) {
+  if (a < 0 || b < 0 || c < 0) return NBLAHIP_EINVAL;
+  if (a == 0 || b == 0 || c == 0) return 1;
+  if (a > kMaxElems || b > kMaxElems || c > kMaxElems) return NBLAHIP_ERANGE;
+  const __int128 total = static_cast<__int128>(a) * b * c;
+  if (total > kMaxElems) return NBLAHIP_ERANGE;
+  return 0;
+}
+
+hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
+
+} // namespace
+
+extern "C" {
+
+// ----------------------------------------------------------------------------
+// BatchNormalization
+// ----------------------------------------------------------------------------
+int nblahip_bn_fwd_infer(const void *x, const float *rmean, const float *rvar,
+                         const float *gamma, const float *beta, void *y, int64_t size0,
+                         int64_t size1, int64_t size2, float eps, int dtype, void *stream) {
+  if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
+  const int d = check_dims3(size0, size1, size2);
+  if (d) return d < 0 ? d : 0;
+  if (!x || !y || !rmean || !rvar) return NBLAHIP_EINVAL;
+  BnProblem p;
+  p.dtype = dtype;
+  p.x = x;
+  p.out = y;
+  p.mean = rmean;
+  p.var = rvar;
+  p.gamma = gamma;
+  p.beta = beta;
+  p.size0 = size0;
+  p.C = size1;
+  p.size2 = size2;
+  p.eps = eps;
+  return launch_bn_infer(p, as_stream(stream));
+}
+
+size_t nblahip_bn_workspace_bytes(int64_t size0, int64_t size1, int64_t size2, int dtype) {
+  if (!dtype_ok(dtype) || check_dims3(size0, size1, size2) != 0) return 0;
+  return bn_workspace_bytes(size0, size1, size2, dtype);
+}
+
+int nblahip_bn_fwd_train(const void *x, const float *gamma, const float *beta, void *y,
+                         float *batch_mean, float *batch_var, float *rmean, float *rvar,
+                         int64_t size0, int64_t size1, int64_t size2, float decay_rate, float eps,
+                         int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+  if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
+  const int d = check_dims3(size0, size1, size2);
+  if (d) return d < 0 ? d : 0;
+  if (!x || !y || !batch_mean || !batch_var) return NBLAHIP_EINVAL;
+  if (int e = check_ws(workspace, workspace_bytes, bn_workspace_bytes(size0, size1, size2, dtype)))
+    return e;
+  BnProblem p;
+  p.dtype = dtype;
+  p.x = x;
+  p.out = y;
+  p.gamma = gamma;
+  p.beta = beta;
+  p.batch_mean = batch_mean;
+  p.batch_var = batch_var;
+  p.rmean = rmean;
+  p.rvar = rvar;
+  p.size0 = size0;
+  p.C = size1;
+  p.size2 = size2;
+  p.decay = decay_rate;
+  p.eps = eps;
+  p.ws = workspace;
+  p.ws_bytes = workspace_bytes;
+  return launch_bn_fwd_train(p, as_stream(stream));
+}
+
+int nblahip_bn_bwd(const void *x, const void *dy, const float *gamma, const float *mean,
+                   const float *var, const float *dmean, const float *dvar, void *dx,
+                   float *dgamma, float *dbeta, int accum_dx, int accum_dgamma, int accum_dbeta,
+                   int64_t size0, int64_t size1, int64_t size2, float eps, int batch_stat,
+                   int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+  if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
+  const int d = check_dims3(size0, size1, size2);
+  if (d) return d < 0 ? d : 0;
+  if (!x || !dy || !mean || !var) return NBLAHIP_EINVAL;
+  if (int e = check_ws(workspace, workspace_bytes, bn_workspace_bytes(size0, size1, size2, dtype)))
+    return e;
+  BnProblem p;
+  p.dtype = dtype;
+  p.x = x;
+  p.dy = dy;
+  p.out = dx;
+  p.gamma = gamma;
+  p.mean = mean;
+  p.var = var;
+  p.dmean = batch_stat ? dmean : nullptr;
+  p.dvar = batch_stat ? dvar : nullptr;
+  p.dgamma = dgamma;
+  p.dbeta = dbeta;
+  p.accum_dx = accum_dx;
+  p.accum_g = accum_dgamma;
+  p.accum_b = accum_dbeta;
+  p.batch_stat = batch_stat;
+  p.size0 = size0;
+  p.C = size1;
+  p.size2 = size2;
+  p.eps = eps;
+  p.ws = workspace;
+  p.ws_bytes = workspace_bytes;
+  return launch_bn_bwd(p, as_stream(stream));
+}
+
+// ----------------------------------------------------------------------------
+// LayerNormalization
+// ----------------------------------------------------------------------------
+int nblahip_ln_fwd(const void *x, const float *gamma, const float *beta, void *y, float *mean,
+                   float *var, int64_t outer, int64_t reduce, float eps, int dtype,
+                   void *stream) {
+  if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
+  const int d = check_dims3(outer, reduce, 1);
+  if (d) return d < 0 ? d : 0;
+  if (!x || !y || !mean || !var) return NBLAHIP_EINVAL;
+  RowProblem p;
+  p.dtype = dtype;
+  p.mode = kRowLN;
+  p.x = x;
+  p.out = y;
+  p.gamma = gamma;
+  p.beta = beta;
+  p.mean = mean;
+  p.var = var;
+  p.rows = outer;
+  p.R = reduce;
+  p.eps = eps;
+  return launch_row_fwd(p, as_stream(stream));
+}
+
+size_t nblahip_ln_bwd_workspace_bytes(int64_t outer, int64_t reduce, int dtype) {
+  if (!dtype_ok(dtype) || check_dims3(outer, reduce, 1) != 0) return 0;
+  return row_bwd_workspace_bytes(kRowLN, outer, reduce, 0);
+}
+
+int nblahip_ln_bwd(const void *x, const void *dy, const float *gamma, const float *mean,
+                   const float *var, const float *dmean, const float *dvar, void *dx,
+                   float *dgamma, float *dbeta, int accum_dx, int accum_dgamma, int accum_dbeta,
+                   int64_t outer, int64_t reduce, float eps, int dtype, void *workspace,
+                   size_t workspace_bytes, void *stream) {
+  if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
+  const int d = check_dims3(outer, reduce, 1);
+  if (d) return d < 0 ? d : 0;
+  if (!x || !dy || !mean || !var) return NBLAHIP_EINVAL;
+  if (int e = check_ws(workspace, workspace_bytes, row_bwd_workspace_bytes(kRowLN, outer, reduce, 0)))
+    return e;
+  RowProblem p;
+  p.dtype = dtype;
+  p.mode = kRowLN;
+  p.x = x;
+  p.dy = dy;
+  p.out = dx;
+  p.gamma = gamma;
+  p.mean = const_cast<float *>(mean);
+  p.var = const_cast<float *>(var);
+  p.dmean = dmean;
+  p.dvar = dvar;
+  p.dgamma = dgamma;
+  p.dbeta = dbeta;
+  p.accum_dx = accum_dx;
+  p.accum_g = accum_dgamma;
+  p.accum_b = accum_dbeta;
+  p.rows = outer;
+  p.R = reduce;
+  p.eps = eps;
+  p.ws = workspace;
+  p.ws_bytes = workspace_bytes;
+  return launch_row_bwd(p, as_stream(stream));
+}
+
+// ----------------------------------------------------------------------------
+// GroupNormalization
+// ----------------------------------------------------------------------------
+static int gn_problem(RowProblem &p, int64_t batch, int64_t channels, int64_t spatial, int groups,
+                      int dtype) {
+  if (!dtype_ok(dtype) || groups <= 0) return NBLAHIP_EINVAL;
+  const int d = check_dims3(batch, channels, spatial);
+  if (d) return d;
+  if (channels % groups != 0) return NBLAHIP_EINVAL;
+  p.dtype = dtype;
+  p.mode = kRowGN;
+  p.batch = batch;
+  p.channels = channels;
+  p.spatial = spatial;
+  p.groups = groups;
+  p.rows = batch * groups;
+  p.R = (channels / groups) * spatial;
+  return 0;
+}
+
+int nblahip_gn_fwd(const void *x, const float *gamma, const float *beta, void *y, float *mean,
+                   float *var, int64_t batch, int64_t channels, int64_t spatial, int groups,
+                   float eps, int dtype, void *stream) {
+  RowProblem p;
+  const int d = gn_problem(p, batch, channels, spatial, groups, dtype);
+  if (d) return d < 0 ? d : 0;
+  if (!x || !y || !mean || !var) return NBLAHIP_EINVAL;
+  p.x = x;
+  p.out = y;
+  p.gamma = gamma;
+  p.beta = beta;
+  p.mean = mean;
+  p.var = var;
+  p.eps = eps;
+  return launch_row_fwd(p, as_stream(stream));
+}
+
+size_t nblahip_gn_bwd_workspace_bytes(int64_t batch, int64_t channels, int64_t spatial,
+                                      int groups, int dtype) {
+  RowProblem p;
+  if (gn_problem(p, batch, channels, spatial, groups, dtype) != 0) return 0;
+  return row_bwd_workspace_bytes(kRowGN, p.rows, p.R, batch * channels);
+}
+
+int nblahip_gn_bwd(const void *x, const void *dy, const float *gamma, const float *mean,
+                   const float *var, const float *dmean, const float *dvar, void *dx,
+                   float *dgamma, float *dbeta, int accum_dx, int accum_dgamma, int accum_dbeta,
+                   int64_t batch, int64_t channels, int64_t spatial, int groups, float eps,
+                   int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+  RowProblem p;
+  const int d = gn_problem(p, batch, channels, spatial, groups, dtype);
+  if (d) return d < 0 ? d : 0;
+  if (!x || !dy || !mean || !var) return NBLAHIP_EINVAL;
+  if (int e = check_ws(workspace, workspace_bytes,
+                       row_bwd_workspace_bytes(kRowGN, p.rows, p.R, batch * channels)))
+    return e;
+  p.x = x;
+  p.dy = dy;
+  p.out = dx;
+  p.gamma = gamma;
+  p.mean = const_cast<float *>(mean);
+  p.var = const_cast<float *>(var);
+  p.dmean = dmean;
+  p.dvar = dvar;
+  p.dgamma = dgamma;
+  p.dbeta = dbeta;
+  p.accum_dx = accum_dx;
+  p.accum_g = accum_dgamma;
+  p.accum_b = accum_dbeta;
+  p.eps = eps;
+  p.ws = workspace;
+  p.ws_bytes = workspace_bytes;
+  return launch_row_bwd(p, as_stream(stream));
+}
+
+// ----------------------------------------------------------------------------
+// InstanceNormalization
+// ----------------------------------------------------------------------------
+static int in_problem(RowProblem &p, int64_t batch, int64_t channels, int64_t spatial,
+                      int bc_gamma, int bc_beta, int dtype) {
+  if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
+  const int d = check_dims3(batch, channels, spatial);
+  if (d) return d;
+  p.dtype = dtype;
+  p.mode = kRowIN;
+  p.batch = batch;
+  p.channels = channels;
+  p.spatial = spatial;
+  p.groups = static_cast<int>(channels);
+  p.bc_gamma = bc_gamma != 0;
+  p.bc_beta = bc_beta != 0;
+  p.rows = batch * channels;
+  p.R = spatial;
+  return 0;
+}
+
+int nblahip_in_fwd(const void *x, const float *gamma, const float *beta, void *y, float *mean,
+                   float *var, int64_t batch, int64_t channels, int64_t spatial, int bc_gamma,
+                   int bc_beta, float eps, int dtype, void *stream) {
+  RowProblem p;
+  const int d = in_problem(p, batch, channels, spatial, bc_gamma, bc_beta, dtype);
+  if (d) return d < 0 ? d : 0;
+  if (!x || !y || !mean || !var) return NBLAHIP_EINVAL;
+  p.x = x;
+  p.out = y;
+  p.gamma = gamma;
+  p.beta = beta;
+  p.mean = mean;
+  p.var = var;
+  p.eps = eps;
+  return launch_row_fwd(p, as_stream(stream));
+}
+
+size_t nblahip_in_bwd_workspace_bytes(int64_t batch, int64_t channels, int64_t spatial,
+                                      int dtype) {
+  RowProblem p;
+  if (in_problem(p, batch, channels, spatial, 1, 1, dtype) != 0) return 0;
+  return row_bwd_workspace_bytes(kRowIN, p.rows, p.R, batch * channels);
+}
+
+int nblahip_in_bwd(const void *x, const void *dy, const float *gamma, const float *mean,
+                   const float *var, const float *dmean, const float *dvar, void *dx,
+                   float *dgamma, float *dbeta, int accum_dx, int accum_dgamma, int accum_dbeta,
+                   int64_t batch, int64_t channels, int64_t spatial, int bc_gamma, int bc_beta,
+                   float eps, int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+  RowProblem p;
+  const int d = in_problem(p, batch, channels, spatial, bc_gamma, bc_beta, dtype);
+  if (d) return d < 0 ? d : 0;
+  if (!x || !dy || !mean || !var) return NBLAHIP_EINVAL;
+  if (int e = check_ws(workspace, workspace_bytes,
+                       row_bwd_workspace_bytes(kRowIN, p.rows, p.R, batch * channels)))
+    return e;
+  p.x = x;
+  p.dy = dy;
+  p.out = dx;
+  p.gamma = gamma;
+  p.mean = const_cast<float *>(mean);
+  p.var = const_cast<float *>(var);
+  p.dmean = dmean;
+  p.dvar = dvar;
+  p.dgamma = dgamma;
+  p.dbeta = dbeta;
+  p.accum_dx = accum_dx;
+  p.accum_g = accum_dgamma;
+  p.accum_b = accum_dbeta;
+  p.eps = eps;
+  p.ws = workspace;
+  p.ws_bytes = workspace_bytes;
+  return launch_row_bwd(p, as_stream(stream));
+}
+
+} // extern "C"

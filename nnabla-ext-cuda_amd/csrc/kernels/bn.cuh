@@ -1,0 +1,569 @@
+// BatchNormalization kernels.  The tensor is [size0, C, size2]; one channel's
+// N = size0*size2 values never fit on chip, so both directions are split
+// reductions:
+//   forward : stats partials (Welford per block) -> finalize (Chan merge,
+//             running stats, per-channel apply parameters) -> apply
+//   backward: (sum dy, sum dy*(x-mean)) partials -> finalize (dgamma, dbeta,
+//             per-channel dx coefficients) -> apply
+// Partials are merged in a fixed order (no atomics): results are reproducible.
+//
+// Two memory layouts get their own reduction kernels:
+//   "planes"       size2 > 1 : a block owns one channel and a slice of its
+//                  size0 planes; lanes run along the contiguous plane.
+//   "channel-last" size2 == 1: x is [M, C]; a lane owns VEC adjacent channels,
+//                  TX lanes span a row segment, TY = 256/TX rows per step.
+#pragma once
+
+#include "common.cuh"
+
+namespace nblahip {
+
+constexpr int kBnBlock = 256;
+constexpr int kBnUnroll = 4;
+
+// Per-channel parameters of the forward apply step: y = (x - mean)*scale + shift.
+// Per-channel parameters of the backward apply step:
+//   dx = c1*dy + c2*(x - mean) + c3.
+struct __align__(16) BnParam {
+  float mean, a, b, c;
+};
+
+// ---------------------------------------------------------------------------
+// Forward statistics, planes layout.  grid = (C, S).
+// vpc = vectors per channel = size0 * nvp; split s covers vectors
+// [s*chunk, min((s+1)*chunk, vpc)).
+// ---------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ void __launch_bounds__(kBnBlock)
+bn_stats_planes_kernel(const T *__restrict__ x, uint32_t C, FastDiv nvp, uint32_t vpc,
+                       uint32_t chunk, float *__restrict__ part /*[C][S][3]*/) {
+  __shared__ float lds[3 * (kBnBlock / kWave)];
+  const uint32_t c = blockIdx.x;
+  const uint32_t s = blockIdx.y;
+  const uint32_t S = gridDim.y;
+  const uint32_t begin = s * chunk;
+  const uint32_t end = min(begin + chunk, vpc);
+  Welford w{0.f, 0.f, 0.f};
+  for (uint32_t v0 = begin + threadIdx.x; v0 < end; v0 += kBnBlock * kBnUnroll) {
+    float vals[kBnUnroll * VEC];
+    int cnt = 0;
+#pragma unroll
+    for (int u = 0; u < kBnUnroll; ++u) {
+      const uint32_t v = v0 + u * kBnBlock;
+      float tmp[VEC];
+      if (v < end) {
+        const uint32_t n = nvp.div(v);
+        const uint32_t i = v - n * nvp.d;
+        const size_t off = (static_cast<size_t>(n) * C + c) * nvp.d + i;
+        load_vec<T, VEC>(x + off * VEC, tmp);
+        cnt += VEC;
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) tmp[j] = 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) vals[u * VEC + j] = tmp[j];
+    }
+    welford_add_chunk<kBnUnroll * VEC>(w, vals, cnt);
+  }
+  w = block_welford(w, lds);
+  if (threadIdx.x == 0) {
+    float *p = part + 3 * (static_cast<size_t>(c) * S + s);
+    p[0] = w.mean;
+    p[1] = w.m2;
+    p[2] = w.n;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Forward statistics, channel-last layout x[M][C].  grid = (ceil(ncv/TX), S),
+// ncv = C/VEC.  Split s covers rows [s*rps, min((s+1)*rps, M)).
+// ---------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ void __launch_bounds__(kBnBlock)
+bn_stats_cl_kernel(const T *__restrict__ x, uint32_t M, uint32_t C, uint32_t ncv,
+                   uint32_t log2tx, uint32_t rps, float *__restrict__ part /*[C][S][3]*/) {
+  // [TY][TX*VEC] means and m2 plus [TY][TX] counts; TY*TX == 256.
+  __shared__ float lmean[kBnBlock * VEC];
+  __shared__ float lm2[kBnBlock * VEC];
+  __shared__ float ln[kBnBlock];
+  const uint32_t TX = 1u << log2tx;
+  const uint32_t TY = kBnBlock >> log2tx;
+  const uint32_t tx = threadIdx.x & (TX - 1);
+  const uint32_t ty = threadIdx.x >> log2tx;
+  const uint32_t cv = blockIdx.x * TX + tx;
+  const bool active = cv < ncv;
+  const uint32_t S = gridDim.y;
+  const uint32_t s = blockIdx.y;
+  const uint32_t rbegin = s * rps;
+  const uint32_t rend = min(rbegin + rps, M);
+
+  float mean[VEC], m2[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) mean[j] = m2[j] = 0.f;
+  float n = 0.f;
+
+  if (active) {
+    for (uint32_t r0 = rbegin + ty; r0 < rend; r0 += TY * kBnUnroll) {
+      float vals[kBnUnroll][VEC];
+      int cnt = 0;
+#pragma unroll
+      for (int u = 0; u < kBnUnroll; ++u) {
+        const uint32_t r = r0 + u * TY;
+        if (r < rend) {
+          load_vec<T, VEC>(x + (static_cast<size_t>(r) * C + static_cast<size_t>(cv) * VEC), vals[u]);
+          ++cnt;
+        } else {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) vals[u][j] = 0.f;
+        }
+      }
+      // cnt >= 1 here.  Chunk statistics per channel, then one Chan merge.
+      const float fc = static_cast<float>(cnt);
+      const float nn = n + fc;
+      const float wb = fc / nn;          // weight of the chunk mean
+      const float wd = n * wb;           // n_a*n_b/(n_a+n_b)
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        float sum = 0.f;
+#pragma unroll
+        for (int u = 0; u < kBnUnroll; ++u) sum += vals[u][j];
+        const float cm = sum / fc;
+        float cm2 = 0.f;
+#pragma unroll
+        for (int u = 0; u < kBnUnroll; ++u) {
+          const float d = vals[u][j] - cm;
+          cm2 += (u < cnt) ? d * d : 0.f;
+        }
+        const float d = cm - mean[j];
+        mean[j] += d * wb;
+        m2[j] += cm2 + d * d * wd;
+      }
+      n = nn;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    lmean[(ty * TX + tx) * VEC + j] = mean[j];
+    lm2[(ty * TX + tx) * VEC + j] = m2[j];
+  }
+  ln[ty * TX + tx] = n;
+  __syncthreads();
+  // Output o = tx*VEC + j of this block; fold the TY row groups in order.
+  for (uint32_t o = threadIdx.x; o < TX * VEC; o += kBnBlock) {
+    const uint32_t otx = o / VEC;
+    const uint32_t ch = blockIdx.x * TX * VEC + o;
+    if (blockIdx.x * TX + otx < ncv) {
+      Welford w{0.f, 0.f, 0.f};
+      for (uint32_t y = 0; y < TY; ++y) {
+        const Welford b{lmean[y * TX * VEC + o], lm2[y * TX * VEC + o], ln[y * TX + otx]};
+        w = welford_merge(w, b);
+      }
+      float *p = part + 3 * (static_cast<size_t>(ch) * S + s);
+      p[0] = w.mean;
+      p[1] = w.m2;
+      p[2] = w.n;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Forward finalize: one block per channel merges its S partials.
+//   mean, var (biased) -> batch_mean/batch_var
+//   running mean/var update (unbiased N/(N-1) factor on the running variance,
+//   the reference's kernel/batch_normalization.cuh:292-302)
+//   apply parameters {mean, gamma*istd, beta}.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(kBnBlock)
+bn_finalize_fwd_kernel(const float *__restrict__ part, uint32_t S, float inv_N,
+                       float unbias, float decay, float eps,
+                       const float *__restrict__ gamma, const float *__restrict__ beta,
+                       float *__restrict__ batch_mean, float *__restrict__ batch_var,
+                       float *__restrict__ rmean, float *__restrict__ rvar,
+                       BnParam *__restrict__ params) {
+  __shared__ float lds[3 * (kBnBlock / kWave)];
+  const uint32_t c = blockIdx.x;
+  Welford w{0.f, 0.f, 0.f};
+  for (uint32_t s = threadIdx.x; s < S; s += kBnBlock) {
+    const float *p = part + 3 * (static_cast<size_t>(c) * S + s);
+    w = welford_merge(w, Welford{p[0], p[1], p[2]});
+  }
+  w = block_welford(w, lds);
+  if (threadIdx.x == 0) {
+    const float mean = w.mean;
+    const float var = w.m2 * inv_N;
+    batch_mean[c] = mean;
+    batch_var[c] = var;
+    if (rmean) rmean[c] = decay * rmean[c] + (1.f - decay) * mean;
+    if (rvar) rvar[c] = decay * rvar[c] + (1.f - decay) * var * unbias;
+    BnParam q;
+    q.mean = mean;
+    q.a = (gamma ? gamma[c] : 1.f) * inv_std(var, eps);
+    q.b = beta ? beta[c] : 0.f;
+    q.c = 0.f;
+    params[c] = q;
+  }
+}
+
+// Inference: apply parameters straight from the running statistics.
+__global__ void __launch_bounds__(256)
+bn_infer_params_kernel(uint32_t C, float eps, const float *__restrict__ rmean,
+                       const float *__restrict__ rvar, const float *__restrict__ gamma,
+                       const float *__restrict__ beta, BnParam *__restrict__ params) {
+  const uint32_t c = blockIdx.x * 256u + threadIdx.x;
+  if (c < C) {
+    BnParam q;
+    q.mean = rmean[c];
+    q.a = (gamma ? gamma[c] : 1.f) * inv_std(rvar[c], eps);
+    q.b = beta ? beta[c] : 0.f;
+    q.c = 0.f;
+    params[c] = q;
+  }
+}
+
+// How the apply kernels obtain a channel's parameters.
+//   params != null : precomputed by a finalize kernel
+//   params == null : inference, computed on the fly from running statistics
+struct BnParamSrc {
+  const BnParam *params;
+  const float *rmean, *rvar, *gamma, *beta;
+  float eps;
+  __device__ __forceinline__ BnParam get(uint32_t c) const {
+    if (params) return params[c];
+    BnParam q;
+    q.mean = rmean[c];
+    q.a = (gamma ? gamma[c] : 1.f) * inv_std(rvar[c], eps);
+    q.b = beta ? beta[c] : 0.f;
+    q.c = 0.f;
+    return q;
+  }
+};
+
+// ---------------------------------------------------------------------------
+// Forward apply, planes layout, flattened over all vectors of the tensor.
+// plane = i / nvp, c = plane % C.
+// ---------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+bn_apply_planes_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
+                       FastDiv nvp, FastDiv cdiv, uint32_t total_vec) {
+  for (uint32_t i0 = blockIdx.x * (256u * kBnUnroll) + threadIdx.x; i0 < total_vec;
+       i0 += gridDim.x * (256u * kBnUnroll)) {
+    float v[kBnUnroll][VEC];
+#pragma unroll
+    for (int u = 0; u < kBnUnroll; ++u) {
+      const uint32_t i = i0 + u * 256u;
+      if (i < total_vec) load_vec<T, VEC>(x + static_cast<size_t>(i) * VEC, v[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < kBnUnroll; ++u) {
+      const uint32_t i = i0 + u * 256u;
+      if (i < total_vec) {
+        const uint32_t plane = nvp.div(i);
+        const uint32_t c = plane - cdiv.div(plane) * cdiv.d;
+        const BnParam q = src.get(c);
+        float o[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) o[j] = (v[u][j] - q.mean) * q.a + q.b;
+        store_vec<T, VEC>(y + static_cast<size_t>(i) * VEC, o);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Forward apply, channel-last with ncv = C/VEC dividing 256: a thread always
+// meets the same VEC channels, so their parameters live in registers.
+// ---------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+bn_apply_cl_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
+                   uint32_t ncv, uint32_t total_vec) {
+  const uint32_t cv = threadIdx.x % ncv;
+  float pm[VEC], pa[VEC], pb[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    const BnParam q = src.get(cv * VEC + j);
+    pm[j] = q.mean;
+    pa[j] = q.a;
+    pb[j] = q.b;
+  }
+  for (uint32_t i0 = blockIdx.x * (256u * kBnUnroll) + threadIdx.x; i0 < total_vec;
+       i0 += gridDim.x * (256u * kBnUnroll)) {
+    float v[kBnUnroll][VEC];
+#pragma unroll
+    for (int u = 0; u < kBnUnroll; ++u) {
+      const uint32_t i = i0 + u * 256u;
+      if (i < total_vec) load_vec<T, VEC>(x + static_cast<size_t>(i) * VEC, v[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < kBnUnroll; ++u) {
+      const uint32_t i = i0 + u * 256u;
+      if (i < total_vec) {
+        float o[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) o[j] = (v[u][j] - pm[j]) * pa[j] + pb[j];
+        store_vec<T, VEC>(y + static_cast<size_t>(i) * VEC, o);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Backward reduction, planes layout.  part2[C][S][2] = (sum dy*(x-mean), sum dy).
+// ---------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ void __launch_bounds__(kBnBlock)
+bn_bwd_reduce_planes_kernel(const T *__restrict__ x, const T *__restrict__ dy,
+                            const float *__restrict__ mean, uint32_t C, FastDiv nvp,
+                            uint32_t vpc, uint32_t chunk, float *__restrict__ part2) {
+  __shared__ float lds[2 * (kBnBlock / kWave)];
+  const uint32_t c = blockIdx.x;
+  const uint32_t s = blockIdx.y;
+  const uint32_t S = gridDim.y;
+  const uint32_t begin = s * chunk;
+  const uint32_t end = min(begin + chunk, vpc);
+  const float m = mean[c];
+  float sdx = 0.f, sdy = 0.f;
+  for (uint32_t v0 = begin + threadIdx.x; v0 < end; v0 += kBnBlock * kBnUnroll) {
+    float xv[kBnUnroll][VEC], dv[kBnUnroll][VEC];
+#pragma unroll
+    for (int u = 0; u < kBnUnroll; ++u) {
+      const uint32_t v = v0 + u * kBnBlock;
+      if (v < end) {
+        const uint32_t n = nvp.div(v);
+        const uint32_t i = v - n * nvp.d;
+        const size_t off = ((static_cast<size_t>(n) * C + c) * nvp.d + i) * VEC;
+        load_vec<T, VEC>(x + off, xv[u]);
+        load_vec<T, VEC>(dy + off, dv[u]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) xv[u][j] = dv[u][j] = 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kBnUnroll; ++u)
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        sdy += dv[u][j];
+        sdx += dv[u][j] * (xv[u][j] - m);
+      }
+  }
+  block_sum2(sdx, sdy, lds);
+  if (threadIdx.x == 0) {
+    float *p = part2 + 2 * (static_cast<size_t>(c) * S + s);
+    p[0] = sdx;
+    p[1] = sdy;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Backward reduction, channel-last.  Same thread layout as bn_stats_cl_kernel.
+// ---------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ void __launch_bounds__(kBnBlock)
+bn_bwd_reduce_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
+                        const float *__restrict__ mean, uint32_t M, uint32_t C,
+                        uint32_t ncv, uint32_t log2tx, uint32_t rps,
+                        float *__restrict__ part2 /*[C][S][2]*/) {
+  __shared__ float lsdx[kBnBlock * VEC];
+  __shared__ float lsdy[kBnBlock * VEC];
+  const uint32_t TX = 1u << log2tx;
+  const uint32_t TY = kBnBlock >> log2tx;
+  const uint32_t tx = threadIdx.x & (TX - 1);
+  const uint32_t ty = threadIdx.x >> log2tx;
+  const uint32_t cv = blockIdx.x * TX + tx;
+  const bool active = cv < ncv;
+  const uint32_t S = gridDim.y;
+  const uint32_t s = blockIdx.y;
+  const uint32_t rbegin = s * rps;
+  const uint32_t rend = min(rbegin + rps, M);
+
+  float sdx[VEC], sdy[VEC], m[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    sdx[j] = sdy[j] = 0.f;
+    m[j] = active ? mean[cv * VEC + j] : 0.f;
+  }
+  if (active) {
+    for (uint32_t r0 = rbegin + ty; r0 < rend; r0 += TY * kBnUnroll) {
+      float xv[kBnUnroll][VEC], dv[kBnUnroll][VEC];
+#pragma unroll
+      for (int u = 0; u < kBnUnroll; ++u) {
+        const uint32_t r = r0 + u * TY;
+        if (r < rend) {
+          const size_t off = static_cast<size_t>(r) * C + static_cast<size_t>(cv) * VEC;
+          load_vec<T, VEC>(x + off, xv[u]);
+          load_vec<T, VEC>(dy + off, dv[u]);
+        } else {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) xv[u][j] = dv[u][j] = 0.f;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kBnUnroll; ++u)
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          sdy[j] += dv[u][j];
+          sdx[j] += dv[u][j] * (xv[u][j] - m[j]);
+        }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    lsdx[(ty * TX + tx) * VEC + j] = sdx[j];
+    lsdy[(ty * TX + tx) * VEC + j] = sdy[j];
+  }
+  __syncthreads();
+  for (uint32_t o = threadIdx.x; o < TX * VEC; o += kBnBlock) {
+    const uint32_t otx = o / VEC;
+    const uint32_t ch = blockIdx.x * TX * VEC + o;
+    if (blockIdx.x * TX + otx < ncv) {
+      float a = 0.f, b = 0.f;
+      for (uint32_t y = 0; y < TY; ++y) {
+        a += lsdx[y * TX * VEC + o];
+        b += lsdy[y * TX * VEC + o];
+      }
+      float *p = part2 + 2 * (static_cast<size_t>(ch) * S + s);
+      p[0] = a;
+      p[1] = b;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Backward finalize (one block per channel).  With sdx = sum dy*(x-mean),
+// sdy = sum dy, g = gamma, i = istd (kernel/batch_normalization.cuh:425-469,
+// 522-540):
+//   dgamma = sdx*i, dbeta = sdy
+//   dvar   = -1/2 * g*sdx * i^3 + dv_in        dmean = -g*sdy*i + dm_in
+//   dx     = g*i*dy + (2*dvar/N)*(x-mean) + dmean/N
+// (the reference's dvar*(-2)*sum(x-mean)/N term vanishes identically).
+// batch_stat == 0: statistics are constants, dx = g*i*dy.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(kBnBlock)
+bn_finalize_bwd_kernel(const float *__restrict__ part2, uint32_t S, float inv_N, float eps,
+                       int batch_stat, const float *__restrict__ gamma,
+                       const float *__restrict__ mean, const float *__restrict__ var,
+                       const float *__restrict__ dmean_in, const float *__restrict__ dvar_in,
+                       float *__restrict__ dgamma, float *__restrict__ dbeta, int accum_g,
+                       int accum_b, BnParam *__restrict__ params) {
+  __shared__ float lds[2 * (kBnBlock / kWave)];
+  const uint32_t c = blockIdx.x;
+  float sdx = 0.f, sdy = 0.f;
+  for (uint32_t s = threadIdx.x; s < S; s += kBnBlock) {
+    const float *p = part2 + 2 * (static_cast<size_t>(c) * S + s);
+    sdx += p[0];
+    sdy += p[1];
+  }
+  block_sum2(sdx, sdy, lds);
+  if (threadIdx.x == 0) {
+    const float istd = inv_std(var[c], eps);
+    const float g = gamma ? gamma[c] : 1.f;
+    if (dgamma) dgamma[c] = sdx * istd + (accum_g ? dgamma[c] : 0.f);
+    if (dbeta) dbeta[c] = sdy + (accum_b ? dbeta[c] : 0.f);
+    BnParam q;
+    q.mean = mean[c];
+    q.a = g * istd;
+    if (batch_stat) {
+      const float dvar = -0.5f * g * sdx * istd * istd * istd + (dvar_in ? dvar_in[c] : 0.f);
+      const float dmean = -g * sdy * istd + (dmean_in ? dmean_in[c] : 0.f);
+      q.b = 2.f * dvar * inv_N;
+      q.c = dmean * inv_N;
+    } else {
+      q.b = 0.f;
+      q.c = 0.f;
+    }
+    params[c] = q;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Backward apply: dx = a*dy + b*(x-mean) + c (+ dx).
+// ---------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+bn_bwd_apply_planes_kernel(const T *__restrict__ x, const T *__restrict__ dy,
+                           T *__restrict__ dx, const BnParam *__restrict__ params,
+                           FastDiv nvp, FastDiv cdiv, uint32_t total_vec, int accum) {
+  constexpr int U = 2;
+  for (uint32_t i0 = blockIdx.x * (256u * U) + threadIdx.x; i0 < total_vec;
+       i0 += gridDim.x * (256u * U)) {
+    float xv[U][VEC], dv[U][VEC];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t i = i0 + u * 256u;
+      if (i < total_vec) {
+        load_vec<T, VEC>(x + static_cast<size_t>(i) * VEC, xv[u]);
+        load_vec<T, VEC>(dy + static_cast<size_t>(i) * VEC, dv[u]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t i = i0 + u * 256u;
+      if (i < total_vec) {
+        const uint32_t plane = nvp.div(i);
+        const uint32_t c = plane - cdiv.div(plane) * cdiv.d;
+        const BnParam q = params[c];
+        float o[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) o[j] = q.a * dv[u][j] + q.b * (xv[u][j] - q.mean) + q.c;
+        if (accum) {
+          float old[VEC];
+          load_vec<T, VEC>(dx + static_cast<size_t>(i) * VEC, old);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) o[j] += old[j];
+        }
+        store_vec<T, VEC>(dx + static_cast<size_t>(i) * VEC, o);
+      }
+    }
+  }
+}
+
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+bn_bwd_apply_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
+                       T *__restrict__ dx, const BnParam *__restrict__ params,
+                       uint32_t ncv, uint32_t total_vec, int accum) {
+  constexpr int U = 2;
+  const uint32_t cv = threadIdx.x % ncv;
+  float pm[VEC], pa[VEC], pb[VEC], pc[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    const BnParam q = params[cv * VEC + j];
+    pm[j] = q.mean;
+    pa[j] = q.a;
+    pb[j] = q.b;
+    pc[j] = q.c;
+  }
+  for (uint32_t i0 = blockIdx.x * (256u * U) + threadIdx.x; i0 < total_vec;
+       i0 += gridDim.x * (256u * U)) {
+    float xv[U][VEC], dv[U][VEC];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t i = i0 + u * 256u;
+      if (i < total_vec) {
+        load_vec<T, VEC>(x + static_cast<size_t>(i) * VEC, xv[u]);
+        load_vec<T, VEC>(dy + static_cast<size_t>(i) * VEC, dv[u]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t i = i0 + u * 256u;
+      if (i < total_vec) {
+        float o[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) o[j] = pa[j] * dv[u][j] + pb[j] * (xv[u][j] - pm[j]) + pc[j];
+        if (accum) {
+          float old[VEC];
+          load_vec<T, VEC>(dx + static_cast<size_t>(i) * VEC, old);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) o[j] += old[j];
+        }
+        store_vec<T, VEC>(dx + static_cast<size_t>(i) * VEC, o);
+      }
+    }
+  }
+}
+
+} // namespace nblahip

@@ -1,0 +1,255 @@
+// Plan selection and launch sequences for BatchNormalization.
+#include <algorithm>
+
+#include "bn.cuh"
+#include "launch.hpp"
+
+namespace nblahip {
+
+namespace {
+
+struct BnPlan {
+  int vec = 1;          // elements per load
+  bool channel_last = false;
+  // planes layout
+  uint32_t nvp = 1;     // vectors per plane
+  uint32_t vpc = 1;     // vectors per channel
+  uint32_t chunk = 1;   // vectors per split
+  // channel-last layout
+  uint32_t ncv = 1;     // channel vectors
+  uint32_t log2tx = 0;
+  uint32_t rps = 1;     // rows per split
+  uint32_t ytiles = 1;  // ceil(ncv / TX)
+  uint32_t S = 1;       // splits
+  bool cl_fast_apply = false;
+  int apply_vec = 1;    // vector width of the apply kernels
+};
+
+uint32_t ceil_div_u(uint64_t a, uint64_t b) { return static_cast<uint32_t>((a + b - 1) / b); }
+
+// Upper bound of S over every plan this shape can get (vector width depends on
+// pointer alignment, unknown when the workspace is sized).
+uint32_t split_target() { return static_cast<uint32_t>(device_cus()) * tune_int("BN_BLOCKS_PER_CU", 16); }
+
+BnPlan make_plan(int64_t size0, int64_t C, int64_t size2, int dtype, bool ptr_aligned) {
+  BnPlan pl;
+  const int full = dtype == NBLAHIP_F16 ? 8 : 4;
+  const uint32_t target = split_target();
+  pl.channel_last = size2 == 1;
+  if (!pl.channel_last) {
+    pl.vec = (ptr_aligned && size2 % full == 0) ? full : 1;
+    pl.nvp = static_cast<uint32_t>(size2 / pl.vec);
+    pl.vpc = static_cast<uint32_t>(size0 * pl.nvp);
+    // Enough blocks to fill the chip, but at least one full unrolled step each.
+    const uint32_t want = std::max<uint32_t>(1, ceil_div_u(target, static_cast<uint64_t>(C)));
+    const uint32_t most = std::max<uint32_t>(1, pl.vpc / (kBnBlock * kBnUnroll));
+    uint32_t S = std::min(want, most);
+    pl.chunk = ceil_div_u(pl.vpc, S);
+    pl.S = ceil_div_u(pl.vpc, pl.chunk);
+  } else {
+    pl.vec = (ptr_aligned && C % full == 0) ? full : 1;
+    pl.ncv = static_cast<uint32_t>(C / pl.vec);
+    uint32_t l2 = 0;
+    while ((1u << l2) < pl.ncv && l2 < 6) ++l2; // TX = min(pow2ceil(ncv), 64)
+    pl.log2tx = l2;
+    const uint32_t TX = 1u << l2;
+    const uint32_t TY = kBnBlock >> l2;
+    pl.ytiles = ceil_div_u(pl.ncv, TX);
+    const uint64_t M = static_cast<uint64_t>(size0);
+    const uint32_t step = TY * kBnUnroll;
+    const uint32_t want = std::max<uint32_t>(1, ceil_div_u(target, pl.ytiles));
+    const uint32_t most = std::max<uint32_t>(1, static_cast<uint32_t>(M / step));
+    const uint32_t S = std::min(want, most);
+    uint32_t rps = ceil_div_u(M, S);
+    rps = ceil_div_u(rps, step) * step;
+    pl.rps = rps;
+    pl.S = ceil_div_u(M, rps);
+    pl.cl_fast_apply = (256u % pl.ncv) == 0;
+  }
+  // Channel-last without the register-resident parameters falls back to one
+  // element per thread, where channel = index % C.
+  pl.apply_vec = (pl.channel_last && !pl.cl_fast_apply) ? 1 : pl.vec;
+  return pl;
+}
+
+size_t part_bytes(uint32_t C, uint32_t S) {
+  return align_up(static_cast<size_t>(C) * S * 3 * sizeof(float), 256);
+}
+
+BnParamSrc param_src(const BnParam *params) {
+  BnParamSrc s{};
+  s.params = params;
+  return s;
+}
+
+int apply_grid(uint32_t total_vec, int unroll) {
+  const uint64_t blocks = (static_cast<uint64_t>(total_vec) + 256ull * unroll - 1) / (256ull * unroll);
+  return static_cast<int>(std::max<uint64_t>(1, std::min<uint64_t>(blocks, 1u << 20)));
+}
+
+template <typename T, int VEC>
+int fwd_apply_t(const BnProblem &p, const BnPlan &pl, const BnParamSrc &src, hipStream_t st) {
+  const T *x = static_cast<const T *>(p.x);
+  T *y = static_cast<T *>(p.out);
+  const uint64_t total = static_cast<uint64_t>(p.size0) * p.C * p.size2;
+  const uint32_t total_vec = static_cast<uint32_t>(total / VEC);
+  if (pl.channel_last && pl.cl_fast_apply) {
+    hipLaunchKernelGGL((bn_apply_cl_kernel<T, VEC>), dim3(apply_grid(total_vec, kBnUnroll)),
+                       dim3(256), 0, st, x, y, src, pl.ncv, total_vec);
+  } else {
+    // channel-last without the register fast path: planes of one vector each.
+    const uint32_t nvp = pl.channel_last ? 1u : pl.nvp;
+    hipLaunchKernelGGL((bn_apply_planes_kernel<T, VEC>), dim3(apply_grid(total_vec, kBnUnroll)),
+                       dim3(256), 0, st, x, y, src, FastDiv(nvp),
+                       FastDiv(static_cast<uint32_t>(p.C)), total_vec);
+  }
+  return last_launch_status();
+}
+
+template <typename T, int VEC>
+int stats_t(const BnProblem &p, const BnPlan &pl, float *part, hipStream_t st) {
+  const T *x = static_cast<const T *>(p.x);
+  if (pl.channel_last) {
+    hipLaunchKernelGGL((bn_stats_cl_kernel<T, VEC>), dim3(pl.ytiles, pl.S), dim3(kBnBlock), 0, st,
+                       x, static_cast<uint32_t>(p.size0), static_cast<uint32_t>(p.C), pl.ncv,
+                       pl.log2tx, pl.rps, part);
+  } else {
+    hipLaunchKernelGGL((bn_stats_planes_kernel<T, VEC>), dim3(static_cast<uint32_t>(p.C), pl.S),
+                       dim3(kBnBlock), 0, st, x, static_cast<uint32_t>(p.C), FastDiv(pl.nvp),
+                       pl.vpc, pl.chunk, part);
+  }
+  return last_launch_status();
+}
+
+template <typename T, int VEC>
+int bwd_reduce_t(const BnProblem &p, const BnPlan &pl, float *part2, hipStream_t st) {
+  const T *x = static_cast<const T *>(p.x);
+  const T *dy = static_cast<const T *>(p.dy);
+  if (pl.channel_last) {
+    hipLaunchKernelGGL((bn_bwd_reduce_cl_kernel<T, VEC>), dim3(pl.ytiles, pl.S), dim3(kBnBlock), 0,
+                       st, x, dy, p.mean, static_cast<uint32_t>(p.size0),
+                       static_cast<uint32_t>(p.C), pl.ncv, pl.log2tx, pl.rps, part2);
+  } else {
+    hipLaunchKernelGGL((bn_bwd_reduce_planes_kernel<T, VEC>),
+                       dim3(static_cast<uint32_t>(p.C), pl.S), dim3(kBnBlock), 0, st, x, dy, p.mean,
+                       static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, part2);
+  }
+  return last_launch_status();
+}
+
+template <typename T, int VEC>
+int bwd_apply_t(const BnProblem &p, const BnPlan &pl, const BnParam *params, hipStream_t st) {
+  const T *x = static_cast<const T *>(p.x);
+  const T *dy = static_cast<const T *>(p.dy);
+  T *dx = static_cast<T *>(p.out);
+  const uint64_t total = static_cast<uint64_t>(p.size0) * p.C * p.size2;
+  const uint32_t total_vec = static_cast<uint32_t>(total / VEC);
+  if (pl.channel_last && pl.cl_fast_apply) {
+    hipLaunchKernelGGL((bn_bwd_apply_cl_kernel<T, VEC>), dim3(apply_grid(total_vec, 2)), dim3(256),
+                       0, st, x, dy, dx, params, pl.ncv, total_vec, p.accum_dx);
+  } else {
+    const uint32_t nvp = pl.channel_last ? 1u : pl.nvp;
+    hipLaunchKernelGGL((bn_bwd_apply_planes_kernel<T, VEC>), dim3(apply_grid(total_vec, 2)),
+                       dim3(256), 0, st, x, dy, dx, params, FastDiv(nvp),
+                       FastDiv(static_cast<uint32_t>(p.C)), total_vec, p.accum_dx);
+  }
+  return last_launch_status();
+}
+
+// Run fn<T, VEC>() for the plan's element type and vector width.
+#define BN_DISPATCH(CALL, VECV)                                                  \
+  do {                                                                           \
+    if (p.dtype == NBLAHIP_F16) {                                                \
+      if ((VECV) == 8) return CALL(__half, 8);                                   \
+      return CALL(__half, 1);                                                    \
+    }                                                                            \
+    if ((VECV) == 4) return CALL(float, 4);                                      \
+    return CALL(float, 1);                                                       \
+  } while (0)
+
+int do_fwd_apply(const BnProblem &p, const BnPlan &pl, const BnParamSrc &src, hipStream_t st) {
+#define CALL(T, V) fwd_apply_t<T, V>(p, pl, src, st)
+  BN_DISPATCH(CALL, pl.apply_vec);
+#undef CALL
+}
+int do_stats(const BnProblem &p, const BnPlan &pl, float *part, hipStream_t st) {
+#define CALL(T, V) stats_t<T, V>(p, pl, part, st)
+  BN_DISPATCH(CALL, pl.vec);
+#undef CALL
+}
+int do_bwd_reduce(const BnProblem &p, const BnPlan &pl, float *part2, hipStream_t st) {
+#define CALL(T, V) bwd_reduce_t<T, V>(p, pl, part2, st)
+  BN_DISPATCH(CALL, pl.vec);
+#undef CALL
+}
+int do_bwd_apply(const BnProblem &p, const BnPlan &pl, const BnParam *params, hipStream_t st) {
+#define CALL(T, V) bwd_apply_t<T, V>(p, pl, params, st)
+  BN_DISPATCH(CALL, pl.apply_vec);
+#undef CALL
+}
+
+} // namespace
+
+size_t bn_workspace_bytes(int64_t size0, int64_t C, int64_t size2, int dtype) {
+  // The aligned plan and the scalar plan may pick different S; size for both.
+  const BnPlan a = make_plan(size0, C, size2, dtype, true);
+  const BnPlan b = make_plan(size0, C, size2, dtype, false);
+  const uint32_t S = std::max(a.S, b.S);
+  return part_bytes(static_cast<uint32_t>(C), S) +
+         align_up(static_cast<size_t>(C) * sizeof(BnParam), 256);
+}
+
+int launch_bn_infer(const BnProblem &p, hipStream_t st) {
+  const bool al = aligned16(p.x) && aligned16(p.out);
+  const BnPlan pl = make_plan(p.size0, p.C, p.size2, p.dtype, al);
+  BnParamSrc src{};
+  src.params = nullptr;
+  src.rmean = p.mean;
+  src.rvar = p.var;
+  src.gamma = p.gamma;
+  src.beta = p.beta;
+  src.eps = p.eps;
+  return do_fwd_apply(p, pl, src, st);
+}
+
+int launch_bn_fwd_train(const BnProblem &p, hipStream_t st) {
+  const bool al = aligned16(p.x) && aligned16(p.out);
+  const BnPlan pl = make_plan(p.size0, p.C, p.size2, p.dtype, al);
+  float *part = static_cast<float *>(p.ws);
+  BnParam *params = reinterpret_cast<BnParam *>(static_cast<char *>(p.ws) +
+                                                part_bytes(static_cast<uint32_t>(p.C), pl.S));
+  if (int e = do_stats(p, pl, part, st)) return e;
+  const double N = static_cast<double>(p.size0) * static_cast<double>(p.size2);
+  const float inv_N = static_cast<float>(1.0 / N);
+  const float unbias = static_cast<float>(N / (N - 1.0)); // inf when N == 1, as the reference
+  hipLaunchKernelGGL(bn_finalize_fwd_kernel, dim3(static_cast<uint32_t>(p.C)), dim3(kBnBlock), 0,
+                     st, part, pl.S, inv_N, unbias, p.decay, p.eps, p.gamma, p.beta, p.batch_mean,
+                     p.batch_var, p.rmean, p.rvar, params);
+  if (int e = last_launch_status()) return e;
+  return do_fwd_apply(p, pl, param_src(params), st);
+}
+
+int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
+  if (!p.out && !p.dgamma && !p.dbeta) return 0;
+  const bool al = aligned16(p.x) && aligned16(p.dy) && (!p.out || aligned16(p.out));
+  const BnPlan pl = make_plan(p.size0, p.C, p.size2, p.dtype, al);
+  float *part2 = static_cast<float *>(p.ws);
+  BnParam *params = reinterpret_cast<BnParam *>(static_cast<char *>(p.ws) +
+                                                part_bytes(static_cast<uint32_t>(p.C), pl.S));
+  const bool need_sums = p.dgamma || p.dbeta || (p.out && p.batch_stat);
+  if (need_sums) {
+    if (int e = do_bwd_reduce(p, pl, part2, st)) return e;
+  }
+  const double N = static_cast<double>(p.size0) * static_cast<double>(p.size2);
+  // Without the reduction (inference-mode dx only) S = 0 leaves the sums at zero.
+  hipLaunchKernelGGL(bn_finalize_bwd_kernel, dim3(static_cast<uint32_t>(p.C)), dim3(kBnBlock), 0,
+                     st, part2, need_sums ? pl.S : 0u, static_cast<float>(1.0 / N), p.eps,
+                     p.batch_stat, p.gamma, p.mean, p.var, p.dmean, p.dvar,
+                     need_sums ? p.dgamma : nullptr, need_sums ? p.dbeta : nullptr, p.accum_g,
+                     p.accum_b, params);
+  if (int e = last_launch_status()) return e;
+  if (p.out) return do_bwd_apply(p, pl, params, st);
+  return 0;
+}
+
+} // namespace nblahip

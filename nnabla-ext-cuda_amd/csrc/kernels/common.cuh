@@ -1,0 +1,346 @@
+// Device-side building blocks shared by every normalization kernel:
+// 128-bit vector access with fp32 conversion, wavefront-64 reductions (DPP for
+// the in-row steps, lane reads for the cross-row steps), LDS block reductions
+// and Welford/Chan merging.  gfx950 only: a wavefront is 64 lanes.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace nblahip {
+
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------------------
+// Element traits: VEC elements per 16-byte access.
+// ---------------------------------------------------------------------------
+template <typename T> struct FullVec;
+template <> struct FullVec<float> { static constexpr int value = 4; };
+template <> struct FullVec<__half> { static constexpr int value = 8; };
+
+template <typename T> __device__ __forceinline__ float to_f32(T v);
+template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ float to_f32<__half>(__half v) {
+  return __half2float(v);
+}
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ __half from_f32<__half>(float v) {
+  return __float2half(v); // round to nearest even
+}
+
+// Load VEC consecutive elements starting at p (p aligned to VEC*sizeof(T))
+// and widen them to float.
+template <typename T, int VEC>
+__device__ __forceinline__ void load_vec(const T *__restrict__ p, float (&out)[VEC]) {
+  if constexpr (VEC == 1) {
+    out[0] = to_f32<T>(p[0]);
+  } else if constexpr (sizeof(T) == 4) {
+    static_assert(VEC == 4, "float vectors are 4 wide");
+    const float4 v = *reinterpret_cast<const float4 *>(p);
+    out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+  } else {
+    static_assert(VEC == 8, "half vectors are 8 wide");
+    const uint4 raw = *reinterpret_cast<const uint4 *>(p);
+    const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float2 f = __half22float2(h[i]);
+      out[2 * i] = f.x;
+      out[2 * i + 1] = f.y;
+    }
+  }
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void store_vec(T *__restrict__ p, const float (&in)[VEC]) {
+  if constexpr (VEC == 1) {
+    p[0] = from_f32<T>(in[0]);
+  } else if constexpr (sizeof(T) == 4) {
+    *reinterpret_cast<float4 *>(p) = make_float4(in[0], in[1], in[2], in[3]);
+  } else {
+    uint4 raw;
+    __half2 *h = reinterpret_cast<__half2 *>(&raw);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      h[i] = __floats2half2_rn(in[2 * i], in[2 * i + 1]);
+    *reinterpret_cast<uint4 *>(p) = raw;
+  }
+}
+
+// Register-resident copy of VEC elements in their storage format (a half
+// vector stays packed: 4 registers for 8 values) with widening on use.
+template <typename T, int VEC> struct RawVec;
+template <> struct RawVec<float, 4> { float4 v; };
+template <> struct RawVec<float, 1> { float v; };
+template <> struct RawVec<__half, 8> { uint4 v; };
+template <> struct RawVec<__half, 1> { __half v; };
+
+template <typename T, int VEC>
+__device__ __forceinline__ RawVec<T, VEC> load_raw(const T *__restrict__ p) {
+  RawVec<T, VEC> r;
+  if constexpr (VEC == 1) {
+    r.v = p[0];
+  } else if constexpr (sizeof(T) == 4) {
+    r.v = *reinterpret_cast<const float4 *>(p);
+  } else {
+    r.v = *reinterpret_cast<const uint4 *>(p);
+  }
+  return r;
+}
+
+template <typename T, int VEC> __device__ __forceinline__ RawVec<T, VEC> zero_raw() {
+  RawVec<T, VEC> r;
+  if constexpr (VEC == 1) {
+    r.v = from_f32<T>(0.f);
+  } else if constexpr (sizeof(T) == 4) {
+    r.v = make_float4(0.f, 0.f, 0.f, 0.f);
+  } else {
+    r.v = make_uint4(0u, 0u, 0u, 0u);
+  }
+  return r;
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void unpack(const RawVec<T, VEC> &r, float (&out)[VEC]) {
+  if constexpr (VEC == 1) {
+    out[0] = to_f32<T>(r.v);
+  } else if constexpr (sizeof(T) == 4) {
+    out[0] = r.v.x; out[1] = r.v.y; out[2] = r.v.z; out[3] = r.v.w;
+  } else {
+    const __half2 *h = reinterpret_cast<const __half2 *>(&r.v);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float2 f = __half22float2(h[i]);
+      out[2 * i] = f.x;
+      out[2 * i + 1] = f.y;
+    }
+  }
+}
+
+// Hides the value of a packed half vector from the optimiser so that the
+// widened floats of one phase are not kept alive for the next one (the point
+// of keeping the row packed).  No instruction is emitted.
+template <typename T, int VEC> __device__ __forceinline__ void keep_packed(RawVec<T, VEC> &r) {
+  if constexpr (sizeof(T) == 2 && VEC == 8) {
+    asm volatile("" : "+v"(r.v.x), "+v"(r.v.y), "+v"(r.v.z), "+v"(r.v.w));
+  }
+}
+
+// VEC consecutive float parameters (gamma/beta style), p aligned to 16 bytes
+// when VEC > 1.
+template <int VEC>
+__device__ __forceinline__ void load_param_vec(const float *__restrict__ p,
+                                               float (&out)[VEC]) {
+  if constexpr (VEC == 1) {
+    out[0] = p[0];
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC / 4; ++i) {
+      const float4 v = reinterpret_cast<const float4 *>(p)[i];
+      out[4 * i] = v.x; out[4 * i + 1] = v.y; out[4 * i + 2] = v.z; out[4 * i + 3] = v.w;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Division by a runtime constant without the integer divider: q = n / d for
+// 0 <= n < 2^31 and 1 <= d < 2^31 (round-up multiplier, 64-bit product).
+// ---------------------------------------------------------------------------
+struct FastDiv {
+  uint32_t d;
+  uint32_t mul;
+  uint32_t shift;
+  __host__ FastDiv() : d(1), mul(0), shift(0) {}
+  __host__ explicit FastDiv(uint32_t divisor) : d(divisor) {
+    if (divisor <= 1) {
+      d = 1; mul = 0; shift = 0;
+      return;
+    }
+    uint32_t s = 0;
+    while ((1ull << s) < divisor) ++s;           // s = ceil(log2 d)
+    const uint64_t m = ((1ull << (31 + s)) + divisor - 1) / divisor; // < 2^32
+    mul = static_cast<uint32_t>(m);
+    shift = s;
+  }
+  __host__ __device__ __forceinline__ uint32_t div(uint32_t n) const {
+    if (d == 1) return n;
+    return static_cast<uint32_t>((static_cast<uint64_t>(n) * mul) >> 31) >> shift;
+  }
+};
+
+// ---------------------------------------------------------------------------
+// Wavefront-64 all-reduce (sum).  Steps 1,2,4,8 stay inside a 16-lane DPP row:
+// quad_perm xor1, quad_perm xor2, row_half_mirror, row_mirror.  After them each
+// row is uniform and the four row values are fetched with lane reads, so the
+// result is wave-uniform and identical in every lane.
+// ---------------------------------------------------------------------------
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf,
+                                         0xf, true));
+}
+
+__device__ __forceinline__ float read_lane(float v, int lane) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+  v += dpp_move<0xB1>(v);  // quad_perm [1,0,3,2]
+  v += dpp_move<0x4E>(v);  // quad_perm [2,3,0,1]
+  v += dpp_move<0x141>(v); // row_half_mirror
+  v += dpp_move<0x140>(v); // row_mirror
+  return (read_lane(v, 0) + read_lane(v, 16)) + (read_lane(v, 32) + read_lane(v, 48));
+}
+
+// Sum over a group of TPR threads that share a row.  TPR == 64: one wave.
+// TPR > 64: the block is exactly one row (blockDim.x == TPR); `lds` holds
+// TPR/64 floats and is reused, so the call ends with a barrier-protected read.
+template <int TPR>
+__device__ __forceinline__ float row_sum(float v, float *lds) {
+  v = wave_sum(v);
+  if constexpr (TPR == kWave) {
+    return v;
+  } else {
+    constexpr int NW = TPR / kWave;
+    const int wave = threadIdx.x / kWave;
+    __syncthreads(); // previous readers of lds are done
+    if ((threadIdx.x & (kWave - 1)) == 0) lds[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) total += lds[i];
+    return total;
+  }
+}
+
+// Two sums at once (halves the number of barriers).
+template <int TPR>
+__device__ __forceinline__ void row_sum2(float &a, float &b, float *lds) {
+  a = wave_sum(a);
+  b = wave_sum(b);
+  if constexpr (TPR > kWave) {
+    constexpr int NW = TPR / kWave;
+    const int wave = threadIdx.x / kWave;
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+      lds[2 * wave] = a;
+      lds[2 * wave + 1] = b;
+    }
+    __syncthreads();
+    float ta = 0.f, tb = 0.f;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+      ta += lds[2 * i];
+      tb += lds[2 * i + 1];
+    }
+    a = ta;
+    b = tb;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Welford state and the Chan/Golub/LeVeque merge (the reference's
+// include/nbla/cuda/utils/reduce_ops/welford.cuh:80-97).  n is kept in float:
+// exact up to 2^24 per partial, which every launch configuration respects.
+// ---------------------------------------------------------------------------
+struct Welford {
+  float mean, m2, n;
+};
+
+__device__ __forceinline__ Welford welford_merge(const Welford &a, const Welford &b) {
+  const float n = a.n + b.n;
+  if (n == 0.f) return Welford{0.f, 0.f, 0.f};
+  const float inv = 1.0f / n;
+  const float d = b.mean - a.mean;
+  Welford r;
+  r.mean = a.mean + d * (b.n * inv);
+  r.m2 = a.m2 + b.m2 + d * d * (a.n * b.n * inv);
+  r.n = n;
+  return r;
+}
+
+// Merge a chunk of CNT values v[] (CNT >= 1, compile-time bound, `cnt` valid)
+// into acc: chunk mean and centred M2 are formed in registers first, so only
+// one reciprocal is spent per chunk.
+template <int CNT>
+__device__ __forceinline__ void welford_add_chunk(Welford &acc, const float (&v)[CNT],
+                                                  int cnt) {
+  if (cnt <= 0) return;
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < CNT; ++i) s += (i < cnt) ? v[i] : 0.f;
+  const float fc = static_cast<float>(cnt);
+  const float cm = s / fc;
+  float m2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < CNT; ++i) {
+    const float d = v[i] - cm;
+    m2 += (i < cnt) ? d * d : 0.f;
+  }
+  acc = welford_merge(acc, Welford{cm, m2, fc});
+}
+
+__device__ __forceinline__ Welford wave_welford(Welford w) {
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    Welford o;
+    o.mean = __shfl_xor(w.mean, off);
+    o.m2 = __shfl_xor(w.m2, off);
+    o.n = __shfl_xor(w.n, off);
+    // Keep the operand order identical in both partners so they agree bitwise.
+    const bool low = (threadIdx.x & off) == 0;
+    w = low ? welford_merge(w, o) : welford_merge(o, w);
+  }
+  return w;
+}
+
+// Block-wide Welford merge; lds holds 3*(blockDim.x/64) floats.  Every thread
+// returns the same merged state.
+__device__ __forceinline__ Welford block_welford(Welford w, float *lds) {
+  w = wave_welford(w);
+  const int nw = blockDim.x / kWave;
+  if (nw == 1) return w;
+  const int wave = threadIdx.x / kWave;
+  __syncthreads();
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    lds[3 * wave] = w.mean;
+    lds[3 * wave + 1] = w.m2;
+    lds[3 * wave + 2] = w.n;
+  }
+  __syncthreads();
+  Welford t{lds[0], lds[1], lds[2]};
+  for (int i = 1; i < nw; ++i)
+    t = welford_merge(t, Welford{lds[3 * i], lds[3 * i + 1], lds[3 * i + 2]});
+  return t;
+}
+
+// Block-wide sum of two values; lds holds 2*(blockDim.x/64) floats.
+__device__ __forceinline__ void block_sum2(float &a, float &b, float *lds) {
+  a = wave_sum(a);
+  b = wave_sum(b);
+  const int nw = blockDim.x / kWave;
+  if (nw == 1) return;
+  const int wave = threadIdx.x / kWave;
+  __syncthreads();
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    lds[2 * wave] = a;
+    lds[2 * wave + 1] = b;
+  }
+  __syncthreads();
+  float ta = 0.f, tb = 0.f;
+  for (int i = 0; i < nw; ++i) {
+    ta += lds[2 * i];
+    tb += lds[2 * i + 1];
+  }
+  a = ta;
+  b = tb;
+}
+
+__device__ __forceinline__ float inv_std(float var, float eps) {
+  return 1.0f / sqrtf(var + eps);
+}
+
+} // namespace nblahip

@@ -1,0 +1,105 @@
+// Host-side launch layer shared by the translation units of the kernel
+// library: problem descriptions, plan selection and the internal launch
+// functions the C-ABI entry points call.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../../include/nblahip.h"
+
+namespace nblahip {
+
+enum RowMode { kRowLN = 0, kRowIN = 1, kRowGN = 2 };
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Number of compute units of the current device (cached per device).
+int device_cus();
+
+// Read-once integer tuning knob from the environment (name without prefix
+// "NBLAHIP_"); returns `fallback` when unset or unparsable.
+int tune_int(const char *name, int fallback);
+
+// One row-normalization problem (LayerNormalization rows,
+// InstanceNormalization planes or GroupNormalization groups).
+struct RowProblem {
+  int dtype = 0;
+  int mode = 0; // RowMode
+  const void *x = nullptr;
+  const void *dy = nullptr;
+  void *out = nullptr; // y or dx
+  const float *gamma = nullptr;
+  const float *beta = nullptr;
+  float *mean = nullptr;
+  float *var = nullptr;
+  const float *dmean = nullptr;
+  const float *dvar = nullptr;
+  float *dgamma = nullptr;
+  float *dbeta = nullptr;
+  int accum_dx = 0, accum_g = 0, accum_b = 0;
+  int64_t rows = 0; // statistics rows
+  int64_t R = 0;    // elements per statistics row
+  // GN / IN geometry: x is [batch, channels, spatial]
+  int64_t batch = 1, channels = 1, spatial = 1;
+  int groups = 1;
+  int bc_gamma = 1, bc_beta = 1;
+  float eps = 0.f;
+  void *ws = nullptr;
+  size_t ws_bytes = 0;
+};
+
+// Register-cached configuration: TPR threads per row, NL 16-byte loads each.
+struct RowCfg {
+  bool ok = false;
+  int vec = 1, tpr = 64, nl = 1;
+};
+
+// vec_ok: whether the full 16-byte vector width may be used (alignment and
+// divisibility already checked by the caller).  max_nl_1024 bounds the loads
+// per thread of the 1024-thread layout; min_tpr is 256 for the
+// GroupNormalization backward.
+RowCfg pick_row_cfg(int dtype, int64_t R, bool vec_ok, int max_nl_1024, int min_tpr);
+
+int launch_row_fwd(const RowProblem &p, hipStream_t st);
+int launch_row_bwd(const RowProblem &p, hipStream_t st);
+size_t row_bwd_workspace_bytes(int mode, int64_t rows, int64_t R, int64_t planes);
+
+struct BnProblem {
+  int dtype = 0;
+  const void *x = nullptr;
+  const void *dy = nullptr;
+  void *out = nullptr; // y or dx
+  const float *gamma = nullptr;
+  const float *beta = nullptr;
+  float *batch_mean = nullptr; // forward: written
+  float *batch_var = nullptr;
+  float *rmean = nullptr;
+  float *rvar = nullptr;
+  const float *mean = nullptr; // backward / inference: read
+  const float *var = nullptr;
+  const float *dmean = nullptr;
+  const float *dvar = nullptr;
+  float *dgamma = nullptr;
+  float *dbeta = nullptr;
+  int accum_dx = 0, accum_g = 0, accum_b = 0;
+  int batch_stat = 1;
+  int64_t size0 = 1, C = 1, size2 = 1;
+  float decay = 0.9f, eps = 1e-5f;
+  void *ws = nullptr;
+  size_t ws_bytes = 0;
+};
+
+int launch_bn_infer(const BnProblem &p, hipStream_t st);
+int launch_bn_fwd_train(const BnProblem &p, hipStream_t st);
+int launch_bn_bwd(const BnProblem &p, hipStream_t st);
+size_t bn_workspace_bytes(int64_t size0, int64_t C, int64_t size2, int dtype);
+
+inline int last_launch_status() {
+  const hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : static_cast<int>(e);
+}
+
+} // namespace nblahip

@@ -1,0 +1,380 @@
+// Row normalizations (LayerNormalization rows, InstanceNormalization planes,
+// GroupNormalization groups) with the row cached in registers: x (and dy) cross
+// HBM exactly once per direction.
+//
+// Thread layout: TPR threads share a row (64 = one wavefront, no barrier at all;
+// 256 / 1024 = one block per row, LDS cross-wave merge).  Thread t issues NL
+// 16-byte loads at element (k*TPR + t)*VEC, k = 0..NL-1, so every load
+// instruction of a wave covers 1 KiB of consecutive memory.
+//
+// Statistics: the row sits in registers, so the mean is an exact-count sum and
+// the variance is the centred second moment taken from the same registers
+// (one pass over memory, no E[x^2]-E[x]^2 cancellation).
+#pragma once
+
+#include "common.cuh"
+#include "launch.hpp"
+
+namespace nblahip {
+
+struct RowArgs {
+  const void *x;
+  const void *dy;     // backward only
+  void *out;          // y (forward) or dx (backward, may be null)
+  const float *gamma; // may be null
+  const float *beta;  // may be null (forward only)
+  float *mean;        // forward: written; backward: read
+  float *var;
+  const float *dmean; // may be null
+  const float *dvar;  // may be null
+  float *ws;          // backward partials
+  int rows;
+  int R;
+  float eps;
+  float inv_R;
+  // Parameter index of element (row, col):
+  //   percol != 0 : col                                   (LayerNormalization)
+  //   percol == 0 : (row % pmod) * pmul + col / pdiv       (Instance / Group)
+  // (beta uses pmod_b in place of pmod: InstanceNormalization may broadcast
+  // gamma and beta differently.)
+  int percol;
+  uint32_t pmod;
+  uint32_t pmod_b;
+  uint32_t pmul;
+  FastDiv pdiv;
+  int accum_dx;
+  // GroupNormalization backward: entries (64*VEC-element runs) per channel and
+  // channels per group.
+  int epc;
+  int cpg;
+};
+
+template <int TPR> struct RowBlock {
+  static constexpr int kBlock = TPR < 256 ? 256 : TPR;
+  static constexpr int kRowsPerBlock = kBlock / TPR;
+};
+
+// ---------------------------------------------------------------------------
+// Forward: y, mean, var.
+// ---------------------------------------------------------------------------
+template <typename T, int VEC, int NL, int TPR>
+__global__ void __launch_bounds__(RowBlock<TPR>::kBlock)
+row_fwd_kernel(const RowArgs a) {
+  constexpr int RPB = RowBlock<TPR>::kRowsPerBlock;
+  __shared__ float lds[2 * 16];
+  const int t = threadIdx.x % TPR;
+  const int sub = threadIdx.x / TPR;
+  const T *__restrict__ x = static_cast<const T *>(a.x);
+  T *__restrict__ y = static_cast<T *>(a.out);
+
+  for (int row = blockIdx.x * RPB + sub; row < a.rows; row += gridDim.x * RPB) {
+    const size_t base = static_cast<size_t>(row) * a.R;
+    RawVec<T, VEC> raw[NL];
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const int col = (k * TPR + t) * VEC;
+      raw[k] = (col < a.R) ? load_raw<T, VEC>(x + base + col) : zero_raw<T, VEC>();
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      float v[VEC];
+      unpack<T, VEC>(raw[k], v);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) s += v[j];
+    }
+    const float mean = row_sum<TPR>(s, lds) * a.inv_R;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+
+    float q = 0.f;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const int col = (k * TPR + t) * VEC;
+      if (col < a.R) {
+        float v[VEC];
+        unpack<T, VEC>(raw[k], v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float d = v[j] - mean;
+          q += d * d;
+        }
+      }
+    }
+    const float var = row_sum<TPR>(q, lds) * a.inv_R;
+    const float istd = inv_std(var, a.eps);
+    if (t == 0) {
+      a.mean[row] = mean;
+      a.var[row] = var;
+    }
+#pragma unroll
+    for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+
+    const uint32_t pbase = a.percol ? 0u : (static_cast<uint32_t>(row) % a.pmod) * a.pmul;
+    const uint32_t bbase = a.percol ? 0u : (static_cast<uint32_t>(row) % a.pmod_b) * a.pmul;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const int col = (k * TPR + t) * VEC;
+      if (col < a.R) {
+        float v[VEC], o[VEC];
+        unpack<T, VEC>(raw[k], v);
+        if (a.percol) {
+          float g[VEC], b[VEC];
+          if (a.gamma) {
+            load_param_vec<VEC>(a.gamma + col, g);
+          } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) g[j] = 1.f;
+          }
+          if (a.beta) {
+            load_param_vec<VEC>(a.beta + col, b);
+          } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) b[j] = 0.f;
+          }
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) o[j] = (v[j] - mean) * (g[j] * istd) + b[j];
+        } else {
+          const uint32_t poff = a.pdiv.div(static_cast<uint32_t>(col));
+          const float g = (a.gamma ? a.gamma[pbase + poff] : 1.f) * istd;
+          const float b = a.beta ? a.beta[bbase + poff] : 0.f;
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) o[j] = (v[j] - mean) * g + b;
+        }
+        store_vec<T, VEC>(y + base + col, o);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Backward: dx plus partial parameter gradients.
+//   s1 = sum(dy*g), t2 = sum(dy*g*(x-mean))
+//   ca = -t2*istd^3/R + 2*dvar/R      cb = -s1*istd/R + dmean/R
+//   dx = dy*g*istd + ca*(x-mean) + cb
+// which is the reference's a*x+b form (kernel/layer_normalization.cuh:50-95)
+// with a*mean folded into the centred term.
+//
+// Partial parameter gradients written to ws:
+//   LN : ws[block][0][R] = sum_rows dy*(x-mean)*istd, ws[block][1][R] = sum_rows dy
+//   IN : ws[2*row] = sum dy*(x-mean)*istd, ws[2*row+1] = sum dy     (row = (n,c))
+//   GN : same pair per (n, channel); requires spatial % (64*VEC) == 0 so that
+//        every wave-wide load belongs to one channel.
+// Padded lanes hold x = dy = 0 in registers, so they add nothing to any sum.
+// ---------------------------------------------------------------------------
+template <typename T, int VEC, int NL, int TPR, int MODE>
+__global__ void __launch_bounds__(RowBlock<TPR>::kBlock)
+row_bwd_kernel(const RowArgs a) {
+  constexpr int RPB = RowBlock<TPR>::kRowsPerBlock;
+  constexpr int NW = TPR / kWave;
+  __shared__ float lds[2 * 16];
+  __shared__ float part[(MODE == kRowGN) ? 2 * NW * NL : 1];
+  __shared__ float xwave[(MODE == kRowLN && RPB > 1) ? (RPB - 1) * kWave * VEC : 1];
+  const int t = threadIdx.x % TPR;
+  const int sub = threadIdx.x / TPR;
+  const T *__restrict__ x = static_cast<const T *>(a.x);
+  const T *__restrict__ dy = static_cast<const T *>(a.dy);
+  T *__restrict__ dx = static_cast<T *>(a.out);
+
+  float acc_g[(MODE == kRowLN) ? NL : 1][VEC];
+  float acc_b[(MODE == kRowLN) ? NL : 1][VEC];
+  if constexpr (MODE == kRowLN) {
+#pragma unroll
+    for (int k = 0; k < NL; ++k)
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) acc_g[k][j] = acc_b[k][j] = 0.f;
+  }
+
+  for (int row = blockIdx.x * RPB + sub; row < a.rows; row += gridDim.x * RPB) {
+    const size_t base = static_cast<size_t>(row) * a.R;
+    RawVec<T, VEC> xr[NL], dr[NL];
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const int col = (k * TPR + t) * VEC;
+      const bool ok = col < a.R;
+      xr[k] = ok ? load_raw<T, VEC>(x + base + col) : zero_raw<T, VEC>();
+      dr[k] = ok ? load_raw<T, VEC>(dy + base + col) : zero_raw<T, VEC>();
+    }
+    const float mean = a.mean[row];
+    const float istd = inv_std(a.var[row], a.eps);
+
+    float s1 = 0.f, t2 = 0.f;
+    float gk[NL]; // per-load scalar gamma (IN / GN)
+    if constexpr (MODE == kRowLN) {
+#pragma unroll
+      for (int k = 0; k < NL; ++k) {
+        const int col = (k * TPR + t) * VEC;
+        if (col < a.R) {
+          float xv[VEC], dv[VEC], g[VEC];
+          unpack<T, VEC>(xr[k], xv);
+          unpack<T, VEC>(dr[k], dv);
+          if (a.gamma) {
+            load_param_vec<VEC>(a.gamma + col, g);
+          } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) g[j] = 1.f;
+          }
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            const float xc = xv[j] - mean;
+            acc_g[k][j] += dv[j] * xc * istd;
+            acc_b[k][j] += dv[j];
+            const float dg = dv[j] * g[j];
+            s1 += dg;
+            t2 += dg * xc;
+          }
+        }
+      }
+      row_sum2<TPR>(s1, t2, lds);
+    } else if constexpr (MODE == kRowIN) {
+      float sdy = 0.f, sdx = 0.f;
+#pragma unroll
+      for (int k = 0; k < NL; ++k) {
+        float xv[VEC], dv[VEC];
+        unpack<T, VEC>(xr[k], xv);
+        unpack<T, VEC>(dr[k], dv);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          sdy += dv[j];
+          sdx += dv[j] * (xv[j] - mean);
+        }
+      }
+      row_sum2<TPR>(sdy, sdx, lds);
+      if (t == 0) {
+        a.ws[2 * static_cast<size_t>(row)] = sdx * istd;
+        a.ws[2 * static_cast<size_t>(row) + 1] = sdy;
+      }
+      const uint32_t pidx = (static_cast<uint32_t>(row) % a.pmod) * a.pmul;
+      const float g = a.gamma ? a.gamma[pidx] : 1.f;
+#pragma unroll
+      for (int k = 0; k < NL; ++k) gk[k] = g;
+      s1 = g * sdy;
+      t2 = g * sdx;
+    } else { // GroupNormalization, RPB == 1
+      static_assert(MODE != kRowGN || RPB == 1, "group rows own the whole block");
+      const int wave = threadIdx.x / kWave;
+      const int lane = threadIdx.x & (kWave - 1);
+      const uint32_t pbase = (static_cast<uint32_t>(row) % a.pmod) * a.pmul;
+      __syncthreads(); // part[] of the previous row has been consumed
+#pragma unroll
+      for (int k = 0; k < NL; ++k) {
+        float xv[VEC], dv[VEC];
+        unpack<T, VEC>(xr[k], xv);
+        unpack<T, VEC>(dr[k], dv);
+        float sdy = 0.f, sdx = 0.f;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          sdy += dv[j];
+          sdx += dv[j] * (xv[j] - mean);
+        }
+        sdy = wave_sum(sdy);
+        sdx = wave_sum(sdx);
+        const int e = k * NW + wave; // run index: elements [e*64*VEC, (e+1)*64*VEC)
+        if (lane == 0) {
+          part[2 * e] = sdx;
+          part[2 * e + 1] = sdy;
+        }
+        const int col = (k * TPR + t) * VEC;
+        const uint32_t ch = (col < a.R) ? a.pdiv.div(static_cast<uint32_t>(col)) : 0u;
+        gk[k] = a.gamma ? a.gamma[pbase + ch] : 1.f;
+      }
+      __syncthreads();
+      // Channel c owns runs [c*epc, (c+1)*epc).
+      float c1 = 0.f, c2 = 0.f;
+      for (int c = threadIdx.x; c < a.cpg; c += TPR) {
+        float sdx = 0.f, sdy = 0.f;
+        for (int e = c * a.epc; e < (c + 1) * a.epc; ++e) {
+          sdx += part[2 * e];
+          sdy += part[2 * e + 1];
+        }
+        const size_t o = 2 * (static_cast<size_t>(row) * a.cpg + c);
+        a.ws[o] = sdx * istd;
+        a.ws[o + 1] = sdy;
+        const float g = a.gamma ? a.gamma[pbase + c] : 1.f;
+        c1 += g * sdy;
+        c2 += g * sdx;
+      }
+      row_sum2<TPR>(c1, c2, lds);
+      s1 = c1;
+      t2 = c2;
+    }
+
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      keep_packed<T, VEC>(xr[k]);
+      keep_packed<T, VEC>(dr[k]);
+    }
+    const float ca = -t2 * istd * istd * istd * a.inv_R +
+                     (a.dvar ? 2.f * a.dvar[row] * a.inv_R : 0.f);
+    const float cb = -s1 * istd * a.inv_R + (a.dmean ? a.dmean[row] * a.inv_R : 0.f);
+
+    if (dx != nullptr) {
+#pragma unroll
+      for (int k = 0; k < NL; ++k) {
+        const int col = (k * TPR + t) * VEC;
+        if (col < a.R) {
+          float xv[VEC], dv[VEC], o[VEC];
+          unpack<T, VEC>(xr[k], xv);
+          unpack<T, VEC>(dr[k], dv);
+          if constexpr (MODE == kRowLN) {
+            float g[VEC];
+            if (a.gamma) {
+              load_param_vec<VEC>(a.gamma + col, g);
+            } else {
+#pragma unroll
+              for (int j = 0; j < VEC; ++j) g[j] = 1.f;
+            }
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+              o[j] = dv[j] * (g[j] * istd) + ca * (xv[j] - mean) + cb;
+          } else {
+            const float gi = gk[k] * istd;
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) o[j] = dv[j] * gi + ca * (xv[j] - mean) + cb;
+          }
+          if (a.accum_dx) {
+            float old[VEC];
+            load_vec<T, VEC>(dx + base + col, old);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) o[j] += old[j];
+          }
+          store_vec<T, VEC>(dx + base + col, o);
+        }
+      }
+    }
+  }
+
+  if constexpr (MODE == kRowLN) {
+    // Fold the RPB waves of a block into wave 0 (fixed order), then write the
+    // block's partial [2][R].
+    float *wsb = a.ws + static_cast<size_t>(blockIdx.x) * 2 * a.R;
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+#pragma unroll
+      for (int k = 0; k < NL; ++k) {
+        float(&acc)[VEC] = (q == 0) ? acc_g[k] : acc_b[k];
+        if constexpr (RPB > 1) {
+          __syncthreads();
+          if (sub > 0) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) xwave[((sub - 1) * kWave + t) * VEC + j] = acc[j];
+          }
+          __syncthreads();
+          if (sub == 0) {
+#pragma unroll
+            for (int r = 0; r < RPB - 1; ++r)
+#pragma unroll
+              for (int j = 0; j < VEC; ++j) acc[j] += xwave[(r * kWave + t) * VEC + j];
+          }
+        }
+        const int col = (k * TPR + t) * VEC;
+        if (sub == 0 && col < a.R) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) wsb[static_cast<size_t>(q) * a.R + col + j] = acc[j];
+        }
+      }
+    }
+  }
+}
+
+} // namespace nblahip

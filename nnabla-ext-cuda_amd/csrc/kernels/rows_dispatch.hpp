@@ -1,0 +1,39 @@
+// Internal: per-family launchers of the register-cached row kernels.  Each
+// lives in its own translation unit so the template instantiations compile
+// in parallel.
+#pragma once
+
+#include "launch.hpp"
+#include "rows.cuh"
+
+namespace nblahip {
+
+int run_row_fwd_cached(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
+                       hipStream_t st);
+int run_row_bwd_cached_ln(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
+                          hipStream_t st);
+int run_row_bwd_cached_in(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
+                          hipStream_t st);
+int run_row_bwd_cached_gn(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
+                          hipStream_t st);
+
+// Expands CASE(T, VEC, NL, TPR) for every supported register-cached shape of
+// element type T.
+#define NBLAHIP_ROW_CASES_TPR(CASE, T, VEC, TPR) \
+  CASE(T, VEC, 1, TPR) CASE(T, VEC, 2, TPR) CASE(T, VEC, 4, TPR) CASE(T, VEC, 8, TPR)
+
+#define NBLAHIP_ROW_CASES(CASE, T)                          \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 64)     \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 256)    \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 1024)   \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 64)                     \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 256)                    \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 1024)
+
+#define NBLAHIP_ROW_CASES_BLOCK(CASE, T)                    \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 256)    \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 1024)   \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 256)                    \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 1024)
+
+} // namespace nblahip

@@ -1,0 +1,255 @@
+// Plan selection and launch sequences for the row normalizations
+// (LayerNormalization, InstanceNormalization, GroupNormalization), plus the
+// instantiations of the streaming kernels.
+#include <algorithm>
+
+#include "rows_dispatch.hpp"
+#include "rows_stream.cuh"
+
+namespace nblahip {
+
+// max_nl_1024 bounds the loads per thread of the 1024-thread layout, whose
+// register budget is 128 VGPRs; the smaller layouts take up to 8.
+RowCfg pick_row_cfg(int dtype, int64_t R, bool vec_ok, int max_nl_1024, int min_tpr) {
+  RowCfg c;
+  const int full = dtype == NBLAHIP_F16 ? 8 : 4;
+  c.vec = vec_ok ? full : 1;
+  const int64_t nv = R / c.vec;
+  static const int tprs[3] = {64, 256, 1024};
+  static const int nls[4] = {1, 2, 4, 8};
+  for (int tpr : tprs) {
+    if (tpr < min_tpr) continue;
+    const int cap = tpr == 1024 ? max_nl_1024 : 8;
+    for (int nl : nls) {
+      if (nl > cap) break;
+      if (static_cast<int64_t>(tpr) * nl >= nv) {
+        c.ok = true;
+        c.tpr = tpr;
+        c.nl = nl;
+        return c;
+      }
+    }
+  }
+  return c;
+}
+
+static int rows_per_block(int tpr) { return tpr < 256 ? 256 / tpr : 1; }
+
+static int cached_grid(int64_t rows, int tpr) {
+  const int rpb = rows_per_block(tpr);
+  const int64_t blocks = (rows + rpb - 1) / rpb;
+  return static_cast<int>(std::min<int64_t>(blocks, 1 << 20));
+}
+
+// Persistent grid of the LayerNormalization backward: each block keeps
+// per-column accumulators, so fewer blocks mean fewer partials to fold.
+static int ln_bwd_grid(int64_t rows, int tpr) {
+  const int per_cu = tune_int("LN_BWD_BLOCKS_PER_CU", 2);
+  const int64_t cap = static_cast<int64_t>(device_cus()) * per_cu;
+  return static_cast<int>(std::min<int64_t>(cached_grid(rows, tpr), cap));
+}
+
+static int stream_grid(int64_t work_blocks) {
+  const int64_t cap = static_cast<int64_t>(device_cus()) * 16;
+  return static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(work_blocks, cap)));
+}
+
+static RowArgs make_args(const RowProblem &p) {
+  RowArgs a{};
+  a.x = p.x;
+  a.dy = p.dy;
+  a.out = p.out;
+  a.gamma = p.gamma;
+  a.beta = p.beta;
+  a.mean = p.mean;
+  a.var = p.var;
+  a.dmean = p.dmean;
+  a.dvar = p.dvar;
+  a.ws = static_cast<float *>(p.ws);
+  a.rows = static_cast<int>(p.rows);
+  a.R = static_cast<int>(p.R);
+  a.eps = p.eps;
+  a.inv_R = 1.0f / static_cast<float>(p.R);
+  a.accum_dx = p.accum_dx;
+  a.epc = 0;
+  a.cpg = 1;
+  if (p.mode == kRowLN) {
+    a.percol = 1;
+    a.pmod = a.pmod_b = 1;
+    a.pmul = 0;
+    a.pdiv = FastDiv(1);
+  } else if (p.mode == kRowIN) {
+    a.percol = 0;
+    a.pmod = static_cast<uint32_t>(p.bc_gamma ? p.channels : p.rows);
+    a.pmod_b = static_cast<uint32_t>(p.bc_beta ? p.channels : p.rows);
+    a.pmul = 1;
+    a.pdiv = FastDiv(static_cast<uint32_t>(p.R)); // col / R == 0
+  } else {
+    a.percol = 0;
+    a.pmod = a.pmod_b = static_cast<uint32_t>(p.groups);
+    a.pmul = static_cast<uint32_t>(p.channels / p.groups);
+    a.pdiv = FastDiv(static_cast<uint32_t>(p.spatial));
+    a.cpg = static_cast<int>(p.channels / p.groups);
+  }
+  return a;
+}
+
+static bool row_vec_ok(const RowProblem &p, bool backward) {
+  const int full = p.dtype == NBLAHIP_F16 ? 8 : 4;
+  if (p.R % full != 0) return false;
+  if (!aligned16(p.x)) return false;
+  if (p.out && !aligned16(p.out)) return false;
+  if (backward && !aligned16(p.dy)) return false;
+  if (p.mode == kRowLN) {
+    if (p.gamma && !aligned16(p.gamma)) return false;
+    if (!backward && p.beta && !aligned16(p.beta)) return false;
+  } else if (p.mode == kRowGN) {
+    if (p.spatial % full != 0) return false;
+  }
+  return true;
+}
+
+template <typename T, int VEC>
+static int stream_fwd_t(const RowProblem &p, const RowArgs &a, hipStream_t st) {
+  hipLaunchKernelGGL((row_stats_stream_kernel<T, VEC>), dim3(stream_grid(p.rows)),
+                     dim3(kStreamBlock), 0, st, static_cast<const T *>(p.x), a.rows, a.R,
+                     a.inv_R, p.mean, p.var);
+  if (int e = last_launch_status()) return e;
+  const uint32_t total_vec = static_cast<uint32_t>(p.rows * p.R / VEC);
+  hipLaunchKernelGGL((row_apply_fwd_kernel<T, VEC>), dim3(stream_grid((total_vec + 255) / 256)),
+                     dim3(256), 0, st, a, FastDiv(static_cast<uint32_t>(p.R / VEC)), total_vec);
+  return last_launch_status();
+}
+
+int launch_row_fwd(const RowProblem &p, hipStream_t st) {
+  const bool vec_ok = row_vec_ok(p, false);
+  const RowArgs a = make_args(p);
+  const RowCfg cfg = pick_row_cfg(p.dtype, p.R, vec_ok, 8, 64);
+  if (cfg.ok && !tune_int("FORCE_STREAM", 0)) {
+    return run_row_fwd_cached(p.dtype, cfg, a, cached_grid(p.rows, cfg.tpr), st);
+  }
+  if (p.dtype == NBLAHIP_F16) {
+    return vec_ok ? stream_fwd_t<__half, 8>(p, a, st) : stream_fwd_t<__half, 1>(p, a, st);
+  }
+  return vec_ok ? stream_fwd_t<float, 4>(p, a, st) : stream_fwd_t<float, 1>(p, a, st);
+}
+
+size_t row_bwd_workspace_bytes(int mode, int64_t rows, int64_t R, int64_t planes) {
+  if (mode == kRowLN) {
+    // Largest persistent grid over the possible thread layouts (one row per
+    // block is the 256/1024-thread case).
+    const size_t cached =
+        static_cast<size_t>(ln_bwd_grid(rows, 1024)) * 2 * static_cast<size_t>(R) * sizeof(float);
+    const size_t stream = static_cast<size_t>(rows) * 2 * sizeof(float);
+    return align_up(std::max(cached, stream), 256);
+  }
+  return align_up(static_cast<size_t>(planes) * 2 * sizeof(float), 256) +
+         align_up(static_cast<size_t>(rows) * 2 * sizeof(float), 256);
+}
+
+template <typename T, int VEC>
+static int stream_bwd_t(const RowProblem &p, const RowArgs &a, hipStream_t st) {
+  const T *x = static_cast<const T *>(p.x);
+  const T *dy = static_cast<const T *>(p.dy);
+  const uint32_t total_vec = static_cast<uint32_t>(p.rows * p.R / VEC);
+  const FastDiv nvr(static_cast<uint32_t>(p.R / VEC));
+  if (p.mode == kRowLN) {
+    float *rs = static_cast<float *>(p.ws);
+    if (p.out) {
+      hipLaunchKernelGGL((ln_row_sums_stream_kernel<T, VEC>), dim3(stream_grid(p.rows)),
+                         dim3(kStreamBlock), 0, st, x, dy, p.gamma, p.mean, a.rows, a.R, rs);
+      if (int e = last_launch_status()) return e;
+      hipLaunchKernelGGL((row_bwd_dx_kernel<T, VEC>), dim3(stream_grid((total_vec + 255) / 256)),
+                         dim3(256), 0, st, a, rs, nvr, total_vec);
+      if (int e = last_launch_status()) return e;
+    }
+    if (p.dgamma || p.dbeta) {
+      hipLaunchKernelGGL((ln_colgrad_stream_kernel<T>), dim3((a.R + 31) / 32), dim3(256), 0, st,
+                         x, dy, p.mean, p.var, a.rows, a.R, p.eps, p.dgamma, p.dbeta, p.accum_g,
+                         p.accum_b);
+      if (int e = last_launch_status()) return e;
+    }
+    return 0;
+  }
+  const int64_t planes = p.batch * p.channels;
+  const int ppr = p.mode == kRowGN ? static_cast<int>(p.channels / p.groups) : 1;
+  float *pairs = static_cast<float *>(p.ws);
+  float *rs = reinterpret_cast<float *>(static_cast<char *>(p.ws) +
+                                        align_up(static_cast<size_t>(planes) * 2 * sizeof(float), 256));
+  hipLaunchKernelGGL((plane_sums_stream_kernel<T, VEC>), dim3(stream_grid(planes)),
+                     dim3(kStreamBlock), 0, st, x, dy, p.mean, static_cast<int>(planes),
+                     static_cast<int>(p.spatial), static_cast<uint32_t>(ppr), pairs);
+  if (int e = last_launch_status()) return e;
+  const uint32_t gmod = (p.mode == kRowGN || p.bc_gamma) ? static_cast<uint32_t>(p.channels) : 0u;
+  hipLaunchKernelGGL(plane_to_row_factors_kernel, dim3(stream_grid(p.rows)), dim3(64), 0, st,
+                     pairs, p.gamma, p.var, a.rows, ppr, gmod, p.eps, rs);
+  if (int e = last_launch_status()) return e;
+  if (p.out) {
+    hipLaunchKernelGGL((row_bwd_dx_kernel<T, VEC>), dim3(stream_grid((total_vec + 255) / 256)),
+                       dim3(256), 0, st, a, rs, nvr, total_vec);
+    if (int e = last_launch_status()) return e;
+  }
+  return 0;
+}
+
+static int launch_pair_reduce(const RowProblem &p, const float *pairs, hipStream_t st) {
+  if (!p.dgamma && !p.dbeta) return 0;
+  const int bcg = p.mode == kRowGN ? 1 : p.bc_gamma;
+  const int bcb = p.mode == kRowGN ? 1 : p.bc_beta;
+  const int64_t count = (bcg && bcb) ? p.channels : p.batch * p.channels;
+  hipLaunchKernelGGL(pair_param_reduce_kernel, dim3(static_cast<unsigned>((count + 255) / 256)),
+                     dim3(256), 0, st, pairs, static_cast<int>(p.batch),
+                     static_cast<int>(p.channels), p.dgamma, p.dbeta, bcg, bcb, p.accum_g,
+                     p.accum_b);
+  return last_launch_status();
+}
+
+int launch_row_bwd(const RowProblem &p, hipStream_t st) {
+  if (!p.out && !p.dgamma && !p.dbeta) return 0;
+  const bool vec_ok = row_vec_ok(p, true);
+  RowArgs a = make_args(p);
+  const int full = p.dtype == NBLAHIP_F16 ? 8 : 4;
+  // LayerNormalization also keeps per-column accumulators in registers.
+  const int nl1024 = p.mode == kRowLN ? (p.dtype == NBLAHIP_F16 ? 2 : 4) : 8;
+  RowCfg cfg = pick_row_cfg(p.dtype, p.R, vec_ok, nl1024, p.mode == kRowGN ? 256 : 64);
+  if (cfg.ok && p.mode == kRowGN) {
+    // Every wave-wide load must fall inside one channel.
+    const int64_t run = 64 * static_cast<int64_t>(cfg.vec);
+    if (p.spatial % run != 0) {
+      // Retry with scalar loads (run = 64 elements) before giving up.
+      cfg = pick_row_cfg(p.dtype, p.R, false, 8, 256);
+      if (cfg.ok && p.spatial % 64 != 0) cfg.ok = false;
+    }
+    if (cfg.ok) a.epc = static_cast<int>(p.spatial / (64 * cfg.vec));
+  }
+  (void)full;
+  if (cfg.ok && !tune_int("FORCE_STREAM", 0)) {
+    if (p.mode == kRowLN) {
+      const int grid = ln_bwd_grid(p.rows, cfg.tpr);
+      if (int e = run_row_bwd_cached_ln(p.dtype, cfg, a, grid, st)) return e;
+      if (p.dgamma || p.dbeta) {
+        hipLaunchKernelGGL(ln_param_reduce_kernel, dim3((2 * a.R + 31) / 32), dim3(256), 0, st,
+                           static_cast<const float *>(p.ws), grid, a.R, p.dgamma, p.dbeta,
+                           p.accum_g, p.accum_b);
+        if (int e = last_launch_status()) return e;
+      }
+      return 0;
+    }
+    const int grid = cached_grid(p.rows, cfg.tpr);
+    const int e = p.mode == kRowIN ? run_row_bwd_cached_in(p.dtype, cfg, a, grid, st)
+                                   : run_row_bwd_cached_gn(p.dtype, cfg, a, grid, st);
+    if (e) return e;
+    return launch_pair_reduce(p, static_cast<const float *>(p.ws), st);
+  }
+  int e;
+  if (p.dtype == NBLAHIP_F16) {
+    e = vec_ok ? stream_bwd_t<__half, 8>(p, a, st) : stream_bwd_t<__half, 1>(p, a, st);
+  } else {
+    e = vec_ok ? stream_bwd_t<float, 4>(p, a, st) : stream_bwd_t<float, 1>(p, a, st);
+  }
+  if (e) return e;
+  if (p.mode == kRowLN) return 0;
+  return launch_pair_reduce(p, static_cast<const float *>(p.ws), st);
+}
+
+} // namespace nblahip

@@ -1,0 +1,329 @@
+// Streaming (any row length, any alignment) versions of the row
+// normalizations.  Used when a row does not fit the register-cached kernels
+// of rows.cuh or the shape breaks their alignment rules.  x is read once for
+// the statistics (single-pass Welford, Chan merges across threads) and once
+// more for the apply step; a row that was just reduced by one block is
+// normally still in that XCD's L2 for the second read.
+#pragma once
+
+#include "common.cuh"
+#include "rows.cuh"
+
+namespace nblahip {
+
+constexpr int kStreamBlock = 256;
+
+// mean/var of each row; one block per row (grid-stride).
+template <typename T, int VEC>
+__global__ void __launch_bounds__(kStreamBlock)
+row_stats_stream_kernel(const T *__restrict__ x, int rows, int R, float inv_R,
+                        float *__restrict__ mean, float *__restrict__ var) {
+  __shared__ float lds[3 * (kStreamBlock / kWave)];
+  constexpr int U = 4;
+  const int nv = R / VEC;
+  for (int row = blockIdx.x; row < rows; row += gridDim.x) {
+    const T *xr = x + static_cast<size_t>(row) * R;
+    Welford w{0.f, 0.f, 0.f};
+    for (int v0 = threadIdx.x; v0 < nv; v0 += kStreamBlock * U) {
+      float vals[U * VEC];
+      int cnt = 0;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int v = v0 + u * kStreamBlock;
+        float tmp[VEC];
+        if (v < nv) {
+          load_vec<T, VEC>(xr + static_cast<size_t>(v) * VEC, tmp);
+          cnt += VEC;
+        } else {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) tmp[j] = 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) vals[u * VEC + j] = tmp[j];
+      }
+      welford_add_chunk<U * VEC>(w, vals, cnt);
+    }
+    w = block_welford(w, lds);
+    if (threadIdx.x == 0) {
+      mean[row] = w.mean;
+      var[row] = w.m2 * inv_R;
+    }
+    __syncthreads();
+  }
+}
+
+// y = (x-mean[row])*gamma[p]*istd[row] + beta[p] over the whole tensor.
+// nvr = vectors per row.
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+row_apply_fwd_kernel(const RowArgs a, FastDiv nvr, uint32_t total_vec) {
+  const T *__restrict__ x = static_cast<const T *>(a.x);
+  T *__restrict__ y = static_cast<T *>(a.out);
+  for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total_vec; i += gridDim.x * 256u) {
+    const uint32_t row = nvr.div(i);
+    const uint32_t col = (i - row * nvr.d) * VEC;
+    const float mean = a.mean[row];
+    const float istd = inv_std(a.var[row], a.eps);
+    float v[VEC], o[VEC];
+    load_vec<T, VEC>(x + static_cast<size_t>(i) * VEC, v);
+    if (a.percol) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float g = a.gamma ? a.gamma[col + j] : 1.f;
+        const float b = a.beta ? a.beta[col + j] : 0.f;
+        o[j] = (v[j] - mean) * (g * istd) + b;
+      }
+    } else {
+      // VEC divides the parameter run length, so one index serves the vector.
+      const uint32_t poff = a.pdiv.div(col);
+      const float g = (a.gamma ? a.gamma[(row % a.pmod) * a.pmul + poff] : 1.f) * istd;
+      const float b = a.beta ? a.beta[(row % a.pmod_b) * a.pmul + poff] : 0.f;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) o[j] = (v[j] - mean) * g + b;
+    }
+    store_vec<T, VEC>(y + static_cast<size_t>(i) * VEC, o);
+  }
+}
+
+// Per-row (s1, t2) for LayerNormalization: s1 = sum dy*gamma[col],
+// t2 = sum dy*gamma[col]*(x-mean).  rs[2*row], rs[2*row+1].
+template <typename T, int VEC>
+__global__ void __launch_bounds__(kStreamBlock)
+ln_row_sums_stream_kernel(const T *__restrict__ x, const T *__restrict__ dy,
+                          const float *__restrict__ gamma,
+                          const float *__restrict__ mean, int rows, int R,
+                          float *__restrict__ rs) {
+  __shared__ float lds[2 * (kStreamBlock / kWave)];
+  const int nv = R / VEC;
+  for (int row = blockIdx.x; row < rows; row += gridDim.x) {
+    const size_t base = static_cast<size_t>(row) * R;
+    const float m = mean[row];
+    float s1 = 0.f, t2 = 0.f;
+    for (int v = threadIdx.x; v < nv; v += kStreamBlock) {
+      float xv[VEC], dv[VEC];
+      load_vec<T, VEC>(x + base + static_cast<size_t>(v) * VEC, xv);
+      load_vec<T, VEC>(dy + base + static_cast<size_t>(v) * VEC, dv);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float dg = dv[j] * (gamma ? gamma[v * VEC + j] : 1.f);
+        s1 += dg;
+        t2 += dg * (xv[j] - m);
+      }
+    }
+    block_sum2(s1, t2, lds);
+    if (threadIdx.x == 0) {
+      rs[2 * static_cast<size_t>(row)] = s1;
+      rs[2 * static_cast<size_t>(row) + 1] = t2;
+    }
+    __syncthreads();
+  }
+}
+
+// Per-plane sums for Instance/GroupNormalization: plane p = (n, c) of length L,
+// statistics row = p / sdiv.  pairs[2p] = sum dy*(x-mean), pairs[2p+1] = sum dy.
+template <typename T, int VEC>
+__global__ void __launch_bounds__(kStreamBlock)
+plane_sums_stream_kernel(const T *__restrict__ x, const T *__restrict__ dy,
+                         const float *__restrict__ mean, int planes, int L,
+                         uint32_t sdiv, float *__restrict__ pairs) {
+  __shared__ float lds[2 * (kStreamBlock / kWave)];
+  const int nv = L / VEC;
+  for (int p = blockIdx.x; p < planes; p += gridDim.x) {
+    const size_t base = static_cast<size_t>(p) * L;
+    const float m = mean[static_cast<uint32_t>(p) / sdiv];
+    float sdx = 0.f, sdy = 0.f;
+    for (int v = threadIdx.x; v < nv; v += kStreamBlock) {
+      float xv[VEC], dv[VEC];
+      load_vec<T, VEC>(x + base + static_cast<size_t>(v) * VEC, xv);
+      load_vec<T, VEC>(dy + base + static_cast<size_t>(v) * VEC, dv);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        sdy += dv[j];
+        sdx += dv[j] * (xv[j] - m);
+      }
+    }
+    block_sum2(sdx, sdy, lds);
+    if (threadIdx.x == 0) {
+      pairs[2 * static_cast<size_t>(p)] = sdx;
+      pairs[2 * static_cast<size_t>(p) + 1] = sdy;
+    }
+    __syncthreads();
+  }
+}
+
+// From per-plane sums to per-statistics-row (s1, t2), weighting each plane with
+// its gamma; also rescales pairs[2p] by istd so that it is the dgamma part.
+//   stat row r owns planes [r*ppr, (r+1)*ppr); gamma index of plane p:
+//   gmod == 0 : p (per-sample parameter)   else p % gmod (broadcast over batch)
+__global__ void __launch_bounds__(64)
+plane_to_row_factors_kernel(float *__restrict__ pairs, const float *__restrict__ gamma,
+                            const float *__restrict__ var, int rows, int ppr,
+                            uint32_t gmod, float eps, float *__restrict__ rs) {
+  for (int r = blockIdx.x; r < rows; r += gridDim.x) {
+    const float istd = inv_std(var[r], eps);
+    float s1 = 0.f, t2 = 0.f;
+    for (int c = threadIdx.x; c < ppr; c += 64) {
+      const uint32_t p = static_cast<uint32_t>(r) * ppr + c;
+      const float g = gamma ? gamma[gmod ? p % gmod : p] : 1.f;
+      const float sdx = pairs[2 * static_cast<size_t>(p)];
+      s1 += g * pairs[2 * static_cast<size_t>(p) + 1];
+      t2 += g * sdx;
+      pairs[2 * static_cast<size_t>(p)] = sdx * istd;
+    }
+    s1 = wave_sum(s1);
+    t2 = wave_sum(t2);
+    if (threadIdx.x == 0) {
+      rs[2 * static_cast<size_t>(r)] = s1;
+      rs[2 * static_cast<size_t>(r) + 1] = t2;
+    }
+  }
+}
+
+// dx = dy*gamma[p]*istd + ca*(x-mean) + cb, elementwise over the tensor.
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+row_bwd_dx_kernel(const RowArgs a, const float *__restrict__ rs, FastDiv nvr,
+                  uint32_t total_vec) {
+  const T *__restrict__ x = static_cast<const T *>(a.x);
+  const T *__restrict__ dy = static_cast<const T *>(a.dy);
+  T *__restrict__ dx = static_cast<T *>(a.out);
+  for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total_vec; i += gridDim.x * 256u) {
+    const uint32_t row = nvr.div(i);
+    const uint32_t col = (i - row * nvr.d) * VEC;
+    const float mean = a.mean[row];
+    const float istd = inv_std(a.var[row], a.eps);
+    const float s1 = rs[2 * static_cast<size_t>(row)];
+    const float t2 = rs[2 * static_cast<size_t>(row) + 1];
+    const float ca = -t2 * istd * istd * istd * a.inv_R +
+                     (a.dvar ? 2.f * a.dvar[row] * a.inv_R : 0.f);
+    const float cb = -s1 * istd * a.inv_R + (a.dmean ? a.dmean[row] * a.inv_R : 0.f);
+    float xv[VEC], dv[VEC], o[VEC];
+    load_vec<T, VEC>(x + static_cast<size_t>(i) * VEC, xv);
+    load_vec<T, VEC>(dy + static_cast<size_t>(i) * VEC, dv);
+    if (a.percol) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float g = a.gamma ? a.gamma[col + j] : 1.f;
+        o[j] = dv[j] * g * istd + ca * (xv[j] - mean) + cb;
+      }
+    } else {
+      const uint32_t pidx = (row % a.pmod) * a.pmul + a.pdiv.div(col);
+      const float gi = (a.gamma ? a.gamma[pidx] : 1.f) * istd;
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) o[j] = dv[j] * gi + ca * (xv[j] - mean) + cb;
+    }
+    if (a.accum_dx) {
+      float old[VEC];
+      load_vec<T, VEC>(dx + static_cast<size_t>(i) * VEC, old);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) o[j] += old[j];
+    }
+    store_vec<T, VEC>(dx + static_cast<size_t>(i) * VEC, o);
+  }
+}
+
+// LayerNormalization dgamma/dbeta, any shape: block = 32 columns x 8 row
+// groups; each block owns a 32-column strip and walks all rows.
+template <typename T>
+__global__ void __launch_bounds__(256)
+ln_colgrad_stream_kernel(const T *__restrict__ x, const T *__restrict__ dy,
+                         const float *__restrict__ mean, const float *__restrict__ var,
+                         int rows, int R, float eps, float *__restrict__ dgamma,
+                         float *__restrict__ dbeta, int accum_g, int accum_b) {
+  __shared__ float rg[8][33];
+  __shared__ float rb[8][33];
+  const int cx = threadIdx.x & 31;
+  const int py = threadIdx.x >> 5;
+  const int col = blockIdx.x * 32 + cx;
+  float sg = 0.f, sb = 0.f;
+  if (col < R) {
+    for (int r = py; r < rows; r += 8) {
+      const size_t i = static_cast<size_t>(r) * R + col;
+      const float d = to_f32<T>(dy[i]);
+      sg += d * (to_f32<T>(x[i]) - mean[r]) * inv_std(var[r], eps);
+      sb += d;
+    }
+  }
+  rg[py][cx] = sg;
+  rb[py][cx] = sb;
+  __syncthreads();
+  if (py == 0 && col < R) {
+    float tg = 0.f, tb = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      tg += rg[i][cx];
+      tb += rb[i][cx];
+    }
+    if (dgamma) dgamma[col] = tg + (accum_g ? dgamma[col] : 0.f);
+    if (dbeta) dbeta[col] = tb + (accum_b ? dbeta[col] : 0.f);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Second stage of the LayerNormalization parameter gradients: column sums of
+// the per-block partials ws[nparts][2][R] -> dgamma[R], dbeta[R].
+// Block = 32 columns x 8 part-groups; coalesced 128-byte reads.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+ln_param_reduce_kernel(const float *__restrict__ ws, int nparts, int R,
+                       float *__restrict__ dgamma, float *__restrict__ dbeta,
+                       int accum_g, int accum_b) {
+  __shared__ float red[8][33];
+  const int cx = threadIdx.x & 31;
+  const int py = threadIdx.x >> 5;
+  const int col2 = blockIdx.x * 32 + cx; // column in the [2R] concatenation
+  float s = 0.f;
+  if (col2 < 2 * R) {
+    for (int p = py; p < nparts; p += 8) s += ws[static_cast<size_t>(p) * 2 * R + col2];
+  }
+  red[py][cx] = s;
+  __syncthreads();
+  if (py == 0 && col2 < 2 * R) {
+    float tot = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) tot += red[i][cx];
+    if (col2 < R) {
+      if (dgamma) dgamma[col2] = tot + (accum_g ? dgamma[col2] : 0.f);
+    } else {
+      if (dbeta) dbeta[col2 - R] = tot + (accum_b ? dbeta[col2 - R] : 0.f);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Second stage of Instance/GroupNormalization parameter gradients:
+// pairs[n][P][2] (dgamma part, dbeta part) -> sum over n when the parameter
+// is broadcast over the batch, otherwise element-wise.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+pair_param_reduce_kernel(const float *__restrict__ pairs, int n, int P,
+                         float *__restrict__ dgamma, float *__restrict__ dbeta,
+                         int bc_gamma, int bc_beta, int accum_g, int accum_b) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (dgamma) {
+    const int count = bc_gamma ? P : n * P;
+    if (i < count) {
+      float s = 0.f;
+      if (bc_gamma) {
+        for (int b = 0; b < n; ++b) s += pairs[2 * (static_cast<size_t>(b) * P + i)];
+      } else {
+        s = pairs[2 * static_cast<size_t>(i)];
+      }
+      dgamma[i] = s + (accum_g ? dgamma[i] : 0.f);
+    }
+  }
+  if (dbeta) {
+    const int count = bc_beta ? P : n * P;
+    if (i < count) {
+      float s = 0.f;
+      if (bc_beta) {
+        for (int b = 0; b < n; ++b) s += pairs[2 * (static_cast<size_t>(b) * P + i) + 1];
+      } else {
+        s = pairs[2 * static_cast<size_t>(i) + 1];
+      }
+      dbeta[i] = s + (accum_b ? dbeta[i] : 0.f);
+    }
+  }
+}
+
+} // namespace nblahip

@@ -1,0 +1,186 @@
+// Runtime shims of the C-ABI (device management, memory, dtype conversion)
+// and the small host utilities shared by the launch code.
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+
+#include "common.cuh"
+#include "launch.hpp"
+
+namespace nblahip {
+
+int device_cus() {
+  static std::mutex mu;
+  static int cus[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  std::lock_guard<std::mutex> lock(mu);
+  if (cus[dev] == 0) {
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+      v = 256;
+    cus[dev] = v;
+  }
+  return cus[dev];
+}
+
+int tune_int(const char *name, int fallback) {
+  static std::mutex mu;
+  static std::unordered_map<std::string, int> cache;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = cache.find(name);
+  if (it != cache.end()) return it->second;
+  int v = fallback;
+  const std::string key = std::string("NBLAHIP_") + name;
+  if (const char *s = std::getenv(key.c_str())) {
+    char *end = nullptr;
+    const long parsed = std::strtol(s, &end, 10);
+    if (end != s && parsed >= 0 && parsed < (1 << 20)) v = static_cast<int>(parsed);
+  }
+  cache.emplace(name, v);
+  return v;
+}
+
+template <typename D, typename S>
+__global__ void __launch_bounds__(256)
+convert_kernel(D *__restrict__ dst, const S *__restrict__ src, int64_t n) {
+  for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < n; i += gridDim.x * 256ll)
+    dst[i] = from_f32<D>(to_f32<S>(src[i]));
+}
+
+template <typename D>
+__global__ void __launch_bounds__(256) fill_kernel(D *__restrict__ dst, float v, int64_t n) {
+  const D d = from_f32<D>(v);
+  for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < n; i += gridDim.x * 256ll) dst[i] = d;
+}
+
+static unsigned flat_grid(int64_t n) {
+  const int64_t b = (n + 255) / 256;
+  return static_cast<unsigned>(b < 1 ? 1 : (b > 65536 ? 65536 : b));
+}
+
+} // namespace nblahip
+
+using namespace nblahip;
+
+static int hip_status(hipError_t e) { return e == hipSuccess ? 0 : static_cast<int>(e); }
+
+extern "C" {
+
+int nblahip_abi_version(void) { return 1; }
+
+const char *nblahip_error_string(int code) {
+  switch (code) {
+  case NBLAHIP_OK: return "success";
+  case NBLAHIP_EINVAL: return "nblahip: invalid argument (null pointer, negative size or unknown dtype)";
+  case NBLAHIP_EWORKSPACE: return "nblahip: workspace is null, misaligned or too small";
+  case NBLAHIP_ERANGE: return "nblahip: tensor has 2^31 or more elements";
+  case NBLAHIP_EALIAS: return "nblahip: output overlaps an input";
+  default: break;
+  }
+  if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+  return "nblahip: unknown status";
+}
+
+int nblahip_device_count(int *count) {
+  if (!count) return NBLAHIP_EINVAL;
+  return hip_status(hipGetDeviceCount(count));
+}
+int nblahip_set_device(int device) { return hip_status(hipSetDevice(device)); }
+int nblahip_get_device(int *device) {
+  if (!device) return NBLAHIP_EINVAL;
+  return hip_status(hipGetDevice(device));
+}
+int nblahip_device_synchronize(void) { return hip_status(hipDeviceSynchronize()); }
+int nblahip_stream_synchronize(void *stream) {
+  return hip_status(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+}
+
+int nblahip_device_info(int device, char *name, size_t name_len, int *compute_units,
+                        int *wave_size, size_t *total_mem) {
+  hipDeviceProp_t prop;
+  const hipError_t e = hipGetDeviceProperties(&prop, device);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (name && name_len) {
+    std::strncpy(name, prop.name, name_len - 1);
+    name[name_len - 1] = '\0';
+  }
+  if (compute_units) *compute_units = prop.multiProcessorCount;
+  if (wave_size) *wave_size = prop.warpSize;
+  if (total_mem) *total_mem = prop.totalGlobalMem;
+  return 0;
+}
+
+int nblahip_malloc(void **ptr, size_t bytes) {
+  if (!ptr) return NBLAHIP_EINVAL;
+  *ptr = nullptr;
+  if (bytes == 0) return 0;
+  return hip_status(hipMalloc(ptr, bytes));
+}
+int nblahip_free(void *ptr) { return ptr ? hip_status(hipFree(ptr)) : 0; }
+
+int nblahip_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream) {
+  if (bytes == 0) return 0;
+  if (!dst || !src) return NBLAHIP_EINVAL;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (int e = hip_status(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, st))) return e;
+  return hip_status(hipStreamSynchronize(st)); // pageable host memory: make the call blocking
+}
+int nblahip_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream) {
+  if (bytes == 0) return 0;
+  if (!dst || !src) return NBLAHIP_EINVAL;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (int e = hip_status(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, st))) return e;
+  return hip_status(hipStreamSynchronize(st));
+}
+int nblahip_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream) {
+  if (bytes == 0) return 0;
+  if (!dst || !src) return NBLAHIP_EINVAL;
+  return hip_status(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice,
+                                   static_cast<hipStream_t>(stream)));
+}
+int nblahip_memset(void *dst, int byte, size_t bytes, void *stream) {
+  if (bytes == 0) return 0;
+  if (!dst) return NBLAHIP_EINVAL;
+  return hip_status(hipMemsetAsync(dst, byte, bytes, static_cast<hipStream_t>(stream)));
+}
+
+int nblahip_convert(void *dst, int dst_dtype, const void *src, int src_dtype, int64_t n,
+                    void *stream) {
+  if (n == 0) return 0;
+  if (!dst || !src || n < 0) return NBLAHIP_EINVAL;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 g(flat_grid(n)), b(256);
+  if (dst_dtype == NBLAHIP_F32 && src_dtype == NBLAHIP_F16) {
+    hipLaunchKernelGGL((convert_kernel<float, __half>), g, b, 0, st, static_cast<float *>(dst),
+                       static_cast<const __half *>(src), n);
+  } else if (dst_dtype == NBLAHIP_F16 && src_dtype == NBLAHIP_F32) {
+    hipLaunchKernelGGL((convert_kernel<__half, float>), g, b, 0, st, static_cast<__half *>(dst),
+                       static_cast<const float *>(src), n);
+  } else if (dst_dtype == src_dtype && (dst_dtype == NBLAHIP_F32 || dst_dtype == NBLAHIP_F16)) {
+    const size_t bytes = static_cast<size_t>(n) * (dst_dtype == NBLAHIP_F32 ? 4 : 2);
+    return hip_status(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, st));
+  } else {
+    return NBLAHIP_EINVAL;
+  }
+  return last_launch_status();
+}
+
+int nblahip_fill(void *dst, int dtype, float value, int64_t n, void *stream) {
+  if (n == 0) return 0;
+  if (!dst || n < 0) return NBLAHIP_EINVAL;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 g(flat_grid(n)), b(256);
+  if (dtype == NBLAHIP_F32) {
+    hipLaunchKernelGGL((fill_kernel<float>), g, b, 0, st, static_cast<float *>(dst), value, n);
+  } else if (dtype == NBLAHIP_F16) {
+    hipLaunchKernelGGL((fill_kernel<__half>), g, b, 0, st, static_cast<__half *>(dst), value, n);
+  } else {
+    return NBLAHIP_EINVAL;
+  }
+  return last_launch_status();
+}
+
+} // extern "C"

@@ -1,0 +1,254 @@
+"""BatchNormalization parity on the GPU: the HIP path, called through the
+C-ABI, against the float64 oracle on the same seeded inputs."""
+import numpy as np
+import pytest
+import torch
+
+from _util import assert_close, dtype_name, load_package, rounded, to_dev, to_np
+from oracle import norm_ref as R
+
+pytestmark = pytest.mark.gpu
+K = load_package()
+
+# (shape, axis): planes layout, channel-last, odd sizes that break 16-byte
+# vectors, single-channel, sizes below one wavefront, 2-D input.
+SMALL = [
+    ((4, 8, 6, 6), 1), ((2, 3, 5, 7), 1), ((3, 16, 49), 1), ((5, 7), 1), ((2, 1, 9), 1),
+    ((1, 4, 64, 64), 1), ((6, 5, 4, 8), 3), ((64, 64), 1), ((33, 24), 1), ((7, 3, 5, 12), 3),
+    ((4, 6, 40), 2), ((2, 300, 3), 1), ((129, 5, 5, 96), 3), ((3, 2, 2, 2050), 3),
+]
+DTYPES = [torch.float32, torch.float16]
+
+
+def make_bn(shape, axis, dtype, seed, mean=0.0, std=1.0):
+    rng = np.random.default_rng(seed)
+    c = shape[axis]
+    x = rounded(rng.standard_normal(shape) * std + mean, dtype)
+    dy = rounded(rng.standard_normal(shape), dtype)
+    g = rng.uniform(0.5, 1.5, c).astype(np.float32).astype(np.float64)
+    b = (rng.standard_normal(c) * 0.1).astype(np.float32).astype(np.float64)
+    rm = (rng.standard_normal(c) * 0.1).astype(np.float32).astype(np.float64)
+    rv = rng.uniform(0.5, 2.0, c).astype(np.float32).astype(np.float64)
+    return x, dy, g, b, rm, rv
+
+
+@pytest.mark.parametrize("shape,axis", SMALL)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("affine", [True, False])
+def test_bn_inference(shape, axis, dtype, affine):
+    x, _, g, b, rm, rv = make_bn(shape, axis, dtype, 0)
+    if not affine:
+        g = b = None
+    ref = R.bn_forward_global(x, b, g, rm, rv, axis, 1e-5)
+    y = K.bn_forward_global(to_dev(x, dtype), to_dev(b), to_dev(g), to_dev(rm), to_dev(rv), axis, 1e-5)
+    assert_close(to_np(y), ref, dtype_name(dtype), "y", "y")
+
+
+@pytest.mark.parametrize("shape,axis", SMALL)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_bn_training_forward_backward(shape, axis, dtype):
+    c = shape[axis]
+    if int(np.prod(shape)) // c < 2:
+        pytest.skip("N == 1")
+    dn = dtype_name(dtype)
+    x, dy, g, b, rm, rv = make_bn(shape, axis, dtype, 1, mean=1.0, std=2.0)
+    y_r, m_r, v_r, rm_r, rv_r = R.bn_forward_batch(x, b, g, rm, rv, axis, 0.9, 1e-5)
+    dx_r, dg_r, db_r = R.bn_backward_batch(x, dy, g, m_r, v_r, axis, 1e-5)
+
+    xd, dyd, gd, bd = to_dev(x, dtype), to_dev(dy, dtype), to_dev(g), to_dev(b)
+    rmd, rvd = to_dev(rm), to_dev(rv)
+    y, m, v = K.bn_forward_batch(xd, bd, gd, rmd, rvd, axis, 0.9, 1e-5)
+    assert_close(to_np(y), y_r, dn, "y", "y")
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    assert_close(to_np(rmd), rm_r, dn, "stat", "running_mean")
+    assert_close(to_np(rvd), rv_r, dn, "stat", "running_var")
+    dx, dg, db = K.bn_backward(xd, dyd, gd, m, v, axis, 1e-5)
+    assert_close(to_np(dx), dx_r, dn, "grad", "dx")
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
+
+
+@pytest.mark.parametrize("shape,axis", [((4, 8, 6, 6), 1), ((37, 24), 1), ((6, 5, 4, 8), 3)])
+def test_bn_flags(shape, axis):
+    """no_scale/no_bias, recompute (no running update), accumulation,
+    propagate_down subsets, 3-output dmean/dvar."""
+    dtype = torch.float32
+    c = shape[axis]
+    x, dy, g, b, rm, rv = make_bn(shape, axis, dtype, 2)
+    rng = np.random.default_rng(3)
+    dm, dv = rng.standard_normal(c), rng.standard_normal(c)
+    xd, dyd = to_dev(x), to_dev(dy)
+
+    # no_scale / no_bias and recompute_impl (running stats untouched = NULL)
+    y_r, m_r, v_r, _, _ = R.bn_forward_batch(x, None, None, None, None, axis, 0.9, 1e-5)
+    y, m, v = K.bn_forward_batch(xd, None, None, None, None, axis, 0.9, 1e-5)
+    assert_close(to_np(y), y_r, "f32", "y", "y no affine")
+    dx_r, dg_r, db_r = R.bn_backward_batch(x, dy, None, m_r, v_r, axis, 1e-5, dm, dv)
+    dx, dg, db = K.bn_backward(xd, dyd, None, m, v, axis, 1e-5, dmean=to_dev(dm), dvar=to_dev(dv))
+    assert_close(to_np(dx), dx_r, "f32", "grad", "dx 3-output")
+    assert_close(to_np(dg), dg_r, "f32", "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, "f32", "pgrad", "dbeta")
+
+    # accumulation onto existing gradients, gamma present
+    _, m_r, v_r, _, _ = R.bn_forward_batch(x, b, g, None, None, axis, 0.9, 1e-5)
+    dx_r, dg_r, db_r = R.bn_backward_batch(x, dy, g, m_r, v_r, axis, 1e-5)
+    pre_dx = rng.standard_normal(shape).astype(np.float32)
+    pre_g = rng.standard_normal(c).astype(np.float32)
+    pre_b = rng.standard_normal(c).astype(np.float32)
+    dxd, dgd, dbd = to_dev(pre_dx), to_dev(pre_g), to_dev(pre_b)
+    K.bn_backward(xd, dyd, to_dev(g), to_dev(m_r), to_dev(v_r), axis, 1e-5, dx=dxd, dgamma=dgd,
+                  dbeta=dbd, accum=(True, True, True))
+    assert_close(to_np(dxd), dx_r + pre_dx, "f32", "grad", "dx accum")
+    assert_close(to_np(dgd), dg_r + pre_g, "f32", "pgrad", "dgamma accum")
+    assert_close(to_np(dbd), db_r + pre_b, "f32", "pgrad", "dbeta accum")
+
+    # propagate_down subsets: only parameters / only dx
+    sentinel = to_dev(np.full(shape, 7.0, np.float32))
+    _, dg, db = K.bn_backward(xd, dyd, to_dev(g), to_dev(m_r), to_dev(v_r), axis, 1e-5,
+                              need=(False, True, True))
+    assert_close(to_np(dg), dg_r, "f32", "pgrad", "dgamma only")
+    assert_close(to_np(db), db_r, "f32", "pgrad", "dbeta only")
+    dx, _, _ = K.bn_backward(xd, dyd, to_dev(g), to_dev(m_r), to_dev(v_r), axis, 1e-5, dx=sentinel,
+                             need=(True, False, False))
+    assert_close(to_np(dx), dx_r, "f32", "grad", "dx only")
+
+
+@pytest.mark.parametrize("shape,axis", [((4, 8, 6, 6), 1), ((6, 5, 4, 8), 3)])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_bn_inference_mode_backward(shape, axis, dtype):
+    dn = dtype_name(dtype)
+    x, dy, g, b, rm, rv = make_bn(shape, axis, dtype, 4)
+    dx_r, dg_r, db_r = R.bn_backward_global(x, dy, g, rm, rv, axis, 1e-5)
+    dx, dg, db = K.bn_backward(to_dev(x, dtype), to_dev(dy, dtype), to_dev(g), to_dev(rm),
+                               to_dev(rv), axis, 1e-5, batch_stat=False)
+    assert_close(to_np(dx), dx_r, dn, "grad", "dx")
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
+
+
+def test_bn_constant_input_and_determinism():
+    x = torch.full((8, 16, 14, 14), 2.5, device="cuda")
+    b = torch.linspace(-1, 1, 16, device="cuda")
+    y, m, v = K.bn_forward_batch(x, b, torch.ones(16, device="cuda"), None, None, 1, 0.9, 1e-5)
+    assert torch.equal(v, torch.zeros_like(v))
+    assert torch.equal(y, b.view(1, 16, 1, 1).expand_as(x).contiguous())
+    xr = torch.randn(16, 32, 28, 28, device="cuda")
+    a1 = K.bn_forward_batch(xr, None, None, None, None, 1, 0.9, 1e-5)
+    a2 = K.bn_forward_batch(xr, None, None, None, None, 1, 0.9, 1e-5)
+    for p, q in zip(a1, a2):
+        assert torch.equal(p, q)
+
+
+def test_bn_misaligned_views():
+    """Pointers that are not 16-byte aligned take the scalar-load plan."""
+    rng = np.random.default_rng(5)
+    shape, axis = (4, 8, 6, 6), 1
+    n = int(np.prod(shape))
+    x = rng.standard_normal(n + 1).astype(np.float32)
+    xd = to_dev(x)[1:].view(shape)
+    assert xd.data_ptr() % 16 != 0
+    xs = x[1:].reshape(shape).astype(np.float64)
+    y_r, m_r, v_r, _, _ = R.bn_forward_batch(xs, None, None, None, None, axis, 0.9, 1e-5)
+    y, m, v = K.bn_forward_batch(xd, None, None, None, None, axis, 0.9, 1e-5)
+    assert_close(to_np(y), y_r, "f32", "y", "y")
+    assert_close(to_np(v), v_r, "f32", "stat", "var")
+
+
+def test_bn_c1_inference_full_size():
+    """BASELINE config 1: x[8,64,56,56] fp32, inference, seed 0."""
+    rng = np.random.default_rng(0)
+    shape = (8, 64, 56, 56)
+    x = rng.standard_normal(shape).astype(np.float32)
+    g = rng.uniform(0.5, 1.5, 64).astype(np.float32)
+    b = (rng.standard_normal(64) * 0.1).astype(np.float32)
+    rm = (rng.standard_normal(64) * 0.1).astype(np.float32)
+    rv = rng.uniform(0.5, 2, 64).astype(np.float32)
+    ref = R.bn_forward_global(x, b, g, rm, rv, 1, 1e-5)
+    y = K.bn_forward_global(to_dev(x), to_dev(b), to_dev(g), to_dev(rm), to_dev(rv), 1, 1e-5)
+    assert_close(to_np(y), ref, "f32", "y", "y")
+
+
+def test_bn_c2_training_full_size():
+    """BASELINE config 2: x[32,256,56,56] ~ N(1,2) fp32, fwd+bwd, seed 1."""
+    rng = np.random.default_rng(1)
+    shape = (32, 256, 56, 56)
+    x = (rng.standard_normal(shape, dtype=np.float32) * 2 + 1).astype(np.float32)
+    dy = rng.standard_normal(shape, dtype=np.float32)
+    g = rng.uniform(0.5, 1.5, 256).astype(np.float32)
+    b = (rng.standard_normal(256) * 0.1).astype(np.float32)
+    rm = np.zeros(256, np.float32)
+    rv = np.ones(256, np.float32)
+    y_r, m_r, v_r, rm_r, rv_r = R.bn_forward_batch(x, b, g, rm, rv, 1, 0.9, 1e-5)
+    dx_r, dg_r, db_r = R.bn_backward_batch(x, dy, g, m_r, v_r, 1, 1e-5)
+    xd, dyd, gd, bd, rmd, rvd = map(to_dev, (x, dy, g, b, rm, rv))
+    y, m, v = K.bn_forward_batch(xd, bd, gd, rmd, rvd, 1, 0.9, 1e-5)
+    dx, dg, db = K.bn_backward(xd, dyd, gd, m, v, 1, 1e-5)
+    assert_close(to_np(y), y_r, "f32", "y", "y")
+    assert_close(to_np(m), m_r, "f32", "stat", "mean")
+    assert_close(to_np(v), v_r, "f32", "stat", "var")
+    assert_close(to_np(rmd), rm_r, "f32", "stat", "running_mean")
+    assert_close(to_np(rvd), rv_r, "f32", "stat", "running_var")
+    assert_close(to_np(dx), dx_r, "f32", "grad", "dx")
+    assert_close(to_np(dg), dg_r, "f32", "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, "f32", "pgrad", "dbeta")
+    # size-independent invariants of the batch backward
+    dxn = to_np(dx).reshape(32, 256, -1)
+    assert np.abs(dxn.sum(axis=(0, 2))).max() < 1e-2
+
+
+def test_bn_c5_channel_last_fp16_full_size():
+    """BASELINE config 5: x[256,56,56,64] fp16 with 1% outliers x50, axes=[3],
+    fp32 statistics, split reduction over 802816 rows, seed 4."""
+    rng = np.random.default_rng(4)
+    shape = (256, 56, 56, 64)
+    x = rng.standard_normal(shape, dtype=np.float32)
+    mask = rng.random(shape, dtype=np.float32) < 0.01
+    x = np.where(mask, x * 50, x).astype(np.float16)
+    del mask
+    dy = rng.standard_normal(shape, dtype=np.float32).astype(np.float16)
+    g = rng.uniform(0.5, 1.5, 64).astype(np.float32)
+    b = (rng.standard_normal(64) * 0.1).astype(np.float32)
+    rm = np.zeros(64, np.float32)
+    rv = np.ones(64, np.float32)
+    xd, dyd = torch.from_numpy(x).cuda(), torch.from_numpy(dy).cuda()
+    gd, bd, rmd, rvd = map(to_dev, (g, b, rm, rv))
+    y, m, v = K.bn_forward_batch(xd, bd, gd, rmd, rvd, 3, 0.9, 1e-5)
+    dx, dg, db = K.bn_backward(xd, dyd, gd, m, v, 3, 1e-5)
+    torch.cuda.synchronize()
+    y_r, m_r, v_r, rm_r, rv_r = R.bn_forward_batch(x, b, g, rm, rv, 3, 0.9, 1e-5)
+    assert_close(to_np(m), m_r, "f16", "stat", "mean")
+    assert_close(to_np(v), v_r, "f16", "stat", "var")
+    assert_close(to_np(rmd), rm_r, "f16", "stat", "running_mean")
+    assert_close(to_np(rvd), rv_r, "f16", "stat", "running_var")
+    assert_close(to_np(y), y_r, "f16", "y", "y")
+    del y_r
+    dx_r, dg_r, db_r = R.bn_backward_batch(x, dy, g, m_r, v_r, 3, 1e-5)
+    assert_close(to_np(dx), dx_r, "f16", "grad", "dx")
+    assert_close(to_np(dg), dg_r, "f16", "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, "f16", "pgrad", "dbeta")
+
+
+def test_bn_argument_errors():
+    x = torch.randn(4, 8, 6, 6, device="cuda")
+    L = K.lib()
+    s = torch.cuda.current_stream().cuda_stream
+    m = torch.empty(8, device="cuda")
+    y = torch.empty_like(x)
+    # unknown dtype
+    assert L.nblahip_bn_fwd_infer(x.data_ptr(), m.data_ptr(), m.data_ptr(), None, None,
+                                  y.data_ptr(), 4, 8, 36, 1e-5, 7, s) == -1
+    # missing required pointer
+    assert L.nblahip_bn_fwd_infer(None, m.data_ptr(), m.data_ptr(), None, None, y.data_ptr(), 4, 8,
+                                  36, 1e-5, 0, s) == -1
+    # workspace too small / missing
+    assert L.nblahip_bn_fwd_train(x.data_ptr(), None, None, y.data_ptr(), m.data_ptr(),
+                                  m.data_ptr(), None, None, 4, 8, 36, 0.9, 1e-5, 0, None, 0, s) == -2
+    # negative size
+    assert L.nblahip_bn_fwd_infer(x.data_ptr(), m.data_ptr(), m.data_ptr(), None, None,
+                                  y.data_ptr(), -1, 8, 36, 1e-5, 0, s) == -1
+    # empty tensor: success, nothing launched
+    assert L.nblahip_bn_fwd_infer(x.data_ptr(), m.data_ptr(), m.data_ptr(), None, None,
+                                  y.data_ptr(), 0, 8, 36, 1e-5, 0, s) == 0
+    with pytest.raises(K.NblaHipError):
+        K.check(-3)

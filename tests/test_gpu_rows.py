@@ -1,0 +1,327 @@
+"""LayerNormalization / GroupNormalization / InstanceNormalization parity on
+the GPU: HIP path through the C-ABI against the float64 oracle."""
+import numpy as np
+import pytest
+import torch
+
+from _util import assert_close, dtype_name, load_package, rounded, to_dev, to_np
+from oracle import norm_ref as R
+
+pytestmark = pytest.mark.gpu
+K = load_package()
+DTYPES = [torch.float32, torch.float16]
+
+
+def f32(a):
+    return np.asarray(a, np.float32).astype(np.float64)
+
+
+# ------------------------------------------------------------------ LN
+# (outer, R): below one wave, odd (scalar loads), one wave per row, one block
+# per row (256 / 1024 threads), longer than the register-cached limit
+# (streaming kernels), single row, R == 1.
+LN_SHAPES = [(5, 1), (7, 3), (16, 17), (33, 64), (9, 1000), (64, 1024), (130, 768), (12, 4096),
+             (5, 8192), (3, 16384), (6, 32768), (2, 70000), (3, 40004), (1, 2048), (300, 256),
+             (2, 131072)]
+
+
+def make_ln(outer, Rr, dtype, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((outer, Rr)) + rng.uniform(-3, 3, (outer, 1))
+    dy = rng.standard_normal((outer, Rr))
+    g = f32(rng.standard_normal(Rr) * 0.1 + 1)
+    b = f32(rng.standard_normal(Rr) * 0.1)
+    return rounded(x, dtype), rounded(dy, dtype), g, b
+
+
+@pytest.mark.parametrize("outer,Rr", LN_SHAPES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_ln_forward_backward(outer, Rr, dtype):
+    dn = dtype_name(dtype)
+    x, dy, g, b = make_ln(outer, Rr, dtype, 2)
+    y_r, m_r, v_r = R.ln_forward(x, b, g, outer, 1e-5)
+    dx_r, dg_r, db_r = R.ln_backward(x, dy, g, m_r, v_r, outer, 1e-5)
+    xd, dyd, gd, bd = to_dev(x, dtype), to_dev(dy, dtype), to_dev(g), to_dev(b)
+    y, m, v = K.ln_forward(xd, bd, gd, outer, 1e-5)
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    assert_close(to_np(y), y_r, dn, "y", "y")
+    dx, dg, db = K.ln_backward(xd, dyd, gd, m, v, outer, 1e-5)
+    assert_close(to_np(dx), dx_r, dn, "grad", "dx")
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
+
+
+@pytest.mark.parametrize("outer,Rr", [(33, 64), (9, 1000), (12, 4096), (2, 70000)])
+def test_ln_flags(outer, Rr):
+    """no_scale/no_bias, 3-output dmean/dvar, accumulation, propagate_down."""
+    dtype = torch.float32
+    x, dy, g, b = make_ln(outer, Rr, dtype, 3)
+    rng = np.random.default_rng(4)
+    dm, dv = f32(rng.standard_normal(outer)), f32(rng.standard_normal(outer))
+    xd, dyd = to_dev(x), to_dev(dy)
+    y_r, m_r, v_r = R.ln_forward(x, None, None, outer, 1e-5)
+    y, m, v = K.ln_forward(xd, None, None, outer, 1e-5)
+    assert_close(to_np(y), y_r, "f32", "y", "y no affine")
+    dx_r, dg_r, db_r = R.ln_backward(x, dy, None, m_r, v_r, outer, 1e-5, dm, dv)
+    dx, dg, db = K.ln_backward(xd, dyd, None, m, v, outer, 1e-5, dmean=to_dev(dm), dvar=to_dev(dv))
+    assert_close(to_np(dx), dx_r, "f32", "grad", "dx 3-output")
+    assert_close(to_np(dg), dg_r, "f32", "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, "f32", "pgrad", "dbeta")
+
+    dx_r, dg_r, db_r = R.ln_backward(x, dy, g, m_r, v_r, outer, 1e-5)
+    pre_dx = rng.standard_normal((outer, Rr)).astype(np.float32)
+    pre_g = rng.standard_normal(Rr).astype(np.float32)
+    pre_b = rng.standard_normal(Rr).astype(np.float32)
+    dxd, dgd, dbd = to_dev(pre_dx), to_dev(pre_g), to_dev(pre_b)
+    K.ln_backward(xd, dyd, to_dev(g), m, v, outer, 1e-5, dx=dxd, dgamma=dgd, dbeta=dbd,
+                  accum=(True, True, True))
+    assert_close(to_np(dxd), dx_r + pre_dx, "f32", "grad", "dx accum")
+    assert_close(to_np(dgd), dg_r + pre_g, "f32", "pgrad", "dgamma accum")
+    assert_close(to_np(dbd), db_r + pre_b, "f32", "pgrad", "dbeta accum")
+
+    _, dg, db = K.ln_backward(xd, dyd, to_dev(g), m, v, outer, 1e-5, need=(False, True, True))
+    assert_close(to_np(dg), dg_r, "f32", "pgrad", "dgamma only")
+    dx, _, _ = K.ln_backward(xd, dyd, to_dev(g), m, v, outer, 1e-5, need=(True, False, False))
+    assert_close(to_np(dx), dx_r, "f32", "grad", "dx only")
+
+
+def test_ln_invariants_and_determinism():
+    torch.manual_seed(0)
+    x = torch.randn(512, 1024, device="cuda")
+    dy = torch.randn(512, 1024, device="cuda")
+    y, m, v = K.ln_forward(x, None, None, 512, 1e-5)
+    # normalised rows: mean 0, var = var/(var+eps)
+    assert y.mean(dim=1).abs().max().item() < 1e-5
+    dx, dg, db = K.ln_backward(x, dy, None, m, v, 512, 1e-5)
+    assert dx.sum(dim=1).abs().max().item() < 1e-3
+    dx2, dg2, db2 = K.ln_backward(x, dy, None, m, v, 512, 1e-5)
+    assert torch.equal(dx, dx2) and torch.equal(dg, dg2) and torch.equal(db, db2)
+    # constant rows give y == beta exactly
+    xc = torch.full((8, 256), 3.25, device="cuda")
+    b = torch.linspace(-1, 1, 256, device="cuda")
+    yc, _, vc = K.ln_forward(xc, b, torch.ones(256, device="cuda"), 8, 1e-5)
+    assert torch.equal(vc, torch.zeros_like(vc))
+    assert torch.equal(yc, b.expand(8, 256).contiguous())
+
+
+def test_ln_misaligned_pointer():
+    rng = np.random.default_rng(6)
+    outer, Rr = 8, 1024
+    flat = rng.standard_normal(outer * Rr + 1).astype(np.float32)
+    xd = to_dev(flat)[1:].view(outer, Rr)
+    assert xd.data_ptr() % 16 != 0
+    x = flat[1:].reshape(outer, Rr).astype(np.float64)
+    y_r, m_r, v_r = R.ln_forward(x, None, None, outer, 1e-5)
+    y, m, v = K.ln_forward(xd, None, None, outer, 1e-5)
+    assert_close(to_np(y), y_r, "f32", "y", "y")
+    assert_close(to_np(v), v_r, "f32", "stat", "var")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_ln_c3_full_size(dtype):
+    """BASELINE config 3: x[32,512,1024] ~ N(0,1) + per-row offset U(-3,3),
+    gamma ~ N(1,0.1), beta ~ N(0,0.1), seed 2, fp32 and fp16."""
+    dn = dtype_name(dtype)
+    rng = np.random.default_rng(2)
+    outer, Rr = 32 * 512, 1024
+    x = rng.standard_normal((outer, Rr), dtype=np.float32) + \
+        rng.uniform(-3, 3, (outer, 1)).astype(np.float32)
+    dy = rng.standard_normal((outer, Rr), dtype=np.float32)
+    g = (rng.standard_normal(Rr) * 0.1 + 1).astype(np.float32)
+    b = (rng.standard_normal(Rr) * 0.1).astype(np.float32)
+    x, dy = rounded(x, dtype), rounded(dy, dtype)
+    y_r, m_r, v_r = R.ln_forward(x, b, g, outer, 1e-5)
+    dx_r, dg_r, db_r = R.ln_backward(x, dy, g, m_r, v_r, outer, 1e-5)
+    xd, dyd, gd, bd = to_dev(x, dtype), to_dev(dy, dtype), to_dev(g), to_dev(b)
+    y, m, v = K.ln_forward(xd, bd, gd, outer, 1e-5)
+    dx, dg, db = K.ln_backward(xd, dyd, gd, m, v, outer, 1e-5)
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    assert_close(to_np(y), y_r, dn, "y", "y")
+    assert_close(to_np(dx), dx_r, dn, "grad", "dx")
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
+
+
+# ------------------------------------------------------------------ GN
+# (n, c, spatial-shape, groups): register-cached with wave-uniform channels,
+# spatial that is not (49, 196), one channel per group, one group, tiny, big
+# groups that stream.
+GN_SHAPES = [(2, 8, (8, 8), 4), (3, 6, (5,), 2), (1, 4, (2, 2), 1), (2, 6, (4,), 6),
+             (2, 32, (7, 7), 8), (2, 32, (14, 14), 4), (4, 64, (16, 16), 8), (2, 16, (32, 32), 2),
+             (2, 256, (64, 64), 32), (1, 8, (128, 128), 1), (2, 12, (512,), 3), (2, 4, (), 2),
+             (3, 10, (64,), 5), (1, 64, (40, 40), 2)]
+
+
+def make_nc(n, c, sp, dtype, seed):
+    rng = np.random.default_rng(seed)
+    shape = (n, c) + sp
+    x = rounded(rng.standard_normal(shape) * 1.5, dtype)
+    dy = rounded(rng.standard_normal(shape), dtype)
+    g = f32(rng.uniform(0.5, 1.5, c))
+    b = f32(rng.standard_normal(c) * 0.1)
+    return x, dy, g, b
+
+
+@pytest.mark.parametrize("n,c,sp,groups", GN_SHAPES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gn_forward_backward(n, c, sp, groups, dtype):
+    dn = dtype_name(dtype)
+    x, dy, g, b = make_nc(n, c, sp, dtype, 3)
+    y_r, m_r, v_r = R.gn_forward(x, b, g, n, c, groups, 1e-5)
+    dx_r, dg_r, db_r = R.gn_backward(x, dy, g, m_r, v_r, n, c, groups, 1e-5)
+    xd, dyd, gd, bd = to_dev(x, dtype), to_dev(dy, dtype), to_dev(g), to_dev(b)
+    y, m, v = K.gn_forward(xd, bd, gd, groups, 1e-5)
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    assert_close(to_np(y), y_r, dn, "y", "y")
+    dx, dg, db = K.gn_backward(xd, dyd, gd, m, v, groups, 1e-5)
+    assert_close(to_np(dx), dx_r, dn, "grad", "dx")
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
+
+
+@pytest.mark.parametrize("n,c,sp,groups", [(4, 64, (16, 16), 8), (2, 32, (7, 7), 8)])
+def test_gn_flags(n, c, sp, groups):
+    dtype = torch.float32
+    x, dy, g, b = make_nc(n, c, sp, dtype, 5)
+    rng = np.random.default_rng(6)
+    rows = n * groups
+    dm, dv = f32(rng.standard_normal(rows)), f32(rng.standard_normal(rows))
+    xd, dyd = to_dev(x), to_dev(dy)
+    y_r, m_r, v_r = R.gn_forward(x, None, None, n, c, groups, 1e-5)
+    y, m, v = K.gn_forward(xd, None, None, groups, 1e-5)
+    assert_close(to_np(y), y_r, "f32", "y", "y no affine")
+    dx_r, dg_r, db_r = R.gn_backward(x, dy, g, m_r, v_r, n, c, groups, 1e-5, dm, dv)
+    pre_dx = rng.standard_normal(x.shape).astype(np.float32)
+    pre_g = rng.standard_normal(c).astype(np.float32)
+    pre_b = rng.standard_normal(c).astype(np.float32)
+    dxd, dgd, dbd = to_dev(pre_dx), to_dev(pre_g), to_dev(pre_b)
+    K.gn_backward(xd, dyd, to_dev(g), m, v, groups, 1e-5, dmean=to_dev(dm), dvar=to_dev(dv), dx=dxd,
+                  dgamma=dgd, dbeta=dbd, accum=(True, True, True))
+    assert_close(to_np(dxd), dx_r + pre_dx, "f32", "grad", "dx accum 3-output")
+    assert_close(to_np(dgd), dg_r + pre_g, "f32", "pgrad", "dgamma accum")
+    assert_close(to_np(dbd), db_r + pre_b, "f32", "pgrad", "dbeta accum")
+    _, dg, db = K.gn_backward(xd, dyd, to_dev(g), m, v, groups, 1e-5, dmean=to_dev(dm),
+                              dvar=to_dev(dv), need=(False, True, True))
+    assert_close(to_np(dg), dg_r, "f32", "pgrad", "dgamma only")
+    assert_close(to_np(db), db_r, "f32", "pgrad", "dbeta only")
+
+
+# ------------------------------------------------------------------ IN
+IN_SHAPES = [(2, 3, (4, 4)), (3, 5, (7,)), (1, 2, (3, 2)), (4, 16, (16, 16)), (2, 8, (64, 64)),
+             (2, 4, (7, 7)), (1, 3, (200, 200)), (2, 2, (300, 300)), (3, 7, (1,)), (2, 3, (1000,))]
+
+
+@pytest.mark.parametrize("n,c,sp", IN_SHAPES)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_in_forward_backward(n, c, sp, dtype):
+    dn = dtype_name(dtype)
+    x, dy, g, b = make_nc(n, c, sp, dtype, 3)
+    y_r, m_r, v_r = R.in_forward(x, b, g, n, c, 1e-5)
+    dx_r, dg_r, db_r = R.in_backward(x, dy, g, m_r, v_r, n, c, 1e-5)
+    xd, dyd, gd, bd = to_dev(x, dtype), to_dev(dy, dtype), to_dev(g), to_dev(b)
+    y, m, v = K.in_forward(xd, bd, gd, 1e-5)
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    assert_close(to_np(y), y_r, dn, "y", "y")
+    dx, dg, db = K.in_backward(xd, dyd, gd, m, v, 1e-5)
+    assert_close(to_np(dx), dx_r, dn, "grad", "dx")
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
+
+
+@pytest.mark.parametrize("n,c,sp", [(3, 4, (6, 6)), (2, 3, (300, 300))])
+@pytest.mark.parametrize("bcg,bcb", [(False, False), (True, False), (False, True)])
+def test_in_per_sample_parameters_and_flags(n, c, sp, bcg, bcb):
+    """gamma/beta of batch*channels elements (no broadcast over the batch),
+    mixed broadcast, 3-output dmean/dvar and accumulation."""
+    dtype = torch.float32
+    rng = np.random.default_rng(7)
+    shape = (n, c) + sp
+    x = f32(rng.standard_normal(shape))
+    dy = f32(rng.standard_normal(shape))
+    g = f32(rng.uniform(0.5, 1.5, c if bcg else n * c))
+    b = f32(rng.standard_normal(c if bcb else n * c))
+    dm, dv = f32(rng.standard_normal(n * c)), f32(rng.standard_normal(n * c))
+    g_full = np.tile(g, n) if bcg else g
+    b_full = np.tile(b, n) if bcb else b
+    y_r, m_r, v_r = R.in_forward(x, b_full, g_full, n, c, 1e-5)
+    dx_r, dg_r, db_r = R.in_backward(x, dy, g, m_r, v_r, n, c, 1e-5, dm, dv, bc_gamma=bcg,
+                                     bc_beta=bcb)
+    xd, dyd = to_dev(x), to_dev(dy)
+    y, m, v = K.in_forward(xd, to_dev(b), to_dev(g), 1e-5, bc_gamma=bcg, bc_beta=bcb)
+    assert_close(to_np(y), y_r, "f32", "y", "y")
+    pre_g = rng.standard_normal(dg_r.size).astype(np.float32)
+    dgd = to_dev(pre_g)
+    dx, _, db = K.in_backward(xd, dyd, to_dev(g), m, v, 1e-5, bc_gamma=bcg, bc_beta=bcb,
+                              dmean=to_dev(dm), dvar=to_dev(dv), dgamma=dgd,
+                              accum=(False, True, False))
+    assert_close(to_np(dx), dx_r, "f32", "grad", "dx")
+    assert_close(to_np(dgd), dg_r + pre_g, "f32", "pgrad", "dgamma accum")
+    assert_close(to_np(db), db_r, "f32", "pgrad", "dbeta")
+
+
+def test_c4_gn_and_in_full_size():
+    """BASELINE config 4: x[16,256,64,64] ~ N(0,1.5) fp16, GN with 32 groups and
+    IN on the same tensor, seed 3."""
+    rng = np.random.default_rng(3)
+    n, c, sp = 16, 256, (64, 64)
+    x = (rng.standard_normal((n, c) + sp, dtype=np.float32) * 1.5).astype(np.float16)
+    dy = rng.standard_normal((n, c) + sp, dtype=np.float32).astype(np.float16)
+    g = rng.uniform(0.5, 1.5, c).astype(np.float32)
+    b = (rng.standard_normal(c) * 0.1).astype(np.float32)
+    xd, dyd = torch.from_numpy(x).cuda(), torch.from_numpy(dy).cuda()
+    gd, bd = to_dev(g), to_dev(b)
+    # GroupNormalization
+    y, m, v = K.gn_forward(xd, bd, gd, 32, 1e-5)
+    dx, dg, db = K.gn_backward(xd, dyd, gd, m, v, 32, 1e-5)
+    y_r, m_r, v_r = R.gn_forward(x, b, g, n, c, 32, 1e-5)
+    dx_r, dg_r, db_r = R.gn_backward(x, dy, g, m_r, v_r, n, c, 32, 1e-5)
+    assert_close(to_np(m), m_r, "f16", "stat", "gn mean")
+    assert_close(to_np(v), v_r, "f16", "stat", "gn var")
+    assert_close(to_np(y), y_r, "f16", "y", "gn y")
+    assert_close(to_np(dx), dx_r, "f16", "grad", "gn dx")
+    assert_close(to_np(dg), dg_r, "f16", "pgrad", "gn dgamma")
+    assert_close(to_np(db), db_r, "f16", "pgrad", "gn dbeta")
+    # InstanceNormalization
+    y, m, v = K.in_forward(xd, bd, gd, 1e-5)
+    dx, dg, db = K.in_backward(xd, dyd, gd, m, v, 1e-5)
+    y_r, m_r, v_r = R.in_forward(x, b, g, n, c, 1e-5)
+    dx_r, dg_r, db_r = R.in_backward(x, dy, g, m_r, v_r, n, c, 1e-5)
+    assert_close(to_np(m), m_r, "f16", "stat", "in mean")
+    assert_close(to_np(v), v_r, "f16", "stat", "in var")
+    assert_close(to_np(y), y_r, "f16", "y", "in y")
+    assert_close(to_np(dx), dx_r, "f16", "grad", "in dx")
+    assert_close(to_np(dg), dg_r, "f16", "pgrad", "in dgamma")
+    assert_close(to_np(db), db_r, "f16", "pgrad", "in dbeta")
+
+
+def test_gn_with_one_channel_per_group_equals_in():
+    torch.manual_seed(1)
+    x = torch.randn(4, 16, 16, 16, device="cuda")
+    g = torch.rand(16, device="cuda") + 0.5
+    b = torch.randn(16, device="cuda")
+    y1, m1, v1 = K.gn_forward(x, b, g, 16, 1e-5)
+    y2, m2, v2 = K.in_forward(x, b, g, 1e-5)
+    assert torch.equal(y1, y2) and torch.equal(m1, m2) and torch.equal(v1, v2)
+
+
+def test_row_argument_errors():
+    L = K.lib()
+    s = torch.cuda.current_stream().cuda_stream
+    x = torch.randn(8, 64, device="cuda")
+    y = torch.empty_like(x)
+    m = torch.empty(8, device="cuda")
+    assert L.nblahip_ln_fwd(x.data_ptr(), None, None, y.data_ptr(), m.data_ptr(), None, 8, 64,
+                            1e-5, 0, s) == -1                      # var missing
+    assert L.nblahip_gn_fwd(x.data_ptr(), None, None, y.data_ptr(), m.data_ptr(), m.data_ptr(), 1,
+                            8, 64, 3, 1e-5, 0, s) == -1            # 8 channels, 3 groups
+    assert L.nblahip_ln_fwd(x.data_ptr(), None, None, y.data_ptr(), m.data_ptr(), m.data_ptr(), 0,
+                            64, 1e-5, 0, s) == 0                   # empty: no-op
+    assert L.nblahip_ln_bwd(x.data_ptr(), x.data_ptr(), None, m.data_ptr(), m.data_ptr(), None,
+                            None, y.data_ptr(), None, None, 0, 0, 0, 8, 64, 1e-5, 0, None, 0,
+                            s) == -2                               # workspace missing
+    assert L.nblahip_ln_fwd(x.data_ptr(), None, None, y.data_ptr(), m.data_ptr(), m.data_ptr(),
+                            1 << 20, 1 << 20, 1e-5, 0, s) == -3    # >= 2^31 elements
