@@ -1,0 +1,330 @@
+#!/usr/bin/env python3
+"""Benchmark of the normalization hot path on one MI355X.
+
+Headline workload (BASELINE.json configs[1]): BatchNormalization training
+forward + backward, fp32 NCHW x[32,256,56,56] ~ N(1,2), dy ~ N(0,1),
+decay_rate 0.9, eps 1e-5.  One step = one forward (batch statistics, running
+statistics update, y) plus one backward (dx, dgamma, dbeta) through the C-ABI,
+inputs resident in HBM.
+
+Prints ONE JSON line.  `value` is algorithmic GB/s of the whole step
+(8 tensor passes: forward x twice + y, backward x and dy twice + dx);
+`roofline` is the dominant kernel (backward apply: x, dy in, dx out) timed with
+HIP events on the launch stream in a second region of the same K steps;
+`cpu_baseline` is the C restatement of the reference arithmetic
+(oracle/norm_ref.c) on the same workload on the host cores; `configs` lists
+every BASELINE configuration (microseconds per call and algorithmic GB/s).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+class Workload:
+    """A named (forward, backward) pair of C-ABI calls over preallocated
+    device buffers, with the algorithmic bytes of each direction."""
+
+    def __init__(self, name, fwd, bwd, fwd_bytes, bwd_bytes, dtype, keep):
+        self.name, self.fwd, self.bwd = name, fwd, bwd
+        self.fwd_bytes, self.bwd_bytes, self.dtype = fwd_bytes, bwd_bytes, dtype
+        self.keep = keep  # references that keep the device buffers alive
+
+
+def _ws(nbytes):
+    import torch
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device="cuda")
+
+
+def make_bn(K, shape, axis, dtype, train, mean=0.0, std=1.0, outliers=False, seed=0):
+    import torch
+    L = K.lib()
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    x = torch.randn(shape, device="cuda", generator=g) * std + mean
+    if outliers:
+        mask = torch.rand(shape, device="cuda", generator=g) < 0.01
+        x = torch.where(mask, x * 50, x)
+    x = x.to(dtype).contiguous()
+    dy = torch.randn(shape, device="cuda", generator=g).to(dtype)
+    c = shape[axis]
+    gamma = torch.rand(c, device="cuda", generator=g) + 0.5
+    beta = torch.randn(c, device="cuda", generator=g) * 0.1
+    rm = torch.zeros(c, device="cuda")
+    rv = torch.ones(c, device="cuda")
+    y, dx = torch.empty_like(x), torch.empty_like(x)
+    bm, bv, dg, db = (torch.empty(c, device="cuda") for _ in range(4))
+    s0, _, s2 = K._bn_sizes(shape, axis)
+    dt = K._dtype_code(x)
+    ws = _ws(L.nblahip_bn_workspace_bytes(s0, c, s2, dt))
+    st = torch.cuda.current_stream().cuda_stream
+    S = x.numel() * x.element_size()
+
+    if train:
+        def fwd():
+            K.check(L.nblahip_bn_fwd_train(x.data_ptr(), gamma.data_ptr(), beta.data_ptr(),
+                                           y.data_ptr(), bm.data_ptr(), bv.data_ptr(),
+                                           rm.data_ptr(), rv.data_ptr(), s0, c, s2, 0.9, 1e-5, dt,
+                                           ws.data_ptr(), ws.numel(), st))
+
+        def bwd():
+            K.check(L.nblahip_bn_bwd(x.data_ptr(), dy.data_ptr(), gamma.data_ptr(), bm.data_ptr(),
+                                     bv.data_ptr(), None, None, dx.data_ptr(), dg.data_ptr(),
+                                     db.data_ptr(), 0, 0, 0, s0, c, s2, 1e-5, 1, dt, ws.data_ptr(),
+                                     ws.numel(), st))
+        return fwd, bwd, 3 * S, 5 * S, (x, dy, gamma, beta, rm, rv, y, dx, bm, bv, dg, db, ws)
+
+    def fwd():
+        K.check(L.nblahip_bn_fwd_infer(x.data_ptr(), rm.data_ptr(), rv.data_ptr(), gamma.data_ptr(),
+                                       beta.data_ptr(), y.data_ptr(), s0, c, s2, 1e-5, dt, st))
+    return fwd, None, 2 * S, 0, (x, gamma, beta, rm, rv, y)
+
+
+def make_rows(K, kind, shape, dtype, seed, **kw):
+    """kind in {"ln", "gn", "in"}; shape [outer..., R] for ln, [N,C,H,W] else."""
+    import torch
+    L = K.lib()
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    x = torch.randn(shape, device="cuda", generator=g) * kw.get("std", 1.0)
+    if kind == "ln":
+        x = x + (torch.rand(shape[:-1] + (1,), device="cuda", generator=g) * 6 - 3)
+    x = x.to(dtype).contiguous()
+    dy = torch.randn(shape, device="cuda", generator=g).to(dtype)
+    y, dx = torch.empty_like(x), torch.empty_like(x)
+    dt = K._dtype_code(x)
+    st = torch.cuda.current_stream().cuda_stream
+    S = x.numel() * x.element_size()
+    if kind == "ln":
+        R = shape[-1]
+        outer = x.numel() // R
+        gamma = torch.randn(R, device="cuda", generator=g) * 0.1 + 1
+        beta = torch.randn(R, device="cuda", generator=g) * 0.1
+        mean, var = torch.empty(outer, device="cuda"), torch.empty(outer, device="cuda")
+        dg, db = torch.empty(R, device="cuda"), torch.empty(R, device="cuda")
+        ws = _ws(L.nblahip_ln_bwd_workspace_bytes(outer, R, dt))
+
+        def fwd():
+            K.check(L.nblahip_ln_fwd(x.data_ptr(), gamma.data_ptr(), beta.data_ptr(), y.data_ptr(),
+                                     mean.data_ptr(), var.data_ptr(), outer, R, 1e-5, dt, st))
+
+        def bwd():
+            K.check(L.nblahip_ln_bwd(x.data_ptr(), dy.data_ptr(), gamma.data_ptr(), mean.data_ptr(),
+                                     var.data_ptr(), None, None, dx.data_ptr(), dg.data_ptr(),
+                                     db.data_ptr(), 0, 0, 0, outer, R, 1e-5, dt, ws.data_ptr(),
+                                     ws.numel(), st))
+    else:
+        n, c = shape[0], shape[1]
+        sp = x.numel() // (n * c)
+        gamma = torch.rand(c, device="cuda", generator=g) + 0.5
+        beta = torch.randn(c, device="cuda", generator=g) * 0.1
+        dg, db = torch.empty(c, device="cuda"), torch.empty(c, device="cuda")
+        if kind == "gn":
+            G = kw["groups"]
+            mean, var = torch.empty(n * G, device="cuda"), torch.empty(n * G, device="cuda")
+            ws = _ws(L.nblahip_gn_bwd_workspace_bytes(n, c, sp, G, dt))
+
+            def fwd():
+                K.check(L.nblahip_gn_fwd(x.data_ptr(), gamma.data_ptr(), beta.data_ptr(),
+                                         y.data_ptr(), mean.data_ptr(), var.data_ptr(), n, c, sp, G,
+                                         1e-5, dt, st))
+
+            def bwd():
+                K.check(L.nblahip_gn_bwd(x.data_ptr(), dy.data_ptr(), gamma.data_ptr(),
+                                         mean.data_ptr(), var.data_ptr(), None, None, dx.data_ptr(),
+                                         dg.data_ptr(), db.data_ptr(), 0, 0, 0, n, c, sp, G, 1e-5,
+                                         dt, ws.data_ptr(), ws.numel(), st))
+        else:
+            mean, var = torch.empty(n * c, device="cuda"), torch.empty(n * c, device="cuda")
+            ws = _ws(L.nblahip_in_bwd_workspace_bytes(n, c, sp, dt))
+
+            def fwd():
+                K.check(L.nblahip_in_fwd(x.data_ptr(), gamma.data_ptr(), beta.data_ptr(),
+                                         y.data_ptr(), mean.data_ptr(), var.data_ptr(), n, c, sp, 1,
+                                         1, 1e-5, dt, st))
+
+            def bwd():
+                K.check(L.nblahip_in_bwd(x.data_ptr(), dy.data_ptr(), gamma.data_ptr(),
+                                         mean.data_ptr(), var.data_ptr(), None, None, dx.data_ptr(),
+                                         dg.data_ptr(), db.data_ptr(), 0, 0, 0, n, c, sp, 1, 1,
+                                         1e-5, dt, ws.data_ptr(), ws.numel(), st))
+    return fwd, bwd, 2 * S, 3 * S, (x, dy, gamma, beta, y, dx, mean, var, dg, db, ws)
+
+
+def time_calls(fns, steps, warmup):
+    """Wall-clock milliseconds per step of calling every fn in fns once."""
+    import torch
+    for _ in range(warmup):
+        for f in fns:
+            f()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        for f in fns:
+            f()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def config_table(K, steps, warmup):
+    """Every BASELINE configuration: us per call and algorithmic GB/s."""
+    import torch
+    specs = [
+        ("C1 BN inference fp32 [8,64,56,56]", lambda: make_bn(K, (8, 64, 56, 56), 1, torch.float32, False, seed=0)),
+        ("C2 BN training fp32 NCHW [32,256,56,56]", lambda: make_bn(K, (32, 256, 56, 56), 1, torch.float32, True, 1.0, 2.0, seed=1)),
+        ("C3 LN fp32 [32,512,1024]", lambda: make_rows(K, "ln", (32, 512, 1024), torch.float32, 2)),
+        ("C3 LN fp16 [32,512,1024]", lambda: make_rows(K, "ln", (32, 512, 1024), torch.float16, 2)),
+        ("C4 GN fp16 [16,256,64,64] G=32", lambda: make_rows(K, "gn", (16, 256, 64, 64), torch.float16, 3, std=1.5, groups=32)),
+        ("C4 IN fp16 [16,256,64,64]", lambda: make_rows(K, "in", (16, 256, 64, 64), torch.float16, 3, std=1.5)),
+        ("C5 BN training fp16 NHWC [256,56,56,64]", lambda: make_bn(K, (256, 56, 56, 64), 3, torch.float16, True, outliers=True, seed=4)),
+    ]
+    out = []
+    for name, make in specs:
+        fwd, bwd, fb, bb, keep = make()
+        row = {"config": name}
+        ms_f = time_calls([fwd], steps, warmup)
+        row["fwd_us"] = round(ms_f * 1e3, 2)
+        row["fwd_GBps"] = round(fb / ms_f / 1e6, 1)
+        if bwd is not None:
+            ms_b = time_calls([bwd], steps, warmup)
+            ms_fb = time_calls([fwd, bwd], steps, warmup)
+            row["bwd_us"] = round(ms_b * 1e3, 2)
+            row["bwd_GBps"] = round(bb / ms_b / 1e6, 1)
+            row["fwd_bwd_us"] = round(ms_fb * 1e3, 2)
+            row["fwd_bwd_GBps"] = round((fb + bb) / ms_fb / 1e6, 1)
+            row["pct_of_hbm_peak"] = round((fb + bb) / ms_fb / 1e6 / HBM_PEAK_GBS * 100, 1)
+        else:
+            row["pct_of_hbm_peak"] = round(fb / ms_f / 1e6 / HBM_PEAK_GBS * 100, 1)
+        log("  ", json.dumps(row))
+        out.append(row)
+        del keep, fwd, bwd
+        torch.cuda.empty_cache()
+    return out
+
+
+def cpu_baseline(budget_s=12.0):
+    """The C restatement (OpenMP over channels) on the full C2 workload."""
+    import numpy as np
+    from oracle import c_ref as C
+    rng = np.random.default_rng(1)
+    shape = (32, 256, 56, 56)
+    x = rng.standard_normal(shape, dtype=np.float32) * 2 + 1
+    dy = rng.standard_normal(shape, dtype=np.float32)
+    g = rng.uniform(0.5, 1.5, 256).astype(np.float32)
+    b = (rng.standard_normal(256) * 0.1).astype(np.float32)
+    rm, rv = np.zeros(256, np.float32), np.ones(256, np.float32)
+    cores = C.lib().nr_num_threads()
+    S = x.nbytes
+    reps, t_total = 0, 0.0
+    while True:
+        t0 = time.perf_counter()
+        y, m, v = C.bn_forward_batch(x, b, g, rm, rv, 32, 256, 3136, 0.9, 1e-5)
+        C.bn_backward_batch(x, dy, g, m, v, 32, 256, 3136, 1e-5)
+        t_total += time.perf_counter() - t0
+        reps += 1
+        if t_total > budget_s or reps >= 20:
+            break
+    sec = t_total / reps
+    return {"value": round(8 * S / sec / 1e9, 3), "unit": "GB/s", "cores": int(cores),
+            "kind": "port", "ms_per_step": round(sec * 1e3, 2),
+            "sample": f"full workload x[32,256,56,56] fwd+bwd, {reps} repetitions, "
+                      f"oracle/norm_ref.c with OpenMP over channels"}
+
+
+def load_traffic():
+    """HBM bytes per launch of the dominant kernel from the committed
+    rocprofv3 --pmc summaries, or None."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get("bn_bwd_apply_planes_kernel", {}).get("hbm_bytes_per_launch")
+    except (OSError, ValueError):
+        return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-table", action="store_true", help="skip the per-config table")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus must be 1 "
+              "(the path shards by batch, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from _util import load_package
+    K = load_package()
+    L = K.lib()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+
+    fwd, bwd, fb, bb, keep = make_bn(K, (32, 256, 56, 56), 1, torch.float32, True, 1.0, 2.0, seed=1)
+    ms = time_calls([fwd, bwd], args.steps, args.warmup)
+    value = (fb + bb) / ms / 1e6  # GB/s
+    log(f"C2 fwd+bwd: {ms * 1e3:.1f} us/step, {value:.0f} GB/s algorithmic")
+
+    # Second region: the same K steps with per-kernel HIP events.
+    kernels = ["bn_stats_planes_kernel", "bn_finalize_fwd_kernel", "bn_apply_planes_kernel",
+               "bn_bwd_reduce_planes_kernel", "bn_finalize_bwd_kernel", "bn_bwd_apply_planes_kernel"]
+    K.check(L.nblahip_profile_enable(args.steps * len(kernels) + 16))
+    for _ in range(args.steps):
+        fwd()
+        bwd()
+    torch.cuda.synchronize()
+    S = fb // 3
+    kbytes = {"bn_stats_planes_kernel": S, "bn_apply_planes_kernel": 2 * S,
+              "bn_bwd_reduce_planes_kernel": 2 * S, "bn_bwd_apply_planes_kernel": 3 * S}
+    per_kernel = {}
+    for k in kernels:
+        tot, cnt = K.profile_query(k)
+        if cnt:
+            per_kernel[k] = {"avg_us": round(tot / cnt * 1e3, 2), "launches": cnt}
+            if k in kbytes:
+                per_kernel[k]["GBps"] = round(kbytes[k] / (tot / cnt) / 1e6, 1)
+    K.check(L.nblahip_profile_enable(0))
+    log("per-kernel:", json.dumps(per_kernel))
+    dom = "bn_bwd_apply_planes_kernel"
+    achieved = per_kernel[dom]["GBps"]
+    roofline = {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "avg_us": per_kernel[dom]["avg_us"], "algorithmic_bytes": 3 * S,
+                "traffic": load_traffic()}
+
+    result = {
+        "metric": "BN training fwd+bwd achieved algorithmic HBM bandwidth (us/call in ms_per_step), 1 MI355X",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "BatchNormalization training fwd+bwd fp32 NCHW x[32,256,56,56] "
+                               "(BASELINE configs[1]), decay_rate 0.9, eps 1e-5",
+                   "algorithmic_bytes_per_step": fb + bb,
+                   "pct_of_hbm_peak": round(value / HBM_PEAK_GBS * 100, 1)},
+        "roofline": roofline,
+        "per_kernel": per_kernel,
+    }
+    del keep
+    torch.cuda.empty_cache()
+    if not args.no_table:
+        result["configs"] = config_table(K, max(20, args.steps // 2), args.warmup)
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline()
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -237,6 +237,27 @@ NBLAHIP_EXPORT int nblahip_convert(void *dst, int dst_dtype, const void *src,
 NBLAHIP_EXPORT int nblahip_fill(void *dst, int dtype, float value, int64_t n,
                                 void *stream);
 
+/* ------------------------------------------------------------------------
+ * Per-kernel event timing, the counterpart of the reference's
+ * CudaEventTimerCallback (python/src/nnabla_ext/cuda/utils/inspection/
+ * profile.py:23-74), which brackets each function with CUDA events.  Here the
+ * brackets sit around every kernel launch, on the launch stream.
+ *   enable(n > 0): pre-create n event pairs and start recording (launches
+ *                  beyond n are not recorded); enable(0): stop and release.
+ *   reset        : forget the records, keep the pool.
+ *   query        : wait for the recorded launches of `kernel_name` (the
+ *                  __global__ function's name, e.g. "bn_bwd_apply_planes_kernel";
+ *                  the row kernels are "row_fwd_kernel", "row_bwd_kernel_ln",
+ *                  "row_bwd_kernel_in", "row_bwd_kernel_gn") and return their
+ *                  summed duration and count.
+ * Not for use while other threads are launching; timing adds two event
+ * records per launch.
+ * ---------------------------------------------------------------------- */
+NBLAHIP_EXPORT int nblahip_profile_enable(int max_records);
+NBLAHIP_EXPORT int nblahip_profile_reset(void);
+NBLAHIP_EXPORT int nblahip_profile_query(const char *kernel_name,
+                                         double *total_ms, int64_t *launches);
+
 #ifdef __cplusplus
 }
 #endif

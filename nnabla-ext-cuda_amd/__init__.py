@@ -61,6 +61,10 @@ SIGNATURES = {
     "nblahip_memset": (_int, [_c_void_p, _int, _sz, _c_void_p]),
     "nblahip_convert": (_int, [_c_void_p, _int, _c_void_p, _int, _i64, _c_void_p]),
     "nblahip_fill": (_int, [_c_void_p, _int, _f, _i64, _c_void_p]),
+    "nblahip_profile_enable": (_int, [_int]),
+    "nblahip_profile_reset": (_int, []),
+    "nblahip_profile_query": (_int, [ctypes.c_char_p, ctypes.POINTER(ctypes.c_double),
+                                     ctypes.POINTER(_i64)]),
 }
 
 _lib = None
@@ -92,6 +96,15 @@ def lib():
 def check(code):
     if code != 0:
         raise NblaHipError(code, lib().nblahip_error_string(code).decode())
+
+
+def profile_query(kernel_name):
+    """(total_ms, launches) of the recorded launches of one kernel."""
+    total = ctypes.c_double(0.0)
+    count = _i64(0)
+    check(lib().nblahip_profile_query(kernel_name.encode(), ctypes.byref(total),
+                                      ctypes.byref(count)))
+    return total.value, count.value
 
 
 # ---------------------------------------------------------------------------

@@ -94,12 +94,12 @@ int fwd_apply_t(const BnProblem &p, const BnPlan &pl, const BnParamSrc &src, hip
   const uint64_t total = static_cast<uint64_t>(p.size0) * p.C * p.size2;
   const uint32_t total_vec = static_cast<uint32_t>(total / VEC);
   if (pl.channel_last && pl.cl_fast_apply) {
-    hipLaunchKernelGGL((bn_apply_cl_kernel<T, VEC>), dim3(apply_grid(total_vec, kBnUnroll)),
+    NBLAHIP_LAUNCH("bn_apply_cl_kernel", (bn_apply_cl_kernel<T, VEC>), dim3(apply_grid(total_vec, kBnUnroll)),
                        dim3(256), 0, st, x, y, src, pl.ncv, total_vec);
   } else {
     // channel-last without the register fast path: planes of one vector each.
     const uint32_t nvp = pl.channel_last ? 1u : pl.nvp;
-    hipLaunchKernelGGL((bn_apply_planes_kernel<T, VEC>), dim3(apply_grid(total_vec, kBnUnroll)),
+    NBLAHIP_LAUNCH("bn_apply_planes_kernel", (bn_apply_planes_kernel<T, VEC>), dim3(apply_grid(total_vec, kBnUnroll)),
                        dim3(256), 0, st, x, y, src, FastDiv(nvp),
                        FastDiv(static_cast<uint32_t>(p.C)), total_vec);
   }
@@ -110,11 +110,11 @@ template <typename T, int VEC>
 int stats_t(const BnProblem &p, const BnPlan &pl, float *part, hipStream_t st) {
   const T *x = static_cast<const T *>(p.x);
   if (pl.channel_last) {
-    hipLaunchKernelGGL((bn_stats_cl_kernel<T, VEC>), dim3(pl.ytiles, pl.S), dim3(kBnBlock), 0, st,
+    NBLAHIP_LAUNCH("bn_stats_cl_kernel", (bn_stats_cl_kernel<T, VEC>), dim3(pl.ytiles, pl.S), dim3(kBnBlock), 0, st,
                        x, static_cast<uint32_t>(p.size0), static_cast<uint32_t>(p.C), pl.ncv,
                        pl.log2tx, pl.rps, part);
   } else {
-    hipLaunchKernelGGL((bn_stats_planes_kernel<T, VEC>), dim3(static_cast<uint32_t>(p.C), pl.S),
+    NBLAHIP_LAUNCH("bn_stats_planes_kernel", (bn_stats_planes_kernel<T, VEC>), dim3(static_cast<uint32_t>(p.C), pl.S),
                        dim3(kBnBlock), 0, st, x, static_cast<uint32_t>(p.C), FastDiv(pl.nvp),
                        pl.vpc, pl.chunk, part);
   }
@@ -126,11 +126,11 @@ int bwd_reduce_t(const BnProblem &p, const BnPlan &pl, float *part2, hipStream_t
   const T *x = static_cast<const T *>(p.x);
   const T *dy = static_cast<const T *>(p.dy);
   if (pl.channel_last) {
-    hipLaunchKernelGGL((bn_bwd_reduce_cl_kernel<T, VEC>), dim3(pl.ytiles, pl.S), dim3(kBnBlock), 0,
+    NBLAHIP_LAUNCH("bn_bwd_reduce_cl_kernel", (bn_bwd_reduce_cl_kernel<T, VEC>), dim3(pl.ytiles, pl.S), dim3(kBnBlock), 0,
                        st, x, dy, p.mean, static_cast<uint32_t>(p.size0),
                        static_cast<uint32_t>(p.C), pl.ncv, pl.log2tx, pl.rps, part2);
   } else {
-    hipLaunchKernelGGL((bn_bwd_reduce_planes_kernel<T, VEC>),
+    NBLAHIP_LAUNCH("bn_bwd_reduce_planes_kernel", (bn_bwd_reduce_planes_kernel<T, VEC>),
                        dim3(static_cast<uint32_t>(p.C), pl.S), dim3(kBnBlock), 0, st, x, dy, p.mean,
                        static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, part2);
   }
@@ -145,11 +145,11 @@ int bwd_apply_t(const BnProblem &p, const BnPlan &pl, const BnParam *params, hip
   const uint64_t total = static_cast<uint64_t>(p.size0) * p.C * p.size2;
   const uint32_t total_vec = static_cast<uint32_t>(total / VEC);
   if (pl.channel_last && pl.cl_fast_apply) {
-    hipLaunchKernelGGL((bn_bwd_apply_cl_kernel<T, VEC>), dim3(apply_grid(total_vec, 2)), dim3(256),
+    NBLAHIP_LAUNCH("bn_bwd_apply_cl_kernel", (bn_bwd_apply_cl_kernel<T, VEC>), dim3(apply_grid(total_vec, 2)), dim3(256),
                        0, st, x, dy, dx, params, pl.ncv, total_vec, p.accum_dx);
   } else {
     const uint32_t nvp = pl.channel_last ? 1u : pl.nvp;
-    hipLaunchKernelGGL((bn_bwd_apply_planes_kernel<T, VEC>), dim3(apply_grid(total_vec, 2)),
+    NBLAHIP_LAUNCH("bn_bwd_apply_planes_kernel", (bn_bwd_apply_planes_kernel<T, VEC>), dim3(apply_grid(total_vec, 2)),
                        dim3(256), 0, st, x, dy, dx, params, FastDiv(nvp),
                        FastDiv(static_cast<uint32_t>(p.C)), total_vec, p.accum_dx);
   }
@@ -222,7 +222,7 @@ int launch_bn_fwd_train(const BnProblem &p, hipStream_t st) {
   const double N = static_cast<double>(p.size0) * static_cast<double>(p.size2);
   const float inv_N = static_cast<float>(1.0 / N);
   const float unbias = static_cast<float>(N / (N - 1.0)); // inf when N == 1, as the reference
-  hipLaunchKernelGGL(bn_finalize_fwd_kernel, dim3(static_cast<uint32_t>(p.C)), dim3(kBnBlock), 0,
+  NBLAHIP_LAUNCH("bn_finalize_fwd_kernel", bn_finalize_fwd_kernel, dim3(static_cast<uint32_t>(p.C)), dim3(kBnBlock), 0,
                      st, part, pl.S, inv_N, unbias, p.decay, p.eps, p.gamma, p.beta, p.batch_mean,
                      p.batch_var, p.rmean, p.rvar, params);
   if (int e = last_launch_status()) return e;
@@ -242,7 +242,7 @@ int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
   }
   const double N = static_cast<double>(p.size0) * static_cast<double>(p.size2);
   // Without the reduction (inference-mode dx only) S = 0 leaves the sums at zero.
-  hipLaunchKernelGGL(bn_finalize_bwd_kernel, dim3(static_cast<uint32_t>(p.C)), dim3(kBnBlock), 0,
+  NBLAHIP_LAUNCH("bn_finalize_bwd_kernel", bn_finalize_bwd_kernel, dim3(static_cast<uint32_t>(p.C)), dim3(kBnBlock), 0,
                      st, part2, need_sums ? pl.S : 0u, static_cast<float>(1.0 / N), p.eps,
                      p.batch_stat, p.gamma, p.mean, p.var, p.dmean, p.dvar,
                      need_sums ? p.dgamma : nullptr, need_sums ? p.dbeta : nullptr, p.accum_g,

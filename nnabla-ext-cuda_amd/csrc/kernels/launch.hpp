@@ -97,6 +97,21 @@ int launch_bn_fwd_train(const BnProblem &p, hipStream_t st);
 int launch_bn_bwd(const BnProblem &p, hipStream_t st);
 size_t bn_workspace_bytes(int64_t size0, int64_t C, int64_t size2, int dtype);
 
+// Optional per-kernel timing (HIP events recorded on the launch stream around
+// every kernel).  Off by default; see nblahip_profile_* in the C-ABI.
+struct ProfScope {
+  int slot;
+  hipStream_t st;
+  ProfScope(const char *tag, hipStream_t s);
+  ~ProfScope();
+};
+
+#define NBLAHIP_LAUNCH(tag, kern, grid, block, shmem, st, ...)       \
+  do {                                                               \
+    ::nblahip::ProfScope prof_scope_(tag, st);                       \
+    hipLaunchKernelGGL(kern, grid, block, shmem, st, __VA_ARGS__);   \
+  } while (0)
+
 inline int last_launch_status() {
   const hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : static_cast<int>(e);

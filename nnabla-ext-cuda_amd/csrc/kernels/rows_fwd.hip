@@ -5,7 +5,7 @@ namespace nblahip {
 
 #define FWD_CASE(T, VEC, NL, TPR)                                                      \
   if (cfg.vec == (VEC) && cfg.nl == (NL) && cfg.tpr == (TPR)) {                        \
-    hipLaunchKernelGGL((row_fwd_kernel<T, VEC, NL, TPR>), dim3(grid),                  \
+    NBLAHIP_LAUNCH("row_fwd_kernel", (row_fwd_kernel<T, VEC, NL, TPR>), dim3(grid),                  \
                        dim3(RowBlock<TPR>::kBlock), 0, st, args);                      \
     return last_launch_status();                                                       \
   }

@@ -111,12 +111,12 @@ static bool row_vec_ok(const RowProblem &p, bool backward) {
 
 template <typename T, int VEC>
 static int stream_fwd_t(const RowProblem &p, const RowArgs &a, hipStream_t st) {
-  hipLaunchKernelGGL((row_stats_stream_kernel<T, VEC>), dim3(stream_grid(p.rows)),
+  NBLAHIP_LAUNCH("row_stats_stream_kernel", (row_stats_stream_kernel<T, VEC>), dim3(stream_grid(p.rows)),
                      dim3(kStreamBlock), 0, st, static_cast<const T *>(p.x), a.rows, a.R,
                      a.inv_R, p.mean, p.var);
   if (int e = last_launch_status()) return e;
   const uint32_t total_vec = static_cast<uint32_t>(p.rows * p.R / VEC);
-  hipLaunchKernelGGL((row_apply_fwd_kernel<T, VEC>), dim3(stream_grid((total_vec + 255) / 256)),
+  NBLAHIP_LAUNCH("row_apply_fwd_kernel", (row_apply_fwd_kernel<T, VEC>), dim3(stream_grid((total_vec + 255) / 256)),
                      dim3(256), 0, st, a, FastDiv(static_cast<uint32_t>(p.R / VEC)), total_vec);
   return last_launch_status();
 }
@@ -156,15 +156,15 @@ static int stream_bwd_t(const RowProblem &p, const RowArgs &a, hipStream_t st) {
   if (p.mode == kRowLN) {
     float *rs = static_cast<float *>(p.ws);
     if (p.out) {
-      hipLaunchKernelGGL((ln_row_sums_stream_kernel<T, VEC>), dim3(stream_grid(p.rows)),
+      NBLAHIP_LAUNCH("ln_row_sums_stream_kernel", (ln_row_sums_stream_kernel<T, VEC>), dim3(stream_grid(p.rows)),
                          dim3(kStreamBlock), 0, st, x, dy, p.gamma, p.mean, a.rows, a.R, rs);
       if (int e = last_launch_status()) return e;
-      hipLaunchKernelGGL((row_bwd_dx_kernel<T, VEC>), dim3(stream_grid((total_vec + 255) / 256)),
+      NBLAHIP_LAUNCH("row_bwd_dx_kernel", (row_bwd_dx_kernel<T, VEC>), dim3(stream_grid((total_vec + 255) / 256)),
                          dim3(256), 0, st, a, rs, nvr, total_vec);
       if (int e = last_launch_status()) return e;
     }
     if (p.dgamma || p.dbeta) {
-      hipLaunchKernelGGL((ln_colgrad_stream_kernel<T>), dim3((a.R + 31) / 32), dim3(256), 0, st,
+      NBLAHIP_LAUNCH("ln_colgrad_stream_kernel", (ln_colgrad_stream_kernel<T>), dim3((a.R + 31) / 32), dim3(256), 0, st,
                          x, dy, p.mean, p.var, a.rows, a.R, p.eps, p.dgamma, p.dbeta, p.accum_g,
                          p.accum_b);
       if (int e = last_launch_status()) return e;
@@ -176,16 +176,16 @@ static int stream_bwd_t(const RowProblem &p, const RowArgs &a, hipStream_t st) {
   float *pairs = static_cast<float *>(p.ws);
   float *rs = reinterpret_cast<float *>(static_cast<char *>(p.ws) +
                                         align_up(static_cast<size_t>(planes) * 2 * sizeof(float), 256));
-  hipLaunchKernelGGL((plane_sums_stream_kernel<T, VEC>), dim3(stream_grid(planes)),
+  NBLAHIP_LAUNCH("plane_sums_stream_kernel", (plane_sums_stream_kernel<T, VEC>), dim3(stream_grid(planes)),
                      dim3(kStreamBlock), 0, st, x, dy, p.mean, static_cast<int>(planes),
                      static_cast<int>(p.spatial), static_cast<uint32_t>(ppr), pairs);
   if (int e = last_launch_status()) return e;
   const uint32_t gmod = (p.mode == kRowGN || p.bc_gamma) ? static_cast<uint32_t>(p.channels) : 0u;
-  hipLaunchKernelGGL(plane_to_row_factors_kernel, dim3(stream_grid(p.rows)), dim3(64), 0, st,
+  NBLAHIP_LAUNCH("plane_to_row_factors_kernel", plane_to_row_factors_kernel, dim3(stream_grid(p.rows)), dim3(64), 0, st,
                      pairs, p.gamma, p.var, a.rows, ppr, gmod, p.eps, rs);
   if (int e = last_launch_status()) return e;
   if (p.out) {
-    hipLaunchKernelGGL((row_bwd_dx_kernel<T, VEC>), dim3(stream_grid((total_vec + 255) / 256)),
+    NBLAHIP_LAUNCH("row_bwd_dx_kernel", (row_bwd_dx_kernel<T, VEC>), dim3(stream_grid((total_vec + 255) / 256)),
                        dim3(256), 0, st, a, rs, nvr, total_vec);
     if (int e = last_launch_status()) return e;
   }
@@ -197,7 +197,7 @@ static int launch_pair_reduce(const RowProblem &p, const float *pairs, hipStream
   const int bcg = p.mode == kRowGN ? 1 : p.bc_gamma;
   const int bcb = p.mode == kRowGN ? 1 : p.bc_beta;
   const int64_t count = (bcg && bcb) ? p.channels : p.batch * p.channels;
-  hipLaunchKernelGGL(pair_param_reduce_kernel, dim3(static_cast<unsigned>((count + 255) / 256)),
+  NBLAHIP_LAUNCH("pair_param_reduce_kernel", pair_param_reduce_kernel, dim3(static_cast<unsigned>((count + 255) / 256)),
                      dim3(256), 0, st, pairs, static_cast<int>(p.batch),
                      static_cast<int>(p.channels), p.dgamma, p.dbeta, bcg, bcb, p.accum_g,
                      p.accum_b);
@@ -228,7 +228,7 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
       const int grid = ln_bwd_grid(p.rows, cfg.tpr);
       if (int e = run_row_bwd_cached_ln(p.dtype, cfg, a, grid, st)) return e;
       if (p.dgamma || p.dbeta) {
-        hipLaunchKernelGGL(ln_param_reduce_kernel, dim3((2 * a.R + 31) / 32), dim3(256), 0, st,
+        NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 31) / 32), dim3(256), 0, st,
                            static_cast<const float *>(p.ws), grid, a.R, p.dgamma, p.dbeta,
                            p.accum_g, p.accum_b);
         if (int e = last_launch_status()) return e;

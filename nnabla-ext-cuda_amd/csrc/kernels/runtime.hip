@@ -5,6 +5,7 @@
 #include <mutex>
 #include <string>
 #include <unordered_map>
+#include <vector>
 
 #include "common.cuh"
 #include "launch.hpp"
@@ -41,6 +42,49 @@ int tune_int(const char *name, int fallback) {
   }
   cache.emplace(name, v);
   return v;
+}
+
+// ---------------------------------------------------------------------------
+// Per-kernel event timing.
+// ---------------------------------------------------------------------------
+namespace {
+struct ProfRecord {
+  const char *tag;
+  hipEvent_t start, stop;
+};
+struct ProfState {
+  std::mutex mu;
+  bool enabled = false;
+  std::vector<ProfRecord> records; // pool, events pre-created
+  size_t used = 0;
+  size_t dropped = 0;
+} g_prof;
+} // namespace
+
+ProfScope::ProfScope(const char *tag, hipStream_t s) : slot(-1), st(s) {
+  if (!g_prof.enabled) return;
+  std::lock_guard<std::mutex> lock(g_prof.mu);
+  if (g_prof.used >= g_prof.records.size()) {
+    ++g_prof.dropped;
+    return;
+  }
+  slot = static_cast<int>(g_prof.used++);
+  g_prof.records[slot].tag = tag;
+  (void)hipEventRecord(g_prof.records[slot].start, st);
+}
+
+ProfScope::~ProfScope() {
+  if (slot >= 0) (void)hipEventRecord(g_prof.records[slot].stop, st);
+}
+
+static void prof_release_locked() {
+  for (auto &r : g_prof.records) {
+    (void)hipEventDestroy(r.start);
+    (void)hipEventDestroy(r.stop);
+  }
+  g_prof.records.clear();
+  g_prof.used = 0;
+  g_prof.dropped = 0;
 }
 
 template <typename D, typename S>
@@ -82,6 +126,53 @@ const char *nblahip_error_string(int code) {
   }
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
   return "nblahip: unknown status";
+}
+
+int nblahip_profile_enable(int max_records) {
+  std::lock_guard<std::mutex> lock(g_prof.mu);
+  g_prof.enabled = false;
+  prof_release_locked();
+  if (max_records <= 0) return 0;
+  g_prof.records.reserve(static_cast<size_t>(max_records));
+  for (int i = 0; i < max_records; ++i) {
+    ProfRecord r{nullptr, nullptr, nullptr};
+    hipError_t e = hipEventCreate(&r.start);
+    if (e == hipSuccess) e = hipEventCreate(&r.stop);
+    if (e != hipSuccess) {
+      if (r.start) (void)hipEventDestroy(r.start);
+      prof_release_locked();
+      return static_cast<int>(e);
+    }
+    g_prof.records.push_back(r);
+  }
+  g_prof.enabled = true;
+  return 0;
+}
+
+int nblahip_profile_reset(void) {
+  std::lock_guard<std::mutex> lock(g_prof.mu);
+  g_prof.used = 0;
+  g_prof.dropped = 0;
+  return 0;
+}
+
+int nblahip_profile_query(const char *kernel_name, double *total_ms, int64_t *launches) {
+  if (!kernel_name || !total_ms || !launches) return NBLAHIP_EINVAL;
+  std::lock_guard<std::mutex> lock(g_prof.mu);
+  *total_ms = 0.0;
+  *launches = 0;
+  for (size_t i = 0; i < g_prof.used; ++i) {
+    const ProfRecord &r = g_prof.records[i];
+    if (std::strcmp(r.tag, kernel_name) != 0) continue;
+    hipError_t e = hipEventSynchronize(r.stop);
+    if (e != hipSuccess) return static_cast<int>(e);
+    float ms = 0.f;
+    e = hipEventElapsedTime(&ms, r.start, r.stop);
+    if (e != hipSuccess) return static_cast<int>(e);
+    *total_ms += ms;
+    *launches += 1;
+  }
+  return 0;
 }
 
 int nblahip_device_count(int *count) {
@@ -154,10 +245,10 @@ int nblahip_convert(void *dst, int dst_dtype, const void *src, int src_dtype, in
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 g(flat_grid(n)), b(256);
   if (dst_dtype == NBLAHIP_F32 && src_dtype == NBLAHIP_F16) {
-    hipLaunchKernelGGL((convert_kernel<float, __half>), g, b, 0, st, static_cast<float *>(dst),
+    NBLAHIP_LAUNCH("convert_kernel", (convert_kernel<float, __half>), g, b, 0, st, static_cast<float *>(dst),
                        static_cast<const __half *>(src), n);
   } else if (dst_dtype == NBLAHIP_F16 && src_dtype == NBLAHIP_F32) {
-    hipLaunchKernelGGL((convert_kernel<__half, float>), g, b, 0, st, static_cast<__half *>(dst),
+    NBLAHIP_LAUNCH("convert_kernel", (convert_kernel<__half, float>), g, b, 0, st, static_cast<__half *>(dst),
                        static_cast<const float *>(src), n);
   } else if (dst_dtype == src_dtype && (dst_dtype == NBLAHIP_F32 || dst_dtype == NBLAHIP_F16)) {
     const size_t bytes = static_cast<size_t>(n) * (dst_dtype == NBLAHIP_F32 ? 4 : 2);
@@ -174,9 +265,9 @@ int nblahip_fill(void *dst, int dtype, float value, int64_t n, void *stream) {
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 g(flat_grid(n)), b(256);
   if (dtype == NBLAHIP_F32) {
-    hipLaunchKernelGGL((fill_kernel<float>), g, b, 0, st, static_cast<float *>(dst), value, n);
+    NBLAHIP_LAUNCH("fill_kernel", (fill_kernel<float>), g, b, 0, st, static_cast<float *>(dst), value, n);
   } else if (dtype == NBLAHIP_F16) {
-    hipLaunchKernelGGL((fill_kernel<__half>), g, b, 0, st, static_cast<__half *>(dst), value, n);
+    NBLAHIP_LAUNCH("fill_kernel", (fill_kernel<__half>), g, b, 0, st, static_cast<__half *>(dst), value, n);
   } else {
     return NBLAHIP_EINVAL;
   }

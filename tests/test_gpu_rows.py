@@ -227,7 +227,10 @@ def test_in_forward_backward(n, c, sp, dtype):
     assert_close(to_np(v), v_r, dn, "stat", "var")
     assert_close(to_np(y), y_r, dn, "y", "y")
     dx, dg, db = K.in_backward(xd, dyd, gd, m, v, 1e-5)
-    assert_close(to_np(dx), dx_r, dn, "grad", "dx")
+    # One element per plane: var == 0 and dx is the exact cancellation of two
+    # terms of size |dy*gamma|/sqrt(eps); the floor follows that size.
+    scale = 1.0 / np.sqrt(1e-5) if int(np.prod(sp)) == 1 else None
+    assert_close(to_np(dx), dx_r, dn, "grad", "dx", scale=scale)
     assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
     assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
 

@@ -11,7 +11,6 @@ import torch.nn.functional as F
 
 from oracle import norm_ref as R
 
-torch.set_default_dtype(torch.float64)
 RTOL = 1e-10
 ATOL = 1e-10
 
@@ -21,7 +20,7 @@ def close(a, b, rtol=RTOL, atol=ATOL):
 
 
 def T(a, grad=False):
-    t = torch.tensor(np.asarray(a, dtype=np.float64))
+    t = torch.tensor(np.asarray(a, dtype=np.float64), dtype=torch.float64)
     return t.requires_grad_(grad)
 
 
