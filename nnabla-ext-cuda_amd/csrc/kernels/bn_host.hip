@@ -84,7 +84,9 @@ BnParamSrc param_src(const BnParam *params) {
 
 int apply_grid(uint32_t total_vec, int unroll) {
   const uint64_t blocks = (static_cast<uint64_t>(total_vec) + 256ull * unroll - 1) / (256ull * unroll);
-  return static_cast<int>(std::max<uint64_t>(1, std::min<uint64_t>(blocks, 1u << 20)));
+  const int per_cu = tune_int("BN_APPLY_BLOCKS_PER_CU", 0);
+  const uint64_t cap = per_cu > 0 ? static_cast<uint64_t>(device_cus()) * per_cu : (1u << 20);
+  return static_cast<int>(std::max<uint64_t>(1, std::min<uint64_t>(blocks, cap)));
 }
 
 template <typename T, int VEC>

@@ -54,10 +54,22 @@ template <int TPR> struct RowBlock {
   static constexpr int kRowsPerBlock = kBlock / TPR;
 };
 
+// Backward blocks.  The LayerNormalization backward is persistent and keeps
+// per-column accumulators, so its wave-per-row layout packs 8 rows into a
+// 512-thread block (256 VGPRs per lane stay available): two blocks per CU,
+// few partials to fold afterwards.
+template <int TPR, int MODE> struct RowBwdBlock {
+  static constexpr int kBlock = (MODE == kRowLN && TPR == kWave) ? 512 : RowBlock<TPR>::kBlock;
+  static constexpr int kRowsPerBlock = kBlock / TPR;
+};
+
 // ---------------------------------------------------------------------------
-// Forward: y, mean, var.
+// Forward: y, mean, var.  PERCOL selects the LayerNormalization parameter
+// layout (gamma/beta per column: loaded once per thread, before the row loop,
+// and kept in registers); otherwise one scalar gamma/beta per 16-byte load,
+// fetched while the row is still in flight.
 // ---------------------------------------------------------------------------
-template <typename T, int VEC, int NL, int TPR>
+template <typename T, int VEC, int NL, int TPR, bool PERCOL>
 __global__ void __launch_bounds__(RowBlock<TPR>::kBlock)
 row_fwd_kernel(const RowArgs a) {
   constexpr int RPB = RowBlock<TPR>::kRowsPerBlock;
@@ -67,6 +79,27 @@ row_fwd_kernel(const RowArgs a) {
   const T *__restrict__ x = static_cast<const T *>(a.x);
   T *__restrict__ y = static_cast<T *>(a.out);
 
+  float gcol[PERCOL ? NL : 1][VEC], bcol[PERCOL ? NL : 1][VEC];
+  if constexpr (PERCOL) {
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const int col = (k * TPR + t) * VEC;
+      const bool ok = col < a.R;
+      if (ok && a.gamma) {
+        load_param_vec<VEC>(a.gamma + col, gcol[k]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) gcol[k][j] = 1.f;
+      }
+      if (ok && a.beta) {
+        load_param_vec<VEC>(a.beta + col, bcol[k]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) bcol[k][j] = 0.f;
+      }
+    }
+  }
+
   for (int row = blockIdx.x * RPB + sub; row < a.rows; row += gridDim.x * RPB) {
     const size_t base = static_cast<size_t>(row) * a.R;
     RawVec<T, VEC> raw[NL];
@@ -74,6 +107,18 @@ row_fwd_kernel(const RowArgs a) {
     for (int k = 0; k < NL; ++k) {
       const int col = (k * TPR + t) * VEC;
       raw[k] = (col < a.R) ? load_raw<T, VEC>(x + base + col) : zero_raw<T, VEC>();
+    }
+    float gk[PERCOL ? 1 : NL], bk[PERCOL ? 1 : NL];
+    if constexpr (!PERCOL) {
+      const uint32_t pbase = (static_cast<uint32_t>(row) % a.pmod) * a.pmul;
+      const uint32_t bbase = (static_cast<uint32_t>(row) % a.pmod_b) * a.pmul;
+#pragma unroll
+      for (int k = 0; k < NL; ++k) {
+        const int col = (k * TPR + t) * VEC;
+        const uint32_t poff = (col < a.R) ? a.pdiv.div(static_cast<uint32_t>(col)) : 0u;
+        gk[k] = a.gamma ? a.gamma[pbase + poff] : 1.f;
+        bk[k] = a.beta ? a.beta[bbase + poff] : 0.f;
+      }
     }
     float s = 0.f;
 #pragma unroll
@@ -110,36 +155,19 @@ row_fwd_kernel(const RowArgs a) {
 #pragma unroll
     for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
 
-    const uint32_t pbase = a.percol ? 0u : (static_cast<uint32_t>(row) % a.pmod) * a.pmul;
-    const uint32_t bbase = a.percol ? 0u : (static_cast<uint32_t>(row) % a.pmod_b) * a.pmul;
 #pragma unroll
     for (int k = 0; k < NL; ++k) {
       const int col = (k * TPR + t) * VEC;
       if (col < a.R) {
         float v[VEC], o[VEC];
         unpack<T, VEC>(raw[k], v);
-        if (a.percol) {
-          float g[VEC], b[VEC];
-          if (a.gamma) {
-            load_param_vec<VEC>(a.gamma + col, g);
-          } else {
+        if constexpr (PERCOL) {
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) g[j] = 1.f;
-          }
-          if (a.beta) {
-            load_param_vec<VEC>(a.beta + col, b);
-          } else {
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) b[j] = 0.f;
-          }
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) o[j] = (v[j] - mean) * (g[j] * istd) + b[j];
+          for (int j = 0; j < VEC; ++j) o[j] = (v[j] - mean) * (gcol[k][j] * istd) + bcol[k][j];
         } else {
-          const uint32_t poff = a.pdiv.div(static_cast<uint32_t>(col));
-          const float g = (a.gamma ? a.gamma[pbase + poff] : 1.f) * istd;
-          const float b = a.beta ? a.beta[bbase + poff] : 0.f;
+          const float g = gk[k] * istd;
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) o[j] = (v[j] - mean) * g + b;
+          for (int j = 0; j < VEC; ++j) o[j] = (v[j] - mean) * g + bk[k];
         }
         store_vec<T, VEC>(y + base + col, o);
       }
@@ -163,9 +191,9 @@ row_fwd_kernel(const RowArgs a) {
 // Padded lanes hold x = dy = 0 in registers, so they add nothing to any sum.
 // ---------------------------------------------------------------------------
 template <typename T, int VEC, int NL, int TPR, int MODE>
-__global__ void __launch_bounds__(RowBlock<TPR>::kBlock)
+__global__ void __launch_bounds__((RowBwdBlock<TPR, MODE>::kBlock))
 row_bwd_kernel(const RowArgs a) {
-  constexpr int RPB = RowBlock<TPR>::kRowsPerBlock;
+  constexpr int RPB = RowBwdBlock<TPR, MODE>::kRowsPerBlock;
   constexpr int NW = TPR / kWave;
   __shared__ float lds[2 * 16];
   __shared__ float part[(MODE == kRowGN) ? 2 * NW * NL : 1];
@@ -178,11 +206,20 @@ row_bwd_kernel(const RowArgs a) {
 
   float acc_g[(MODE == kRowLN) ? NL : 1][VEC];
   float acc_b[(MODE == kRowLN) ? NL : 1][VEC];
+  float gcol[(MODE == kRowLN) ? NL : 1][VEC]; // per-column gamma, loaded once
   if constexpr (MODE == kRowLN) {
 #pragma unroll
-    for (int k = 0; k < NL; ++k)
+    for (int k = 0; k < NL; ++k) {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) acc_g[k][j] = acc_b[k][j] = 0.f;
+      const int col = (k * TPR + t) * VEC;
+      if (col < a.R && a.gamma) {
+        load_param_vec<VEC>(a.gamma + col, gcol[k]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) gcol[k][j] = 1.f;
+      }
+    }
   }
 
   for (int row = blockIdx.x * RPB + sub; row < a.rows; row += gridDim.x * RPB) {
@@ -205,21 +242,15 @@ row_bwd_kernel(const RowArgs a) {
       for (int k = 0; k < NL; ++k) {
         const int col = (k * TPR + t) * VEC;
         if (col < a.R) {
-          float xv[VEC], dv[VEC], g[VEC];
+          float xv[VEC], dv[VEC];
           unpack<T, VEC>(xr[k], xv);
           unpack<T, VEC>(dr[k], dv);
-          if (a.gamma) {
-            load_param_vec<VEC>(a.gamma + col, g);
-          } else {
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) g[j] = 1.f;
-          }
 #pragma unroll
           for (int j = 0; j < VEC; ++j) {
             const float xc = xv[j] - mean;
             acc_g[k][j] += dv[j] * xc * istd;
             acc_b[k][j] += dv[j];
-            const float dg = dv[j] * g[j];
+            const float dg = dv[j] * gcol[k][j];
             s1 += dg;
             t2 += dg * xc;
           }
@@ -317,16 +348,9 @@ row_bwd_kernel(const RowArgs a) {
           unpack<T, VEC>(xr[k], xv);
           unpack<T, VEC>(dr[k], dv);
           if constexpr (MODE == kRowLN) {
-            float g[VEC];
-            if (a.gamma) {
-              load_param_vec<VEC>(a.gamma + col, g);
-            } else {
-#pragma unroll
-              for (int j = 0; j < VEC; ++j) g[j] = 1.f;
-            }
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
-              o[j] = dv[j] * (g[j] * istd) + ca * (xv[j] - mean) + cb;
+              o[j] = dv[j] * (gcol[k][j] * istd) + ca * (xv[j] - mean) + cb;
           } else {
             const float gi = gk[k] * istd;
 #pragma unroll

@@ -7,7 +7,7 @@ namespace nblahip {
 #define BWD_CASE(T, VEC, NL, TPR)                                                      \
   if (cfg.vec == (VEC) && cfg.nl == (NL) && cfg.tpr == (TPR)) {                        \
     NBLAHIP_LAUNCH("row_bwd_kernel_in", (row_bwd_kernel<T, VEC, NL, TPR, kRowIN>), dim3(grid),           \
-                       dim3(RowBlock<TPR>::kBlock), 0, st, args);                      \
+                       dim3(RowBwdBlock<TPR, kRowIN>::kBlock), 0, st, args);                      \
     return last_launch_status();                                                       \
   }
 

@@ -5,8 +5,13 @@ namespace nblahip {
 
 #define FWD_CASE(T, VEC, NL, TPR)                                                      \
   if (cfg.vec == (VEC) && cfg.nl == (NL) && cfg.tpr == (TPR)) {                        \
-    NBLAHIP_LAUNCH("row_fwd_kernel", (row_fwd_kernel<T, VEC, NL, TPR>), dim3(grid),                  \
-                       dim3(RowBlock<TPR>::kBlock), 0, st, args);                      \
+    if (args.percol) {                                                                 \
+      NBLAHIP_LAUNCH("row_fwd_kernel", (row_fwd_kernel<T, VEC, NL, TPR, true>), dim3(grid), \
+                     dim3(RowBlock<TPR>::kBlock), 0, st, args);                        \
+    } else {                                                                           \
+      NBLAHIP_LAUNCH("row_fwd_kernel", (row_fwd_kernel<T, VEC, NL, TPR, false>), dim3(grid), \
+                     dim3(RowBlock<TPR>::kBlock), 0, st, args);                        \
+    }                                                                                  \
     return last_launch_status();                                                       \
   }
 

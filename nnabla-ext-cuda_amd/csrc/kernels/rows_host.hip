@@ -44,9 +44,12 @@ static int cached_grid(int64_t rows, int tpr) {
 // Persistent grid of the LayerNormalization backward: each block keeps
 // per-column accumulators, so fewer blocks mean fewer partials to fold.
 static int ln_bwd_grid(int64_t rows, int tpr) {
-  const int per_cu = tune_int("LN_BWD_BLOCKS_PER_CU", 2);
+  // Wave-per-row rows run 8 to a 512-thread block; longer rows own a block.
+  const int rpb = tpr == 64 ? 8 : 1;
+  const int per_cu = tune_int("LN_BWD_BLOCKS_PER_CU", tpr == 1024 ? 1 : 2);
   const int64_t cap = static_cast<int64_t>(device_cus()) * per_cu;
-  return static_cast<int>(std::min<int64_t>(cached_grid(rows, tpr), cap));
+  const int64_t blocks = (rows + rpb - 1) / rpb;
+  return static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(blocks, cap)));
 }
 
 static int stream_grid(int64_t work_blocks) {
@@ -138,8 +141,8 @@ size_t row_bwd_workspace_bytes(int mode, int64_t rows, int64_t R, int64_t planes
   if (mode == kRowLN) {
     // Largest persistent grid over the possible thread layouts (one row per
     // block is the 256/1024-thread case).
-    const size_t cached =
-        static_cast<size_t>(ln_bwd_grid(rows, 1024)) * 2 * static_cast<size_t>(R) * sizeof(float);
+    const int g = std::max(ln_bwd_grid(rows, 64), std::max(ln_bwd_grid(rows, 256), ln_bwd_grid(rows, 1024)));
+    const size_t cached = static_cast<size_t>(g) * 2 * static_cast<size_t>(R) * sizeof(float);
     const size_t stream = static_cast<size_t>(rows) * 2 * sizeof(float);
     return align_up(std::max(cached, stream), 256);
   }
@@ -228,7 +231,7 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
       const int grid = ln_bwd_grid(p.rows, cfg.tpr);
       if (int e = run_row_bwd_cached_ln(p.dtype, cfg, a, grid, st)) return e;
       if (p.dgamma || p.dbeta) {
-        NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 31) / 32), dim3(256), 0, st,
+        NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 31) / 32), dim3(1024), 0, st,
                            static_cast<const float *>(p.ws), grid, a.R, p.dgamma, p.dbeta,
                            p.accum_g, p.accum_b);
         if (int e = last_launch_status()) return e;

@@ -262,26 +262,38 @@ ln_colgrad_stream_kernel(const T *__restrict__ x, const T *__restrict__ dy,
 // ---------------------------------------------------------------------------
 // Second stage of the LayerNormalization parameter gradients: column sums of
 // the per-block partials ws[nparts][2][R] -> dgamma[R], dbeta[R].
-// Block = 32 columns x 8 part-groups; coalesced 128-byte reads.
+// Block = 32 columns x 32 part groups; every thread issues its (up to 8 per
+// batch) independent 128-byte-coalesced loads before adding, so the whole
+// fold costs a few load latencies.
 // ---------------------------------------------------------------------------
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 ln_param_reduce_kernel(const float *__restrict__ ws, int nparts, int R,
                        float *__restrict__ dgamma, float *__restrict__ dbeta,
                        int accum_g, int accum_b) {
-  __shared__ float red[8][33];
+  __shared__ float red[32][33];
   const int cx = threadIdx.x & 31;
   const int py = threadIdx.x >> 5;
   const int col2 = blockIdx.x * 32 + cx; // column in the [2R] concatenation
+  const size_t stride = 2 * static_cast<size_t>(R);
   float s = 0.f;
   if (col2 < 2 * R) {
-    for (int p = py; p < nparts; p += 8) s += ws[static_cast<size_t>(p) * 2 * R + col2];
+    for (int p0 = py; p0 < nparts; p0 += 32 * 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int p = p0 + 32 * u;
+        v[u] = (p < nparts) ? ws[static_cast<size_t>(p) * stride + col2] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) s += v[u];
+    }
   }
   red[py][cx] = s;
   __syncthreads();
   if (py == 0 && col2 < 2 * R) {
     float tot = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) tot += red[i][cx];
+    for (int i = 0; i < 32; ++i) tot += red[i][cx];
     if (col2 < R) {
       if (dgamma) dgamma[col2] = tot + (accum_g ? dgamma[col2] : 0.f);
     } else {
