@@ -246,7 +246,7 @@ def load_traffic():
     path = os.path.join(ROOT, "profiles", "traffic.json")
     try:
         with open(path) as f:
-            return json.load(f).get("bn_bwd_apply_planes_kernel", {}).get("hbm_bytes_per_launch")
+            return json.load(f).get("bn_bwd_apply_planes_fused_kernel", {}).get("hbm_bytes_per_launch")
     except (OSError, ValueError):
         return None
 
@@ -278,7 +278,9 @@ def main():
 
     # Second region: the same K steps with per-kernel HIP events.
     kernels = ["bn_stats_planes_kernel", "bn_finalize_fwd_kernel", "bn_apply_planes_kernel",
-               "bn_bwd_reduce_planes_kernel", "bn_finalize_bwd_kernel", "bn_bwd_apply_planes_kernel"]
+               "bn_apply_planes_fused_kernel", "bn_bwd_reduce_planes_kernel",
+               "bn_finalize_bwd_kernel", "bn_bwd_apply_planes_kernel",
+               "bn_bwd_apply_planes_fused_kernel"]
     K.check(L.nblahip_profile_enable(args.steps * len(kernels) + 16))
     for _ in range(args.steps):
         fwd()
@@ -286,7 +288,8 @@ def main():
     torch.cuda.synchronize()
     S = fb // 3
     kbytes = {"bn_stats_planes_kernel": S, "bn_apply_planes_kernel": 2 * S,
-              "bn_bwd_reduce_planes_kernel": 2 * S, "bn_bwd_apply_planes_kernel": 3 * S}
+              "bn_apply_planes_fused_kernel": 2 * S, "bn_bwd_reduce_planes_kernel": 2 * S,
+              "bn_bwd_apply_planes_kernel": 3 * S, "bn_bwd_apply_planes_fused_kernel": 3 * S}
     per_kernel = {}
     for k in kernels:
         tot, cnt = K.profile_query(k)
@@ -296,7 +299,9 @@ def main():
                 per_kernel[k]["GBps"] = round(kbytes[k] / (tot / cnt) / 1e6, 1)
     K.check(L.nblahip_profile_enable(0))
     log("per-kernel:", json.dumps(per_kernel))
-    dom = "bn_bwd_apply_planes_kernel"
+    # dominant kernel = the backward apply (3 tensor passes), fused or not
+    dom = max((k for k in per_kernel if k.startswith("bn_bwd_apply")),
+              key=lambda k: per_kernel[k]["launches"])
     achieved = per_kernel[dom]["GBps"]
     roofline = {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),

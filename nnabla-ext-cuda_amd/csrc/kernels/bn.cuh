@@ -19,7 +19,7 @@
 namespace nblahip {
 
 constexpr int kBnBlock = 256;
-constexpr int kBnUnroll = 4;
+constexpr int kBnUnroll = 4; // 16-byte loads in flight per thread and input
 
 // Per-channel parameters of the forward apply step: y = (x - mean)*scale + shift.
 // Per-channel parameters of the backward apply step:
@@ -87,6 +87,7 @@ bn_stats_cl_kernel(const T *__restrict__ x, uint32_t M, uint32_t C, uint32_t ncv
   __shared__ float lmean[kBnBlock * VEC];
   __shared__ float lm2[kBnBlock * VEC];
   __shared__ float ln[kBnBlock];
+  __shared__ float l2[3 * kBnBlock]; // second merge level: [q][o] triples
   const uint32_t TX = 1u << log2tx;
   const uint32_t TY = kBnBlock >> log2tx;
   const uint32_t tx = threadIdx.x & (TX - 1);
@@ -120,15 +121,16 @@ bn_stats_cl_kernel(const T *__restrict__ x, uint32_t M, uint32_t C, uint32_t ncv
       }
       // cnt >= 1 here.  Chunk statistics per channel, then one Chan merge.
       const float fc = static_cast<float>(cnt);
+      const float inv_fc = fast_rcp(fc);
       const float nn = n + fc;
-      const float wb = fc / nn;          // weight of the chunk mean
-      const float wd = n * wb;           // n_a*n_b/(n_a+n_b)
+      const float wb = fc * fast_rcp(nn); // weight of the chunk mean
+      const float wd = n * wb;            // n_a*n_b/(n_a+n_b)
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
         float sum = 0.f;
 #pragma unroll
         for (int u = 0; u < kBnUnroll; ++u) sum += vals[u][j];
-        const float cm = sum / fc;
+        const float cm = sum * inv_fc;
         float cm2 = 0.f;
 #pragma unroll
         for (int u = 0; u < kBnUnroll; ++u) {
@@ -149,20 +151,52 @@ bn_stats_cl_kernel(const T *__restrict__ x, uint32_t M, uint32_t C, uint32_t ncv
   }
   ln[ty * TX + tx] = n;
   __syncthreads();
-  // Output o = tx*VEC + j of this block; fold the TY row groups in order.
-  for (uint32_t o = threadIdx.x; o < TX * VEC; o += kBnBlock) {
+  // Output o = tx*VEC + j of this block needs its TY row groups folded.  With
+  // nout = TX*VEC outputs and 256 threads, Q = 256/nout threads share an
+  // output: each folds TY/Q row groups in order, then the Q results are
+  // folded in order by the first of them (fixed order: reproducible).
+  const uint32_t nout = TX * VEC;
+  if (nout <= kBnBlock) {
+    const uint32_t Q = kBnBlock / nout;
+    const uint32_t per = (TY + Q - 1) / Q;
+    const uint32_t o = threadIdx.x % nout;
+    const uint32_t q = threadIdx.x / nout;
     const uint32_t otx = o / VEC;
-    const uint32_t ch = blockIdx.x * TX * VEC + o;
-    if (blockIdx.x * TX + otx < ncv) {
-      Welford w{0.f, 0.f, 0.f};
-      for (uint32_t y = 0; y < TY; ++y) {
-        const Welford b{lmean[y * TX * VEC + o], lm2[y * TX * VEC + o], ln[y * TX + otx]};
-        w = welford_merge(w, b);
+    Welford w{0.f, 0.f, 0.f};
+    for (uint32_t y = q * per; y < min((q + 1) * per, TY); ++y) {
+      const Welford b{lmean[y * nout + o], lm2[y * nout + o], ln[y * TX + otx]};
+      w = welford_merge(w, b);
+    }
+    l2[3 * threadIdx.x] = w.mean;
+    l2[3 * threadIdx.x + 1] = w.m2;
+    l2[3 * threadIdx.x + 2] = w.n;
+    __syncthreads();
+    if (q == 0 && blockIdx.x * TX + otx < ncv) {
+      for (uint32_t k = 1; k < Q; ++k) {
+        const uint32_t t = k * nout + o;
+        w = welford_merge(w, Welford{l2[3 * t], l2[3 * t + 1], l2[3 * t + 2]});
       }
+      const uint32_t ch = blockIdx.x * nout + o;
       float *p = part + 3 * (static_cast<size_t>(ch) * S + s);
       p[0] = w.mean;
       p[1] = w.m2;
       p[2] = w.n;
+    }
+  } else {
+    for (uint32_t o = threadIdx.x; o < nout; o += kBnBlock) {
+      const uint32_t otx = o / VEC;
+      if (blockIdx.x * TX + otx < ncv) {
+        Welford w{0.f, 0.f, 0.f};
+        for (uint32_t y = 0; y < TY; ++y) {
+          const Welford b{lmean[y * nout + o], lm2[y * nout + o], ln[y * TX + otx]};
+          w = welford_merge(w, b);
+        }
+        const uint32_t ch = blockIdx.x * nout + o;
+        float *p = part + 3 * (static_cast<size_t>(ch) * S + s);
+        p[0] = w.mean;
+        p[1] = w.m2;
+        p[2] = w.n;
+      }
     }
   }
 }
@@ -263,8 +297,16 @@ bn_apply_planes_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc sr
         const uint32_t c = plane - cdiv.div(plane) * cdiv.d;
         const BnParam q = src.get(c);
         float o[VEC];
+        if constexpr (sizeof(T) == 2) {
+          // Half output: one mixed-precision fma per element; the folded shift
+          // loses nothing a 10-bit mantissa can hold.
+          const float shift = fmaf(-q.mean, q.a, q.b);
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) o[j] = (v[u][j] - q.mean) * q.a + q.b;
+          for (int j = 0; j < VEC; ++j) o[j] = fmaf(v[u][j], q.a, shift);
+        } else {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) o[j] = (v[u][j] - q.mean) * q.a + q.b;
+        }
         store_vec<T, VEC>(y + static_cast<size_t>(i) * VEC, o);
       }
     }

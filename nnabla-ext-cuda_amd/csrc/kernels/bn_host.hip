@@ -29,13 +29,19 @@ uint32_t ceil_div_u(uint64_t a, uint64_t b) { return static_cast<uint32_t>((a + 
 
 // Upper bound of S over every plan this shape can get (vector width depends on
 // pointer alignment, unknown when the workspace is sized).
-uint32_t split_target() { return static_cast<uint32_t>(device_cus()) * tune_int("BN_BLOCKS_PER_CU", 16); }
+// Blocks a split reduction aims for.  The planes kernels end with one cheap
+// block merge and like many blocks; the channel-last kernels end with an LDS
+// fold over 256/TX row groups and like fewer, longer blocks.
+uint32_t split_target(bool channel_last) {
+  return static_cast<uint32_t>(device_cus()) *
+         (channel_last ? tune_int("BN_CL_BLOCKS_PER_CU", 4) : tune_int("BN_BLOCKS_PER_CU", 16));
+}
 
 BnPlan make_plan(int64_t size0, int64_t C, int64_t size2, int dtype, bool ptr_aligned) {
   BnPlan pl;
   const int full = dtype == NBLAHIP_F16 ? 8 : 4;
-  const uint32_t target = split_target();
   pl.channel_last = size2 == 1;
+  const uint32_t target = split_target(pl.channel_last);
   if (!pl.channel_last) {
     pl.vec = (ptr_aligned && size2 % full == 0) ? full : 1;
     pl.nvp = static_cast<uint32_t>(size2 / pl.vec);
@@ -82,9 +88,11 @@ BnParamSrc param_src(const BnParam *params) {
   return s;
 }
 
-int apply_grid(uint32_t total_vec, int unroll) {
+// Channel-last apply kernels load their per-channel parameters into registers
+// once per thread, so they run as a persistent grid (cl = true).
+int apply_grid(uint32_t total_vec, int unroll, bool cl = false) {
   const uint64_t blocks = (static_cast<uint64_t>(total_vec) + 256ull * unroll - 1) / (256ull * unroll);
-  const int per_cu = tune_int("BN_APPLY_BLOCKS_PER_CU", 0);
+  const int per_cu = cl ? tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 4) : tune_int("BN_APPLY_BLOCKS_PER_CU", 0);
   const uint64_t cap = per_cu > 0 ? static_cast<uint64_t>(device_cus()) * per_cu : (1u << 20);
   return static_cast<int>(std::max<uint64_t>(1, std::min<uint64_t>(blocks, cap)));
 }
@@ -96,7 +104,7 @@ int fwd_apply_t(const BnProblem &p, const BnPlan &pl, const BnParamSrc &src, hip
   const uint64_t total = static_cast<uint64_t>(p.size0) * p.C * p.size2;
   const uint32_t total_vec = static_cast<uint32_t>(total / VEC);
   if (pl.channel_last && pl.cl_fast_apply) {
-    NBLAHIP_LAUNCH("bn_apply_cl_kernel", (bn_apply_cl_kernel<T, VEC>), dim3(apply_grid(total_vec, kBnUnroll)),
+    NBLAHIP_LAUNCH("bn_apply_cl_kernel", (bn_apply_cl_kernel<T, VEC>), dim3(apply_grid(total_vec, kBnUnroll, true)),
                        dim3(256), 0, st, x, y, src, pl.ncv, total_vec);
   } else {
     // channel-last without the register fast path: planes of one vector each.
@@ -147,7 +155,7 @@ int bwd_apply_t(const BnProblem &p, const BnPlan &pl, const BnParam *params, hip
   const uint64_t total = static_cast<uint64_t>(p.size0) * p.C * p.size2;
   const uint32_t total_vec = static_cast<uint32_t>(total / VEC);
   if (pl.channel_last && pl.cl_fast_apply) {
-    NBLAHIP_LAUNCH("bn_bwd_apply_cl_kernel", (bn_bwd_apply_cl_kernel<T, VEC>), dim3(apply_grid(total_vec, 2)), dim3(256),
+    NBLAHIP_LAUNCH("bn_bwd_apply_cl_kernel", (bn_bwd_apply_cl_kernel<T, VEC>), dim3(apply_grid(total_vec, 2, true)), dim3(256),
                        0, st, x, dy, dx, params, pl.ncv, total_vec, p.accum_dx);
   } else {
     const uint32_t nvp = pl.channel_last ? 1u : pl.nvp;

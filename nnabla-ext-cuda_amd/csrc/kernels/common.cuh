@@ -128,6 +128,79 @@ template <typename T, int VEC> __device__ __forceinline__ void keep_packed(RawVe
   }
 }
 
+// ---------------------------------------------------------------------------
+// Element access on packed vectors with the widening folded into the
+// arithmetic.  For half data, fma(float(h), a, b) with a half operand taken
+// straight from the packed register compiles to ONE v_fma_mix_f32, provided
+// the multiplier is not a literal 1.0 (the optimiser would turn the fma into
+// an add and need a separate conversion): callers that only want float(h)+b
+// pass a 1.0f that arrives as a kernel argument.  raw_sum adds two halves per
+// v_dot2_f32_f16.
+// ---------------------------------------------------------------------------
+typedef _Float16 half2_native __attribute__((ext_vector_type(2)));
+
+// float(x[j]) * a + b for element j of the vector (j is a compile-time
+// constant after unrolling).
+template <typename T, int VEC>
+__device__ __forceinline__ float elem_fma(const RawVec<T, VEC> &r, int j, float a, float b) {
+  if constexpr (VEC == 1) {
+    return fmaf(to_f32<T>(r.v), a, b);
+  } else if constexpr (sizeof(T) == 4) {
+    const float x = j == 0 ? r.v.x : j == 1 ? r.v.y : j == 2 ? r.v.z : r.v.w;
+    return fmaf(x, a, b);
+  } else {
+    const uint32_t w = j < 2 ? r.v.x : j < 4 ? r.v.y : j < 6 ? r.v.z : r.v.w;
+    const half2_native h = __builtin_bit_cast(half2_native, w);
+    return fmaf(static_cast<float>((j & 1) ? h.y : h.x), a, b);
+  }
+}
+
+// (x[j] - mean) * istd.  Half data takes the folded one-instruction form
+// x*istd + (-mean*istd): its extra error, eps32*|mean|*istd, is far below half
+// resolution.  Float data keeps the centred two-instruction form, exact for
+// x == mean and insensitive to |mean| >> std.
+template <typename T, int VEC>
+__device__ __forceinline__ float norm_elem(const RawVec<T, VEC> &r, int j, float mean,
+                                           float istd, float nmi) {
+  if constexpr (sizeof(T) == 2) {
+    return elem_fma<T, VEC>(r, j, istd, nmi);
+  } else {
+    return (elem_fma<T, VEC>(r, j, 1.0f, 0.f) - mean) * istd;
+  }
+}
+
+// r when ok, zeros otherwise (branch-free: the load itself is unconditional).
+template <typename T, int VEC>
+__device__ __forceinline__ RawVec<T, VEC> raw_or_zero(bool ok, RawVec<T, VEC> r) {
+  if constexpr (VEC == 1) {
+    r.v = ok ? r.v : from_f32<T>(0.f);
+  } else if constexpr (sizeof(T) == 4) {
+    r.v.x = ok ? r.v.x : 0.f; r.v.y = ok ? r.v.y : 0.f;
+    r.v.z = ok ? r.v.z : 0.f; r.v.w = ok ? r.v.w : 0.f;
+  } else {
+    r.v.x = ok ? r.v.x : 0u; r.v.y = ok ? r.v.y : 0u;
+    r.v.z = ok ? r.v.z : 0u; r.v.w = ok ? r.v.w : 0u;
+  }
+  return r;
+}
+
+// acc + sum of the VEC elements (fp32 accumulation).
+template <typename T, int VEC>
+__device__ __forceinline__ float raw_sum(const RawVec<T, VEC> &r, float acc) {
+  if constexpr (VEC == 1) {
+    return acc + to_f32<T>(r.v);
+  } else if constexpr (sizeof(T) == 4) {
+    return acc + ((r.v.x + r.v.y) + (r.v.z + r.v.w));
+  } else {
+    const half2_native ones = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
+    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_native, r.v.x), ones, acc, false);
+    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_native, r.v.y), ones, acc, false);
+    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_native, r.v.z), ones, acc, false);
+    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_native, r.v.w), ones, acc, false);
+    return acc;
+  }
+}
+
 // VEC consecutive float parameters (gamma/beta style), p aligned to 16 bytes
 // when VEC > 1.
 template <int VEC>
@@ -250,10 +323,14 @@ struct Welford {
   float mean, m2, n;
 };
 
+// 1/x to within one ulp (v_rcp_f32); the merge weights do not need the
+// correctly rounded quotient and the full division costs ten instructions.
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
 __device__ __forceinline__ Welford welford_merge(const Welford &a, const Welford &b) {
   const float n = a.n + b.n;
   if (n == 0.f) return Welford{0.f, 0.f, 0.f};
-  const float inv = 1.0f / n;
+  const float inv = fast_rcp(n);
   const float d = b.mean - a.mean;
   Welford r;
   r.mean = a.mean + d * (b.n * inv);
@@ -273,7 +350,7 @@ __device__ __forceinline__ void welford_add_chunk(Welford &acc, const float (&v)
 #pragma unroll
   for (int i = 0; i < CNT; ++i) s += (i < cnt) ? v[i] : 0.f;
   const float fc = static_cast<float>(cnt);
-  const float cm = s / fc;
+  const float cm = s * fast_rcp(fc);
   float m2 = 0.f;
 #pragma unroll
   for (int i = 0; i < CNT; ++i) {

@@ -43,6 +43,9 @@ struct RowArgs {
   uint32_t pmul;
   FastDiv pdiv;
   int accum_dx;
+  // 1.0f delivered at run time: keeps fma(float(half), one, b) a single
+  // mixed-precision instruction (see elem_fma).
+  float one;
   // GroupNormalization backward: entries (64*VEC-element runs) per channel and
   // channels per group.
   int epc;
@@ -105,8 +108,11 @@ row_fwd_kernel(const RowArgs a) {
     RawVec<T, VEC> raw[NL];
 #pragma unroll
     for (int k = 0; k < NL; ++k) {
+      // Out-of-row lanes load column 0 (always valid) and are zeroed after:
+      // no branch, so the NL loads are in flight together.
       const int col = (k * TPR + t) * VEC;
-      raw[k] = (col < a.R) ? load_raw<T, VEC>(x + base + col) : zero_raw<T, VEC>();
+      const bool ok = col < a.R;
+      raw[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + base + (ok ? col : 0)));
     }
     float gk[PERCOL ? 1 : NL], bk[PERCOL ? 1 : NL];
     if constexpr (!PERCOL) {
@@ -122,12 +128,7 @@ row_fwd_kernel(const RowArgs a) {
     }
     float s = 0.f;
 #pragma unroll
-    for (int k = 0; k < NL; ++k) {
-      float v[VEC];
-      unpack<T, VEC>(raw[k], v);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) s += v[j];
-    }
+    for (int k = 0; k < NL; ++k) s = raw_sum<T, VEC>(raw[k], s);
     const float mean = row_sum<TPR>(s, lds) * a.inv_R;
 #pragma unroll
     for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
@@ -137,12 +138,10 @@ row_fwd_kernel(const RowArgs a) {
     for (int k = 0; k < NL; ++k) {
       const int col = (k * TPR + t) * VEC;
       if (col < a.R) {
-        float v[VEC];
-        unpack<T, VEC>(raw[k], v);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
-          const float d = v[j] - mean;
-          q += d * d;
+          const float d = elem_fma<T, VEC>(raw[k], j, a.one, -mean);
+          q = fmaf(d, d, q);
         }
       }
     }
@@ -159,15 +158,23 @@ row_fwd_kernel(const RowArgs a) {
     for (int k = 0; k < NL; ++k) {
       const int col = (k * TPR + t) * VEC;
       if (col < a.R) {
-        float v[VEC], o[VEC];
-        unpack<T, VEC>(raw[k], v);
+        float o[VEC];
         if constexpr (PERCOL) {
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) o[j] = (v[j] - mean) * (gcol[k][j] * istd) + bcol[k][j];
+          for (int j = 0; j < VEC; ++j)
+            o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mean), gcol[k][j] * istd, bcol[k][j]);
+        } else if constexpr (sizeof(T) == 2) {
+          // Half output: x*g + (b - mean*g) in one mixed fma per element; the
+          // folded shift loses nothing a 10-bit mantissa can hold.
+          const float g = gk[k] * istd;
+          const float sh = fmaf(-mean, g, bk[k]);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) o[j] = elem_fma<T, VEC>(raw[k], j, g, sh);
         } else {
           const float g = gk[k] * istd;
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) o[j] = (v[j] - mean) * g + bk[k];
+          for (int j = 0; j < VEC; ++j)
+            o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mean), g, bk[k]);
         }
         store_vec<T, VEC>(y + base + col, o);
       }
@@ -176,25 +183,30 @@ row_fwd_kernel(const RowArgs a) {
 }
 
 // ---------------------------------------------------------------------------
-// Backward: dx plus partial parameter gradients.
-//   s1 = sum(dy*g), t2 = sum(dy*g*(x-mean))
-//   ca = -t2*istd^3/R + 2*dvar/R      cb = -s1*istd/R + dmean/R
-//   dx = dy*g*istd + ca*(x-mean) + cb
+// Backward: dx plus partial parameter gradients.  With xh = (x-mean)*istd
+// (one fma per element: x*istd - mean*istd) and dg = dy*gamma:
+//   s1 = sum(dg), t2 = sum(dg*xh)
+//   cA = -istd*t2/R + 2*dvar*std/R        cb = -s1*istd/R + dmean/R
+//   dx = dg*istd + cA*xh + cb
 // which is the reference's a*x+b form (kernel/layer_normalization.cuh:50-95)
-// with a*mean folded into the centred term.
+// rewritten on the normalised variable (std = (var+eps)*istd).
 //
 // Partial parameter gradients written to ws:
-//   LN : ws[block][0][R] = sum_rows dy*(x-mean)*istd, ws[block][1][R] = sum_rows dy
-//   IN : ws[2*row] = sum dy*(x-mean)*istd, ws[2*row+1] = sum dy     (row = (n,c))
+//   LN : ws[block][0][R] = sum_rows dy*xh, ws[block][1][R] = sum_rows dy
+//   IN : ws[2*row] = sum dy*xh, ws[2*row+1] = sum dy             (row = (n,c))
 //   GN : same pair per (n, channel); requires spatial % (64*VEC) == 0 so that
 //        every wave-wide load belongs to one channel.
-// Padded lanes hold x = dy = 0 in registers, so they add nothing to any sum.
+// Padded lanes hold x = dy = 0 in registers; dy == 0 keeps them out of every
+// sum.
 // ---------------------------------------------------------------------------
 template <typename T, int VEC, int NL, int TPR, int MODE>
 __global__ void __launch_bounds__((RowBwdBlock<TPR, MODE>::kBlock))
 row_bwd_kernel(const RowArgs a) {
   constexpr int RPB = RowBwdBlock<TPR, MODE>::kRowsPerBlock;
   constexpr int NW = TPR / kWave;
+  // LayerNormalization keeps xh and dg of a row in registers between the
+  // reduction and the dx step when they are few; otherwise they are recomputed.
+  constexpr bool KEEP = (MODE == kRowLN) && (NL * VEC <= 16);
   __shared__ float lds[2 * 16];
   __shared__ float part[(MODE == kRowGN) ? 2 * NW * NL : 1];
   __shared__ float xwave[(MODE == kRowLN && RPB > 1) ? (RPB - 1) * kWave * VEC : 1];
@@ -229,30 +241,32 @@ row_bwd_kernel(const RowArgs a) {
     for (int k = 0; k < NL; ++k) {
       const int col = (k * TPR + t) * VEC;
       const bool ok = col < a.R;
-      xr[k] = ok ? load_raw<T, VEC>(x + base + col) : zero_raw<T, VEC>();
-      dr[k] = ok ? load_raw<T, VEC>(dy + base + col) : zero_raw<T, VEC>();
+      const int colc = ok ? col : 0; // branch-free: all loads in flight together
+      xr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + base + colc));
+      dr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(dy + base + colc));
     }
     const float mean = a.mean[row];
-    const float istd = inv_std(a.var[row], a.eps);
+    const float vpe = a.var[row] + a.eps;
+    const float istd = 1.0f / sqrtf(vpe);
+    const float nmi = -mean * istd;
 
     float s1 = 0.f, t2 = 0.f;
-    float gk[NL]; // per-load scalar gamma (IN / GN)
+    float gk[NL];                                   // per-load scalar gamma (IN / GN)
+    float xh_keep[KEEP ? NL : 1][VEC], dg_keep[KEEP ? NL : 1][VEC];
     if constexpr (MODE == kRowLN) {
 #pragma unroll
       for (int k = 0; k < NL; ++k) {
-        const int col = (k * TPR + t) * VEC;
-        if (col < a.R) {
-          float xv[VEC], dv[VEC];
-          unpack<T, VEC>(xr[k], xv);
-          unpack<T, VEC>(dr[k], dv);
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) {
-            const float xc = xv[j] - mean;
-            acc_g[k][j] += dv[j] * xc * istd;
-            acc_b[k][j] += dv[j];
-            const float dg = dv[j] * gcol[k][j];
-            s1 += dg;
-            t2 += dg * xc;
+        for (int j = 0; j < VEC; ++j) {
+          const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+          const float dg = elem_fma<T, VEC>(dr[k], j, gcol[k][j], 0.f);
+          acc_g[k][j] = elem_fma<T, VEC>(dr[k], j, xh, acc_g[k][j]);
+          acc_b[k][j] = elem_fma<T, VEC>(dr[k], j, a.one, acc_b[k][j]);
+          s1 += dg;
+          t2 = fmaf(dg, xh, t2);
+          if constexpr (KEEP) {
+            xh_keep[k][j] = xh;
+            dg_keep[k][j] = dg;
           }
         }
       }
@@ -261,18 +275,16 @@ row_bwd_kernel(const RowArgs a) {
       float sdy = 0.f, sdx = 0.f;
 #pragma unroll
       for (int k = 0; k < NL; ++k) {
-        float xv[VEC], dv[VEC];
-        unpack<T, VEC>(xr[k], xv);
-        unpack<T, VEC>(dr[k], dv);
+        sdy = raw_sum<T, VEC>(dr[k], sdy);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
-          sdy += dv[j];
-          sdx += dv[j] * (xv[j] - mean);
+          const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+          sdx = elem_fma<T, VEC>(dr[k], j, xh, sdx);
         }
       }
       row_sum2<TPR>(sdy, sdx, lds);
       if (t == 0) {
-        a.ws[2 * static_cast<size_t>(row)] = sdx * istd;
+        a.ws[2 * static_cast<size_t>(row)] = sdx;
         a.ws[2 * static_cast<size_t>(row) + 1] = sdy;
       }
       const uint32_t pidx = (static_cast<uint32_t>(row) % a.pmod) * a.pmul;
@@ -289,14 +301,12 @@ row_bwd_kernel(const RowArgs a) {
       __syncthreads(); // part[] of the previous row has been consumed
 #pragma unroll
       for (int k = 0; k < NL; ++k) {
-        float xv[VEC], dv[VEC];
-        unpack<T, VEC>(xr[k], xv);
-        unpack<T, VEC>(dr[k], dv);
-        float sdy = 0.f, sdx = 0.f;
+        float sdy = raw_sum<T, VEC>(dr[k], 0.f);
+        float sdx = 0.f;
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
-          sdy += dv[j];
-          sdx += dv[j] * (xv[j] - mean);
+          const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+          sdx = elem_fma<T, VEC>(dr[k], j, xh, sdx);
         }
         sdy = wave_sum(sdy);
         sdx = wave_sum(sdx);
@@ -319,7 +329,7 @@ row_bwd_kernel(const RowArgs a) {
           sdy += part[2 * e + 1];
         }
         const size_t o = 2 * (static_cast<size_t>(row) * a.cpg + c);
-        a.ws[o] = sdx * istd;
+        a.ws[o] = sdx;
         a.ws[o + 1] = sdy;
         const float g = a.gamma ? a.gamma[pbase + c] : 1.f;
         c1 += g * sdy;
@@ -335,8 +345,8 @@ row_bwd_kernel(const RowArgs a) {
       keep_packed<T, VEC>(xr[k]);
       keep_packed<T, VEC>(dr[k]);
     }
-    const float ca = -t2 * istd * istd * istd * a.inv_R +
-                     (a.dvar ? 2.f * a.dvar[row] * a.inv_R : 0.f);
+    const float cA = -istd * t2 * a.inv_R +
+                     (a.dvar ? 2.f * a.dvar[row] * (vpe * istd) * a.inv_R : 0.f);
     const float cb = -s1 * istd * a.inv_R + (a.dmean ? a.dmean[row] * a.inv_R : 0.f);
 
     if (dx != nullptr) {
@@ -344,17 +354,24 @@ row_bwd_kernel(const RowArgs a) {
       for (int k = 0; k < NL; ++k) {
         const int col = (k * TPR + t) * VEC;
         if (col < a.R) {
-          float xv[VEC], dv[VEC], o[VEC];
-          unpack<T, VEC>(xr[k], xv);
-          unpack<T, VEC>(dr[k], dv);
-          if constexpr (MODE == kRowLN) {
+          float o[VEC];
+          if constexpr (KEEP) {
 #pragma unroll
             for (int j = 0; j < VEC; ++j)
-              o[j] = dv[j] * (gcol[k][j] * istd) + ca * (xv[j] - mean) + cb;
+              o[j] = fmaf(dg_keep[k][j], istd, fmaf(xh_keep[k][j], cA, cb));
+          } else if constexpr (MODE == kRowLN) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+              const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+              o[j] = elem_fma<T, VEC>(dr[k], j, gcol[k][j] * istd, fmaf(xh, cA, cb));
+            }
           } else {
             const float gi = gk[k] * istd;
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) o[j] = dv[j] * gi + ca * (xv[j] - mean) + cb;
+            for (int j = 0; j < VEC; ++j) {
+              const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+              o[j] = elem_fma<T, VEC>(dr[k], j, gi, fmaf(xh, cA, cb));
+            }
           }
           if (a.accum_dx) {
             float old[VEC];

@@ -74,6 +74,7 @@ static RowArgs make_args(const RowProblem &p) {
   a.eps = p.eps;
   a.inv_R = 1.0f / static_cast<float>(p.R);
   a.accum_dx = p.accum_dx;
+  a.one = 1.0f;
   a.epc = 0;
   a.cpg = 1;
   if (p.mode == kRowLN) {

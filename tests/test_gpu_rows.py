@@ -47,7 +47,10 @@ def test_ln_forward_backward(outer, Rr, dtype):
     assert_close(to_np(v), v_r, dn, "stat", "var")
     assert_close(to_np(y), y_r, dn, "y", "y")
     dx, dg, db = K.ln_backward(xd, dyd, gd, m, v, outer, 1e-5)
-    assert_close(to_np(dx), dx_r, dn, "grad", "dx")
+    # One element per row: var == 0 and dx is the exact cancellation of two
+    # terms of size |dy*gamma|/sqrt(eps); the floor follows that size.
+    scale = 1.0 / np.sqrt(1e-5) if Rr == 1 else None
+    assert_close(to_np(dx), dx_r, dn, "grad", "dx", scale=scale)
     assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
     assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
 
