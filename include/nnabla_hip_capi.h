@@ -1,0 +1,86 @@
+/*
+ * nnabla_hip_capi.h - flat C surface over the "hip" backend's C++ layer
+ * (libnnabla_hip.so): initialisation, Variables, and the four normalization
+ * Functions created through the function registry by context, exactly the
+ * calls a language binding makes.  It plays the part of the reference's
+ * Cython layer (python/src/nnabla_ext/cuda/init.pyx:28-71 calls init_cuda()
+ * and registers the context; the core's function bindings then create
+ * functions by name and context).  Errors of the C++ layer (nbla::Exception)
+ * are caught here: functions return 0 on success and non-zero otherwise, and
+ * nnabla_hip_last_error() returns the message of the calling thread's last
+ * failure.
+ */
+#ifndef NNABLA_HIP_CAPI_H_
+#define NNABLA_HIP_CAPI_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NNABLA_HIP_EXPORT __attribute__((visibility("default")))
+
+typedef struct nnabla_hip_variable nnabla_hip_variable;
+typedef struct nnabla_hip_function nnabla_hip_function;
+
+/* nbla::init_hip() (idempotent). */
+NNABLA_HIP_EXPORT int nnabla_hip_init(void);
+NNABLA_HIP_EXPORT const char *nnabla_hip_last_error(void);
+/* Array classes of the backend, comma separated ("HipCachedArray,HipArray"). */
+NNABLA_HIP_EXPORT const char *nnabla_hip_array_classes(void);
+NNABLA_HIP_EXPORT int nnabla_hip_device_synchronize(const char *device_id);
+/* Bytes held by live device arrays / kept in the allocator cache. */
+NNABLA_HIP_EXPORT int nnabla_hip_memory_stats(uint64_t *live_bytes, uint64_t *cached_bytes);
+NNABLA_HIP_EXPORT int nnabla_hip_clear_memory_cache(void);
+
+/* Variables.  which: 0 = data, 1 = grad.  dtype: 0 = float32, 1 = float16
+ * (the host buffer is always float32; float16 storage rounds to nearest). */
+NNABLA_HIP_EXPORT nnabla_hip_variable *nnabla_hip_variable_new(int ndim, const int64_t *shape);
+NNABLA_HIP_EXPORT void nnabla_hip_variable_delete(nnabla_hip_variable *v);
+NNABLA_HIP_EXPORT int nnabla_hip_variable_ndim(nnabla_hip_variable *v);
+NNABLA_HIP_EXPORT int nnabla_hip_variable_shape(nnabla_hip_variable *v, int64_t *shape_out);
+NNABLA_HIP_EXPORT int nnabla_hip_variable_set(nnabla_hip_variable *v, int which, const float *host,
+                                              int64_t n, int dtype);
+NNABLA_HIP_EXPORT int nnabla_hip_variable_get(nnabla_hip_variable *v, int which, float *host,
+                                              int64_t n);
+NNABLA_HIP_EXPORT int nnabla_hip_variable_zero(nnabla_hip_variable *v, int which);
+NNABLA_HIP_EXPORT int nnabla_hip_variable_fill(nnabla_hip_variable *v, int which, float value);
+
+/* Function creation through the registry.  `backends` is the context's backend
+ * preference list, comma separated (e.g. "hip:half,hip:float"). */
+NNABLA_HIP_EXPORT nnabla_hip_function *nnabla_hip_create_batch_normalization(
+    const char *backends, const char *array_class, const char *device_id, const int *axes,
+    int n_axes, float decay_rate, float eps, int batch_stat, int no_scale, int no_bias);
+NNABLA_HIP_EXPORT nnabla_hip_function *nnabla_hip_create_layer_normalization(
+    const char *backends, const char *array_class, const char *device_id, const int *batch_axis,
+    int n_batch_axis, float eps, int no_scale, int no_bias);
+NNABLA_HIP_EXPORT nnabla_hip_function *nnabla_hip_create_group_normalization(
+    const char *backends, const char *array_class, const char *device_id, int num_groups,
+    int channel_axis, const int *batch_axis, int n_batch_axis, float eps, int no_scale,
+    int no_bias);
+NNABLA_HIP_EXPORT nnabla_hip_function *nnabla_hip_create_instance_normalization(
+    const char *backends, const char *array_class, const char *device_id, int channel_axis,
+    const int *batch_axis, int n_batch_axis, float eps, int no_scale, int no_bias);
+NNABLA_HIP_EXPORT void nnabla_hip_function_delete(nnabla_hip_function *f);
+NNABLA_HIP_EXPORT const char *nnabla_hip_function_name(nnabla_hip_function *f);
+
+/* Function::setup / forward / backward / recompute. */
+NNABLA_HIP_EXPORT int nnabla_hip_function_setup(nnabla_hip_function *f,
+                                                nnabla_hip_variable **inputs, int n_inputs,
+                                                nnabla_hip_variable **outputs, int n_outputs);
+NNABLA_HIP_EXPORT int nnabla_hip_function_forward(nnabla_hip_function *f,
+                                                  nnabla_hip_variable **inputs, int n_inputs,
+                                                  nnabla_hip_variable **outputs, int n_outputs);
+NNABLA_HIP_EXPORT int nnabla_hip_function_recompute(nnabla_hip_function *f,
+                                                    nnabla_hip_variable **inputs, int n_inputs,
+                                                    nnabla_hip_variable **outputs, int n_outputs);
+NNABLA_HIP_EXPORT int nnabla_hip_function_backward(nnabla_hip_function *f,
+                                                   nnabla_hip_variable **inputs, int n_inputs,
+                                                   nnabla_hip_variable **outputs, int n_outputs,
+                                                   const int *propagate_down, const int *accum);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NNABLA_HIP_CAPI_H_ */

@@ -1,0 +1,221 @@
+"""ctypes binding of libnnabla_hip.so (include/nnabla_hip_capi.h): the C++
+backend layer - context-selected nbla::Function objects over Variables - as a
+language binding sees it.  Used by the tests that exercise the Function
+classes the way NNabla's own function tests do (create by name and context,
+setup, forward, backward with propagate_down/accum)."""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+HOST_LIB_PATH = os.path.join(_HERE, "lib", "libnnabla_hip.so")
+
+_P = ctypes.c_void_p
+_PP = ctypes.POINTER(ctypes.c_void_p)
+_I = ctypes.c_int
+_I64 = ctypes.c_int64
+_F = ctypes.c_float
+_S = ctypes.c_char_p
+_IP = ctypes.POINTER(ctypes.c_int)
+_FP = ctypes.POINTER(ctypes.c_float)
+
+SIGNATURES = {
+    "nnabla_hip_init": (_I, []),
+    "nnabla_hip_last_error": (_S, []),
+    "nnabla_hip_array_classes": (_S, []),
+    "nnabla_hip_device_synchronize": (_I, [_S]),
+    "nnabla_hip_memory_stats": (_I, [ctypes.POINTER(ctypes.c_uint64)] * 2),
+    "nnabla_hip_clear_memory_cache": (_I, []),
+    "nnabla_hip_variable_new": (_P, [_I, ctypes.POINTER(_I64)]),
+    "nnabla_hip_variable_delete": (None, [_P]),
+    "nnabla_hip_variable_ndim": (_I, [_P]),
+    "nnabla_hip_variable_shape": (_I, [_P, ctypes.POINTER(_I64)]),
+    "nnabla_hip_variable_set": (_I, [_P, _I, _FP, _I64, _I]),
+    "nnabla_hip_variable_get": (_I, [_P, _I, _FP, _I64]),
+    "nnabla_hip_variable_zero": (_I, [_P, _I]),
+    "nnabla_hip_variable_fill": (_I, [_P, _I, _F]),
+    "nnabla_hip_create_batch_normalization": (_P, [_S, _S, _S, _IP, _I, _F, _F, _I, _I, _I]),
+    "nnabla_hip_create_layer_normalization": (_P, [_S, _S, _S, _IP, _I, _F, _I, _I]),
+    "nnabla_hip_create_group_normalization": (_P, [_S, _S, _S, _I, _I, _IP, _I, _F, _I, _I]),
+    "nnabla_hip_create_instance_normalization": (_P, [_S, _S, _S, _I, _IP, _I, _F, _I, _I]),
+    "nnabla_hip_function_delete": (None, [_P]),
+    "nnabla_hip_function_name": (_S, [_P]),
+    "nnabla_hip_function_setup": (_I, [_P, _PP, _I, _PP, _I]),
+    "nnabla_hip_function_forward": (_I, [_P, _PP, _I, _PP, _I]),
+    "nnabla_hip_function_recompute": (_I, [_P, _PP, _I, _PP, _I]),
+    "nnabla_hip_function_backward": (_I, [_P, _PP, _I, _PP, _I, _IP, _IP]),
+}
+
+_lib = None
+
+
+class NblaError(RuntimeError):
+    """An nbla::Exception that crossed the C surface."""
+
+    def __init__(self, code, text):
+        super().__init__(text)
+        self.code = code
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(HOST_LIB_PATH):
+            raise RuntimeError(f"{HOST_LIB_PATH} is missing: build it first (make -C csrc)")
+        h = ctypes.CDLL(HOST_LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(h, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = h
+    return _lib
+
+
+def _check(code):
+    if code != 0:
+        raise NblaError(code, lib().nnabla_hip_last_error().decode())
+
+
+def init():
+    _check(lib().nnabla_hip_init())
+
+
+def context(type_config="float", device_id="0", array_class="HipCachedArray"):
+    """Backend preference list the way the reference's context() builds it
+    (python/src/nnabla_ext/cuda/__init__.py:138-149): half falls back to float."""
+    backends = ["hip:half", "hip:float"] if type_config == "half" else ["hip:float"]
+    return {"backends": ",".join(backends), "array_class": array_class, "device_id": str(device_id)}
+
+
+def _ints(seq):
+    arr = (ctypes.c_int * max(len(seq), 1))(*seq)
+    return arr, len(seq)
+
+
+class Variable:
+    def __init__(self, shape):
+        self.shape = tuple(int(s) for s in shape)
+        arr = (_I64 * max(len(self.shape), 1))(*self.shape)
+        self._h = lib().nnabla_hip_variable_new(len(self.shape), arr)
+        if not self._h:
+            raise NblaError(-1, lib().nnabla_hip_last_error().decode())
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().nnabla_hip_variable_delete(self._h)
+            self._h = None
+
+    @property
+    def current_shape(self):
+        n = lib().nnabla_hip_variable_ndim(self._h)
+        out = (_I64 * max(n, 1))()
+        _check(lib().nnabla_hip_variable_shape(self._h, out))
+        return tuple(out[i] for i in range(n))
+
+    def _set(self, which, a, half):
+        a = np.ascontiguousarray(a, dtype=np.float32).reshape(-1)
+        _check(lib().nnabla_hip_variable_set(self._h, which, a.ctypes.data_as(_FP), a.size,
+                                             1 if half else 0))
+
+    def _get(self, which):
+        shape = self.current_shape
+        out = np.empty(int(np.prod(shape, dtype=np.int64)), np.float32)
+        _check(lib().nnabla_hip_variable_get(self._h, which, out.ctypes.data_as(_FP), out.size))
+        return out.reshape(shape)
+
+    def set_data(self, a, half=False):
+        self._set(0, a, half)
+
+    def set_grad(self, a, half=False):
+        self._set(1, a, half)
+
+    @property
+    def d(self):
+        return self._get(0)
+
+    @property
+    def g(self):
+        return self._get(1)
+
+    def zero_grad(self):
+        _check(lib().nnabla_hip_variable_zero(self._h, 1))
+
+    def fill_grad(self, v):
+        _check(lib().nnabla_hip_variable_fill(self._h, 1, float(v)))
+
+
+def _handles(vs):
+    arr = (ctypes.c_void_p * max(len(vs), 1))(*[v._h for v in vs])
+    return ctypes.cast(arr, _PP), len(vs)
+
+
+class Function:
+    def __init__(self, handle):
+        if not handle:
+            raise NblaError(-1, lib().nnabla_hip_last_error().decode())
+        self._h = handle
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().nnabla_hip_function_delete(self._h)
+            self._h = None
+
+    @property
+    def name(self):
+        return lib().nnabla_hip_function_name(self._h).decode()
+
+    def setup(self, inputs, outputs):
+        i, ni = _handles(inputs)
+        o, no = _handles(outputs)
+        _check(lib().nnabla_hip_function_setup(self._h, i, ni, o, no))
+
+    def forward(self, inputs, outputs):
+        i, ni = _handles(inputs)
+        o, no = _handles(outputs)
+        _check(lib().nnabla_hip_function_forward(self._h, i, ni, o, no))
+
+    def recompute(self, inputs, outputs):
+        i, ni = _handles(inputs)
+        o, no = _handles(outputs)
+        _check(lib().nnabla_hip_function_recompute(self._h, i, ni, o, no))
+
+    def backward(self, inputs, outputs, propagate_down=None, accum=None):
+        i, ni = _handles(inputs)
+        o, no = _handles(outputs)
+        pd = [1] * ni if propagate_down is None else [int(bool(p)) for p in propagate_down]
+        ac = [0] * ni if accum is None else [int(bool(a)) for a in accum]
+        pda, _ = _ints(pd)
+        aca, _ = _ints(ac)
+        _check(lib().nnabla_hip_function_backward(self._h, i, ni, o, no, pda, aca))
+
+
+def _ctx_args(ctx):
+    return ctx["backends"].encode(), ctx["array_class"].encode(), ctx["device_id"].encode()
+
+
+def BatchNormalization(ctx, axes=(1,), decay_rate=0.9, eps=1e-5, batch_stat=True, no_scale=False,
+                       no_bias=False):
+    ax, n = _ints(list(axes))
+    return Function(lib().nnabla_hip_create_batch_normalization(
+        *_ctx_args(ctx), ax, n, decay_rate, eps, int(batch_stat), int(no_scale), int(no_bias)))
+
+
+def LayerNormalization(ctx, batch_axis=(0,), eps=1e-5, no_scale=False, no_bias=False):
+    ba, n = _ints(list(batch_axis))
+    return Function(lib().nnabla_hip_create_layer_normalization(
+        *_ctx_args(ctx), ba, n, eps, int(no_scale), int(no_bias)))
+
+
+def GroupNormalization(ctx, num_groups=1, channel_axis=1, batch_axis=(0,), eps=1e-5, no_scale=False,
+                       no_bias=False):
+    ba, n = _ints(list(batch_axis))
+    return Function(lib().nnabla_hip_create_group_normalization(
+        *_ctx_args(ctx), num_groups, channel_axis, ba, n, eps, int(no_scale), int(no_bias)))
+
+
+def InstanceNormalization(ctx, channel_axis=1, batch_axis=(0,), eps=1e-5, no_scale=False,
+                          no_bias=False):
+    ba, n = _ints(list(batch_axis))
+    return Function(lib().nnabla_hip_create_instance_normalization(
+        *_ctx_args(ctx), channel_axis, ba, n, eps, int(no_scale), int(no_bias)))

@@ -1,0 +1,42 @@
+// BatchNormalizationHip<T>: the "hip" implementation of BatchNormalization,
+// same constructor, name()/allowed_array_classes() and *_impl overrides as
+// BatchNormalizationCuda<T> (include/nbla/cuda/function/batch_normalization.hpp:31-85).
+// Statistics, gamma/beta and their gradients are float32 for every T, as in
+// the reference's cudnn context
+// (src/nbla/cuda/cudnn/function/generic/batch_normalization.cu:94-99,193-227).
+#pragma once
+
+#include <nbla/function/batch_normalization.hpp>
+#include <nbla/hip/common.hpp>
+#include <nbla/hip/hip.hpp>
+
+namespace nbla {
+
+template <typename T> class BatchNormalizationHip : public BatchNormalization<T> {
+protected:
+  int device_;
+  Variable workspace_; // split-reduction partials + per-channel parameters
+  size_t workspace_bytes_ = 0;
+
+public:
+  BatchNormalizationHip(const Context &ctx, const vector<int> axes, float decay_rate, float eps,
+                        bool batch_stat, bool no_scale, bool no_bias)
+      : BatchNormalization<T>(ctx, axes, decay_rate, eps, batch_stat, no_scale, no_bias),
+        device_(std::stoi(ctx.device_id)) {}
+  virtual ~BatchNormalizationHip() {}
+  virtual string name() { return "BatchNormalizationHip"; }
+  virtual vector<string> allowed_array_classes() {
+    return SingletonManager::get<Hip>()->array_classes();
+  }
+
+protected:
+  virtual void setup_impl(const Variables &inputs, const Variables &outputs);
+  virtual void forward_impl(const Variables &inputs, const Variables &outputs);
+  virtual void backward_impl(const Variables &inputs, const Variables &outputs,
+                             const vector<bool> &propagate_down, const vector<bool> &accum);
+  virtual void forward_impl_batch(const Variables &inputs, const Variables &outputs,
+                                  const bool update_inputs);
+  virtual void forward_impl_global(const Variables &inputs, const Variables &outputs);
+  virtual void recompute_impl(const Variables &inputs, const Variables &outputs);
+};
+} // namespace nbla

@@ -1,0 +1,138 @@
+// BatchNormalizationHip<T>: host-side control flow of the reference's
+// BatchNormalizationCuda<T> (src/nbla/cuda/function/generic/batch_normalization.cu)
+// over the nblahip kernel layer.
+#include <nbla/hip/function/batch_normalization.hpp>
+#include <nbla/variable.hpp>
+
+namespace nbla {
+
+template <typename T>
+void BatchNormalizationHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
+  BatchNormalization<T>::setup_impl(inputs, outputs);
+  hip_set_device(this->device_);
+  NBLA_CHECK(inputs[0]->size() < (Size_t(1) << 31), error_code::value,
+             "BatchNormalizationHip indexes with 32 bits: fewer than 2^31 elements required.");
+  workspace_bytes_ = nblahip_bn_workspace_bytes(this->size0_, this->size1_, this->size2_,
+                                                HipDtype<T>::code);
+  workspace_.reshape(Shape_t{static_cast<Size_t>((workspace_bytes_ + 3) / 4)}, true);
+}
+
+template <typename T>
+void BatchNormalizationHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->device_);
+  if (this->batch_stat_) { // Training mode.
+    forward_impl_batch(inputs, outputs, true /* update_inputs */);
+  } else { // Testing mode.
+    forward_impl_global(inputs, outputs);
+  }
+}
+
+template <typename T>
+void BatchNormalizationHip<T>::recompute_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->device_);
+  if (this->batch_stat_) {
+    forward_impl_batch(inputs, outputs, false /* update_inputs */);
+  } else {
+    forward_impl_global(inputs, outputs);
+  }
+}
+
+template <typename T>
+void BatchNormalizationHip<T>::forward_impl_batch(const Variables &inputs, const Variables &outputs,
+                                                  const bool update_inputs) {
+  // Batch statistics go to the outputs when they are exposed, otherwise to
+  // the members backward reads them from.
+  Variable *batch_mean = &this->mean_;
+  Variable *batch_var = &this->var_;
+  if (outputs.size() == 3) {
+    batch_mean = outputs[1];
+    batch_var = outputs[2];
+  }
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  const float *beta =
+      this->no_bias_ ? nullptr : inputs[this->b_idx_]->template get_data_pointer<float>(this->ctx_);
+  const float *gamma =
+      this->no_scale_ ? nullptr : inputs[this->g_idx_]->template get_data_pointer<float>(this->ctx_);
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  float *m = batch_mean->cast_data_and_get_pointer<float>(this->ctx_, true);
+  float *v = batch_var->cast_data_and_get_pointer<float>(this->ctx_, true);
+  // Running statistics are read-modify-write inputs; recompute leaves them.
+  float *rm = !update_inputs
+                  ? nullptr
+                  : inputs[this->m_idx_]->template cast_data_and_get_pointer<float>(this->ctx_);
+  float *rv = !update_inputs
+                  ? nullptr
+                  : inputs[this->v_idx_]->template cast_data_and_get_pointer<float>(this->ctx_);
+  float *ws = workspace_.cast_data_and_get_pointer<float>(this->ctx_, true);
+  NBLA_HIP_CHECK(nblahip_bn_fwd_train(x, gamma, beta, y, m, v, rm, rv, this->size0_, this->size1_,
+                                      this->size2_, this->decay_rate_, this->eps_,
+                                      HipDtype<T>::code, ws, workspace_bytes_, nullptr));
+}
+
+template <typename T>
+void BatchNormalizationHip<T>::forward_impl_global(const Variables &inputs,
+                                                   const Variables &outputs) {
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  const float *beta =
+      this->no_bias_ ? nullptr : inputs[this->b_idx_]->template get_data_pointer<float>(this->ctx_);
+  const float *gamma =
+      this->no_scale_ ? nullptr : inputs[this->g_idx_]->template get_data_pointer<float>(this->ctx_);
+  const float *rm = inputs[this->m_idx_]->template get_data_pointer<float>(this->ctx_);
+  const float *rv = inputs[this->v_idx_]->template get_data_pointer<float>(this->ctx_);
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  NBLA_HIP_CHECK(nblahip_bn_fwd_infer(x, rm, rv, gamma, beta, y, this->size0_, this->size1_,
+                                      this->size2_, this->eps_, HipDtype<T>::code, nullptr));
+}
+
+template <typename T>
+void BatchNormalizationHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
+                                             const vector<bool> &propagate_down,
+                                             const vector<bool> &accum) {
+  hip_set_device(this->device_);
+  const bool pd_x = propagate_down[0];
+  const bool pd_beta = !this->no_bias_ && propagate_down[this->b_idx_];
+  const bool pd_gamma = !this->no_scale_ && propagate_down[this->g_idx_];
+  if (!(pd_x || pd_beta || pd_gamma)) return;
+
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
+  const float *gamma =
+      this->no_scale_ ? nullptr : inputs[this->g_idx_]->template get_data_pointer<float>(this->ctx_);
+
+  // Statistics the forward normalised with, and the gradients that reach the
+  // mean/var outputs in the three-output form.
+  const float *mean, *var, *dmean = nullptr, *dvar = nullptr;
+  if (this->batch_stat_) {
+    Variable *batch_mean = &this->mean_;
+    Variable *batch_var = &this->var_;
+    if (outputs.size() == 3) {
+      batch_mean = outputs[1];
+      batch_var = outputs[2];
+      dmean = batch_mean->get_grad_pointer<float>(this->ctx_);
+      dvar = batch_var->get_grad_pointer<float>(this->ctx_);
+    }
+    mean = batch_mean->get_data_pointer<float>(this->ctx_);
+    var = batch_var->get_data_pointer<float>(this->ctx_);
+  } else {
+    mean = inputs[this->m_idx_]->template get_data_pointer<float>(this->ctx_);
+    var = inputs[this->v_idx_]->template get_data_pointer<float>(this->ctx_);
+  }
+
+  T *dx = !pd_x ? nullptr : inputs[0]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[0]);
+  float *dbeta = !pd_beta ? nullptr
+                          : inputs[this->b_idx_]->template cast_grad_and_get_pointer<float>(
+                                this->ctx_, !accum[this->b_idx_]);
+  float *dgamma = !pd_gamma ? nullptr
+                            : inputs[this->g_idx_]->template cast_grad_and_get_pointer<float>(
+                                  this->ctx_, !accum[this->g_idx_]);
+  float *ws = workspace_.cast_data_and_get_pointer<float>(this->ctx_, true);
+  NBLA_HIP_CHECK(nblahip_bn_bwd(
+      x, dy, gamma, mean, var, dmean, dvar, dx, dgamma, dbeta, pd_x && accum[0],
+      pd_gamma && accum[this->g_idx_], pd_beta && accum[this->b_idx_], this->size0_, this->size1_,
+      this->size2_, this->eps_, this->batch_stat_ ? 1 : 0, HipDtype<T>::code, ws, workspace_bytes_,
+      nullptr));
+}
+
+template class BatchNormalizationHip<float>;
+template class BatchNormalizationHip<Half>;
+} // namespace nbla

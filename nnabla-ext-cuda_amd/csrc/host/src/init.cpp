@@ -1,0 +1,81 @@
+// init_hip(): registration of the "hip" backend (src/nbla/cuda/init.cpp.tmpl:65-270
+// is the reference's equivalent; here the table is four functions by two type
+// configs, written out by hand instead of generated from yaml).
+#include <mutex>
+
+#include <nbla/cpu.hpp>
+#include <nbla/function_registry.hpp>
+#include <nbla/hip/array/hip_array.hpp>
+#include <nbla/hip/function/batch_normalization.hpp>
+#include <nbla/hip/function/group_normalization.hpp>
+#include <nbla/hip/function/instance_normalization.hpp>
+#include <nbla/hip/function/layer_normalization.hpp>
+#include <nbla/hip/hip.hpp>
+#include <nbla/hip/init.hpp>
+
+namespace nbla {
+
+#ifdef NBLA_HIP_USE_CORE_STANDIN
+// With the real core these registries live in libnnabla.
+NBLA_REGISTER_FUNCTION_SOURCE(BatchNormalization, const vector<int> &, float, float, bool, bool, bool);
+NBLA_REGISTER_FUNCTION_SOURCE(LayerNormalization, const vector<int> &, float, bool, bool);
+NBLA_REGISTER_FUNCTION_SOURCE(GroupNormalization, int, int, const vector<int> &, float, bool, bool);
+NBLA_REGISTER_FUNCTION_SOURCE(InstanceNormalization, int, const vector<int> &, float, bool, bool);
+#endif
+
+void init_hip() {
+  static std::mutex mtx;
+  static bool is_initialized = false;
+  std::lock_guard<std::mutex> lock(mtx);
+  if (is_initialized) return;
+
+  init_cpu();
+
+  // Backend
+  NBLA_REGISTER_BACKEND("hip", [] { return static_cast<BackendBase *>(SingletonManager::get<Hip>()); });
+
+  // Array classes and synchronizers
+  ArrayCreator::add_creator("HipArray", [](Size_t s, dtypes d, const Context &c) -> Array * {
+    return new HipArray(s, d, c);
+  });
+  ArrayCreator::add_creator("HipCachedArray", [](Size_t s, dtypes d, const Context &c) -> Array * {
+    return new HipCachedArray(s, d, c);
+  });
+  const char *device_classes[] = {"HipArray", "HipCachedArray"};
+  for (const char *dc : device_classes) {
+    ArraySynchronizer::add_synchronizer(dc, "CpuArray", synchronizer_hip_array_cpu_array);
+    ArraySynchronizer::add_synchronizer("CpuArray", dc, synchronizer_cpu_array_hip_array);
+    for (const char *dc2 : device_classes)
+      ArraySynchronizer::add_synchronizer(dc, dc2, [](Array *src, Array *dst) { dst->copy_from(src); });
+  }
+
+  // Functions: same names as the reference registers, new backend key.
+  typedef BatchNormalizationHip<float> BatchNormalizationHip_float;
+  typedef BatchNormalizationHip<Half> BatchNormalizationHip_half;
+  NBLA_REGISTER_FUNCTION_IMPL(BatchNormalization, BatchNormalizationHip_float, "hip:float",
+                              const vector<int> &, float, float, bool, bool, bool);
+  NBLA_REGISTER_FUNCTION_IMPL(BatchNormalization, BatchNormalizationHip_half, "hip:half",
+                              const vector<int> &, float, float, bool, bool, bool);
+  typedef LayerNormalizationHip<float> LayerNormalizationHip_float;
+  typedef LayerNormalizationHip<Half> LayerNormalizationHip_half;
+  NBLA_REGISTER_FUNCTION_IMPL(LayerNormalization, LayerNormalizationHip_float, "hip:float",
+                              const vector<int> &, float, bool, bool);
+  NBLA_REGISTER_FUNCTION_IMPL(LayerNormalization, LayerNormalizationHip_half, "hip:half",
+                              const vector<int> &, float, bool, bool);
+  typedef GroupNormalizationHip<float> GroupNormalizationHip_float;
+  typedef GroupNormalizationHip<Half> GroupNormalizationHip_half;
+  NBLA_REGISTER_FUNCTION_IMPL(GroupNormalization, GroupNormalizationHip_float, "hip:float", int, int,
+                              const vector<int> &, float, bool, bool);
+  NBLA_REGISTER_FUNCTION_IMPL(GroupNormalization, GroupNormalizationHip_half, "hip:half", int, int,
+                              const vector<int> &, float, bool, bool);
+  typedef InstanceNormalizationHip<float> InstanceNormalizationHip_float;
+  typedef InstanceNormalizationHip<Half> InstanceNormalizationHip_half;
+  NBLA_REGISTER_FUNCTION_IMPL(InstanceNormalization, InstanceNormalizationHip_float, "hip:float", int,
+                              const vector<int> &, float, bool, bool);
+  NBLA_REGISTER_FUNCTION_IMPL(InstanceNormalization, InstanceNormalizationHip_half, "hip:half", int,
+                              const vector<int> &, float, bool, bool);
+
+  is_initialized = true;
+}
+
+} // namespace nbla

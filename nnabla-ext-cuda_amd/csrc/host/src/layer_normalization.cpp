@@ -1,0 +1,100 @@
+// LayerNormalizationHip<T>: host-side control flow of LayerNormalizationCuda<T>
+// (src/nbla/cuda/function/generic/layer_normalization.cu) over nblahip.
+#include <nbla/hip/function/layer_normalization.hpp>
+#include <nbla/variable.hpp>
+
+namespace nbla {
+
+template <typename T>
+void LayerNormalizationHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
+  LayerNormalization<T>::setup_shapes(inputs, outputs);
+  hip_set_device(this->device_);
+  const auto x_shape = inputs[0]->shape();
+  // The kernels reduce over trailing axes: batch axes must be the leading
+  // ones (the reference hands any other layout to the core's CPU function,
+  // layer_normalization.cu:43-51; this backend has no CPU path and refuses).
+  const auto &ba = this->batch_axis_;
+  const bool leading = *std::max_element(ba.begin(), ba.end()) < static_cast<int>(ba.size());
+  NBLA_CHECK(leading, error_code::not_implemented,
+             "LayerNormalizationHip supports batch_axis = [0, ..., k-1] only.");
+  batch_size_ = 1;
+  for (const auto b : ba) batch_size_ *= x_shape[b];
+  reduce_size_ = inputs[0]->size() / std::max<Size_t>(batch_size_, 1);
+  NBLA_CHECK(inputs[0]->size() < (Size_t(1) << 31), error_code::value,
+             "LayerNormalizationHip indexes with 32 bits: fewer than 2^31 elements required.");
+  mean_.reshape(Shape_t{batch_size_}, true);
+  var_.reshape(Shape_t{batch_size_}, true);
+  workspace_bytes_ = nblahip_ln_bwd_workspace_bytes(batch_size_, reduce_size_, HipDtype<T>::code);
+  workspace_.reshape(Shape_t{static_cast<Size_t>((workspace_bytes_ + 3) / 4)}, true);
+}
+
+template <typename T>
+void LayerNormalizationHip<T>::forward_impl(const Variables &inputs, const Variables &outputs) {
+  hip_set_device(this->device_);
+  Variable *v_mean = &mean_;
+  Variable *v_var = &var_;
+  if (outputs.size() == 3) { // statistics are exposed
+    v_mean = outputs[1];
+    v_var = outputs[2];
+  }
+  const int beta_idx = 1;
+  const int gamma_idx = this->no_bias_ ? 1 : 2;
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  const float *beta =
+      this->no_bias_ ? nullptr : inputs[beta_idx]->template get_data_pointer<float>(this->ctx_);
+  const float *gamma =
+      this->no_scale_ ? nullptr : inputs[gamma_idx]->template get_data_pointer<float>(this->ctx_);
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  float *mean = v_mean->cast_data_and_get_pointer<float>(this->ctx_, true);
+  float *var = v_var->cast_data_and_get_pointer<float>(this->ctx_, true);
+  NBLA_HIP_CHECK(nblahip_ln_fwd(x, gamma, beta, y, mean, var, batch_size_, reduce_size_,
+                                this->eps_, HipDtype<T>::code, nullptr));
+}
+
+template <typename T>
+void LayerNormalizationHip<T>::backward_impl(const Variables &inputs, const Variables &outputs,
+                                             const vector<bool> &propagate_down,
+                                             const vector<bool> &accum) {
+  hip_set_device(this->device_);
+  const int beta_idx = 1;
+  const int gamma_idx = this->no_bias_ ? 1 : 2;
+  const bool pd_x = propagate_down[0];
+  const bool pd_beta = !this->no_bias_ && propagate_down[beta_idx];
+  const bool pd_gamma = !this->no_scale_ && propagate_down[gamma_idx];
+  if (!(pd_x || pd_beta || pd_gamma)) return;
+
+  Variable *v_mean = &mean_;
+  Variable *v_var = &var_;
+  const float *dmean = nullptr, *dvar = nullptr;
+  if (outputs.size() == 3) {
+    v_mean = outputs[1];
+    v_var = outputs[2];
+    dmean = v_mean->get_grad_pointer<float>(this->ctx_);
+    dvar = v_var->get_grad_pointer<float>(this->ctx_);
+  }
+  const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
+  const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
+  const float *gamma =
+      this->no_scale_ ? nullptr : inputs[gamma_idx]->template get_data_pointer<float>(this->ctx_);
+  const float *mean = v_mean->get_data_pointer<float>(this->ctx_);
+  const float *var = v_var->get_data_pointer<float>(this->ctx_);
+  T *dx = !pd_x ? nullptr : inputs[0]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[0]);
+  float *dbeta = !pd_beta ? nullptr
+                          : inputs[beta_idx]->template cast_grad_and_get_pointer<float>(
+                                this->ctx_, !accum[beta_idx]);
+  float *dgamma = !pd_gamma ? nullptr
+                            : inputs[gamma_idx]->template cast_grad_and_get_pointer<float>(
+                                  this->ctx_, !accum[gamma_idx]);
+  float *ws = workspace_.cast_data_and_get_pointer<float>(this->ctx_, true);
+  NBLA_HIP_CHECK(nblahip_ln_bwd(x, dy, gamma, mean, var, dmean, dvar, dx, dgamma, dbeta,
+                                pd_x && accum[0], pd_gamma && accum[gamma_idx],
+                                pd_beta && accum[beta_idx], batch_size_, reduce_size_, this->eps_,
+                                HipDtype<T>::code, ws, workspace_bytes_, nullptr));
+  // Scratch is only needed inside the call (the reference clears its buffers
+  // the same way, layer_normalization.cu:202-203,236-237).
+  workspace_.data()->array()->clear();
+}
+
+template class LayerNormalizationHip<float>;
+template class LayerNormalizationHip<Half>;
+} // namespace nbla

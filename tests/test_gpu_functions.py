@@ -1,0 +1,272 @@
+"""The nbla::Function classes of the "hip" backend, driven the way NNabla's
+function tests drive a backend: create by name and context, setup, forward,
+backward with propagate_down/accum flags, compared with the oracle."""
+import numpy as np
+import pytest
+
+from _util import assert_close, load_package
+from oracle import norm_ref as R
+
+load_package()
+from nnabla_ext_cuda_amd import binding as B  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+CONFIGS = ["float", "half"]
+
+
+def dn(tc):
+    return "f16" if tc == "half" else "f32"
+
+
+def rnd(a, tc):
+    a = np.asarray(a, np.float32)
+    return a.astype(np.float16).astype(np.float64) if tc == "half" else a.astype(np.float64)
+
+
+def var(a, half=False):
+    v = B.Variable(np.shape(a))
+    v.set_data(a, half=half)
+    return v
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    B.init()
+
+
+@pytest.mark.parametrize("tc", CONFIGS)
+@pytest.mark.parametrize("shape,axis", [((4, 8, 6, 6), 1), ((6, 5, 4, 8), 3), ((16, 24), 1)])
+def test_batch_normalization_training(tc, shape, axis):
+    rng = np.random.default_rng(1)
+    half = tc == "half"
+    c = shape[axis]
+    pshape = tuple(c if i == axis else 1 for i in range(len(shape)))
+    x = rnd(rng.standard_normal(shape) * 2 + 1, tc)
+    dy = rnd(rng.standard_normal(shape), tc)
+    g = rng.uniform(0.5, 1.5, pshape).astype(np.float32)
+    b = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
+    rm = np.zeros(pshape, np.float32)
+    rv = np.ones(pshape, np.float32)
+    f = B.BatchNormalization(B.context(tc), axes=[axis], decay_rate=0.9, eps=1e-5, batch_stat=True)
+    assert f.name == "BatchNormalizationHip"
+    vx, vb, vg, vm, vv = var(x, half), var(b), var(g), var(rm), var(rv)
+    vy = B.Variable(shape)
+    ins = [vx, vb, vg, vm, vv]
+    f.setup(ins, [vy])
+    f.forward(ins, [vy])
+    y_r, m_r, v_r, rm_r, rv_r = R.bn_forward_batch(x, b, g, rm, rv, axis, 0.9, 1e-5)
+    assert_close(vy.d, y_r, dn(tc), "y", "y")
+    assert_close(vm.d, rm_r, dn(tc), "stat", "running mean (updated in place)")
+    assert_close(vv.d, rv_r, dn(tc), "stat", "running var (updated in place)")
+
+    # recompute must not touch the running statistics
+    f.recompute(ins, [vy])
+    assert_close(vm.d, rm_r, dn(tc), "stat", "running mean after recompute")
+    assert_close(vy.d, y_r, dn(tc), "y", "y after recompute")
+
+    vy.set_grad(dy, half)
+    f.backward(ins, [vy], propagate_down=[1, 1, 1, 0, 0], accum=[0, 0, 0, 0, 0])
+    dx_r, dg_r, db_r = R.bn_backward_batch(x, dy, g, m_r, v_r, axis, 1e-5)
+    assert_close(vx.g, dx_r, dn(tc), "grad", "dx")
+    assert_close(vg.g, dg_r, dn(tc), "pgrad", "dgamma")
+    assert_close(vb.g, db_r, dn(tc), "pgrad", "dbeta")
+
+    # accumulation: run backward again onto the existing gradients
+    f.backward(ins, [vy], propagate_down=[1, 1, 1, 0, 0], accum=[1, 1, 1, 0, 0])
+    assert_close(vx.g, 2 * dx_r, dn(tc), "grad", "dx accum")
+    assert_close(vg.g, 2 * dg_r, dn(tc), "pgrad", "dgamma accum")
+    # propagate_down subset: only beta; the others keep their values
+    before = vx.g.copy()
+    f.backward(ins, [vy], propagate_down=[0, 1, 0, 0, 0], accum=[0, 0, 0, 0, 0])
+    assert_close(vb.g, db_r, dn(tc), "pgrad", "dbeta only")
+    np.testing.assert_array_equal(vx.g, before)
+
+
+@pytest.mark.parametrize("tc", CONFIGS)
+def test_batch_normalization_three_outputs_and_flags(tc):
+    rng = np.random.default_rng(2)
+    half = tc == "half"
+    shape, axis, c = (4, 6, 5, 5), 1, 6
+    pshape = (1, c, 1, 1)
+    x = rnd(rng.standard_normal(shape), tc)
+    dy = rnd(rng.standard_normal(shape), tc)
+    dm = rng.standard_normal(pshape).astype(np.float32)
+    dv = rng.standard_normal(pshape).astype(np.float32)
+    rm, rv = np.zeros(pshape, np.float32), np.ones(pshape, np.float32)
+    f = B.BatchNormalization(B.context(tc), axes=[axis], batch_stat=True, no_scale=True, no_bias=True)
+    vx, vm, vv = var(x, half), var(rm), var(rv)
+    vy, om, ov = B.Variable(shape), B.Variable(()), B.Variable(())
+    f.setup([vx, vm, vv], [vy, om, ov])
+    assert om.current_shape == pshape and ov.current_shape == pshape
+    f.forward([vx, vm, vv], [vy, om, ov])
+    y_r, m_r, v_r, _, _ = R.bn_forward_batch(x, None, None, None, None, axis, 0.9, 1e-5)
+    assert_close(vy.d, y_r, dn(tc), "y", "y")
+    assert_close(om.d, m_r, dn(tc), "stat", "mean output")
+    assert_close(ov.d, v_r, dn(tc), "stat", "var output")
+    vy.set_grad(dy, half)
+    om.set_grad(dm)
+    ov.set_grad(dv)
+    f.backward([vx, vm, vv], [vy, om, ov], propagate_down=[1, 0, 0], accum=[0, 0, 0])
+    dx_r, _, _ = R.bn_backward_batch(x, dy, None, m_r, v_r, axis, 1e-5, dm, dv)
+    assert_close(vx.g, dx_r, dn(tc), "grad", "dx with dmean/dvar")
+
+
+@pytest.mark.parametrize("tc", CONFIGS)
+def test_batch_normalization_inference(tc):
+    rng = np.random.default_rng(3)
+    half = tc == "half"
+    shape, c = (8, 16, 7, 7), 16
+    pshape = (1, c, 1, 1)
+    x = rnd(rng.standard_normal(shape), tc)
+    dy = rnd(rng.standard_normal(shape), tc)
+    g = rng.uniform(0.5, 1.5, pshape).astype(np.float32)
+    b = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
+    rm = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
+    rv = rng.uniform(0.5, 2, pshape).astype(np.float32)
+    f = B.BatchNormalization(B.context(tc), axes=[1], batch_stat=False)
+    vx, vb, vg, vm, vv = var(x, half), var(b), var(g), var(rm), var(rv)
+    vy = B.Variable(shape)
+    ins = [vx, vb, vg, vm, vv]
+    f.setup(ins, [vy])
+    f.forward(ins, [vy])
+    assert_close(vy.d, R.bn_forward_global(x, b, g, rm, rv, 1, 1e-5), dn(tc), "y", "y")
+    np.testing.assert_array_equal(vm.d, rm)          # running stats are read-only here
+    vy.set_grad(dy, half)
+    f.backward(ins, [vy], propagate_down=[1, 1, 1, 0, 0], accum=[0] * 5)
+    dx_r, dg_r, db_r = R.bn_backward_global(x, dy, g, rm, rv, 1, 1e-5)
+    assert_close(vx.g, dx_r, dn(tc), "grad", "dx")
+    assert_close(vg.g, dg_r, dn(tc), "pgrad", "dgamma")
+    assert_close(vb.g, db_r, dn(tc), "pgrad", "dbeta")
+
+
+@pytest.mark.parametrize("tc", CONFIGS)
+@pytest.mark.parametrize("shape,batch_axis", [((4, 6, 64), (0, 1)), ((8, 1000), (0,)), ((3, 5, 7, 16), (0,))])
+def test_layer_normalization(tc, shape, batch_axis):
+    rng = np.random.default_rng(4)
+    half = tc == "half"
+    outer = int(np.prod([shape[a] for a in batch_axis]))
+    pshape = tuple(1 if i in batch_axis else s for i, s in enumerate(shape))
+    x = rnd(rng.standard_normal(shape) + 2, tc)
+    dy = rnd(rng.standard_normal(shape), tc)
+    g = (rng.standard_normal(pshape) * 0.1 + 1).astype(np.float32)
+    b = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
+    f = B.LayerNormalization(B.context(tc), batch_axis=list(batch_axis), eps=1e-5)
+    vx, vb, vg = var(x, half), var(b), var(g)
+    vy, om, ov = B.Variable(shape), B.Variable(()), B.Variable(())
+    f.setup([vx, vb, vg], [vy, om, ov])
+    f.forward([vx, vb, vg], [vy, om, ov])
+    y_r, m_r, v_r = R.ln_forward(x, b, g, outer, 1e-5)
+    assert_close(vy.d, y_r, dn(tc), "y", "y")
+    assert_close(om.d, m_r, dn(tc), "stat", "mean output")
+    assert_close(ov.d, v_r, dn(tc), "stat", "var output")
+    dm = rng.standard_normal(om.current_shape).astype(np.float32)
+    dv = rng.standard_normal(ov.current_shape).astype(np.float32)
+    vy.set_grad(dy, half)
+    om.set_grad(dm)
+    ov.set_grad(dv)
+    pre = rng.standard_normal(shape).astype(np.float32)
+    vx.set_grad(pre, half)
+    f.backward([vx, vb, vg], [vy, om, ov], propagate_down=[1, 1, 1], accum=[1, 0, 0])
+    dx_r, dg_r, db_r = R.ln_backward(x, dy, g, m_r, v_r, outer, 1e-5, dm, dv)
+    assert_close(vx.g, dx_r + rnd(pre, tc), dn(tc), "grad", "dx accum with dmean/dvar")
+    assert_close(vg.g, dg_r, dn(tc), "pgrad", "dgamma")
+    assert_close(vb.g, db_r, dn(tc), "pgrad", "dbeta")
+
+
+@pytest.mark.parametrize("tc", CONFIGS)
+@pytest.mark.parametrize("shape,groups", [((4, 16, 8, 8), 4), ((2, 6, 5), 3), ((3, 8, 7, 7), 8)])
+def test_group_normalization(tc, shape, groups):
+    rng = np.random.default_rng(5)
+    half = tc == "half"
+    n, c = shape[0], shape[1]
+    pshape = (1, c) + (1,) * (len(shape) - 2)
+    x = rnd(rng.standard_normal(shape) * 1.5, tc)
+    dy = rnd(rng.standard_normal(shape), tc)
+    g = rng.uniform(0.5, 1.5, pshape).astype(np.float32)
+    b = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
+    f = B.GroupNormalization(B.context(tc), num_groups=groups, channel_axis=1, batch_axis=[0])
+    vx, vb, vg = var(x, half), var(b), var(g)
+    vy = B.Variable(shape)
+    f.setup([vx, vb, vg], [vy])
+    f.forward([vx, vb, vg], [vy])
+    y_r, m_r, v_r = R.gn_forward(x, b, g, n, c, groups, 1e-5)
+    assert_close(vy.d, y_r, dn(tc), "y", "y")
+    vy.set_grad(dy, half)
+    f.backward([vx, vb, vg], [vy], propagate_down=[1, 1, 1], accum=[0, 0, 0])
+    dx_r, dg_r, db_r = R.gn_backward(x, dy, g, m_r, v_r, n, c, groups, 1e-5)
+    assert_close(vx.g, dx_r, dn(tc), "grad", "dx")
+    assert_close(vg.g, dg_r, dn(tc), "pgrad", "dgamma")
+    assert_close(vb.g, db_r, dn(tc), "pgrad", "dbeta")
+
+
+@pytest.mark.parametrize("tc", CONFIGS)
+@pytest.mark.parametrize("per_sample", [False, True])
+def test_instance_normalization(tc, per_sample):
+    rng = np.random.default_rng(6)
+    half = tc == "half"
+    shape = (3, 5, 9, 9)
+    n, c = shape[0], shape[1]
+    pshape = (n if per_sample else 1, c, 1, 1)
+    x = rnd(rng.standard_normal(shape) * 1.5, tc)
+    dy = rnd(rng.standard_normal(shape), tc)
+    g = rng.uniform(0.5, 1.5, pshape).astype(np.float32)
+    b = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
+    f = B.InstanceNormalization(B.context(tc), channel_axis=1, batch_axis=[0])
+    vx, vb, vg = var(x, half), var(b), var(g)
+    vy = B.Variable(shape)
+    f.setup([vx, vb, vg], [vy])
+    f.forward([vx, vb, vg], [vy])
+    g_full = g.reshape(-1) if per_sample else np.tile(g.reshape(-1), n)
+    b_full = b.reshape(-1) if per_sample else np.tile(b.reshape(-1), n)
+    y_r, m_r, v_r = R.in_forward(x, b_full, g_full, n, c, 1e-5)
+    assert_close(vy.d, y_r, dn(tc), "y", "y")
+    vy.set_grad(dy, half)
+    f.backward([vx, vb, vg], [vy], propagate_down=[1, 1, 1], accum=[0, 0, 0])
+    dx_r, dg_r, db_r = R.in_backward(x, dy, g.reshape(-1), m_r, v_r, n, c, 1e-5,
+                                     bc_gamma=not per_sample, bc_beta=not per_sample)
+    assert_close(vx.g, dx_r, dn(tc), "grad", "dx")
+    assert_close(vg.g, dg_r, dn(tc), "pgrad", "dgamma")
+    assert_close(vb.g, db_r, dn(tc), "pgrad", "dbeta")
+
+
+def test_unsupported_layouts_raise_not_implemented():
+    ctx = B.context("float")
+    x, y = B.Variable((4, 6, 8)), B.Variable((4, 6, 8))
+    f = B.LayerNormalization(ctx, batch_axis=[1], no_scale=True, no_bias=True)
+    with pytest.raises(B.NblaError, match="batch_axis"):
+        f.setup([x], [y])
+    g = B.GroupNormalization(ctx, num_groups=2, channel_axis=2, batch_axis=[0], no_scale=True,
+                             no_bias=True)
+    with pytest.raises(B.NblaError, match="channel-first"):
+        g.setup([x], [y])
+    h = B.GroupNormalization(ctx, num_groups=4, channel_axis=1, batch_axis=[0], no_scale=True,
+                             no_bias=True)
+    with pytest.raises(B.NblaError, match="divisible"):
+        h.setup([x], [y])
+
+
+def test_caching_allocator_reuses_blocks():
+    import ctypes
+    L = B.lib()
+    live, cached = ctypes.c_uint64(), ctypes.c_uint64()
+    ctx = B.context("float")
+    x = np.random.default_rng(7).standard_normal((64, 256)).astype(np.float32)
+
+    def run():
+        f = B.LayerNormalization(ctx, batch_axis=[0], no_scale=True, no_bias=True)
+        vx, vy = var(x), B.Variable(x.shape)
+        f.setup([vx], [vy])
+        f.forward([vx], [vy])
+        return vy.d
+
+    a = run()
+    L.nnabla_hip_memory_stats(ctypes.byref(live), ctypes.byref(cached))
+    assert cached.value > 0                      # freed arrays went to the cache
+    c1 = cached.value
+    b = run()
+    np.testing.assert_array_equal(a, b)
+    L.nnabla_hip_memory_stats(ctypes.byref(live), ctypes.byref(cached))
+    assert cached.value == c1                    # second run was served from it
+    assert L.nnabla_hip_clear_memory_cache() == 0
+    L.nnabla_hip_memory_stats(ctypes.byref(live), ctypes.byref(cached))
+    assert cached.value == 0
