@@ -243,10 +243,10 @@ def cpu_baseline(budget_s=12.0):
 def load_traffic():
     """HBM bytes per launch of the dominant kernel from the committed
     rocprofv3 --pmc summaries, or None."""
-    path = os.path.join(ROOT, "profiles", "traffic.json")
+    path = os.path.join(ROOT, "profiles", "bn_bwd_apply_planes_c2_traffic.txt")
     try:
         with open(path) as f:
-            return json.load(f).get("bn_bwd_apply_planes_fused_kernel", {}).get("hbm_bytes_per_launch")
+            return json.load(f).get("bn_bwd_apply_planes_kernel", {}).get("hbm_bytes_per_launch")
     except (OSError, ValueError):
         return None
 
@@ -258,6 +258,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-table", action="store_true", help="skip the per-config table")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch a float32->float16 convert of the workload's x (a plain "
+                         "streaming kernel of known traffic: 4 B read, 2 B written per element) "
+                         "so that rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE readings can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus must be 1 "
@@ -272,6 +276,14 @@ def main():
     torch.cuda.set_device(0)
 
     fwd, bwd, fb, bb, keep = make_bn(K, (32, 256, 56, 56), 1, torch.float32, True, 1.0, 2.0, seed=1)
+    if args.calibrate:
+        xs = keep[0]
+        half = torch.empty(xs.shape, dtype=torch.float16, device="cuda")
+        st = torch.cuda.current_stream().cuda_stream
+        for _ in range(args.steps):
+            K.check(L.nblahip_convert(half.data_ptr(), K.F16, xs.data_ptr(), K.F32, xs.numel(), st))
+        torch.cuda.synchronize()
+        del half
     ms = time_calls([fwd, bwd], args.steps, args.warmup)
     value = (fb + bb) / ms / 1e6  # GB/s
     log(f"C2 fwd+bwd: {ms * 1e3:.1f} us/step, {value:.0f} GB/s algorithmic")

@@ -240,8 +240,9 @@ NBLAHIP_EXPORT int nblahip_fill(void *dst, int dtype, float value, int64_t n,
 /* ------------------------------------------------------------------------
  * Per-kernel event timing, the counterpart of the reference's
  * CudaEventTimerCallback (python/src/nnabla_ext/cuda/utils/inspection/
- * profile.py:23-74), which brackets each function with CUDA events.  Here the
- * brackets sit around every kernel launch, on the launch stream.
+ * profile.py:23-74), which brackets each function with CUDA events.  Here every
+ * kernel launch carries its own start/stop event pair on the launch stream
+ * (stamped at the begin and end of the kernel's execution).
  *   enable(n > 0): pre-create n event pairs and start recording (launches
  *                  beyond n are not recorded); enable(0): stop and release.
  *   reset        : forget the records, keep the pool.
@@ -250,8 +251,7 @@ NBLAHIP_EXPORT int nblahip_fill(void *dst, int dtype, float value, int64_t n,
  *                  the row kernels are "row_fwd_kernel", "row_bwd_kernel_ln",
  *                  "row_bwd_kernel_in", "row_bwd_kernel_gn") and return their
  *                  summed duration and count.
- * Not for use while other threads are launching; timing adds two event
- * records per launch.
+ * Not for use while other threads are launching.
  * ---------------------------------------------------------------------- */
 NBLAHIP_EXPORT int nblahip_profile_enable(int max_records);
 NBLAHIP_EXPORT int nblahip_profile_reset(void);

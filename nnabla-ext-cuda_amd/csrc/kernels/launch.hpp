@@ -4,6 +4,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -97,19 +98,23 @@ int launch_bn_fwd_train(const BnProblem &p, hipStream_t st);
 int launch_bn_bwd(const BnProblem &p, hipStream_t st);
 size_t bn_workspace_bytes(int64_t size0, int64_t C, int64_t size2, int dtype);
 
-// Optional per-kernel timing (HIP events recorded on the launch stream around
-// every kernel).  Off by default; see nblahip_profile_* in the C-ABI.
-struct ProfScope {
-  int slot;
-  hipStream_t st;
-  ProfScope(const char *tag, hipStream_t s);
-  ~ProfScope();
-};
+// Optional per-kernel timing.  When enabled, a launch goes through
+// hipExtLaunchKernelGGL with a start/stop event pair, which stamps the
+// kernel's own dispatch (begin and end of execution on the device), the same
+// interval a kernel trace reports.  Off by default; see nblahip_profile_* in
+// the C-ABI.  Returns false (and leaves the events untouched) when timing is
+// off or the pool is exhausted.
+bool prof_acquire(const char *tag, hipEvent_t *start, hipEvent_t *stop);
 
-#define NBLAHIP_LAUNCH(tag, kern, grid, block, shmem, st, ...)       \
-  do {                                                               \
-    ::nblahip::ProfScope prof_scope_(tag, st);                       \
-    hipLaunchKernelGGL(kern, grid, block, shmem, st, __VA_ARGS__);   \
+#define NBLAHIP_LAUNCH(tag, kern, grid, block, shmem, st, ...)                          \
+  do {                                                                                  \
+    hipEvent_t prof_ev0_, prof_ev1_;                                                    \
+    if (::nblahip::prof_acquire(tag, &prof_ev0_, &prof_ev1_)) {                         \
+      hipExtLaunchKernelGGL(kern, grid, block, shmem, st, prof_ev0_, prof_ev1_, 0,      \
+                            __VA_ARGS__);                                               \
+    } else {                                                                            \
+      hipLaunchKernelGGL(kern, grid, block, shmem, st, __VA_ARGS__);                    \
+    }                                                                                   \
   } while (0)
 
 inline int last_launch_status() {

@@ -61,20 +61,18 @@ struct ProfState {
 } g_prof;
 } // namespace
 
-ProfScope::ProfScope(const char *tag, hipStream_t s) : slot(-1), st(s) {
-  if (!g_prof.enabled) return;
+bool prof_acquire(const char *tag, hipEvent_t *start, hipEvent_t *stop) {
+  if (!g_prof.enabled) return false;
   std::lock_guard<std::mutex> lock(g_prof.mu);
   if (g_prof.used >= g_prof.records.size()) {
     ++g_prof.dropped;
-    return;
+    return false;
   }
-  slot = static_cast<int>(g_prof.used++);
-  g_prof.records[slot].tag = tag;
-  (void)hipEventRecord(g_prof.records[slot].start, st);
-}
-
-ProfScope::~ProfScope() {
-  if (slot >= 0) (void)hipEventRecord(g_prof.records[slot].stop, st);
+  ProfRecord &r = g_prof.records[g_prof.used++];
+  r.tag = tag;
+  *start = r.start;
+  *stop = r.stop;
+  return true;
 }
 
 static void prof_release_locked() {
