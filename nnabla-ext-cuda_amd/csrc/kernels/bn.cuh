@@ -78,11 +78,44 @@ bn_stats_planes_kernel(const T *__restrict__ x, uint32_t C, FastDiv nvp, uint32_
 // ---------------------------------------------------------------------------
 // Forward statistics, channel-last layout x[M][C].  grid = (ceil(ncv/TX), S),
 // ncv = C/VEC.  Split s covers rows [s*rps, min((s+1)*rps, M)).
+// A thread keeps VEC Welford states (one per channel it owns) and feeds them
+// chunks of kBnClRows rows: chunk mean, centred chunk M2, one Chan merge.
 // ---------------------------------------------------------------------------
+constexpr int kBnClRows = 8;
+
+template <typename T, int VEC, bool FULL>
+__device__ __forceinline__ void bn_cl_chunk(const RawVec<T, VEC> (&raw)[kBnClRows], int cnt,
+                                            float one, float (&mean)[VEC], float (&m2)[VEC],
+                                            float &n) {
+  const float fc = static_cast<float>(cnt);
+  const float inv_fc = fast_rcp(fc);
+  const float nn = n + fc;
+  const float wb = fc * fast_rcp(nn); // weight of the chunk mean
+  const float wd = n * wb;            // n_a*n_b/(n_a+n_b)
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    float sum = 0.f; // rows beyond cnt were zeroed at load time
+#pragma unroll
+    for (int u = 0; u < kBnClRows; ++u) sum = elem_fma<T, VEC>(raw[u], j, one, sum);
+    const float cm = sum * inv_fc;
+    float cm2 = 0.f;
+#pragma unroll
+    for (int u = 0; u < kBnClRows; ++u) {
+      const float d = elem_fma<T, VEC>(raw[u], j, one, -cm);
+      if (FULL || u < cnt) cm2 = fmaf(d, d, cm2);
+    }
+    const float d = cm - mean[j];
+    mean[j] = fmaf(d, wb, mean[j]);
+    m2[j] += fmaf(d * d, wd, cm2);
+  }
+  n = nn;
+}
+
 template <typename T, int VEC>
 __global__ void __launch_bounds__(kBnBlock)
 bn_stats_cl_kernel(const T *__restrict__ x, uint32_t M, uint32_t C, uint32_t ncv,
-                   uint32_t log2tx, uint32_t rps, float *__restrict__ part /*[C][S][3]*/) {
+                   uint32_t log2tx, uint32_t rps, float one,
+                   float *__restrict__ part /*[C][S][3]*/) {
   // [TY][TX*VEC] means and m2 plus [TY][TX] counts; TY*TX == 256.
   __shared__ float lmean[kBnBlock * VEC];
   __shared__ float lm2[kBnBlock * VEC];
@@ -105,43 +138,27 @@ bn_stats_cl_kernel(const T *__restrict__ x, uint32_t M, uint32_t C, uint32_t ncv
   float n = 0.f;
 
   if (active) {
-    for (uint32_t r0 = rbegin + ty; r0 < rend; r0 += TY * kBnUnroll) {
-      float vals[kBnUnroll][VEC];
+    const T *xc = x + static_cast<size_t>(cv) * VEC;
+    uint32_t r0 = rbegin + ty;
+    // full chunks: every row valid, no masks
+    for (; r0 + (kBnClRows - 1) * TY < rend; r0 += TY * kBnClRows) {
+      RawVec<T, VEC> raw[kBnClRows];
+#pragma unroll
+      for (int u = 0; u < kBnClRows; ++u)
+        raw[u] = load_raw<T, VEC>(xc + static_cast<size_t>(r0 + u * TY) * C);
+      bn_cl_chunk<T, VEC, true>(raw, kBnClRows, one, mean, m2, n);
+    }
+    if (r0 < rend) { // tail chunk: clamp the row, zero what lies beyond
+      RawVec<T, VEC> raw[kBnClRows];
       int cnt = 0;
 #pragma unroll
-      for (int u = 0; u < kBnUnroll; ++u) {
+      for (int u = 0; u < kBnClRows; ++u) {
         const uint32_t r = r0 + u * TY;
-        if (r < rend) {
-          load_vec<T, VEC>(x + (static_cast<size_t>(r) * C + static_cast<size_t>(cv) * VEC), vals[u]);
-          ++cnt;
-        } else {
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) vals[u][j] = 0.f;
-        }
+        const bool ok = r < rend;
+        raw[u] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(xc + static_cast<size_t>(ok ? r : r0) * C));
+        cnt += ok ? 1 : 0;
       }
-      // cnt >= 1 here.  Chunk statistics per channel, then one Chan merge.
-      const float fc = static_cast<float>(cnt);
-      const float inv_fc = fast_rcp(fc);
-      const float nn = n + fc;
-      const float wb = fc * fast_rcp(nn); // weight of the chunk mean
-      const float wd = n * wb;            // n_a*n_b/(n_a+n_b)
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        float sum = 0.f;
-#pragma unroll
-        for (int u = 0; u < kBnUnroll; ++u) sum += vals[u][j];
-        const float cm = sum * inv_fc;
-        float cm2 = 0.f;
-#pragma unroll
-        for (int u = 0; u < kBnUnroll; ++u) {
-          const float d = vals[u][j] - cm;
-          cm2 += (u < cnt) ? d * d : 0.f;
-        }
-        const float d = cm - mean[j];
-        mean[j] += d * wb;
-        m2[j] += cm2 + d * d * wd;
-      }
-      n = nn;
+      bn_cl_chunk<T, VEC, false>(raw, cnt, one, mean, m2, n);
     }
   }
 #pragma unroll
@@ -322,21 +339,23 @@ __global__ void __launch_bounds__(256)
 bn_apply_cl_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
                    uint32_t ncv, uint32_t total_vec) {
   const uint32_t cv = threadIdx.x % ncv;
+  // y = x*pa + ps with ps = pb - mean*pa for half output (one mixed fma per
+  // element); the centred form (x-mean)*pa + pb for float output.
   float pm[VEC], pa[VEC], pb[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
     const BnParam q = src.get(cv * VEC + j);
     pm[j] = q.mean;
     pa[j] = q.a;
-    pb[j] = q.b;
+    pb[j] = (sizeof(T) == 2) ? fmaf(-q.mean, q.a, q.b) : q.b;
   }
   for (uint32_t i0 = blockIdx.x * (256u * kBnUnroll) + threadIdx.x; i0 < total_vec;
        i0 += gridDim.x * (256u * kBnUnroll)) {
-    float v[kBnUnroll][VEC];
+    RawVec<T, VEC> raw[kBnUnroll];
 #pragma unroll
     for (int u = 0; u < kBnUnroll; ++u) {
-      const uint32_t i = i0 + u * 256u;
-      if (i < total_vec) load_vec<T, VEC>(x + static_cast<size_t>(i) * VEC, v[u]);
+      const uint32_t i = min(i0 + u * 256u, total_vec - 1); // clamped: loads stay branch-free
+      raw[u] = load_raw<T, VEC>(x + static_cast<size_t>(i) * VEC);
     }
 #pragma unroll
     for (int u = 0; u < kBnUnroll; ++u) {
@@ -344,7 +363,13 @@ bn_apply_cl_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
       if (i < total_vec) {
         float o[VEC];
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) o[j] = (v[u][j] - pm[j]) * pa[j] + pb[j];
+        for (int j = 0; j < VEC; ++j) {
+          if constexpr (sizeof(T) == 2) {
+            o[j] = elem_fma<T, VEC>(raw[u], j, pa[j], pb[j]);
+          } else {
+            o[j] = (elem_fma<T, VEC>(raw[u], j, 1.0f, 0.f) - pm[j]) * pa[j] + pb[j];
+          }
+        }
         store_vec<T, VEC>(y + static_cast<size_t>(i) * VEC, o);
       }
     }
@@ -406,7 +431,7 @@ template <typename T, int VEC>
 __global__ void __launch_bounds__(kBnBlock)
 bn_bwd_reduce_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                         const float *__restrict__ mean, uint32_t M, uint32_t C,
-                        uint32_t ncv, uint32_t log2tx, uint32_t rps,
+                        uint32_t ncv, uint32_t log2tx, uint32_t rps, float one,
                         float *__restrict__ part2 /*[C][S][2]*/) {
   __shared__ float lsdx[kBnBlock * VEC];
   __shared__ float lsdy[kBnBlock * VEC];
@@ -421,33 +446,41 @@ bn_bwd_reduce_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
   const uint32_t rbegin = s * rps;
   const uint32_t rend = min(rbegin + rps, M);
 
-  float sdx[VEC], sdy[VEC], m[VEC];
+  float sdx[VEC], sdy[VEC], nm[VEC];
+  {
+    // Clamped index instead of a branch: one vector load of the VEC means.
+    float mv[VEC];
+    const uint32_t cvc = active ? cv : 0u;
 #pragma unroll
-  for (int j = 0; j < VEC; ++j) {
-    sdx[j] = sdy[j] = 0.f;
-    m[j] = active ? mean[cv * VEC + j] : 0.f;
+    for (int j = 0; j < VEC; ++j) mv[j] = mean[cvc * VEC + j];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      sdx[j] = sdy[j] = 0.f;
+      nm[j] = -mv[j];
+    }
   }
   if (active) {
     for (uint32_t r0 = rbegin + ty; r0 < rend; r0 += TY * kBnUnroll) {
-      float xv[kBnUnroll][VEC], dv[kBnUnroll][VEC];
+      RawVec<T, VEC> xr[kBnUnroll], dr[kBnUnroll];
+      // All loads first (rows beyond the split re-read row r0), selects after:
+      // the eight loads are in flight together.
 #pragma unroll
       for (int u = 0; u < kBnUnroll; ++u) {
         const uint32_t r = r0 + u * TY;
-        if (r < rend) {
-          const size_t off = static_cast<size_t>(r) * C + static_cast<size_t>(cv) * VEC;
-          load_vec<T, VEC>(x + off, xv[u]);
-          load_vec<T, VEC>(dy + off, dv[u]);
-        } else {
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) xv[u][j] = dv[u][j] = 0.f;
-        }
+        const size_t off = static_cast<size_t>(r < rend ? r : r0) * C + static_cast<size_t>(cv) * VEC;
+        xr[u] = load_raw<T, VEC>(x + off);
+        dr[u] = load_raw<T, VEC>(dy + off);
       }
+#pragma unroll
+      for (int u = 0; u < kBnUnroll; ++u) // dy zeroed beyond the split: adds nothing
+        dr[u] = raw_or_zero<T, VEC>(r0 + u * TY < rend, dr[u]);
 #pragma unroll
       for (int u = 0; u < kBnUnroll; ++u)
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
-          sdy[j] += dv[u][j];
-          sdx[j] += dv[u][j] * (xv[u][j] - m[j]);
+          const float xc = elem_fma<T, VEC>(xr[u], j, one, nm[j]);
+          sdy[j] = elem_fma<T, VEC>(dr[u], j, one, sdy[j]);
+          sdx[j] = elem_fma<T, VEC>(dr[u], j, xc, sdx[j]);
         }
     }
   }
@@ -569,25 +602,25 @@ bn_bwd_apply_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                        uint32_t ncv, uint32_t total_vec, int accum) {
   constexpr int U = 2;
   const uint32_t cv = threadIdx.x % ncv;
-  float pm[VEC], pa[VEC], pb[VEC], pc[VEC];
+  // dx = pa*dy + pb*(x - mean) + pc = pa*dy + (pb*x + ps), ps = pc - pb*mean:
+  // pb*(x-mean) is the small curvature term, so folding the mean costs nothing
+  // measurable in float either (|pb*mean| <= |dvar|*2|mean|/N).
+  float pa[VEC], pb[VEC], ps[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
     const BnParam q = params[cv * VEC + j];
-    pm[j] = q.mean;
     pa[j] = q.a;
     pb[j] = q.b;
-    pc[j] = q.c;
+    ps[j] = fmaf(-q.b, q.mean, q.c);
   }
   for (uint32_t i0 = blockIdx.x * (256u * U) + threadIdx.x; i0 < total_vec;
        i0 += gridDim.x * (256u * U)) {
-    float xv[U][VEC], dv[U][VEC];
+    RawVec<T, VEC> xr[U], dr[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const uint32_t i = i0 + u * 256u;
-      if (i < total_vec) {
-        load_vec<T, VEC>(x + static_cast<size_t>(i) * VEC, xv[u]);
-        load_vec<T, VEC>(dy + static_cast<size_t>(i) * VEC, dv[u]);
-      }
+      const uint32_t i = min(i0 + u * 256u, total_vec - 1);
+      xr[u] = load_raw<T, VEC>(x + static_cast<size_t>(i) * VEC);
+      dr[u] = load_raw<T, VEC>(dy + static_cast<size_t>(i) * VEC);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -595,7 +628,8 @@ bn_bwd_apply_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
       if (i < total_vec) {
         float o[VEC];
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) o[j] = pa[j] * dv[u][j] + pb[j] * (xv[u][j] - pm[j]) + pc[j];
+        for (int j = 0; j < VEC; ++j)
+          o[j] = elem_fma<T, VEC>(dr[u], j, pa[j], elem_fma<T, VEC>(xr[u], j, pb[j], ps[j]));
         if (accum) {
           float old[VEC];
           load_vec<T, VEC>(dx + static_cast<size_t>(i) * VEC, old);

@@ -62,14 +62,15 @@ BnPlan make_plan(int64_t size0, int64_t C, int64_t size2, int dtype, bool ptr_al
     const uint32_t TY = kBnBlock >> l2;
     pl.ytiles = ceil_div_u(pl.ncv, TX);
     const uint64_t M = static_cast<uint64_t>(size0);
+    // Equal row ranges, a whole number of blocks per CU when the tensor is
+    // large enough (an uneven last wave of blocks costs a full block time);
+    // the kernels mask the ragged end of a range themselves.
     const uint32_t step = TY * kBnUnroll;
     const uint32_t want = std::max<uint32_t>(1, ceil_div_u(target, pl.ytiles));
     const uint32_t most = std::max<uint32_t>(1, static_cast<uint32_t>(M / step));
     const uint32_t S = std::min(want, most);
-    uint32_t rps = ceil_div_u(M, S);
-    rps = ceil_div_u(rps, step) * step;
-    pl.rps = rps;
-    pl.S = ceil_div_u(M, rps);
+    pl.rps = ceil_div_u(M, S);
+    pl.S = ceil_div_u(M, pl.rps);
     pl.cl_fast_apply = (256u % pl.ncv) == 0;
   }
   // Channel-last without the register-resident parameters falls back to one
@@ -122,7 +123,7 @@ int stats_t(const BnProblem &p, const BnPlan &pl, float *part, hipStream_t st) {
   if (pl.channel_last) {
     NBLAHIP_LAUNCH("bn_stats_cl_kernel", (bn_stats_cl_kernel<T, VEC>), dim3(pl.ytiles, pl.S), dim3(kBnBlock), 0, st,
                        x, static_cast<uint32_t>(p.size0), static_cast<uint32_t>(p.C), pl.ncv,
-                       pl.log2tx, pl.rps, part);
+                       pl.log2tx, pl.rps, 1.0f, part);
   } else {
     NBLAHIP_LAUNCH("bn_stats_planes_kernel", (bn_stats_planes_kernel<T, VEC>), dim3(static_cast<uint32_t>(p.C), pl.S),
                        dim3(kBnBlock), 0, st, x, static_cast<uint32_t>(p.C), FastDiv(pl.nvp),
@@ -138,7 +139,7 @@ int bwd_reduce_t(const BnProblem &p, const BnPlan &pl, float *part2, hipStream_t
   if (pl.channel_last) {
     NBLAHIP_LAUNCH("bn_bwd_reduce_cl_kernel", (bn_bwd_reduce_cl_kernel<T, VEC>), dim3(pl.ytiles, pl.S), dim3(kBnBlock), 0,
                        st, x, dy, p.mean, static_cast<uint32_t>(p.size0),
-                       static_cast<uint32_t>(p.C), pl.ncv, pl.log2tx, pl.rps, part2);
+                       static_cast<uint32_t>(p.C), pl.ncv, pl.log2tx, pl.rps, 1.0f, part2);
   } else {
     NBLAHIP_LAUNCH("bn_bwd_reduce_planes_kernel", (bn_bwd_reduce_planes_kernel<T, VEC>),
                        dim3(static_cast<uint32_t>(p.C), pl.S), dim3(kBnBlock), 0, st, x, dy, p.mean,

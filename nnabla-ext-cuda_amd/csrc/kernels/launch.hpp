@@ -12,7 +12,9 @@
 
 namespace nblahip {
 
-enum RowMode { kRowLN = 0, kRowIN = 1, kRowGN = 2 };
+// kRowINc: InstanceNormalization backward with a block per channel that walks
+// the batch itself, so dgamma/dbeta need no second kernel.
+enum RowMode { kRowLN = 0, kRowIN = 1, kRowGN = 2, kRowINc = 3 };
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

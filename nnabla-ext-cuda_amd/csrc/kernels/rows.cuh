@@ -46,6 +46,12 @@ struct RowArgs {
   // 1.0f delivered at run time: keeps fma(float(half), one, b) a single
   // mixed-precision instruction (see elem_fma).
   float one;
+  // Channel-per-block InstanceNormalization backward writes the parameter
+  // gradients itself.
+  float *dgamma;
+  float *dbeta;
+  int accum_g;
+  int accum_b;
   // GroupNormalization backward: entries (64*VEC-element runs) per channel and
   // channels per group.
   int epc;
@@ -62,7 +68,9 @@ template <int TPR> struct RowBlock {
 // 512-thread block (256 VGPRs per lane stay available): two blocks per CU,
 // few partials to fold afterwards.
 template <int TPR, int MODE> struct RowBwdBlock {
-  static constexpr int kBlock = (MODE == kRowLN && TPR == kWave) ? 512 : RowBlock<TPR>::kBlock;
+  static constexpr int kBlock = (MODE == kRowLN && TPR == kWave)    ? 512
+                                : (MODE == kRowINc && TPR == kWave) ? 1024
+                                                                    : RowBlock<TPR>::kBlock;
   static constexpr int kRowsPerBlock = kBlock / TPR;
 };
 
@@ -234,7 +242,19 @@ row_bwd_kernel(const RowArgs a) {
     }
   }
 
-  for (int row = blockIdx.x * RPB + sub; row < a.rows; row += gridDim.x * RPB) {
+  // Iteration space.  Every mode but kRowINc: one unit = one row, rows strided
+  // over the grid.  kRowINc: one unit = one channel (block-strided), whose
+  // batch*1 rows (n, c) are strided over the block's waves / walked in turn.
+  constexpr bool CH = (MODE == kRowINc);
+  const int channels = static_cast<int>(a.pmod);
+  const int nunits = CH ? channels : a.rows;
+  const int u0 = CH ? static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x) * RPB + sub;
+  const int ustride = CH ? static_cast<int>(gridDim.x) : static_cast<int>(gridDim.x) * RPB;
+  const int inner_n = CH ? a.rows / channels : 1;
+  for (int unit = u0; unit < nunits; unit += ustride) {
+  float ch_sdx = 0.f, ch_sdy = 0.f; // kRowINc: this wave's share of the channel sums
+  for (int rr = CH ? sub : 0; rr < inner_n; rr += CH ? RPB : 1) {
+    const int row = CH ? rr * channels + unit : unit;
     const size_t base = static_cast<size_t>(row) * a.R;
     RawVec<T, VEC> xr[NL], dr[NL];
 #pragma unroll
@@ -271,7 +291,7 @@ row_bwd_kernel(const RowArgs a) {
         }
       }
       row_sum2<TPR>(s1, t2, lds);
-    } else if constexpr (MODE == kRowIN) {
+    } else if constexpr (MODE == kRowIN || MODE == kRowINc) {
       float sdy = 0.f, sdx = 0.f;
 #pragma unroll
       for (int k = 0; k < NL; ++k) {
@@ -283,9 +303,14 @@ row_bwd_kernel(const RowArgs a) {
         }
       }
       row_sum2<TPR>(sdy, sdx, lds);
-      if (t == 0) {
-        a.ws[2 * static_cast<size_t>(row)] = sdx;
-        a.ws[2 * static_cast<size_t>(row) + 1] = sdy;
+      if constexpr (CH) {
+        ch_sdx += sdx;
+        ch_sdy += sdy;
+      } else {
+        if (t == 0) {
+          a.ws[2 * static_cast<size_t>(row)] = sdx;
+          a.ws[2 * static_cast<size_t>(row) + 1] = sdy;
+        }
       }
       const uint32_t pidx = (static_cast<uint32_t>(row) % a.pmod) * a.pmul;
       const float g = a.gamma ? a.gamma[pidx] : 1.f;
@@ -383,7 +408,31 @@ row_bwd_kernel(const RowArgs a) {
         }
       }
     }
+  } // rows of the unit
+  if constexpr (CH) {
+    // Fold the waves' shares in wave order and publish dgamma[c], dbeta[c].
+    __shared__ float chfold[2 * 16];
+    if constexpr (RPB > 1) {
+      __syncthreads();
+      if (t == 0) {
+        chfold[2 * sub] = ch_sdx;
+        chfold[2 * sub + 1] = ch_sdy;
+      }
+      __syncthreads();
+      ch_sdx = 0.f;
+      ch_sdy = 0.f;
+#pragma unroll
+      for (int w = 0; w < RPB; ++w) {
+        ch_sdx += chfold[2 * w];
+        ch_sdy += chfold[2 * w + 1];
+      }
+    }
+    if (threadIdx.x == 0) {
+      if (a.dgamma) a.dgamma[unit] = ch_sdx + (a.accum_g ? a.dgamma[unit] : 0.f);
+      if (a.dbeta) a.dbeta[unit] = ch_sdy + (a.accum_b ? a.dbeta[unit] : 0.f);
+    }
   }
+  } // units
 
   if constexpr (MODE == kRowLN) {
     // Fold the RPB waves of a block into wave 0 (fixed order), then write the

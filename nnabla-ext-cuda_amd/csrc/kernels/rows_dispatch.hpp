@@ -14,6 +14,8 @@ int run_row_bwd_cached_ln(int dtype, const RowCfg &cfg, const RowArgs &args, int
                           hipStream_t st);
 int run_row_bwd_cached_in(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
                           hipStream_t st);
+int run_row_bwd_cached_inc(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
+                           hipStream_t st);
 int run_row_bwd_cached_gn(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
                           hipStream_t st);
 

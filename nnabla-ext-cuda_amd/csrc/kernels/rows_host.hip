@@ -74,6 +74,10 @@ static RowArgs make_args(const RowProblem &p) {
   a.eps = p.eps;
   a.inv_R = 1.0f / static_cast<float>(p.R);
   a.accum_dx = p.accum_dx;
+  a.dgamma = p.dgamma;
+  a.dbeta = p.dbeta;
+  a.accum_g = p.accum_g;
+  a.accum_b = p.accum_b;
   a.one = 1.0f;
   a.epc = 0;
   a.cpg = 1;
@@ -238,6 +242,15 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
         if (int e = last_launch_status()) return e;
       }
       return 0;
+    }
+    // InstanceNormalization with parameters shared by the batch and enough
+    // channels to fill the chip: a block per channel sums over the batch
+    // itself, no second kernel.
+    if (p.mode == kRowIN && p.bc_gamma && p.bc_beta && p.batch > 1 &&
+        p.channels * 2 >= device_cus() && !(cfg.tpr == 1024 && cfg.nl == 8) &&
+        !tune_int("IN_NO_CHANNEL_BLOCKS", 0)) {
+      const int grid = static_cast<int>(std::min<int64_t>(p.channels, 1 << 20));
+      return run_row_bwd_cached_inc(p.dtype, cfg, a, grid, st);
     }
     const int grid = cached_grid(p.rows, cfg.tpr);
     const int e = p.mode == kRowIN ? run_row_bwd_cached_in(p.dtype, cfg, a, grid, st)

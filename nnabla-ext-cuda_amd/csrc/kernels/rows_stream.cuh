@@ -312,29 +312,28 @@ pair_param_reduce_kernel(const float *__restrict__ pairs, int n, int P,
                          float *__restrict__ dgamma, float *__restrict__ dbeta,
                          int bc_gamma, int bc_beta, int accum_g, int accum_b) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (dgamma) {
-    const int count = bc_gamma ? P : n * P;
-    if (i < count) {
-      float s = 0.f;
-      if (bc_gamma) {
-        for (int b = 0; b < n; ++b) s += pairs[2 * (static_cast<size_t>(b) * P + i)];
-      } else {
-        s = pairs[2 * static_cast<size_t>(i)];
+  const float2 *__restrict__ pp = reinterpret_cast<const float2 *>(pairs);
+  if (i < P) {
+    // Both batch sums in one sweep; the loads of a sweep are independent.
+    float sg = 0.f, sb = 0.f;
+    for (int b0 = 0; b0 < n; b0 += 8) {
+      float2 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        v[u] = (b0 + u < n) ? pp[static_cast<size_t>(b0 + u) * P + i] : make_float2(0.f, 0.f);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        sg += v[u].x;
+        sb += v[u].y;
       }
-      dgamma[i] = s + (accum_g ? dgamma[i] : 0.f);
     }
+    if (dgamma && bc_gamma) dgamma[i] = sg + (accum_g ? dgamma[i] : 0.f);
+    if (dbeta && bc_beta) dbeta[i] = sb + (accum_b ? dbeta[i] : 0.f);
   }
-  if (dbeta) {
-    const int count = bc_beta ? P : n * P;
-    if (i < count) {
-      float s = 0.f;
-      if (bc_beta) {
-        for (int b = 0; b < n; ++b) s += pairs[2 * (static_cast<size_t>(b) * P + i) + 1];
-      } else {
-        s = pairs[2 * static_cast<size_t>(i) + 1];
-      }
-      dbeta[i] = s + (accum_b ? dbeta[i] : 0.f);
-    }
+  if (i < n * P) { // per-sample parameters: element-wise
+    const float2 v = pp[i];
+    if (dgamma && !bc_gamma) dgamma[i] = v.x + (accum_g ? dgamma[i] : 0.f);
+    if (dbeta && !bc_beta) dbeta[i] = v.y + (accum_b ? dbeta[i] : 0.f);
   }
 }
 
