@@ -28,50 +28,137 @@ struct __align__(16) BnParam {
   float mean, a, b, c;
 };
 
+// What a channel's finished statistics turn into (shared by the finalize
+// kernel and by reduction blocks that own a whole channel):
+//   mean, var (biased) -> batch_mean/batch_var
+//   running mean/var update (unbiased N/(N-1) factor on the running variance,
+//   the reference's kernel/batch_normalization.cuh:292-302)
+//   apply parameters {mean, gamma*istd, beta}.
+struct BnFwdFinal {
+  float inv_N, unbias, decay, eps;
+  const float *gamma, *beta;
+  float *batch_mean, *batch_var, *rmean, *rvar;
+  BnParam *params;
+  __device__ __forceinline__ void publish(uint32_t c, const Welford &w) const {
+    const float mean = w.mean;
+    const float var = w.m2 * inv_N;
+    batch_mean[c] = mean;
+    batch_var[c] = var;
+    if (rmean) rmean[c] = decay * rmean[c] + (1.f - decay) * mean;
+    if (rvar) rvar[c] = decay * rvar[c] + (1.f - decay) * var * unbias;
+    BnParam q;
+    q.mean = mean;
+    q.a = (gamma ? gamma[c] : 1.f) * inv_std(var, eps);
+    q.b = beta ? beta[c] : 0.f;
+    q.c = 0.f;
+    params[c] = q;
+  }
+};
+
+// Backward counterpart.  With sdx = sum dy*(x-mean), sdy = sum dy, g = gamma,
+// i = istd (kernel/batch_normalization.cuh:425-469,522-540):
+//   dgamma = sdx*i, dbeta = sdy
+//   dvar   = -1/2 * g*sdx * i^3 + dv_in        dmean = -g*sdy*i + dm_in
+//   dx     = g*i*dy + (2*dvar/N)*(x-mean) + dmean/N
+// (the reference's dvar*(-2)*sum(x-mean)/N term vanishes identically).
+// batch_stat == 0: statistics are constants, dx = g*i*dy.
+struct BnBwdFinal {
+  float inv_N, eps;
+  int batch_stat;
+  const float *gamma, *mean, *var, *dmean_in, *dvar_in;
+  float *dgamma, *dbeta;
+  int accum_g, accum_b;
+  BnParam *params;
+  __device__ __forceinline__ void publish(uint32_t c, float sdx, float sdy) const {
+    const float istd = inv_std(var[c], eps);
+    const float g = gamma ? gamma[c] : 1.f;
+    if (dgamma) dgamma[c] = sdx * istd + (accum_g ? dgamma[c] : 0.f);
+    if (dbeta) dbeta[c] = sdy + (accum_b ? dbeta[c] : 0.f);
+    BnParam q;
+    q.mean = mean[c];
+    q.a = g * istd;
+    if (batch_stat) {
+      const float dvar = -0.5f * g * sdx * istd * istd * istd + (dvar_in ? dvar_in[c] : 0.f);
+      const float dmean = -g * sdy * istd + (dmean_in ? dmean_in[c] : 0.f);
+      q.b = 2.f * dvar * inv_N;
+      q.c = dmean * inv_N;
+    } else {
+      q.b = 0.f;
+      q.c = 0.f;
+    }
+    params[c] = q;
+  }
+};
+
+// Offset (in vectors) of vector v of channel c in the planes layout.
+__device__ __forceinline__ size_t bn_plane_offset(uint32_t v, uint32_t c, uint32_t C,
+                                                  const FastDiv &nvp) {
+  const uint32_t n = nvp.div(v);
+  const uint32_t i = v - n * nvp.d;
+  return (static_cast<size_t>(n) * C + c) * nvp.d + i;
+}
+
 // ---------------------------------------------------------------------------
 // Forward statistics, planes layout.  grid = (C, S).
 // vpc = vectors per channel = size0 * nvp; split s covers vectors
-// [s*chunk, min((s+1)*chunk, vpc)).
+// [s*chunk, min((s+1)*chunk, vpc)).  DIRECT (S == 1, BLOCK = 1024): the block
+// owns the whole channel and publishes its statistics itself; used when there
+// are enough channels to give every CU a block, which removes the partial
+// buffer and the finalize launch.  U = 16-byte loads in flight per thread.
 // ---------------------------------------------------------------------------
-template <typename T, int VEC>
-__global__ void __launch_bounds__(kBnBlock)
+template <typename T, int VEC, int BLOCK, bool DIRECT, int U>
+__global__ void __launch_bounds__(BLOCK)
 bn_stats_planes_kernel(const T *__restrict__ x, uint32_t C, FastDiv nvp, uint32_t vpc,
-                       uint32_t chunk, float *__restrict__ part /*[C][S][3]*/) {
-  __shared__ float lds[3 * (kBnBlock / kWave)];
+                       uint32_t chunk, float *__restrict__ part /*[C][S][3]*/, BnFwdFinal fin) {
+  __shared__ float lds[3 * (BLOCK / kWave)];
   const uint32_t c = blockIdx.x;
   const uint32_t s = blockIdx.y;
   const uint32_t S = gridDim.y;
   const uint32_t begin = s * chunk;
   const uint32_t end = min(begin + chunk, vpc);
   Welford w{0.f, 0.f, 0.f};
-  for (uint32_t v0 = begin + threadIdx.x; v0 < end; v0 += kBnBlock * kBnUnroll) {
-    float vals[kBnUnroll * VEC];
-    int cnt = 0;
+  uint32_t v0 = begin + threadIdx.x;
+  // full steps: every load valid, all U loads in flight together
+  for (; v0 + (U - 1) * BLOCK < end; v0 += BLOCK * U) {
+    RawVec<T, VEC> raw[U];
 #pragma unroll
-    for (int u = 0; u < kBnUnroll; ++u) {
-      const uint32_t v = v0 + u * kBnBlock;
+    for (int u = 0; u < U; ++u)
+      raw[u] = load_raw<T, VEC>(x + bn_plane_offset(v0 + u * BLOCK, c, C, nvp) * VEC);
+    float vals[U * VEC];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
       float tmp[VEC];
-      if (v < end) {
-        const uint32_t n = nvp.div(v);
-        const uint32_t i = v - n * nvp.d;
-        const size_t off = (static_cast<size_t>(n) * C + c) * nvp.d + i;
-        load_vec<T, VEC>(x + off * VEC, tmp);
-        cnt += VEC;
-      } else {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) tmp[j] = 0.f;
-      }
+      unpack<T, VEC>(raw[u], tmp);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) vals[u * VEC + j] = tmp[j];
     }
-    welford_add_chunk<kBnUnroll * VEC>(w, vals, cnt);
+    welford_add_chunk<U * VEC>(w, vals, U * VEC);
+  }
+  if (v0 < end) { // ragged last step: clamp the index, count what is real
+    float vals[U * VEC];
+    int cnt = 0;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t v = v0 + u * BLOCK;
+      const bool ok = v < end;
+      float tmp[VEC];
+      unpack<T, VEC>(load_raw<T, VEC>(x + bn_plane_offset(ok ? v : v0, c, C, nvp) * VEC), tmp);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) vals[u * VEC + j] = ok ? tmp[j] : 0.f;
+      cnt += ok ? VEC : 0;
+    }
+    welford_add_chunk<U * VEC>(w, vals, cnt);
   }
   w = block_welford(w, lds);
   if (threadIdx.x == 0) {
-    float *p = part + 3 * (static_cast<size_t>(c) * S + s);
-    p[0] = w.mean;
-    p[1] = w.m2;
-    p[2] = w.n;
+    if constexpr (DIRECT) {
+      fin.publish(c, w);
+    } else {
+      float *p = part + 3 * (static_cast<size_t>(c) * S + s);
+      p[0] = w.mean;
+      p[1] = w.m2;
+      p[2] = w.n;
+    }
   }
 }
 
@@ -220,18 +307,9 @@ bn_stats_cl_kernel(const T *__restrict__ x, uint32_t M, uint32_t C, uint32_t ncv
 
 // ---------------------------------------------------------------------------
 // Forward finalize: one block per channel merges its S partials.
-//   mean, var (biased) -> batch_mean/batch_var
-//   running mean/var update (unbiased N/(N-1) factor on the running variance,
-//   the reference's kernel/batch_normalization.cuh:292-302)
-//   apply parameters {mean, gamma*istd, beta}.
 // ---------------------------------------------------------------------------
 __global__ void __launch_bounds__(kBnBlock)
-bn_finalize_fwd_kernel(const float *__restrict__ part, uint32_t S, float inv_N,
-                       float unbias, float decay, float eps,
-                       const float *__restrict__ gamma, const float *__restrict__ beta,
-                       float *__restrict__ batch_mean, float *__restrict__ batch_var,
-                       float *__restrict__ rmean, float *__restrict__ rvar,
-                       BnParam *__restrict__ params) {
+bn_finalize_fwd_kernel(const float *__restrict__ part, uint32_t S, BnFwdFinal fin) {
   __shared__ float lds[3 * (kBnBlock / kWave)];
   const uint32_t c = blockIdx.x;
   Welford w{0.f, 0.f, 0.f};
@@ -240,20 +318,7 @@ bn_finalize_fwd_kernel(const float *__restrict__ part, uint32_t S, float inv_N,
     w = welford_merge(w, Welford{p[0], p[1], p[2]});
   }
   w = block_welford(w, lds);
-  if (threadIdx.x == 0) {
-    const float mean = w.mean;
-    const float var = w.m2 * inv_N;
-    batch_mean[c] = mean;
-    batch_var[c] = var;
-    if (rmean) rmean[c] = decay * rmean[c] + (1.f - decay) * mean;
-    if (rvar) rvar[c] = decay * rvar[c] + (1.f - decay) * var * unbias;
-    BnParam q;
-    q.mean = mean;
-    q.a = (gamma ? gamma[c] : 1.f) * inv_std(var, eps);
-    q.b = beta ? beta[c] : 0.f;
-    q.c = 0.f;
-    params[c] = q;
-  }
+  if (threadIdx.x == 0) fin.publish(c, w);
 }
 
 // Inference: apply parameters straight from the running statistics.
@@ -378,49 +443,53 @@ bn_apply_cl_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
 
 // ---------------------------------------------------------------------------
 // Backward reduction, planes layout.  part2[C][S][2] = (sum dy*(x-mean), sum dy).
+// DIRECT as in bn_stats_planes_kernel.
 // ---------------------------------------------------------------------------
-template <typename T, int VEC>
-__global__ void __launch_bounds__(kBnBlock)
+template <typename T, int VEC, int BLOCK, bool DIRECT>
+__global__ void __launch_bounds__(BLOCK)
 bn_bwd_reduce_planes_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                             const float *__restrict__ mean, uint32_t C, FastDiv nvp,
-                            uint32_t vpc, uint32_t chunk, float *__restrict__ part2) {
-  __shared__ float lds[2 * (kBnBlock / kWave)];
+                            uint32_t vpc, uint32_t chunk, float one, float *__restrict__ part2,
+                            BnBwdFinal fin) {
+  __shared__ float lds[2 * (BLOCK / kWave)];
   const uint32_t c = blockIdx.x;
   const uint32_t s = blockIdx.y;
   const uint32_t S = gridDim.y;
   const uint32_t begin = s * chunk;
   const uint32_t end = min(begin + chunk, vpc);
-  const float m = mean[c];
+  const float nm = -mean[c];
   float sdx = 0.f, sdy = 0.f;
-  for (uint32_t v0 = begin + threadIdx.x; v0 < end; v0 += kBnBlock * kBnUnroll) {
-    float xv[kBnUnroll][VEC], dv[kBnUnroll][VEC];
+  for (uint32_t v0 = begin + threadIdx.x; v0 < end; v0 += BLOCK * kBnUnroll) {
+    RawVec<T, VEC> xr[kBnUnroll], dr[kBnUnroll];
+    // all loads first (indices past the end re-read v0), selects after
 #pragma unroll
     for (int u = 0; u < kBnUnroll; ++u) {
-      const uint32_t v = v0 + u * kBnBlock;
-      if (v < end) {
-        const uint32_t n = nvp.div(v);
-        const uint32_t i = v - n * nvp.d;
-        const size_t off = ((static_cast<size_t>(n) * C + c) * nvp.d + i) * VEC;
-        load_vec<T, VEC>(x + off, xv[u]);
-        load_vec<T, VEC>(dy + off, dv[u]);
-      } else {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) xv[u][j] = dv[u][j] = 0.f;
-      }
+      const uint32_t v = v0 + u * BLOCK;
+      const size_t off = bn_plane_offset(v < end ? v : v0, c, C, nvp) * VEC;
+      xr[u] = load_raw<T, VEC>(x + off);
+      dr[u] = load_raw<T, VEC>(dy + off);
     }
 #pragma unroll
-    for (int u = 0; u < kBnUnroll; ++u)
+    for (int u = 0; u < kBnUnroll; ++u) dr[u] = raw_or_zero<T, VEC>(v0 + u * BLOCK < end, dr[u]);
+#pragma unroll
+    for (int u = 0; u < kBnUnroll; ++u) {
+      sdy = raw_sum<T, VEC>(dr[u], sdy);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        sdy += dv[u][j];
-        sdx += dv[u][j] * (xv[u][j] - m);
+        const float xc = elem_fma<T, VEC>(xr[u], j, one, nm);
+        sdx = elem_fma<T, VEC>(dr[u], j, xc, sdx);
       }
+    }
   }
   block_sum2(sdx, sdy, lds);
   if (threadIdx.x == 0) {
-    float *p = part2 + 2 * (static_cast<size_t>(c) * S + s);
-    p[0] = sdx;
-    p[1] = sdy;
+    if constexpr (DIRECT) {
+      fin.publish(c, sdx, sdy);
+    } else {
+      float *p = part2 + 2 * (static_cast<size_t>(c) * S + s);
+      p[0] = sdx;
+      p[1] = sdy;
+    }
   }
 }
 
@@ -507,22 +576,10 @@ bn_bwd_reduce_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
 }
 
 // ---------------------------------------------------------------------------
-// Backward finalize (one block per channel).  With sdx = sum dy*(x-mean),
-// sdy = sum dy, g = gamma, i = istd (kernel/batch_normalization.cuh:425-469,
-// 522-540):
-//   dgamma = sdx*i, dbeta = sdy
-//   dvar   = -1/2 * g*sdx * i^3 + dv_in        dmean = -g*sdy*i + dm_in
-//   dx     = g*i*dy + (2*dvar/N)*(x-mean) + dmean/N
-// (the reference's dvar*(-2)*sum(x-mean)/N term vanishes identically).
-// batch_stat == 0: statistics are constants, dx = g*i*dy.
+// Backward finalize (one block per channel): sums the S partial pairs.
 // ---------------------------------------------------------------------------
 __global__ void __launch_bounds__(kBnBlock)
-bn_finalize_bwd_kernel(const float *__restrict__ part2, uint32_t S, float inv_N, float eps,
-                       int batch_stat, const float *__restrict__ gamma,
-                       const float *__restrict__ mean, const float *__restrict__ var,
-                       const float *__restrict__ dmean_in, const float *__restrict__ dvar_in,
-                       float *__restrict__ dgamma, float *__restrict__ dbeta, int accum_g,
-                       int accum_b, BnParam *__restrict__ params) {
+bn_finalize_bwd_kernel(const float *__restrict__ part2, uint32_t S, BnBwdFinal fin) {
   __shared__ float lds[2 * (kBnBlock / kWave)];
   const uint32_t c = blockIdx.x;
   float sdx = 0.f, sdy = 0.f;
@@ -532,25 +589,7 @@ bn_finalize_bwd_kernel(const float *__restrict__ part2, uint32_t S, float inv_N,
     sdy += p[1];
   }
   block_sum2(sdx, sdy, lds);
-  if (threadIdx.x == 0) {
-    const float istd = inv_std(var[c], eps);
-    const float g = gamma ? gamma[c] : 1.f;
-    if (dgamma) dgamma[c] = sdx * istd + (accum_g ? dgamma[c] : 0.f);
-    if (dbeta) dbeta[c] = sdy + (accum_b ? dbeta[c] : 0.f);
-    BnParam q;
-    q.mean = mean[c];
-    q.a = g * istd;
-    if (batch_stat) {
-      const float dvar = -0.5f * g * sdx * istd * istd * istd + (dvar_in ? dvar_in[c] : 0.f);
-      const float dmean = -g * sdy * istd + (dmean_in ? dmean_in[c] : 0.f);
-      q.b = 2.f * dvar * inv_N;
-      q.c = dmean * inv_N;
-    } else {
-      q.b = 0.f;
-      q.c = 0.f;
-    }
-    params[c] = q;
-  }
+  if (threadIdx.x == 0) fin.publish(c, sdx, sdy);
 }
 
 // ---------------------------------------------------------------------------

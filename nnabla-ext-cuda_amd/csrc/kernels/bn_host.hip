@@ -23,6 +23,7 @@ struct BnPlan {
   uint32_t S = 1;       // splits
   bool cl_fast_apply = false;
   int apply_vec = 1;    // vector width of the apply kernels
+  bool direct = false;  // planes: one 1024-thread block owns a whole channel
 };
 
 uint32_t ceil_div_u(uint64_t a, uint64_t b) { return static_cast<uint32_t>((a + b - 1) / b); }
@@ -52,6 +53,16 @@ BnPlan make_plan(int64_t size0, int64_t C, int64_t size2, int dtype, bool ptr_al
     uint32_t S = std::min(want, most);
     pl.chunk = ceil_div_u(pl.vpc, S);
     pl.S = ceil_div_u(pl.vpc, pl.chunk);
+    // A whole number of channels per CU and enough work per channel: let a
+    // 1024-thread block own its channel (no partials, no finalize launch).
+    const uint32_t cus = static_cast<uint32_t>(device_cus());
+    const int direct = tune_int("BN_DIRECT", 2); // 0 never, 1 always, 2 automatic
+    const bool balanced = (static_cast<uint64_t>(C) % cus == 0) || static_cast<uint64_t>(C) >= 8ull * cus;
+    if (direct == 1 || (direct == 2 && balanced && pl.vpc >= 4u * 1024u * kBnUnroll)) {
+      pl.direct = true;
+      pl.S = 1;
+      pl.chunk = pl.vpc;
+    }
   } else {
     pl.vec = (ptr_aligned && C % full == 0) ? full : 1;
     pl.ncv = static_cast<uint32_t>(C / pl.vec);
@@ -118,32 +129,45 @@ int fwd_apply_t(const BnProblem &p, const BnPlan &pl, const BnParamSrc &src, hip
 }
 
 template <typename T, int VEC>
-int stats_t(const BnProblem &p, const BnPlan &pl, float *part, hipStream_t st) {
+int stats_t(const BnProblem &p, const BnPlan &pl, float *part, const BnFwdFinal &fin,
+            hipStream_t st) {
   const T *x = static_cast<const T *>(p.x);
   if (pl.channel_last) {
-    NBLAHIP_LAUNCH("bn_stats_cl_kernel", (bn_stats_cl_kernel<T, VEC>), dim3(pl.ytiles, pl.S), dim3(kBnBlock), 0, st,
-                       x, static_cast<uint32_t>(p.size0), static_cast<uint32_t>(p.C), pl.ncv,
-                       pl.log2tx, pl.rps, 1.0f, part);
+    NBLAHIP_LAUNCH("bn_stats_cl_kernel", (bn_stats_cl_kernel<T, VEC>), dim3(pl.ytiles, pl.S),
+                   dim3(kBnBlock), 0, st, x, static_cast<uint32_t>(p.size0),
+                   static_cast<uint32_t>(p.C), pl.ncv, pl.log2tx, pl.rps, 1.0f, part);
+  } else if (pl.direct) {
+    NBLAHIP_LAUNCH("bn_stats_planes_kernel", (bn_stats_planes_kernel<T, VEC, 1024, true, 8>),
+                   dim3(static_cast<uint32_t>(p.C), 1), dim3(1024), 0, st, x,
+                   static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, part, fin);
   } else {
-    NBLAHIP_LAUNCH("bn_stats_planes_kernel", (bn_stats_planes_kernel<T, VEC>), dim3(static_cast<uint32_t>(p.C), pl.S),
-                       dim3(kBnBlock), 0, st, x, static_cast<uint32_t>(p.C), FastDiv(pl.nvp),
-                       pl.vpc, pl.chunk, part);
+    NBLAHIP_LAUNCH("bn_stats_planes_kernel", (bn_stats_planes_kernel<T, VEC, kBnBlock, false, kBnUnroll>),
+                   dim3(static_cast<uint32_t>(p.C), pl.S), dim3(kBnBlock), 0, st, x,
+                   static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, part, fin);
   }
   return last_launch_status();
 }
 
 template <typename T, int VEC>
-int bwd_reduce_t(const BnProblem &p, const BnPlan &pl, float *part2, hipStream_t st) {
+int bwd_reduce_t(const BnProblem &p, const BnPlan &pl, float *part2, const BnBwdFinal &fin,
+                 hipStream_t st) {
   const T *x = static_cast<const T *>(p.x);
   const T *dy = static_cast<const T *>(p.dy);
   if (pl.channel_last) {
-    NBLAHIP_LAUNCH("bn_bwd_reduce_cl_kernel", (bn_bwd_reduce_cl_kernel<T, VEC>), dim3(pl.ytiles, pl.S), dim3(kBnBlock), 0,
-                       st, x, dy, p.mean, static_cast<uint32_t>(p.size0),
-                       static_cast<uint32_t>(p.C), pl.ncv, pl.log2tx, pl.rps, 1.0f, part2);
+    NBLAHIP_LAUNCH("bn_bwd_reduce_cl_kernel", (bn_bwd_reduce_cl_kernel<T, VEC>),
+                   dim3(pl.ytiles, pl.S), dim3(kBnBlock), 0, st, x, dy, p.mean,
+                   static_cast<uint32_t>(p.size0), static_cast<uint32_t>(p.C), pl.ncv, pl.log2tx,
+                   pl.rps, 1.0f, part2);
+  } else if (pl.direct) {
+    NBLAHIP_LAUNCH("bn_bwd_reduce_planes_kernel",
+                   (bn_bwd_reduce_planes_kernel<T, VEC, 1024, true>),
+                   dim3(static_cast<uint32_t>(p.C), 1), dim3(1024), 0, st, x, dy, p.mean,
+                   static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, 1.0f, part2, fin);
   } else {
-    NBLAHIP_LAUNCH("bn_bwd_reduce_planes_kernel", (bn_bwd_reduce_planes_kernel<T, VEC>),
-                       dim3(static_cast<uint32_t>(p.C), pl.S), dim3(kBnBlock), 0, st, x, dy, p.mean,
-                       static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, part2);
+    NBLAHIP_LAUNCH("bn_bwd_reduce_planes_kernel",
+                   (bn_bwd_reduce_planes_kernel<T, VEC, kBnBlock, false>),
+                   dim3(static_cast<uint32_t>(p.C), pl.S), dim3(kBnBlock), 0, st, x, dy, p.mean,
+                   static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, 1.0f, part2, fin);
   }
   return last_launch_status();
 }
@@ -183,13 +207,15 @@ int do_fwd_apply(const BnProblem &p, const BnPlan &pl, const BnParamSrc &src, hi
   BN_DISPATCH(CALL, pl.apply_vec);
 #undef CALL
 }
-int do_stats(const BnProblem &p, const BnPlan &pl, float *part, hipStream_t st) {
-#define CALL(T, V) stats_t<T, V>(p, pl, part, st)
+int do_stats(const BnProblem &p, const BnPlan &pl, float *part, const BnFwdFinal &fin,
+             hipStream_t st) {
+#define CALL(T, V) stats_t<T, V>(p, pl, part, fin, st)
   BN_DISPATCH(CALL, pl.vec);
 #undef CALL
 }
-int do_bwd_reduce(const BnProblem &p, const BnPlan &pl, float *part2, hipStream_t st) {
-#define CALL(T, V) bwd_reduce_t<T, V>(p, pl, part2, st)
+int do_bwd_reduce(const BnProblem &p, const BnPlan &pl, float *part2, const BnBwdFinal &fin,
+                  hipStream_t st) {
+#define CALL(T, V) bwd_reduce_t<T, V>(p, pl, part2, fin, st)
   BN_DISPATCH(CALL, pl.vec);
 #undef CALL
 }
@@ -229,14 +255,25 @@ int launch_bn_fwd_train(const BnProblem &p, hipStream_t st) {
   float *part = static_cast<float *>(p.ws);
   BnParam *params = reinterpret_cast<BnParam *>(static_cast<char *>(p.ws) +
                                                 part_bytes(static_cast<uint32_t>(p.C), pl.S));
-  if (int e = do_stats(p, pl, part, st)) return e;
   const double N = static_cast<double>(p.size0) * static_cast<double>(p.size2);
-  const float inv_N = static_cast<float>(1.0 / N);
-  const float unbias = static_cast<float>(N / (N - 1.0)); // inf when N == 1, as the reference
-  NBLAHIP_LAUNCH("bn_finalize_fwd_kernel", bn_finalize_fwd_kernel, dim3(static_cast<uint32_t>(p.C)), dim3(kBnBlock), 0,
-                     st, part, pl.S, inv_N, unbias, p.decay, p.eps, p.gamma, p.beta, p.batch_mean,
-                     p.batch_var, p.rmean, p.rvar, params);
-  if (int e = last_launch_status()) return e;
+  BnFwdFinal fin{};
+  fin.inv_N = static_cast<float>(1.0 / N);
+  fin.unbias = static_cast<float>(N / (N - 1.0)); // inf when N == 1, as the reference
+  fin.decay = p.decay;
+  fin.eps = p.eps;
+  fin.gamma = p.gamma;
+  fin.beta = p.beta;
+  fin.batch_mean = p.batch_mean;
+  fin.batch_var = p.batch_var;
+  fin.rmean = p.rmean;
+  fin.rvar = p.rvar;
+  fin.params = params;
+  if (int e = do_stats(p, pl, part, fin, st)) return e;
+  if (!pl.direct) {
+    NBLAHIP_LAUNCH("bn_finalize_fwd_kernel", bn_finalize_fwd_kernel,
+                   dim3(static_cast<uint32_t>(p.C)), dim3(kBnBlock), 0, st, part, pl.S, fin);
+    if (int e = last_launch_status()) return e;
+  }
   return do_fwd_apply(p, pl, param_src(params), st);
 }
 
@@ -248,17 +285,31 @@ int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
   BnParam *params = reinterpret_cast<BnParam *>(static_cast<char *>(p.ws) +
                                                 part_bytes(static_cast<uint32_t>(p.C), pl.S));
   const bool need_sums = p.dgamma || p.dbeta || (p.out && p.batch_stat);
-  if (need_sums) {
-    if (int e = do_bwd_reduce(p, pl, part2, st)) return e;
-  }
   const double N = static_cast<double>(p.size0) * static_cast<double>(p.size2);
-  // Without the reduction (inference-mode dx only) S = 0 leaves the sums at zero.
-  NBLAHIP_LAUNCH("bn_finalize_bwd_kernel", bn_finalize_bwd_kernel, dim3(static_cast<uint32_t>(p.C)), dim3(kBnBlock), 0,
-                     st, part2, need_sums ? pl.S : 0u, static_cast<float>(1.0 / N), p.eps,
-                     p.batch_stat, p.gamma, p.mean, p.var, p.dmean, p.dvar,
-                     need_sums ? p.dgamma : nullptr, need_sums ? p.dbeta : nullptr, p.accum_g,
-                     p.accum_b, params);
-  if (int e = last_launch_status()) return e;
+  BnBwdFinal fin{};
+  fin.inv_N = static_cast<float>(1.0 / N);
+  fin.eps = p.eps;
+  fin.batch_stat = p.batch_stat;
+  fin.gamma = p.gamma;
+  fin.mean = p.mean;
+  fin.var = p.var;
+  fin.dmean_in = p.dmean;
+  fin.dvar_in = p.dvar;
+  fin.dgamma = need_sums ? p.dgamma : nullptr;
+  fin.dbeta = need_sums ? p.dbeta : nullptr;
+  fin.accum_g = p.accum_g;
+  fin.accum_b = p.accum_b;
+  fin.params = params;
+  if (need_sums) {
+    if (int e = do_bwd_reduce(p, pl, part2, fin, st)) return e;
+  }
+  if (!need_sums || !pl.direct) {
+    // Without the reduction (inference-mode dx only) S = 0 leaves the sums at zero.
+    NBLAHIP_LAUNCH("bn_finalize_bwd_kernel", bn_finalize_bwd_kernel,
+                   dim3(static_cast<uint32_t>(p.C)), dim3(kBnBlock), 0, st, part2,
+                   need_sums ? pl.S : 0u, fin);
+    if (int e = last_launch_status()) return e;
+  }
   if (p.out) return do_bwd_apply(p, pl, params, st);
   return 0;
 }
