@@ -61,10 +61,10 @@ struct RowCfg {
 };
 
 // vec_ok: whether the full 16-byte vector width may be used (alignment and
-// divisibility already checked by the caller).  max_nl_1024 bounds the loads
-// per thread of the 1024-thread layout; min_tpr is 256 for the
+// divisibility already checked by the caller).  max_nl / max_nl_1024 bound the
+// loads per thread below / at 1024 threads; min_tpr is 256 for the
 // GroupNormalization backward.
-RowCfg pick_row_cfg(int dtype, int64_t R, bool vec_ok, int max_nl_1024, int min_tpr);
+RowCfg pick_row_cfg(int dtype, int64_t R, bool vec_ok, int max_nl, int max_nl_1024, int min_tpr);
 
 int launch_row_fwd(const RowProblem &p, hipStream_t st);
 int launch_row_bwd(const RowProblem &p, hipStream_t st);

@@ -27,15 +27,19 @@ int run_row_bwd_cached_gn(int dtype, const RowCfg &cfg, const RowArgs &args, int
 #define NBLAHIP_ROW_CASES(CASE, T)                          \
   NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 64)     \
   NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 256)    \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 512)    \
   NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 1024)   \
   NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 64)                     \
   NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 256)                    \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 512)                    \
   NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 1024)
 
 #define NBLAHIP_ROW_CASES_BLOCK(CASE, T)                    \
   NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 256)    \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 512)    \
   NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 1024)   \
   NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 256)                    \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 512)                    \
   NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 1024)
 
 } // namespace nblahip

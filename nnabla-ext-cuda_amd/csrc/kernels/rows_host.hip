@@ -8,18 +8,19 @@
 
 namespace nblahip {
 
-// max_nl_1024 bounds the loads per thread of the 1024-thread layout, whose
-// register budget is 128 VGPRs; the smaller layouts take up to 8.
-RowCfg pick_row_cfg(int dtype, int64_t R, bool vec_ok, int max_nl_1024, int min_tpr) {
+// max_nl bounds the loads per thread of the layouts below 1024 threads,
+// max_nl_1024 those of the 1024-thread layout, whose register budget is 128
+// VGPRs; both are chosen per kernel family so that no variant in use spills.
+RowCfg pick_row_cfg(int dtype, int64_t R, bool vec_ok, int max_nl, int max_nl_1024, int min_tpr) {
   RowCfg c;
   const int full = dtype == NBLAHIP_F16 ? 8 : 4;
   c.vec = vec_ok ? full : 1;
   const int64_t nv = R / c.vec;
-  static const int tprs[3] = {64, 256, 1024};
+  static const int tprs[4] = {64, 256, 512, 1024};
   static const int nls[4] = {1, 2, 4, 8};
   for (int tpr : tprs) {
     if (tpr < min_tpr) continue;
-    const int cap = tpr == 1024 ? max_nl_1024 : 8;
+    const int cap = tpr == 1024 ? max_nl_1024 : max_nl;
     for (int nl : nls) {
       if (nl > cap) break;
       if (static_cast<int64_t>(tpr) * nl >= nv) {
@@ -132,7 +133,8 @@ static int stream_fwd_t(const RowProblem &p, const RowArgs &a, hipStream_t st) {
 int launch_row_fwd(const RowProblem &p, hipStream_t st) {
   const bool vec_ok = row_vec_ok(p, false);
   const RowArgs a = make_args(p);
-  const RowCfg cfg = pick_row_cfg(p.dtype, p.R, vec_ok, 8, 64);
+  // LayerNormalization keeps gamma/beta of its columns in registers too.
+  const RowCfg cfg = pick_row_cfg(p.dtype, p.R, vec_ok, 8, p.mode == kRowLN ? 4 : 8, 64);
   if (cfg.ok && !tune_int("FORCE_STREAM", 0)) {
     return run_row_fwd_cached(p.dtype, cfg, a, cached_grid(p.rows, cfg.tpr), st);
   }
@@ -146,7 +148,8 @@ size_t row_bwd_workspace_bytes(int mode, int64_t rows, int64_t R, int64_t planes
   if (mode == kRowLN) {
     // Largest persistent grid over the possible thread layouts (one row per
     // block is the 256/1024-thread case).
-    const int g = std::max(ln_bwd_grid(rows, 64), std::max(ln_bwd_grid(rows, 256), ln_bwd_grid(rows, 1024)));
+    const int g = std::max(std::max(ln_bwd_grid(rows, 64), ln_bwd_grid(rows, 256)),
+                           std::max(ln_bwd_grid(rows, 512), ln_bwd_grid(rows, 1024)));
     const size_t cached = static_cast<size_t>(g) * 2 * static_cast<size_t>(R) * sizeof(float);
     const size_t stream = static_cast<size_t>(rows) * 2 * sizeof(float);
     return align_up(std::max(cached, stream), 256);
@@ -217,15 +220,18 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
   const bool vec_ok = row_vec_ok(p, true);
   RowArgs a = make_args(p);
   const int full = p.dtype == NBLAHIP_F16 ? 8 : 4;
-  // LayerNormalization also keeps per-column accumulators in registers.
-  const int nl1024 = p.mode == kRowLN ? (p.dtype == NBLAHIP_F16 ? 2 : 4) : 8;
-  RowCfg cfg = pick_row_cfg(p.dtype, p.R, vec_ok, nl1024, p.mode == kRowGN ? 256 : 64);
+  // LayerNormalization also keeps per-column accumulators, gamma and the
+  // normalised row in registers.
+  const bool ln = p.mode == kRowLN;
+  const int nl_small = ln ? 4 : 8;
+  const int nl_1024 = ln ? (p.dtype == NBLAHIP_F16 ? 1 : 2) : 8;
+  RowCfg cfg = pick_row_cfg(p.dtype, p.R, vec_ok, nl_small, nl_1024, p.mode == kRowGN ? 256 : 64);
   if (cfg.ok && p.mode == kRowGN) {
     // Every wave-wide load must fall inside one channel.
     const int64_t run = 64 * static_cast<int64_t>(cfg.vec);
     if (p.spatial % run != 0) {
       // Retry with scalar loads (run = 64 elements) before giving up.
-      cfg = pick_row_cfg(p.dtype, p.R, false, 8, 256);
+      cfg = pick_row_cfg(p.dtype, p.R, false, 8, 8, 256);
       if (cfg.ok && p.spatial % 64 != 0) cfg.ok = false;
     }
     if (cfg.ok) a.epc = static_cast<int>(p.spatial / (64 * cfg.vec));
