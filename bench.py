@@ -91,7 +91,8 @@ def make_bn(K, shape, axis, dtype, train, mean=0.0, std=1.0, outliers=False, see
 
 
 def make_rows(K, kind, shape, dtype, seed, **kw):
-    """kind in {"ln", "gn", "in"}; shape [outer..., R] for ln, [N,C,H,W] else."""
+    """kind in {"ln", "gn", "in"}; shape [outer..., R] for ln, [N,C,H,W] else
+    ([N,H,W,C] with channel_last=True)."""
     import torch
     L = K.lib()
     g = torch.Generator(device="cuda").manual_seed(seed)
@@ -123,7 +124,8 @@ def make_rows(K, kind, shape, dtype, seed, **kw):
                                      db.data_ptr(), 0, 0, 0, outer, R, 1e-5, dt, ws.data_ptr(),
                                      ws.numel(), st))
     else:
-        n, c = shape[0], shape[1]
+        cl = kw.get("channel_last", False)
+        n, c = shape[0], shape[-1] if cl else shape[1]
         sp = x.numel() // (n * c)
         gamma = torch.rand(c, device="cuda", generator=g) + 0.5
         beta = torch.randn(c, device="cuda", generator=g) * 0.1
@@ -131,7 +133,19 @@ def make_rows(K, kind, shape, dtype, seed, **kw):
         if kind == "gn":
             G = kw["groups"]
             mean, var = torch.empty(n * G, device="cuda"), torch.empty(n * G, device="cuda")
-            ws = _ws(L.nblahip_gn_bwd_workspace_bytes(n, c, sp, G, dt))
+            ws = _ws(L.nblahip_gn_cl_workspace_bytes(n, sp, c, G, dt) if cl else
+                     L.nblahip_gn_bwd_workspace_bytes(n, c, sp, G, dt))
+
+            def fwd_cl():
+                K.check(L.nblahip_gn_cl_fwd(x.data_ptr(), gamma.data_ptr(), beta.data_ptr(),
+                                            y.data_ptr(), mean.data_ptr(), var.data_ptr(), n, sp, c,
+                                            G, 1e-5, dt, ws.data_ptr(), ws.numel(), st))
+
+            def bwd_cl():
+                K.check(L.nblahip_gn_cl_bwd(x.data_ptr(), dy.data_ptr(), gamma.data_ptr(),
+                                            mean.data_ptr(), var.data_ptr(), None, None,
+                                            dx.data_ptr(), dg.data_ptr(), db.data_ptr(), 0, 0, 0, n,
+                                            sp, c, G, 1e-5, dt, ws.data_ptr(), ws.numel(), st))
 
             def fwd():
                 K.check(L.nblahip_gn_fwd(x.data_ptr(), gamma.data_ptr(), beta.data_ptr(),
@@ -145,7 +159,19 @@ def make_rows(K, kind, shape, dtype, seed, **kw):
                                          dt, ws.data_ptr(), ws.numel(), st))
         else:
             mean, var = torch.empty(n * c, device="cuda"), torch.empty(n * c, device="cuda")
-            ws = _ws(L.nblahip_in_bwd_workspace_bytes(n, c, sp, dt))
+            ws = _ws(L.nblahip_in_cl_workspace_bytes(n, sp, c, dt) if cl else
+                     L.nblahip_in_bwd_workspace_bytes(n, c, sp, dt))
+
+            def fwd_cl():
+                K.check(L.nblahip_in_cl_fwd(x.data_ptr(), gamma.data_ptr(), beta.data_ptr(),
+                                            y.data_ptr(), mean.data_ptr(), var.data_ptr(), n, sp, c,
+                                            1, 1, 1e-5, dt, ws.data_ptr(), ws.numel(), st))
+
+            def bwd_cl():
+                K.check(L.nblahip_in_cl_bwd(x.data_ptr(), dy.data_ptr(), gamma.data_ptr(),
+                                            mean.data_ptr(), var.data_ptr(), None, None,
+                                            dx.data_ptr(), dg.data_ptr(), db.data_ptr(), 0, 0, 0, n,
+                                            sp, c, 1, 1, 1e-5, dt, ws.data_ptr(), ws.numel(), st))
 
             def fwd():
                 K.check(L.nblahip_in_fwd(x.data_ptr(), gamma.data_ptr(), beta.data_ptr(),
@@ -157,6 +183,8 @@ def make_rows(K, kind, shape, dtype, seed, **kw):
                                          mean.data_ptr(), var.data_ptr(), None, None, dx.data_ptr(),
                                          dg.data_ptr(), db.data_ptr(), 0, 0, 0, n, c, sp, 1, 1,
                                          1e-5, dt, ws.data_ptr(), ws.numel(), st))
+        if cl:
+            fwd, bwd = fwd_cl, bwd_cl
     return fwd, bwd, 2 * S, 3 * S, (x, dy, gamma, beta, y, dx, mean, var, dg, db, ws)
 
 
@@ -185,6 +213,8 @@ def config_table(K, steps, warmup):
         ("C3 LN fp16 [32,512,1024]", lambda: make_rows(K, "ln", (32, 512, 1024), torch.float16, 2)),
         ("C4 GN fp16 [16,256,64,64] G=32", lambda: make_rows(K, "gn", (16, 256, 64, 64), torch.float16, 3, std=1.5, groups=32)),
         ("C4 IN fp16 [16,256,64,64]", lambda: make_rows(K, "in", (16, 256, 64, 64), torch.float16, 3, std=1.5)),
+        ("C4 GN fp16 NHWC [16,64,64,256] G=32", lambda: make_rows(K, "gn", (16, 64, 64, 256), torch.float16, 3, std=1.5, groups=32, channel_last=True)),
+        ("C4 IN fp16 NHWC [16,64,64,256]", lambda: make_rows(K, "in", (16, 64, 64, 256), torch.float16, 3, std=1.5, channel_last=True)),
         ("C5 BN training fp16 NHWC [256,56,56,64]", lambda: make_bn(K, (256, 56, 56, 64), 3, torch.float16, True, outliers=True, seed=4)),
     ]
     out = []

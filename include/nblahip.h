@@ -204,6 +204,70 @@ NBLAHIP_EXPORT int nblahip_in_bwd(const void *x, const void *dy,
                                   size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------
+ * Channel-last Group/InstanceNormalization.  x viewed as
+ * [batch, spatial, channels] (channel axis last).  The reference transposes
+ * to channel-first through ChannelFirstAdaptor before and after its kernels
+ * (group_normalization.cu:39-55, :93-106, :203-224;
+ * instance_normalization.cu:40-51, :81-94, :187-207); these entry points read
+ * and write the channel-last tensor in place of those transposes.  Results
+ * equal the channel-first entry points applied to the transposed tensor.
+ * Both directions need a workspace of *_cl_workspace_bytes; batch <= 65535.
+ * ---------------------------------------------------------------------- */
+NBLAHIP_EXPORT size_t nblahip_gn_cl_workspace_bytes(int64_t batch,
+                                                    int64_t spatial,
+                                                    int64_t channels,
+                                                    int groups, int dtype);
+
+/* Replaces convert_to_channel_first + forward_channel_first +
+ * convert_from_channel_first (group_normalization.cu:93-106). */
+NBLAHIP_EXPORT int nblahip_gn_cl_fwd(const void *x, const float *gamma,
+                                     const float *beta, void *y, float *mean,
+                                     float *var, int64_t batch, int64_t spatial,
+                                     int64_t channels, int groups, float eps,
+                                     int dtype, void *workspace,
+                                     size_t workspace_bytes, void *stream);
+
+/* Replaces the adaptor backward + backward_channel_first
+ * (group_normalization.cu:203-224). */
+NBLAHIP_EXPORT int nblahip_gn_cl_bwd(const void *x, const void *dy,
+                                     const float *gamma, const float *mean,
+                                     const float *var, const float *dmean,
+                                     const float *dvar, void *dx, float *dgamma,
+                                     float *dbeta, int accum_dx,
+                                     int accum_dgamma, int accum_dbeta,
+                                     int64_t batch, int64_t spatial,
+                                     int64_t channels, int groups, float eps,
+                                     int dtype, void *workspace,
+                                     size_t workspace_bytes, void *stream);
+
+NBLAHIP_EXPORT size_t nblahip_in_cl_workspace_bytes(int64_t batch,
+                                                    int64_t spatial,
+                                                    int64_t channels,
+                                                    int dtype);
+
+/* Replaces convert_to_channel_first + forward_channel_first +
+ * convert_from_channel_first (instance_normalization.cu:81-94). */
+NBLAHIP_EXPORT int nblahip_in_cl_fwd(const void *x, const float *gamma,
+                                     const float *beta, void *y, float *mean,
+                                     float *var, int64_t batch, int64_t spatial,
+                                     int64_t channels, int bc_gamma, int bc_beta,
+                                     float eps, int dtype, void *workspace,
+                                     size_t workspace_bytes, void *stream);
+
+/* Replaces the adaptor backward + backward_channel_first
+ * (instance_normalization.cu:187-207). */
+NBLAHIP_EXPORT int nblahip_in_cl_bwd(const void *x, const void *dy,
+                                     const float *gamma, const float *mean,
+                                     const float *var, const float *dmean,
+                                     const float *dvar, void *dx, float *dgamma,
+                                     float *dbeta, int accum_dx,
+                                     int accum_dgamma, int accum_dbeta,
+                                     int64_t batch, int64_t spatial,
+                                     int64_t channels, int bc_gamma, int bc_beta,
+                                     float eps, int dtype, void *workspace,
+                                     size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------
  * Runtime shims used by the backend's array class and singleton so that host
  * C++ never includes a HIP header.  They replace the cudaMalloc / cudaMemcpy /
  * cudaMemset / dtype-converting copy paths of src/nbla/cuda/memory/

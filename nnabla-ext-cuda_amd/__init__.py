@@ -46,6 +46,16 @@ SIGNATURES = {
     "nblahip_in_bwd_workspace_bytes": (_sz, [_i64] * 3 + [_int]),
     "nblahip_in_bwd": (_int, [_c_void_p] * 10 + [_int] * 3 + [_i64] * 3 + [_int, _int, _f, _int,
                                                                    _c_void_p, _sz, _c_void_p]),
+    "nblahip_gn_cl_workspace_bytes": (_sz, [_i64] * 3 + [_int, _int]),
+    "nblahip_gn_cl_fwd": (_int, [_c_void_p] * 6 + [_i64] * 3 + [_int, _f, _int, _c_void_p, _sz,
+                                                                _c_void_p]),
+    "nblahip_gn_cl_bwd": (_int, [_c_void_p] * 10 + [_int] * 3 + [_i64] * 3 + [_int, _f, _int,
+                                                                      _c_void_p, _sz, _c_void_p]),
+    "nblahip_in_cl_workspace_bytes": (_sz, [_i64] * 3 + [_int]),
+    "nblahip_in_cl_fwd": (_int, [_c_void_p] * 6 + [_i64] * 3 + [_int, _int, _f, _int, _c_void_p,
+                                                                _sz, _c_void_p]),
+    "nblahip_in_cl_bwd": (_int, [_c_void_p] * 10 + [_int] * 3 + [_i64] * 3 + [_int, _int, _f, _int,
+                                                                      _c_void_p, _sz, _c_void_p]),
     "nblahip_device_count": (_int, [ctypes.POINTER(_int)]),
     "nblahip_set_device": (_int, [_int]),
     "nblahip_get_device": (_int, [ctypes.POINTER(_int)]),
@@ -240,21 +250,32 @@ def ln_backward(x, dy, gamma, mean, var, outer, eps=1e-5, dmean=None, dvar=None,
     return (dx if need[0] else None, dgamma if need[1] else None, dbeta if need[2] else None)
 
 
-def _ncs(x):
-    n, c = x.shape[0], x.shape[1]
+def _ncs(x, channel_last=False):
+    """(batch, channels, spatial) of [N, C, *spatial] or, channel-last, [N, *spatial, C]."""
+    n = x.shape[0]
+    c = x.shape[-1] if channel_last else x.shape[1]
     sp = 1
-    for s in x.shape[2:]:
+    for s in (x.shape[1:-1] if channel_last else x.shape[2:]):
         sp *= s
     return n, c, sp
 
 
-def gn_forward(x, beta, gamma, num_groups, eps=1e-5):
+def gn_forward(x, beta, gamma, num_groups, eps=1e-5, channel_last=False, ws=None):
     import torch
     assert x.is_contiguous()
-    n, c, sp = _ncs(x)
+    n, c, sp = _ncs(x, channel_last)
     y = torch.empty_like(x)
     mean = torch.empty(n * num_groups, dtype=torch.float32, device=x.device)
     var = torch.empty(n * num_groups, dtype=torch.float32, device=x.device)
+    if channel_last:
+        dt = _dtype_code(x)
+        nbytes = lib().nblahip_gn_cl_workspace_bytes(n, sp, c, num_groups, dt)
+        ws = ws if ws is not None else _workspace(nbytes, x.device)
+        check(lib().nblahip_gn_cl_fwd(_ptr(x), _ptr(_f32(gamma, "gamma")),
+                                      _ptr(_f32(beta, "beta")), _ptr(y), _ptr(mean), _ptr(var),
+                                      n, sp, c, num_groups, eps, dt, _ptr(ws), ws.numel(),
+                                      _stream()))
+        return y, mean, var
     check(lib().nblahip_gn_fwd(_ptr(x), _ptr(_f32(gamma, "gamma")), _ptr(_f32(beta, "beta")),
                                _ptr(y), _ptr(mean), _ptr(var), n, c, sp, num_groups, eps,
                                _dtype_code(x), _stream()))
@@ -263,10 +284,10 @@ def gn_forward(x, beta, gamma, num_groups, eps=1e-5):
 
 def gn_backward(x, dy, gamma, mean, var, num_groups, eps=1e-5, dmean=None, dvar=None, dx=None,
                 dgamma=None, dbeta=None, accum=(False, False, False), need=(True, True, True),
-                ws=None):
+                ws=None, channel_last=False):
     import torch
     assert x.is_contiguous() and dy.is_contiguous()
-    n, c, sp = _ncs(x)
+    n, c, sp = _ncs(x, channel_last)
     dt = _dtype_code(x)
     if need[0] and dx is None:
         dx = torch.empty_like(x)
@@ -274,6 +295,15 @@ def gn_backward(x, dy, gamma, mean, var, num_groups, eps=1e-5, dmean=None, dvar=
         dgamma = torch.empty(c, dtype=torch.float32, device=x.device)
     if need[2] and dbeta is None:
         dbeta = torch.empty(c, dtype=torch.float32, device=x.device)
+    if channel_last:
+        nbytes = lib().nblahip_gn_cl_workspace_bytes(n, sp, c, num_groups, dt)
+        ws = ws if ws is not None else _workspace(nbytes, x.device)
+        check(lib().nblahip_gn_cl_bwd(
+            _ptr(x), _ptr(dy), _ptr(_f32(gamma, "gamma")), _ptr(mean), _ptr(var), _ptr(dmean),
+            _ptr(dvar), _ptr(dx if need[0] else None), _ptr(dgamma if need[1] else None),
+            _ptr(dbeta if need[2] else None), int(accum[0]), int(accum[1]), int(accum[2]), n, sp, c,
+            num_groups, eps, dt, _ptr(ws), ws.numel(), _stream()))
+        return (dx if need[0] else None, dgamma if need[1] else None, dbeta if need[2] else None)
     nbytes = lib().nblahip_gn_bwd_workspace_bytes(n, c, sp, num_groups, dt)
     ws = ws if ws is not None else _workspace(nbytes, x.device)
     check(lib().nblahip_gn_bwd(_ptr(x), _ptr(dy), _ptr(_f32(gamma, "gamma")), _ptr(mean), _ptr(var),
@@ -284,13 +314,23 @@ def gn_backward(x, dy, gamma, mean, var, num_groups, eps=1e-5, dmean=None, dvar=
     return (dx if need[0] else None, dgamma if need[1] else None, dbeta if need[2] else None)
 
 
-def in_forward(x, beta, gamma, eps=1e-5, bc_gamma=True, bc_beta=True):
+def in_forward(x, beta, gamma, eps=1e-5, bc_gamma=True, bc_beta=True, channel_last=False,
+               ws=None):
     import torch
     assert x.is_contiguous()
-    n, c, sp = _ncs(x)
+    n, c, sp = _ncs(x, channel_last)
     y = torch.empty_like(x)
     mean = torch.empty(n * c, dtype=torch.float32, device=x.device)
     var = torch.empty(n * c, dtype=torch.float32, device=x.device)
+    if channel_last:
+        dt = _dtype_code(x)
+        nbytes = lib().nblahip_in_cl_workspace_bytes(n, sp, c, dt)
+        ws = ws if ws is not None else _workspace(nbytes, x.device)
+        check(lib().nblahip_in_cl_fwd(_ptr(x), _ptr(_f32(gamma, "gamma")),
+                                      _ptr(_f32(beta, "beta")), _ptr(y), _ptr(mean), _ptr(var),
+                                      n, sp, c, int(bc_gamma), int(bc_beta), eps, dt, _ptr(ws),
+                                      ws.numel(), _stream()))
+        return y, mean, var
     check(lib().nblahip_in_fwd(_ptr(x), _ptr(_f32(gamma, "gamma")), _ptr(_f32(beta, "beta")),
                                _ptr(y), _ptr(mean), _ptr(var), n, c, sp, int(bc_gamma),
                                int(bc_beta), eps, _dtype_code(x), _stream()))
@@ -299,10 +339,10 @@ def in_forward(x, beta, gamma, eps=1e-5, bc_gamma=True, bc_beta=True):
 
 def in_backward(x, dy, gamma, mean, var, eps=1e-5, bc_gamma=True, bc_beta=True, dmean=None,
                 dvar=None, dx=None, dgamma=None, dbeta=None, accum=(False, False, False),
-                need=(True, True, True), ws=None):
+                need=(True, True, True), ws=None, channel_last=False):
     import torch
     assert x.is_contiguous() and dy.is_contiguous()
-    n, c, sp = _ncs(x)
+    n, c, sp = _ncs(x, channel_last)
     dt = _dtype_code(x)
     if need[0] and dx is None:
         dx = torch.empty_like(x)
@@ -310,6 +350,15 @@ def in_backward(x, dy, gamma, mean, var, eps=1e-5, bc_gamma=True, bc_beta=True, 
         dgamma = torch.empty(c if bc_gamma else n * c, dtype=torch.float32, device=x.device)
     if need[2] and dbeta is None:
         dbeta = torch.empty(c if bc_beta else n * c, dtype=torch.float32, device=x.device)
+    if channel_last:
+        nbytes = lib().nblahip_in_cl_workspace_bytes(n, sp, c, dt)
+        ws = ws if ws is not None else _workspace(nbytes, x.device)
+        check(lib().nblahip_in_cl_bwd(
+            _ptr(x), _ptr(dy), _ptr(_f32(gamma, "gamma")), _ptr(mean), _ptr(var), _ptr(dmean),
+            _ptr(dvar), _ptr(dx if need[0] else None), _ptr(dgamma if need[1] else None),
+            _ptr(dbeta if need[2] else None), int(accum[0]), int(accum[1]), int(accum[2]), n, sp, c,
+            int(bc_gamma), int(bc_beta), eps, dt, _ptr(ws), ws.numel(), _stream()))
+        return (dx if need[0] else None, dgamma if need[1] else None, dbeta if need[2] else None)
     nbytes = lib().nblahip_in_bwd_workspace_bytes(n, c, sp, dt)
     ws = ws if ws is not None else _workspace(nbytes, x.device)
     check(lib().nblahip_in_bwd(_ptr(x), _ptr(dy), _ptr(_f32(gamma, "gamma")), _ptr(mean), _ptr(var),

@@ -27,7 +27,7 @@ public:
 
 protected:
   // y like x; with three outputs, mean and var have x's rank with the channel
-  // axis holding num_groups and every later axis 1.
+  // axis holding num_groups and every axis that is neither batch nor channel 1.
   void setup_shapes(const Variables &inputs, const Variables &outputs) {
     const size_t n_in = 1 + (no_bias_ ? 0 : 1) + (no_scale_ ? 0 : 1);
     NBLA_CHECK(inputs.size() == n_in, error_code::value,
@@ -54,8 +54,11 @@ protected:
     outputs[0]->reshape(shape, true);
     if (outputs.size() == 3) {
       Shape_t stat_shape = shape;
+      for (int i = 0; i < ndim; ++i) {
+        const bool is_batch = std::find(batch_axis_.begin(), batch_axis_.end(), i) != batch_axis_.end();
+        if (!is_batch) stat_shape[i] = 1;
+      }
       stat_shape[channel_axis_] = num_groups_;
-      for (int i = channel_axis_ + 1; i < ndim; ++i) stat_shape[i] = 1;
       outputs[1]->reshape(stat_shape, true);
       outputs[2]->reshape(stat_shape, true);
     }

@@ -13,6 +13,7 @@ template <typename T> class InstanceNormalizationHip : public InstanceNormalizat
 protected:
   int device_;
   Size_t batch_size_ = 0, channel_size_ = 0, spatial_size_ = 0;
+  bool channel_last_ = false; // x is [batch..., spatial..., channel]
   Variable mean_, var_;   // float32 per-(n, c) statistics kept for backward
   Variable workspace_;
   size_t workspace_bytes_ = 0;

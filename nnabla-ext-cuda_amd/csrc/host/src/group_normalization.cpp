@@ -11,24 +11,33 @@ void GroupNormalizationHip<T>::setup_impl(const Variables &inputs, const Variabl
   hip_set_device(this->device_);
   const auto x = inputs[0];
   const int c = this->channel_axis_;
-  // Channel-first only: the channel axis follows the (leading) batch axes.
-  // The reference transposes any other layout through the core's
-  // ChannelFirstAdaptor (group_normalization.cu:40-55); that adaptor is not
-  // part of this backend.
-  bool channel_first = c == static_cast<int>(this->batch_axis_.size());
-  for (int b : this->batch_axis_) channel_first = channel_first && b < c;
-  NBLA_CHECK(channel_first, error_code::not_implemented,
-             "GroupNormalizationHip supports channel-first layouts only "
-             "(batch axes leading, channel_axis right after them).");
+  // Two layouts run without a transpose: channel-first (the channel axis
+  // right after the leading batch axes) and channel-last (batch axes leading,
+  // channel axis last).  The reference brings every other layout to
+  // channel-first through the core's ChannelFirstAdaptor
+  // (group_normalization.cu:40-55); that adaptor is not part of this backend.
+  const int nb = static_cast<int>(this->batch_axis_.size());
+  const int ndim = static_cast<int>(x->shape().size());
+  bool batch_leading = true;
+  for (int b : this->batch_axis_) batch_leading = batch_leading && b < nb;
+  const bool channel_first = batch_leading && c == nb;
+  channel_last_ = batch_leading && !channel_first && c == ndim - 1;
+  NBLA_CHECK(channel_first || channel_last_, error_code::not_implemented,
+             "GroupNormalizationHip supports batch axes leading with the channel axis right "
+             "after them (channel-first) or last (channel-last).");
   channel_size_ = x->shape()[c];
-  batch_size_ = x->size() / x->size(c);
-  spatial_size_ = x->size(c + 1);
+  batch_size_ = 1;
+  for (int b : this->batch_axis_) batch_size_ *= x->shape()[b];
+  spatial_size_ = batch_size_ * channel_size_ ? x->size() / (batch_size_ * channel_size_) : 0;
   NBLA_CHECK(x->size() < (Size_t(1) << 31), error_code::value,
              "GroupNormalizationHip indexes with 32 bits: fewer than 2^31 elements required.");
   mean_.reshape(Shape_t{batch_size_ * this->num_groups_}, true);
   var_.reshape(Shape_t{batch_size_ * this->num_groups_}, true);
-  workspace_bytes_ = nblahip_gn_bwd_workspace_bytes(batch_size_, channel_size_, spatial_size_,
-                                                    this->num_groups_, HipDtype<T>::code);
+  workspace_bytes_ =
+      channel_last_ ? nblahip_gn_cl_workspace_bytes(batch_size_, spatial_size_, channel_size_,
+                                                    this->num_groups_, HipDtype<T>::code)
+                    : nblahip_gn_bwd_workspace_bytes(batch_size_, channel_size_, spatial_size_,
+                                                     this->num_groups_, HipDtype<T>::code);
   workspace_.reshape(Shape_t{static_cast<Size_t>((workspace_bytes_ + 3) / 4)}, true);
 }
 
@@ -51,6 +60,14 @@ void GroupNormalizationHip<T>::forward_impl(const Variables &inputs, const Varia
   T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
   float *mean = v_mean->cast_data_and_get_pointer<float>(this->ctx_, true);
   float *var = v_var->cast_data_and_get_pointer<float>(this->ctx_, true);
+  if (channel_last_) {
+    float *ws = workspace_.cast_data_and_get_pointer<float>(this->ctx_, true);
+    NBLA_HIP_CHECK(nblahip_gn_cl_fwd(x, gamma, beta, y, mean, var, batch_size_, spatial_size_,
+                                     channel_size_, this->num_groups_, this->eps_,
+                                     HipDtype<T>::code, ws, workspace_bytes_, nullptr));
+    workspace_.data()->array()->clear();
+    return;
+  }
   NBLA_HIP_CHECK(nblahip_gn_fwd(x, gamma, beta, y, mean, var, batch_size_, channel_size_,
                                 spatial_size_, this->num_groups_, this->eps_, HipDtype<T>::code,
                                 nullptr));
@@ -91,11 +108,19 @@ void GroupNormalizationHip<T>::backward_impl(const Variables &inputs, const Vari
                             : inputs[gamma_idx]->template cast_grad_and_get_pointer<float>(
                                   this->ctx_, !accum[gamma_idx]);
   float *ws = workspace_.cast_data_and_get_pointer<float>(this->ctx_, true);
-  NBLA_HIP_CHECK(nblahip_gn_bwd(x, dy, gamma, mean, var, dmean, dvar, dx, dgamma, dbeta,
-                                pd_x && accum[0], pd_gamma && accum[gamma_idx],
-                                pd_beta && accum[beta_idx], batch_size_, channel_size_,
-                                spatial_size_, this->num_groups_, this->eps_, HipDtype<T>::code, ws,
-                                workspace_bytes_, nullptr));
+  if (channel_last_) {
+    NBLA_HIP_CHECK(nblahip_gn_cl_bwd(x, dy, gamma, mean, var, dmean, dvar, dx, dgamma, dbeta,
+                                     pd_x && accum[0], pd_gamma && accum[gamma_idx],
+                                     pd_beta && accum[beta_idx], batch_size_, spatial_size_,
+                                     channel_size_, this->num_groups_, this->eps_,
+                                     HipDtype<T>::code, ws, workspace_bytes_, nullptr));
+  } else {
+    NBLA_HIP_CHECK(nblahip_gn_bwd(x, dy, gamma, mean, var, dmean, dvar, dx, dgamma, dbeta,
+                                  pd_x && accum[0], pd_gamma && accum[gamma_idx],
+                                  pd_beta && accum[beta_idx], batch_size_, channel_size_,
+                                  spatial_size_, this->num_groups_, this->eps_, HipDtype<T>::code,
+                                  ws, workspace_bytes_, nullptr));
+  }
   workspace_.data()->array()->clear();
 }
 

@@ -345,4 +345,139 @@ int nblahip_in_bwd(const void *x, const void *dy, const float *gamma, const floa
   return launch_row_bwd(p, as_stream(stream));
 }
 
+// ---------------------------------------------------------------------------
+// Channel-last Group/InstanceNormalization: x is [batch, spatial, channels].
+// ---------------------------------------------------------------------------
+namespace {
+// 0: run; >0: nothing to do; <0: error.
+int cl_problem(ClProblem &p, int64_t batch, int64_t spatial, int64_t channels, int groups,
+               int dtype) {
+  if (!dtype_ok(dtype) || groups <= 0) return NBLAHIP_EINVAL;
+  const int d = check_dims3(batch, spatial, channels);
+  if (d) return d;
+  if (channels % groups != 0) return NBLAHIP_EINVAL;
+  if (batch > 65535) return NBLAHIP_ERANGE; // one slab per grid y/z index
+  p.dtype = dtype;
+  p.batch = batch;
+  p.spatial = spatial;
+  p.channels = channels;
+  p.groups = groups;
+  return 0;
+}
+
+int cl_fwd(ClProblem &p, const void *x, const float *gamma, const float *beta, void *y,
+           float *mean, float *var, float eps, void *workspace, size_t workspace_bytes,
+           void *stream) {
+  if (!x || !y || !mean || !var) return NBLAHIP_EINVAL;
+  if (int e = check_ws(workspace, workspace_bytes,
+                       cl_workspace_bytes(p.batch, p.spatial, p.channels, p.dtype)))
+    return e;
+  p.x = x;
+  p.out = y;
+  p.gamma = gamma;
+  p.beta = beta;
+  p.mean = mean;
+  p.var = var;
+  p.eps = eps;
+  p.ws = workspace;
+  p.ws_bytes = workspace_bytes;
+  return launch_cl_fwd(p, as_stream(stream));
+}
+
+int cl_bwd(ClProblem &p, const void *x, const void *dy, const float *gamma, const float *mean,
+           const float *var, const float *dmean, const float *dvar, void *dx, float *dgamma,
+           float *dbeta, int accum_dx, int accum_dgamma, int accum_dbeta, float eps,
+           void *workspace, size_t workspace_bytes, void *stream) {
+  if (!x || !dy || !mean || !var) return NBLAHIP_EINVAL;
+  if (int e = check_ws(workspace, workspace_bytes,
+                       cl_workspace_bytes(p.batch, p.spatial, p.channels, p.dtype)))
+    return e;
+  p.x = x;
+  p.dy = dy;
+  p.out = dx;
+  p.gamma = gamma;
+  p.mean = const_cast<float *>(mean);
+  p.var = const_cast<float *>(var);
+  p.dmean = dmean;
+  p.dvar = dvar;
+  p.dgamma = dgamma;
+  p.dbeta = dbeta;
+  p.accum_dx = accum_dx;
+  p.accum_g = accum_dgamma;
+  p.accum_b = accum_dbeta;
+  p.eps = eps;
+  p.ws = workspace;
+  p.ws_bytes = workspace_bytes;
+  return launch_cl_bwd(p, as_stream(stream));
+}
+} // namespace
+
+size_t nblahip_gn_cl_workspace_bytes(int64_t batch, int64_t spatial, int64_t channels, int groups,
+                                     int dtype) {
+  ClProblem p;
+  if (cl_problem(p, batch, spatial, channels, groups, dtype) != 0) return 0;
+  return cl_workspace_bytes(batch, spatial, channels, dtype);
+}
+
+int nblahip_gn_cl_fwd(const void *x, const float *gamma, const float *beta, void *y, float *mean,
+                      float *var, int64_t batch, int64_t spatial, int64_t channels, int groups,
+                      float eps, int dtype, void *workspace, size_t workspace_bytes,
+                      void *stream) {
+  ClProblem p;
+  const int d = cl_problem(p, batch, spatial, channels, groups, dtype);
+  if (d) return d < 0 ? d : 0;
+  return cl_fwd(p, x, gamma, beta, y, mean, var, eps, workspace, workspace_bytes, stream);
+}
+
+int nblahip_gn_cl_bwd(const void *x, const void *dy, const float *gamma, const float *mean,
+                      const float *var, const float *dmean, const float *dvar, void *dx,
+                      float *dgamma, float *dbeta, int accum_dx, int accum_dgamma,
+                      int accum_dbeta, int64_t batch, int64_t spatial, int64_t channels,
+                      int groups, float eps, int dtype, void *workspace, size_t workspace_bytes,
+                      void *stream) {
+  ClProblem p;
+  const int d = cl_problem(p, batch, spatial, channels, groups, dtype);
+  if (d) return d < 0 ? d : 0;
+  return cl_bwd(p, x, dy, gamma, mean, var, dmean, dvar, dx, dgamma, dbeta, accum_dx,
+                accum_dgamma, accum_dbeta, eps, workspace, workspace_bytes, stream);
+}
+
+size_t nblahip_in_cl_workspace_bytes(int64_t batch, int64_t spatial, int64_t channels,
+                                     int dtype) {
+  ClProblem p;
+  if (cl_problem(p, batch, spatial, channels, static_cast<int>(std::max<int64_t>(channels, 1)),
+                 dtype) != 0)
+    return 0;
+  return cl_workspace_bytes(batch, spatial, channels, dtype);
+}
+
+int nblahip_in_cl_fwd(const void *x, const float *gamma, const float *beta, void *y, float *mean,
+                      float *var, int64_t batch, int64_t spatial, int64_t channels, int bc_gamma,
+                      int bc_beta, float eps, int dtype, void *workspace, size_t workspace_bytes,
+                      void *stream) {
+  ClProblem p;
+  const int d = cl_problem(p, batch, spatial, channels,
+                           static_cast<int>(std::max<int64_t>(channels, 1)), dtype);
+  if (d) return d < 0 ? d : 0;
+  p.bc_gamma = bc_gamma;
+  p.bc_beta = bc_beta;
+  return cl_fwd(p, x, gamma, beta, y, mean, var, eps, workspace, workspace_bytes, stream);
+}
+
+int nblahip_in_cl_bwd(const void *x, const void *dy, const float *gamma, const float *mean,
+                      const float *var, const float *dmean, const float *dvar, void *dx,
+                      float *dgamma, float *dbeta, int accum_dx, int accum_dgamma,
+                      int accum_dbeta, int64_t batch, int64_t spatial, int64_t channels,
+                      int bc_gamma, int bc_beta, float eps, int dtype, void *workspace,
+                      size_t workspace_bytes, void *stream) {
+  ClProblem p;
+  const int d = cl_problem(p, batch, spatial, channels,
+                           static_cast<int>(std::max<int64_t>(channels, 1)), dtype);
+  if (d) return d < 0 ? d : 0;
+  p.bc_gamma = bc_gamma;
+  p.bc_beta = bc_beta;
+  return cl_bwd(p, x, dy, gamma, mean, var, dmean, dvar, dx, dgamma, dbeta, accum_dx,
+                accum_dgamma, accum_dbeta, eps, workspace, workspace_bytes, stream);
+}
+
 } // extern "C"

@@ -218,6 +218,10 @@ bn_stats_cl_kernel(const T *__restrict__ x, uint32_t M, uint32_t C, uint32_t ncv
   const uint32_t s = blockIdx.y;
   const uint32_t rbegin = s * rps;
   const uint32_t rend = min(rbegin + rps, M);
+  // blockIdx.z: independent [M, C] slabs (the samples of a channel-last
+  // Group/InstanceNormalization); BatchNormalization launches one slab.
+  x += static_cast<size_t>(blockIdx.z) * M * C;
+  part += static_cast<size_t>(blockIdx.z) * C * S * 3;
 
   float mean[VEC], m2[VEC];
 #pragma unroll
@@ -403,6 +407,10 @@ template <typename T, int VEC>
 __global__ void __launch_bounds__(256)
 bn_apply_cl_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
                    uint32_t ncv, uint32_t total_vec) {
+  // blockIdx.y: slab (sample) index; each slab has its own ncv*VEC parameters.
+  x += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
+  y += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
+  if (src.params) src.params += static_cast<size_t>(blockIdx.y) * ncv * VEC;
   const uint32_t cv = threadIdx.x % ncv;
   // y = x*pa + ps with ps = pb - mean*pa for half output (one mixed fma per
   // element); the centred form (x-mean)*pa + pb for float output.
@@ -501,7 +509,8 @@ __global__ void __launch_bounds__(kBnBlock)
 bn_bwd_reduce_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                         const float *__restrict__ mean, uint32_t M, uint32_t C,
                         uint32_t ncv, uint32_t log2tx, uint32_t rps, float one,
-                        float *__restrict__ part2 /*[C][S][2]*/) {
+                        float *__restrict__ part2 /*[C][S][2]*/, uint32_t mean_slab_stride,
+                        FastDiv cpg) {
   __shared__ float lsdx[kBnBlock * VEC];
   __shared__ float lsdy[kBnBlock * VEC];
   const uint32_t TX = 1u << log2tx;
@@ -518,10 +527,17 @@ bn_bwd_reduce_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
   float sdx[VEC], sdy[VEC], nm[VEC];
   {
     // Clamped index instead of a branch: one vector load of the VEC means.
+    // Mean of channel c in slab z: mean[z*mean_slab_stride + c/cpg]
+    // (BatchNormalization: stride 0, cpg 1; GroupNormalization: stride G,
+    // cpg channels per group).
+    x += static_cast<size_t>(blockIdx.z) * M * C;
+    dy += static_cast<size_t>(blockIdx.z) * M * C;
+    part2 += static_cast<size_t>(blockIdx.z) * C * gridDim.y * 2;
+    mean += static_cast<size_t>(blockIdx.z) * mean_slab_stride;
     float mv[VEC];
     const uint32_t cvc = active ? cv : 0u;
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) mv[j] = mean[cvc * VEC + j];
+    for (int j = 0; j < VEC; ++j) mv[j] = mean[cpg.div(cvc * VEC + j)];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
       sdx[j] = sdy[j] = 0.f;
@@ -640,6 +656,10 @@ bn_bwd_apply_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                        T *__restrict__ dx, const BnParam *__restrict__ params,
                        uint32_t ncv, uint32_t total_vec, int accum) {
   constexpr int U = 2;
+  x += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
+  dy += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
+  dx += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
+  params += static_cast<size_t>(blockIdx.y) * ncv * VEC;
   const uint32_t cv = threadIdx.x % ncv;
   // dx = pa*dy + pb*(x - mean) + pc = pa*dy + (pb*x + ps), ps = pc - pb*mean:
   // pb*(x-mean) is the small curvature term, so folding the mean costs nothing
@@ -678,6 +698,161 @@ bn_bwd_apply_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
         store_vec<T, VEC>(dx + static_cast<size_t>(i) * VEC, o);
       }
     }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Channel-last Group/InstanceNormalization on the BatchNormalization
+// channel-last machinery: x is N slabs [S, C]; the split reductions above
+// leave partials per (n, c, split).  One block per (n, group) merges the
+// partials of the group's cpg channels (cpg = 1: InstanceNormalization) and
+// publishes mean/var of the group plus the apply parameters of its channels.
+//   gamma/beta index of channel c in sample n: gmod == 0 ? n*C + c : c
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(kBnBlock)
+gn_cl_finalize_fwd_kernel(const float *__restrict__ part, uint32_t S, uint32_t C, uint32_t cpg,
+                          float inv_R, float eps, const float *__restrict__ gamma,
+                          const float *__restrict__ beta, uint32_t gmod, uint32_t bmod,
+                          float *__restrict__ mean, float *__restrict__ var,
+                          BnParam *__restrict__ params) {
+  __shared__ float lds[3 * (kBnBlock / kWave)];
+  const uint32_t G = C / cpg;
+  const uint32_t n = blockIdx.x / G, g = blockIdx.x % G;
+  const float *p0 = part + 3 * (static_cast<size_t>(n) * C + static_cast<size_t>(g) * cpg) * S;
+  Welford w{0.f, 0.f, 0.f};
+  for (uint32_t i = threadIdx.x; i < cpg * S; i += kBnBlock) { // (channel, split) pairs, contiguous
+    const float *p = p0 + 3 * static_cast<size_t>(i);
+    w = welford_merge(w, Welford{p[0], p[1], p[2]});
+  }
+  w = block_welford(w, lds);
+  const float m = w.mean;
+  const float v = w.m2 * inv_R;
+  const float istd = inv_std(v, eps);
+  if (threadIdx.x == 0) {
+    mean[blockIdx.x] = m;
+    var[blockIdx.x] = v;
+  }
+  for (uint32_t cl = threadIdx.x; cl < cpg; cl += kBnBlock) {
+    const uint32_t c = g * cpg + cl;
+    const uint32_t nc = n * C + c;
+    BnParam q;
+    q.mean = m;
+    q.a = (gamma ? gamma[gmod ? c : nc] : 1.f) * istd;
+    q.b = beta ? beta[bmod ? c : nc] : 0.f;
+    q.c = 0.f;
+    params[nc] = q;
+  }
+}
+
+// Backward: per (n, group) s1 = sum_c gamma_c*sdy_c, t2 = sum_c gamma_c*sdx_c
+// with sdx_c = sum dy*(x-mean) over the channel (kernel/group_normalization.cuh
+// :98-149 on centred sums), then per channel
+//   dx = gamma_c*istd*dy + f1*(x-mean) + f2',  f1 = -t2*istd^3/R + 2*dvar/R,
+//   f2' = -s1*istd/R + dmean/R
+// and the pair (sdx_c*istd, sdy_c) for the batch sum of dgamma/dbeta.
+__global__ void __launch_bounds__(kBnBlock)
+gn_cl_finalize_bwd_kernel(const float *__restrict__ part2, uint32_t S, uint32_t C, uint32_t cpg,
+                          float inv_R, float eps, const float *__restrict__ gamma, uint32_t gmod,
+                          const float *__restrict__ mean, const float *__restrict__ var,
+                          const float *__restrict__ dmean, const float *__restrict__ dvar,
+                          float *__restrict__ pairs, BnParam *__restrict__ params) {
+  __shared__ float lds[2 * (kBnBlock / kWave)];
+  const uint32_t G = C / cpg;
+  const uint32_t n = blockIdx.x / G, g = blockIdx.x % G;
+  const float m = mean[blockIdx.x];
+  const float istd = inv_std(var[blockIdx.x], eps);
+  // Pass 1: channel sums over the splits, s1/t2 over the group.
+  float s1 = 0.f, t2 = 0.f;
+  for (uint32_t cl = threadIdx.x; cl < cpg; cl += kBnBlock) {
+    const uint32_t c = g * cpg + cl;
+    const uint32_t nc = n * C + c;
+    const float *p = part2 + 2 * static_cast<size_t>(nc) * S;
+    float sdx = 0.f, sdy = 0.f;
+    for (uint32_t s = 0; s < S; ++s) {
+      sdx += p[2 * s];
+      sdy += p[2 * s + 1];
+    }
+    pairs[2 * static_cast<size_t>(nc)] = sdx * istd;
+    pairs[2 * static_cast<size_t>(nc) + 1] = sdy;
+    const float gm = gamma ? gamma[gmod ? c : nc] : 1.f;
+    s1 += gm * sdy;
+    t2 += gm * sdx;
+  }
+  block_sum2(s1, t2, lds);
+  const float f1 = -t2 * istd * istd * istd * inv_R + (dvar ? 2.f * dvar[blockIdx.x] * inv_R : 0.f);
+  const float f2 = -s1 * istd * inv_R + (dmean ? dmean[blockIdx.x] * inv_R : 0.f);
+  for (uint32_t cl = threadIdx.x; cl < cpg; cl += kBnBlock) {
+    const uint32_t c = g * cpg + cl;
+    const uint32_t nc = n * C + c;
+    BnParam q;
+    q.mean = m;
+    q.a = (gamma ? gamma[gmod ? c : nc] : 1.f) * istd;
+    q.b = f1;
+    q.c = f2;
+    params[nc] = q;
+  }
+}
+
+// Generic (scalar) apply steps for channel-last slabs whose channel count
+// does not fit the register-resident parameter layout: element i of the whole
+// tensor belongs to slab i / slab_elems and channel i % C.
+template <typename T>
+__global__ void __launch_bounds__(256)
+cl_slab_apply_kernel(const T *__restrict__ x, T *__restrict__ y,
+                     const BnParam *__restrict__ params, FastDiv slab_elems, FastDiv cdiv,
+                     uint32_t total) {
+  for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
+    const uint32_t n = slab_elems.div(i);
+    const uint32_t c = i - cdiv.div(i) * cdiv.d;
+    const BnParam q = params[n * cdiv.d + c];
+    y[i] = from_f32<T>((to_f32<T>(x[i]) - q.mean) * q.a + q.b);
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+cl_slab_bwd_apply_kernel(const T *__restrict__ x, const T *__restrict__ dy, T *__restrict__ dx,
+                         const BnParam *__restrict__ params, FastDiv slab_elems, FastDiv cdiv,
+                         uint32_t total, int accum) {
+  for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
+    const uint32_t n = slab_elems.div(i);
+    const uint32_t c = i - cdiv.div(i) * cdiv.d;
+    const BnParam q = params[n * cdiv.d + c];
+    float o = q.a * to_f32<T>(dy[i]) + q.b * (to_f32<T>(x[i]) - q.mean) + q.c;
+    if (accum) o += to_f32<T>(dx[i]);
+    dx[i] = from_f32<T>(o);
+  }
+}
+
+// Batch sum of per-(n, c) pairs (dgamma part, dbeta part) for the channel-last
+// Group/InstanceNormalization backward; element-wise when a parameter is per
+// sample.
+__global__ void __launch_bounds__(256)
+cl_pair_param_reduce_kernel(const float *__restrict__ pairs, int n, int P,
+                            float *__restrict__ dgamma, float *__restrict__ dbeta, int bc_gamma,
+                            int bc_beta, int accum_g, int accum_b) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  const float2 *__restrict__ pp = reinterpret_cast<const float2 *>(pairs);
+  if (i < P) {
+    float sg = 0.f, sb = 0.f;
+    for (int b0 = 0; b0 < n; b0 += 8) {
+      float2 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        v[u] = (b0 + u < n) ? pp[static_cast<size_t>(b0 + u) * P + i] : make_float2(0.f, 0.f);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        sg += v[u].x;
+        sb += v[u].y;
+      }
+    }
+    if (dgamma && bc_gamma) dgamma[i] = sg + (accum_g ? dgamma[i] : 0.f);
+    if (dbeta && bc_beta) dbeta[i] = sb + (accum_b ? dbeta[i] : 0.f);
+  }
+  if (i < n * P) {
+    const float2 v = pp[i];
+    if (dgamma && !bc_gamma) dgamma[i] = v.x + (accum_g ? dgamma[i] : 0.f);
+    if (dbeta && !bc_beta) dbeta[i] = v.y + (accum_b ? dbeta[i] : 0.f);
   }
 }
 

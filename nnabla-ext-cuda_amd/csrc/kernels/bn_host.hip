@@ -157,7 +157,7 @@ int bwd_reduce_t(const BnProblem &p, const BnPlan &pl, float *part2, const BnBwd
     NBLAHIP_LAUNCH("bn_bwd_reduce_cl_kernel", (bn_bwd_reduce_cl_kernel<T, VEC>),
                    dim3(pl.ytiles, pl.S), dim3(kBnBlock), 0, st, x, dy, p.mean,
                    static_cast<uint32_t>(p.size0), static_cast<uint32_t>(p.C), pl.ncv, pl.log2tx,
-                   pl.rps, 1.0f, part2);
+                   pl.rps, 1.0f, part2, 0u, FastDiv(1));
   } else if (pl.direct) {
     NBLAHIP_LAUNCH("bn_bwd_reduce_planes_kernel",
                    (bn_bwd_reduce_planes_kernel<T, VEC, 1024, true>),
@@ -311,6 +311,186 @@ int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
     if (int e = last_launch_status()) return e;
   }
   if (p.out) return do_bwd_apply(p, pl, params, st);
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Channel-last Group/InstanceNormalization (N slabs of [S, C]).
+// ---------------------------------------------------------------------------
+namespace {
+
+BnPlan make_cl_plan(int64_t batch, int64_t spatial, int64_t C, int dtype, bool ptr_aligned) {
+  BnPlan pl;
+  const int full = dtype == NBLAHIP_F16 ? 8 : 4;
+  pl.channel_last = true;
+  pl.vec = (ptr_aligned && C % full == 0) ? full : 1;
+  pl.ncv = static_cast<uint32_t>(C / pl.vec);
+  uint32_t l2 = 0;
+  while ((1u << l2) < pl.ncv && l2 < 6) ++l2;
+  pl.log2tx = l2;
+  const uint32_t TX = 1u << l2;
+  const uint32_t TY = kBnBlock >> l2;
+  pl.ytiles = ceil_div_u(pl.ncv, TX);
+  const uint64_t M = static_cast<uint64_t>(spatial);
+  const uint32_t step = TY * kBnUnroll;
+  // the batch already multiplies the block count
+  const uint64_t per_slab = std::max<uint64_t>(1, split_target(true) / static_cast<uint64_t>(batch));
+  const uint32_t want = std::max<uint32_t>(1, ceil_div_u(per_slab, pl.ytiles));
+  const uint32_t most = std::max<uint32_t>(1, static_cast<uint32_t>(M / step));
+  const uint32_t S = std::min(want, most);
+  pl.rps = ceil_div_u(M, S);
+  pl.S = ceil_div_u(M, pl.rps);
+  pl.cl_fast_apply = (256u % pl.ncv) == 0;
+  pl.apply_vec = pl.cl_fast_apply ? pl.vec : 1;
+  return pl;
+}
+
+struct ClWs {
+  float *part;
+  BnParam *params;
+  float *pairs;
+};
+
+size_t cl_part_bytes(int64_t batch, int64_t C, uint32_t S) {
+  return align_up(static_cast<size_t>(batch) * C * S * 3 * sizeof(float), 256);
+}
+
+ClWs cl_carve(const ClProblem &p, const BnPlan &pl) {
+  ClWs w;
+  char *base = static_cast<char *>(p.ws);
+  w.part = reinterpret_cast<float *>(base);
+  base += cl_part_bytes(p.batch, p.channels, pl.S);
+  w.params = reinterpret_cast<BnParam *>(base);
+  base += align_up(static_cast<size_t>(p.batch) * p.channels * sizeof(BnParam), 256);
+  w.pairs = reinterpret_cast<float *>(base);
+  return w;
+}
+
+template <typename T, int VEC>
+int cl_stats_t(const ClProblem &p, const BnPlan &pl, float *part, hipStream_t st) {
+  NBLAHIP_LAUNCH("bn_stats_cl_kernel", (bn_stats_cl_kernel<T, VEC>),
+                 dim3(pl.ytiles, pl.S, static_cast<uint32_t>(p.batch)), dim3(kBnBlock), 0, st,
+                 static_cast<const T *>(p.x), static_cast<uint32_t>(p.spatial),
+                 static_cast<uint32_t>(p.channels), pl.ncv, pl.log2tx, pl.rps, 1.0f, part);
+  return last_launch_status();
+}
+
+template <typename T, int VEC>
+int cl_apply_t(const ClProblem &p, const BnPlan &pl, const BnParam *params, hipStream_t st) {
+  const uint64_t slab = static_cast<uint64_t>(p.spatial) * p.channels;
+  if (pl.cl_fast_apply) {
+    const uint32_t slab_vec = static_cast<uint32_t>(slab / VEC);
+    const uint64_t per_slab = std::max<uint64_t>(
+        1, static_cast<uint64_t>(device_cus()) * tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 4) / p.batch);
+    const uint64_t need = (static_cast<uint64_t>(slab_vec) + 256ull * kBnUnroll - 1) / (256ull * kBnUnroll);
+    NBLAHIP_LAUNCH("bn_apply_cl_kernel", (bn_apply_cl_kernel<T, VEC>),
+                   dim3(static_cast<uint32_t>(std::min(need, per_slab)), static_cast<uint32_t>(p.batch)),
+                   dim3(256), 0, st, static_cast<const T *>(p.x), static_cast<T *>(p.out),
+                   param_src(params), pl.ncv, slab_vec);
+  } else {
+    const uint32_t total = static_cast<uint32_t>(slab * p.batch);
+    NBLAHIP_LAUNCH("cl_slab_apply_kernel", (cl_slab_apply_kernel<T>),
+                   dim3(apply_grid(total, 1)), dim3(256), 0, st, static_cast<const T *>(p.x),
+                   static_cast<T *>(p.out), params, FastDiv(static_cast<uint32_t>(slab)),
+                   FastDiv(static_cast<uint32_t>(p.channels)), total);
+  }
+  return last_launch_status();
+}
+
+template <typename T, int VEC>
+int cl_bwd_reduce_t(const ClProblem &p, const BnPlan &pl, float *part2, hipStream_t st) {
+  const uint32_t cpg = static_cast<uint32_t>(p.channels / p.groups);
+  NBLAHIP_LAUNCH("bn_bwd_reduce_cl_kernel", (bn_bwd_reduce_cl_kernel<T, VEC>),
+                 dim3(pl.ytiles, pl.S, static_cast<uint32_t>(p.batch)), dim3(kBnBlock), 0, st,
+                 static_cast<const T *>(p.x), static_cast<const T *>(p.dy), p.mean,
+                 static_cast<uint32_t>(p.spatial), static_cast<uint32_t>(p.channels), pl.ncv,
+                 pl.log2tx, pl.rps, 1.0f, part2, static_cast<uint32_t>(p.groups), FastDiv(cpg));
+  return last_launch_status();
+}
+
+template <typename T, int VEC>
+int cl_bwd_apply_t(const ClProblem &p, const BnPlan &pl, const BnParam *params, hipStream_t st) {
+  const uint64_t slab = static_cast<uint64_t>(p.spatial) * p.channels;
+  if (pl.cl_fast_apply) {
+    const uint32_t slab_vec = static_cast<uint32_t>(slab / VEC);
+    const uint64_t per_slab = std::max<uint64_t>(
+        1, static_cast<uint64_t>(device_cus()) * tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 4) / p.batch);
+    const uint64_t need = (static_cast<uint64_t>(slab_vec) + 256ull * 2 - 1) / (256ull * 2);
+    NBLAHIP_LAUNCH("bn_bwd_apply_cl_kernel", (bn_bwd_apply_cl_kernel<T, VEC>),
+                   dim3(static_cast<uint32_t>(std::min(need, per_slab)), static_cast<uint32_t>(p.batch)),
+                   dim3(256), 0, st, static_cast<const T *>(p.x), static_cast<const T *>(p.dy),
+                   static_cast<T *>(p.out), params, pl.ncv, slab_vec, p.accum_dx);
+  } else {
+    const uint32_t total = static_cast<uint32_t>(slab * p.batch);
+    NBLAHIP_LAUNCH("cl_slab_bwd_apply_kernel", (cl_slab_bwd_apply_kernel<T>),
+                   dim3(apply_grid(total, 1)), dim3(256), 0, st, static_cast<const T *>(p.x),
+                   static_cast<const T *>(p.dy), static_cast<T *>(p.out), params,
+                   FastDiv(static_cast<uint32_t>(slab)), FastDiv(static_cast<uint32_t>(p.channels)),
+                   total, p.accum_dx);
+  }
+  return last_launch_status();
+}
+
+} // namespace
+
+size_t cl_workspace_bytes(int64_t batch, int64_t spatial, int64_t channels, int dtype) {
+  const BnPlan a = make_cl_plan(batch, spatial, channels, dtype, true);
+  const BnPlan b = make_cl_plan(batch, spatial, channels, dtype, false);
+  return cl_part_bytes(batch, channels, std::max(a.S, b.S)) +
+         align_up(static_cast<size_t>(batch) * channels * sizeof(BnParam), 256) +
+         align_up(static_cast<size_t>(batch) * channels * 2 * sizeof(float), 256);
+}
+
+int launch_cl_fwd(const ClProblem &p, hipStream_t st) {
+  const bool al = aligned16(p.x) && aligned16(p.out);
+  const BnPlan pl = make_cl_plan(p.batch, p.spatial, p.channels, p.dtype, al);
+  const ClWs w = cl_carve(p, pl);
+  const uint32_t cpg = static_cast<uint32_t>(p.channels / p.groups);
+#define CALL(T, V) cl_stats_t<T, V>(p, pl, w.part, st)
+  const int e1 = [&]() -> int { BN_DISPATCH(CALL, pl.vec); }();
+#undef CALL
+  if (e1) return e1;
+  const float inv_R = static_cast<float>(1.0 / (static_cast<double>(p.spatial) * cpg));
+  NBLAHIP_LAUNCH("gn_cl_finalize_fwd_kernel", gn_cl_finalize_fwd_kernel,
+                 dim3(static_cast<uint32_t>(p.batch * p.groups)), dim3(kBnBlock), 0, st, w.part, pl.S,
+                 static_cast<uint32_t>(p.channels), cpg, inv_R, p.eps, p.gamma, p.beta,
+                 p.bc_gamma ? 1u : 0u, p.bc_beta ? 1u : 0u, p.mean, p.var, w.params);
+  if (int e = last_launch_status()) return e;
+#define CALL(T, V) cl_apply_t<T, V>(p, pl, w.params, st)
+  BN_DISPATCH(CALL, pl.apply_vec);
+#undef CALL
+}
+
+int launch_cl_bwd(const ClProblem &p, hipStream_t st) {
+  if (!p.out && !p.dgamma && !p.dbeta) return 0;
+  const bool al = aligned16(p.x) && aligned16(p.dy) && (!p.out || aligned16(p.out));
+  const BnPlan pl = make_cl_plan(p.batch, p.spatial, p.channels, p.dtype, al);
+  const ClWs w = cl_carve(p, pl);
+  const uint32_t cpg = static_cast<uint32_t>(p.channels / p.groups);
+#define CALL(T, V) cl_bwd_reduce_t<T, V>(p, pl, w.part, st)
+  const int e1 = [&]() -> int { BN_DISPATCH(CALL, pl.vec); }();
+#undef CALL
+  if (e1) return e1;
+  const float inv_R = static_cast<float>(1.0 / (static_cast<double>(p.spatial) * cpg));
+  NBLAHIP_LAUNCH("gn_cl_finalize_bwd_kernel", gn_cl_finalize_bwd_kernel,
+                 dim3(static_cast<uint32_t>(p.batch * p.groups)), dim3(kBnBlock), 0, st, w.part, pl.S,
+                 static_cast<uint32_t>(p.channels), cpg, inv_R, p.eps, p.gamma, p.bc_gamma ? 1u : 0u,
+                 p.mean, p.var, p.dmean, p.dvar, w.pairs, w.params);
+  if (int e = last_launch_status()) return e;
+  if (p.out) {
+#define CALL(T, V) cl_bwd_apply_t<T, V>(p, pl, w.params, st)
+    const int e2 = [&]() -> int { BN_DISPATCH(CALL, pl.apply_vec); }();
+#undef CALL
+    if (e2) return e2;
+  }
+  if (p.dgamma || p.dbeta) {
+    const int64_t count = (p.bc_gamma && p.bc_beta) ? p.channels : p.batch * p.channels;
+    NBLAHIP_LAUNCH("pair_param_reduce_cl_kernel", cl_pair_param_reduce_kernel,
+                   dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, st, w.pairs,
+                   static_cast<int>(p.batch), static_cast<int>(p.channels), p.dgamma, p.dbeta,
+                   p.bc_gamma, p.bc_beta, p.accum_g, p.accum_b);
+    if (int e = last_launch_status()) return e;
+  }
   return 0;
 }
 

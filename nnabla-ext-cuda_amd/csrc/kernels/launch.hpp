@@ -119,6 +119,32 @@ bool prof_acquire(const char *tag, hipEvent_t *start, hipEvent_t *stop);
     }                                                                                   \
   } while (0)
 
+// Channel-last Group/InstanceNormalization: x is [batch, spatial, channels].
+struct ClProblem {
+  int dtype = 0;
+  const void *x = nullptr;
+  const void *dy = nullptr;
+  void *out = nullptr; // y or dx
+  const float *gamma = nullptr;
+  const float *beta = nullptr;
+  float *mean = nullptr; // [batch*groups], forward: written; backward: read
+  float *var = nullptr;
+  const float *dmean = nullptr;
+  const float *dvar = nullptr;
+  float *dgamma = nullptr;
+  float *dbeta = nullptr;
+  int accum_dx = 0, accum_g = 0, accum_b = 0;
+  int64_t batch = 1, spatial = 1, channels = 1;
+  int groups = 1;
+  int bc_gamma = 1, bc_beta = 1; // parameters shared by the batch (always for groups)
+  float eps = 0.f;
+  void *ws = nullptr;
+  size_t ws_bytes = 0;
+};
+int launch_cl_fwd(const ClProblem &p, hipStream_t st);
+int launch_cl_bwd(const ClProblem &p, hipStream_t st);
+size_t cl_workspace_bytes(int64_t batch, int64_t spatial, int64_t channels, int dtype);
+
 inline int last_launch_status() {
   const hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : static_cast<int>(e);

@@ -229,16 +229,91 @@ def test_instance_normalization(tc, per_sample):
     assert_close(vb.g, db_r, dn(tc), "pgrad", "dbeta")
 
 
+@pytest.mark.parametrize("tc", CONFIGS)
+@pytest.mark.parametrize("shape,groups", [((4, 8, 8, 16), 4), ((2, 5, 6), 3), ((3, 7, 7, 24), 8)])
+def test_group_normalization_channel_last(tc, shape, groups):
+    """x[N, *spatial, C] with channel_axis = -1: no transposes, statistics as
+    outputs [N, 1.., G], same numbers as the channel-first function on the
+    transposed tensor (the reference's adaptor path, group_normalization.cu:93-106)."""
+    rng = np.random.default_rng(8)
+    half = tc == "half"
+    n, c = shape[0], shape[-1]
+    pshape = (1,) * (len(shape) - 1) + (c,)
+    x = rnd(rng.standard_normal(shape) * 1.5, tc)
+    dy = rnd(rng.standard_normal(shape), tc)
+    g = rng.uniform(0.5, 1.5, pshape).astype(np.float32)
+    b = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
+    f = B.GroupNormalization(B.context(tc), num_groups=groups, channel_axis=len(shape) - 1,
+                             batch_axis=[0])
+    vx, vb, vg = var(x, half), var(b), var(g)
+    vy, om, ov = B.Variable(shape), B.Variable(()), B.Variable(())
+    f.setup([vx, vb, vg], [vy, om, ov])
+    assert tuple(om.current_shape) == (n,) + (1,) * (len(shape) - 2) + (groups,)
+    f.forward([vx, vb, vg], [vy, om, ov])
+    xt, dyt = np.moveaxis(x, -1, 1), np.moveaxis(dy, -1, 1)
+    y_r, m_r, v_r = R.gn_forward(xt, b, g, n, c, groups, 1e-5)
+    back = lambda a: np.moveaxis(np.asarray(a).reshape(xt.shape), 1, -1)
+    assert_close(vy.d, back(y_r), dn(tc), "y", "y")
+    assert_close(om.d, m_r, dn(tc), "stat", "mean output")
+    assert_close(ov.d, v_r, dn(tc), "stat", "var output")
+    dm = rng.standard_normal(om.current_shape).astype(np.float32)
+    dv = rng.standard_normal(ov.current_shape).astype(np.float32)
+    vy.set_grad(dy, half)
+    om.set_grad(dm)
+    ov.set_grad(dv)
+    f.backward([vx, vb, vg], [vy, om, ov], propagate_down=[1, 1, 1], accum=[0, 0, 0])
+    dx_r, dg_r, db_r = R.gn_backward(xt, dyt, g, m_r, v_r, n, c, groups, 1e-5, dm, dv)
+    assert_close(vx.g, back(dx_r), dn(tc), "grad", "dx")
+    assert_close(vg.g, dg_r, dn(tc), "pgrad", "dgamma")
+    assert_close(vb.g, db_r, dn(tc), "pgrad", "dbeta")
+
+
+@pytest.mark.parametrize("tc", CONFIGS)
+@pytest.mark.parametrize("per_sample", [False, True])
+def test_instance_normalization_channel_last(tc, per_sample):
+    rng = np.random.default_rng(9)
+    half = tc == "half"
+    shape = (3, 9, 9, 8)
+    n, c = shape[0], shape[-1]
+    pshape = (n if per_sample else 1, 1, 1, c)
+    x = rnd(rng.standard_normal(shape) * 1.5, tc)
+    dy = rnd(rng.standard_normal(shape), tc)
+    g = rng.uniform(0.5, 1.5, pshape).astype(np.float32)
+    b = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
+    f = B.InstanceNormalization(B.context(tc), channel_axis=3, batch_axis=[0])
+    vx, vb, vg = var(x, half), var(b), var(g)
+    vy = B.Variable(shape)
+    f.setup([vx, vb, vg], [vy])
+    f.forward([vx, vb, vg], [vy])
+    xt, dyt = np.moveaxis(x, -1, 1), np.moveaxis(dy, -1, 1)
+    back = lambda a: np.moveaxis(np.asarray(a).reshape(xt.shape), 1, -1)
+    g_full = g.reshape(-1) if per_sample else np.tile(g.reshape(-1), n)
+    b_full = b.reshape(-1) if per_sample else np.tile(b.reshape(-1), n)
+    y_r, m_r, v_r = R.in_forward(xt, b_full, g_full, n, c, 1e-5)
+    assert_close(vy.d, back(y_r), dn(tc), "y", "y")
+    vy.set_grad(dy, half)
+    f.backward([vx, vb, vg], [vy], propagate_down=[1, 1, 1], accum=[0, 0, 0])
+    dx_r, dg_r, db_r = R.in_backward(xt, dyt, g.reshape(-1), m_r, v_r, n, c, 1e-5,
+                                     bc_gamma=not per_sample, bc_beta=not per_sample)
+    assert_close(vx.g, back(dx_r), dn(tc), "grad", "dx")
+    assert_close(vg.g, dg_r, dn(tc), "pgrad", "dgamma")
+    assert_close(vb.g, db_r, dn(tc), "pgrad", "dbeta")
+
+
 def test_unsupported_layouts_raise_not_implemented():
     ctx = B.context("float")
     x, y = B.Variable((4, 6, 8)), B.Variable((4, 6, 8))
     f = B.LayerNormalization(ctx, batch_axis=[1], no_scale=True, no_bias=True)
     with pytest.raises(B.NblaError, match="batch_axis"):
         f.setup([x], [y])
+    x4, y4 = B.Variable((4, 6, 8, 5)), B.Variable((4, 6, 8, 5))
     g = B.GroupNormalization(ctx, num_groups=2, channel_axis=2, batch_axis=[0], no_scale=True,
                              no_bias=True)
     with pytest.raises(B.NblaError, match="channel-first"):
-        g.setup([x], [y])
+        g.setup([x4], [y4])                      # channel axis in the middle
+    i = B.InstanceNormalization(ctx, channel_axis=0, batch_axis=[1], no_scale=True, no_bias=True)
+    with pytest.raises(B.NblaError, match="channel-first"):
+        i.setup([x], [y])                        # batch axis behind the channel axis
     h = B.GroupNormalization(ctx, num_groups=4, channel_axis=1, batch_axis=[0], no_scale=True,
                              no_bias=True)
     with pytest.raises(B.NblaError, match="divisible"):
