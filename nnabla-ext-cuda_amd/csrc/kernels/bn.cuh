@@ -704,35 +704,48 @@ bn_bwd_apply_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
 // ---------------------------------------------------------------------------
 // Channel-last Group/InstanceNormalization on the BatchNormalization
 // channel-last machinery: x is N slabs [S, C]; the split reductions above
-// leave partials per (n, c, split).  One block per (n, group) merges the
-// partials of the group's cpg channels (cpg = 1: InstanceNormalization) and
-// publishes mean/var of the group plus the apply parameters of its channels.
+// leave partials per (n, c, split).  The finalize kernels merge the partials
+// of each (n, group)'s cpg channels (cpg = 1: InstanceNormalization) and
+// publish mean/var of the group plus the apply parameters of its channels.
+// WAVE: one wave per (n, group) (small groups, no LDS), else one block.
 //   gamma/beta index of channel c in sample n: gmod == 0 ? n*C + c : c
 // ---------------------------------------------------------------------------
+__device__ __forceinline__ float subgroup_sum(float v, uint32_t width /* power of two <= 64 */) {
+  for (uint32_t o = width >> 1; o; o >>= 1) v += __shfl_xor(v, static_cast<int>(o));
+  return v;
+}
+
+template <bool WAVE>
 __global__ void __launch_bounds__(kBnBlock)
 gn_cl_finalize_fwd_kernel(const float *__restrict__ part, uint32_t S, uint32_t C, uint32_t cpg,
-                          float inv_R, float eps, const float *__restrict__ gamma,
+                          uint32_t NG, float inv_R, float eps, const float *__restrict__ gamma,
                           const float *__restrict__ beta, uint32_t gmod, uint32_t bmod,
                           float *__restrict__ mean, float *__restrict__ var,
                           BnParam *__restrict__ params) {
   __shared__ float lds[3 * (kBnBlock / kWave)];
+  constexpr uint32_t kWaves = kBnBlock / kWave;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t ng = WAVE ? blockIdx.x * kWaves + threadIdx.x / kWave : blockIdx.x;
+  if (WAVE && ng >= NG) return; // wave-uniform; no block barrier in this mode
+  const uint32_t tid = WAVE ? lane : threadIdx.x;
+  const uint32_t nthr = WAVE ? kWave : kBnBlock;
   const uint32_t G = C / cpg;
-  const uint32_t n = blockIdx.x / G, g = blockIdx.x % G;
+  const uint32_t n = ng / G, g = ng % G;
   const float *p0 = part + 3 * (static_cast<size_t>(n) * C + static_cast<size_t>(g) * cpg) * S;
   Welford w{0.f, 0.f, 0.f};
-  for (uint32_t i = threadIdx.x; i < cpg * S; i += kBnBlock) { // (channel, split) pairs, contiguous
+  for (uint32_t i = tid; i < cpg * S; i += nthr) { // (channel, split) pairs, contiguous
     const float *p = p0 + 3 * static_cast<size_t>(i);
     w = welford_merge(w, Welford{p[0], p[1], p[2]});
   }
-  w = block_welford(w, lds);
+  w = WAVE ? wave_welford(w) : block_welford(w, lds);
   const float m = w.mean;
   const float v = w.m2 * inv_R;
   const float istd = inv_std(v, eps);
-  if (threadIdx.x == 0) {
-    mean[blockIdx.x] = m;
-    var[blockIdx.x] = v;
+  if (tid == 0) {
+    mean[ng] = m;
+    var[ng] = v;
   }
-  for (uint32_t cl = threadIdx.x; cl < cpg; cl += kBnBlock) {
+  for (uint32_t cl = tid; cl < cpg; cl += nthr) {
     const uint32_t c = g * cpg + cl;
     const uint32_t nc = n * C + c;
     BnParam q;
@@ -750,38 +763,63 @@ gn_cl_finalize_fwd_kernel(const float *__restrict__ part, uint32_t S, uint32_t C
 //   dx = gamma_c*istd*dy + f1*(x-mean) + f2',  f1 = -t2*istd^3/R + 2*dvar/R,
 //   f2' = -s1*istd/R + dmean/R
 // and the pair (sdx_c*istd, sdy_c) for the batch sum of dgamma/dbeta.
+// A wave covers 64/sp channels at a time, sp lanes (a power of two) sharing
+// the S splits of one channel.
+template <bool WAVE>
 __global__ void __launch_bounds__(kBnBlock)
-gn_cl_finalize_bwd_kernel(const float *__restrict__ part2, uint32_t S, uint32_t C, uint32_t cpg,
-                          float inv_R, float eps, const float *__restrict__ gamma, uint32_t gmod,
+gn_cl_finalize_bwd_kernel(const float *__restrict__ part2, uint32_t S, uint32_t sp, uint32_t C,
+                          uint32_t cpg, uint32_t NG, float inv_R, float eps,
+                          const float *__restrict__ gamma, uint32_t gmod,
                           const float *__restrict__ mean, const float *__restrict__ var,
                           const float *__restrict__ dmean, const float *__restrict__ dvar,
                           float *__restrict__ pairs, BnParam *__restrict__ params) {
   __shared__ float lds[2 * (kBnBlock / kWave)];
+  constexpr uint32_t kWaves = kBnBlock / kWave;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t wave = threadIdx.x / kWave;
+  const uint32_t ng = WAVE ? blockIdx.x * kWaves + wave : blockIdx.x;
+  if (WAVE && ng >= NG) return; // wave-uniform; no block barrier in this mode
+  const uint32_t tid = WAVE ? lane : threadIdx.x;
+  const uint32_t nthr = WAVE ? kWave : kBnBlock;
   const uint32_t G = C / cpg;
-  const uint32_t n = blockIdx.x / G, g = blockIdx.x % G;
-  const float m = mean[blockIdx.x];
-  const float istd = inv_std(var[blockIdx.x], eps);
-  // Pass 1: channel sums over the splits, s1/t2 over the group.
+  const uint32_t n = ng / G, g = ng % G;
+  const float m = mean[ng];
+  const float istd = inv_std(var[ng], eps);
+  const uint32_t chw = kWave / sp;          // channels per wave pass
+  const uint32_t sub = lane / sp, sl = lane & (sp - 1);
+  const uint32_t first = (WAVE ? 0u : wave) * chw;
+  const uint32_t stride = (WAVE ? 1u : kWaves) * chw;
+  const float2 *__restrict__ pp = reinterpret_cast<const float2 *>(part2);
   float s1 = 0.f, t2 = 0.f;
-  for (uint32_t cl = threadIdx.x; cl < cpg; cl += kBnBlock) {
-    const uint32_t c = g * cpg + cl;
+  for (uint32_t cl0 = first; cl0 < cpg; cl0 += stride) {
+    const uint32_t cl = cl0 + sub;
+    const bool ok = cl < cpg;
+    const uint32_t c = g * cpg + (ok ? cl : 0u);
     const uint32_t nc = n * C + c;
-    const float *p = part2 + 2 * static_cast<size_t>(nc) * S;
     float sdx = 0.f, sdy = 0.f;
-    for (uint32_t s = 0; s < S; ++s) {
-      sdx += p[2 * s];
-      sdy += p[2 * s + 1];
+    for (uint32_t s = sl; s < S; s += sp) {
+      const float2 v = pp[static_cast<size_t>(nc) * S + s];
+      sdx += v.x;
+      sdy += v.y;
     }
-    pairs[2 * static_cast<size_t>(nc)] = sdx * istd;
-    pairs[2 * static_cast<size_t>(nc) + 1] = sdy;
-    const float gm = gamma ? gamma[gmod ? c : nc] : 1.f;
-    s1 += gm * sdy;
-    t2 += gm * sdx;
+    sdx = subgroup_sum(sdx, sp);
+    sdy = subgroup_sum(sdy, sp);
+    if (ok && sl == 0) {
+      reinterpret_cast<float2 *>(pairs)[nc] = make_float2(sdx * istd, sdy);
+      const float gm = gamma ? gamma[gmod ? c : nc] : 1.f;
+      s1 += gm * sdy;
+      t2 += gm * sdx;
+    }
   }
-  block_sum2(s1, t2, lds);
-  const float f1 = -t2 * istd * istd * istd * inv_R + (dvar ? 2.f * dvar[blockIdx.x] * inv_R : 0.f);
-  const float f2 = -s1 * istd * inv_R + (dmean ? dmean[blockIdx.x] * inv_R : 0.f);
-  for (uint32_t cl = threadIdx.x; cl < cpg; cl += kBnBlock) {
+  if (WAVE) {
+    s1 = wave_sum(s1);
+    t2 = wave_sum(t2);
+  } else {
+    block_sum2(s1, t2, lds);
+  }
+  const float f1 = -t2 * istd * istd * istd * inv_R + (dvar ? 2.f * dvar[ng] * inv_R : 0.f);
+  const float f2 = -s1 * istd * inv_R + (dmean ? dmean[ng] * inv_R : 0.f);
+  for (uint32_t cl = tid; cl < cpg; cl += nthr) {
     const uint32_t c = g * cpg + cl;
     const uint32_t nc = n * C + c;
     BnParam q;

@@ -345,6 +345,12 @@ BnPlan make_cl_plan(int64_t batch, int64_t spatial, int64_t C, int dtype, bool p
   return pl;
 }
 
+// Groups small enough for one wave each (at most 2 partials per lane: the
+// merges of one lane are a serial chain).
+bool cl_wave_finalize(uint32_t cpg, uint32_t S) {
+  return static_cast<uint64_t>(cpg) * S <= 2u * kWave;
+}
+
 struct ClWs {
   float *part;
   BnParam *params;
@@ -451,10 +457,18 @@ int launch_cl_fwd(const ClProblem &p, hipStream_t st) {
 #undef CALL
   if (e1) return e1;
   const float inv_R = static_cast<float>(1.0 / (static_cast<double>(p.spatial) * cpg));
-  NBLAHIP_LAUNCH("gn_cl_finalize_fwd_kernel", gn_cl_finalize_fwd_kernel,
-                 dim3(static_cast<uint32_t>(p.batch * p.groups)), dim3(kBnBlock), 0, st, w.part, pl.S,
-                 static_cast<uint32_t>(p.channels), cpg, inv_R, p.eps, p.gamma, p.beta,
-                 p.bc_gamma ? 1u : 0u, p.bc_beta ? 1u : 0u, p.mean, p.var, w.params);
+  const uint32_t NG = static_cast<uint32_t>(p.batch * p.groups);
+  if (cl_wave_finalize(cpg, pl.S)) {
+    NBLAHIP_LAUNCH("gn_cl_finalize_fwd_kernel", gn_cl_finalize_fwd_kernel<true>,
+                   dim3(ceil_div_u(NG, kBnBlock / kWave)), dim3(kBnBlock), 0, st, w.part, pl.S,
+                   static_cast<uint32_t>(p.channels), cpg, NG, inv_R, p.eps, p.gamma, p.beta,
+                   p.bc_gamma ? 1u : 0u, p.bc_beta ? 1u : 0u, p.mean, p.var, w.params);
+  } else {
+    NBLAHIP_LAUNCH("gn_cl_finalize_fwd_kernel", gn_cl_finalize_fwd_kernel<false>, dim3(NG),
+                   dim3(kBnBlock), 0, st, w.part, pl.S, static_cast<uint32_t>(p.channels), cpg, NG,
+                   inv_R, p.eps, p.gamma, p.beta, p.bc_gamma ? 1u : 0u, p.bc_beta ? 1u : 0u,
+                   p.mean, p.var, w.params);
+  }
   if (int e = last_launch_status()) return e;
 #define CALL(T, V) cl_apply_t<T, V>(p, pl, w.params, st)
   BN_DISPATCH(CALL, pl.apply_vec);
@@ -472,10 +486,20 @@ int launch_cl_bwd(const ClProblem &p, hipStream_t st) {
 #undef CALL
   if (e1) return e1;
   const float inv_R = static_cast<float>(1.0 / (static_cast<double>(p.spatial) * cpg));
-  NBLAHIP_LAUNCH("gn_cl_finalize_bwd_kernel", gn_cl_finalize_bwd_kernel,
-                 dim3(static_cast<uint32_t>(p.batch * p.groups)), dim3(kBnBlock), 0, st, w.part, pl.S,
-                 static_cast<uint32_t>(p.channels), cpg, inv_R, p.eps, p.gamma, p.bc_gamma ? 1u : 0u,
-                 p.mean, p.var, p.dmean, p.dvar, w.pairs, w.params);
+  const uint32_t NG = static_cast<uint32_t>(p.batch * p.groups);
+  uint32_t sp = 1; // lanes sharing the splits of one channel: power of two, at most a wave
+  while (sp < pl.S && sp < kWave) sp <<= 1;
+  if (cl_wave_finalize(cpg, pl.S)) {
+    NBLAHIP_LAUNCH("gn_cl_finalize_bwd_kernel", gn_cl_finalize_bwd_kernel<true>,
+                   dim3(ceil_div_u(NG, kBnBlock / kWave)), dim3(kBnBlock), 0, st, w.part, pl.S, sp,
+                   static_cast<uint32_t>(p.channels), cpg, NG, inv_R, p.eps, p.gamma,
+                   p.bc_gamma ? 1u : 0u, p.mean, p.var, p.dmean, p.dvar, w.pairs, w.params);
+  } else {
+    NBLAHIP_LAUNCH("gn_cl_finalize_bwd_kernel", gn_cl_finalize_bwd_kernel<false>, dim3(NG),
+                   dim3(kBnBlock), 0, st, w.part, pl.S, sp, static_cast<uint32_t>(p.channels), cpg,
+                   NG, inv_R, p.eps, p.gamma, p.bc_gamma ? 1u : 0u, p.mean, p.var, p.dmean, p.dvar,
+                   w.pairs, w.params);
+  }
   if (int e = last_launch_status()) return e;
   if (p.out) {
 #define CALL(T, V) cl_bwd_apply_t<T, V>(p, pl, w.params, st)
