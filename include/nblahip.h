@@ -110,6 +110,50 @@ NBLAHIP_EXPORT int nblahip_bn_bwd(const void *x, const void *dy,
                                   size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------
+ * FusedBatchNormalization: y = max(0, BatchNormalization(x) + z), z optional
+ * (NULL: no residual input).  Same tensor view, statistics and workspace as
+ * BatchNormalization above; gamma and beta are always present in the
+ * reference (fused_batch_normalization.hpp:30-37) but may be NULL here.
+ * ---------------------------------------------------------------------- */
+
+/* Replaces the batch_stat == false forward of the composite
+ * FusedBatchNormalization (BatchNormalization forward_impl_global,
+ * batch_normalization.cu:175-199, then add2 and relu,
+ * include/nbla/cuda/utils/add2.cuh:23-27, relu.cuh:48-52). */
+NBLAHIP_EXPORT int nblahip_fused_bn_fwd_infer(const void *x, const void *z,
+                                              const float *rmean,
+                                              const float *rvar,
+                                              const float *gamma,
+                                              const float *beta, void *y,
+                                              int64_t size0, int64_t size1,
+                                              int64_t size2, float eps,
+                                              int dtype, void *stream);
+
+/* Replaces fused_batch_norm_forward: cudnnBatchNormalizationForwardTrainingEx
+ * with BN_ADD_ACTIVATION / BN_ACTIVATION
+ * (cudnn/function/generic/fused_batch_normalization.cu:136-216). */
+NBLAHIP_EXPORT int nblahip_fused_bn_fwd_train(
+    const void *x, const void *z, const float *gamma, const float *beta,
+    void *y, float *batch_mean, float *batch_var, float *rmean, float *rvar,
+    int64_t size0, int64_t size1, int64_t size2, float decay_rate, float eps,
+    int dtype, void *workspace, size_t workspace_bytes, void *stream);
+
+/* Replaces cudnnBatchNormalizationBackwardEx
+ * (cudnn/function/generic/fused_batch_normalization.cu:230-357) and the
+ * composite relu_add2_backward (function/generic/fused_batch_normalization.cu
+ * :47-75) followed by the BatchNormalization backward: with
+ * g = dy where y > 0 else 0,  dz (+)= g  and (dx, dgamma, dbeta) are the
+ * BatchNormalization backward of g.  y is the forward output (required);
+ * dx, dz, dgamma, dbeta may each be NULL (not propagated); dz may alias dy. */
+NBLAHIP_EXPORT int nblahip_fused_bn_bwd(
+    const void *x, const void *y, const void *dy, const float *gamma,
+    const float *mean, const float *var, const float *dmean, const float *dvar,
+    void *dx, void *dz, float *dgamma, float *dbeta, int accum_dx, int accum_dz,
+    int accum_dgamma, int accum_dbeta, int64_t size0, int64_t size1,
+    int64_t size2, float eps, int batch_stat, int dtype, void *workspace,
+    size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------
  * LayerNormalization.  x viewed as [outer, reduce]
  * (src/nbla/cuda/function/generic/layer_normalization.cu:53-59).
  * ---------------------------------------------------------------------- */

@@ -34,6 +34,11 @@ SIGNATURES = {
                                                               _c_void_p]),
     "nblahip_bn_bwd": (_int, [_c_void_p] * 10 + [_int] * 3 + [_i64] * 3 + [_f, _int, _int,
                                                                    _c_void_p, _sz, _c_void_p]),
+    "nblahip_fused_bn_fwd_infer": (_int, [_c_void_p] * 7 + [_i64] * 3 + [_f, _int, _c_void_p]),
+    "nblahip_fused_bn_fwd_train": (_int, [_c_void_p] * 9 + [_i64] * 3 + [_f, _f, _int, _c_void_p,
+                                                                         _sz, _c_void_p]),
+    "nblahip_fused_bn_bwd": (_int, [_c_void_p] * 12 + [_int] * 4 + [_i64] * 3 + [_f, _int, _int,
+                                                                         _c_void_p, _sz, _c_void_p]),
     "nblahip_ln_fwd": (_int, [_c_void_p] * 6 + [_i64] * 2 + [_f, _int, _c_void_p]),
     "nblahip_ln_bwd_workspace_bytes": (_sz, [_i64] * 2 + [_int]),
     "nblahip_ln_bwd": (_int, [_c_void_p] * 10 + [_int] * 3 + [_i64] * 2 + [_f, _int, _c_void_p,
@@ -212,6 +217,66 @@ def bn_backward(x, dy, gamma, mean, var, axis=1, eps=1e-5, batch_stat=True, dmea
                                int(accum[0]), int(accum[1]), int(accum[2]), s0, c, s2, eps,
                                int(batch_stat), dt, _ptr(ws), ws.numel(), _stream()))
     return (dx if need[0] else None, dgamma if need[1] else None, dbeta if need[2] else None)
+
+
+def fused_bn_forward_global(x, z, beta, gamma, rmean, rvar, axis=1, eps=1e-5):
+    """y = max(0, bn_inference(x) + z); z may be None."""
+    import torch
+    assert x.is_contiguous() and (z is None or z.is_contiguous())
+    s0, c, s2 = _bn_sizes(x.shape, axis)
+    y = torch.empty_like(x)
+    check(lib().nblahip_fused_bn_fwd_infer(
+        _ptr(x), _ptr(z), _ptr(_f32(rmean, "rmean")), _ptr(_f32(rvar, "rvar")),
+        _ptr(_f32(gamma, "gamma")), _ptr(_f32(beta, "beta")), _ptr(y), s0, c, s2, eps,
+        _dtype_code(x), _stream()))
+    return y
+
+
+def fused_bn_forward_batch(x, z, beta, gamma, rmean, rvar, axis=1, decay_rate=0.9, eps=1e-5,
+                           ws=None):
+    """y = max(0, bn_training(x) + z); returns y, batch_mean, batch_var."""
+    import torch
+    assert x.is_contiguous() and (z is None or z.is_contiguous())
+    s0, c, s2 = _bn_sizes(x.shape, axis)
+    dt = _dtype_code(x)
+    y = torch.empty_like(x)
+    mean = torch.empty(c, dtype=torch.float32, device=x.device)
+    var = torch.empty(c, dtype=torch.float32, device=x.device)
+    need = lib().nblahip_bn_workspace_bytes(s0, c, s2, dt)
+    ws = ws if ws is not None else _workspace(need, x.device)
+    check(lib().nblahip_fused_bn_fwd_train(
+        _ptr(x), _ptr(z), _ptr(_f32(gamma, "gamma")), _ptr(_f32(beta, "beta")), _ptr(y),
+        _ptr(mean), _ptr(var), _ptr(_f32(rmean, "rmean")), _ptr(_f32(rvar, "rvar")), s0, c, s2,
+        decay_rate, eps, dt, _ptr(ws), ws.numel(), _stream()))
+    return y, mean, var
+
+
+def fused_bn_backward(x, y, dy, gamma, mean, var, axis=1, eps=1e-5, batch_stat=True, dmean=None,
+                      dvar=None, dx=None, dz=None, dgamma=None, dbeta=None,
+                      accum=(False, False, False, False), need=(True, True, True, True), ws=None):
+    """need / accum = (dx, dz, dgamma, dbeta).  Returns dx, dz, dgamma, dbeta."""
+    import torch
+    assert x.is_contiguous() and dy.is_contiguous() and y.is_contiguous()
+    s0, c, s2 = _bn_sizes(x.shape, axis)
+    dt = _dtype_code(x)
+    if need[0] and dx is None:
+        dx = torch.empty_like(x)
+    if need[1] and dz is None:
+        dz = torch.empty_like(x)
+    if need[2] and dgamma is None:
+        dgamma = torch.empty(c, dtype=torch.float32, device=x.device)
+    if need[3] and dbeta is None:
+        dbeta = torch.empty(c, dtype=torch.float32, device=x.device)
+    nbytes = lib().nblahip_bn_workspace_bytes(s0, c, s2, dt)
+    ws = ws if ws is not None else _workspace(nbytes, x.device)
+    check(lib().nblahip_fused_bn_bwd(
+        _ptr(x), _ptr(y), _ptr(dy), _ptr(_f32(gamma, "gamma")), _ptr(mean), _ptr(var), _ptr(dmean),
+        _ptr(dvar), _ptr(dx if need[0] else None), _ptr(dz if need[1] else None),
+        _ptr(dgamma if need[2] else None), _ptr(dbeta if need[3] else None), int(accum[0]),
+        int(accum[1]), int(accum[2]), int(accum[3]), s0, c, s2, eps, int(batch_stat), dt, _ptr(ws),
+        ws.numel(), _stream()))
+    return (dx if need[0] else None, dz if need[1] else None, dgamma if need[2] else None,
+            dbeta if need[3] else None)
 
 
 def ln_forward(x, beta, gamma, outer, eps=1e-5):

@@ -31,14 +31,15 @@ hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
 
 } // namespace
 
-extern "C" {
-
 // ----------------------------------------------------------------------------
-// BatchNormalization
+// BatchNormalization and FusedBatchNormalization (relu != 0: y = max(0, bn + z);
+// y_out != null in the backward: dy masked by y_out > 0, masked dy -> dz)
 // ----------------------------------------------------------------------------
-int nblahip_bn_fwd_infer(const void *x, const float *rmean, const float *rvar,
-                         const float *gamma, const float *beta, void *y, int64_t size0,
-                         int64_t size1, int64_t size2, float eps, int dtype, void *stream) {
+namespace {
+int bn_fwd_infer_impl(const void *x, const void *z, int relu, const float *rmean,
+                      const float *rvar, const float *gamma, const float *beta, void *y,
+                      int64_t size0, int64_t size1, int64_t size2, float eps, int dtype,
+                      void *stream) {
   if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
   const int d = check_dims3(size0, size1, size2);
   if (d) return d < 0 ? d : 0;
@@ -55,18 +56,16 @@ int nblahip_bn_fwd_infer(const void *x, const float *rmean, const float *rvar,
   p.C = size1;
   p.size2 = size2;
   p.eps = eps;
+  p.relu = relu;
+  p.z = z;
   return launch_bn_infer(p, as_stream(stream));
 }
 
-size_t nblahip_bn_workspace_bytes(int64_t size0, int64_t size1, int64_t size2, int dtype) {
-  if (!dtype_ok(dtype) || check_dims3(size0, size1, size2) != 0) return 0;
-  return bn_workspace_bytes(size0, size1, size2, dtype);
-}
-
-int nblahip_bn_fwd_train(const void *x, const float *gamma, const float *beta, void *y,
-                         float *batch_mean, float *batch_var, float *rmean, float *rvar,
-                         int64_t size0, int64_t size1, int64_t size2, float decay_rate, float eps,
-                         int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+int bn_fwd_train_impl(const void *x, const void *z, int relu, const float *gamma,
+                      const float *beta, void *y, float *batch_mean, float *batch_var,
+                      float *rmean, float *rvar, int64_t size0, int64_t size1, int64_t size2,
+                      float decay_rate, float eps, int dtype, void *workspace,
+                      size_t workspace_bytes, void *stream) {
   if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
   const int d = check_dims3(size0, size1, size2);
   if (d) return d < 0 ? d : 0;
@@ -90,18 +89,22 @@ int nblahip_bn_fwd_train(const void *x, const float *gamma, const float *beta, v
   p.eps = eps;
   p.ws = workspace;
   p.ws_bytes = workspace_bytes;
+  p.relu = relu;
+  p.z = z;
   return launch_bn_fwd_train(p, as_stream(stream));
 }
 
-int nblahip_bn_bwd(const void *x, const void *dy, const float *gamma, const float *mean,
-                   const float *var, const float *dmean, const float *dvar, void *dx,
-                   float *dgamma, float *dbeta, int accum_dx, int accum_dgamma, int accum_dbeta,
-                   int64_t size0, int64_t size1, int64_t size2, float eps, int batch_stat,
-                   int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+int bn_bwd_impl(int fused, const void *x, const void *y_out, const void *dy, const float *gamma,
+                const float *mean, const float *var, const float *dmean, const float *dvar,
+                void *dx, void *dz, float *dgamma, float *dbeta, int accum_dx, int accum_dz,
+                int accum_dgamma, int accum_dbeta, int64_t size0, int64_t size1, int64_t size2,
+                float eps, int batch_stat, int dtype, void *workspace, size_t workspace_bytes,
+                void *stream) {
   if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
   const int d = check_dims3(size0, size1, size2);
   if (d) return d < 0 ? d : 0;
   if (!x || !dy || !mean || !var) return NBLAHIP_EINVAL;
+  if (fused ? !y_out : (y_out || dz)) return NBLAHIP_EINVAL;
   if (int e = check_ws(workspace, workspace_bytes, bn_workspace_bytes(size0, size1, size2, dtype)))
     return e;
   BnProblem p;
@@ -126,7 +129,73 @@ int nblahip_bn_bwd(const void *x, const void *dy, const float *gamma, const floa
   p.eps = eps;
   p.ws = workspace;
   p.ws_bytes = workspace_bytes;
+  p.y = y_out;
+  p.dz = dz;
+  p.accum_dz = accum_dz;
   return launch_bn_bwd(p, as_stream(stream));
+}
+} // namespace
+
+extern "C" {
+
+int nblahip_bn_fwd_infer(const void *x, const float *rmean, const float *rvar,
+                         const float *gamma, const float *beta, void *y, int64_t size0,
+                         int64_t size1, int64_t size2, float eps, int dtype, void *stream) {
+  return bn_fwd_infer_impl(x, nullptr, 0, rmean, rvar, gamma, beta, y, size0, size1, size2, eps,
+                           dtype, stream);
+}
+
+size_t nblahip_bn_workspace_bytes(int64_t size0, int64_t size1, int64_t size2, int dtype) {
+  if (!dtype_ok(dtype) || check_dims3(size0, size1, size2) != 0) return 0;
+  return bn_workspace_bytes(size0, size1, size2, dtype);
+}
+
+int nblahip_bn_fwd_train(const void *x, const float *gamma, const float *beta, void *y,
+                         float *batch_mean, float *batch_var, float *rmean, float *rvar,
+                         int64_t size0, int64_t size1, int64_t size2, float decay_rate, float eps,
+                         int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+  return bn_fwd_train_impl(x, nullptr, 0, gamma, beta, y, batch_mean, batch_var, rmean, rvar,
+                           size0, size1, size2, decay_rate, eps, dtype, workspace,
+                           workspace_bytes, stream);
+}
+
+int nblahip_bn_bwd(const void *x, const void *dy, const float *gamma, const float *mean,
+                   const float *var, const float *dmean, const float *dvar, void *dx,
+                   float *dgamma, float *dbeta, int accum_dx, int accum_dgamma, int accum_dbeta,
+                   int64_t size0, int64_t size1, int64_t size2, float eps, int batch_stat,
+                   int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+  return bn_bwd_impl(0, x, nullptr, dy, gamma, mean, var, dmean, dvar, dx, nullptr, dgamma, dbeta,
+                     accum_dx, 0, accum_dgamma, accum_dbeta, size0, size1, size2, eps, batch_stat,
+                     dtype, workspace, workspace_bytes, stream);
+}
+
+int nblahip_fused_bn_fwd_infer(const void *x, const void *z, const float *rmean,
+                               const float *rvar, const float *gamma, const float *beta, void *y,
+                               int64_t size0, int64_t size1, int64_t size2, float eps, int dtype,
+                               void *stream) {
+  return bn_fwd_infer_impl(x, z, 1, rmean, rvar, gamma, beta, y, size0, size1, size2, eps, dtype,
+                           stream);
+}
+
+int nblahip_fused_bn_fwd_train(const void *x, const void *z, const float *gamma,
+                               const float *beta, void *y, float *batch_mean, float *batch_var,
+                               float *rmean, float *rvar, int64_t size0, int64_t size1,
+                               int64_t size2, float decay_rate, float eps, int dtype,
+                               void *workspace, size_t workspace_bytes, void *stream) {
+  return bn_fwd_train_impl(x, z, 1, gamma, beta, y, batch_mean, batch_var, rmean, rvar, size0,
+                           size1, size2, decay_rate, eps, dtype, workspace, workspace_bytes,
+                           stream);
+}
+
+int nblahip_fused_bn_bwd(const void *x, const void *y, const void *dy, const float *gamma,
+                         const float *mean, const float *var, const float *dmean,
+                         const float *dvar, void *dx, void *dz, float *dgamma, float *dbeta,
+                         int accum_dx, int accum_dz, int accum_dgamma, int accum_dbeta,
+                         int64_t size0, int64_t size1, int64_t size2, float eps, int batch_stat,
+                         int dtype, void *workspace, size_t workspace_bytes, void *stream) {
+  return bn_bwd_impl(1, x, y, dy, gamma, mean, var, dmean, dvar, dx, dz, dgamma, dbeta, accum_dx,
+                     accum_dz, accum_dgamma, accum_dbeta, size0, size1, size2, eps, batch_stat,
+                     dtype, workspace, workspace_bytes, stream);
 }
 
 // ----------------------------------------------------------------------------

@@ -363,17 +363,23 @@ struct BnParamSrc {
 // Forward apply, planes layout, flattened over all vectors of the tensor.
 // plane = i / nvp, c = plane % C.
 // ---------------------------------------------------------------------------
-template <typename T, int VEC>
+// FUSE (FusedBatchNormalization): 0 plain, 1 y = max(0, bn), 2 y = max(0, bn + z).
+template <typename T, int VEC, int FUSE = 0>
 __global__ void __launch_bounds__(256)
 bn_apply_planes_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
-                       FastDiv nvp, FastDiv cdiv, uint32_t total_vec) {
+                       FastDiv nvp, FastDiv cdiv, uint32_t total_vec,
+                       const T *__restrict__ z) {
   for (uint32_t i0 = blockIdx.x * (256u * kBnUnroll) + threadIdx.x; i0 < total_vec;
        i0 += gridDim.x * (256u * kBnUnroll)) {
     float v[kBnUnroll][VEC];
+    float zv[FUSE == 2 ? kBnUnroll : 1][VEC];
 #pragma unroll
     for (int u = 0; u < kBnUnroll; ++u) {
       const uint32_t i = i0 + u * 256u;
-      if (i < total_vec) load_vec<T, VEC>(x + static_cast<size_t>(i) * VEC, v[u]);
+      if (i < total_vec) {
+        load_vec<T, VEC>(x + static_cast<size_t>(i) * VEC, v[u]);
+        if constexpr (FUSE == 2) load_vec<T, VEC>(z + static_cast<size_t>(i) * VEC, zv[u]);
+      }
     }
 #pragma unroll
     for (int u = 0; u < kBnUnroll; ++u) {
@@ -393,6 +399,14 @@ bn_apply_planes_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc sr
 #pragma unroll
           for (int j = 0; j < VEC; ++j) o[j] = (v[u][j] - q.mean) * q.a + q.b;
         }
+        if constexpr (FUSE == 2) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) o[j] += zv[u][j];
+        }
+        if constexpr (FUSE != 0) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) o[j] = fmaxf(0.f, o[j]);
+        }
         store_vec<T, VEC>(y + static_cast<size_t>(i) * VEC, o);
       }
     }
@@ -403,13 +417,14 @@ bn_apply_planes_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc sr
 // Forward apply, channel-last with ncv = C/VEC dividing 256: a thread always
 // meets the same VEC channels, so their parameters live in registers.
 // ---------------------------------------------------------------------------
-template <typename T, int VEC>
+template <typename T, int VEC, int FUSE = 0>
 __global__ void __launch_bounds__(256)
 bn_apply_cl_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
-                   uint32_t ncv, uint32_t total_vec) {
+                   uint32_t ncv, uint32_t total_vec, const T *__restrict__ z, float one) {
   // blockIdx.y: slab (sample) index; each slab has its own ncv*VEC parameters.
   x += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
   y += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
+  if constexpr (FUSE == 2) z += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
   if (src.params) src.params += static_cast<size_t>(blockIdx.y) * ncv * VEC;
   const uint32_t cv = threadIdx.x % ncv;
   // y = x*pa + ps with ps = pb - mean*pa for half output (one mixed fma per
@@ -425,10 +440,12 @@ bn_apply_cl_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
   for (uint32_t i0 = blockIdx.x * (256u * kBnUnroll) + threadIdx.x; i0 < total_vec;
        i0 += gridDim.x * (256u * kBnUnroll)) {
     RawVec<T, VEC> raw[kBnUnroll];
+    RawVec<T, VEC> zr[FUSE == 2 ? kBnUnroll : 1];
 #pragma unroll
     for (int u = 0; u < kBnUnroll; ++u) {
       const uint32_t i = min(i0 + u * 256u, total_vec - 1); // clamped: loads stay branch-free
       raw[u] = load_raw<T, VEC>(x + static_cast<size_t>(i) * VEC);
+      if constexpr (FUSE == 2) zr[u] = load_raw<T, VEC>(z + static_cast<size_t>(i) * VEC);
     }
 #pragma unroll
     for (int u = 0; u < kBnUnroll; ++u) {
@@ -442,6 +459,8 @@ bn_apply_cl_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
           } else {
             o[j] = (elem_fma<T, VEC>(raw[u], j, 1.0f, 0.f) - pm[j]) * pa[j] + pb[j];
           }
+          if constexpr (FUSE == 2) o[j] = elem_fma<T, VEC>(zr[u], j, one, o[j]);
+          if constexpr (FUSE != 0) o[j] = fmaxf(0.f, o[j]);
         }
         store_vec<T, VEC>(y + static_cast<size_t>(i) * VEC, o);
       }
@@ -453,12 +472,13 @@ bn_apply_cl_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
 // Backward reduction, planes layout.  part2[C][S][2] = (sum dy*(x-mean), sum dy).
 // DIRECT as in bn_stats_planes_kernel.
 // ---------------------------------------------------------------------------
-template <typename T, int VEC, int BLOCK, bool DIRECT>
+// FUSED (FusedBatchNormalization): dy is first masked by y > 0 (ReLU backward).
+template <typename T, int VEC, int BLOCK, bool DIRECT, bool FUSED = false>
 __global__ void __launch_bounds__(BLOCK)
 bn_bwd_reduce_planes_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                             const float *__restrict__ mean, uint32_t C, FastDiv nvp,
                             uint32_t vpc, uint32_t chunk, float one, float *__restrict__ part2,
-                            BnBwdFinal fin) {
+                            BnBwdFinal fin, const T *__restrict__ y) {
   __shared__ float lds[2 * (BLOCK / kWave)];
   const uint32_t c = blockIdx.x;
   const uint32_t s = blockIdx.y;
@@ -469,6 +489,7 @@ bn_bwd_reduce_planes_kernel(const T *__restrict__ x, const T *__restrict__ dy,
   float sdx = 0.f, sdy = 0.f;
   for (uint32_t v0 = begin + threadIdx.x; v0 < end; v0 += BLOCK * kBnUnroll) {
     RawVec<T, VEC> xr[kBnUnroll], dr[kBnUnroll];
+    RawVec<T, VEC> yr[FUSED ? kBnUnroll : 1];
     // all loads first (indices past the end re-read v0), selects after
 #pragma unroll
     for (int u = 0; u < kBnUnroll; ++u) {
@@ -476,9 +497,14 @@ bn_bwd_reduce_planes_kernel(const T *__restrict__ x, const T *__restrict__ dy,
       const size_t off = bn_plane_offset(v < end ? v : v0, c, C, nvp) * VEC;
       xr[u] = load_raw<T, VEC>(x + off);
       dr[u] = load_raw<T, VEC>(dy + off);
+      if constexpr (FUSED) yr[u] = load_raw<T, VEC>(y + off);
     }
 #pragma unroll
     for (int u = 0; u < kBnUnroll; ++u) dr[u] = raw_or_zero<T, VEC>(v0 + u * BLOCK < end, dr[u]);
+    if constexpr (FUSED) {
+#pragma unroll
+      for (int u = 0; u < kBnUnroll; ++u) dr[u] = raw_relu_mask<T, VEC>(dr[u], yr[u]);
+    }
 #pragma unroll
     for (int u = 0; u < kBnUnroll; ++u) {
       sdy = raw_sum<T, VEC>(dr[u], sdy);
@@ -504,13 +530,13 @@ bn_bwd_reduce_planes_kernel(const T *__restrict__ x, const T *__restrict__ dy,
 // ---------------------------------------------------------------------------
 // Backward reduction, channel-last.  Same thread layout as bn_stats_cl_kernel.
 // ---------------------------------------------------------------------------
-template <typename T, int VEC>
+template <typename T, int VEC, bool FUSED = false>
 __global__ void __launch_bounds__(kBnBlock)
 bn_bwd_reduce_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                         const float *__restrict__ mean, uint32_t M, uint32_t C,
                         uint32_t ncv, uint32_t log2tx, uint32_t rps, float one,
                         float *__restrict__ part2 /*[C][S][2]*/, uint32_t mean_slab_stride,
-                        FastDiv cpg) {
+                        FastDiv cpg, const T *__restrict__ y) {
   __shared__ float lsdx[kBnBlock * VEC];
   __shared__ float lsdy[kBnBlock * VEC];
   const uint32_t TX = 1u << log2tx;
@@ -547,6 +573,7 @@ bn_bwd_reduce_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
   if (active) {
     for (uint32_t r0 = rbegin + ty; r0 < rend; r0 += TY * kBnUnroll) {
       RawVec<T, VEC> xr[kBnUnroll], dr[kBnUnroll];
+      RawVec<T, VEC> yr[FUSED ? kBnUnroll : 1];
       // All loads first (rows beyond the split re-read row r0), selects after:
       // the eight loads are in flight together.
 #pragma unroll
@@ -555,10 +582,15 @@ bn_bwd_reduce_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
         const size_t off = static_cast<size_t>(r < rend ? r : r0) * C + static_cast<size_t>(cv) * VEC;
         xr[u] = load_raw<T, VEC>(x + off);
         dr[u] = load_raw<T, VEC>(dy + off);
+        if constexpr (FUSED) yr[u] = load_raw<T, VEC>(y + off);
       }
 #pragma unroll
       for (int u = 0; u < kBnUnroll; ++u) // dy zeroed beyond the split: adds nothing
         dr[u] = raw_or_zero<T, VEC>(r0 + u * TY < rend, dr[u]);
+      if constexpr (FUSED) {
+#pragma unroll
+        for (int u = 0; u < kBnUnroll; ++u) dr[u] = raw_relu_mask<T, VEC>(dr[u], yr[u]);
+      }
 #pragma unroll
       for (int u = 0; u < kBnUnroll; ++u)
 #pragma unroll
@@ -611,27 +643,50 @@ bn_finalize_bwd_kernel(const float *__restrict__ part2, uint32_t S, BnBwdFinal f
 // ---------------------------------------------------------------------------
 // Backward apply: dx = a*dy + b*(x-mean) + c (+ dx).
 // ---------------------------------------------------------------------------
-template <typename T, int VEC>
+// FUSED (FusedBatchNormalization): dy is first masked by y > 0; the masked dy
+// is also the gradient of the residual input z (dz, optional).  dx may be
+// null when FUSED (only dz wanted).
+template <typename T, int VEC, bool FUSED = false>
 __global__ void __launch_bounds__(256)
 bn_bwd_apply_planes_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                            T *__restrict__ dx, const BnParam *__restrict__ params,
-                           FastDiv nvp, FastDiv cdiv, uint32_t total_vec, int accum) {
+                           FastDiv nvp, FastDiv cdiv, uint32_t total_vec, int accum,
+                           const T *__restrict__ y, T *__restrict__ dz, int accum_dz) {
   constexpr int U = 2;
   for (uint32_t i0 = blockIdx.x * (256u * U) + threadIdx.x; i0 < total_vec;
        i0 += gridDim.x * (256u * U)) {
     float xv[U][VEC], dv[U][VEC];
+    float yv[FUSED ? U : 1][VEC];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t i = i0 + u * 256u;
       if (i < total_vec) {
         load_vec<T, VEC>(x + static_cast<size_t>(i) * VEC, xv[u]);
         load_vec<T, VEC>(dy + static_cast<size_t>(i) * VEC, dv[u]);
+        if constexpr (FUSED) load_vec<T, VEC>(y + static_cast<size_t>(i) * VEC, yv[u]);
       }
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t i = i0 + u * 256u;
       if (i < total_vec) {
+        if constexpr (FUSED) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) dv[u][j] = yv[u][j] > 0.f ? dv[u][j] : 0.f;
+          if (dz) {
+            float g[VEC];
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) g[j] = dv[u][j];
+            if (accum_dz) {
+              float old[VEC];
+              load_vec<T, VEC>(dz + static_cast<size_t>(i) * VEC, old);
+#pragma unroll
+              for (int j = 0; j < VEC; ++j) g[j] += old[j];
+            }
+            store_vec<T, VEC>(dz + static_cast<size_t>(i) * VEC, g);
+          }
+          if (!dx) continue;
+        }
         const uint32_t plane = nvp.div(i);
         const uint32_t c = plane - cdiv.div(plane) * cdiv.d;
         const BnParam q = params[c];
@@ -650,15 +705,20 @@ bn_bwd_apply_planes_kernel(const T *__restrict__ x, const T *__restrict__ dy,
   }
 }
 
-template <typename T, int VEC>
+template <typename T, int VEC, bool FUSED = false>
 __global__ void __launch_bounds__(256)
 bn_bwd_apply_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                        T *__restrict__ dx, const BnParam *__restrict__ params,
-                       uint32_t ncv, uint32_t total_vec, int accum) {
+                       uint32_t ncv, uint32_t total_vec, int accum, const T *__restrict__ y,
+                       T *__restrict__ dz, int accum_dz) {
   constexpr int U = 2;
   x += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
   dy += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
-  dx += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
+  if (!FUSED || dx) dx += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
+  if constexpr (FUSED) {
+    y += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
+    if (dz) dz += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
+  }
   params += static_cast<size_t>(blockIdx.y) * ncv * VEC;
   const uint32_t cv = threadIdx.x % ncv;
   // dx = pa*dy + pb*(x - mean) + pc = pa*dy + (pb*x + ps), ps = pc - pb*mean:
@@ -675,16 +735,38 @@ bn_bwd_apply_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
   for (uint32_t i0 = blockIdx.x * (256u * U) + threadIdx.x; i0 < total_vec;
        i0 += gridDim.x * (256u * U)) {
     RawVec<T, VEC> xr[U], dr[U];
+    RawVec<T, VEC> yr[FUSED ? U : 1];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t i = min(i0 + u * 256u, total_vec - 1);
       xr[u] = load_raw<T, VEC>(x + static_cast<size_t>(i) * VEC);
       dr[u] = load_raw<T, VEC>(dy + static_cast<size_t>(i) * VEC);
+      if constexpr (FUSED) yr[u] = load_raw<T, VEC>(y + static_cast<size_t>(i) * VEC);
+    }
+    if constexpr (FUSED) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) dr[u] = raw_relu_mask<T, VEC>(dr[u], yr[u]);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t i = i0 + u * 256u;
       if (i < total_vec) {
+        if constexpr (FUSED) {
+          if (dz) {
+            T *dzp = dz + static_cast<size_t>(i) * VEC;
+            if (accum_dz) {
+              float g[VEC], old[VEC];
+              unpack<T, VEC>(dr[u], g);
+              load_vec<T, VEC>(dzp, old);
+#pragma unroll
+              for (int j = 0; j < VEC; ++j) g[j] += old[j];
+              store_vec<T, VEC>(dzp, g);
+            } else {
+              store_raw<T, VEC>(dzp, dr[u]);
+            }
+          }
+          if (!dx) continue;
+        }
         float o[VEC];
 #pragma unroll
         for (int j = 0; j < VEC; ++j)

@@ -109,23 +109,33 @@ int apply_grid(uint32_t total_vec, int unroll, bool cl = false) {
   return static_cast<int>(std::max<uint64_t>(1, std::min<uint64_t>(blocks, cap)));
 }
 
-template <typename T, int VEC>
-int fwd_apply_t(const BnProblem &p, const BnPlan &pl, const BnParamSrc &src, hipStream_t st) {
+template <typename T, int VEC, int FUSE>
+int fwd_apply_fuse_t(const BnProblem &p, const BnPlan &pl, const BnParamSrc &src, hipStream_t st) {
   const T *x = static_cast<const T *>(p.x);
+  const T *z = static_cast<const T *>(p.z);
   T *y = static_cast<T *>(p.out);
   const uint64_t total = static_cast<uint64_t>(p.size0) * p.C * p.size2;
   const uint32_t total_vec = static_cast<uint32_t>(total / VEC);
   if (pl.channel_last && pl.cl_fast_apply) {
-    NBLAHIP_LAUNCH("bn_apply_cl_kernel", (bn_apply_cl_kernel<T, VEC>), dim3(apply_grid(total_vec, kBnUnroll, true)),
-                       dim3(256), 0, st, x, y, src, pl.ncv, total_vec);
+    NBLAHIP_LAUNCH(FUSE ? "bn_apply_cl_kernel_fused" : "bn_apply_cl_kernel",
+                   (bn_apply_cl_kernel<T, VEC, FUSE>), dim3(apply_grid(total_vec, kBnUnroll, true)),
+                   dim3(256), 0, st, x, y, src, pl.ncv, total_vec, z, 1.0f);
   } else {
     // channel-last without the register fast path: planes of one vector each.
     const uint32_t nvp = pl.channel_last ? 1u : pl.nvp;
-    NBLAHIP_LAUNCH("bn_apply_planes_kernel", (bn_apply_planes_kernel<T, VEC>), dim3(apply_grid(total_vec, kBnUnroll)),
-                       dim3(256), 0, st, x, y, src, FastDiv(nvp),
-                       FastDiv(static_cast<uint32_t>(p.C)), total_vec);
+    NBLAHIP_LAUNCH(FUSE ? "bn_apply_planes_kernel_fused" : "bn_apply_planes_kernel",
+                   (bn_apply_planes_kernel<T, VEC, FUSE>), dim3(apply_grid(total_vec, kBnUnroll)),
+                   dim3(256), 0, st, x, y, src, FastDiv(nvp), FastDiv(static_cast<uint32_t>(p.C)),
+                   total_vec, z);
   }
   return last_launch_status();
+}
+
+template <typename T, int VEC>
+int fwd_apply_t(const BnProblem &p, const BnPlan &pl, const BnParamSrc &src, hipStream_t st) {
+  if (!p.relu) return fwd_apply_fuse_t<T, VEC, 0>(p, pl, src, st);
+  return p.z ? fwd_apply_fuse_t<T, VEC, 2>(p, pl, src, st)
+             : fwd_apply_fuse_t<T, VEC, 1>(p, pl, src, st);
 }
 
 template <typename T, int VEC>
@@ -148,47 +158,69 @@ int stats_t(const BnProblem &p, const BnPlan &pl, float *part, const BnFwdFinal 
   return last_launch_status();
 }
 
+template <typename T, int VEC, bool FUSED>
+int bwd_reduce_fuse_t(const BnProblem &p, const BnPlan &pl, float *part2, const BnBwdFinal &fin,
+                      hipStream_t st) {
+  const T *x = static_cast<const T *>(p.x);
+  const T *dy = static_cast<const T *>(p.dy);
+  const T *y = static_cast<const T *>(p.y);
+  if (pl.channel_last) {
+    NBLAHIP_LAUNCH(FUSED ? "bn_bwd_reduce_cl_kernel_fused" : "bn_bwd_reduce_cl_kernel",
+                   (bn_bwd_reduce_cl_kernel<T, VEC, FUSED>), dim3(pl.ytiles, pl.S), dim3(kBnBlock),
+                   0, st, x, dy, p.mean, static_cast<uint32_t>(p.size0),
+                   static_cast<uint32_t>(p.C), pl.ncv, pl.log2tx, pl.rps, 1.0f, part2, 0u,
+                   FastDiv(1), y);
+  } else if (pl.direct) {
+    NBLAHIP_LAUNCH(FUSED ? "bn_bwd_reduce_planes_kernel_fused" : "bn_bwd_reduce_planes_kernel",
+                   (bn_bwd_reduce_planes_kernel<T, VEC, 1024, true, FUSED>),
+                   dim3(static_cast<uint32_t>(p.C), 1), dim3(1024), 0, st, x, dy, p.mean,
+                   static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, 1.0f, part2, fin,
+                   y);
+  } else {
+    NBLAHIP_LAUNCH(FUSED ? "bn_bwd_reduce_planes_kernel_fused" : "bn_bwd_reduce_planes_kernel",
+                   (bn_bwd_reduce_planes_kernel<T, VEC, kBnBlock, false, FUSED>),
+                   dim3(static_cast<uint32_t>(p.C), pl.S), dim3(kBnBlock), 0, st, x, dy, p.mean,
+                   static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, 1.0f, part2, fin,
+                   y);
+  }
+  return last_launch_status();
+}
+
 template <typename T, int VEC>
 int bwd_reduce_t(const BnProblem &p, const BnPlan &pl, float *part2, const BnBwdFinal &fin,
                  hipStream_t st) {
+  return p.y ? bwd_reduce_fuse_t<T, VEC, true>(p, pl, part2, fin, st)
+             : bwd_reduce_fuse_t<T, VEC, false>(p, pl, part2, fin, st);
+}
+
+template <typename T, int VEC, bool FUSED>
+int bwd_apply_fuse_t(const BnProblem &p, const BnPlan &pl, const BnParam *params, hipStream_t st) {
   const T *x = static_cast<const T *>(p.x);
   const T *dy = static_cast<const T *>(p.dy);
-  if (pl.channel_last) {
-    NBLAHIP_LAUNCH("bn_bwd_reduce_cl_kernel", (bn_bwd_reduce_cl_kernel<T, VEC>),
-                   dim3(pl.ytiles, pl.S), dim3(kBnBlock), 0, st, x, dy, p.mean,
-                   static_cast<uint32_t>(p.size0), static_cast<uint32_t>(p.C), pl.ncv, pl.log2tx,
-                   pl.rps, 1.0f, part2, 0u, FastDiv(1));
-  } else if (pl.direct) {
-    NBLAHIP_LAUNCH("bn_bwd_reduce_planes_kernel",
-                   (bn_bwd_reduce_planes_kernel<T, VEC, 1024, true>),
-                   dim3(static_cast<uint32_t>(p.C), 1), dim3(1024), 0, st, x, dy, p.mean,
-                   static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, 1.0f, part2, fin);
+  const T *y = static_cast<const T *>(p.y);
+  T *dx = static_cast<T *>(p.out);
+  T *dz = static_cast<T *>(p.dz);
+  const uint64_t total = static_cast<uint64_t>(p.size0) * p.C * p.size2;
+  const uint32_t total_vec = static_cast<uint32_t>(total / VEC);
+  if (pl.channel_last && pl.cl_fast_apply) {
+    NBLAHIP_LAUNCH(FUSED ? "bn_bwd_apply_cl_kernel_fused" : "bn_bwd_apply_cl_kernel",
+                   (bn_bwd_apply_cl_kernel<T, VEC, FUSED>), dim3(apply_grid(total_vec, 2, true)),
+                   dim3(256), 0, st, x, dy, dx, params, pl.ncv, total_vec, p.accum_dx, y, dz,
+                   p.accum_dz);
   } else {
-    NBLAHIP_LAUNCH("bn_bwd_reduce_planes_kernel",
-                   (bn_bwd_reduce_planes_kernel<T, VEC, kBnBlock, false>),
-                   dim3(static_cast<uint32_t>(p.C), pl.S), dim3(kBnBlock), 0, st, x, dy, p.mean,
-                   static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, 1.0f, part2, fin);
+    const uint32_t nvp = pl.channel_last ? 1u : pl.nvp;
+    NBLAHIP_LAUNCH(FUSED ? "bn_bwd_apply_planes_kernel_fused" : "bn_bwd_apply_planes_kernel",
+                   (bn_bwd_apply_planes_kernel<T, VEC, FUSED>), dim3(apply_grid(total_vec, 2)),
+                   dim3(256), 0, st, x, dy, dx, params, FastDiv(nvp),
+                   FastDiv(static_cast<uint32_t>(p.C)), total_vec, p.accum_dx, y, dz, p.accum_dz);
   }
   return last_launch_status();
 }
 
 template <typename T, int VEC>
 int bwd_apply_t(const BnProblem &p, const BnPlan &pl, const BnParam *params, hipStream_t st) {
-  const T *x = static_cast<const T *>(p.x);
-  const T *dy = static_cast<const T *>(p.dy);
-  T *dx = static_cast<T *>(p.out);
-  const uint64_t total = static_cast<uint64_t>(p.size0) * p.C * p.size2;
-  const uint32_t total_vec = static_cast<uint32_t>(total / VEC);
-  if (pl.channel_last && pl.cl_fast_apply) {
-    NBLAHIP_LAUNCH("bn_bwd_apply_cl_kernel", (bn_bwd_apply_cl_kernel<T, VEC>), dim3(apply_grid(total_vec, 2, true)), dim3(256),
-                       0, st, x, dy, dx, params, pl.ncv, total_vec, p.accum_dx);
-  } else {
-    const uint32_t nvp = pl.channel_last ? 1u : pl.nvp;
-    NBLAHIP_LAUNCH("bn_bwd_apply_planes_kernel", (bn_bwd_apply_planes_kernel<T, VEC>), dim3(apply_grid(total_vec, 2)),
-                       dim3(256), 0, st, x, dy, dx, params, FastDiv(nvp),
-                       FastDiv(static_cast<uint32_t>(p.C)), total_vec, p.accum_dx);
-  }
-  return last_launch_status();
+  return p.y ? bwd_apply_fuse_t<T, VEC, true>(p, pl, params, st)
+             : bwd_apply_fuse_t<T, VEC, false>(p, pl, params, st);
 }
 
 // Run fn<T, VEC>() for the plan's element type and vector width.
@@ -237,7 +269,7 @@ size_t bn_workspace_bytes(int64_t size0, int64_t C, int64_t size2, int dtype) {
 }
 
 int launch_bn_infer(const BnProblem &p, hipStream_t st) {
-  const bool al = aligned16(p.x) && aligned16(p.out);
+  const bool al = aligned16(p.x) && aligned16(p.out) && (!p.z || aligned16(p.z));
   const BnPlan pl = make_plan(p.size0, p.C, p.size2, p.dtype, al);
   BnParamSrc src{};
   src.params = nullptr;
@@ -250,7 +282,7 @@ int launch_bn_infer(const BnProblem &p, hipStream_t st) {
 }
 
 int launch_bn_fwd_train(const BnProblem &p, hipStream_t st) {
-  const bool al = aligned16(p.x) && aligned16(p.out);
+  const bool al = aligned16(p.x) && aligned16(p.out) && (!p.z || aligned16(p.z));
   const BnPlan pl = make_plan(p.size0, p.C, p.size2, p.dtype, al);
   float *part = static_cast<float *>(p.ws);
   BnParam *params = reinterpret_cast<BnParam *>(static_cast<char *>(p.ws) +
@@ -278,8 +310,9 @@ int launch_bn_fwd_train(const BnProblem &p, hipStream_t st) {
 }
 
 int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
-  if (!p.out && !p.dgamma && !p.dbeta) return 0;
-  const bool al = aligned16(p.x) && aligned16(p.dy) && (!p.out || aligned16(p.out));
+  if (!p.out && !p.dgamma && !p.dbeta && !p.dz) return 0;
+  const bool al = aligned16(p.x) && aligned16(p.dy) && (!p.out || aligned16(p.out)) &&
+                  (!p.y || aligned16(p.y)) && (!p.dz || aligned16(p.dz));
   const BnPlan pl = make_plan(p.size0, p.C, p.size2, p.dtype, al);
   float *part2 = static_cast<float *>(p.ws);
   BnParam *params = reinterpret_cast<BnParam *>(static_cast<char *>(p.ws) +
@@ -303,14 +336,14 @@ int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
   if (need_sums) {
     if (int e = do_bwd_reduce(p, pl, part2, fin, st)) return e;
   }
-  if (!need_sums || !pl.direct) {
+  if ((p.out || need_sums) && (!need_sums || !pl.direct)) {
     // Without the reduction (inference-mode dx only) S = 0 leaves the sums at zero.
     NBLAHIP_LAUNCH("bn_finalize_bwd_kernel", bn_finalize_bwd_kernel,
                    dim3(static_cast<uint32_t>(p.C)), dim3(kBnBlock), 0, st, part2,
                    need_sums ? pl.S : 0u, fin);
     if (int e = last_launch_status()) return e;
   }
-  if (p.out) return do_bwd_apply(p, pl, params, st);
+  if (p.out || p.dz) return do_bwd_apply(p, pl, params, st);
   return 0;
 }
 
@@ -392,7 +425,7 @@ int cl_apply_t(const ClProblem &p, const BnPlan &pl, const BnParam *params, hipS
     NBLAHIP_LAUNCH("bn_apply_cl_kernel", (bn_apply_cl_kernel<T, VEC>),
                    dim3(static_cast<uint32_t>(std::min(need, per_slab)), static_cast<uint32_t>(p.batch)),
                    dim3(256), 0, st, static_cast<const T *>(p.x), static_cast<T *>(p.out),
-                   param_src(params), pl.ncv, slab_vec);
+                   param_src(params), pl.ncv, slab_vec, static_cast<const T *>(nullptr), 1.0f);
   } else {
     const uint32_t total = static_cast<uint32_t>(slab * p.batch);
     NBLAHIP_LAUNCH("cl_slab_apply_kernel", (cl_slab_apply_kernel<T>),
@@ -410,7 +443,8 @@ int cl_bwd_reduce_t(const ClProblem &p, const BnPlan &pl, float *part2, hipStrea
                  dim3(pl.ytiles, pl.S, static_cast<uint32_t>(p.batch)), dim3(kBnBlock), 0, st,
                  static_cast<const T *>(p.x), static_cast<const T *>(p.dy), p.mean,
                  static_cast<uint32_t>(p.spatial), static_cast<uint32_t>(p.channels), pl.ncv,
-                 pl.log2tx, pl.rps, 1.0f, part2, static_cast<uint32_t>(p.groups), FastDiv(cpg));
+                 pl.log2tx, pl.rps, 1.0f, part2, static_cast<uint32_t>(p.groups), FastDiv(cpg),
+                 static_cast<const T *>(nullptr));
   return last_launch_status();
 }
 
@@ -425,7 +459,8 @@ int cl_bwd_apply_t(const ClProblem &p, const BnPlan &pl, const BnParam *params, 
     NBLAHIP_LAUNCH("bn_bwd_apply_cl_kernel", (bn_bwd_apply_cl_kernel<T, VEC>),
                    dim3(static_cast<uint32_t>(std::min(need, per_slab)), static_cast<uint32_t>(p.batch)),
                    dim3(256), 0, st, static_cast<const T *>(p.x), static_cast<const T *>(p.dy),
-                   static_cast<T *>(p.out), params, pl.ncv, slab_vec, p.accum_dx);
+                   static_cast<T *>(p.out), params, pl.ncv, slab_vec, p.accum_dx,
+                   static_cast<const T *>(nullptr), static_cast<T *>(nullptr), 0);
   } else {
     const uint32_t total = static_cast<uint32_t>(slab * p.batch);
     NBLAHIP_LAUNCH("cl_slab_bwd_apply_kernel", (cl_slab_bwd_apply_kernel<T>),

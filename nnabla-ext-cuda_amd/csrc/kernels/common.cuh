@@ -184,6 +184,43 @@ __device__ __forceinline__ RawVec<T, VEC> raw_or_zero(bool ok, RawVec<T, VEC> r)
   return r;
 }
 
+// 0xFFFF in each 16-bit half of the result whose half-precision value in w is
+// greater than zero (positive, not NaN), 0 elsewhere.  Per half: magnitude
+// != 0 (adding 0x7FFF carries into bit 15), magnitude <= 0x7C00 (0xFC00 minus
+// it keeps bit 15) and sign clear; neither step crosses the 16-bit boundary.
+__device__ __forceinline__ uint32_t half2_gt_zero_mask(uint32_t w) {
+  const uint32_t mag = w & 0x7FFF7FFFu;
+  const uint32_t bit = (mag + 0x7FFF7FFFu) & (0xFC00FC00u - mag) & ~w & 0x80008000u;
+  return (bit >> 15) * 0xFFFFu;
+}
+
+// ReLU backward on the storage format: dy where y > 0, zero elsewhere
+// (kernel_relu_backward, include/nbla/cuda/utils/relu.cuh:56-62).
+template <typename T, int VEC>
+__device__ __forceinline__ RawVec<T, VEC> raw_relu_mask(RawVec<T, VEC> dy, const RawVec<T, VEC> &y) {
+  if constexpr (VEC == 1) {
+    dy.v = to_f32<T>(y.v) > 0.f ? dy.v : from_f32<T>(0.f);
+  } else if constexpr (sizeof(T) == 4) {
+    dy.v.x = y.v.x > 0.f ? dy.v.x : 0.f; dy.v.y = y.v.y > 0.f ? dy.v.y : 0.f;
+    dy.v.z = y.v.z > 0.f ? dy.v.z : 0.f; dy.v.w = y.v.w > 0.f ? dy.v.w : 0.f;
+  } else {
+    dy.v.x &= half2_gt_zero_mask(y.v.x); dy.v.y &= half2_gt_zero_mask(y.v.y);
+    dy.v.z &= half2_gt_zero_mask(y.v.z); dy.v.w &= half2_gt_zero_mask(y.v.w);
+  }
+  return dy;
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void store_raw(T *__restrict__ p, const RawVec<T, VEC> &r) {
+  if constexpr (VEC == 1) {
+    p[0] = r.v;
+  } else if constexpr (sizeof(T) == 4) {
+    *reinterpret_cast<float4 *>(p) = r.v;
+  } else {
+    *reinterpret_cast<uint4 *>(p) = r.v;
+  }
+}
+
 // acc + sum of the VEC elements (fp32 accumulation).
 template <typename T, int VEC>
 __device__ __forceinline__ float raw_sum(const RawVec<T, VEC> &r, float acc) {

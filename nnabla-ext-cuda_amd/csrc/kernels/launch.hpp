@@ -89,6 +89,13 @@ struct BnProblem {
   float *dbeta = nullptr;
   int accum_dx = 0, accum_g = 0, accum_b = 0;
   int batch_stat = 1;
+  // FusedBatchNormalization: forward y = max(0, bn(x) [+ z]) when relu != 0;
+  // backward masks dy by y > 0 when y != null and writes the masked dy to dz.
+  int relu = 0;
+  const void *z = nullptr;
+  const void *y = nullptr;
+  void *dz = nullptr;
+  int accum_dz = 0;
   int64_t size0 = 1, C = 1, size2 = 1;
   float decay = 0.9f, eps = 1e-5f;
   void *ws = nullptr;

@@ -18,6 +18,9 @@ How each function is pinned (see tests/test_oracle_pins.py):
       -> torch CPU float64 F.batch_norm / layer_norm / group_norm /
          instance_norm + autograd (library routines), incl. the 3-output
          dmean/dvar terms through an autograd loss that consumes mean and var;
+  fused_bn_forward / fused_bn_backward
+      -> torch CPU float64 relu(F.batch_norm(x) + z) + autograd (training and
+         eval mode, with and without z);
   welford_update / welford_merge / welford_rows
       -> equality with the two-pass mean/variance, merge associativity,
          brute-force split enumeration on tiny inputs, n=0 identity;
@@ -197,6 +200,44 @@ def bn_backward_global(x, dy, gamma, rmean, rvar, axis=1, eps=1e-5):
     dgamma = (dy3 * (x3 - _bc(rmean, c, 0)) * inv).sum(axis=(0, 2))
     dbeta = dy3.sum(axis=(0, 2))
     return dx.reshape(shape), dgamma, dbeta
+
+
+# --------------------------------------------------------------------------
+# FusedBatchNormalization: y = relu(BatchNormalization(x) + z)
+# --------------------------------------------------------------------------
+def fused_bn_forward(x, z, beta, gamma, rmean, rvar, axis=1, decay_rate=0.9,
+                     eps=1e-5, batch_stat=True):
+    """BatchNormalization, then the residual add (add2.cuh:23-27) and
+    max(0, .) (relu.cuh:48-52); what cudnnBatchNormalizationForwardTrainingEx
+    computes with BN_ADD_ACTIVATION (cudnn/function/generic/
+    fused_batch_normalization.cu:136-216).  z None: BN_ACTIVATION.
+    Returns y, mean, var, new_rmean, new_rvar (statistics None when
+    batch_stat is false)."""
+    if batch_stat:
+        y, mean, var, nrm, nrv = bn_forward_batch(x, beta, gamma, rmean, rvar,
+                                                  axis, decay_rate, eps)
+    else:
+        y = bn_forward_global(x, beta, gamma, rmean, rvar, axis, eps)
+        mean = var = nrm = nrv = None
+    if z is not None:
+        y = y + _f64(z)
+    return np.maximum(y, 0.0), mean, var, nrm, nrv
+
+
+def fused_bn_backward(x, y, dy, gamma, mean, var, axis=1, eps=1e-5,
+                      batch_stat=True, dmean=None, dvar=None):
+    """relu_add2_backward (function/generic/fused_batch_normalization.cu:
+    47-75): g = dy where y > 0 else 0 (relu.cuh:56-62), dz = g (add2.cuh:
+    30-35), then the BatchNormalization backward of g.  Returns dx, dz,
+    dgamma, dbeta."""
+    g = np.where(_f64(y) > 0, _f64(dy), 0.0)
+    if batch_stat:
+        dx, dgamma, dbeta = bn_backward_batch(x, g, gamma, mean, var, axis,
+                                              eps, dmean, dvar)
+    else:
+        dx, dgamma, dbeta = bn_backward_global(x, g, gamma, mean, var, axis,
+                                               eps)
+    return dx, g, dgamma, dbeta
 
 
 # --------------------------------------------------------------------------

@@ -103,6 +103,50 @@ def test_bn_forward_global_vs_torch(shape, axis, no_scale, no_bias):
 
 
 @pytest.mark.parametrize("shape,axis", BN_CASES)
+@pytest.mark.parametrize("with_z", [True, False])
+@pytest.mark.parametrize("batch_stat", [True, False])
+def test_fused_bn_vs_torch_autograd(shape, axis, with_z, batch_stat):
+    """relu(batch_norm(x) + z) and its gradients w.r.t. x, z, gamma, beta from
+    torch float64 autograd, training and eval mode."""
+    rng = np.random.default_rng(31)
+    c = shape[axis]
+    if batch_stat and int(np.prod(shape)) // c < 2:
+        pytest.skip("degenerate")
+    x = rng.standard_normal(shape) * 2 + 1
+    z = rng.standard_normal(shape) if with_z else None
+    dy = rng.standard_normal(shape)
+    g = rng.uniform(0.5, 1.5, c)
+    b = rng.standard_normal(c)
+    rm = rng.standard_normal(c) * 0.3 + 1
+    rv = rng.uniform(1.0, 4.0, c)
+    y, mean, var, nrm, nrv = R.fused_bn_forward(x, z, b, g, rm, rv, axis, 0.9, 1e-5, batch_stat)
+    xt, gt, bt = T(x, True), T(g, True), T(b, True)
+    zt = T(z, True) if with_z else None
+    trm, trv = T(rm).clone(), T(rv).clone()
+    bn = F.batch_norm(torch.movedim(xt, axis, 1), trm, trv, gt, bt, batch_stat, 0.1, 1e-5)
+    pre = torch.movedim(bn, 1, axis)
+    if with_z:
+        pre = pre + zt
+    yt = torch.relu(pre)
+    close(y, yt.detach().numpy())
+    if c > 1:
+        assert (y > 0).any() and (y == 0).any()  # both branches of the ReLU occur
+    if batch_stat:
+        close(nrm, trm.numpy())
+        close(nrv, trv.numpy())
+    (yt * T(dy)).sum().backward()
+    st_m, st_v = (mean, var) if batch_stat else (rm, rv)
+    dx, dz, dg, db = R.fused_bn_backward(x, y, dy, g, st_m, st_v, axis, 1e-5, batch_stat)
+    close(dx, xt.grad.numpy(), rtol=1e-9, atol=1e-9)
+    close(dg, gt.grad.numpy(), rtol=1e-9, atol=1e-9)
+    close(db, bt.grad.numpy(), rtol=1e-9, atol=1e-9)
+    if with_z:
+        close(dz, zt.grad.numpy())
+    # dz is dy gated by the sign of the OUTPUT (relu.cuh:59-61)
+    np.testing.assert_array_equal(dz, np.where(y > 0, dy, 0.0))
+
+
+@pytest.mark.parametrize("shape,axis", BN_CASES)
 @pytest.mark.parametrize("decay", [0.9, 0.5])
 def test_bn_forward_batch_vs_torch(shape, axis, decay):
     rng = np.random.default_rng(11)
