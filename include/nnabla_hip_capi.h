@@ -52,6 +52,11 @@ NNABLA_HIP_EXPORT int nnabla_hip_variable_fill(nnabla_hip_variable *v, int which
 NNABLA_HIP_EXPORT nnabla_hip_function *nnabla_hip_create_batch_normalization(
     const char *backends, const char *array_class, const char *device_id, const int *axes,
     int n_axes, float decay_rate, float eps, int batch_stat, int no_scale, int no_bias);
+/* inputs [x, beta, gamma, mean, var] or [x, beta, gamma, mean, var, z];
+ * nonlinearity must be "relu". */
+NNABLA_HIP_EXPORT nnabla_hip_function *nnabla_hip_create_fused_batch_normalization(
+    const char *backends, const char *array_class, const char *device_id, const int *axes,
+    int n_axes, float decay_rate, float eps, int batch_stat, const char *nonlinearity);
 NNABLA_HIP_EXPORT nnabla_hip_function *nnabla_hip_create_layer_normalization(
     const char *backends, const char *array_class, const char *device_id, const int *batch_axis,
     int n_batch_axis, float eps, int no_scale, int no_bias);

@@ -36,6 +36,7 @@ SIGNATURES = {
     "nnabla_hip_variable_zero": (_I, [_P, _I]),
     "nnabla_hip_variable_fill": (_I, [_P, _I, _F]),
     "nnabla_hip_create_batch_normalization": (_P, [_S, _S, _S, _IP, _I, _F, _F, _I, _I, _I]),
+    "nnabla_hip_create_fused_batch_normalization": (_P, [_S, _S, _S, _IP, _I, _F, _F, _I, _S]),
     "nnabla_hip_create_layer_normalization": (_P, [_S, _S, _S, _IP, _I, _F, _I, _I]),
     "nnabla_hip_create_group_normalization": (_P, [_S, _S, _S, _I, _I, _IP, _I, _F, _I, _I]),
     "nnabla_hip_create_instance_normalization": (_P, [_S, _S, _S, _I, _IP, _I, _F, _I, _I]),
@@ -199,6 +200,13 @@ def BatchNormalization(ctx, axes=(1,), decay_rate=0.9, eps=1e-5, batch_stat=True
     ax, n = _ints(list(axes))
     return Function(lib().nnabla_hip_create_batch_normalization(
         *_ctx_args(ctx), ax, n, decay_rate, eps, int(batch_stat), int(no_scale), int(no_bias)))
+
+
+def FusedBatchNormalization(ctx, axes=(1,), decay_rate=0.9, eps=1e-5, batch_stat=True,
+                            nonlinearity="relu"):
+    ax, n = _ints(list(axes))
+    return Function(lib().nnabla_hip_create_fused_batch_normalization(
+        *_ctx_args(ctx), ax, n, decay_rate, eps, int(batch_stat), nonlinearity.encode()))
 
 
 def LayerNormalization(ctx, batch_axis=(0,), eps=1e-5, no_scale=False, no_bias=False):

@@ -3,6 +3,7 @@
 
 #include <nbla/cpu.hpp>
 #include <nbla/function/batch_normalization.hpp>
+#include <nbla/function/fused_batch_normalization.hpp>
 #include <nbla/function/group_normalization.hpp>
 #include <nbla/function/instance_normalization.hpp>
 #include <nbla/function/layer_normalization.hpp>
@@ -190,6 +191,19 @@ nnabla_hip_function *nnabla_hip_create_batch_normalization(const char *backends,
     const vector<int> ax(axes, axes + n_axes);
     out = wrap(create_BatchNormalization(make_ctx(backends, array_class, device_id), ax, decay_rate,
                                          eps, batch_stat != 0, no_scale != 0, no_bias != 0));
+  });
+  return out;
+}
+
+nnabla_hip_function *nnabla_hip_create_fused_batch_normalization(
+    const char *backends, const char *array_class, const char *device_id, const int *axes,
+    int n_axes, float decay_rate, float eps, int batch_stat, const char *nonlinearity) {
+  nnabla_hip_function *out = nullptr;
+  guarded([&] {
+    const vector<int> ax(axes, axes + n_axes);
+    out = wrap(create_FusedBatchNormalization(make_ctx(backends, array_class, device_id), ax,
+                                              decay_rate, eps, batch_stat != 0,
+                                              string(nonlinearity ? nonlinearity : "")));
   });
   return out;
 }

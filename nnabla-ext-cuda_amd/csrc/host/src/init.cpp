@@ -1,5 +1,5 @@
 // init_hip(): registration of the "hip" backend (src/nbla/cuda/init.cpp.tmpl:65-270
-// is the reference's equivalent; here the table is four functions by two type
+// is the reference's equivalent; here the table is five functions by two type
 // configs, written out by hand instead of generated from yaml).
 #include <mutex>
 
@@ -7,6 +7,7 @@
 #include <nbla/function_registry.hpp>
 #include <nbla/hip/array/hip_array.hpp>
 #include <nbla/hip/function/batch_normalization.hpp>
+#include <nbla/hip/function/fused_batch_normalization.hpp>
 #include <nbla/hip/function/group_normalization.hpp>
 #include <nbla/hip/function/instance_normalization.hpp>
 #include <nbla/hip/function/layer_normalization.hpp>
@@ -18,6 +19,8 @@ namespace nbla {
 #ifdef NBLA_HIP_USE_CORE_STANDIN
 // With the real core these registries live in libnnabla.
 NBLA_REGISTER_FUNCTION_SOURCE(BatchNormalization, const vector<int> &, float, float, bool, bool, bool);
+NBLA_REGISTER_FUNCTION_SOURCE(FusedBatchNormalization, const vector<int> &, float, float, bool,
+                              const string &);
 NBLA_REGISTER_FUNCTION_SOURCE(LayerNormalization, const vector<int> &, float, bool, bool);
 NBLA_REGISTER_FUNCTION_SOURCE(GroupNormalization, int, int, const vector<int> &, float, bool, bool);
 NBLA_REGISTER_FUNCTION_SOURCE(InstanceNormalization, int, const vector<int> &, float, bool, bool);
@@ -56,6 +59,13 @@ void init_hip() {
                               const vector<int> &, float, float, bool, bool, bool);
   NBLA_REGISTER_FUNCTION_IMPL(BatchNormalization, BatchNormalizationHip_half, "hip:half",
                               const vector<int> &, float, float, bool, bool, bool);
+  typedef FusedBatchNormalizationHip<float> FusedBatchNormalizationHip_float;
+  typedef FusedBatchNormalizationHip<Half> FusedBatchNormalizationHip_half;
+  NBLA_REGISTER_FUNCTION_IMPL(FusedBatchNormalization, FusedBatchNormalizationHip_float,
+                              "hip:float", const vector<int> &, float, float, bool,
+                              const string &);
+  NBLA_REGISTER_FUNCTION_IMPL(FusedBatchNormalization, FusedBatchNormalizationHip_half, "hip:half",
+                              const vector<int> &, float, float, bool, const string &);
   typedef LayerNormalizationHip<float> LayerNormalizationHip_float;
   typedef LayerNormalizationHip<Half> LayerNormalizationHip_half;
   NBLA_REGISTER_FUNCTION_IMPL(LayerNormalization, LayerNormalizationHip_float, "hip:float",

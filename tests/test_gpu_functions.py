@@ -140,6 +140,80 @@ def test_batch_normalization_inference(tc):
 
 
 @pytest.mark.parametrize("tc", CONFIGS)
+@pytest.mark.parametrize("shape,axis", [((4, 8, 7, 7), 1), ((4, 7, 7, 16), 3)])
+@pytest.mark.parametrize("with_z", [True, False])
+def test_fused_batch_normalization(tc, shape, axis, with_z):
+    """y = relu(bn(x) + z): forward with running-stat update, recompute,
+    backward to x, beta, gamma and z, accumulation on z."""
+    rng = np.random.default_rng(21)
+    half = tc == "half"
+    c = shape[axis]
+    pshape = tuple(c if i == axis else 1 for i in range(len(shape)))
+    x = rnd(rng.standard_normal(shape) * 2 + 1, tc)
+    z = rnd(rng.standard_normal(shape), tc)
+    dy = rnd(rng.standard_normal(shape), tc)
+    g = rng.uniform(0.5, 1.5, pshape).astype(np.float32)
+    b = (rng.standard_normal(pshape) * 0.3).astype(np.float32)
+    rm, rv = np.zeros(pshape, np.float32), np.ones(pshape, np.float32)
+    f = B.FusedBatchNormalization(B.context(tc), axes=[axis], decay_rate=0.9, eps=1e-5,
+                                  batch_stat=True, nonlinearity="relu")
+    assert f.name == "FusedBatchNormalizationHip"
+    vx, vb, vg, vm, vv, vz = var(x, half), var(b), var(g), var(rm), var(rv), var(z, half)
+    ins = [vx, vb, vg, vm, vv] + ([vz] if with_z else [])
+    vy = B.Variable(shape)
+    f.setup(ins, [vy])
+    f.forward(ins, [vy])
+    y_r, m_r, v_r, rm_r, rv_r = R.fused_bn_forward(x, z if with_z else None, b, g, rm, rv, axis,
+                                                   0.9, 1e-5, True)
+    assert_close(vy.d, y_r, dn(tc), "y", "y")
+    assert_close(vm.d, rm_r, dn(tc), "stat", "running mean")
+    assert_close(vv.d, rv_r, dn(tc), "stat", "running var")
+    f.recompute(ins, [vy])
+    assert_close(vm.d, rm_r, dn(tc), "stat", "running mean after recompute")
+    y_gpu = vy.d.astype(np.float64)
+    vy.set_grad(dy, half)
+    n_in = len(ins)
+    pd = [1, 1, 1, 0, 0] + ([1] if with_z else [])
+    f.backward(ins, [vy], propagate_down=pd, accum=[0] * n_in)
+    dx_r, dz_r, dg_r, db_r = R.fused_bn_backward(x, y_gpu, dy, g, m_r, v_r, axis, 1e-5, True)
+    assert_close(vx.g, dx_r, dn(tc), "grad", "dx")
+    assert_close(vg.g, dg_r, dn(tc), "pgrad", "dgamma")
+    assert_close(vb.g, db_r, dn(tc), "pgrad", "dbeta")
+    if with_z:
+        np.testing.assert_array_equal(vz.g.astype(np.float64), dz_r)
+        f.backward(ins, [vy], propagate_down=[0, 0, 0, 0, 0, 1], accum=[0, 0, 0, 0, 0, 1])
+        assert_close(vz.g, 2 * dz_r, dn(tc), "grad", "dz accum")
+
+
+@pytest.mark.parametrize("tc", CONFIGS)
+def test_fused_batch_normalization_inference_and_errors(tc):
+    rng = np.random.default_rng(22)
+    half = tc == "half"
+    shape, axis, c = (4, 6, 5, 5), 1, 6
+    pshape = (1, c, 1, 1)
+    x = rnd(rng.standard_normal(shape), tc)
+    z = rnd(rng.standard_normal(shape), tc)
+    g = rng.uniform(0.5, 1.5, pshape).astype(np.float32)
+    b = (rng.standard_normal(pshape) * 0.3).astype(np.float32)
+    rm = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
+    rv = rng.uniform(0.5, 2, pshape).astype(np.float32)
+    f = B.FusedBatchNormalization(B.context(tc), axes=[axis], batch_stat=False)
+    ins = [var(x, half), var(b), var(g), var(rm), var(rv), var(z, half)]
+    vy = B.Variable(shape)
+    f.setup(ins, [vy])
+    f.forward(ins, [vy])
+    y_r, _, _, _, _ = R.fused_bn_forward(x, z, b, g, rm, rv, axis, 0.9, 1e-5, False)
+    assert_close(vy.d, y_r, dn(tc), "y", "y")
+    np.testing.assert_array_equal(ins[3].d, rm)
+    bad = B.FusedBatchNormalization(B.context(tc), axes=[axis], nonlinearity="tanh")
+    with pytest.raises(B.NblaError, match="relu"):
+        bad.setup(ins, [vy])
+    few = B.FusedBatchNormalization(B.context(tc), axes=[axis])
+    with pytest.raises(B.NblaError, match="at least 5 inputs"):
+        few.setup(ins[:3], [vy])
+
+
+@pytest.mark.parametrize("tc", CONFIGS)
 @pytest.mark.parametrize("shape,batch_axis", [((4, 6, 64), (0, 1)), ((8, 1000), (0,)), ((3, 5, 7, 16), (0,))])
 def test_layer_normalization(tc, shape, batch_axis):
     rng = np.random.default_rng(4)
