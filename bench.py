@@ -47,7 +47,7 @@ def _ws(nbytes):
     return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device="cuda")
 
 
-def make_bn(K, shape, axis, dtype, train, mean=0.0, std=1.0, outliers=False, seed=0):
+def make_bn(K, shape, axis, dtype, train, mean=0.0, std=1.0, outliers=False, seed=0, fused=False):
     import torch
     L = K.lib()
     g = torch.Generator(device="cuda").manual_seed(seed)
@@ -69,6 +69,27 @@ def make_bn(K, shape, axis, dtype, train, mean=0.0, std=1.0, outliers=False, see
     ws = _ws(L.nblahip_bn_workspace_bytes(s0, c, s2, dt))
     st = torch.cuda.current_stream().cuda_stream
     S = x.numel() * x.element_size()
+
+    if train and fused:
+        # FusedBatchNormalization: y = relu(bn(x) + z); backward also yields dz.
+        z = torch.randn(shape, device="cuda", generator=g).to(dtype)
+        dz = torch.empty_like(x)
+
+        def fwd():
+            K.check(L.nblahip_fused_bn_fwd_train(x.data_ptr(), z.data_ptr(), gamma.data_ptr(),
+                                                 beta.data_ptr(), y.data_ptr(), bm.data_ptr(),
+                                                 bv.data_ptr(), rm.data_ptr(), rv.data_ptr(), s0, c,
+                                                 s2, 0.9, 1e-5, dt, ws.data_ptr(), ws.numel(), st))
+
+        def bwd():
+            K.check(L.nblahip_fused_bn_bwd(x.data_ptr(), y.data_ptr(), dy.data_ptr(),
+                                           gamma.data_ptr(), bm.data_ptr(), bv.data_ptr(), None,
+                                           None, dx.data_ptr(), dz.data_ptr(), dg.data_ptr(),
+                                           db.data_ptr(), 0, 0, 0, 0, s0, c, s2, 1e-5, 1, dt,
+                                           ws.data_ptr(), ws.numel(), st))
+        # fwd: x (stats), x, z (apply), y; bwd: x, dy, y, dz (reduce), x, dz, dx (apply)
+        return fwd, bwd, 4 * S, 7 * S, (x, z, dy, gamma, beta, rm, rv, y, dx, dz, bm, bv, dg, db,
+                                        ws)
 
     if train:
         def fwd():
@@ -216,6 +237,7 @@ def config_table(K, steps, warmup):
         ("C4 GN fp16 NHWC [16,64,64,256] G=32", lambda: make_rows(K, "gn", (16, 64, 64, 256), torch.float16, 3, std=1.5, groups=32, channel_last=True)),
         ("C4 IN fp16 NHWC [16,64,64,256]", lambda: make_rows(K, "in", (16, 64, 64, 256), torch.float16, 3, std=1.5, channel_last=True)),
         ("C5 BN training fp16 NHWC [256,56,56,64]", lambda: make_bn(K, (256, 56, 56, 64), 3, torch.float16, True, outliers=True, seed=4)),
+        ("Fused BN+add+ReLU training fp16 NHWC [256,56,56,64]", lambda: make_bn(K, (256, 56, 56, 64), 3, torch.float16, True, outliers=True, seed=4, fused=True)),
     ]
     out = []
     for name, make in specs:

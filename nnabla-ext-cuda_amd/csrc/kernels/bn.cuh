@@ -472,13 +472,15 @@ bn_apply_cl_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
 // Backward reduction, planes layout.  part2[C][S][2] = (sum dy*(x-mean), sum dy).
 // DIRECT as in bn_stats_planes_kernel.
 // ---------------------------------------------------------------------------
-// FUSED (FusedBatchNormalization): dy is first masked by y > 0 (ReLU backward).
+// FUSED (FusedBatchNormalization): dy is first masked by y > 0 (ReLU backward);
+// the masked dy is stored to dz when dz != null (the gradient of the residual
+// input, which the apply step can then read in place of dy and y).
 template <typename T, int VEC, int BLOCK, bool DIRECT, bool FUSED = false>
 __global__ void __launch_bounds__(BLOCK)
 bn_bwd_reduce_planes_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                             const float *__restrict__ mean, uint32_t C, FastDiv nvp,
                             uint32_t vpc, uint32_t chunk, float one, float *__restrict__ part2,
-                            BnBwdFinal fin, const T *__restrict__ y) {
+                            BnBwdFinal fin, const T *__restrict__ y, T *__restrict__ dz) {
   __shared__ float lds[2 * (BLOCK / kWave)];
   const uint32_t c = blockIdx.x;
   const uint32_t s = blockIdx.y;
@@ -504,6 +506,13 @@ bn_bwd_reduce_planes_kernel(const T *__restrict__ x, const T *__restrict__ dy,
     if constexpr (FUSED) {
 #pragma unroll
       for (int u = 0; u < kBnUnroll; ++u) dr[u] = raw_relu_mask<T, VEC>(dr[u], yr[u]);
+      if (dz) {
+#pragma unroll
+        for (int u = 0; u < kBnUnroll; ++u) {
+          const uint32_t v = v0 + u * BLOCK;
+          if (v < end) store_raw<T, VEC>(dz + bn_plane_offset(v, c, C, nvp) * VEC, dr[u]);
+        }
+      }
     }
 #pragma unroll
     for (int u = 0; u < kBnUnroll; ++u) {
@@ -536,7 +545,7 @@ bn_bwd_reduce_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                         const float *__restrict__ mean, uint32_t M, uint32_t C,
                         uint32_t ncv, uint32_t log2tx, uint32_t rps, float one,
                         float *__restrict__ part2 /*[C][S][2]*/, uint32_t mean_slab_stride,
-                        FastDiv cpg, const T *__restrict__ y) {
+                        FastDiv cpg, const T *__restrict__ y, T *__restrict__ dz) {
   __shared__ float lsdx[kBnBlock * VEC];
   __shared__ float lsdy[kBnBlock * VEC];
   const uint32_t TX = 1u << log2tx;
@@ -590,6 +599,15 @@ bn_bwd_reduce_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
       if constexpr (FUSED) {
 #pragma unroll
         for (int u = 0; u < kBnUnroll; ++u) dr[u] = raw_relu_mask<T, VEC>(dr[u], yr[u]);
+        if (dz) {
+#pragma unroll
+          for (int u = 0; u < kBnUnroll; ++u) {
+            const uint32_t r = r0 + u * TY;
+            if (r < rend)
+              store_raw<T, VEC>(dz + static_cast<size_t>(r) * C + static_cast<size_t>(cv) * VEC,
+                                dr[u]);
+          }
+        }
       }
 #pragma unroll
       for (int u = 0; u < kBnUnroll; ++u)

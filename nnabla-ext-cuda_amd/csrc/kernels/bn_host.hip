@@ -158,30 +158,35 @@ int stats_t(const BnProblem &p, const BnPlan &pl, float *part, const BnFwdFinal 
   return last_launch_status();
 }
 
+// The reduction also stores the gated dy as dz when that is a plain store: the
+// apply step then reads dz in place of (dy, y).
+bool gate_in_reduce(const BnProblem &p) { return p.y && p.dz && !p.accum_dz; }
+
 template <typename T, int VEC, bool FUSED>
 int bwd_reduce_fuse_t(const BnProblem &p, const BnPlan &pl, float *part2, const BnBwdFinal &fin,
                       hipStream_t st) {
   const T *x = static_cast<const T *>(p.x);
   const T *dy = static_cast<const T *>(p.dy);
   const T *y = static_cast<const T *>(p.y);
+  T *dz = gate_in_reduce(p) ? static_cast<T *>(p.dz) : nullptr;
   if (pl.channel_last) {
     NBLAHIP_LAUNCH(FUSED ? "bn_bwd_reduce_cl_kernel_fused" : "bn_bwd_reduce_cl_kernel",
                    (bn_bwd_reduce_cl_kernel<T, VEC, FUSED>), dim3(pl.ytiles, pl.S), dim3(kBnBlock),
                    0, st, x, dy, p.mean, static_cast<uint32_t>(p.size0),
                    static_cast<uint32_t>(p.C), pl.ncv, pl.log2tx, pl.rps, 1.0f, part2, 0u,
-                   FastDiv(1), y);
+                   FastDiv(1), y, dz);
   } else if (pl.direct) {
     NBLAHIP_LAUNCH(FUSED ? "bn_bwd_reduce_planes_kernel_fused" : "bn_bwd_reduce_planes_kernel",
                    (bn_bwd_reduce_planes_kernel<T, VEC, 1024, true, FUSED>),
                    dim3(static_cast<uint32_t>(p.C), 1), dim3(1024), 0, st, x, dy, p.mean,
                    static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, 1.0f, part2, fin,
-                   y);
+                   y, dz);
   } else {
     NBLAHIP_LAUNCH(FUSED ? "bn_bwd_reduce_planes_kernel_fused" : "bn_bwd_reduce_planes_kernel",
                    (bn_bwd_reduce_planes_kernel<T, VEC, kBnBlock, false, FUSED>),
                    dim3(static_cast<uint32_t>(p.C), pl.S), dim3(kBnBlock), 0, st, x, dy, p.mean,
                    static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, 1.0f, part2, fin,
-                   y);
+                   y, dz);
   }
   return last_launch_status();
 }
@@ -343,6 +348,15 @@ int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
                    need_sums ? pl.S : 0u, fin);
     if (int e = last_launch_status()) return e;
   }
+  if (need_sums && gate_in_reduce(p)) {
+    // dz already holds the gated dy: a plain BatchNormalization apply over it.
+    if (!p.out) return 0;
+    BnProblem q = p;
+    q.dy = p.dz;
+    q.y = nullptr;
+    q.dz = nullptr;
+    return do_bwd_apply(q, pl, params, st);
+  }
   if (p.out || p.dz) return do_bwd_apply(p, pl, params, st);
   return 0;
 }
@@ -444,7 +458,7 @@ int cl_bwd_reduce_t(const ClProblem &p, const BnPlan &pl, float *part2, hipStrea
                  static_cast<const T *>(p.x), static_cast<const T *>(p.dy), p.mean,
                  static_cast<uint32_t>(p.spatial), static_cast<uint32_t>(p.channels), pl.ncv,
                  pl.log2tx, pl.rps, 1.0f, part2, static_cast<uint32_t>(p.groups), FastDiv(cpg),
-                 static_cast<const T *>(nullptr));
+                 static_cast<const T *>(nullptr), static_cast<T *>(nullptr));
   return last_launch_status();
 }
 
