@@ -47,7 +47,8 @@ def _ws(nbytes):
     return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device="cuda")
 
 
-def make_bn(K, shape, axis, dtype, train, mean=0.0, std=1.0, outliers=False, seed=0, fused=False):
+def make_bn(K, shape, axis, dtype, train, mean=0.0, std=1.0, outliers=False, seed=0, fused=False,
+            stream=None):
     import torch
     L = K.lib()
     g = torch.Generator(device="cuda").manual_seed(seed)
@@ -67,7 +68,7 @@ def make_bn(K, shape, axis, dtype, train, mean=0.0, std=1.0, outliers=False, see
     s0, _, s2 = K._bn_sizes(shape, axis)
     dt = K._dtype_code(x)
     ws = _ws(L.nblahip_bn_workspace_bytes(s0, c, s2, dt))
-    st = torch.cuda.current_stream().cuda_stream
+    st = stream if stream is not None else torch.cuda.current_stream().cuda_stream
     S = x.numel() * x.element_size()
 
     if train and fused:
@@ -224,6 +225,27 @@ def time_calls(fns, steps, warmup):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
+def time_in_graph(K, calls, steps, warmup):
+    """Milliseconds per call of the C1 inference forward when `calls` of them
+    are captured into one graph and the graph is replayed."""
+    import torch
+    side = torch.cuda.Stream()
+    fn, _, _, _, keep = make_bn(K, (8, 64, 56, 56), 1, torch.float32, False, seed=0,
+                                stream=side.cuda_stream)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(calls):
+                fn()
+    ms = time_calls([graph.replay], max(1, steps // 4), max(1, warmup // 4)) / calls
+    del graph, keep
+    return ms
+
+
 def config_table(K, steps, warmup):
     """Every BASELINE configuration: us per call and algorithmic GB/s."""
     import torch
@@ -256,6 +278,9 @@ def config_table(K, steps, warmup):
             row["pct_of_hbm_peak"] = round((fb + bb) / ms_fb / 1e6 / HBM_PEAK_GBS * 100, 1)
         else:
             row["pct_of_hbm_peak"] = round(fb / ms_f / 1e6 / HBM_PEAK_GBS * 100, 1)
+            # A 13 MB pass is bounded by the cost of a dispatch: the same call
+            # replayed from a captured graph of 20 calls, per call.
+            row["fwd_us_in_graph"] = round(time_in_graph(K, 20, steps, warmup) * 1e3, 2)
         log("  ", json.dumps(row))
         out.append(row)
         del keep, fwd, bwd
