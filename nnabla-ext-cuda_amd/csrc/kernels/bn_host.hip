@@ -102,9 +102,11 @@ BnParamSrc param_src(const BnParam *params) {
 
 // Channel-last apply kernels load their per-channel parameters into registers
 // once per thread, so they run as a persistent grid (cl = true).
-int apply_grid(uint32_t total_vec, int unroll, bool cl = false) {
+int apply_grid(uint32_t total_vec, int unroll, bool cl = false, bool fwd = false) {
   const uint64_t blocks = (static_cast<uint64_t>(total_vec) + 256ull * unroll - 1) / (256ull * unroll);
-  const int per_cu = cl ? tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 4) : tune_int("BN_APPLY_BLOCKS_PER_CU", 0);
+  const int per_cu = !cl ? tune_int("BN_APPLY_BLOCKS_PER_CU", 0)
+                         : fwd ? tune_int("BN_CL_FWD_APPLY_BLOCKS_PER_CU", 2)
+                               : tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 4);
   const uint64_t cap = per_cu > 0 ? static_cast<uint64_t>(device_cus()) * per_cu : (1u << 20);
   return static_cast<int>(std::max<uint64_t>(1, std::min<uint64_t>(blocks, cap)));
 }
@@ -118,7 +120,7 @@ int fwd_apply_fuse_t(const BnProblem &p, const BnPlan &pl, const BnParamSrc &src
   const uint32_t total_vec = static_cast<uint32_t>(total / VEC);
   if (pl.channel_last && pl.cl_fast_apply) {
     NBLAHIP_LAUNCH(FUSE ? "bn_apply_cl_kernel_fused" : "bn_apply_cl_kernel",
-                   (bn_apply_cl_kernel<T, VEC, FUSE>), dim3(apply_grid(total_vec, kBnUnroll, true)),
+                   (bn_apply_cl_kernel<T, VEC, FUSE>), dim3(apply_grid(total_vec, kBnUnroll, true, true)),
                    dim3(256), 0, st, x, y, src, pl.ncv, total_vec, z, 1.0f);
   } else {
     // channel-last without the register fast path: planes of one vector each.
