@@ -258,7 +258,7 @@ bn_stats_cl_kernel(const T *__restrict__ x, uint32_t M, uint32_t C, uint32_t ncv
     lm2[(ty * TX + tx) * VEC + j] = m2[j];
   }
   ln[ty * TX + tx] = n;
-  __syncthreads();
+  lds_barrier();
   // Output o = tx*VEC + j of this block needs its TY row groups folded.  With
   // nout = TX*VEC outputs and 256 threads, Q = 256/nout threads share an
   // output: each folds TY/Q row groups in order, then the Q results are
@@ -278,7 +278,7 @@ bn_stats_cl_kernel(const T *__restrict__ x, uint32_t M, uint32_t C, uint32_t ncv
     l2[3 * threadIdx.x] = w.mean;
     l2[3 * threadIdx.x + 1] = w.m2;
     l2[3 * threadIdx.x + 2] = w.n;
-    __syncthreads();
+    lds_barrier();
     if (q == 0 && blockIdx.x * TX + otx < ncv) {
       for (uint32_t k = 1; k < Q; ++k) {
         const uint32_t t = k * nout + o;
@@ -624,7 +624,7 @@ bn_bwd_reduce_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
     lsdx[(ty * TX + tx) * VEC + j] = sdx[j];
     lsdy[(ty * TX + tx) * VEC + j] = sdy[j];
   }
-  __syncthreads();
+  lds_barrier();
   for (uint32_t o = threadIdx.x; o < TX * VEC; o += kBnBlock) {
     const uint32_t otx = o / VEC;
     const uint32_t ch = blockIdx.x * TX * VEC + o;

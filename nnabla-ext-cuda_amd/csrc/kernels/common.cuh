@@ -128,6 +128,18 @@ template <typename T, int VEC> __device__ __forceinline__ void keep_packed(RawVe
   }
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences
+// global memory, i.e. waits for every outstanding global load and store of the
+// wave (s_waitcnt vmcnt(0)) before the barrier: loads prefetched for the next
+// row and stores of the previous one would all have to land first.  No kernel
+// here communicates between threads through global memory, so the barriers
+// only need the LDS writes of each wave to have landed (s_waitcnt lgkmcnt(0)).
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // ---------------------------------------------------------------------------
 // Element access on packed vectors with the widening folded into the
 // arithmetic.  For half data, fma(float(h), a, b) with a half operand taken
@@ -316,9 +328,9 @@ __device__ __forceinline__ float row_sum(float v, float *lds) {
   } else {
     constexpr int NW = TPR / kWave;
     const int wave = threadIdx.x / kWave;
-    __syncthreads(); // previous readers of lds are done
+    lds_barrier(); // previous readers of lds are done
     if ((threadIdx.x & (kWave - 1)) == 0) lds[wave] = v;
-    __syncthreads();
+    lds_barrier();
     float total = 0.f;
 #pragma unroll
     for (int i = 0; i < NW; ++i) total += lds[i];
@@ -334,12 +346,12 @@ __device__ __forceinline__ void row_sum2(float &a, float &b, float *lds) {
   if constexpr (TPR > kWave) {
     constexpr int NW = TPR / kWave;
     const int wave = threadIdx.x / kWave;
-    __syncthreads();
+    lds_barrier();
     if ((threadIdx.x & (kWave - 1)) == 0) {
       lds[2 * wave] = a;
       lds[2 * wave + 1] = b;
     }
-    __syncthreads();
+    lds_barrier();
     float ta = 0.f, tb = 0.f;
 #pragma unroll
     for (int i = 0; i < NW; ++i) {
@@ -418,13 +430,13 @@ __device__ __forceinline__ Welford block_welford(Welford w, float *lds) {
   const int nw = blockDim.x / kWave;
   if (nw == 1) return w;
   const int wave = threadIdx.x / kWave;
-  __syncthreads();
+  lds_barrier();
   if ((threadIdx.x & (kWave - 1)) == 0) {
     lds[3 * wave] = w.mean;
     lds[3 * wave + 1] = w.m2;
     lds[3 * wave + 2] = w.n;
   }
-  __syncthreads();
+  lds_barrier();
   Welford t{lds[0], lds[1], lds[2]};
   for (int i = 1; i < nw; ++i)
     t = welford_merge(t, Welford{lds[3 * i], lds[3 * i + 1], lds[3 * i + 2]});
@@ -438,12 +450,12 @@ __device__ __forceinline__ void block_sum2(float &a, float &b, float *lds) {
   const int nw = blockDim.x / kWave;
   if (nw == 1) return;
   const int wave = threadIdx.x / kWave;
-  __syncthreads();
+  lds_barrier();
   if ((threadIdx.x & (kWave - 1)) == 0) {
     lds[2 * wave] = a;
     lds[2 * wave + 1] = b;
   }
-  __syncthreads();
+  lds_barrier();
   float ta = 0.f, tb = 0.f;
   for (int i = 0; i < nw; ++i) {
     ta += lds[2 * i];

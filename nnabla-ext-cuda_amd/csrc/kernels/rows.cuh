@@ -256,6 +256,19 @@ row_bwd_kernel(const RowArgs a) {
   for (int rr = CH ? sub : 0; rr < inner_n; rr += CH ? RPB : 1) {
     const int row = CH ? rr * channels + unit : unit;
     const size_t base = static_cast<size_t>(row) * a.R;
+    float gk[NL];                                   // per-load scalar gamma (IN / GN)
+    float gch = 1.f;                                // GN: gamma of channel threadIdx.x
+    if constexpr (MODE == kRowGN) {
+      // Issued ahead of the row data, so their latency hides behind it.
+      const uint32_t pb = (static_cast<uint32_t>(row) % a.pmod) * a.pmul;
+#pragma unroll
+      for (int k = 0; k < NL; ++k) {
+        const int col = (k * TPR + t) * VEC;
+        const uint32_t ch = (col < a.R) ? a.pdiv.div(static_cast<uint32_t>(col)) : 0u;
+        gk[k] = a.gamma ? a.gamma[pb + ch] : 1.f;
+      }
+      if (a.gamma && static_cast<int>(threadIdx.x) < a.cpg) gch = a.gamma[pb + threadIdx.x];
+    }
     RawVec<T, VEC> xr[NL], dr[NL];
 #pragma unroll
     for (int k = 0; k < NL; ++k) {
@@ -271,7 +284,6 @@ row_bwd_kernel(const RowArgs a) {
     const float nmi = -mean * istd;
 
     float s1 = 0.f, t2 = 0.f;
-    float gk[NL];                                   // per-load scalar gamma (IN / GN)
     float xh_keep[KEEP ? NL : 1][VEC], dg_keep[KEEP ? NL : 1][VEC];
     if constexpr (MODE == kRowLN) {
 #pragma unroll
@@ -323,7 +335,7 @@ row_bwd_kernel(const RowArgs a) {
       const int wave = threadIdx.x / kWave;
       const int lane = threadIdx.x & (kWave - 1);
       const uint32_t pbase = (static_cast<uint32_t>(row) % a.pmod) * a.pmul;
-      __syncthreads(); // part[] of the previous row has been consumed
+      lds_barrier(); // part[] of the previous row has been consumed
 #pragma unroll
       for (int k = 0; k < NL; ++k) {
         float sdy = raw_sum<T, VEC>(dr[k], 0.f);
@@ -340,11 +352,8 @@ row_bwd_kernel(const RowArgs a) {
           part[2 * e] = sdx;
           part[2 * e + 1] = sdy;
         }
-        const int col = (k * TPR + t) * VEC;
-        const uint32_t ch = (col < a.R) ? a.pdiv.div(static_cast<uint32_t>(col)) : 0u;
-        gk[k] = a.gamma ? a.gamma[pbase + ch] : 1.f;
       }
-      __syncthreads();
+      lds_barrier();
       // Channel c owns runs [c*epc, (c+1)*epc).
       float c1 = 0.f, c2 = 0.f;
       for (int c = threadIdx.x; c < a.cpg; c += TPR) {
@@ -356,7 +365,7 @@ row_bwd_kernel(const RowArgs a) {
         const size_t o = 2 * (static_cast<size_t>(row) * a.cpg + c);
         a.ws[o] = sdx;
         a.ws[o + 1] = sdy;
-        const float g = a.gamma ? a.gamma[pbase + c] : 1.f;
+        const float g = c < TPR ? gch : (a.gamma ? a.gamma[pbase + c] : 1.f);
         c1 += g * sdy;
         c2 += g * sdx;
       }
@@ -413,12 +422,12 @@ row_bwd_kernel(const RowArgs a) {
     // Fold the waves' shares in wave order and publish dgamma[c], dbeta[c].
     __shared__ float chfold[2 * 16];
     if constexpr (RPB > 1) {
-      __syncthreads();
+      lds_barrier();
       if (t == 0) {
         chfold[2 * sub] = ch_sdx;
         chfold[2 * sub + 1] = ch_sdy;
       }
-      __syncthreads();
+      lds_barrier();
       ch_sdx = 0.f;
       ch_sdy = 0.f;
 #pragma unroll
@@ -444,12 +453,12 @@ row_bwd_kernel(const RowArgs a) {
       for (int k = 0; k < NL; ++k) {
         float(&acc)[VEC] = (q == 0) ? acc_g[k] : acc_b[k];
         if constexpr (RPB > 1) {
-          __syncthreads();
+          lds_barrier();
           if (sub > 0) {
 #pragma unroll
             for (int j = 0; j < VEC; ++j) xwave[((sub - 1) * kWave + t) * VEC + j] = acc[j];
           }
-          __syncthreads();
+          lds_barrier();
           if (sub == 0) {
 #pragma unroll
             for (int r = 0; r < RPB - 1; ++r)

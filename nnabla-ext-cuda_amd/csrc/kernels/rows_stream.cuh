@@ -48,7 +48,7 @@ row_stats_stream_kernel(const T *__restrict__ x, int rows, int R, float inv_R,
       mean[row] = w.mean;
       var[row] = w.m2 * inv_R;
     }
-    __syncthreads();
+    lds_barrier();
   }
 }
 
@@ -115,7 +115,7 @@ ln_row_sums_stream_kernel(const T *__restrict__ x, const T *__restrict__ dy,
       rs[2 * static_cast<size_t>(row)] = s1;
       rs[2 * static_cast<size_t>(row) + 1] = t2;
     }
-    __syncthreads();
+    lds_barrier();
   }
 }
 
@@ -147,7 +147,7 @@ plane_sums_stream_kernel(const T *__restrict__ x, const T *__restrict__ dy,
       pairs[2 * static_cast<size_t>(p)] = sdx;
       pairs[2 * static_cast<size_t>(p) + 1] = sdy;
     }
-    __syncthreads();
+    lds_barrier();
   }
 }
 
@@ -246,7 +246,7 @@ ln_colgrad_stream_kernel(const T *__restrict__ x, const T *__restrict__ dy,
   }
   rg[py][cx] = sg;
   rb[py][cx] = sb;
-  __syncthreads();
+  lds_barrier();
   if (py == 0 && col < R) {
     float tg = 0.f, tb = 0.f;
 #pragma unroll
@@ -289,7 +289,7 @@ ln_param_reduce_kernel(const float *__restrict__ ws, int nparts, int R,
     }
   }
   red[py][cx] = s;
-  __syncthreads();
+  lds_barrier();
   if (py == 0 && col2 < 2 * R) {
     float tot = 0.f;
 #pragma unroll
