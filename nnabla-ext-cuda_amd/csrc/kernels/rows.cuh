@@ -74,6 +74,19 @@ template <int TPR, int MODE> struct RowBwdBlock {
   static constexpr int kRowsPerBlock = kBlock / TPR;
 };
 
+// Waves per SIMD the backward kernel must leave room for (second argument of
+// __launch_bounds__).  Two 512-thread blocks per CU need 4, i.e. at most 128
+// VGPRs; the layout named here would otherwise take a few registers more,
+// halve its occupancy and run a grid of two blocks per CU in two rounds
+// (GroupNormalization backward of 64 KB groups: 21.5 -> 17.1 us).  The
+// wave-per-row LayerNormalization float kernel (133 VGPRs) is left alone: the
+// spill the cap costs it sits in its row loop and is worth more than the
+// occupancy.
+template <typename T, int VEC, int NL, int TPR, int MODE> struct RowBwdOccupancy {
+  static constexpr bool kGn512 = MODE == kRowGN && TPR == 512 && NL == 8;
+  static constexpr int kMinWaves = kGn512 ? 4 : 1;
+};
+
 // ---------------------------------------------------------------------------
 // Forward: y, mean, var.  PERCOL selects the LayerNormalization parameter
 // layout (gamma/beta per column: loaded once per thread, before the row loop,
@@ -208,7 +221,8 @@ row_fwd_kernel(const RowArgs a) {
 // sum.
 // ---------------------------------------------------------------------------
 template <typename T, int VEC, int NL, int TPR, int MODE>
-__global__ void __launch_bounds__((RowBwdBlock<TPR, MODE>::kBlock))
+__global__ void __launch_bounds__((RowBwdBlock<TPR, MODE>::kBlock),
+                                   (RowBwdOccupancy<T, VEC, NL, TPR, MODE>::kMinWaves))
 row_bwd_kernel(const RowArgs a) {
   constexpr int RPB = RowBwdBlock<TPR, MODE>::kRowsPerBlock;
   constexpr int NW = TPR / kWave;

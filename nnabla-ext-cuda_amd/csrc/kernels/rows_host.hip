@@ -44,10 +44,12 @@ static int cached_grid(int64_t rows, int tpr) {
 
 // Persistent grid of the LayerNormalization backward: each block keeps
 // per-column accumulators, so fewer blocks mean fewer partials to fold.
-static int ln_bwd_grid(int64_t rows, int tpr) {
+static int ln_bwd_grid(int64_t rows, int tpr, bool wide_regs = false) {
   // Wave-per-row rows run 8 to a 512-thread block; longer rows own a block.
+  // wide_regs: the float wave-per-row kernel with 4 loads per lane needs more
+  // than 128 VGPRs, so one of its 512-thread blocks is resident per CU.
   const int rpb = tpr == 64 ? 8 : 1;
-  const int per_cu = tune_int("LN_BWD_BLOCKS_PER_CU", tpr == 1024 ? 1 : 2);
+  const int per_cu = tune_int("LN_BWD_BLOCKS_PER_CU", (tpr == 1024 || wide_regs) ? 1 : 2);
   const int64_t cap = static_cast<int64_t>(device_cus()) * per_cu;
   const int64_t blocks = (rows + rpb - 1) / rpb;
   return static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(blocks, cap)));
@@ -239,7 +241,8 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
   (void)full;
   if (cfg.ok && !tune_int("FORCE_STREAM", 0)) {
     if (p.mode == kRowLN) {
-      const int grid = ln_bwd_grid(p.rows, cfg.tpr);
+      const int grid = ln_bwd_grid(p.rows, cfg.tpr,
+                                   p.dtype == NBLAHIP_F32 && cfg.tpr == 64 && cfg.nl * cfg.vec >= 16);
       if (int e = run_row_bwd_cached_ln(p.dtype, cfg, a, grid, st)) return e;
       if (p.dgamma || p.dbeta) {
         NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 31) / 32), dim3(1024), 0, st,
