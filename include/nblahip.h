@@ -110,6 +110,58 @@ NBLAHIP_EXPORT int nblahip_bn_bwd(const void *x, const void *dy,
                                   size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------
+ * BatchNormalization of a batch that is split over several workers
+ * (SyncBatchNormalization): the device steps of one worker.  The exchange
+ * between the steps (all-gather of the statistics, all-reduce of the backward
+ * pairs) belongs to the caller's communicator; with one worker the sequence
+ * equals nblahip_bn_fwd_train / nblahip_bn_bwd.
+ *   forward : local_stats -> [all-gather stats] -> merge_stats ->
+ *             nblahip_bn_fwd_infer(x, batch_mean, batch_var, gamma, beta, y)
+ *   backward: bwd_local_sums -> [all-reduce sums] -> bwd_apply_sums
+ * ---------------------------------------------------------------------- */
+
+/* Replaces forward_collect_statistics(_channels_last)
+ * (sync_batch_normalization.cu:122-131): mean[C] and biased var[C] of this
+ * worker's shard.  (The reference exchanges 1/sqrt(var+eps); the variance
+ * itself loses nothing when eps dominates it.) */
+NBLAHIP_EXPORT int nblahip_bn_local_stats(const void *x, float *mean,
+                                          float *var, int64_t size0,
+                                          int64_t size1, int64_t size2,
+                                          int dtype, void *workspace,
+                                          size_t workspace_bytes, void *stream);
+
+/* Replaces forward_reduce_statistics (sync_batch_normalization.cu:146-150,
+ * kernel/sync_batch_normalization.cuh:448-487).  stats: `workers` records of
+ * 2*channels+1 floats {mean[C], var[C], count}, as gathered.  Writes the
+ * statistics of the whole batch and updates the running ones (NULL: not). */
+NBLAHIP_EXPORT int nblahip_bn_merge_stats(const float *stats, int workers,
+                                          int64_t channels, float *batch_mean,
+                                          float *batch_var, float *rmean,
+                                          float *rvar, float decay_rate,
+                                          void *stream);
+
+/* Replaces backward_reduce(_channels_last) (sync_batch_normalization.cu:
+ * 216-231).  mean/var: statistics of the whole batch.  sums[C][2] =
+ * (sum dy*(x-mean), sum dy) over this worker's shard, to be summed over the
+ * workers; dgamma/dbeta (optional) are this worker's contributions. */
+NBLAHIP_EXPORT int nblahip_bn_bwd_local_sums(
+    const void *x, const void *dy, const float *mean, const float *var,
+    float *sums, float *dgamma, float *dbeta, int accum_dgamma, int accum_dbeta,
+    int64_t size0, int64_t size1, int64_t size2, float eps, int dtype,
+    void *workspace, size_t workspace_bytes, void *stream);
+
+/* Replaces backward_dx_post(_channels_last) (sync_batch_normalization.cu:
+ * 258-283, kernel/sync_batch_normalization.cuh:899-960).  sums: the pairs
+ * summed over all workers; total_count: elements per channel over all
+ * workers. */
+NBLAHIP_EXPORT int nblahip_bn_bwd_apply_sums(
+    const void *x, const void *dy, const float *gamma, const float *mean,
+    const float *var, const float *sums, double total_count,
+    const float *dmean, const float *dvar, void *dx, int accum_dx,
+    int64_t size0, int64_t size1, int64_t size2, float eps, int dtype,
+    void *workspace, size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------
  * FusedBatchNormalization: y = max(0, BatchNormalization(x) + z), z optional
  * (NULL: no residual input).  Same tensor view, statistics and workspace as
  * BatchNormalization above; gamma and beta are always present in the

@@ -34,6 +34,12 @@ SIGNATURES = {
                                                               _c_void_p]),
     "nblahip_bn_bwd": (_int, [_c_void_p] * 10 + [_int] * 3 + [_i64] * 3 + [_f, _int, _int,
                                                                    _c_void_p, _sz, _c_void_p]),
+    "nblahip_bn_local_stats": (_int, [_c_void_p] * 3 + [_i64] * 3 + [_int, _c_void_p, _sz, _c_void_p]),
+    "nblahip_bn_merge_stats": (_int, [_c_void_p, _int, _i64] + [_c_void_p] * 4 + [_f, _c_void_p]),
+    "nblahip_bn_bwd_local_sums": (_int, [_c_void_p] * 7 + [_int, _int] + [_i64] * 3 + [_f, _int,
+                                                                          _c_void_p, _sz, _c_void_p]),
+    "nblahip_bn_bwd_apply_sums": (_int, [_c_void_p] * 6 + [ctypes.c_double] + [_c_void_p] * 3 +
+                                  [_int] + [_i64] * 3 + [_f, _int, _c_void_p, _sz, _c_void_p]),
     "nblahip_fused_bn_fwd_infer": (_int, [_c_void_p] * 7 + [_i64] * 3 + [_f, _int, _c_void_p]),
     "nblahip_fused_bn_fwd_train": (_int, [_c_void_p] * 9 + [_i64] * 3 + [_f, _f, _int, _c_void_p,
                                                                          _sz, _c_void_p]),
@@ -217,6 +223,67 @@ def bn_backward(x, dy, gamma, mean, var, axis=1, eps=1e-5, batch_stat=True, dmea
                                int(accum[0]), int(accum[1]), int(accum[2]), s0, c, s2, eps,
                                int(batch_stat), dt, _ptr(ws), ws.numel(), _stream()))
     return (dx if need[0] else None, dgamma if need[1] else None, dbeta if need[2] else None)
+
+
+def bn_local_stats(x, axis=1, ws=None):
+    """mean[C], biased var[C] of this shard of the batch."""
+    import torch
+    assert x.is_contiguous()
+    s0, c, s2 = _bn_sizes(x.shape, axis)
+    dt = _dtype_code(x)
+    mean = torch.empty(c, dtype=torch.float32, device=x.device)
+    var = torch.empty(c, dtype=torch.float32, device=x.device)
+    need = lib().nblahip_bn_workspace_bytes(s0, c, s2, dt)
+    ws = ws if ws is not None else _workspace(need, x.device)
+    check(lib().nblahip_bn_local_stats(_ptr(x), _ptr(mean), _ptr(var), s0, c, s2, dt, _ptr(ws),
+                                       ws.numel(), _stream()))
+    return mean, var
+
+
+def bn_merge_stats(stats, channels, rmean=None, rvar=None, decay_rate=0.9):
+    """stats: float32 [workers, 2*channels+1] = {mean, var, count} per worker."""
+    import torch
+    assert stats.is_contiguous() and stats.dtype == torch.float32
+    mean = torch.empty(channels, dtype=torch.float32, device=stats.device)
+    var = torch.empty(channels, dtype=torch.float32, device=stats.device)
+    check(lib().nblahip_bn_merge_stats(_ptr(stats), stats.shape[0], channels, _ptr(mean), _ptr(var),
+                                       _ptr(_f32(rmean, "rmean")), _ptr(_f32(rvar, "rvar")),
+                                       decay_rate, _stream()))
+    return mean, var
+
+
+def bn_backward_local_sums(x, dy, mean, var, axis=1, eps=1e-5, need_params=True, ws=None):
+    """Returns sums[C, 2] = (sum dy*(x-mean), sum dy) of this shard, dgamma, dbeta."""
+    import torch
+    assert x.is_contiguous() and dy.is_contiguous()
+    s0, c, s2 = _bn_sizes(x.shape, axis)
+    dt = _dtype_code(x)
+    sums = torch.empty(c, 2, dtype=torch.float32, device=x.device)
+    dg = torch.empty(c, dtype=torch.float32, device=x.device) if need_params else None
+    db = torch.empty(c, dtype=torch.float32, device=x.device) if need_params else None
+    need = lib().nblahip_bn_workspace_bytes(s0, c, s2, dt)
+    ws = ws if ws is not None else _workspace(need, x.device)
+    check(lib().nblahip_bn_bwd_local_sums(_ptr(x), _ptr(dy), _ptr(mean), _ptr(var), _ptr(sums),
+                                          _ptr(dg), _ptr(db), 0, 0, s0, c, s2, eps, dt, _ptr(ws),
+                                          ws.numel(), _stream()))
+    return sums, dg, db
+
+
+def bn_backward_apply_sums(x, dy, gamma, mean, var, sums, total_count, axis=1, eps=1e-5,
+                           dmean=None, dvar=None, dx=None, accum=False, ws=None):
+    import torch
+    assert x.is_contiguous() and dy.is_contiguous() and sums.is_contiguous()
+    s0, c, s2 = _bn_sizes(x.shape, axis)
+    dt = _dtype_code(x)
+    if dx is None:
+        dx = torch.empty_like(x)
+    need = lib().nblahip_bn_workspace_bytes(s0, c, s2, dt)
+    ws = ws if ws is not None else _workspace(need, x.device)
+    check(lib().nblahip_bn_bwd_apply_sums(_ptr(x), _ptr(dy), _ptr(_f32(gamma, "gamma")), _ptr(mean),
+                                          _ptr(var), _ptr(sums), float(total_count), _ptr(dmean),
+                                          _ptr(dvar), _ptr(dx), int(accum), s0, c, s2, eps, dt,
+                                          _ptr(ws), ws.numel(), _stream()))
+    return dx
 
 
 def fused_bn_forward_global(x, z, beta, gamma, rmean, rvar, axis=1, eps=1e-5):

@@ -29,7 +29,7 @@ void InstanceNormalizationHip<T>::setup_impl(const Variables &inputs, const Vari
   channel_size_ = x->shape()[c];
   batch_size_ = 1;
   for (int b : this->batch_axis_) batch_size_ *= x->shape()[b];
-  spatial_size_ = batch_size_ * channel_size_ ? x->size() / (batch_size_ * channel_size_) : 0;
+  spatial_size_ = (batch_size_ > 0 && channel_size_ > 0) ? x->size() / (batch_size_ * channel_size_) : 0;
   NBLA_CHECK(x->size() < (Size_t(1) << 31), error_code::value,
              "InstanceNormalizationHip indexes with 32 bits: fewer than 2^31 elements required.");
   mean_.reshape(Shape_t{batch_size_ * channel_size_}, true);

@@ -169,6 +169,107 @@ int nblahip_bn_bwd(const void *x, const void *dy, const float *gamma, const floa
                      dtype, workspace, workspace_bytes, stream);
 }
 
+// ----------------------------------------------------------------------------
+// Steps of a BatchNormalization whose batch is split over several workers
+// ----------------------------------------------------------------------------
+int nblahip_bn_local_stats(const void *x, float *mean, float *var, int64_t size0, int64_t size1,
+                           int64_t size2, int dtype, void *workspace, size_t workspace_bytes,
+                           void *stream) {
+  if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
+  const int d = check_dims3(size0, size1, size2);
+  if (d) return d < 0 ? d : 0;
+  if (!x || !mean || !var) return NBLAHIP_EINVAL;
+  if (int e = check_ws(workspace, workspace_bytes, bn_workspace_bytes(size0, size1, size2, dtype)))
+    return e;
+  BnProblem p;
+  p.dtype = dtype;
+  p.x = x;
+  p.batch_mean = mean;
+  p.batch_var = var;
+  p.size0 = size0;
+  p.C = size1;
+  p.size2 = size2;
+  p.ws = workspace;
+  p.ws_bytes = workspace_bytes;
+  return launch_bn_local_stats(p, as_stream(stream));
+}
+
+int nblahip_bn_merge_stats(const float *stats, int workers, int64_t channels, float *batch_mean,
+                           float *batch_var, float *rmean, float *rvar, float decay_rate,
+                           void *stream) {
+  if (workers < 0 || channels < 0) return NBLAHIP_EINVAL;
+  if (workers == 0 || channels == 0) return 0;
+  if (channels > kMaxElems) return NBLAHIP_ERANGE;
+  if (!stats || !batch_mean || !batch_var) return NBLAHIP_EINVAL;
+  return launch_bn_merge_stats(stats, workers, channels, batch_mean, batch_var, rmean, rvar,
+                               decay_rate, as_stream(stream));
+}
+
+int nblahip_bn_bwd_local_sums(const void *x, const void *dy, const float *mean, const float *var,
+                              float *sums, float *dgamma, float *dbeta, int accum_dgamma,
+                              int accum_dbeta, int64_t size0, int64_t size1, int64_t size2,
+                              float eps, int dtype, void *workspace, size_t workspace_bytes,
+                              void *stream) {
+  if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
+  const int d = check_dims3(size0, size1, size2);
+  if (d) return d < 0 ? d : 0;
+  if (!x || !dy || !mean || !var || !sums) return NBLAHIP_EINVAL;
+  if (int e = check_ws(workspace, workspace_bytes, bn_workspace_bytes(size0, size1, size2, dtype)))
+    return e;
+  BnProblem p;
+  p.dtype = dtype;
+  p.x = x;
+  p.dy = dy;
+  p.mean = mean;
+  p.var = var;
+  p.sums_out = sums;
+  p.dgamma = dgamma;
+  p.dbeta = dbeta;
+  p.accum_g = accum_dgamma;
+  p.accum_b = accum_dbeta;
+  p.batch_stat = 1;
+  p.size0 = size0;
+  p.C = size1;
+  p.size2 = size2;
+  p.eps = eps;
+  p.ws = workspace;
+  p.ws_bytes = workspace_bytes;
+  return launch_bn_bwd(p, as_stream(stream));
+}
+
+int nblahip_bn_bwd_apply_sums(const void *x, const void *dy, const float *gamma, const float *mean,
+                              const float *var, const float *sums, double total_count,
+                              const float *dmean, const float *dvar, void *dx, int accum_dx,
+                              int64_t size0, int64_t size1, int64_t size2, float eps, int dtype,
+                              void *workspace, size_t workspace_bytes, void *stream) {
+  if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
+  const int d = check_dims3(size0, size1, size2);
+  if (d) return d < 0 ? d : 0;
+  if (!x || !dy || !mean || !var || !sums || !dx || !(total_count >= 1.0)) return NBLAHIP_EINVAL;
+  if (int e = check_ws(workspace, workspace_bytes, bn_workspace_bytes(size0, size1, size2, dtype)))
+    return e;
+  BnProblem p;
+  p.dtype = dtype;
+  p.x = x;
+  p.dy = dy;
+  p.out = dx;
+  p.gamma = gamma;
+  p.mean = mean;
+  p.var = var;
+  p.dmean = dmean;
+  p.dvar = dvar;
+  p.sums_in = sums;
+  p.total_count = total_count;
+  p.accum_dx = accum_dx;
+  p.size0 = size0;
+  p.C = size1;
+  p.size2 = size2;
+  p.eps = eps;
+  p.ws = workspace;
+  p.ws_bytes = workspace_bytes;
+  return launch_bn_bwd_from_sums(p, as_stream(stream));
+}
+
 int nblahip_fused_bn_fwd_infer(const void *x, const void *z, const float *rmean,
                                const float *rvar, const float *gamma, const float *beta, void *y,
                                int64_t size0, int64_t size1, int64_t size2, float eps, int dtype,

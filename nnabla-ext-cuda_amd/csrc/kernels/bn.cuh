@@ -69,7 +69,14 @@ struct BnBwdFinal {
   float *dgamma, *dbeta;
   int accum_g, accum_b;
   BnParam *params;
+  // Optional: the channel's raw pair (sum dy*(x-mean), sum dy), for callers that
+  // add the pairs of several shards of the batch before the apply step.
+  float *sums;
   __device__ __forceinline__ void publish(uint32_t c, float sdx, float sdy) const {
+    if (sums) {
+      sums[2 * c] = sdx;
+      sums[2 * c + 1] = sdy;
+    }
     const float istd = inv_std(var[c], eps);
     const float g = gamma ? gamma[c] : 1.f;
     if (dgamma) dgamma[c] = sdx * istd + (accum_g ? dgamma[c] : 0.f);
@@ -639,6 +646,34 @@ bn_bwd_reduce_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
       p[1] = b;
     }
   }
+}
+
+// ---------------------------------------------------------------------------
+// Statistics of a batch that is split over `workers` shards (the exchange step
+// of the reference's SyncBatchNormalization,
+// batch_norm_reduce_statistics_kernel, kernel/sync_batch_normalization.cuh:
+// 448-487): stats[w] = {mean[C], var[C] (biased, over the shard), count}.
+// Chan merge in shard order -> mean/var of the whole batch, running statistics
+// with the unbiased N/(N-1) factor on the total count.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+bn_merge_stats_kernel(const float *__restrict__ stats, uint32_t workers, uint32_t C,
+                      float *__restrict__ batch_mean, float *__restrict__ batch_var,
+                      float *__restrict__ rmean, float *__restrict__ rvar, float decay) {
+  const uint32_t c = blockIdx.x * 256u + threadIdx.x;
+  if (c >= C) return;
+  const size_t stride = 2 * static_cast<size_t>(C) + 1;
+  Welford w{0.f, 0.f, 0.f};
+  for (uint32_t j = 0; j < workers; ++j) {
+    const float *s = stats + j * stride;
+    const float n = s[2 * C];
+    w = welford_merge(w, Welford{s[c], s[C + c] * n, n});
+  }
+  const float var = w.n > 0.f ? w.m2 / w.n : 0.f;
+  batch_mean[c] = w.mean;
+  batch_var[c] = var;
+  if (rmean) rmean[c] = decay * rmean[c] + (1.f - decay) * w.mean;
+  if (rvar) rvar[c] = decay * rvar[c] + (1.f - decay) * (w.m2 / (w.n - 1.f));
 }
 
 // ---------------------------------------------------------------------------

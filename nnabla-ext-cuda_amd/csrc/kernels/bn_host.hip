@@ -288,8 +288,9 @@ int launch_bn_infer(const BnProblem &p, hipStream_t st) {
   return do_fwd_apply(p, pl, src, st);
 }
 
-int launch_bn_fwd_train(const BnProblem &p, hipStream_t st) {
-  const bool al = aligned16(p.x) && aligned16(p.out) && (!p.z || aligned16(p.z));
+namespace {
+int bn_fwd_train_impl(const BnProblem &p, bool stats_only, hipStream_t st) {
+  const bool al = aligned16(p.x) && (stats_only || aligned16(p.out)) && (!p.z || aligned16(p.z));
   const BnPlan pl = make_plan(p.size0, p.C, p.size2, p.dtype, al);
   float *part = static_cast<float *>(p.ws);
   BnParam *params = reinterpret_cast<BnParam *>(static_cast<char *>(p.ws) +
@@ -313,18 +314,38 @@ int launch_bn_fwd_train(const BnProblem &p, hipStream_t st) {
                    dim3(static_cast<uint32_t>(p.C)), dim3(kBnBlock), 0, st, part, pl.S, fin);
     if (int e = last_launch_status()) return e;
   }
+  if (stats_only) return 0;
   return do_fwd_apply(p, pl, param_src(params), st);
+}
+} // namespace
+
+int launch_bn_fwd_train(const BnProblem &p, hipStream_t st) {
+  return bn_fwd_train_impl(p, false, st);
+}
+
+int launch_bn_local_stats(const BnProblem &p, hipStream_t st) {
+  return bn_fwd_train_impl(p, true, st);
+}
+
+int launch_bn_merge_stats(const float *stats, int workers, int64_t C, float *batch_mean,
+                          float *batch_var, float *rmean, float *rvar, float decay,
+                          hipStream_t st) {
+  NBLAHIP_LAUNCH("bn_merge_stats_kernel", bn_merge_stats_kernel,
+                 dim3(static_cast<uint32_t>((C + 255) / 256)), dim3(256), 0, st, stats,
+                 static_cast<uint32_t>(workers), static_cast<uint32_t>(C), batch_mean, batch_var,
+                 rmean, rvar, decay);
+  return last_launch_status();
 }
 
 int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
-  if (!p.out && !p.dgamma && !p.dbeta && !p.dz) return 0;
+  if (!p.out && !p.dgamma && !p.dbeta && !p.dz && !p.sums_out) return 0;
   const bool al = aligned16(p.x) && aligned16(p.dy) && (!p.out || aligned16(p.out)) &&
                   (!p.y || aligned16(p.y)) && (!p.dz || aligned16(p.dz));
   const BnPlan pl = make_plan(p.size0, p.C, p.size2, p.dtype, al);
   float *part2 = static_cast<float *>(p.ws);
   BnParam *params = reinterpret_cast<BnParam *>(static_cast<char *>(p.ws) +
                                                 part_bytes(static_cast<uint32_t>(p.C), pl.S));
-  const bool need_sums = p.dgamma || p.dbeta || (p.out && p.batch_stat);
+  const bool need_sums = p.dgamma || p.dbeta || p.sums_out || (p.out && p.batch_stat);
   const double N = static_cast<double>(p.size0) * static_cast<double>(p.size2);
   BnBwdFinal fin{};
   fin.inv_N = static_cast<float>(1.0 / N);
@@ -340,6 +361,7 @@ int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
   fin.accum_g = p.accum_g;
   fin.accum_b = p.accum_b;
   fin.params = params;
+  fin.sums = p.sums_out;
   if (need_sums) {
     if (int e = do_bwd_reduce(p, pl, part2, fin, st)) return e;
   }
@@ -361,6 +383,29 @@ int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
   }
   if (p.out || p.dz) return do_bwd_apply(p, pl, params, st);
   return 0;
+}
+
+int launch_bn_bwd_from_sums(const BnProblem &p, hipStream_t st) {
+  if (!p.out) return 0;
+  const bool al = aligned16(p.x) && aligned16(p.dy) && aligned16(p.out);
+  const BnPlan pl = make_plan(p.size0, p.C, p.size2, p.dtype, al);
+  BnParam *params = reinterpret_cast<BnParam *>(static_cast<char *>(p.ws) +
+                                                part_bytes(static_cast<uint32_t>(p.C), pl.S));
+  BnBwdFinal fin{};
+  fin.inv_N = static_cast<float>(1.0 / p.total_count);
+  fin.eps = p.eps;
+  fin.batch_stat = 1;
+  fin.gamma = p.gamma;
+  fin.mean = p.mean;
+  fin.var = p.var;
+  fin.dmean_in = p.dmean;
+  fin.dvar_in = p.dvar;
+  fin.params = params;
+  // The summed pairs are laid out like one split of the partial buffer.
+  NBLAHIP_LAUNCH("bn_finalize_bwd_kernel", bn_finalize_bwd_kernel,
+                 dim3(static_cast<uint32_t>(p.C)), dim3(kBnBlock), 0, st, p.sums_in, 1u, fin);
+  if (int e = last_launch_status()) return e;
+  return do_bwd_apply(p, pl, params, st);
 }
 
 // ---------------------------------------------------------------------------

@@ -96,6 +96,11 @@ struct BnProblem {
   const void *y = nullptr;
   void *dz = nullptr;
   int accum_dz = 0;
+  // Split-batch (SyncBatchNormalization) steps: backward pair sums out
+  // ([C][2] = sum dy*(x-mean), sum dy), or in together with the total count.
+  float *sums_out = nullptr;
+  const float *sums_in = nullptr;
+  double total_count = 0.0;
   int64_t size0 = 1, C = 1, size2 = 1;
   float decay = 0.9f, eps = 1e-5f;
   void *ws = nullptr;
@@ -105,6 +110,13 @@ struct BnProblem {
 int launch_bn_infer(const BnProblem &p, hipStream_t st);
 int launch_bn_fwd_train(const BnProblem &p, hipStream_t st);
 int launch_bn_bwd(const BnProblem &p, hipStream_t st);
+// Local statistics only (p.out unused), merge of per-shard statistics, and the
+// backward apply step from summed pairs (p.sums_in, p.total_count).
+int launch_bn_local_stats(const BnProblem &p, hipStream_t st);
+int launch_bn_merge_stats(const float *stats, int workers, int64_t C, float *batch_mean,
+                          float *batch_var, float *rmean, float *rvar, float decay,
+                          hipStream_t st);
+int launch_bn_bwd_from_sums(const BnProblem &p, hipStream_t st);
 size_t bn_workspace_bytes(int64_t size0, int64_t C, int64_t size2, int dtype);
 
 // Optional per-kernel timing.  When enabled, a launch goes through

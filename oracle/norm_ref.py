@@ -18,6 +18,10 @@ How each function is pinned (see tests/test_oracle_pins.py):
       -> torch CPU float64 F.batch_norm / layer_norm / group_norm /
          instance_norm + autograd (library routines), incl. the 3-output
          dmean/dvar terms through an autograd loss that consumes mean and var;
+  syncbn_merge_stats
+      -> equality with the statistics of the concatenated batch (two-pass
+         numpy mean/var) for even and uneven splits, and with torch's running
+         statistics of the whole batch;
   fused_bn_forward / fused_bn_backward
       -> torch CPU float64 relu(F.batch_norm(x) + z) + autograd (training and
          eval mode, with and without z);
@@ -200,6 +204,39 @@ def bn_backward_global(x, dy, gamma, rmean, rvar, axis=1, eps=1e-5):
     dgamma = (dy3 * (x3 - _bc(rmean, c, 0)) * inv).sum(axis=(0, 2))
     dbeta = dy3.sum(axis=(0, 2))
     return dx.reshape(shape), dgamma, dbeta
+
+
+# --------------------------------------------------------------------------
+# BatchNormalization statistics of a batch split over several workers
+# --------------------------------------------------------------------------
+def syncbn_merge_stats(means, variances, counts, rmean=None, rvar=None,
+                       decay_rate=0.9):
+    """batch_norm_reduce_statistics_kernel (kernel/sync_batch_normalization.cuh:
+    448-487): per channel, fold the workers' (mean, biased var, count) in
+    worker order,
+      var_n += v*count + (avg - m)^2 * n*count/(n+count)
+      avg    = (n*avg + count*m)/(n+count);  n += count
+    mean = avg, var = var_n/n; running var with var_n/(n-1).
+    means, variances: [W, C]; counts: [W].  Returns mean, var, new_rmean,
+    new_rvar."""
+    means, variances = _f64(means), _f64(variances)
+    counts = _f64(counts)
+    c = means.shape[1]
+    avg = np.zeros(c, F64)
+    var_n = np.zeros(c, F64)
+    n = 0.0
+    for j in range(means.shape[0]):
+        cnt = counts[j]
+        factor = 1.0 / (n + cnt)
+        var_n = var_n + variances[j] * cnt + (avg - means[j]) ** 2 * n * cnt * factor
+        avg = n * factor * avg + cnt * factor * means[j]
+        n += cnt
+    new_rm = new_rv = None
+    if rmean is not None:
+        new_rm = decay_rate * _f64(rmean).reshape(c) + (1 - decay_rate) * avg
+    if rvar is not None:
+        new_rv = decay_rate * _f64(rvar).reshape(c) + (1 - decay_rate) * var_n / (n - 1)
+    return avg, var_n / n, new_rm, new_rv
 
 
 # --------------------------------------------------------------------------

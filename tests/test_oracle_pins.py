@@ -102,6 +102,28 @@ def test_bn_forward_global_vs_torch(shape, axis, no_scale, no_bias):
     close(y, torch.movedim(yt, 1, axis).numpy())
 
 
+@pytest.mark.parametrize("splits", [[7], [3, 4], [1, 5, 2, 8], [10, 1]])
+def test_syncbn_merge_equals_whole_batch_statistics(splits):
+    """Per-shard (mean, biased var, count) folded by the reference's update
+    equal the statistics of the concatenated batch; the running statistics
+    equal torch's on the whole batch."""
+    rng = np.random.default_rng(41)
+    c = 5
+    shards = [rng.standard_normal((n, c, 3, 2)) * (i + 1) + i for i, n in enumerate(splits)]
+    means = np.stack([s.mean(axis=(0, 2, 3)) for s in shards])
+    variances = np.stack([s.var(axis=(0, 2, 3)) for s in shards])
+    counts = np.array([s.shape[0] * 6 for s in shards], np.float64)
+    rm, rv = rng.standard_normal(c), rng.uniform(0.5, 2, c)
+    mean, var, nrm, nrv = R.syncbn_merge_stats(means, variances, counts, rm, rv, 0.9)
+    whole = np.concatenate(shards, axis=0)
+    close(mean, whole.mean(axis=(0, 2, 3)))
+    close(var, whole.var(axis=(0, 2, 3)))
+    trm, trv = T(rm).clone(), T(rv).clone()
+    F.batch_norm(T(whole), trm, trv, None, None, True, 0.1, 1e-5)
+    close(nrm, trm.numpy())
+    close(nrv, trv.numpy())
+
+
 @pytest.mark.parametrize("shape,axis", BN_CASES)
 @pytest.mark.parametrize("with_z", [True, False])
 @pytest.mark.parametrize("batch_stat", [True, False])
