@@ -59,9 +59,10 @@ def test_registry_selects_by_context_and_has_no_cpu_implementation():
     assert B.LayerNormalization(B.context("half")).name == "LayerNormalizationHip"
     assert B.GroupNormalization(B.context("float"), num_groups=2).name == "GroupNormalizationHip"
     assert B.InstanceNormalization(B.context("half")).name == "InstanceNormalizationHip"
+    assert B.FusedBatchNormalization(B.context("half")).name == "FusedBatchNormalizationHip"
     cpu_only = {"backends": "cpu:float", "array_class": "CpuArray", "device_id": "0"}
     for make in (B.BatchNormalization, B.LayerNormalization, B.GroupNormalization,
-                 B.InstanceNormalization):
+                 B.InstanceNormalization, B.FusedBatchNormalization):
         with pytest.raises(B.NblaError, match="No implementation"):
             make(cpu_only)
 
@@ -77,3 +78,26 @@ def test_setup_rejects_wrong_array_class_before_any_device_work():
     f2 = B.LayerNormalization(B.context("float"))
     with pytest.raises(B.NblaError, match="setup"):
         f2.forward([x, beta, gamma], [y])          # forward before setup
+
+
+def test_product_has_no_fallback_and_never_touches_the_oracle(tmp_path):
+    """The package raises when its kernel library is missing, and no file of
+    the package imports, loads or names the oracle."""
+    import importlib.util
+    import pathlib
+    import re
+    root = pathlib.Path(__file__).resolve().parents[1]
+    pkg = root / "nnabla-ext-cuda_amd"
+    spec = importlib.util.spec_from_file_location("nblahip_missing", pkg / "__init__.py")
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    mod.LIB_PATH = str(tmp_path / "libnblahip.so")          # not there
+    with pytest.raises(RuntimeError, match="no fallback"):
+        mod.lib()
+    pat = re.compile(r"oracle|norm_ref|libnorm_ref")
+    offenders = []
+    for f in pkg.rglob("*"):
+        if f.is_file() and f.suffix in {".py", ".cpp", ".hpp", ".h", ".hip", ".cuh"} or f.name == "Makefile":
+            if f.is_file() and pat.search(f.read_text(errors="ignore")):
+                offenders.append(str(f.relative_to(root)))
+    assert not offenders, offenders
