@@ -8,7 +8,6 @@ namespace nbla {
 template <typename T>
 void GroupNormalizationHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
   GroupNormalization<T>::setup_shapes(inputs, outputs);
-  hip_set_device(this->device_);
   const auto x = inputs[0];
   const int c = this->channel_axis_;
   // Two layouts run without a transpose: channel-first (the channel axis
@@ -33,6 +32,7 @@ void GroupNormalizationHip<T>::setup_impl(const Variables &inputs, const Variabl
              "GroupNormalizationHip indexes with 32 bits: fewer than 2^31 elements required.");
   mean_.reshape(Shape_t{batch_size_ * this->num_groups_}, true);
   var_.reshape(Shape_t{batch_size_ * this->num_groups_}, true);
+  hip_set_device(this->device_); // argument errors above are reported without a device
   workspace_bytes_ =
       channel_last_ ? nblahip_gn_cl_workspace_bytes(batch_size_, spatial_size_, channel_size_,
                                                     this->num_groups_, HipDtype<T>::code)

@@ -9,7 +9,6 @@ namespace nbla {
 template <typename T>
 void InstanceNormalizationHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
   InstanceNormalization<T>::setup_shapes(inputs, outputs);
-  hip_set_device(this->device_);
   const auto x = inputs[0];
   const int c = this->channel_axis_;
   // Two layouts run without a transpose: channel-first (the channel axis
@@ -34,6 +33,7 @@ void InstanceNormalizationHip<T>::setup_impl(const Variables &inputs, const Vari
              "InstanceNormalizationHip indexes with 32 bits: fewer than 2^31 elements required.");
   mean_.reshape(Shape_t{batch_size_ * channel_size_}, true);
   var_.reshape(Shape_t{batch_size_ * channel_size_}, true);
+  hip_set_device(this->device_); // argument errors above are reported without a device
   workspace_bytes_ =
       channel_last_ ? nblahip_in_cl_workspace_bytes(batch_size_, spatial_size_, channel_size_,
                                                     HipDtype<T>::code)

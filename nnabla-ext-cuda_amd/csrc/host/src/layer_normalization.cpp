@@ -8,7 +8,6 @@ namespace nbla {
 template <typename T>
 void LayerNormalizationHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
   LayerNormalization<T>::setup_shapes(inputs, outputs);
-  hip_set_device(this->device_);
   const auto x_shape = inputs[0]->shape();
   // The kernels reduce over trailing axes: batch axes must be the leading
   // ones (the reference hands any other layout to the core's CPU function,
@@ -24,6 +23,7 @@ void LayerNormalizationHip<T>::setup_impl(const Variables &inputs, const Variabl
              "LayerNormalizationHip indexes with 32 bits: fewer than 2^31 elements required.");
   mean_.reshape(Shape_t{batch_size_}, true);
   var_.reshape(Shape_t{batch_size_}, true);
+  hip_set_device(this->device_); // argument errors above are reported without a device
   workspace_bytes_ = nblahip_ln_bwd_workspace_bytes(batch_size_, reduce_size_, HipDtype<T>::code);
   workspace_.reshape(Shape_t{static_cast<Size_t>((workspace_bytes_ + 3) / 4)}, true);
 }
