@@ -28,20 +28,23 @@ int device_cus() {
 }
 
 int tune_int(const char *name, int fallback) {
+  // Only the environment's answer is cached (-1: not set): callers may pass
+  // different fallbacks for the same knob.
   static std::mutex mu;
   static std::unordered_map<std::string, int> cache;
   std::lock_guard<std::mutex> lock(mu);
   auto it = cache.find(name);
-  if (it != cache.end()) return it->second;
-  int v = fallback;
-  const std::string key = std::string("NBLAHIP_") + name;
-  if (const char *s = std::getenv(key.c_str())) {
-    char *end = nullptr;
-    const long parsed = std::strtol(s, &end, 10);
-    if (end != s && parsed >= 0 && parsed < (1 << 20)) v = static_cast<int>(parsed);
+  if (it == cache.end()) {
+    int v = -1;
+    const std::string key = std::string("NBLAHIP_") + name;
+    if (const char *s = std::getenv(key.c_str())) {
+      char *end = nullptr;
+      const long parsed = std::strtol(s, &end, 10);
+      if (end != s && parsed >= 0 && parsed < (1 << 20)) v = static_cast<int>(parsed);
+    }
+    it = cache.emplace(name, v).first;
   }
-  cache.emplace(name, v);
-  return v;
+  return it->second >= 0 ? it->second : fallback;
 }
 
 // ---------------------------------------------------------------------------
