@@ -382,6 +382,12 @@ NBLAHIP_EXPORT int nblahip_device_info(int device, char *name, size_t name_len,
                                        size_t *total_mem);
 NBLAHIP_EXPORT int nblahip_malloc(void **ptr, size_t bytes);
 NBLAHIP_EXPORT int nblahip_free(void *ptr);
+/* Page-locked host memory (hipHostMalloc), the storage of the pinned host
+ * array class (CudaCachedHostArray / CudaHostMemory,
+ * include/nbla/cuda/array/cuda_array.hpp:92-108).  Copies to and from it are
+ * direct DMA transfers. */
+NBLAHIP_EXPORT int nblahip_host_malloc(void **ptr, size_t bytes);
+NBLAHIP_EXPORT int nblahip_host_free(void *ptr);
 NBLAHIP_EXPORT int nblahip_memcpy_h2d(void *dst, const void *src, size_t bytes,
                                       void *stream);
 NBLAHIP_EXPORT int nblahip_memcpy_d2h(void *dst, const void *src, size_t bytes,

@@ -31,6 +31,9 @@ NNABLA_HIP_EXPORT const char *nnabla_hip_last_error(void);
 NNABLA_HIP_EXPORT const char *nnabla_hip_array_classes(void);
 NNABLA_HIP_EXPORT int nnabla_hip_device_synchronize(const char *device_id);
 /* Bytes held by live device arrays / kept in the allocator cache. */
+/* Host array class variable_set/get stage through: "CpuArray" (default) or
+ * "HipCachedHostArray" (page-locked memory, direct DMA transfers). */
+NNABLA_HIP_EXPORT int nnabla_hip_set_host_array_class(const char *name);
 NNABLA_HIP_EXPORT int nnabla_hip_memory_stats(uint64_t *live_bytes, uint64_t *cached_bytes);
 NNABLA_HIP_EXPORT int nnabla_hip_clear_memory_cache(void);
 

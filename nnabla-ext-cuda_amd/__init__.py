@@ -76,6 +76,8 @@ SIGNATURES = {
                                    ctypes.POINTER(_int), ctypes.POINTER(_sz)]),
     "nblahip_malloc": (_int, [ctypes.POINTER(_c_void_p), _sz]),
     "nblahip_free": (_int, [_c_void_p]),
+    "nblahip_host_malloc": (_int, [ctypes.POINTER(_c_void_p), _sz]),
+    "nblahip_host_free": (_int, [_c_void_p]),
     "nblahip_memcpy_h2d": (_int, [_c_void_p, _c_void_p, _sz, _c_void_p]),
     "nblahip_memcpy_d2h": (_int, [_c_void_p, _c_void_p, _sz, _c_void_p]),
     "nblahip_memcpy_d2d": (_int, [_c_void_p, _c_void_p, _sz, _c_void_p]),

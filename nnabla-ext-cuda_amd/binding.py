@@ -25,6 +25,7 @@ SIGNATURES = {
     "nnabla_hip_last_error": (_S, []),
     "nnabla_hip_array_classes": (_S, []),
     "nnabla_hip_device_synchronize": (_I, [_S]),
+    "nnabla_hip_set_host_array_class": (_I, [_S]),
     "nnabla_hip_memory_stats": (_I, [ctypes.POINTER(ctypes.c_uint64)] * 2),
     "nnabla_hip_clear_memory_cache": (_I, []),
     "nnabla_hip_variable_new": (_P, [_I, ctypes.POINTER(_I64)]),
@@ -80,6 +81,12 @@ def _check(code):
 
 def init():
     _check(lib().nnabla_hip_init())
+
+
+def set_host_array_class(name):
+    """"CpuArray" (default) or "HipCachedHostArray": the host array class
+    Variable.d / set_data stage through."""
+    _check(lib().nnabla_hip_set_host_array_class(name.encode()))
 
 
 def context(type_config="float", device_id="0", array_class="HipCachedArray"):

@@ -281,12 +281,23 @@ public:
 
 // Host array (the core's CpuArray, minimal).
 class NBLA_API CpuArray : public Array {
+protected:
+  bool owns_ = true;
+  // For subclasses that bring their own host storage (the core passes an
+  // AllocatorMemoryPtr: src/nbla/cuda/array/cuda_array.cpp:283-296).
+  CpuArray(Size_t size, dtypes dtype, const Context &ctx, void *storage)
+      : Array(size, dtype, ctx), owns_(false) {
+    ptr_ = storage;
+  }
+
 public:
   CpuArray(Size_t size, dtypes dtype, const Context &ctx) : Array(size, dtype, ctx) {
     ptr_ = std::malloc(std::max<size_t>(nbytes(), 1));
     NBLA_CHECK(ptr_, error_code::memory, "host allocation of %zu bytes failed", nbytes());
   }
-  ~CpuArray() override { std::free(ptr_); }
+  ~CpuArray() override {
+    if (owns_) std::free(ptr_);
+  }
   void zero() override { std::memset(ptr_, 0, nbytes()); }
   void fill(float value) override {
     if (dtype_ == dtypes::FLOAT) {

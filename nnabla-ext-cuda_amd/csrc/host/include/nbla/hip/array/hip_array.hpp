@@ -29,6 +29,18 @@ public:
   HipCachedArray(Size_t size, dtypes dtype, const Context &ctx) : HipArray(size, dtype, ctx, true) {}
 };
 
+// Host array in page-locked memory (counterpart of CudaCachedHostArray,
+// include/nbla/cuda/array/cuda_array.hpp:92-108): behaves as a CpuArray, and
+// transfers between it and the device arrays are direct DMA copies.
+class NBLA_HIP_API HipCachedHostArray : public CpuArray {
+public:
+  HipCachedHostArray(Size_t size, dtypes dtype, const Context &ctx);
+  ~HipCachedHostArray() override;
+  static Context filter_context(const Context &ctx) {
+    return Context({}, "HipCachedHostArray", "");
+  }
+};
+
 // Blocking copies between a host array and a device array of the same dtype.
 NBLA_HIP_API void synchronizer_hip_array_cpu_array(Array *src, Array *dst);
 NBLA_HIP_API void synchronizer_cpu_array_hip_array(Array *src, Array *dst);

@@ -76,10 +76,13 @@ NdArrayPtr pick(nnabla_hip_variable *v, int which) {
   return which == 0 ? v->var.data() : v->var.grad();
 }
 
-const Context &host_ctx() {
-  static const Context ctx({"cpu:float"}, "CpuArray", "0");
-  return ctx;
+// Array class the host side of variable_set/get stages through.
+std::string &host_array_class() {
+  static std::string name = "CpuArray";
+  return name;
 }
+
+Context host_ctx() { return Context({"cpu:float"}, host_array_class(), "0"); }
 
 nnabla_hip_function *wrap(FunctionPtr fn) {
   nnabla_hip_function *f = new nnabla_hip_function;
@@ -140,6 +143,16 @@ int nnabla_hip_variable_shape(nnabla_hip_variable *v, int64_t *shape_out) {
     NBLA_CHECK(v && shape_out, error_code::value, "null argument");
     const Shape_t s = v->var.shape();
     std::copy(s.begin(), s.end(), shape_out);
+  });
+}
+
+int nnabla_hip_set_host_array_class(const char *name) {
+  return guarded([&] {
+    const std::string n = name ? name : "";
+    NBLA_CHECK(n == "CpuArray" || n == "HipCachedHostArray", error_code::value,
+               "host array class must be CpuArray or HipCachedHostArray, given '%s'", n.c_str());
+    if (n != "CpuArray") init_hip();
+    host_array_class() = n;
   });
 }
 

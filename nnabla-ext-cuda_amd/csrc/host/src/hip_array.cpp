@@ -41,6 +41,20 @@ void HipArray::copy_from(const Array *src) {
                                  hip_dtype_code(src->dtype()), size_, nullptr));
 }
 
+namespace {
+void *pinned_alloc(size_t bytes) {
+  void *p = nullptr;
+  NBLA_HIP_CHECK(nblahip_host_malloc(&p, std::max<size_t>(bytes, 1)));
+  return p;
+}
+} // namespace
+
+HipCachedHostArray::HipCachedHostArray(Size_t size, dtypes dtype, const Context &ctx)
+    : CpuArray(size, dtype, ctx,
+               pinned_alloc(static_cast<size_t>(size) * sizeof_dtype(dtype))) {}
+
+HipCachedHostArray::~HipCachedHostArray() { NBLA_HIP_FORCE_ASSERT(nblahip_host_free(ptr_)); }
+
 void synchronizer_hip_array_cpu_array(Array *src, Array *dst) {
   NBLA_CHECK(src->size() == dst->size() && src->dtype() == dst->dtype(), error_code::value,
              "device-to-host copy needs equal size and dtype");

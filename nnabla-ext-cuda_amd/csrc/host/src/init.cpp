@@ -44,10 +44,22 @@ void init_hip() {
   ArrayCreator::add_creator("HipCachedArray", [](Size_t s, dtypes d, const Context &c) -> Array * {
     return new HipCachedArray(s, d, c);
   });
+  ArrayCreator::add_creator("HipCachedHostArray", [](Size_t s, dtypes d, const Context &c) -> Array * {
+    return new HipCachedHostArray(s, d, c);
+  });
+  // The pinned host array is a host array: plain copies to and from CpuArray.
+  ArraySynchronizer::add_synchronizer("HipCachedHostArray", "CpuArray",
+                                      [](Array *src, Array *dst) { dst->copy_from(src); });
+  ArraySynchronizer::add_synchronizer("CpuArray", "HipCachedHostArray",
+                                      [](Array *src, Array *dst) { dst->copy_from(src); });
+  ArraySynchronizer::add_synchronizer("HipCachedHostArray", "HipCachedHostArray",
+                                      [](Array *src, Array *dst) { dst->copy_from(src); });
   const char *device_classes[] = {"HipArray", "HipCachedArray"};
   for (const char *dc : device_classes) {
     ArraySynchronizer::add_synchronizer(dc, "CpuArray", synchronizer_hip_array_cpu_array);
     ArraySynchronizer::add_synchronizer("CpuArray", dc, synchronizer_cpu_array_hip_array);
+    ArraySynchronizer::add_synchronizer(dc, "HipCachedHostArray", synchronizer_hip_array_cpu_array);
+    ArraySynchronizer::add_synchronizer("HipCachedHostArray", dc, synchronizer_cpu_array_hip_array);
     for (const char *dc2 : device_classes)
       ArraySynchronizer::add_synchronizer(dc, dc2, [](Array *src, Array *dst) { dst->copy_from(src); });
   }

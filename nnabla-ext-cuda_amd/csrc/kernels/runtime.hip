@@ -213,6 +213,14 @@ int nblahip_malloc(void **ptr, size_t bytes) {
 }
 int nblahip_free(void *ptr) { return ptr ? hip_status(hipFree(ptr)) : 0; }
 
+int nblahip_host_malloc(void **ptr, size_t bytes) {
+  if (!ptr) return NBLAHIP_EINVAL;
+  *ptr = nullptr;
+  if (bytes == 0) return 0;
+  return hip_status(hipHostMalloc(ptr, bytes, hipHostMallocDefault));
+}
+int nblahip_host_free(void *ptr) { return ptr ? hip_status(hipHostFree(ptr)) : 0; }
+
 int nblahip_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream) {
   if (bytes == 0) return 0;
   if (!dst || !src) return NBLAHIP_EINVAL;

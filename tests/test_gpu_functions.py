@@ -394,6 +394,35 @@ def test_unsupported_layouts_raise_not_implemented():
         h.setup([x], [y])
 
 
+def test_pinned_host_array_class_gives_the_same_results():
+    """Staging through HipCachedHostArray (page-locked memory) instead of
+    CpuArray changes nothing but the transfer path."""
+    rng = np.random.default_rng(23)
+    x = rng.standard_normal((16, 8, 12, 12)).astype(np.float32)
+    dy = rng.standard_normal(x.shape).astype(np.float32)
+
+    def run():
+        f = B.InstanceNormalization(B.context("half"), channel_axis=1, batch_axis=[0], no_scale=True,
+                                    no_bias=True)
+        vx, vy = var(x, True), B.Variable(x.shape)
+        f.setup([vx], [vy])
+        f.forward([vx], [vy])
+        vy.set_grad(dy, True)
+        f.backward([vx], [vy], propagate_down=[1], accum=[0])
+        return vy.d.copy(), vx.g.copy()
+
+    y0, dx0 = run()
+    B.set_host_array_class("HipCachedHostArray")
+    try:
+        y1, dx1 = run()
+    finally:
+        B.set_host_array_class("CpuArray")
+    np.testing.assert_array_equal(y0, y1)
+    np.testing.assert_array_equal(dx0, dx1)
+    with pytest.raises(B.NblaError, match="host array class"):
+        B.set_host_array_class("NoSuchArray")
+
+
 def test_caching_allocator_reuses_blocks():
     import ctypes
     L = B.lib()
