@@ -31,6 +31,7 @@ NNABLA_HIP_EXPORT const char *nnabla_hip_last_error(void);
 NNABLA_HIP_EXPORT const char *nnabla_hip_array_classes(void);
 NNABLA_HIP_EXPORT int nnabla_hip_device_synchronize(const char *device_id);
 /* Bytes held by live device arrays / kept in the allocator cache. */
+NNABLA_HIP_EXPORT int nnabla_hip_device_count(int *count);
 /* Host array class variable_set/get stage through: "CpuArray" (default) or
  * "HipCachedHostArray" (page-locked memory, direct DMA transfers). */
 NNABLA_HIP_EXPORT int nnabla_hip_set_host_array_class(const char *name);

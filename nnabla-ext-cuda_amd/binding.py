@@ -26,6 +26,7 @@ SIGNATURES = {
     "nnabla_hip_array_classes": (_S, []),
     "nnabla_hip_device_synchronize": (_I, [_S]),
     "nnabla_hip_set_host_array_class": (_I, [_S]),
+    "nnabla_hip_device_count": (_I, [ctypes.POINTER(ctypes.c_int)]),
     "nnabla_hip_memory_stats": (_I, [ctypes.POINTER(ctypes.c_uint64)] * 2),
     "nnabla_hip_clear_memory_cache": (_I, []),
     "nnabla_hip_variable_new": (_P, [_I, ctypes.POINTER(_I64)]),
@@ -89,11 +90,56 @@ def set_host_array_class(name):
     _check(lib().nnabla_hip_set_host_array_class(name.encode()))
 
 
-def context(type_config="float", device_id="0", array_class="HipCachedArray"):
+def array_classes():
+    """Array classes of the backend, the default one first
+    (python/src/nnabla_ext/cuda/init.pyx:137-138)."""
+    init()
+    return lib().nnabla_hip_array_classes().decode().split(",")
+
+
+def context(device_id=0, type_config="float", **kw):
     """Backend preference list the way the reference's context() builds it
-    (python/src/nnabla_ext/cuda/__init__.py:138-149): half falls back to float."""
-    backends = ["hip:half", "hip:float"] if type_config == "half" else ["hip:float"]
-    return {"backends": ",".join(backends), "array_class": array_class, "device_id": str(device_id)}
+    (python/src/nnabla_ext/cuda/__init__.py:138-149): half falls back to
+    float.  There is no 'cpu:float' tail: this backend has no CPU path."""
+    if type_config == "half":
+        backends = ["hip:half", "hip:float"]
+    elif type_config == "float":
+        backends = ["hip:float"]
+    else:
+        raise ValueError("Unknown data type config is given %s" % type_config)
+    return {"backends": ",".join(backends), "array_class": kw.get("array_class", "HipCachedArray"),
+            "device_id": str(device_id)}
+
+
+def device_synchronize(device="0"):
+    """hipDeviceSynchronize on one device (init.pyx:179-186)."""
+    _check(lib().nnabla_hip_device_synchronize(str(device).encode()))
+
+
+def synchronize(device_id=0, **kw):
+    return device_synchronize(device_id)
+
+
+def get_device_count():
+    n = ctypes.c_int(0)
+    _check(lib().nnabla_hip_device_count(ctypes.byref(n)))
+    return n.value
+
+
+def get_devices():
+    return [str(i) for i in range(get_device_count())]
+
+
+def clear_memory_cache():
+    """Returns every cached device block to the driver (init.pyx:74-75)."""
+    _check(lib().nnabla_hip_clear_memory_cache())
+
+
+def memory_stats():
+    """(bytes handed out, bytes held in the cache) of the caching allocator."""
+    live, cached = ctypes.c_uint64(0), ctypes.c_uint64(0)
+    _check(lib().nnabla_hip_memory_stats(ctypes.byref(live), ctypes.byref(cached)))
+    return live.value, cached.value
 
 
 def _ints(seq):

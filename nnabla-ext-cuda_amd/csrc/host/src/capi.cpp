@@ -146,6 +146,13 @@ int nnabla_hip_variable_shape(nnabla_hip_variable *v, int64_t *shape_out) {
   });
 }
 
+int nnabla_hip_device_count(int *count) {
+  return guarded([&] {
+    NBLA_CHECK(count, error_code::value, "count must not be null");
+    NBLA_HIP_CHECK(nblahip_device_count(count));
+  });
+}
+
 int nnabla_hip_set_host_array_class(const char *name) {
   return guarded([&] {
     const std::string n = name ? name : "";

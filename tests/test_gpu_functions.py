@@ -47,7 +47,7 @@ def test_batch_normalization_training(tc, shape, axis):
     b = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
     rm = np.zeros(pshape, np.float32)
     rv = np.ones(pshape, np.float32)
-    f = B.BatchNormalization(B.context(tc), axes=[axis], decay_rate=0.9, eps=1e-5, batch_stat=True)
+    f = B.BatchNormalization(B.context(type_config=tc), axes=[axis], decay_rate=0.9, eps=1e-5, batch_stat=True)
     assert f.name == "BatchNormalizationHip"
     vx, vb, vg, vm, vv = var(x, half), var(b), var(g), var(rm), var(rv)
     vy = B.Variable(shape)
@@ -93,7 +93,7 @@ def test_batch_normalization_three_outputs_and_flags(tc):
     dm = rng.standard_normal(pshape).astype(np.float32)
     dv = rng.standard_normal(pshape).astype(np.float32)
     rm, rv = np.zeros(pshape, np.float32), np.ones(pshape, np.float32)
-    f = B.BatchNormalization(B.context(tc), axes=[axis], batch_stat=True, no_scale=True, no_bias=True)
+    f = B.BatchNormalization(B.context(type_config=tc), axes=[axis], batch_stat=True, no_scale=True, no_bias=True)
     vx, vm, vv = var(x, half), var(rm), var(rv)
     vy, om, ov = B.Variable(shape), B.Variable(()), B.Variable(())
     f.setup([vx, vm, vv], [vy, om, ov])
@@ -123,7 +123,7 @@ def test_batch_normalization_inference(tc):
     b = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
     rm = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
     rv = rng.uniform(0.5, 2, pshape).astype(np.float32)
-    f = B.BatchNormalization(B.context(tc), axes=[1], batch_stat=False)
+    f = B.BatchNormalization(B.context(type_config=tc), axes=[1], batch_stat=False)
     vx, vb, vg, vm, vv = var(x, half), var(b), var(g), var(rm), var(rv)
     vy = B.Variable(shape)
     ins = [vx, vb, vg, vm, vv]
@@ -155,7 +155,7 @@ def test_fused_batch_normalization(tc, shape, axis, with_z):
     g = rng.uniform(0.5, 1.5, pshape).astype(np.float32)
     b = (rng.standard_normal(pshape) * 0.3).astype(np.float32)
     rm, rv = np.zeros(pshape, np.float32), np.ones(pshape, np.float32)
-    f = B.FusedBatchNormalization(B.context(tc), axes=[axis], decay_rate=0.9, eps=1e-5,
+    f = B.FusedBatchNormalization(B.context(type_config=tc), axes=[axis], decay_rate=0.9, eps=1e-5,
                                   batch_stat=True, nonlinearity="relu")
     assert f.name == "FusedBatchNormalizationHip"
     vx, vb, vg, vm, vv, vz = var(x, half), var(b), var(g), var(rm), var(rv), var(z, half)
@@ -197,7 +197,7 @@ def test_fused_batch_normalization_inference_and_errors(tc):
     b = (rng.standard_normal(pshape) * 0.3).astype(np.float32)
     rm = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
     rv = rng.uniform(0.5, 2, pshape).astype(np.float32)
-    f = B.FusedBatchNormalization(B.context(tc), axes=[axis], batch_stat=False)
+    f = B.FusedBatchNormalization(B.context(type_config=tc), axes=[axis], batch_stat=False)
     ins = [var(x, half), var(b), var(g), var(rm), var(rv), var(z, half)]
     vy = B.Variable(shape)
     f.setup(ins, [vy])
@@ -205,10 +205,10 @@ def test_fused_batch_normalization_inference_and_errors(tc):
     y_r, _, _, _, _ = R.fused_bn_forward(x, z, b, g, rm, rv, axis, 0.9, 1e-5, False)
     assert_close(vy.d, y_r, dn(tc), "y", "y")
     np.testing.assert_array_equal(ins[3].d, rm)
-    bad = B.FusedBatchNormalization(B.context(tc), axes=[axis], nonlinearity="tanh")
+    bad = B.FusedBatchNormalization(B.context(type_config=tc), axes=[axis], nonlinearity="tanh")
     with pytest.raises(B.NblaError, match="relu"):
         bad.setup(ins, [vy])
-    few = B.FusedBatchNormalization(B.context(tc), axes=[axis])
+    few = B.FusedBatchNormalization(B.context(type_config=tc), axes=[axis])
     with pytest.raises(B.NblaError, match="at least 5 inputs"):
         few.setup(ins[:3], [vy])
 
@@ -224,7 +224,7 @@ def test_layer_normalization(tc, shape, batch_axis):
     dy = rnd(rng.standard_normal(shape), tc)
     g = (rng.standard_normal(pshape) * 0.1 + 1).astype(np.float32)
     b = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
-    f = B.LayerNormalization(B.context(tc), batch_axis=list(batch_axis), eps=1e-5)
+    f = B.LayerNormalization(B.context(type_config=tc), batch_axis=list(batch_axis), eps=1e-5)
     vx, vb, vg = var(x, half), var(b), var(g)
     vy, om, ov = B.Variable(shape), B.Variable(()), B.Variable(())
     f.setup([vx, vb, vg], [vy, om, ov])
@@ -258,7 +258,7 @@ def test_group_normalization(tc, shape, groups):
     dy = rnd(rng.standard_normal(shape), tc)
     g = rng.uniform(0.5, 1.5, pshape).astype(np.float32)
     b = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
-    f = B.GroupNormalization(B.context(tc), num_groups=groups, channel_axis=1, batch_axis=[0])
+    f = B.GroupNormalization(B.context(type_config=tc), num_groups=groups, channel_axis=1, batch_axis=[0])
     vx, vb, vg = var(x, half), var(b), var(g)
     vy = B.Variable(shape)
     f.setup([vx, vb, vg], [vy])
@@ -285,7 +285,7 @@ def test_instance_normalization(tc, per_sample):
     dy = rnd(rng.standard_normal(shape), tc)
     g = rng.uniform(0.5, 1.5, pshape).astype(np.float32)
     b = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
-    f = B.InstanceNormalization(B.context(tc), channel_axis=1, batch_axis=[0])
+    f = B.InstanceNormalization(B.context(type_config=tc), channel_axis=1, batch_axis=[0])
     vx, vb, vg = var(x, half), var(b), var(g)
     vy = B.Variable(shape)
     f.setup([vx, vb, vg], [vy])
@@ -317,7 +317,7 @@ def test_group_normalization_channel_last(tc, shape, groups):
     dy = rnd(rng.standard_normal(shape), tc)
     g = rng.uniform(0.5, 1.5, pshape).astype(np.float32)
     b = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
-    f = B.GroupNormalization(B.context(tc), num_groups=groups, channel_axis=len(shape) - 1,
+    f = B.GroupNormalization(B.context(type_config=tc), num_groups=groups, channel_axis=len(shape) - 1,
                              batch_axis=[0])
     vx, vb, vg = var(x, half), var(b), var(g)
     vy, om, ov = B.Variable(shape), B.Variable(()), B.Variable(())
@@ -354,7 +354,7 @@ def test_instance_normalization_channel_last(tc, per_sample):
     dy = rnd(rng.standard_normal(shape), tc)
     g = rng.uniform(0.5, 1.5, pshape).astype(np.float32)
     b = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
-    f = B.InstanceNormalization(B.context(tc), channel_axis=3, batch_axis=[0])
+    f = B.InstanceNormalization(B.context(type_config=tc), channel_axis=3, batch_axis=[0])
     vx, vb, vg = var(x, half), var(b), var(g)
     vy = B.Variable(shape)
     f.setup([vx, vb, vg], [vy])
@@ -375,7 +375,7 @@ def test_instance_normalization_channel_last(tc, per_sample):
 
 
 def test_unsupported_layouts_raise_not_implemented():
-    ctx = B.context("float")
+    ctx = B.context(type_config="float")
     x, y = B.Variable((4, 6, 8)), B.Variable((4, 6, 8))
     f = B.LayerNormalization(ctx, batch_axis=[1], no_scale=True, no_bias=True)
     with pytest.raises(B.NblaError, match="batch_axis"):
@@ -394,6 +394,24 @@ def test_unsupported_layouts_raise_not_implemented():
         h.setup([x], [y])
 
 
+def test_extension_module_utilities():
+    """The helpers the reference's Python package exports
+    (python/src/nnabla_ext/cuda/__init__.py:124-160, init.pyx:74-205)."""
+    assert B.array_classes()[0] == "HipCachedArray" and "HipArray" in B.array_classes()
+    assert B.get_device_count() >= 1
+    assert B.get_devices()[0] == "0"
+    ctx = B.context(0, "half")
+    assert ctx["backends"] == "hip:half,hip:float" and ctx["device_id"] == "0"
+    assert B.context(device_id=0)["backends"] == "hip:float"
+    with pytest.raises(ValueError):
+        B.context(0, "mixed")
+    B.synchronize(0)
+    B.device_synchronize("0")
+    B.clear_memory_cache()
+    live, cached = B.memory_stats()
+    assert cached == 0 and live >= 0
+
+
 def test_pinned_host_array_class_gives_the_same_results():
     """Staging through HipCachedHostArray (page-locked memory) instead of
     CpuArray changes nothing but the transfer path."""
@@ -402,7 +420,7 @@ def test_pinned_host_array_class_gives_the_same_results():
     dy = rng.standard_normal(x.shape).astype(np.float32)
 
     def run():
-        f = B.InstanceNormalization(B.context("half"), channel_axis=1, batch_axis=[0], no_scale=True,
+        f = B.InstanceNormalization(B.context(type_config="half"), channel_axis=1, batch_axis=[0], no_scale=True,
                                     no_bias=True)
         vx, vy = var(x, True), B.Variable(x.shape)
         f.setup([vx], [vy])
@@ -427,7 +445,7 @@ def test_caching_allocator_reuses_blocks():
     import ctypes
     L = B.lib()
     live, cached = ctypes.c_uint64(), ctypes.c_uint64()
-    ctx = B.context("float")
+    ctx = B.context(type_config="float")
     x = np.random.default_rng(7).standard_normal((64, 256)).astype(np.float32)
 
     def run():

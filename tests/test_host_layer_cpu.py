@@ -54,12 +54,12 @@ def test_variable_roundtrip_on_host_float_and_half():
 
 def test_registry_selects_by_context_and_has_no_cpu_implementation():
     B.init()
-    f = B.BatchNormalization(B.context("float"))
+    f = B.BatchNormalization(B.context(type_config="float"))
     assert f.name == "BatchNormalizationHip"
-    assert B.LayerNormalization(B.context("half")).name == "LayerNormalizationHip"
-    assert B.GroupNormalization(B.context("float"), num_groups=2).name == "GroupNormalizationHip"
-    assert B.InstanceNormalization(B.context("half")).name == "InstanceNormalizationHip"
-    assert B.FusedBatchNormalization(B.context("half")).name == "FusedBatchNormalizationHip"
+    assert B.LayerNormalization(B.context(type_config="half")).name == "LayerNormalizationHip"
+    assert B.GroupNormalization(B.context(type_config="float"), num_groups=2).name == "GroupNormalizationHip"
+    assert B.InstanceNormalization(B.context(type_config="half")).name == "InstanceNormalizationHip"
+    assert B.FusedBatchNormalization(B.context(type_config="half")).name == "FusedBatchNormalizationHip"
     cpu_only = {"backends": "cpu:float", "array_class": "CpuArray", "device_id": "0"}
     for make in (B.BatchNormalization, B.LayerNormalization, B.GroupNormalization,
                  B.InstanceNormalization, B.FusedBatchNormalization):
@@ -75,9 +75,19 @@ def test_setup_rejects_wrong_array_class_before_any_device_work():
     beta, gamma = B.Variable((1, 8)), B.Variable((1, 8))
     with pytest.raises(B.NblaError, match="not allowed"):
         f.setup([x, beta, gamma], [y])
-    f2 = B.LayerNormalization(B.context("float"))
+    f2 = B.LayerNormalization(B.context(type_config="float"))
     with pytest.raises(B.NblaError, match="setup"):
         f2.forward([x, beta, gamma], [y])          # forward before setup
+
+
+def test_context_follows_the_reference_signature():
+    assert B.context() == {"backends": "hip:float", "array_class": "HipCachedArray",
+                           "device_id": "0"}
+    assert B.context(1, "half")["backends"] == "hip:half,hip:float"
+    assert B.context(device_id=3)["device_id"] == "3"
+    with pytest.raises(ValueError, match="Unknown data type config"):
+        B.context(0, "mixed_half")
+    assert B.array_classes() == ["HipCachedArray", "HipArray"]
 
 
 def test_product_has_no_fallback_and_never_touches_the_oracle(tmp_path):
