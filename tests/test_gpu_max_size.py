@@ -1,0 +1,139 @@
+"""Tensors just below the 2^31-element limit of the C-ABI (fp16, 4.3 GB each):
+the 32-bit index arithmetic of the kernels must not wrap.  The input is a small
+block tiled along the batch, so every tile must reproduce the result of the
+block alone, which the float64 oracle checks; parameter gradients scale with
+the number of tiles."""
+import numpy as np
+import pytest
+import torch
+
+from _util import assert_close, load_package, to_dev, to_np
+from oracle import norm_ref as R
+
+pytestmark = pytest.mark.gpu
+K = load_package()
+
+
+def _need(gib):
+    free, _ = torch.cuda.mem_get_info()
+    if free < gib * (1 << 30):
+        pytest.skip(f"needs {gib} GiB of free device memory")
+
+
+def test_layer_normalization_just_below_2_31_elements():
+    _need(24)
+    Rr, blk = 8192, 64
+    tiles = ((1 << 31) - 1) // (Rr * blk)            # 4095 tiles -> 2 146 959 360 elements
+    rows = tiles * blk
+    assert rows * Rr < (1 << 31) and rows * Rr > (1 << 31) - (1 << 21)
+    rng = np.random.default_rng(61)
+    xb = (rng.standard_normal((blk, Rr)) + rng.uniform(-3, 3, (blk, 1))).astype(np.float16)
+    dyb = rng.standard_normal((blk, Rr)).astype(np.float16)
+    g = (rng.standard_normal(Rr) * 0.1 + 1).astype(np.float32)
+    b = (rng.standard_normal(Rr) * 0.1).astype(np.float32)
+    x = torch.from_numpy(xb).cuda().repeat(tiles, 1)
+    dy = torch.from_numpy(dyb).cuda().repeat(tiles, 1)
+    gd, bd = to_dev(g), to_dev(b)
+    y, m, v = K.ln_forward(x, bd, gd, rows, 1e-5)
+    y_r, m_r, v_r = R.ln_forward(xb, b, g, blk, 1e-5)
+    assert_close(to_np(y[:blk]), y_r, "f16", "y", "first tile y")
+    assert_close(to_np(m[:blk]), m_r, "f16", "stat", "first tile mean")
+    yt = y.view(tiles, blk, Rr)
+    assert torch.equal(yt[-1], yt[0]) and torch.equal(yt[tiles // 2], yt[0])
+    assert bool((yt == yt[0]).all())
+    assert torch.equal(m.view(tiles, blk)[-1], m[:blk]) and torch.equal(v.view(tiles, blk)[-1], v[:blk])
+    del yt, y
+    dx, dg, db = K.ln_backward(x, dy, gd, m, v, rows, 1e-5)
+    dx_r, dg_r, db_r = R.ln_backward(xb, dyb, g, m_r, v_r, blk, 1e-5)
+    assert_close(to_np(dx[:blk]), dx_r, "f16", "grad", "first tile dx")
+    dxt = dx.view(tiles, blk, Rr)
+    assert bool((dxt == dxt[0]).all())
+    assert_close(to_np(dg) / tiles, dg_r, "f16", "pgrad", "dgamma / tiles")
+    assert_close(to_np(db) / tiles, db_r, "f16", "pgrad", "dbeta / tiles")
+
+
+@pytest.mark.parametrize("layout", ["planes", "channel_last"])
+def test_batch_normalization_just_below_2_31_elements(layout):
+    _need(24)
+    c, sp = 256, 4096
+    n = ((1 << 31) - 1) // (c * sp)                  # 2047 samples -> 2 146 435 072 elements
+    rng = np.random.default_rng(62)
+    shape_b = (1, c, sp) if layout == "planes" else (1, sp, c)
+    axis = 1 if layout == "planes" else 2
+    xb = (rng.standard_normal(shape_b) * 2 + 1).astype(np.float16)
+    dyb = rng.standard_normal(shape_b).astype(np.float16)
+    g = rng.uniform(0.5, 1.5, c).astype(np.float32)
+    b = (rng.standard_normal(c) * 0.1).astype(np.float32)
+    x = torch.from_numpy(xb).cuda().repeat(n, 1, 1)
+    dy = torch.from_numpy(dyb).cuda().repeat(n, 1, 1)
+    assert x.numel() < (1 << 31) and x.numel() > (1 << 31) - (1 << 21)
+    gd, bd = to_dev(g), to_dev(b)
+    # statistics of n identical samples are those of one sample
+    y_r, m_r, v_r, _, _ = R.bn_forward_batch(xb, b, g, None, None, axis, 0.9, 1e-5)
+    y, m, v = K.bn_forward_batch(x, bd, gd, None, None, axis, 0.9, 1e-5)
+    assert_close(to_np(m), m_r, "f16", "stat", "mean")
+    assert_close(to_np(v), v_r, "f16", "stat", "var")
+    assert_close(to_np(y[:1]), y_r, "f16", "y", "first sample y")
+    assert bool((y == y[0]).all())
+    del y
+    # backward of the tiled batch: sums scale with n, dx = per-sample result with N -> n*N
+    dx, dg, db = K.bn_backward(x, dy, gd, m, v, axis, 1e-5)
+    dx_r, dg_r, db_r = R.bn_backward_batch(xb, dyb, g, m_r, v_r, axis, 1e-5)
+    assert bool((dx == dx[0]).all())
+    assert_close(to_np(dx[:1]), dx_r, "f16", "grad", "first sample dx")
+    assert_close(to_np(dg) / n, dg_r, "f16", "pgrad", "dgamma / n")
+    assert_close(to_np(db) / n, db_r, "f16", "pgrad", "dbeta / n")
+
+
+@pytest.mark.parametrize("kind", ["gn", "in", "gn_cl", "in_cl"])
+def test_group_and_instance_normalization_just_below_2_31_elements(kind):
+    _need(24)
+    c, sp, groups = 256, 4096, 32
+    n = ((1 << 31) - 1) // (c * sp)
+    cl = kind.endswith("_cl")
+    rng = np.random.default_rng(63)
+    shape_b = (1, sp, c) if cl else (1, c, sp)
+    xb = (rng.standard_normal(shape_b) * 1.5).astype(np.float16)
+    dyb = rng.standard_normal(shape_b).astype(np.float16)
+    g = rng.uniform(0.5, 1.5, c).astype(np.float32)
+    b = (rng.standard_normal(c) * 0.1).astype(np.float32)
+    x = torch.from_numpy(xb).cuda().repeat(n, 1, 1)
+    dy = torch.from_numpy(dyb).cuda().repeat(n, 1, 1)
+    gd, bd = to_dev(g), to_dev(b)
+    xt = np.moveaxis(xb, -1, 1) if cl else xb
+    dyt = np.moveaxis(dyb, -1, 1) if cl else dyb
+    back = (lambda a: np.moveaxis(np.asarray(a).reshape(xt.shape), 1, -1)) if cl else \
+        (lambda a: np.asarray(a).reshape(xt.shape))
+    if kind.startswith("gn"):
+        y, m, v = K.gn_forward(x, bd, gd, groups, 1e-5, channel_last=cl)
+        y_r, m_r, v_r = R.gn_forward(xt, b, g, 1, c, groups, 1e-5)
+        dx_r, dg_r, db_r = R.gn_backward(xt, dyt, g, m_r, v_r, 1, c, groups, 1e-5)
+    else:
+        y, m, v = K.in_forward(x, bd, gd, 1e-5, channel_last=cl)
+        y_r, m_r, v_r = R.in_forward(xt, b, g, 1, c, 1e-5)
+        dx_r, dg_r, db_r = R.in_backward(xt, dyt, g, m_r, v_r, 1, c, 1e-5)
+    per = m.numel() // n
+    assert_close(to_np(m[:per]), m_r, "f16", "stat", "first sample mean")
+    assert torch.equal(m.view(n, per)[-1], m[:per])
+    assert_close(to_np(y[:1]), back(y_r), "f16", "y", "first sample y")
+    assert bool((y == y[0]).all())
+    del y
+    if kind.startswith("gn"):
+        dx, dg, db = K.gn_backward(x, dy, gd, m, v, groups, 1e-5, channel_last=cl)
+    else:
+        dx, dg, db = K.in_backward(x, dy, gd, m, v, 1e-5, channel_last=cl)
+    assert_close(to_np(dx[:1]), back(dx_r), "f16", "grad", "first sample dx")
+    assert bool((dx == dx[0]).all())
+    assert_close(to_np(dg) / n, dg_r, "f16", "pgrad", "dgamma / n")
+    assert_close(to_np(db) / n, db_r, "f16", "pgrad", "dbeta / n")
+
+
+def test_one_more_element_is_refused():
+    L = K.lib()
+    s = torch.cuda.current_stream().cuda_stream
+    t = torch.empty(16, device="cuda")
+    p = t.data_ptr()
+    assert L.nblahip_bn_fwd_infer(p, p, p, None, None, p, 1 << 11, 1 << 10, 1 << 10, 1e-5, 1,
+                                  s) == -3                 # 2^31 elements
+    assert L.nblahip_in_fwd(p, None, None, p, p, p, 1 << 11, 1 << 10, 1 << 10, 1, 1, 1e-5, 1,
+                            s) == -3
