@@ -341,8 +341,9 @@ def main():
                          "so that rocprofv3 --pmc FETCH_SIZE/WRITE_SIZE readings can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build measures one GPU; --gpus must be 1 "
-              "(the path shards by batch, see DESIGN.md)", file=sys.stderr)
+        print("bench.py: this build measures one GPU; --gpus must be 1 (the path shards by "
+              "batch; the exchange between shards belongs to the caller's communicator)",
+              file=sys.stderr)
         sys.exit(2)
 
     import torch
