@@ -78,12 +78,14 @@ template <int TPR, int MODE> struct RowBwdBlock {
 // __launch_bounds__).  Two 512-thread blocks per CU need 4, i.e. at most 128
 // VGPRs; the layout named here would otherwise take a few registers more,
 // halve its occupancy and run a grid of two blocks per CU in two rounds
-// (GroupNormalization backward of 64 KB groups: 21.5 -> 17.1 us).  The
+// (GroupNormalization backward of 64 KB half groups: 21.5 -> 17.1 us; the
+// float layout would spill 96 bytes per lane under the cap and is slower with
+// it: 22.4 vs 21.0 us on 16 384-element groups).  The
 // wave-per-row LayerNormalization float kernel (133 VGPRs) is left alone: the
 // spill the cap costs it sits in its row loop and is worth more than the
 // occupancy.
 template <typename T, int VEC, int NL, int TPR, int MODE> struct RowBwdOccupancy {
-  static constexpr bool kGn512 = MODE == kRowGN && TPR == 512 && NL == 8;
+  static constexpr bool kGn512 = MODE == kRowGN && TPR == 512 && NL == 8 && sizeof(T) == 2;
   static constexpr int kMinWaves = kGn512 ? 4 : 1;
 };
 
