@@ -1,5 +1,9 @@
 // Instantiations and launcher of the register-cached backward row kernel,
 // mode kRowLN.
+#include <map>
+#include <mutex>
+#include <tuple>
+
 #include "rows_dispatch.hpp"
 
 namespace nblahip {
@@ -15,6 +19,37 @@ template <typename T>
 static int run_bwd_t(const RowCfg &cfg, const RowArgs &args, int grid, hipStream_t st) {
   NBLAHIP_ROW_CASES(BWD_CASE, T)
   return NBLAHIP_EINVAL;
+}
+
+// Blocks of the selected kernel that fit one CU at the same time (register and
+// LDS use decide), asked of the runtime once per layout: the persistent grid
+// of the LayerNormalization backward should fill the chip in one round.
+#define OCC_CASE(T, VEC, NL, TPR)                                                      \
+  if (cfg.vec == (VEC) && cfg.nl == (NL) && cfg.tpr == (TPR)) {                        \
+    int n = 0;                                                                         \
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(                                  \
+            &n, row_bwd_kernel<T, VEC, NL, TPR, kRowLN>,                               \
+            RowBwdBlock<TPR, kRowLN>::kBlock, 0) != hipSuccess)                        \
+      n = 0;                                                                           \
+    return n;                                                                          \
+  }
+
+template <typename T> static int occupancy_t(const RowCfg &cfg) {
+  NBLAHIP_ROW_CASES(OCC_CASE, T)
+  return 0;
+}
+
+int row_bwd_ln_resident_blocks(int dtype, const RowCfg &cfg) {
+  static std::mutex mu;
+  static std::map<std::tuple<int, int, int, int>, int> cache;
+  const auto key = std::make_tuple(dtype, cfg.vec, cfg.nl, cfg.tpr);
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = cache.find(key);
+  if (it == cache.end()) {
+    const int n = dtype == NBLAHIP_F16 ? occupancy_t<__half>(cfg) : occupancy_t<float>(cfg);
+    it = cache.emplace(key, n).first;
+  }
+  return it->second;
 }
 
 int run_row_bwd_cached_ln(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,

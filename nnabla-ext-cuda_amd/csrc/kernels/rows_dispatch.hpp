@@ -12,6 +12,9 @@ int run_row_fwd_cached(int dtype, const RowCfg &cfg, const RowArgs &args, int gr
                        hipStream_t st);
 int run_row_bwd_cached_ln(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
                           hipStream_t st);
+// Resident blocks per CU of the LayerNormalization backward kernel for cfg
+// (0 when the runtime cannot tell).
+int row_bwd_ln_resident_blocks(int dtype, const RowCfg &cfg);
 int run_row_bwd_cached_in(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
                           hipStream_t st);
 int run_row_bwd_cached_inc(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,

@@ -44,12 +44,13 @@ static int cached_grid(int64_t rows, int tpr) {
 
 // Persistent grid of the LayerNormalization backward: each block keeps
 // per-column accumulators, so fewer blocks mean fewer partials to fold.
-static int ln_bwd_grid(int64_t rows, int tpr, bool wide_regs = false) {
+static int ln_bwd_grid(int64_t rows, int tpr, int resident = 2) {
   // Wave-per-row rows run 8 to a 512-thread block; longer rows own a block.
-  // wide_regs: the float wave-per-row kernel with 4 loads per lane needs more
-  // than 128 VGPRs, so one of its 512-thread blocks is resident per CU.
+  // resident: blocks of the chosen kernel that fit a CU together; the grid
+  // never exceeds what is resident (one round) nor two blocks per CU (the
+  // workspace holds one partial per block).
   const int rpb = tpr == 64 ? 8 : 1;
-  const int per_cu = tune_int("LN_BWD_BLOCKS_PER_CU", (tpr == 1024 || wide_regs) ? 1 : 2);
+  const int per_cu = tune_int("LN_BWD_BLOCKS_PER_CU", std::max(1, std::min(2, resident)));
   const int64_t cap = static_cast<int64_t>(device_cus()) * per_cu;
   const int64_t blocks = (rows + rpb - 1) / rpb;
   return static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(blocks, cap)));
@@ -146,6 +147,15 @@ int launch_row_fwd(const RowProblem &p, hipStream_t st) {
   return vec_ok ? stream_fwd_t<float, 4>(p, a, st) : stream_fwd_t<float, 1>(p, a, st);
 }
 
+// Row chunks of the streaming LayerNormalization column gradients: enough
+// (strip, chunk) blocks for 8 per CU, at least 64 rows per chunk.
+static int ln_stream_chunks(int64_t rows, int64_t R) {
+  const int64_t strips = (R + 63) / 64;
+  const int64_t want = (8 * static_cast<int64_t>(device_cus()) + strips - 1) / strips;
+  const int64_t most = std::max<int64_t>(1, rows / 64);
+  return static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(std::min(want, most), 65535)));
+}
+
 size_t row_bwd_workspace_bytes(int mode, int64_t rows, int64_t R, int64_t planes) {
   if (mode == kRowLN) {
     // Largest persistent grid over the possible thread layouts (one row per
@@ -153,7 +163,9 @@ size_t row_bwd_workspace_bytes(int mode, int64_t rows, int64_t R, int64_t planes
     const int g = std::max(std::max(ln_bwd_grid(rows, 64), ln_bwd_grid(rows, 256)),
                            std::max(ln_bwd_grid(rows, 512), ln_bwd_grid(rows, 1024)));
     const size_t cached = static_cast<size_t>(g) * 2 * static_cast<size_t>(R) * sizeof(float);
-    const size_t stream = static_cast<size_t>(rows) * 2 * sizeof(float);
+    const size_t stream = align_up(static_cast<size_t>(rows) * 2 * sizeof(float), 256) +
+                          static_cast<size_t>(ln_stream_chunks(rows, R)) * 2 *
+                              static_cast<size_t>(R) * sizeof(float);
     return align_up(std::max(cached, stream), 256);
   }
   return align_up(static_cast<size_t>(planes) * 2 * sizeof(float), 256) +
@@ -177,9 +189,17 @@ static int stream_bwd_t(const RowProblem &p, const RowArgs &a, hipStream_t st) {
       if (int e = last_launch_status()) return e;
     }
     if (p.dgamma || p.dbeta) {
-      NBLAHIP_LAUNCH("ln_colgrad_stream_kernel", (ln_colgrad_stream_kernel<T>), dim3((a.R + 31) / 32), dim3(256), 0, st,
-                         x, dy, p.mean, p.var, a.rows, a.R, p.eps, p.dgamma, p.dbeta, p.accum_g,
-                         p.accum_b);
+      // Column partials over row chunks, after the row sums in the workspace.
+      float *part = reinterpret_cast<float *>(
+          static_cast<char *>(p.ws) + align_up(static_cast<size_t>(p.rows) * 2 * sizeof(float), 256));
+      const int Y = ln_stream_chunks(p.rows, p.R);
+      const int rpc = static_cast<int>((p.rows + Y - 1) / Y);
+      NBLAHIP_LAUNCH("ln_colgrad_stream_kernel", (ln_colgrad_stream_kernel<T>),
+                     dim3((a.R + 63) / 64, Y), dim3(256), 0, st, x, dy, p.mean, p.var, a.rows, a.R,
+                     rpc, p.eps, part);
+      if (int e = last_launch_status()) return e;
+      NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 31) / 32),
+                     dim3(1024), 0, st, part, Y, a.R, p.dgamma, p.dbeta, p.accum_g, p.accum_b);
       if (int e = last_launch_status()) return e;
     }
     return 0;
@@ -241,8 +261,8 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
   (void)full;
   if (cfg.ok && !tune_int("FORCE_STREAM", 0)) {
     if (p.mode == kRowLN) {
-      const int grid = ln_bwd_grid(p.rows, cfg.tpr,
-                                   p.dtype == NBLAHIP_F32 && cfg.tpr == 64 && cfg.nl * cfg.vec >= 16);
+      const int resident = row_bwd_ln_resident_blocks(p.dtype, cfg);
+      const int grid = ln_bwd_grid(p.rows, cfg.tpr, resident > 0 ? resident : 2);
       if (int e = run_row_bwd_cached_ln(p.dtype, cfg, a, grid, st)) return e;
       if (p.dgamma || p.dbeta) {
         NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 31) / 32), dim3(1024), 0, st,

@@ -222,40 +222,53 @@ row_bwd_dx_kernel(const RowArgs a, const float *__restrict__ rs, FastDiv nvr,
   }
 }
 
-// LayerNormalization dgamma/dbeta, any shape: block = 32 columns x 8 row
-// groups; each block owns a 32-column strip and walks all rows.
+// LayerNormalization dgamma/dbeta partials, any shape.  grid = (ceil(R/64), Y):
+// a block owns a 64-column strip (one wave-wide, fully coalesced access per
+// row) and the rows [y*rpc, (y+1)*rpc); its 4 waves take every 4th row, 4 rows
+// in flight each.  part[y][0][R] = sum dy*(x-mean)*istd, part[y][1][R] = sum dy;
+// ln_param_reduce_kernel folds the Y partials.
 template <typename T>
 __global__ void __launch_bounds__(256)
 ln_colgrad_stream_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                          const float *__restrict__ mean, const float *__restrict__ var,
-                         int rows, int R, float eps, float *__restrict__ dgamma,
-                         float *__restrict__ dbeta, int accum_g, int accum_b) {
-  __shared__ float rg[8][33];
-  __shared__ float rb[8][33];
-  const int cx = threadIdx.x & 31;
-  const int py = threadIdx.x >> 5;
-  const int col = blockIdx.x * 32 + cx;
+                         int rows, int R, int rpc, float eps, float *__restrict__ part) {
+  __shared__ float rg[4][64];
+  __shared__ float rb[4][64];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int col = blockIdx.x * 64 + lane;
+  const int colc = col < R ? col : R - 1; // clamped: loads stay unconditional
+  const int rbegin = blockIdx.y * rpc;
+  const int rend = min(rbegin + rpc, rows);
   float sg = 0.f, sb = 0.f;
-  if (col < R) {
-    for (int r = py; r < rows; r += 8) {
-      const size_t i = static_cast<size_t>(r) * R + col;
-      const float d = to_f32<T>(dy[i]);
-      sg += d * (to_f32<T>(x[i]) - mean[r]) * inv_std(var[r], eps);
+  for (int r0 = rbegin + wave; r0 < rend; r0 += 16) {
+    float xv[4], dv[4], mu[4], is[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int r = r0 + 4 * u;
+      const int rc = r < rend ? r : r0;
+      const size_t i = static_cast<size_t>(rc) * R + colc;
+      xv[u] = to_f32<T>(x[i]);
+      dv[u] = to_f32<T>(dy[i]);
+      mu[u] = mean[rc];
+      is[u] = var[rc];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float d = (r0 + 4 * u < rend) ? dv[u] : 0.f;
+      sg += d * (xv[u] - mu[u]) * inv_std(is[u], eps);
       sb += d;
     }
   }
-  rg[py][cx] = sg;
-  rb[py][cx] = sb;
+  rg[wave][lane] = sg;
+  rb[wave][lane] = sb;
   lds_barrier();
-  if (py == 0 && col < R) {
-    float tg = 0.f, tb = 0.f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      tg += rg[i][cx];
-      tb += rb[i][cx];
-    }
-    if (dgamma) dgamma[col] = tg + (accum_g ? dgamma[col] : 0.f);
-    if (dbeta) dbeta[col] = tb + (accum_b ? dbeta[col] : 0.f);
+  if (wave == 0 && col < R) {
+    const float tg = (rg[0][lane] + rg[1][lane]) + (rg[2][lane] + rg[3][lane]);
+    const float tb = (rb[0][lane] + rb[1][lane]) + (rb[2][lane] + rb[3][lane]);
+    float *p = part + static_cast<size_t>(blockIdx.y) * 2 * R;
+    p[col] = tg;
+    p[R + col] = tb;
   }
 }
 
