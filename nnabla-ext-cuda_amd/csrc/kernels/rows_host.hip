@@ -136,8 +136,11 @@ static int stream_fwd_t(const RowProblem &p, const RowArgs &a, hipStream_t st) {
 int launch_row_fwd(const RowProblem &p, hipStream_t st) {
   const bool vec_ok = row_vec_ok(p, false);
   const RowArgs a = make_args(p);
-  // LayerNormalization keeps gamma/beta of its columns in registers too.
-  const RowCfg cfg = pick_row_cfg(p.dtype, p.R, vec_ok, 8, p.mode == kRowLN ? 4 : 8, 64);
+  // LayerNormalization keeps gamma/beta of its columns in registers too: with
+  // 8 loads per thread it needs 140-210 VGPRs (8 waves per CU), so it spreads
+  // a row over more threads instead.
+  const int max_nl = p.mode == kRowLN ? 4 : 8;
+  const RowCfg cfg = pick_row_cfg(p.dtype, p.R, vec_ok, max_nl, max_nl, 64);
   if (cfg.ok && !tune_int("FORCE_STREAM", 0)) {
     return run_row_fwd_cached(p.dtype, cfg, a, cached_grid(p.rows, cfg.tpr), st);
   }
