@@ -44,7 +44,10 @@ BnPlan make_plan(int64_t size0, int64_t C, int64_t size2, int dtype, bool ptr_al
   pl.channel_last = size2 == 1;
   const uint32_t target = split_target(pl.channel_last);
   if (!pl.channel_last) {
-    pl.vec = (ptr_aligned && size2 % full == 0) ? full : 1;
+    // Planes of 14x14 = 196 half elements are common: 8-byte accesses there.
+    pl.vec = (ptr_aligned && size2 % full == 0)                          ? full
+             : (ptr_aligned && dtype == NBLAHIP_F16 && size2 % 4 == 0) ? 4
+                                                                        : 1;
     pl.nvp = static_cast<uint32_t>(size2 / pl.vec);
     pl.vpc = static_cast<uint32_t>(size0 * pl.nvp);
     // Enough blocks to fill the chip, but at least one full unrolled step each.
@@ -235,6 +238,7 @@ int bwd_apply_t(const BnProblem &p, const BnPlan &pl, const BnParam *params, hip
   do {                                                                           \
     if (p.dtype == NBLAHIP_F16) {                                                \
       if ((VECV) == 8) return CALL(__half, 8);                                   \
+      if ((VECV) == 4) return CALL(__half, 4);                                   \
       return CALL(__half, 1);                                                    \
     }                                                                            \
     if ((VECV) == 4) return CALL(float, 4);                                      \

@@ -40,8 +40,17 @@ __device__ __forceinline__ void load_vec(const T *__restrict__ p, float (&out)[V
     static_assert(VEC == 4, "float vectors are 4 wide");
     const float4 v = *reinterpret_cast<const float4 *>(p);
     out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+  } else if constexpr (VEC == 4) { // half, 8-byte access
+    const uint2 raw = *reinterpret_cast<const uint2 *>(p);
+    const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const float2 f = __half22float2(h[i]);
+      out[2 * i] = f.x;
+      out[2 * i + 1] = f.y;
+    }
   } else {
-    static_assert(VEC == 8, "half vectors are 8 wide");
+    static_assert(VEC == 8, "half vectors are 8 or 4 wide");
     const uint4 raw = *reinterpret_cast<const uint4 *>(p);
     const __half2 *h = reinterpret_cast<const __half2 *>(&raw);
 #pragma unroll
@@ -59,6 +68,13 @@ __device__ __forceinline__ void store_vec(T *__restrict__ p, const float (&in)[V
     p[0] = from_f32<T>(in[0]);
   } else if constexpr (sizeof(T) == 4) {
     *reinterpret_cast<float4 *>(p) = make_float4(in[0], in[1], in[2], in[3]);
+  } else if constexpr (VEC == 4) {
+    uint2 raw;
+    __half2 *h = reinterpret_cast<__half2 *>(&raw);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      h[i] = __floats2half2_rn(in[2 * i], in[2 * i + 1]);
+    *reinterpret_cast<uint2 *>(p) = raw;
   } else {
     uint4 raw;
     __half2 *h = reinterpret_cast<__half2 *>(&raw);
@@ -75,6 +91,7 @@ template <typename T, int VEC> struct RawVec;
 template <> struct RawVec<float, 4> { float4 v; };
 template <> struct RawVec<float, 1> { float v; };
 template <> struct RawVec<__half, 8> { uint4 v; };
+template <> struct RawVec<__half, 4> { uint2 v; }; // 8-byte access (planes of 4k elements)
 template <> struct RawVec<__half, 1> { __half v; };
 
 template <typename T, int VEC>
@@ -84,6 +101,8 @@ __device__ __forceinline__ RawVec<T, VEC> load_raw(const T *__restrict__ p) {
     r.v = p[0];
   } else if constexpr (sizeof(T) == 4) {
     r.v = *reinterpret_cast<const float4 *>(p);
+  } else if constexpr (VEC == 4) {
+    r.v = *reinterpret_cast<const uint2 *>(p);
   } else {
     r.v = *reinterpret_cast<const uint4 *>(p);
   }
@@ -96,6 +115,8 @@ template <typename T, int VEC> __device__ __forceinline__ RawVec<T, VEC> zero_ra
     r.v = from_f32<T>(0.f);
   } else if constexpr (sizeof(T) == 4) {
     r.v = make_float4(0.f, 0.f, 0.f, 0.f);
+  } else if constexpr (VEC == 4) {
+    r.v = make_uint2(0u, 0u);
   } else {
     r.v = make_uint4(0u, 0u, 0u, 0u);
   }
@@ -111,7 +132,7 @@ __device__ __forceinline__ void unpack(const RawVec<T, VEC> &r, float (&out)[VEC
   } else {
     const __half2 *h = reinterpret_cast<const __half2 *>(&r.v);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < VEC / 2; ++i) {
       const float2 f = __half22float2(h[i]);
       out[2 * i] = f.x;
       out[2 * i + 1] = f.y;
@@ -125,6 +146,8 @@ __device__ __forceinline__ void unpack(const RawVec<T, VEC> &r, float (&out)[VEC
 template <typename T, int VEC> __device__ __forceinline__ void keep_packed(RawVec<T, VEC> &r) {
   if constexpr (sizeof(T) == 2 && VEC == 8) {
     asm volatile("" : "+v"(r.v.x), "+v"(r.v.y), "+v"(r.v.z), "+v"(r.v.w));
+  } else if constexpr (sizeof(T) == 2 && VEC == 4) {
+    asm volatile("" : "+v"(r.v.x), "+v"(r.v.y));
   }
 }
 
@@ -160,6 +183,10 @@ __device__ __forceinline__ float elem_fma(const RawVec<T, VEC> &r, int j, float 
   } else if constexpr (sizeof(T) == 4) {
     const float x = j == 0 ? r.v.x : j == 1 ? r.v.y : j == 2 ? r.v.z : r.v.w;
     return fmaf(x, a, b);
+  } else if constexpr (VEC == 4) {
+    const uint32_t w = j < 2 ? r.v.x : r.v.y;
+    const half2_native h = __builtin_bit_cast(half2_native, w);
+    return fmaf(static_cast<float>((j & 1) ? h.y : h.x), a, b);
   } else {
     const uint32_t w = j < 2 ? r.v.x : j < 4 ? r.v.y : j < 6 ? r.v.z : r.v.w;
     const half2_native h = __builtin_bit_cast(half2_native, w);
@@ -189,6 +216,8 @@ __device__ __forceinline__ RawVec<T, VEC> raw_or_zero(bool ok, RawVec<T, VEC> r)
   } else if constexpr (sizeof(T) == 4) {
     r.v.x = ok ? r.v.x : 0.f; r.v.y = ok ? r.v.y : 0.f;
     r.v.z = ok ? r.v.z : 0.f; r.v.w = ok ? r.v.w : 0.f;
+  } else if constexpr (VEC == 4) {
+    r.v.x = ok ? r.v.x : 0u; r.v.y = ok ? r.v.y : 0u;
   } else {
     r.v.x = ok ? r.v.x : 0u; r.v.y = ok ? r.v.y : 0u;
     r.v.z = ok ? r.v.z : 0u; r.v.w = ok ? r.v.w : 0u;
@@ -215,6 +244,8 @@ __device__ __forceinline__ RawVec<T, VEC> raw_relu_mask(RawVec<T, VEC> dy, const
   } else if constexpr (sizeof(T) == 4) {
     dy.v.x = y.v.x > 0.f ? dy.v.x : 0.f; dy.v.y = y.v.y > 0.f ? dy.v.y : 0.f;
     dy.v.z = y.v.z > 0.f ? dy.v.z : 0.f; dy.v.w = y.v.w > 0.f ? dy.v.w : 0.f;
+  } else if constexpr (VEC == 4) {
+    dy.v.x &= half2_gt_zero_mask(y.v.x); dy.v.y &= half2_gt_zero_mask(y.v.y);
   } else {
     dy.v.x &= half2_gt_zero_mask(y.v.x); dy.v.y &= half2_gt_zero_mask(y.v.y);
     dy.v.z &= half2_gt_zero_mask(y.v.z); dy.v.w &= half2_gt_zero_mask(y.v.w);
@@ -228,6 +259,8 @@ __device__ __forceinline__ void store_raw(T *__restrict__ p, const RawVec<T, VEC
     p[0] = r.v;
   } else if constexpr (sizeof(T) == 4) {
     *reinterpret_cast<float4 *>(p) = r.v;
+  } else if constexpr (VEC == 4) {
+    *reinterpret_cast<uint2 *>(p) = r.v;
   } else {
     *reinterpret_cast<uint4 *>(p) = r.v;
   }
@@ -244,8 +277,10 @@ __device__ __forceinline__ float raw_sum(const RawVec<T, VEC> &r, float acc) {
     const half2_native ones = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
     acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_native, r.v.x), ones, acc, false);
     acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_native, r.v.y), ones, acc, false);
-    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_native, r.v.z), ones, acc, false);
-    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_native, r.v.w), ones, acc, false);
+    if constexpr (VEC == 8) {
+      acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_native, r.v.z), ones, acc, false);
+      acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_native, r.v.w), ones, acc, false);
+    }
     return acc;
   }
 }

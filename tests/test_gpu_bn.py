@@ -16,6 +16,8 @@ SMALL = [
     ((4, 8, 6, 6), 1), ((2, 3, 5, 7), 1), ((3, 16, 49), 1), ((5, 7), 1), ((2, 1, 9), 1),
     ((1, 4, 64, 64), 1), ((6, 5, 4, 8), 3), ((64, 64), 1), ((33, 24), 1), ((7, 3, 5, 12), 3),
     ((4, 6, 40), 2), ((2, 300, 3), 1), ((129, 5, 5, 96), 3), ((3, 2, 2, 2050), 3),
+    # planes of 4k (not 8k) elements: 8-byte accesses for fp16
+    ((8, 12, 14, 14), 1), ((3, 5, 4), 1), ((16, 256, 14, 14), 1),
 ]
 DTYPES = [torch.float32, torch.float16]
 
