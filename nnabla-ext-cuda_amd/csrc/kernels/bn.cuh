@@ -105,6 +105,40 @@ __device__ __forceinline__ size_t bn_plane_offset(uint32_t v, uint32_t c, uint32
   return (static_cast<size_t>(n) * C + c) * nvp.d + i;
 }
 
+// A plane whose length is no multiple of the vector width: the kernels still
+// use vectors aligned in the TENSOR (base pointers 16-byte aligned, element
+// count a multiple of VEC), and a plane is covered by the nvp = ceil((VEC - 1 +
+// size2) / VEC) aligned vectors that can overlap it; elements of a vector
+// outside the plane (they belong to the neighbouring channels) are masked.
+// PlaneVec: element offset of the vector and the range [lo, hi) of its
+// elements that lie in the plane.
+struct PlaneVec {
+  size_t off;
+  int lo, hi;
+};
+
+template <int VEC, bool MASKED>
+__device__ __forceinline__ PlaneVec bn_plane_vec(uint32_t v, uint32_t c, uint32_t C,
+                                                 const FastDiv &nvp, uint32_t size2,
+                                                 uint32_t last_vec) {
+  PlaneVec r;
+  if constexpr (!MASKED) {
+    r.off = bn_plane_offset(v, c, C, nvp) * VEC;
+    r.lo = 0;
+    r.hi = VEC;
+  } else {
+    const uint32_t n = nvp.div(v);
+    const uint32_t i = v - n * nvp.d;
+    const uint32_t first = (n * C + c) * size2; // first element of the plane
+    r.lo = static_cast<int>(first % VEC) - static_cast<int>(i * VEC);
+    r.hi = r.lo + static_cast<int>(size2);
+    // A vector past the plane's end has hi <= 0 (nothing valid); keep its
+    // address inside the tensor.
+    r.off = static_cast<size_t>(min(first / VEC + i, last_vec)) * VEC;
+  }
+  return r;
+}
+
 // ---------------------------------------------------------------------------
 // Forward statistics, planes layout.  grid = (C, S).
 // vpc = vectors per channel = size0 * nvp; split s covers vectors
@@ -113,10 +147,11 @@ __device__ __forceinline__ size_t bn_plane_offset(uint32_t v, uint32_t c, uint32
 // are enough channels to give every CU a block, which removes the partial
 // buffer and the finalize launch.  U = 16-byte loads in flight per thread.
 // ---------------------------------------------------------------------------
-template <typename T, int VEC, int BLOCK, bool DIRECT, int U>
+template <typename T, int VEC, int BLOCK, bool DIRECT, int U, bool MASKED = false>
 __global__ void __launch_bounds__(BLOCK)
 bn_stats_planes_kernel(const T *__restrict__ x, uint32_t C, FastDiv nvp, uint32_t vpc,
-                       uint32_t chunk, float *__restrict__ part /*[C][S][3]*/, BnFwdFinal fin) {
+                       uint32_t chunk, float *__restrict__ part /*[C][S][3]*/, BnFwdFinal fin,
+                       uint32_t size2, uint32_t last_vec) {
   __shared__ float lds[3 * (BLOCK / kWave)];
   const uint32_t c = blockIdx.x;
   const uint32_t s = blockIdx.y;
@@ -125,8 +160,34 @@ bn_stats_planes_kernel(const T *__restrict__ x, uint32_t C, FastDiv nvp, uint32_
   const uint32_t end = min(begin + chunk, vpc);
   Welford w{0.f, 0.f, 0.f};
   uint32_t v0 = begin + threadIdx.x;
+  if constexpr (MASKED) {
+    for (; v0 < end; v0 += BLOCK * U) {
+      RawVec<T, VEC> raw[U];
+      PlaneVec pv[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint32_t v = v0 + u * BLOCK;
+        pv[u] = bn_plane_vec<VEC, true>(v < end ? v : v0, c, C, nvp, size2, last_vec);
+        raw[u] = load_raw<T, VEC>(x + pv[u].off);
+        if (v >= end) pv[u].hi = pv[u].lo;
+      }
+      float vals[U * VEC];
+      bool ok[U * VEC];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        float tmp[VEC];
+        unpack<T, VEC>(raw[u], tmp);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          ok[u * VEC + j] = j >= pv[u].lo && j < pv[u].hi;
+          vals[u * VEC + j] = tmp[j];
+        }
+      }
+      welford_add_chunk_masked<U * VEC>(w, vals, ok);
+    }
+  }
   // full steps: every load valid, all U loads in flight together
-  for (; v0 + (U - 1) * BLOCK < end; v0 += BLOCK * U) {
+  for (; !MASKED && v0 + (U - 1) * BLOCK < end; v0 += BLOCK * U) {
     RawVec<T, VEC> raw[U];
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -141,7 +202,7 @@ bn_stats_planes_kernel(const T *__restrict__ x, uint32_t C, FastDiv nvp, uint32_
     }
     welford_add_chunk<U * VEC>(w, vals, U * VEC);
   }
-  if (v0 < end) { // ragged last step: clamp the index, count what is real
+  if (!MASKED && v0 < end) { // ragged last step: clamp the index, count what is real
     float vals[U * VEC];
     int cnt = 0;
 #pragma unroll
@@ -371,7 +432,10 @@ struct BnParamSrc {
 // plane = i / nvp, c = plane % C.
 // ---------------------------------------------------------------------------
 // FUSE (FusedBatchNormalization): 0 plain, 1 y = max(0, bn), 2 y = max(0, bn + z).
-template <typename T, int VEC, int FUSE = 0>
+// STRADDLE: planes of nvp.d ELEMENTS (>= VEC, no multiple of VEC); a vector
+// then holds the end of one plane and the start of the next at most, and each
+// element picks the parameters of its own channel.
+template <typename T, int VEC, int FUSE = 0, bool STRADDLE = false>
 __global__ void __launch_bounds__(256)
 bn_apply_planes_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
                        FastDiv nvp, FastDiv cdiv, uint32_t total_vec,
@@ -392,11 +456,20 @@ bn_apply_planes_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc sr
     for (int u = 0; u < kBnUnroll; ++u) {
       const uint32_t i = i0 + u * 256u;
       if (i < total_vec) {
-        const uint32_t plane = nvp.div(i);
+        const uint32_t plane = nvp.div(STRADDLE ? i * VEC : i);
         const uint32_t c = plane - cdiv.div(plane) * cdiv.d;
         const BnParam q = src.get(c);
         float o[VEC];
-        if constexpr (sizeof(T) == 2) {
+        if constexpr (STRADDLE) {
+          // elements j >= cross belong to the next plane
+          const int cross = static_cast<int>(nvp.d - (i * VEC - plane * nvp.d));
+          const BnParam q1 = src.get(c + 1 == cdiv.d ? 0u : c + 1);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            const bool nx = j >= cross;
+            o[j] = (v[u][j] - (nx ? q1.mean : q.mean)) * (nx ? q1.a : q.a) + (nx ? q1.b : q.b);
+          }
+        } else if constexpr (sizeof(T) == 2) {
           // Half output: one mixed-precision fma per element; the folded shift
           // loses nothing a 10-bit mantissa can hold.
           const float shift = fmaf(-q.mean, q.a, q.b);
@@ -482,12 +555,13 @@ bn_apply_cl_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
 // FUSED (FusedBatchNormalization): dy is first masked by y > 0 (ReLU backward);
 // the masked dy is stored to dz when dz != null (the gradient of the residual
 // input, which the apply step can then read in place of dy and y).
-template <typename T, int VEC, int BLOCK, bool DIRECT, bool FUSED = false>
+template <typename T, int VEC, int BLOCK, bool DIRECT, bool FUSED = false, bool MASKED = false>
 __global__ void __launch_bounds__(BLOCK)
 bn_bwd_reduce_planes_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                             const float *__restrict__ mean, uint32_t C, FastDiv nvp,
                             uint32_t vpc, uint32_t chunk, float one, float *__restrict__ part2,
-                            BnBwdFinal fin, const T *__restrict__ y, T *__restrict__ dz) {
+                            BnBwdFinal fin, const T *__restrict__ y, T *__restrict__ dz,
+                            uint32_t size2, uint32_t last_vec) {
   __shared__ float lds[2 * (BLOCK / kWave)];
   const uint32_t c = blockIdx.x;
   const uint32_t s = blockIdx.y;
@@ -499,17 +573,21 @@ bn_bwd_reduce_planes_kernel(const T *__restrict__ x, const T *__restrict__ dy,
   for (uint32_t v0 = begin + threadIdx.x; v0 < end; v0 += BLOCK * kBnUnroll) {
     RawVec<T, VEC> xr[kBnUnroll], dr[kBnUnroll];
     RawVec<T, VEC> yr[FUSED ? kBnUnroll : 1];
+    PlaneVec pv[kBnUnroll];
     // all loads first (indices past the end re-read v0), selects after
 #pragma unroll
     for (int u = 0; u < kBnUnroll; ++u) {
       const uint32_t v = v0 + u * BLOCK;
-      const size_t off = bn_plane_offset(v < end ? v : v0, c, C, nvp) * VEC;
-      xr[u] = load_raw<T, VEC>(x + off);
-      dr[u] = load_raw<T, VEC>(dy + off);
-      if constexpr (FUSED) yr[u] = load_raw<T, VEC>(y + off);
+      pv[u] = bn_plane_vec<VEC, MASKED>(v < end ? v : v0, c, C, nvp, size2, last_vec);
+      xr[u] = load_raw<T, VEC>(x + pv[u].off);
+      dr[u] = load_raw<T, VEC>(dy + pv[u].off);
+      if constexpr (FUSED) yr[u] = load_raw<T, VEC>(y + pv[u].off);
     }
 #pragma unroll
-    for (int u = 0; u < kBnUnroll; ++u) dr[u] = raw_or_zero<T, VEC>(v0 + u * BLOCK < end, dr[u]);
+    for (int u = 0; u < kBnUnroll; ++u) {
+      dr[u] = raw_or_zero<T, VEC>(v0 + u * BLOCK < end, dr[u]);
+      if constexpr (MASKED) dr[u] = raw_keep_range<T, VEC>(dr[u], pv[u].lo, pv[u].hi);
+    }
     if constexpr (FUSED) {
 #pragma unroll
       for (int u = 0; u < kBnUnroll; ++u) dr[u] = raw_relu_mask<T, VEC>(dr[u], yr[u]);
@@ -517,7 +595,17 @@ bn_bwd_reduce_planes_kernel(const T *__restrict__ x, const T *__restrict__ dy,
 #pragma unroll
         for (int u = 0; u < kBnUnroll; ++u) {
           const uint32_t v = v0 + u * BLOCK;
-          if (v < end) store_raw<T, VEC>(dz + bn_plane_offset(v, c, C, nvp) * VEC, dr[u]);
+          if (v < end) {
+            if (!MASKED || (pv[u].lo <= 0 && pv[u].hi >= VEC)) {
+              store_raw<T, VEC>(dz + pv[u].off, dr[u]);
+            } else { // a vector shared with the neighbouring planes: element stores
+              float g[VEC];
+              unpack<T, VEC>(dr[u], g);
+#pragma unroll
+              for (int j = 0; j < VEC; ++j)
+                if (j >= pv[u].lo && j < pv[u].hi) dz[pv[u].off + j] = from_f32<T>(g[j]);
+            }
+          }
         }
       }
     }
@@ -699,7 +787,7 @@ bn_finalize_bwd_kernel(const float *__restrict__ part2, uint32_t S, BnBwdFinal f
 // FUSED (FusedBatchNormalization): dy is first masked by y > 0; the masked dy
 // is also the gradient of the residual input z (dz, optional).  dx may be
 // null when FUSED (only dz wanted).
-template <typename T, int VEC, bool FUSED = false>
+template <typename T, int VEC, bool FUSED = false, bool STRADDLE = false>
 __global__ void __launch_bounds__(256)
 bn_bwd_apply_planes_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                            T *__restrict__ dx, const BnParam *__restrict__ params,
@@ -740,12 +828,23 @@ bn_bwd_apply_planes_kernel(const T *__restrict__ x, const T *__restrict__ dy,
           }
           if (!dx) continue;
         }
-        const uint32_t plane = nvp.div(i);
+        const uint32_t plane = nvp.div(STRADDLE ? i * VEC : i);
         const uint32_t c = plane - cdiv.div(plane) * cdiv.d;
         const BnParam q = params[c];
         float o[VEC];
+        if constexpr (STRADDLE) { // as in bn_apply_planes_kernel
+          const int cross = static_cast<int>(nvp.d - (i * VEC - plane * nvp.d));
+          const BnParam q1 = params[c + 1 == cdiv.d ? 0u : c + 1];
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) o[j] = q.a * dv[u][j] + q.b * (xv[u][j] - q.mean) + q.c;
+          for (int j = 0; j < VEC; ++j) {
+            const bool nx = j >= cross;
+            o[j] = (nx ? q1.a : q.a) * dv[u][j] +
+                   (nx ? q1.b : q.b) * (xv[u][j] - (nx ? q1.mean : q.mean)) + (nx ? q1.c : q.c);
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) o[j] = q.a * dv[u][j] + q.b * (xv[u][j] - q.mean) + q.c;
+        }
         if (accum) {
           float old[VEC];
           load_vec<T, VEC>(dx + static_cast<size_t>(i) * VEC, old);

@@ -24,6 +24,12 @@ struct BnPlan {
   bool cl_fast_apply = false;
   int apply_vec = 1;    // vector width of the apply kernels
   bool direct = false;  // planes: one 1024-thread block owns a whole channel
+  // planes whose length is no multiple of the vector width: tensor-aligned
+  // vectors, masked at the plane's ends (reductions) or split between the two
+  // channels they touch (apply)
+  bool masked = false;
+  uint32_t size2 = 1;
+  uint32_t last_vec = 0;
 };
 
 uint32_t ceil_div_u(uint64_t a, uint64_t b) { return static_cast<uint32_t>((a + b - 1) / b); }
@@ -49,6 +55,15 @@ BnPlan make_plan(int64_t size0, int64_t C, int64_t size2, int dtype, bool ptr_al
              : (ptr_aligned && dtype == NBLAHIP_F16 && size2 % 4 == 0) ? 4
                                                                         : 1;
     pl.nvp = static_cast<uint32_t>(size2 / pl.vec);
+    const uint64_t total = static_cast<uint64_t>(size0) * C * size2;
+    if (pl.vec == 1 && ptr_aligned && size2 > full && total % full == 0 &&
+        tune_int("BN_MASKED_PLANES", 1)) {
+      pl.masked = true;
+      pl.vec = full;
+      pl.size2 = static_cast<uint32_t>(size2);
+      pl.last_vec = static_cast<uint32_t>(total / full - 1);
+      pl.nvp = static_cast<uint32_t>((size2 + 2 * full - 2) / full); // most vectors a plane meets
+    }
     pl.vpc = static_cast<uint32_t>(size0 * pl.nvp);
     // Enough blocks to fill the chip, but at least one full unrolled step each.
     const uint32_t want = std::max<uint32_t>(1, ceil_div_u(target, static_cast<uint64_t>(C)));
@@ -114,6 +129,10 @@ int apply_grid(uint32_t total_vec, int unroll, bool cl = false, bool fwd = false
   return static_cast<int>(std::max<uint64_t>(1, std::min<uint64_t>(blocks, cap)));
 }
 
+// The widest vector of the element type: only that one has the masked-plane
+// kernel variants.
+template <typename T, int VEC> constexpr bool kFullVec = VEC == (sizeof(T) == 2 ? 8 : 4);
+
 template <typename T, int VEC, int FUSE>
 int fwd_apply_fuse_t(const BnProblem &p, const BnPlan &pl, const BnParamSrc &src, hipStream_t st) {
   const T *x = static_cast<const T *>(p.x);
@@ -128,6 +147,15 @@ int fwd_apply_fuse_t(const BnProblem &p, const BnPlan &pl, const BnParamSrc &src
   } else {
     // channel-last without the register fast path: planes of one vector each.
     const uint32_t nvp = pl.channel_last ? 1u : pl.nvp;
+    if constexpr (kFullVec<T, VEC>) {
+      if (pl.masked) {
+        NBLAHIP_LAUNCH(FUSE ? "bn_apply_planes_kernel_fused" : "bn_apply_planes_kernel",
+                       (bn_apply_planes_kernel<T, VEC, FUSE, true>),
+                       dim3(apply_grid(total_vec, kBnUnroll)), dim3(256), 0, st, x, y, src,
+                       FastDiv(pl.size2), FastDiv(static_cast<uint32_t>(p.C)), total_vec, z);
+        return last_launch_status();
+      }
+    }
     NBLAHIP_LAUNCH(FUSE ? "bn_apply_planes_kernel_fused" : "bn_apply_planes_kernel",
                    (bn_apply_planes_kernel<T, VEC, FUSE>), dim3(apply_grid(total_vec, kBnUnroll)),
                    dim3(256), 0, st, x, y, src, FastDiv(nvp), FastDiv(static_cast<uint32_t>(p.C)),
@@ -151,14 +179,34 @@ int stats_t(const BnProblem &p, const BnPlan &pl, float *part, const BnFwdFinal 
     NBLAHIP_LAUNCH("bn_stats_cl_kernel", (bn_stats_cl_kernel<T, VEC>), dim3(pl.ytiles, pl.S),
                    dim3(kBnBlock), 0, st, x, static_cast<uint32_t>(p.size0),
                    static_cast<uint32_t>(p.C), pl.ncv, pl.log2tx, pl.rps, 1.0f, part);
+  } else if (pl.masked) {
+    if constexpr (kFullVec<T, VEC>) {
+      if (pl.direct) {
+        NBLAHIP_LAUNCH("bn_stats_planes_kernel",
+                       (bn_stats_planes_kernel<T, VEC, 1024, true, 4, true>),
+                       dim3(static_cast<uint32_t>(p.C), 1), dim3(1024), 0, st, x,
+                       static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, part, fin,
+                       pl.size2, pl.last_vec);
+      } else {
+        NBLAHIP_LAUNCH("bn_stats_planes_kernel",
+                       (bn_stats_planes_kernel<T, VEC, kBnBlock, false, kBnUnroll, true>),
+                       dim3(static_cast<uint32_t>(p.C), pl.S), dim3(kBnBlock), 0, st, x,
+                       static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, part, fin,
+                       pl.size2, pl.last_vec);
+      }
+    } else {
+      return NBLAHIP_EINVAL;
+    }
   } else if (pl.direct) {
     NBLAHIP_LAUNCH("bn_stats_planes_kernel", (bn_stats_planes_kernel<T, VEC, 1024, true, 8>),
                    dim3(static_cast<uint32_t>(p.C), 1), dim3(1024), 0, st, x,
-                   static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, part, fin);
+                   static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, part, fin, 0u,
+                   0u);
   } else {
     NBLAHIP_LAUNCH("bn_stats_planes_kernel", (bn_stats_planes_kernel<T, VEC, kBnBlock, false, kBnUnroll>),
                    dim3(static_cast<uint32_t>(p.C), pl.S), dim3(kBnBlock), 0, st, x,
-                   static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, part, fin);
+                   static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, part, fin, 0u,
+                   0u);
   }
   return last_launch_status();
 }
@@ -180,18 +228,36 @@ int bwd_reduce_fuse_t(const BnProblem &p, const BnPlan &pl, float *part2, const 
                    0, st, x, dy, p.mean, static_cast<uint32_t>(p.size0),
                    static_cast<uint32_t>(p.C), pl.ncv, pl.log2tx, pl.rps, 1.0f, part2, 0u,
                    FastDiv(1), y, dz);
+  } else if (pl.masked) {
+    if constexpr (kFullVec<T, VEC>) {
+      if (pl.direct) {
+        NBLAHIP_LAUNCH(FUSED ? "bn_bwd_reduce_planes_kernel_fused" : "bn_bwd_reduce_planes_kernel",
+                       (bn_bwd_reduce_planes_kernel<T, VEC, 1024, true, FUSED, true>),
+                       dim3(static_cast<uint32_t>(p.C), 1), dim3(1024), 0, st, x, dy, p.mean,
+                       static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, 1.0f, part2,
+                       fin, y, dz, pl.size2, pl.last_vec);
+      } else {
+        NBLAHIP_LAUNCH(FUSED ? "bn_bwd_reduce_planes_kernel_fused" : "bn_bwd_reduce_planes_kernel",
+                       (bn_bwd_reduce_planes_kernel<T, VEC, kBnBlock, false, FUSED, true>),
+                       dim3(static_cast<uint32_t>(p.C), pl.S), dim3(kBnBlock), 0, st, x, dy, p.mean,
+                       static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, 1.0f, part2,
+                       fin, y, dz, pl.size2, pl.last_vec);
+      }
+    } else {
+      return NBLAHIP_EINVAL;
+    }
   } else if (pl.direct) {
     NBLAHIP_LAUNCH(FUSED ? "bn_bwd_reduce_planes_kernel_fused" : "bn_bwd_reduce_planes_kernel",
                    (bn_bwd_reduce_planes_kernel<T, VEC, 1024, true, FUSED>),
                    dim3(static_cast<uint32_t>(p.C), 1), dim3(1024), 0, st, x, dy, p.mean,
                    static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, 1.0f, part2, fin,
-                   y, dz);
+                   y, dz, 0u, 0u);
   } else {
     NBLAHIP_LAUNCH(FUSED ? "bn_bwd_reduce_planes_kernel_fused" : "bn_bwd_reduce_planes_kernel",
                    (bn_bwd_reduce_planes_kernel<T, VEC, kBnBlock, false, FUSED>),
                    dim3(static_cast<uint32_t>(p.C), pl.S), dim3(kBnBlock), 0, st, x, dy, p.mean,
                    static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, 1.0f, part2, fin,
-                   y, dz);
+                   y, dz, 0u, 0u);
   }
   return last_launch_status();
 }
@@ -219,6 +285,16 @@ int bwd_apply_fuse_t(const BnProblem &p, const BnPlan &pl, const BnParam *params
                    p.accum_dz);
   } else {
     const uint32_t nvp = pl.channel_last ? 1u : pl.nvp;
+    if constexpr (kFullVec<T, VEC>) {
+      if (pl.masked) {
+        NBLAHIP_LAUNCH(FUSED ? "bn_bwd_apply_planes_kernel_fused" : "bn_bwd_apply_planes_kernel",
+                       (bn_bwd_apply_planes_kernel<T, VEC, FUSED, true>),
+                       dim3(apply_grid(total_vec, 2)), dim3(256), 0, st, x, dy, dx, params,
+                       FastDiv(pl.size2), FastDiv(static_cast<uint32_t>(p.C)), total_vec,
+                       p.accum_dx, y, dz, p.accum_dz);
+        return last_launch_status();
+      }
+    }
     NBLAHIP_LAUNCH(FUSED ? "bn_bwd_apply_planes_kernel_fused" : "bn_bwd_apply_planes_kernel",
                    (bn_bwd_apply_planes_kernel<T, VEC, FUSED>), dim3(apply_grid(total_vec, 2)),
                    dim3(256), 0, st, x, dy, dx, params, FastDiv(nvp),

@@ -253,6 +253,28 @@ __device__ __forceinline__ RawVec<T, VEC> raw_relu_mask(RawVec<T, VEC> dy, const
   return dy;
 }
 
+// Zeroes the elements of a raw vector outside [lo, hi).
+template <typename T, int VEC>
+__device__ __forceinline__ RawVec<T, VEC> raw_keep_range(RawVec<T, VEC> r, int lo, int hi) {
+  if constexpr (VEC == 1) {
+    if (!(0 >= lo && 0 < hi)) r = zero_raw<T, VEC>();
+  } else if constexpr (sizeof(T) == 4) {
+    r.v.x = (0 >= lo && 0 < hi) ? r.v.x : 0.f;
+    r.v.y = (1 >= lo && 1 < hi) ? r.v.y : 0.f;
+    r.v.z = (2 >= lo && 2 < hi) ? r.v.z : 0.f;
+    r.v.w = (3 >= lo && 3 < hi) ? r.v.w : 0.f;
+  } else {
+    uint32_t *w = reinterpret_cast<uint32_t *>(&r.v);
+#pragma unroll
+    for (int k = 0; k < VEC / 2; ++k) {
+      const uint32_t m = ((2 * k >= lo && 2 * k < hi) ? 0x0000ffffu : 0u) |
+                         ((2 * k + 1 >= lo && 2 * k + 1 < hi) ? 0xffff0000u : 0u);
+      w[k] &= m;
+    }
+  }
+  return r;
+}
+
 template <typename T, int VEC>
 __device__ __forceinline__ void store_raw(T *__restrict__ p, const RawVec<T, VEC> &r) {
   if constexpr (VEC == 1) {
@@ -440,6 +462,29 @@ __device__ __forceinline__ void welford_add_chunk(Welford &acc, const float (&v)
   for (int i = 0; i < CNT; ++i) {
     const float d = v[i] - cm;
     m2 += (i < cnt) ? d * d : 0.f;
+  }
+  acc = welford_merge(acc, Welford{cm, m2, fc});
+}
+
+// The same with an arbitrary subset of the chunk valid (ok[i]).
+template <int CNT>
+__device__ __forceinline__ void welford_add_chunk_masked(Welford &acc, const float (&v)[CNT],
+                                                         const bool (&ok)[CNT]) {
+  float s = 0.f;
+  int cnt = 0;
+#pragma unroll
+  for (int i = 0; i < CNT; ++i) {
+    s += ok[i] ? v[i] : 0.f;
+    cnt += ok[i] ? 1 : 0;
+  }
+  if (cnt == 0) return;
+  const float fc = static_cast<float>(cnt);
+  const float cm = s * fast_rcp(fc);
+  float m2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < CNT; ++i) {
+    const float d = v[i] - cm;
+    m2 += ok[i] ? d * d : 0.f;
   }
   acc = welford_merge(acc, Welford{cm, m2, fc});
 }

@@ -18,6 +18,9 @@ SMALL = [
     ((4, 6, 40), 2), ((2, 300, 3), 1), ((129, 5, 5, 96), 3), ((3, 2, 2, 2050), 3),
     # planes of 4k (not 8k) elements: 8-byte accesses for fp16
     ((8, 12, 14, 14), 1), ((3, 5, 4), 1), ((16, 256, 14, 14), 1),
+    # planes that are no multiple of the vector width, tensor a multiple: masked vectors
+    ((4, 8, 7, 7), 1), ((2, 16, 9, 9), 1), ((3, 8, 3, 11), 1), ((1, 24, 5, 5), 1),
+    ((64, 32, 7, 7), 1), ((5, 16, 13), 1),
 ]
 DTYPES = [torch.float32, torch.float16]
 
@@ -155,6 +158,28 @@ def test_bn_misaligned_views():
     y, m, v = K.bn_forward_batch(xd, None, None, None, None, axis, 0.9, 1e-5)
     assert_close(to_np(y), y_r, "f32", "y", "y")
     assert_close(to_np(v), v_r, "f32", "stat", "var")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_bn_odd_planes_channel_owning_blocks(dtype):
+    """33x33 planes (no multiple of the vector width) with enough data per
+    channel for the blocks that own a whole channel."""
+    dn = dtype_name(dtype)
+    shape, axis = (128, 256, 33, 33), 1
+    x, dy, g, b, rm, rv = make_bn(shape, axis, dtype, 17, mean=0.5, std=1.5)
+    y_r, m_r, v_r, rm_r, rv_r = R.bn_forward_batch(x, b, g, rm, rv, axis, 0.9, 1e-5)
+    xd, dyd, gd, bd, rmd, rvd = to_dev(x, dtype), to_dev(dy, dtype), to_dev(g), to_dev(b), to_dev(rm), to_dev(rv)
+    y, m, v = K.bn_forward_batch(xd, bd, gd, rmd, rvd, axis, 0.9, 1e-5)
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    assert_close(to_np(rvd), rv_r, dn, "stat", "running_var")
+    assert_close(to_np(y), y_r, dn, "y", "y")
+    del y_r
+    dx_r, dg_r, db_r = R.bn_backward_batch(x, dy, g, m_r, v_r, axis, 1e-5)
+    dx, dg, db = K.bn_backward(xd, dyd, gd, m, v, axis, 1e-5)
+    assert_close(to_np(dx), dx_r, dn, "grad", "dx")
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
 
 
 def test_bn_c1_inference_full_size():

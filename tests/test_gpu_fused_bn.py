@@ -24,6 +24,7 @@ SHAPES = [
     ((6, 5, 4, 8), 3), ((64, 64), 1), ((7, 3, 5, 12), 3), ((129, 5, 5, 96), 3),
     ((3, 2, 2, 2050), 3), ((2, 256, 9, 9), 1), ((8, 14, 14, 64), 3),
     ((8, 12, 14, 14), 1), ((16, 256, 14, 14), 1),
+    ((4, 8, 7, 7), 1), ((64, 32, 7, 7), 1), ((5, 16, 13), 1),
 ]
 
 
