@@ -494,19 +494,54 @@ bn_apply_planes_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc sr
 }
 
 // ---------------------------------------------------------------------------
-// Forward apply, channel-last with ncv = C/VEC dividing 256: a thread always
-// meets the same VEC channels, so their parameters live in registers.
+// Thread layout of the channel-last apply kernels over a slab x[M][ncv] of
+// vectors: a thread always meets the same VEC channels, so their parameters
+// live in registers.  A block covers cols = min(ncv, 256) channel vectors of
+// R = 256 / cols rows per step (threads past R*cols idle; for ncv dividing 256
+// there are none and the block walks the slab as one contiguous run).  Wider
+// rows are cut into ntiles = ceil(ncv / 256) column tiles;
+// gridDim.x = ntiles * row blocks.
+// ---------------------------------------------------------------------------
+struct ClApplyMap {
+  uint32_t cv;       // channel vector of this thread
+  uint32_t row0;     // first row
+  uint32_t R;        // rows between the U loads of one step
+  uint32_t row_step; // rows between steps
+  bool active;
+};
+
+template <int U>
+__device__ __forceinline__ ClApplyMap cl_apply_map(uint32_t ncv, uint32_t ntiles) {
+  ClApplyMap m;
+  const uint32_t cols = min(ncv, 256u);
+  m.R = 256u / cols;
+  const uint32_t tr = threadIdx.x / cols;
+  const uint32_t tile = blockIdx.x % ntiles;
+  const uint32_t rb = blockIdx.x / ntiles;
+  m.cv = tile * 256u + (threadIdx.x - tr * cols);
+  m.active = tr < m.R && m.cv < ncv;
+  m.row0 = rb * m.R * U + tr;
+  m.row_step = (gridDim.x / ntiles) * m.R * U;
+  return m;
+}
+
+// ---------------------------------------------------------------------------
+// Forward apply, channel-last.
 // ---------------------------------------------------------------------------
 template <typename T, int VEC, int FUSE = 0>
 __global__ void __launch_bounds__(256)
 bn_apply_cl_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
-                   uint32_t ncv, uint32_t total_vec, const T *__restrict__ z, float one) {
+                   uint32_t ncv, uint32_t ntiles, uint32_t M, const T *__restrict__ z,
+                   float one) {
   // blockIdx.y: slab (sample) index; each slab has its own ncv*VEC parameters.
-  x += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
-  y += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
-  if constexpr (FUSE == 2) z += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
+  const size_t slab = static_cast<size_t>(blockIdx.y) * M * ncv * VEC;
+  x += slab;
+  y += slab;
+  if constexpr (FUSE == 2) z += slab;
   if (src.params) src.params += static_cast<size_t>(blockIdx.y) * ncv * VEC;
-  const uint32_t cv = threadIdx.x % ncv;
+  const ClApplyMap map = cl_apply_map<kBnUnroll>(ncv, ntiles);
+  if (!map.active) return;
+  const uint32_t cv = map.cv;
   // y = x*pa + ps with ps = pb - mean*pa for half output (one mixed fma per
   // element); the centred form (x-mean)*pa + pb for float output.
   float pm[VEC], pa[VEC], pb[VEC];
@@ -517,20 +552,21 @@ bn_apply_cl_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
     pa[j] = q.a;
     pb[j] = (sizeof(T) == 2) ? fmaf(-q.mean, q.a, q.b) : q.b;
   }
-  for (uint32_t i0 = blockIdx.x * (256u * kBnUnroll) + threadIdx.x; i0 < total_vec;
-       i0 += gridDim.x * (256u * kBnUnroll)) {
+  for (uint32_t r0 = map.row0; r0 < M; r0 += map.row_step) {
     RawVec<T, VEC> raw[kBnUnroll];
     RawVec<T, VEC> zr[FUSE == 2 ? kBnUnroll : 1];
 #pragma unroll
     for (int u = 0; u < kBnUnroll; ++u) {
-      const uint32_t i = min(i0 + u * 256u, total_vec - 1); // clamped: loads stay branch-free
+      // clamped: loads stay branch-free
+      const uint32_t i = min(r0 + u * map.R, M - 1) * ncv + cv;
       raw[u] = load_raw<T, VEC>(x + static_cast<size_t>(i) * VEC);
       if constexpr (FUSE == 2) zr[u] = load_raw<T, VEC>(z + static_cast<size_t>(i) * VEC);
     }
 #pragma unroll
     for (int u = 0; u < kBnUnroll; ++u) {
-      const uint32_t i = i0 + u * 256u;
-      if (i < total_vec) {
+      const uint32_t row = r0 + u * map.R;
+      const uint32_t i = row * ncv + cv;
+      if (row < M) {
         float o[VEC];
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
@@ -861,18 +897,21 @@ template <typename T, int VEC, bool FUSED = false>
 __global__ void __launch_bounds__(256)
 bn_bwd_apply_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                        T *__restrict__ dx, const BnParam *__restrict__ params,
-                       uint32_t ncv, uint32_t total_vec, int accum, const T *__restrict__ y,
-                       T *__restrict__ dz, int accum_dz) {
+                       uint32_t ncv, uint32_t ntiles, uint32_t M, int accum,
+                       const T *__restrict__ y, T *__restrict__ dz, int accum_dz) {
   constexpr int U = 2;
-  x += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
-  dy += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
-  if (!FUSED || dx) dx += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
+  const size_t slab = static_cast<size_t>(blockIdx.y) * M * ncv * VEC;
+  x += slab;
+  dy += slab;
+  if (!FUSED || dx) dx += slab;
   if constexpr (FUSED) {
-    y += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
-    if (dz) dz += static_cast<size_t>(blockIdx.y) * total_vec * VEC;
+    y += slab;
+    if (dz) dz += slab;
   }
   params += static_cast<size_t>(blockIdx.y) * ncv * VEC;
-  const uint32_t cv = threadIdx.x % ncv;
+  const ClApplyMap map = cl_apply_map<U>(ncv, ntiles);
+  if (!map.active) return;
+  const uint32_t cv = map.cv;
   // dx = pa*dy + pb*(x - mean) + pc = pa*dy + (pb*x + ps), ps = pc - pb*mean:
   // pb*(x-mean) is the small curvature term, so folding the mean costs nothing
   // measurable in float either (|pb*mean| <= |dvar|*2|mean|/N).
@@ -884,13 +923,12 @@ bn_bwd_apply_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
     pb[j] = q.b;
     ps[j] = fmaf(-q.b, q.mean, q.c);
   }
-  for (uint32_t i0 = blockIdx.x * (256u * U) + threadIdx.x; i0 < total_vec;
-       i0 += gridDim.x * (256u * U)) {
+  for (uint32_t r0 = map.row0; r0 < M; r0 += map.row_step) {
     RawVec<T, VEC> xr[U], dr[U];
     RawVec<T, VEC> yr[FUSED ? U : 1];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const uint32_t i = min(i0 + u * 256u, total_vec - 1);
+      const uint32_t i = min(r0 + u * map.R, M - 1) * ncv + cv;
       xr[u] = load_raw<T, VEC>(x + static_cast<size_t>(i) * VEC);
       dr[u] = load_raw<T, VEC>(dy + static_cast<size_t>(i) * VEC);
       if constexpr (FUSED) yr[u] = load_raw<T, VEC>(y + static_cast<size_t>(i) * VEC);
@@ -901,8 +939,9 @@ bn_bwd_apply_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const uint32_t i = i0 + u * 256u;
-      if (i < total_vec) {
+      const uint32_t row = r0 + u * map.R;
+      const uint32_t i = row * ncv + cv;
+      if (row < M) {
         if constexpr (FUSED) {
           if (dz) {
             T *dzp = dz + static_cast<size_t>(i) * VEC;
@@ -1062,37 +1101,6 @@ gn_cl_finalize_bwd_kernel(const float *__restrict__ part2, uint32_t S, uint32_t 
     q.b = f1;
     q.c = f2;
     params[nc] = q;
-  }
-}
-
-// Generic (scalar) apply steps for channel-last slabs whose channel count
-// does not fit the register-resident parameter layout: element i of the whole
-// tensor belongs to slab i / slab_elems and channel i % C.
-template <typename T>
-__global__ void __launch_bounds__(256)
-cl_slab_apply_kernel(const T *__restrict__ x, T *__restrict__ y,
-                     const BnParam *__restrict__ params, FastDiv slab_elems, FastDiv cdiv,
-                     uint32_t total) {
-  for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
-    const uint32_t n = slab_elems.div(i);
-    const uint32_t c = i - cdiv.div(i) * cdiv.d;
-    const BnParam q = params[n * cdiv.d + c];
-    y[i] = from_f32<T>((to_f32<T>(x[i]) - q.mean) * q.a + q.b);
-  }
-}
-
-template <typename T>
-__global__ void __launch_bounds__(256)
-cl_slab_bwd_apply_kernel(const T *__restrict__ x, const T *__restrict__ dy, T *__restrict__ dx,
-                         const BnParam *__restrict__ params, FastDiv slab_elems, FastDiv cdiv,
-                         uint32_t total, int accum) {
-  for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
-    const uint32_t n = slab_elems.div(i);
-    const uint32_t c = i - cdiv.div(i) * cdiv.d;
-    const BnParam q = params[n * cdiv.d + c];
-    float o = q.a * to_f32<T>(dy[i]) + q.b * (to_f32<T>(x[i]) - q.mean) + q.c;
-    if (accum) o += to_f32<T>(dx[i]);
-    dx[i] = from_f32<T>(o);
   }
 }
 

@@ -21,7 +21,6 @@ struct BnPlan {
   uint32_t rps = 1;     // rows per split
   uint32_t ytiles = 1;  // ceil(ncv / TX)
   uint32_t S = 1;       // splits
-  bool cl_fast_apply = false;
   int apply_vec = 1;    // vector width of the apply kernels
   bool direct = false;  // planes: one 1024-thread block owns a whole channel
   // planes whose length is no multiple of the vector width: tensor-aligned
@@ -42,6 +41,35 @@ uint32_t ceil_div_u(uint64_t a, uint64_t b) { return static_cast<uint32_t>((a + 
 uint32_t split_target(bool channel_last) {
   return static_cast<uint32_t>(device_cus()) *
          (channel_last ? tune_int("BN_CL_BLOCKS_PER_CU", 4) : tune_int("BN_BLOCKS_PER_CU", 16));
+}
+
+// Vector width of the channel-last kernels: rows of C elements must be a whole
+// number of vectors (16 bytes; 8 bytes for fp16 rows of 4k channels).
+int cl_vec(int64_t C, int dtype, bool ptr_aligned) {
+  if (!ptr_aligned) return 1;
+  const int full = dtype == NBLAHIP_F16 ? 8 : 4;
+  if (C % full == 0) return full;
+  return (dtype == NBLAHIP_F16 && C % 4 == 0) ? 4 : 1;
+}
+
+// Grid of a channel-last apply kernel over `slabs` slabs of M rows of ncv
+// vectors: column tiles times row blocks, about per_cu blocks per CU in all
+// (the kernels load their parameters into registers once per thread, so they
+// run as a persistent grid).
+struct ClApplyGrid {
+  uint32_t x, ntiles;
+};
+ClApplyGrid cl_apply_grid(uint64_t M, uint32_t ncv, int unroll, int per_cu, uint64_t slabs) {
+  ClApplyGrid g;
+  const uint32_t cols = std::min(ncv, 256u);
+  const uint64_t rows_per_step = static_cast<uint64_t>(256u / cols) * unroll;
+  g.ntiles = ceil_div_u(ncv, 256);
+  const uint64_t need = (M + rows_per_step - 1) / rows_per_step;
+  const uint64_t cap =
+      per_cu > 0 ? std::max<uint64_t>(1, static_cast<uint64_t>(device_cus()) * per_cu / slabs / g.ntiles)
+                 : (1u << 20);
+  g.x = g.ntiles * static_cast<uint32_t>(std::max<uint64_t>(1, std::min(need, cap)));
+  return g;
 }
 
 BnPlan make_plan(int64_t size0, int64_t C, int64_t size2, int dtype, bool ptr_aligned) {
@@ -82,7 +110,7 @@ BnPlan make_plan(int64_t size0, int64_t C, int64_t size2, int dtype, bool ptr_al
       pl.chunk = pl.vpc;
     }
   } else {
-    pl.vec = (ptr_aligned && C % full == 0) ? full : 1;
+    pl.vec = cl_vec(C, dtype, ptr_aligned);
     pl.ncv = static_cast<uint32_t>(C / pl.vec);
     uint32_t l2 = 0;
     while ((1u << l2) < pl.ncv && l2 < 6) ++l2; // TX = min(pow2ceil(ncv), 64)
@@ -100,11 +128,8 @@ BnPlan make_plan(int64_t size0, int64_t C, int64_t size2, int dtype, bool ptr_al
     const uint32_t S = std::min(want, most);
     pl.rps = ceil_div_u(M, S);
     pl.S = ceil_div_u(M, pl.rps);
-    pl.cl_fast_apply = (256u % pl.ncv) == 0;
   }
-  // Channel-last without the register-resident parameters falls back to one
-  // element per thread, where channel = index % C.
-  pl.apply_vec = (pl.channel_last && !pl.cl_fast_apply) ? 1 : pl.vec;
+  pl.apply_vec = pl.vec;
   return pl;
 }
 
@@ -118,13 +143,9 @@ BnParamSrc param_src(const BnParam *params) {
   return s;
 }
 
-// Channel-last apply kernels load their per-channel parameters into registers
-// once per thread, so they run as a persistent grid (cl = true).
-int apply_grid(uint32_t total_vec, int unroll, bool cl = false, bool fwd = false) {
+int apply_grid(uint32_t total_vec, int unroll) {
   const uint64_t blocks = (static_cast<uint64_t>(total_vec) + 256ull * unroll - 1) / (256ull * unroll);
-  const int per_cu = !cl ? tune_int("BN_APPLY_BLOCKS_PER_CU", 0)
-                         : fwd ? tune_int("BN_CL_FWD_APPLY_BLOCKS_PER_CU", 2)
-                               : tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 4);
+  const int per_cu = tune_int("BN_APPLY_BLOCKS_PER_CU", 0);
   const uint64_t cap = per_cu > 0 ? static_cast<uint64_t>(device_cus()) * per_cu : (1u << 20);
   return static_cast<int>(std::max<uint64_t>(1, std::min<uint64_t>(blocks, cap)));
 }
@@ -140,13 +161,13 @@ int fwd_apply_fuse_t(const BnProblem &p, const BnPlan &pl, const BnParamSrc &src
   T *y = static_cast<T *>(p.out);
   const uint64_t total = static_cast<uint64_t>(p.size0) * p.C * p.size2;
   const uint32_t total_vec = static_cast<uint32_t>(total / VEC);
-  if (pl.channel_last && pl.cl_fast_apply) {
+  if (pl.channel_last) {
+    const ClApplyGrid g = cl_apply_grid(static_cast<uint64_t>(p.size0), pl.ncv, kBnUnroll,
+                                        tune_int("BN_CL_FWD_APPLY_BLOCKS_PER_CU", 2), 1);
     NBLAHIP_LAUNCH(FUSE ? "bn_apply_cl_kernel_fused" : "bn_apply_cl_kernel",
-                   (bn_apply_cl_kernel<T, VEC, FUSE>), dim3(apply_grid(total_vec, kBnUnroll, true, true)),
-                   dim3(256), 0, st, x, y, src, pl.ncv, total_vec, z, 1.0f);
+                   (bn_apply_cl_kernel<T, VEC, FUSE>), dim3(g.x), dim3(256), 0, st, x, y, src,
+                   pl.ncv, g.ntiles, static_cast<uint32_t>(p.size0), z, 1.0f);
   } else {
-    // channel-last without the register fast path: planes of one vector each.
-    const uint32_t nvp = pl.channel_last ? 1u : pl.nvp;
     if constexpr (kFullVec<T, VEC>) {
       if (pl.masked) {
         NBLAHIP_LAUNCH(FUSE ? "bn_apply_planes_kernel_fused" : "bn_apply_planes_kernel",
@@ -158,8 +179,8 @@ int fwd_apply_fuse_t(const BnProblem &p, const BnPlan &pl, const BnParamSrc &src
     }
     NBLAHIP_LAUNCH(FUSE ? "bn_apply_planes_kernel_fused" : "bn_apply_planes_kernel",
                    (bn_apply_planes_kernel<T, VEC, FUSE>), dim3(apply_grid(total_vec, kBnUnroll)),
-                   dim3(256), 0, st, x, y, src, FastDiv(nvp), FastDiv(static_cast<uint32_t>(p.C)),
-                   total_vec, z);
+                   dim3(256), 0, st, x, y, src, FastDiv(pl.nvp),
+                   FastDiv(static_cast<uint32_t>(p.C)), total_vec, z);
   }
   return last_launch_status();
 }
@@ -278,13 +299,14 @@ int bwd_apply_fuse_t(const BnProblem &p, const BnPlan &pl, const BnParam *params
   T *dz = static_cast<T *>(p.dz);
   const uint64_t total = static_cast<uint64_t>(p.size0) * p.C * p.size2;
   const uint32_t total_vec = static_cast<uint32_t>(total / VEC);
-  if (pl.channel_last && pl.cl_fast_apply) {
+  if (pl.channel_last) {
+    const ClApplyGrid g = cl_apply_grid(static_cast<uint64_t>(p.size0), pl.ncv, 2,
+                                        tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 4), 1);
     NBLAHIP_LAUNCH(FUSED ? "bn_bwd_apply_cl_kernel_fused" : "bn_bwd_apply_cl_kernel",
-                   (bn_bwd_apply_cl_kernel<T, VEC, FUSED>), dim3(apply_grid(total_vec, 2, true)),
-                   dim3(256), 0, st, x, dy, dx, params, pl.ncv, total_vec, p.accum_dx, y, dz,
+                   (bn_bwd_apply_cl_kernel<T, VEC, FUSED>), dim3(g.x), dim3(256), 0, st, x, dy, dx,
+                   params, pl.ncv, g.ntiles, static_cast<uint32_t>(p.size0), p.accum_dx, y, dz,
                    p.accum_dz);
   } else {
-    const uint32_t nvp = pl.channel_last ? 1u : pl.nvp;
     if constexpr (kFullVec<T, VEC>) {
       if (pl.masked) {
         NBLAHIP_LAUNCH(FUSED ? "bn_bwd_apply_planes_kernel_fused" : "bn_bwd_apply_planes_kernel",
@@ -297,7 +319,7 @@ int bwd_apply_fuse_t(const BnProblem &p, const BnPlan &pl, const BnParam *params
     }
     NBLAHIP_LAUNCH(FUSED ? "bn_bwd_apply_planes_kernel_fused" : "bn_bwd_apply_planes_kernel",
                    (bn_bwd_apply_planes_kernel<T, VEC, FUSED>), dim3(apply_grid(total_vec, 2)),
-                   dim3(256), 0, st, x, dy, dx, params, FastDiv(nvp),
+                   dim3(256), 0, st, x, dy, dx, params, FastDiv(pl.nvp),
                    FastDiv(static_cast<uint32_t>(p.C)), total_vec, p.accum_dx, y, dz, p.accum_dz);
   }
   return last_launch_status();
@@ -497,7 +519,7 @@ BnPlan make_cl_plan(int64_t batch, int64_t spatial, int64_t C, int dtype, bool p
   BnPlan pl;
   const int full = dtype == NBLAHIP_F16 ? 8 : 4;
   pl.channel_last = true;
-  pl.vec = (ptr_aligned && C % full == 0) ? full : 1;
+  pl.vec = cl_vec(C, dtype, ptr_aligned);
   pl.ncv = static_cast<uint32_t>(C / pl.vec);
   uint32_t l2 = 0;
   while ((1u << l2) < pl.ncv && l2 < 6) ++l2;
@@ -514,8 +536,7 @@ BnPlan make_cl_plan(int64_t batch, int64_t spatial, int64_t C, int dtype, bool p
   const uint32_t S = std::min(want, most);
   pl.rps = ceil_div_u(M, S);
   pl.S = ceil_div_u(M, pl.rps);
-  pl.cl_fast_apply = (256u % pl.ncv) == 0;
-  pl.apply_vec = pl.cl_fast_apply ? pl.vec : 1;
+  pl.apply_vec = pl.vec;
   return pl;
 }
 
@@ -557,23 +578,13 @@ int cl_stats_t(const ClProblem &p, const BnPlan &pl, float *part, hipStream_t st
 
 template <typename T, int VEC>
 int cl_apply_t(const ClProblem &p, const BnPlan &pl, const BnParam *params, hipStream_t st) {
-  const uint64_t slab = static_cast<uint64_t>(p.spatial) * p.channels;
-  if (pl.cl_fast_apply) {
-    const uint32_t slab_vec = static_cast<uint32_t>(slab / VEC);
-    const uint64_t per_slab = std::max<uint64_t>(
-        1, static_cast<uint64_t>(device_cus()) * tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 4) / p.batch);
-    const uint64_t need = (static_cast<uint64_t>(slab_vec) + 256ull * kBnUnroll - 1) / (256ull * kBnUnroll);
-    NBLAHIP_LAUNCH("bn_apply_cl_kernel", (bn_apply_cl_kernel<T, VEC>),
-                   dim3(static_cast<uint32_t>(std::min(need, per_slab)), static_cast<uint32_t>(p.batch)),
-                   dim3(256), 0, st, static_cast<const T *>(p.x), static_cast<T *>(p.out),
-                   param_src(params), pl.ncv, slab_vec, static_cast<const T *>(nullptr), 1.0f);
-  } else {
-    const uint32_t total = static_cast<uint32_t>(slab * p.batch);
-    NBLAHIP_LAUNCH("cl_slab_apply_kernel", (cl_slab_apply_kernel<T>),
-                   dim3(apply_grid(total, 1)), dim3(256), 0, st, static_cast<const T *>(p.x),
-                   static_cast<T *>(p.out), params, FastDiv(static_cast<uint32_t>(slab)),
-                   FastDiv(static_cast<uint32_t>(p.channels)), total);
-  }
+  const ClApplyGrid g = cl_apply_grid(static_cast<uint64_t>(p.spatial), pl.ncv, kBnUnroll,
+                                      tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 4),
+                                      static_cast<uint64_t>(p.batch));
+  NBLAHIP_LAUNCH("bn_apply_cl_kernel", (bn_apply_cl_kernel<T, VEC>),
+                 dim3(g.x, static_cast<uint32_t>(p.batch)), dim3(256), 0, st,
+                 static_cast<const T *>(p.x), static_cast<T *>(p.out), param_src(params), pl.ncv,
+                 g.ntiles, static_cast<uint32_t>(p.spatial), static_cast<const T *>(nullptr), 1.0f);
   return last_launch_status();
 }
 
@@ -591,25 +602,14 @@ int cl_bwd_reduce_t(const ClProblem &p, const BnPlan &pl, float *part2, hipStrea
 
 template <typename T, int VEC>
 int cl_bwd_apply_t(const ClProblem &p, const BnPlan &pl, const BnParam *params, hipStream_t st) {
-  const uint64_t slab = static_cast<uint64_t>(p.spatial) * p.channels;
-  if (pl.cl_fast_apply) {
-    const uint32_t slab_vec = static_cast<uint32_t>(slab / VEC);
-    const uint64_t per_slab = std::max<uint64_t>(
-        1, static_cast<uint64_t>(device_cus()) * tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 4) / p.batch);
-    const uint64_t need = (static_cast<uint64_t>(slab_vec) + 256ull * 2 - 1) / (256ull * 2);
-    NBLAHIP_LAUNCH("bn_bwd_apply_cl_kernel", (bn_bwd_apply_cl_kernel<T, VEC>),
-                   dim3(static_cast<uint32_t>(std::min(need, per_slab)), static_cast<uint32_t>(p.batch)),
-                   dim3(256), 0, st, static_cast<const T *>(p.x), static_cast<const T *>(p.dy),
-                   static_cast<T *>(p.out), params, pl.ncv, slab_vec, p.accum_dx,
-                   static_cast<const T *>(nullptr), static_cast<T *>(nullptr), 0);
-  } else {
-    const uint32_t total = static_cast<uint32_t>(slab * p.batch);
-    NBLAHIP_LAUNCH("cl_slab_bwd_apply_kernel", (cl_slab_bwd_apply_kernel<T>),
-                   dim3(apply_grid(total, 1)), dim3(256), 0, st, static_cast<const T *>(p.x),
-                   static_cast<const T *>(p.dy), static_cast<T *>(p.out), params,
-                   FastDiv(static_cast<uint32_t>(slab)), FastDiv(static_cast<uint32_t>(p.channels)),
-                   total, p.accum_dx);
-  }
+  const ClApplyGrid g = cl_apply_grid(static_cast<uint64_t>(p.spatial), pl.ncv, 2,
+                                      tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 4),
+                                      static_cast<uint64_t>(p.batch));
+  NBLAHIP_LAUNCH("bn_bwd_apply_cl_kernel", (bn_bwd_apply_cl_kernel<T, VEC>),
+                 dim3(g.x, static_cast<uint32_t>(p.batch)), dim3(256), 0, st,
+                 static_cast<const T *>(p.x), static_cast<const T *>(p.dy), static_cast<T *>(p.out),
+                 params, pl.ncv, g.ntiles, static_cast<uint32_t>(p.spatial), p.accum_dx,
+                 static_cast<const T *>(nullptr), static_cast<T *>(nullptr), 0);
   return last_launch_status();
 }
 

@@ -21,6 +21,9 @@ SMALL = [
     # planes that are no multiple of the vector width, tensor a multiple: masked vectors
     ((4, 8, 7, 7), 1), ((2, 16, 9, 9), 1), ((3, 8, 3, 11), 1), ((1, 24, 5, 5), 1),
     ((64, 32, 7, 7), 1), ((5, 16, 13), 1),
+    # channel-last: channel vectors that do not divide 256, rows wider than 256 vectors,
+    # 8-byte fp16 rows
+    ((6, 9, 9, 96), 3), ((3, 5, 5, 4104), 3), ((37, 100), 1), ((4, 6, 6, 20), 3), ((700, 1032), 1),
 ]
 DTYPES = [torch.float32, torch.float16]
 

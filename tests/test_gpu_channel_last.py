@@ -45,7 +45,9 @@ GN_CL_SHAPES = [(2, (8, 8), 8, 4), (3, (5,), 6, 2), (1, (2, 2), 4, 1), (2, (4,),
                 (2, (7, 7), 32, 8), (2, (14, 14), 24, 4), (4, (16, 16), 64, 8),
                 (2, (32, 32), 16, 2), (2, (64, 64), 256, 32), (1, (128, 128), 8, 1),
                 (2, (512,), 12, 3), (2, (), 4, 2), (3, (64,), 10, 5), (1, (40, 40), 40, 2),
-                (2, (3, 3), 2048, 32), (2, (4096,), 32, 4), (5, (33,), 7, 7), (1, (1,), 5, 1)]
+                (2, (3, 3), 2048, 32), (2, (4096,), 32, 4), (5, (33,), 7, 7), (1, (1,), 5, 1),
+                # channel vectors that do not divide 256, rows wider than 256 vectors, 8-byte fp16 rows
+                (2, (9, 9), 96, 4), (2, (5, 5), 4104, 8), (3, (11,), 100, 5), (2, (6, 6), 20, 2)]
 
 
 @pytest.mark.parametrize("n,sp,c,groups", GN_CL_SHAPES)
@@ -70,7 +72,8 @@ def test_gn_channel_last(n, sp, c, groups, dtype):
 
 IN_CL_SHAPES = [(2, (4, 4), 3), (3, (7,), 5), (1, (3, 2), 2), (4, (16, 16), 16), (2, (64, 64), 8),
                 (2, (7, 7), 24), (1, (200, 200), 3), (2, (300, 300), 2), (3, (1,), 7),
-                (2, (1000,), 64), (2, (5, 5), 1024), (16, (32, 32), 256)]
+                (2, (1000,), 64), (2, (5, 5), 1024), (16, (32, 32), 256),
+                (2, (9, 9), 96), (2, (5, 5), 4104), (3, (11,), 100), (2, (300,), 1032)]
 
 
 @pytest.mark.parametrize("n,sp,c", IN_CL_SHAPES)

@@ -25,6 +25,7 @@ SHAPES = [
     ((3, 2, 2, 2050), 3), ((2, 256, 9, 9), 1), ((8, 14, 14, 64), 3),
     ((8, 12, 14, 14), 1), ((16, 256, 14, 14), 1),
     ((4, 8, 7, 7), 1), ((64, 32, 7, 7), 1), ((5, 16, 13), 1),
+    ((6, 9, 9, 96), 3), ((3, 5, 5, 4104), 3), ((37, 100), 1),
 ]
 
 
