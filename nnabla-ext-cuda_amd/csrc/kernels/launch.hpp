@@ -14,7 +14,9 @@ namespace nblahip {
 
 // kRowINc: InstanceNormalization backward with a block per channel that walks
 // the batch itself, so dgamma/dbeta need no second kernel.
-enum RowMode { kRowLN = 0, kRowIN = 1, kRowGN = 2, kRowINc = 3 };
+// kRowGNm: GroupNormalization backward with the run-time thread map (planes
+// that are no multiple of a wave-wide load); kRowGN is the fixed map.
+enum RowMode { kRowLN = 0, kRowIN = 1, kRowGN = 2, kRowINc = 3, kRowGNm = 4 };
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

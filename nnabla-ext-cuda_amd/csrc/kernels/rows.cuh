@@ -52,11 +52,45 @@ struct RowArgs {
   float *dbeta;
   int accum_g;
   int accum_b;
-  // GroupNormalization backward: entries (64*VEC-element runs) per channel and
-  // channels per group.
+  // GroupNormalization backward: runs (wave-wide loads) per channel and
+  // channels per group, and the thread map (see GnSlot).
   int epc;
   int cpg;
+  int gn_wpc;      // waves sharing one channel
+  int gn_nwc;      // channels the block's waves cover at once (NW / gn_wpc)
+  int gn_pv;       // vectors per plane (spatial / VEC)
+  uint64_t gn_map; // per load k, 8 bits: (pass over the channels) | (load within the channel) << 4; 0xff unused
 };
+
+// GroupNormalization backward thread map.  A wave-wide load never crosses a
+// channel, so the per-channel sums the parameter gradients need are wave sums.
+// The block's NW waves are split into gn_nwc sets of gn_wpc waves; in pass ci a
+// set works on channel ci*gn_nwc + set, whose plane its waves cover in runs of
+// 64 vectors: load m of wave j of the set is run m*gn_wpc + j of that channel
+// (lanes past the plane's end idle).  Channels with small planes therefore
+// share a wave's loads over several passes, channels with large planes spread
+// over several waves, and the plane only has to be a whole number of vectors.
+struct GnSlot {
+  uint32_t ch; // channel within the group
+  int run;     // index into the block's run sums: ch*epc + run within the channel
+  int col;     // first element within the row
+  bool ok;     // this lane holds data
+  bool live;   // the wave's run exists (its sums are recorded, zeros included)
+};
+
+template <int VEC>
+__device__ __forceinline__ GnSlot gn_slot(const RowArgs &a, int k, int set, int j, int lane) {
+  GnSlot s;
+  const uint32_t code = static_cast<uint32_t>(a.gn_map >> (8 * k)) & 0xffu;
+  const int ci = code & 15, m = code >> 4;
+  s.ch = static_cast<uint32_t>(ci * a.gn_nwc + set);
+  const int part = m * a.gn_wpc + j;
+  s.live = code != 0xffu && set < a.gn_nwc && static_cast<int>(s.ch) < a.cpg;
+  s.ok = s.live && lane < a.gn_pv - part * kWave;
+  s.run = static_cast<int>(s.ch) * a.epc + part;
+  s.col = (static_cast<int>(s.ch * a.pdiv.d) + part * (kWave * VEC)) + lane * VEC;
+  return s;
+}
 
 template <int TPR> struct RowBlock {
   static constexpr int kBlock = TPR < 256 ? 256 : TPR;
@@ -85,7 +119,8 @@ template <int TPR, int MODE> struct RowBwdBlock {
 // spill the cap costs it sits in its row loop and is worth more than the
 // occupancy.
 template <typename T, int VEC, int NL, int TPR, int MODE> struct RowBwdOccupancy {
-  static constexpr bool kGn512 = MODE == kRowGN && TPR == 512 && NL == 8 && sizeof(T) == 2;
+  static constexpr bool kGn512 =
+      (MODE == kRowGN || MODE == kRowGNm) && TPR == 512 && NL == 8 && sizeof(T) == 2;
   static constexpr int kMinWaves = kGn512 ? 4 : 1;
 };
 
@@ -217,8 +252,9 @@ row_fwd_kernel(const RowArgs a) {
 // Partial parameter gradients written to ws:
 //   LN : ws[block][0][R] = sum_rows dy*xh, ws[block][1][R] = sum_rows dy
 //   IN : ws[2*row] = sum dy*xh, ws[2*row+1] = sum dy             (row = (n,c))
-//   GN : same pair per (n, channel); requires spatial % (64*VEC) == 0 so that
-//        every wave-wide load belongs to one channel.
+//   GN : same pair per (n, channel); every wave-wide load lies inside one
+//        channel, by the fixed map when spatial % (64*VEC) == 0 (kRowGN), else by
+//        the run-time map of GnSlot (kRowGNm).
 // Padded lanes hold x = dy = 0 in registers; dy == 0 keeps them out of every
 // sum.
 // ---------------------------------------------------------------------------
@@ -231,8 +267,10 @@ row_bwd_kernel(const RowArgs a) {
   // LayerNormalization keeps xh and dg of a row in registers between the
   // reduction and the dx step when they are few; otherwise they are recomputed.
   constexpr bool KEEP = (MODE == kRowLN) && (NL * VEC <= 16);
+  constexpr bool GN = MODE == kRowGN || MODE == kRowGNm;
+  constexpr bool GNM = MODE == kRowGNm; // run-time thread map (GnSlot)
   __shared__ float lds[2 * 16];
-  __shared__ float part[(MODE == kRowGN) ? 2 * NW * NL : 1];
+  __shared__ float part[GN ? 2 * NW * NL : 1];
   __shared__ float xwave[(MODE == kRowLN && RPB > 1) ? (RPB - 1) * kWave * VEC : 1];
   const int t = threadIdx.x % TPR;
   const int sub = threadIdx.x / TPR;
@@ -258,6 +296,16 @@ row_bwd_kernel(const RowArgs a) {
     }
   }
 
+  // GroupNormalization: this wave's set, its place within the set, the lane.
+  int gn_set = 0, gn_j = 0, gn_lane = 0;
+  if constexpr (GNM) {
+    // wave-uniform, and told so: the map then costs scalar instructions only
+    const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x / kWave));
+    gn_set = wave / a.gn_wpc;
+    gn_j = wave - gn_set * a.gn_wpc;
+    gn_lane = threadIdx.x & (kWave - 1);
+  }
+
   // Iteration space.  Every mode but kRowINc: one unit = one row, rows strided
   // over the grid.  kRowINc: one unit = one channel (block-strided), whose
   // batch*1 rows (n, c) are strided over the block's waves / walked in turn.
@@ -274,22 +322,32 @@ row_bwd_kernel(const RowArgs a) {
     const size_t base = static_cast<size_t>(row) * a.R;
     float gk[NL];                                   // per-load scalar gamma (IN / GN)
     float gch = 1.f;                                // GN: gamma of channel threadIdx.x
-    if constexpr (MODE == kRowGN) {
+    if constexpr (GN) {
       // Issued ahead of the row data, so their latency hides behind it.
       const uint32_t pb = (static_cast<uint32_t>(row) % a.pmod) * a.pmul;
 #pragma unroll
       for (int k = 0; k < NL; ++k) {
-        const int col = (k * TPR + t) * VEC;
-        const uint32_t ch = (col < a.R) ? a.pdiv.div(static_cast<uint32_t>(col)) : 0u;
-        gk[k] = a.gamma ? a.gamma[pb + ch] : 1.f;
+        if constexpr (GNM) {
+          const GnSlot sl = gn_slot<VEC>(a, k, gn_set, gn_j, gn_lane);
+          gk[k] = (a.gamma && sl.live) ? a.gamma[pb + sl.ch] : 1.f;
+        } else {
+          const int col = (k * TPR + t) * VEC;
+          const uint32_t ch = (col < a.R) ? a.pdiv.div(static_cast<uint32_t>(col)) : 0u;
+          gk[k] = a.gamma ? a.gamma[pb + ch] : 1.f;
+        }
       }
       if (a.gamma && static_cast<int>(threadIdx.x) < a.cpg) gch = a.gamma[pb + threadIdx.x];
     }
     RawVec<T, VEC> xr[NL], dr[NL];
 #pragma unroll
     for (int k = 0; k < NL; ++k) {
-      const int col = (k * TPR + t) * VEC;
-      const bool ok = col < a.R;
+      int col = (k * TPR + t) * VEC;
+      bool ok = col < a.R;
+      if constexpr (GNM) {
+        const GnSlot sl = gn_slot<VEC>(a, k, gn_set, gn_j, gn_lane);
+        col = sl.col;
+        ok = sl.ok;
+      }
       const int colc = ok ? col : 0; // branch-free: all loads in flight together
       xr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + base + colc));
       dr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(dy + base + colc));
@@ -347,8 +405,7 @@ row_bwd_kernel(const RowArgs a) {
       s1 = g * sdy;
       t2 = g * sdx;
     } else { // GroupNormalization, RPB == 1
-      static_assert(MODE != kRowGN || RPB == 1, "group rows own the whole block");
-      const int wave = threadIdx.x / kWave;
+      static_assert(!GN || RPB == 1, "group rows own the whole block");
       const int lane = threadIdx.x & (kWave - 1);
       const uint32_t pbase = (static_cast<uint32_t>(row) % a.pmod) * a.pmul;
       lds_barrier(); // part[] of the previous row has been consumed
@@ -363,10 +420,19 @@ row_bwd_kernel(const RowArgs a) {
         }
         sdy = wave_sum(sdy);
         sdx = wave_sum(sdx);
-        const int e = k * NW + wave; // run index: elements [e*64*VEC, (e+1)*64*VEC)
-        if (lane == 0) {
-          part[2 * e] = sdx;
-          part[2 * e + 1] = sdy;
+        if constexpr (GNM) {
+          const GnSlot sl = gn_slot<VEC>(a, k, gn_set, gn_j, gn_lane);
+          if (lane == 0 && sl.live) {
+            part[2 * sl.run] = sdx;
+            part[2 * sl.run + 1] = sdy;
+          }
+        } else {
+          // fixed map: run e covers elements [e*64*VEC, (e+1)*64*VEC) of the row
+          const int e = k * NW + static_cast<int>(threadIdx.x / kWave);
+          if (lane == 0) {
+            part[2 * e] = sdx;
+            part[2 * e + 1] = sdy;
+          }
         }
       }
       lds_barrier();
@@ -402,8 +468,14 @@ row_bwd_kernel(const RowArgs a) {
     if (dx != nullptr) {
 #pragma unroll
       for (int k = 0; k < NL; ++k) {
-        const int col = (k * TPR + t) * VEC;
-        if (col < a.R) {
+        int col = (k * TPR + t) * VEC;
+        bool ok = col < a.R;
+        if constexpr (GNM) {
+          const GnSlot sl = gn_slot<VEC>(a, k, gn_set, gn_j, gn_lane);
+          col = sl.col;
+          ok = sl.ok;
+        }
+        if (ok) {
           float o[VEC];
           if constexpr (KEEP) {
 #pragma unroll

@@ -21,6 +21,8 @@ int run_row_bwd_cached_inc(int dtype, const RowCfg &cfg, const RowArgs &args, in
                            hipStream_t st);
 int run_row_bwd_cached_gn(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
                           hipStream_t st);
+int run_row_bwd_cached_gnm(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
+                           hipStream_t st);
 
 // Expands CASE(T, VEC, NL, TPR) for every supported register-cached shape of
 // element type T.

@@ -61,6 +61,54 @@ static RowCfg pick_ln_bwd_cfg(int dtype, int64_t R, bool vec_ok) {
   return c;
 }
 
+// GroupNormalization backward: vector width, block size, loads per thread and
+// the thread map of GnSlot (written into a).  Candidates are the widest vector
+// and scalar loads, and the block sizes whose map fits 8 loads per thread; the
+// cost of one is its lane slots (threads x loads) weighted by 4 + VEC: a load
+// costs the same whether 8 or 64 of its lanes carry data, but the arithmetic
+// behind it grows with the vector, so sparse wide loads lose to dense narrow
+// ones (planes of 64 half elements: 15.5 us with 8 of 64 lanes busy, 9.4 us
+// with scalar loads).
+static RowCfg pick_gn_bwd_cfg(const RowProblem &p, bool vec_ok, RowArgs &a) {
+  RowCfg best;
+  const int full = p.dtype == NBLAHIP_F16 ? 8 : 4;
+  const int64_t cpg = p.channels / p.groups;
+  int64_t best_cost = 0;
+  for (int vec : {full, 1}) {
+    if (vec > 1 && !vec_ok) continue;
+    const int64_t pv = p.spatial / vec;
+    for (int tpr : {256, 512, 1024}) {
+      const int64_t nw = tpr / 64;
+      const int64_t wpc = cpg < nw ? nw / cpg : 1;
+      const int64_t nwc = nw / wpc;
+      const int64_t cpw = (cpg + nwc - 1) / nwc;            // passes over the channels
+      const int64_t nlc = (pv + 64 * wpc - 1) / (64 * wpc); // loads per channel
+      const int64_t need = cpw * nlc;
+      if (need > 8 || nlc > 15 || cpw > 15) continue;
+      int nl = 1;
+      while (nl < need) nl <<= 1;
+      const int64_t cost = static_cast<int64_t>(tpr) * nl * (4 + vec);
+      if (best.ok && cost >= best_cost) continue;
+      best.ok = true;
+      best.vec = vec;
+      best.tpr = tpr;
+      best.nl = nl;
+      best_cost = cost;
+      a.gn_wpc = static_cast<int>(wpc);
+      a.gn_nwc = static_cast<int>(nwc);
+      a.gn_pv = static_cast<int>(pv);
+      a.epc = static_cast<int>(nlc * wpc);
+      uint64_t map = ~0ull;
+      for (int64_t k = 0; k < need; ++k) {
+        const uint64_t code = static_cast<uint64_t>(k / nlc) | (static_cast<uint64_t>(k % nlc) << 4);
+        map = (map & ~(0xffull << (8 * k))) | (code << (8 * k));
+      }
+      a.gn_map = map;
+    }
+  }
+  return best;
+}
+
 static int rows_per_block(int tpr) { return tpr < 256 ? 256 / tpr : 1; }
 
 static int cached_grid(int64_t rows, int tpr) {
@@ -278,17 +326,36 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
   const int nl_small = ln ? 4 : 8;
   const int nl_1024 = ln ? (p.dtype == NBLAHIP_F16 ? 1 : 2) : 8;
   RowCfg cfg = ln ? pick_ln_bwd_cfg(p.dtype, p.R, vec_ok)
-                  : pick_row_cfg(p.dtype, p.R, vec_ok, nl_small, nl_1024,
-                                 p.mode == kRowGN ? 256 : 64);
-  if (cfg.ok && p.mode == kRowGN) {
-    // Every wave-wide load must fall inside one channel.
-    const int64_t run = 64 * static_cast<int64_t>(cfg.vec);
-    if (p.spatial % run != 0) {
-      // Retry with scalar loads (run = 64 elements) before giving up.
-      cfg = pick_row_cfg(p.dtype, p.R, false, 8, 8, 256);
-      if (cfg.ok && p.spatial % 64 != 0) cfg.ok = false;
+                  : pick_row_cfg(p.dtype, p.R, vec_ok, nl_small, nl_1024, 64);
+  bool gn_map = false;
+  if (p.mode == kRowGN) {
+    // Fixed map (every wave-wide load of the plain row layout falls inside one
+    // channel), with the widest vector or with scalar loads, against the
+    // run-time map, by the cost of pick_gn_bwd_cfg; the run-time map pays
+    // about 15 % for its address arithmetic (64 KB half groups: 24.5 vs 21.3 us).
+    auto cost = [](const RowCfg &c) { return static_cast<int64_t>(c.tpr) * c.nl * (4 + c.vec); };
+    RowCfg fixed;
+    for (bool v : {true, false}) {
+      if (v && !vec_ok) continue;
+      const RowCfg c = pick_row_cfg(p.dtype, p.R, v, 8, 8, 256);
+      if (c.ok && p.spatial % (64 * static_cast<int64_t>(c.vec)) == 0 &&
+          (!fixed.ok || cost(c) < cost(fixed)))
+        fixed = c;
     }
-    if (cfg.ok) a.epc = static_cast<int>(p.spatial / (64 * cfg.vec));
+    RowArgs am = a;
+    const RowCfg mapped = pick_gn_bwd_cfg(p, vec_ok, am);
+    if (mapped.ok && (!fixed.ok || cost(mapped) * 115 < cost(fixed) * 100)) {
+      cfg = mapped;
+      a = am;
+      gn_map = true;
+    } else {
+      cfg = fixed;
+      if (cfg.ok) a.epc = static_cast<int>(p.spatial / (64 * cfg.vec));
+    }
+    // The float 1024 x 8 layout (one block per CU, 128 KB of row data in its
+    // registers) loses to the streaming kernels: 92-105 vs 85 us on
+    // 25 088-element groups, 55 vs 56 us on 32 768-element ones.
+    if (cfg.ok && p.dtype == NBLAHIP_F32 && cfg.tpr == 1024 && cfg.nl == 8) cfg.ok = false;
   }
   (void)full;
   if (cfg.ok && !tune_int("FORCE_STREAM", 0)) {
@@ -315,6 +382,7 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
     }
     const int grid = cached_grid(p.rows, cfg.tpr);
     const int e = p.mode == kRowIN ? run_row_bwd_cached_in(p.dtype, cfg, a, grid, st)
+                  : gn_map         ? run_row_bwd_cached_gnm(p.dtype, cfg, a, grid, st)
                                    : run_row_bwd_cached_gn(p.dtype, cfg, a, grid, st);
     if (e) return e;
     return launch_pair_reduce(p, static_cast<const float *>(p.ws), st);

@@ -154,7 +154,12 @@ def test_ln_c3_full_size(dtype):
 GN_SHAPES = [(2, 8, (8, 8), 4), (3, 6, (5,), 2), (1, 4, (2, 2), 1), (2, 6, (4,), 6),
              (2, 32, (7, 7), 8), (2, 32, (14, 14), 4), (4, 64, (16, 16), 8), (2, 16, (32, 32), 2),
              (2, 256, (64, 64), 32), (1, 8, (128, 128), 1), (2, 12, (512,), 3), (2, 4, (), 2),
-             (3, 10, (64,), 5), (1, 64, (40, 40), 2)]
+             (3, 10, (64,), 5), (1, 64, (40, 40), 2),
+             # thread maps of the backward: several channels per wave, several waves per
+             # channel, wave sets that do not divide the block, planes that end inside a load
+             (2, 64, (56, 56), 8), (2, 64, (28, 28), 4), (2, 6, (8, 8), 2), (2, 4, (64, 64), 4),
+             (1, 10, (48, 48), 2), (2, 64, (14, 14), 2), (2, 128, (7, 7), 2), (1, 80, (8, 8), 2),
+             (3, 24, (24, 24), 3), (2, 14, (72,), 2)]
 
 
 def make_nc(n, c, sp, dtype, seed):
