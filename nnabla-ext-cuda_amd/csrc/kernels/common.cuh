@@ -18,6 +18,8 @@ constexpr int kWave = 64;
 template <typename T> struct FullVec;
 template <> struct FullVec<float> { static constexpr int value = 4; };
 template <> struct FullVec<__half> { static constexpr int value = 8; };
+// 8-byte vectors for half rows of 4k elements (float: the full vector again).
+template <typename T> struct MidVec { static constexpr int value = 4; };
 
 template <typename T> __device__ __forceinline__ float to_f32(T v);
 template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }

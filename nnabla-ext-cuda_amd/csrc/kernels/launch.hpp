@@ -56,17 +56,16 @@ struct RowProblem {
   size_t ws_bytes = 0;
 };
 
-// Register-cached configuration: TPR threads per row, NL 16-byte loads each.
+// Register-cached configuration: TPR threads per row, NL loads of vec elements each.
 struct RowCfg {
   bool ok = false;
   int vec = 1, tpr = 64, nl = 1;
 };
 
-// vec_ok: whether the full 16-byte vector width may be used (alignment and
-// divisibility already checked by the caller).  max_nl / max_nl_1024 bound the
-// loads per thread below / at 1024 threads; min_tpr is 256 for the
-// GroupNormalization backward.
-RowCfg pick_row_cfg(int dtype, int64_t R, bool vec_ok, int max_nl, int max_nl_1024, int min_tpr);
+// vec: elements per load (alignment and divisibility already checked by the
+// caller).  max_nl / max_nl_1024 bound the loads per thread below / at 1024
+// threads; min_tpr is 256 for the GroupNormalization backward.
+RowCfg pick_row_cfg(int vec, int64_t R, int max_nl, int max_nl_1024, int min_tpr);
 
 int launch_row_fwd(const RowProblem &p, hipStream_t st);
 int launch_row_bwd(const RowProblem &p, hipStream_t st);

@@ -25,7 +25,8 @@ int run_row_bwd_cached_gnm(int dtype, const RowCfg &cfg, const RowArgs &args, in
                            hipStream_t st);
 
 // Expands CASE(T, VEC, NL, TPR) for every supported register-cached shape of
-// element type T.
+// element type T (for float the MidVec lines repeat the FullVec ones: same
+// instantiations, unreachable branches).
 #define NBLAHIP_ROW_CASES_TPR(CASE, T, VEC, TPR) \
   CASE(T, VEC, 1, TPR) CASE(T, VEC, 2, TPR) CASE(T, VEC, 4, TPR) CASE(T, VEC, 8, TPR)
 
@@ -34,6 +35,10 @@ int run_row_bwd_cached_gnm(int dtype, const RowCfg &cfg, const RowArgs &args, in
   NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 256)    \
   NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 512)    \
   NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 1024)   \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, MidVec<T>::value, 64)      \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, MidVec<T>::value, 256)     \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, MidVec<T>::value, 512)     \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, MidVec<T>::value, 1024)    \
   NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 64)                     \
   NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 256)                    \
   NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 512)                    \
@@ -43,6 +48,9 @@ int run_row_bwd_cached_gnm(int dtype, const RowCfg &cfg, const RowArgs &args, in
   NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 256)    \
   NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 512)    \
   NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 1024)   \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, MidVec<T>::value, 256)     \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, MidVec<T>::value, 512)     \
+  NBLAHIP_ROW_CASES_TPR(CASE, T, MidVec<T>::value, 1024)    \
   NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 256)                    \
   NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 512)                    \
   NBLAHIP_ROW_CASES_TPR(CASE, T, 1, 1024)

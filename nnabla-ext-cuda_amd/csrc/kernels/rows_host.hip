@@ -11,10 +11,9 @@ namespace nblahip {
 // max_nl bounds the loads per thread of the layouts below 1024 threads,
 // max_nl_1024 those of the 1024-thread layout, whose register budget is 128
 // VGPRs; both are chosen per kernel family so that no variant in use spills.
-RowCfg pick_row_cfg(int dtype, int64_t R, bool vec_ok, int max_nl, int max_nl_1024, int min_tpr) {
+RowCfg pick_row_cfg(int vec, int64_t R, int max_nl, int max_nl_1024, int min_tpr) {
   RowCfg c;
-  const int full = dtype == NBLAHIP_F16 ? 8 : 4;
-  c.vec = vec_ok ? full : 1;
+  c.vec = vec;
   const int64_t nv = R / c.vec;
   static const int tprs[4] = {64, 256, 512, 1024};
   static const int nls[4] = {1, 2, 4, 8};
@@ -39,10 +38,9 @@ RowCfg pick_row_cfg(int dtype, int64_t R, bool vec_ok, int max_nl, int max_nl_10
 // 256 or 512 threads with the fewest loads per thread (the per-column
 // accumulators make every load cost about 27 VGPRs), and the 1024-thread
 // layout, the slowest, only for rows nothing else holds.
-static RowCfg pick_ln_bwd_cfg(int dtype, int64_t R, bool vec_ok) {
+static RowCfg pick_ln_bwd_cfg(int dtype, int64_t R, int vec) {
   RowCfg c;
-  const int full = dtype == NBLAHIP_F16 ? 8 : 4;
-  c.vec = vec_ok ? full : 1;
+  c.vec = vec;
   const int64_t nv = R / c.vec;
   auto take = [&](int tpr, int nl) {
     c.ok = true;
@@ -69,13 +67,11 @@ static RowCfg pick_ln_bwd_cfg(int dtype, int64_t R, bool vec_ok) {
 // behind it grows with the vector, so sparse wide loads lose to dense narrow
 // ones (planes of 64 half elements: 15.5 us with 8 of 64 lanes busy, 9.4 us
 // with scalar loads).
-static RowCfg pick_gn_bwd_cfg(const RowProblem &p, bool vec_ok, RowArgs &a) {
+static RowCfg pick_gn_bwd_cfg(const RowProblem &p, int row_vec, RowArgs &a) {
   RowCfg best;
-  const int full = p.dtype == NBLAHIP_F16 ? 8 : 4;
   const int64_t cpg = p.channels / p.groups;
   int64_t best_cost = 0;
-  for (int vec : {full, 1}) {
-    if (vec > 1 && !vec_ok) continue;
+  for (int vec : {row_vec, 1}) {
     const int64_t pv = p.spatial / vec;
     for (int tpr : {256, 512, 1024}) {
       const int64_t nw = tpr / 64;
@@ -181,19 +177,24 @@ static RowArgs make_args(const RowProblem &p) {
   return a;
 }
 
-static bool row_vec_ok(const RowProblem &p, bool backward) {
-  const int full = p.dtype == NBLAHIP_F16 ? 8 : 4;
-  if (p.R % full != 0) return false;
-  if (!aligned16(p.x)) return false;
-  if (p.out && !aligned16(p.out)) return false;
-  if (backward && !aligned16(p.dy)) return false;
+// Vector width of the row kernels: rows (and GroupNormalization planes) must
+// be a whole number of vectors and every pointer 16-byte aligned; 16 bytes, or
+// 8 bytes for half rows of 4k elements, else scalar.
+static int row_vec(const RowProblem &p, bool backward) {
+  if (!aligned16(p.x)) return 1;
+  if (p.out && !aligned16(p.out)) return 1;
+  if (backward && !aligned16(p.dy)) return 1;
   if (p.mode == kRowLN) {
-    if (p.gamma && !aligned16(p.gamma)) return false;
-    if (!backward && p.beta && !aligned16(p.beta)) return false;
-  } else if (p.mode == kRowGN) {
-    if (p.spatial % full != 0) return false;
+    if (p.gamma && !aligned16(p.gamma)) return 1;
+    if (!backward && p.beta && !aligned16(p.beta)) return 1;
   }
-  return true;
+  const int full = p.dtype == NBLAHIP_F16 ? 8 : 4;
+  for (int vec : {full, 4}) {
+    if (p.R % vec != 0) continue;
+    if (p.mode == kRowGN && p.spatial % vec != 0) continue;
+    return vec;
+  }
+  return 1;
 }
 
 template <typename T, int VEC>
@@ -209,20 +210,22 @@ static int stream_fwd_t(const RowProblem &p, const RowArgs &a, hipStream_t st) {
 }
 
 int launch_row_fwd(const RowProblem &p, hipStream_t st) {
-  const bool vec_ok = row_vec_ok(p, false);
+  const int vec = row_vec(p, false);
   const RowArgs a = make_args(p);
   // LayerNormalization keeps gamma/beta of its columns in registers too: with
   // 8 loads per thread it needs 140-210 VGPRs (8 waves per CU), so it spreads
   // a row over more threads instead.
   const int max_nl = p.mode == kRowLN ? 4 : 8;
-  const RowCfg cfg = pick_row_cfg(p.dtype, p.R, vec_ok, max_nl, max_nl, 64);
+  const RowCfg cfg = pick_row_cfg(vec, p.R, max_nl, max_nl, 64);
   if (cfg.ok && !tune_int("FORCE_STREAM", 0)) {
     return run_row_fwd_cached(p.dtype, cfg, a, cached_grid(p.rows, cfg.tpr), st);
   }
   if (p.dtype == NBLAHIP_F16) {
-    return vec_ok ? stream_fwd_t<__half, 8>(p, a, st) : stream_fwd_t<__half, 1>(p, a, st);
+    return vec == 8   ? stream_fwd_t<__half, 8>(p, a, st)
+           : vec == 4 ? stream_fwd_t<__half, 4>(p, a, st)
+                      : stream_fwd_t<__half, 1>(p, a, st);
   }
-  return vec_ok ? stream_fwd_t<float, 4>(p, a, st) : stream_fwd_t<float, 1>(p, a, st);
+  return vec == 4 ? stream_fwd_t<float, 4>(p, a, st) : stream_fwd_t<float, 1>(p, a, st);
 }
 
 // Row chunks of the streaming LayerNormalization column gradients: enough
@@ -317,16 +320,15 @@ static int launch_pair_reduce(const RowProblem &p, const float *pairs, hipStream
 
 int launch_row_bwd(const RowProblem &p, hipStream_t st) {
   if (!p.out && !p.dgamma && !p.dbeta) return 0;
-  const bool vec_ok = row_vec_ok(p, true);
+  const int vec = row_vec(p, true);
   RowArgs a = make_args(p);
-  const int full = p.dtype == NBLAHIP_F16 ? 8 : 4;
   // LayerNormalization also keeps per-column accumulators, gamma and the
   // normalised row in registers.
   const bool ln = p.mode == kRowLN;
   const int nl_small = ln ? 4 : 8;
   const int nl_1024 = ln ? (p.dtype == NBLAHIP_F16 ? 1 : 2) : 8;
-  RowCfg cfg = ln ? pick_ln_bwd_cfg(p.dtype, p.R, vec_ok)
-                  : pick_row_cfg(p.dtype, p.R, vec_ok, nl_small, nl_1024, 64);
+  RowCfg cfg = ln ? pick_ln_bwd_cfg(p.dtype, p.R, vec)
+                  : pick_row_cfg(vec, p.R, nl_small, nl_1024, 64);
   bool gn_map = false;
   if (p.mode == kRowGN) {
     // Fixed map (every wave-wide load of the plain row layout falls inside one
@@ -335,15 +337,14 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
     // about 15 % for its address arithmetic (64 KB half groups: 24.5 vs 21.3 us).
     auto cost = [](const RowCfg &c) { return static_cast<int64_t>(c.tpr) * c.nl * (4 + c.vec); };
     RowCfg fixed;
-    for (bool v : {true, false}) {
-      if (v && !vec_ok) continue;
-      const RowCfg c = pick_row_cfg(p.dtype, p.R, v, 8, 8, 256);
+    for (int v : {vec, 1}) {
+      const RowCfg c = pick_row_cfg(v, p.R, 8, 8, 256);
       if (c.ok && p.spatial % (64 * static_cast<int64_t>(c.vec)) == 0 &&
           (!fixed.ok || cost(c) < cost(fixed)))
         fixed = c;
     }
     RowArgs am = a;
-    const RowCfg mapped = pick_gn_bwd_cfg(p, vec_ok, am);
+    const RowCfg mapped = pick_gn_bwd_cfg(p, vec, am);
     if (mapped.ok && (!fixed.ok || cost(mapped) * 115 < cost(fixed) * 100)) {
       cfg = mapped;
       a = am;
@@ -357,7 +358,6 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
     // 25 088-element groups, 55 vs 56 us on 32 768-element ones.
     if (cfg.ok && p.dtype == NBLAHIP_F32 && cfg.tpr == 1024 && cfg.nl == 8) cfg.ok = false;
   }
-  (void)full;
   if (cfg.ok && !tune_int("FORCE_STREAM", 0)) {
     if (p.mode == kRowLN) {
       const int resident = row_bwd_ln_resident_blocks(p.dtype, cfg);
@@ -389,9 +389,11 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
   }
   int e;
   if (p.dtype == NBLAHIP_F16) {
-    e = vec_ok ? stream_bwd_t<__half, 8>(p, a, st) : stream_bwd_t<__half, 1>(p, a, st);
+    e = vec == 8   ? stream_bwd_t<__half, 8>(p, a, st)
+        : vec == 4 ? stream_bwd_t<__half, 4>(p, a, st)
+                   : stream_bwd_t<__half, 1>(p, a, st);
   } else {
-    e = vec_ok ? stream_bwd_t<float, 4>(p, a, st) : stream_bwd_t<float, 1>(p, a, st);
+    e = vec == 4 ? stream_bwd_t<float, 4>(p, a, st) : stream_bwd_t<float, 1>(p, a, st);
   }
   if (e) return e;
   if (p.mode == kRowLN) return 0;

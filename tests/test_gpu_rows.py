@@ -22,7 +22,9 @@ def f32(a):
 # (streaming kernels), single row, R == 1.
 LN_SHAPES = [(5, 1), (7, 3), (16, 17), (33, 64), (9, 1000), (64, 1024), (130, 768), (12, 4096),
              (5, 8192), (3, 16384), (6, 32768), (2, 70000), (3, 40004), (1, 2048), (300, 256),
-             (2, 131072)]
+             (2, 131072),
+             # half rows of 4k (not 8k) elements: 8-byte loads
+             (40, 1004), (9, 20), (70, 516), (4, 8196), (3, 2052)]
 
 
 def make_ln(outer, Rr, dtype, seed):
@@ -219,7 +221,8 @@ def test_gn_flags(n, c, sp, groups):
 
 # ------------------------------------------------------------------ IN
 IN_SHAPES = [(2, 3, (4, 4)), (3, 5, (7,)), (1, 2, (3, 2)), (4, 16, (16, 16)), (2, 8, (64, 64)),
-             (2, 4, (7, 7)), (1, 3, (200, 200)), (2, 2, (300, 300)), (3, 7, (1,)), (2, 3, (1000,))]
+             (2, 4, (7, 7)), (1, 3, (200, 200)), (2, 2, (300, 300)), (3, 7, (1,)), (2, 3, (1000,)),
+             (4, 8, (14, 14)), (2, 3, (6, 6)), (2, 300, (14, 14)), (3, 2, (90, 90))]
 
 
 @pytest.mark.parametrize("n,c,sp", IN_SHAPES)
