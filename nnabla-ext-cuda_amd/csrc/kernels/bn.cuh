@@ -1104,36 +1104,4 @@ gn_cl_finalize_bwd_kernel(const float *__restrict__ part2, uint32_t S, uint32_t 
   }
 }
 
-// Batch sum of per-(n, c) pairs (dgamma part, dbeta part) for the channel-last
-// Group/InstanceNormalization backward; element-wise when a parameter is per
-// sample.
-__global__ void __launch_bounds__(256)
-cl_pair_param_reduce_kernel(const float *__restrict__ pairs, int n, int P,
-                            float *__restrict__ dgamma, float *__restrict__ dbeta, int bc_gamma,
-                            int bc_beta, int accum_g, int accum_b) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  const float2 *__restrict__ pp = reinterpret_cast<const float2 *>(pairs);
-  if (i < P) {
-    float sg = 0.f, sb = 0.f;
-    for (int b0 = 0; b0 < n; b0 += 8) {
-      float2 v[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-        v[u] = (b0 + u < n) ? pp[static_cast<size_t>(b0 + u) * P + i] : make_float2(0.f, 0.f);
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        sg += v[u].x;
-        sb += v[u].y;
-      }
-    }
-    if (dgamma && bc_gamma) dgamma[i] = sg + (accum_g ? dgamma[i] : 0.f);
-    if (dbeta && bc_beta) dbeta[i] = sb + (accum_b ? dbeta[i] : 0.f);
-  }
-  if (i < n * P) {
-    const float2 v = pp[i];
-    if (dgamma && !bc_gamma) dgamma[i] = v.x + (accum_g ? dgamma[i] : 0.f);
-    if (dbeta && !bc_beta) dbeta[i] = v.y + (accum_b ? dbeta[i] : 0.f);
-  }
-}
-
 } // namespace nblahip

@@ -2,6 +2,7 @@
 #include <algorithm>
 
 #include "bn.cuh"
+#include "pair_reduce.cuh"
 #include "launch.hpp"
 
 namespace nblahip {
@@ -684,12 +685,10 @@ int launch_cl_bwd(const ClProblem &p, hipStream_t st) {
     if (e2) return e2;
   }
   if (p.dgamma || p.dbeta) {
-    const int64_t count = (p.bc_gamma && p.bc_beta) ? p.channels : p.batch * p.channels;
-    NBLAHIP_LAUNCH("pair_param_reduce_cl_kernel", cl_pair_param_reduce_kernel,
-                   dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, st, w.pairs,
-                   static_cast<int>(p.batch), static_cast<int>(p.channels), p.dgamma, p.dbeta,
-                   p.bc_gamma, p.bc_beta, p.accum_g, p.accum_b);
-    if (int e = last_launch_status()) return e;
+    if (int e = launch_pair_param_reduce("pair_param_reduce_cl_kernel", w.pairs, p.batch, p.channels,
+                                         p.dgamma, p.dbeta, p.bc_gamma, p.bc_beta, p.accum_g,
+                                         p.accum_b, st))
+      return e;
   }
   return 0;
 }

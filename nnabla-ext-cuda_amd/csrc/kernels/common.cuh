@@ -376,15 +376,32 @@ __device__ __forceinline__ float wave_sum(float v) {
   return (read_lane(v, 0) + read_lane(v, 16)) + (read_lane(v, 32) + read_lane(v, 48));
 }
 
-// Sum over a group of TPR threads that share a row.  TPR == 64: one wave.
-// TPR > 64: the block is exactly one row (blockDim.x == TPR); `lds` holds
-// TPR/64 floats and is reused, so the call ends with a barrier-protected read.
+// Sum over aligned groups of G = 4, 8, 16 or 32 adjacent lanes (every lane of
+// a group returns the group's sum): the first steps of wave_sum, and one lane
+// exchange between the two 16-lane rows for G = 32.  Lanes of a group must be
+// active together.
+template <int G> __device__ __forceinline__ float group_sum(float v) {
+  static_assert(G == 4 || G == 8 || G == 16 || G == 32, "sub-wave group size");
+  v += dpp_move<0xB1>(v);
+  v += dpp_move<0x4E>(v);
+  if constexpr (G >= 8) v += dpp_move<0x141>(v);
+  if constexpr (G >= 16) v += dpp_move<0x140>(v);
+  if constexpr (G == 32) v += __shfl_xor(v, 16);
+  return v;
+}
+
+// Sum over a group of TPR threads that share a row.  TPR < 64: several rows
+// per wave.  TPR == 64: one wave.  TPR > 64: the block is exactly one row
+// (blockDim.x == TPR); `lds` holds TPR/64 floats and is reused, so the call
+// ends with a barrier-protected read.
 template <int TPR>
 __device__ __forceinline__ float row_sum(float v, float *lds) {
-  v = wave_sum(v);
-  if constexpr (TPR == kWave) {
-    return v;
+  if constexpr (TPR < kWave) {
+    return group_sum<TPR>(v);
+  } else if constexpr (TPR == kWave) {
+    return wave_sum(v);
   } else {
+    v = wave_sum(v);
     constexpr int NW = TPR / kWave;
     const int wave = threadIdx.x / kWave;
     lds_barrier(); // previous readers of lds are done
@@ -400,8 +417,14 @@ __device__ __forceinline__ float row_sum(float v, float *lds) {
 // Two sums at once (halves the number of barriers).
 template <int TPR>
 __device__ __forceinline__ void row_sum2(float &a, float &b, float *lds) {
-  a = wave_sum(a);
-  b = wave_sum(b);
+  if constexpr (TPR < kWave) {
+    a = group_sum<TPR>(a);
+    b = group_sum<TPR>(b);
+    return;
+  } else {
+    a = wave_sum(a);
+    b = wave_sum(b);
+  }
   if constexpr (TPR > kWave) {
     constexpr int NW = TPR / kWave;
     const int wave = threadIdx.x / kWave;

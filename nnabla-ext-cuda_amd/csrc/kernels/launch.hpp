@@ -64,8 +64,9 @@ struct RowCfg {
 
 // vec: elements per load (alignment and divisibility already checked by the
 // caller).  max_nl / max_nl_1024 bound the loads per thread below / at 1024
-// threads; min_tpr is 256 for the GroupNormalization backward.
-RowCfg pick_row_cfg(int vec, int64_t R, int max_nl, int max_nl_1024, int min_tpr);
+// threads; min_tpr is 256 for the GroupNormalization backward and 4 where
+// several rows may share a wave; percol: LayerNormalization parameter layout.
+RowCfg pick_row_cfg(int vec, int64_t R, int max_nl, int max_nl_1024, int min_tpr, bool percol);
 
 int launch_row_fwd(const RowProblem &p, hipStream_t st);
 int launch_row_bwd(const RowProblem &p, hipStream_t st);

@@ -2,7 +2,8 @@
 // GroupNormalization groups) with the row cached in registers: x (and dy) cross
 // HBM exactly once per direction.
 //
-// Thread layout: TPR threads share a row (64 = one wavefront, no barrier at all;
+// Thread layout: TPR threads share a row (4..32 = several rows per wavefront,
+// for rows of a few hundred bytes; 64 = one wavefront, no barrier at all;
 // 256 / 1024 = one block per row, LDS cross-wave merge).  Thread t issues NL
 // 16-byte loads at element (k*TPR + t)*VEC, k = 0..NL-1, so every load
 // instruction of a wave covers 1 KiB of consecutive memory.
@@ -102,7 +103,7 @@ template <int TPR> struct RowBlock {
 // 512-thread block (256 VGPRs per lane stay available): two blocks per CU,
 // few partials to fold afterwards.
 template <int TPR, int MODE> struct RowBwdBlock {
-  static constexpr int kBlock = (MODE == kRowLN && TPR == kWave)    ? 512
+  static constexpr int kBlock = (MODE == kRowLN && TPR <= kWave)    ? 512
                                 : (MODE == kRowINc && TPR == kWave) ? 1024
                                                                     : RowBlock<TPR>::kBlock;
   static constexpr int kRowsPerBlock = kBlock / TPR;
@@ -271,7 +272,7 @@ row_bwd_kernel(const RowArgs a) {
   constexpr bool GNM = MODE == kRowGNm; // run-time thread map (GnSlot)
   __shared__ float lds[2 * 16];
   __shared__ float part[GN ? 2 * NW * NL : 1];
-  __shared__ float xwave[(MODE == kRowLN && RPB > 1) ? (RPB - 1) * kWave * VEC : 1];
+  __shared__ float xfold[(MODE == kRowLN && RPB > 1) ? (RPB / 2) * TPR * VEC : 1];
   const int t = threadIdx.x % TPR;
   const int sub = threadIdx.x / TPR;
   const T *__restrict__ x = static_cast<const T *>(a.x);
@@ -532,8 +533,8 @@ row_bwd_kernel(const RowArgs a) {
   } // units
 
   if constexpr (MODE == kRowLN) {
-    // Fold the RPB waves of a block into wave 0 (fixed order), then write the
-    // block's partial [2][R].
+    // Fold the RPB row groups of a block into group 0 (a halving tree, fixed
+    // order), then write the block's partial [2][R].
     float *wsb = a.ws + static_cast<size_t>(blockIdx.x) * 2 * a.R;
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
@@ -541,17 +542,18 @@ row_bwd_kernel(const RowArgs a) {
       for (int k = 0; k < NL; ++k) {
         float(&acc)[VEC] = (q == 0) ? acc_g[k] : acc_b[k];
         if constexpr (RPB > 1) {
-          lds_barrier();
-          if (sub > 0) {
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) xwave[((sub - 1) * kWave + t) * VEC + j] = acc[j];
-          }
-          lds_barrier();
-          if (sub == 0) {
+          for (int half = RPB / 2; half >= 1; half /= 2) {
+            lds_barrier(); // the previous level has been read
+            if (sub >= half && sub < 2 * half) {
 #pragma unroll
-            for (int r = 0; r < RPB - 1; ++r)
+              for (int j = 0; j < VEC; ++j) xfold[((sub - half) * TPR + t) * VEC + j] = acc[j];
+            }
+            lds_barrier();
+            if (sub < half) {
 #pragma unroll
-              for (int j = 0; j < VEC; ++j) acc[j] += xwave[(r * kWave + t) * VEC + j];
+              for (int j = 0; j < VEC; ++j) acc[j] += xfold[(sub * TPR + t) * VEC + j];
+            }
           }
         }
         const int col = (k * TPR + t) * VEC;

@@ -13,7 +13,7 @@ namespace nblahip {
 
 template <typename T>
 static int run_bwd_t(const RowCfg &cfg, const RowArgs &args, int grid, hipStream_t st) {
-  NBLAHIP_ROW_CASES(BWD_CASE, T)
+  NBLAHIP_ROW_CASES_WAVE(BWD_CASE, T)
   return NBLAHIP_EINVAL;
 }
 

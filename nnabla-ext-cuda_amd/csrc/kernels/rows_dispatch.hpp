@@ -30,7 +30,21 @@ int run_row_bwd_cached_gnm(int dtype, const RowCfg &cfg, const RowArgs &args, in
 #define NBLAHIP_ROW_CASES_TPR(CASE, T, VEC, TPR) \
   CASE(T, VEC, 1, TPR) CASE(T, VEC, 2, TPR) CASE(T, VEC, 4, TPR) CASE(T, VEC, 8, TPR)
 
+// Rows of a few hundred bytes: several rows per wave, at most 4 loads each.
+#define NBLAHIP_ROW_CASES_SUBWAVE(CASE, T, VEC)                                   \
+  CASE(T, VEC, 1, 4) CASE(T, VEC, 2, 4) CASE(T, VEC, 4, 4)                        \
+  CASE(T, VEC, 1, 8) CASE(T, VEC, 2, 8) CASE(T, VEC, 4, 8)                        \
+  CASE(T, VEC, 1, 16) CASE(T, VEC, 2, 16) CASE(T, VEC, 4, 16)                     \
+  CASE(T, VEC, 1, 32) CASE(T, VEC, 2, 32) CASE(T, VEC, 4, 32)
+
 #define NBLAHIP_ROW_CASES(CASE, T)                          \
+  NBLAHIP_ROW_CASES_SUBWAVE(CASE, T, FullVec<T>::value)     \
+  NBLAHIP_ROW_CASES_SUBWAVE(CASE, T, MidVec<T>::value)      \
+  NBLAHIP_ROW_CASES_SUBWAVE(CASE, T, 1)                     \
+  NBLAHIP_ROW_CASES_WAVE(CASE, T)
+
+// One wave or more per row.
+#define NBLAHIP_ROW_CASES_WAVE(CASE, T)                     \
   NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 64)     \
   NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 256)    \
   NBLAHIP_ROW_CASES_TPR(CASE, T, FullVec<T>::value, 512)    \

@@ -4,6 +4,7 @@
 #include <algorithm>
 
 #include "rows_dispatch.hpp"
+#include "pair_reduce.cuh"
 #include "rows_stream.cuh"
 
 namespace nblahip {
@@ -11,10 +12,37 @@ namespace nblahip {
 // max_nl bounds the loads per thread of the layouts below 1024 threads,
 // max_nl_1024 those of the 1024-thread layout, whose register budget is 128
 // VGPRs; both are chosen per kernel family so that no variant in use spills.
-RowCfg pick_row_cfg(int vec, int64_t R, int max_nl, int max_nl_1024, int min_tpr) {
+// Rows of fewer than 64 vectors: several rows per wave, 4 to 32 lanes each.
+// Measured on 64 MB tensors (LayerNormalization of 32- to 256-element half
+// rows: 219 / 106 / 56 / 31 us with a wave per row, 23 / 22 / 22 / 21 us here):
+// layouts that pad the row to the next power of two and no further are
+// equivalent within 5 %, two loads per lane being the best or next to it in
+// both directions; rows of 33 to 63 vectors (7x7 planes) want four loads per
+// lane in the forward pass (12.5 vs 18.3 us), which the LayerNormalization
+// backward cannot afford in registers.
+static bool pick_subwave(RowCfg &c, int64_t nv, bool percol) {
+  const int ftpr = tune_int("ROW_TPR", 0), fnl = tune_int("ROW_NL", 0);
+  auto take = [&](int tpr, int nl) {
+    c.ok = true;
+    c.tpr = tpr;
+    c.nl = nl;
+    return true;
+  };
+  if (ftpr > 0 && ftpr < 64 && fnl > 0 && static_cast<int64_t>(ftpr) * fnl >= nv)
+    return take(ftpr, fnl);
+  if (nv >= 64 || !tune_int("ROW_SUBWAVE", 1)) return false;
+  if (nv <= 4) return take(4, 1);
+  int pad = 8;
+  while (pad < nv) pad <<= 1;
+  if (pad < 64) return take(pad / 2, 2);
+  return percol ? take(32, 2) : take(16, 4);
+}
+
+RowCfg pick_row_cfg(int vec, int64_t R, int max_nl, int max_nl_1024, int min_tpr, bool percol) {
   RowCfg c;
   c.vec = vec;
   const int64_t nv = R / c.vec;
+  if (min_tpr < 64 && pick_subwave(c, nv, percol)) return c;
   static const int tprs[4] = {64, 256, 512, 1024};
   static const int nls[4] = {1, 2, 4, 8};
   for (int tpr : tprs) {
@@ -48,6 +76,7 @@ static RowCfg pick_ln_bwd_cfg(int dtype, int64_t R, int vec) {
     c.nl = nl;
     return c;
   };
+  if (pick_subwave(c, nv, true)) return c;
   for (int nl : {1, 2, 4})
     if (64 * nl >= nv) return take(64, nl);
   for (int nl : {1, 2, 4})
@@ -120,7 +149,7 @@ static int ln_bwd_grid(int64_t rows, int tpr, int resident = 2) {
   // resident: blocks of the chosen kernel that fit a CU together; the grid
   // never exceeds what is resident (one round) nor two blocks per CU (the
   // workspace holds one partial per block).
-  const int rpb = tpr == 64 ? 8 : 1;
+  const int rpb = tpr <= 64 ? 512 / tpr : 1;
   const int per_cu = tune_int("LN_BWD_BLOCKS_PER_CU", std::max(1, std::min(2, resident)));
   const int64_t cap = static_cast<int64_t>(device_cus()) * per_cu;
   const int64_t blocks = (rows + rpb - 1) / rpb;
@@ -216,7 +245,7 @@ int launch_row_fwd(const RowProblem &p, hipStream_t st) {
   // 8 loads per thread it needs 140-210 VGPRs (8 waves per CU), so it spreads
   // a row over more threads instead.
   const int max_nl = p.mode == kRowLN ? 4 : 8;
-  const RowCfg cfg = pick_row_cfg(vec, p.R, max_nl, max_nl, 64);
+  const RowCfg cfg = pick_row_cfg(vec, p.R, max_nl, max_nl, 4, p.mode == kRowLN);
   if (cfg.ok && !tune_int("FORCE_STREAM", 0)) {
     return run_row_fwd_cached(p.dtype, cfg, a, cached_grid(p.rows, cfg.tpr), st);
   }
@@ -310,12 +339,8 @@ static int launch_pair_reduce(const RowProblem &p, const float *pairs, hipStream
   if (!p.dgamma && !p.dbeta) return 0;
   const int bcg = p.mode == kRowGN ? 1 : p.bc_gamma;
   const int bcb = p.mode == kRowGN ? 1 : p.bc_beta;
-  const int64_t count = (bcg && bcb) ? p.channels : p.batch * p.channels;
-  NBLAHIP_LAUNCH("pair_param_reduce_kernel", pair_param_reduce_kernel, dim3(static_cast<unsigned>((count + 255) / 256)),
-                     dim3(256), 0, st, pairs, static_cast<int>(p.batch),
-                     static_cast<int>(p.channels), p.dgamma, p.dbeta, bcg, bcb, p.accum_g,
-                     p.accum_b);
-  return last_launch_status();
+  return launch_pair_param_reduce("pair_param_reduce_kernel", pairs, p.batch, p.channels, p.dgamma,
+                                  p.dbeta, bcg, bcb, p.accum_g, p.accum_b, st);
 }
 
 int launch_row_bwd(const RowProblem &p, hipStream_t st) {
@@ -328,7 +353,7 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
   const int nl_small = ln ? 4 : 8;
   const int nl_1024 = ln ? (p.dtype == NBLAHIP_F16 ? 1 : 2) : 8;
   RowCfg cfg = ln ? pick_ln_bwd_cfg(p.dtype, p.R, vec)
-                  : pick_row_cfg(vec, p.R, nl_small, nl_1024, 64);
+                  : pick_row_cfg(vec, p.R, nl_small, nl_1024, p.mode == kRowGN ? 256 : 4, false);
   bool gn_map = false;
   if (p.mode == kRowGN) {
     // Fixed map (every wave-wide load of the plain row layout falls inside one
@@ -338,7 +363,7 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
     auto cost = [](const RowCfg &c) { return static_cast<int64_t>(c.tpr) * c.nl * (4 + c.vec); };
     RowCfg fixed;
     for (int v : {vec, 1}) {
-      const RowCfg c = pick_row_cfg(v, p.R, 8, 8, 256);
+      const RowCfg c = pick_row_cfg(v, p.R, 8, 8, 256, false);
       if (c.ok && p.spatial % (64 * static_cast<int64_t>(c.vec)) == 0 &&
           (!fixed.ok || cost(c) < cost(fixed)))
         fixed = c;
@@ -375,7 +400,7 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
     // channels to fill the chip: a block per channel sums over the batch
     // itself, no second kernel.
     if (p.mode == kRowIN && p.bc_gamma && p.bc_beta && p.batch > 1 &&
-        p.channels * 2 >= device_cus() && !(cfg.tpr == 1024 && cfg.nl == 8) &&
+        p.channels * 2 >= device_cus() && !(cfg.tpr == 1024 && cfg.nl == 8) && cfg.tpr >= 64 &&
         !tune_int("IN_NO_CHANNEL_BLOCKS", 0)) {
       const int grid = static_cast<int>(std::min<int64_t>(p.channels, 1 << 20));
       return run_row_bwd_cached_inc(p.dtype, cfg, a, grid, st);

@@ -24,7 +24,9 @@ LN_SHAPES = [(5, 1), (7, 3), (16, 17), (33, 64), (9, 1000), (64, 1024), (130, 76
              (5, 8192), (3, 16384), (6, 32768), (2, 70000), (3, 40004), (1, 2048), (300, 256),
              (2, 131072),
              # half rows of 4k (not 8k) elements: 8-byte loads
-             (40, 1004), (9, 20), (70, 516), (4, 8196), (3, 2052)]
+             (40, 1004), (9, 20), (70, 516), (4, 8196), (3, 2052),
+             # several rows per wave (4 to 32 lanes each), ragged row counts
+             (1000, 32), (513, 128), (100, 48), (77, 200), (2049, 64), (31, 8), (129, 24), (65, 392)]
 
 
 def make_ln(outer, Rr, dtype, seed):
@@ -222,7 +224,8 @@ def test_gn_flags(n, c, sp, groups):
 # ------------------------------------------------------------------ IN
 IN_SHAPES = [(2, 3, (4, 4)), (3, 5, (7,)), (1, 2, (3, 2)), (4, 16, (16, 16)), (2, 8, (64, 64)),
              (2, 4, (7, 7)), (1, 3, (200, 200)), (2, 2, (300, 300)), (3, 7, (1,)), (2, 3, (1000,)),
-             (4, 8, (14, 14)), (2, 3, (6, 6)), (2, 300, (14, 14)), (3, 2, (90, 90))]
+             (4, 8, (14, 14)), (2, 3, (6, 6)), (2, 300, (14, 14)), (3, 2, (90, 90)),
+             (8, 64, (8, 8)), (5, 33, (7, 7)), (3, 300, (4, 4)), (2, 129, (3, 5)), (7, 11, (6,))]
 
 
 @pytest.mark.parametrize("n,c,sp", IN_SHAPES)
