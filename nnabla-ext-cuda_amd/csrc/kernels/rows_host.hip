@@ -226,12 +226,35 @@ static int row_vec(const RowProblem &p, bool backward) {
   return 1;
 }
 
+// Splits per row (or plane) of the streaming reductions: 1 when the units
+// alone give every CU two blocks, else enough runs for four blocks per CU, each
+// at least four unrolled steps long, at most 64.
+static int stream_splits(int64_t units, int64_t nv) {
+  const int64_t cus = device_cus();
+  if (units >= 2 * cus) return 1;
+  const int64_t want = (4 * cus + units - 1) / units;
+  const int64_t most = std::max<int64_t>(1, nv / (kStreamBlock * 16));
+  return static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(std::min(want, most), 64)));
+}
+
 template <typename T, int VEC>
 static int stream_fwd_t(const RowProblem &p, const RowArgs &a, hipStream_t st) {
-  NBLAHIP_LAUNCH("row_stats_stream_kernel", (row_stats_stream_kernel<T, VEC>), dim3(stream_grid(p.rows)),
-                     dim3(kStreamBlock), 0, st, static_cast<const T *>(p.x), a.rows, a.R,
-                     a.inv_R, p.mean, p.var);
+  // A few very long rows: split them.  The partial states live in the first
+  // bytes of y, which the apply step below overwrites (not when y is x).
+  int S = (p.out != p.x && aligned16(p.out)) ? stream_splits(p.rows, p.R / VEC) : 1;
+  float *part = static_cast<float *>(p.out);
+  if (static_cast<size_t>(p.rows) * S * 3 * sizeof(float) >
+      static_cast<size_t>(p.rows) * p.R * sizeof(T))
+    S = 1;
+  NBLAHIP_LAUNCH("row_stats_stream_kernel", (row_stats_stream_kernel<T, VEC>),
+                 dim3(stream_grid(p.rows), S), dim3(kStreamBlock), 0, st,
+                 static_cast<const T *>(p.x), a.rows, a.R, a.inv_R, p.mean, p.var, part);
   if (int e = last_launch_status()) return e;
+  if (S > 1) {
+    NBLAHIP_LAUNCH("row_stats_merge_kernel", row_stats_merge_kernel, dim3((a.rows + 63) / 64),
+                   dim3(64), 0, st, part, a.rows, S, a.inv_R, p.mean, p.var);
+    if (int e = last_launch_status()) return e;
+  }
   const uint32_t total_vec = static_cast<uint32_t>(p.rows * p.R / VEC);
   NBLAHIP_LAUNCH("row_apply_fwd_kernel", (row_apply_fwd_kernel<T, VEC>), dim3(stream_grid((total_vec + 255) / 256)),
                      dim3(256), 0, st, a, FastDiv(static_cast<uint32_t>(p.R / VEC)), total_vec);
@@ -273,13 +296,24 @@ size_t row_bwd_workspace_bytes(int mode, int64_t rows, int64_t R, int64_t planes
     const int g = std::max(std::max(ln_bwd_grid(rows, 64), ln_bwd_grid(rows, 256)),
                            std::max(ln_bwd_grid(rows, 512), ln_bwd_grid(rows, 1024)));
     const size_t cached = static_cast<size_t>(g) * 2 * static_cast<size_t>(R) * sizeof(float);
+    // row sums, column partials over row chunks, partial sums of split rows
+    const size_t split = rows < 2 * static_cast<int64_t>(device_cus())
+                             ? static_cast<size_t>(rows) * 64 * 2 * sizeof(float)
+                             : 0;
     const size_t stream = align_up(static_cast<size_t>(rows) * 2 * sizeof(float), 256) +
-                          static_cast<size_t>(ln_stream_chunks(rows, R)) * 2 *
-                              static_cast<size_t>(R) * sizeof(float);
+                          align_up(static_cast<size_t>(ln_stream_chunks(rows, R)) * 2 *
+                                       static_cast<size_t>(R) * sizeof(float),
+                                   256) +
+                          split;
     return align_up(std::max(cached, stream), 256);
   }
+  // plane pairs, row factors, and the partial pairs of split planes (at most
+  // 64 runs each, only taken for fewer than 2 planes per CU)
+  const size_t split = planes < 2 * static_cast<int64_t>(device_cus())
+                           ? static_cast<size_t>(planes) * 64 * 2 * sizeof(float)
+                           : 0;
   return align_up(static_cast<size_t>(planes) * 2 * sizeof(float), 256) +
-         align_up(static_cast<size_t>(rows) * 2 * sizeof(float), 256);
+         align_up(static_cast<size_t>(rows) * 2 * sizeof(float), 256) + align_up(split, 256);
 }
 
 template <typename T, int VEC>
@@ -291,9 +325,22 @@ static int stream_bwd_t(const RowProblem &p, const RowArgs &a, hipStream_t st) {
   if (p.mode == kRowLN) {
     float *rs = static_cast<float *>(p.ws);
     if (p.out) {
-      NBLAHIP_LAUNCH("ln_row_sums_stream_kernel", (ln_row_sums_stream_kernel<T, VEC>), dim3(stream_grid(p.rows)),
-                         dim3(kStreamBlock), 0, st, x, dy, p.gamma, p.mean, a.rows, a.R, rs);
+      const int S = stream_splits(p.rows, p.R / VEC);
+      float *split = reinterpret_cast<float *>(
+          static_cast<char *>(p.ws) + align_up(static_cast<size_t>(p.rows) * 2 * sizeof(float), 256) +
+          align_up(static_cast<size_t>(ln_stream_chunks(p.rows, p.R)) * 2 *
+                       static_cast<size_t>(p.R) * sizeof(float),
+                   256));
+      NBLAHIP_LAUNCH("ln_row_sums_stream_kernel", (ln_row_sums_stream_kernel<T, VEC>),
+                     dim3(stream_grid(p.rows), S), dim3(kStreamBlock), 0, st, x, dy, p.gamma,
+                     p.mean, a.rows, a.R, S > 1 ? split : rs);
       if (int e = last_launch_status()) return e;
+      if (S > 1) {
+        NBLAHIP_LAUNCH("pair_split_merge_kernel", pair_split_merge_kernel,
+                       dim3(static_cast<unsigned>((p.rows + 63) / 64)), dim3(64), 0, st, split,
+                       a.rows, S, rs);
+        if (int e = last_launch_status()) return e;
+      }
       NBLAHIP_LAUNCH("row_bwd_dx_kernel", (row_bwd_dx_kernel<T, VEC>), dim3(stream_grid((total_vec + 255) / 256)),
                          dim3(256), 0, st, a, rs, nvr, total_vec);
       if (int e = last_launch_status()) return e;
@@ -319,10 +366,20 @@ static int stream_bwd_t(const RowProblem &p, const RowArgs &a, hipStream_t st) {
   float *pairs = static_cast<float *>(p.ws);
   float *rs = reinterpret_cast<float *>(static_cast<char *>(p.ws) +
                                         align_up(static_cast<size_t>(planes) * 2 * sizeof(float), 256));
-  NBLAHIP_LAUNCH("plane_sums_stream_kernel", (plane_sums_stream_kernel<T, VEC>), dim3(stream_grid(planes)),
-                     dim3(kStreamBlock), 0, st, x, dy, p.mean, static_cast<int>(planes),
-                     static_cast<int>(p.spatial), static_cast<uint32_t>(ppr), pairs);
+  const int S = stream_splits(planes, p.spatial / VEC);
+  float *part = reinterpret_cast<float *>(
+      reinterpret_cast<char *>(rs) + align_up(static_cast<size_t>(p.rows) * 2 * sizeof(float), 256));
+  NBLAHIP_LAUNCH("plane_sums_stream_kernel", (plane_sums_stream_kernel<T, VEC>),
+                 dim3(stream_grid(planes), S), dim3(kStreamBlock), 0, st, x, dy, p.mean,
+                 static_cast<int>(planes), static_cast<int>(p.spatial), static_cast<uint32_t>(ppr),
+                 S > 1 ? part : pairs);
   if (int e = last_launch_status()) return e;
+  if (S > 1) {
+    NBLAHIP_LAUNCH("pair_split_merge_kernel", pair_split_merge_kernel,
+                   dim3(static_cast<unsigned>((planes + 63) / 64)), dim3(64), 0, st, part,
+                   static_cast<int>(planes), S, pairs);
+    if (int e = last_launch_status()) return e;
+  }
   const uint32_t gmod = (p.mode == kRowGN || p.bc_gamma) ? static_cast<uint32_t>(p.channels) : 0u;
   NBLAHIP_LAUNCH("plane_to_row_factors_kernel", plane_to_row_factors_kernel, dim3(stream_grid(p.rows)), dim3(64), 0, st,
                      pairs, p.gamma, p.var, a.rows, ppr, gmod, p.eps, rs);

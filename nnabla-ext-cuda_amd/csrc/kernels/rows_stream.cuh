@@ -13,18 +13,27 @@ namespace nblahip {
 
 constexpr int kStreamBlock = 256;
 
-// mean/var of each row; one block per row (grid-stride).
+// mean/var of each row; one block per row (grid-stride over blockIdx.x).
+// gridDim.y = S > 1 splits every row into S runs of vectors, for tensors of a
+// few very long rows (3-D InstanceNormalization, GroupNormalization with one
+// group): block (., s) then leaves its Welford state in part[row][s][3] and
+// row_stats_merge_kernel finishes.
 template <typename T, int VEC>
 __global__ void __launch_bounds__(kStreamBlock)
 row_stats_stream_kernel(const T *__restrict__ x, int rows, int R, float inv_R,
-                        float *__restrict__ mean, float *__restrict__ var) {
+                        float *__restrict__ mean, float *__restrict__ var,
+                        float *__restrict__ part) {
   __shared__ float lds[3 * (kStreamBlock / kWave)];
   constexpr int U = 4;
-  const int nv = R / VEC;
+  const int nv_row = R / VEC;
+  const int S = gridDim.y;
+  const int chunk = (nv_row + S - 1) / S;
+  const int vbegin = static_cast<int>(blockIdx.y) * chunk;
+  const int nv = min(nv_row, vbegin + chunk);
   for (int row = blockIdx.x; row < rows; row += gridDim.x) {
     const T *xr = x + static_cast<size_t>(row) * R;
     Welford w{0.f, 0.f, 0.f};
-    for (int v0 = threadIdx.x; v0 < nv; v0 += kStreamBlock * U) {
+    for (int v0 = vbegin + threadIdx.x; v0 < nv; v0 += kStreamBlock * U) {
       float vals[U * VEC];
       int cnt = 0;
 #pragma unroll
@@ -45,11 +54,33 @@ row_stats_stream_kernel(const T *__restrict__ x, int rows, int R, float inv_R,
     }
     w = block_welford(w, lds);
     if (threadIdx.x == 0) {
-      mean[row] = w.mean;
-      var[row] = w.m2 * inv_R;
+      if (S == 1) {
+        mean[row] = w.mean;
+        var[row] = w.m2 * inv_R;
+      } else {
+        float *o = part + 3 * (static_cast<size_t>(row) * S + blockIdx.y);
+        o[0] = w.mean;
+        o[1] = w.m2;
+        o[2] = w.n;
+      }
     }
     lds_barrier();
   }
+}
+
+// Chan merge of the S partial states of each row, in split order.
+__global__ void __launch_bounds__(64)
+row_stats_merge_kernel(const float *__restrict__ part, int rows, int S, float inv_R,
+                       float *__restrict__ mean, float *__restrict__ var) {
+  const int row = blockIdx.x * 64 + threadIdx.x;
+  if (row >= rows) return;
+  Welford w{0.f, 0.f, 0.f};
+  for (int s = 0; s < S; ++s) {
+    const float *q = part + 3 * (static_cast<size_t>(row) * S + s);
+    w = welford_merge(w, Welford{q[0], q[1], q[2]});
+  }
+  mean[row] = w.mean;
+  var[row] = w.m2 * inv_R;
 }
 
 // y = (x-mean[row])*gamma[p]*istd[row] + beta[p] over the whole tensor.
@@ -94,12 +125,18 @@ ln_row_sums_stream_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                           const float *__restrict__ mean, int rows, int R,
                           float *__restrict__ rs) {
   __shared__ float lds[2 * (kStreamBlock / kWave)];
-  const int nv = R / VEC;
+  // gridDim.y = S > 1: every row in S runs of vectors, partial pairs to
+  // rs[(row*S + s)*2] (a partial buffer then), summed by pair_split_merge_kernel.
+  const int nv_row = R / VEC;
+  const int S = gridDim.y;
+  const int chunk = (nv_row + S - 1) / S;
+  const int vbegin = static_cast<int>(blockIdx.y) * chunk;
+  const int nv = min(nv_row, vbegin + chunk);
   for (int row = blockIdx.x; row < rows; row += gridDim.x) {
     const size_t base = static_cast<size_t>(row) * R;
     const float m = mean[row];
     float s1 = 0.f, t2 = 0.f;
-    for (int v = threadIdx.x; v < nv; v += kStreamBlock) {
+    for (int v = vbegin + threadIdx.x; v < nv; v += kStreamBlock) {
       float xv[VEC], dv[VEC];
       load_vec<T, VEC>(x + base + static_cast<size_t>(v) * VEC, xv);
       load_vec<T, VEC>(dy + base + static_cast<size_t>(v) * VEC, dv);
@@ -112,8 +149,9 @@ ln_row_sums_stream_kernel(const T *__restrict__ x, const T *__restrict__ dy,
     }
     block_sum2(s1, t2, lds);
     if (threadIdx.x == 0) {
-      rs[2 * static_cast<size_t>(row)] = s1;
-      rs[2 * static_cast<size_t>(row) + 1] = t2;
+      const size_t o = 2 * (static_cast<size_t>(row) * S + blockIdx.y);
+      rs[o] = s1;
+      rs[o + 1] = t2;
     }
     lds_barrier();
   }
@@ -127,12 +165,19 @@ plane_sums_stream_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                          const float *__restrict__ mean, int planes, int L,
                          uint32_t sdiv, float *__restrict__ pairs) {
   __shared__ float lds[2 * (kStreamBlock / kWave)];
-  const int nv = L / VEC;
+  // gridDim.y = S > 1: every plane in S runs of vectors, partial pairs to
+  // pairs[(p*S + s)*2] (the caller passes a partial buffer then) and
+  // pair_split_merge_kernel adds them up.
+  const int nv_plane = L / VEC;
+  const int S = gridDim.y;
+  const int chunk = (nv_plane + S - 1) / S;
+  const int vbegin = static_cast<int>(blockIdx.y) * chunk;
+  const int nv = min(nv_plane, vbegin + chunk);
   for (int p = blockIdx.x; p < planes; p += gridDim.x) {
     const size_t base = static_cast<size_t>(p) * L;
     const float m = mean[static_cast<uint32_t>(p) / sdiv];
     float sdx = 0.f, sdy = 0.f;
-    for (int v = threadIdx.x; v < nv; v += kStreamBlock) {
+    for (int v = vbegin + threadIdx.x; v < nv; v += kStreamBlock) {
       float xv[VEC], dv[VEC];
       load_vec<T, VEC>(x + base + static_cast<size_t>(v) * VEC, xv);
       load_vec<T, VEC>(dy + base + static_cast<size_t>(v) * VEC, dv);
@@ -144,11 +189,27 @@ plane_sums_stream_kernel(const T *__restrict__ x, const T *__restrict__ dy,
     }
     block_sum2(sdx, sdy, lds);
     if (threadIdx.x == 0) {
-      pairs[2 * static_cast<size_t>(p)] = sdx;
-      pairs[2 * static_cast<size_t>(p) + 1] = sdy;
+      const size_t o = 2 * (static_cast<size_t>(p) * S + blockIdx.y);
+      pairs[o] = sdx;
+      pairs[o + 1] = sdy;
     }
     lds_barrier();
   }
+}
+
+// Sum of the S partial pairs of each plane, in split order.
+__global__ void __launch_bounds__(64)
+pair_split_merge_kernel(const float *__restrict__ part, int planes, int S,
+                        float *__restrict__ pairs) {
+  const int p = blockIdx.x * 64 + threadIdx.x;
+  if (p >= planes) return;
+  float a = 0.f, b = 0.f;
+  for (int s = 0; s < S; ++s) {
+    a += part[2 * (static_cast<size_t>(p) * S + s)];
+    b += part[2 * (static_cast<size_t>(p) * S + s) + 1];
+  }
+  pairs[2 * static_cast<size_t>(p)] = a;
+  pairs[2 * static_cast<size_t>(p) + 1] = b;
 }
 
 // From per-plane sums to per-statistics-row (s1, t2), weighting each plane with

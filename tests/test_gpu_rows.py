@@ -163,7 +163,9 @@ GN_SHAPES = [(2, 8, (8, 8), 4), (3, 6, (5,), 2), (1, 4, (2, 2), 1), (2, 6, (4,),
              # channel, wave sets that do not divide the block, planes that end inside a load
              (2, 64, (56, 56), 8), (2, 64, (28, 28), 4), (2, 6, (8, 8), 2), (2, 4, (64, 64), 4),
              (1, 10, (48, 48), 2), (2, 64, (14, 14), 2), (2, 128, (7, 7), 2), (1, 80, (8, 8), 2),
-             (3, 24, (24, 24), 3), (2, 14, (72,), 2)]
+             (3, 24, (24, 24), 3), (2, 14, (72,), 2),
+             # one group of 2M elements per sample: split streaming reductions
+             (2, 32, (256, 256), 1), (1, 6, (333, 333), 2)]
 
 
 def make_nc(n, c, sp, dtype, seed):
@@ -225,7 +227,9 @@ def test_gn_flags(n, c, sp, groups):
 IN_SHAPES = [(2, 3, (4, 4)), (3, 5, (7,)), (1, 2, (3, 2)), (4, 16, (16, 16)), (2, 8, (64, 64)),
              (2, 4, (7, 7)), (1, 3, (200, 200)), (2, 2, (300, 300)), (3, 7, (1,)), (2, 3, (1000,)),
              (4, 8, (14, 14)), (2, 3, (6, 6)), (2, 300, (14, 14)), (3, 2, (90, 90)),
-             (8, 64, (8, 8)), (5, 33, (7, 7)), (3, 300, (4, 4)), (2, 129, (3, 5)), (7, 11, (6,))]
+             (8, 64, (8, 8)), (5, 33, (7, 7)), (3, 300, (4, 4)), (2, 129, (3, 5)), (7, 11, (6,)),
+             # a few very long rows: split streaming reductions
+             (2, 4, (64, 64, 64)), (1, 2, (999, 1001))]
 
 
 @pytest.mark.parametrize("n,c,sp", IN_SHAPES)
