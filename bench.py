@@ -288,6 +288,86 @@ def config_table(K, steps, warmup):
     return out
 
 
+def torch_native_table(K, steps, warmup):
+    """This library beside the framework's own kernels on the same GPU:
+    torch.ops.aten.native_{batch,layer,group}_norm and their backward ops on the
+    same shapes (wall clock per call, microseconds)."""
+    import torch
+    A = torch.ops.aten
+
+    def bn(shape, dt, cl):
+        n, c, h, w = shape
+        x = torch.randn(shape, device="cuda", dtype=dt)
+        dy = torch.randn_like(x)
+        if cl:
+            x = x.contiguous(memory_format=torch.channels_last)
+            dy = dy.contiguous(memory_format=torch.channels_last)
+        g, b = torch.rand(c, device="cuda") + 0.5, torch.randn(c, device="cuda")
+        rm, rv = torch.zeros(c, device="cuda"), torch.ones(c, device="cuda")
+        fwd_t = lambda: A.native_batch_norm(x, g, b, rm, rv, True, 0.1, 1e-5)
+        _, sm, si = fwd_t()
+        bwd_t = lambda: A.native_batch_norm_backward(dy, x, g, rm, rv, sm, si, True, 1e-5,
+                                                     [True, True, True])
+        ours = make_bn(K, (n, h, w, c) if cl else shape, 3 if cl else 1, dt, True, seed=1)
+        return fwd_t, bwd_t, ours
+
+    def ln(shape, dt):
+        rows, r = shape
+        x = torch.randn(shape, device="cuda", dtype=dt)
+        dy = torch.randn_like(x)
+        g, b = (torch.rand(r, device="cuda") + 0.5).to(dt), torch.randn(r, device="cuda").to(dt)
+        fwd_t = lambda: A.native_layer_norm(x, [r], g, b, 1e-5)
+        _, m, rs = fwd_t()
+        bwd_t = lambda: A.native_layer_norm_backward(dy, x, [r], m, rs, g, b, [True, True, True])
+        return fwd_t, bwd_t, make_rows(K, "ln", shape, dt, 3)
+
+    def gn(shape, groups, dt):
+        n, c, h, w = shape
+        x = torch.randn(shape, device="cuda", dtype=dt)
+        dy = torch.randn_like(x)
+        g, b = (torch.rand(c, device="cuda") + 0.5).to(dt), torch.randn(c, device="cuda").to(dt)
+        fwd_t = lambda: A.native_group_norm(x, g, b, n, c, h * w, groups, 1e-5)
+        _, m, rs = fwd_t()
+        bwd_t = lambda: A.native_group_norm_backward(dy, x, m, rs, g, n, c, h * w, groups,
+                                                     [True, True, True])
+        ours = (make_rows(K, "in", shape, dt, 3) if groups == c
+                else make_rows(K, "gn", shape, dt, 3, groups=groups))
+        return fwd_t, bwd_t, ours
+
+    f32, f16 = torch.float32, torch.float16
+    specs = []
+    for dt in (f32, f16):
+        n = str(dt)[6:]
+        specs += [
+            (f"BN {n} NCHW [32,256,56,56]", lambda dt=dt: bn((32, 256, 56, 56), dt, False)),
+            (f"BN {n} NHWC [256,56,56,64]", lambda dt=dt: bn((256, 64, 56, 56), dt, True)),
+            (f"BN {n} NCHW [256,1024,14,14]", lambda dt=dt: bn((256, 1024, 14, 14), dt, False)),
+            (f"BN {n} NCHW [256,2048,7,7]", lambda dt=dt: bn((256, 2048, 7, 7), dt, False)),
+            (f"LN {n} [16384,1024]", lambda dt=dt: ln((16384, 1024), dt)),
+            (f"LN {n} [8192,4096]", lambda dt=dt: ln((8192, 4096), dt)),
+            (f"LN {n} [262144,128]", lambda dt=dt: ln((262144, 128), dt)),
+            (f"GN {n} [16,256,64,64] G=32", lambda dt=dt: gn((16, 256, 64, 64), 32, dt)),
+            (f"GN {n} [32,512,28,28] G=32", lambda dt=dt: gn((32, 512, 28, 28), 32, dt)),
+            (f"GN {n} [32,1024,14,14] G=32", lambda dt=dt: gn((32, 1024, 14, 14), 32, dt)),
+            (f"IN {n} [16,256,64,64]", lambda dt=dt: gn((16, 256, 64, 64), 256, dt)),
+        ]
+    out = []
+    for name, make in specs:
+        fwd_t, bwd_t, (fwd, bwd, _, _, keep) = make()
+        row = {"config": name}
+        for key, ours, theirs in (("fwd", fwd, fwd_t), ("bwd", bwd, bwd_t)):
+            a = time_calls([ours], steps, warmup) * 1e3
+            b = time_calls([theirs], steps, warmup) * 1e3
+            row[key + "_us"] = round(a, 1)
+            row["torch_" + key + "_us"] = round(b, 1)
+            row[key + "_speedup"] = round(b / a, 2)
+        log("  ", json.dumps(row))
+        out.append(row)
+        del keep, fwd, bwd, fwd_t, bwd_t
+        torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline(budget_s=12.0):
     """The C restatement (OpenMP over channels) on the full C2 workload."""
     import numpy as np
@@ -335,6 +415,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-table", action="store_true", help="skip the per-config table")
+    ap.add_argument("--torch-native", action="store_true",
+                    help="also time torch's own normalization kernels on the same shapes")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a float32->float16 convert of the workload's x (a plain "
                          "streaming kernel of known traffic: 4 B read, 2 B written per element) "
@@ -414,6 +496,8 @@ def main():
     torch.cuda.empty_cache()
     if not args.no_table:
         result["configs"] = config_table(K, max(20, args.steps // 2), args.warmup)
+    if args.torch_native:
+        result["torch_native"] = torch_native_table(K, max(20, args.steps // 2), args.warmup)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
     else:
