@@ -626,6 +626,10 @@ size_t cl_workspace_bytes(int64_t batch, int64_t spatial, int64_t channels, int 
 
 int launch_cl_fwd(const ClProblem &p, hipStream_t st) {
   const bool al = aligned16(p.x) && aligned16(p.out);
+  {
+    int status = 0;
+    if (gn_cl_cached_fwd(p, al, st, &status)) return status;
+  }
   const BnPlan pl = make_cl_plan(p.batch, p.spatial, p.channels, p.dtype, al);
   const ClWs w = cl_carve(p, pl);
   const uint32_t cpg = static_cast<uint32_t>(p.channels / p.groups);
@@ -657,6 +661,17 @@ int launch_cl_bwd(const ClProblem &p, hipStream_t st) {
   const bool al = aligned16(p.x) && aligned16(p.dy) && (!p.out || aligned16(p.out));
   const BnPlan pl = make_cl_plan(p.batch, p.spatial, p.channels, p.dtype, al);
   const ClWs w = cl_carve(p, pl);
+  {
+    int status = 0;
+    if (gn_cl_cached_bwd(p, al, w.pairs, st, &status)) {
+      if (status) return status;
+      if (p.dgamma || p.dbeta)
+        return launch_pair_param_reduce("pair_param_reduce_cl_kernel", w.pairs, p.batch, p.channels,
+                                        p.dgamma, p.dbeta, p.bc_gamma, p.bc_beta, p.accum_g,
+                                        p.accum_b, st);
+      return 0;
+    }
+  }
   const uint32_t cpg = static_cast<uint32_t>(p.channels / p.groups);
 #define CALL(T, V) cl_bwd_reduce_t<T, V>(p, pl, w.part, st)
   const int e1 = [&]() -> int { BN_DISPATCH(CALL, pl.vec); }();

@@ -1,0 +1,271 @@
+// Channel-last GroupNormalization with the group cached in registers: one
+// pass over HBM per direction, like the channel-first row kernels of rows.cuh.
+//
+// x is [N][P][C] (P spatial positions).  The reduction unit (n, g) is the
+// strided tile of P positions x cpg adjacent channels; with cpg a multiple of
+// the vector width a thread's vector holds VEC channels of one position, and
+// because cvg = cpg / VEC divides the block size a thread always meets the
+// same VEC channels: their gamma/beta (and, backward, their dgamma/dbeta
+// partial sums) live in registers.
+//
+// A vector is 16 bytes of a 128-byte line that the neighbouring groups of the
+// same position fill: gpl = 128 B / (cpg * sizeof(T)) groups share every line.
+// Workgroups are handed to the 8 XCDs round-robin by linear index, so the block
+// index is decoded such that the gpl blocks that share lines are neighbours on
+// ONE XCD: its L2 then fetches each line from memory once instead of gpl times
+// (one fetch per XCD that holds a sharer).
+#pragma once
+
+#include "common.cuh"
+#include "launch.hpp"
+
+namespace nblahip {
+
+struct GnClArgs {
+  const void *x;
+  const void *dy;     // backward only
+  void *out;          // y (forward) or dx (backward, may be null)
+  const float *gamma; // [C], may be null
+  const float *beta;  // [C], may be null (forward only)
+  float *mean;        // [N*G] forward: written; backward: read
+  float *var;
+  const float *dmean; // may be null
+  const float *dvar;  // may be null
+  float *pairs;       // backward: [N][C][2] = (sum dy*xh, sum dy) per sample and channel
+  int P, C, G, cpg;
+  int units;          // N * G
+  FastDiv cvg;        // channel vectors per group (cpg / VEC); divides the block size
+  int gpl;            // groups sharing a cache line, 1: plain block order
+  float eps, inv_R, one;
+  int accum_dx;
+};
+
+constexpr int kXcds = 8;
+
+// Unit (n*G + g) of this block, or -1 for the padding blocks of the XCD map:
+// block b runs on XCD b % 8; consecutive blocks of one XCD take the gpl
+// members of one line-sharing set, then the next set of that XCD.
+__device__ __forceinline__ int gn_cl_unit(const GnClArgs &a) {
+  const uint32_t b = blockIdx.x;
+  if (a.gpl <= 1) return static_cast<int>(b);
+  const uint32_t xcd = b % kXcds, r = b / kXcds;
+  const uint32_t m = r % a.gpl, set = (r / a.gpl) * kXcds + xcd;
+  const uint32_t unit = set * a.gpl + m;
+  return unit < static_cast<uint32_t>(a.units) ? static_cast<int>(unit) : -1;
+}
+
+template <int TPR> __device__ __forceinline__ float gn_cl_block_sum(float v, float *lds) {
+  v = wave_sum(v);
+  constexpr int NW = TPR / kWave;
+  const int wave = threadIdx.x / kWave;
+  lds_barrier();
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[wave] = v;
+  lds_barrier();
+  float total = 0.f;
+#pragma unroll
+  for (int i = 0; i < NW; ++i) total += lds[i];
+  return total;
+}
+
+// ---------------------------------------------------------------------------
+// Forward.  Block = one (n, g); thread t owns channel vector t % cvg and the
+// positions t / cvg + k * (TPR / cvg), k < NL.
+// ---------------------------------------------------------------------------
+template <typename T, int VEC, int NL, int TPR>
+__global__ void __launch_bounds__(TPR)
+gn_cl_row_fwd_kernel(const GnClArgs a) {
+  __shared__ float lds[TPR / kWave];
+  const int unit = gn_cl_unit(a);
+  if (unit < 0) return;
+  const uint32_t n = static_cast<uint32_t>(unit) / a.G, g = static_cast<uint32_t>(unit) % a.G;
+  const uint32_t pos0 = a.cvg.div(threadIdx.x);
+  const uint32_t cv = threadIdx.x - pos0 * a.cvg.d;
+  const uint32_t pstep = TPR / a.cvg.d;
+  const uint32_t ch = g * a.cpg + cv * VEC; // first of this thread's channels
+  const T *__restrict__ x = static_cast<const T *>(a.x) + static_cast<size_t>(n) * a.P * a.C + ch;
+  T *__restrict__ y = static_cast<T *>(a.out) + static_cast<size_t>(n) * a.P * a.C + ch;
+
+  RawVec<T, VEC> raw[NL];
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = pos0 + k * pstep;
+    const bool ok = pos < static_cast<uint32_t>(a.P);
+    raw[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + static_cast<size_t>(ok ? pos : 0u) * a.C));
+  }
+  float gam[VEC], bet[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    gam[j] = a.gamma ? a.gamma[ch + j] : 1.f;
+    bet[j] = a.beta ? a.beta[ch + j] : 0.f;
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) s = raw_sum<T, VEC>(raw[k], s);
+  const float mean = gn_cl_block_sum<TPR>(s, lds) * a.inv_R;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+  float q = 0.f;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    if (pos0 + k * pstep < static_cast<uint32_t>(a.P)) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float d = elem_fma<T, VEC>(raw[k], j, a.one, -mean);
+        q = fmaf(d, d, q);
+      }
+    }
+  }
+  const float var = gn_cl_block_sum<TPR>(q, lds) * a.inv_R;
+  const float istd = inv_std(var, a.eps);
+  if (threadIdx.x == 0) {
+    a.mean[unit] = mean;
+    a.var[unit] = var;
+  }
+#pragma unroll
+  for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+  float sc[VEC], sh[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    sc[j] = gam[j] * istd;
+    sh[j] = fmaf(-mean, sc[j], bet[j]); // half output: x*sc + sh in one mixed fma
+  }
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = pos0 + k * pstep;
+    if (pos < static_cast<uint32_t>(a.P)) {
+      float o[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        if constexpr (sizeof(T) == 2) {
+          o[j] = elem_fma<T, VEC>(raw[k], j, sc[j], sh[j]);
+        } else {
+          o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mean), sc[j], bet[j]);
+        }
+      }
+      store_vec<T, VEC>(y + static_cast<size_t>(pos) * a.C, o);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Backward: dx and the per-(n, channel) pairs behind dgamma/dbeta.  With
+// xh = (x-mean)*istd and dg = dy*gamma:
+//   s1 = sum dg, t2 = sum dg*xh, cA = -istd*t2/R + 2*dvar*std/R,
+//   cb = -s1*istd/R + dmean/R, dx = dg*istd + cA*xh + cb
+// (the algebra of the channel-first row kernel).  A thread's channels are
+// fixed, so its VEC pairs (sum dy*xh, sum dy) accumulate in registers; threads
+// with the same channel vector are folded by wave sums and an LDS pass.
+// ---------------------------------------------------------------------------
+template <typename T, int VEC, int NL, int TPR>
+__global__ void __launch_bounds__(TPR, (TPR == 512 ? 4 : 1))
+gn_cl_row_bwd_kernel(const GnClArgs a) {
+  constexpr int NW = TPR / kWave;
+  __shared__ float fold[NW][2 * VEC * 8]; // per wave: up to 8 channel vectors x 2*VEC sums
+  __shared__ float chs[2 * VEC * 8];      // folded per-channel sums of the group (cpg <= 8*VEC)
+  const int unit = gn_cl_unit(a);
+  if (unit < 0) return;
+  const uint32_t n = static_cast<uint32_t>(unit) / a.G, g = static_cast<uint32_t>(unit) % a.G;
+  const uint32_t pos0 = a.cvg.div(threadIdx.x);
+  const uint32_t cv = threadIdx.x - pos0 * a.cvg.d;
+  const uint32_t pstep = TPR / a.cvg.d;
+  const uint32_t ch = g * a.cpg + cv * VEC;
+  const size_t slab = static_cast<size_t>(n) * a.P * a.C + ch;
+  const T *__restrict__ x = static_cast<const T *>(a.x) + slab;
+  const T *__restrict__ dy = static_cast<const T *>(a.dy) + slab;
+  T *__restrict__ dx = a.out ? static_cast<T *>(a.out) + slab : nullptr;
+
+  RawVec<T, VEC> xr[NL], dr[NL];
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = pos0 + k * pstep;
+    const bool ok = pos < static_cast<uint32_t>(a.P);
+    const size_t off = static_cast<size_t>(ok ? pos : 0u) * a.C;
+    xr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + off));
+    dr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(dy + off));
+  }
+  float gam[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) gam[j] = a.gamma ? a.gamma[ch + j] : 1.f;
+  const float mean = a.mean[unit];
+  const float vpe = a.var[unit] + a.eps;
+  const float istd = 1.0f / sqrtf(vpe);
+  const float nmi = -mean * istd;
+
+  // per-channel partial sums of this thread (padded positions hold dy = 0)
+  float sdx[VEC], sdy[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) sdx[j] = sdy[j] = 0.f;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+      sdx[j] = elem_fma<T, VEC>(dr[k], j, xh, sdx[j]);
+      sdy[j] = elem_fma<T, VEC>(dr[k], j, a.one, sdy[j]);
+    }
+  }
+  // Lanes with equal lane % cvg share channels (cvg is a power of two <= 8):
+  // butterfly over the lane bits above log2(cvg), then one LDS row per wave.
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    for (int off = static_cast<int>(a.cvg.d); off < kWave; off <<= 1) {
+      sdx[j] += __shfl_xor(sdx[j], off);
+      sdy[j] += __shfl_xor(sdy[j], off);
+    }
+  }
+  if (lane < static_cast<int>(a.cvg.d)) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      fold[wave][(lane * VEC + j) * 2] = sdx[j];
+      fold[wave][(lane * VEC + j) * 2 + 1] = sdy[j];
+    }
+  }
+  lds_barrier();
+  if (static_cast<int>(threadIdx.x) < 2 * a.cpg) {
+    float t = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) t += fold[w][threadIdx.x];
+    chs[threadIdx.x] = t;
+    // entry 2*c of the group is (sum dy*xh) of its channel c, 2*c+1 (sum dy)
+    a.pairs[2 * (static_cast<size_t>(n) * a.C + g * a.cpg) + threadIdx.x] = t;
+  }
+  lds_barrier();
+  float s1 = 0.f, t2 = 0.f;
+  for (int c = 0; c < a.cpg; ++c) {
+    const float gc = a.gamma ? a.gamma[g * a.cpg + c] : 1.f;
+    t2 = fmaf(gc, chs[2 * c], t2);
+    s1 = fmaf(gc, chs[2 * c + 1], s1);
+  }
+  if (dx == nullptr) return;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    keep_packed<T, VEC>(xr[k]);
+    keep_packed<T, VEC>(dr[k]);
+  }
+  const float cA = -istd * t2 * a.inv_R + (a.dvar ? 2.f * a.dvar[unit] * (vpe * istd) * a.inv_R : 0.f);
+  const float cb = -s1 * istd * a.inv_R + (a.dmean ? a.dmean[unit] * a.inv_R : 0.f);
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = pos0 + k * pstep;
+    if (pos < static_cast<uint32_t>(a.P)) {
+      float o[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+        o[j] = elem_fma<T, VEC>(dr[k], j, gam[j] * istd, fmaf(xh, cA, cb));
+      }
+      T *p = dx + static_cast<size_t>(pos) * a.C;
+      if (a.accum_dx) {
+        float old[VEC];
+        load_vec<T, VEC>(p, old);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) o[j] += old[j];
+      }
+      store_vec<T, VEC>(p, o);
+    }
+  }
+}
+
+} // namespace nblahip

@@ -1,0 +1,142 @@
+// Instantiations and launcher of the register-cached channel-last
+// GroupNormalization kernels.
+#include <algorithm>
+
+#include "gn_cl_rows.cuh"
+
+namespace nblahip {
+
+namespace {
+
+struct GnClCfg {
+  bool ok = false;
+  int vec = 1, tpr = 256, nl = 1;
+};
+
+// The cached kernels apply when a group is at least one vector of channels
+// wide (cpg = VEC * cvg, cvg in {1, 2, 4, 8}), fits 8 loads per thread of a
+// block, and is big enough to be worth a block; parameters shared by the batch.
+GnClCfg pick_cfg(const ClProblem &p, bool aligned, bool backward, GnClArgs &a) {
+  GnClCfg c;
+  if (!aligned || !tune_int("GN_CL_CACHED", 1)) return c;
+  if (!p.bc_gamma || !p.bc_beta) return c;
+  const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
+  const int64_t cpg = p.channels / p.groups;
+  if (cpg % vec != 0) return c;
+  const int64_t cvg = cpg / vec;
+  if (cvg != 1 && cvg != 2 && cvg != 4 && cvg != 8) return c;
+  const int64_t nv = p.spatial * cvg;
+  if (nv < 256) return c;
+  // Backward, beyond 2048 vectors per group the three-kernel path is as fast
+  // or faster (64 KB half groups: 41.9 vs 42.4 us; 50 KB ones: 56.1 vs 52.6 us),
+  // the strided 16-byte accesses of two tensors being the limit; below it the
+  // single pass wins clearly (28x28 planes: 24 vs 39 us).
+  if (backward && nv > 2048) return c;
+  for (int tpr : {256, 512, 1024}) {
+    for (int nl : {1, 2, 4, 8}) {
+      if (static_cast<int64_t>(tpr) * nl < nv) continue;
+      // the float 1024 x 8 layout (128 KB of x and dy in one block's registers)
+      // is left to the three-kernel path
+      if (p.dtype == NBLAHIP_F32 && tpr == 1024 && nl == 8) continue;
+      c.ok = true;
+      c.vec = vec;
+      c.tpr = tpr;
+      c.nl = nl;
+      break;
+    }
+    if (c.ok) break;
+  }
+  if (!c.ok) return c;
+  a.P = static_cast<int>(p.spatial);
+  a.C = static_cast<int>(p.channels);
+  a.G = p.groups;
+  a.cpg = static_cast<int>(cpg);
+  a.units = static_cast<int>(p.batch * p.groups);
+  a.cvg = FastDiv(static_cast<uint32_t>(cvg));
+  const int64_t line = 128 / (p.dtype == NBLAHIP_F16 ? 2 : 4); // elements per 128-byte line
+  const int64_t gpl = line / cpg;
+  a.gpl = (gpl >= 2 && p.groups % gpl == 0 && tune_int("GN_CL_XCD_MAP", 1)) ? static_cast<int>(gpl) : 1;
+  a.eps = p.eps;
+  a.inv_R = static_cast<float>(1.0 / (static_cast<double>(p.spatial) * cpg));
+  a.one = 1.0f;
+  a.accum_dx = p.accum_dx;
+  return c;
+}
+
+unsigned grid_of(const GnClArgs &a) {
+  if (a.gpl <= 1) return static_cast<unsigned>(a.units);
+  const unsigned sets = static_cast<unsigned>(a.units / a.gpl);
+  return (sets + kXcds - 1) / kXcds * kXcds * static_cast<unsigned>(a.gpl);
+}
+
+#define GN_CL_CASES_TPR(CASE, T, VEC, TPR) \
+  CASE(T, VEC, 1, TPR) CASE(T, VEC, 2, TPR) CASE(T, VEC, 4, TPR) CASE(T, VEC, 8, TPR)
+#define GN_CL_CASES(CASE, T, VEC) \
+  GN_CL_CASES_TPR(CASE, T, VEC, 256) GN_CL_CASES_TPR(CASE, T, VEC, 512) GN_CL_CASES_TPR(CASE, T, VEC, 1024)
+
+#define FWD_CASE(T, VEC, NL, TPR)                                                              \
+  if (c.nl == (NL) && c.tpr == (TPR)) {                                                        \
+    NBLAHIP_LAUNCH("gn_cl_row_fwd_kernel", (gn_cl_row_fwd_kernel<T, VEC, NL, TPR>),            \
+                   dim3(grid_of(a)), dim3(TPR), 0, st, a);                                     \
+    return last_launch_status();                                                               \
+  }
+#define BWD_CASE(T, VEC, NL, TPR)                                                              \
+  if (c.nl == (NL) && c.tpr == (TPR)) {                                                        \
+    NBLAHIP_LAUNCH("gn_cl_row_bwd_kernel", (gn_cl_row_bwd_kernel<T, VEC, NL, TPR>),            \
+                   dim3(grid_of(a)), dim3(TPR), 0, st, a);                                     \
+    return last_launch_status();                                                               \
+  }
+
+int run_fwd(int dtype, const GnClCfg &c, const GnClArgs &a, hipStream_t st) {
+  if (dtype == NBLAHIP_F16) {
+    GN_CL_CASES(FWD_CASE, __half, 8)
+  } else {
+    GN_CL_CASES(FWD_CASE, float, 4)
+  }
+  return NBLAHIP_EINVAL;
+}
+
+int run_bwd(int dtype, const GnClCfg &c, const GnClArgs &a, hipStream_t st) {
+  if (dtype == NBLAHIP_F16) {
+    GN_CL_CASES(BWD_CASE, __half, 8)
+  } else {
+    GN_CL_CASES(BWD_CASE, float, 4)
+  }
+  return NBLAHIP_EINVAL;
+}
+
+} // namespace
+
+bool gn_cl_cached_fwd(const ClProblem &p, bool aligned, hipStream_t st, int *status) {
+  GnClArgs a{};
+  const GnClCfg c = pick_cfg(p, aligned, false, a);
+  if (!c.ok) return false;
+  a.x = p.x;
+  a.out = p.out;
+  a.gamma = p.gamma;
+  a.beta = p.beta;
+  a.mean = p.mean;
+  a.var = p.var;
+  *status = run_fwd(p.dtype, c, a, st);
+  return true;
+}
+
+bool gn_cl_cached_bwd(const ClProblem &p, bool aligned, float *pairs, hipStream_t st,
+                      int *status) {
+  GnClArgs a{};
+  const GnClCfg c = pick_cfg(p, aligned, true, a);
+  if (!c.ok) return false;
+  a.x = p.x;
+  a.dy = p.dy;
+  a.out = p.out;
+  a.gamma = p.gamma;
+  a.mean = p.mean;
+  a.var = p.var;
+  a.dmean = p.dmean;
+  a.dvar = p.dvar;
+  a.pairs = pairs;
+  *status = run_bwd(p.dtype, c, a, st);
+  return true;
+}
+
+} // namespace nblahip

@@ -162,6 +162,11 @@ struct ClProblem {
   void *ws = nullptr;
   size_t ws_bytes = 0;
 };
+// Register-cached channel-last GroupNormalization (gn_cl_rows.hip): false when
+// the shape is not theirs, else *status holds the launch result.  The backward
+// leaves the per-(n, channel) pairs in `pairs` for the batch sum.
+bool gn_cl_cached_fwd(const ClProblem &p, bool aligned, hipStream_t st, int *status);
+bool gn_cl_cached_bwd(const ClProblem &p, bool aligned, float *pairs, hipStream_t st, int *status);
 int launch_cl_fwd(const ClProblem &p, hipStream_t st);
 int launch_cl_bwd(const ClProblem &p, hipStream_t st);
 size_t cl_workspace_bytes(int64_t batch, int64_t spatial, int64_t channels, int dtype);

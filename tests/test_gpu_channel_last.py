@@ -47,7 +47,11 @@ GN_CL_SHAPES = [(2, (8, 8), 8, 4), (3, (5,), 6, 2), (1, (2, 2), 4, 1), (2, (4,),
                 (2, (512,), 12, 3), (2, (), 4, 2), (3, (64,), 10, 5), (1, (40, 40), 40, 2),
                 (2, (3, 3), 2048, 32), (2, (4096,), 32, 4), (5, (33,), 7, 7), (1, (1,), 5, 1),
                 # channel vectors that do not divide 256, rows wider than 256 vectors, 8-byte fp16 rows
-                (2, (9, 9), 96, 4), (2, (5, 5), 4104, 8), (3, (11,), 100, 5), (2, (6, 6), 20, 2)]
+                (2, (9, 9), 96, 4), (2, (5, 5), 4104, 8), (3, (11,), 100, 5), (2, (6, 6), 20, 2),
+                # group cached in registers: 1 to 8 channel vectors per group, ragged last load,
+                # groups that share cache lines (the XCD block map) and groups that do not
+                (3, (33, 33), 64, 2), (2, (20, 20), 128, 2), (5, (17, 17), 16, 1), (3, (24, 24), 96, 12),
+                (2, (56, 56), 64, 8), (9, (16, 16), 32, 4), (1, (90, 90), 8, 1)]
 
 
 @pytest.mark.parametrize("n,sp,c,groups", GN_CL_SHAPES)
