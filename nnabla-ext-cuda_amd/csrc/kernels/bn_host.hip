@@ -423,6 +423,8 @@ int bn_fwd_train_impl(const BnProblem &p, bool stats_only, hipStream_t st) {
 } // namespace
 
 int launch_bn_fwd_train(const BnProblem &p, hipStream_t st) {
+  int status = 0;
+  if (bn_rows_fwd_train(p, st, &status)) return status;
   return bn_fwd_train_impl(p, false, st);
 }
 
@@ -442,6 +444,10 @@ int launch_bn_merge_stats(const float *stats, int workers, int64_t C, float *bat
 
 int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
   if (!p.out && !p.dgamma && !p.dbeta && !p.dz && !p.sums_out) return 0;
+  {
+    int status = 0;
+    if (bn_rows_bwd(p, st, &status)) return status;
+  }
   const bool al = aligned16(p.x) && aligned16(p.dy) && (!p.out || aligned16(p.out)) &&
                   (!p.y || aligned16(p.y)) && (!p.dz || aligned16(p.dz));
   const BnPlan pl = make_plan(p.size0, p.C, p.size2, p.dtype, al);

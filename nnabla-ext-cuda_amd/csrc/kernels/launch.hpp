@@ -16,7 +16,9 @@ namespace nblahip {
 // the batch itself, so dgamma/dbeta need no second kernel.
 // kRowGNm: GroupNormalization backward with the run-time thread map (planes
 // that are no multiple of a wave-wide load); kRowGN is the fixed map.
-enum RowMode { kRowLN = 0, kRowIN = 1, kRowGN = 2, kRowINc = 3, kRowGNm = 4 };
+// kRowBN: BatchNormalization of tensors whose channel (all its planes) fits a
+// block's registers: a row is the strided set of planes of one channel.
+enum RowMode { kRowLN = 0, kRowIN = 1, kRowGN = 2, kRowINc = 3, kRowGNm = 4, kRowBN = 5 };
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -109,6 +111,11 @@ struct BnProblem {
   size_t ws_bytes = 0;
 };
 
+// BatchNormalization training forward / backward with a channel cached in
+// registers (one launch, x and dy cross HBM once per direction): false when
+// the shape or the flags are not theirs, else *status holds the launch result.
+bool bn_rows_fwd_train(const BnProblem &p, hipStream_t st, int *status);
+bool bn_rows_bwd(const BnProblem &p, hipStream_t st, int *status);
 int launch_bn_infer(const BnProblem &p, hipStream_t st);
 int launch_bn_fwd_train(const BnProblem &p, hipStream_t st);
 int launch_bn_bwd(const BnProblem &p, hipStream_t st);

@@ -61,7 +61,26 @@ struct RowArgs {
   int gn_nwc;      // channels the block's waves cover at once (NW / gn_wpc)
   int gn_pv;       // vectors per plane (spatial / VEC)
   uint64_t gn_map; // per load k, 8 bits: (pass over the channels) | (load within the channel) << 4; 0xff unused
+  // BatchNormalization rows (STRIDED / kRowBN): row c is the planes (n, c),
+  // n = 0..N-1, each `plane.d` contiguous elements, plane_jump = (C-1)*plane.d
+  // elements between the end of one and the start of the next.
+  FastDiv plane;
+  uint32_t plane_jump;
+  float *rmean; // running statistics, may be null
+  float *rvar;
+  float decay, unbias;
 };
+
+// Offset of element col of a row from the row's first element.
+template <bool STRIDED>
+__device__ __forceinline__ size_t row_elem_offset(const RowArgs &a, int col) {
+  if constexpr (STRIDED) {
+    return static_cast<size_t>(col) +
+           static_cast<size_t>(a.plane.div(static_cast<uint32_t>(col))) * a.plane_jump;
+  } else {
+    return static_cast<size_t>(col);
+  }
+}
 
 // GroupNormalization backward thread map.  A wave-wide load never crosses a
 // channel, so the per-channel sums the parameter gradients need are wave sums.
@@ -131,7 +150,9 @@ template <typename T, int VEC, int NL, int TPR, int MODE> struct RowBwdOccupancy
 // and kept in registers); otherwise one scalar gamma/beta per 16-byte load,
 // fetched while the row is still in flight.
 // ---------------------------------------------------------------------------
-template <typename T, int VEC, int NL, int TPR, bool PERCOL>
+// STRIDED: BatchNormalization rows (see RowArgs::plane); also updates the
+// running statistics.
+template <typename T, int VEC, int NL, int TPR, bool PERCOL, bool STRIDED = false>
 __global__ void __launch_bounds__(RowBlock<TPR>::kBlock)
 row_fwd_kernel(const RowArgs a) {
   constexpr int RPB = RowBlock<TPR>::kRowsPerBlock;
@@ -163,7 +184,7 @@ row_fwd_kernel(const RowArgs a) {
   }
 
   for (int row = blockIdx.x * RPB + sub; row < a.rows; row += gridDim.x * RPB) {
-    const size_t base = static_cast<size_t>(row) * a.R;
+    const size_t base = static_cast<size_t>(row) * (STRIDED ? a.plane.d : a.R);
     RawVec<T, VEC> raw[NL];
 #pragma unroll
     for (int k = 0; k < NL; ++k) {
@@ -171,7 +192,8 @@ row_fwd_kernel(const RowArgs a) {
       // no branch, so the NL loads are in flight together.
       const int col = (k * TPR + t) * VEC;
       const bool ok = col < a.R;
-      raw[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + base + (ok ? col : 0)));
+      raw[k] = raw_or_zero<T, VEC>(
+          ok, load_raw<T, VEC>(x + base + row_elem_offset<STRIDED>(a, ok ? col : 0)));
     }
     float gk[PERCOL ? 1 : NL], bk[PERCOL ? 1 : NL];
     if constexpr (!PERCOL) {
@@ -209,6 +231,10 @@ row_fwd_kernel(const RowArgs a) {
     if (t == 0) {
       a.mean[row] = mean;
       a.var[row] = var;
+      if constexpr (STRIDED) {
+        if (a.rmean) a.rmean[row] = a.decay * a.rmean[row] + (1.f - a.decay) * mean;
+        if (a.rvar) a.rvar[row] = a.decay * a.rvar[row] + (1.f - a.decay) * var * a.unbias;
+      }
     }
 #pragma unroll
     for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
@@ -235,7 +261,7 @@ row_fwd_kernel(const RowArgs a) {
           for (int j = 0; j < VEC; ++j)
             o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mean), g, bk[k]);
         }
-        store_vec<T, VEC>(y + base + col, o);
+        store_vec<T, VEC>(y + base + row_elem_offset<STRIDED>(a, col), o);
       }
     }
   }
@@ -269,6 +295,7 @@ row_bwd_kernel(const RowArgs a) {
   // reduction and the dx step when they are few; otherwise they are recomputed.
   constexpr bool KEEP = (MODE == kRowLN) && (NL * VEC <= 16);
   constexpr bool GN = MODE == kRowGN || MODE == kRowGNm;
+  constexpr bool BN = MODE == kRowBN; // strided rows, dgamma/dbeta written here
   constexpr bool GNM = MODE == kRowGNm; // run-time thread map (GnSlot)
   __shared__ float lds[2 * 16];
   __shared__ float part[GN ? 2 * NW * NL : 1];
@@ -320,7 +347,7 @@ row_bwd_kernel(const RowArgs a) {
   float ch_sdx = 0.f, ch_sdy = 0.f; // kRowINc: this wave's share of the channel sums
   for (int rr = CH ? sub : 0; rr < inner_n; rr += CH ? RPB : 1) {
     const int row = CH ? rr * channels + unit : unit;
-    const size_t base = static_cast<size_t>(row) * a.R;
+    const size_t base = static_cast<size_t>(row) * (BN ? a.plane.d : a.R);
     float gk[NL];                                   // per-load scalar gamma (IN / GN)
     float gch = 1.f;                                // GN: gamma of channel threadIdx.x
     if constexpr (GN) {
@@ -349,9 +376,10 @@ row_bwd_kernel(const RowArgs a) {
         col = sl.col;
         ok = sl.ok;
       }
-      const int colc = ok ? col : 0; // branch-free: all loads in flight together
-      xr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + base + colc));
-      dr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(dy + base + colc));
+      // branch-free: all loads in flight together
+      const size_t off = base + row_elem_offset<BN>(a, ok ? col : 0);
+      xr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + off));
+      dr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(dy + off));
     }
     const float mean = a.mean[row];
     const float vpe = a.var[row] + a.eps;
@@ -378,7 +406,7 @@ row_bwd_kernel(const RowArgs a) {
         }
       }
       row_sum2<TPR>(s1, t2, lds);
-    } else if constexpr (MODE == kRowIN || MODE == kRowINc) {
+    } else if constexpr (MODE == kRowIN || MODE == kRowINc || BN) {
       float sdy = 0.f, sdx = 0.f;
 #pragma unroll
       for (int k = 0; k < NL; ++k) {
@@ -393,6 +421,11 @@ row_bwd_kernel(const RowArgs a) {
       if constexpr (CH) {
         ch_sdx += sdx;
         ch_sdy += sdy;
+      } else if constexpr (BN) {
+        if (t == 0) {
+          if (a.dgamma) a.dgamma[row] = sdx + (a.accum_g ? a.dgamma[row] : 0.f);
+          if (a.dbeta) a.dbeta[row] = sdy + (a.accum_b ? a.dbeta[row] : 0.f);
+        }
       } else {
         if (t == 0) {
           a.ws[2 * static_cast<size_t>(row)] = sdx;
@@ -496,13 +529,14 @@ row_bwd_kernel(const RowArgs a) {
               o[j] = elem_fma<T, VEC>(dr[k], j, gi, fmaf(xh, cA, cb));
             }
           }
+          T *dst = dx + base + row_elem_offset<BN>(a, col);
           if (a.accum_dx) {
             float old[VEC];
-            load_vec<T, VEC>(dx + base + col, old);
+            load_vec<T, VEC>(dst, old);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) o[j] += old[j];
           }
-          store_vec<T, VEC>(dx + base + col, o);
+          store_vec<T, VEC>(dst, o);
         }
       }
     }

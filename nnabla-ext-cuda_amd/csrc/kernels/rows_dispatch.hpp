@@ -21,6 +21,10 @@ int run_row_bwd_cached_inc(int dtype, const RowCfg &cfg, const RowArgs &args, in
                            hipStream_t st);
 int run_row_bwd_cached_gn(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
                           hipStream_t st);
+int run_row_fwd_cached_bn(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
+                          hipStream_t st);
+int run_row_bwd_cached_bn(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
+                          hipStream_t st);
 int run_row_bwd_cached_gnm(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
                            hipStream_t st);
 

@@ -1,0 +1,26 @@
+// Instantiations and launcher of the register-cached forward row kernel for
+// BatchNormalization rows (a row = the planes of one channel).
+#include "rows_dispatch.hpp"
+
+namespace nblahip {
+
+#define FWD_CASE(T, VEC, NL, TPR)                                                      \
+  if (cfg.vec == (VEC) && cfg.nl == (NL) && cfg.tpr == (TPR)) {                        \
+    NBLAHIP_LAUNCH("row_fwd_kernel_bn", (row_fwd_kernel<T, VEC, NL, TPR, false, true>), \
+                   dim3(grid), dim3(RowBlock<TPR>::kBlock), 0, st, args);              \
+    return last_launch_status();                                                       \
+  }
+
+template <typename T>
+static int run_fwd_t(const RowCfg &cfg, const RowArgs &args, int grid, hipStream_t st) {
+  NBLAHIP_ROW_CASES(FWD_CASE, T)
+  return NBLAHIP_EINVAL;
+}
+
+int run_row_fwd_cached_bn(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
+                          hipStream_t st) {
+  return dtype == NBLAHIP_F16 ? run_fwd_t<__half>(cfg, args, grid, st)
+                              : run_fwd_t<float>(cfg, args, grid, st);
+}
+
+} // namespace nblahip

@@ -21,6 +21,9 @@ SMALL = [
     # planes that are no multiple of the vector width, tensor a multiple: masked vectors
     ((4, 8, 7, 7), 1), ((2, 16, 9, 9), 1), ((3, 8, 3, 11), 1), ((1, 24, 5, 5), 1),
     ((64, 32, 7, 7), 1), ((5, 16, 13), 1),
+    # a channel (all its planes) in one block's registers: every row layout
+    ((32, 64, 28, 28), 1), ((16, 128, 14, 14), 1), ((6, 256, 3, 3), 1), ((2, 512, 2, 2), 1),
+    ((64, 40, 32, 32), 1), ((9, 33, 5, 5), 1), ((2, 64, 64, 64), 1),
     # channel-last: channel vectors that do not divide 256, rows wider than 256 vectors,
     # 8-byte fp16 rows
     ((6, 9, 9, 96), 3), ((3, 5, 5, 4104), 3), ((37, 100), 1), ((4, 6, 6, 20), 3), ((700, 1032), 1),
@@ -77,7 +80,9 @@ def test_bn_training_forward_backward(shape, axis, dtype):
     assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
 
 
-@pytest.mark.parametrize("shape,axis", [((4, 8, 6, 6), 1), ((37, 24), 1), ((6, 5, 4, 8), 3)])
+@pytest.mark.parametrize("shape,axis", [((4, 8, 6, 6), 1), ((37, 24), 1), ((6, 5, 4, 8), 3),
+                                        # a channel per block, cached in registers
+                                        ((8, 64, 12, 12), 1), ((4, 48, 7, 9), 1), ((3, 300, 2, 2), 1)])
 def test_bn_flags(shape, axis):
     """no_scale/no_bias, recompute (no running update), accumulation,
     propagate_down subsets, 3-output dmean/dvar."""
