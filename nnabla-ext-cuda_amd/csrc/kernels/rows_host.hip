@@ -456,9 +456,14 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
     // InstanceNormalization with parameters shared by the batch and enough
     // channels to fill the chip: a block per channel sums over the batch
     // itself, no second kernel.
+    // Not with fewer channels than CUs (half the chip idles: [64,128,64,64]
+    // float 126 vs 75 us) nor for float planes of 512 vectors and more in
+    // batches of 8 and more (10-18 % slower than a row per block plus the
+    // batch sum; smaller batches save more on the second launch).
+    const bool big_float = p.dtype == NBLAHIP_F32 && cfg.tpr * cfg.nl >= 512 && p.batch >= 8;
     if (p.mode == kRowIN && p.bc_gamma && p.bc_beta && p.batch > 1 &&
-        p.channels * 2 >= device_cus() && !(cfg.tpr == 1024 && cfg.nl == 8) && cfg.tpr >= 64 &&
-        !tune_int("IN_NO_CHANNEL_BLOCKS", 0)) {
+        p.channels >= device_cus() && !big_float && !(cfg.tpr == 1024 && cfg.nl == 8) &&
+        cfg.tpr >= 64 && !tune_int("IN_NO_CHANNEL_BLOCKS", 0)) {
       const int grid = static_cast<int>(std::min<int64_t>(p.channels, 1 << 20));
       return run_row_bwd_cached_inc(p.dtype, cfg, a, grid, st);
     }
