@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the normalization hot path on one MI355X.
 
-Headline workload (BASELINE.json configs[1]): BatchNormalization training
+Headline workload (benchmark configuration 2): BatchNormalization training
 forward + backward, fp32 NCHW x[32,256,56,56] ~ N(1,2), dy ~ N(0,1),
 decay_rate 0.9, eps 1e-5.  One step = one forward (batch statistics, running
 statistics update, y) plus one backward (dx, dgamma, dbeta) through the C-ABI,
@@ -13,7 +13,7 @@ Prints ONE JSON line.  `value` is algorithmic GB/s of the whole step
 HIP events on the launch stream in a second region of the same K steps;
 `cpu_baseline` is the C restatement of the reference arithmetic
 (oracle/norm_ref.c) on the same workload on the host cores; `configs` lists
-every BASELINE configuration (microseconds per call and algorithmic GB/s).
+every benchmark configuration (microseconds per call and algorithmic GB/s).
 """
 import argparse
 import json
@@ -247,7 +247,7 @@ def time_in_graph(K, calls, steps, warmup):
 
 
 def config_table(K, steps, warmup):
-    """Every BASELINE configuration: us per call and algorithmic GB/s."""
+    """Every benchmark configuration: us per call and algorithmic GB/s."""
     import torch
     specs = [
         ("C1 BN inference fp32 [8,64,56,56]", lambda: make_bn(K, (8, 64, 56, 56), 1, torch.float32, False, seed=0)),
@@ -486,7 +486,7 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "BatchNormalization training fwd+bwd fp32 NCHW x[32,256,56,56] "
-                               "(BASELINE configs[1]), decay_rate 0.9, eps 1e-5",
+                               "(benchmark configuration 2), decay_rate 0.9, eps 1e-5",
                    "algorithmic_bytes_per_step": fb + bb,
                    "pct_of_hbm_peak": round(value / HBM_PEAK_GBS * 100, 1)},
         "roofline": roofline,

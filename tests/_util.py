@@ -1,5 +1,5 @@
 """Shared helpers of the test-suite: package loading, tolerances, input
-generators for the BASELINE configurations."""
+generators for the benchmark configurations."""
 import importlib.util
 import os
 import sys

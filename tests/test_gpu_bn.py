@@ -191,7 +191,7 @@ def test_bn_odd_planes_channel_owning_blocks(dtype):
 
 
 def test_bn_c1_inference_full_size():
-    """BASELINE config 1: x[8,64,56,56] fp32, inference, seed 0."""
+    """Benchmark configuration 1: x[8,64,56,56] fp32, inference, seed 0."""
     rng = np.random.default_rng(0)
     shape = (8, 64, 56, 56)
     x = rng.standard_normal(shape).astype(np.float32)
@@ -205,7 +205,7 @@ def test_bn_c1_inference_full_size():
 
 
 def test_bn_c2_training_full_size():
-    """BASELINE config 2: x[32,256,56,56] ~ N(1,2) fp32, fwd+bwd, seed 1."""
+    """Benchmark configuration 2: x[32,256,56,56] ~ N(1,2) fp32, fwd+bwd, seed 1."""
     rng = np.random.default_rng(1)
     shape = (32, 256, 56, 56)
     x = (rng.standard_normal(shape, dtype=np.float32) * 2 + 1).astype(np.float32)
@@ -233,7 +233,7 @@ def test_bn_c2_training_full_size():
 
 
 def test_bn_c5_channel_last_fp16_full_size():
-    """BASELINE config 5: x[256,56,56,64] fp16 with 1% outliers x50, axes=[3],
+    """Benchmark configuration 5: x[256,56,56,64] fp16 with 1% outliers x50, axes=[3],
     fp32 statistics, split reduction over 802816 rows, seed 4."""
     rng = np.random.default_rng(4)
     shape = (256, 56, 56, 64)

@@ -215,7 +215,7 @@ def test_channel_last_misaligned_pointer():
 
 
 def test_c4_channel_last_full_size():
-    """BASELINE config 4 stored channel-last: x[16,64,64,256] fp16, GN with 32
+    """Benchmark configuration 4 stored channel-last: x[16,64,64,256] fp16, GN with 32
     groups and IN, seed 3."""
     rng = np.random.default_rng(3)
     n, c, sp = 16, 256, (64, 64)

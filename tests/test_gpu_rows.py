@@ -127,7 +127,7 @@ def test_ln_misaligned_pointer():
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_ln_c3_full_size(dtype):
-    """BASELINE config 3: x[32,512,1024] ~ N(0,1) + per-row offset U(-3,3),
+    """Benchmark configuration 3: x[32,512,1024] ~ N(0,1) + per-row offset U(-3,3),
     gamma ~ N(1,0.1), beta ~ N(0,0.1), seed 2, fp32 and fp16."""
     dn = dtype_name(dtype)
     rng = np.random.default_rng(2)
@@ -285,7 +285,7 @@ def test_in_per_sample_parameters_and_flags(n, c, sp, bcg, bcb):
 
 
 def test_c4_gn_and_in_full_size():
-    """BASELINE config 4: x[16,256,64,64] ~ N(0,1.5) fp16, GN with 32 groups and
+    """Benchmark configuration 4: x[16,256,64,64] ~ N(0,1.5) fp16, GN with 32 groups and
     IN on the same tensor, seed 3."""
     rng = np.random.default_rng(3)
     n, c, sp = 16, 256, (64, 64)
