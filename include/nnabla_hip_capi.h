@@ -71,6 +71,16 @@ NNABLA_HIP_EXPORT nnabla_hip_function *nnabla_hip_create_group_normalization(
 NNABLA_HIP_EXPORT nnabla_hip_function *nnabla_hip_create_instance_normalization(
     const char *backends, const char *array_class, const char *device_id, int channel_axis,
     const int *batch_axis, int n_batch_axis, float eps, int no_scale, int no_bias);
+/* TensorNormalizationCuda / WeightStandardizationCuda
+ * (include/nbla/cuda/function/tensor_normalization.hpp:22-46,
+ * weight_standardization.hpp:22-46).  axes: the axes the statistics keep; they
+ * must be adjacent (the reference's composite transposes for other sets). */
+NNABLA_HIP_EXPORT nnabla_hip_function *nnabla_hip_create_tensor_normalization(
+    const char *backends, const char *array_class, const char *device_id, const int *axes,
+    int n_axes, float eps, int no_scale, int no_bias);
+NNABLA_HIP_EXPORT nnabla_hip_function *nnabla_hip_create_weight_standardization(
+    const char *backends, const char *array_class, const char *device_id, int channel_axis,
+    float eps);
 NNABLA_HIP_EXPORT void nnabla_hip_function_delete(nnabla_hip_function *f);
 NNABLA_HIP_EXPORT const char *nnabla_hip_function_name(nnabla_hip_function *f);
 

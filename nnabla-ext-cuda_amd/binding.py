@@ -42,6 +42,8 @@ SIGNATURES = {
     "nnabla_hip_create_layer_normalization": (_P, [_S, _S, _S, _IP, _I, _F, _I, _I]),
     "nnabla_hip_create_group_normalization": (_P, [_S, _S, _S, _I, _I, _IP, _I, _F, _I, _I]),
     "nnabla_hip_create_instance_normalization": (_P, [_S, _S, _S, _I, _IP, _I, _F, _I, _I]),
+    "nnabla_hip_create_tensor_normalization": (_P, [_S, _S, _S, _IP, _I, _F, _I, _I]),
+    "nnabla_hip_create_weight_standardization": (_P, [_S, _S, _S, _I, _F]),
     "nnabla_hip_function_delete": (None, [_P]),
     "nnabla_hip_function_name": (_S, [_P]),
     "nnabla_hip_function_setup": (_I, [_P, _PP, _I, _PP, _I]),
@@ -280,3 +282,15 @@ def InstanceNormalization(ctx, channel_axis=1, batch_axis=(0,), eps=1e-5, no_sca
     ba, n = _ints(list(batch_axis))
     return Function(lib().nnabla_hip_create_instance_normalization(
         *_ctx_args(ctx), channel_axis, ba, n, eps, int(no_scale), int(no_bias)))
+
+
+def TensorNormalization(ctx, axes=(1,), eps=1e-5, no_scale=False, no_bias=False):
+    """axes: the axes the statistics keep (adjacent); beta/gamma have their extent."""
+    ax, n = _ints(list(axes))
+    return Function(lib().nnabla_hip_create_tensor_normalization(
+        *_ctx_args(ctx), ax, n, eps, int(no_scale), int(no_bias)))
+
+
+def WeightStandardization(ctx, channel_axis=0, eps=1e-5):
+    return Function(lib().nnabla_hip_create_weight_standardization(
+        *_ctx_args(ctx), channel_axis, eps))

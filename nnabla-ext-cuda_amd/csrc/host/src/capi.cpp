@@ -7,6 +7,8 @@
 #include <nbla/function/group_normalization.hpp>
 #include <nbla/function/instance_normalization.hpp>
 #include <nbla/function/layer_normalization.hpp>
+#include <nbla/function/tensor_normalization.hpp>
+#include <nbla/function/weight_standardization.hpp>
 #include <nbla/hip/hip.hpp>
 #include <nbla/hip/init.hpp>
 #include <nbla/variable.hpp>
@@ -269,6 +271,32 @@ nnabla_hip_function *nnabla_hip_create_instance_normalization(const char *backen
     const vector<int> ba(batch_axis, batch_axis + n_batch_axis);
     out = wrap(create_InstanceNormalization(make_ctx(backends, array_class, device_id),
                                             channel_axis, ba, eps, no_scale != 0, no_bias != 0));
+  });
+  return out;
+}
+
+nnabla_hip_function *nnabla_hip_create_tensor_normalization(const char *backends,
+                                                            const char *array_class,
+                                                            const char *device_id, const int *axes,
+                                                            int n_axes, float eps, int no_scale,
+                                                            int no_bias) {
+  nnabla_hip_function *out = nullptr;
+  guarded([&] {
+    const vector<int> ax(axes, axes + n_axes);
+    out = wrap(create_TensorNormalization(make_ctx(backends, array_class, device_id), ax, eps,
+                                          no_scale != 0, no_bias != 0));
+  });
+  return out;
+}
+
+nnabla_hip_function *nnabla_hip_create_weight_standardization(const char *backends,
+                                                              const char *array_class,
+                                                              const char *device_id,
+                                                              int channel_axis, float eps) {
+  nnabla_hip_function *out = nullptr;
+  guarded([&] {
+    out = wrap(create_WeightStandardization(make_ctx(backends, array_class, device_id),
+                                            channel_axis, eps));
   });
   return out;
 }

@@ -11,6 +11,8 @@
 #include <nbla/hip/function/group_normalization.hpp>
 #include <nbla/hip/function/instance_normalization.hpp>
 #include <nbla/hip/function/layer_normalization.hpp>
+#include <nbla/hip/function/tensor_normalization.hpp>
+#include <nbla/hip/function/weight_standardization.hpp>
 #include <nbla/hip/hip.hpp>
 #include <nbla/hip/init.hpp>
 
@@ -24,6 +26,8 @@ NBLA_REGISTER_FUNCTION_SOURCE(FusedBatchNormalization, const vector<int> &, floa
 NBLA_REGISTER_FUNCTION_SOURCE(LayerNormalization, const vector<int> &, float, bool, bool);
 NBLA_REGISTER_FUNCTION_SOURCE(GroupNormalization, int, int, const vector<int> &, float, bool, bool);
 NBLA_REGISTER_FUNCTION_SOURCE(InstanceNormalization, int, const vector<int> &, float, bool, bool);
+NBLA_REGISTER_FUNCTION_SOURCE(TensorNormalization, const vector<int> &, float, bool, bool);
+NBLA_REGISTER_FUNCTION_SOURCE(WeightStandardization, int, float);
 #endif
 
 void init_hip() {
@@ -96,6 +100,18 @@ void init_hip() {
                               const vector<int> &, float, bool, bool);
   NBLA_REGISTER_FUNCTION_IMPL(InstanceNormalization, InstanceNormalizationHip_half, "hip:half", int,
                               const vector<int> &, float, bool, bool);
+  typedef TensorNormalizationHip<float> TensorNormalizationHip_float;
+  typedef TensorNormalizationHip<Half> TensorNormalizationHip_half;
+  NBLA_REGISTER_FUNCTION_IMPL(TensorNormalization, TensorNormalizationHip_float, "hip:float",
+                              const vector<int> &, float, bool, bool);
+  NBLA_REGISTER_FUNCTION_IMPL(TensorNormalization, TensorNormalizationHip_half, "hip:half",
+                              const vector<int> &, float, bool, bool);
+  typedef WeightStandardizationHip<float> WeightStandardizationHip_float;
+  typedef WeightStandardizationHip<Half> WeightStandardizationHip_half;
+  NBLA_REGISTER_FUNCTION_IMPL(WeightStandardization, WeightStandardizationHip_float, "hip:float",
+                              int, float);
+  NBLA_REGISTER_FUNCTION_IMPL(WeightStandardization, WeightStandardizationHip_half, "hip:half", int,
+                              float);
 
   is_initialized = true;
 }

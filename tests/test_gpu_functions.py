@@ -3,6 +3,7 @@ function tests drive a backend: create by name and context, setup, forward,
 backward with propagate_down/accum flags, compared with the oracle."""
 import numpy as np
 import pytest
+import torch
 
 from _util import assert_close, load_package
 from oracle import norm_ref as R
@@ -466,3 +467,120 @@ def test_caching_allocator_reuses_blocks():
     assert L.nnabla_hip_clear_memory_cache() == 0
     L.nnabla_hip_memory_stats(ctypes.byref(live), ctypes.byref(cached))
     assert cached.value == 0
+
+
+def _tensor_norm_reference(x, dy, g, b, keep, eps, dm=None, dv=None):
+    """float64 torch autograd of y = (x - mean) / sqrt(var + eps) * g + b with
+    statistics over every axis not in `keep` (biased variance)."""
+    red = [i for i in range(x.ndim) if i not in keep]
+    xt = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    gt = None if g is None else torch.tensor(g, dtype=torch.float64, requires_grad=True)
+    bt = None if b is None else torch.tensor(b, dtype=torch.float64, requires_grad=True)
+    m = xt.mean(red, keepdim=True)
+    v = xt.var(red, unbiased=False, keepdim=True)
+    y = (xt - m) / torch.sqrt(v + eps)
+    if gt is not None:
+        y = y * gt
+    if bt is not None:
+        y = y + bt
+    loss = (y * torch.tensor(dy, dtype=torch.float64)).sum()
+    if dm is not None:
+        loss = loss + (m * torch.tensor(dm, dtype=torch.float64)).sum()
+        loss = loss + (v * torch.tensor(dv, dtype=torch.float64)).sum()
+    loss.backward()
+    out = lambda t: None if t is None else t.grad.numpy()
+    return (y.detach().numpy(), m.detach().numpy(), v.detach().numpy(), xt.grad.numpy(), out(gt),
+            out(bt))
+
+
+@pytest.mark.parametrize("tc", CONFIGS)
+@pytest.mark.parametrize("shape,axes", [((4, 6, 5, 8), [1]), ((4, 6, 5, 8), [0, 1]),
+                                        ((4, 6, 5, 8), [3]), ((4, 6, 5, 8), [2, 3]),
+                                        ((4, 6, 5, 8), [1, 2]), ((3, 40, 14, 14), [-3]),
+                                        ((64, 48), [0]), ((2, 3, 4, 5, 6), [1, 2, 3])])
+def test_tensor_normalization(tc, shape, axes):
+    """TensorNormalization over adjacent kept axes against float64 autograd of the
+    defining formula; statistics as outputs with gradients flowing into them."""
+    rng = np.random.default_rng(21)
+    half = tc == "half"
+    keep = sorted(a % len(shape) for a in axes)
+    pshape = tuple(s if i in keep else 1 for i, s in enumerate(shape))
+    x = rnd(rng.standard_normal(shape) * 1.5 + 0.5, tc)
+    dy = rnd(rng.standard_normal(shape), tc)
+    g = rng.uniform(0.5, 1.5, pshape).astype(np.float32)
+    b = (rng.standard_normal(pshape) * 0.1).astype(np.float32)
+    dm = rng.standard_normal(pshape).astype(np.float32)
+    dv = rng.standard_normal(pshape).astype(np.float32)
+    f = B.TensorNormalization(B.context(type_config=tc), axes=axes, eps=1e-5)
+    assert f.name == "TensorNormalizationHip"
+    vx, vb, vg = var(x, half), var(b), var(g)
+    vy, om, ov = B.Variable(shape), B.Variable(()), B.Variable(())
+    f.setup([vx, vb, vg], [vy, om, ov])
+    assert om.current_shape == pshape and ov.current_shape == pshape
+    f.forward([vx, vb, vg], [vy, om, ov])
+    y_r, m_r, v_r, dx_r, dg_r, db_r = _tensor_norm_reference(x, dy, g, b, keep, 1e-5, dm, dv)
+    assert_close(vy.d, y_r, dn(tc), "y", "y")
+    assert_close(om.d, m_r, dn(tc), "stat", "mean")
+    assert_close(ov.d, v_r, dn(tc), "stat", "var")
+    vy.set_grad(dy, half)
+    om.set_grad(dm)
+    ov.set_grad(dv)
+    f.backward([vx, vb, vg], [vy, om, ov], propagate_down=[1, 1, 1], accum=[0, 0, 0])
+    assert_close(vx.g, dx_r, dn(tc), "grad", "dx")
+    assert_close(vg.g, dg_r, dn(tc), "pgrad", "dgamma")
+    assert_close(vb.g, db_r, dn(tc), "pgrad", "dbeta")
+    # one output, no scale / no bias, accumulation onto dx
+    f1 = B.TensorNormalization(B.context(type_config=tc), axes=axes, eps=1e-5, no_scale=True,
+                               no_bias=True)
+    vy1 = B.Variable(shape)
+    f1.setup([vx], [vy1])
+    f1.forward([vx], [vy1])
+    y1, _, _, dx1, _, _ = _tensor_norm_reference(x, dy, None, None, keep, 1e-5)
+    assert_close(vy1.d, y1, dn(tc), "y", "y plain")
+    pre = rnd(rng.standard_normal(shape), tc)
+    vx.set_grad(pre, half)
+    vy1.set_grad(dy, half)
+    f1.backward([vx], [vy1], propagate_down=[1], accum=[1])
+    assert_close(vx.g, dx1 + pre, dn(tc), "grad", "dx accumulated")
+
+
+@pytest.mark.parametrize("tc", CONFIGS)
+@pytest.mark.parametrize("shape,axis", [((16, 8, 3, 3), 0), ((8, 16, 3, 3), 1), ((64, 576), 0),
+                                        ((3, 3, 8, 32), -1)])
+def test_weight_standardization(tc, shape, axis):
+    rng = np.random.default_rng(22)
+    half = tc == "half"
+    keep = [axis % len(shape)]
+    pshape = tuple(s if i in keep else 1 for i, s in enumerate(shape))
+    w = rnd(rng.standard_normal(shape) * 0.2 + 0.05, tc)
+    dy = rnd(rng.standard_normal(shape), tc)
+    f = B.WeightStandardization(B.context(type_config=tc), channel_axis=axis, eps=1e-5)
+    assert f.name == "WeightStandardizationHip"
+    vw, vy = var(w, half), B.Variable(shape)
+    f.setup([vw], [vy])
+    f.forward([vw], [vy])
+    y_r, m_r, v_r, dw_r, _, _ = _tensor_norm_reference(w, dy, None, None, keep, 1e-5)
+    assert_close(vy.d, y_r, dn(tc), "y", "y")
+    vy.set_grad(dy, half)
+    f.backward([vw], [vy], propagate_down=[1], accum=[0])
+    assert_close(vw.g, dw_r, dn(tc), "grad", "dw")
+    # statistics as outputs
+    om, ov = B.Variable(()), B.Variable(())
+    f.setup([vw], [vy, om, ov])
+    f.forward([vw], [vy, om, ov])
+    assert om.current_shape == pshape
+    assert_close(om.d, m_r, dn(tc), "stat", "mean")
+    assert_close(ov.d, v_r, dn(tc), "stat", "var")
+
+
+def test_tensor_normalization_argument_errors():
+    ctx = B.context(type_config="float")
+    x, y = B.Variable((4, 6, 5, 8)), B.Variable((4, 6, 5, 8))
+    with pytest.raises(RuntimeError, match="adjacent"):
+        B.TensorNormalization(ctx, axes=[0, 2], no_scale=True, no_bias=True).setup([x], [y])
+    with pytest.raises(RuntimeError, match="out of range"):
+        B.TensorNormalization(ctx, axes=[4], no_scale=True, no_bias=True).setup([x], [y])
+    with pytest.raises(RuntimeError, match="elements"):
+        B.TensorNormalization(ctx, axes=[1], no_scale=True).setup([x, B.Variable((1, 5, 1, 1))], [y])
+    with pytest.raises(RuntimeError, match="out of range"):
+        B.WeightStandardization(ctx, channel_axis=7).setup([x], [y])

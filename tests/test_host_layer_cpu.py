@@ -60,9 +60,12 @@ def test_registry_selects_by_context_and_has_no_cpu_implementation():
     assert B.GroupNormalization(B.context(type_config="float"), num_groups=2).name == "GroupNormalizationHip"
     assert B.InstanceNormalization(B.context(type_config="half")).name == "InstanceNormalizationHip"
     assert B.FusedBatchNormalization(B.context(type_config="half")).name == "FusedBatchNormalizationHip"
+    assert B.TensorNormalization(B.context(type_config="float")).name == "TensorNormalizationHip"
+    assert B.WeightStandardization(B.context(type_config="half")).name == "WeightStandardizationHip"
     cpu_only = {"backends": "cpu:float", "array_class": "CpuArray", "device_id": "0"}
     for make in (B.BatchNormalization, B.LayerNormalization, B.GroupNormalization,
-                 B.InstanceNormalization, B.FusedBatchNormalization):
+                 B.InstanceNormalization, B.FusedBatchNormalization, B.TensorNormalization,
+                 B.WeightStandardization):
         with pytest.raises(B.NblaError, match="No implementation"):
             make(cpu_only)
 
