@@ -71,14 +71,15 @@ struct RowArgs {
   float decay, unbias;
 };
 
-// Offset of element col of a row from the row's first element.
+// Offset of element col of a row from the row's first element.  32 bits (a
+// tensor has fewer than 2^31 elements): the row base stays a wave-uniform
+// 64-bit value and the per-lane part of every address one register.
 template <bool STRIDED>
-__device__ __forceinline__ size_t row_elem_offset(const RowArgs &a, int col) {
+__device__ __forceinline__ uint32_t row_elem_offset(const RowArgs &a, int col) {
   if constexpr (STRIDED) {
-    return static_cast<size_t>(col) +
-           static_cast<size_t>(a.plane.div(static_cast<uint32_t>(col))) * a.plane_jump;
+    return static_cast<uint32_t>(col) + a.plane.div(static_cast<uint32_t>(col)) * a.plane_jump;
   } else {
-    return static_cast<size_t>(col);
+    return static_cast<uint32_t>(col);
   }
 }
 
@@ -377,9 +378,9 @@ row_bwd_kernel(const RowArgs a) {
         ok = sl.ok;
       }
       // branch-free: all loads in flight together
-      const size_t off = base + row_elem_offset<BN>(a, ok ? col : 0);
-      xr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + off));
-      dr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(dy + off));
+      const uint32_t off = row_elem_offset<BN>(a, ok ? col : 0);
+      xr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + base + off));
+      dr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(dy + base + off));
     }
     const float mean = a.mean[row];
     const float vpe = a.var[row] + a.eps;
