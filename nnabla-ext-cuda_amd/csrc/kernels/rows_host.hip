@@ -438,7 +438,9 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
     // The float 1024 x 8 layout (one block per CU, 128 KB of row data in its
     // registers) loses to the streaming kernels: 92-105 vs 85 us on
     // 25 088-element groups, 55 vs 56 us on 32 768-element ones.
-    if (cfg.ok && p.dtype == NBLAHIP_F32 && cfg.tpr == 1024 && cfg.nl == 8) cfg.ok = false;
+    if (cfg.ok && p.dtype == NBLAHIP_F32 && cfg.vec == 4 && cfg.tpr == 1024 && cfg.nl == 8 &&
+        !tune_int("GN_FLOAT_1024X8", 0))
+      cfg.ok = false;
   }
   if (cfg.ok && !tune_int("FORCE_STREAM", 0)) {
     if (p.mode == kRowLN) {
