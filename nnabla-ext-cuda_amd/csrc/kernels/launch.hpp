@@ -18,7 +18,18 @@ namespace nblahip {
 // that are no multiple of a wave-wide load); kRowGN is the fixed map.
 // kRowBN: BatchNormalization of tensors whose channel (all its planes) fits a
 // block's registers: a row is the strided set of planes of one channel.
-enum RowMode { kRowLN = 0, kRowIN = 1, kRowGN = 2, kRowINc = 3, kRowGNm = 4, kRowBN = 5 };
+// kRowLNx: LayerNormalization backward of rows too long for the per-column
+// accumulators of kRowLN: dx only (gamma read per row), the column gradients
+// come from the streaming kernel.
+enum RowMode {
+  kRowLN = 0,
+  kRowIN = 1,
+  kRowGN = 2,
+  kRowINc = 3,
+  kRowGNm = 4,
+  kRowBN = 5,
+  kRowLNx = 6
+};
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

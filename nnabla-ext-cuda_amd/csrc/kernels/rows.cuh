@@ -407,6 +407,26 @@ row_bwd_kernel(const RowArgs a) {
         }
       }
       row_sum2<TPR>(s1, t2, lds);
+    } else if constexpr (MODE == kRowLNx) {
+#pragma unroll
+      for (int k = 0; k < NL; ++k) {
+        const int col = (k * TPR + t) * VEC;
+        float gv[VEC];
+        if (col < a.R && a.gamma) {
+          load_param_vec<VEC>(a.gamma + col, gv);
+        } else {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) gv[j] = 1.f;
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+          const float dg = elem_fma<T, VEC>(dr[k], j, gv[j], 0.f);
+          s1 += dg;
+          t2 = fmaf(dg, xh, t2);
+        }
+      }
+      row_sum2<TPR>(s1, t2, lds);
     } else if constexpr (MODE == kRowIN || MODE == kRowINc || BN) {
       float sdy = 0.f, sdx = 0.f;
 #pragma unroll
@@ -521,6 +541,19 @@ row_bwd_kernel(const RowArgs a) {
             for (int j = 0; j < VEC; ++j) {
               const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
               o[j] = elem_fma<T, VEC>(dr[k], j, gcol[k][j] * istd, fmaf(xh, cA, cb));
+            }
+          } else if constexpr (MODE == kRowLNx) {
+            float gv[VEC]; // read again rather than kept: NL*VEC registers otherwise
+            if (a.gamma) {
+              load_param_vec<VEC>(a.gamma + col, gv);
+            } else {
+#pragma unroll
+              for (int j = 0; j < VEC; ++j) gv[j] = 1.f;
+            }
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+              const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+              o[j] = elem_fma<T, VEC>(dr[k], j, gv[j] * istd, fmaf(xh, cA, cb));
             }
           } else {
             const float gi = gk[k] * istd;

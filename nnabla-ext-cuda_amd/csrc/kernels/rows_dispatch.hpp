@@ -25,6 +25,8 @@ int run_row_fwd_cached_bn(int dtype, const RowCfg &cfg, const RowArgs &args, int
                           hipStream_t st);
 int run_row_bwd_cached_bn(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
                           hipStream_t st);
+int run_row_bwd_cached_lnx(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
+                           hipStream_t st);
 int run_row_bwd_cached_gnm(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
                            hipStream_t st);
 

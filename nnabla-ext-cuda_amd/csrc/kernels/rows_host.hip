@@ -282,8 +282,10 @@ int launch_row_fwd(const RowProblem &p, hipStream_t st) {
 
 // Row chunks of the streaming LayerNormalization column gradients: enough
 // (strip, chunk) blocks for 8 per CU, at least 64 rows per chunk.
-static int ln_stream_chunks(int64_t rows, int64_t R) {
-  const int64_t strips = (R + 63) / 64;
+static int ln_stream_chunks(int64_t rows, int64_t R, int vec = 8) {
+  // (the default is the widest strip: the fewest strips, hence the most
+  // chunks - the bound the workspace is sized for)
+  const int64_t strips = (R + 64 * vec - 1) / (64 * vec);
   const int64_t want = (8 * static_cast<int64_t>(device_cus()) + strips - 1) / strips;
   const int64_t most = std::max<int64_t>(1, rows / 64);
   return static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(std::min(want, most), 65535)));
@@ -316,6 +318,35 @@ size_t row_bwd_workspace_bytes(int mode, int64_t rows, int64_t R, int64_t planes
          align_up(static_cast<size_t>(rows) * 2 * sizeof(float), 256) + align_up(split, 256);
 }
 
+// LayerNormalization dgamma/dbeta by the streaming kernel: column partials over
+// row chunks (kept after the row sums in the workspace), then their fold.
+template <typename T, int VEC>
+static int stream_ln_colgrad_t(const RowProblem &p, const RowArgs &a, hipStream_t st) {
+  float *part = reinterpret_cast<float *>(
+      static_cast<char *>(p.ws) + align_up(static_cast<size_t>(p.rows) * 2 * sizeof(float), 256));
+  const int Y = ln_stream_chunks(p.rows, p.R, VEC);
+  const int rpc = static_cast<int>((p.rows + Y - 1) / Y);
+  NBLAHIP_LAUNCH("ln_colgrad_stream_kernel", (ln_colgrad_stream_kernel<T, VEC>),
+                 dim3((a.R + 64 * VEC - 1) / (64 * VEC), Y), dim3(256), 0, st,
+                 static_cast<const T *>(p.x), static_cast<const T *>(p.dy), p.mean, p.var, a.rows,
+                 a.R, rpc, p.eps, part);
+  if (int e = last_launch_status()) return e;
+  NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 31) / 32),
+                 dim3(1024), 0, st, part, Y, a.R, p.dgamma, p.dbeta, p.accum_g, p.accum_b);
+  return last_launch_status();
+}
+
+// vec: the row kernels' vector width for this problem (x and dy aligned, R a
+// multiple of it).
+static int stream_ln_colgrad(const RowProblem &p, const RowArgs &a, int vec, hipStream_t st) {
+  if (p.dtype == NBLAHIP_F16) {
+    return vec == 8   ? stream_ln_colgrad_t<__half, 8>(p, a, st)
+           : vec == 4 ? stream_ln_colgrad_t<__half, 4>(p, a, st)
+                      : stream_ln_colgrad_t<__half, 1>(p, a, st);
+  }
+  return vec == 4 ? stream_ln_colgrad_t<float, 4>(p, a, st) : stream_ln_colgrad_t<float, 1>(p, a, st);
+}
+
 template <typename T, int VEC>
 static int stream_bwd_t(const RowProblem &p, const RowArgs &a, hipStream_t st) {
   const T *x = static_cast<const T *>(p.x);
@@ -345,20 +376,7 @@ static int stream_bwd_t(const RowProblem &p, const RowArgs &a, hipStream_t st) {
                          dim3(256), 0, st, a, rs, nvr, total_vec);
       if (int e = last_launch_status()) return e;
     }
-    if (p.dgamma || p.dbeta) {
-      // Column partials over row chunks, after the row sums in the workspace.
-      float *part = reinterpret_cast<float *>(
-          static_cast<char *>(p.ws) + align_up(static_cast<size_t>(p.rows) * 2 * sizeof(float), 256));
-      const int Y = ln_stream_chunks(p.rows, p.R);
-      const int rpc = static_cast<int>((p.rows + Y - 1) / Y);
-      NBLAHIP_LAUNCH("ln_colgrad_stream_kernel", (ln_colgrad_stream_kernel<T>),
-                     dim3((a.R + 63) / 64, Y), dim3(256), 0, st, x, dy, p.mean, p.var, a.rows, a.R,
-                     rpc, p.eps, part);
-      if (int e = last_launch_status()) return e;
-      NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 31) / 32),
-                     dim3(1024), 0, st, part, Y, a.R, p.dgamma, p.dbeta, p.accum_g, p.accum_b);
-      if (int e = last_launch_status()) return e;
-    }
+    if (p.dgamma || p.dbeta) return stream_ln_colgrad(p, a, VEC, st);
     return 0;
   }
   const int64_t planes = p.batch * p.channels;
@@ -475,6 +493,23 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
                                    : run_row_bwd_cached_gn(p.dtype, cfg, a, grid, st);
     if (e) return e;
     return launch_pair_reduce(p, static_cast<const float *>(p.ws), st);
+  }
+  if (p.mode == kRowLN && !tune_int("FORCE_STREAM", 0) && tune_int("LN_LONG_ROWS_CACHED", 1)) {
+    // Rows too long for the per-column accumulators but not for a block's
+    // registers: dx in one pass over x and dy (3 S), the column gradients by
+    // the streaming kernel (2 S) - 5 S instead of the 7 S of the all-streaming
+    // sequence below.
+    // (Not the 1024 x 8 layouts with vectors: 128 KB of row data in one
+    // block's registers, 210-256 us against 160-167 us streamed in float,
+    // 96 against about 60 us in half.)
+    const RowCfg lx = pick_row_cfg(vec, p.R, 8, vec > 1 ? 4 : 8, 256, true);
+    if (lx.ok) {
+      if (p.out) {
+        if (int e = run_row_bwd_cached_lnx(p.dtype, lx, a, cached_grid(p.rows, lx.tpr), st)) return e;
+      }
+      if (p.dgamma || p.dbeta) return stream_ln_colgrad(p, a, vec, st);
+      return 0;
+    }
   }
   int e;
   if (p.dtype == NBLAHIP_F16) {

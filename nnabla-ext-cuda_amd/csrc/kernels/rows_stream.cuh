@@ -98,12 +98,23 @@ row_apply_fwd_kernel(const RowArgs a, FastDiv nvr, uint32_t total_vec) {
     float v[VEC], o[VEC];
     load_vec<T, VEC>(x + static_cast<size_t>(i) * VEC, v);
     if (a.percol) {
+      // gamma/beta of VEC columns in one or two 16-byte loads each (vectors
+      // are only used when the parameter pointers are aligned)
+      float gv[VEC], bv[VEC];
+      if (a.gamma) {
+        load_param_vec<VEC>(a.gamma + col, gv);
+      } else {
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const float g = a.gamma ? a.gamma[col + j] : 1.f;
-        const float b = a.beta ? a.beta[col + j] : 0.f;
-        o[j] = (v[j] - mean) * (g * istd) + b;
+        for (int j = 0; j < VEC; ++j) gv[j] = 1.f;
       }
+      if (a.beta) {
+        load_param_vec<VEC>(a.beta + col, bv);
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) bv[j] = 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) o[j] = (v[j] - mean) * (gv[j] * istd) + bv[j];
     } else {
       // VEC divides the parameter run length, so one index serves the vector.
       const uint32_t poff = a.pdiv.div(col);
@@ -262,11 +273,15 @@ row_bwd_dx_kernel(const RowArgs a, const float *__restrict__ rs, FastDiv nvr,
     load_vec<T, VEC>(x + static_cast<size_t>(i) * VEC, xv);
     load_vec<T, VEC>(dy + static_cast<size_t>(i) * VEC, dv);
     if (a.percol) {
+      float gv[VEC];
+      if (a.gamma) {
+        load_param_vec<VEC>(a.gamma + col, gv);
+      } else {
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const float g = a.gamma ? a.gamma[col + j] : 1.f;
-        o[j] = dv[j] * g * istd + ca * (xv[j] - mean) + cb;
+        for (int j = 0; j < VEC; ++j) gv[j] = 1.f;
       }
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) o[j] = dv[j] * gv[j] * istd + ca * (xv[j] - mean) + cb;
     } else {
       const uint32_t pidx = (row % a.pmod) * a.pmul + a.pdiv.div(col);
       const float gi = (a.gamma ? a.gamma[pidx] : 1.f) * istd;
@@ -283,53 +298,69 @@ row_bwd_dx_kernel(const RowArgs a, const float *__restrict__ rs, FastDiv nvr,
   }
 }
 
-// LayerNormalization dgamma/dbeta partials, any shape.  grid = (ceil(R/64), Y):
-// a block owns a 64-column strip (one wave-wide, fully coalesced access per
-// row) and the rows [y*rpc, (y+1)*rpc); its 4 waves take every 4th row, 4 rows
-// in flight each.  part[y][0][R] = sum dy*(x-mean)*istd, part[y][1][R] = sum dy;
+// LayerNormalization dgamma/dbeta partials, any shape.  grid = (ceil(R/(64*VEC)), Y):
+// a block owns a strip of 64*VEC columns (a lane VEC adjacent ones: one
+// wave-wide, fully coalesced access per row) and the rows [y*rpc, (y+1)*rpc);
+// its 4 waves take every 4th row, 4 rows in flight each.
+// part[y][0][R] = sum dy*(x-mean)*istd, part[y][1][R] = sum dy;
 // ln_param_reduce_kernel folds the Y partials.
-template <typename T>
+template <typename T, int VEC>
 __global__ void __launch_bounds__(256)
 ln_colgrad_stream_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                          const float *__restrict__ mean, const float *__restrict__ var,
                          int rows, int R, int rpc, float eps, float *__restrict__ part) {
-  __shared__ float rg[4][64];
-  __shared__ float rb[4][64];
+  __shared__ float rg[4][64 * VEC];
+  __shared__ float rb[4][64 * VEC];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int col = blockIdx.x * 64 + lane;
-  const int colc = col < R ? col : R - 1; // clamped: loads stay unconditional
+  const int col = (blockIdx.x * 64 + lane) * VEC;
+  const int colc = col < R ? col : R - VEC; // clamped: loads stay unconditional
   const int rbegin = blockIdx.y * rpc;
   const int rend = min(rbegin + rpc, rows);
-  float sg = 0.f, sb = 0.f;
+  float sg[VEC], sb[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) sg[j] = sb[j] = 0.f;
   for (int r0 = rbegin + wave; r0 < rend; r0 += 16) {
-    float xv[4], dv[4], mu[4], is[4];
+    RawVec<T, VEC> xv[4], dv[4];
+    float mu[4], is[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int r = r0 + 4 * u;
       const int rc = r < rend ? r : r0;
       const size_t i = static_cast<size_t>(rc) * R + colc;
-      xv[u] = to_f32<T>(x[i]);
-      dv[u] = to_f32<T>(dy[i]);
+      xv[u] = load_raw<T, VEC>(x + i);
+      dv[u] = raw_or_zero<T, VEC>(r < rend, load_raw<T, VEC>(dy + i));
       mu[u] = mean[rc];
       is[u] = var[rc];
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const float d = (r0 + 4 * u < rend) ? dv[u] : 0.f;
-      sg += d * (xv[u] - mu[u]) * inv_std(is[u], eps);
-      sb += d;
+      const float istd = inv_std(is[u], eps);
+      const float nmi = -mu[u] * istd;
+      float xf[VEC], df[VEC];
+      unpack<T, VEC>(xv[u], xf);
+      unpack<T, VEC>(dv[u], df);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        sg[j] = fmaf(df[j], fmaf(xf[j], istd, nmi), sg[j]);
+        sb[j] += df[j];
+      }
     }
   }
-  rg[wave][lane] = sg;
-  rb[wave][lane] = sb;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    rg[wave][lane * VEC + j] = sg[j];
+    rb[wave][lane * VEC + j] = sb[j];
+  }
   lds_barrier();
   if (wave == 0 && col < R) {
-    const float tg = (rg[0][lane] + rg[1][lane]) + (rg[2][lane] + rg[3][lane]);
-    const float tb = (rb[0][lane] + rb[1][lane]) + (rb[2][lane] + rb[3][lane]);
     float *p = part + static_cast<size_t>(blockIdx.y) * 2 * R;
-    p[col] = tg;
-    p[R + col] = tb;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const int l = lane * VEC + j;
+      p[col + j] = (rg[0][l] + rg[1][l]) + (rg[2][l] + rg[3][l]);
+      p[R + col + j] = (rb[0][l] + rb[1][l]) + (rb[2][l] + rb[3][l]);
+    }
   }
 }
 
