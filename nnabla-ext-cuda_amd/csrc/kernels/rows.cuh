@@ -154,7 +154,8 @@ template <typename T, int VEC, int NL, int TPR, int MODE> struct RowBwdOccupancy
 // STRIDED: BatchNormalization rows (see RowArgs::plane); also updates the
 // running statistics.
 template <typename T, int VEC, int NL, int TPR, bool PERCOL, bool STRIDED = false>
-__global__ void __launch_bounds__(RowBlock<TPR>::kBlock)
+__global__ void __launch_bounds__(RowBlock<TPR>::kBlock,
+                                  ((PERCOL && TPR == 1024 && NL <= 4) ? 8 : 1))
 row_fwd_kernel(const RowArgs a) {
   constexpr int RPB = RowBlock<TPR>::kRowsPerBlock;
   __shared__ float lds[2 * 16];
@@ -163,8 +164,12 @@ row_fwd_kernel(const RowArgs a) {
   const T *__restrict__ x = static_cast<const T *>(a.x);
   T *__restrict__ y = static_cast<T *>(a.out);
 
-  float gcol[PERCOL ? NL : 1][VEC], bcol[PERCOL ? NL : 1][VEC];
-  if constexpr (PERCOL) {
+  // 1024-thread blocks (rows of thousands of vectors, one row per block): the
+  // parameters are fetched where they are used instead, which keeps the kernel
+  // at 64 VGPRs and two blocks per CU.
+  constexpr bool LATE = PERCOL && TPR == 1024;
+  float gcol[(PERCOL && !LATE) ? NL : 1][VEC], bcol[(PERCOL && !LATE) ? NL : 1][VEC];
+  if constexpr (PERCOL && !LATE) {
 #pragma unroll
     for (int k = 0; k < NL; ++k) {
       const int col = (k * TPR + t) * VEC;
@@ -245,7 +250,24 @@ row_fwd_kernel(const RowArgs a) {
       const int col = (k * TPR + t) * VEC;
       if (col < a.R) {
         float o[VEC];
-        if constexpr (PERCOL) {
+        if constexpr (LATE) {
+          float gv[VEC], bv[VEC];
+          if (a.gamma) {
+            load_param_vec<VEC>(a.gamma + col, gv);
+          } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) gv[j] = 1.f;
+          }
+          if (a.beta) {
+            load_param_vec<VEC>(a.beta + col, bv);
+          } else {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) bv[j] = 0.f;
+          }
+#pragma unroll
+          for (int j = 0; j < VEC; ++j)
+            o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mean), gv[j] * istd, bv[j]);
+        } else if constexpr (PERCOL) {
 #pragma unroll
           for (int j = 0; j < VEC; ++j)
             o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mean), gcol[k][j] * istd, bcol[k][j]);
