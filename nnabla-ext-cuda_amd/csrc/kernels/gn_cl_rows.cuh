@@ -223,13 +223,13 @@ gn_cl_row_bwd_kernel(const GnClArgs a) {
     }
   }
   lds_barrier();
-  if (static_cast<int>(threadIdx.x) < 2 * a.cpg) {
+  for (int e = threadIdx.x; e < 2 * a.cpg; e += TPR) { // up to 128 entries, 64 threads and more
     float t = 0.f;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) t += fold[w][threadIdx.x];
-    chs[threadIdx.x] = t;
+    for (int w = 0; w < NW; ++w) t += fold[w][e];
+    chs[e] = t;
     // entry 2*c of the group is (sum dy*xh) of its channel c, 2*c+1 (sum dy)
-    a.pairs[2 * (static_cast<size_t>(n) * a.C + g * a.cpg) + threadIdx.x] = t;
+    a.pairs[2 * (static_cast<size_t>(n) * a.C + g * a.cpg) + e] = t;
   }
   lds_barrier();
   float s1 = 0.f, t2 = 0.f;
@@ -255,6 +255,221 @@ gn_cl_row_bwd_kernel(const GnClArgs a) {
       for (int j = 0; j < VEC; ++j) {
         const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
         o[j] = elem_fma<T, VEC>(dr[k], j, gam[j] * istd, fmaf(xh, cA, cb));
+      }
+      T *p = dx + static_cast<size_t>(pos) * a.C;
+      if (a.accum_dx) {
+        float old[VEC];
+        load_vec<T, VEC>(p, old);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) o[j] += old[j];
+      }
+      store_vec<T, VEC>(p, o);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Channel-last InstanceNormalization with the instances cached in registers.
+// A block owns sample n and one channel vector (VEC adjacent channels, i.e.
+// VEC instances): thread t holds positions t + k*TPR, its vector element j
+// always belongs to channel ch + j, so the statistics are VEC sums per thread,
+// folded over the block (wave sums, then LDS).  GnClArgs as above with
+// G = C / VEC "groups", cpg = VEC, cvg = 1; mean/var/dmean/dvar are indexed
+// n*C + channel.  The block order shares cache lines between neighbouring
+// channel vectors exactly as for the groups.
+// ---------------------------------------------------------------------------
+template <int TPR, int VEC>
+__device__ __forceinline__ void in_cl_block_sums(float (&v)[VEC], float (*lds)[VEC]) {
+  constexpr int NW = TPR / kWave;
+  const int wave = threadIdx.x / kWave;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) v[j] = wave_sum(v[j]);
+  lds_barrier(); // previous readers of lds are done
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) lds[wave][j] = v[j];
+  }
+  lds_barrier();
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    float t = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) t += lds[w][j];
+    v[j] = t;
+  }
+}
+
+template <typename T, int VEC, int NL, int TPR>
+__global__ void __launch_bounds__(TPR)
+in_cl_row_fwd_kernel(const GnClArgs a) {
+  __shared__ float lds[TPR / kWave][VEC];
+  const int unit = gn_cl_unit(a);
+  if (unit < 0) return;
+  const uint32_t n = static_cast<uint32_t>(unit) / a.G, cv = static_cast<uint32_t>(unit) % a.G;
+  const uint32_t ch = cv * VEC;
+  const T *__restrict__ x = static_cast<const T *>(a.x) + static_cast<size_t>(n) * a.P * a.C + ch;
+  T *__restrict__ y = static_cast<T *>(a.out) + static_cast<size_t>(n) * a.P * a.C + ch;
+
+  RawVec<T, VEC> raw[NL];
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = threadIdx.x + k * TPR;
+    const bool ok = pos < static_cast<uint32_t>(a.P);
+    raw[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + static_cast<size_t>(ok ? pos : 0u) * a.C));
+  }
+  float gam[VEC], bet[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    gam[j] = a.gamma ? a.gamma[ch + j] : 1.f;
+    bet[j] = a.beta ? a.beta[ch + j] : 0.f;
+  }
+  float mean[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) mean[j] = 0.f;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) mean[j] = elem_fma<T, VEC>(raw[k], j, a.one, mean[j]);
+  }
+  in_cl_block_sums<TPR, VEC>(mean, lds);
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) mean[j] *= a.inv_R;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+  float var[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) var[j] = 0.f;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    if (threadIdx.x + k * TPR < static_cast<uint32_t>(a.P)) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float d = elem_fma<T, VEC>(raw[k], j, a.one, -mean[j]);
+        var[j] = fmaf(d, d, var[j]);
+      }
+    }
+  }
+  in_cl_block_sums<TPR, VEC>(var, lds);
+  float sc[VEC], sh[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    var[j] *= a.inv_R;
+    sc[j] = gam[j] * inv_std(var[j], a.eps);
+    sh[j] = fmaf(-mean[j], sc[j], bet[j]);
+  }
+  if (threadIdx.x < VEC) {
+    // lane j publishes channel j (every lane holds all VEC values)
+    float m = mean[0], v = var[0];
+#pragma unroll
+    for (int j = 1; j < VEC; ++j) {
+      m = threadIdx.x == j ? mean[j] : m;
+      v = threadIdx.x == j ? var[j] : v;
+    }
+    a.mean[static_cast<size_t>(n) * a.C + ch + threadIdx.x] = m;
+    a.var[static_cast<size_t>(n) * a.C + ch + threadIdx.x] = v;
+  }
+#pragma unroll
+  for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = threadIdx.x + k * TPR;
+    if (pos < static_cast<uint32_t>(a.P)) {
+      float o[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        if constexpr (sizeof(T) == 2) {
+          o[j] = elem_fma<T, VEC>(raw[k], j, sc[j], sh[j]);
+        } else {
+          o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mean[j]), sc[j], bet[j]);
+        }
+      }
+      store_vec<T, VEC>(y + static_cast<size_t>(pos) * a.C, o);
+    }
+  }
+}
+
+// Backward, per channel c of the block: sdx = sum dy*xh, sdy = sum dy (also the
+// pair behind dgamma/dbeta), dx = g*istd*dy + cA*xh + cb with
+// cA = -istd*g*sdx/P + 2*dvar*std/P, cb = -g*sdy*istd/P + dmean/P.
+template <typename T, int VEC, int NL, int TPR>
+__global__ void __launch_bounds__(TPR, (TPR == 512 ? 4 : 1))
+in_cl_row_bwd_kernel(const GnClArgs a) {
+  __shared__ float lds[TPR / kWave][VEC];
+  const int unit = gn_cl_unit(a);
+  if (unit < 0) return;
+  const uint32_t n = static_cast<uint32_t>(unit) / a.G, cv = static_cast<uint32_t>(unit) % a.G;
+  const uint32_t ch = cv * VEC;
+  const size_t slab = static_cast<size_t>(n) * a.P * a.C + ch;
+  const size_t stat = static_cast<size_t>(n) * a.C + ch;
+  const T *__restrict__ x = static_cast<const T *>(a.x) + slab;
+  const T *__restrict__ dy = static_cast<const T *>(a.dy) + slab;
+  T *__restrict__ dx = a.out ? static_cast<T *>(a.out) + slab : nullptr;
+
+  RawVec<T, VEC> xr[NL], dr[NL];
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = threadIdx.x + k * TPR;
+    const bool ok = pos < static_cast<uint32_t>(a.P);
+    const size_t off = static_cast<size_t>(ok ? pos : 0u) * a.C;
+    xr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + off));
+    dr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(dy + off));
+  }
+  float istd[VEC], nmi[VEC], mean[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    mean[j] = a.mean[stat + j];
+    istd[j] = 1.0f / sqrtf(a.var[stat + j] + a.eps);
+    nmi[j] = -mean[j] * istd[j];
+  }
+  float sdx[VEC], sdy[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) sdx[j] = sdy[j] = 0.f;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float xh = norm_elem<T, VEC>(xr[k], j, mean[j], istd[j], nmi[j]);
+      sdx[j] = elem_fma<T, VEC>(dr[k], j, xh, sdx[j]);
+      sdy[j] = elem_fma<T, VEC>(dr[k], j, a.one, sdy[j]);
+    }
+  }
+  in_cl_block_sums<TPR, VEC>(sdx, lds);
+  in_cl_block_sums<TPR, VEC>(sdy, lds);
+  if (threadIdx.x < VEC) {
+    float px = sdx[0], py = sdy[0];
+#pragma unroll
+    for (int j = 1; j < VEC; ++j) {
+      px = threadIdx.x == j ? sdx[j] : px;
+      py = threadIdx.x == j ? sdy[j] : py;
+    }
+    a.pairs[2 * (stat + threadIdx.x)] = px;
+    a.pairs[2 * (stat + threadIdx.x) + 1] = py;
+  }
+  if (dx == nullptr) return;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    keep_packed<T, VEC>(xr[k]);
+    keep_packed<T, VEC>(dr[k]);
+  }
+  float gi[VEC], cA[VEC], cb[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    const float g = a.gamma ? a.gamma[ch + j] : 1.f;
+    const float vpe = a.var[stat + j] + a.eps;
+    gi[j] = g * istd[j];
+    cA[j] = -istd[j] * g * sdx[j] * a.inv_R +
+            (a.dvar ? 2.f * a.dvar[stat + j] * (vpe * istd[j]) * a.inv_R : 0.f);
+    cb[j] = -g * sdy[j] * istd[j] * a.inv_R + (a.dmean ? a.dmean[stat + j] * a.inv_R : 0.f);
+  }
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = threadIdx.x + k * TPR;
+    if (pos < static_cast<uint32_t>(a.P)) {
+      float o[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float xh = norm_elem<T, VEC>(xr[k], j, mean[j], istd[j], nmi[j]);
+        o[j] = elem_fma<T, VEC>(dr[k], j, gi[j], fmaf(xh, cA[j], cb[j]));
       }
       T *p = dx + static_cast<size_t>(pos) * a.C;
       if (a.accum_dx) {

@@ -26,15 +26,17 @@ GnClCfg pick_cfg(const ClProblem &p, bool aligned, bool backward, GnClArgs &a) {
   const int64_t cvg = cpg / vec;
   if (cvg != 1 && cvg != 2 && cvg != 4 && cvg != 8) return c;
   const int64_t nv = p.spatial * cvg;
-  if (nv < 256) return c;
+  if (nv < 32) return c;
   // Backward, beyond 2048 vectors per group the three-kernel path is as fast
   // or faster (64 KB half groups: 41.9 vs 42.4 us; 50 KB ones: 56.1 vs 52.6 us),
   // the strided 16-byte accesses of two tensors being the limit; below it the
   // single pass wins clearly (28x28 planes: 24 vs 39 us).
   if (backward && nv > 2048) return c;
-  for (int tpr : {256, 512, 1024}) {
+  // small groups: one wave per group (no LDS, no barrier), at most 4 loads
+  for (int tpr : {64, 256, 512, 1024}) {
     for (int nl : {1, 2, 4, 8}) {
       if (static_cast<int64_t>(tpr) * nl < nv) continue;
+      if (tpr == 64 && nl > 4) continue;
       // the float 1024 x 8 layout (128 KB of x and dy in one block's registers)
       // is left to the three-kernel path
       if (p.dtype == NBLAHIP_F32 && tpr == 1024 && nl == 8) continue;
@@ -63,6 +65,49 @@ GnClCfg pick_cfg(const ClProblem &p, bool aligned, bool backward, GnClArgs &a) {
   return c;
 }
 
+// InstanceNormalization: a block per (sample, channel vector); P positions of
+// one vector each.
+GnClCfg pick_in_cfg(const ClProblem &p, bool aligned, bool backward, GnClArgs &a) {
+  GnClCfg c;
+  if (!aligned || !tune_int("IN_CL_CACHED", 1)) return c;
+  if (!p.bc_gamma || !p.bc_beta) return c;
+  const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
+  if (p.channels % vec != 0) return c;
+  const int64_t nv = p.spatial;
+  if (nv < tune_int("IN_CL_MIN", 32)) return c;
+  // Beyond 2048 positions the three-kernel path is as fast or faster in float
+  // and in the backward pass (64x64 planes, half: backward 49 vs 44 us; 56x56
+  // float: 62 / 130 vs 57 / 92 us); below, the single pass wins by 1.3-2x.
+  if ((backward || p.dtype == NBLAHIP_F32) && nv > 2048) return c;
+  for (int tpr : {64, 256, 512, 1024}) {
+    for (int nl : {1, 2, 4, 8}) {
+      if (static_cast<int64_t>(tpr) * nl < nv) continue;
+      if (tpr == 64 && nl > 4) continue; // one wave per unit: at most 4 loads
+      if (p.dtype == NBLAHIP_F32 && tpr == 1024 && nl == 8) continue;
+      c.ok = true;
+      c.vec = vec;
+      c.tpr = tpr;
+      c.nl = nl;
+      break;
+    }
+    if (c.ok) break;
+  }
+  if (!c.ok) return c;
+  a.P = static_cast<int>(p.spatial);
+  a.C = static_cast<int>(p.channels);
+  a.G = static_cast<int>(p.channels / vec);
+  a.cpg = vec;
+  a.units = static_cast<int>(p.batch * a.G);
+  a.cvg = FastDiv(1);
+  const int gpl = 128 / (vec * (p.dtype == NBLAHIP_F16 ? 2 : 4)); // vectors per 128-byte line
+  a.gpl = (a.G % gpl == 0 && tune_int("GN_CL_XCD_MAP", 1)) ? gpl : 1;
+  a.eps = p.eps;
+  a.inv_R = static_cast<float>(1.0 / static_cast<double>(p.spatial));
+  a.one = 1.0f;
+  a.accum_dx = p.accum_dx;
+  return c;
+}
+
 unsigned grid_of(const GnClArgs &a) {
   if (a.gpl <= 1) return static_cast<unsigned>(a.units);
   const unsigned sets = static_cast<unsigned>(a.units / a.gpl);
@@ -73,6 +118,8 @@ unsigned grid_of(const GnClArgs &a) {
   CASE(T, VEC, 1, TPR) CASE(T, VEC, 2, TPR) CASE(T, VEC, 4, TPR) CASE(T, VEC, 8, TPR)
 #define GN_CL_CASES(CASE, T, VEC) \
   GN_CL_CASES_TPR(CASE, T, VEC, 256) GN_CL_CASES_TPR(CASE, T, VEC, 512) GN_CL_CASES_TPR(CASE, T, VEC, 1024)
+// ... and one wave per unit (small planes or groups).
+#define IN_CL_CASES(CASE, T, VEC) GN_CL_CASES_TPR(CASE, T, VEC, 64) GN_CL_CASES(CASE, T, VEC)
 
 #define FWD_CASE(T, VEC, NL, TPR)                                                              \
   if (c.nl == (NL) && c.tpr == (TPR)) {                                                        \
@@ -87,20 +134,51 @@ unsigned grid_of(const GnClArgs &a) {
     return last_launch_status();                                                               \
   }
 
+#define IN_FWD_CASE(T, VEC, NL, TPR)                                                           \
+  if (c.nl == (NL) && c.tpr == (TPR)) {                                                        \
+    NBLAHIP_LAUNCH("in_cl_row_fwd_kernel", (in_cl_row_fwd_kernel<T, VEC, NL, TPR>),            \
+                   dim3(grid_of(a)), dim3(TPR), 0, st, a);                                     \
+    return last_launch_status();                                                               \
+  }
+#define IN_BWD_CASE(T, VEC, NL, TPR)                                                           \
+  if (c.nl == (NL) && c.tpr == (TPR)) {                                                        \
+    NBLAHIP_LAUNCH("in_cl_row_bwd_kernel", (in_cl_row_bwd_kernel<T, VEC, NL, TPR>),            \
+                   dim3(grid_of(a)), dim3(TPR), 0, st, a);                                     \
+    return last_launch_status();                                                               \
+  }
+
+int run_in_fwd(int dtype, const GnClCfg &c, const GnClArgs &a, hipStream_t st) {
+  if (dtype == NBLAHIP_F16) {
+    IN_CL_CASES(IN_FWD_CASE, __half, 8)
+  } else {
+    IN_CL_CASES(IN_FWD_CASE, float, 4)
+  }
+  return NBLAHIP_EINVAL;
+}
+
+int run_in_bwd(int dtype, const GnClCfg &c, const GnClArgs &a, hipStream_t st) {
+  if (dtype == NBLAHIP_F16) {
+    IN_CL_CASES(IN_BWD_CASE, __half, 8)
+  } else {
+    IN_CL_CASES(IN_BWD_CASE, float, 4)
+  }
+  return NBLAHIP_EINVAL;
+}
+
 int run_fwd(int dtype, const GnClCfg &c, const GnClArgs &a, hipStream_t st) {
   if (dtype == NBLAHIP_F16) {
-    GN_CL_CASES(FWD_CASE, __half, 8)
+    IN_CL_CASES(FWD_CASE, __half, 8)
   } else {
-    GN_CL_CASES(FWD_CASE, float, 4)
+    IN_CL_CASES(FWD_CASE, float, 4)
   }
   return NBLAHIP_EINVAL;
 }
 
 int run_bwd(int dtype, const GnClCfg &c, const GnClArgs &a, hipStream_t st) {
   if (dtype == NBLAHIP_F16) {
-    GN_CL_CASES(BWD_CASE, __half, 8)
+    IN_CL_CASES(BWD_CASE, __half, 8)
   } else {
-    GN_CL_CASES(BWD_CASE, float, 4)
+    IN_CL_CASES(BWD_CASE, float, 4)
   }
   return NBLAHIP_EINVAL;
 }
@@ -109,7 +187,8 @@ int run_bwd(int dtype, const GnClCfg &c, const GnClArgs &a, hipStream_t st) {
 
 bool gn_cl_cached_fwd(const ClProblem &p, bool aligned, hipStream_t st, int *status) {
   GnClArgs a{};
-  const GnClCfg c = pick_cfg(p, aligned, false, a);
+  const bool instance = p.groups == p.channels;
+  const GnClCfg c = instance ? pick_in_cfg(p, aligned, false, a) : pick_cfg(p, aligned, false, a);
   if (!c.ok) return false;
   a.x = p.x;
   a.out = p.out;
@@ -117,14 +196,15 @@ bool gn_cl_cached_fwd(const ClProblem &p, bool aligned, hipStream_t st, int *sta
   a.beta = p.beta;
   a.mean = p.mean;
   a.var = p.var;
-  *status = run_fwd(p.dtype, c, a, st);
+  *status = instance ? run_in_fwd(p.dtype, c, a, st) : run_fwd(p.dtype, c, a, st);
   return true;
 }
 
 bool gn_cl_cached_bwd(const ClProblem &p, bool aligned, float *pairs, hipStream_t st,
                       int *status) {
   GnClArgs a{};
-  const GnClCfg c = pick_cfg(p, aligned, true, a);
+  const bool instance = p.groups == p.channels;
+  const GnClCfg c = instance ? pick_in_cfg(p, aligned, true, a) : pick_cfg(p, aligned, true, a);
   if (!c.ok) return false;
   a.x = p.x;
   a.dy = p.dy;
@@ -135,7 +215,7 @@ bool gn_cl_cached_bwd(const ClProblem &p, bool aligned, float *pairs, hipStream_
   a.dmean = p.dmean;
   a.dvar = p.dvar;
   a.pairs = pairs;
-  *status = run_bwd(p.dtype, c, a, st);
+  *status = instance ? run_in_bwd(p.dtype, c, a, st) : run_bwd(p.dtype, c, a, st);
   return true;
 }
 

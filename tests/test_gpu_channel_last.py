@@ -77,7 +77,10 @@ def test_gn_channel_last(n, sp, c, groups, dtype):
 IN_CL_SHAPES = [(2, (4, 4), 3), (3, (7,), 5), (1, (3, 2), 2), (4, (16, 16), 16), (2, (64, 64), 8),
                 (2, (7, 7), 24), (1, (200, 200), 3), (2, (300, 300), 2), (3, (1,), 7),
                 (2, (1000,), 64), (2, (5, 5), 1024), (16, (32, 32), 256),
-                (2, (9, 9), 96), (2, (5, 5), 4104), (3, (11,), 100), (2, (300,), 1032)]
+                (2, (9, 9), 96), (2, (5, 5), 4104), (3, (11,), 100), (2, (300,), 1032),
+                # instances cached in registers (256 positions and more)
+                (3, (33, 33), 24), (2, (20, 20), 128), (5, (17, 17), 16), (2, (56, 56), 64),
+                (1, (90, 90), 8), (9, (16, 16), 32)]
 
 
 @pytest.mark.parametrize("n,sp,c", IN_CL_SHAPES)
@@ -101,7 +104,7 @@ def test_in_channel_last(n, sp, c, dtype):
 
 
 @pytest.mark.parametrize("n,sp,c", [(3, (6, 6), 4), (2, (50, 50), 16)])
-@pytest.mark.parametrize("bcg,bcb", [(False, False), (True, False), (False, True)])
+@pytest.mark.parametrize("bcg,bcb", [(False, False), (True, False), (False, True), (True, True)])
 def test_in_channel_last_per_sample_parameters_and_flags(n, sp, c, bcg, bcb):
     rng = np.random.default_rng(7)
     shape = (n,) + sp + (c,)
