@@ -38,6 +38,14 @@ struct GnClArgs {
   int gpl;            // groups sharing a cache line, 1: plain block order
   float eps, inv_R, one;
   int accum_dx;
+  // BatchNormalization [M, C] through the instance kernels (one "sample" of M
+  // positions): running statistics of the forward, and dgamma/dbeta written
+  // by the backward itself (there is no batch to sum over; pairs unused).
+  float *rmean, *rvar;
+  float decay, unbias;
+  float *dgamma, *dbeta;
+  int accum_g, accum_b;
+  int direct_params;
 };
 
 constexpr int kXcds = 8;
@@ -365,8 +373,11 @@ in_cl_row_fwd_kernel(const GnClArgs a) {
       m = threadIdx.x == j ? mean[j] : m;
       v = threadIdx.x == j ? var[j] : v;
     }
-    a.mean[static_cast<size_t>(n) * a.C + ch + threadIdx.x] = m;
-    a.var[static_cast<size_t>(n) * a.C + ch + threadIdx.x] = v;
+    const size_t c = static_cast<size_t>(n) * a.C + ch + threadIdx.x;
+    a.mean[c] = m;
+    a.var[c] = v;
+    if (a.rmean) a.rmean[c] = a.decay * a.rmean[c] + (1.f - a.decay) * m;
+    if (a.rvar) a.rvar[c] = a.decay * a.rvar[c] + (1.f - a.decay) * v * a.unbias;
   }
 #pragma unroll
   for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
@@ -442,8 +453,14 @@ in_cl_row_bwd_kernel(const GnClArgs a) {
       px = threadIdx.x == j ? sdx[j] : px;
       py = threadIdx.x == j ? sdy[j] : py;
     }
-    a.pairs[2 * (stat + threadIdx.x)] = px;
-    a.pairs[2 * (stat + threadIdx.x) + 1] = py;
+    const size_t c = stat + threadIdx.x;
+    if (a.direct_params) {
+      if (a.dgamma) a.dgamma[c] = px + (a.accum_g ? a.dgamma[c] : 0.f);
+      if (a.dbeta) a.dbeta[c] = py + (a.accum_b ? a.dbeta[c] : 0.f);
+    } else {
+      a.pairs[2 * c] = px;
+      a.pairs[2 * c + 1] = py;
+    }
   }
   if (dx == nullptr) return;
 #pragma unroll

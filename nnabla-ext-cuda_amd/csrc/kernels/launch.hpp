@@ -127,6 +127,10 @@ struct BnProblem {
 // the shape or the flags are not theirs, else *status holds the launch result.
 bool bn_rows_fwd_train(const BnProblem &p, hipStream_t st, int *status);
 bool bn_rows_bwd(const BnProblem &p, hipStream_t st, int *status);
+// The same for channel-last tensors of few rows (gn_cl_rows.hip): a block per
+// channel vector keeps its column in registers.
+bool bn_cl_cached_fwd_train(const BnProblem &p, hipStream_t st, int *status);
+bool bn_cl_cached_bwd(const BnProblem &p, hipStream_t st, int *status);
 int launch_bn_infer(const BnProblem &p, hipStream_t st);
 int launch_bn_fwd_train(const BnProblem &p, hipStream_t st);
 int launch_bn_bwd(const BnProblem &p, hipStream_t st);

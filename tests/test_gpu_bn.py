@@ -27,6 +27,9 @@ SMALL = [
     # channel-last: channel vectors that do not divide 256, rows wider than 256 vectors,
     # 8-byte fp16 rows
     ((6, 9, 9, 96), 3), ((3, 5, 5, 4104), 3), ((37, 100), 1), ((4, 6, 6, 20), 3), ((700, 1032), 1),
+    # channel-last with few rows: a channel vector's column in one block's registers
+    ((32, 7, 7, 512), 3), ((8, 14, 14, 256), 3), ((100, 2048), 1), ((33, 8, 8, 320), 3),
+    ((5000, 256), 1),
 ]
 DTYPES = [torch.float32, torch.float16]
 
@@ -82,7 +85,9 @@ def test_bn_training_forward_backward(shape, axis, dtype):
 
 @pytest.mark.parametrize("shape,axis", [((4, 8, 6, 6), 1), ((37, 24), 1), ((6, 5, 4, 8), 3),
                                         # a channel per block, cached in registers
-                                        ((8, 64, 12, 12), 1), ((4, 48, 7, 9), 1), ((3, 300, 2, 2), 1)])
+                                        ((8, 64, 12, 12), 1), ((4, 48, 7, 9), 1), ((3, 300, 2, 2), 1),
+                                        # channel-last, a channel vector's column per block
+                                        ((8, 7, 7, 256), 3), ((300, 512), 1)])
 def test_bn_flags(shape, axis):
     """no_scale/no_bias, recompute (no running update), accumulation,
     propagate_down subsets, 3-output dmean/dvar."""
