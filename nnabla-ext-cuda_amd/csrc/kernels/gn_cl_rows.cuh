@@ -46,6 +46,13 @@ struct GnClArgs {
   float *dgamma, *dbeta;
   int accum_g, accum_b;
   int direct_params;
+  // FusedBatchNormalization through the same kernels: forward
+  // y = max(0, bn(x) [+ z]); backward dy is first gated by y > 0 and the gated
+  // dy is the gradient of z (dz, optional).
+  const void *z;
+  const void *y;
+  void *dz;
+  int accum_dz;
 };
 
 constexpr int kXcds = 8;
@@ -307,7 +314,8 @@ __device__ __forceinline__ void in_cl_block_sums(float (&v)[VEC], float (*lds)[V
   }
 }
 
-template <typename T, int VEC, int NL, int TPR>
+// FUSE: 0 plain, 1 y = max(0, .), 2 y = max(0, . + z).
+template <typename T, int VEC, int NL, int TPR, int FUSE = 0>
 __global__ void __launch_bounds__(TPR)
 in_cl_row_fwd_kernel(const GnClArgs a) {
   __shared__ float lds[TPR / kWave][VEC];
@@ -394,6 +402,16 @@ in_cl_row_fwd_kernel(const GnClArgs a) {
           o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mean[j]), sc[j], bet[j]);
         }
       }
+      if constexpr (FUSE == 2) {
+        const T *zp = static_cast<const T *>(a.z) + static_cast<size_t>(n) * a.P * a.C + ch;
+        const RawVec<T, VEC> zr = load_raw<T, VEC>(zp + static_cast<size_t>(pos) * a.C);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) o[j] = elem_fma<T, VEC>(zr, j, a.one, o[j]);
+      }
+      if constexpr (FUSE != 0) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) o[j] = fmaxf(0.f, o[j]);
+      }
       store_vec<T, VEC>(y + static_cast<size_t>(pos) * a.C, o);
     }
   }
@@ -402,7 +420,8 @@ in_cl_row_fwd_kernel(const GnClArgs a) {
 // Backward, per channel c of the block: sdx = sum dy*xh, sdy = sum dy (also the
 // pair behind dgamma/dbeta), dx = g*istd*dy + cA*xh + cb with
 // cA = -istd*g*sdx/P + 2*dvar*std/P, cb = -g*sdy*istd/P + dmean/P.
-template <typename T, int VEC, int NL, int TPR>
+// FUSED: dy := dy where y > 0 else 0 first; dz (optional) receives it.
+template <typename T, int VEC, int NL, int TPR, bool FUSED = false>
 __global__ void __launch_bounds__(TPR, (TPR == 512 ? 4 : 1))
 in_cl_row_bwd_kernel(const GnClArgs a) {
   __shared__ float lds[TPR / kWave][VEC];
@@ -424,6 +443,23 @@ in_cl_row_bwd_kernel(const GnClArgs a) {
     const size_t off = static_cast<size_t>(ok ? pos : 0u) * a.C;
     xr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + off));
     dr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(dy + off));
+    if constexpr (FUSED) {
+      const RawVec<T, VEC> yr = load_raw<T, VEC>(static_cast<const T *>(a.y) + slab + off);
+      dr[k] = raw_relu_mask<T, VEC>(dr[k], yr);
+      if (a.dz && ok) {
+        T *dzp = static_cast<T *>(a.dz) + slab + off;
+        if (a.accum_dz) {
+          float g[VEC], old[VEC];
+          unpack<T, VEC>(dr[k], g);
+          load_vec<T, VEC>(dzp, old);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) g[j] += old[j];
+          store_vec<T, VEC>(dzp, g);
+        } else {
+          store_raw<T, VEC>(dzp, dr[k]);
+        }
+      }
+    }
   }
   float istd[VEC], nmi[VEC], mean[VEC];
 #pragma unroll

@@ -6,6 +6,11 @@
 
 namespace nblahip {
 
+// gn_cl_rows_fused.hip
+int run_in_fwd_fused(int dtype, int tpr, int nl, const GnClArgs &a, unsigned grid, int fuse,
+                     hipStream_t st);
+int run_in_bwd_fused(int dtype, int tpr, int nl, const GnClArgs &a, unsigned grid, hipStream_t st);
+
 namespace {
 
 struct GnClCfg {
@@ -226,8 +231,9 @@ bool gn_cl_cached_bwd(const ClProblem &p, bool aligned, float *pairs, hipStream_
 // ---------------------------------------------------------------------------
 static bool bn_cl_cfg(const BnProblem &p, bool backward, GnClCfg &c, GnClArgs &a) {
   if (!tune_int("BN_CL_CACHED", 1)) return false;
-  if (p.size2 != 1 || p.relu || p.z || p.y || p.dz || p.sums_out || p.sums_in) return false;
-  const bool al = aligned16(p.x) && (!p.out || aligned16(p.out)) && (!backward || aligned16(p.dy));
+  if (p.size2 != 1 || p.sums_out || p.sums_in) return false;
+  const bool al = aligned16(p.x) && (!p.out || aligned16(p.out)) && (!backward || aligned16(p.dy)) &&
+                  (!p.z || aligned16(p.z)) && (!p.y || aligned16(p.y)) && (!p.dz || aligned16(p.dz));
   ClProblem q;
   q.dtype = p.dtype;
   q.batch = 1;
@@ -262,14 +268,16 @@ bool bn_cl_cached_fwd_train(const BnProblem &p, hipStream_t st, int *status) {
   a.rvar = p.rvar;
   a.decay = p.decay;
   a.unbias = static_cast<float>(N / (N - 1.0));
-  *status = run_in_fwd(p.dtype, c, a, st);
+  a.z = p.z;
+  *status = !p.relu ? run_in_fwd(p.dtype, c, a, st)
+                    : run_in_fwd_fused(p.dtype, c.tpr, c.nl, a, grid_of(a), p.z ? 2 : 1, st);
   return true;
 }
 
 bool bn_cl_cached_bwd(const BnProblem &p, hipStream_t st, int *status) {
   GnClCfg c;
   GnClArgs a{};
-  if (!p.batch_stat || (!p.out && !p.dgamma && !p.dbeta)) return false;
+  if (!p.batch_stat || (!p.out && !p.dgamma && !p.dbeta && !p.dz)) return false;
   if (!bn_cl_cfg(p, true, c, a)) return false;
   a.x = p.x;
   a.dy = p.dy;
@@ -284,7 +292,11 @@ bool bn_cl_cached_bwd(const BnProblem &p, hipStream_t st, int *status) {
   a.dbeta = p.dbeta;
   a.accum_g = p.accum_g;
   a.accum_b = p.accum_b;
-  *status = run_in_bwd(p.dtype, c, a, st);
+  a.y = p.y;
+  a.dz = p.dz;
+  a.accum_dz = p.accum_dz;
+  *status = !p.y ? run_in_bwd(p.dtype, c, a, st)
+                 : run_in_bwd_fused(p.dtype, c.tpr, c.nl, a, grid_of(a), st);
   return true;
 }
 

@@ -26,6 +26,8 @@ SHAPES = [
     ((8, 12, 14, 14), 1), ((16, 256, 14, 14), 1),
     ((4, 8, 7, 7), 1), ((64, 32, 7, 7), 1), ((5, 16, 13), 1),
     ((6, 9, 9, 96), 3), ((3, 5, 5, 4104), 3), ((37, 100), 1),
+    # channel-last with few rows: a channel vector's column in one block's registers
+    ((32, 7, 7, 512), 3), ((8, 14, 14, 256), 3), ((100, 2048), 1), ((33, 8, 8, 320), 3),
 ]
 
 
