@@ -114,7 +114,10 @@ BnPlan make_plan(int64_t size0, int64_t C, int64_t size2, int dtype, bool ptr_al
     const uint32_t cus = static_cast<uint32_t>(device_cus());
     const int direct = tune_int("BN_DIRECT", 2); // 0 never, 1 always, 2 automatic
     const bool balanced = (static_cast<uint64_t>(C) % cus == 0) || static_cast<uint64_t>(C) >= 8ull * cus;
-    if (direct == 1 || (direct == 2 && balanced && pl.vpc >= 4u * 1024u * kBnUnroll)) {
+    // (two steps of the 1024-thread block and more: [32,256,56,56] half, 12 544
+    // vectors per channel, 72 vs 81 us forward + backward; smaller channels fit
+    // the row kernels' registers and do not come here)
+    if (direct == 1 || (direct == 2 && balanced && pl.vpc >= 2u * 1024u * kBnUnroll)) {
       pl.direct = true;
       pl.S = 1;
       pl.chunk = pl.vpc;
