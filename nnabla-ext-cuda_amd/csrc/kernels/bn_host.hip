@@ -23,7 +23,8 @@ struct BnPlan {
   uint32_t ytiles = 1;  // ceil(ncv / TX)
   uint32_t S = 1;       // splits
   int apply_vec = 1;    // vector width of the apply kernels
-  bool direct = false;  // planes: one 1024-thread block owns a whole channel
+  bool direct = false;  // planes: one 1024-thread block owns a whole channel (statistics)
+  bool direct_bwd = false; // the same for the backward reduction
   // planes whose length is no multiple of the vector width: tensor-aligned
   // vectors, masked at the plane's ends (reductions) or split between the two
   // channels they touch (apply)
@@ -117,11 +118,13 @@ BnPlan make_plan(int64_t size0, int64_t C, int64_t size2, int dtype, bool ptr_al
     // (two steps of the 1024-thread block and more: [32,256,56,56] half, 12 544
     // vectors per channel, 72 vs 81 us forward + backward; smaller channels fit
     // the row kernels' registers and do not come here)
-    if (direct == 1 || (direct == 2 && balanced && pl.vpc >= 2u * 1024u * kBnUnroll)) {
-      pl.direct = true;
-      pl.S = 1;
-      pl.chunk = pl.vpc;
-    }
+    // The backward reduction takes them from 8192 vectors per channel; the
+    // statistics only with one channel per CU below 16 384 (with four rounds of
+    // 1024-thread blocks, [256,1024,14,14] half, they lose: 75 vs 64 us forward).
+    const bool enough = pl.vpc >= 2u * 1024u * kBnUnroll;
+    pl.direct_bwd = direct == 1 || (direct == 2 && balanced && enough);
+    pl.direct = direct == 1 || (direct == 2 && balanced && enough &&
+                                (pl.vpc >= 4u * 1024u * kBnUnroll || static_cast<uint64_t>(C) <= cus));
   } else {
     pl.vec = cl_vec(C, dtype, ptr_aligned);
     pl.ncv = static_cast<uint32_t>(C / pl.vec);
@@ -219,7 +222,7 @@ int stats_t(const BnProblem &p, const BnPlan &pl, float *part, const BnFwdFinal 
         NBLAHIP_LAUNCH("bn_stats_planes_kernel",
                        (bn_stats_planes_kernel<T, VEC, 1024, true, 4, true>),
                        dim3(static_cast<uint32_t>(p.C), 1), dim3(1024), 0, st, x,
-                       static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, part, fin,
+                       static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.vpc, part, fin,
                        pl.size2, pl.last_vec);
       } else {
         NBLAHIP_LAUNCH("bn_stats_planes_kernel",
@@ -234,7 +237,7 @@ int stats_t(const BnProblem &p, const BnPlan &pl, float *part, const BnFwdFinal 
   } else if (pl.direct) {
     NBLAHIP_LAUNCH("bn_stats_planes_kernel", (bn_stats_planes_kernel<T, VEC, 1024, true, 8>),
                    dim3(static_cast<uint32_t>(p.C), 1), dim3(1024), 0, st, x,
-                   static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, part, fin, 0u,
+                   static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.vpc, part, fin, 0u,
                    0u);
   } else {
     NBLAHIP_LAUNCH("bn_stats_planes_kernel", (bn_stats_planes_kernel<T, VEC, kBnBlock, false, kBnUnroll>),
@@ -264,11 +267,11 @@ int bwd_reduce_fuse_t(const BnProblem &p, const BnPlan &pl, float *part2, const 
                    FastDiv(1), y, dz);
   } else if (pl.masked) {
     if constexpr (kFullVec<T, VEC>) {
-      if (pl.direct) {
+      if (pl.direct_bwd) {
         NBLAHIP_LAUNCH(FUSED ? "bn_bwd_reduce_planes_kernel_fused" : "bn_bwd_reduce_planes_kernel",
                        (bn_bwd_reduce_planes_kernel<T, VEC, 1024, true, FUSED, true>),
                        dim3(static_cast<uint32_t>(p.C), 1), dim3(1024), 0, st, x, dy, p.mean,
-                       static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, 1.0f, part2,
+                       static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.vpc, 1.0f, part2,
                        fin, y, dz, pl.size2, pl.last_vec);
       } else {
         NBLAHIP_LAUNCH(FUSED ? "bn_bwd_reduce_planes_kernel_fused" : "bn_bwd_reduce_planes_kernel",
@@ -280,11 +283,11 @@ int bwd_reduce_fuse_t(const BnProblem &p, const BnPlan &pl, float *part2, const 
     } else {
       return NBLAHIP_EINVAL;
     }
-  } else if (pl.direct) {
+  } else if (pl.direct_bwd) {
     NBLAHIP_LAUNCH(FUSED ? "bn_bwd_reduce_planes_kernel_fused" : "bn_bwd_reduce_planes_kernel",
                    (bn_bwd_reduce_planes_kernel<T, VEC, 1024, true, FUSED>),
                    dim3(static_cast<uint32_t>(p.C), 1), dim3(1024), 0, st, x, dy, p.mean,
-                   static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.chunk, 1.0f, part2, fin,
+                   static_cast<uint32_t>(p.C), FastDiv(pl.nvp), pl.vpc, pl.vpc, 1.0f, part2, fin,
                    y, dz, 0u, 0u);
   } else {
     NBLAHIP_LAUNCH(FUSED ? "bn_bwd_reduce_planes_kernel_fused" : "bn_bwd_reduce_planes_kernel",
@@ -488,7 +491,7 @@ int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
   if (need_sums) {
     if (int e = do_bwd_reduce(p, pl, part2, fin, st)) return e;
   }
-  if ((p.out || need_sums) && (!need_sums || !pl.direct)) {
+  if ((p.out || need_sums) && (!need_sums || !pl.direct_bwd)) {
     // Without the reduction (inference-mode dx only) S = 0 leaves the sums at zero.
     NBLAHIP_LAUNCH("bn_finalize_bwd_kernel", bn_finalize_bwd_kernel,
                    dim3(static_cast<uint32_t>(p.C)), dim3(kBnBlock), 0, st, part2,
