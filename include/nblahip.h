@@ -208,6 +208,12 @@ NBLAHIP_EXPORT int nblahip_fused_bn_bwd(
 /* ------------------------------------------------------------------------
  * LayerNormalization.  x viewed as [outer, reduce]
  * (src/nbla/cuda/function/generic/layer_normalization.cu:53-59).
+ *
+ * The forward entry points of the three row normalizations below take no
+ * workspace.  For tensors of a few very long rows they keep partial statistics
+ * in the first bytes of y until the pass that writes y overwrites them: y must
+ * not overlap x other than being x itself (in place, y == x, is detected and
+ * handled without the scratch use).
  * ---------------------------------------------------------------------- */
 
 /* Replaces forward_impl (layer_normalization.cu:77-133): reduce_2d_x<WelfordOp>
