@@ -346,3 +346,37 @@ def test_row_argument_errors():
                             s) == -2                               # workspace missing
     assert L.nblahip_ln_fwd(x.data_ptr(), None, None, y.data_ptr(), m.data_ptr(), m.data_ptr(),
                             1 << 20, 1 << 20, 1e-5, 0, s) == -3    # >= 2^31 elements
+
+
+@pytest.mark.parametrize("outer,Rr", [(64, 1024), (300, 48), (2, 131072), (3, 40004)])
+def test_ln_forward_in_place(outer, Rr):
+    """y == x: register-cached, several rows per wave, and the streaming path
+    (which must then not keep its partial statistics in y)."""
+    x, _, g, b = make_ln(outer, Rr, torch.float32, 31)
+    y_r, m_r, v_r = R.ln_forward(x, b, g, outer, 1e-5)
+    xd, gd, bd = to_dev(x), to_dev(g), to_dev(b)
+    mean = torch.empty(outer, device="cuda")
+    var = torch.empty(outer, device="cuda")
+    L = K.lib()
+    K.check(L.nblahip_ln_fwd(xd.data_ptr(), gd.data_ptr(), bd.data_ptr(), xd.data_ptr(),
+                             mean.data_ptr(), var.data_ptr(), outer, Rr, 1e-5, 0,
+                             torch.cuda.current_stream().cuda_stream))
+    assert_close(to_np(xd), y_r, "f32", "y", "y in place")
+    assert_close(to_np(mean), m_r, "f32", "stat", "mean")
+    assert_close(to_np(var), v_r, "f32", "stat", "var")
+
+
+@pytest.mark.parametrize("n,c,sp", [(2, 8, (16, 16)), (1, 3, (300, 300)), (4, 64, (7, 7))])
+def test_in_forward_in_place(n, c, sp):
+    x, _, g, b = make_nc(n, c, sp, torch.float16, 32)
+    y_r, m_r, v_r = R.in_forward(x, b, g, n, c, 1e-5)
+    xd, gd, bd = to_dev(x, torch.float16), to_dev(g), to_dev(b)
+    mean = torch.empty(n * c, device="cuda")
+    var = torch.empty(n * c, device="cuda")
+    L = K.lib()
+    spatial = int(np.prod(sp))
+    K.check(L.nblahip_in_fwd(xd.data_ptr(), gd.data_ptr(), bd.data_ptr(), xd.data_ptr(),
+                             mean.data_ptr(), var.data_ptr(), n, c, spatial, 1, 1, 1e-5, 1,
+                             torch.cuda.current_stream().cuda_stream))
+    assert_close(to_np(xd), y_r.reshape(x.shape), "f16", "y", "y in place")
+    assert_close(to_np(mean), m_r, "f16", "stat", "mean")
