@@ -72,14 +72,15 @@ GnClCfg pick_cfg(const ClProblem &p, bool aligned, bool backward, GnClArgs &a) {
 
 // InstanceNormalization: a block per (sample, channel vector); P positions of
 // one vector each.
-GnClCfg pick_in_cfg(const ClProblem &p, bool aligned, bool backward, GnClArgs &a) {
+GnClCfg pick_in_cfg(const ClProblem &p, bool aligned, bool backward, GnClArgs &a,
+                    int64_t min_positions = -1) {
   GnClCfg c;
   if (!aligned || !tune_int("IN_CL_CACHED", 1)) return c;
   if (!p.bc_gamma || !p.bc_beta) return c;
   const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
   if (p.channels % vec != 0) return c;
   const int64_t nv = p.spatial;
-  if (nv < tune_int("IN_CL_MIN", 32)) return c;
+  if (nv < (min_positions >= 0 ? min_positions : tune_int("IN_CL_MIN", 32))) return c;
   // Beyond 2048 positions the three-kernel path is as fast or faster in float
   // and in the backward pass (64x64 planes, half: backward 49 vs 44 us; 56x56
   // float: 62 / 130 vs 57 / 92 us); below, the single pass wins by 1.3-2x.
@@ -246,9 +247,12 @@ static bool bn_cl_cfg(const BnProblem &p, bool backward, GnClCfg &c, GnClArgs &a
   // half: 17 / 17 -> 9 / 10 us); the forward still does up to 4096 rows when
   // there are at least 64 blocks (14 vs 23 us), the backward does not (24 vs 24 us
   // at 3136 rows, 49 vs 25 us at 6272).
-  c = pick_in_cfg(q, al, backward, a);
+  c = pick_in_cfg(q, al, backward, a, 2); // also the few rows of a fully connected layer's batch
   if (!c.ok) return false;
-  if (a.units < 32) return false; // a handful of blocks: the split reduction fills the chip
+  // a handful of blocks: the split reduction fills the chip (tensors of up to
+  // 2 MB excepted: there its three launches cost more than idle CUs)
+  const int64_t bytes = p.size0 * p.C * (p.dtype == NBLAHIP_F16 ? 2 : 4);
+  if (a.units < 32 && bytes > (2 << 20)) return false;
   if (p.size0 > 2048 && (p.size0 > 4096 || a.units < 64)) return false;
   return true;
 }

@@ -548,8 +548,11 @@ static bool bn_rows_cfg(const BnProblem &p, bool backward, RowCfg &cfg, RowArgs 
   cfg = pick_row_cfg(vec, R, 8, 8, 4, false);
   if (!cfg.ok) return false;
   // a handful of blocks leaves the chip idle: the split reduction spreads
-  // such tensors over all CUs
-  if ((p.C + rows_per_block(cfg.tpr) - 1) / rows_per_block(cfg.tpr) < 32) return false;
+  // such tensors over all CUs - unless the tensor is so small (2 MB) that the
+  // three launches of that path are what costs (14 vs 6 us)
+  const int64_t bytes = R * p.C * (p.dtype == NBLAHIP_F16 ? 2 : 4);
+  if ((p.C + rows_per_block(cfg.tpr) - 1) / rows_per_block(cfg.tpr) < 32 && bytes > (2 << 20))
+    return false;
   a = RowArgs{};
   a.x = p.x;
   a.dy = p.dy;

@@ -29,7 +29,7 @@ SMALL = [
     ((6, 9, 9, 96), 3), ((3, 5, 5, 4104), 3), ((37, 100), 1), ((4, 6, 6, 20), 3), ((700, 1032), 1),
     # channel-last with few rows: a channel vector's column in one block's registers
     ((32, 7, 7, 512), 3), ((8, 14, 14, 256), 3), ((100, 2048), 1), ((33, 8, 8, 320), 3),
-    ((5000, 256), 1),
+    ((5000, 256), 1), ((16, 1024), 1), ((4, 2048), 1), ((6, 64), 1),
 ]
 DTYPES = [torch.float32, torch.float16]
 
