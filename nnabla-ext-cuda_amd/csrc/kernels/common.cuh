@@ -64,26 +64,63 @@ __device__ __forceinline__ void load_vec(const T *__restrict__ p, float (&out)[V
   }
 }
 
-template <typename T, int VEC>
+// Vector stores of outputs are non-temporal by default: an output is written
+// once and not read again by the call, so it should not displace the inputs
+// (which the second pass of a split reduction reads again) from L2 and the
+// Infinity Cache.  Measured on [32,256,56,56] fp32 BatchNormalization: backward
+// apply 44.4 -> 41.9 us, the four kernels 125.8 -> 118.9 us.  (Non-temporal
+// loads were measured too and lose: the second pass then misses the cache.)
+// STREAM = false keeps the ordinary store: for kernels whose wave writes short
+// pieces of many cache lines (the channel-last tiles), where neighbouring
+// blocks complete the lines in L2; non-temporal stores of such pieces cost 3x.
+typedef float native_f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t native_u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t native_u2 __attribute__((ext_vector_type(2)));
+template <bool STREAM> __device__ __forceinline__ void store_wide(float *p, const float4 &v) {
+  if constexpr (STREAM) {
+    const native_f4 t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<native_f4 *>(p));
+  } else {
+    *reinterpret_cast<float4 *>(p) = v;
+  }
+}
+template <bool STREAM> __device__ __forceinline__ void store_wide(__half *p, const uint4 &v) {
+  if constexpr (STREAM) {
+    const native_u4 t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<native_u4 *>(p));
+  } else {
+    *reinterpret_cast<uint4 *>(p) = v;
+  }
+}
+template <bool STREAM> __device__ __forceinline__ void store_wide(__half *p, const uint2 &v) {
+  if constexpr (STREAM) {
+    const native_u2 t = {v.x, v.y};
+    __builtin_nontemporal_store(t, reinterpret_cast<native_u2 *>(p));
+  } else {
+    *reinterpret_cast<uint2 *>(p) = v;
+  }
+}
+
+template <typename T, int VEC, bool STREAM = true>
 __device__ __forceinline__ void store_vec(T *__restrict__ p, const float (&in)[VEC]) {
   if constexpr (VEC == 1) {
     p[0] = from_f32<T>(in[0]);
   } else if constexpr (sizeof(T) == 4) {
-    *reinterpret_cast<float4 *>(p) = make_float4(in[0], in[1], in[2], in[3]);
+    store_wide<STREAM>(p, make_float4(in[0], in[1], in[2], in[3]));
   } else if constexpr (VEC == 4) {
     uint2 raw;
     __half2 *h = reinterpret_cast<__half2 *>(&raw);
 #pragma unroll
     for (int i = 0; i < 2; ++i)
       h[i] = __floats2half2_rn(in[2 * i], in[2 * i + 1]);
-    *reinterpret_cast<uint2 *>(p) = raw;
+    store_wide<STREAM>(p, raw);
   } else {
     uint4 raw;
     __half2 *h = reinterpret_cast<__half2 *>(&raw);
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       h[i] = __floats2half2_rn(in[2 * i], in[2 * i + 1]);
-    *reinterpret_cast<uint4 *>(p) = raw;
+    store_wide<STREAM>(p, raw);
   }
 }
 
@@ -277,16 +314,16 @@ __device__ __forceinline__ RawVec<T, VEC> raw_keep_range(RawVec<T, VEC> r, int l
   return r;
 }
 
-template <typename T, int VEC>
+template <typename T, int VEC, bool STREAM = true>
 __device__ __forceinline__ void store_raw(T *__restrict__ p, const RawVec<T, VEC> &r) {
   if constexpr (VEC == 1) {
     p[0] = r.v;
   } else if constexpr (sizeof(T) == 4) {
-    *reinterpret_cast<float4 *>(p) = r.v;
+    store_wide<STREAM>(p, r.v);
   } else if constexpr (VEC == 4) {
-    *reinterpret_cast<uint2 *>(p) = r.v;
+    store_wide<STREAM>(p, r.v);
   } else {
-    *reinterpret_cast<uint4 *>(p) = r.v;
+    store_wide<STREAM>(p, r.v);
   }
 }
 

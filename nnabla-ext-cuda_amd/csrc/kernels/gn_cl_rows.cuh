@@ -157,7 +157,7 @@ gn_cl_row_fwd_kernel(const GnClArgs a) {
           o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mean), sc[j], bet[j]);
         }
       }
-      store_vec<T, VEC>(y + static_cast<size_t>(pos) * a.C, o);
+      store_vec<T, VEC, false>(y + static_cast<size_t>(pos) * a.C, o);
     }
   }
 }
@@ -278,7 +278,7 @@ gn_cl_row_bwd_kernel(const GnClArgs a) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) o[j] += old[j];
       }
-      store_vec<T, VEC>(p, o);
+      store_vec<T, VEC, false>(p, o);
     }
   }
 }
@@ -412,7 +412,7 @@ in_cl_row_fwd_kernel(const GnClArgs a) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) o[j] = fmaxf(0.f, o[j]);
       }
-      store_vec<T, VEC>(y + static_cast<size_t>(pos) * a.C, o);
+      store_vec<T, VEC, false>(y + static_cast<size_t>(pos) * a.C, o);
     }
   }
 }
@@ -454,9 +454,9 @@ in_cl_row_bwd_kernel(const GnClArgs a) {
           load_vec<T, VEC>(dzp, old);
 #pragma unroll
           for (int j = 0; j < VEC; ++j) g[j] += old[j];
-          store_vec<T, VEC>(dzp, g);
+          store_vec<T, VEC, false>(dzp, g);
         } else {
-          store_raw<T, VEC>(dzp, dr[k]);
+          store_raw<T, VEC, false>(dzp, dr[k]);
         }
       }
     }
@@ -531,7 +531,7 @@ in_cl_row_bwd_kernel(const GnClArgs a) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) o[j] += old[j];
       }
-      store_vec<T, VEC>(p, o);
+      store_vec<T, VEC, false>(p, o);
     }
   }
 }
