@@ -158,7 +158,8 @@ class Variable:
             raise NblaError(-1, lib().nnabla_hip_last_error().decode())
 
     def __del__(self):
-        if getattr(self, "_h", None):
+        # (at interpreter shutdown the module globals may be gone already)
+        if getattr(self, "_h", None) and lib is not None:
             lib().nnabla_hip_variable_delete(self._h)
             self._h = None
 
@@ -213,7 +214,7 @@ class Function:
         self._h = handle
 
     def __del__(self):
-        if getattr(self, "_h", None):
+        if getattr(self, "_h", None) and lib is not None:
             lib().nnabla_hip_function_delete(self._h)
             self._h = None
 

@@ -24,6 +24,7 @@
 #include <cstring>
 #include <functional>
 #include <map>
+#include <set>
 #include <memory>
 #include <mutex>
 #include <sstream>
@@ -340,6 +341,7 @@ class NBLA_API SyncedArray {
   std::map<Key, ArrayPtr> arrays_;
   bool has_head_ = false;
   Key head_;
+  std::set<Key> current_; // materialisations that hold the head's content (head included)
   bool zeroing_ = false, filling_ = false;
   float fill_value_ = 0.f;
 
@@ -364,7 +366,7 @@ class NBLA_API SyncedArray {
       if (filling_) dst->fill(fill_value_); else dst->zero();
       return dst;
     }
-    if (key == head_) return dst;
+    if (key == head_ || current_.count(key)) return dst; // a reader's copy stays good until the next write
     ArrayPtr src = arrays_.at(head_);
     if (head_.first == key.first) {
       dst->copy_from(src.get()); // same class: dtype conversion on its device
@@ -374,10 +376,12 @@ class NBLA_API SyncedArray {
       if (head_.second != key.second) {
         const Key skey(head_.first, key.second);
         staged = materialize(skey, src->context());
-        staged->copy_from(src.get());
+        if (!current_.count(skey)) staged->copy_from(src.get());
+        current_.insert(skey);
       }
       ArraySynchronizer::synchronize(head_.first, staged.get(), key.first, dst.get());
     }
+    current_.insert(key);
     return dst;
   }
 
@@ -392,6 +396,7 @@ public:
     // every other materialisation is stale now
     for (auto it = arrays_.begin(); it != arrays_.end();)
       it = (it->first == head_) ? std::next(it) : arrays_.erase(it);
+    current_.clear();
     return a;
   }
   Array *cast(dtypes dtype, const Context &ctx, bool write_only = false) {
@@ -408,6 +413,7 @@ public:
   }
   void zero() {
     arrays_.clear();
+    current_.clear();
     has_head_ = true;
     zeroing_ = true;
     filling_ = false;
@@ -415,6 +421,7 @@ public:
   }
   void fill(float v) {
     arrays_.clear();
+    current_.clear();
     has_head_ = true;
     zeroing_ = false;
     filling_ = true;
@@ -423,6 +430,7 @@ public:
   }
   void clear() {
     arrays_.clear();
+    current_.clear();
     has_head_ = false;
     zeroing_ = filling_ = false;
   }

@@ -79,6 +79,17 @@ static void test_variable_and_arrays() {
   EXPECT(static_cast<float>(h[5]) == 2.5f);
   const float *f = v.get_data_pointer<float>(cpu);
   EXPECT(f[23] == 11.5f);
+  // A reader's converted copy stays good until the next write: reading again
+  // returns the same buffer without converting (a value planted in it
+  // survives), and a write through cast() refreshes what the reader sees.
+  const_cast<Half *>(h)[5] = Half(-7.f);
+  const Half *h2 = v.get_data_pointer<Half>(cpu);
+  EXPECT(h2 == h && static_cast<float>(h2[5]) == -7.f);
+  EXPECT(v.get_data_pointer<float>(cpu)[5] == 2.5f);        // the head is untouched
+  d = v.cast_data_and_get_pointer<float>(cpu, false);
+  EXPECT(d[5] == 2.5f);
+  d[5] = 9.f;
+  EXPECT(static_cast<float>(v.get_data_pointer<Half>(cpu)[5]) == 9.f);
   v.grad()->fill(3.f);
   EXPECT(v.get_grad_pointer<float>(cpu)[7] == 3.f);
   v.grad()->zero();
