@@ -393,22 +393,6 @@ bn_finalize_fwd_kernel(const float *__restrict__ part, uint32_t S, BnFwdFinal fi
   if (threadIdx.x == 0) fin.publish(c, w);
 }
 
-// Inference: apply parameters straight from the running statistics.
-__global__ void __launch_bounds__(256)
-bn_infer_params_kernel(uint32_t C, float eps, const float *__restrict__ rmean,
-                       const float *__restrict__ rvar, const float *__restrict__ gamma,
-                       const float *__restrict__ beta, BnParam *__restrict__ params) {
-  const uint32_t c = blockIdx.x * 256u + threadIdx.x;
-  if (c < C) {
-    BnParam q;
-    q.mean = rmean[c];
-    q.a = (gamma ? gamma[c] : 1.f) * inv_std(rvar[c], eps);
-    q.b = beta ? beta[c] : 0.f;
-    q.c = 0.f;
-    params[c] = q;
-  }
-}
-
 // How the apply kernels obtain a channel's parameters.
 //   params != null : precomputed by a finalize kernel
 //   params == null : inference, computed on the fly from running statistics
