@@ -12,7 +12,9 @@ Canonical layouts (row-major, the reference's own flattening):
   GN/IN   x viewed as [N, C, spatial]     (group_normalization.cu:57-62,
                                            instance_normalization.cu:53-55)
 
-How each function is pinned (see tests/test_oracle_pins.py):
+How each function is pinned (see tests/test_oracle_pins.py; the same torch
+operators also wrote the stored vectors of tests/golden/*.npz, which
+tests/test_golden.py holds the oracle and the HIP path to):
   bn_forward_global, bn_forward_batch, bn_backward_batch, bn_backward_global,
   ln_forward/backward, gn_forward/backward, in_forward/backward
       -> torch CPU float64 F.batch_norm / layer_norm / group_norm /
