@@ -7,8 +7,9 @@ decay_rate 0.9, eps 1e-5.  One step = one forward (batch statistics, running
 statistics update, y) plus one backward (dx, dgamma, dbeta) through the C-ABI,
 inputs resident in HBM.
 
-Prints ONE JSON line.  `value` is algorithmic GB/s of the whole step
-(8 tensor passes: forward x twice + y, backward x and dy twice + dx);
+Prints ONE JSON line.  `value` is algorithmic GB/s of the whole step (the
+tensor passes the chosen plan makes: forward x + y with the channel held on
+chip, else x twice + y; backward x and dy twice + dx);
 `roofline` is the dominant kernel (backward apply: x, dy in, dx out) timed with
 HIP events on the launch stream in a second region of the same K steps;
 `cpu_baseline` is the C restatement of the reference arithmetic
@@ -45,6 +46,32 @@ class Workload:
 def _ws(nbytes):
     import torch
     return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device="cuda")
+
+
+# Kernels that keep a BatchNormalization channel on chip (registers, LDS) and
+# the tensor passes their direction then makes; the split reduction makes 3
+# forward (x for the statistics, x again, y) and 5 backward.
+BN_ONCHIP_FWD = ("bn_onchip_fwd_kernel", "row_fwd_kernel_bn", "in_cl_row_fwd_kernel")
+BN_ONCHIP_BWD = {"bn_onchip_bwd_kernel": 4, "row_bwd_kernel_bn": 3, "in_cl_row_bwd_kernel": 3}
+
+
+def bn_tensor_passes(K, fwd, bwd):
+    """(forward, backward) tensor passes of the plan the library picks for this
+    workload: a pass counts when the channel cannot stay on chip between the
+    statistics and the apply phase.  Read off the kernels one call launches."""
+    import torch
+    L = K.lib()
+    K.check(L.nblahip_profile_enable(64))
+    fwd()
+    bwd()
+    torch.cuda.synchronize()
+    pf = 2 if any(K.profile_query(k)[1] for k in BN_ONCHIP_FWD) else 3
+    pb = 5
+    for k, passes in BN_ONCHIP_BWD.items():
+        if K.profile_query(k)[1]:
+            pb = passes
+    K.check(L.nblahip_profile_enable(0))
+    return pf, pb
 
 
 def make_bn(K, shape, axis, dtype, train, mean=0.0, std=1.0, outliers=False, seed=0, fused=False,
@@ -104,7 +131,8 @@ def make_bn(K, shape, axis, dtype, train, mean=0.0, std=1.0, outliers=False, see
                                      bv.data_ptr(), None, None, dx.data_ptr(), dg.data_ptr(),
                                      db.data_ptr(), 0, 0, 0, s0, c, s2, 1e-5, 1, dt, ws.data_ptr(),
                                      ws.numel(), st))
-        return fwd, bwd, 3 * S, 5 * S, (x, dy, gamma, beta, rm, rv, y, dx, bm, bv, dg, db, ws)
+        pf, pb = bn_tensor_passes(K, fwd, bwd)
+        return fwd, bwd, pf * S, pb * S, (x, dy, gamma, beta, rm, rv, y, dx, bm, bv, dg, db, ws)
 
     def fwd():
         K.check(L.nblahip_bn_fwd_infer(x.data_ptr(), rm.data_ptr(), rv.data_ptr(), gamma.data_ptr(),
@@ -449,7 +477,8 @@ def main():
     log(f"C2 fwd+bwd: {ms * 1e3:.1f} us/step, {value:.0f} GB/s algorithmic")
 
     # Second region: the same K steps with per-kernel HIP events.
-    kernels = ["bn_stats_planes_kernel", "bn_finalize_fwd_kernel", "bn_apply_planes_kernel",
+    kernels = ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel",
+               "bn_stats_planes_kernel", "bn_finalize_fwd_kernel", "bn_apply_planes_kernel",
                "bn_apply_planes_fused_kernel", "bn_bwd_reduce_planes_kernel",
                "bn_finalize_bwd_kernel", "bn_bwd_apply_planes_kernel",
                "bn_bwd_apply_planes_fused_kernel"]
@@ -458,8 +487,9 @@ def main():
         fwd()
         bwd()
     torch.cuda.synchronize()
-    S = fb // 3
-    kbytes = {"bn_stats_planes_kernel": S, "bn_apply_planes_kernel": 2 * S,
+    S = keep[0].numel() * keep[0].element_size()
+    kbytes = {"bn_onchip_fwd_kernel": 2 * S, "bn_onchip_bwd_kernel": 4 * S,
+              "bn_stats_planes_kernel": S, "bn_apply_planes_kernel": 2 * S,
               "bn_apply_planes_fused_kernel": 2 * S, "bn_bwd_reduce_planes_kernel": 2 * S,
               "bn_bwd_apply_planes_kernel": 3 * S, "bn_bwd_apply_planes_fused_kernel": 3 * S}
     per_kernel = {}
@@ -488,6 +518,10 @@ def main():
         "config": {"workload": "BatchNormalization training fwd+bwd fp32 NCHW x[32,256,56,56] "
                                "(benchmark configuration 2), decay_rate 0.9, eps 1e-5",
                    "algorithmic_bytes_per_step": fb + bb,
+                   "tensor_passes": {"forward": fb // S, "backward": bb // S,
+                                     "note": "a pass counts when the channel cannot stay on chip "
+                                             "between statistics and apply; the forward keeps "
+                                             "its channel in registers and LDS (x read once)"},
                    "pct_of_hbm_peak": round(value / HBM_PEAK_GBS * 100, 1)},
         "roofline": roofline,
         "per_kernel": per_kernel,

@@ -440,6 +440,7 @@ int bn_fwd_train_impl(const BnProblem &p, bool stats_only, hipStream_t st) {
 int launch_bn_fwd_train(const BnProblem &p, hipStream_t st) {
   int status = 0;
   if (bn_rows_fwd_train(p, st, &status)) return status;
+  if (bn_onchip_fwd_train(p, st, &status)) return status;
   if (bn_cl_cached_fwd_train(p, st, &status)) return status;
   return bn_fwd_train_impl(p, false, st);
 }
@@ -463,6 +464,7 @@ int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
   {
     int status = 0;
     if (bn_rows_bwd(p, st, &status)) return status;
+    if (bn_onchip_bwd(p, st, &status)) return status;
     if (bn_cl_cached_bwd(p, st, &status)) return status;
   }
   const bool al = aligned16(p.x) && aligned16(p.dy) && (!p.out || aligned16(p.out)) &&

@@ -1,0 +1,462 @@
+// BatchNormalization training forward with a whole channel held on one CU:
+// registers first, LDS for what exceeds them.  One 1024-thread block per
+// channel reads its N planes once, reduces, and writes y: x crosses the memory
+// system once (2 S per call) where the split reduction reads it twice (3 S).
+//
+// A CU holds 512 KB of vector registers and 160 KB of LDS; a 1024-thread block
+// may use 128 registers per thread, of which NR 16-byte vectors (4 registers
+// each) are data, and NS more vectors per thread live in LDS (each thread
+// reads back only what it wrote: no barrier, no bank conflict).  NR + NS = 25
+// covers 25600 vectors = 400 KB per channel: [32, C, 56, 56] in float,
+// [64, C, 56, 56] in half.
+//
+// The backward keeps x on the CU the same way and streams dy past it twice
+// (sums, then dx): x once, dy twice, dx once = 4 S where the split reduction
+// moves 5 S; dgamma/dbeta are written by the channel's block, no finalize.
+//
+// Worth it only when there is a channel for (nearly) every CU: the block is
+// alone on its CU, so fewer channels than CUs leave the rest of the chip idle
+// and the split reduction wins.
+#include <algorithm>
+
+#include "common.cuh"
+#include "launch.hpp"
+
+namespace nblahip {
+
+namespace {
+
+constexpr int kOnchipBlock = 1024;
+
+struct BnOnchipArgs {
+  const void *x;
+  void *y;
+  const float *gamma, *beta;
+  float *mean, *var, *rmean, *rvar;
+  uint32_t C;
+  uint32_t size2;      // elements per plane
+  uint32_t nv;         // vectors per channel = size0 * vpp
+  FastDiv vpp;         // vectors per plane
+  float inv_N, unbias, decay, eps, one;
+  // backward
+  const void *dy;
+  void *dx;                 // may be null
+  const float *dmean, *dvar; // may be null
+  float *dgamma, *dbeta;    // may be null
+  int accum_dx, accum_g, accum_b;
+};
+
+__device__ __forceinline__ float onchip_block_sum(float v, float *red) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / kWave;
+  lds_barrier(); // earlier readers of red are done
+  if ((threadIdx.x & (kWave - 1)) == 0) red[wave] = v;
+  lds_barrier();
+  float t = 0.f;
+#pragma unroll
+  for (int i = 0; i < kOnchipBlock / kWave; ++i) t += red[i];
+  return t;
+}
+
+// The same value, opaque to the optimiser: offsets computed from it are not
+// merged with those of an earlier pass (kept alive across the passes, the 25
+// offsets of a thread cost 25 registers and the kernel spills).
+__device__ __forceinline__ uint32_t fresh(uint32_t v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
+// Hides a register-held vector from the optimiser (keep_packed does so for
+// half data only): what pass 1 derived from it (x - mean, xh) is then computed
+// again in pass 2 instead of being kept alive, or spilled, across the passes.
+template <typename T, int VEC> __device__ __forceinline__ void forget(RawVec<T, VEC> &r) {
+  if constexpr (sizeof(T) == 4) {
+    asm volatile("" : "+v"(r.v.x), "+v"(r.v.y), "+v"(r.v.z), "+v"(r.v.w));
+  } else {
+    keep_packed<T, VEC>(r);
+  }
+}
+
+// v again, but only once `after` has been computed: ties the addresses of a
+// batch of loads to the previous batch's results, so the compiler cannot issue
+// every batch up front (25 batches' worth of registers).
+__device__ __forceinline__ uint32_t fresh_after(uint32_t v, float after) {
+  asm volatile("" : "+v"(v) : "v"(after));
+  return v;
+}
+
+__device__ __forceinline__ uint32_t fresh_after(uint32_t v, uint32_t after) {
+  asm volatile("" : "+v"(v) : "v"(after));
+  return v;
+}
+
+// Element offset of vector v of channel c (planes are contiguous, a channel's
+// planes lie C*size2 apart).
+__device__ __forceinline__ uint32_t onchip_offset(const BnOnchipArgs &a, uint32_t c, uint32_t v,
+                                                  int vec) {
+  const uint32_t n = a.vpp.div(v);
+  const uint32_t w = v - n * a.vpp.d;
+  return (n * a.C + c) * a.size2 + w * static_cast<uint32_t>(vec);
+}
+
+template <typename T, int VEC, int NR, int NS>
+__global__ void __launch_bounds__(kOnchipBlock)
+bn_onchip_fwd_kernel(const BnOnchipArgs a) {
+  static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors only");
+  __shared__ float red[kOnchipBlock / kWave];
+  __shared__ uint4 spill[NS > 0 ? NS * kOnchipBlock : 1];
+  const uint32_t c = blockIdx.x;
+  const uint32_t t = threadIdx.x;
+  const T *__restrict__ x = static_cast<const T *>(a.x);
+  T *__restrict__ y = static_cast<T *>(a.y);
+
+  // Loads, all in flight together (no branch: a slot beyond the channel reads
+  // the channel's last vector and is left out of every sum and store): the LDS
+  // part first (its registers are handed back as soon as the values are
+  // parked), then the register part.
+  RawVec<T, VEC> parked[NS > 0 ? NS : 1];
+#pragma unroll
+  for (int k = 0; k < NS; ++k) {
+    const uint32_t v = static_cast<uint32_t>(NR + k) * kOnchipBlock + t;
+    parked[k] = load_raw<T, VEC>(x + onchip_offset(a, c, min(v, a.nv - 1u), VEC));
+  }
+  RawVec<T, VEC> raw[NR];
+#pragma unroll
+  for (int k = 0; k < NR; ++k) {
+    const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t;
+    raw[k] = load_raw<T, VEC>(x + onchip_offset(a, c, min(v, a.nv - 1u), VEC));
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < NS; ++k) {
+    const float part = raw_sum<T, VEC>(parked[k], 0.f);
+    s += (static_cast<uint32_t>(NR + k) * kOnchipBlock + t < a.nv) ? part : 0.f;
+    spill[k * kOnchipBlock + t] = __builtin_bit_cast(uint4, parked[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < NR; ++k) {
+    const float part = raw_sum<T, VEC>(raw[k], 0.f);
+    s += (static_cast<uint32_t>(k) * kOnchipBlock + t < a.nv) ? part : 0.f;
+  }
+  const float mean = onchip_block_sum(s, red) * a.inv_N;
+#pragma unroll
+  for (int k = 0; k < NR; ++k) keep_packed<T, VEC>(raw[k]);
+
+  float q = 0.f;
+#pragma unroll
+  for (int k = 0; k < NR; ++k) {
+    if (static_cast<uint32_t>(k) * kOnchipBlock + t < a.nv) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float d = elem_fma<T, VEC>(raw[k], j, a.one, -mean);
+        q = fmaf(d, d, q);
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < NS; ++k) {
+    if (static_cast<uint32_t>(NR + k) * kOnchipBlock + t < a.nv) {
+      const RawVec<T, VEC> r = __builtin_bit_cast(RawVec<T, VEC>, spill[k * kOnchipBlock + t]);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float d = elem_fma<T, VEC>(r, j, a.one, -mean);
+        q = fmaf(d, d, q);
+      }
+    }
+  }
+  const float var = onchip_block_sum(q, red) * a.inv_N;
+  const float istd = inv_std(var, a.eps);
+  if (t == 0) {
+    a.mean[c] = mean;
+    a.var[c] = var;
+    if (a.rmean) a.rmean[c] = a.decay * a.rmean[c] + (1.f - a.decay) * mean;
+    if (a.rvar) a.rvar[c] = a.decay * a.rvar[c] + (1.f - a.decay) * var * a.unbias;
+  }
+#pragma unroll
+  for (int k = 0; k < NR; ++k) keep_packed<T, VEC>(raw[k]);
+  const float g = (a.gamma ? a.gamma[c] : 1.f) * istd;
+  const float b = a.beta ? a.beta[c] : 0.f;
+  const float sh = fmaf(-mean, g, b);
+
+  auto emit = [&](const RawVec<T, VEC> &r, uint32_t v) {
+    float o[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      if constexpr (sizeof(T) == 2) {
+        o[j] = elem_fma<T, VEC>(r, j, g, sh); // x*g + (b - mean*g): one mixed fma, rounded once
+      } else {
+        o[j] = fmaf(elem_fma<T, VEC>(r, j, a.one, -mean), g, b);
+      }
+    }
+    store_vec<T, VEC>(y + onchip_offset(a, c, v, VEC), o);
+  };
+  const uint32_t t2 = fresh(t);
+#pragma unroll
+  for (int k = 0; k < NR; ++k) {
+    const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t2;
+    if (v < a.nv) emit(raw[k], v);
+  }
+#pragma unroll
+  for (int k = 0; k < NS; ++k) {
+    const uint32_t v = static_cast<uint32_t>(NR + k) * kOnchipBlock + t2;
+    if (v < a.nv) emit(__builtin_bit_cast(RawVec<T, VEC>, spill[k * kOnchipBlock + t]), v);
+  }
+}
+
+
+// Backward (batch statistics).  mean/var are read; with xh = (x-mean)*istd:
+//   sdy = sum dy, sdx = sum dy*xh  (= dbeta, dgamma)
+//   dx = dy*g*istd + xh*cA + cb,  cA = -istd*g*sdx/N + 2*dvar*std/N,
+//   cb = -g*sdy*istd/N + dmean/N.
+// dy is streamed in batches of B vectors per thread, twice.
+template <typename T, int VEC, int NR, int NS, int B>
+__global__ void __launch_bounds__(kOnchipBlock)
+bn_onchip_bwd_kernel(const BnOnchipArgs a) {
+  static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors only");
+  constexpr int NL = NR + NS;
+  __shared__ float red[kOnchipBlock / kWave];
+  __shared__ uint4 spill[NS > 0 ? NS * kOnchipBlock : 1];
+  const uint32_t c = blockIdx.x;
+  const uint32_t t = threadIdx.x;
+  const T *__restrict__ x = static_cast<const T *>(a.x);
+  const T *__restrict__ dy = static_cast<const T *>(a.dy);
+  T *__restrict__ dx = static_cast<T *>(a.dx);
+
+  RawVec<T, VEC> raw[NR];
+  {
+    RawVec<T, VEC> parked[NS > 0 ? NS : 1];
+#pragma unroll
+    for (int k = 0; k < NS; ++k) {
+      const uint32_t v = static_cast<uint32_t>(NR + k) * kOnchipBlock + t;
+      parked[k] = load_raw<T, VEC>(x + onchip_offset(a, c, min(v, a.nv - 1u), VEC));
+    }
+    // Here the parked vectors are stored away before the register part is
+    // requested (its addresses wait for the last parked value): with all 25
+    // loads in flight plus the first batch of dy the kernel spills.
+    uint32_t tr = t;
+#pragma unroll
+    for (int k = 0; k < NS; ++k) {
+      const uint4 w = __builtin_bit_cast(uint4, parked[k]);
+      spill[k * kOnchipBlock + t] = w;
+      tr = fresh_after(tr, w.x);
+    }
+    __builtin_amdgcn_sched_barrier(0); // every LDS store above, every load of the register part below
+    // The parked values must be read back from LDS, not forwarded from the
+    // registers that held them (which would keep those registers alive).
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int k = 0; k < NR; ++k) {
+      const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + tr;
+      raw[k] = load_raw<T, VEC>(x + onchip_offset(a, c, min(v, a.nv - 1u), VEC));
+    }
+  }
+  const float mean = a.mean[c];
+  const float vpe = a.var[c] + a.eps;
+  const float istd = 1.0f / sqrtf(vpe);
+  const float nmi = -mean * istd;
+
+  // (k is a compile-time constant after unrolling; tid is the batch's own
+  // copy of the thread index, so that the LDS reads of a batch are not issued
+  // before the batch before it is done)
+  auto xvec = [&](int k, uint32_t tid) -> RawVec<T, VEC> {
+    if (k < NR) return raw[k < NR ? k : 0];
+    return __builtin_bit_cast(RawVec<T, VEC>, spill[(k - NR) * kOnchipBlock + tid]);
+  };
+
+  float sdy = 0.f, sdx = 0.f;
+#pragma unroll
+  for (int k0 = 0; k0 < NL; k0 += B) {
+    const uint32_t t1 = fresh_after(t, sdx);
+    RawVec<T, VEC> d[B];
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      const int k = k0 + b;
+      d[b] = zero_raw<T, VEC>();
+      if (k < NL) { // compile-time
+        const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t1;
+        d[b] = load_raw<T, VEC>(dy + onchip_offset(a, c, min(v, a.nv - 1u), VEC));
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      const int k = k0 + b;
+      if (k < NL) {
+        const RawVec<T, VEC> xr = xvec(k, t1);
+        float py = raw_sum<T, VEC>(d[b], 0.f), px = 0.f;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float xh = norm_elem<T, VEC>(xr, j, mean, istd, nmi);
+          px = elem_fma<T, VEC>(d[b], j, xh, px);
+        }
+        const bool ok = static_cast<uint32_t>(k) * kOnchipBlock + t < a.nv;
+        sdy += ok ? py : 0.f;
+        sdx += ok ? px : 0.f;
+      }
+    }
+    // keep the next batch's loads below this point: hoisted, the batches'
+    // registers add up and spill
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  sdy = onchip_block_sum(sdy, red);
+  sdx = onchip_block_sum(sdx, red);
+  if (t == 0) {
+    if (a.dgamma) a.dgamma[c] = sdx + (a.accum_g ? a.dgamma[c] : 0.f);
+    if (a.dbeta) a.dbeta[c] = sdy + (a.accum_b ? a.dbeta[c] : 0.f);
+  }
+  if (dx == nullptr) return;
+#pragma unroll
+  for (int k = 0; k < NR; ++k) forget<T, VEC>(raw[k]);
+  const float g = a.gamma ? a.gamma[c] : 1.f;
+  const float gi = g * istd;
+  const float cA = -istd * g * sdx * a.inv_N + (a.dvar ? 2.f * a.dvar[c] * (vpe * istd) * a.inv_N : 0.f);
+  const float cb = -g * sdy * istd * a.inv_N + (a.dmean ? a.dmean[c] * a.inv_N : 0.f);
+  float last = cb; // something the previous batch computed
+#pragma unroll
+  for (int k0 = 0; k0 < NL; k0 += B) {
+    const uint32_t t2 = fresh_after(t, last);
+    RawVec<T, VEC> d[B];
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      const int k = k0 + b;
+      d[b] = zero_raw<T, VEC>();
+      if (k < NL) { // compile-time
+        const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t2;
+        d[b] = load_raw<T, VEC>(dy + onchip_offset(a, c, min(v, a.nv - 1u), VEC));
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+      const int k = k0 + b;
+      const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t2;
+      if (k < NL && v < a.nv) {
+        const RawVec<T, VEC> xr = xvec(k, t2);
+        float o[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float xh = norm_elem<T, VEC>(xr, j, mean, istd, nmi);
+          o[j] = elem_fma<T, VEC>(d[b], j, gi, fmaf(xh, cA, cb));
+        }
+        T *dst = dx + onchip_offset(a, c, v, VEC);
+        if (a.accum_dx) {
+          float old[VEC];
+          load_vec<T, VEC>(dst, old);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) o[j] += old[j];
+        }
+        store_vec<T, VEC>(dst, o);
+        last = o[0];
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+template <typename T, int VEC>
+int run_onchip_fwd(int nl, const BnOnchipArgs &a, hipStream_t st) {
+#define ONCHIP_CASE(NR, NS)                                                                      \
+  if (nl <= (NR) + (NS)) {                                                                       \
+    NBLAHIP_LAUNCH("bn_onchip_fwd_kernel", (bn_onchip_fwd_kernel<T, VEC, NR, NS>), dim3(a.C),    \
+                   dim3(kOnchipBlock), 0, st, a);                                                \
+    return last_launch_status();                                                                 \
+  }
+  ONCHIP_CASE(10, 0)
+  ONCHIP_CASE(12, 0)
+  ONCHIP_CASE(14, 0)
+  ONCHIP_CASE(16, 0)
+  ONCHIP_CASE(16, 3)
+  ONCHIP_CASE(16, 6)
+  ONCHIP_CASE(16, 9)
+#undef ONCHIP_CASE
+  return NBLAHIP_EINVAL;
+}
+
+template <typename T, int VEC>
+int run_onchip_bwd(int nl, const BnOnchipArgs &a, hipStream_t st) {
+#define ONCHIP_CASE(NR, NS)                                                                      \
+  if (nl <= (NR) + (NS)) {                                                                       \
+    NBLAHIP_LAUNCH("bn_onchip_bwd_kernel", (bn_onchip_bwd_kernel<T, VEC, NR, NS, 4>),            \
+                   dim3(a.C), dim3(kOnchipBlock), 0, st, a);                                     \
+    return last_launch_status();                                                                 \
+  }
+  ONCHIP_CASE(10, 0)
+  ONCHIP_CASE(12, 0)
+  ONCHIP_CASE(14, 0)
+  ONCHIP_CASE(12, 3)
+  ONCHIP_CASE(12, 6)
+#undef ONCHIP_CASE
+  return NBLAHIP_EINVAL;
+}
+
+// Shape test shared by both directions; fills the common arguments.
+bool onchip_args(const BnProblem &p, bool backward, BnOnchipArgs &a, int &nl) {
+  if (!tune_int("BN_ONCHIP", 1)) return false;
+  if (p.size2 <= 1 || p.relu || p.z || p.y || p.dz || p.sums_out || p.sums_in) return false;
+  const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
+  if (p.size2 % vec != 0 || !aligned16(p.x) || (p.out && !aligned16(p.out))) return false;
+  if (backward && !aligned16(p.dy)) return false;
+  const int64_t nv = p.size0 * (p.size2 / vec);
+  nl = static_cast<int>((nv + kOnchipBlock - 1) / kOnchipBlock);
+  // up to 8 loads per thread the row kernels take the channel; above 25 it
+  // does not fit
+  if (nl <= 8 || nl > 25) return false;
+  // a block is alone on its CU: fewer channels than (nearly all) CUs idle the rest
+  if (p.C * 8 < static_cast<int64_t>(device_cus()) * 7) return false;
+  a = BnOnchipArgs{};
+  a.x = p.x;
+  a.gamma = p.gamma;
+  a.C = static_cast<uint32_t>(p.C);
+  a.size2 = static_cast<uint32_t>(p.size2);
+  a.nv = static_cast<uint32_t>(nv);
+  a.vpp = FastDiv(static_cast<uint32_t>(p.size2 / vec));
+  const double N = static_cast<double>(p.size0) * static_cast<double>(p.size2);
+  a.inv_N = static_cast<float>(1.0 / N);
+  a.unbias = static_cast<float>(N / (N - 1.0));
+  a.decay = p.decay;
+  a.eps = p.eps;
+  a.one = 1.0f;
+  return true;
+}
+
+} // namespace
+
+bool bn_onchip_bwd(const BnProblem &p, hipStream_t st, int *status) {
+  BnOnchipArgs a;
+  int nl = 0;
+  if (!p.batch_stat || (!p.out && !p.dgamma && !p.dbeta)) return false;
+  if (!onchip_args(p, true, a, nl)) return false;
+  // Beside x a thread holds a batch of dy: the layouts beyond 18 vectors per
+  // thread spill and lose to the split reduction (25 vectors, float
+  // [32,256,56,56]: 76 vs 71 us).
+  if (nl > tune_int("BN_ONCHIP_BWD_MAX", 18)) return false;
+  a.dy = p.dy;
+  a.dx = p.out;
+  a.mean = const_cast<float *>(p.mean);
+  a.var = const_cast<float *>(p.var);
+  a.dmean = p.dmean;
+  a.dvar = p.dvar;
+  a.dgamma = p.dgamma;
+  a.dbeta = p.dbeta;
+  a.accum_dx = p.accum_dx;
+  a.accum_g = p.accum_g;
+  a.accum_b = p.accum_b;
+  *status = p.dtype == NBLAHIP_F16 ? run_onchip_bwd<__half, 8>(nl, a, st)
+                                   : run_onchip_bwd<float, 4>(nl, a, st);
+  return true;
+}
+
+bool bn_onchip_fwd_train(const BnProblem &p, hipStream_t st, int *status) {
+  BnOnchipArgs a;
+  int nl = 0;
+  if (!p.out || !onchip_args(p, false, a, nl)) return false;
+  a.y = p.out;
+  a.beta = p.beta;
+  a.mean = p.batch_mean;
+  a.var = p.batch_var;
+  a.rmean = p.rmean;
+  a.rvar = p.rvar;
+  *status = p.dtype == NBLAHIP_F16 ? run_onchip_fwd<__half, 8>(nl, a, st)
+                                   : run_onchip_fwd<float, 4>(nl, a, st);
+  return true;
+}
+
+} // namespace nblahip

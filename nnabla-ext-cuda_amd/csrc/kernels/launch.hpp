@@ -126,6 +126,11 @@ struct BnProblem {
 // registers (one launch, x and dy cross HBM once per direction): false when
 // the shape or the flags are not theirs, else *status holds the launch result.
 bool bn_rows_fwd_train(const BnProblem &p, hipStream_t st, int *status);
+// Training forward with a channel of up to 25600 vectors held on one CU
+// (registers and LDS), for tensors with a channel per CU (bn_onchip.hip).
+bool bn_onchip_fwd_train(const BnProblem &p, hipStream_t st, int *status);
+// ... and the backward with x held there and dy streamed past it twice.
+bool bn_onchip_bwd(const BnProblem &p, hipStream_t st, int *status);
 bool bn_rows_bwd(const BnProblem &p, hipStream_t st, int *status);
 // The same for channel-last tensors of few rows (gn_cl_rows.hip): a block per
 // channel vector keeps its column in registers.

@@ -292,3 +292,50 @@ def test_bn_argument_errors():
                                   y.data_ptr(), 0, 8, 36, 1e-5, 0, s) == 0
     with pytest.raises(K.NblaHipError):
         K.check(-3)
+
+
+# A channel held on one CU (registers, then LDS): needs a channel for (nearly)
+# every CU and 8193 to 25600 vectors per channel.  N picks the vectors per
+# thread (9 to 25), hence the register/LDS layout; odd N leaves the last slot
+# partly filled.  Backward layouts end at 18 vectors per thread (beyond, the
+# split reduction runs), so 19+ checks the hand-over too.
+ONCHIP_CASES = [(torch.float32, 33), (torch.float32, 47), (torch.float32, 55), (torch.float32, 63),
+                (torch.float32, 71), (torch.float32, 85), (torch.float32, 99),
+                (torch.float16, 67), (torch.float16, 111), (torch.float16, 141),
+                (torch.float16, 197)]
+
+
+@pytest.mark.parametrize("dtype,n", ONCHIP_CASES)
+def test_bn_channel_on_chip(dtype, n):
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    c = (cus * 7 + 7) // 8
+    shape, axis = (n, c, 32, 32), 1
+    dn = dtype_name(dtype)
+    x, dy, g, b, rm, rv = make_bn(shape, axis, dtype, 21, mean=1.0, std=2.0)
+    y_r, m_r, v_r, rm_r, rv_r = R.bn_forward_batch(x, b, g, rm, rv, axis, 0.9, 1e-5)
+    rng = np.random.default_rng(22)
+    dm, dv = rng.standard_normal(c), rng.standard_normal(c)
+    dx_r, dg_r, db_r = R.bn_backward_batch(x, dy, g, m_r, v_r, axis, 1e-5, dm, dv)
+    xd, dyd, gd, bd = to_dev(x, dtype), to_dev(dy, dtype), to_dev(g), to_dev(b)
+    rmd, rvd = to_dev(rm), to_dev(rv)
+    y, m, v = K.bn_forward_batch(xd, bd, gd, rmd, rvd, axis, 0.9, 1e-5)
+    assert_close(to_np(y), y_r, dn, "y", "y")
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    assert_close(to_np(rmd), rm_r, dn, "stat", "running_mean")
+    assert_close(to_np(rvd), rv_r, dn, "stat", "running_var")
+    if dtype == torch.float32:  # accumulated onto an existing gradient
+        pre = torch.randn_like(xd)
+        dx, dg, db = K.bn_backward(xd, dyd, gd, m, v, axis, 1e-5, dmean=to_dev(dm), dvar=to_dev(dv),
+                                   dx=pre.clone(), accum=(True, False, False))
+        assert_close(to_np(dx) - to_np(pre), dx_r, dn, "grad", "dx (accumulated)")
+    else:
+        dx, dg, db = K.bn_backward(xd, dyd, gd, m, v, axis, 1e-5, dmean=to_dev(dm), dvar=to_dev(dv))
+        assert_close(to_np(dx), dx_r, dn, "grad", "dx")
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
+    # run to run, and without dx
+    y2, _, _ = K.bn_forward_batch(xd, bd, gd, to_dev(rm), to_dev(rv), axis, 0.9, 1e-5)
+    assert torch.equal(y2, y)
+    _, dg2, db2 = K.bn_backward(xd, dyd, gd, m, v, axis, 1e-5, need=(False, True, True))
+    assert torch.equal(dg2, dg) and torch.equal(db2, db)
