@@ -46,6 +46,7 @@ struct BnOnchipArgs {
   int accum_dx, accum_g, accum_b;
 };
 
+template <int TB = kOnchipBlock>
 __device__ __forceinline__ float onchip_block_sum(float v, float *red) {
   v = wave_sum(v);
   const int wave = threadIdx.x / kWave;
@@ -54,7 +55,7 @@ __device__ __forceinline__ float onchip_block_sum(float v, float *red) {
   lds_barrier();
   float t = 0.f;
 #pragma unroll
-  for (int i = 0; i < kOnchipBlock / kWave; ++i) t += red[i];
+  for (int i = 0; i < TB / kWave; ++i) t += red[i];
   return t;
 }
 
@@ -209,13 +210,17 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
 //   dx = dy*g*istd + xh*cA + cb,  cA = -istd*g*sdx/N + 2*dvar*std/N,
 //   cb = -g*sdy*istd/N + dmean/N.
 // dy is streamed in batches of B vectors per thread, twice.
-template <typename T, int VEC, int NR, int NS, int B>
-__global__ void __launch_bounds__(kOnchipBlock)
+// TB threads per block: a CU's 512 KB of registers are 128 per thread for 1024
+// threads and 256 for 512, and what a thread needs beside its data (addresses,
+// sums, a batch of dy) is paid once per thread - the long channels take 512
+// threads (and 320 bytes of LDS per thread instead of 160).
+template <typename T, int VEC, int NR, int NS, int B, int TB>
+__global__ void __launch_bounds__(TB)
 bn_onchip_bwd_kernel(const BnOnchipArgs a) {
   static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors only");
   constexpr int NL = NR + NS;
-  __shared__ float red[kOnchipBlock / kWave];
-  __shared__ uint4 spill[NS > 0 ? NS * kOnchipBlock : 1];
+  __shared__ float red[TB / kWave];
+  __shared__ uint4 spill[NS > 0 ? NS * TB : 1];
   const uint32_t c = blockIdx.x;
   const uint32_t t = threadIdx.x;
   const T *__restrict__ x = static_cast<const T *>(a.x);
@@ -227,7 +232,7 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
     RawVec<T, VEC> parked[NS > 0 ? NS : 1];
 #pragma unroll
     for (int k = 0; k < NS; ++k) {
-      const uint32_t v = static_cast<uint32_t>(NR + k) * kOnchipBlock + t;
+      const uint32_t v = static_cast<uint32_t>(NR + k) * TB + t;
       parked[k] = load_raw<T, VEC>(x + onchip_offset(a, c, min(v, a.nv - 1u), VEC));
     }
     // Here the parked vectors are stored away before the register part is
@@ -237,7 +242,7 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
 #pragma unroll
     for (int k = 0; k < NS; ++k) {
       const uint4 w = __builtin_bit_cast(uint4, parked[k]);
-      spill[k * kOnchipBlock + t] = w;
+      spill[k * TB + t] = w;
       tr = fresh_after(tr, w.x);
     }
     __builtin_amdgcn_sched_barrier(0); // every LDS store above, every load of the register part below
@@ -246,7 +251,7 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
     asm volatile("" ::: "memory");
 #pragma unroll
     for (int k = 0; k < NR; ++k) {
-      const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + tr;
+      const uint32_t v = static_cast<uint32_t>(k) * TB + tr;
       raw[k] = load_raw<T, VEC>(x + onchip_offset(a, c, min(v, a.nv - 1u), VEC));
     }
   }
@@ -260,7 +265,7 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
   // before the batch before it is done)
   auto xvec = [&](int k, uint32_t tid) -> RawVec<T, VEC> {
     if (k < NR) return raw[k < NR ? k : 0];
-    return __builtin_bit_cast(RawVec<T, VEC>, spill[(k - NR) * kOnchipBlock + tid]);
+    return __builtin_bit_cast(RawVec<T, VEC>, spill[(k - NR) * TB + tid]);
   };
 
   float sdy = 0.f, sdx = 0.f;
@@ -273,7 +278,7 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
       const int k = k0 + b;
       d[b] = zero_raw<T, VEC>();
       if (k < NL) { // compile-time
-        const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t1;
+        const uint32_t v = static_cast<uint32_t>(k) * TB + t1;
         d[b] = load_raw<T, VEC>(dy + onchip_offset(a, c, min(v, a.nv - 1u), VEC));
       }
     }
@@ -288,7 +293,7 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
           const float xh = norm_elem<T, VEC>(xr, j, mean, istd, nmi);
           px = elem_fma<T, VEC>(d[b], j, xh, px);
         }
-        const bool ok = static_cast<uint32_t>(k) * kOnchipBlock + t < a.nv;
+        const bool ok = static_cast<uint32_t>(k) * TB + t < a.nv;
         sdy += ok ? py : 0.f;
         sdx += ok ? px : 0.f;
       }
@@ -297,8 +302,8 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
     // registers add up and spill
     __builtin_amdgcn_sched_barrier(0);
   }
-  sdy = onchip_block_sum(sdy, red);
-  sdx = onchip_block_sum(sdx, red);
+  sdy = onchip_block_sum<TB>(sdy, red);
+  sdx = onchip_block_sum<TB>(sdx, red);
   if (t == 0) {
     if (a.dgamma) a.dgamma[c] = sdx + (a.accum_g ? a.dgamma[c] : 0.f);
     if (a.dbeta) a.dbeta[c] = sdy + (a.accum_b ? a.dbeta[c] : 0.f);
@@ -320,14 +325,14 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
       const int k = k0 + b;
       d[b] = zero_raw<T, VEC>();
       if (k < NL) { // compile-time
-        const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t2;
+        const uint32_t v = static_cast<uint32_t>(k) * TB + t2;
         d[b] = load_raw<T, VEC>(dy + onchip_offset(a, c, min(v, a.nv - 1u), VEC));
       }
     }
 #pragma unroll
     for (int b = 0; b < B; ++b) {
       const int k = k0 + b;
-      const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t2;
+      const uint32_t v = static_cast<uint32_t>(k) * TB + t2;
       if (k < NL && v < a.nv) {
         const RawVec<T, VEC> xr = xvec(k, t2);
         float o[VEC];
@@ -371,18 +376,19 @@ int run_onchip_fwd(int nl, const BnOnchipArgs &a, hipStream_t st) {
 }
 
 template <typename T, int VEC>
-int run_onchip_bwd(int nl, const BnOnchipArgs &a, hipStream_t st) {
-#define ONCHIP_CASE(NR, NS)                                                                      \
-  if (nl <= (NR) + (NS)) {                                                                       \
-    NBLAHIP_LAUNCH("bn_onchip_bwd_kernel", (bn_onchip_bwd_kernel<T, VEC, NR, NS, 4>),            \
-                   dim3(a.C), dim3(kOnchipBlock), 0, st, a);                                     \
+int run_onchip_bwd(int64_t nv, const BnOnchipArgs &a, hipStream_t st) {
+#define ONCHIP_CASE(NR, NS, B, TB)                                                               \
+  if (nv <= static_cast<int64_t>((NR) + (NS)) * (TB)) {                                          \
+    NBLAHIP_LAUNCH("bn_onchip_bwd_kernel", (bn_onchip_bwd_kernel<T, VEC, NR, NS, B, TB>),        \
+                   dim3(a.C), dim3(TB), 0, st, a);                                               \
     return last_launch_status();                                                                 \
   }
-  ONCHIP_CASE(10, 0)
-  ONCHIP_CASE(12, 0)
-  ONCHIP_CASE(14, 0)
-  ONCHIP_CASE(12, 3)
-  ONCHIP_CASE(12, 6)
+  ONCHIP_CASE(10, 0, 4, 1024)
+  ONCHIP_CASE(12, 0, 4, 1024)
+  ONCHIP_CASE(14, 0, 4, 1024)
+  ONCHIP_CASE(12, 3, 4, 1024)
+  ONCHIP_CASE(12, 6, 4, 1024)
+  ONCHIP_CASE(24, 16, 8, 512)
 #undef ONCHIP_CASE
   return NBLAHIP_EINVAL;
 }
@@ -424,10 +430,10 @@ bool bn_onchip_bwd(const BnProblem &p, hipStream_t st, int *status) {
   int nl = 0;
   if (!p.batch_stat || (!p.out && !p.dgamma && !p.dbeta)) return false;
   if (!onchip_args(p, true, a, nl)) return false;
-  // Beside x a thread holds a batch of dy: the layouts beyond 18 vectors per
-  // thread spill and lose to the split reduction (25 vectors, float
-  // [32,256,56,56]: 76 vs 71 us).
-  if (nl > tune_int("BN_ONCHIP_BWD_MAX", 18)) return false;
+  // Beside x a thread holds a batch of dy: the layouts for more than 20480
+  // vectors per channel spill and lose to the split reduction (25088 vectors,
+  // float [32,256,56,56]: 72-76 vs 71 us; half [64,256,56,56]: 115 vs 71 us).
+  if (nl > tune_int("BN_ONCHIP_BWD_MAX", 20)) return false;
   a.dy = p.dy;
   a.dx = p.out;
   a.mean = const_cast<float *>(p.mean);
@@ -439,8 +445,8 @@ bool bn_onchip_bwd(const BnProblem &p, hipStream_t st, int *status) {
   a.accum_dx = p.accum_dx;
   a.accum_g = p.accum_g;
   a.accum_b = p.accum_b;
-  *status = p.dtype == NBLAHIP_F16 ? run_onchip_bwd<__half, 8>(nl, a, st)
-                                   : run_onchip_bwd<float, 4>(nl, a, st);
+  *status = p.dtype == NBLAHIP_F16 ? run_onchip_bwd<__half, 8>(a.nv, a, st)
+                                   : run_onchip_bwd<float, 4>(a.nv, a, st);
   return true;
 }
 
