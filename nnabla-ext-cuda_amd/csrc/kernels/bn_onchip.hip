@@ -100,6 +100,8 @@ __device__ __forceinline__ uint32_t onchip_offset(const BnOnchipArgs &a, uint32_
   return (n * a.C + c) * a.size2 + w * static_cast<uint32_t>(vec);
 }
 
+} // namespace
+
 template <typename T, int VEC, int NR, int NS>
 __global__ void __launch_bounds__(kOnchipBlock)
 bn_onchip_fwd_kernel(const BnOnchipArgs a) {
@@ -355,6 +357,8 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
     __builtin_amdgcn_sched_barrier(0);
   }
 }
+
+namespace {
 
 template <typename T, int VEC>
 int run_onchip_fwd(int nl, const BnOnchipArgs &a, hipStream_t st) {
