@@ -53,9 +53,13 @@ def _ws(nbytes):
 # forward (x for the statistics, x again, y) and 5 backward.
 BN_ONCHIP_FWD = ("bn_onchip_fwd_kernel", "row_fwd_kernel_bn", "in_cl_row_fwd_kernel")
 BN_ONCHIP_BWD = {"bn_onchip_bwd_kernel": 4, "row_bwd_kernel_bn": 3, "in_cl_row_bwd_kernel": 3}
+# bn_onchip_bwd_kernel holds x of a channel on its CU and streams dy twice
+# (x, 2 dy, dx = 4 passes); of a channel beyond 20480 16-byte vectors it holds
+# 18432 and reads the rest of x twice as well.
+BN_ONCHIP_BWD_HELD, BN_ONCHIP_BWD_WHOLE = 18432, 20480
 
 
-def bn_tensor_passes(K, fwd, bwd):
+def bn_tensor_passes(K, fwd, bwd, vectors_per_channel=0):
     """(forward, backward) tensor passes of the plan the library picks for this
     workload: a pass counts when the channel cannot stay on chip between the
     statistics and the apply phase.  Read off the kernels one call launches."""
@@ -70,6 +74,8 @@ def bn_tensor_passes(K, fwd, bwd):
     for k, passes in BN_ONCHIP_BWD.items():
         if K.profile_query(k)[1]:
             pb = passes
+            if k == "bn_onchip_bwd_kernel" and vectors_per_channel > BN_ONCHIP_BWD_WHOLE:
+                pb += (vectors_per_channel - BN_ONCHIP_BWD_HELD) / vectors_per_channel
     K.check(L.nblahip_profile_enable(0))
     return pf, pb
 
@@ -131,8 +137,9 @@ def make_bn(K, shape, axis, dtype, train, mean=0.0, std=1.0, outliers=False, see
                                      bv.data_ptr(), None, None, dx.data_ptr(), dg.data_ptr(),
                                      db.data_ptr(), 0, 0, 0, s0, c, s2, 1e-5, 1, dt, ws.data_ptr(),
                                      ws.numel(), st))
-        pf, pb = bn_tensor_passes(K, fwd, bwd)
-        return fwd, bwd, pf * S, pb * S, (x, dy, gamma, beta, rm, rv, y, dx, bm, bv, dg, db, ws)
+        pf, pb = bn_tensor_passes(K, fwd, bwd, s0 * s2 * x.element_size() // 16)
+        return fwd, bwd, pf * S, int(round(pb * S)), (x, dy, gamma, beta, rm, rv, y, dx, bm, bv, dg,
+                                                      db, ws)
 
     def fwd():
         K.check(L.nblahip_bn_fwd_infer(x.data_ptr(), rm.data_ptr(), rv.data_ptr(), gamma.data_ptr(),
@@ -425,13 +432,14 @@ def cpu_baseline(budget_s=12.0):
                       f"oracle/norm_ref.c with OpenMP over channels"}
 
 
-def load_traffic():
-    """HBM bytes per launch of the dominant kernel from the committed
-    rocprofv3 --pmc summaries, or None."""
-    path = os.path.join(ROOT, "profiles", "bn_bwd_apply_planes_c2_traffic.txt")
+def load_traffic(kernel):
+    """HBM bytes per launch of a kernel of the headline workload from the
+    committed rocprofv3 --pmc summary (FETCH_SIZE and WRITE_SIZE scaled by a
+    convert kernel of known traffic), or None."""
+    path = os.path.join(ROOT, "profiles", "c2_kernel_traffic.txt")
     try:
         with open(path) as f:
-            return json.load(f).get("bn_bwd_apply_planes_kernel", {}).get("hbm_bytes_per_launch")
+            return json.load(f).get(kernel, {}).get("hbm_bytes_per_launch")
     except (OSError, ValueError):
         return None
 
@@ -488,7 +496,7 @@ def main():
         bwd()
     torch.cuda.synchronize()
     S = keep[0].numel() * keep[0].element_size()
-    kbytes = {"bn_onchip_fwd_kernel": 2 * S, "bn_onchip_bwd_kernel": 4 * S,
+    kbytes = {"bn_onchip_fwd_kernel": fb, "bn_onchip_bwd_kernel": bb,
               "bn_stats_planes_kernel": S, "bn_apply_planes_kernel": 2 * S,
               "bn_apply_planes_fused_kernel": 2 * S, "bn_bwd_reduce_planes_kernel": 2 * S,
               "bn_bwd_apply_planes_kernel": 3 * S, "bn_bwd_apply_planes_fused_kernel": 3 * S}
@@ -501,14 +509,13 @@ def main():
                 per_kernel[k]["GBps"] = round(kbytes[k] / (tot / cnt) / 1e6, 1)
     K.check(L.nblahip_profile_enable(0))
     log("per-kernel:", json.dumps(per_kernel))
-    # dominant kernel = the backward apply (3 tensor passes), fused or not
-    dom = max((k for k in per_kernel if k.startswith("bn_bwd_apply")),
-              key=lambda k: per_kernel[k]["launches"])
+    # dominant kernel = the one with the most time per step
+    dom = max((k for k in per_kernel if k in kbytes), key=lambda k: per_kernel[k]["avg_us"])
     achieved = per_kernel[dom]["GBps"]
     roofline = {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "avg_us": per_kernel[dom]["avg_us"], "algorithmic_bytes": 3 * S,
-                "traffic": load_traffic()}
+                "avg_us": per_kernel[dom]["avg_us"], "algorithmic_bytes": kbytes[dom],
+                "traffic": load_traffic(dom)}
 
     result = {
         "metric": "BN training fwd+bwd achieved algorithmic HBM bandwidth (us/call in ms_per_step), 1 MI355X",
@@ -518,10 +525,12 @@ def main():
         "config": {"workload": "BatchNormalization training fwd+bwd fp32 NCHW x[32,256,56,56] "
                                "(benchmark configuration 2), decay_rate 0.9, eps 1e-5",
                    "algorithmic_bytes_per_step": fb + bb,
-                   "tensor_passes": {"forward": fb // S, "backward": bb // S,
+                   "tensor_passes": {"forward": round(fb / S, 3), "backward": round(bb / S, 3),
                                      "note": "a pass counts when the channel cannot stay on chip "
                                              "between statistics and apply; the forward keeps "
-                                             "its channel in registers and LDS (x read once)"},
+                                             "its channel in registers and LDS (x read once), the "
+                                             "backward 18432 of its 25088 vectors (that part of x "
+                                             "read once, the rest and dy twice)"},
                    "pct_of_hbm_peak": round(value / HBM_PEAK_GBS * 100, 1)},
         "roofline": roofline,
         "per_kernel": per_kernel,

@@ -216,7 +216,11 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
 // threads and 256 for 512, and what a thread needs beside its data (addresses,
 // sums, a batch of dy) is paid once per thread - the long channels take 512
 // threads (and 320 bytes of LDS per thread instead of 160).
-template <typename T, int VEC, int NR, int NS, int B, int TB>
+// OVER: the channel is longer than the NR + NS slots held on chip; the
+// vectors beyond them are streamed like dy (x and dy read in both passes, a
+// rolled loop of small batches), so only the held part saves its second read:
+// (18432 / nv) S of the 5 S.
+template <typename T, int VEC, int NR, int NS, int B, int TB, bool OVER = false>
 __global__ void __launch_bounds__(TB)
 bn_onchip_bwd_kernel(const BnOnchipArgs a) {
   static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors only");
@@ -304,6 +308,31 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
     // registers add up and spill
     __builtin_amdgcn_sched_barrier(0);
   }
+  if constexpr (OVER) {
+    constexpr int BO = 2;
+#pragma unroll 1
+    for (uint32_t v0 = static_cast<uint32_t>(NL) * TB; v0 < a.nv; v0 += BO * TB) {
+      RawVec<T, VEC> xo[BO], d[BO];
+#pragma unroll
+      for (int b = 0; b < BO; ++b) {
+        const uint32_t off = onchip_offset(a, c, min(v0 + b * TB + t, a.nv - 1u), VEC);
+        xo[b] = load_raw<T, VEC>(x + off);
+        d[b] = load_raw<T, VEC>(dy + off);
+      }
+#pragma unroll
+      for (int b = 0; b < BO; ++b) {
+        float py = raw_sum<T, VEC>(d[b], 0.f), px = 0.f;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float xh = norm_elem<T, VEC>(xo[b], j, mean, istd, nmi);
+          px = elem_fma<T, VEC>(d[b], j, xh, px);
+        }
+        const bool ok = v0 + b * TB + t < a.nv;
+        sdy += ok ? py : 0.f;
+        sdx += ok ? px : 0.f;
+      }
+    }
+  }
   sdy = onchip_block_sum<TB>(sdy, red);
   sdx = onchip_block_sum<TB>(sdx, red);
   if (t == 0) {
@@ -356,6 +385,39 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
     }
     __builtin_amdgcn_sched_barrier(0);
   }
+  if constexpr (OVER) {
+    constexpr int BO = 2;
+#pragma unroll 1
+    for (uint32_t v0 = static_cast<uint32_t>(NL) * TB; v0 < a.nv; v0 += BO * TB) {
+      RawVec<T, VEC> xo[BO], d[BO];
+      uint32_t off[BO];
+#pragma unroll
+      for (int b = 0; b < BO; ++b) {
+        off[b] = onchip_offset(a, c, min(v0 + b * TB + t, a.nv - 1u), VEC);
+        xo[b] = load_raw<T, VEC>(x + off[b]);
+        d[b] = load_raw<T, VEC>(dy + off[b]);
+      }
+#pragma unroll
+      for (int b = 0; b < BO; ++b) {
+        if (v0 + b * TB + t < a.nv) {
+          float o[VEC];
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            const float xh = norm_elem<T, VEC>(xo[b], j, mean, istd, nmi);
+            o[j] = elem_fma<T, VEC>(d[b], j, gi, fmaf(xh, cA, cb));
+          }
+          T *dst = dx + off[b];
+          if (a.accum_dx) {
+            float old[VEC];
+            load_vec<T, VEC>(dst, old);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) o[j] += old[j];
+          }
+          store_vec<T, VEC>(dst, o);
+        }
+      }
+    }
+  }
 }
 
 namespace {
@@ -394,11 +456,14 @@ int run_onchip_bwd(int64_t nv, const BnOnchipArgs &a, hipStream_t st) {
   ONCHIP_CASE(12, 6, 4, 1024)
   ONCHIP_CASE(24, 16, 8, 512)
 #undef ONCHIP_CASE
-  return NBLAHIP_EINVAL;
+  // longer channels: 18 slots held, the rest streamed
+  NBLAHIP_LAUNCH("bn_onchip_bwd_kernel", (bn_onchip_bwd_kernel<T, VEC, 12, 6, 4, 1024, true>),
+                 dim3(a.C), dim3(1024), 0, st, a);
+  return last_launch_status();
 }
 
 // Shape test shared by both directions; fills the common arguments.
-bool onchip_args(const BnProblem &p, bool backward, BnOnchipArgs &a, int &nl) {
+bool onchip_args(const BnProblem &p, bool backward, BnOnchipArgs &a, int &nl, int max_nl = 25) {
   if (!tune_int("BN_ONCHIP", 1)) return false;
   if (p.size2 <= 1 || p.relu || p.z || p.y || p.dz || p.sums_out || p.sums_in) return false;
   const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
@@ -408,7 +473,7 @@ bool onchip_args(const BnProblem &p, bool backward, BnOnchipArgs &a, int &nl) {
   nl = static_cast<int>((nv + kOnchipBlock - 1) / kOnchipBlock);
   // up to 8 loads per thread the row kernels take the channel; above 25 it
   // does not fit
-  if (nl <= 8 || nl > 25) return false;
+  if (nl <= 8 || nl > max_nl) return false;
   // a block is alone on its CU: fewer channels than (nearly all) CUs idle the rest
   if (p.C * 8 < static_cast<int64_t>(device_cus()) * 7) return false;
   a = BnOnchipArgs{};
@@ -433,11 +498,11 @@ bool bn_onchip_bwd(const BnProblem &p, hipStream_t st, int *status) {
   BnOnchipArgs a;
   int nl = 0;
   if (!p.batch_stat || (!p.out && !p.dgamma && !p.dbeta)) return false;
-  if (!onchip_args(p, true, a, nl)) return false;
-  // Beside x a thread holds a batch of dy: the layouts for more than 20480
+  // Beside x a thread holds a batch of dy: layouts that hold more than 20480
   // vectors per channel spill and lose to the split reduction (25088 vectors,
   // float [32,256,56,56]: 72-76 vs 71 us; half [64,256,56,56]: 115 vs 71 us).
-  if (nl > tune_int("BN_ONCHIP_BWD_MAX", 20)) return false;
+  // Longer channels keep 18432 vectors on chip and stream the rest.
+  if (!onchip_args(p, true, a, nl, tune_int("BN_ONCHIP_BWD_MAX", 48))) return false;
   a.dy = p.dy;
   a.dx = p.out;
   a.mean = const_cast<float *>(p.mean);
