@@ -57,6 +57,9 @@ BN_ONCHIP_BWD = {"bn_onchip_bwd_kernel": 4, "row_bwd_kernel_bn": 3, "in_cl_row_b
 # (x, 2 dy, dx = 4 passes); of a channel beyond 20480 16-byte vectors it holds
 # 18432 and reads the rest of x twice as well.
 BN_ONCHIP_BWD_HELD, BN_ONCHIP_BWD_WHOLE = 18432, 20480
+# bn_onchip_fwd_kernel holds up to 25600 vectors of a channel; the rest of a
+# longer channel is read twice.
+BN_ONCHIP_FWD_HELD = 25600
 
 
 def bn_tensor_passes(K, fwd, bwd, vectors_per_channel=0):
@@ -70,6 +73,8 @@ def bn_tensor_passes(K, fwd, bwd, vectors_per_channel=0):
     bwd()
     torch.cuda.synchronize()
     pf = 2 if any(K.profile_query(k)[1] for k in BN_ONCHIP_FWD) else 3
+    if K.profile_query("bn_onchip_fwd_kernel")[1] and vectors_per_channel > BN_ONCHIP_FWD_HELD:
+        pf += (vectors_per_channel - BN_ONCHIP_FWD_HELD) / vectors_per_channel
     pb = 5
     for k, passes in BN_ONCHIP_BWD.items():
         if K.profile_query(k)[1]:
@@ -138,7 +143,7 @@ def make_bn(K, shape, axis, dtype, train, mean=0.0, std=1.0, outliers=False, see
                                      db.data_ptr(), 0, 0, 0, s0, c, s2, 1e-5, 1, dt, ws.data_ptr(),
                                      ws.numel(), st))
         pf, pb = bn_tensor_passes(K, fwd, bwd, s0 * s2 * x.element_size() // 16)
-        return fwd, bwd, pf * S, int(round(pb * S)), (x, dy, gamma, beta, rm, rv, y, dx, bm, bv, dg,
+        return fwd, bwd, int(round(pf * S)), int(round(pb * S)), (x, dy, gamma, beta, rm, rv, y, dx, bm, bv, dg,
                                                       db, ws)
 
     def fwd():

@@ -102,7 +102,14 @@ __device__ __forceinline__ uint32_t onchip_offset(const BnOnchipArgs &a, uint32_
 
 } // namespace
 
-template <typename T, int VEC, int NR, int NS>
+// OVER: the channel is longer than the NR + NS slots held on chip.  The mean
+// of the held part serves as the shift K of the whole channel: the held part's
+// second pass and ONE read of the rest accumulate sum (x - K) and
+// sum (x - K)^2, from which mean = K + s1/N and var = q/N - (s1/N)^2 (K is the
+// mean of 25600 vectors of the same channel, so the subtracted square is tiny
+// against the variance: no cancellation).  The rest is read a second time for
+// y: 2 S + (1 - 25600 / nv) S instead of 3 S.
+template <typename T, int VEC, int NR, int NS, bool OVER = false>
 __global__ void __launch_bounds__(kOnchipBlock)
 bn_onchip_fwd_kernel(const BnOnchipArgs a) {
   static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors only");
@@ -141,11 +148,14 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
     const float part = raw_sum<T, VEC>(raw[k], 0.f);
     s += (static_cast<uint32_t>(k) * kOnchipBlock + t < a.nv) ? part : 0.f;
   }
-  const float mean = onchip_block_sum(s, red) * a.inv_N;
+  // (OVER: the shift K, over the held elements only)
+  constexpr uint32_t kHeld = static_cast<uint32_t>(NR + NS) * kOnchipBlock;
+  float mean = onchip_block_sum(s, red) * (OVER ? 1.0f / (static_cast<float>(kHeld) * VEC) : a.inv_N);
 #pragma unroll
   for (int k = 0; k < NR; ++k) keep_packed<T, VEC>(raw[k]);
 
   float q = 0.f;
+  float s1 = 0.f; // OVER: sum (x - K), the held part's rounding residue included
 #pragma unroll
   for (int k = 0; k < NR; ++k) {
     if (static_cast<uint32_t>(k) * kOnchipBlock + t < a.nv) {
@@ -153,6 +163,7 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
       for (int j = 0; j < VEC; ++j) {
         const float d = elem_fma<T, VEC>(raw[k], j, a.one, -mean);
         q = fmaf(d, d, q);
+        if constexpr (OVER) s1 += d;
       }
     }
   }
@@ -164,10 +175,39 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
       for (int j = 0; j < VEC; ++j) {
         const float d = elem_fma<T, VEC>(r, j, a.one, -mean);
         q = fmaf(d, d, q);
+        if constexpr (OVER) s1 += d;
       }
     }
   }
-  const float var = onchip_block_sum(q, red) * a.inv_N;
+  if constexpr (OVER) {
+    constexpr int BO = 4;
+#pragma unroll 1
+    for (uint32_t v0 = kHeld; v0 < a.nv; v0 += BO * kOnchipBlock) {
+      RawVec<T, VEC> xo[BO];
+#pragma unroll
+      for (int b = 0; b < BO; ++b)
+        xo[b] = load_raw<T, VEC>(x + onchip_offset(a, c, min(v0 + b * kOnchipBlock + t, a.nv - 1u), VEC));
+#pragma unroll
+      for (int b = 0; b < BO; ++b) {
+        float ps = 0.f, pq = 0.f;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float d = elem_fma<T, VEC>(xo[b], j, a.one, -mean);
+          ps += d;
+          pq = fmaf(d, d, pq);
+        }
+        const bool ok = v0 + b * kOnchipBlock + t < a.nv;
+        s1 += ok ? ps : 0.f;
+        q += ok ? pq : 0.f;
+      }
+    }
+    s1 = onchip_block_sum(s1, red) * a.inv_N; // mean - K
+  }
+  float var = onchip_block_sum(q, red) * a.inv_N;
+  if constexpr (OVER) {
+    var = fmaxf(var - s1 * s1, 0.f);
+    mean += s1;
+  }
   const float istd = inv_std(var, a.eps);
   if (t == 0) {
     a.mean[c] = mean;
@@ -203,6 +243,21 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
   for (int k = 0; k < NS; ++k) {
     const uint32_t v = static_cast<uint32_t>(NR + k) * kOnchipBlock + t2;
     if (v < a.nv) emit(__builtin_bit_cast(RawVec<T, VEC>, spill[k * kOnchipBlock + t]), v);
+  }
+  if constexpr (OVER) {
+    constexpr int BO = 4;
+#pragma unroll 1
+    for (uint32_t v0 = kHeld; v0 < a.nv; v0 += BO * kOnchipBlock) {
+      RawVec<T, VEC> xo[BO];
+#pragma unroll
+      for (int b = 0; b < BO; ++b)
+        xo[b] = load_raw<T, VEC>(x + onchip_offset(a, c, min(v0 + b * kOnchipBlock + t, a.nv - 1u), VEC));
+#pragma unroll
+      for (int b = 0; b < BO; ++b) {
+        const uint32_t v = v0 + b * kOnchipBlock + t;
+        if (v < a.nv) emit(xo[b], v);
+      }
+    }
   }
 }
 
@@ -438,7 +493,10 @@ int run_onchip_fwd(int nl, const BnOnchipArgs &a, hipStream_t st) {
   ONCHIP_CASE(16, 6)
   ONCHIP_CASE(16, 9)
 #undef ONCHIP_CASE
-  return NBLAHIP_EINVAL;
+  // longer channels: 25 slots held, the rest streamed
+  NBLAHIP_LAUNCH("bn_onchip_fwd_kernel", (bn_onchip_fwd_kernel<T, VEC, 16, 9, true>), dim3(a.C),
+                 dim3(kOnchipBlock), 0, st, a);
+  return last_launch_status();
 }
 
 template <typename T, int VEC>
@@ -502,7 +560,7 @@ bool bn_onchip_bwd(const BnProblem &p, hipStream_t st, int *status) {
   // vectors per channel spill and lose to the split reduction (25088 vectors,
   // float [32,256,56,56]: 72-76 vs 71 us; half [64,256,56,56]: 115 vs 71 us).
   // Longer channels keep 18432 vectors on chip and stream the rest.
-  if (!onchip_args(p, true, a, nl, tune_int("BN_ONCHIP_BWD_MAX", 48))) return false;
+  if (!onchip_args(p, true, a, nl, tune_int("BN_ONCHIP_BWD_MAX", 64))) return false;
   a.dy = p.dy;
   a.dx = p.out;
   a.mean = const_cast<float *>(p.mean);
@@ -522,7 +580,7 @@ bool bn_onchip_bwd(const BnProblem &p, hipStream_t st, int *status) {
 bool bn_onchip_fwd_train(const BnProblem &p, hipStream_t st, int *status) {
   BnOnchipArgs a;
   int nl = 0;
-  if (!p.out || !onchip_args(p, false, a, nl)) return false;
+  if (!p.out || !onchip_args(p, false, a, nl, tune_int("BN_ONCHIP_FWD_MAX", 64))) return false;
   a.y = p.out;
   a.beta = p.beta;
   a.mean = p.batch_mean;
