@@ -9,8 +9,9 @@ inputs resident in HBM.
 
 Prints ONE JSON line.  `value` is algorithmic GB/s of the whole step (the
 tensor passes the chosen plan makes: forward x + y with the channel held on
-chip, else x twice + y; backward x and dy twice + dx);
-`roofline` is the dominant kernel (backward apply: x, dy in, dx out) timed with
+chip, else x twice + y; backward dy twice + dx + x once for the part of the
+channel held on chip, twice for the rest);
+`roofline` is the kernel with the most time per step (the backward), timed with
 HIP events on the launch stream in a second region of the same K steps;
 `cpu_baseline` is the C restatement of the reference arithmetic
 (oracle/norm_ref.c) on the same workload on the host cores; `configs` lists
