@@ -1,22 +1,31 @@
-// BatchNormalization training forward with a whole channel held on one CU:
-// registers first, LDS for what exceeds them.  One 1024-thread block per
-// channel reads its N planes once, reduces, and writes y: x crosses the memory
-// system once (2 S per call) where the split reduction reads it twice (3 S).
+// BatchNormalization training with a channel held on one CU: registers first,
+// LDS for what exceeds them.  One 1024-thread block per channel reads its N
+// planes once, reduces, and writes y: x crosses the memory system once (2 S
+// per call) where the split reduction reads it twice (3 S).
 //
 // A CU holds 512 KB of vector registers and 160 KB of LDS; a 1024-thread block
 // may use 128 registers per thread, of which NR 16-byte vectors (4 registers
 // each) are data, and NS more vectors per thread live in LDS (each thread
 // reads back only what it wrote: no barrier, no bank conflict).  NR + NS = 25
 // covers 25600 vectors = 400 KB per channel: [32, C, 56, 56] in float,
-// [64, C, 56, 56] in half.
+// [64, C, 56, 56] in half.  A longer channel keeps that many vectors and
+// streams the rest (read twice, as in the split reduction).
 //
 // The backward keeps x on the CU the same way and streams dy past it twice
 // (sums, then dx): x once, dy twice, dx once = 4 S where the split reduction
 // moves 5 S; dgamma/dbeta are written by the channel's block, no finalize.
+// Beside x a thread needs a batch of dy, so it holds fewer vectors: 18432 per
+// channel with 1024 threads, 20480 with 512; the rest of x is streamed with dy.
 //
 // Worth it only when there is a channel for (nearly) every CU: the block is
 // alone on its CU, so fewer channels than CUs leave the rest of the chip idle
 // and the split reduction wins.
+//
+// The kernels are fully unrolled over the slots of a thread, and most of what
+// looks odd below (opaque copies of the thread index, vectors hidden from the
+// optimiser, addresses tied to earlier results) keeps the compiler from
+// holding across the passes what is cheaper to compute again: each such value
+// costs a register in every one of 1024 threads, and the layouts leave none.
 #include <algorithm>
 
 #include "common.cuh"
