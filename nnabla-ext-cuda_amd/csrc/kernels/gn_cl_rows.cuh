@@ -53,6 +53,11 @@ struct GnClArgs {
   const void *y;
   void *dz;
   int accum_dz;
+  // Wide forward kernels (a block takes several neighbouring groups / channel
+  // vectors): G counts the blocks per sample there, groups the real groups
+  // per sample, chunk the vectors a block covers per position.
+  int groups;
+  FastDiv chunk;
 };
 
 constexpr int kXcds = 8;
@@ -532,6 +537,222 @@ in_cl_row_bwd_kernel(const GnClArgs a) {
         for (int j = 0; j < VEC; ++j) o[j] += old[j];
       }
       store_vec<T, VEC, false>(p, o);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Wide forward kernels.  A 16-byte vector is an eighth of the 128-byte line
+// that L2 hands to the CU: with one group (or channel vector) per block every
+// line crosses that path once per sharer, and the forward runs at the rate of
+// that path, not of HBM (the same 33 MB tensor: 24 us at 16-byte pieces per
+// position, 17 us at 32, 13.5 us at 64).  Here a block takes GPB neighbouring
+// groups (CVB channel vectors): its threads read 32- or 64-byte pieces.  The
+// statistics stay per group (per channel), so the block sums are segmented:
+// a butterfly over the lanes that hold the same piece of the chunk, then LDS.
+// ---------------------------------------------------------------------------
+template <typename T, int VEC, int NL, int TPR, int CVB>
+__global__ void __launch_bounds__(TPR)
+in_cl_wide_fwd_kernel(const GnClArgs a) {
+  constexpr int NW = TPR / kWave;
+  constexpr uint32_t PST = TPR / CVB; // positions a block covers per load
+  __shared__ float lds[NW][CVB][VEC];
+  const int unit = gn_cl_unit(a);
+  if (unit < 0) return;
+  const uint32_t n = static_cast<uint32_t>(unit) / a.G, cb = static_cast<uint32_t>(unit) % a.G;
+  const uint32_t cvx = threadIdx.x % CVB, pos0 = threadIdx.x / CVB;
+  const uint32_t ch = (cb * CVB + cvx) * VEC;
+  const T *__restrict__ x = static_cast<const T *>(a.x) + static_cast<size_t>(n) * a.P * a.C + ch;
+  T *__restrict__ y = static_cast<T *>(a.out) + static_cast<size_t>(n) * a.P * a.C + ch;
+
+  RawVec<T, VEC> raw[NL];
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = pos0 + k * PST;
+    const bool ok = pos < static_cast<uint32_t>(a.P);
+    raw[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + static_cast<size_t>(ok ? pos : 0u) * a.C));
+  }
+  float gam[VEC], bet[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    gam[j] = a.gamma ? a.gamma[ch + j] : 1.f;
+    bet[j] = a.beta ? a.beta[ch + j] : 0.f;
+  }
+  // sums over the threads with the same channel vector (lane % CVB == cvx)
+  auto block_sums = [&](float (&v)[VEC]) {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+#pragma unroll
+      for (int off = CVB; off < kWave; off <<= 1) v[j] += __shfl_xor(v[j], off);
+    }
+    lds_barrier(); // previous readers of lds are done
+    if (lane < CVB) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) lds[wave][lane][j] = v[j];
+    }
+    lds_barrier();
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      float t = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) t += lds[w][cvx][j];
+      v[j] = t;
+    }
+  };
+  float mean[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) mean[j] = 0.f;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) mean[j] = elem_fma<T, VEC>(raw[k], j, a.one, mean[j]);
+  }
+  block_sums(mean);
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) mean[j] *= a.inv_R;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+  float var[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) var[j] = 0.f;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    if (pos0 + k * PST < static_cast<uint32_t>(a.P)) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float d = elem_fma<T, VEC>(raw[k], j, a.one, -mean[j]);
+        var[j] = fmaf(d, d, var[j]);
+      }
+    }
+  }
+  block_sums(var);
+  float sc[VEC], sh[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    var[j] *= a.inv_R;
+    sc[j] = gam[j] * inv_std(var[j], a.eps);
+    sh[j] = fmaf(-mean[j], sc[j], bet[j]);
+  }
+  if (threadIdx.x < CVB) { // thread t < CVB holds channel vector t of the block
+    const size_t c = static_cast<size_t>(n) * a.C + ch;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      a.mean[c + j] = mean[j];
+      a.var[c + j] = var[j];
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = pos0 + k * PST;
+    if (pos < static_cast<uint32_t>(a.P)) {
+      float o[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        if constexpr (sizeof(T) == 2) {
+          o[j] = elem_fma<T, VEC>(raw[k], j, sc[j], sh[j]);
+        } else {
+          o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mean[j]), sc[j], bet[j]);
+        }
+      }
+      store_vec<T, VEC, false>(y + static_cast<size_t>(pos) * a.C, o);
+    }
+  }
+}
+
+// GroupNormalization: the chunk of a position holds GPB groups of cvg vectors
+// each; thread t owns vector t % chunk of the positions t / chunk + k * (TPR /
+// chunk).  Lanes with the same t % chunk are folded first, then the cvg lanes
+// of a group (aligned runs of a power of two), then the waves through LDS.
+template <typename T, int VEC, int NL, int TPR, int GPB>
+__global__ void __launch_bounds__(TPR)
+gn_cl_wide_fwd_kernel(const GnClArgs a) {
+  constexpr int NW = TPR / kWave;
+  __shared__ float lds[NW][GPB];
+  const int unit = gn_cl_unit(a);
+  if (unit < 0) return;
+  const uint32_t n = static_cast<uint32_t>(unit) / a.G, gb = static_cast<uint32_t>(unit) % a.G;
+  const uint32_t pos0 = a.chunk.div(threadIdx.x);
+  const uint32_t cvx = threadIdx.x - pos0 * a.chunk.d;
+  const uint32_t sg = a.cvg.div(cvx); // group of the block this thread belongs to
+  const uint32_t pstep = TPR / a.chunk.d;
+  const uint32_t ch = gb * GPB * a.cpg + cvx * VEC;
+  const T *__restrict__ x = static_cast<const T *>(a.x) + static_cast<size_t>(n) * a.P * a.C + ch;
+  T *__restrict__ y = static_cast<T *>(a.out) + static_cast<size_t>(n) * a.P * a.C + ch;
+
+  RawVec<T, VEC> raw[NL];
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = pos0 + k * pstep;
+    const bool ok = pos < static_cast<uint32_t>(a.P);
+    raw[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + static_cast<size_t>(ok ? pos : 0u) * a.C));
+  }
+  float gam[VEC], bet[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    gam[j] = a.gamma ? a.gamma[ch + j] : 1.f;
+    bet[j] = a.beta ? a.beta[ch + j] : 0.f;
+  }
+  auto group_block_sum = [&](float v) -> float {
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    for (int off = static_cast<int>(a.chunk.d); off < kWave; off <<= 1) v += __shfl_xor(v, off);
+    for (int off = 1; off < static_cast<int>(a.cvg.d); off <<= 1) v += __shfl_xor(v, off);
+    lds_barrier(); // previous readers of lds are done
+    if (lane < static_cast<int>(a.chunk.d) && cvx == sg * a.cvg.d) lds[wave][sg] = v;
+    lds_barrier();
+    float t = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) t += lds[w][sg];
+    return t;
+  };
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) s = raw_sum<T, VEC>(raw[k], s);
+  const float mean = group_block_sum(s) * a.inv_R;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+  float q = 0.f;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    if (pos0 + k * pstep < static_cast<uint32_t>(a.P)) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float d = elem_fma<T, VEC>(raw[k], j, a.one, -mean);
+        q = fmaf(d, d, q);
+      }
+    }
+  }
+  const float var = group_block_sum(q) * a.inv_R;
+  const float istd = inv_std(var, a.eps);
+  if (threadIdx.x < a.chunk.d && cvx == sg * a.cvg.d) {
+    const uint32_t u = n * static_cast<uint32_t>(a.groups) + gb * GPB + sg;
+    a.mean[u] = mean;
+    a.var[u] = var;
+  }
+#pragma unroll
+  for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+  float sc[VEC], sh[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    sc[j] = gam[j] * istd;
+    sh[j] = fmaf(-mean, sc[j], bet[j]);
+  }
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = pos0 + k * pstep;
+    if (pos < static_cast<uint32_t>(a.P)) {
+      float o[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        if constexpr (sizeof(T) == 2) {
+          o[j] = elem_fma<T, VEC>(raw[k], j, sc[j], sh[j]);
+        } else {
+          o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mean), sc[j], bet[j]);
+        }
+      }
+      store_vec<T, VEC, false>(y + static_cast<size_t>(pos) * a.C, o);
     }
   }
 }

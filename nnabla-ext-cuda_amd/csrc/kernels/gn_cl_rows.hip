@@ -191,7 +191,88 @@ int run_bwd(int dtype, const GnClCfg &c, const GnClArgs &a, hipStream_t st) {
 
 } // namespace
 
+namespace {
+
+// Wide forward (half data, planes of 1024 positions and more): the widest
+// chunk - 4 or 2 neighbouring groups / channel vectors per block, 64 or 32
+// bytes per position - that still leaves a block for every CU and fits a
+// block's registers.
+template <int W>
+int run_wide(bool instance, int tpr, int nl, const GnClArgs &a, hipStream_t st) {
+#define WIDE_CASE(NL, TPR)                                                                       \
+  if (nl == (NL) && tpr == (TPR)) {                                                              \
+    if (instance) {                                                                              \
+      NBLAHIP_LAUNCH("in_cl_wide_fwd_kernel", (in_cl_wide_fwd_kernel<__half, 8, NL, TPR, W>),    \
+                     dim3(grid_of(a)), dim3(TPR), 0, st, a);                                     \
+    } else {                                                                                     \
+      NBLAHIP_LAUNCH("gn_cl_wide_fwd_kernel", (gn_cl_wide_fwd_kernel<__half, 8, NL, TPR, W>),    \
+                     dim3(grid_of(a)), dim3(TPR), 0, st, a);                                     \
+    }                                                                                            \
+    return last_launch_status();                                                                 \
+  }
+  WIDE_CASE(4, 512)
+  WIDE_CASE(8, 512)
+  WIDE_CASE(4, 1024)
+  WIDE_CASE(8, 1024)
+#undef WIDE_CASE
+  return NBLAHIP_EINVAL;
+}
+
+bool wide_fwd(const ClProblem &p, bool aligned, hipStream_t st, int *status) {
+  if (!aligned || p.dtype != NBLAHIP_F16 || !tune_int("GN_CL_WIDE", 1)) return false;
+  if (!p.bc_gamma || !p.bc_beta || p.spatial < 1024) return false;
+  constexpr int vec = 8;
+  const bool instance = p.groups == p.channels;
+  const int64_t cpg = instance ? vec : p.channels / p.groups; // channels of one unit of the chunk
+  if (cpg % vec != 0 || p.channels % vec != 0) return false;
+  const int64_t cvg = cpg / vec;                               // vectors per unit
+  // Only 16-byte pieces gain: from 32-byte pieces on it is a wash or a loss
+  // ([64,32,32,512] in 32 groups 28.3 -> 29.9 us, [64,32,32,256] in 8 groups 13.5 -> 15.9 us).
+  if (cvg != 1) return false;
+  const int64_t per_sample = instance ? p.channels / vec : p.groups; // units per sample
+  for (int w : {4, 2}) {
+    if (per_sample % w != 0 || cvg * w > 8) continue;
+    const int64_t blocks = p.batch * (per_sample / w);
+    if (blocks < device_cus()) continue;
+    const int64_t nv = p.spatial * cvg * w; // vectors a block holds
+    for (int tpr : {512, 1024}) {
+      for (int nl : {4, 8}) {
+        if (static_cast<int64_t>(tpr) * nl < nv) continue;
+        // the instance kernel's 1024 x 8 layout spills (8 statistics per thread)
+        // and loses: [8,64,64,512] 26.2 -> 28.6 us
+        if (instance && tpr == 1024 && nl == 8) continue;
+        GnClArgs a{};
+        a.x = p.x;
+        a.out = p.out;
+        a.gamma = p.gamma;
+        a.beta = p.beta;
+        a.mean = p.mean;
+        a.var = p.var;
+        a.P = static_cast<int>(p.spatial);
+        a.C = static_cast<int>(p.channels);
+        a.G = static_cast<int>(per_sample / w);
+        a.groups = static_cast<int>(per_sample);
+        a.cpg = static_cast<int>(cpg);
+        a.units = static_cast<int>(blocks);
+        a.cvg = FastDiv(static_cast<uint32_t>(cvg));
+        a.chunk = FastDiv(static_cast<uint32_t>(cvg * w));
+        const int64_t gpl = 128 / (cpg * w * 2); // blocks sharing a 128-byte line
+        a.gpl = (gpl >= 2 && a.G % gpl == 0 && tune_int("GN_CL_XCD_MAP", 1)) ? static_cast<int>(gpl) : 1;
+        a.eps = p.eps;
+        a.inv_R = static_cast<float>(1.0 / (static_cast<double>(p.spatial) * (instance ? 1 : cpg)));
+        a.one = 1.0f;
+        *status = w == 4 ? run_wide<4>(instance, tpr, nl, a, st) : run_wide<2>(instance, tpr, nl, a, st);
+        return true;
+      }
+    }
+  }
+  return false;
+}
+
+} // namespace
+
 bool gn_cl_cached_fwd(const ClProblem &p, bool aligned, hipStream_t st, int *status) {
+  if (wide_fwd(p, aligned, st, status)) return true;
   GnClArgs a{};
   const bool instance = p.groups == p.channels;
   const GnClCfg c = instance ? pick_in_cfg(p, aligned, false, a) : pick_cfg(p, aligned, false, a);

@@ -51,7 +51,10 @@ GN_CL_SHAPES = [(2, (8, 8), 8, 4), (3, (5,), 6, 2), (1, (2, 2), 4, 1), (2, (4,),
                 # group cached in registers: 1 to 8 channel vectors per group, ragged last load,
                 # groups that share cache lines (the XCD block map) and groups that do not
                 (3, (33, 33), 64, 2), (2, (20, 20), 128, 2), (5, (17, 17), 16, 1), (3, (24, 24), 96, 12),
-                (2, (56, 56), 64, 8), (9, (16, 16), 32, 4), (1, (90, 90), 8, 1)]
+                (2, (56, 56), 64, 8), (9, (16, 16), 32, 4), (1, (90, 90), 8, 1),
+                # half data, 8 channels per group, a block for every CU left: blocks that
+                # take 2 or 4 neighbouring groups (ragged planes; the 1024 x 8 layout)
+                (4, (32, 32), 1024, 128), (8, (33, 33), 1024, 128), (16, (64, 64), 256, 32)]
 
 
 @pytest.mark.parametrize("n,sp,c,groups", GN_CL_SHAPES)
@@ -80,7 +83,9 @@ IN_CL_SHAPES = [(2, (4, 4), 3), (3, (7,), 5), (1, (3, 2), 2), (4, (16, 16), 16),
                 (2, (9, 9), 96), (2, (5, 5), 4104), (3, (11,), 100), (2, (300,), 1032),
                 # instances cached in registers (256 positions and more)
                 (3, (33, 33), 24), (2, (20, 20), 128), (5, (17, 17), 16), (2, (56, 56), 64),
-                (1, (90, 90), 8), (9, (16, 16), 32)]
+                (1, (90, 90), 8), (9, (16, 16), 32),
+                # half data, a block for every CU left: blocks of 2 or 4 channel vectors
+                (4, (32, 32), 1024), (8, (33, 33), 1024), (16, (64, 32), 256)]
 
 
 @pytest.mark.parametrize("n,sp,c", IN_CL_SHAPES)
