@@ -757,4 +757,154 @@ gn_cl_wide_fwd_kernel(const GnClArgs a) {
   }
 }
 
+// Wide backward (half data, 8 channels per group, or instances): a block takes
+// GPB neighbouring groups / channel vectors of a sample, keeps x in registers
+// and parks dy in LDS (each thread reads back what it wrote), so both tensors
+// cross the memory system once, in 32- or 64-byte pieces: one launch, 3 S,
+// where planes beyond 2048 positions otherwise take the three-kernel path
+// (6 S).  A thread's vector is the 8 channels of one group (INSTANCE: 8
+// instances) at one position; per-channel sums fold over the threads with the
+// same piece of the chunk.  Algebra as in gn_cl_row_bwd_kernel /
+// in_cl_row_bwd_kernel.
+template <int NL, int TPR, int GPB, bool INSTANCE>
+__global__ void __launch_bounds__(TPR)
+cl_wide_bwd_kernel(const GnClArgs a) {
+  using T = __half;
+  constexpr int VEC = 8;
+  constexpr int NW = TPR / kWave;
+  constexpr uint32_t PST = TPR / GPB;
+  __shared__ uint4 park[NL * TPR];
+  __shared__ float fold[NW][GPB][2 * VEC];
+  __shared__ float chs[GPB][2 * VEC];
+  const int unit = gn_cl_unit(a);
+  if (unit < 0) return;
+  const uint32_t n = static_cast<uint32_t>(unit) / a.G, gb = static_cast<uint32_t>(unit) % a.G;
+  const uint32_t cvx = threadIdx.x % GPB, pos0 = threadIdx.x / GPB;
+  const uint32_t ch = (gb * GPB + cvx) * VEC;
+  const size_t slab = static_cast<size_t>(n) * a.P * a.C + ch;
+  const T *__restrict__ x = static_cast<const T *>(a.x) + slab;
+  const T *__restrict__ dy = static_cast<const T *>(a.dy) + slab;
+  T *__restrict__ dx = a.out ? static_cast<T *>(a.out) + slab : nullptr;
+
+  RawVec<T, VEC> xr[NL];
+  {
+    RawVec<T, VEC> dr[NL];
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const uint32_t pos = pos0 + k * PST;
+      const bool ok = pos < static_cast<uint32_t>(a.P);
+      const size_t off = static_cast<size_t>(ok ? pos : 0u) * a.C;
+      xr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + off));
+      dr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(dy + off)); // padded positions: dy = 0
+    }
+#pragma unroll
+    for (int k = 0; k < NL; ++k) park[k * TPR + threadIdx.x] = dr[k].v;
+  }
+  asm volatile("" ::: "memory"); // dy is read back from LDS, not kept in registers
+  // statistics of this thread's channels: one pair per group, or one per channel
+  constexpr int NS = INSTANCE ? VEC : 1;
+  const uint32_t stat = INSTANCE ? n * static_cast<uint32_t>(a.C) + ch
+                                 : n * static_cast<uint32_t>(a.groups) + gb * GPB + cvx;
+  float mean[NS], istd[NS], nmi[NS];
+#pragma unroll
+  for (int i = 0; i < NS; ++i) {
+    mean[i] = a.mean[stat + i];
+    istd[i] = 1.0f / sqrtf(a.var[stat + i] + a.eps);
+    nmi[i] = -mean[i] * istd[i];
+  }
+  float sdx[VEC], sdy[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) sdx[j] = sdy[j] = 0.f;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    RawVec<T, VEC> dr;
+    dr.v = park[k * TPR + threadIdx.x];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const int i = INSTANCE ? j : 0;
+      const float xh = norm_elem<T, VEC>(xr[k], j, mean[i], istd[i], nmi[i]);
+      sdx[j] = elem_fma<T, VEC>(dr, j, xh, sdx[j]);
+      sdy[j] = elem_fma<T, VEC>(dr, j, a.one, sdy[j]);
+    }
+  }
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+#pragma unroll
+    for (int off = GPB; off < kWave; off <<= 1) {
+      sdx[j] += __shfl_xor(sdx[j], off);
+      sdy[j] += __shfl_xor(sdy[j], off);
+    }
+  }
+  if (lane < GPB) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      fold[wave][lane][2 * j] = sdx[j];
+      fold[wave][lane][2 * j + 1] = sdy[j];
+    }
+  }
+  lds_barrier();
+  if (threadIdx.x < GPB * 2 * VEC) {
+    const int cv = threadIdx.x / (2 * VEC), e = threadIdx.x % (2 * VEC);
+    float t = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) t += fold[w][cv][e];
+    chs[cv][e] = t;
+    // entry 2*c is (sum dy*xh) of channel c of the block's chunk, 2*c+1 (sum dy)
+    a.pairs[2 * (static_cast<size_t>(n) * a.C + gb * GPB * VEC) + threadIdx.x] = t;
+  }
+  lds_barrier();
+  if (dx == nullptr) return;
+#pragma unroll
+  for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(xr[k]);
+  float gi[VEC], cA[NS], cb[NS];
+  if constexpr (INSTANCE) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float g = a.gamma ? a.gamma[ch + j] : 1.f;
+      const float vpe = a.var[stat + j] + a.eps;
+      gi[j] = g * istd[j];
+      cA[j] = -istd[j] * g * chs[cvx][2 * j] * a.inv_R +
+              (a.dvar ? 2.f * a.dvar[stat + j] * (vpe * istd[j]) * a.inv_R : 0.f);
+      cb[j] = -g * chs[cvx][2 * j + 1] * istd[j] * a.inv_R +
+              (a.dmean ? a.dmean[stat + j] * a.inv_R : 0.f);
+    }
+  } else {
+    float s1 = 0.f, t2 = 0.f;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float g = a.gamma ? a.gamma[ch + j] : 1.f;
+      gi[j] = g * istd[0];
+      t2 = fmaf(g, chs[cvx][2 * j], t2);
+      s1 = fmaf(g, chs[cvx][2 * j + 1], s1);
+    }
+    const float vpe = a.var[stat] + a.eps;
+    cA[0] = -istd[0] * t2 * a.inv_R + (a.dvar ? 2.f * a.dvar[stat] * (vpe * istd[0]) * a.inv_R : 0.f);
+    cb[0] = -s1 * istd[0] * a.inv_R + (a.dmean ? a.dmean[stat] * a.inv_R : 0.f);
+  }
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = pos0 + k * PST;
+    if (pos < static_cast<uint32_t>(a.P)) {
+      RawVec<T, VEC> dr;
+      dr.v = park[k * TPR + threadIdx.x];
+      float o[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const int i = INSTANCE ? j : 0;
+        const float xh = norm_elem<T, VEC>(xr[k], j, mean[i], istd[i], nmi[i]);
+        o[j] = elem_fma<T, VEC>(dr, j, gi[j], fmaf(xh, cA[i], cb[i]));
+      }
+      T *p = dx + static_cast<size_t>(pos) * a.C;
+      if (a.accum_dx) {
+        float old[VEC];
+        load_vec<T, VEC>(p, old);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) o[j] += old[j];
+      }
+      store_vec<T, VEC, false>(p, o);
+    }
+  }
+}
+
 } // namespace nblahip

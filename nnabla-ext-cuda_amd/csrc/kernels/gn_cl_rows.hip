@@ -287,8 +287,82 @@ bool gn_cl_cached_fwd(const ClProblem &p, bool aligned, hipStream_t st, int *sta
   return true;
 }
 
+namespace {
+
+template <int W>
+int run_wide_bwd(bool instance, int tpr, int nl, const GnClArgs &a, hipStream_t st) {
+#define WIDE_CASE(NL, TPR)                                                                       \
+  if (nl == (NL) && tpr == (TPR)) {                                                              \
+    if (instance) {                                                                              \
+      NBLAHIP_LAUNCH("cl_wide_bwd_kernel", (cl_wide_bwd_kernel<NL, TPR, W, true>),               \
+                     dim3(grid_of(a)), dim3(TPR), 0, st, a);                                     \
+    } else {                                                                                     \
+      NBLAHIP_LAUNCH("cl_wide_bwd_kernel", (cl_wide_bwd_kernel<NL, TPR, W, false>),              \
+                     dim3(grid_of(a)), dim3(TPR), 0, st, a);                                     \
+    }                                                                                            \
+    return last_launch_status();                                                                 \
+  }
+  WIDE_CASE(4, 512)
+  WIDE_CASE(8, 512)
+  WIDE_CASE(4, 1024)
+  WIDE_CASE(8, 1024)
+#undef WIDE_CASE
+  return NBLAHIP_EINVAL;
+}
+
+// Same shapes as the wide forward (half data, 8 channels per group or
+// instances, planes of 1024 positions and more, a block for every CU left).
+bool wide_bwd(const ClProblem &p, bool aligned, float *pairs, hipStream_t st, int *status) {
+  if (!aligned || p.dtype != NBLAHIP_F16 || !tune_int("GN_CL_WIDE_BWD", 1)) return false;
+  if (!p.bc_gamma || !p.bc_beta || p.spatial < 1024) return false;
+  constexpr int vec = 8;
+  const bool instance = p.groups == p.channels;
+  if (p.channels % vec != 0 || (!instance && p.channels / p.groups != vec)) return false;
+  const int64_t per_sample = instance ? p.channels / vec : p.groups;
+  for (int w : {4, 2}) {
+    if (per_sample % w != 0) continue;
+    const int64_t blocks = p.batch * (per_sample / w);
+    if (blocks < device_cus()) continue;
+    const int64_t nv = p.spatial * w;
+    for (int tpr : {512, 1024}) {
+      for (int nl : {4, 8}) {
+        if (static_cast<int64_t>(tpr) * nl < nv) continue;
+        GnClArgs a{};
+        a.x = p.x;
+        a.dy = p.dy;
+        a.out = p.out;
+        a.gamma = p.gamma;
+        a.mean = p.mean;
+        a.var = p.var;
+        a.dmean = p.dmean;
+        a.dvar = p.dvar;
+        a.pairs = pairs;
+        a.P = static_cast<int>(p.spatial);
+        a.C = static_cast<int>(p.channels);
+        a.G = static_cast<int>(per_sample / w);
+        a.groups = static_cast<int>(per_sample);
+        a.cpg = vec;
+        a.units = static_cast<int>(blocks);
+        const int64_t gpl = 128 / (vec * w * 2); // blocks sharing a 128-byte line
+        a.gpl = (gpl >= 2 && a.G % gpl == 0 && tune_int("GN_CL_XCD_MAP", 1)) ? static_cast<int>(gpl) : 1;
+        a.eps = p.eps;
+        a.inv_R = static_cast<float>(1.0 / (static_cast<double>(p.spatial) * (instance ? 1 : vec)));
+        a.one = 1.0f;
+        a.accum_dx = p.accum_dx;
+        *status = w == 4 ? run_wide_bwd<4>(instance, tpr, nl, a, st)
+                         : run_wide_bwd<2>(instance, tpr, nl, a, st);
+        return true;
+      }
+    }
+  }
+  return false;
+}
+
+} // namespace
+
 bool gn_cl_cached_bwd(const ClProblem &p, bool aligned, float *pairs, hipStream_t st,
                       int *status) {
+  if (wide_bwd(p, aligned, pairs, st, status)) return true;
   GnClArgs a{};
   const bool instance = p.groups == p.channels;
   const GnClCfg c = instance ? pick_in_cfg(p, aligned, true, a) : pick_cfg(p, aligned, true, a);
