@@ -551,9 +551,13 @@ in_cl_row_bwd_kernel(const GnClArgs a) {
 // statistics stay per group (per channel), so the block sums are segmented:
 // a butterfly over the lanes that hold the same piece of the chunk, then LDS.
 // ---------------------------------------------------------------------------
-template <typename T, int VEC, int NL, int TPR, int CVB>
+// PARK: x waits in LDS instead of registers (the 1024 x 8 layout: with 8
+// statistics per thread beside 8 vectors of x the registers run out).
+template <typename T, int VEC, int NL, int TPR, int CVB, bool PARK = false>
 __global__ void __launch_bounds__(TPR)
 in_cl_wide_fwd_kernel(const GnClArgs a) {
+  static_assert(!PARK || sizeof(RawVec<T, VEC>) == 16, "parked vectors are 16 bytes");
+  __shared__ uint4 park[PARK ? NL * TPR : 1];
   constexpr int NW = TPR / kWave;
   constexpr uint32_t PST = TPR / CVB; // positions a block covers per load
   __shared__ float lds[NW][CVB][VEC];
@@ -572,6 +576,18 @@ in_cl_wide_fwd_kernel(const GnClArgs a) {
     const bool ok = pos < static_cast<uint32_t>(a.P);
     raw[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + static_cast<size_t>(ok ? pos : 0u) * a.C));
   }
+  if constexpr (PARK) {
+#pragma unroll
+    for (int k = 0; k < NL; ++k) park[k * TPR + threadIdx.x] = __builtin_bit_cast(uint4, raw[k]);
+    asm volatile("" ::: "memory"); // read back from LDS from here on
+  }
+  auto xv = [&](int k) -> RawVec<T, VEC> {
+    if constexpr (PARK) {
+      return __builtin_bit_cast(RawVec<T, VEC>, park[k * TPR + threadIdx.x]);
+    } else {
+      return raw[k];
+    }
+  };
   float gam[VEC], bet[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
@@ -605,23 +621,27 @@ in_cl_wide_fwd_kernel(const GnClArgs a) {
   for (int j = 0; j < VEC; ++j) mean[j] = 0.f;
 #pragma unroll
   for (int k = 0; k < NL; ++k) {
+    const RawVec<T, VEC> r = xv(k);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) mean[j] = elem_fma<T, VEC>(raw[k], j, a.one, mean[j]);
+    for (int j = 0; j < VEC; ++j) mean[j] = elem_fma<T, VEC>(r, j, a.one, mean[j]);
   }
   block_sums(mean);
 #pragma unroll
   for (int j = 0; j < VEC; ++j) mean[j] *= a.inv_R;
 #pragma unroll
-  for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+  for (int k = 0; k < NL; ++k) {
+    if constexpr (!PARK) keep_packed<T, VEC>(raw[k]);
+  }
   float var[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) var[j] = 0.f;
 #pragma unroll
   for (int k = 0; k < NL; ++k) {
     if (pos0 + k * PST < static_cast<uint32_t>(a.P)) {
+      const RawVec<T, VEC> r = xv(k);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        const float d = elem_fma<T, VEC>(raw[k], j, a.one, -mean[j]);
+        const float d = elem_fma<T, VEC>(r, j, a.one, -mean[j]);
         var[j] = fmaf(d, d, var[j]);
       }
     }
@@ -643,18 +663,21 @@ in_cl_wide_fwd_kernel(const GnClArgs a) {
     }
   }
 #pragma unroll
-  for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+  for (int k = 0; k < NL; ++k) {
+    if constexpr (!PARK) keep_packed<T, VEC>(raw[k]);
+  }
 #pragma unroll
   for (int k = 0; k < NL; ++k) {
     const uint32_t pos = pos0 + k * PST;
     if (pos < static_cast<uint32_t>(a.P)) {
+      const RawVec<T, VEC> r = xv(k);
       float o[VEC];
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
         if constexpr (sizeof(T) == 2) {
-          o[j] = elem_fma<T, VEC>(raw[k], j, sc[j], sh[j]);
+          o[j] = elem_fma<T, VEC>(r, j, sc[j], sh[j]);
         } else {
-          o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mean[j]), sc[j], bet[j]);
+          o[j] = fmaf(elem_fma<T, VEC>(r, j, a.one, -mean[j]), sc[j], bet[j]);
         }
       }
       store_vec<T, VEC, false>(y + static_cast<size_t>(pos) * a.C, o);

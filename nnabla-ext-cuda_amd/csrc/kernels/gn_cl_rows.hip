@@ -202,7 +202,8 @@ int run_wide(bool instance, int tpr, int nl, const GnClArgs &a, hipStream_t st) 
 #define WIDE_CASE(NL, TPR)                                                                       \
   if (nl == (NL) && tpr == (TPR)) {                                                              \
     if (instance) {                                                                              \
-      NBLAHIP_LAUNCH("in_cl_wide_fwd_kernel", (in_cl_wide_fwd_kernel<__half, 8, NL, TPR, W>),    \
+      NBLAHIP_LAUNCH("in_cl_wide_fwd_kernel",                                                    \
+                     (in_cl_wide_fwd_kernel<__half, 8, NL, TPR, W, (NL) * (TPR) == 8192>),       \
                      dim3(grid_of(a)), dim3(TPR), 0, st, a);                                     \
     } else {                                                                                     \
       NBLAHIP_LAUNCH("gn_cl_wide_fwd_kernel", (gn_cl_wide_fwd_kernel<__half, 8, NL, TPR, W>),    \
@@ -238,9 +239,6 @@ bool wide_fwd(const ClProblem &p, bool aligned, hipStream_t st, int *status) {
     for (int tpr : {512, 1024}) {
       for (int nl : {4, 8}) {
         if (static_cast<int64_t>(tpr) * nl < nv) continue;
-        // the instance kernel's 1024 x 8 layout spills (8 statistics per thread)
-        // and loses: [8,64,64,512] 26.2 -> 28.6 us
-        if (instance && tpr == 1024 && nl == 8) continue;
         GnClArgs a{};
         a.x = p.x;
         a.out = p.out;
