@@ -320,6 +320,12 @@ row_bwd_kernel(const RowArgs a) {
   constexpr bool GN = MODE == kRowGN || MODE == kRowGNm;
   constexpr bool BN = MODE == kRowBN; // strided rows, dgamma/dbeta written here
   constexpr bool GNM = MODE == kRowGNm; // run-time thread map (GnSlot)
+  // Float groups of 64-128 KB (1024 threads x 8 loads): dy waits in LDS, not
+  // in registers (each thread reads back what it wrote) - with x and dy both
+  // in registers the block is alone on its CU at 128 registers per thread and
+  // loses to the five-pass streaming kernels.
+  constexpr bool PARK = GN && sizeof(T) == 4 && VEC == 4 && TPR == 1024 && NL == 8;
+  __shared__ uint4 park[PARK ? NL * TPR : 1];
   __shared__ float lds[2 * 16];
   __shared__ float part[GN ? 2 * NW * NL : 1];
   __shared__ float xfold[(MODE == kRowLN && RPB > 1) ? (RPB / 2) * TPR * VEC : 1];
@@ -404,6 +410,18 @@ row_bwd_kernel(const RowArgs a) {
       xr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + base + off));
       dr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(dy + base + off));
     }
+    if constexpr (PARK) {
+#pragma unroll
+      for (int k = 0; k < NL; ++k) park[k * TPR + threadIdx.x] = __builtin_bit_cast(uint4, dr[k]);
+      asm volatile("" ::: "memory"); // read back from LDS from here on
+    }
+    auto dyv = [&](int k) -> RawVec<T, VEC> {
+      if constexpr (PARK) {
+        return __builtin_bit_cast(RawVec<T, VEC>, park[k * TPR + threadIdx.x]);
+      } else {
+        return dr[k];
+      }
+    };
     const float mean = a.mean[row];
     const float vpe = a.var[row] + a.eps;
     const float istd = 1.0f / sqrtf(vpe);
@@ -488,12 +506,13 @@ row_bwd_kernel(const RowArgs a) {
       lds_barrier(); // part[] of the previous row has been consumed
 #pragma unroll
       for (int k = 0; k < NL; ++k) {
-        float sdy = raw_sum<T, VEC>(dr[k], 0.f);
+        const RawVec<T, VEC> dk = dyv(k);
+        float sdy = raw_sum<T, VEC>(dk, 0.f);
         float sdx = 0.f;
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
           const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
-          sdx = elem_fma<T, VEC>(dr[k], j, xh, sdx);
+          sdx = elem_fma<T, VEC>(dk, j, xh, sdx);
         }
         sdy = wave_sum(sdy);
         sdx = wave_sum(sdx);
@@ -536,7 +555,7 @@ row_bwd_kernel(const RowArgs a) {
 #pragma unroll
     for (int k = 0; k < NL; ++k) {
       keep_packed<T, VEC>(xr[k]);
-      keep_packed<T, VEC>(dr[k]);
+      if constexpr (!PARK) keep_packed<T, VEC>(dr[k]);
     }
     const float cA = -istd * t2 * a.inv_R +
                      (a.dvar ? 2.f * a.dvar[row] * (vpe * istd) * a.inv_R : 0.f);
@@ -579,10 +598,11 @@ row_bwd_kernel(const RowArgs a) {
             }
           } else {
             const float gi = gk[k] * istd;
+            const RawVec<T, VEC> dk = dyv(k);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) {
               const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
-              o[j] = elem_fma<T, VEC>(dr[k], j, gi, fmaf(xh, cA, cb));
+              o[j] = elem_fma<T, VEC>(dk, j, gi, fmaf(xh, cA, cb));
             }
           }
           T *dst = dx + base + row_elem_offset<BN>(a, col);

@@ -453,11 +453,12 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
       cfg = fixed;
       if (cfg.ok) a.epc = static_cast<int>(p.spatial / (64 * cfg.vec));
     }
-    // The float 1024 x 8 layout (one block per CU, 128 KB of row data in its
-    // registers) loses to the streaming kernels: 92-105 vs 85 us on
-    // 25 088-element groups, 55 vs 56 us on 32 768-element ones.
+    // The float 1024 x 8 layout (one block per CU, 128 KB of x and as much of
+    // dy) lost to the streaming kernels with both in registers (92-105 vs 85 us
+    // on 25 088-element groups, 55 vs 56 us on 32 768-element ones); with dy
+    // parked in LDS it wins: 80 -> 62 us and 55.5 -> 41 us.
     if (cfg.ok && p.dtype == NBLAHIP_F32 && cfg.vec == 4 && cfg.tpr == 1024 && cfg.nl == 8 &&
-        !tune_int("GN_FLOAT_1024X8", 0))
+        !tune_int("GN_FLOAT_1024X8", 1))
       cfg.ok = false;
   }
   if (cfg.ok && !tune_int("FORCE_STREAM", 0)) {

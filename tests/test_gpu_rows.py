@@ -164,6 +164,8 @@ GN_SHAPES = [(2, 8, (8, 8), 4), (3, 6, (5,), 2), (1, 4, (2, 2), 1), (2, 6, (4,),
              (2, 64, (56, 56), 8), (2, 64, (28, 28), 4), (2, 6, (8, 8), 2), (2, 4, (64, 64), 4),
              (1, 10, (48, 48), 2), (2, 64, (14, 14), 2), (2, 128, (7, 7), 2), (1, 80, (8, 8), 2),
              (3, 24, (24, 24), 3), (2, 14, (72,), 2),
+             # float groups of 64-128 KB: 1024 threads x 8 loads, dy parked in LDS (fixed map)
+             (2, 16, (64, 64), 2),
              # one group of 2M elements per sample: split streaming reductions
              (2, 32, (256, 256), 1), (1, 6, (333, 333), 2)]
 
