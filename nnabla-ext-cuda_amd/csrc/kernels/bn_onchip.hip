@@ -17,9 +17,9 @@
 // Beside x a thread needs a batch of dy, so it holds fewer vectors: 18432 per
 // channel with 1024 threads, 20480 with 512; the rest of x is streamed with dy.
 //
-// Worth it only when there is a channel for (nearly) every CU: the block is
-// alone on its CU, so fewer channels than CUs leave the rest of the chip idle
-// and the split reduction wins.
+// The block is alone on its CU, so fewer channels than CUs leave CUs idle; the
+// path still wins down to an eighth (forward) or a quarter (backward) of the
+// CUs, because a CU alone pulls far more than its share of the bandwidth.
 //
 // The kernels are fully unrolled over the slots of a thread, and most of what
 // looks odd below (opaque copies of the thread index, vectors hidden from the
@@ -541,8 +541,19 @@ bool onchip_args(const BnProblem &p, bool backward, BnOnchipArgs &a, int &nl, in
   // up to 8 loads per thread the row kernels take the channel; above 25 it
   // does not fit
   if (nl <= 8 || nl > max_nl) return false;
-  // a block is alone on its CU: fewer channels than (nearly all) CUs idle the rest
-  if (p.C * 8 < static_cast<int64_t>(device_cus()) * 7) return false;
+  // A block is alone on its CU, so fewer channels than CUs leave CUs idle -
+  // but a CU alone pulls far more than its 1/256 share of the bandwidth, and
+  // the split reduction pays a finalize launch: the forward wins down to an
+  // eighth of the CUs ([32,32,56,56] float 15.3 -> 10.4 us), the backward down
+  // to a quarter ([32,64,56,56] 25.6 -> 22.8 us; with 32 channels 16 -> 19 us).
+  // With a streamed remainder (channels beyond what the layouts hold) only
+  // with a channel for nearly every CU: [32,64,112,112] half (50176 vectors)
+  // 33.6 / 43.1 vs 35.7 / 52.0 us.
+  const bool whole = nv <= (backward ? 20480 : 25600);
+  const int min_pct = !whole     ? tune_int("BN_ONCHIP_STREAMED_MIN_PCT", 88)
+                      : backward ? tune_int("BN_ONCHIP_BWD_MIN_PCT", 25)
+                                 : tune_int("BN_ONCHIP_FWD_MIN_PCT", 12);
+  if (p.C * 100 < static_cast<int64_t>(device_cus()) * min_pct) return false;
   a = BnOnchipArgs{};
   a.x = p.x;
   a.gamma = p.gamma;

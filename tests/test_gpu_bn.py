@@ -310,9 +310,12 @@ ONCHIP_CASES = [(torch.float32, 33), (torch.float32, 47), (torch.float32, 55), (
 
 
 @pytest.mark.parametrize("dtype,n", ONCHIP_CASES)
-def test_bn_channel_on_chip(dtype, n):
+@pytest.mark.parametrize("few_channels", [False, True])
+def test_bn_channel_on_chip(dtype, n, few_channels):
     cus = torch.cuda.get_device_properties(0).multi_processor_count
-    c = (cus * 7 + 7) // 8
+    # a channel for (nearly) every CU, or for a quarter of them (whole-channel
+    # layouts only; the others then take the split reduction)
+    c = (cus + 3) // 4 + 1 if few_channels else (cus * 7 + 7) // 8
     shape, axis = (n, c, 32, 32), 1
     dn = dtype_name(dtype)
     x, dy, g, b, rm, rv = make_bn(shape, axis, dtype, 21, mean=1.0, std=2.0)
