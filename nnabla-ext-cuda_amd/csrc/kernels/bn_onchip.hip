@@ -47,6 +47,7 @@ struct BnOnchipArgs {
   uint32_t nv;         // vectors per channel = size0 * vpp
   FastDiv vpp;         // vectors per plane
   float inv_N, unbias, decay, eps, one;
+  const void *z; // FusedBatchNormalization forward: y = max(0, bn(x) [+ z]); may be null
   // backward
   const void *dy;
   void *dx;                 // may be null
@@ -118,7 +119,8 @@ __device__ __forceinline__ uint32_t onchip_offset(const BnOnchipArgs &a, uint32_
 // mean of 25600 vectors of the same channel, so the subtracted square is tiny
 // against the variance: no cancellation).  The rest is read a second time for
 // y: 2 S + (1 - 25600 / nv) S instead of 3 S.
-template <typename T, int VEC, int NR, int NS, bool OVER = false>
+// FUSED (FusedBatchNormalization): y = max(0, bn(x) + z), z optional.
+template <typename T, int VEC, int NR, int NS, bool OVER = false, bool FUSED = false>
 __global__ void __launch_bounds__(kOnchipBlock)
 bn_onchip_fwd_kernel(const BnOnchipArgs a) {
   static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors only");
@@ -240,7 +242,17 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
         o[j] = fmaf(elem_fma<T, VEC>(r, j, a.one, -mean), g, b);
       }
     }
-    store_vec<T, VEC>(y + onchip_offset(a, c, v, VEC), o);
+    const uint32_t off = onchip_offset(a, c, v, VEC);
+    if constexpr (FUSED) {
+      if (a.z) {
+        const RawVec<T, VEC> zr = load_raw<T, VEC>(static_cast<const T *>(a.z) + off);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) o[j] = elem_fma<T, VEC>(zr, j, a.one, o[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) o[j] = fmaxf(0.f, o[j]);
+    }
+    store_vec<T, VEC>(y + off, o);
   };
   const uint32_t t2 = fresh(t);
 #pragma unroll
@@ -486,11 +498,12 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
 
 namespace {
 
-template <typename T, int VEC>
+template <typename T, int VEC, bool FUSED>
 int run_onchip_fwd(int nl, const BnOnchipArgs &a, hipStream_t st) {
 #define ONCHIP_CASE(NR, NS)                                                                      \
   if (nl <= (NR) + (NS)) {                                                                       \
-    NBLAHIP_LAUNCH("bn_onchip_fwd_kernel", (bn_onchip_fwd_kernel<T, VEC, NR, NS>), dim3(a.C),    \
+    NBLAHIP_LAUNCH(FUSED ? "bn_onchip_fwd_kernel_fused" : "bn_onchip_fwd_kernel",                \
+                   (bn_onchip_fwd_kernel<T, VEC, NR, NS, false, FUSED>), dim3(a.C),              \
                    dim3(kOnchipBlock), 0, st, a);                                                \
     return last_launch_status();                                                                 \
   }
@@ -503,8 +516,9 @@ int run_onchip_fwd(int nl, const BnOnchipArgs &a, hipStream_t st) {
   ONCHIP_CASE(16, 9)
 #undef ONCHIP_CASE
   // longer channels: 25 slots held, the rest streamed
-  NBLAHIP_LAUNCH("bn_onchip_fwd_kernel", (bn_onchip_fwd_kernel<T, VEC, 16, 9, true>), dim3(a.C),
-                 dim3(kOnchipBlock), 0, st, a);
+  NBLAHIP_LAUNCH(FUSED ? "bn_onchip_fwd_kernel_fused" : "bn_onchip_fwd_kernel",
+                 (bn_onchip_fwd_kernel<T, VEC, 16, 9, true, FUSED>), dim3(a.C), dim3(kOnchipBlock),
+                 0, st, a);
   return last_launch_status();
 }
 
@@ -532,7 +546,9 @@ int run_onchip_bwd(int64_t nv, const BnOnchipArgs &a, hipStream_t st) {
 // Shape test shared by both directions; fills the common arguments.
 bool onchip_args(const BnProblem &p, bool backward, BnOnchipArgs &a, int &nl, int max_nl = 25) {
   if (!tune_int("BN_ONCHIP", 1)) return false;
-  if (p.size2 <= 1 || p.relu || p.z || p.y || p.dz || p.sums_out || p.sums_in) return false;
+  if (p.size2 <= 1 || p.y || p.dz || p.sums_out || p.sums_in) return false;
+  if (backward && (p.relu || p.z)) return false;
+  if (p.z && !aligned16(p.z)) return false;
   const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
   if (p.size2 % vec != 0 || !aligned16(p.x) || (p.out && !aligned16(p.out))) return false;
   if (backward && !aligned16(p.dy)) return false;
@@ -607,8 +623,14 @@ bool bn_onchip_fwd_train(const BnProblem &p, hipStream_t st, int *status) {
   a.var = p.batch_var;
   a.rmean = p.rmean;
   a.rvar = p.rvar;
-  *status = p.dtype == NBLAHIP_F16 ? run_onchip_fwd<__half, 8>(nl, a, st)
-                                   : run_onchip_fwd<float, 4>(nl, a, st);
+  a.z = p.z;
+  if (p.relu || p.z) {
+    *status = p.dtype == NBLAHIP_F16 ? run_onchip_fwd<__half, 8, true>(nl, a, st)
+                                     : run_onchip_fwd<float, 4, true>(nl, a, st);
+  } else {
+    *status = p.dtype == NBLAHIP_F16 ? run_onchip_fwd<__half, 8, false>(nl, a, st)
+                                     : run_onchip_fwd<float, 4, false>(nl, a, st);
+  }
   return true;
 }
 

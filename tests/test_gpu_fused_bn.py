@@ -28,6 +28,9 @@ SHAPES = [
     ((6, 9, 9, 96), 3), ((3, 5, 5, 4104), 3), ((37, 100), 1),
     # channel-last with few rows: a channel vector's column in one block's registers
     ((32, 7, 7, 512), 3), ((8, 14, 14, 256), 3), ((100, 2048), 1), ((33, 8, 8, 320), 3),
+    # planes layout with a channel held on one CU in the forward (registers, then LDS;
+    # the last one with a streamed remainder)
+    ((36, 64, 32, 32), 1), ((73, 48, 32, 32), 1), ((230, 232, 16, 32), 1),
 ]
 
 
