@@ -346,3 +346,34 @@ def test_bn_channel_on_chip(dtype, n, few_channels):
     assert torch.equal(y2, y)
     _, dg2, db2 = K.bn_backward(xd, dyd, gd, m, v, axis, 1e-5, need=(False, True, True))
     assert torch.equal(dg2, dg) and torch.equal(db2, db)
+
+
+@pytest.mark.parametrize("shape,axis,dtype", [
+    ((8, 12, 14, 14), 1, torch.float32),      # split reduction
+    ((8, 64, 12, 12), 1, torch.float32),      # channel in one block's registers
+    ((37, 64, 32, 32), 1, torch.float32),     # channel held on one CU
+    ((131, 232, 16, 32), 1, torch.float16),   # ... with a streamed remainder
+    ((8, 7, 7, 256), 3, torch.float16),       # channel-last, column in registers
+    ((300, 9, 64), 2, torch.float32),         # channel-last split reduction
+])
+def test_bn_training_forward_in_place(shape, axis, dtype):
+    """y == x through the C-ABI on every forward path."""
+    dn = dtype_name(dtype)
+    x, _, g, b, rm, rv = make_bn(shape, axis, dtype, 33, mean=0.5, std=1.5)
+    y_r, m_r, v_r, rm_r, rv_r = R.bn_forward_batch(x, b, g, rm, rv, axis, 0.9, 1e-5)
+    xd, gd, bd, rmd, rvd = to_dev(x, dtype), to_dev(g), to_dev(b), to_dev(rm), to_dev(rv)
+    c = shape[axis]
+    m, v = torch.empty(c, device="cuda"), torch.empty(c, device="cuda")
+    s0, _, s2 = K._bn_sizes(shape, axis)
+    L = K.lib()
+    dt = K._dtype_code(xd)
+    ws = torch.empty(max(int(L.nblahip_bn_workspace_bytes(s0, c, s2, dt)), 256), dtype=torch.uint8,
+                     device="cuda")
+    K.check(L.nblahip_bn_fwd_train(xd.data_ptr(), gd.data_ptr(), bd.data_ptr(), xd.data_ptr(),
+                                   m.data_ptr(), v.data_ptr(), rmd.data_ptr(), rvd.data_ptr(), s0, c,
+                                   s2, 0.9, 1e-5, dt, ws.data_ptr(), ws.numel(),
+                                   torch.cuda.current_stream().cuda_stream))
+    assert_close(to_np(xd), y_r, dn, "y", "y in place")
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    assert_close(to_np(rmd), rm_r, dn, "stat", "running_mean")
