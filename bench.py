@@ -143,7 +143,9 @@ def make_bn(K, shape, axis, dtype, train, mean=0.0, std=1.0, outliers=False, see
                                      bv.data_ptr(), None, None, dx.data_ptr(), dg.data_ptr(),
                                      db.data_ptr(), 0, 0, 0, s0, c, s2, 1e-5, 1, dt, ws.data_ptr(),
                                      ws.numel(), st))
-        pf, pb = bn_tensor_passes(K, fwd, bwd, s0 * s2 * x.element_size() // 16)
+        # (vectors are 16 bytes, 8 for half planes of 4k - not 8k - elements)
+        vec_bytes = 8 if x.element_size() == 2 and s2 % 8 != 0 and s2 % 4 == 0 else 16
+        pf, pb = bn_tensor_passes(K, fwd, bwd, s0 * s2 * x.element_size() // vec_bytes)
         return fwd, bwd, int(round(pf * S)), int(round(pb * S)), (x, dy, gamma, beta, rm, rv, y, dx, bm, bv, dg,
                                                       db, ws)
 

@@ -27,6 +27,7 @@
 // holding across the passes what is cheaper to compute again: each such value
 // costs a register in every one of 1024 threads, and the layouts leave none.
 #include <algorithm>
+#include <type_traits>
 
 #include "common.cuh"
 #include "launch.hpp"
@@ -47,6 +48,7 @@ struct BnOnchipArgs {
   uint32_t nv;         // vectors per channel = size0 * vpp
   FastDiv vpp;         // vectors per plane
   float inv_N, unbias, decay, eps, one;
+  int vec;       // elements per vector (8-byte vectors for half planes of 4k elements)
   const void *z; // FusedBatchNormalization forward: y = max(0, bn(x) [+ z]); may be null
   // backward
   const void *dy;
@@ -101,6 +103,11 @@ __device__ __forceinline__ uint32_t fresh_after(uint32_t v, uint32_t after) {
   return v;
 }
 
+// LDS slot of a parked vector: 16 bytes, or 8 for half planes of 4k (not 8k)
+// elements, which are read in 8-byte vectors.
+template <typename T, int VEC>
+using Slot = std::conditional_t<sizeof(RawVec<T, VEC>) == 16, uint4, uint2>;
+
 // Element offset of vector v of channel c (planes are contiguous, a channel's
 // planes lie C*size2 apart).
 __device__ __forceinline__ uint32_t onchip_offset(const BnOnchipArgs &a, uint32_t c, uint32_t v,
@@ -123,9 +130,9 @@ __device__ __forceinline__ uint32_t onchip_offset(const BnOnchipArgs &a, uint32_
 template <typename T, int VEC, int NR, int NS, bool OVER = false, bool FUSED = false>
 __global__ void __launch_bounds__(kOnchipBlock)
 bn_onchip_fwd_kernel(const BnOnchipArgs a) {
-  static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors only");
+  static_assert(sizeof(RawVec<T, VEC>) == sizeof(Slot<T, VEC>), "8- or 16-byte vectors");
   __shared__ float red[kOnchipBlock / kWave];
-  __shared__ uint4 spill[NS > 0 ? NS * kOnchipBlock : 1];
+  __shared__ Slot<T, VEC> spill[NS > 0 ? NS * kOnchipBlock : 1];
   const uint32_t c = blockIdx.x;
   const uint32_t t = threadIdx.x;
   const T *__restrict__ x = static_cast<const T *>(a.x);
@@ -152,7 +159,7 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
   for (int k = 0; k < NS; ++k) {
     const float part = raw_sum<T, VEC>(parked[k], 0.f);
     s += (static_cast<uint32_t>(NR + k) * kOnchipBlock + t < a.nv) ? part : 0.f;
-    spill[k * kOnchipBlock + t] = __builtin_bit_cast(uint4, parked[k]);
+    spill[k * kOnchipBlock + t] = __builtin_bit_cast(Slot<T, VEC>, parked[k]);
   }
 #pragma unroll
   for (int k = 0; k < NR; ++k) {
@@ -299,10 +306,10 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
 template <typename T, int VEC, int NR, int NS, int B, int TB, bool OVER = false>
 __global__ void __launch_bounds__(TB)
 bn_onchip_bwd_kernel(const BnOnchipArgs a) {
-  static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors only");
+  static_assert(sizeof(RawVec<T, VEC>) == sizeof(Slot<T, VEC>), "8- or 16-byte vectors");
   constexpr int NL = NR + NS;
   __shared__ float red[TB / kWave];
-  __shared__ uint4 spill[NS > 0 ? NS * TB : 1];
+  __shared__ Slot<T, VEC> spill[NS > 0 ? NS * TB : 1];
   const uint32_t c = blockIdx.x;
   const uint32_t t = threadIdx.x;
   const T *__restrict__ x = static_cast<const T *>(a.x);
@@ -323,7 +330,7 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
     uint32_t tr = t;
 #pragma unroll
     for (int k = 0; k < NS; ++k) {
-      const uint4 w = __builtin_bit_cast(uint4, parked[k]);
+      const Slot<T, VEC> w = __builtin_bit_cast(Slot<T, VEC>, parked[k]);
       spill[k * TB + t] = w;
       tr = fresh_after(tr, w.x);
     }
@@ -549,7 +556,8 @@ bool onchip_args(const BnProblem &p, bool backward, BnOnchipArgs &a, int &nl, in
   if (p.size2 <= 1 || p.y || p.dz || p.sums_out || p.sums_in) return false;
   if (backward && (p.relu || p.z)) return false;
   if (p.z && !aligned16(p.z)) return false;
-  const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
+  int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
+  if (p.dtype == NBLAHIP_F16 && p.size2 % 8 != 0 && p.size2 % 4 == 0) vec = 4; // 8-byte vectors
   if (p.size2 % vec != 0 || !aligned16(p.x) || (p.out && !aligned16(p.out))) return false;
   if (backward && !aligned16(p.dy)) return false;
   const int64_t nv = p.size0 * (p.size2 / vec);
@@ -557,6 +565,10 @@ bool onchip_args(const BnProblem &p, bool backward, BnOnchipArgs &a, int &nl, in
   // up to 8 loads per thread the row kernels take the channel; above 25 it
   // does not fit
   if (nl <= 8 || nl > max_nl) return false;
+  // 8-byte vectors move half as much per instruction: a gain for channels of
+  // up to 16384 of them ([256,1024,14,14] 61 / 84 -> 58 / 77 us, [256,256,14,14]
+  // 24 / 24.5 -> 15 / 18.5 us), a loss beyond ([512,1024,14,14] 115 / 175 -> 130 / 176 us)
+  if (vec == 4 && p.dtype == NBLAHIP_F16 && nl > 16) return false;
   // A block is alone on its CU, so fewer channels than CUs leave CUs idle -
   // but a CU alone pulls far more than its 1/256 share of the bandwidth, and
   // the split reduction pays a finalize launch: the forward wins down to an
@@ -577,6 +589,7 @@ bool onchip_args(const BnProblem &p, bool backward, BnOnchipArgs &a, int &nl, in
   a.size2 = static_cast<uint32_t>(p.size2);
   a.nv = static_cast<uint32_t>(nv);
   a.vpp = FastDiv(static_cast<uint32_t>(p.size2 / vec));
+  a.vec = vec;
   const double N = static_cast<double>(p.size0) * static_cast<double>(p.size2);
   a.inv_N = static_cast<float>(1.0 / N);
   a.unbias = static_cast<float>(N / (N - 1.0));
@@ -608,8 +621,9 @@ bool bn_onchip_bwd(const BnProblem &p, hipStream_t st, int *status) {
   a.accum_dx = p.accum_dx;
   a.accum_g = p.accum_g;
   a.accum_b = p.accum_b;
-  *status = p.dtype == NBLAHIP_F16 ? run_onchip_bwd<__half, 8>(a.nv, a, st)
-                                   : run_onchip_bwd<float, 4>(a.nv, a, st);
+  *status = p.dtype != NBLAHIP_F16 ? run_onchip_bwd<float, 4>(a.nv, a, st)
+            : a.vec == 8           ? run_onchip_bwd<__half, 8>(a.nv, a, st)
+                                   : run_onchip_bwd<__half, 4>(a.nv, a, st);
   return true;
 }
 
@@ -625,11 +639,13 @@ bool bn_onchip_fwd_train(const BnProblem &p, hipStream_t st, int *status) {
   a.rvar = p.rvar;
   a.z = p.z;
   if (p.relu || p.z) {
-    *status = p.dtype == NBLAHIP_F16 ? run_onchip_fwd<__half, 8, true>(nl, a, st)
-                                     : run_onchip_fwd<float, 4, true>(nl, a, st);
+    *status = p.dtype != NBLAHIP_F16 ? run_onchip_fwd<float, 4, true>(nl, a, st)
+              : a.vec == 8           ? run_onchip_fwd<__half, 8, true>(nl, a, st)
+                                     : run_onchip_fwd<__half, 4, true>(nl, a, st);
   } else {
-    *status = p.dtype == NBLAHIP_F16 ? run_onchip_fwd<__half, 8, false>(nl, a, st)
-                                     : run_onchip_fwd<float, 4, false>(nl, a, st);
+    *status = p.dtype != NBLAHIP_F16 ? run_onchip_fwd<float, 4, false>(nl, a, st)
+              : a.vec == 8           ? run_onchip_fwd<__half, 8, false>(nl, a, st)
+                                     : run_onchip_fwd<__half, 4, false>(nl, a, st);
   }
   return true;
 }

@@ -316,7 +316,18 @@ def test_bn_channel_on_chip(dtype, n, few_channels):
     # a channel for (nearly) every CU, or for a quarter of them (whole-channel
     # layouts only; the others then take the split reduction)
     c = (cus + 3) // 4 + 1 if few_channels else (cus * 7 + 7) // 8
-    shape, axis = (n, c, 32, 32), 1
+    check_channel_on_chip((n, c, 32, 32), dtype)
+
+
+# Half planes of 4k (not 8k) elements (14 x 14) are held as 8-byte vectors, up
+# to 16384 of them per channel (the last shape is beyond: split reduction).
+@pytest.mark.parametrize("shape", [(180, 64, 14, 14), (330, 72, 14, 14), (420, 72, 14, 14)])
+def test_bn_channel_on_chip_8_byte_vectors(shape):
+    check_channel_on_chip(shape, torch.float16)
+
+
+def check_channel_on_chip(shape, dtype):
+    axis, c = 1, shape[1]
     dn = dtype_name(dtype)
     x, dy, g, b, rm, rv = make_bn(shape, axis, dtype, 21, mean=1.0, std=2.0)
     y_r, m_r, v_r, rm_r, rv_r = R.bn_forward_batch(x, b, g, rm, rv, axis, 0.9, 1e-5)
