@@ -532,9 +532,16 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
 // ---------------------------------------------------------------------------
 static bool bn_rows_cfg(const BnProblem &p, bool backward, RowCfg &cfg, RowArgs &a) {
   if (!tune_int("BN_ROWS", 1)) return false;
-  if (p.size2 <= 1 || p.relu || p.z || p.y || p.dz || p.sums_out || p.sums_in) return false;
+  if (p.relu || p.z || p.y || p.dz || p.sums_out || p.sums_in) return false;
+  // channel-last (planes of one element): a row is strided by C, which only a
+  // handful of channels keeps inside a cache line (RGB-like inputs); wider
+  // channel-last tensors have their own kernels
+  if (p.size2 <= 1 && p.C > 8) return false;
   const int64_t R = p.size0 * p.size2;
   if (R < 2 || R > (int64_t{1} << 20)) return false;
+  const int64_t bytes = R * p.C * (p.dtype == NBLAHIP_F16 ? 2 : 4);
+  const bool tiny = bytes <= (2 << 20); // launches, not bytes, are what costs
+  if (p.size2 <= 1 && !tiny) return false;
   int vec = 1;
   const bool al = aligned16(p.x) && (!p.out || aligned16(p.out)) && (!backward || aligned16(p.dy));
   if (al) {
@@ -544,15 +551,15 @@ static bool bn_rows_cfg(const BnProblem &p, bool backward, RowCfg &cfg, RowArgs 
   }
   // Scalar loads (planes of odd length) pay off for short rows only: beyond,
   // the split path with its tensor-aligned vectors is as fast or faster
-  // ([128,2048,7,7] fp16 forward: 34 vs 29 us).
-  if (vec == 1 && R > 4096) return false;
+  // ([128,2048,7,7] fp16 forward: 34 vs 29 us) - except on tensors so small
+  // that its three launches are the cost ([32,64,13,13] fp32: 14 us).
+  if (vec == 1 && R > 4096 && !tiny) return false;
   cfg = pick_row_cfg(vec, R, 8, 8, 4, false);
   if (!cfg.ok) return false;
   // a handful of blocks leaves the chip idle: the split reduction spreads
   // such tensors over all CUs - unless the tensor is so small (2 MB) that the
   // three launches of that path are what costs (14 vs 6 us)
-  const int64_t bytes = R * p.C * (p.dtype == NBLAHIP_F16 ? 2 : 4);
-  if ((p.C + rows_per_block(cfg.tpr) - 1) / rows_per_block(cfg.tpr) < 32 && bytes > (2 << 20))
+  if ((p.C + rows_per_block(cfg.tpr) - 1) / rows_per_block(cfg.tpr) < 32 && !tiny)
     return false;
   a = RowArgs{};
   a.x = p.x;

@@ -30,6 +30,10 @@ SMALL = [
     # channel-last with few rows: a channel vector's column in one block's registers
     ((32, 7, 7, 512), 3), ((8, 14, 14, 256), 3), ((100, 2048), 1), ((33, 8, 8, 320), 3),
     ((5000, 256), 1), ((16, 1024), 1), ((4, 2048), 1), ((6, 64), 1),
+    # tiny tensors in one launch: odd planes of 4k-8k elements per channel through
+    # scalar loads, channel-last with a handful of channels as strided rows
+    ((32, 64, 13, 13), 1), ((40, 5, 13, 15), 1), ((8, 14, 14, 3), 3), ((1, 64, 64, 3), 3),
+    ((64, 13, 13, 3), 3), ((90, 7), 1), ((1000, 1), 1), ((2, 31, 33, 8), 3),
 ]
 DTYPES = [torch.float32, torch.float16]
 
