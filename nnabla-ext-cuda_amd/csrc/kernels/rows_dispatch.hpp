@@ -10,6 +10,9 @@ namespace nblahip {
 
 int run_row_fwd_cached(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
                        hipStream_t st);
+// A row of up to 400 KB held on one CU (registers + LDS), GroupNormalization and
+// InstanceNormalization forward; false: not taken.
+bool row_onchip_fwd(const RowProblem &p, const RowArgs &args, int vec, hipStream_t st, int *status);
 int run_row_bwd_cached_ln(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
                           hipStream_t st);
 // Resident blocks per CU of the LayerNormalization backward kernel for cfg

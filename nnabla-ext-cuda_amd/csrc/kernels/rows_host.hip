@@ -272,6 +272,8 @@ int launch_row_fwd(const RowProblem &p, hipStream_t st) {
   if (cfg.ok && !tune_int("FORCE_STREAM", 0)) {
     return run_row_fwd_cached(p.dtype, cfg, a, cached_grid(p.rows, cfg.tpr), st);
   }
+  if (int status = 0; !tune_int("FORCE_STREAM", 0) && row_onchip_fwd(p, a, vec, st, &status))
+    return status;
   if (p.dtype == NBLAHIP_F16) {
     return vec == 8   ? stream_fwd_t<__half, 8>(p, a, st)
            : vec == 4 ? stream_fwd_t<__half, 4>(p, a, st)

@@ -1,0 +1,163 @@
+// GroupNormalization / InstanceNormalization forward for rows beyond what a
+// block's registers alone hold (128 KB) with the row held on one CU all the
+// same: NR 16-byte vectors per thread in registers, NS more in LDS (each
+// thread reads back what it wrote).  One 1024-thread block per row reads it
+// once, reduces, and writes y: 2 S where the streaming kernels move 3 S.
+// NR + NS = 25 covers rows of 400 KB: float groups of 100 k elements
+// ([N,320,64,64] in 32 groups, 256x256 planes), half groups of 200 k.
+#include <algorithm>
+
+#include "common.cuh"
+#include "launch.hpp"
+#include "onchip.cuh"
+#include "rows.cuh"
+
+namespace nblahip {
+
+template <typename T, int VEC, int NR, int NS>
+__global__ void __launch_bounds__(kOnchipBlock)
+row_onchip_fwd_kernel(const RowArgs a) {
+  static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors");
+  __shared__ float red[kOnchipBlock / kWave];
+  __shared__ uint4 spill[NS > 0 ? NS * kOnchipBlock : 1];
+  const uint32_t row = blockIdx.x;
+  const uint32_t t = threadIdx.x;
+  const uint32_t nv = static_cast<uint32_t>(a.R) / VEC;
+  const T *__restrict__ x = static_cast<const T *>(a.x) + static_cast<size_t>(row) * a.R;
+  T *__restrict__ y = static_cast<T *>(a.out) + static_cast<size_t>(row) * a.R;
+
+  // All loads in flight together, without a branch: a slot beyond the row
+  // reads the row's last vector and is left out of every sum and store.  The
+  // LDS part first: its registers are free again once the values are parked.
+  RawVec<T, VEC> parked[NS > 0 ? NS : 1];
+#pragma unroll
+  for (int k = 0; k < NS; ++k) {
+    const uint32_t v = static_cast<uint32_t>(NR + k) * kOnchipBlock + t;
+    parked[k] = load_raw<T, VEC>(x + min(v, nv - 1u) * VEC);
+  }
+  RawVec<T, VEC> raw[NR];
+#pragma unroll
+  for (int k = 0; k < NR; ++k) {
+    const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t;
+    raw[k] = load_raw<T, VEC>(x + min(v, nv - 1u) * VEC);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < NS; ++k) {
+    const float part = raw_sum<T, VEC>(parked[k], 0.f);
+    s += (static_cast<uint32_t>(NR + k) * kOnchipBlock + t < nv) ? part : 0.f;
+    spill[k * kOnchipBlock + t] = __builtin_bit_cast(uint4, parked[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < NR; ++k) {
+    const float part = raw_sum<T, VEC>(raw[k], 0.f);
+    s += (static_cast<uint32_t>(k) * kOnchipBlock + t < nv) ? part : 0.f;
+  }
+  const float mean = onchip_block_sum(s, red) * a.inv_R;
+#pragma unroll
+  for (int k = 0; k < NR; ++k) keep_packed<T, VEC>(raw[k]);
+
+  float q = 0.f;
+#pragma unroll
+  for (int k = 0; k < NR; ++k) {
+    if (static_cast<uint32_t>(k) * kOnchipBlock + t < nv) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float d = elem_fma<T, VEC>(raw[k], j, a.one, -mean);
+        q = fmaf(d, d, q);
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < NS; ++k) {
+    if (static_cast<uint32_t>(NR + k) * kOnchipBlock + t < nv) {
+      const RawVec<T, VEC> r = __builtin_bit_cast(RawVec<T, VEC>, spill[k * kOnchipBlock + t]);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float d = elem_fma<T, VEC>(r, j, a.one, -mean);
+        q = fmaf(d, d, q);
+      }
+    }
+  }
+  const float var = onchip_block_sum(q, red) * a.inv_R;
+  const float istd = inv_std(var, a.eps);
+  if (t == 0) {
+    a.mean[row] = mean;
+    a.var[row] = var;
+  }
+#pragma unroll
+  for (int k = 0; k < NR; ++k) keep_packed<T, VEC>(raw[k]);
+
+  // gamma/beta of a vector: one channel (a plane is a whole number of vectors)
+  const uint32_t pbase = (row % a.pmod) * a.pmul;
+  const uint32_t bbase = (row % a.pmod_b) * a.pmul;
+  auto emit = [&](const RawVec<T, VEC> &r, uint32_t v) {
+    const uint32_t poff = a.pdiv.div(v * VEC);
+    const float g = (a.gamma ? a.gamma[pbase + poff] : 1.f) * istd;
+    const float b = a.beta ? a.beta[bbase + poff] : 0.f;
+    float o[VEC];
+    if constexpr (sizeof(T) == 2) {
+      const float sh = fmaf(-mean, g, b); // x*g + (b - mean*g): one mixed fma, rounded once
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) o[j] = elem_fma<T, VEC>(r, j, g, sh);
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) o[j] = fmaf(elem_fma<T, VEC>(r, j, a.one, -mean), g, b);
+    }
+    store_vec<T, VEC>(y + v * VEC, o);
+  };
+  const uint32_t t2 = fresh(t);
+#pragma unroll
+  for (int k = 0; k < NR; ++k) {
+    const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t2;
+    if (v < nv) emit(raw[k], v);
+  }
+#pragma unroll
+  for (int k = 0; k < NS; ++k) {
+    const uint32_t v = static_cast<uint32_t>(NR + k) * kOnchipBlock + t2;
+    if (v < nv) emit(__builtin_bit_cast(RawVec<T, VEC>, spill[k * kOnchipBlock + t]), v);
+  }
+}
+
+namespace {
+
+template <typename T, int VEC>
+int run_onchip_fwd(int nl, const RowArgs &a, int grid, hipStream_t st) {
+#define ONCHIP_ROW_FWD(NR, NS)                                                              \
+  if (nl <= (NR) + (NS)) {                                                                  \
+    NBLAHIP_LAUNCH("row_onchip_fwd_kernel", (row_onchip_fwd_kernel<T, VEC, NR, NS>),        \
+                   dim3(grid), dim3(kOnchipBlock), 0, st, a);                               \
+    return last_launch_status();                                                            \
+  }
+  ONCHIP_ROW_FWD(10, 0)
+  ONCHIP_ROW_FWD(12, 0)
+  ONCHIP_ROW_FWD(14, 0)
+  ONCHIP_ROW_FWD(16, 0)
+  ONCHIP_ROW_FWD(16, 3)
+  ONCHIP_ROW_FWD(16, 6)
+  ONCHIP_ROW_FWD(16, 9)
+#undef ONCHIP_ROW_FWD
+  return NBLAHIP_EINVAL;
+}
+
+} // namespace
+
+// Rows of 8193..25600 full vectors, at least a quarter as many as there are
+// CUs (the block is alone on its CU; with fewer rows the streaming kernels,
+// which split a row over many blocks, use more of the chip).
+bool row_onchip_fwd(const RowProblem &p, const RowArgs &a, int vec, hipStream_t st, int *status) {
+  if (!tune_int("ROW_ONCHIP", 1)) return false;
+  if (p.mode == kRowLN || !p.out) return false;
+  if (vec != (p.dtype == NBLAHIP_F16 ? 8 : 4)) return false;
+  const int64_t nv = p.R / vec;
+  if (nv <= 8192 || nv > 25 * kOnchipBlock) return false;
+  if (p.rows * 100 < static_cast<int64_t>(device_cus()) * tune_int("ROW_ONCHIP_MIN_PCT", 25))
+    return false;
+  const int nl = static_cast<int>((nv + kOnchipBlock - 1) / kOnchipBlock);
+  const int grid = static_cast<int>(p.rows);
+  *status = p.dtype == NBLAHIP_F16 ? run_onchip_fwd<__half, 8>(nl, a, grid, st)
+                                   : run_onchip_fwd<float, 4>(nl, a, grid, st);
+  return true;
+}
+
+} // namespace nblahip

@@ -368,7 +368,50 @@ def test_ln_forward_in_place(outer, Rr):
     assert_close(to_np(var), v_r, "f32", "stat", "var")
 
 
-@pytest.mark.parametrize("n,c,sp", [(2, 8, (16, 16)), (1, 3, (300, 300)), (4, 64, (7, 7))])
+# Rows of 128-400 KB on at least a quarter as many rows as CUs: the forward holds
+# a row on one CU (registers + LDS).  One shape per layout (10 to 25 vectors per
+# thread), a row that ends inside a wave's load, several channels per row.
+ONCHIP_ROWS = [
+    ("in", torch.float32, 1, 64, (200, 200), 0), ("in", torch.float32, 1, 64, (216, 216), 0),
+    ("in", torch.float32, 2, 32, (232, 232), 0), ("in", torch.float32, 1, 64, (250, 256), 0),
+    ("in", torch.float32, 1, 64, (272, 272), 0), ("in", torch.float32, 1, 64, (296, 296), 0),
+    ("in", torch.float32, 1, 64, (316, 316), 0), ("in", torch.float32, 1, 70, (2, 50002), 0),
+    ("gn", torch.float32, 2, 320, (64, 64), 32), ("gn", torch.float32, 2, 512, (52, 52), 32),
+    ("gn", torch.float16, 2, 640, (64, 64), 32), ("gn", torch.float16, 1, 128, (284, 284), 64),
+    ("gn", torch.float16, 1, 192, (2, 2, 16666), 64), ("in", torch.float16, 1, 64, (400, 400), 0),
+    ("in", torch.float16, 1, 64, (448, 446), 0), ("gn", torch.float16, 1, 1536, (90, 90), 64),
+]
+
+
+@pytest.mark.parametrize("kind,dtype,n,c,sp,groups", ONCHIP_ROWS)
+def test_long_rows_held_on_chip(kind, dtype, n, c, sp, groups):
+    dn = dtype_name(dtype)
+    x, dy, g, b = make_nc(n, c, sp, dtype, 41)
+    xd, gd, bd = to_dev(x, dtype), to_dev(g), to_dev(b)
+    if kind == "in":
+        y_r, m_r, v_r = R.in_forward(x, b, g, n, c, 1e-5)
+        y, m, v = K.in_forward(xd, bd, gd, 1e-5)
+    else:
+        y_r, m_r, v_r = R.gn_forward(x, b, g, n, c, groups, 1e-5)
+        y, m, v = K.gn_forward(xd, bd, gd, groups, 1e-5)
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    assert_close(to_np(y), y_r, dn, "y", "y")
+    # the backward (streaming kernels) on the statistics the forward produced
+    dyd = to_dev(dy, dtype)
+    if kind == "in":
+        dx_r, dg_r, db_r = R.in_backward(x, dy, g, m_r, v_r, n, c, 1e-5)
+        dx, dg, db = K.in_backward(xd, dyd, gd, m, v, 1e-5)
+    else:
+        dx_r, dg_r, db_r = R.gn_backward(x, dy, g, m_r, v_r, n, c, groups, 1e-5)
+        dx, dg, db = K.gn_backward(xd, dyd, gd, m, v, groups, 1e-5)
+    assert_close(to_np(dx), dx_r, dn, "grad", "dx")
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
+
+
+@pytest.mark.parametrize("n,c,sp", [(2, 8, (16, 16)), (1, 3, (300, 300)), (4, 64, (7, 7)),
+                                    (1, 64, (400, 400))])
 def test_in_forward_in_place(n, c, sp):
     x, _, g, b = make_nc(n, c, sp, torch.float16, 32)
     y_r, m_r, v_r = R.in_forward(x, b, g, n, c, 1e-5)
