@@ -54,6 +54,11 @@ struct BnOnchipArgs {
   void *dx;                 // may be null
   const float *dmean, *dvar; // may be null
   float *dgamma, *dbeta;    // may be null
+  // InstanceNormalization backward through these kernels (a channel = one
+  // plane (n, c), C = N*C of them): gamma of channel c % gmod, and the sums
+  // go to pairs[c] = (dgamma part, dbeta part) for the batch sum that follows
+  uint32_t gmod;
+  float *pairs; // may be null
   int accum_dx, accum_g, accum_b;
 };
 
@@ -370,11 +375,15 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
   if (t == 0) {
     if (a.dgamma) a.dgamma[c] = sdx + (a.accum_g ? a.dgamma[c] : 0.f);
     if (a.dbeta) a.dbeta[c] = sdy + (a.accum_b ? a.dbeta[c] : 0.f);
+    if (a.pairs) {
+      a.pairs[2 * c] = sdx;
+      a.pairs[2 * c + 1] = sdy;
+    }
   }
   if (dx == nullptr) return;
 #pragma unroll
   for (int k = 0; k < NR; ++k) forget<T, VEC>(raw[k]);
-  const float g = a.gamma ? a.gamma[c] : 1.f;
+  const float g = a.gamma ? a.gamma[c % a.gmod] : 1.f;
   const float gi = g * istd;
   const float cA = -istd * g * sdx * a.inv_N + (a.dvar ? 2.f * a.dvar[c] * (vpe * istd) * a.inv_N : 0.f);
   const float cb = -g * sdy * istd * a.inv_N + (a.dmean ? a.dmean[c] * a.inv_N : 0.f);
@@ -545,6 +554,7 @@ bool onchip_args(const BnProblem &p, bool backward, BnOnchipArgs &a, int &nl, in
   a.decay = p.decay;
   a.eps = p.eps;
   a.one = 1.0f;
+  a.gmod = a.C;
   return true;
 }
 
@@ -573,6 +583,46 @@ bool bn_onchip_bwd(const BnProblem &p, hipStream_t st, int *status) {
   *status = p.dtype != NBLAHIP_F16 ? run_onchip_bwd<float, 4>(a.nv, a, st)
             : a.vec == 8           ? run_onchip_bwd<__half, 8>(a.nv, a, st)
                                    : run_onchip_bwd<__half, 4>(a.nv, a, st);
+  return true;
+}
+
+// InstanceNormalization backward for planes beyond what a block's registers
+// hold of x and dy together: x of a plane stays on its CU while dy is streamed
+// past it twice (4 S; the streaming kernels move 5 S).  Planes of 8193..20480
+// full vectors, at least a quarter as many as there are CUs.  The per-plane
+// sums are left in p.ws for the batch sum (or the split) that follows.
+bool in_onchip_bwd(const RowProblem &p, hipStream_t st, int *status) {
+  if (!tune_int("ROW_ONCHIP", 1) || p.mode != kRowIN) return false;
+  if (!p.out && !p.dgamma && !p.dbeta) return false;
+  const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
+  if (p.R % vec != 0 || !aligned16(p.x) || !aligned16(p.dy) || (p.out && !aligned16(p.out)))
+    return false;
+  const int64_t nv = p.R / vec;
+  if (nv <= 8192 || nv > 20480) return false;
+  if (p.rows * 100 < static_cast<int64_t>(device_cus()) * tune_int("ROW_ONCHIP_BWD_MIN_PCT", 25))
+    return false;
+  BnOnchipArgs a{};
+  a.x = p.x;
+  a.dy = p.dy;
+  a.dx = p.out;
+  a.gamma = p.gamma;
+  a.gmod = static_cast<uint32_t>(p.bc_gamma ? p.channels : p.rows);
+  a.mean = p.mean;
+  a.var = p.var;
+  a.dmean = p.dmean;
+  a.dvar = p.dvar;
+  a.pairs = (p.dgamma || p.dbeta) ? static_cast<float *>(p.ws) : nullptr;
+  a.accum_dx = p.accum_dx;
+  a.C = static_cast<uint32_t>(p.rows);
+  a.size2 = static_cast<uint32_t>(p.R);
+  a.nv = static_cast<uint32_t>(nv);
+  a.vpp = FastDiv(static_cast<uint32_t>(nv)); // one plane per channel
+  a.vec = vec;
+  a.inv_N = static_cast<float>(1.0 / static_cast<double>(p.R));
+  a.eps = p.eps;
+  a.one = 1.0f;
+  *status = p.dtype != NBLAHIP_F16 ? run_onchip_bwd<float, 4>(nv, a, st)
+                                   : run_onchip_bwd<__half, 8>(nv, a, st);
   return true;
 }
 

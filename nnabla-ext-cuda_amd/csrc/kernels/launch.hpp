@@ -70,6 +70,10 @@ struct RowProblem {
 };
 
 // Register-cached configuration: TPR threads per row, NL loads of vec elements each.
+// InstanceNormalization backward with a plane's x held on one CU (bn_onchip.hip);
+// false: not taken.  Leaves the per-plane (dgamma, dbeta) parts in p.ws.
+bool in_onchip_bwd(const RowProblem &p, hipStream_t st, int *status);
+
 struct RowCfg {
   bool ok = false;
   int vec = 1, tpr = 64, nl = 1;

@@ -380,6 +380,10 @@ ONCHIP_ROWS = [
     ("gn", torch.float16, 2, 640, (64, 64), 32), ("gn", torch.float16, 1, 128, (284, 284), 64),
     ("gn", torch.float16, 1, 192, (2, 2, 16666), 64), ("in", torch.float16, 1, 64, (400, 400), 0),
     ("in", torch.float16, 1, 64, (448, 446), 0), ("gn", torch.float16, 1, 1536, (90, 90), 64),
+    # InstanceNormalization backward with x of a plane held on its CU (every layout)
+    ("in", torch.float32, 2, 40, (190, 190), 0), ("in", torch.float32, 1, 72, (236, 236), 0),
+    ("in", torch.float32, 1, 64, (256, 256), 0), ("in", torch.float32, 1, 64, (284, 284), 0),
+    ("in", torch.float16, 1, 64, (360, 360), 0), ("in", torch.float16, 2, 33, (2, 70004), 0),
 ]
 
 
@@ -397,7 +401,7 @@ def test_long_rows_held_on_chip(kind, dtype, n, c, sp, groups):
     assert_close(to_np(m), m_r, dn, "stat", "mean")
     assert_close(to_np(v), v_r, dn, "stat", "var")
     assert_close(to_np(y), y_r, dn, "y", "y")
-    # the backward (streaming kernels) on the statistics the forward produced
+    # the backward on the statistics the forward produced
     dyd = to_dev(dy, dtype)
     if kind == "in":
         dx_r, dg_r, db_r = R.in_backward(x, dy, g, m_r, v_r, n, c, 1e-5)
