@@ -589,7 +589,8 @@ bool bn_onchip_bwd(const BnProblem &p, hipStream_t st, int *status) {
 // InstanceNormalization backward for planes beyond what a block's registers
 // hold of x and dy together: x of a plane stays on its CU while dy is streamed
 // past it twice (4 S; the streaming kernels move 5 S).  Planes of 8193..20480
-// full vectors, at least a quarter as many as there are CUs.  The per-plane
+// full vectors, at least a quarter as many as there are CUs; up to 65536 with
+// the first 18432 held.  The per-plane
 // sums are left in p.ws for the batch sum (or the split) that follows.
 bool in_onchip_bwd(const RowProblem &p, hipStream_t st, int *status) {
   if (!tune_int("ROW_ONCHIP", 1) || p.mode != kRowIN) return false;
@@ -598,9 +599,12 @@ bool in_onchip_bwd(const RowProblem &p, hipStream_t st, int *status) {
   if (p.R % vec != 0 || !aligned16(p.x) || !aligned16(p.dy) || (p.out && !aligned16(p.out)))
     return false;
   const int64_t nv = p.R / vec;
-  if (nv <= 8192 || nv > 20480) return false;
-  if (p.rows * 100 < static_cast<int64_t>(device_cus()) * tune_int("ROW_ONCHIP_BWD_MIN_PCT", 25))
-    return false;
+  if (nv <= 8192 || nv > 65536) return false;
+  // (longer planes keep 18432 vectors and stream the rest, which pays with a
+  // plane for nearly every CU, as for BatchNormalization)
+  const int min_pct = nv <= 20480 ? tune_int("ROW_ONCHIP_BWD_MIN_PCT", 25)
+                                  : tune_int("BN_ONCHIP_STREAMED_MIN_PCT", 88);
+  if (p.rows * 100 < static_cast<int64_t>(device_cus()) * min_pct) return false;
   BnOnchipArgs a{};
   a.x = p.x;
   a.dy = p.dy;

@@ -198,7 +198,8 @@ def test_gn_forward_backward(n, c, sp, groups, dtype):
     assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
 
 
-@pytest.mark.parametrize("n,c,sp,groups", [(4, 64, (16, 16), 8), (2, 32, (7, 7), 8)])
+@pytest.mark.parametrize("n,c,sp,groups", [(4, 64, (16, 16), 8), (2, 32, (7, 7), 8),
+                                           (2, 160, (64, 64), 16)])
 def test_gn_flags(n, c, sp, groups):
     dtype = torch.float32
     x, dy, g, b = make_nc(n, c, sp, dtype, 5)
@@ -255,7 +256,7 @@ def test_in_forward_backward(n, c, sp, dtype):
     assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
 
 
-@pytest.mark.parametrize("n,c,sp", [(3, 4, (6, 6)), (2, 3, (300, 300))])
+@pytest.mark.parametrize("n,c,sp", [(3, 4, (6, 6)), (2, 3, (300, 300)), (2, 32, (190, 190))])
 @pytest.mark.parametrize("bcg,bcb", [(False, False), (True, False), (False, True)])
 def test_in_per_sample_parameters_and_flags(n, c, sp, bcg, bcb):
     """gamma/beta of batch*channels elements (no broadcast over the batch),
@@ -384,6 +385,8 @@ ONCHIP_ROWS = [
     ("in", torch.float32, 2, 40, (190, 190), 0), ("in", torch.float32, 1, 72, (236, 236), 0),
     ("in", torch.float32, 1, 64, (256, 256), 0), ("in", torch.float32, 1, 64, (284, 284), 0),
     ("in", torch.float16, 1, 64, (360, 360), 0), ("in", torch.float16, 2, 33, (2, 70004), 0),
+    # ... with the first 18432 vectors held and the rest streamed
+    ("in", torch.float32, 1, 230, (300, 300), 0), ("in", torch.float16, 1, 240, (2, 150004), 0),
 ]
 
 
@@ -412,6 +415,24 @@ def test_long_rows_held_on_chip(kind, dtype, n, c, sp, groups):
     assert_close(to_np(dx), dx_r, dn, "grad", "dx")
     assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
     assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_in_backward_held_on_chip_accumulate_and_parameter_gradients_only(dtype):
+    dn = dtype_name(dtype)
+    n, c, sp = 2, 40, ((2, 24580) if dtype == torch.float32 else (2, 49156))  # 12290 vectors
+    x, dy, g, b = make_nc(n, c, sp, dtype, 43)
+    _, m_r, v_r = R.in_forward(x, b, g, n, c, 1e-5)
+    dx_r, dg_r, db_r = R.in_backward(x, dy, g, m_r, v_r, n, c, 1e-5)
+    xd, dyd, gd = to_dev(x, dtype), to_dev(dy, dtype), to_dev(g)
+    m, v = to_dev(m_r), to_dev(v_r)
+    pre = rounded(np.random.default_rng(44).standard_normal(x.shape), dtype)
+    dxd = to_dev(pre, dtype)
+    K.in_backward(xd, dyd, gd, m, v, 1e-5, dx=dxd, accum=(True, False, False))
+    assert_close(to_np(dxd), dx_r + pre, dn, "grad", "dx accumulated")
+    _, dg, db = K.in_backward(xd, dyd, gd, m, v, 1e-5, need=(False, True, True))
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma only")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta only")
 
 
 @pytest.mark.parametrize("n,c,sp", [(2, 8, (16, 16)), (1, 3, (300, 300)), (4, 64, (7, 7)),
