@@ -603,7 +603,7 @@ bool in_onchip_bwd(const RowProblem &p, hipStream_t st, int *status) {
   // (longer planes keep 18432 vectors and stream the rest, which pays with a
   // plane for nearly every CU, as for BatchNormalization)
   const int min_pct = nv <= 20480 ? tune_int("ROW_ONCHIP_BWD_MIN_PCT", 25)
-                                  : tune_int("BN_ONCHIP_STREAMED_MIN_PCT", 88);
+                                  : tune_int("ROW_ONCHIP_STREAMED_MIN_PCT", 88);
   if (p.rows * 100 < static_cast<int64_t>(device_cus()) * min_pct) return false;
   BnOnchipArgs a{};
   a.x = p.x;

@@ -14,7 +14,13 @@
 
 namespace nblahip {
 
-template <typename T, int VEC, int NR, int NS>
+// OVER: the row is longer than the NR + NS slots.  The mean of the held part
+// serves as the shift K of the whole row: the held part's second pass and ONE
+// read of the rest accumulate sum (x - K) and sum (x - K)^2, from which
+// mean = K + s1/R and var = q/R - (s1/R)^2 (K is the mean of 10^5 elements of
+// the same row: the subtracted square is tiny against the variance).  The rest
+// is read a second time for y: 2 S + (1 - 25600 / nv) S.
+template <typename T, int VEC, int NR, int NS, bool OVER = false>
 __global__ void __launch_bounds__(kOnchipBlock)
 row_onchip_fwd_kernel(const RowArgs a) {
   static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors");
@@ -53,11 +59,14 @@ row_onchip_fwd_kernel(const RowArgs a) {
     const float part = raw_sum<T, VEC>(raw[k], 0.f);
     s += (static_cast<uint32_t>(k) * kOnchipBlock + t < nv) ? part : 0.f;
   }
-  const float mean = onchip_block_sum(s, red) * a.inv_R;
+  // (OVER: the shift K, over the held elements only)
+  constexpr uint32_t kHeld = static_cast<uint32_t>(NR + NS) * kOnchipBlock;
+  float mean = onchip_block_sum(s, red) * (OVER ? 1.0f / (static_cast<float>(kHeld) * VEC) : a.inv_R);
 #pragma unroll
   for (int k = 0; k < NR; ++k) keep_packed<T, VEC>(raw[k]);
 
   float q = 0.f;
+  float s1 = 0.f; // OVER: sum (x - K), the held part's rounding residue included
 #pragma unroll
   for (int k = 0; k < NR; ++k) {
     if (static_cast<uint32_t>(k) * kOnchipBlock + t < nv) {
@@ -65,6 +74,7 @@ row_onchip_fwd_kernel(const RowArgs a) {
       for (int j = 0; j < VEC; ++j) {
         const float d = elem_fma<T, VEC>(raw[k], j, a.one, -mean);
         q = fmaf(d, d, q);
+        if constexpr (OVER) s1 += d;
       }
     }
   }
@@ -76,10 +86,39 @@ row_onchip_fwd_kernel(const RowArgs a) {
       for (int j = 0; j < VEC; ++j) {
         const float d = elem_fma<T, VEC>(r, j, a.one, -mean);
         q = fmaf(d, d, q);
+        if constexpr (OVER) s1 += d;
       }
     }
   }
-  const float var = onchip_block_sum(q, red) * a.inv_R;
+  constexpr int BO = 4; // vectors per thread and step of the streamed rest
+  if constexpr (OVER) {
+#pragma unroll 1
+    for (uint32_t v0 = kHeld; v0 < nv; v0 += BO * kOnchipBlock) {
+      RawVec<T, VEC> xo[BO];
+#pragma unroll
+      for (int b = 0; b < BO; ++b)
+        xo[b] = load_raw<T, VEC>(x + min(v0 + b * kOnchipBlock + t, nv - 1u) * VEC);
+#pragma unroll
+      for (int b = 0; b < BO; ++b) {
+        float ps = 0.f, pq = 0.f;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float d = elem_fma<T, VEC>(xo[b], j, a.one, -mean);
+          ps += d;
+          pq = fmaf(d, d, pq);
+        }
+        const bool ok = v0 + b * kOnchipBlock + t < nv;
+        s1 += ok ? ps : 0.f;
+        q += ok ? pq : 0.f;
+      }
+    }
+    s1 = onchip_block_sum(s1, red) * a.inv_R; // mean - K
+  }
+  float var = onchip_block_sum(q, red) * a.inv_R;
+  if constexpr (OVER) {
+    var = fmaxf(var - s1 * s1, 0.f);
+    mean += s1;
+  }
   const float istd = inv_std(var, a.eps);
   if (t == 0) {
     a.mean[row] = mean;
@@ -117,6 +156,20 @@ row_onchip_fwd_kernel(const RowArgs a) {
     const uint32_t v = static_cast<uint32_t>(NR + k) * kOnchipBlock + t2;
     if (v < nv) emit(__builtin_bit_cast(RawVec<T, VEC>, spill[k * kOnchipBlock + t]), v);
   }
+  if constexpr (OVER) {
+#pragma unroll 1
+    for (uint32_t v0 = kHeld; v0 < nv; v0 += BO * kOnchipBlock) {
+      RawVec<T, VEC> xo[BO];
+#pragma unroll
+      for (int b = 0; b < BO; ++b)
+        xo[b] = load_raw<T, VEC>(x + min(v0 + b * kOnchipBlock + t, nv - 1u) * VEC);
+#pragma unroll
+      for (int b = 0; b < BO; ++b) {
+        const uint32_t v = v0 + b * kOnchipBlock + t;
+        if (v < nv) emit(xo[b], v);
+      }
+    }
+  }
 }
 
 namespace {
@@ -137,7 +190,10 @@ int run_onchip_fwd(int nl, const RowArgs &a, int grid, hipStream_t st) {
   ONCHIP_ROW_FWD(16, 6)
   ONCHIP_ROW_FWD(16, 9)
 #undef ONCHIP_ROW_FWD
-  return NBLAHIP_EINVAL;
+  // longer rows: 25 slots held, the rest streamed
+  NBLAHIP_LAUNCH("row_onchip_fwd_kernel", (row_onchip_fwd_kernel<T, VEC, 16, 9, true>), dim3(grid),
+                 dim3(kOnchipBlock), 0, st, a);
+  return last_launch_status();
 }
 
 } // namespace
@@ -145,15 +201,17 @@ int run_onchip_fwd(int nl, const RowArgs &a, int grid, hipStream_t st) {
 // Rows of 8193..25600 full vectors, at least an eighth as many as there are
 // CUs (the block is alone on its CU; with fewer rows the streaming kernels,
 // which split a row over many blocks, use more of the chip: 32 groups of 160 KB
-// 8.3 vs 11.8 us, 16 of 320 KB 12.6 vs 11.7 us).
+// 8.3 vs 11.8 us, 16 of 320 KB 12.6 vs 11.7 us); up to 65536 vectors with the
+// first 25600 held, given a row for nearly every CU.
 bool row_onchip_fwd(const RowProblem &p, const RowArgs &a, int vec, hipStream_t st, int *status) {
   if (!tune_int("ROW_ONCHIP", 1)) return false;
   if (p.mode == kRowLN || !p.out) return false;
   if (vec != (p.dtype == NBLAHIP_F16 ? 8 : 4)) return false;
   const int64_t nv = p.R / vec;
-  if (nv <= 8192 || nv > 25 * kOnchipBlock) return false;
-  if (p.rows * 100 < static_cast<int64_t>(device_cus()) * tune_int("ROW_ONCHIP_MIN_PCT", 12))
-    return false;
+  if (nv <= 8192 || nv > 65536) return false;
+  const int min_pct = nv <= 25 * kOnchipBlock ? tune_int("ROW_ONCHIP_MIN_PCT", 12)
+                                              : tune_int("ROW_ONCHIP_STREAMED_MIN_PCT", 88);
+  if (p.rows * 100 < static_cast<int64_t>(device_cus()) * min_pct) return false;
   const int nl = static_cast<int>((nv + kOnchipBlock - 1) / kOnchipBlock);
   const int grid = static_cast<int>(p.rows);
   *status = p.dtype == NBLAHIP_F16 ? run_onchip_fwd<__half, 8>(nl, a, grid, st)

@@ -381,6 +381,9 @@ ONCHIP_ROWS = [
     ("gn", torch.float16, 2, 640, (64, 64), 32), ("gn", torch.float16, 1, 128, (284, 284), 64),
     ("gn", torch.float16, 1, 192, (2, 2, 16666), 64), ("in", torch.float16, 1, 64, (400, 400), 0),
     ("in", torch.float16, 1, 64, (448, 446), 0), ("gn", torch.float16, 1, 1536, (90, 90), 64),
+    # rows of 25601-65536 vectors: the first 25600 held, the rest streamed (forward)
+    ("in", torch.float32, 1, 226, (322, 322), 0), ("gn", torch.float16, 2, 452, (2, 130004), 226),
+    ("in", torch.float16, 1, 226, (2, 131076), 0),
     # InstanceNormalization backward with x of a plane held on its CU (every layout)
     ("in", torch.float32, 2, 40, (190, 190), 0), ("in", torch.float32, 1, 72, (236, 236), 0),
     ("in", torch.float32, 1, 64, (256, 256), 0), ("in", torch.float32, 1, 64, (284, 284), 0),
@@ -436,7 +439,7 @@ def test_in_backward_held_on_chip_accumulate_and_parameter_gradients_only(dtype)
 
 
 @pytest.mark.parametrize("n,c,sp", [(2, 8, (16, 16)), (1, 3, (300, 300)), (4, 64, (7, 7)),
-                                    (1, 64, (400, 400))])
+                                    (1, 64, (400, 400)), (1, 226, (2, 104008))])
 def test_in_forward_in_place(n, c, sp):
     x, _, g, b = make_nc(n, c, sp, torch.float16, 32)
     y_r, m_r, v_r = R.in_forward(x, b, g, n, c, 1e-5)
