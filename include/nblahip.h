@@ -92,6 +92,27 @@ NBLAHIP_EXPORT int nblahip_bn_fwd_train(const void *x, const float *gamma,
                                         float eps, int dtype, void *workspace,
                                         size_t workspace_bytes, void *stream);
 
+/* nblahip_bn_fwd_train for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  It has no counterpart in the reference.  Same arguments and
+ * results as nblahip_bn_fwd_train minus the workspace: the partials of the
+ * split reduction live in an array of
+ * nblahip_bn_fwd_train_static_max_workspace() bytes (4 MiB) inside the
+ * library's code object, one per GPU, held until the process ends.  A shape
+ * whose nblahip_bn_workspace_bytes() exceeds that returns NBLAHIP_EWORKSPACE.
+ * The call allocates and frees nothing.  All calls on one GPU share the array:
+ * calls that overlap in time on the same GPU (different streams or threads)
+ * race, so keep them on one stream.  The array's address is looked up on the
+ * first call per device; a call with an empty tensor (size0 == 0) does that
+ * look-up and launches nothing, which is the set-up step to make before a
+ * capture starts. */
+NBLAHIP_EXPORT size_t nblahip_bn_fwd_train_static_max_workspace(void);
+NBLAHIP_EXPORT int nblahip_bn_fwd_train_static(
+    const void *x, const float *gamma, const float *beta, void *y,
+    float *batch_mean, float *batch_var, float *rmean, float *rvar,
+    int64_t size0, int64_t size1, int64_t size2, float decay_rate, float eps,
+    int dtype, void *stream);
+
 /* Replaces backward_impl_batch (batch_normalization.cu:215-316, kernels
  * cuh:402-540) and cudnnBatchNormalizationBackward(Ex)
  * (cudnn/.../batch_normalization.cu:328-457).  mean/var are the statistics the

@@ -32,6 +32,8 @@ SIGNATURES = {
     "nblahip_bn_workspace_bytes": (_sz, [_i64] * 3 + [_int]),
     "nblahip_bn_fwd_train": (_int, [_c_void_p] * 8 + [_i64] * 3 + [_f, _f, _int, _c_void_p, _sz,
                                                               _c_void_p]),
+    "nblahip_bn_fwd_train_static_max_workspace": (_sz, []),
+    "nblahip_bn_fwd_train_static": (_int, [_c_void_p] * 8 + [_i64] * 3 + [_f, _f, _int, _c_void_p]),
     "nblahip_bn_bwd": (_int, [_c_void_p] * 10 + [_int] * 3 + [_i64] * 3 + [_f, _int, _int,
                                                                    _c_void_p, _sz, _c_void_p]),
     "nblahip_bn_local_stats": (_int, [_c_void_p] * 3 + [_i64] * 3 + [_int, _c_void_p, _sz, _c_void_p]),
@@ -199,6 +201,24 @@ def bn_forward_batch(x, beta, gamma, rmean, rvar, axis=1, decay_rate=0.9, eps=1e
                                      _ptr(y), _ptr(mean), _ptr(var), _ptr(_f32(rmean, "rmean")),
                                      _ptr(_f32(rvar, "rvar")), s0, c, s2, decay_rate, eps, dt,
                                      _ptr(ws), ws.numel(), _stream()))
+    return y, mean, var
+
+
+def bn_forward_batch_static(x, beta, gamma, rmean, rvar, axis=1, decay_rate=0.9, eps=1e-5,
+                            out=None):
+    """bn_forward_batch through the entry point that allocates nothing; out =
+    (y, mean, var) preallocated by the caller (allocated here when None)."""
+    import torch
+    assert x.is_contiguous()
+    s0, c, s2 = _bn_sizes(x.shape, axis)
+    if out is None:
+        out = (torch.empty_like(x), torch.empty(c, dtype=torch.float32, device=x.device),
+               torch.empty(c, dtype=torch.float32, device=x.device))
+    y, mean, var = out
+    check(lib().nblahip_bn_fwd_train_static(
+        _ptr(x), _ptr(_f32(gamma, "gamma")), _ptr(_f32(beta, "beta")), _ptr(y), _ptr(mean),
+        _ptr(var), _ptr(_f32(rmean, "rmean")), _ptr(_f32(rvar, "rvar")), s0, c, s2, decay_rate,
+        eps, _dtype_code(x), _stream()))
     return y, mean, var
 
 

@@ -1,6 +1,8 @@
 // C-ABI entry points of the normalization kernels: argument validation and
 // translation into launch-layer problems.  Nothing here allocates, throws or
 // waits for the device.
+#include <atomic>
+
 #include "launch.hpp"
 
 using namespace nblahip;
@@ -28,6 +30,34 @@ int check_dims3(int64_t a, int64_t b, int64_t c) {
 }
 
 hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
+
+// Scratch of nblahip_bn_fwd_train_static, the entry point for callers that
+// cannot allocate: one array per GPU in the code object's own data segment,
+// held until the process ends.  `scratch` below is only the host-side handle
+// of that array; the device address is looked up once per device and kept in
+// g_scratch_ptr, and host code passes that pointer, never the handle, to
+// kernels.
+constexpr size_t kStaticScratchBytes = size_t{4} << 20;
+constexpr int kMaxDevices = 64;
+__device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+std::atomic<void *> g_scratch_ptr[kMaxDevices];
+
+// Device address of the current device's scratch array (resolved on the first
+// call per device; two threads resolving at once store the same address).
+int static_scratch(void **out) {
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return static_cast<int>(e);
+  if (dev < 0 || dev >= kMaxDevices) return NBLAHIP_EINVAL;
+  void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    if (hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)); e != hipSuccess)
+      return static_cast<int>(e);
+    if (!ptr) return static_cast<int>(hipErrorInvalidSymbol);
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return 0;
+}
 
 } // namespace
 
@@ -157,6 +187,26 @@ int nblahip_bn_fwd_train(const void *x, const float *gamma, const float *beta, v
   return bn_fwd_train_impl(x, nullptr, 0, gamma, beta, y, batch_mean, batch_var, rmean, rvar,
                            size0, size1, size2, decay_rate, eps, dtype, workspace,
                            workspace_bytes, stream);
+}
+
+size_t nblahip_bn_fwd_train_static_max_workspace(void) { return kStaticScratchBytes; }
+
+int nblahip_bn_fwd_train_static(const void *x, const float *gamma, const float *beta, void *y,
+                                float *batch_mean, float *batch_var, float *rmean, float *rvar,
+                                int64_t size0, int64_t size1, int64_t size2, float decay_rate,
+                                float eps, int dtype, void *stream) {
+  // Shapes whose partials do not fit the static array are turned away before
+  // anything touches the device.
+  if (dtype_ok(dtype) && check_dims3(size0, size1, size2) == 0 &&
+      bn_workspace_bytes(size0, size1, size2, dtype) > kStaticScratchBytes)
+    return NBLAHIP_EWORKSPACE;
+  void *ws = nullptr;
+  if (int e = static_scratch(&ws)) return e;
+  // The split reduction writes every partial before it reads it: nothing in
+  // the array has to start at zero.
+  return bn_fwd_train_impl(x, nullptr, 0, gamma, beta, y, batch_mean, batch_var, rmean, rvar,
+                           size0, size1, size2, decay_rate, eps, dtype, ws, kStaticScratchBytes,
+                           stream);
 }
 
 int nblahip_bn_bwd(const void *x, const void *dy, const float *gamma, const float *mean,
