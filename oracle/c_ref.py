@@ -23,6 +23,8 @@ def lib():
             raise RuntimeError(f"{LIB_PATH} missing: run `make -C {_HERE}`")
         L = ctypes.CDLL(LIB_PATH)
         L.nr_num_threads.restype = _i
+        L.nr_set_num_threads.argtypes = [_i]
+        L.nr_set_num_threads.restype = None
         L.nr_bn_forward_global.argtypes = [_P] * 6 + [_I] * 3 + [_F]
         L.nr_bn_forward_batch.argtypes = [_P] * 8 + [_I] * 3 + [_F, _F]
         L.nr_bn_backward_batch.argtypes = [_P] * 10 + [_I] * 3 + [_F]

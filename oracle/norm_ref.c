@@ -30,6 +30,15 @@ NR_EXPORT int nr_num_threads(void) {
 #endif
 }
 
+/* n >= 1: threads of the following calls (1 = the scalar port). */
+NR_EXPORT void nr_set_num_threads(int n) {
+#ifdef _OPENMP
+  if (n >= 1) omp_set_num_threads(n);
+#else
+  (void)n;
+#endif
+}
+
 /* ---- Welford, include/nbla/cuda/utils/reduce_ops/welford.cuh:62-97 ------ */
 typedef struct {
   double mean, m2;
