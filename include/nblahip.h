@@ -430,6 +430,18 @@ NBLAHIP_EXPORT int nblahip_convert(void *dst, int dst_dtype, const void *src,
 NBLAHIP_EXPORT int nblahip_fill(void *dst, int dtype, float value, int64_t n,
                                 void *stream);
 
+/* Axis permutation of a contiguous tensor (float32 or float16):
+ *   dst[i_perm[0], ..., i_perm[ndim-1]] = src[i_0, ..., i_{ndim-1}]
+ * i.e. axis k of dst is axis perm[k] of src, whose extents are shape[0..ndim-1]
+ * (ndim <= 8); accum != 0 adds onto dst.  The Function classes use it for the
+ * layouts the normalization kernels do not read in place; it replaces the
+ * transposes of the core's ChannelFirstAdaptor the reference calls
+ * (group_normalization.cu:40-55,93-109, instance_normalization.cu:40-51,81-94)
+ * and its generic transpose kernel (kernel/transpose.cuh:19-53). */
+NBLAHIP_EXPORT int nblahip_permute(const void *src, void *dst, int ndim,
+                                   const int64_t *shape, const int *perm,
+                                   int accum, int dtype, void *stream);
+
 /* ------------------------------------------------------------------------
  * Per-kernel event timing, the counterpart of the reference's
  * CudaEventTimerCallback (python/src/nnabla_ext/cuda/utils/inspection/

@@ -73,8 +73,9 @@ NNABLA_HIP_EXPORT nnabla_hip_function *nnabla_hip_create_instance_normalization(
     const int *batch_axis, int n_batch_axis, float eps, int no_scale, int no_bias);
 /* TensorNormalizationCuda / WeightStandardizationCuda
  * (include/nbla/cuda/function/tensor_normalization.hpp:22-46,
- * weight_standardization.hpp:22-46).  axes: the axes the statistics keep; they
- * must be adjacent (the reference's composite transposes for other sets). */
+ * weight_standardization.hpp:22-46).  axes: the axes the statistics keep,
+ * read in place when adjacent, gathered by a device permutation otherwise (the
+ * reference's composite transposes for such sets). */
 NNABLA_HIP_EXPORT nnabla_hip_function *nnabla_hip_create_tensor_normalization(
     const char *backends, const char *array_class, const char *device_id, const int *axes,
     int n_axes, float eps, int no_scale, int no_bias);

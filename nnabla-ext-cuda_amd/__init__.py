@@ -86,6 +86,8 @@ SIGNATURES = {
     "nblahip_memset": (_int, [_c_void_p, _int, _sz, _c_void_p]),
     "nblahip_convert": (_int, [_c_void_p, _int, _c_void_p, _int, _i64, _c_void_p]),
     "nblahip_fill": (_int, [_c_void_p, _int, _f, _i64, _c_void_p]),
+    "nblahip_permute": (_int, [_c_void_p, _c_void_p, _int, ctypes.POINTER(_i64),
+                               ctypes.POINTER(_int), _int, _int, _c_void_p]),
     "nblahip_profile_enable": (_int, [_int]),
     "nblahip_profile_reset": (_int, []),
     "nblahip_profile_query": (_int, [ctypes.c_char_p, ctypes.POINTER(ctypes.c_double),
@@ -522,3 +524,17 @@ def in_backward(x, dy, gamma, mean, var, eps=1e-5, bc_gamma=True, bc_beta=True, 
                                int(bc_gamma), int(bc_beta), eps, dt, _ptr(ws), ws.numel(),
                                _stream()))
     return (dx if need[0] else None, dgamma if need[1] else None, dbeta if need[2] else None)
+
+
+def permute(x, perm, out=None, accum=False):
+    """out (+)= x.permute(perm), contiguous (nblahip_permute)."""
+    import torch
+    assert x.is_contiguous()
+    nd = x.dim()
+    shape = (_i64 * nd)(*x.shape)
+    pm = (_int * nd)(*perm)
+    if out is None:
+        out = torch.empty([x.shape[p] for p in perm], dtype=x.dtype, device=x.device)
+    check(lib().nblahip_permute(_ptr(x), _ptr(out), nd, shape, pm, int(accum), _dtype_code(x),
+                                _stream()))
+    return out

@@ -6,6 +6,7 @@
 #include <nbla/function/group_normalization.hpp>
 #include <nbla/hip/common.hpp>
 #include <nbla/hip/hip.hpp>
+#include <nbla/hip/utils/channel_layout.hpp>
 
 namespace nbla {
 
@@ -17,6 +18,10 @@ protected:
   Variable mean_, var_;   // float32 per-(n, group) statistics kept for backward
   Variable workspace_;
   size_t workspace_bytes_ = 0;
+  // Layouts that are neither channel-first nor channel-last: permuted copies
+  // of x / dy / y / dx and of the statistics, alive only inside a call.
+  ChannelLayout layout_;
+  Variable adapt_a_, adapt_b_, adapt_c_, stat_a_, stat_b_, stat_c_, stat_d_;
 
 public:
   GroupNormalizationHip(const Context &ctx, int num_groups, int channel_axis,

@@ -6,6 +6,7 @@
 #include <nbla/function/instance_normalization.hpp>
 #include <nbla/hip/common.hpp>
 #include <nbla/hip/hip.hpp>
+#include <nbla/hip/utils/channel_layout.hpp>
 
 namespace nbla {
 
@@ -17,6 +18,12 @@ protected:
   Variable mean_, var_;   // float32 per-(n, c) statistics kept for backward
   Variable workspace_;
   size_t workspace_bytes_ = 0;
+  // Layouts that are neither channel-first nor channel-last: permuted copies
+  // of x / dy / y / dx, of the statistics and of per-sample parameters, alive
+  // only inside a call.
+  ChannelLayout layout_;
+  Variable adapt_a_, adapt_b_, adapt_c_;
+  Variable stat_a_, stat_b_, stat_c_, stat_d_, stat_e_, stat_f_, stat_g_;
 
 public:
   InstanceNormalizationHip(const Context &ctx, int channel_axis, const vector<int> &batch_axis,

@@ -6,6 +6,7 @@
 #include <nbla/function/layer_normalization.hpp>
 #include <nbla/hip/common.hpp>
 #include <nbla/hip/hip.hpp>
+#include <nbla/hip/utils/axis_adaptor.hpp>
 
 namespace nbla {
 
@@ -16,6 +17,10 @@ protected:
   Variable mean_, var_;   // float32 row statistics kept for backward
   Variable workspace_;
   size_t workspace_bytes_ = 0;
+  // Batch axes that are not the leading ones: permuted copies of x / dy / y /
+  // dx, alive only inside a call.
+  AxisAdaptor adaptor_;
+  Variable adapt_a_, adapt_b_, adapt_c_;
 
 public:
   LayerNormalizationHip(const Context &ctx, const vector<int> &batch_axis, float eps,

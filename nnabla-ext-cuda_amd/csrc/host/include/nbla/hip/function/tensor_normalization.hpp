@@ -9,6 +9,7 @@
 #include <nbla/function/tensor_normalization.hpp>
 #include <nbla/hip/common.hpp>
 #include <nbla/hip/hip.hpp>
+#include <nbla/hip/utils/axis_adaptor.hpp>
 
 namespace nbla {
 
@@ -19,6 +20,10 @@ protected:
   Variable mean_, var_; // float32 statistics kept for backward
   Variable workspace_;
   size_t workspace_bytes_ = 0;
+  // Kept axes that are not adjacent: permuted copies of x / dy / y / dx, alive
+  // only inside a call.
+  AxisAdaptor adaptor_;
+  Variable adapt_a_, adapt_b_, adapt_c_;
 
 public:
   TensorNormalizationHip(const Context &ctx, const vector<int> &axes, float eps, bool no_scale,

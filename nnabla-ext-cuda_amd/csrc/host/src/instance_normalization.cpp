@@ -10,25 +10,15 @@ template <typename T>
 void InstanceNormalizationHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
   InstanceNormalization<T>::setup_shapes(inputs, outputs);
   const auto x = inputs[0];
-  const int c = this->channel_axis_;
-  // Two layouts run without a transpose: channel-first (the channel axis
-  // right after the leading batch axes) and channel-last (batch axes leading,
-  // channel axis last).  The reference brings every other layout to
-  // channel-first through the core's ChannelFirstAdaptor
-  // (instance_normalization.cu:40-55); that adaptor is not part of this backend.
-  const int nb = static_cast<int>(this->batch_axis_.size());
-  const int ndim = static_cast<int>(x->shape().size());
-  bool batch_leading = true;
-  for (int b : this->batch_axis_) batch_leading = batch_leading && b < nb;
-  const bool channel_first = batch_leading && c == nb;
-  channel_last_ = batch_leading && !channel_first && c == ndim - 1;
-  NBLA_CHECK(channel_first || channel_last_, error_code::not_implemented,
-             "InstanceNormalizationHip supports batch axes leading with the channel axis right "
-             "after them (channel-first) or last (channel-last).");
-  channel_size_ = x->shape()[c];
-  batch_size_ = 1;
-  for (int b : this->batch_axis_) batch_size_ *= x->shape()[b];
-  spatial_size_ = (batch_size_ > 0 && channel_size_ > 0) ? x->size() / (batch_size_ * channel_size_) : 0;
+  // Channel-first and channel-last tensors are read in place; any other
+  // position of the channel and batch axes goes through a device permutation
+  // to channel-first and back, the counterpart of the ChannelFirstAdaptor the
+  // reference uses (instance_normalization.cu:40-55,81-94,187-207).
+  layout_.setup(x->shape(), this->batch_axis_, this->channel_axis_, x->shape()[this->channel_axis_]);
+  channel_last_ = layout_.channel_last;
+  channel_size_ = layout_.channels;
+  batch_size_ = layout_.batch;
+  spatial_size_ = layout_.spatial;
   NBLA_CHECK(x->size() < (Size_t(1) << 31), error_code::value,
              "InstanceNormalizationHip indexes with 32 bits: fewer than 2^31 elements required.");
   mean_.reshape(Shape_t{batch_size_ * channel_size_}, true);
@@ -59,19 +49,54 @@ void InstanceNormalizationHip<T>::forward_impl(const Variables &inputs, const Va
   T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
   float *mean = v_mean->cast_data_and_get_pointer<float>(this->ctx_, true);
   float *var = v_var->cast_data_and_get_pointer<float>(this->ctx_, true);
+  const int bc_gamma = this->need_gamma_broadcast_ ? 1 : 0, bc_beta = this->need_beta_broadcast_ ? 1 : 0;
   if (channel_last_) {
     float *ws = workspace_.cast_data_and_get_pointer<float>(this->ctx_, true);
     NBLA_HIP_CHECK(nblahip_in_cl_fwd(x, gamma, beta, y, mean, var, batch_size_, spatial_size_,
-                                     channel_size_, this->need_gamma_broadcast_ ? 1 : 0,
-                                     this->need_beta_broadcast_ ? 1 : 0, this->eps_,
+                                     channel_size_, bc_gamma, bc_beta, this->eps_,
                                      HipDtype<T>::code, ws, workspace_bytes_, nullptr));
     workspace_.data()->array()->clear();
     return;
   }
-  NBLA_HIP_CHECK(nblahip_in_fwd(x, gamma, beta, y, mean, var, batch_size_, channel_size_,
-                                spatial_size_, this->need_gamma_broadcast_ ? 1 : 0,
-                                this->need_beta_broadcast_ ? 1 : 0, this->eps_, HipDtype<T>::code,
+  const bool adapt = layout_.data.needed(), adapt_stats = layout_.stats.needed();
+  const Size_t n = inputs[0]->size(), ns = batch_size_ * channel_size_;
+  const T *xk = x;
+  T *yk = y;
+  float *mk = mean, *vk = var;
+  if (adapt) {
+    T *xs = adaptor_scratch<T>(adapt_a_, n, this->ctx_);
+    layout_.data.to_kernel(x, xs, HipDtype<T>::code);
+    xk = xs;
+    yk = adaptor_scratch<T>(adapt_b_, n, this->ctx_);
+  }
+  if (adapt_stats) {
+    // statistics and per-sample parameters are [batch..., channel] for the kernels
+    mk = adaptor_scratch<float>(stat_a_, ns, this->ctx_);
+    vk = adaptor_scratch<float>(stat_b_, ns, this->ctx_);
+    if (gamma && !bc_gamma) {
+      float *gk = adaptor_scratch<float>(stat_c_, ns, this->ctx_);
+      layout_.stats.to_kernel(gamma, gk, NBLAHIP_F32);
+      gamma = gk;
+    }
+    if (beta && !bc_beta) {
+      float *bk = adaptor_scratch<float>(stat_d_, ns, this->ctx_);
+      layout_.stats.to_kernel(beta, bk, NBLAHIP_F32);
+      beta = bk;
+    }
+  }
+  NBLA_HIP_CHECK(nblahip_in_fwd(xk, gamma, beta, yk, mk, vk, batch_size_, channel_size_,
+                                spatial_size_, bc_gamma, bc_beta, this->eps_, HipDtype<T>::code,
                                 nullptr));
+  if (adapt) {
+    layout_.data.to_caller(yk, y, false, HipDtype<T>::code);
+    adaptor_release(adapt_a_);
+    adaptor_release(adapt_b_);
+  }
+  if (adapt_stats) {
+    layout_.stats.to_caller(mk, mean, false, NBLAHIP_F32);
+    layout_.stats.to_caller(vk, var, false, NBLAHIP_F32);
+    for (Variable *v : {&stat_a_, &stat_b_, &stat_c_, &stat_d_}) adaptor_release(*v);
+  }
 }
 
 template <typename T>
@@ -109,20 +134,73 @@ void InstanceNormalizationHip<T>::backward_impl(const Variables &inputs, const V
                             : inputs[gamma_idx]->template cast_grad_and_get_pointer<float>(
                                   this->ctx_, !accum[gamma_idx]);
   float *ws = workspace_.cast_data_and_get_pointer<float>(this->ctx_, true);
+  const int bc_gamma = this->need_gamma_broadcast_ ? 1 : 0, bc_beta = this->need_beta_broadcast_ ? 1 : 0;
   if (channel_last_) {
     NBLA_HIP_CHECK(nblahip_in_cl_bwd(x, dy, gamma, mean, var, dmean, dvar, dx, dgamma, dbeta,
                                      pd_x && accum[0], pd_gamma && accum[gamma_idx],
                                      pd_beta && accum[beta_idx], batch_size_, spatial_size_,
-                                     channel_size_, this->need_gamma_broadcast_ ? 1 : 0,
-                                     this->need_beta_broadcast_ ? 1 : 0, this->eps_,
+                                     channel_size_, bc_gamma, bc_beta, this->eps_,
                                      HipDtype<T>::code, ws, workspace_bytes_, nullptr));
-  } else {
-    NBLA_HIP_CHECK(nblahip_in_bwd(x, dy, gamma, mean, var, dmean, dvar, dx, dgamma, dbeta,
-                                  pd_x && accum[0], pd_gamma && accum[gamma_idx],
-                                  pd_beta && accum[beta_idx], batch_size_, channel_size_,
-                                  spatial_size_, this->need_gamma_broadcast_ ? 1 : 0,
-                                  this->need_beta_broadcast_ ? 1 : 0, this->eps_,
-                                  HipDtype<T>::code, ws, workspace_bytes_, nullptr));
+    workspace_.data()->array()->clear();
+    return;
+  }
+  const bool adapt = layout_.data.needed(), adapt_stats = layout_.stats.needed();
+  const Size_t n = inputs[0]->size(), ns = batch_size_ * channel_size_;
+  const T *xk = x, *dyk = dy;
+  T *dxk = dx;
+  if (adapt) {
+    T *xs = adaptor_scratch<T>(adapt_a_, n, this->ctx_);
+    T *dys = adaptor_scratch<T>(adapt_b_, n, this->ctx_);
+    layout_.data.to_kernel(x, xs, HipDtype<T>::code);
+    layout_.data.to_kernel(dy, dys, HipDtype<T>::code);
+    xk = xs;
+    dyk = dys;
+    if (pd_x) dxk = adaptor_scratch<T>(adapt_c_, n, this->ctx_);
+  }
+  // Per-sample parameter gradients come back in the kernels' [batch...,
+  // channel] order and are added to the caller's afterwards.
+  float *dgk = dgamma, *dbk = dbeta;
+  const bool own_dg = adapt_stats && dgamma && !bc_gamma, own_db = adapt_stats && dbeta && !bc_beta;
+  if (adapt_stats) {
+    float *mk = adaptor_scratch<float>(stat_a_, ns, this->ctx_);
+    float *vk = adaptor_scratch<float>(stat_b_, ns, this->ctx_);
+    layout_.stats.to_kernel(mean, mk, NBLAHIP_F32);
+    layout_.stats.to_kernel(var, vk, NBLAHIP_F32);
+    mean = mk;
+    var = vk;
+    if (dmean) {
+      float *dmk = adaptor_scratch<float>(stat_c_, ns, this->ctx_);
+      float *dvk = adaptor_scratch<float>(stat_d_, ns, this->ctx_);
+      layout_.stats.to_kernel(dmean, dmk, NBLAHIP_F32);
+      layout_.stats.to_kernel(dvar, dvk, NBLAHIP_F32);
+      dmean = dmk;
+      dvar = dvk;
+    }
+    if (gamma && !bc_gamma) {
+      float *gk = adaptor_scratch<float>(stat_e_, ns, this->ctx_);
+      layout_.stats.to_kernel(gamma, gk, NBLAHIP_F32);
+      gamma = gk;
+    }
+    if (own_dg) dgk = adaptor_scratch<float>(stat_f_, ns, this->ctx_);
+    if (own_db) dbk = adaptor_scratch<float>(stat_g_, ns, this->ctx_);
+  }
+  NBLA_HIP_CHECK(nblahip_in_bwd(xk, dyk, gamma, mean, var, dmean, dvar, dxk, dgk, dbk,
+                                !adapt && pd_x && accum[0],
+                                !own_dg && pd_gamma && accum[gamma_idx],
+                                !own_db && pd_beta && accum[beta_idx], batch_size_, channel_size_,
+                                spatial_size_, bc_gamma, bc_beta, this->eps_, HipDtype<T>::code, ws,
+                                workspace_bytes_, nullptr));
+  if (adapt) {
+    if (pd_x) layout_.data.to_caller(dxk, dx, accum[0], HipDtype<T>::code);
+    adaptor_release(adapt_a_);
+    adaptor_release(adapt_b_);
+    adaptor_release(adapt_c_);
+  }
+  if (adapt_stats) {
+    if (own_dg) layout_.stats.to_caller(dgk, dgamma, accum[gamma_idx], NBLAHIP_F32);
+    if (own_db) layout_.stats.to_caller(dbk, dbeta, accum[beta_idx], NBLAHIP_F32);
+    for (Variable *v : {&stat_a_, &stat_b_, &stat_c_, &stat_d_, &stat_e_, &stat_f_, &stat_g_})
+      adaptor_release(*v);
   }
   workspace_.data()->array()->clear();
 }

@@ -9,13 +9,15 @@ template <typename T>
 void LayerNormalizationHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
   LayerNormalization<T>::setup_shapes(inputs, outputs);
   const auto x_shape = inputs[0]->shape();
-  // The kernels reduce over trailing axes: batch axes must be the leading
-  // ones (the reference hands any other layout to the core's CPU function,
-  // layer_normalization.cu:43-51; this backend has no CPU path and refuses).
-  const auto &ba = this->batch_axis_;
-  const bool leading = *std::max_element(ba.begin(), ba.end()) < static_cast<int>(ba.size());
-  NBLA_CHECK(leading, error_code::not_implemented,
-             "LayerNormalizationHip supports batch_axis = [0, ..., k-1] only.");
+  // The kernels reduce over trailing axes.  Batch axes that are not the
+  // leading ones are brought to the front by a device permutation, and y / dx
+  // are permuted back (the reference hands such layouts to the core's
+  // function instead, layer_normalization.cu:43-51).  The non-batch axes keep
+  // their order, so beta and gamma are read as they are, and the statistics
+  // come out in batch-axis order, as the caller lays them out.
+  vector<int> ba(this->batch_axis_);
+  std::sort(ba.begin(), ba.end());
+  adaptor_.setup(x_shape, ba);
   batch_size_ = 1;
   for (const auto b : ba) batch_size_ *= x_shape[b];
   reduce_size_ = inputs[0]->size() / std::max<Size_t>(batch_size_, 1);
@@ -47,8 +49,22 @@ void LayerNormalizationHip<T>::forward_impl(const Variables &inputs, const Varia
   T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
   float *mean = v_mean->cast_data_and_get_pointer<float>(this->ctx_, true);
   float *var = v_var->cast_data_and_get_pointer<float>(this->ctx_, true);
-  NBLA_HIP_CHECK(nblahip_ln_fwd(x, gamma, beta, y, mean, var, batch_size_, reduce_size_,
+  const T *xk = x;
+  T *yk = y;
+  if (adaptor_.needed()) {
+    const Size_t n = inputs[0]->size();
+    T *xs = adaptor_scratch<T>(adapt_a_, n, this->ctx_);
+    adaptor_.to_kernel(x, xs, HipDtype<T>::code);
+    xk = xs;
+    yk = adaptor_scratch<T>(adapt_b_, n, this->ctx_);
+  }
+  NBLA_HIP_CHECK(nblahip_ln_fwd(xk, gamma, beta, yk, mean, var, batch_size_, reduce_size_,
                                 this->eps_, HipDtype<T>::code, nullptr));
+  if (adaptor_.needed()) {
+    adaptor_.to_caller(yk, y, false, HipDtype<T>::code);
+    adaptor_release(adapt_a_);
+    adaptor_release(adapt_b_);
+  }
 }
 
 template <typename T>
@@ -86,10 +102,28 @@ void LayerNormalizationHip<T>::backward_impl(const Variables &inputs, const Vari
                             : inputs[gamma_idx]->template cast_grad_and_get_pointer<float>(
                                   this->ctx_, !accum[gamma_idx]);
   float *ws = workspace_.cast_data_and_get_pointer<float>(this->ctx_, true);
-  NBLA_HIP_CHECK(nblahip_ln_bwd(x, dy, gamma, mean, var, dmean, dvar, dx, dgamma, dbeta,
-                                pd_x && accum[0], pd_gamma && accum[gamma_idx],
+  const bool adapt = adaptor_.needed();
+  T *dxk = dx;
+  if (adapt) {
+    const Size_t n = inputs[0]->size();
+    T *xs = adaptor_scratch<T>(adapt_a_, n, this->ctx_);
+    T *dys = adaptor_scratch<T>(adapt_b_, n, this->ctx_);
+    adaptor_.to_kernel(x, xs, HipDtype<T>::code);
+    adaptor_.to_kernel(dy, dys, HipDtype<T>::code);
+    x = xs;
+    dy = dys;
+    if (pd_x) dxk = adaptor_scratch<T>(adapt_c_, n, this->ctx_);
+  }
+  NBLA_HIP_CHECK(nblahip_ln_bwd(x, dy, gamma, mean, var, dmean, dvar, dxk, dgamma, dbeta,
+                                !adapt && pd_x && accum[0], pd_gamma && accum[gamma_idx],
                                 pd_beta && accum[beta_idx], batch_size_, reduce_size_, this->eps_,
                                 HipDtype<T>::code, ws, workspace_bytes_, nullptr));
+  if (adapt) {
+    if (pd_x) adaptor_.to_caller(dxk, dx, accum[0], HipDtype<T>::code);
+    adaptor_release(adapt_a_);
+    adaptor_release(adapt_b_);
+    adaptor_release(adapt_c_);
+  }
   // Scratch is only needed inside the call (the reference clears its buffers
   // the same way, layer_normalization.cu:202-203,236-237).
   workspace_.data()->array()->clear();

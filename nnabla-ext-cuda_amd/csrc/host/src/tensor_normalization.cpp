@@ -3,7 +3,8 @@
 // (src/nbla/cuda/function/generic/tensor_normalization.cu:22-46,
 // weight_standardization.cu:22-46) set the device and call the core's
 // composites; here both run on the batch-statistics BatchNormalization entry
-// points of nblahip (no running statistics, no transposes).
+// points of nblahip (no running statistics; no transposes when the kept axes
+// are adjacent).
 #include <nbla/hip/function/tensor_normalization.hpp>
 #include <nbla/hip/function/weight_standardization.hpp>
 #include <nbla/variable.hpp>
@@ -12,14 +13,17 @@ namespace nbla {
 
 namespace {
 
-// Shared forward: x viewed as [size0, size1, size2], statistics per index of size1.
+// Shared forward: x viewed as [size0, size1, size2], statistics per index of
+// size1; through `adaptor` (when needed) for kept axes that are not adjacent.
 template <typename T> struct NormView {
   Size_t size0, size1, size2;
   float eps;
   size_t ws_bytes;
 
   void forward(const Context &ctx, Variable *x_v, Variable *beta_v, Variable *gamma_v,
-               Variable *y_v, Variable *mean_v, Variable *var_v, Variable &ws_v) const {
+               Variable *y_v, Variable *mean_v, Variable *var_v, Variable &ws_v,
+               const AxisAdaptor *adaptor = nullptr, Variable *buf_a = nullptr,
+               Variable *buf_b = nullptr) const {
     const T *x = x_v->get_data_pointer<T>(ctx);
     const float *beta = beta_v ? beta_v->get_data_pointer<float>(ctx) : nullptr;
     const float *gamma = gamma_v ? gamma_v->get_data_pointer<float>(ctx) : nullptr;
@@ -27,25 +31,51 @@ template <typename T> struct NormView {
     float *m = mean_v->cast_data_and_get_pointer<float>(ctx, true);
     float *v = var_v->cast_data_and_get_pointer<float>(ctx, true);
     float *ws = ws_v.cast_data_and_get_pointer<float>(ctx, true);
-    NBLA_HIP_CHECK(nblahip_bn_fwd_train(x, gamma, beta, y, m, v, nullptr, nullptr, size0, size1,
+    const bool adapt = adaptor && adaptor->needed();
+    T *yk = y;
+    if (adapt) {
+      T *xs = adaptor_scratch<T>(*buf_a, x_v->size(), ctx);
+      adaptor->to_kernel(x, xs, HipDtype<T>::code);
+      x = xs;
+      yk = adaptor_scratch<T>(*buf_b, x_v->size(), ctx);
+    }
+    NBLA_HIP_CHECK(nblahip_bn_fwd_train(x, gamma, beta, yk, m, v, nullptr, nullptr, size0, size1,
                                         size2, 0.f, eps, HipDtype<T>::code, ws, ws_bytes, nullptr));
+    if (adapt) {
+      adaptor->to_caller(yk, y, false, HipDtype<T>::code);
+      adaptor_release(*buf_a);
+      adaptor_release(*buf_b);
+    }
     ws_v.data()->array()->clear();
   }
 };
 
 } // namespace
 
-// The kept axes must be adjacent: they become the "channel" extent of the
-// [size0, C, size2] view.  (The core's composite handles any set of axes by
-// transposing; that is not part of this backend.)
+// Adjacent kept axes are the "channel" extent of the [size0, C, size2] view of
+// the tensor as it lies in memory.  Any other set is gathered behind the
+// remaining axes by a device permutation ([others..., kept...], i.e. the
+// channel-last view [size0, C, 1]) and y / dx are permuted back; the core's
+// composite the reference calls transposes for such sets as well
+// (tensor_normalization.cu:22-46).  The kept axes keep their order, so beta,
+// gamma and the statistics are read and written as the caller lays them out.
 static void view_of_axes(const Shape_t &shape, const vector<int> &sorted_axes, Size_t &s0,
-                         Size_t &s1, Size_t &s2) {
-  for (size_t i = 1; i < sorted_axes.size(); ++i) {
-    NBLA_CHECK(sorted_axes[i] == sorted_axes[i - 1] + 1, error_code::not_implemented,
-               "TensorNormalizationHip supports adjacent axes only (no transposes).");
-  }
-  const int first = sorted_axes.front(), last = sorted_axes.back();
+                         Size_t &s1, Size_t &s2, AxisAdaptor *adaptor = nullptr) {
+  bool adjacent = true;
+  for (size_t i = 1; i < sorted_axes.size(); ++i)
+    adjacent = adjacent && sorted_axes[i] == sorted_axes[i - 1] + 1;
   s0 = s1 = s2 = 1;
+  if (!adjacent) {
+    NBLA_CHECK(adaptor != nullptr, error_code::value, "axes must be adjacent.");
+    adaptor->setup(shape, sorted_axes, true);
+    for (int i = 0; i < static_cast<int>(shape.size()); ++i) {
+      const bool kept = std::find(sorted_axes.begin(), sorted_axes.end(), i) != sorted_axes.end();
+      (kept ? s1 : s0) *= shape[i];
+    }
+    return;
+  }
+  if (adaptor) adaptor->setup(Shape_t{1}, vector<int>{0}); // not needed
+  const int first = sorted_axes.front(), last = sorted_axes.back();
   for (int i = 0; i < static_cast<int>(shape.size()); ++i) {
     if (i < first) s0 *= shape[i];
     else if (i <= last) s1 *= shape[i];
@@ -56,7 +86,7 @@ static void view_of_axes(const Shape_t &shape, const vector<int> &sorted_axes, S
 template <typename T>
 void TensorNormalizationHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
   TensorNormalization<T>::setup_shapes(inputs, outputs);
-  view_of_axes(inputs[0]->shape(), this->axes_, size0_, size1_, size2_);
+  view_of_axes(inputs[0]->shape(), this->axes_, size0_, size1_, size2_, &adaptor_);
   NBLA_CHECK(inputs[0]->size() < (Size_t(1) << 31), error_code::value,
              "TensorNormalizationHip indexes with 32 bits: fewer than 2^31 elements required.");
   mean_.reshape(Shape_t{size1_}, true);
@@ -73,7 +103,8 @@ void TensorNormalizationHip<T>::forward_impl(const Variables &inputs, const Vari
   const NormView<T> view{size0_, size1_, size2_, this->eps_, workspace_bytes_};
   view.forward(this->ctx_, inputs[0], this->no_bias_ ? nullptr : inputs[this->beta_idx_],
                this->no_scale_ ? nullptr : inputs[this->gamma_idx_], outputs[0],
-               three ? outputs[1] : &mean_, three ? outputs[2] : &var_, workspace_);
+               three ? outputs[1] : &mean_, three ? outputs[2] : &var_, workspace_, &adaptor_,
+               &adapt_a_, &adapt_b_);
 }
 
 template <typename T>
@@ -104,10 +135,28 @@ void TensorNormalizationHip<T>::backward_impl(const Variables &inputs, const Var
                             : inputs[this->gamma_idx_]->template cast_grad_and_get_pointer<float>(
                                   this->ctx_, !accum[this->gamma_idx_]);
   float *ws = workspace_.cast_data_and_get_pointer<float>(this->ctx_, true);
-  NBLA_HIP_CHECK(nblahip_bn_bwd(x, dy, gamma, mean, var, dmean, dvar, dx, dgamma, dbeta,
-                                pd_x && accum[0], pd_gamma && accum[this->gamma_idx_],
+  const bool adapt = adaptor_.needed();
+  T *dxk = dx;
+  if (adapt) {
+    const Size_t n = inputs[0]->size();
+    T *xs = adaptor_scratch<T>(adapt_a_, n, this->ctx_);
+    T *dys = adaptor_scratch<T>(adapt_b_, n, this->ctx_);
+    adaptor_.to_kernel(x, xs, HipDtype<T>::code);
+    adaptor_.to_kernel(dy, dys, HipDtype<T>::code);
+    x = xs;
+    dy = dys;
+    if (pd_x) dxk = adaptor_scratch<T>(adapt_c_, n, this->ctx_);
+  }
+  NBLA_HIP_CHECK(nblahip_bn_bwd(x, dy, gamma, mean, var, dmean, dvar, dxk, dgamma, dbeta,
+                                !adapt && pd_x && accum[0], pd_gamma && accum[this->gamma_idx_],
                                 pd_beta && accum[this->beta_idx_], size0_, size1_, size2_,
                                 this->eps_, 1, HipDtype<T>::code, ws, workspace_bytes_, nullptr));
+  if (adapt) {
+    if (pd_x) adaptor_.to_caller(dxk, dx, accum[0], HipDtype<T>::code);
+    adaptor_release(adapt_a_);
+    adaptor_release(adapt_b_);
+    adaptor_release(adapt_c_);
+  }
   workspace_.data()->array()->clear();
 }
 

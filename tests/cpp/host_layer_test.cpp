@@ -156,14 +156,14 @@ static void test_setup_errors() {
     EXPECT_THROW(g->setup({&x, &p6, &p6, &m6, &v6, &z}, {&y}), "shape of x");
   }
   {
-    auto f = create_LayerNormalization(ctx, vector<int>{1}, 1e-5f, true, true);
-    EXPECT_THROW(f->setup({&x}, {&y}), "batch_axis");
+    auto f = create_LayerNormalization(ctx, vector<int>{9}, 1e-5f, true, true);
+    EXPECT_THROW(f->setup({&x}, {&y}), "batch_axis out of range");
   }
   {
     auto f = create_GroupNormalization(ctx, 4, 1, vector<int>{0}, 1e-5f, true, true);
     EXPECT_THROW(f->setup({&x}, {&y}), "divisible");
-    auto g = create_GroupNormalization(ctx, 1, 2, vector<int>{0}, 1e-5f, true, true);
-    EXPECT_THROW(g->setup({&x}, {&y}), "channel-first");   // channel axis in the middle
+    auto g = create_GroupNormalization(ctx, 1, 2, vector<int>{2}, 1e-5f, true, true);
+    EXPECT_THROW(g->setup({&x}, {&y}), "batch_axis");   // batch axis equal to the channel axis
   }
   {
     auto f = create_InstanceNormalization(ctx, 1, vector<int>{0}, 1e-5f, false, false);
