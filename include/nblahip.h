@@ -421,6 +421,25 @@ NBLAHIP_EXPORT int nblahip_memcpy_d2h(void *dst, const void *src, size_t bytes,
                                       void *stream);
 NBLAHIP_EXPORT int nblahip_memcpy_d2d(void *dst, const void *src, size_t bytes,
                                       void *stream);
+/* Asynchronous transfers (src/nbla/cuda/array/cuda_array.cpp:83-158: the
+ * AsyncFlag::ASYNC synchronizers issue cudaMemcpyAsync on the backend's
+ * stream_HtoD / stream_DtoH and order it against the null stream with events).
+ * The *_async copies return without waiting and are meant for page-locked host
+ * memory (nblahip_host_malloc); streams are created non-blocking with the
+ * default priority, events without timing.  nblahip_event_query: *done = 1
+ * when everything recorded before the event has finished. */
+NBLAHIP_EXPORT int nblahip_memcpy_h2d_async(void *dst, const void *src,
+                                            size_t bytes, void *stream);
+NBLAHIP_EXPORT int nblahip_memcpy_d2h_async(void *dst, const void *src,
+                                            size_t bytes, void *stream);
+NBLAHIP_EXPORT int nblahip_stream_create(void **stream);
+NBLAHIP_EXPORT int nblahip_stream_destroy(void *stream);
+NBLAHIP_EXPORT int nblahip_event_create(void **event);
+NBLAHIP_EXPORT int nblahip_event_destroy(void *event);
+NBLAHIP_EXPORT int nblahip_event_record(void *event, void *stream);
+NBLAHIP_EXPORT int nblahip_stream_wait_event(void *stream, void *event);
+NBLAHIP_EXPORT int nblahip_event_synchronize(void *event);
+NBLAHIP_EXPORT int nblahip_event_query(void *event, int *done);
 NBLAHIP_EXPORT int nblahip_memset(void *dst, int byte, size_t bytes,
                                   void *stream);
 /* dst[i] = (dst_dtype) src[i] for n elements (float32 <-> float16). */

@@ -48,6 +48,18 @@ NNABLA_HIP_EXPORT int nnabla_hip_variable_set(nnabla_hip_variable *v, int which,
                                               int64_t n, int dtype);
 NNABLA_HIP_EXPORT int nnabla_hip_variable_get(nnabla_hip_variable *v, int which, float *host,
                                               int64_t n);
+/* NdArray::cast(dtype, Context({}, array_class, device_id), write_only,
+ * async_flags): moves the variable's content into an array of that class.
+ * async_flags as the core's AsyncFlag (1 = ASYNC, 2 = UNSAFE): with ASYNC and a
+ * page-locked host array on the other side the transfer is enqueued on the
+ * backend's transfer stream and the call returns at once
+ * (src/nbla/cuda/array/cuda_array.cpp:83-158); the next use of the array waits
+ * for it.  nnabla_hip_pending_transfers: host-to-device transfers whose source
+ * array the backend still keeps alive. */
+NNABLA_HIP_EXPORT int nnabla_hip_variable_cast(nnabla_hip_variable *v, int which,
+                                               const char *array_class, const char *device_id,
+                                               int dtype, int write_only, int async_flags);
+NNABLA_HIP_EXPORT int nnabla_hip_pending_transfers(uint64_t *count);
 NNABLA_HIP_EXPORT int nnabla_hip_variable_zero(nnabla_hip_variable *v, int which);
 NNABLA_HIP_EXPORT int nnabla_hip_variable_fill(nnabla_hip_variable *v, int which, float value);
 

@@ -83,6 +83,16 @@ SIGNATURES = {
     "nblahip_memcpy_h2d": (_int, [_c_void_p, _c_void_p, _sz, _c_void_p]),
     "nblahip_memcpy_d2h": (_int, [_c_void_p, _c_void_p, _sz, _c_void_p]),
     "nblahip_memcpy_d2d": (_int, [_c_void_p, _c_void_p, _sz, _c_void_p]),
+    "nblahip_memcpy_h2d_async": (_int, [_c_void_p, _c_void_p, _sz, _c_void_p]),
+    "nblahip_memcpy_d2h_async": (_int, [_c_void_p, _c_void_p, _sz, _c_void_p]),
+    "nblahip_stream_create": (_int, [ctypes.POINTER(_c_void_p)]),
+    "nblahip_stream_destroy": (_int, [_c_void_p]),
+    "nblahip_event_create": (_int, [ctypes.POINTER(_c_void_p)]),
+    "nblahip_event_destroy": (_int, [_c_void_p]),
+    "nblahip_event_record": (_int, [_c_void_p, _c_void_p]),
+    "nblahip_stream_wait_event": (_int, [_c_void_p, _c_void_p]),
+    "nblahip_event_synchronize": (_int, [_c_void_p]),
+    "nblahip_event_query": (_int, [_c_void_p, ctypes.POINTER(_int)]),
     "nblahip_memset": (_int, [_c_void_p, _int, _sz, _c_void_p]),
     "nblahip_convert": (_int, [_c_void_p, _int, _c_void_p, _int, _i64, _c_void_p]),
     "nblahip_fill": (_int, [_c_void_p, _int, _f, _i64, _c_void_p]),

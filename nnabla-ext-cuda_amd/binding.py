@@ -35,6 +35,8 @@ SIGNATURES = {
     "nnabla_hip_variable_shape": (_I, [_P, ctypes.POINTER(_I64)]),
     "nnabla_hip_variable_set": (_I, [_P, _I, _FP, _I64, _I]),
     "nnabla_hip_variable_get": (_I, [_P, _I, _FP, _I64]),
+    "nnabla_hip_variable_cast": (_I, [_P, _I, _S, _S, _I, _I, _I]),
+    "nnabla_hip_pending_transfers": (_I, [ctypes.POINTER(ctypes.c_uint64)]),
     "nnabla_hip_variable_zero": (_I, [_P, _I]),
     "nnabla_hip_variable_fill": (_I, [_P, _I, _F]),
     "nnabla_hip_create_batch_normalization": (_P, [_S, _S, _S, _IP, _I, _F, _F, _I, _I, _I]),
@@ -111,6 +113,16 @@ def context(device_id=0, type_config="float", **kw):
         raise ValueError("Unknown data type config is given %s" % type_config)
     return {"backends": ",".join(backends), "array_class": kw.get("array_class", "HipCachedArray"),
             "device_id": str(device_id)}
+
+
+ASYNC, UNSAFE = 1, 2
+
+
+def pending_transfers():
+    """Host-to-device transfers whose source array the backend still holds."""
+    n = ctypes.c_uint64(0)
+    _check(lib().nnabla_hip_pending_transfers(ctypes.byref(n)))
+    return n.value
 
 
 def device_synchronize(device="0"):
@@ -194,6 +206,13 @@ class Variable:
     @property
     def g(self):
         return self._get(1)
+
+    def cast(self, array_class, device_id="0", which=0, half=False, write_only=False,
+             async_flags=0):
+        """NdArray.cast to an array class; async_flags: ASYNC = 1, UNSAFE = 2."""
+        _check(lib().nnabla_hip_variable_cast(self._h, which, array_class.encode(),
+                                              str(device_id).encode(), 1 if half else 0,
+                                              1 if write_only else 0, int(async_flags)))
 
     def zero_grad(self):
         _check(lib().nnabla_hip_variable_zero(self._h, 1))

@@ -219,17 +219,53 @@ public:
 };
 
 // ---------------------------------------------------------------- arrays
+// Flags of a cast / get / synchronizer call (used as AsyncFlag::ASYNC etc. at
+// src/nbla/cuda/array/cuda_array.cpp:130,149,191,199): ASYNC asks for a
+// non-blocking transfer, UNSAFE waives keeping the source alive until the
+// transfer has run, OFFREC belongs to the core's array-use recorder.
+namespace AsyncFlag {
+enum Flags { NONE = 0, ASYNC = 1, UNSAFE = 2, OFFREC = 4 };
+}
+
+inline bool is_cpu_context(const Context &ctx) {
+  return ctx.array_class.find("Cpu") == 0 || ctx.array_class.find("HostArray") != string::npos;
+}
+
+// An asynchronous transfer still on its way into an array
+// (include/nbla/cuda/event.hpp: CudaEvent derives from this).
+class NBLA_API Event {
+public:
+  virtual ~Event() {}
+  // Makes the consumer (the function stream, and the host for a host
+  // consumer without ASYNC / UNSAFE) wait for the transfer.
+  virtual void wait_event(const Context ctx, const int async_flags = AsyncFlag::NONE) = 0;
+};
+typedef shared_ptr<Event> EventPtr;
+
 // (Array interface as subclassed at include/nbla/cuda/array/cuda_array.hpp:36-49.)
-class NBLA_API Array {
+class NBLA_API Array : public std::enable_shared_from_this<Array> {
 protected:
   Size_t size_;
   dtypes dtype_;
   Context ctx_;
   void *ptr_ = nullptr;
+  EventPtr event_;
 
 public:
   Array(Size_t size, dtypes dtype, const Context &ctx) : size_(size), dtype_(dtype), ctx_(ctx) {}
   virtual ~Array() {}
+  shared_ptr<Array> getptr() { return shared_from_this(); }
+  // The transfer that fills this array, if one is still outstanding
+  // (cuda_array.cpp:87-91,113-114: set by the asynchronous synchronizers,
+  // consumed by wait_event).
+  void set_event(EventPtr e) { event_ = e; }
+  bool have_event() const { return static_cast<bool>(event_); }
+  void wait_event(const Context ctx, const int async_flags = AsyncFlag::NONE) {
+    if (event_) {
+      event_->wait_event(ctx, async_flags);
+      event_.reset();
+    }
+  }
   template <typename T = void> T *pointer() { return reinterpret_cast<T *>(ptr_); }
   template <typename T = void> const T *const_pointer() const {
     return reinterpret_cast<const T *>(ptr_);
@@ -264,7 +300,7 @@ public:
 
 class NBLA_API ArraySynchronizer {
 public:
-  typedef std::function<void(Array *, Array *)> Synchronizer; // (src, dst)
+  typedef std::function<void(Array *, Array *, const int)> Synchronizer; // (src, dst, async_flags)
   static std::map<std::pair<string, string>, Synchronizer> &registry() {
     static std::map<std::pair<string, string>, Synchronizer> r;
     return r;
@@ -272,11 +308,12 @@ public:
   static void add_synchronizer(const string &src, const string &dst, Synchronizer s) {
     registry()[std::make_pair(src, dst)] = s;
   }
-  static void synchronize(const string &src_class, Array *src, const string &dst_class, Array *dst) {
+  static void synchronize(const string &src_class, Array *src, const string &dst_class, Array *dst,
+                          const int async_flags = AsyncFlag::NONE) {
     auto it = registry().find(std::make_pair(src_class, dst_class));
     NBLA_CHECK(it != registry().end(), error_code::unclassified,
                "No synchronizer registered from %s to %s.", src_class.c_str(), dst_class.c_str());
-    it->second(src, dst);
+    it->second(src, dst, async_flags);
   }
 };
 
@@ -353,9 +390,13 @@ class NBLA_API SyncedArray {
     return a;
   }
 
-  ArrayPtr sync(dtypes dtype, const Context &ctx, bool write_only) {
+  ArrayPtr sync(dtypes dtype, const Context &ctx, bool write_only, const int async_flags) {
     const Key key(ctx.array_class, static_cast<int>(dtype));
     ArrayPtr dst = materialize(key, ctx);
+    // A transfer into this materialisation that is still outstanding: its
+    // consumer waits here (the function stream; the host too for a host
+    // context without ASYNC / UNSAFE).
+    dst->wait_event(ctx, async_flags);
     if (write_only) return dst;
     if (!has_head_) {
       // Never written: defined content is zero (or the pending fill value).
@@ -369,6 +410,7 @@ class NBLA_API SyncedArray {
     if (key == head_ || current_.count(key)) return dst; // a reader's copy stays good until the next write
     ArrayPtr src = arrays_.at(head_);
     if (head_.first == key.first) {
+      src->wait_event(ctx, async_flags);
       dst->copy_from(src.get()); // same class: dtype conversion on its device
     } else {
       // Cross-class: convert on the source side when dtypes differ, then move.
@@ -376,10 +418,13 @@ class NBLA_API SyncedArray {
       if (head_.second != key.second) {
         const Key skey(head_.first, key.second);
         staged = materialize(skey, src->context());
-        if (!current_.count(skey)) staged->copy_from(src.get());
+        if (!current_.count(skey)) {
+          src->wait_event(src->context(), async_flags);
+          staged->copy_from(src.get());
+        }
         current_.insert(skey);
       }
-      ArraySynchronizer::synchronize(head_.first, staged.get(), key.first, dst.get());
+      ArraySynchronizer::synchronize(head_.first, staged.get(), key.first, dst.get(), async_flags);
     }
     current_.insert(key);
     return dst;
@@ -388,8 +433,9 @@ class NBLA_API SyncedArray {
 public:
   explicit SyncedArray(Size_t size) : size_(size) {}
   Size_t size() const { return size_; }
-  ArrayPtr cast_sp(dtypes dtype, const Context &ctx, bool write_only = false) {
-    ArrayPtr a = sync(dtype, ctx, write_only);
+  ArrayPtr cast_sp(dtypes dtype, const Context &ctx, bool write_only = false,
+                   const int async_flags = AsyncFlag::NONE) {
+    ArrayPtr a = sync(dtype, ctx, write_only, async_flags);
     head_ = Key(ctx.array_class, static_cast<int>(dtype));
     has_head_ = true;
     zeroing_ = filling_ = false;
@@ -399,11 +445,12 @@ public:
     current_.clear();
     return a;
   }
-  Array *cast(dtypes dtype, const Context &ctx, bool write_only = false) {
-    return cast_sp(dtype, ctx, write_only).get();
+  Array *cast(dtypes dtype, const Context &ctx, bool write_only = false,
+              const int async_flags = AsyncFlag::NONE) {
+    return cast_sp(dtype, ctx, write_only, async_flags).get();
   }
-  const Array *get(dtypes dtype, const Context &ctx) {
-    ArrayPtr a = sync(dtype, ctx, false);
+  const Array *get(dtypes dtype, const Context &ctx, const int async_flags = AsyncFlag::NONE) {
+    ArrayPtr a = sync(dtype, ctx, false, async_flags);
     if (!has_head_ || zeroing_ || filling_) {
       head_ = Key(ctx.array_class, static_cast<int>(dtype));
       has_head_ = true;
@@ -461,10 +508,13 @@ public:
   SyncedArrayPtr array() { return array_; }
   void zero() { array_->zero(); }
   void fill(float v) { array_->fill(v); }
-  Array *cast(dtypes dtype, const Context &ctx, bool write_only = false) {
-    return array_->cast(dtype, ctx, write_only);
+  Array *cast(dtypes dtype, const Context &ctx, bool write_only = false,
+              const int async_flags = AsyncFlag::NONE) {
+    return array_->cast(dtype, ctx, write_only, async_flags);
   }
-  const Array *get(dtypes dtype, const Context &ctx) { return array_->get(dtype, ctx); }
+  const Array *get(dtypes dtype, const Context &ctx, const int async_flags = AsyncFlag::NONE) {
+    return array_->get(dtype, ctx, async_flags);
+  }
 };
 typedef shared_ptr<NdArray> NdArrayPtr;
 
@@ -668,7 +718,7 @@ inline void init_cpu() {
     ArrayCreator::add_creator("CpuArray", [](Size_t s, dtypes d, const Context &c) -> Array * {
       return new CpuArray(s, d, c);
     });
-    ArraySynchronizer::add_synchronizer("CpuArray", "CpuArray", [](Array *src, Array *dst) {
+    ArraySynchronizer::add_synchronizer("CpuArray", "CpuArray", [](Array *src, Array *dst, const int) {
       dst->copy_from(src);
     });
   });

@@ -41,8 +41,34 @@ public:
   }
 };
 
-// Blocking copies between a host array and a device array of the same dtype.
-NBLA_HIP_API void synchronizer_hip_array_cpu_array(Array *src, Array *dst);
-NBLA_HIP_API void synchronizer_cpu_array_hip_array(Array *src, Array *dst);
+// Copies between a host array and a device array of the same dtype
+// (src/nbla/cuda/array/cuda_array.cpp:83-235).  Blocking by default.  With
+// AsyncFlag::ASYNC and a page-locked host array (HipCachedHostArray) the copy is
+// enqueued on the backend's transfer stream of its direction, after whatever
+// the function stream (the null stream) holds at that moment, and recorded as
+// an event in the destination array: the next cast / get of that array makes
+// the function stream wait for it (and the host too, when the consumer is a
+// host context and passes neither ASYNC nor UNSAFE).  A host-to-device copy
+// keeps its source array alive until it has run unless AsyncFlag::UNSAFE is
+// given.  Pageable host memory (CpuArray) is always copied with blocking
+// semantics, whatever the flags say.
+NBLA_HIP_API void synchronizer_hip_array_cpu_array(Array *src, Array *dst, const int async_flags);
+NBLA_HIP_API void synchronizer_cpu_array_hip_array(Array *src, Array *dst, const int async_flags);
+
+// A transfer enqueued on one of the backend's transfer streams (counterpart of
+// CudaEvent, src/nbla/cuda/event.cpp:20-60).  Holds the source array so that it
+// outlives the transfer for as long as the destination remembers the event.
+class NBLA_HIP_API HipEvent : public Event {
+  void *raw_event_;
+  ArrayPtr src_;
+  int device_;
+
+public:
+  HipEvent(void *raw_event, ArrayPtr src, int device)
+      : raw_event_(raw_event), src_(src), device_(device) {}
+  ~HipEvent() override;
+  void *raw_event() { return raw_event_; }
+  void wait_event(const Context ctx, const int async_flags = AsyncFlag::NONE) override;
+};
 
 } // namespace nbla

@@ -6,6 +6,7 @@
 #pragma once
 
 #include <map>
+#include <memory>
 #include <mutex>
 #include <nbla/backend_registry.hpp>
 #include <nbla/hip/common.hpp>
@@ -31,7 +32,20 @@ public:
   size_t cached_bytes() const;
   size_t live_bytes() const;
 
+  // Transfer streams of a device, one per direction (the reference's
+  // stream_HtoD / stream_DtoH, include/nbla/cuda/cuda.hpp:118-119): created on
+  // first use, non-blocking, default priority.
+  void *transfer_stream(int device, bool to_device);
+  // Keeps `event` (and with it the source array of its transfer) alive until
+  // the transfer has finished; finished ones are dropped on later calls and by
+  // device_synchronize.
+  void keep_until_done(std::shared_ptr<class HipEvent> event);
+  size_t pending_transfers();
+
 private:
+  void reap_locked();
+  std::map<std::pair<int, bool>, void *> streams_;
+  vector<std::shared_ptr<class HipEvent>> pending_;
   mutable std::mutex mu_;
   std::map<std::pair<int, size_t>, vector<void *>> cache_;
   size_t cached_bytes_ = 0, live_bytes_ = 0;

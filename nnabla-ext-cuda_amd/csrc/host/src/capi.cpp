@@ -194,6 +194,25 @@ int nnabla_hip_variable_get(nnabla_hip_variable *v, int which, float *host, int6
   });
 }
 
+int nnabla_hip_variable_cast(nnabla_hip_variable *v, int which, const char *array_class,
+                             const char *device_id, int dtype, int write_only, int async_flags) {
+  return guarded([&] {
+    NdArrayPtr a = pick(v, which);
+    NBLA_CHECK(dtype == 0 || dtype == 1, error_code::value, "dtype must be 0 (float) or 1 (half)");
+    NBLA_CHECK(array_class != nullptr, error_code::value, "array_class must be given");
+    init_hip();
+    const Context ctx({}, array_class, device_id ? device_id : "0");
+    a->cast(dtype == 0 ? dtypes::FLOAT : dtypes::HALF, ctx, write_only != 0, async_flags);
+  });
+}
+
+int nnabla_hip_pending_transfers(uint64_t *count) {
+  return guarded([&] {
+    NBLA_CHECK(count != nullptr, error_code::value, "count must not be null");
+    *count = SingletonManager::get<Hip>()->pending_transfers();
+  });
+}
+
 int nnabla_hip_variable_zero(nnabla_hip_variable *v, int which) {
   return guarded([&] { pick(v, which)->zero(); });
 }

@@ -1,4 +1,5 @@
 // Hip backend singleton and device helpers.
+#include <nbla/hip/array/hip_array.hpp>
 #include <nbla/hip/hip.hpp>
 
 namespace nbla {
@@ -14,6 +15,8 @@ int hip_get_device() {
 Hip::Hip() {}
 
 Hip::~Hip() {
+  pending_.clear();
+  for (auto &kv : streams_) NBLA_HIP_FORCE_ASSERT(nblahip_stream_destroy(kv.second));
   for (auto &kv : cache_)
     for (void *p : kv.second) NBLA_HIP_FORCE_ASSERT(nblahip_free(p));
 }
@@ -23,6 +26,41 @@ vector<string> Hip::array_classes() const { return {"HipCachedArray", "HipArray"
 void Hip::device_synchronize(const string &device) {
   hip_set_device(std::stoi(device));
   NBLA_HIP_CHECK(nblahip_device_synchronize());
+  std::lock_guard<std::mutex> lock(mu_);
+  reap_locked();
+}
+
+void *Hip::transfer_stream(int device, bool to_device) {
+  std::lock_guard<std::mutex> lock(mu_);
+  auto it = streams_.find(std::make_pair(device, to_device));
+  if (it != streams_.end()) return it->second;
+  hip_set_device(device);
+  void *st = nullptr;
+  NBLA_HIP_CHECK(nblahip_stream_create(&st));
+  streams_[std::make_pair(device, to_device)] = st;
+  return st;
+}
+
+void Hip::reap_locked() {
+  size_t kept = 0;
+  for (auto &e : pending_) {
+    int done = 0;
+    if (nblahip_event_query(e->raw_event(), &done) == 0 && done) continue;
+    pending_[kept++] = e;
+  }
+  pending_.resize(kept);
+}
+
+void Hip::keep_until_done(std::shared_ptr<HipEvent> event) {
+  std::lock_guard<std::mutex> lock(mu_);
+  reap_locked();
+  pending_.push_back(event);
+}
+
+size_t Hip::pending_transfers() {
+  std::lock_guard<std::mutex> lock(mu_);
+  reap_locked();
+  return pending_.size();
 }
 
 void Hip::default_stream_synchronize(const string &device) {

@@ -53,11 +53,11 @@ void init_hip() {
   });
   // The pinned host array is a host array: plain copies to and from CpuArray.
   ArraySynchronizer::add_synchronizer("HipCachedHostArray", "CpuArray",
-                                      [](Array *src, Array *dst) { dst->copy_from(src); });
+                                      [](Array *src, Array *dst, const int) { dst->copy_from(src); });
   ArraySynchronizer::add_synchronizer("CpuArray", "HipCachedHostArray",
-                                      [](Array *src, Array *dst) { dst->copy_from(src); });
+                                      [](Array *src, Array *dst, const int) { dst->copy_from(src); });
   ArraySynchronizer::add_synchronizer("HipCachedHostArray", "HipCachedHostArray",
-                                      [](Array *src, Array *dst) { dst->copy_from(src); });
+                                      [](Array *src, Array *dst, const int) { dst->copy_from(src); });
   const char *device_classes[] = {"HipArray", "HipCachedArray"};
   for (const char *dc : device_classes) {
     ArraySynchronizer::add_synchronizer(dc, "CpuArray", synchronizer_hip_array_cpu_array);
@@ -65,7 +65,7 @@ void init_hip() {
     ArraySynchronizer::add_synchronizer(dc, "HipCachedHostArray", synchronizer_hip_array_cpu_array);
     ArraySynchronizer::add_synchronizer("HipCachedHostArray", dc, synchronizer_cpu_array_hip_array);
     for (const char *dc2 : device_classes)
-      ArraySynchronizer::add_synchronizer(dc, dc2, [](Array *src, Array *dst) { dst->copy_from(src); });
+      ArraySynchronizer::add_synchronizer(dc, dc2, [](Array *src, Array *dst, const int) { dst->copy_from(src); });
   }
 
   // Functions: same names as the reference registers, new backend key.

@@ -235,6 +235,66 @@ int nblahip_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream) {
   if (int e = hip_status(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, st))) return e;
   return hip_status(hipStreamSynchronize(st));
 }
+// Non-blocking copies for page-locked host memory: enqueued on `stream`, the
+// caller orders them with events.
+int nblahip_memcpy_h2d_async(void *dst, const void *src, size_t bytes, void *stream) {
+  if (bytes == 0) return 0;
+  if (!dst || !src) return NBLAHIP_EINVAL;
+  return hip_status(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice,
+                                   static_cast<hipStream_t>(stream)));
+}
+int nblahip_memcpy_d2h_async(void *dst, const void *src, size_t bytes, void *stream) {
+  if (bytes == 0) return 0;
+  if (!dst || !src) return NBLAHIP_EINVAL;
+  return hip_status(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost,
+                                   static_cast<hipStream_t>(stream)));
+}
+
+int nblahip_stream_create(void **stream) {
+  if (!stream) return NBLAHIP_EINVAL;
+  hipStream_t st = nullptr;
+  // default priority; non-blocking: ordered against the null stream by events only
+  const int e = hip_status(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+  *stream = st;
+  return e;
+}
+int nblahip_stream_destroy(void *stream) {
+  return stream ? hip_status(hipStreamDestroy(static_cast<hipStream_t>(stream))) : 0;
+}
+int nblahip_event_create(void **event) {
+  if (!event) return NBLAHIP_EINVAL;
+  hipEvent_t ev = nullptr;
+  const int e = hip_status(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+  *event = ev;
+  return e;
+}
+int nblahip_event_destroy(void *event) {
+  return event ? hip_status(hipEventDestroy(static_cast<hipEvent_t>(event))) : 0;
+}
+int nblahip_event_record(void *event, void *stream) {
+  if (!event) return NBLAHIP_EINVAL;
+  return hip_status(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
+}
+int nblahip_stream_wait_event(void *stream, void *event) {
+  if (!event) return NBLAHIP_EINVAL;
+  return hip_status(hipStreamWaitEvent(static_cast<hipStream_t>(stream),
+                                       static_cast<hipEvent_t>(event), 0));
+}
+int nblahip_event_synchronize(void *event) {
+  if (!event) return NBLAHIP_EINVAL;
+  return hip_status(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+}
+int nblahip_event_query(void *event, int *done) {
+  if (!event || !done) return NBLAHIP_EINVAL;
+  const hipError_t e = hipEventQuery(static_cast<hipEvent_t>(event));
+  if (e == hipErrorNotReady) {
+    *done = 0;
+    return 0;
+  }
+  *done = e == hipSuccess ? 1 : 0;
+  return hip_status(e);
+}
+
 int nblahip_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream) {
   if (bytes == 0) return 0;
   if (!dst || !src) return NBLAHIP_EINVAL;

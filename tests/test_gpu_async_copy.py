@@ -1,0 +1,92 @@
+"""Asynchronous host<->device copies of the array layer (the reference's
+AsyncFlag::ASYNC / UNSAFE synchronizers, src/nbla/cuda/array/cuda_array.cpp:
+83-158): enqueued on the backend's transfer streams for page-locked host
+arrays, ordered against the function stream by events, blocking for pageable
+memory.  Every case checks the data that arrives, through a Function or a
+read-back."""
+import numpy as np
+import pytest
+
+from _util import assert_close, load_package
+from oracle import norm_ref as R
+
+load_package()
+from nnabla_ext_cuda_amd import binding as B  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _host_class():
+    B.init()
+    yield
+    B.set_host_array_class("CpuArray")
+    B.device_synchronize()
+
+
+def _ln(x_var, shape, outer):
+    f = B.LayerNormalization(B.context(), batch_axis=[0], eps=1e-5, no_scale=True, no_bias=True)
+    y = B.Variable(shape)
+    f.setup([x_var], [y])
+    f.forward([x_var], [y])
+    return y
+
+
+@pytest.mark.parametrize("host_class", ["HipCachedHostArray", "CpuArray"])
+@pytest.mark.parametrize("flags", [B.ASYNC, B.ASYNC | B.UNSAFE, 0])
+def test_async_upload_feeds_a_function_and_async_download_returns_its_output(host_class, flags):
+    B.set_host_array_class(host_class)
+    rng = np.random.default_rng(41)
+    shape = (512, 1024)
+    x = rng.standard_normal(shape).astype(np.float32) + 2
+    vx = B.Variable(shape)
+    vx.set_data(x)                                   # lives in a host array of host_class
+    vx.cast("HipCachedArray", async_flags=flags)     # upload, enqueued when pinned + ASYNC
+    vy = _ln(vx, shape, shape[0])                    # the kernel's stream waits for the upload
+    y_r, _, _ = R.ln_forward(x, None, None, shape[0], 1e-5)
+    vy.cast(host_class, device_id="", async_flags=flags)   # download, enqueued likewise
+    assert_close(vy.d, y_r, "f32", "y", "y after asynchronous transfers")  # the host waits here
+    B.device_synchronize()
+    assert B.pending_transfers() == 0
+
+
+def test_source_of_an_async_upload_outlives_its_variable_slot():
+    """The upload drops the host array from the variable at once; its memory
+    must stay valid until the copy has run even when new page-locked arrays are
+    allocated and filled right behind it."""
+    B.set_host_array_class("HipCachedHostArray")
+    n = 16 << 20
+    x = np.arange(n, dtype=np.float32)
+    vx = B.Variable((n,))
+    vx.set_data(x)
+    vx.cast("HipCachedArray", async_flags=B.ASYNC)
+    others = []
+    for k in range(3):                               # same size: likely the same pages again
+        v = B.Variable((n,))
+        v.set_data(np.full(n, -1.0 - k, np.float32))
+        others.append(v)
+    assert B.pending_transfers() <= 1
+    np.testing.assert_array_equal(vx.d, x)
+    B.device_synchronize()
+    assert B.pending_transfers() == 0
+
+
+def test_unsafe_upload_keeps_no_guard():
+    B.set_host_array_class("HipCachedHostArray")
+    x = np.linspace(-1, 1, 4096, dtype=np.float32)
+    vx = B.Variable((4096,))
+    vx.set_data(x)
+    vx.cast("HipCachedArray", async_flags=B.ASYNC | B.UNSAFE)
+    assert B.pending_transfers() == 0
+    B.device_synchronize()
+    np.testing.assert_array_equal(vx.d, x)
+
+
+def test_half_storage_goes_through_the_same_path():
+    B.set_host_array_class("HipCachedHostArray")
+    x = np.linspace(-4, 4, 8192, dtype=np.float32)
+    vx = B.Variable((8192,))
+    vx.set_data(x, half=True)
+    vx.cast("HipCachedArray", half=True, async_flags=B.ASYNC)
+    vx.cast("HipCachedArray", half=False)            # device-side conversion after the upload
+    np.testing.assert_array_equal(vx.d, x.astype(np.float16).astype(np.float32))
