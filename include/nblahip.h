@@ -481,6 +481,30 @@ NBLAHIP_EXPORT int nblahip_profile_enable(int max_records);
 NBLAHIP_EXPORT int nblahip_profile_reset(void);
 NBLAHIP_EXPORT int nblahip_profile_query(const char *kernel_name,
                                          double *total_ms, int64_t *launches);
+/* Names of the kernels recorded since the last reset, one per line, each once,
+ * in order of first launch.  Writes at most `capacity` bytes (terminated);
+ * *needed = bytes for the whole list. */
+NBLAHIP_EXPORT int nblahip_profile_kernels(char *names, size_t capacity,
+                                           size_t *needed);
+
+/* ------------------------------------------------------------------------
+ * Plan knobs.  Which kernel family serves a shape is decided per call from a
+ * few integers (block counts per CU, size limits of the on-chip paths, on/off
+ * switches of each specialised plan).  Every one has a default; the environment
+ * variable NBLAHIP_<NAME> (read once, at the knob's first use) overrides the
+ * default and nblahip_tune_set overrides both, from the next call on.  Results
+ * never depend on a knob beyond the summation order of partial sums.  No
+ * counterpart in the reference, whose launch shapes are compile-time macros
+ * (include/nbla/cuda/common.hpp:337-343: NBLA_CUDA_NUM_THREADS,
+ * NBLA_CUDA_GET_BLOCKS).
+ *   set(name, value >= 0): override; set(name, -1): back to environment/default.
+ *   get(name, fallback)  : the value a launch would use now.
+ *   reset()              : drop every override made through set.
+ * `name` is the knob without the NBLAHIP_ prefix, e.g. "BN_ONCHIP".
+ * ---------------------------------------------------------------------- */
+NBLAHIP_EXPORT int nblahip_tune_set(const char *name, int value);
+NBLAHIP_EXPORT int nblahip_tune_get(const char *name, int fallback);
+NBLAHIP_EXPORT int nblahip_tune_reset(void);
 
 #ifdef __cplusplus
 }

@@ -102,6 +102,10 @@ SIGNATURES = {
     "nblahip_profile_reset": (_int, []),
     "nblahip_profile_query": (_int, [ctypes.c_char_p, ctypes.POINTER(ctypes.c_double),
                                      ctypes.POINTER(_i64)]),
+    "nblahip_profile_kernels": (_int, [ctypes.c_char_p, _sz, ctypes.POINTER(_sz)]),
+    "nblahip_tune_set": (_int, [ctypes.c_char_p, _int]),
+    "nblahip_tune_get": (_int, [ctypes.c_char_p, _int]),
+    "nblahip_tune_reset": (_int, []),
 }
 
 _lib = None
@@ -142,6 +146,29 @@ def profile_query(kernel_name):
     check(lib().nblahip_profile_query(kernel_name.encode(), ctypes.byref(total),
                                       ctypes.byref(count)))
     return total.value, count.value
+
+
+def profile_kernels():
+    """Names of the kernels recorded since the last profile reset, in order of
+    first launch."""
+    need = _sz(0)
+    check(lib().nblahip_profile_kernels(None, 0, ctypes.byref(need)))
+    buf = ctypes.create_string_buffer(need.value)
+    check(lib().nblahip_profile_kernels(buf, need.value, ctypes.byref(need)))
+    return [n for n in buf.value.decode().split("\n") if n]
+
+
+def tune_set(name, value):
+    """Override plan knob NBLAHIP_<name> from the next call on (-1: undo)."""
+    check(lib().nblahip_tune_set(name.encode(), int(value)))
+
+
+def tune_get(name, fallback=-1):
+    return lib().nblahip_tune_get(name.encode(), int(fallback))
+
+
+def tune_reset():
+    check(lib().nblahip_tune_reset())
 
 
 # ---------------------------------------------------------------------------

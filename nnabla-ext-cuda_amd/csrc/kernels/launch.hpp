@@ -37,8 +37,8 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 // Number of compute units of the current device (cached per device).
 int device_cus();
 
-// Read-once integer tuning knob from the environment (name without prefix
-// "NBLAHIP_"); returns `fallback` when unset or unparsable.
+// Integer plan knob (name without the prefix "NBLAHIP_"): the value set through
+// nblahip_tune_set, else the environment's (read once), else `fallback`.
 int tune_int(const char *name, int fallback);
 
 // One row-normalization problem (LayerNormalization rows,

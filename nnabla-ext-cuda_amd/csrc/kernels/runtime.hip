@@ -27,24 +27,37 @@ int device_cus() {
   return cus[dev];
 }
 
-int tune_int(const char *name, int fallback) {
-  // Only the environment's answer is cached (-1: not set): callers may pass
-  // different fallbacks for the same knob.
-  static std::mutex mu;
-  static std::unordered_map<std::string, int> cache;
-  std::lock_guard<std::mutex> lock(mu);
-  auto it = cache.find(name);
-  if (it == cache.end()) {
-    int v = -1;
+namespace {
+// name -> value from the environment (-1: not set) and the value set through
+// nblahip_tune_set (-1: none); the latter wins.
+struct TuneEntry {
+  int env = -1, set = -1;
+};
+std::mutex g_tune_mu;
+std::unordered_map<std::string, TuneEntry> g_tune;
+
+TuneEntry &tune_entry_locked(const char *name) {
+  auto it = g_tune.find(name);
+  if (it == g_tune.end()) {
+    TuneEntry e;
     const std::string key = std::string("NBLAHIP_") + name;
     if (const char *s = std::getenv(key.c_str())) {
       char *end = nullptr;
       const long parsed = std::strtol(s, &end, 10);
-      if (end != s && parsed >= 0 && parsed < (1 << 20)) v = static_cast<int>(parsed);
+      if (end != s && parsed >= 0 && parsed < (1 << 20)) e.env = static_cast<int>(parsed);
     }
-    it = cache.emplace(name, v).first;
+    it = g_tune.emplace(name, e).first;
   }
-  return it->second >= 0 ? it->second : fallback;
+  return it->second;
+}
+} // namespace
+
+int tune_int(const char *name, int fallback) {
+  // Only the environment's answer is cached: callers may pass different
+  // fallbacks for the same knob.
+  std::lock_guard<std::mutex> lock(g_tune_mu);
+  const TuneEntry &e = tune_entry_locked(name);
+  return e.set >= 0 ? e.set : e.env >= 0 ? e.env : fallback;
 }
 
 // ---------------------------------------------------------------------------
@@ -173,6 +186,47 @@ int nblahip_profile_query(const char *kernel_name, double *total_ms, int64_t *la
     *total_ms += ms;
     *launches += 1;
   }
+  return 0;
+}
+
+int nblahip_profile_kernels(char *names, size_t capacity, size_t *needed) {
+  if (!needed || (!names && capacity)) return NBLAHIP_EINVAL;
+  std::lock_guard<std::mutex> lock(g_prof.mu);
+  std::vector<const char *> seen;
+  std::string out;
+  for (size_t i = 0; i < g_prof.used; ++i) {
+    const char *tag = g_prof.records[i].tag;
+    bool dup = false;
+    for (const char *t : seen) dup = dup || std::strcmp(t, tag) == 0;
+    if (dup) continue;
+    seen.push_back(tag);
+    if (!out.empty()) out += '\n';
+    out += tag;
+  }
+  *needed = out.size() + 1;
+  if (capacity) {
+    const size_t n = out.size() < capacity - 1 ? out.size() : capacity - 1;
+    std::memcpy(names, out.data(), n);
+    names[n] = '\0';
+  }
+  return 0;
+}
+
+int nblahip_tune_set(const char *name, int value) {
+  if (!name || !*name || value >= (1 << 20)) return NBLAHIP_EINVAL;
+  std::lock_guard<std::mutex> lock(g_tune_mu);
+  tune_entry_locked(name).set = value < 0 ? -1 : value;
+  return 0;
+}
+
+int nblahip_tune_get(const char *name, int fallback) {
+  if (!name || !*name) return fallback;
+  return tune_int(name, fallback);
+}
+
+int nblahip_tune_reset(void) {
+  std::lock_guard<std::mutex> lock(g_tune_mu);
+  for (auto &kv : g_tune) kv.second.set = -1;
   return 0;
 }
 

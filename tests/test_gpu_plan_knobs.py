@@ -1,0 +1,282 @@
+"""Every plan a knob can switch on is held to the oracle.
+
+A shape is served by one of several kernel families, chosen per call from the
+plan knobs (NBLAHIP_<NAME> in the environment, or nblahip_tune_set).  The
+default choice is what the other test files exercise; here each knob that
+selects another kernel, or another grid for the same kernel, is set through
+nblahip_tune_set, the forward and backward of a shape that the knob affects
+run through the C-ABI, the results are compared with the float64 oracle, and
+the kernels that ran (read back from the library's per-kernel timing) are
+compared with the kernels of the default plan."""
+import numpy as np
+import pytest
+import torch
+
+from _util import assert_close, dtype_name, load_package, rounded, to_dev, to_np
+from oracle import norm_ref as R
+
+pytestmark = pytest.mark.gpu
+K = load_package()
+F32, F16 = torch.float32, torch.float16
+
+
+def f32(a):
+    return np.asarray(a, np.float32).astype(np.float64)
+
+
+@pytest.fixture(autouse=True)
+def _default_knobs_afterwards():
+    K.tune_reset()
+    yield
+    K.tune_reset()
+    K.check(K.lib().nblahip_profile_enable(0))
+
+
+# --------------------------------------------------------------- runners
+# Each runs forward + backward on the device, checks every output against the
+# oracle and returns nothing; inputs are seeded per case.
+def run_bn(shape, axis, dtype, seed=1):
+    dn = dtype_name(dtype)
+    rng = np.random.default_rng(seed)
+    c = shape[axis]
+    x = rounded(rng.standard_normal(shape) * 2 + 1, dtype)
+    dy = rounded(rng.standard_normal(shape), dtype)
+    g, b = f32(rng.uniform(0.5, 1.5, c)), f32(rng.standard_normal(c) * 0.1)
+    rm, rv = f32(rng.standard_normal(c) * 0.1), f32(rng.uniform(0.5, 2.0, c))
+    y_r, m_r, v_r, rm_r, rv_r = R.bn_forward_batch(x, b, g, rm, rv, axis, 0.9, 1e-5)
+    dx_r, dg_r, db_r = R.bn_backward_batch(x, dy, g, m_r, v_r, axis, 1e-5)
+    xd, dyd, gd, bd = to_dev(x, dtype), to_dev(dy, dtype), to_dev(g), to_dev(b)
+    rmd, rvd = to_dev(rm), to_dev(rv)
+    y, m, v = K.bn_forward_batch(xd, bd, gd, rmd, rvd, axis, 0.9, 1e-5)
+    assert_close(to_np(y), y_r, dn, "y", "y")
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    assert_close(to_np(rmd), rm_r, dn, "stat", "running mean")
+    assert_close(to_np(rvd), rv_r, dn, "stat", "running var")
+    dx, dg, db = K.bn_backward(xd, dyd, gd, m, v, axis, 1e-5)
+    assert_close(to_np(dx), dx_r, dn, "grad", "dx")
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
+
+
+def run_ln(outer, Rr, dtype, seed=2):
+    dn = dtype_name(dtype)
+    rng = np.random.default_rng(seed)
+    x = rounded(rng.standard_normal((outer, Rr)) + rng.uniform(-3, 3, (outer, 1)), dtype)
+    dy = rounded(rng.standard_normal((outer, Rr)), dtype)
+    g, b = f32(rng.standard_normal(Rr) * 0.1 + 1), f32(rng.standard_normal(Rr) * 0.1)
+    y_r, m_r, v_r = R.ln_forward(x, b, g, outer, 1e-5)
+    dx_r, dg_r, db_r = R.ln_backward(x, dy, g, m_r, v_r, outer, 1e-5)
+    xd, dyd, gd, bd = to_dev(x, dtype), to_dev(dy, dtype), to_dev(g), to_dev(b)
+    y, m, v = K.ln_forward(xd, bd, gd, outer, 1e-5)
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    assert_close(to_np(y), y_r, dn, "y", "y")
+    dx, dg, db = K.ln_backward(xd, dyd, gd, m, v, outer, 1e-5)
+    assert_close(to_np(dx), dx_r, dn, "grad", "dx")
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
+
+
+def _nc_inputs(n, c, sp, dtype, seed, channel_last):
+    """Channel-first float64 views of the inputs (for the oracle) and the
+    arrays in the caller's layout (for the device)."""
+    rng = np.random.default_rng(seed)
+    shape = (n, c) + tuple(sp)
+    x = rounded(rng.standard_normal(shape) * 1.5 + rng.uniform(-2, 2, (n, c) + (1,) * len(sp)), dtype)
+    dy = rounded(rng.standard_normal(shape), dtype)
+    g, b = f32(rng.uniform(0.5, 1.5, c)), f32(rng.standard_normal(c) * 0.1)
+    lay = (lambda a: np.ascontiguousarray(np.moveaxis(a, 1, -1))) if channel_last else (lambda a: a)
+    return x, dy, g, b, lay
+
+
+def run_gn(n, c, sp, groups, dtype, channel_last=False, seed=3):
+    dn = dtype_name(dtype)
+    x, dy, g, b, lay = _nc_inputs(n, c, sp, dtype, seed, channel_last)
+    y_r, m_r, v_r = R.gn_forward(x, b, g, n, c, groups, 1e-5)
+    dx_r, dg_r, db_r = R.gn_backward(x, dy, g, m_r, v_r, n, c, groups, 1e-5)
+    xd, dyd, gd, bd = to_dev(lay(x), dtype), to_dev(lay(dy), dtype), to_dev(g), to_dev(b)
+    y, m, v = K.gn_forward(xd, bd, gd, groups, 1e-5, channel_last=channel_last)
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    assert_close(to_np(y), lay(y_r.reshape(x.shape)), dn, "y", "y")
+    dx, dg, db = K.gn_backward(xd, dyd, gd, m, v, groups, 1e-5, channel_last=channel_last)
+    assert_close(to_np(dx), lay(dx_r.reshape(x.shape)), dn, "grad", "dx")
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
+
+
+def run_in(n, c, sp, dtype, channel_last=False, seed=4):
+    dn = dtype_name(dtype)
+    x, dy, g, b, lay = _nc_inputs(n, c, sp, dtype, seed, channel_last)
+    y_r, m_r, v_r = R.in_forward(x, b, g, n, c, 1e-5)
+    dx_r, dg_r, db_r = R.in_backward(x, dy, g, m_r, v_r, n, c, 1e-5)
+    xd, dyd, gd, bd = to_dev(lay(x), dtype), to_dev(lay(dy), dtype), to_dev(g), to_dev(b)
+    y, m, v = K.in_forward(xd, bd, gd, 1e-5, channel_last=channel_last)
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    assert_close(to_np(y), lay(y_r.reshape(x.shape)), dn, "y", "y")
+    dx, dg, db = K.in_backward(xd, dyd, gd, m, v, 1e-5, channel_last=channel_last)
+    assert_close(to_np(dx), lay(dx_r.reshape(x.shape)), dn, "grad", "dx")
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
+
+
+def kernels_of(run, args, knobs):
+    """Runs `run(*args)` (with its oracle checks) under `knobs`; returns the
+    names of the kernels the library launched."""
+    K.tune_reset()
+    for name, value in knobs.items():
+        K.tune_set(name, value)
+    K.check(K.lib().nblahip_profile_enable(256))
+    run(*args)
+    torch.cuda.synchronize()
+    names = K.profile_kernels()
+    K.check(K.lib().nblahip_profile_enable(0))
+    K.tune_reset()
+    return names
+
+
+# --------------------------------------------------------------- the table
+# (id, runner, arguments, knobs, kernels the knob must bring in, kernels of the
+# default plan that it must keep out).  The default plan of every row is run
+# as well (same oracle checks) and must contain the "out" kernels: that pins
+# that the shape is one the knob decides about.
+SWITCHES = [
+    # BatchNormalization, planes layout
+    ("bn_onchip_off", run_bn, ((32, 64, 56, 56), 1, F16), {"BN_ONCHIP": 0},
+     ["bn_stats_planes_kernel", "bn_apply_planes_kernel", "bn_bwd_reduce_planes_kernel",
+      "bn_bwd_apply_planes_kernel"],
+     ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"]),
+    ("bn_onchip_fwd_max", run_bn, ((32, 32, 56, 56), 1, F32), {"BN_ONCHIP_FWD_MAX": 16},
+     ["bn_stats_planes_kernel"], ["bn_onchip_fwd_kernel"]),
+    ("bn_onchip_bwd_max", run_bn, ((32, 64, 56, 56), 1, F16), {"BN_ONCHIP_BWD_MAX": 8},
+     ["bn_onchip_fwd_kernel", "bn_bwd_reduce_planes_kernel"], ["bn_onchip_bwd_kernel"]),
+    ("bn_onchip_min_pct_up", run_bn, ((32, 64, 56, 56), 1, F16),
+     {"BN_ONCHIP_FWD_MIN_PCT": 100, "BN_ONCHIP_BWD_MIN_PCT": 100},
+     ["bn_stats_planes_kernel", "bn_bwd_reduce_planes_kernel"],
+     ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"]),
+    ("bn_rows_off", run_bn, ((32, 64, 14, 14), 1, F16), {"BN_ROWS": 0},
+     ["bn_stats_planes_kernel", "bn_finalize_fwd_kernel", "bn_apply_planes_kernel",
+      "bn_finalize_bwd_kernel"], ["row_fwd_kernel_bn", "row_bwd_kernel_bn"]),
+    ("bn_cl_cached_off", run_bn, ((32, 7, 7, 256), 3, F16), {"BN_CL_CACHED": 0},
+     ["bn_stats_cl_kernel", "bn_apply_cl_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
+     ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"]),
+    # rows: LayerNormalization / GroupNormalization / InstanceNormalization
+    ("ln_force_stream", run_ln, (64, 1024, F32), {"FORCE_STREAM": 1},
+     ["row_stats_stream_kernel", "row_apply_fwd_kernel", "ln_row_sums_stream_kernel",
+      "row_bwd_dx_kernel", "ln_colgrad_stream_kernel"], ["row_fwd_kernel", "row_bwd_kernel_ln"]),
+    ("gn_force_stream", run_gn, (4, 32, (16, 16), 8, F16), {"FORCE_STREAM": 1},
+     ["row_stats_stream_kernel", "plane_sums_stream_kernel", "plane_to_row_factors_kernel"],
+     ["row_fwd_kernel", "row_bwd_kernel_gn"]),
+    ("in_force_stream", run_in, (4, 16, (32, 32), F32), {"FORCE_STREAM": 1},
+     ["row_stats_stream_kernel", "plane_sums_stream_kernel"], ["row_fwd_kernel", "row_bwd_kernel_in"]),
+    ("ln_long_rows_all_streaming", run_ln, (24, 18432, F16), {"LN_LONG_ROWS_CACHED": 0},
+     ["ln_row_sums_stream_kernel", "row_bwd_dx_kernel"], ["row_bwd_kernel_lnx"]),
+    ("in_rows_instead_of_channel_blocks", run_in, (4, 256, (32, 32), F16), {"IN_NO_CHANNEL_BLOCKS": 1},
+     ["row_bwd_kernel_in", "pair_param_reduce_kernel"], ["row_bwd_kernel_inc"]),
+    ("gn_float_groups_streamed", run_gn, (4, 64, (64, 64), 8, F32), {"GN_FLOAT_1024X8": 0},
+     ["plane_sums_stream_kernel", "row_bwd_dx_kernel"], ["row_bwd_kernel_gn"]),
+    ("gn_rows_onchip_off", run_gn, (4, 320, (64, 64), 32, F32), {"ROW_ONCHIP": 0},
+     ["row_stats_stream_kernel", "row_apply_fwd_kernel"], ["row_onchip_fwd_kernel"]),
+    ("in_rows_onchip_off", run_in, (2, 64, (256, 256), F32), {"ROW_ONCHIP": 0},
+     ["row_stats_stream_kernel", "plane_sums_stream_kernel"],
+     ["row_onchip_fwd_kernel", "bn_onchip_bwd_kernel"]),
+    ("rows_onchip_min_pct_up", run_gn, (4, 320, (64, 64), 32, F32), {"ROW_ONCHIP_MIN_PCT": 100},
+     ["row_stats_stream_kernel"], ["row_onchip_fwd_kernel"]),
+    ("in_rows_onchip_bwd_min_pct_up", run_in, (2, 64, (256, 256), F32), {"ROW_ONCHIP_BWD_MIN_PCT": 100},
+     ["row_onchip_fwd_kernel", "plane_sums_stream_kernel"], ["bn_onchip_bwd_kernel"]),
+    # channel-last GroupNormalization / InstanceNormalization
+    ("gn_cl_wide_off", run_gn, (4, 1024, (32, 32), 128, F16, True),
+     {"GN_CL_WIDE": 0, "GN_CL_WIDE_BWD": 0}, ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"],
+     ["gn_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"]),
+    ("in_cl_wide_off", run_in, (4, 1024, (32, 32), F16, True),
+     {"GN_CL_WIDE": 0, "GN_CL_WIDE_BWD": 0}, ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"],
+     ["in_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"]),
+    ("gn_cl_cached_off", run_gn, (2, 128, (20, 20), 8, F32, True), {"GN_CL_CACHED": 0},
+     ["bn_stats_cl_kernel", "gn_cl_finalize_fwd_kernel", "bn_bwd_reduce_cl_kernel",
+      "gn_cl_finalize_bwd_kernel"], ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"]),
+    ("in_cl_cached_off", run_in, (2, 128, (20, 20), F32, True), {"IN_CL_CACHED": 0},
+     ["bn_stats_cl_kernel", "gn_cl_finalize_fwd_kernel", "gn_cl_finalize_bwd_kernel"],
+     ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"]),
+    ("in_cl_min_positions_up", run_in, (4, 64, (8, 8), F16, True), {"IN_CL_MIN": 128},
+     ["bn_stats_cl_kernel", "bn_bwd_reduce_cl_kernel"], ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"]),
+]
+
+
+@pytest.mark.parametrize("case", SWITCHES, ids=[c[0] for c in SWITCHES])
+def test_plan_switch_changes_the_kernels_and_keeps_parity(case):
+    _, run, args, knobs, must_run, must_not_run = case
+    default = kernels_of(run, args, {})
+    for name in must_not_run:
+        assert name in default, f"default plan of {args} ran {default}, expected {name} among them"
+    switched = kernels_of(run, args, knobs)
+    for name in must_run:
+        assert name in switched, f"{knobs}: ran {switched}, expected {name}"
+    for name in must_not_run:
+        assert name not in switched, f"{knobs}: {name} still ran ({switched})"
+
+
+# Knobs that keep the kernel names and change grids, thread maps, template
+# instances or limits: parity under each value.  (id, runner, arguments, list
+# of knob settings, kernels that must run, kernels that must not.)
+GRIDS = [
+    ("bn_blocks_per_cu", run_bn, ((16, 48, 28, 28), 1, F32),
+     [{"BN_ROWS": 0, "BN_BLOCKS_PER_CU": v} for v in (1, 4, 64)],
+     ["bn_stats_planes_kernel", "bn_finalize_fwd_kernel", "bn_finalize_bwd_kernel"], []),
+    # channel-owning 1024-thread reduction blocks: no partials, no finalize kernel
+    ("bn_direct_always", run_bn, ((16, 24, 28, 28), 1, F32), [{"BN_ROWS": 0, "BN_DIRECT": 1}],
+     ["bn_stats_planes_kernel", "bn_bwd_reduce_planes_kernel"],
+     ["bn_finalize_fwd_kernel", "bn_finalize_bwd_kernel"]),
+    ("bn_direct_never", run_bn, ((8, 256, 28, 28), 1, F16), [{"BN_ROWS": 0, "BN_DIRECT": 0}],
+     ["bn_stats_planes_kernel", "bn_finalize_fwd_kernel", "bn_finalize_bwd_kernel"], []),
+    ("bn_apply_persistent", run_bn, ((16, 48, 28, 28), 1, F32),
+     [{"BN_ROWS": 0, "BN_APPLY_BLOCKS_PER_CU": v} for v in (1, 3)],
+     ["bn_apply_planes_kernel", "bn_bwd_apply_planes_kernel"], []),
+    ("bn_masked_planes_off", run_bn, ((64, 64, 7, 7), 1, F16), [{"BN_ROWS": 0, "BN_MASKED_PLANES": 0}],
+     ["bn_stats_planes_kernel", "bn_apply_planes_kernel"], []),
+    ("bn_cl_grids", run_bn, ((64, 28, 28, 64), 3, F16),
+     [{"BN_CL_BLOCKS_PER_CU": a, "BN_CL_FWD_APPLY_BLOCKS_PER_CU": b, "BN_CL_APPLY_BLOCKS_PER_CU": c}
+      for a, b, c in ((1, 1, 1), (2, 4, 2), (8, 3, 7))],
+     ["bn_stats_cl_kernel", "bn_apply_cl_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
+     []),
+    ("bn_onchip_few_channels", run_bn, ((32, 4, 56, 56), 1, F16),
+     [{"BN_ONCHIP_FWD_MIN_PCT": 1, "BN_ONCHIP_BWD_MIN_PCT": 1}],
+     ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
+    ("bn_onchip_streamed_few_channels", run_bn, ((64, 8, 56, 56), 1, F32),
+     [{"BN_ONCHIP_STREAMED_MIN_PCT": 1}], ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
+    ("ln_bwd_blocks_per_cu", run_ln, (4096, 1024, F16), [{"LN_BWD_BLOCKS_PER_CU": v} for v in (1, 2, 4)],
+     ["row_bwd_kernel_ln", "ln_param_reduce_kernel"], []),
+    ("ln_wave_per_short_row", run_ln, (1000, 32, F32), [{"ROW_SUBWAVE": 0}],
+     ["row_fwd_kernel", "row_bwd_kernel_ln"], []),
+    ("ln_forced_subwave_layout", run_ln, (513, 128, F32), [{"ROW_TPR": 8, "ROW_NL": 4},
+                                                           {"ROW_TPR": 16, "ROW_NL": 2}],
+     ["row_fwd_kernel", "row_bwd_kernel_ln"], []),
+    ("rows_onchip_few_rows", run_in, (1, 8, (256, 256), F32),
+     [{"ROW_ONCHIP_MIN_PCT": 1, "ROW_ONCHIP_BWD_MIN_PCT": 1}],
+     ["row_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
+    ("rows_onchip_streamed_few_rows", run_in, (1, 8, (512, 512), F16),
+     [{"ROW_ONCHIP_STREAMED_MIN_PCT": 1}], ["row_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
+    ("gn_cl_wide_plain_block_order", run_gn, (4, 1024, (32, 32), 128, F16, True), [{"GN_CL_XCD_MAP": 0}],
+     ["gn_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], []),
+    ("in_cl_wide_plain_block_order", run_in, (4, 1024, (32, 32), F16, True), [{"GN_CL_XCD_MAP": 0}],
+     ["in_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], []),
+    ("gn_cl_rows_plain_block_order", run_gn, (2, 128, (20, 20), 8, F32, True), [{"GN_CL_XCD_MAP": 0}],
+     ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"], []),
+    ("in_cl_rows_plain_block_order", run_in, (2, 128, (20, 20), F16, True),
+     [{"GN_CL_XCD_MAP": 0, "GN_CL_WIDE": 0, "GN_CL_WIDE_BWD": 0}],
+     ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"], []),
+    ("in_cl_fewer_positions", run_in, (4, 64, (4, 4), F16, True), [{"IN_CL_MIN": 8}],
+     ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"], []),
+]
+
+
+@pytest.mark.parametrize("case", GRIDS, ids=[c[0] for c in GRIDS])
+def test_grid_and_limit_knobs_keep_parity(case):
+    _, run, args, settings, expected, absent = case
+    for knobs in settings:
+        ran = kernels_of(run, args, knobs)
+        for name in expected:
+            assert name in ran, f"{knobs}: ran {ran}, expected {name}"
+        for name in absent:
+            assert name not in ran, f"{knobs}: {name} ran ({ran})"
