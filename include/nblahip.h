@@ -234,7 +234,8 @@ NBLAHIP_EXPORT int nblahip_fused_bn_bwd(
  * workspace.  For tensors of a few very long rows they keep partial statistics
  * in the first bytes of y until the pass that writes y overwrites them: y must
  * not overlap x other than being x itself (in place, y == x, is detected and
- * handled without the scratch use).
+ * handled without the scratch use), nor gamma, beta, mean or var.  A y that
+ * does is rejected with NBLAHIP_EALIAS before anything is launched.
  * ---------------------------------------------------------------------- */
 
 /* Replaces forward_impl (layer_normalization.cu:77-133): reduce_2d_x<WelfordOp>

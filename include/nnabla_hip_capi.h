@@ -59,6 +59,16 @@ NNABLA_HIP_EXPORT int nnabla_hip_variable_get(nnabla_hip_variable *v, int which,
 NNABLA_HIP_EXPORT int nnabla_hip_variable_cast(nnabla_hip_variable *v, int which,
                                                const char *array_class, const char *device_id,
                                                int dtype, int write_only, int async_flags);
+/* dtype above: 0 float, 1 half, or 0x100 + the core's dtypes enumerator (BOOL 0,
+ * BYTE 1, UBYTE 2, SHORT 3, USHORT 4, INT 5, UINT 6, LONG 7, ULONG 8, FLOAT 9,
+ * DOUBLE 10, HALF 23): device arrays store and copy every dtype, as CudaArray
+ * does (src/nbla/cuda/array/cuda_array.cpp:211-279); only float and half are
+ * filled with values and converted.  set_raw / get_raw move n elements of that
+ * dtype between host memory and the variable without conversion. */
+NNABLA_HIP_EXPORT int nnabla_hip_variable_set_raw(nnabla_hip_variable *v, int which,
+                                                  const void *host, int64_t n, int dtype);
+NNABLA_HIP_EXPORT int nnabla_hip_variable_get_raw(nnabla_hip_variable *v, int which, void *host,
+                                                  int64_t n, int dtype);
 NNABLA_HIP_EXPORT int nnabla_hip_pending_transfers(uint64_t *count);
 NNABLA_HIP_EXPORT int nnabla_hip_variable_zero(nnabla_hip_variable *v, int which);
 NNABLA_HIP_EXPORT int nnabla_hip_variable_fill(nnabla_hip_variable *v, int which, float value);

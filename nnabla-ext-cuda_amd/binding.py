@@ -36,6 +36,8 @@ SIGNATURES = {
     "nnabla_hip_variable_set": (_I, [_P, _I, _FP, _I64, _I]),
     "nnabla_hip_variable_get": (_I, [_P, _I, _FP, _I64]),
     "nnabla_hip_variable_cast": (_I, [_P, _I, _S, _S, _I, _I, _I]),
+    "nnabla_hip_variable_set_raw": (_I, [_P, _I, ctypes.c_void_p, _I64, _I]),
+    "nnabla_hip_variable_get_raw": (_I, [_P, _I, ctypes.c_void_p, _I64, _I]),
     "nnabla_hip_pending_transfers": (_I, [ctypes.POINTER(ctypes.c_uint64)]),
     "nnabla_hip_variable_zero": (_I, [_P, _I]),
     "nnabla_hip_variable_fill": (_I, [_P, _I, _F]),
@@ -213,6 +215,32 @@ class Variable:
         _check(lib().nnabla_hip_variable_cast(self._h, which, array_class.encode(),
                                               str(device_id).encode(), 1 if half else 0,
                                               1 if write_only else 0, int(async_flags)))
+
+    # numpy dtype -> 0x100 + the core's dtypes enumerator
+    _RAW = {"bool": 0, "int8": 1, "uint8": 2, "int16": 3, "uint16": 4, "int32": 5, "uint32": 6,
+            "int64": 7, "uint64": 8, "float32": 9, "float64": 10, "float16": 23}
+
+    def set_raw(self, a, which=0):
+        """Stores `a` in its own dtype (no conversion)."""
+        a = np.ascontiguousarray(a).reshape(-1)
+        _check(lib().nnabla_hip_variable_set_raw(self._h, which, a.ctypes.data, a.size,
+                                                 0x100 + self._RAW[a.dtype.name]))
+
+    def get_raw(self, dtype, which=0):
+        shape = self.current_shape
+        out = np.empty(int(np.prod(shape, dtype=np.int64)), np.dtype(dtype))
+        _check(lib().nnabla_hip_variable_get_raw(self._h, which, out.ctypes.data, out.size,
+                                                 0x100 + self._RAW[out.dtype.name]))
+        return out.reshape(shape)
+
+    def cast_raw(self, array_class, dtype, device_id="0", which=0, async_flags=0):
+        _check(lib().nnabla_hip_variable_cast(self._h, which, array_class.encode(),
+                                              str(device_id).encode(),
+                                              0x100 + self._RAW[np.dtype(dtype).name], 0,
+                                              int(async_flags)))
+
+    def zero_data(self):
+        _check(lib().nnabla_hip_variable_zero(self._h, 0))
 
     def zero_grad(self):
         _check(lib().nnabla_hip_variable_zero(self._h, 1))

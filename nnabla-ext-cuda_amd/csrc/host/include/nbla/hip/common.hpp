@@ -42,7 +42,8 @@ template <> struct HipDtype<Half> { static constexpr int code = NBLAHIP_F16; };
 
 inline int hip_dtype_code(dtypes d) {
   NBLA_CHECK(d == dtypes::FLOAT || d == dtypes::HALF, error_code::type,
-             "The hip backend stores float32 and float16 only.");
+             "The hip backend fills and converts float32 and float16 only (other dtypes are "
+             "stored and copied).");
   return d == dtypes::FLOAT ? NBLAHIP_F32 : NBLAHIP_F16;
 }
 

@@ -1,4 +1,5 @@
 // Flat C surface over the C++ backend (see include/nnabla_hip_capi.h).
+#include <cstring>
 #include <nnabla_hip_capi.h>
 
 #include <nbla/cpu.hpp>
@@ -194,15 +195,53 @@ int nnabla_hip_variable_get(nnabla_hip_variable *v, int which, float *host, int6
   });
 }
 
+namespace {
+// 0: float, 1: half, 0x100 + n: the core's dtypes enumerator n (any stored type).
+dtypes storage_dtype(int dtype) {
+  if (dtype == 0) return dtypes::FLOAT;
+  if (dtype == 1) return dtypes::HALF;
+  const int n = dtype - 0x100;
+  NBLA_CHECK((n >= static_cast<int>(dtypes::BOOL) && n <= static_cast<int>(dtypes::DOUBLE)) ||
+                 n == static_cast<int>(dtypes::HALF),
+             error_code::value, "dtype must be 0 (float), 1 (half) or 0x100 + a core dtype");
+  return static_cast<dtypes>(n);
+}
+} // namespace
+
 int nnabla_hip_variable_cast(nnabla_hip_variable *v, int which, const char *array_class,
                              const char *device_id, int dtype, int write_only, int async_flags) {
   return guarded([&] {
     NdArrayPtr a = pick(v, which);
-    NBLA_CHECK(dtype == 0 || dtype == 1, error_code::value, "dtype must be 0 (float) or 1 (half)");
     NBLA_CHECK(array_class != nullptr, error_code::value, "array_class must be given");
     init_hip();
     const Context ctx({}, array_class, device_id ? device_id : "0");
-    a->cast(dtype == 0 ? dtypes::FLOAT : dtypes::HALF, ctx, write_only != 0, async_flags);
+    a->cast(storage_dtype(dtype), ctx, write_only != 0, async_flags);
+  });
+}
+
+int nnabla_hip_variable_set_raw(nnabla_hip_variable *v, int which, const void *host, int64_t n,
+                                int dtype) {
+  return guarded([&] {
+    NdArrayPtr a = pick(v, which);
+    NBLA_CHECK(host && n == a->size(), error_code::value, "expected %lld elements, given %lld",
+               static_cast<long long>(a->size()), static_cast<long long>(n));
+    init_cpu();
+    const dtypes d = storage_dtype(dtype);
+    void *dst = a->cast(d, host_ctx(), true)->pointer<void>();
+    std::memcpy(dst, host, static_cast<size_t>(n) * sizeof_dtype(d));
+  });
+}
+
+int nnabla_hip_variable_get_raw(nnabla_hip_variable *v, int which, void *host, int64_t n,
+                                int dtype) {
+  return guarded([&] {
+    NdArrayPtr a = pick(v, which);
+    NBLA_CHECK(host && n == a->size(), error_code::value, "expected %lld elements, given %lld",
+               static_cast<long long>(a->size()), static_cast<long long>(n));
+    init_cpu();
+    const dtypes d = storage_dtype(dtype);
+    const void *src = a->get(d, host_ctx())->const_pointer<void>();
+    std::memcpy(host, src, static_cast<size_t>(n) * sizeof_dtype(d));
   });
 }
 

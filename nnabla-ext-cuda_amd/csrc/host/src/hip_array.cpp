@@ -6,7 +6,6 @@ namespace nbla {
 
 HipArray::HipArray(Size_t size, dtypes dtype, const Context &ctx, bool cached)
     : Array(size, dtype, ctx), device_(std::stoi(ctx.device_id)), cached_(cached) {
-  hip_dtype_code(dtype); // rejects unsupported dtypes up front
   if (cached_) {
     ptr_ = SingletonManager::get<Hip>()->alloc(nbytes(), device_);
   } else {
@@ -24,12 +23,24 @@ HipArray::~HipArray() {
   }
 }
 
+namespace {
+bool is_float_dtype(dtypes d) { return d == dtypes::FLOAT || d == dtypes::HALF; }
+} // namespace
+
+// Any dtype is stored and moved (the reference's CudaArray holds every dtype,
+// src/nbla/cuda/array/cuda_array.cpp:211-279); value fills and conversions
+// exist for the two float types the normalization functions compute in.
 void HipArray::zero() {
   hip_set_device(device_);
-  NBLA_HIP_CHECK(nblahip_fill(ptr_, hip_dtype_code(dtype_), 0.f, size_, nullptr));
+  if (is_float_dtype(dtype_)) {
+    NBLA_HIP_CHECK(nblahip_fill(ptr_, hip_dtype_code(dtype_), 0.f, size_, nullptr));
+  } else {
+    NBLA_HIP_CHECK(nblahip_memset(ptr_, 0, nbytes(), nullptr));
+  }
 }
 
 void HipArray::fill(float value) {
+  if (value == 0.f) return zero();
   hip_set_device(device_);
   NBLA_HIP_CHECK(nblahip_fill(ptr_, hip_dtype_code(dtype_), value, size_, nullptr));
 }
@@ -37,6 +48,10 @@ void HipArray::fill(float value) {
 void HipArray::copy_from(const Array *src) {
   NBLA_CHECK(src->size() == size_, error_code::value, "size mismatch in HipArray::copy_from");
   hip_set_device(device_);
+  if (src->dtype() == dtype_) {
+    NBLA_HIP_CHECK(nblahip_memcpy_d2d(ptr_, src->const_pointer<void>(), nbytes(), nullptr));
+    return;
+  }
   NBLA_HIP_CHECK(nblahip_convert(ptr_, hip_dtype_code(dtype_), src->const_pointer<void>(),
                                  hip_dtype_code(src->dtype()), size_, nullptr));
 }

@@ -31,6 +31,27 @@ int check_dims3(int64_t a, int64_t b, int64_t c) {
 
 hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
 
+bool ranges_overlap(const void *a, size_t a_bytes, const void *b, size_t b_bytes) {
+  if (!a || !b || !a_bytes || !b_bytes) return false;
+  const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+  return a0 < b0 + b_bytes && b0 < a0 + a_bytes;
+}
+
+// The row forwards may keep partial statistics in y before they write it, and
+// they read gamma/beta while writing y: y may be x itself (in place) but must
+// not overlap x partially, nor the parameters, nor the statistics outputs.
+int check_fwd_alias(const void *x, void *y, size_t tensor_bytes, const float *gamma, size_t g_bytes,
+                    const float *beta, size_t b_bytes, const float *mean, const float *var,
+                    size_t stat_bytes) {
+  if (y != x && ranges_overlap(x, tensor_bytes, y, tensor_bytes)) return NBLAHIP_EALIAS;
+  if (ranges_overlap(y, tensor_bytes, gamma, g_bytes) || ranges_overlap(y, tensor_bytes, beta, b_bytes) ||
+      ranges_overlap(y, tensor_bytes, mean, stat_bytes) || ranges_overlap(y, tensor_bytes, var, stat_bytes))
+    return NBLAHIP_EALIAS;
+  return 0;
+}
+
+size_t elem_bytes(int dtype) { return dtype == NBLAHIP_F16 ? 2 : 4; }
+
 // Scratch of nblahip_bn_fwd_train_static, the entry point for callers that
 // cannot allocate: one array per GPU in the code object's own data segment,
 // held until the process ends.  `scratch` below is only the host-side handle
@@ -359,6 +380,10 @@ int nblahip_ln_fwd(const void *x, const float *gamma, const float *beta, void *y
   const int d = check_dims3(outer, reduce, 1);
   if (d) return d < 0 ? d : 0;
   if (!x || !y || !mean || !var) return NBLAHIP_EINVAL;
+  if (int e = check_fwd_alias(x, y, static_cast<size_t>(outer) * reduce * elem_bytes(dtype), gamma,
+                              reduce * sizeof(float), beta, reduce * sizeof(float), mean, var,
+                              outer * sizeof(float)))
+    return e;
   RowProblem p;
   p.dtype = dtype;
   p.mode = kRowLN;
@@ -441,6 +466,10 @@ int nblahip_gn_fwd(const void *x, const float *gamma, const float *beta, void *y
   const int d = gn_problem(p, batch, channels, spatial, groups, dtype);
   if (d) return d < 0 ? d : 0;
   if (!x || !y || !mean || !var) return NBLAHIP_EINVAL;
+  if (int e = check_fwd_alias(x, y, static_cast<size_t>(batch) * channels * spatial * elem_bytes(dtype),
+                              gamma, channels * sizeof(float), beta, channels * sizeof(float), mean,
+                              var, static_cast<size_t>(batch) * groups * sizeof(float)))
+    return e;
   p.x = x;
   p.out = y;
   p.gamma = gamma;
@@ -517,6 +546,11 @@ int nblahip_in_fwd(const void *x, const float *gamma, const float *beta, void *y
   const int d = in_problem(p, batch, channels, spatial, bc_gamma, bc_beta, dtype);
   if (d) return d < 0 ? d : 0;
   if (!x || !y || !mean || !var) return NBLAHIP_EINVAL;
+  if (int e = check_fwd_alias(x, y, static_cast<size_t>(batch) * channels * spatial * elem_bytes(dtype),
+                              gamma, (bc_gamma ? 1 : batch) * channels * sizeof(float), beta,
+                              (bc_beta ? 1 : batch) * channels * sizeof(float), mean, var,
+                              static_cast<size_t>(batch) * channels * sizeof(float)))
+    return e;
   p.x = x;
   p.out = y;
   p.gamma = gamma;

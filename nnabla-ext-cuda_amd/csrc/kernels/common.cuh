@@ -4,6 +4,13 @@
 // and Welford/Chan merging.  gfx950 only: a wavefront is 64 lanes.
 #pragma once
 
+// The kernels assume the CDNA4 part they are tuned for: 64-lane waves, 160 KB of
+// LDS per workgroup (the on-chip layouts declare up to 147 KB statically), 512
+// vector registers per SIMD lane.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "nblahip kernels are written for gfx950 (MI355X); build with ARCH=gfx950"
+#endif
+
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 #include <stdint.h>

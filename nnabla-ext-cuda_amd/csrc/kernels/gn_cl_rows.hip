@@ -216,6 +216,13 @@ int run_wide(bool instance, int tpr, int nl, const GnClArgs &a, hipStream_t st) 
   WIDE_CASE(4, 1024)
   WIDE_CASE(8, 1024)
 #undef WIDE_CASE
+  // 16 vectors per thread: GroupNormalization only (the instance kernel keeps
+  // 8 statistics per thread beside its vectors and would spill)
+  if (nl == 16 && tpr == 1024 && !instance) {
+    NBLAHIP_LAUNCH("gn_cl_wide_fwd_kernel", (gn_cl_wide_fwd_kernel<__half, 8, 16, 1024, W>),
+                   dim3(grid_of(a)), dim3(1024), 0, st, a);
+    return last_launch_status();
+  }
   return NBLAHIP_EINVAL;
 }
 
@@ -234,10 +241,17 @@ bool wide_fwd(const ClProblem &p, bool aligned, hipStream_t st, int *status) {
   for (int w : {4, 2}) {
     if (per_sample % w != 0 || cvg * w > 8) continue;
     const int64_t blocks = p.batch * (per_sample / w);
-    if (blocks < device_cus()) continue;
     const int64_t nv = p.spatial * cvg * w; // vectors a block holds
+    // A block for every CU, except where four groups of a long plane (16
+    // vectors per thread, GroupNormalization only) leave one for every other
+    // CU: 64-byte pieces from half the CUs beat 32-byte pieces from all of them
+    // ([16,64,64,256] G=32: 19.0 -> 17.8 us).
+    const bool long_tile = w == 4 && !instance && nv > 8192;
+    if (blocks * 100 < static_cast<int64_t>(device_cus()) * tune_int("GN_CL_WIDE_MIN_PCT", long_tile ? 50 : 100))
+      continue;
     for (int tpr : {512, 1024}) {
-      for (int nl : {4, 8}) {
+      for (int nl : {4, 8, 16}) {
+        if (nl == 16 && (tpr != 1024 || instance)) continue;
         if (static_cast<int64_t>(tpr) * nl < nv) continue;
         GnClArgs a{};
         a.x = p.x;

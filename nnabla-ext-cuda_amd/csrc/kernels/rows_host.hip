@@ -333,7 +333,7 @@ static int stream_ln_colgrad_t(const RowProblem &p, const RowArgs &a, hipStream_
                  static_cast<const T *>(p.x), static_cast<const T *>(p.dy), p.mean, p.var, a.rows,
                  a.R, rpc, p.eps, part);
   if (int e = last_launch_status()) return e;
-  NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 31) / 32),
+  NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 15) / 16),
                  dim3(1024), 0, st, part, Y, a.R, p.dgamma, p.dbeta, p.accum_g, p.accum_b);
   return last_launch_status();
 }
@@ -473,7 +473,7 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
       const int grid = ln_bwd_grid(p.rows, cfg.tpr, resident > 0 ? resident : 2);
       if (int e = run_row_bwd_cached_ln(p.dtype, cfg, a, grid, st)) return e;
       if (p.dgamma || p.dbeta) {
-        NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 31) / 32), dim3(1024), 0, st,
+        NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 15) / 16), dim3(1024), 0, st,
                            static_cast<const float *>(p.ws), grid, a.R, p.dgamma, p.dbeta,
                            p.accum_g, p.accum_b);
         if (int e = last_launch_status()) return e;

@@ -367,38 +367,41 @@ ln_colgrad_stream_kernel(const T *__restrict__ x, const T *__restrict__ dy,
 // ---------------------------------------------------------------------------
 // Second stage of the LayerNormalization parameter gradients: column sums of
 // the per-block partials ws[nparts][2][R] -> dgamma[R], dbeta[R].
-// Block = 32 columns x 32 part groups; every thread issues its (up to 8 per
-// batch) independent 128-byte-coalesced loads before adding, so the whole
-// fold costs a few load latencies.
+// Block = 16 columns x 64 part groups: up to 512 partials are one batch of 8
+// independent loads per thread (one memory round trip), a 64-byte run per
+// part, and 2R/16 blocks spread the fold over the chip.  The fold order is
+// fixed: parts py, py+64, ... per thread, lanes by butterfly, waves in order.
 // ---------------------------------------------------------------------------
 __global__ void __launch_bounds__(1024)
 ln_param_reduce_kernel(const float *__restrict__ ws, int nparts, int R,
                        float *__restrict__ dgamma, float *__restrict__ dbeta,
                        int accum_g, int accum_b) {
-  __shared__ float red[32][33];
-  const int cx = threadIdx.x & 31;
-  const int py = threadIdx.x >> 5;
-  const int col2 = blockIdx.x * 32 + cx; // column in the [2R] concatenation
+  __shared__ float red[16][16];
+  const int cx = threadIdx.x & 15;
+  const int py = threadIdx.x >> 4;
+  const int wave = threadIdx.x >> 6;
+  const int col2 = blockIdx.x * 16 + cx; // column in the [2R] concatenation
+  const bool live = col2 < 2 * R;
   const size_t stride = 2 * static_cast<size_t>(R);
   float s = 0.f;
-  if (col2 < 2 * R) {
-    for (int p0 = py; p0 < nparts; p0 += 32 * 8) {
-      float v[8];
+  for (int p0 = py; p0 < nparts; p0 += 64 * 8) {
+    float v[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int p = p0 + 32 * u;
-        v[u] = (p < nparts) ? ws[static_cast<size_t>(p) * stride + col2] : 0.f;
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u) s += v[u];
+    for (int u = 0; u < 8; ++u) {
+      const int p = p0 + 64 * u;
+      v[u] = (live && p < nparts) ? ws[static_cast<size_t>(p) * stride + col2] : 0.f;
     }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s += v[u];
   }
-  red[py][cx] = s;
+  s += __shfl_xor(s, 16);
+  s += __shfl_xor(s, 32);
+  if ((threadIdx.x & 63) < 16) red[wave][cx] = s;
   lds_barrier();
-  if (py == 0 && col2 < 2 * R) {
+  if (threadIdx.x < 16 && live) {
     float tot = 0.f;
 #pragma unroll
-    for (int i = 0; i < 32; ++i) tot += red[i][cx];
+    for (int i = 0; i < 16; ++i) tot += red[i][cx];
     if (col2 < R) {
       if (dgamma) dgamma[col2] = tot + (accum_g ? dgamma[col2] : 0.f);
     } else {

@@ -1,5 +1,6 @@
 // Runtime shims of the C-ABI (device management, memory, dtype conversion)
 // and the small host utilities shared by the launch code.
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -70,7 +71,7 @@ struct ProfRecord {
 };
 struct ProfState {
   std::mutex mu;
-  bool enabled = false;
+  std::atomic<bool> enabled{false}; // read by launching threads without the lock
   std::vector<ProfRecord> records; // pool, events pre-created
   size_t used = 0;
   size_t dropped = 0;
@@ -78,7 +79,7 @@ struct ProfState {
 } // namespace
 
 bool prof_acquire(const char *tag, hipEvent_t *start, hipEvent_t *stop) {
-  if (!g_prof.enabled) return false;
+  if (!g_prof.enabled.load(std::memory_order_acquire)) return false;
   std::lock_guard<std::mutex> lock(g_prof.mu);
   if (g_prof.used >= g_prof.records.size()) {
     ++g_prof.dropped;

@@ -58,3 +58,26 @@ def test_argument_validation_needs_no_gpu():
     assert L.nblahip_bn_fwd_infer(None, None, None, None, None, None, 4, 4, 4, 1e-5, 9, None) == -1
     assert L.nblahip_ln_fwd(None, None, None, None, None, None, 0, 4, 1e-5, 0, None) == 0
     assert L.nblahip_convert(None, 0, None, 1, 0, None) == 0
+
+
+def test_row_forwards_reject_an_output_that_overlaps_an_input():
+    """y may be x itself; any other overlap with x, the parameters or the
+    statistics is refused from the pointer ranges alone (no device access)."""
+    L = K.lib()
+    base = 0x7f0000000000                      # never dereferenced
+    n_ln, r_ln = 64, 256                       # fp32: 65536 bytes
+    x, far = base, base + (1 << 24)
+    g, b, m, v = far, far + 4096, far + 8192, far + 12288
+
+    def ln(y, gamma=g, beta=b, mean=m, var=v):
+        return L.nblahip_ln_fwd(x, gamma, beta, y, mean, var, n_ln, r_ln, 1e-5, 0, None)
+
+    assert ln(x + 1024) == -4 and ln(x - 1024) == -4 and ln(x + 65532) == -4
+    assert ln(far - 32768, gamma=far) == -4     # y runs into gamma
+    assert ln(x + (1 << 20), mean=x + (1 << 20) + 100) == -4
+    assert "overlaps" in L.nblahip_error_string(-4).decode()
+    gn = lambda y: L.nblahip_gn_fwd(x, g, b, y, m, v, 4, 16, 64, 4, 1e-5, 1, None)   # fp16: 8192 bytes
+    assert gn(x + 4096) == -4 and gn(x - 8190) == -4
+    inn = lambda y, beta=b: L.nblahip_in_fwd(x, g, beta, y, m, v, 4, 16, 64, 1, 0, 1e-5, 1, None)
+    assert inn(x + 2) == -4
+    assert inn(far + 4096 - 8192 + 4 * 16 * 4, beta=b) == -4   # per-sample beta: 4*16 floats

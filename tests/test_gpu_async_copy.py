@@ -90,3 +90,19 @@ def test_half_storage_goes_through_the_same_path():
     vx.cast("HipCachedArray", half=True, async_flags=B.ASYNC)
     vx.cast("HipCachedArray", half=False)            # device-side conversion after the upload
     np.testing.assert_array_equal(vx.d, x.astype(np.float16).astype(np.float32))
+
+
+@pytest.mark.parametrize("dtype", ["int32", "uint8", "int64", "bool", "float64"])
+def test_device_arrays_store_every_dtype(dtype):
+    """Stored and copied without conversion, host -> device -> host, also
+    through the asynchronous path; zero() clears them."""
+    B.set_host_array_class("HipCachedHostArray")
+    rng = np.random.default_rng(5)
+    a = (rng.integers(0, 200, 5000) % (2 if dtype == "bool" else 200)).astype(dtype)
+    v = B.Variable((5000,))
+    v.set_raw(a)
+    v.cast_raw("HipCachedArray", dtype, async_flags=B.ASYNC)
+    np.testing.assert_array_equal(v.get_raw(dtype), a)
+    v.cast_raw("HipArray", dtype)
+    v.zero_data()
+    np.testing.assert_array_equal(v.get_raw(dtype), np.zeros(5000, dtype))

@@ -261,6 +261,9 @@ GRIDS = [
      ["gn_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], []),
     ("in_cl_wide_plain_block_order", run_in, (4, 1024, (32, 32), F16, True), [{"GN_CL_XCD_MAP": 0}],
      ["in_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], []),
+    # four groups per block, 16 vectors per thread, on a quarter of the CUs
+    ("gn_cl_wide_fewer_blocks", run_gn, (8, 256, (64, 64), 32, F16, True), [{"GN_CL_WIDE_MIN_PCT": 25}],
+     ["gn_cl_wide_fwd_kernel"], []),
     ("gn_cl_rows_plain_block_order", run_gn, (2, 128, (20, 20), 8, F32, True), [{"GN_CL_XCD_MAP": 0}],
      ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"], []),
     ("in_cl_rows_plain_block_order", run_in, (2, 128, (20, 20), F16, True),
