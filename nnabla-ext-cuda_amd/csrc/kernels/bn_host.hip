@@ -655,6 +655,7 @@ int launch_cl_fwd(const ClProblem &p, hipStream_t st) {
   const bool al = aligned16(p.x) && aligned16(p.out);
   {
     int status = 0;
+    if (cl_split_fwd(p, al, st, &status)) return status;
     if (gn_cl_cached_fwd(p, al, st, &status)) return status;
   }
   const BnPlan pl = make_cl_plan(p.batch, p.spatial, p.channels, p.dtype, al);
@@ -690,6 +691,15 @@ int launch_cl_bwd(const ClProblem &p, hipStream_t st) {
   const ClWs w = cl_carve(p, pl);
   {
     int status = 0;
+    float *pairs = nullptr;
+    int64_t pair_batches = 0;
+    if (cl_split_bwd(p, al, &pairs, &pair_batches, st, &status)) {
+      if (status) return status;
+      if (p.dgamma || p.dbeta)
+        return launch_pair_param_reduce("pair_param_reduce_cl_kernel", pairs, pair_batches,
+                                        p.channels, p.dgamma, p.dbeta, 1, 1, p.accum_g, p.accum_b, st);
+      return 0;
+    }
     if (gn_cl_cached_bwd(p, al, w.pairs, st, &status)) {
       if (status) return status;
       if (p.dgamma || p.dbeta)

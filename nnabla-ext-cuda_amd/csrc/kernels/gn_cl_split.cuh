@@ -1,0 +1,618 @@
+// Channel-last Group/InstanceNormalization with a reduction unit SPLIT over
+// several workgroups that exchange their partial sums.
+//
+// x is [N][P][C].  A statistics unit (a group of a sample, or one channel of a
+// sample) is a strided tile of P positions x a few channels, i.e. a 2- to
+// 128-byte piece of every 128-byte cache line it touches.  A block that owns
+// whole units therefore reads pieces of lines (gn_cl_rows.cuh), and the other
+// pieces are fetched again by the blocks that own the neighbouring units.
+//
+// Here a block owns whole LINES instead: a column tile of 8 sixteen-byte
+// vectors (128 bytes: 64 half or 32 float channels, all the units inside it)
+// over PB consecutive positions.  The `split` blocks that cover the P positions
+// of one (sample, column tile) each reduce their part in registers, publish the
+// partial sums of every unit in the tile, read the partials of their partner
+// blocks, merge all of them in the same fixed order (every block arrives at
+// bit-identical statistics) and finish their part from registers: one pass
+// over HBM per direction, in whole lines, with many small blocks per CU.
+//
+// The exchange needs no barrier, no fence and no zeroed memory: a partial is
+// one 64-bit word {value, epoch} written and read with relaxed device-scope
+// atomics.  `epoch` is unique per call (the exchange array lives in the
+// library, starts zeroed and only ever holds such words), so a word either
+// carries this call's epoch - then its value is the partner's partial - or it
+// does not count.  A block polls each word at most `spin` times.  If a partner
+// has not published by then (it has not been scheduled yet, or another call
+// overwrote the slot), the block computes that partner's partial itself from
+// global memory: every wave reaches the end of the kernel whatever the other
+// blocks do, and the result is correct either way.
+#pragma once
+
+#include "common.cuh"
+#include "launch.hpp"
+
+namespace nblahip {
+
+constexpr int kSplitTV = 8;    // 16-byte vectors per column tile (one 128-byte line per position)
+constexpr int kSplitMax = 16;  // most blocks per (sample, column tile)
+
+struct ClSplitArgs {
+  const void *x;
+  const void *dy; // backward
+  void *out;      // y or dx (dx may be null)
+  const float *gamma;
+  const float *beta;
+  float *mean; // forward: written, backward: read; [N * C / cpg]
+  float *var;
+  const float *dmean;
+  const float *dvar;
+  float *pairs;             // backward: [N * split][C][2] = (sum dy*xh, sum dy) per block and channel
+  unsigned long long *xchg; // this call's exchange words
+  uint32_t epoch;
+  int spin;  // polls per exchange word before the partner's part is recomputed
+  int P, C;
+  int tiles; // column tiles per position = C * sizeof(T) / 128
+  int split; // blocks per (sample, column tile)
+  int PB;    // positions per block = NL * TPR / 8
+  int cpg;   // channels per unit (1: instances)
+  int cvg_shift; // log2 of the vectors per unit (groups only)
+  float eps, inv_R, one;
+  int accum_dx;
+};
+
+__device__ __forceinline__ unsigned long long split_pack(float v, uint32_t epoch) {
+  return (static_cast<unsigned long long>(epoch) << 32) | __float_as_uint(v);
+}
+
+__device__ __forceinline__ void split_publish(unsigned long long *slot, float v, uint32_t epoch) {
+  __hip_atomic_store(slot, split_pack(v, epoch), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Polls the partner words this thread is responsible for into part[]; words
+// that do not turn up mark their block in missing[].
+template <int TPR>
+__device__ __forceinline__ void split_collect(const ClSplitArgs &a, const unsigned long long *base,
+                                              uint32_t self, int per, float *part, int *missing) {
+  const int total = a.split * per;
+  for (int idx = threadIdx.x; idx < total; idx += TPR) {
+    const int sp = idx / per;
+    if (sp == static_cast<int>(self)) continue;
+    bool ok = false;
+    unsigned long long w = 0;
+    for (int it = 0; it < a.spin; ++it) {
+      w = __hip_atomic_load(base + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (static_cast<uint32_t>(w >> 32) == a.epoch) {
+        ok = true;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(8);
+    }
+    if (ok) {
+      part[idx] = __uint_as_float(static_cast<uint32_t>(w));
+    } else {
+      missing[sp] = 1;
+    }
+  }
+}
+
+// Sum of v over the threads of the block that hold the same unit of the tile
+// (groups: the 2^cvg_shift neighbouring vectors of a position; every thread of
+// a unit receives the total).  fold: [TPR / 64][8].
+template <int TPR>
+__device__ __forceinline__ float split_group_sum(float v, int cvg_shift, uint32_t cvx, uint32_t gi,
+                                                 float (*fold)[kSplitTV]) {
+  constexpr int NW = TPR / kWave;
+  for (int off = 1; off < (1 << cvg_shift); off <<= 1) v += __shfl_xor(v, off);
+  v += __shfl_xor(v, 8);
+  v += __shfl_xor(v, 16);
+  v += __shfl_xor(v, 32);
+  lds_barrier(); // earlier readers of fold are done
+  if ((threadIdx.x & (kWave - 1)) < kSplitTV && (cvx & ((1u << cvg_shift) - 1)) == 0)
+    fold[threadIdx.x / kWave][gi] = v;
+  lds_barrier();
+  float t = 0.f;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) t += fold[w][gi];
+  return t;
+}
+
+// The same for VEC per-channel values of a thread (instances; channel-wise
+// sums of the backward): threads with equal cvx hold the same channels.
+// fold: [TPR / 64][8 * VEC]; out[j] = total of channel cvx * VEC + j.
+template <int TPR, int VEC>
+__device__ __forceinline__ void split_channel_sums(float (&v)[VEC], uint32_t cvx,
+                                                   float (*fold)[kSplitTV * VEC]) {
+  constexpr int NW = TPR / kWave;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    v[j] += __shfl_xor(v[j], 8);
+    v[j] += __shfl_xor(v[j], 16);
+    v[j] += __shfl_xor(v[j], 32);
+  }
+  lds_barrier();
+  if ((threadIdx.x & (kWave - 1)) < kSplitTV) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) fold[threadIdx.x / kWave][cvx * VEC + j] = v[j];
+  }
+  lds_barrier();
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    float t = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) t += fold[w][cvx * VEC + j];
+    v[j] = t;
+  }
+}
+
+__device__ __forceinline__ float split_count(const ClSplitArgs &a, int sp) {
+  const int left = a.P - sp * a.PB;
+  return static_cast<float>(left < a.PB ? left : a.PB);
+}
+
+// Chan merge of the (mean, m2) partials of one unit over the blocks, in block
+// order; counts follow from the geometry.  Returns mean, var (biased).
+__device__ __forceinline__ void split_merge_stats(const ClSplitArgs &a, const float *part, int per,
+                                                  int u, float per_pos, float &mean, float &var) {
+  float m = part[u * 2], m2 = part[u * 2 + 1], n = split_count(a, 0) * per_pos;
+  for (int sp = 1; sp < a.split; ++sp) {
+    const float nb = split_count(a, sp) * per_pos;
+    const float mb = part[sp * per + u * 2], qb = part[sp * per + u * 2 + 1];
+    const float tot = n + nb;
+    const float d = mb - m;
+    const float wgt = nb / tot;
+    m = fmaf(d, wgt, m);
+    m2 = m2 + qb + d * d * (n * wgt);
+    n = tot;
+  }
+  mean = m;
+  var = m2 * a.inv_R;
+}
+
+// ---------------------------------------------------------------------------
+// Forward.  Block b = ((n * split + s) * tiles + tile); thread t owns vector
+// t % 8 of the tile at positions s * PB + t / 8 + k * (TPR / 8), k < NL.
+// ---------------------------------------------------------------------------
+template <typename T, int VEC, int NL, int TPR, bool INSTANCE>
+__global__ void __launch_bounds__(TPR)
+cl_split_fwd_kernel(const ClSplitArgs a) {
+  constexpr int TV = kSplitTV;
+  constexpr int PR = TPR / TV;
+  constexpr int NW = TPR / kWave;
+  constexpr int UMAX = INSTANCE ? TV * VEC : TV;
+  __shared__ float fold[NW][UMAX];
+  __shared__ float part[kSplitMax * UMAX * 2];
+  __shared__ int missing[kSplitMax];
+  const uint32_t tile = blockIdx.x % a.tiles, ns = blockIdx.x / a.tiles;
+  const uint32_t s = ns % a.split, n = ns / a.split;
+  const uint32_t cvx = threadIdx.x % TV, prow = threadIdx.x / TV;
+  const uint32_t ch = (tile * TV + cvx) * VEC;
+  const uint32_t gi = INSTANCE ? 0u : (cvx >> a.cvg_shift);
+  const int U = INSTANCE ? TV * VEC : (TV >> a.cvg_shift); // units in the tile
+  const int per = 2 * U;
+  const float per_pos = INSTANCE ? 1.f : static_cast<float>(a.cpg);
+  const T *__restrict__ x = static_cast<const T *>(a.x) + static_cast<size_t>(n) * a.P * a.C + ch;
+  T *__restrict__ y = static_cast<T *>(a.out) + static_cast<size_t>(n) * a.P * a.C + ch;
+  unsigned long long *slots =
+      a.xchg + (static_cast<size_t>(n) * a.tiles + tile) * a.split * per;
+  const bool writer = prow == 0 && (INSTANCE || (cvx & ((1u << a.cvg_shift) - 1)) == 0);
+
+  if (threadIdx.x < kSplitMax) missing[threadIdx.x] = 0;
+  RawVec<T, VEC> raw[NL];
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = s * a.PB + prow + k * PR;
+    const bool ok = pos < static_cast<uint32_t>(a.P);
+    raw[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + static_cast<size_t>(ok ? pos : s * a.PB) * a.C));
+  }
+  float gam[VEC], bet[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    gam[j] = a.gamma ? a.gamma[ch + j] : 1.f;
+    bet[j] = a.beta ? a.beta[ch + j] : 0.f;
+  }
+
+  float mean[INSTANCE ? VEC : 1], var[INSTANCE ? VEC : 1];
+  if constexpr (!INSTANCE) {
+    // ---- this block's part: mean, then the second moment about it
+    float sum = 0.f;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) sum = raw_sum<T, VEC>(raw[k], sum);
+    const float cnt = split_count(a, s) * per_pos;
+    const float m = split_group_sum<TPR>(sum, a.cvg_shift, cvx, gi, fold) / cnt;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+    float q = 0.f;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      if (s * a.PB + prow + k * PR < static_cast<uint32_t>(a.P)) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float d = elem_fma<T, VEC>(raw[k], j, a.one, -m);
+          q = fmaf(d, d, q);
+        }
+      }
+    }
+    q = split_group_sum<TPR>(q, a.cvg_shift, cvx, gi, fold);
+    if (writer) {
+      part[s * per + gi * 2] = m;
+      part[s * per + gi * 2 + 1] = q;
+      split_publish(slots + s * per + gi * 2, m, a.epoch);
+      split_publish(slots + s * per + gi * 2 + 1, q, a.epoch);
+    }
+  } else {
+    float sum[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) sum[j] = 0.f;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) sum[j] = elem_fma<T, VEC>(raw[k], j, a.one, sum[j]);
+    }
+    split_channel_sums<TPR, VEC>(sum, cvx, fold);
+    const float icnt = 1.0f / split_count(a, s);
+    float m[VEC], q[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      m[j] = sum[j] * icnt;
+      q[j] = 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      if (s * a.PB + prow + k * PR < static_cast<uint32_t>(a.P)) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float d = elem_fma<T, VEC>(raw[k], j, a.one, -m[j]);
+          q[j] = fmaf(d, d, q[j]);
+        }
+      }
+    }
+    split_channel_sums<TPR, VEC>(q, cvx, fold);
+    if (writer) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const int u = cvx * VEC + j;
+        part[s * per + u * 2] = m[j];
+        part[s * per + u * 2 + 1] = q[j];
+        split_publish(slots + s * per + u * 2, m[j], a.epoch);
+        split_publish(slots + s * per + u * 2 + 1, q[j], a.epoch);
+      }
+    }
+  }
+
+  // ---- the partners' parts
+  split_collect<TPR>(a, slots, s, per, part, missing);
+  lds_barrier();
+  for (int sp = 0; sp < a.split; ++sp) {
+    if (sp == static_cast<int>(s) || !missing[sp]) continue; // same answer in every thread
+    // Partner sp has not published: its part from global memory, one vector
+    // at a time (the block's own vectors stay in registers).
+    const float cnt = split_count(a, sp);
+    if constexpr (!INSTANCE) {
+      float sum = 0.f;
+#pragma unroll 1
+      for (int k = 0; k < NL; ++k) {
+        const uint32_t pos = sp * a.PB + prow + k * PR;
+        const bool ok = pos < static_cast<uint32_t>(a.P);
+        const RawVec<T, VEC> r = raw_or_zero<T, VEC>(
+            ok, load_raw<T, VEC>(x + static_cast<size_t>(ok ? pos : sp * a.PB) * a.C));
+        sum = raw_sum<T, VEC>(r, sum);
+      }
+      const float m = split_group_sum<TPR>(sum, a.cvg_shift, cvx, gi, fold) / (cnt * per_pos);
+      float q = 0.f;
+#pragma unroll 1
+      for (int k = 0; k < NL; ++k) {
+        const uint32_t pos = sp * a.PB + prow + k * PR;
+        if (pos < static_cast<uint32_t>(a.P)) {
+          const RawVec<T, VEC> r = load_raw<T, VEC>(x + static_cast<size_t>(pos) * a.C);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            const float d = elem_fma<T, VEC>(r, j, a.one, -m);
+            q = fmaf(d, d, q);
+          }
+        }
+      }
+      q = split_group_sum<TPR>(q, a.cvg_shift, cvx, gi, fold);
+      if (writer) {
+        part[sp * per + gi * 2] = m;
+        part[sp * per + gi * 2 + 1] = q;
+      }
+    } else {
+      float sum[VEC], m[VEC], q[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) sum[j] = 0.f;
+#pragma unroll 1
+      for (int k = 0; k < NL; ++k) {
+        const uint32_t pos = sp * a.PB + prow + k * PR;
+        const bool ok = pos < static_cast<uint32_t>(a.P);
+        const RawVec<T, VEC> r = raw_or_zero<T, VEC>(
+            ok, load_raw<T, VEC>(x + static_cast<size_t>(ok ? pos : sp * a.PB) * a.C));
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) sum[j] = elem_fma<T, VEC>(r, j, a.one, sum[j]);
+      }
+      split_channel_sums<TPR, VEC>(sum, cvx, fold);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        m[j] = sum[j] / cnt;
+        q[j] = 0.f;
+      }
+#pragma unroll 1
+      for (int k = 0; k < NL; ++k) {
+        const uint32_t pos = sp * a.PB + prow + k * PR;
+        if (pos < static_cast<uint32_t>(a.P)) {
+          const RawVec<T, VEC> r = load_raw<T, VEC>(x + static_cast<size_t>(pos) * a.C);
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            const float d = elem_fma<T, VEC>(r, j, a.one, -m[j]);
+            q[j] = fmaf(d, d, q[j]);
+          }
+        }
+      }
+      split_channel_sums<TPR, VEC>(q, cvx, fold);
+      if (writer) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          part[sp * per + (cvx * VEC + j) * 2] = m[j];
+          part[sp * per + (cvx * VEC + j) * 2 + 1] = q[j];
+        }
+      }
+    }
+    lds_barrier();
+  }
+
+  // ---- merge in block order, write the statistics (first block), normalize
+  if constexpr (!INSTANCE) {
+    split_merge_stats(a, part, per, gi, per_pos, mean[0], var[0]);
+    if (s == 0 && writer) {
+      const size_t u = static_cast<size_t>(n) * (a.C / a.cpg) + (tile * TV * VEC) / a.cpg + gi;
+      a.mean[u] = mean[0];
+      a.var[u] = var[0];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) split_merge_stats(a, part, per, cvx * VEC + j, 1.f, mean[j], var[j]);
+    if (s == 0 && writer) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        a.mean[static_cast<size_t>(n) * a.C + ch + j] = mean[j];
+        a.var[static_cast<size_t>(n) * a.C + ch + j] = var[j];
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+  float sc[VEC], sh[VEC], mu[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    const int ju = INSTANCE ? j : 0;
+    sc[j] = gam[j] * inv_std(var[ju], a.eps);
+    mu[j] = mean[ju];
+    sh[j] = fmaf(-mean[ju], sc[j], bet[j]);
+  }
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = s * a.PB + prow + k * PR;
+    if (pos < static_cast<uint32_t>(a.P)) {
+      float o[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        if constexpr (sizeof(T) == 2) {
+          o[j] = elem_fma<T, VEC>(raw[k], j, sc[j], sh[j]);
+        } else {
+          o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mu[j]), sc[j], bet[j]);
+        }
+      }
+      store_vec<T, VEC>(y + static_cast<size_t>(pos) * a.C, o);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Backward.  With xh = (x-mean)*istd, per unit: s1 = sum gamma*dy,
+// t2 = sum gamma*dy*xh (over the unit's channels and all positions),
+//   cA = -istd*t2/R + 2*dvar*std/R,  cb = -s1*istd/R + dmean/R,
+//   dx = gamma*istd*dy + cA*xh + cb
+// (gn_cl_row_bwd_kernel / in_cl_row_bwd_kernel).  A block reduces the
+// per-channel pairs (sum dy*xh, sum dy) of its positions, stores them for the
+// batch sum behind dgamma/dbeta as "sample" n * split + s, publishes the
+// partial (t2, s1) of each unit, collects its partners' and writes its dx.
+// x stays in registers, dy is parked in LDS (each thread reads back what it
+// wrote): both in registers cost more than the 128 a thread may use with two
+// blocks of 512 on a CU.
+// ---------------------------------------------------------------------------
+template <typename T, int VEC, int NL, int TPR, bool INSTANCE>
+__global__ void __launch_bounds__(TPR, 4)
+cl_split_bwd_kernel(const ClSplitArgs a) {
+  constexpr int TV = kSplitTV;
+  constexpr int PR = TPR / TV;
+  constexpr int NW = TPR / kWave;
+  constexpr int CH = TV * VEC; // channels of the tile
+  constexpr int UMAX = INSTANCE ? CH : TV;
+  constexpr int SV = INSTANCE ? VEC : 1; // statistics units of a thread's vector
+  __shared__ RawVec<T, VEC> park[NL * TPR];
+  __shared__ float fold[NW][CH];
+  __shared__ float chs[2][CH]; // [0]: sum dy*xh, [1]: sum dy per channel of the tile
+  __shared__ float part[kSplitMax * UMAX * 2];
+  __shared__ int missing[kSplitMax];
+  const uint32_t tile = blockIdx.x % a.tiles, ns = blockIdx.x / a.tiles;
+  const uint32_t s = ns % a.split, n = ns / a.split;
+  const uint32_t cvx = threadIdx.x % TV, prow = threadIdx.x / TV;
+  const uint32_t ch0 = tile * CH, ch = ch0 + cvx * VEC;
+  const uint32_t gi = INSTANCE ? 0u : (cvx >> a.cvg_shift);
+  const int U = INSTANCE ? CH : (TV >> a.cvg_shift);
+  const int per = 2 * U;
+  const size_t slab = static_cast<size_t>(n) * a.P * a.C + ch;
+  const T *__restrict__ x = static_cast<const T *>(a.x) + slab;
+  const T *__restrict__ dy = static_cast<const T *>(a.dy) + slab;
+  T *__restrict__ dx = a.out ? static_cast<T *>(a.out) + slab : nullptr;
+  unsigned long long *slots =
+      a.xchg + (static_cast<size_t>(n) * a.tiles + tile) * a.split * per;
+  // statistics index of this thread's first unit
+  const size_t stat = INSTANCE ? static_cast<size_t>(n) * a.C + ch
+                               : static_cast<size_t>(n) * (a.C / a.cpg) + ch0 / a.cpg + gi;
+
+  if (threadIdx.x < kSplitMax) missing[threadIdx.x] = 0;
+  RawVec<T, VEC> xr[NL];
+  {
+    RawVec<T, VEC> dr[NL];
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const uint32_t pos = s * a.PB + prow + k * PR;
+      const bool ok = pos < static_cast<uint32_t>(a.P);
+      const size_t off = static_cast<size_t>(ok ? pos : s * a.PB) * a.C;
+      xr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + off));
+      dr[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(dy + off));
+    }
+#pragma unroll
+    for (int k = 0; k < NL; ++k) park[k * TPR + threadIdx.x] = dr[k];
+  }
+  float mean[SV], istd[SV], nmi[SV];
+#pragma unroll
+  for (int j = 0; j < SV; ++j) {
+    mean[j] = a.mean[stat + j];
+    istd[j] = 1.0f / sqrtf(a.var[stat + j] + a.eps);
+    nmi[j] = -mean[j] * istd[j];
+  }
+
+  // chs -> the partial (t2, s1) of every unit of the tile, into part[sp]
+  auto unit_partials = [&](uint32_t sp, bool publish) {
+    for (int e = threadIdx.x; e < per; e += TPR) {
+      const int u = e >> 1, w = e & 1; // w = 0: t2 (from sum dy*xh), 1: s1 (from sum dy)
+      float v;
+      if constexpr (INSTANCE) {
+        v = chs[w][u];
+      } else {
+        v = 0.f;
+        for (int c = 0; c < a.cpg; ++c) {
+          const float gc = a.gamma ? a.gamma[ch0 + u * a.cpg + c] : 1.f;
+          v = fmaf(gc, chs[w][u * a.cpg + c], v);
+        }
+      }
+      part[sp * per + e] = v;
+      if (publish) split_publish(slots + sp * per + e, v, a.epoch);
+    }
+  };
+
+  // ---- this block's positions (own LDS entries only: no barrier needed before)
+  {
+    float sdx[VEC], sdy[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) sdx[j] = sdy[j] = 0.f;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const RawVec<T, VEC> dv = park[k * TPR + threadIdx.x];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const int ju = INSTANCE ? j : 0;
+        const float xh = norm_elem<T, VEC>(xr[k], j, mean[ju], istd[ju], nmi[ju]);
+        sdx[j] = elem_fma<T, VEC>(dv, j, xh, sdx[j]);
+        sdy[j] = elem_fma<T, VEC>(dv, j, a.one, sdy[j]);
+      }
+    }
+    split_channel_sums<TPR, VEC>(sdx, cvx, fold);
+    split_channel_sums<TPR, VEC>(sdy, cvx, fold);
+    if (prow == 0) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        chs[0][cvx * VEC + j] = sdx[j];
+        chs[1][cvx * VEC + j] = sdy[j];
+      }
+    }
+    lds_barrier();
+    if (a.pairs) {
+      for (int e = threadIdx.x; e < 2 * CH; e += TPR) {
+        const int c = e >> 1, w = e & 1;
+        a.pairs[2 * ((static_cast<size_t>(n) * a.split + s) * a.C + ch0 + c) + w] = chs[w][c];
+      }
+    }
+    unit_partials(s, true);
+  }
+  if (dx == nullptr) return;
+
+  // ---- the partners' parts
+  split_collect<TPR>(a, slots, s, per, part, missing);
+  lds_barrier();
+  for (int sp = 0; sp < a.split; ++sp) {
+    if (sp == static_cast<int>(s) || !missing[sp]) continue; // same answer in every thread
+    // Partner sp has not published: its sums from global memory, a vector at a time.
+    float sdx[VEC], sdy[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) sdx[j] = sdy[j] = 0.f;
+#pragma unroll 1
+    for (int k = 0; k < NL; ++k) {
+      const uint32_t pos = sp * a.PB + prow + k * PR;
+      const bool ok = pos < static_cast<uint32_t>(a.P);
+      const size_t off = static_cast<size_t>(ok ? pos : sp * a.PB) * a.C;
+      const RawVec<T, VEC> xv = load_raw<T, VEC>(x + off);
+      const RawVec<T, VEC> dv = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(dy + off));
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const int ju = INSTANCE ? j : 0;
+        const float xh = norm_elem<T, VEC>(xv, j, mean[ju], istd[ju], nmi[ju]);
+        sdx[j] = elem_fma<T, VEC>(dv, j, xh, sdx[j]);
+        sdy[j] = elem_fma<T, VEC>(dv, j, a.one, sdy[j]);
+      }
+    }
+    split_channel_sums<TPR, VEC>(sdx, cvx, fold);
+    split_channel_sums<TPR, VEC>(sdy, cvx, fold);
+    if (prow == 0) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        chs[0][cvx * VEC + j] = sdx[j];
+        chs[1][cvx * VEC + j] = sdy[j];
+      }
+    }
+    lds_barrier();
+    unit_partials(static_cast<uint32_t>(sp), false);
+    lds_barrier();
+  }
+
+  // ---- totals in block order, dx
+#pragma unroll
+  for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(xr[k]);
+  float gis[VEC], cA[SV], cb[SV];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) gis[j] = (a.gamma ? a.gamma[ch + j] : 1.f) * istd[INSTANCE ? j : 0];
+#pragma unroll
+  for (int j = 0; j < SV; ++j) {
+    const int u = INSTANCE ? static_cast<int>(cvx) * VEC + j : static_cast<int>(gi);
+    float t2 = 0.f, s1 = 0.f;
+    for (int sp = 0; sp < a.split; ++sp) {
+      t2 += part[sp * per + u * 2];
+      s1 += part[sp * per + u * 2 + 1];
+    }
+    if constexpr (INSTANCE) { // the exchanged sums are per channel, without gamma
+      const float g = a.gamma ? a.gamma[ch + j] : 1.f;
+      t2 *= g;
+      s1 *= g;
+    }
+    const float vpe = a.var[stat + j] + a.eps;
+    cA[j] = -istd[j] * t2 * a.inv_R + (a.dvar ? 2.f * a.dvar[stat + j] * (vpe * istd[j]) * a.inv_R : 0.f);
+    cb[j] = -s1 * istd[j] * a.inv_R + (a.dmean ? a.dmean[stat + j] * a.inv_R : 0.f);
+  }
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = s * a.PB + prow + k * PR;
+    if (pos < static_cast<uint32_t>(a.P)) {
+      const RawVec<T, VEC> dv = park[k * TPR + threadIdx.x];
+      float o[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const int ju = INSTANCE ? j : 0;
+        const float xh = norm_elem<T, VEC>(xr[k], j, mean[ju], istd[ju], nmi[ju]);
+        o[j] = elem_fma<T, VEC>(dv, j, gis[j], fmaf(xh, cA[ju], cb[ju]));
+      }
+      T *p = dx + static_cast<size_t>(pos) * a.C;
+      if (a.accum_dx) {
+        float old[VEC];
+        load_vec<T, VEC>(p, old);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) o[j] += old[j];
+      }
+      store_vec<T, VEC>(p, o);
+    }
+  }
+}
+
+} // namespace nblahip

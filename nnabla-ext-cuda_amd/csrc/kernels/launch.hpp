@@ -198,6 +198,12 @@ struct ClProblem {
 // leaves the per-(n, channel) pairs in `pairs` for the batch sum.
 bool gn_cl_cached_fwd(const ClProblem &p, bool aligned, hipStream_t st, int *status);
 bool gn_cl_cached_bwd(const ClProblem &p, bool aligned, float *pairs, hipStream_t st, int *status);
+// Split channel-last kernels (gn_cl_split.hip): a block owns whole 128-byte
+// lines of a position range, the blocks of a sample exchange partial sums.  The
+// backward leaves per-block pairs in the workspace: *pairs is [*pair_batches][C][2].
+bool cl_split_fwd(const ClProblem &p, bool aligned, hipStream_t st, int *status);
+bool cl_split_bwd(const ClProblem &p, bool aligned, float **pairs, int64_t *pair_batches,
+                  hipStream_t st, int *status);
 int launch_cl_fwd(const ClProblem &p, hipStream_t st);
 int launch_cl_bwd(const ClProblem &p, hipStream_t st);
 size_t cl_workspace_bytes(int64_t batch, int64_t spatial, int64_t channels, int dtype);

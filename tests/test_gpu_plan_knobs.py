@@ -122,6 +122,11 @@ def run_in(n, c, sp, dtype, channel_last=False, seed=4):
     assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
 
 
+# GroupNormalization rows about the channel-last kernels that own whole groups
+# run with the split kernels (which take those shapes by default) switched off.
+NO_SPLIT = {"GN_CL_SPLIT": 0}
+
+
 def kernels_of(run, args, knobs):
     """Runs `run(*args)` (with its oracle checks) under `knobs`; returns the
     names of the kernels the library launched."""
@@ -187,15 +192,23 @@ SWITCHES = [
     ("in_rows_onchip_bwd_min_pct_up", run_in, (2, 64, (256, 256), F32), {"ROW_ONCHIP_BWD_MIN_PCT": 100},
      ["row_onchip_fwd_kernel", "plane_sums_stream_kernel"], ["bn_onchip_bwd_kernel"]),
     # channel-last GroupNormalization / InstanceNormalization
+    ("gn_cl_split_off", run_gn, (4, 1024, (32, 32), 128, F16, True), {"GN_CL_SPLIT": 0},
+     ["gn_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], ["cl_split_fwd_kernel", "cl_split_bwd_kernel"]),
+    ("gn_cl_split_off_float", run_gn, (2, 128, (20, 20), 8, F32, True), {"GN_CL_SPLIT": 0},
+     ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"], ["cl_split_fwd_kernel", "cl_split_bwd_kernel"]),
+    ("in_cl_split_on", run_in, (4, 1024, (32, 32), F16, True), {"GN_CL_SPLIT_INSTANCES": 1},
+     ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], ["in_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"]),
+    ("in_cl_split_on_float", run_in, (3, 64, (19, 19), F32, True), {"GN_CL_SPLIT_INSTANCES": 1},
+     ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"]),
     ("gn_cl_wide_off", run_gn, (4, 1024, (32, 32), 128, F16, True),
      {"GN_CL_WIDE": 0, "GN_CL_WIDE_BWD": 0}, ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"],
-     ["gn_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"]),
+     ["gn_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], NO_SPLIT),
     ("in_cl_wide_off", run_in, (4, 1024, (32, 32), F16, True),
      {"GN_CL_WIDE": 0, "GN_CL_WIDE_BWD": 0}, ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"],
      ["in_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"]),
     ("gn_cl_cached_off", run_gn, (2, 128, (20, 20), 8, F32, True), {"GN_CL_CACHED": 0},
      ["bn_stats_cl_kernel", "gn_cl_finalize_fwd_kernel", "bn_bwd_reduce_cl_kernel",
-      "gn_cl_finalize_bwd_kernel"], ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"]),
+      "gn_cl_finalize_bwd_kernel"], ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"], NO_SPLIT),
     ("in_cl_cached_off", run_in, (2, 128, (20, 20), F32, True), {"IN_CL_CACHED": 0},
      ["bn_stats_cl_kernel", "gn_cl_finalize_fwd_kernel", "gn_cl_finalize_bwd_kernel"],
      ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"]),
@@ -206,11 +219,12 @@ SWITCHES = [
 
 @pytest.mark.parametrize("case", SWITCHES, ids=[c[0] for c in SWITCHES])
 def test_plan_switch_changes_the_kernels_and_keeps_parity(case):
-    _, run, args, knobs, must_run, must_not_run = case
-    default = kernels_of(run, args, {})
+    _, run, args, knobs, must_run, must_not_run = case[:6]
+    base = case[6] if len(case) > 6 else {}
+    default = kernels_of(run, args, base)
     for name in must_not_run:
         assert name in default, f"default plan of {args} ran {default}, expected {name} among them"
-    switched = kernels_of(run, args, knobs)
+    switched = kernels_of(run, args, {**base, **knobs})
     for name in must_run:
         assert name in switched, f"{knobs}: ran {switched}, expected {name}"
     for name in must_not_run:
@@ -257,14 +271,32 @@ GRIDS = [
      ["row_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
     ("rows_onchip_streamed_few_rows", run_in, (1, 8, (512, 512), F16),
      [{"ROW_ONCHIP_STREAMED_MIN_PCT": 1}], ["row_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
-    ("gn_cl_wide_plain_block_order", run_gn, (4, 1024, (32, 32), 128, F16, True), [{"GN_CL_XCD_MAP": 0}],
+    # the split kernels: every block shape, and every partner's part recomputed
+    # because no poll is allowed (what a block does when a partner is late)
+    ("gn_cl_split_shapes", run_gn, (3, 128, (40, 40), 16, F16, True),
+     [{"GN_CL_SPLIT_TPR": t, "GN_CL_SPLIT_NL": n} for t, n in ((256, 4), (256, 8), (512, 4), (512, 8),
+                                                                (1024, 4), (1024, 8))],
+     ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], []),
+    ("gn_cl_split_shapes_float", run_gn, (2, 64, (37, 37), 8, F32, True),
+     [{"GN_CL_SPLIT_TPR": t, "GN_CL_SPLIT_NL": n} for t, n in ((256, 4), (256, 8), (512, 4), (512, 8),
+                                                                (1024, 4), (1024, 8))],
+     ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], []),
+    ("gn_cl_split_no_polls", run_gn, (3, 128, (40, 40), 16, F16, True), [{"GN_CL_SPLIT_SPIN": 0}],
+     ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], []),
+    ("in_cl_split_no_polls", run_in, (2, 64, (30, 30), F32, True),
+     [{"GN_CL_SPLIT_SPIN": 0, "GN_CL_SPLIT_INSTANCES": 1}],
+     ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], []),
+    ("gn_cl_wide_plain_block_order", run_gn, (4, 1024, (32, 32), 128, F16, True),
+     [{"GN_CL_XCD_MAP": 0, **NO_SPLIT}],
      ["gn_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], []),
     ("in_cl_wide_plain_block_order", run_in, (4, 1024, (32, 32), F16, True), [{"GN_CL_XCD_MAP": 0}],
      ["in_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], []),
     # four groups per block, 16 vectors per thread, on a quarter of the CUs
-    ("gn_cl_wide_fewer_blocks", run_gn, (8, 256, (64, 64), 32, F16, True), [{"GN_CL_WIDE_MIN_PCT": 25}],
+    ("gn_cl_wide_fewer_blocks", run_gn, (8, 256, (64, 64), 32, F16, True),
+     [{"GN_CL_WIDE_MIN_PCT": 25, **NO_SPLIT}],
      ["gn_cl_wide_fwd_kernel"], []),
-    ("gn_cl_rows_plain_block_order", run_gn, (2, 128, (20, 20), 8, F32, True), [{"GN_CL_XCD_MAP": 0}],
+    ("gn_cl_rows_plain_block_order", run_gn, (2, 128, (20, 20), 8, F32, True),
+     [{"GN_CL_XCD_MAP": 0, **NO_SPLIT}],
      ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"], []),
     ("in_cl_rows_plain_block_order", run_in, (2, 128, (20, 20), F16, True),
      [{"GN_CL_XCD_MAP": 0, "GN_CL_WIDE": 0, "GN_CL_WIDE_BWD": 0}],

@@ -23,6 +23,8 @@ def test_every_knob_the_library_reads_has_a_parity_case():
     used = set()
     for case in T.SWITCHES:
         used |= set(case[3])
+        if len(case) > 6:
+            used |= set(case[6])
     for case in T.GRIDS:
         for knobs in case[3]:
             used |= set(knobs)
