@@ -16,20 +16,17 @@
 // bit-identical statistics) and finish their part from registers: one pass
 // over HBM per direction, in whole lines, with many small blocks per CU.
 //
-// The exchange needs no barrier, no fence and no zeroed memory: a partial is
-// one 64-bit word {value, epoch} written and read with relaxed device-scope
-// atomics.  `epoch` is unique per call (the exchange array lives in the
-// library, starts zeroed and only ever holds such words), so a word either
-// carries this call's epoch - then its value is the partner's partial - or it
-// does not count.  A block polls each word at most `spin` times.  If a partner
-// has not published by then (it has not been scheduled yet, or another call
-// overwrote the slot), the block computes that partner's partial itself from
-// global memory: every wave reaches the end of the kernel whatever the other
-// blocks do, and the result is correct either way.
+// The partials travel as {value, epoch} words (xchg.cuh): no barrier, no fence,
+// no zeroed memory.  A block polls each word at most `spin` times; if a partner
+// has not published by then, the block computes that partner's partial itself
+// from global memory, in the partner's own arithmetic: every wave reaches the
+// end of the kernel whatever the other blocks do, and the result is the same
+// bit for bit either way.
 #pragma once
 
 #include "common.cuh"
 #include "launch.hpp"
+#include "xchg.cuh"
 
 namespace nblahip {
 
@@ -60,39 +57,32 @@ struct ClSplitArgs {
   int accum_dx;
 };
 
-__device__ __forceinline__ unsigned long long split_pack(float v, uint32_t epoch) {
-  return (static_cast<unsigned long long>(epoch) << 32) | __float_as_uint(v);
-}
-
-__device__ __forceinline__ void split_publish(unsigned long long *slot, float v, uint32_t epoch) {
-  __hip_atomic_store(slot, split_pack(v, epoch), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Polls the partner words this thread is responsible for into part[]; words
-// that do not turn up mark their block in missing[].
+// Polls the partners' words into part[] (a thread takes the two words of a
+// unit at a time); words that do not turn up mark their block in missing[].
 template <int TPR>
 __device__ __forceinline__ void split_collect(const ClSplitArgs &a, const unsigned long long *base,
                                               uint32_t self, int per, float *part, int *missing) {
   const int total = a.split * per;
-  for (int idx = threadIdx.x; idx < total; idx += TPR) {
+  for (int idx = 2 * threadIdx.x; idx < total; idx += 2 * TPR) {
     const int sp = idx / per;
     if (sp == static_cast<int>(self)) continue;
-    bool ok = false;
-    unsigned long long w = 0;
-    for (int it = 0; it < a.spin; ++it) {
-      w = __hip_atomic_load(base + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (static_cast<uint32_t>(w >> 32) == a.epoch) {
-        ok = true;
-        break;
-      }
-      __builtin_amdgcn_s_sleep(8);
-    }
-    if (ok) {
-      part[idx] = __uint_as_float(static_cast<uint32_t>(w));
+    float v0, v1;
+    if (xchg_poll2(base + idx, a.epoch, a.spin, &v0, &v1)) {
+      part[idx] = v0;
+      part[idx + 1] = v1;
     } else {
       missing[sp] = 1;
     }
   }
+}
+
+// Publishes this block's entries of part[] (a word per thread).
+template <int TPR>
+__device__ __forceinline__ void split_publish_own(const ClSplitArgs &a, unsigned long long *base,
+                                                  uint32_t self, int per, const float *part) {
+  lds_barrier(); // part[self] as its writers left it
+  for (int e = threadIdx.x; e < per; e += TPR)
+    xchg_publish(base + self * per + e, part[self * per + e], a.epoch);
 }
 
 // Sum of v over the threads of the block that hold the same unit of the tile
@@ -236,8 +226,6 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
     if (writer) {
       part[s * per + gi * 2] = m;
       part[s * per + gi * 2 + 1] = q;
-      split_publish(slots + s * per + gi * 2, m, a.epoch);
-      split_publish(slots + s * per + gi * 2 + 1, q, a.epoch);
     }
   } else {
     float sum[VEC];
@@ -275,13 +263,12 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
         const int u = cvx * VEC + j;
         part[s * per + u * 2] = m[j];
         part[s * per + u * 2 + 1] = q[j];
-        split_publish(slots + s * per + u * 2, m[j], a.epoch);
-        split_publish(slots + s * per + u * 2 + 1, q[j], a.epoch);
       }
     }
   }
 
   // ---- the partners' parts
+  split_publish_own<TPR>(a, slots, s, per, part);
   split_collect<TPR>(a, slots, s, per, part, missing);
   lds_barrier();
   for (int sp = 0; sp < a.split; ++sp) {
@@ -490,7 +477,7 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
         }
       }
       part[sp * per + e] = v;
-      if (publish) split_publish(slots + sp * per + e, v, a.epoch);
+      if (publish) xchg_publish(slots + sp * per + e, v, a.epoch);
     }
   };
 

@@ -2,49 +2,12 @@
 // (gn_cl_split.cuh): eligibility, the block shape, the exchange array and the
 // per-call epoch.
 #include <algorithm>
-#include <atomic>
 
 #include "gn_cl_split.cuh"
 
 namespace nblahip {
 
 namespace {
-
-// Exchange words of all calls: a ring inside the library's own data segment,
-// zero when the code object is loaded and from then on written only by the
-// split kernels ({value, epoch} words), which is what makes an epoch match
-// proof of a partner's publication.  One array per GPU.
-constexpr size_t kXchgWords = size_t{1} << 19; // 4 MiB
-constexpr int kMaxDevices = 64;
-__device__ __align__(256) unsigned long long split_xchg[kXchgWords];
-std::atomic<unsigned long long *> g_xchg_ptr[kMaxDevices];
-std::atomic<uint32_t> g_epoch[kMaxDevices];
-std::atomic<uint64_t> g_ring[kMaxDevices];
-
-// Device address of this device's exchange array, this call's epoch (never 0:
-// the array starts zeroed) and its region of the ring.  Regions of calls in
-// flight at the same time may overlap once the ring wraps; an overwritten word
-// fails the epoch test and its reader recomputes the value.
-int exchange_region(size_t words, unsigned long long **region, uint32_t *epoch) {
-  int dev = 0;
-  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return static_cast<int>(e);
-  if (dev < 0 || dev >= kMaxDevices) return NBLAHIP_EINVAL;
-  unsigned long long *base = g_xchg_ptr[dev].load(std::memory_order_acquire);
-  if (!base) {
-    void *p = nullptr;
-    if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(split_xchg)); e != hipSuccess)
-      return static_cast<int>(e);
-    if (!p) return static_cast<int>(hipErrorInvalidSymbol);
-    base = static_cast<unsigned long long *>(p);
-    g_xchg_ptr[dev].store(base, std::memory_order_release);
-  }
-  uint32_t ep = g_epoch[dev].fetch_add(1, std::memory_order_relaxed) + 1;
-  if (ep == 0) ep = g_epoch[dev].fetch_add(1, std::memory_order_relaxed) + 1;
-  *epoch = ep;
-  const uint64_t at = g_ring[dev].fetch_add(words, std::memory_order_relaxed) % kXchgWords;
-  *region = base + (at + words <= kXchgWords ? at : 0);
-  return 0;
-}
 
 struct SplitPlan {
   bool ok = false;
@@ -54,7 +17,7 @@ struct SplitPlan {
   size_t words = 0;
 };
 
-SplitPlan plan_split(const ClProblem &p, bool aligned, bool backward, hipStream_t st) {
+SplitPlan plan_split(const ClProblem &p, bool aligned, bool backward) {
   SplitPlan s;
   if (!aligned || !tune_int("GN_CL_SPLIT", 1)) return s;
   if (!p.bc_gamma || !p.bc_beta) return s;
@@ -76,13 +39,6 @@ SplitPlan plan_split(const ClProblem &p, bool aligned, bool backward, hipStream_
   }
   s.units = s.instance ? static_cast<int>(tile_ch) : kSplitTV >> s.cvg_shift;
   s.tiles = static_cast<int>(p.channels / tile_ch);
-  // An exchanged epoch is only proof of publication while every launch has
-  // its own: a captured launch would replay one epoch.
-  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(st, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
-    (void)hipGetLastError();
-    return s;
-  }
   // Block shape: positions per block PB = NL * TPR / 8.  256 threads x 8
   // vectors (32 KB of half data, four blocks to a CU) is the fastest shape in
   // both directions over a sweep of shapes (C4 stored NHWC backward 25.5 us
@@ -117,7 +73,7 @@ SplitPlan plan_split(const ClProblem &p, bool aligned, bool backward, hipStream_
   if (!s.ok) return s;
   const int64_t blocks = p.batch * s.tiles * static_cast<int64_t>(s.split);
   s.words = static_cast<size_t>(blocks) * 2 * s.units;
-  if (blocks > (1ll << 30) || s.words > kXchgWords) s.ok = false;
+  if (blocks > (1ll << 30) || s.words > xchg_capacity()) s.ok = false;
   if (backward &&
       static_cast<size_t>(p.batch) * s.split * p.channels * 2 * sizeof(float) > p.ws_bytes)
     s.ok = false;
@@ -135,7 +91,7 @@ ClSplitArgs make_args(const ClProblem &p, const SplitPlan &s) {
   a.var = p.var;
   a.dmean = p.dmean;
   a.dvar = p.dvar;
-  a.spin = tune_int("GN_CL_SPLIT_SPIN", 64);
+  a.spin = tune_int("XCHG_SPIN", 64);
   a.P = static_cast<int>(p.spatial);
   a.C = static_cast<int>(p.channels);
   a.tiles = s.tiles;
@@ -173,8 +129,8 @@ int run(bool backward, const SplitPlan &s, const ClSplitArgs &a, unsigned grid, 
   return NBLAHIP_EINVAL;
 }
 
-int dispatch(const ClProblem &p, const SplitPlan &s, bool backward, ClSplitArgs &a, hipStream_t st) {
-  if (int e = exchange_region(s.words, &a.xchg, &a.epoch)) return e;
+int dispatch(const ClProblem &p, const SplitPlan &s, bool backward, const ClSplitArgs &a,
+             hipStream_t st) {
   const unsigned grid = static_cast<unsigned>(p.batch * s.tiles * s.split);
   if (p.dtype == NBLAHIP_F16) {
     return s.instance ? run<__half, 8, true>(backward, s, a, grid, st)
@@ -187,18 +143,20 @@ int dispatch(const ClProblem &p, const SplitPlan &s, bool backward, ClSplitArgs 
 } // namespace
 
 bool cl_split_fwd(const ClProblem &p, bool aligned, hipStream_t st, int *status) {
-  const SplitPlan s = plan_split(p, aligned, false, st);
+  const SplitPlan s = plan_split(p, aligned, false);
   if (!s.ok) return false;
   ClSplitArgs a = make_args(p, s);
+  if (!xchg_acquire(s.words, st, &a.xchg, &a.epoch, status)) return *status != 0;
   *status = dispatch(p, s, false, a, st);
   return true;
 }
 
 bool cl_split_bwd(const ClProblem &p, bool aligned, float **pairs, int64_t *pair_batches,
                   hipStream_t st, int *status) {
-  const SplitPlan s = plan_split(p, aligned, true, st);
+  const SplitPlan s = plan_split(p, aligned, true);
   if (!s.ok) return false;
   ClSplitArgs a = make_args(p, s);
+  if (!xchg_acquire(s.words, st, &a.xchg, &a.epoch, status)) return *status != 0;
   a.pairs = static_cast<float *>(p.ws); // [batch * split][C][2], summed over its first axis afterwards
   *pairs = a.pairs;
   *pair_batches = p.batch * s.split;

@@ -95,7 +95,7 @@ def test_split_kernels_match_the_oracle_with_and_without_the_exchange(n, sp, c, 
         return
     # no poll allowed: every block recomputes all its partners' parts, in the
     # arithmetic the partners use, so not a bit may change
-    K.tune_set("GN_CL_SPLIT_SPIN", 0)
+    K.tune_set("XCHG_SPIN", 0)
     out2, names2 = run()
     assert ran(names2)
     for a_, b_ in zip(out, out2):
@@ -111,7 +111,7 @@ def test_split_kernels_match_the_oracle_with_and_without_the_exchange(n, sp, c, 
 def test_split_flags(spin):
     """no_scale/no_bias, dmean/dvar, accumulation onto dx/dgamma/dbeta, parameter
     gradients only, dx only."""
-    K.tune_set("GN_CL_SPLIT_SPIN", spin)
+    K.tune_set("XCHG_SPIN", spin)
     n, sp, c, groups = 3, (24, 24), 64, 4
     rng = np.random.default_rng(9)
     x, dy, g, b = make(n, sp, c, F32, 31)

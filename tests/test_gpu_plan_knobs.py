@@ -281,10 +281,10 @@ GRIDS = [
      [{"GN_CL_SPLIT_TPR": t, "GN_CL_SPLIT_NL": n} for t, n in ((256, 4), (256, 8), (512, 4), (512, 8),
                                                                 (1024, 4), (1024, 8))],
      ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], []),
-    ("gn_cl_split_no_polls", run_gn, (3, 128, (40, 40), 16, F16, True), [{"GN_CL_SPLIT_SPIN": 0}],
+    ("gn_cl_split_no_polls", run_gn, (3, 128, (40, 40), 16, F16, True), [{"XCHG_SPIN": 0}],
      ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], []),
     ("in_cl_split_no_polls", run_in, (2, 64, (30, 30), F32, True),
-     [{"GN_CL_SPLIT_SPIN": 0, "GN_CL_SPLIT_INSTANCES": 1}],
+     [{"XCHG_SPIN": 0, "GN_CL_SPLIT_INSTANCES": 1}],
      ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], []),
     ("gn_cl_wide_plain_block_order", run_gn, (4, 1024, (32, 32), 128, F16, True),
      [{"GN_CL_XCD_MAP": 0, **NO_SPLIT}],
