@@ -1,0 +1,427 @@
+// Channel-last BatchNormalization training with the whole tensor held on the
+// chip between the statistics and the normalization.
+//
+// x is [M][C].  A channel's column runs through every row, so no block can own
+// a channel, and the split reduction reads x twice (statistics, then apply:
+// 3 S forward, 5 S backward).  But the 256 CUs together hold 256 x 400 KB in
+// registers and LDS - a [256,56,56,64] half tensor (103 MB) fits.  One
+// 1024-thread block per CU takes a contiguous range of rows (NR 16-byte vectors
+// per thread in registers, NS more in LDS, as in bn_onchip.hip); a thread's
+// vectors always hold the same VEC channels (C / VEC divides 1024), so the
+// per-channel sums are VEC accumulators per thread, folded over the block.
+// The blocks then exchange their per-channel partials as {value, epoch} words
+// (xchg.cuh) in two stages: block c merges the partials of channel c from all
+// blocks (fixed order), writes mean / var / running statistics and publishes
+// the result once per block (were all blocks to poll the same C words, the one
+// memory channel that holds them would queue the polls of 16 000 threads); every
+// block reads its copy of the C results and normalizes what it holds: x
+// crosses the memory system once (2 S).
+//
+// Every wait is a bounded poll.  A partial that does not turn up is computed
+// by the block that needs it, from global memory, in the arithmetic of the
+// block that owes it (same thread map, same order: the same bits); a channel
+// result that does not turn up is merged by the block that needs it.  So every
+// wave reaches the end whatever the other blocks do, and the results do not
+// depend on who computed what.
+#include <algorithm>
+#include <type_traits>
+
+#include "common.cuh"
+#include "launch.hpp"
+#include "onchip.cuh"
+#include "xchg.cuh"
+
+namespace nblahip {
+
+namespace {
+
+constexpr int kGridMaxBlocks = 256; // partials per channel a block merges (one per thread of a wave quad)
+constexpr int kGridMaxC = 128;      // channels (LDS fold of the per-channel sums)
+
+struct BnClGridArgs {
+  const void *x;
+  void *y;
+  const float *gamma, *beta;
+  float *mean, *var, *rmean, *rvar;
+  uint32_t C;
+  uint32_t cv;      // channel vectors per row = C / VEC (a power of two)
+  uint32_t nv;      // vectors of the tensor = M * cv
+  uint32_t vb;      // vectors per block (whole rows)
+  uint32_t nblocks;
+  float inv_N, unbias, decay, eps, one;
+  unsigned long long *x1; // stage 1: [nblocks][C][2] = (mean, m2) of the block's rows
+  unsigned long long *x2; // stage 2: [nblocks][C][2] = (mean, var), a copy for every block
+  uint32_t epoch;
+  int spin;
+};
+
+// Vectors of block b.
+__device__ __forceinline__ uint32_t grid_block_vectors(const BnClGridArgs &a, uint32_t b) {
+  const uint32_t first = b * a.vb;
+  return first >= a.nv ? 0u : min(a.vb, a.nv - first);
+}
+
+// Per-channel totals of v[VEC] over the threads of the block that hold the
+// same channel vector (t % cv): butterfly over the lanes cv apart, one row of
+// fold[16][C] per wave, the rows added in wave order by one thread per channel
+// (tot[C]), and every thread reads back its channels' totals.
+template <int VEC>
+__device__ __forceinline__ void grid_channel_sums(float (&v)[VEC], uint32_t cv, uint32_t cvx,
+                                                  float *fold, float *tot, uint32_t C) {
+  constexpr int NW = kOnchipBlock / kWave;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    for (uint32_t off = cv; off < kWave; off <<= 1) v[j] += __shfl_xor(v[j], off);
+  }
+  lds_barrier(); // earlier readers of fold / tot are done
+  if ((threadIdx.x & (kWave - 1)) < cv) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) fold[(threadIdx.x / kWave) * C + cvx * VEC + j] = v[j];
+  }
+  lds_barrier();
+  if (threadIdx.x < C) {
+    float t = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) t += fold[w * C + threadIdx.x];
+    tot[threadIdx.x] = t;
+  }
+  lds_barrier();
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) v[j] = tot[cvx * VEC + j];
+}
+
+// The same fold for ONE channel (element e of the vectors of channel vector
+// c / VEC): identical butterfly and wave order, so identical bits.
+__device__ __forceinline__ float grid_channel_sum1(float v, uint32_t cv, uint32_t cvx, uint32_t c,
+                                                   bool mine, float *fold, uint32_t C) {
+  constexpr int NW = kOnchipBlock / kWave;
+  for (uint32_t off = cv; off < kWave; off <<= 1) v += __shfl_xor(v, off);
+  lds_barrier(); // earlier readers of fold are done
+  if ((threadIdx.x & (kWave - 1)) < cv && mine) fold[(threadIdx.x / kWave) * C + c] = v;
+  lds_barrier();
+  float t = 0.f;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) t += fold[w * C + c];
+  return t;
+}
+
+// (mean, m2) of the rows of block p for channel c, from global memory, in the
+// order block p itself uses (its thread map, slots ascending per thread, the
+// same folds): what block p publishes for c, bit for bit.  Only the threads of
+// c's channel vector load (the folds never mix channel vectors) and only c's
+// element is accumulated, so this costs a handful of registers.
+template <typename T, int VEC>
+__device__ __forceinline__ void grid_partial_from_memory(const BnClGridArgs &a, uint32_t p,
+                                                         uint32_t c, float *fold, float &m,
+                                                         float &q) {
+  const T *__restrict__ x = static_cast<const T *>(a.x);
+  const uint32_t t = threadIdx.x;
+  const uint32_t cvx = t % a.cv, e = c % VEC;
+  const uint32_t vbp = cvx == c / VEC ? grid_block_vectors(a, p) : 0u;
+  const uint32_t rows = grid_block_vectors(a, p) / a.cv;
+  const size_t first = static_cast<size_t>(p) * a.vb;
+  float s = 0.f;
+#pragma unroll 1
+  for (uint32_t v = t; v < vbp; v += kOnchipBlock) {
+    const RawVec<T, VEC> r = load_raw<T, VEC>(x + (first + v) * VEC);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float n = elem_fma<T, VEC>(r, j, a.one, s);
+      s = static_cast<uint32_t>(j) == e ? n : s;
+    }
+  }
+  s = grid_channel_sum1(s, a.cv, cvx, c, cvx == c / VEC, fold, a.C);
+  m = s * (1.0f / static_cast<float>(rows));
+  q = 0.f;
+#pragma unroll 1
+  for (uint32_t v = t; v < vbp; v += kOnchipBlock) {
+    const RawVec<T, VEC> r = load_raw<T, VEC>(x + (first + v) * VEC);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float d = elem_fma<T, VEC>(r, j, a.one, -m);
+      const float n = fmaf(d, d, q);
+      q = static_cast<uint32_t>(j) == e ? n : q;
+    }
+  }
+  q = grid_channel_sum1(q, a.cv, cvx, c, cvx == c / VEC, fold, a.C);
+}
+
+// Merged (mean, var) of channel c over all blocks: thread p < nblocks takes
+// block p's partial (polled; computed here if it does not arrive), the block
+// merges them in a fixed tree.  Same result in every thread and in every block
+// that calls it.  scratch: miss[kGridMaxBlocks] ints, got[2 * kGridMaxBlocks],
+// wel[3 * 16], fold[16 * C].
+template <typename T, int VEC>
+__device__ __forceinline__ void grid_channel_result(const BnClGridArgs &a, uint32_t c, int *miss,
+                                                    float *got, float *wel, float *fold,
+                                                    float &mean, float &var) {
+  const uint32_t t = threadIdx.x;
+  lds_barrier(); // got / miss of an earlier call have been consumed
+  if (t == 0) miss[kGridMaxBlocks] = 0; // any partial missing at all?
+  lds_barrier();
+  if (t < a.nblocks) {
+    float v0 = 0.f, v1 = 0.f;
+    const bool ok = xchg_poll2(a.x1 + (static_cast<size_t>(t) * a.C + c) * 2, a.epoch, a.spin, &v0, &v1);
+    got[2 * t] = v0;
+    got[2 * t + 1] = v1;
+    miss[t] = ok ? 0 : 1;
+    if (!ok) miss[kGridMaxBlocks] = 1;
+  }
+  lds_barrier();
+  for (uint32_t p = 0; miss[kGridMaxBlocks] && p < a.nblocks; ++p) {
+    if (!miss[p]) continue; // same answer in every thread
+    float m, q;
+    grid_partial_from_memory<T, VEC>(a, p, c, fold, m, q);
+    if (t == 0) {
+      got[2 * p] = m;
+      got[2 * p + 1] = q;
+    }
+    lds_barrier();
+  }
+  Welford w{0.f, 0.f, 0.f};
+  if (t < a.nblocks) {
+    w.mean = got[2 * t];
+    w.m2 = got[2 * t + 1];
+    w.n = static_cast<float>(grid_block_vectors(a, t) / a.cv);
+  }
+  w = block_welford(w, wel);
+  mean = w.mean;
+  var = w.m2 * a.inv_N;
+}
+
+} // namespace
+
+template <typename T, int VEC, int NR, int NS>
+__global__ void __launch_bounds__(kOnchipBlock)
+bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
+  static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors");
+  constexpr int NL = NR + NS;
+  __shared__ uint4 spill[NS > 0 ? NS * kOnchipBlock : 1];
+  __shared__ float fold[16 * kGridMaxC];
+  __shared__ float tot[kGridMaxC];
+  __shared__ float fin[2 * kGridMaxC];   // (mean, var) per channel
+  __shared__ float got[2 * kGridMaxBlocks];
+  __shared__ int miss[kGridMaxBlocks + 2]; // [kGridMaxBlocks], [+1]: any partial / any result missing
+  __shared__ float wel[3 * 16];
+  const uint32_t b = blockIdx.x;
+  const uint32_t t = threadIdx.x;
+  const uint32_t cvx = t % a.cv;
+  const uint32_t ch = cvx * VEC;
+  const uint32_t vbb = grid_block_vectors(a, b);
+  const T *__restrict__ x = static_cast<const T *>(a.x) + static_cast<size_t>(b) * a.vb * VEC;
+  T *__restrict__ y = static_cast<T *>(a.y) + static_cast<size_t>(b) * a.vb * VEC;
+
+  // ---- loads: slot k is vector k * 1024 + t of the block (a slot past the
+  // block's end reads the block's last vector and stays out of sums and stores)
+  const uint32_t last = vbb - 1;
+  RawVec<T, VEC> raw[NR];
+  {
+    RawVec<T, VEC> parked[NS > 0 ? NS : 1];
+#pragma unroll
+    for (int k = 0; k < NS; ++k) {
+      const uint32_t v = static_cast<uint32_t>(NR + k) * kOnchipBlock + t;
+      parked[k] = load_raw<T, VEC>(x + static_cast<size_t>(min(v, last)) * VEC);
+    }
+#pragma unroll
+    for (int k = 0; k < NR; ++k) {
+      const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t;
+      raw[k] = load_raw<T, VEC>(x + static_cast<size_t>(min(v, last)) * VEC);
+    }
+#pragma unroll
+    for (int k = 0; k < NS; ++k) spill[k * kOnchipBlock + t] = __builtin_bit_cast(uint4, parked[k]);
+  }
+  auto slot = [&](int k) -> RawVec<T, VEC> {
+    if (k < NR) return raw[k < NR ? k : 0];
+    return __builtin_bit_cast(RawVec<T, VEC>, spill[(k - NR) * kOnchipBlock + t]);
+  };
+
+  // ---- this block's partial per channel: mean, then the second moment about it
+  float m[VEC], q[VEC];
+  {
+    float s[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) s[j] = 0.f;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      if (static_cast<uint32_t>(k) * kOnchipBlock + t < vbb) {
+        const RawVec<T, VEC> r = slot(k);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) s[j] = elem_fma<T, VEC>(r, j, a.one, s[j]);
+      }
+    }
+    grid_channel_sums<VEC>(s, a.cv, cvx, fold, tot, a.C);
+    const float icnt = 1.0f / static_cast<float>(vbb / a.cv);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      m[j] = s[j] * icnt;
+      q[j] = 0.f;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < NR; ++k) forget<T, VEC>(raw[k]);
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    if (static_cast<uint32_t>(k) * kOnchipBlock + t < vbb) {
+      const RawVec<T, VEC> r = slot(k);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float d = elem_fma<T, VEC>(r, j, a.one, -m[j]);
+        q[j] = fmaf(d, d, q[j]);
+      }
+    }
+  }
+  grid_channel_sums<VEC>(q, a.cv, cvx, fold, tot, a.C);
+  // publish (mean, m2) of every channel: a word per thread (tot holds the m2
+  // totals; the means go through fin, which is free until the results arrive)
+  if (t < a.cv) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) fin[ch + j] = m[j];
+  }
+  lds_barrier();
+  for (uint32_t e = t; e < 2 * a.C; e += kOnchipBlock)
+    xchg_publish(a.x1 + static_cast<size_t>(b) * a.C * 2 + e, (e & 1) ? tot[e >> 1] : fin[e >> 1], a.epoch);
+
+  // ---- stage 2: block c merges channel c, writes its statistics, publishes
+  for (uint32_t c = b; c < a.C; c += a.nblocks) {
+    float mean, var;
+    grid_channel_result<T, VEC>(a, c, miss, got, wel, fold, mean, var);
+    if (t == 0) {
+      a.mean[c] = mean;
+      a.var[c] = var;
+      if (a.rmean) a.rmean[c] = a.decay * a.rmean[c] + (1.f - a.decay) * mean;
+      if (a.rvar) a.rvar[c] = a.decay * a.rvar[c] + (1.f - a.decay) * var * a.unbias;
+    }
+    if (t < a.nblocks) { // a copy for block t
+      unsigned long long *w = a.x2 + (static_cast<size_t>(t) * a.C + c) * 2;
+      xchg_publish(w, mean, a.epoch);
+      xchg_publish(w + 1, var, a.epoch);
+    }
+  }
+
+  // ---- every block: the C results (merged here where one does not arrive)
+  lds_barrier();
+  if (t == 0) miss[kGridMaxBlocks + 1] = 0;
+  lds_barrier();
+  for (uint32_t c = t; c < a.C; c += kOnchipBlock) {
+    float v0 = 0.f, v1 = 0.f;
+    const bool ok = xchg_poll2(a.x2 + (static_cast<size_t>(b) * a.C + c) * 2, a.epoch, a.spin, &v0, &v1);
+    fin[2 * c] = v0;
+    fin[2 * c + 1] = ok ? v1 : -1.f; // a variance is never negative: marks "missing"
+    if (!ok) miss[kGridMaxBlocks + 1] = 1;
+  }
+  lds_barrier();
+  for (uint32_t c = 0; miss[kGridMaxBlocks + 1] && c < a.C; ++c) {
+    if (fin[2 * c + 1] >= 0.f) continue; // same answer in every thread
+    float mean, var;
+    grid_channel_result<T, VEC>(a, c, miss, got, wel, fold, mean, var);
+    lds_barrier();
+    if (t == 0) {
+      fin[2 * c] = mean;
+      fin[2 * c + 1] = var;
+    }
+    lds_barrier();
+  }
+
+  // ---- normalize what the block holds
+#pragma unroll
+  for (int k = 0; k < NR; ++k) forget<T, VEC>(raw[k]);
+  float sc[VEC], sh[VEC], mu[VEC], be[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    mu[j] = fin[2 * (ch + j)];
+    sc[j] = (a.gamma ? a.gamma[ch + j] : 1.f) * inv_std(fin[2 * (ch + j) + 1], a.eps);
+    be[j] = a.beta ? a.beta[ch + j] : 0.f;
+    sh[j] = fmaf(-mu[j], sc[j], be[j]);
+  }
+  const uint32_t t2 = fresh(t);
+#pragma unroll
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t2;
+    if (v < vbb) {
+      const RawVec<T, VEC> r = slot(k);
+      float o[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        if constexpr (sizeof(T) == 2) {
+          o[j] = elem_fma<T, VEC>(r, j, sc[j], sh[j]);
+        } else {
+          o[j] = fmaf(elem_fma<T, VEC>(r, j, a.one, -mu[j]), sc[j], be[j]);
+        }
+      }
+      store_vec<T, VEC>(y + static_cast<size_t>(v) * VEC, o);
+    }
+  }
+}
+
+namespace {
+
+template <typename T, int VEC>
+int run_grid_fwd(int nl, const BnClGridArgs &a, hipStream_t st) {
+#define GRID_CASE(NR, NS)                                                                        \
+  if (nl <= (NR) + (NS)) {                                                                       \
+    NBLAHIP_LAUNCH("bn_cl_grid_fwd_kernel", (bn_cl_grid_fwd_kernel<T, VEC, NR, NS>),             \
+                   dim3(a.nblocks), dim3(kOnchipBlock), 0, st, a);                               \
+    return last_launch_status();                                                                 \
+  }
+  GRID_CASE(4, 0)
+  GRID_CASE(8, 0)
+  GRID_CASE(12, 0)
+  GRID_CASE(16, 0)
+  GRID_CASE(16, 3)
+  GRID_CASE(16, 6)
+  GRID_CASE(16, 9)
+#undef GRID_CASE
+  return NBLAHIP_EINVAL;
+}
+
+} // namespace
+
+bool bn_cl_grid_fwd_train(const BnProblem &p, hipStream_t st, int *status) {
+  if (!tune_int("BN_CL_GRID", 1)) return false;
+  if (p.size2 != 1 || p.relu || p.z || p.y || p.sums_out || p.sums_in || !p.out) return false;
+  const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
+  if (p.C % vec != 0 || p.C > kGridMaxC || !aligned16(p.x) || !aligned16(p.out)) return false;
+  const int64_t cv = p.C / vec;
+  if ((cv & (cv - 1)) != 0 || cv > kWave) return false;
+  const int64_t M = p.size0;
+  const int64_t nv = M * cv;
+  const int blocks = std::min(device_cus(), kGridMaxBlocks);
+  // whole rows per block, the same for every block but the last
+  const int64_t rows_pb = (M + blocks - 1) / blocks;
+  const int64_t vb = rows_pb * cv;
+  const int nl = static_cast<int>((vb + kOnchipBlock - 1) / kOnchipBlock);
+  const int64_t nblocks = (M + rows_pb - 1) / rows_pb;
+  // Up to what the chip holds, and from 10 vectors per thread: the exchange and
+  // the folds cost about 12 us whatever the size, one read of x saves 0.16 us
+  // per MB ([256,56,56,64] half 57.5 -> 51.2 us, [128,56,56,64] 35.6 -> 32.7 us,
+  // [64,56,56,64] 24.1 us either way, [32,56,56,64] 18.4 -> 21.8 us).
+  if (nl < tune_int("BN_CL_GRID_MIN_SLOTS", 10) || nl > 25 || nblocks < blocks / 2) return false;
+  BnClGridArgs a{};
+  a.x = p.x;
+  a.y = p.out;
+  a.gamma = p.gamma;
+  a.beta = p.beta;
+  a.mean = p.batch_mean;
+  a.var = p.batch_var;
+  a.rmean = p.rmean;
+  a.rvar = p.rvar;
+  a.C = static_cast<uint32_t>(p.C);
+  a.cv = static_cast<uint32_t>(cv);
+  a.nv = static_cast<uint32_t>(nv);
+  a.vb = static_cast<uint32_t>(vb);
+  a.nblocks = static_cast<uint32_t>(nblocks);
+  const double N = static_cast<double>(M);
+  a.inv_N = static_cast<float>(1.0 / N);
+  a.unbias = static_cast<float>(N / (N - 1.0));
+  a.decay = p.decay;
+  a.eps = p.eps;
+  a.one = 1.0f;
+  a.spin = tune_int("XCHG_SPIN", 64) * 16; // a whole-chip exchange: wait longer before recomputing
+  const size_t words = static_cast<size_t>(nblocks) * p.C * 4;
+  if (!xchg_acquire(words, st, &a.x1, &a.epoch, status)) return *status != 0;
+  a.x2 = a.x1 + static_cast<size_t>(nblocks) * p.C * 2;
+  *status = p.dtype == NBLAHIP_F16 ? run_grid_fwd<__half, 8>(nl, a, st) : run_grid_fwd<float, 4>(nl, a, st);
+  return true;
+}
+
+} // namespace nblahip

@@ -442,6 +442,7 @@ int launch_bn_fwd_train(const BnProblem &p, hipStream_t st) {
   if (bn_rows_fwd_train(p, st, &status)) return status;
   if (bn_onchip_fwd_train(p, st, &status)) return status;
   if (bn_cl_cached_fwd_train(p, st, &status)) return status;
+  if (bn_cl_grid_fwd_train(p, st, &status)) return status;
   return bn_fwd_train_impl(p, false, st);
 }
 

@@ -392,3 +392,99 @@ def test_bn_training_forward_in_place(shape, axis, dtype):
     assert_close(to_np(m), m_r, dn, "stat", "mean")
     assert_close(to_np(v), v_r, dn, "stat", "var")
     assert_close(to_np(rmd), rm_r, dn, "stat", "running_mean")
+
+
+# ------------------------------------------------------------------
+# Channel-last training forward with the whole tensor held on the chip and the
+# per-channel partials exchanged between the blocks.
+@pytest.mark.parametrize("m,c,dtype", [(100352, 64, torch.float16), (100353, 64, torch.float16),
+                                       (200000, 32, torch.float32), (150000, 128, torch.float16),
+                                       (1000001, 8, torch.float16), (40000, 128, torch.float32)])
+def test_bn_channel_last_held_on_the_chip(m, c, dtype):
+    """Against the oracle; bit-identical when no poll is allowed (every block
+    then computes the partials and channel results it needs itself); close to
+    the split reduction; running statistics updated once."""
+    dn = dtype_name(dtype)
+    x, _, g, b, rm, rv = make_bn((m, c), 1, dtype, 5, mean=1.0, std=2.0)
+    y_r, m_r, v_r, rm_r, rv_r = R.bn_forward_batch(x, b, g, rm, rv, 1, 0.9, 1e-5)
+    xd, gd, bd = to_dev(x, dtype), to_dev(g), to_dev(b)
+
+    def run(knobs):
+        K.tune_reset()
+        for k_, val in knobs.items():
+            K.tune_set(k_, val)
+        rmd, rvd = to_dev(rm), to_dev(rv)
+        K.check(K.lib().nblahip_profile_enable(16))
+        y, mean, var = K.bn_forward_batch(xd, bd, gd, rmd, rvd, 1, 0.9, 1e-5)
+        torch.cuda.synchronize()
+        names = K.profile_kernels()
+        K.check(K.lib().nblahip_profile_enable(0))
+        K.tune_reset()
+        return [y, mean, var, rmd, rvd], names
+
+    try:
+        held, names = run({"BN_CL_GRID_MIN_SLOTS": 1})
+        assert names == ["bn_cl_grid_fwd_kernel"], names
+        alone, names = run({"BN_CL_GRID_MIN_SLOTS": 1, "XCHG_SPIN": 0})
+        assert names == ["bn_cl_grid_fwd_kernel"], names
+        split, names = run({"BN_CL_GRID": 0})
+        assert "bn_cl_grid_fwd_kernel" not in names
+    finally:
+        K.tune_reset()
+    y, mean, var, rmd, rvd = held
+    assert_close(to_np(mean), m_r, dn, "stat", "mean")
+    assert_close(to_np(var), v_r, dn, "stat", "var")
+    assert_close(to_np(rmd), rm_r, dn, "stat", "running mean")
+    assert_close(to_np(rvd), rv_r, dn, "stat", "running var")
+    assert_close(to_np(y), y_r, dn, "y", "y")
+    for a_, b_ in zip(held, alone):
+        assert torch.equal(a_, b_)
+    assert_close(to_np(split[0]), to_np(y), dn, "y", "y against the split reduction")
+    assert_close(to_np(split[2]), to_np(var), dn, "stat", "var against the split reduction")
+
+
+def test_two_chip_filling_forwards_at_once():
+    """Two host threads, each on its own stream, run the forward that holds the
+    whole tensor on the chip at the same time: each launch wants every CU, so
+    blocks of the two launches wait for partners that are not resident yet, time
+    out and compute what they need themselves.  Both must finish and give the
+    single-threaded results bit for bit."""
+    import threading
+    m, c = 256 * 56 * 56, 64
+
+    def work(seed, reps):
+        gen = torch.Generator(device="cuda").manual_seed(seed)
+        x = (torch.randn(m, c, device="cuda", generator=gen) * 2 + 1).half()
+        gamma = torch.rand(c, device="cuda", generator=gen) + 0.5
+        beta = torch.randn(c, device="cuda", generator=gen)
+        out = None
+        for _ in range(reps):
+            out = K.bn_forward_batch(x, beta, gamma, None, None, 1, 0.9, 1e-5)
+        return list(out)
+
+    K.check(K.lib().nblahip_profile_enable(8))
+    want = [[t.clone() for t in work(300 + i, 1)] for i in range(2)]
+    torch.cuda.synchronize()
+    assert K.profile_kernels() == ["bn_cl_grid_fwd_kernel"]
+    K.check(K.lib().nblahip_profile_enable(0))
+    got, errors = [None, None], []
+
+    def run(i):
+        try:
+            s = torch.cuda.Stream()
+            with torch.cuda.stream(s):
+                out = work(300 + i, 4)
+                s.synchronize()
+            got[i] = out
+        except Exception as e:  # noqa: BLE001 - reported below
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=run, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for w, g_ in zip(want, got):
+        for a_, b_ in zip(w, g_):
+            assert torch.equal(a_, b_)

@@ -164,6 +164,11 @@ SWITCHES = [
     ("bn_rows_off", run_bn, ((32, 64, 14, 14), 1, F16), {"BN_ROWS": 0},
      ["bn_stats_planes_kernel", "bn_finalize_fwd_kernel", "bn_apply_planes_kernel",
       "bn_finalize_bwd_kernel"], ["row_fwd_kernel_bn", "row_bwd_kernel_bn"]),
+    ("bn_cl_grid_off", run_bn, ((100352, 64), 1, F16), {"BN_CL_GRID": 0},
+     ["bn_stats_cl_kernel", "bn_finalize_fwd_kernel", "bn_apply_cl_kernel"], ["bn_cl_grid_fwd_kernel"],
+     {"BN_CL_GRID_MIN_SLOTS": 1}),
+    ("bn_cl_grid_from_fewer_vectors", run_bn, ((100352, 64), 1, F16), {"BN_CL_GRID_MIN_SLOTS": 1},
+     ["bn_cl_grid_fwd_kernel"], ["bn_stats_cl_kernel"]),
     ("bn_cl_cached_off", run_bn, ((32, 7, 7, 256), 3, F16), {"BN_CL_CACHED": 0},
      ["bn_stats_cl_kernel", "bn_apply_cl_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
      ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"]),
