@@ -106,12 +106,13 @@ __device__ __forceinline__ float split_group_sum(float v, int cvg_shift, uint32_
   return t;
 }
 
-// The same for VEC per-channel values of a thread (instances; channel-wise
-// sums of the backward): threads with equal cvx hold the same channels.
-// fold: [TPR / 64][8 * VEC]; out[j] = total of channel cvx * VEC + j.
+// The same for VEC per-channel values of a thread (instances): threads with
+// equal cvx hold the same channels.  Butterfly over the lanes 8 apart, a row of
+// fold[TPR / 64][8 * VEC] per wave, the rows added in wave order by one thread
+// per channel (tot[8 * VEC]); v[j] = total of channel cvx * VEC + j.
 template <int TPR, int VEC>
 __device__ __forceinline__ void split_channel_sums(float (&v)[VEC], uint32_t cvx,
-                                                   float (*fold)[kSplitTV * VEC]) {
+                                                   float (*fold)[kSplitTV * VEC], float *tot) {
   constexpr int NW = TPR / kWave;
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
@@ -119,19 +120,57 @@ __device__ __forceinline__ void split_channel_sums(float (&v)[VEC], uint32_t cvx
     v[j] += __shfl_xor(v[j], 16);
     v[j] += __shfl_xor(v[j], 32);
   }
-  lds_barrier();
+  lds_barrier(); // earlier readers of fold / tot are done
   if ((threadIdx.x & (kWave - 1)) < kSplitTV) {
 #pragma unroll
     for (int j = 0; j < VEC; ++j) fold[threadIdx.x / kWave][cvx * VEC + j] = v[j];
   }
   lds_barrier();
-#pragma unroll
-  for (int j = 0; j < VEC; ++j) {
+  if (threadIdx.x < kSplitTV * VEC) {
     float t = 0.f;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) t += fold[w][cvx * VEC + j];
-    v[j] = t;
+    for (int w = 0; w < NW; ++w) t += fold[w][threadIdx.x];
+    tot[threadIdx.x] = t;
   }
+  lds_barrier();
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) v[j] = tot[cvx * VEC + j];
+}
+
+// Backward: the per-channel pairs (sum dy*xh, sum dy) of the block, both at
+// once, straight into chs[2][8 * VEC] (nothing returns to the threads).
+// fold: [TPR / 64][2 * 8 * VEC].
+template <int TPR, int VEC>
+__device__ __forceinline__ void split_pair_sums(float (&sdx)[VEC], float (&sdy)[VEC], uint32_t cvx,
+                                                float (*fold)[2 * kSplitTV * VEC],
+                                                float (*chs)[kSplitTV * VEC]) {
+  constexpr int NW = TPR / kWave;
+  constexpr int CH = kSplitTV * VEC;
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    sdx[j] += __shfl_xor(sdx[j], 8);
+    sdy[j] += __shfl_xor(sdy[j], 8);
+    sdx[j] += __shfl_xor(sdx[j], 16);
+    sdy[j] += __shfl_xor(sdy[j], 16);
+    sdx[j] += __shfl_xor(sdx[j], 32);
+    sdy[j] += __shfl_xor(sdy[j], 32);
+  }
+  lds_barrier(); // earlier readers of fold / chs are done
+  if ((threadIdx.x & (kWave - 1)) < kSplitTV) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      fold[threadIdx.x / kWave][cvx * VEC + j] = sdx[j];
+      fold[threadIdx.x / kWave][CH + cvx * VEC + j] = sdy[j];
+    }
+  }
+  lds_barrier();
+  for (int e = threadIdx.x; e < 2 * CH; e += TPR) {
+    float t = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) t += fold[w][e];
+    chs[e / CH][e % CH] = t;
+  }
+  lds_barrier();
 }
 
 __device__ __forceinline__ float split_count(const ClSplitArgs &a, int sp) {
@@ -170,6 +209,7 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
   constexpr int NW = TPR / kWave;
   constexpr int UMAX = INSTANCE ? TV * VEC : TV;
   __shared__ float fold[NW][UMAX];
+  __shared__ float tot[UMAX];
   __shared__ float part[kSplitMax * UMAX * 2];
   __shared__ int missing[kSplitMax];
   const uint32_t tile = blockIdx.x % a.tiles, ns = blockIdx.x / a.tiles;
@@ -236,7 +276,7 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) sum[j] = elem_fma<T, VEC>(raw[k], j, a.one, sum[j]);
     }
-    split_channel_sums<TPR, VEC>(sum, cvx, fold);
+    split_channel_sums<TPR, VEC>(sum, cvx, fold, tot);
     const float icnt = 1.0f / split_count(a, s);
     float m[VEC], q[VEC];
 #pragma unroll
@@ -256,7 +296,7 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
         }
       }
     }
-    split_channel_sums<TPR, VEC>(q, cvx, fold);
+    split_channel_sums<TPR, VEC>(q, cvx, fold, tot);
     if (writer) {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
@@ -318,10 +358,10 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) sum[j] = elem_fma<T, VEC>(r, j, a.one, sum[j]);
       }
-      split_channel_sums<TPR, VEC>(sum, cvx, fold);
+      split_channel_sums<TPR, VEC>(sum, cvx, fold, tot);
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
-        m[j] = sum[j] / cnt;
+        m[j] = sum[j] * (1.0f / cnt); // as the owner computes it
         q[j] = 0.f;
       }
 #pragma unroll 1
@@ -336,7 +376,7 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
           }
         }
       }
-      split_channel_sums<TPR, VEC>(q, cvx, fold);
+      split_channel_sums<TPR, VEC>(q, cvx, fold, tot);
       if (writer) {
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
@@ -418,7 +458,7 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
   constexpr int UMAX = INSTANCE ? CH : TV;
   constexpr int SV = INSTANCE ? VEC : 1; // statistics units of a thread's vector
   __shared__ RawVec<T, VEC> park[NL * TPR];
-  __shared__ float fold[NW][CH];
+  __shared__ float fold[NW][2 * CH];
   __shared__ float chs[2][CH]; // [0]: sum dy*xh, [1]: sum dy per channel of the tile
   __shared__ float part[kSplitMax * UMAX * 2];
   __shared__ int missing[kSplitMax];
@@ -497,16 +537,7 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
         sdy[j] = elem_fma<T, VEC>(dv, j, a.one, sdy[j]);
       }
     }
-    split_channel_sums<TPR, VEC>(sdx, cvx, fold);
-    split_channel_sums<TPR, VEC>(sdy, cvx, fold);
-    if (prow == 0) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        chs[0][cvx * VEC + j] = sdx[j];
-        chs[1][cvx * VEC + j] = sdy[j];
-      }
-    }
-    lds_barrier();
+    split_pair_sums<TPR, VEC>(sdx, sdy, cvx, fold, chs);
     if (a.pairs) {
       for (int e = threadIdx.x; e < 2 * CH; e += TPR) {
         const int c = e >> 1, w = e & 1;
@@ -541,16 +572,7 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
         sdy[j] = elem_fma<T, VEC>(dv, j, a.one, sdy[j]);
       }
     }
-    split_channel_sums<TPR, VEC>(sdx, cvx, fold);
-    split_channel_sums<TPR, VEC>(sdy, cvx, fold);
-    if (prow == 0) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        chs[0][cvx * VEC + j] = sdx[j];
-        chs[1][cvx * VEC + j] = sdy[j];
-      }
-    }
-    lds_barrier();
+    split_pair_sums<TPR, VEC>(sdx, sdy, cvx, fold, chs);
     unit_partials(static_cast<uint32_t>(sp), false);
     lds_barrier();
   }

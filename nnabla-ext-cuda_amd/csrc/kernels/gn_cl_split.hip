@@ -21,10 +21,7 @@ SplitPlan plan_split(const ClProblem &p, bool aligned, bool backward) {
   SplitPlan s;
   if (!aligned || !tune_int("GN_CL_SPLIT", 1)) return s;
   if (!p.bc_gamma || !p.bc_beta) return s;
-  // Instances exchange 64 channels x 2 words per block and partner: the polls
-  // cost what the whole lines save (C4 stored NHWC forward 27 vs 22 us), so
-  // they stay with the kernels of gn_cl_rows.cuh unless asked for.
-  if (p.groups == p.channels && !tune_int("GN_CL_SPLIT_INSTANCES", 0)) return s;
+  if (p.groups == p.channels && !tune_int("GN_CL_SPLIT_INSTANCES", 1)) return s;
   const int esz = p.dtype == NBLAHIP_F16 ? 2 : 4;
   s.vec = 16 / esz;
   const int64_t tile_ch = static_cast<int64_t>(kSplitTV) * s.vec; // channels of a 128-byte line
@@ -39,36 +36,51 @@ SplitPlan plan_split(const ClProblem &p, bool aligned, bool backward) {
   }
   s.units = s.instance ? static_cast<int>(tile_ch) : kSplitTV >> s.cvg_shift;
   s.tiles = static_cast<int>(p.channels / tile_ch);
-  // Block shape: positions per block PB = NL * TPR / 8.  256 threads x 8
-  // vectors (32 KB of half data, four blocks to a CU) is the fastest shape in
-  // both directions over a sweep of shapes (C4 stored NHWC backward 25.5 us
-  // against 31.5 with 512 x 8, whose half instantiation spills); the forward of
-  // long planes and float data gain a little from 512 x 8 (15.6 vs 16.4 us,
-  // float backward 40.0 vs 43.0 us).  Planes beyond 16 blocks of the largest
-  // shape are left to the other kernels.
+  // Block shape: positions per block PB = NL * TPR / 8 (128, 256, 512 or 1024);
+  // planes beyond 16 blocks of the largest shape are left to the other kernels.
+  // First choice, from a sweep of shapes (cold, forward / backward us):
+  //  groups, forward: 256 x 8, four blocks to a CU (float and planes from 4096
+  //    positions: 512 x 8 - [16,64,64,256] half 15.5 vs 15.7, float 25.0 vs 26.7);
+  //  groups, backward: 512 x 8 where that still gives two blocks per CU
+  //    ([16,64,64,256] 23.5 vs 25.4, [32,56,56,256] 38.7 vs 41.6), else 256 x 8
+  //    ([4,32,32,1024] 11.4 vs 12.4);
+  //  instances exchange 64 channels x 2 words per block and partner, so fewer,
+  //    larger blocks: 512 x 8 up to 2048 positions ([32,28,28,512] 14.6 / 21.6
+  //    against 20.9 / 40.9 with the line-piece kernels), 1024 x 8 beyond
+  //    ([16,64,64,256] 19.0 / 27.4 against 21.6 / 40.4);
+  //  any plane that one block of a smaller shape holds whole takes that shape.
   static const int shapes[][2] = {{256, 4}, {256, 8}, {512, 8}, {1024, 8}, {512, 4}, {1024, 4}};
   const int ftpr = tune_int("GN_CL_SPLIT_TPR", 0), fnl = tune_int("GN_CL_SPLIT_NL", 0);
   const bool forced = ftpr && fnl;
-  const bool large_first = p.spatial >= 4096 && (!backward || p.dtype == NBLAHIP_F32);
-  for (int pass = 0; pass < 2 && !s.ok; ++pass) {
-    for (int i = 0; i < (forced ? 6 : 4); ++i) {
-      const int *sh = shapes[i];
-      if (forced && (sh[0] != ftpr || sh[1] != fnl)) continue;
-      const int64_t pb = static_cast<int64_t>(sh[0]) * sh[1] / kSplitTV;
-      const int64_t split = (p.spatial + pb - 1) / pb;
-      if (split > kSplitMax) continue;
-      if (!forced) {
-        if (pass == 0 && large_first && sh[0] != 512) continue; // first choice for these
-        if (i == 0 && p.spatial > pb) continue;                 // 256 x 4 only for planes it holds whole
-      }
-      s.tpr = sh[0];
-      s.nl = sh[1];
-      s.pb = static_cast<int>(pb);
-      s.split = static_cast<int>(split);
-      s.ok = true;
-      break;
+  auto take = [&](int i) {
+    const int64_t pb = static_cast<int64_t>(shapes[i][0]) * shapes[i][1] / kSplitTV;
+    const int64_t split = (p.spatial + pb - 1) / pb;
+    if (split > kSplitMax) return false;
+    s.tpr = shapes[i][0];
+    s.nl = shapes[i][1];
+    s.pb = static_cast<int>(pb);
+    s.split = static_cast<int>(split);
+    s.ok = true;
+    return true;
+  };
+  if (forced) {
+    for (int i = 0; i < 6 && !s.ok; ++i)
+      if (shapes[i][0] == ftpr && shapes[i][1] == fnl) take(i);
+  } else {
+    int first = 1; // 256 x 8
+    if (p.spatial <= 128) {
+      first = 0;
+    } else if (p.spatial <= 256) {
+      first = 1;
+    } else if (s.instance) {
+      first = p.spatial <= 2048 ? 2 : 3;
+    } else if (backward) {
+      const int64_t blocks512 = p.batch * s.tiles * ((p.spatial + 511) / 512);
+      if (blocks512 >= 2 * static_cast<int64_t>(device_cus())) first = 2;
+    } else if (p.spatial >= 4096 || (p.dtype == NBLAHIP_F32 && p.spatial >= 2048)) {
+      first = 2;
     }
-    if (!large_first || forced) break;
+    for (int i = first; i < 4 && !s.ok; ++i) take(i);
   }
   if (!s.ok) return s;
   const int64_t blocks = p.batch * s.tiles * static_cast<int64_t>(s.split);

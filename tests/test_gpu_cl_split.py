@@ -1,4 +1,4 @@
-"""Channel-last GroupNormalization through the split kernels: a block owns
+"""Channel-last Group/InstanceNormalization through the split kernels: a block owns
 whole 128-byte lines of a range of positions and the blocks of a sample
 exchange partial sums (each partial one {value, epoch} word).  Parity against
 the oracle on the transposed tensor; the path a block takes when a partner's
@@ -223,3 +223,75 @@ def test_a_captured_graph_takes_the_other_kernels_and_replays_correctly():
             assert torch.equal(a_, b_), rep
         for a_, b_ in zip(split, outs):                      # same function, other summation order
             torch.testing.assert_close(a_.float(), b_.float(), rtol=2e-2, atol=2e-2)
+
+
+IN_SHAPES = [(3, (33, 33), 64), (2, (70, 70), 64), (5, (9, 9), 128), (2, (100, 100), 32), (2, (7,), 64),
+             (1, (127, 129), 64), (4, (16, 16), 256)]
+
+
+@pytest.mark.parametrize("n,sp,c", IN_SHAPES)
+@pytest.mark.parametrize("dtype", [F32, F16])
+def test_instances_through_the_split_kernels(n, sp, c, dtype):
+    dn = dtype_name(dtype)
+    eligible = c % (64 if dtype == F16 else 32) == 0
+    x, dy, g, b = make(n, sp, c, dtype, 23)
+    xt, dyt = to_cf(x), to_cf(dy)
+    y_r, m_r, v_r = R.in_forward(xt, b, g, n, c, 1e-5)
+    dx_r, dg_r, db_r = R.in_backward(xt, dyt, g, m_r, v_r, n, c, 1e-5)
+    xd, dyd, gd, bd = to_dev(x, dtype), to_dev(dy, dtype), to_dev(g), to_dev(b)
+
+    def run():
+        K.check(K.lib().nblahip_profile_enable(64))
+        y, m, v = K.in_forward(xd, bd, gd, 1e-5, channel_last=True)
+        dx, dgam, dbet = K.in_backward(xd, dyd, gd, m, v, 1e-5, channel_last=True)
+        torch.cuda.synchronize()
+        names = K.profile_kernels()
+        K.check(K.lib().nblahip_profile_enable(0))
+        return [y, m, v, dx, dgam, dbet], names
+
+    out, names = run()
+    assert ran(names) == eligible, names
+    y, m, v, dx, dgam, dbet = out
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    assert_close(to_np(y), to_cl(y_r.reshape(xt.shape)), dn, "y", "y")
+    assert_close(to_np(dx), to_cl(dx_r.reshape(xt.shape)), dn, "grad", "dx")
+    assert_close(to_np(dgam), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(dbet), db_r, dn, "pgrad", "dbeta")
+    if not eligible:
+        return
+    K.tune_set("XCHG_SPIN", 0)     # every partner's part recomputed: not a bit may change
+    out2, names2 = run()
+    assert ran(names2)
+    for a_, b_ in zip(out, out2):
+        assert torch.equal(a_, b_)
+
+
+def test_instance_flags_through_the_split_kernels():
+    """dmean/dvar, accumulation, parameter gradients only, no parameters."""
+    n, sp, c = 3, (24, 24), 64
+    rng = np.random.default_rng(10)
+    x, dy, g, b = make(n, sp, c, F32, 33)
+    xt, dyt = to_cf(x), to_cf(dy)
+    xd, dyd = to_dev(x), to_dev(dy)
+    K.check(K.lib().nblahip_profile_enable(64))
+    y_r, m_r, v_r = R.in_forward(xt, None, None, n, c, 1e-5)
+    y, m, v = K.in_forward(xd, None, None, 1e-5, channel_last=True)
+    assert_close(to_np(y), to_cl(y_r.reshape(xt.shape)), "f32", "y", "y no params")
+    dm, dv = f32(rng.standard_normal(n * c)), f32(rng.standard_normal(n * c))
+    y_r, m_r, v_r = R.in_forward(xt, b, g, n, c, 1e-5)
+    dx_r, dg_r, db_r = R.in_backward(xt, dyt, g, m_r, v_r, n, c, 1e-5, dmean=dm, dvar=dv)
+    y, m, v = K.in_forward(xd, to_dev(b), to_dev(g), 1e-5, channel_last=True)
+    pre_dx = rng.standard_normal(x.shape).astype(np.float32)
+    pre_g = rng.standard_normal(c).astype(np.float32)
+    dxd, dgd = to_dev(pre_dx), to_dev(pre_g)
+    K.in_backward(xd, dyd, to_dev(g), m, v, 1e-5, dmean=to_dev(dm), dvar=to_dev(dv), dx=dxd,
+                  dgamma=dgd, accum=(True, True, False), channel_last=True)
+    assert_close(to_np(dxd), to_cl(dx_r.reshape(xt.shape)) + pre_dx, "f32", "grad", "dx accum")
+    assert_close(to_np(dgd), dg_r + pre_g, "f32", "pgrad", "dgamma accum")
+    _, dgam, dbet = K.in_backward(xd, dyd, to_dev(g), m, v, 1e-5, dmean=to_dev(dm), dvar=to_dev(dv),
+                                  need=(False, True, True), channel_last=True)
+    assert_close(to_np(dgam), dg_r, "f32", "pgrad", "dgamma only")
+    assert_close(to_np(dbet), db_r, "f32", "pgrad", "dbeta only")
+    torch.cuda.synchronize()
+    assert ran(K.profile_kernels())

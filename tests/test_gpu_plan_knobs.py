@@ -201,24 +201,25 @@ SWITCHES = [
      ["gn_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], ["cl_split_fwd_kernel", "cl_split_bwd_kernel"]),
     ("gn_cl_split_off_float", run_gn, (2, 128, (20, 20), 8, F32, True), {"GN_CL_SPLIT": 0},
      ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"], ["cl_split_fwd_kernel", "cl_split_bwd_kernel"]),
-    ("in_cl_split_on", run_in, (4, 1024, (32, 32), F16, True), {"GN_CL_SPLIT_INSTANCES": 1},
-     ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], ["in_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"]),
-    ("in_cl_split_on_float", run_in, (3, 64, (19, 19), F32, True), {"GN_CL_SPLIT_INSTANCES": 1},
-     ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"]),
+    ("in_cl_split_off", run_in, (4, 1024, (32, 32), F16, True), {"GN_CL_SPLIT_INSTANCES": 0},
+     ["in_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], ["cl_split_fwd_kernel", "cl_split_bwd_kernel"]),
+    ("in_cl_split_off_float", run_in, (3, 64, (19, 19), F32, True), {"GN_CL_SPLIT_INSTANCES": 0},
+     ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"], ["cl_split_fwd_kernel", "cl_split_bwd_kernel"]),
     ("gn_cl_wide_off", run_gn, (4, 1024, (32, 32), 128, F16, True),
      {"GN_CL_WIDE": 0, "GN_CL_WIDE_BWD": 0}, ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"],
      ["gn_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], NO_SPLIT),
     ("in_cl_wide_off", run_in, (4, 1024, (32, 32), F16, True),
      {"GN_CL_WIDE": 0, "GN_CL_WIDE_BWD": 0}, ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"],
-     ["in_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"]),
+     ["in_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], NO_SPLIT),
     ("gn_cl_cached_off", run_gn, (2, 128, (20, 20), 8, F32, True), {"GN_CL_CACHED": 0},
      ["bn_stats_cl_kernel", "gn_cl_finalize_fwd_kernel", "bn_bwd_reduce_cl_kernel",
       "gn_cl_finalize_bwd_kernel"], ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"], NO_SPLIT),
     ("in_cl_cached_off", run_in, (2, 128, (20, 20), F32, True), {"IN_CL_CACHED": 0},
      ["bn_stats_cl_kernel", "gn_cl_finalize_fwd_kernel", "gn_cl_finalize_bwd_kernel"],
-     ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"]),
+     ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"], NO_SPLIT),
     ("in_cl_min_positions_up", run_in, (4, 64, (8, 8), F16, True), {"IN_CL_MIN": 128},
-     ["bn_stats_cl_kernel", "bn_bwd_reduce_cl_kernel"], ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"]),
+     ["bn_stats_cl_kernel", "bn_bwd_reduce_cl_kernel"], ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"],
+     NO_SPLIT),
 ]
 
 
@@ -288,13 +289,13 @@ GRIDS = [
      ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], []),
     ("gn_cl_split_no_polls", run_gn, (3, 128, (40, 40), 16, F16, True), [{"XCHG_SPIN": 0}],
      ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], []),
-    ("in_cl_split_no_polls", run_in, (2, 64, (30, 30), F32, True),
-     [{"XCHG_SPIN": 0, "GN_CL_SPLIT_INSTANCES": 1}],
+    ("in_cl_split_no_polls", run_in, (2, 64, (30, 30), F32, True), [{"XCHG_SPIN": 0}],
      ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], []),
     ("gn_cl_wide_plain_block_order", run_gn, (4, 1024, (32, 32), 128, F16, True),
      [{"GN_CL_XCD_MAP": 0, **NO_SPLIT}],
      ["gn_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], []),
-    ("in_cl_wide_plain_block_order", run_in, (4, 1024, (32, 32), F16, True), [{"GN_CL_XCD_MAP": 0}],
+    ("in_cl_wide_plain_block_order", run_in, (4, 1024, (32, 32), F16, True),
+     [{"GN_CL_XCD_MAP": 0, **NO_SPLIT}],
      ["in_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], []),
     # four groups per block, 16 vectors per thread, on a quarter of the CUs
     ("gn_cl_wide_fewer_blocks", run_gn, (8, 256, (64, 64), 32, F16, True),
@@ -304,9 +305,9 @@ GRIDS = [
      [{"GN_CL_XCD_MAP": 0, **NO_SPLIT}],
      ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"], []),
     ("in_cl_rows_plain_block_order", run_in, (2, 128, (20, 20), F16, True),
-     [{"GN_CL_XCD_MAP": 0, "GN_CL_WIDE": 0, "GN_CL_WIDE_BWD": 0}],
+     [{"GN_CL_XCD_MAP": 0, "GN_CL_WIDE": 0, "GN_CL_WIDE_BWD": 0, **NO_SPLIT}],
      ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"], []),
-    ("in_cl_fewer_positions", run_in, (4, 64, (4, 4), F16, True), [{"IN_CL_MIN": 8}],
+    ("in_cl_fewer_positions", run_in, (4, 64, (4, 4), F16, True), [{"IN_CL_MIN": 8, **NO_SPLIT}],
      ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"], []),
 ]
 
