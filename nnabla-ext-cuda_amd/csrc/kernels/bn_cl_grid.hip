@@ -65,6 +65,9 @@ __device__ __forceinline__ uint32_t grid_block_vectors(const BnClGridArgs &a, ui
 // same channel vector (t % cv): butterfly over the lanes cv apart, one row of
 // fold[16][C] per wave, the rows added in wave order by one thread per channel
 // (tot[C]), and every thread reads back its channels' totals.
+// (No barrier ahead of the first write: every earlier reader of fold has passed
+// the last barrier of the call before, and so has every reader of tot by the
+// time tot is written again, two barriers further on.)
 template <int VEC>
 __device__ __forceinline__ void grid_channel_sums(float (&v)[VEC], uint32_t cv, uint32_t cvx,
                                                   float *fold, float *tot, uint32_t C) {
@@ -73,7 +76,6 @@ __device__ __forceinline__ void grid_channel_sums(float (&v)[VEC], uint32_t cv, 
   for (int j = 0; j < VEC; ++j) {
     for (uint32_t off = cv; off < kWave; off <<= 1) v[j] += __shfl_xor(v[j], off);
   }
-  lds_barrier(); // earlier readers of fold / tot are done
   if ((threadIdx.x & (kWave - 1)) < cv) {
 #pragma unroll
     for (int j = 0; j < VEC; ++j) fold[(threadIdx.x / kWave) * C + cvx * VEC + j] = v[j];
@@ -148,7 +150,7 @@ __device__ __forceinline__ void grid_partial_from_memory(const BnClGridArgs &a, 
 
 // Merged (mean, var) of channel c over all blocks: thread p < nblocks takes
 // block p's partial (polled; computed here if it does not arrive), the block
-// merges them in a fixed tree.  Same result in every thread and in every block
+// merges them in a fixed order.  Same result in every thread and in every block
 // that calls it.  scratch: miss[kGridMaxBlocks] ints, got[2 * kGridMaxBlocks],
 // wel[3 * 16], fold[16 * C].
 template <typename T, int VEC>
@@ -178,15 +180,17 @@ __device__ __forceinline__ void grid_channel_result(const BnClGridArgs &a, uint3
     }
     lds_barrier();
   }
-  Welford w{0.f, 0.f, 0.f};
+  // mean = sum n_p * mean_p / N, m2 = sum (m2_p + n_p * (mean_p - mean)^2): two
+  // block sums in a fixed order (a Chan merge tree over 256 partials took 2.5 us)
+  float np = 0.f, mp = 0.f, qp = 0.f;
   if (t < a.nblocks) {
-    w.mean = got[2 * t];
-    w.m2 = got[2 * t + 1];
-    w.n = static_cast<float>(grid_block_vectors(a, t) / a.cv);
+    mp = got[2 * t];
+    qp = got[2 * t + 1];
+    np = static_cast<float>(grid_block_vectors(a, t) / a.cv);
   }
-  w = block_welford(w, wel);
-  mean = w.mean;
-  var = w.m2 * a.inv_N;
+  mean = onchip_block_sum(np * mp, wel) * a.inv_N;
+  const float d = mp - mean;
+  var = onchip_block_sum(fmaf(np * d, d, qp), wel) * a.inv_N;
 }
 
 } // namespace
@@ -391,11 +395,11 @@ bool bn_cl_grid_fwd_train(const BnProblem &p, hipStream_t st, int *status) {
   const int64_t vb = rows_pb * cv;
   const int nl = static_cast<int>((vb + kOnchipBlock - 1) / kOnchipBlock);
   const int64_t nblocks = (M + rows_pb - 1) / rows_pb;
-  // Up to what the chip holds, and from 10 vectors per thread: the exchange and
-  // the folds cost about 12 us whatever the size, one read of x saves 0.16 us
-  // per MB ([256,56,56,64] half 57.5 -> 51.2 us, [128,56,56,64] 35.6 -> 32.7 us,
-  // [64,56,56,64] 24.1 us either way, [32,56,56,64] 18.4 -> 21.8 us).
-  if (nl < tune_int("BN_CL_GRID_MIN_SLOTS", 10) || nl > 25 || nblocks < blocks / 2) return false;
+  // Up to what the chip holds, and from 6 vectors per thread: the exchange and
+  // the folds cost about 9 us whatever the size, one read of x saves 0.16 us
+  // per MB ([256,56,56,64] half 57.8 -> 49.4 us, [128,56,56,64] 35.0 -> 30.9 us,
+  // [64,56,56,64] 24.1 -> 22.0 us, [32,56,56,64] 18.4 -> 19.5 us).
+  if (nl < tune_int("BN_CL_GRID_MIN_SLOTS", 6) || nl > 25 || nblocks < blocks / 2) return false;
   BnClGridArgs a{};
   a.x = p.x;
   a.y = p.out;
