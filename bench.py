@@ -105,7 +105,13 @@ BN_ONCHIP_BWD_HELD, BN_ONCHIP_BWD_WHOLE = 18432, 20480
 BN_ONCHIP_FWD_HELD = 25600
 
 
-def bn_tensor_passes(K, fwd, bwd, vectors_per_channel=0):
+# bn_cl_grid_bwd_kernel (channel-last, the whole tensor on the chip's 256 CUs)
+# holds 21 x 1024 vectors of x per block and reads what a block has beyond that
+# twice, like dy: x, 2 dy, dx = 4 passes + the part of x not held.
+BN_CL_GRID_BWD_HELD, BN_CL_GRID_BLOCKS = 21 * 1024, 256
+
+
+def bn_tensor_passes(K, fwd, bwd, vectors_per_channel=0, channel_last_vectors=0):
     """(forward, backward) tensor passes of the plan the library picks for this
     workload: a pass counts when the channel cannot stay on chip between the
     statistics and the apply phase.  Read off the kernels one call launches."""
@@ -124,6 +130,9 @@ def bn_tensor_passes(K, fwd, bwd, vectors_per_channel=0):
             pb = passes
             if k == "bn_onchip_bwd_kernel" and vectors_per_channel > BN_ONCHIP_BWD_WHOLE:
                 pb += (vectors_per_channel - BN_ONCHIP_BWD_HELD) / vectors_per_channel
+    if K.profile_query("bn_cl_grid_bwd_kernel")[1]:
+        per_block = -(-channel_last_vectors // BN_CL_GRID_BLOCKS)
+        pb = 4 + max(0, per_block - BN_CL_GRID_BWD_HELD) / max(1, per_block)
     K.check(L.nblahip_profile_enable(0))
     return pf, pb
 
@@ -221,7 +230,8 @@ def make_bn(K, name, shape, axis, dtype, train, mean=0.0, std=1.0, outliers=Fals
         # (vectors are 16 bytes, 8 for half planes of 4k - not 8k - elements)
         esz = sets[0]["x"].element_size()
         vec_bytes = 8 if esz == 2 and s2 % 8 != 0 and s2 % 4 == 0 else 16
-        pf, pb = bn_tensor_passes(K, fwd, bwd, s0 * s2 * esz // vec_bytes)
+        pf, pb = bn_tensor_passes(K, fwd, bwd, s0 * s2 * esz // vec_bytes,
+                                  s0 * c * esz // 16 if s2 == 1 else 0)
         # the probe call moved the running statistics of set 0: start over
         sets[0]["rm"].copy_(up(rm0))
         sets[0]["rv"].copy_(up(rv0))

@@ -49,7 +49,14 @@ struct BnClGridArgs {
   uint32_t vb;      // vectors per block (whole rows)
   uint32_t nblocks;
   float inv_N, unbias, decay, eps, one;
+  // backward
+  const void *dy;
+  void *dx;                  // may be null
+  const float *dmean, *dvar; // may be null
+  float *dgamma, *dbeta;     // may be null
+  int accum_dx, accum_g, accum_b;
   unsigned long long *x1; // stage 1: [nblocks][C][2] = (mean, m2) of the block's rows
+                          //          (backward: (sum dy*xh, sum dy))
   unsigned long long *x2; // stage 2: [nblocks][C][2] = (mean, var), a copy for every block
   uint32_t epoch;
   int spin;
@@ -191,6 +198,74 @@ __device__ __forceinline__ void grid_channel_result(const BnClGridArgs &a, uint3
   mean = onchip_block_sum(np * mp, wel) * a.inv_N;
   const float d = mp - mean;
   var = onchip_block_sum(fmaf(np * d, d, qp), wel) * a.inv_N;
+}
+
+// Backward: (sum dy*xh, sum dy) of the rows of block p for channel c, from
+// global memory, in block p's own order (vectors k * 1024 + t ascending per
+// thread, the same folds): what block p publishes for c, bit for bit.
+template <typename T, int VEC>
+__device__ __forceinline__ void grid_pair_from_memory(const BnClGridArgs &a, uint32_t p,
+                                                      uint32_t c, float *fold, float &sdx,
+                                                      float &sdy) {
+  const T *__restrict__ x = static_cast<const T *>(a.x);
+  const T *__restrict__ dy = static_cast<const T *>(a.dy);
+  const uint32_t t = threadIdx.x;
+  const uint32_t cvx = t % a.cv, e = c % VEC;
+  const uint32_t vbp = cvx == c / VEC ? grid_block_vectors(a, p) : 0u;
+  const size_t first = static_cast<size_t>(p) * a.vb;
+  const float mean = a.mean[c];
+  const float istd = 1.0f / sqrtf(a.var[c] + a.eps);
+  const float nmi = -mean * istd;
+  sdx = 0.f;
+  sdy = 0.f;
+#pragma unroll 1
+  for (uint32_t v = t; v < vbp; v += kOnchipBlock) {
+    const RawVec<T, VEC> xr = load_raw<T, VEC>(x + (first + v) * VEC);
+    const RawVec<T, VEC> dr = load_raw<T, VEC>(dy + (first + v) * VEC);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float xh = norm_elem<T, VEC>(xr, j, mean, istd, nmi);
+      const float nx = elem_fma<T, VEC>(dr, j, xh, sdx);
+      const float ny = elem_fma<T, VEC>(dr, j, a.one, sdy);
+      sdx = static_cast<uint32_t>(j) == e ? nx : sdx;
+      sdy = static_cast<uint32_t>(j) == e ? ny : sdy;
+    }
+  }
+  sdx = grid_channel_sum1(sdx, a.cv, cvx, c, cvx == c / VEC, fold, a.C);
+  sdy = grid_channel_sum1(sdy, a.cv, cvx, c, cvx == c / VEC, fold, a.C);
+}
+
+// Backward: (sum dy*xh, sum dy) of channel c over all blocks, in block order.
+// Same structure and scratch as grid_channel_result.
+template <typename T, int VEC>
+__device__ __forceinline__ void grid_pair_result(const BnClGridArgs &a, uint32_t c, int *miss,
+                                                 float *got, float *wel, float *fold, float &sdx,
+                                                 float &sdy) {
+  const uint32_t t = threadIdx.x;
+  lds_barrier(); // got / miss of an earlier call have been consumed
+  if (t == 0) miss[kGridMaxBlocks] = 0;
+  lds_barrier();
+  if (t < a.nblocks) {
+    float v0 = 0.f, v1 = 0.f;
+    const bool ok = xchg_poll2(a.x1 + (static_cast<size_t>(t) * a.C + c) * 2, a.epoch, a.spin, &v0, &v1);
+    got[2 * t] = v0;
+    got[2 * t + 1] = v1;
+    miss[t] = ok ? 0 : 1;
+    if (!ok) miss[kGridMaxBlocks] = 1;
+  }
+  lds_barrier();
+  for (uint32_t p = 0; miss[kGridMaxBlocks] && p < a.nblocks; ++p) {
+    if (!miss[p]) continue; // same answer in every thread
+    float px, py;
+    grid_pair_from_memory<T, VEC>(a, p, c, fold, px, py);
+    if (t == 0) {
+      got[2 * p] = px;
+      got[2 * p + 1] = py;
+    }
+    lds_barrier();
+  }
+  sdx = onchip_block_sum(t < a.nblocks ? got[2 * t] : 0.f, wel);
+  sdy = onchip_block_sum(t < a.nblocks ? got[2 * t + 1] : 0.f, wel);
 }
 
 } // namespace
@@ -357,6 +432,222 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
   }
 }
 
+// Backward (batch statistics).  With xh = (x-mean)*istd per channel:
+//   sdx = sum dy*xh (= dgamma), sdy = sum dy (= dbeta),
+//   dx = dy*g*istd + xh*cA + cb,  cA = -istd*g*sdx/N + 2*dvar*std/N,
+//   cb = -g*sdy*istd/N + dmean/N.
+// x is held as in the forward (NR + NS vectors per thread; what a block has
+// beyond that is streamed with dy in both passes), dy is streamed twice in
+// batches of B vectors; the blocks exchange (sdx, sdy) per channel in the
+// forward's two stages, block c writing dgamma[c] / dbeta[c].
+template <typename T, int VEC, int NR, int NS, int B>
+__global__ void __launch_bounds__(kOnchipBlock)
+bn_cl_grid_bwd_kernel(const BnClGridArgs a) {
+  static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors");
+  constexpr int NL = NR + NS;
+  __shared__ uint4 spill[NS > 0 ? NS * kOnchipBlock : 1];
+  __shared__ float fold[16 * kGridMaxC];
+  __shared__ float tot[kGridMaxC];
+  __shared__ float fin[2 * kGridMaxC]; // (sdx, sdy) totals per channel
+  __shared__ int finmiss[kGridMaxC];
+  __shared__ float got[2 * kGridMaxBlocks];
+  __shared__ int miss[kGridMaxBlocks + 2];
+  __shared__ float wel[16];
+  const uint32_t b = blockIdx.x;
+  const uint32_t t = threadIdx.x;
+  const uint32_t cvx = t % a.cv;
+  const uint32_t ch = cvx * VEC;
+  const uint32_t vbb = grid_block_vectors(a, b);
+  const size_t base = static_cast<size_t>(b) * a.vb * VEC;
+  const T *__restrict__ x = static_cast<const T *>(a.x) + base;
+  const T *__restrict__ dy = static_cast<const T *>(a.dy) + base;
+  T *__restrict__ dx = a.dx ? static_cast<T *>(a.dx) + base : nullptr;
+  const uint32_t last = vbb - 1;
+
+  RawVec<T, VEC> raw[NR];
+  {
+    RawVec<T, VEC> parked[NS > 0 ? NS : 1];
+#pragma unroll
+    for (int k = 0; k < NS; ++k) {
+      const uint32_t v = static_cast<uint32_t>(NR + k) * kOnchipBlock + t;
+      parked[k] = load_raw<T, VEC>(x + static_cast<size_t>(min(v, last)) * VEC);
+    }
+#pragma unroll
+    for (int k = 0; k < NR; ++k) {
+      const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t;
+      raw[k] = load_raw<T, VEC>(x + static_cast<size_t>(min(v, last)) * VEC);
+    }
+#pragma unroll
+    for (int k = 0; k < NS; ++k) spill[k * kOnchipBlock + t] = __builtin_bit_cast(uint4, parked[k]);
+  }
+  auto slot = [&](int k) -> RawVec<T, VEC> {
+    if (k < NR) return raw[k < NR ? k : 0];
+    return __builtin_bit_cast(RawVec<T, VEC>, spill[(k - NR) * kOnchipBlock + t]);
+  };
+  float mean[VEC], istd[VEC], nmi[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    mean[j] = a.mean[ch + j];
+    istd[j] = 1.0f / sqrtf(a.var[ch + j] + a.eps);
+    nmi[j] = -mean[j] * istd[j];
+  }
+
+  // ---- pass 1: the block's (sum dy*xh, sum dy) per channel, vectors ascending
+  float sdx[VEC], sdy[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) sdx[j] = sdy[j] = 0.f;
+#pragma unroll
+  for (int k0 = 0; k0 < NL; k0 += B) {
+    const uint32_t t1 = fresh_after(t, sdx[0]);
+    RawVec<T, VEC> d[B];
+#pragma unroll
+    for (int i = 0; i < B; ++i) {
+      const uint32_t v = static_cast<uint32_t>(k0 + i) * kOnchipBlock + t1;
+      d[i] = load_raw<T, VEC>(dy + static_cast<size_t>(min(v, last)) * VEC);
+    }
+#pragma unroll
+    for (int i = 0; i < B; ++i) {
+      const int k = k0 + i;
+      if (k < NL && static_cast<uint32_t>(k) * kOnchipBlock + t < vbb) {
+        const RawVec<T, VEC> xr = slot(k);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float xh = norm_elem<T, VEC>(xr, j, mean[j], istd[j], nmi[j]);
+          sdx[j] = elem_fma<T, VEC>(d[i], j, xh, sdx[j]);
+          sdy[j] = elem_fma<T, VEC>(d[i], j, a.one, sdy[j]);
+        }
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0); // the next batch's loads stay below: hoisted, the batches add up
+  }
+#pragma unroll 1
+  for (uint32_t v = static_cast<uint32_t>(NL) * kOnchipBlock + t; v < vbb; v += kOnchipBlock) {
+    const RawVec<T, VEC> xr = load_raw<T, VEC>(x + static_cast<size_t>(v) * VEC);
+    const RawVec<T, VEC> dr = load_raw<T, VEC>(dy + static_cast<size_t>(v) * VEC);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float xh = norm_elem<T, VEC>(xr, j, mean[j], istd[j], nmi[j]);
+      sdx[j] = elem_fma<T, VEC>(dr, j, xh, sdx[j]);
+      sdy[j] = elem_fma<T, VEC>(dr, j, a.one, sdy[j]);
+    }
+  }
+  grid_channel_sums<VEC>(sdx, a.cv, cvx, fold, tot, a.C);
+  if (t < a.cv) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) fin[ch + j] = sdx[j];
+  }
+  grid_channel_sums<VEC>(sdy, a.cv, cvx, fold, tot, a.C);
+  // (fin's stores precede the barriers of the second fold: visible by now)
+  for (uint32_t e = t; e < 2 * a.C; e += kOnchipBlock)
+    xchg_publish(a.x1 + static_cast<size_t>(b) * a.C * 2 + e, (e & 1) ? tot[e >> 1] : fin[e >> 1], a.epoch);
+
+  // ---- stage 2: block c sums channel c over the blocks, writes dgamma / dbeta, publishes
+  for (uint32_t c = b; c < a.C; c += a.nblocks) {
+    float tx, ty;
+    grid_pair_result<T, VEC>(a, c, miss, got, wel, fold, tx, ty);
+    if (t == 0) {
+      if (a.dgamma) a.dgamma[c] = tx + (a.accum_g ? a.dgamma[c] : 0.f);
+      if (a.dbeta) a.dbeta[c] = ty + (a.accum_b ? a.dbeta[c] : 0.f);
+    }
+    if (t < a.nblocks) { // a copy for block t
+      unsigned long long *w = a.x2 + (static_cast<size_t>(t) * a.C + c) * 2;
+      xchg_publish(w, tx, a.epoch);
+      xchg_publish(w + 1, ty, a.epoch);
+    }
+  }
+  if (dx == nullptr) return;
+
+  // ---- every block: the C totals (summed here where one does not arrive)
+  lds_barrier();
+  if (t == 0) miss[kGridMaxBlocks + 1] = 0;
+  lds_barrier();
+  for (uint32_t c = t; c < a.C; c += kOnchipBlock) {
+    float v0 = 0.f, v1 = 0.f;
+    const bool ok = xchg_poll2(a.x2 + (static_cast<size_t>(b) * a.C + c) * 2, a.epoch, a.spin, &v0, &v1);
+    fin[2 * c] = v0;
+    fin[2 * c + 1] = v1;
+    finmiss[c] = ok ? 0 : 1;
+    if (!ok) miss[kGridMaxBlocks + 1] = 1;
+  }
+  lds_barrier();
+  for (uint32_t c = 0; miss[kGridMaxBlocks + 1] && c < a.C; ++c) {
+    if (!finmiss[c]) continue; // same answer in every thread
+    float tx, ty;
+    grid_pair_result<T, VEC>(a, c, miss, got, wel, fold, tx, ty);
+    lds_barrier();
+    if (t == 0) {
+      fin[2 * c] = tx;
+      fin[2 * c + 1] = ty;
+    }
+    lds_barrier();
+  }
+
+  // ---- pass 2: dx = dy*gi + (x - mean)*A2 + cb  (half: x*A2 + B2, one mixed fma)
+#pragma unroll
+  for (int k = 0; k < NR; ++k) forget<T, VEC>(raw[k]);
+  float gi[VEC], A2[VEC], B2[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    const float g = a.gamma ? a.gamma[ch + j] : 1.f;
+    const float vpe = a.var[ch + j] + a.eps;
+    const float cA = -istd[j] * g * fin[2 * (ch + j)] * a.inv_N +
+                     (a.dvar ? 2.f * a.dvar[ch + j] * (vpe * istd[j]) * a.inv_N : 0.f);
+    const float cb = -g * fin[2 * (ch + j) + 1] * istd[j] * a.inv_N +
+                     (a.dmean ? a.dmean[ch + j] * a.inv_N : 0.f);
+    gi[j] = g * istd[j];
+    A2[j] = istd[j] * cA;
+    B2[j] = sizeof(T) == 2 ? fmaf(nmi[j], cA, cb) : cb;
+  }
+  auto emit = [&](const RawVec<T, VEC> &xr, const RawVec<T, VEC> &dr, uint32_t v) {
+    float o[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      float xt;
+      if constexpr (sizeof(T) == 2) {
+        xt = elem_fma<T, VEC>(xr, j, A2[j], B2[j]);
+      } else {
+        xt = fmaf(elem_fma<T, VEC>(xr, j, a.one, -mean[j]), A2[j], B2[j]);
+      }
+      o[j] = elem_fma<T, VEC>(dr, j, gi[j], xt);
+    }
+    T *dst = dx + static_cast<size_t>(v) * VEC;
+    if (a.accum_dx) {
+      float old[VEC];
+      load_vec<T, VEC>(dst, old);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) o[j] += old[j];
+    }
+    store_vec<T, VEC>(dst, o);
+  };
+  float lastv = B2[0];
+#pragma unroll
+  for (int k0 = 0; k0 < NL; k0 += B) {
+    const uint32_t t2 = fresh_after(t, lastv);
+    RawVec<T, VEC> d[B];
+#pragma unroll
+    for (int i = 0; i < B; ++i) {
+      const uint32_t v = static_cast<uint32_t>(k0 + i) * kOnchipBlock + t2;
+      d[i] = load_raw<T, VEC>(dy + static_cast<size_t>(min(v, last)) * VEC);
+    }
+#pragma unroll
+    for (int i = 0; i < B; ++i) {
+      const int k = k0 + i;
+      const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t2;
+      if (k < NL && v < vbb) {
+        emit(slot(k), d[i], v);
+        lastv = __builtin_bit_cast(float, __builtin_bit_cast(uint4, d[i]).x);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll 1
+  for (uint32_t v = static_cast<uint32_t>(NL) * kOnchipBlock + t; v < vbb; v += kOnchipBlock) {
+    const RawVec<T, VEC> xr = load_raw<T, VEC>(x + static_cast<size_t>(v) * VEC);
+    const RawVec<T, VEC> dr = load_raw<T, VEC>(dy + static_cast<size_t>(v) * VEC);
+    emit(xr, dr, v);
+  }
+}
+
 namespace {
 
 template <typename T, int VEC>
@@ -380,38 +671,55 @@ int run_grid_fwd(int nl, const BnClGridArgs &a, hipStream_t st) {
 
 } // namespace
 
-bool bn_cl_grid_fwd_train(const BnProblem &p, hipStream_t st, int *status) {
+namespace {
+
+template <typename T, int VEC>
+int run_grid_bwd(int nl, const BnClGridArgs &a, hipStream_t st) {
+#define GRID_CASE(NR, NS)                                                                        \
+  if (nl <= (NR) + (NS)) {                                                                       \
+    NBLAHIP_LAUNCH("bn_cl_grid_bwd_kernel", (bn_cl_grid_bwd_kernel<T, VEC, NR, NS, (sizeof(T) == 2 ? 2 : 4)>),          \
+                   dim3(a.nblocks), dim3(kOnchipBlock), 0, st, a);                               \
+    return last_launch_status();                                                                 \
+  }
+  GRID_CASE(4, 0)
+  GRID_CASE(8, 0)
+  GRID_CASE(12, 0)
+  GRID_CASE(12, 3)
+  GRID_CASE(12, 6)
+  GRID_CASE(12, 9)
+#undef GRID_CASE
+  // more per thread than the 21 vectors held: the rest is streamed with dy
+  NBLAHIP_LAUNCH("bn_cl_grid_bwd_kernel", (bn_cl_grid_bwd_kernel<T, VEC, 12, 9, (sizeof(T) == 2 ? 2 : 4)>),
+                 dim3(a.nblocks), dim3(kOnchipBlock), 0, st, a);
+  return last_launch_status();
+}
+
+// Shape test and the arguments both directions share; nl = vectors per thread.
+bool grid_args(const BnProblem &p, BnClGridArgs &a, int &nl) {
   if (!tune_int("BN_CL_GRID", 1)) return false;
-  if (p.size2 != 1 || p.relu || p.z || p.y || p.sums_out || p.sums_in || !p.out) return false;
+  if (p.size2 != 1 || p.relu || p.z || p.y || p.dz || p.sums_out || p.sums_in) return false;
   const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
-  if (p.C % vec != 0 || p.C > kGridMaxC || !aligned16(p.x) || !aligned16(p.out)) return false;
+  if (p.C % vec != 0 || p.C > kGridMaxC || !aligned16(p.x) || (p.out && !aligned16(p.out))) return false;
   const int64_t cv = p.C / vec;
   if ((cv & (cv - 1)) != 0 || cv > kWave) return false;
   const int64_t M = p.size0;
-  const int64_t nv = M * cv;
   const int blocks = std::min(device_cus(), kGridMaxBlocks);
   // whole rows per block, the same for every block but the last
   const int64_t rows_pb = (M + blocks - 1) / blocks;
   const int64_t vb = rows_pb * cv;
-  const int nl = static_cast<int>((vb + kOnchipBlock - 1) / kOnchipBlock);
+  nl = static_cast<int>((vb + kOnchipBlock - 1) / kOnchipBlock);
   const int64_t nblocks = (M + rows_pb - 1) / rows_pb;
   // Up to what the chip holds, and from 6 vectors per thread: the exchange and
   // the folds cost about 9 us whatever the size, one read of x saves 0.16 us
   // per MB ([256,56,56,64] half 57.8 -> 49.4 us, [128,56,56,64] 35.0 -> 30.9 us,
   // [64,56,56,64] 24.1 -> 22.0 us, [32,56,56,64] 18.4 -> 19.5 us).
   if (nl < tune_int("BN_CL_GRID_MIN_SLOTS", 6) || nl > 25 || nblocks < blocks / 2) return false;
-  BnClGridArgs a{};
+  a = BnClGridArgs{};
   a.x = p.x;
-  a.y = p.out;
   a.gamma = p.gamma;
-  a.beta = p.beta;
-  a.mean = p.batch_mean;
-  a.var = p.batch_var;
-  a.rmean = p.rmean;
-  a.rvar = p.rvar;
   a.C = static_cast<uint32_t>(p.C);
   a.cv = static_cast<uint32_t>(cv);
-  a.nv = static_cast<uint32_t>(nv);
+  a.nv = static_cast<uint32_t>(M * cv);
   a.vb = static_cast<uint32_t>(vb);
   a.nblocks = static_cast<uint32_t>(nblocks);
   const double N = static_cast<double>(M);
@@ -421,10 +729,52 @@ bool bn_cl_grid_fwd_train(const BnProblem &p, hipStream_t st, int *status) {
   a.eps = p.eps;
   a.one = 1.0f;
   a.spin = tune_int("XCHG_SPIN", 64) * 16; // a whole-chip exchange: wait longer before recomputing
-  const size_t words = static_cast<size_t>(nblocks) * p.C * 4;
-  if (!xchg_acquire(words, st, &a.x1, &a.epoch, status)) return *status != 0;
-  a.x2 = a.x1 + static_cast<size_t>(nblocks) * p.C * 2;
+  return true;
+}
+
+// Exchange words of both stages.
+bool grid_exchange(const BnProblem &p, BnClGridArgs &a, hipStream_t st, int *status) {
+  const size_t words = static_cast<size_t>(a.nblocks) * p.C * 4;
+  if (!xchg_acquire(words, st, &a.x1, &a.epoch, status)) return false;
+  a.x2 = a.x1 + static_cast<size_t>(a.nblocks) * p.C * 2;
+  return true;
+}
+
+} // namespace
+
+bool bn_cl_grid_fwd_train(const BnProblem &p, hipStream_t st, int *status) {
+  BnClGridArgs a;
+  int nl = 0;
+  if (!p.out || !grid_args(p, a, nl)) return false;
+  a.y = p.out;
+  a.beta = p.beta;
+  a.mean = p.batch_mean;
+  a.var = p.batch_var;
+  a.rmean = p.rmean;
+  a.rvar = p.rvar;
+  if (!grid_exchange(p, a, st, status)) return *status != 0;
   *status = p.dtype == NBLAHIP_F16 ? run_grid_fwd<__half, 8>(nl, a, st) : run_grid_fwd<float, 4>(nl, a, st);
+  return true;
+}
+
+bool bn_cl_grid_bwd(const BnProblem &p, hipStream_t st, int *status) {
+  BnClGridArgs a;
+  int nl = 0;
+  if (!p.batch_stat || !tune_int("BN_CL_GRID_BWD", 1) || !grid_args(p, a, nl)) return false;
+  if (!aligned16(p.dy)) return false;
+  a.dy = p.dy;
+  a.dx = p.out;
+  a.mean = const_cast<float *>(p.mean);
+  a.var = const_cast<float *>(p.var);
+  a.dmean = p.dmean;
+  a.dvar = p.dvar;
+  a.dgamma = p.dgamma;
+  a.dbeta = p.dbeta;
+  a.accum_dx = p.accum_dx;
+  a.accum_g = p.accum_g;
+  a.accum_b = p.accum_b;
+  if (!grid_exchange(p, a, st, status)) return *status != 0;
+  *status = p.dtype == NBLAHIP_F16 ? run_grid_bwd<__half, 8>(nl, a, st) : run_grid_bwd<float, 4>(nl, a, st);
   return true;
 }
 

@@ -467,6 +467,7 @@ int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
     if (bn_rows_bwd(p, st, &status)) return status;
     if (bn_onchip_bwd(p, st, &status)) return status;
     if (bn_cl_cached_bwd(p, st, &status)) return status;
+    if (bn_cl_grid_bwd(p, st, &status)) return status;
   }
   const bool al = aligned16(p.x) && aligned16(p.dy) && (!p.out || aligned16(p.out)) &&
                   (!p.y || aligned16(p.y)) && (!p.dz || aligned16(p.dz));

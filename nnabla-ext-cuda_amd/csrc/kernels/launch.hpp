@@ -142,6 +142,7 @@ bool bn_cl_cached_fwd_train(const BnProblem &p, hipStream_t st, int *status);
 // Channel-last training forward with the whole tensor held on the chip's CUs
 // and the per-channel partials exchanged between the blocks (bn_cl_grid.hip).
 bool bn_cl_grid_fwd_train(const BnProblem &p, hipStream_t st, int *status);
+bool bn_cl_grid_bwd(const BnProblem &p, hipStream_t st, int *status);
 bool bn_cl_cached_bwd(const BnProblem &p, hipStream_t st, int *status);
 int launch_bn_infer(const BnProblem &p, hipStream_t st);
 int launch_bn_fwd_train(const BnProblem &p, hipStream_t st);

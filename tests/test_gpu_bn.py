@@ -443,6 +443,68 @@ def test_bn_channel_last_held_on_the_chip(m, c, dtype):
     assert_close(to_np(split[2]), to_np(var), dn, "stat", "var against the split reduction")
 
 
+@pytest.mark.parametrize("m,c,dtype", [(100352, 64, torch.float16), (100353, 64, torch.float16),
+                                       (200000, 32, torch.float32), (150000, 128, torch.float16),
+                                       (1000001, 8, torch.float16), (40000, 128, torch.float32),
+                                       # more of x than a block holds: the rest is read again
+                                       (750000, 64, torch.float16), (380000, 64, torch.float32)])
+def test_bn_channel_last_backward_held_on_the_chip(m, c, dtype):
+    """Backward with x held on the chip and the (sum dy*xh, sum dy) pairs
+    exchanged: against the oracle with the 3-output terms, bit-identical when no
+    poll is allowed, close to the split reduction; accumulation and the
+    parameters-only call."""
+    dn = dtype_name(dtype)
+    x, dy, g, b, _, _ = make_bn((m, c), 1, dtype, 6, mean=1.0, std=2.0)
+    rng = np.random.default_rng(7)
+    dm, dv = rng.standard_normal(c), rng.standard_normal(c)
+    _, m_r, v_r, _, _ = R.bn_forward_batch(x, b, g, None, None, 1, 0.9, 1e-5)
+    dx_r, dg_r, db_r = R.bn_backward_batch(x, dy, g, m_r, v_r, 1, 1e-5, dm, dv)
+    xd, dyd, gd = to_dev(x, dtype), to_dev(dy, dtype), to_dev(g)
+    md, vd, dmd, dvd = to_dev(m_r), to_dev(v_r), to_dev(dm), to_dev(dv)
+    pre_dx = rounded(rng.standard_normal((m, c)), dtype)
+    pre_g, pre_b = rng.standard_normal(c), rng.standard_normal(c)
+
+    def run(knobs, **kw):
+        K.tune_reset()
+        for k_, val in knobs.items():
+            K.tune_set(k_, val)
+        K.check(K.lib().nblahip_profile_enable(16))
+        out = K.bn_backward(xd, dyd, gd, md, vd, 1, 1e-5, dmean=dmd, dvar=dvd, **kw)
+        torch.cuda.synchronize()
+        names = K.profile_kernels()
+        K.check(K.lib().nblahip_profile_enable(0))
+        K.tune_reset()
+        return out, names
+
+    try:
+        held, names = run({"BN_CL_GRID_MIN_SLOTS": 1})
+        assert names == ["bn_cl_grid_bwd_kernel"], names
+        alone, names = run({"BN_CL_GRID_MIN_SLOTS": 1, "XCHG_SPIN": 0})
+        assert names == ["bn_cl_grid_bwd_kernel"], names
+        split, names = run({"BN_CL_GRID_BWD": 0, "BN_CL_GRID_MIN_SLOTS": 1})
+        assert "bn_cl_grid_bwd_kernel" not in names
+        acc, names = run({"BN_CL_GRID_MIN_SLOTS": 1}, dx=to_dev(pre_dx, dtype), dgamma=to_dev(pre_g),
+                         dbeta=to_dev(pre_b), accum=(True, True, True))
+        assert names == ["bn_cl_grid_bwd_kernel"], names
+        params, names = run({"BN_CL_GRID_MIN_SLOTS": 1}, need=(False, True, True))
+        assert names == ["bn_cl_grid_bwd_kernel"], names
+    finally:
+        K.tune_reset()
+    dx, dg, db = held
+    assert_close(to_np(dx), dx_r, dn, "grad", "dx")
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
+    for a_, b_ in zip(held, alone):
+        assert torch.equal(a_, b_)
+    assert_close(to_np(split[0]), to_np(dx), dn, "grad", "dx against the split reduction")
+    assert_close(to_np(split[1]), to_np(dg), dn, "pgrad", "dgamma against the split reduction")
+    assert_close(to_np(acc[0]), dx_r + pre_dx, dn, "grad", "dx accumulated")
+    assert_close(to_np(acc[1]), dg_r + pre_g, dn, "pgrad", "dgamma accumulated")
+    assert_close(to_np(acc[2]), db_r + pre_b, dn, "pgrad", "dbeta accumulated")
+    assert params[0] is None
+    assert torch.equal(params[1], dg) and torch.equal(params[2], db)
+
+
 def test_two_chip_filling_forwards_at_once():
     """Two host threads, each on its own stream, run the forward that holds the
     whole tensor on the chip at the same time: each launch wants every CU, so

@@ -169,6 +169,9 @@ SWITCHES = [
      {"BN_CL_GRID_MIN_SLOTS": 1}),
     ("bn_cl_grid_from_fewer_vectors", run_bn, ((100352, 64), 1, F16), {"BN_CL_GRID_MIN_SLOTS": 1},
      ["bn_cl_grid_fwd_kernel"], ["bn_stats_cl_kernel"]),
+    ("bn_cl_grid_bwd_off", run_bn, ((100352, 64), 1, F16), {"BN_CL_GRID_BWD": 0},
+     ["bn_cl_grid_fwd_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
+     ["bn_cl_grid_bwd_kernel"], {"BN_CL_GRID_MIN_SLOTS": 1}),
     ("bn_cl_cached_off", run_bn, ((32, 7, 7, 256), 3, F16), {"BN_CL_CACHED": 0},
      ["bn_stats_cl_kernel", "bn_apply_cl_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
      ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"]),
