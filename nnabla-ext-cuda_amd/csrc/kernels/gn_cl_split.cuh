@@ -58,20 +58,46 @@ struct ClSplitArgs {
 };
 
 // Polls the partners' words into part[] (a thread takes the two words of a
-// unit at a time); words that do not turn up mark their block in missing[].
+// unit at a time, the first reads of up to four units in flight together: a
+// tile of an instance in 16 blocks of 256 threads has 1920 words to collect per
+// block, four round trips one after the other when polled unit by unit); words
+// that do not turn up mark their block in missing[].
 template <int TPR>
 __device__ __forceinline__ void split_collect(const ClSplitArgs &a, const unsigned long long *base,
                                               uint32_t self, int per, float *part, int *missing) {
+  constexpr int kFly = TPR >= 1024 ? 1 : (TPR >= 512 ? 2 : 4); // 2048 words a sweep
   const int total = a.split * per;
-  for (int idx = 2 * threadIdx.x; idx < total; idx += 2 * TPR) {
-    const int sp = idx / per;
-    if (sp == static_cast<int>(self)) continue;
-    float v0, v1;
-    if (xchg_poll2(base + idx, a.epoch, a.spin, &v0, &v1)) {
-      part[idx] = v0;
-      part[idx + 1] = v1;
-    } else {
-      missing[sp] = 1;
+  for (int i0 = 2 * threadIdx.x; i0 < total; i0 += 2 * TPR * kFly) {
+    unsigned long long w[kFly][2];
+    bool want[kFly];
+#pragma unroll
+    for (int f = 0; f < kFly; ++f) {
+      const int idx = i0 + f * 2 * TPR;
+      want[f] = idx < total && idx / per != static_cast<int>(self);
+      if (want[f]) {
+        w[f][0] = __hip_atomic_load(base + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        w[f][1] = __hip_atomic_load(base + idx + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+#pragma unroll
+    for (int f = 0; f < kFly; ++f) {
+      if (!want[f]) continue;
+      const int idx = i0 + f * 2 * TPR;
+      float v0, v1;
+      bool ok = a.spin > 0 && static_cast<uint32_t>(w[f][0] >> 32) == a.epoch &&
+                static_cast<uint32_t>(w[f][1] >> 32) == a.epoch;
+      if (ok) {
+        v0 = __uint_as_float(static_cast<uint32_t>(w[f][0]));
+        v1 = __uint_as_float(static_cast<uint32_t>(w[f][1]));
+      } else {
+        ok = xchg_poll2(base + idx, a.epoch, a.spin - 1, &v0, &v1);
+      }
+      if (ok) {
+        part[idx] = v0;
+        part[idx + 1] = v1;
+      } else {
+        missing[idx / per] = 1;
+      }
     }
   }
 }
@@ -211,6 +237,7 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
   __shared__ float fold[NW][UMAX];
   __shared__ float tot[UMAX];
   __shared__ float part[kSplitMax * UMAX * 2];
+  __shared__ float merged[UMAX * 2];
   __shared__ int missing[kSplitMax];
   const uint32_t tile = blockIdx.x % a.tiles, ns = blockIdx.x / a.tiles;
   const uint32_t s = ns % a.split, n = ns / a.split;
@@ -388,24 +415,28 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
     lds_barrier();
   }
 
-  // ---- merge in block order, write the statistics (first block), normalize
-  if constexpr (!INSTANCE) {
-    split_merge_stats(a, part, per, gi, per_pos, mean[0], var[0]);
-    if (s == 0 && writer) {
-      const size_t u = static_cast<size_t>(n) * (a.C / a.cpg) + (tile * TV * VEC) / a.cpg + gi;
-      a.mean[u] = mean[0];
-      a.var[u] = var[0];
+  // ---- merge in block order (a thread per unit: every thread merging its own
+  // units again cost 2.6 us in a 1024-thread block of an instance), write the
+  // statistics (first block), normalize
+  if (static_cast<int>(threadIdx.x) < U) {
+    const int u = static_cast<int>(threadIdx.x);
+    float m, v;
+    split_merge_stats(a, part, per, u, per_pos, m, v);
+    merged[2 * u] = m;
+    merged[2 * u + 1] = v;
+    if (s == 0) {
+      const size_t ug = INSTANCE ? static_cast<size_t>(n) * a.C + tile * TV * VEC + u
+                                 : static_cast<size_t>(n) * (a.C / a.cpg) + (tile * TV * VEC) / a.cpg + u;
+      a.mean[ug] = m;
+      a.var[ug] = v;
     }
-  } else {
+  }
+  lds_barrier();
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) split_merge_stats(a, part, per, cvx * VEC + j, 1.f, mean[j], var[j]);
-    if (s == 0 && writer) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        a.mean[static_cast<size_t>(n) * a.C + ch + j] = mean[j];
-        a.var[static_cast<size_t>(n) * a.C + ch + j] = var[j];
-      }
-    }
+  for (int j = 0; j < (INSTANCE ? VEC : 1); ++j) {
+    const int u = INSTANCE ? static_cast<int>(cvx) * VEC + j : static_cast<int>(gi);
+    mean[j] = merged[2 * u];
+    var[j] = merged[2 * u + 1];
   }
 #pragma unroll
   for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
@@ -435,6 +466,38 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
   }
 }
 
+// The per-channel pairs of block (sample of x / dy, sp) from global memory into
+// chs, a vector at a time, in the arithmetic of the block that owns them: the
+// positions in the order of its registers, the same folds.  x, dy: the
+// thread's column of the sample; mean, istd, nmi: the sample's statistics for
+// the thread's units.
+template <typename T, int VEC, int NL, int TPR, bool INSTANCE, int SV>
+__device__ __forceinline__ void split_pairs_from_memory(
+    const ClSplitArgs &a, const T *__restrict__ x, const T *__restrict__ dy, int sp, uint32_t prow,
+    uint32_t cvx, const float (&mean)[SV], const float (&istd)[SV], const float (&nmi)[SV],
+    float (*fold)[2 * kSplitTV * VEC], float (*chs)[kSplitTV * VEC]) {
+  constexpr int PR = TPR / kSplitTV;
+  float sdx[VEC], sdy[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) sdx[j] = sdy[j] = 0.f;
+#pragma unroll 1
+  for (int k = 0; k < NL; ++k) {
+    const uint32_t pos = sp * a.PB + prow + k * PR;
+    const bool ok = pos < static_cast<uint32_t>(a.P);
+    const size_t off = static_cast<size_t>(ok ? pos : sp * a.PB) * a.C;
+    const RawVec<T, VEC> xv = load_raw<T, VEC>(x + off);
+    const RawVec<T, VEC> dv = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(dy + off));
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const int ju = INSTANCE ? j : 0;
+      const float xh = norm_elem<T, VEC>(xv, j, mean[ju], istd[ju], nmi[ju]);
+      sdx[j] = elem_fma<T, VEC>(dv, j, xh, sdx[j]);
+      sdy[j] = elem_fma<T, VEC>(dv, j, a.one, sdy[j]);
+    }
+  }
+  split_pair_sums<TPR, VEC>(sdx, sdy, cvx, fold, chs);
+}
+
 // ---------------------------------------------------------------------------
 // Backward.  With xh = (x-mean)*istd, per unit: s1 = sum gamma*dy,
 // t2 = sum gamma*dy*xh (over the unit's channels and all positions),
@@ -461,6 +524,7 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
   __shared__ float fold[NW][2 * CH];
   __shared__ float chs[2][CH]; // [0]: sum dy*xh, [1]: sum dy per channel of the tile
   __shared__ float part[kSplitMax * UMAX * 2];
+  __shared__ float totals[UMAX * 2];
   __shared__ int missing[kSplitMax];
   const uint32_t tile = blockIdx.x % a.tiles, ns = blockIdx.x / a.tiles;
   const uint32_t s = ns % a.split, n = ns / a.split;
@@ -554,30 +618,19 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
   for (int sp = 0; sp < a.split; ++sp) {
     if (sp == static_cast<int>(s) || !missing[sp]) continue; // same answer in every thread
     // Partner sp has not published: its sums from global memory, a vector at a time.
-    float sdx[VEC], sdy[VEC];
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) sdx[j] = sdy[j] = 0.f;
-#pragma unroll 1
-    for (int k = 0; k < NL; ++k) {
-      const uint32_t pos = sp * a.PB + prow + k * PR;
-      const bool ok = pos < static_cast<uint32_t>(a.P);
-      const size_t off = static_cast<size_t>(ok ? pos : sp * a.PB) * a.C;
-      const RawVec<T, VEC> xv = load_raw<T, VEC>(x + off);
-      const RawVec<T, VEC> dv = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(dy + off));
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const int ju = INSTANCE ? j : 0;
-        const float xh = norm_elem<T, VEC>(xv, j, mean[ju], istd[ju], nmi[ju]);
-        sdx[j] = elem_fma<T, VEC>(dv, j, xh, sdx[j]);
-        sdy[j] = elem_fma<T, VEC>(dv, j, a.one, sdy[j]);
-      }
-    }
-    split_pair_sums<TPR, VEC>(sdx, sdy, cvx, fold, chs);
+    split_pairs_from_memory<T, VEC, NL, TPR, INSTANCE, SV>(a, x, dy, sp, prow, cvx, mean, istd, nmi,
+                                                           fold, chs);
     unit_partials(static_cast<uint32_t>(sp), false);
     lds_barrier();
   }
 
-  // ---- totals in block order, dx
+  // ---- totals in block order (a thread per word), dx
+  for (int e = threadIdx.x; e < per; e += TPR) {
+    float t = 0.f;
+    for (int sp = 0; sp < a.split; ++sp) t += part[sp * per + e];
+    totals[e] = t;
+  }
+  lds_barrier();
 #pragma unroll
   for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(xr[k]);
   float gis[VEC], cA[SV], cb[SV];
@@ -586,11 +639,7 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
 #pragma unroll
   for (int j = 0; j < SV; ++j) {
     const int u = INSTANCE ? static_cast<int>(cvx) * VEC + j : static_cast<int>(gi);
-    float t2 = 0.f, s1 = 0.f;
-    for (int sp = 0; sp < a.split; ++sp) {
-      t2 += part[sp * per + u * 2];
-      s1 += part[sp * per + u * 2 + 1];
-    }
+    float t2 = totals[2 * u], s1 = totals[2 * u + 1];
     if constexpr (INSTANCE) { // the exchanged sums are per channel, without gamma
       const float g = a.gamma ? a.gamma[ch + j] : 1.f;
       t2 *= g;

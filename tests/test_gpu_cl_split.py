@@ -57,7 +57,9 @@ def ran(names):
 # block shape covers, several column tiles
 SHAPES = [(3, (33, 33), 64, 8), (2, (20, 20), 128, 4), (5, (9, 9), 64, 1), (2, (70, 70), 64, 8),
           (1, (127, 129), 64, 2), (2, (100, 100), 32, 4), (4, (16, 16), 512, 16), (2, (7,), 64, 8),
-          (1, (300,), 192, 12)]
+          (1, (300,), 192, 12),
+          # many (sample, block) rows of pairs behind dgamma / dbeta
+          (40, (20, 20), 64, 8), (70, (6, 6), 128, 16)]
 
 
 @pytest.mark.parametrize("n,sp,c,groups", SHAPES)
@@ -142,6 +144,10 @@ def test_split_flags(spin):
                                   dvar=to_dev(dv), need=(False, True, True), channel_last=True)
     assert_close(to_np(dgam), dg_r, "f32", "pgrad", "dgamma only")
     assert_close(to_np(dbet), db_r, "f32", "pgrad", "dbeta only")
+    _, dgam, none = K.gn_backward(xd, dyd, to_dev(g), m, v, groups, 1e-5, dmean=to_dev(dm),
+                                  dvar=to_dev(dv), need=(True, True, False), channel_last=True)
+    assert none is None
+    assert_close(to_np(dgam), dg_r, "f32", "pgrad", "dgamma without dbeta")
     torch.cuda.synchronize()
     assert ran(K.profile_kernels())
 
