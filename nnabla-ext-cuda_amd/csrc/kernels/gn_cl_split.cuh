@@ -254,18 +254,18 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
   const bool writer = prow == 0 && (INSTANCE || (cvx & ((1u << a.cvg_shift) - 1)) == 0);
 
   if (threadIdx.x < kSplitMax) missing[threadIdx.x] = 0;
+  float gam[VEC], bet[VEC]; // ahead of the tensor's loads: they travel together
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    gam[j] = a.gamma ? a.gamma[ch + j] : 1.f;
+    bet[j] = a.beta ? a.beta[ch + j] : 0.f;
+  }
   RawVec<T, VEC> raw[NL];
 #pragma unroll
   for (int k = 0; k < NL; ++k) {
     const uint32_t pos = s * a.PB + prow + k * PR;
     const bool ok = pos < static_cast<uint32_t>(a.P);
     raw[k] = raw_or_zero<T, VEC>(ok, load_raw<T, VEC>(x + static_cast<size_t>(ok ? pos : s * a.PB) * a.C));
-  }
-  float gam[VEC], bet[VEC];
-#pragma unroll
-  for (int j = 0; j < VEC; ++j) {
-    gam[j] = a.gamma ? a.gamma[ch + j] : 1.f;
-    bet[j] = a.beta ? a.beta[ch + j] : 0.f;
   }
 
   float mean[INSTANCE ? VEC : 1], var[INSTANCE ? VEC : 1];
@@ -524,7 +524,8 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
   __shared__ float fold[NW][2 * CH];
   __shared__ float chs[2][CH]; // [0]: sum dy*xh, [1]: sum dy per channel of the tile
   __shared__ float part[kSplitMax * UMAX * 2];
-  __shared__ float totals[UMAX * 2];
+  __shared__ float coef[UMAX * 2]; // (cA, cb) per unit
+  __shared__ float gch[CH];        // gamma of the tile's channels
   __shared__ int missing[kSplitMax];
   const uint32_t tile = blockIdx.x % a.tiles, ns = blockIdx.x / a.tiles;
   const uint32_t s = ns % a.split, n = ns / a.split;
@@ -544,6 +545,25 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
                                : static_cast<size_t>(n) * (a.C / a.cpg) + ch0 / a.cpg + gi;
 
   if (threadIdx.x < kSplitMax) missing[threadIdx.x] = 0;
+  // Small loads first, so that they travel with the tensor's: the thread's
+  // statistics, gamma of channel threadIdx.x of the tile, and what the thread
+  // of unit threadIdx.x needs for the unit's coefficients.
+  float mean[SV], uvar[SV];
+#pragma unroll
+  for (int j = 0; j < SV; ++j) {
+    mean[j] = a.mean[stat + j];
+    uvar[j] = a.var[stat + j];
+  }
+  const bool unit_thread = static_cast<int>(threadIdx.x) < U;
+  const size_t ustat = INSTANCE ? static_cast<size_t>(n) * a.C + ch0 + threadIdx.x
+                                : static_cast<size_t>(n) * (a.C / a.cpg) + ch0 / a.cpg + threadIdx.x;
+  float g_c = 1.f, u_var = 1.f, u_dvar = 0.f, u_dmean = 0.f;
+  if (threadIdx.x < CH && a.gamma) g_c = a.gamma[ch0 + threadIdx.x];
+  if (unit_thread) {
+    u_var = a.var[ustat];
+    if (a.dvar) u_dvar = a.dvar[ustat];
+    if (a.dmean) u_dmean = a.dmean[ustat];
+  }
   RawVec<T, VEC> xr[NL];
   {
     RawVec<T, VEC> dr[NL];
@@ -558,13 +578,13 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
 #pragma unroll
     for (int k = 0; k < NL; ++k) park[k * TPR + threadIdx.x] = dr[k];
   }
-  float mean[SV], istd[SV], nmi[SV];
+  float istd[SV], nmi[SV];
 #pragma unroll
   for (int j = 0; j < SV; ++j) {
-    mean[j] = a.mean[stat + j];
-    istd[j] = 1.0f / sqrtf(a.var[stat + j] + a.eps);
+    istd[j] = 1.0f / sqrtf(uvar[j] + a.eps);
     nmi[j] = -mean[j] * istd[j];
   }
+  if (threadIdx.x < CH) gch[threadIdx.x] = g_c; // (read behind the barriers of the first fold)
 
   // chs -> the partial (t2, s1) of every unit of the tile, into part[sp]
   auto unit_partials = [&](uint32_t sp, bool publish) {
@@ -576,8 +596,7 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
       } else {
         v = 0.f;
         for (int c = 0; c < a.cpg; ++c) {
-          const float gc = a.gamma ? a.gamma[ch0 + u * a.cpg + c] : 1.f;
-          v = fmaf(gc, chs[w][u * a.cpg + c], v);
+          v = fmaf(gch[u * a.cpg + c], chs[w][u * a.cpg + c], v);
         }
       }
       part[sp * per + e] = v;
@@ -624,30 +643,42 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
     lds_barrier();
   }
 
-  // ---- totals in block order (a thread per word), dx
-  for (int e = threadIdx.x; e < per; e += TPR) {
-    float t = 0.f;
-    for (int sp = 0; sp < a.split; ++sp) t += part[sp * per + e];
-    totals[e] = t;
+  // ---- totals in block order and the unit's coefficients (a thread per unit), dx
+  if (unit_thread) {
+    const int u = static_cast<int>(threadIdx.x);
+    float t2 = 0.f, s1 = 0.f;
+    for (int sp = 0; sp < a.split; ++sp) {
+      t2 += part[sp * per + 2 * u];
+      s1 += part[sp * per + 2 * u + 1];
+    }
+    if constexpr (INSTANCE) { // the exchanged sums are per channel, without gamma
+      t2 *= g_c;
+      s1 *= g_c;
+    }
+    const float vpe = u_var + a.eps;
+    const float is = 1.0f / sqrtf(vpe);
+    coef[2 * u] = -is * t2 * a.inv_R + (a.dvar ? 2.f * u_dvar * (vpe * is) * a.inv_R : 0.f);
+    coef[2 * u + 1] = -s1 * is * a.inv_R + (a.dmean ? u_dmean * a.inv_R : 0.f);
   }
   lds_barrier();
 #pragma unroll
   for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(xr[k]);
+  // half: dx = dy*gis + x*A2 + B2 with A2 = istd*cA, B2 = nmi*cA + cb, two
+  // mixed-precision fmas per element; float: dx = dy*gis + xh*cA + cb
   float gis[VEC], cA[SV], cb[SV];
 #pragma unroll
-  for (int j = 0; j < VEC; ++j) gis[j] = (a.gamma ? a.gamma[ch + j] : 1.f) * istd[INSTANCE ? j : 0];
+  for (int j = 0; j < VEC; ++j) gis[j] = gch[cvx * VEC + j] * istd[INSTANCE ? j : 0];
 #pragma unroll
   for (int j = 0; j < SV; ++j) {
     const int u = INSTANCE ? static_cast<int>(cvx) * VEC + j : static_cast<int>(gi);
-    float t2 = totals[2 * u], s1 = totals[2 * u + 1];
-    if constexpr (INSTANCE) { // the exchanged sums are per channel, without gamma
-      const float g = a.gamma ? a.gamma[ch + j] : 1.f;
-      t2 *= g;
-      s1 *= g;
+    const float ca = coef[2 * u], cbu = coef[2 * u + 1];
+    if constexpr (sizeof(T) == 2) {
+      cA[j] = istd[j] * ca;
+      cb[j] = fmaf(nmi[j], ca, cbu);
+    } else {
+      cA[j] = ca;
+      cb[j] = cbu;
     }
-    const float vpe = a.var[stat + j] + a.eps;
-    cA[j] = -istd[j] * t2 * a.inv_R + (a.dvar ? 2.f * a.dvar[stat + j] * (vpe * istd[j]) * a.inv_R : 0.f);
-    cb[j] = -s1 * istd[j] * a.inv_R + (a.dmean ? a.dmean[stat + j] * a.inv_R : 0.f);
   }
 #pragma unroll
   for (int k = 0; k < NL; ++k) {
@@ -658,8 +689,12 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
         const int ju = INSTANCE ? j : 0;
-        const float xh = norm_elem<T, VEC>(xr[k], j, mean[ju], istd[ju], nmi[ju]);
-        o[j] = elem_fma<T, VEC>(dv, j, gis[j], fmaf(xh, cA[ju], cb[ju]));
+        if constexpr (sizeof(T) == 2) {
+          o[j] = elem_fma<T, VEC>(dv, j, gis[j], elem_fma<T, VEC>(xr[k], j, cA[ju], cb[ju]));
+        } else {
+          const float xh = norm_elem<T, VEC>(xr[k], j, mean[ju], istd[ju], nmi[ju]);
+          o[j] = elem_fma<T, VEC>(dv, j, gis[j], fmaf(xh, cA[ju], cb[ju]));
+        }
       }
       T *p = dx + static_cast<size_t>(pos) * a.C;
       if (a.accum_dx) {
