@@ -282,8 +282,16 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
   __shared__ float got[2 * kGridMaxBlocks];
   __shared__ int miss[kGridMaxBlocks + 2]; // [kGridMaxBlocks], [+1]: any partial / any result missing
   __shared__ float wel[3 * 16];
+  __shared__ float gb[2 * kGridMaxC]; // gamma, beta
   const uint32_t b = blockIdx.x;
   const uint32_t t = threadIdx.x;
+  // gamma and beta of channel t, asked for ahead of the tensor (behind the
+  // exchange they would cost a memory round trip of their own)
+  float gamma_t = 1.f, beta_t = 0.f;
+  if (t < a.C) {
+    if (a.gamma) gamma_t = a.gamma[t];
+    if (a.beta) beta_t = a.beta[t];
+  }
   const uint32_t cvx = t % a.cv;
   const uint32_t ch = cvx * VEC;
   const uint32_t vbb = grid_block_vectors(a, b);
@@ -305,6 +313,10 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
     for (int k = 0; k < NR; ++k) {
       const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t;
       raw[k] = load_raw<T, VEC>(x + static_cast<size_t>(min(v, last)) * VEC);
+    }
+    if (t < a.C) { // (they arrive first; read behind the barriers of the folds)
+      gb[t] = gamma_t;
+      gb[kGridMaxC + t] = beta_t;
     }
 #pragma unroll
     for (int k = 0; k < NS; ++k) spill[k * kOnchipBlock + t] = __builtin_bit_cast(uint4, parked[k]);
@@ -408,8 +420,8 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
     mu[j] = fin[2 * (ch + j)];
-    sc[j] = (a.gamma ? a.gamma[ch + j] : 1.f) * inv_std(fin[2 * (ch + j) + 1], a.eps);
-    be[j] = a.beta ? a.beta[ch + j] : 0.f;
+    sc[j] = gb[ch + j] * inv_std(fin[2 * (ch + j) + 1], a.eps);
+    be[j] = gb[kGridMaxC + ch + j];
     sh[j] = fmaf(-mu[j], sc[j], be[j]);
   }
   const uint32_t t2 = fresh(t);
@@ -453,8 +465,20 @@ bn_cl_grid_bwd_kernel(const BnClGridArgs a) {
   __shared__ float got[2 * kGridMaxBlocks];
   __shared__ int miss[kGridMaxBlocks + 2];
   __shared__ float wel[16];
+  __shared__ float par[5 * kGridMaxC]; // mean, var, gamma, dvar, dmean
   const uint32_t b = blockIdx.x;
   const uint32_t t = threadIdx.x;
+  // The parameters of channel t, asked for ahead of the tensor: behind the LDS
+  // stores of x, or behind the exchange, each would cost a memory round trip
+  // of its own.
+  float p_mean = 0.f, p_var = 1.f, p_gamma = 1.f, p_dvar = 0.f, p_dmean = 0.f;
+  if (t < a.C) {
+    p_mean = a.mean[t];
+    p_var = a.var[t];
+    if (a.gamma) p_gamma = a.gamma[t];
+    if (a.dvar) p_dvar = a.dvar[t];
+    if (a.dmean) p_dmean = a.dmean[t];
+  }
   const uint32_t cvx = t % a.cv;
   const uint32_t ch = cvx * VEC;
   const uint32_t vbb = grid_block_vectors(a, b);
@@ -484,11 +508,19 @@ bn_cl_grid_bwd_kernel(const BnClGridArgs a) {
     if (k < NR) return raw[k < NR ? k : 0];
     return __builtin_bit_cast(RawVec<T, VEC>, spill[(k - NR) * kOnchipBlock + t]);
   };
+  if (t < a.C) {
+    par[t] = p_mean;
+    par[kGridMaxC + t] = p_var;
+    par[2 * kGridMaxC + t] = p_gamma;
+    par[3 * kGridMaxC + t] = p_dvar;
+    par[4 * kGridMaxC + t] = p_dmean;
+  }
+  lds_barrier();
   float mean[VEC], istd[VEC], nmi[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
-    mean[j] = a.mean[ch + j];
-    istd[j] = 1.0f / sqrtf(a.var[ch + j] + a.eps);
+    mean[j] = par[ch + j];
+    istd[j] = 1.0f / sqrtf(par[kGridMaxC + ch + j] + a.eps);
     nmi[j] = -mean[j] * istd[j];
   }
 
@@ -588,12 +620,12 @@ bn_cl_grid_bwd_kernel(const BnClGridArgs a) {
   float gi[VEC], A2[VEC], B2[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
-    const float g = a.gamma ? a.gamma[ch + j] : 1.f;
-    const float vpe = a.var[ch + j] + a.eps;
+    const float g = par[2 * kGridMaxC + ch + j];
+    const float vpe = par[kGridMaxC + ch + j] + a.eps;
     const float cA = -istd[j] * g * fin[2 * (ch + j)] * a.inv_N +
-                     (a.dvar ? 2.f * a.dvar[ch + j] * (vpe * istd[j]) * a.inv_N : 0.f);
+                     (a.dvar ? 2.f * par[3 * kGridMaxC + ch + j] * (vpe * istd[j]) * a.inv_N : 0.f);
     const float cb = -g * fin[2 * (ch + j) + 1] * istd[j] * a.inv_N +
-                     (a.dmean ? a.dmean[ch + j] * a.inv_N : 0.f);
+                     (a.dmean ? par[4 * kGridMaxC + ch + j] * a.inv_N : 0.f);
     gi[j] = g * istd[j];
     A2[j] = istd[j] * cA;
     B2[j] = sizeof(T) == 2 ? fmaf(nmi[j], cA, cb) : cb;

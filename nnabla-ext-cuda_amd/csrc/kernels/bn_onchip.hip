@@ -91,6 +91,9 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
   const uint32_t t = threadIdx.x;
   const T *__restrict__ x = static_cast<const T *>(a.x);
   T *__restrict__ y = static_cast<T *>(a.y);
+  // (asked for now: behind the block sums they would cost a round trip of their own)
+  const float gamma_c = a.gamma ? a.gamma[c] : 1.f;
+  const float beta_c = a.beta ? a.beta[c] : 0.f;
 
   // Loads, all in flight together (no branch: a slot beyond the channel reads
   // the channel's last vector and is left out of every sum and store): the LDS
@@ -189,8 +192,8 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
   }
 #pragma unroll
   for (int k = 0; k < NR; ++k) keep_packed<T, VEC>(raw[k]);
-  const float g = (a.gamma ? a.gamma[c] : 1.f) * istd;
-  const float b = a.beta ? a.beta[c] : 0.f;
+  const float g = gamma_c * istd;
+  const float b = beta_c;
   const float sh = fmaf(-mean, g, b);
 
   auto emit = [&](const RawVec<T, VEC> &r, uint32_t v) {
@@ -269,6 +272,8 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
   const T *__restrict__ x = static_cast<const T *>(a.x);
   const T *__restrict__ dy = static_cast<const T *>(a.dy);
   T *__restrict__ dx = static_cast<T *>(a.dx);
+  // (asked for now: behind the block sums they would cost a round trip of their own)
+  const float g = a.gamma ? a.gamma[c % a.gmod] : 1.f;
 
   RawVec<T, VEC> raw[NR];
   {
@@ -383,7 +388,6 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
   if (dx == nullptr) return;
 #pragma unroll
   for (int k = 0; k < NR; ++k) forget<T, VEC>(raw[k]);
-  const float g = a.gamma ? a.gamma[c % a.gmod] : 1.f;
   const float gi = g * istd;
   const float cA = -istd * g * sdx * a.inv_N + (a.dvar ? 2.f * a.dvar[c] * (vpe * istd) * a.inv_N : 0.f);
   const float cb = -g * sdy * istd * a.inv_N + (a.dmean ? a.dmean[c] * a.inv_N : 0.f);

@@ -395,6 +395,19 @@ row_bwd_kernel(const RowArgs a) {
       }
       if (a.gamma && static_cast<int>(threadIdx.x) < a.cpg) gch = a.gamma[pb + threadIdx.x];
     }
+    // IN: the row's gamma, asked for ahead of the row (behind the reduction it
+    // would cost a memory round trip of its own; the BN rows have no register
+    // to spare for it).
+    float g_row = 1.f;
+    if constexpr (MODE == kRowIN || MODE == kRowINc) {
+      if (a.gamma) g_row = a.gamma[(static_cast<uint32_t>(row) % a.pmod) * a.pmul];
+    }
+    // (with dy parked in LDS the statistics too: the stores wait for the row)
+    float mean_early = 0.f, var_early = 0.f;
+    if constexpr (PARK) {
+      mean_early = a.mean[row];
+      var_early = a.var[row];
+    }
     RawVec<T, VEC> xr[NL], dr[NL];
 #pragma unroll
     for (int k = 0; k < NL; ++k) {
@@ -422,8 +435,8 @@ row_bwd_kernel(const RowArgs a) {
         return dr[k];
       }
     };
-    const float mean = a.mean[row];
-    const float vpe = a.var[row] + a.eps;
+    const float mean = PARK ? mean_early : a.mean[row];
+    const float vpe = (PARK ? var_early : a.var[row]) + a.eps;
     const float istd = 1.0f / sqrtf(vpe);
     const float nmi = -mean * istd;
 
@@ -493,8 +506,8 @@ row_bwd_kernel(const RowArgs a) {
           a.ws[2 * static_cast<size_t>(row) + 1] = sdy;
         }
       }
-      const uint32_t pidx = (static_cast<uint32_t>(row) % a.pmod) * a.pmul;
-      const float g = a.gamma ? a.gamma[pidx] : 1.f;
+      float g = g_row;
+      if constexpr (BN) g = a.gamma ? a.gamma[(static_cast<uint32_t>(row) % a.pmod) * a.pmul] : 1.f;
 #pragma unroll
       for (int k = 0; k < NL; ++k) gk[k] = g;
       s1 = g * sdy;
