@@ -116,9 +116,10 @@ __device__ __forceinline__ float grid_channel_sum1(float v, uint32_t cv, uint32_
 
 // (mean, m2) of the rows of block p for channel c, from global memory, in the
 // order block p itself uses (its thread map, slots ascending per thread, the
-// same folds): what block p publishes for c, bit for bit.  Only the threads of
-// c's channel vector load (the folds never mix channel vectors) and only c's
-// element is accumulated, so this costs a handful of registers.
+// thread's first element as the shift, the same folds): what block p
+// publishes for c, bit for bit.  Only the threads of c's channel vector load
+// (the folds never mix channel vectors) and only c's element is accumulated,
+// so this costs a handful of registers.
 template <typename T, int VEC>
 __device__ __forceinline__ void grid_partial_from_memory(const BnClGridArgs &a, uint32_t p,
                                                          uint32_t c, float *fold, float &m,
@@ -126,33 +127,35 @@ __device__ __forceinline__ void grid_partial_from_memory(const BnClGridArgs &a, 
   const T *__restrict__ x = static_cast<const T *>(a.x);
   const uint32_t t = threadIdx.x;
   const uint32_t cvx = t % a.cv, e = c % VEC;
-  const uint32_t vbp = cvx == c / VEC ? grid_block_vectors(a, p) : 0u;
-  const uint32_t rows = grid_block_vectors(a, p) / a.cv;
+  const uint32_t vbb = grid_block_vectors(a, p);
+  const bool mine = cvx == c / VEC;
   const size_t first = static_cast<size_t>(p) * a.vb;
-  float s = 0.f;
-#pragma unroll 1
-  for (uint32_t v = t; v < vbp; v += kOnchipBlock) {
-    const RawVec<T, VEC> r = load_raw<T, VEC>(x + (first + v) * VEC);
+  float kk = 0.f, s1 = 0.f, s2 = 0.f, nt = 0.f;
+  if (mine && t < vbb) {
+    const RawVec<T, VEC> r0 = load_raw<T, VEC>(x + (first + t) * VEC);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-      const float n = elem_fma<T, VEC>(r, j, a.one, s);
-      s = static_cast<uint32_t>(j) == e ? n : s;
+      const float v0 = elem_fma<T, VEC>(r0, j, a.one, 0.f);
+      kk = static_cast<uint32_t>(j) == e ? v0 : kk;
     }
-  }
-  s = grid_channel_sum1(s, a.cv, cvx, c, cvx == c / VEC, fold, a.C);
-  m = s * (1.0f / static_cast<float>(rows));
-  q = 0.f;
+    nt = static_cast<float>((vbb - 1u - t) / kOnchipBlock + 1u);
 #pragma unroll 1
-  for (uint32_t v = t; v < vbp; v += kOnchipBlock) {
-    const RawVec<T, VEC> r = load_raw<T, VEC>(x + (first + v) * VEC);
+    for (uint32_t v = t + kOnchipBlock; v < vbb; v += kOnchipBlock) {
+      const RawVec<T, VEC> r = load_raw<T, VEC>(x + (first + v) * VEC);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      const float d = elem_fma<T, VEC>(r, j, a.one, -m);
-      const float n = fmaf(d, d, q);
-      q = static_cast<uint32_t>(j) == e ? n : q;
+      for (int j = 0; j < VEC; ++j) {
+        const float d = elem_fma<T, VEC>(r, j, a.one, -kk);
+        const float n1 = s1 + d;
+        const float n2 = fmaf(d, d, s2);
+        s1 = static_cast<uint32_t>(j) == e ? n1 : s1;
+        s2 = static_cast<uint32_t>(j) == e ? n2 : s2;
+      }
     }
   }
-  q = grid_channel_sum1(q, a.cv, cvx, c, cvx == c / VEC, fold, a.C);
+  m = grid_channel_sum1(fmaf(nt, kk, s1), a.cv, cvx, c, mine, fold, a.C);
+  m *= 1.0f / static_cast<float>(vbb / a.cv);
+  const float d = kk - m;
+  q = grid_channel_sum1(mine ? fmaf(d, fmaf(nt, d, 2.f * s1), s2) : 0.f, a.cv, cvx, c, mine, fold, a.C);
 }
 
 // Merged (mean, var) of channel c over all blocks: thread p < nblocks takes
@@ -326,51 +329,68 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
     return __builtin_bit_cast(RawVec<T, VEC>, spill[(k - NR) * kOnchipBlock + t]);
   };
 
-  // ---- this block's partial per channel: mean, then the second moment about it
+  // (slot k holds a vector of the block: t against a scalar, no register per slot)
+  auto holds = [&](int k) { return static_cast<int>(t) < static_cast<int>(vbb) - k * kOnchipBlock; };
+
+  // ---- this block's partial per channel, in ONE pass over the slots, taken by
+  // every wave as its own loads arrive (the memory system serves a CU's waves
+  // one after the other, 2 to 18 us after the start here: what a wave does
+  // before the block's first barrier hides behind the other waves' loads, what
+  // comes after it keeps memory idle - a second pass about the block's mean
+  // cost 5.8 us of [256,56,56,64]'s 49).  Per thread and channel, with the
+  // thread's first element as the shift K: s1 = sum (x - K), s2 = sum (x - K)^2
+  // over its n slots.  Then mean = sum_t (n K + s1) / rows, and about it
+  // m2 = sum_t (s2 + 2 e s1 + n e^2), e = K - mean: two block sums of a few
+  // operations per thread.  K is one of the thread's own values, so the three
+  // terms cancel to no less than that element's own share of m2.
   float m[VEC], q[VEC];
   {
-    float s[VEC];
+    float kk[VEC], s1[VEC], s2[VEC];
+    {
+      const RawVec<T, VEC> r0 = slot(0);
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) s[j] = 0.f;
-#pragma unroll
-    for (int k = 0; k < NL; ++k) {
-      if (static_cast<uint32_t>(k) * kOnchipBlock + t < vbb) {
-        const RawVec<T, VEC> r = slot(k);
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) s[j] = elem_fma<T, VEC>(r, j, a.one, s[j]);
+      for (int j = 0; j < VEC; ++j) {
+        kk[j] = holds(0) ? elem_fma<T, VEC>(r0, j, a.one, 0.f) : 0.f;
+        s1[j] = s2[j] = 0.f;
       }
     }
-    grid_channel_sums<VEC>(s, a.cv, cvx, fold, tot, a.C);
+#pragma unroll
+    for (int k = 1; k < NL; ++k) {
+      if (holds(k)) {
+        const RawVec<T, VEC> r = slot(k);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float d = elem_fma<T, VEC>(r, j, a.one, -kk[j]);
+          s1[j] += d;
+          s2[j] = fmaf(d, d, s2[j]);
+        }
+      }
+    }
+    const float nt = t < vbb ? static_cast<float>((vbb - 1u - t) / kOnchipBlock + 1u) : 0.f;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) m[j] = fmaf(nt, kk[j], s1[j]);
+    grid_channel_sums<VEC>(m, a.cv, cvx, fold, tot, a.C);
     const float icnt = 1.0f / static_cast<float>(vbb / a.cv);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-      m[j] = s[j] * icnt;
-      q[j] = 0.f;
+      m[j] *= icnt;
+      const float e = kk[j] - m[j];
+      q[j] = fmaf(e, fmaf(nt, e, 2.f * s1[j]), s2[j]);
     }
+    grid_channel_sums<VEC>(q, a.cv, cvx, fold, tot, a.C);
   }
-#pragma unroll
-  for (int k = 0; k < NR; ++k) forget<T, VEC>(raw[k]);
-#pragma unroll
-  for (int k = 0; k < NL; ++k) {
-    if (static_cast<uint32_t>(k) * kOnchipBlock + t < vbb) {
-      const RawVec<T, VEC> r = slot(k);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const float d = elem_fma<T, VEC>(r, j, a.one, -m[j]);
-        q[j] = fmaf(d, d, q[j]);
-      }
-    }
-  }
-  grid_channel_sums<VEC>(q, a.cv, cvx, fold, tot, a.C);
-  // publish (mean, m2) of every channel: a word per thread (tot holds the m2
-  // totals; the means go through fin, which is free until the results arrive)
+  // publish (mean, m2) of every channel: a word per thread (through fin, which
+  // is free until the results arrive)
   if (t < a.cv) {
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) fin[ch + j] = m[j];
+    for (int j = 0; j < VEC; ++j) {
+      fin[2 * (ch + j)] = m[j];
+      fin[2 * (ch + j) + 1] = q[j];
+    }
   }
   lds_barrier();
   for (uint32_t e = t; e < 2 * a.C; e += kOnchipBlock)
-    xchg_publish(a.x1 + static_cast<size_t>(b) * a.C * 2 + e, (e & 1) ? tot[e >> 1] : fin[e >> 1], a.epoch);
+    xchg_publish(a.x1 + static_cast<size_t>(b) * a.C * 2 + e, fin[e], a.epoch);
 
   // ---- stage 2: block c merges channel c, writes its statistics, publishes
   for (uint32_t c = b; c < a.C; c += a.nblocks) {
