@@ -73,13 +73,9 @@ __device__ __forceinline__ uint32_t onchip_offset(const BnOnchipArgs &a, uint32_
 
 } // namespace
 
-// OVER: the channel is longer than the NR + NS slots held on chip.  The mean
-// of the held part serves as the shift K of the whole channel: the held part's
-// second pass and ONE read of the rest accumulate sum (x - K) and
-// sum (x - K)^2, from which mean = K + s1/N and var = q/N - (s1/N)^2 (K is the
-// mean of 25600 vectors of the same channel, so the subtracted square is tiny
-// against the variance: no cancellation).  The rest is read a second time for
-// y: 2 S + (1 - 25600 / nv) S instead of 3 S.
+// OVER: the channel is longer than the NR + NS slots held on chip.  The rest
+// is read once for the statistics (into the same per-thread sums as the held
+// part) and a second time for y: 2 S + (1 - 25600 / nv) S instead of 3 S.
 // FUSED (FusedBatchNormalization): y = max(0, bn(x) + z), z optional.
 template <typename T, int VEC, int NR, int NS, bool OVER = false, bool FUSED = false>
 __global__ void __launch_bounds__(kOnchipBlock)
@@ -111,49 +107,37 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
     const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t;
     raw[k] = load_raw<T, VEC>(x + onchip_offset(a, c, min(v, a.nv - 1u), VEC));
   }
-  float s = 0.f;
+  // Statistics in ONE pass, taken by every wave as its own loads arrive (the
+  // memory system serves a CU's waves one after the other: what a wave does
+  // before the block's first barrier hides behind the other waves' loads, a
+  // second pass about the mean would keep memory idle).  Per thread, with its
+  // first element as the shift K: s1 = sum (x - K), s2 = sum (x - K)^2 over its
+  // n elements; mean = sum_t (n K + s1) / N and, about it,
+  // var = sum_t (s2 + 2 e s1 + n e^2) / N with e = K - mean: two block sums of
+  // a few operations per thread.  K is one of the thread's own elements, so
+  // the three terms cancel to no less than that element's own share.
+  // (OVER: the vectors beyond the held ones are read here once, and once more for y.)
+  auto held = [&](int k) { return static_cast<int>(t) < static_cast<int>(a.nv) - k * kOnchipBlock; };
+  const float kk = held(0) ? elem_fma<T, VEC>(raw[0], 0, a.one, 0.f) : 0.f;
+  float s1 = 0.f, s2 = 0.f;
+  auto take = [&](const RawVec<T, VEC> &r) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float d = elem_fma<T, VEC>(r, j, a.one, -kk);
+      s1 += d;
+      s2 = fmaf(d, d, s2);
+    }
+  };
 #pragma unroll
   for (int k = 0; k < NS; ++k) {
-    const float part = raw_sum<T, VEC>(parked[k], 0.f);
-    s += (static_cast<uint32_t>(NR + k) * kOnchipBlock + t < a.nv) ? part : 0.f;
+    if (held(NR + k)) take(parked[k]);
     spill[k * kOnchipBlock + t] = __builtin_bit_cast(Slot<T, VEC>, parked[k]);
   }
 #pragma unroll
   for (int k = 0; k < NR; ++k) {
-    const float part = raw_sum<T, VEC>(raw[k], 0.f);
-    s += (static_cast<uint32_t>(k) * kOnchipBlock + t < a.nv) ? part : 0.f;
+    if (held(k)) take(raw[k]);
   }
-  // (OVER: the shift K, over the held elements only)
   constexpr uint32_t kHeld = static_cast<uint32_t>(NR + NS) * kOnchipBlock;
-  float mean = onchip_block_sum(s, red) * (OVER ? 1.0f / (static_cast<float>(kHeld) * VEC) : a.inv_N);
-#pragma unroll
-  for (int k = 0; k < NR; ++k) keep_packed<T, VEC>(raw[k]);
-
-  float q = 0.f;
-  float s1 = 0.f; // OVER: sum (x - K), the held part's rounding residue included
-#pragma unroll
-  for (int k = 0; k < NR; ++k) {
-    if (static_cast<uint32_t>(k) * kOnchipBlock + t < a.nv) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const float d = elem_fma<T, VEC>(raw[k], j, a.one, -mean);
-        q = fmaf(d, d, q);
-        if constexpr (OVER) s1 += d;
-      }
-    }
-  }
-#pragma unroll
-  for (int k = 0; k < NS; ++k) {
-    if (static_cast<uint32_t>(NR + k) * kOnchipBlock + t < a.nv) {
-      const RawVec<T, VEC> r = __builtin_bit_cast(RawVec<T, VEC>, spill[k * kOnchipBlock + t]);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const float d = elem_fma<T, VEC>(r, j, a.one, -mean);
-        q = fmaf(d, d, q);
-        if constexpr (OVER) s1 += d;
-      }
-    }
-  }
   if constexpr (OVER) {
     constexpr int BO = 4;
 #pragma unroll 1
@@ -164,25 +148,16 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
         xo[b] = load_raw<T, VEC>(x + onchip_offset(a, c, min(v0 + b * kOnchipBlock + t, a.nv - 1u), VEC));
 #pragma unroll
       for (int b = 0; b < BO; ++b) {
-        float ps = 0.f, pq = 0.f;
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          const float d = elem_fma<T, VEC>(xo[b], j, a.one, -mean);
-          ps += d;
-          pq = fmaf(d, d, pq);
-        }
-        const bool ok = v0 + b * kOnchipBlock + t < a.nv;
-        s1 += ok ? ps : 0.f;
-        q += ok ? pq : 0.f;
+        if (v0 + b * kOnchipBlock + t < a.nv) take(xo[b]);
       }
     }
-    s1 = onchip_block_sum(s1, red) * a.inv_N; // mean - K
   }
-  float var = onchip_block_sum(q, red) * a.inv_N;
-  if constexpr (OVER) {
-    var = fmaxf(var - s1 * s1, 0.f);
-    mean += s1;
-  }
+  const float nt = t < a.nv ? static_cast<float>(((a.nv - 1u - t) / kOnchipBlock + 1u) * VEC) : 0.f;
+  const float mean = onchip_block_sum(fmaf(nt, kk, s1), red) * a.inv_N;
+  const float e = kk - mean;
+  const float var = onchip_block_sum(fmaf(e, fmaf(nt, e, 2.f * s1), s2), red) * a.inv_N;
+#pragma unroll
+  for (int k = 0; k < NR; ++k) keep_packed<T, VEC>(raw[k]);
   const float istd = inv_std(var, a.eps);
   if (t == 0) {
     a.mean[c] = mean;

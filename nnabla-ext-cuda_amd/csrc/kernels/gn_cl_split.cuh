@@ -223,6 +223,86 @@ __device__ __forceinline__ void split_merge_stats(const ClSplitArgs &a, const fl
   var = m2 * a.inv_R;
 }
 
+// The (mean, m2) part of block sp of a sample for the thread's units, in ONE
+// pass over the block's vectors, which every wave takes as its own loads
+// arrive (the memory system serves a CU's waves one after the other: what a
+// wave does before the block's first barrier hides behind the other waves'
+// loads; a second pass about the block's mean kept memory idle for 2.2 us of
+// an instance's 18).  Per thread and unit, with the thread's first element as
+// the shift K: s1 = sum (x - K), s2 = sum (x - K)^2 over its n elements; then
+// mean = sum_t (n K + s1) / count and, about it, m2 = sum_t (s2 + 2 e s1 + n e^2)
+// with e = K - mean: two block sums of a few operations per thread.  K is one
+// of the thread's own elements, so the three terms cancel to no less than that
+// element's own share of m2.  get(k): the vector at position
+// sp * PB + prow + k * PR (asked for only where that lies inside the plane).
+// ROLLED: a loop (vectors from global memory, few registers) instead of
+// straight-line code; the arithmetic is the same, element by element.
+template <typename T, int VEC, int NL, int TPR, bool INSTANCE, bool ROLLED, class Get>
+__device__ __forceinline__ void split_block_part(const ClSplitArgs &a, int sp, uint32_t prow,
+                                                 uint32_t cvx, uint32_t gi, float per_pos, Get get,
+                                                 float (*fold)[kSplitTV * (INSTANCE ? VEC : 1)],
+                                                 float *tot, float (&m)[INSTANCE ? VEC : 1],
+                                                 float (&q)[INSTANCE ? VEC : 1]) {
+  constexpr int PR = TPR / kSplitTV;
+  constexpr int SV = INSTANCE ? VEC : 1;
+  const int left = a.P - sp * a.PB - static_cast<int>(prow); // positions from the thread's first on
+  const int nk = left <= 0 ? 0 : min(NL, (left + PR - 1) / PR); // the thread's vectors
+  float kk[SV], s1[SV], s2[SV];
+#pragma unroll
+  for (int j = 0; j < SV; ++j) kk[j] = s1[j] = s2[j] = 0.f;
+  if (nk > 0) {
+    const RawVec<T, VEC> r0 = get(0);
+#pragma unroll
+    for (int j = 0; j < SV; ++j) kk[j] = elem_fma<T, VEC>(r0, j, a.one, 0.f);
+    if constexpr (!INSTANCE) {
+#pragma unroll
+      for (int j = 1; j < VEC; ++j) {
+        const float d = elem_fma<T, VEC>(r0, j, a.one, -kk[0]);
+        s1[0] += d;
+        s2[0] = fmaf(d, d, s2[0]);
+      }
+    }
+  }
+  auto take = [&](int k) {
+    const RawVec<T, VEC> r = get(k);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const int ju = INSTANCE ? j : 0;
+      const float d = elem_fma<T, VEC>(r, j, a.one, -kk[ju]);
+      s1[ju] += d;
+      s2[ju] = fmaf(d, d, s2[ju]);
+    }
+  };
+  if constexpr (ROLLED) {
+#pragma unroll 1
+    for (int k = 1; k < nk; ++k) take(k);
+  } else {
+#pragma unroll
+    for (int k = 1; k < NL; ++k) {
+      if (k < nk) take(k);
+    }
+  }
+  const float nt = static_cast<float>(nk * (INSTANCE ? 1 : VEC));
+  const float cnt = split_count(a, sp) * per_pos;
+  if constexpr (INSTANCE) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) m[j] = fmaf(nt, kk[j], s1[j]);
+    split_channel_sums<TPR, VEC>(m, cvx, fold, tot);
+    const float icnt = 1.0f / cnt;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      m[j] *= icnt;
+      const float e = kk[j] - m[j];
+      q[j] = fmaf(e, fmaf(nt, e, 2.f * s1[j]), s2[j]);
+    }
+    split_channel_sums<TPR, VEC>(q, cvx, fold, tot);
+  } else {
+    m[0] = split_group_sum<TPR>(fmaf(nt, kk[0], s1[0]), a.cvg_shift, cvx, gi, fold) / cnt;
+    const float e = kk[0] - m[0];
+    q[0] = split_group_sum<TPR>(fmaf(e, fmaf(nt, e, 2.f * s1[0]), s2[0]), a.cvg_shift, cvx, gi, fold);
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Forward.  Block b = ((n * split + s) * tiles + tile); thread t owns vector
 // t % 8 of the tile at positions s * PB + t / 8 + k * (TPR / 8), k < NL.
@@ -269,68 +349,15 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
   }
 
   float mean[INSTANCE ? VEC : 1], var[INSTANCE ? VEC : 1];
-  if constexpr (!INSTANCE) {
-    // ---- this block's part: mean, then the second moment about it
-    float sum = 0.f;
+  // ---- this block's part
+  split_block_part<T, VEC, NL, TPR, INSTANCE, false>(
+      a, static_cast<int>(s), prow, cvx, gi, per_pos, [&](int k) { return raw[k]; }, fold, tot, mean, var);
+  if (writer) {
 #pragma unroll
-    for (int k = 0; k < NL; ++k) sum = raw_sum<T, VEC>(raw[k], sum);
-    const float cnt = split_count(a, s) * per_pos;
-    const float m = split_group_sum<TPR>(sum, a.cvg_shift, cvx, gi, fold) / cnt;
-#pragma unroll
-    for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
-    float q = 0.f;
-#pragma unroll
-    for (int k = 0; k < NL; ++k) {
-      if (s * a.PB + prow + k * PR < static_cast<uint32_t>(a.P)) {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          const float d = elem_fma<T, VEC>(raw[k], j, a.one, -m);
-          q = fmaf(d, d, q);
-        }
-      }
-    }
-    q = split_group_sum<TPR>(q, a.cvg_shift, cvx, gi, fold);
-    if (writer) {
-      part[s * per + gi * 2] = m;
-      part[s * per + gi * 2 + 1] = q;
-    }
-  } else {
-    float sum[VEC];
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) sum[j] = 0.f;
-#pragma unroll
-    for (int k = 0; k < NL; ++k) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) sum[j] = elem_fma<T, VEC>(raw[k], j, a.one, sum[j]);
-    }
-    split_channel_sums<TPR, VEC>(sum, cvx, fold, tot);
-    const float icnt = 1.0f / split_count(a, s);
-    float m[VEC], q[VEC];
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      m[j] = sum[j] * icnt;
-      q[j] = 0.f;
-    }
-#pragma unroll
-    for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
-#pragma unroll
-    for (int k = 0; k < NL; ++k) {
-      if (s * a.PB + prow + k * PR < static_cast<uint32_t>(a.P)) {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          const float d = elem_fma<T, VEC>(raw[k], j, a.one, -m[j]);
-          q[j] = fmaf(d, d, q[j]);
-        }
-      }
-    }
-    split_channel_sums<TPR, VEC>(q, cvx, fold, tot);
-    if (writer) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const int u = cvx * VEC + j;
-        part[s * per + u * 2] = m[j];
-        part[s * per + u * 2 + 1] = q[j];
-      }
+    for (int j = 0; j < (INSTANCE ? VEC : 1); ++j) {
+      const int u = INSTANCE ? static_cast<int>(cvx) * VEC + j : static_cast<int>(gi);
+      part[s * per + u * 2] = mean[j];
+      part[s * per + u * 2 + 1] = var[j];
     }
   }
 
@@ -342,74 +369,18 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
     if (sp == static_cast<int>(s) || !missing[sp]) continue; // same answer in every thread
     // Partner sp has not published: its part from global memory, one vector
     // at a time (the block's own vectors stay in registers).
-    const float cnt = split_count(a, sp);
-    if constexpr (!INSTANCE) {
-      float sum = 0.f;
-#pragma unroll 1
-      for (int k = 0; k < NL; ++k) {
-        const uint32_t pos = sp * a.PB + prow + k * PR;
-        const bool ok = pos < static_cast<uint32_t>(a.P);
-        const RawVec<T, VEC> r = raw_or_zero<T, VEC>(
-            ok, load_raw<T, VEC>(x + static_cast<size_t>(ok ? pos : sp * a.PB) * a.C));
-        sum = raw_sum<T, VEC>(r, sum);
-      }
-      const float m = split_group_sum<TPR>(sum, a.cvg_shift, cvx, gi, fold) / (cnt * per_pos);
-      float q = 0.f;
-#pragma unroll 1
-      for (int k = 0; k < NL; ++k) {
-        const uint32_t pos = sp * a.PB + prow + k * PR;
-        if (pos < static_cast<uint32_t>(a.P)) {
-          const RawVec<T, VEC> r = load_raw<T, VEC>(x + static_cast<size_t>(pos) * a.C);
+    split_block_part<T, VEC, NL, TPR, INSTANCE, true>(
+        a, sp, prow, cvx, gi, per_pos,
+        [&](int k) {
+          return load_raw<T, VEC>(x + static_cast<size_t>(sp * a.PB + prow + k * PR) * a.C);
+        },
+        fold, tot, mean, var);
+    if (writer) {
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) {
-            const float d = elem_fma<T, VEC>(r, j, a.one, -m);
-            q = fmaf(d, d, q);
-          }
-        }
-      }
-      q = split_group_sum<TPR>(q, a.cvg_shift, cvx, gi, fold);
-      if (writer) {
-        part[sp * per + gi * 2] = m;
-        part[sp * per + gi * 2 + 1] = q;
-      }
-    } else {
-      float sum[VEC], m[VEC], q[VEC];
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) sum[j] = 0.f;
-#pragma unroll 1
-      for (int k = 0; k < NL; ++k) {
-        const uint32_t pos = sp * a.PB + prow + k * PR;
-        const bool ok = pos < static_cast<uint32_t>(a.P);
-        const RawVec<T, VEC> r = raw_or_zero<T, VEC>(
-            ok, load_raw<T, VEC>(x + static_cast<size_t>(ok ? pos : sp * a.PB) * a.C));
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) sum[j] = elem_fma<T, VEC>(r, j, a.one, sum[j]);
-      }
-      split_channel_sums<TPR, VEC>(sum, cvx, fold, tot);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        m[j] = sum[j] * (1.0f / cnt); // as the owner computes it
-        q[j] = 0.f;
-      }
-#pragma unroll 1
-      for (int k = 0; k < NL; ++k) {
-        const uint32_t pos = sp * a.PB + prow + k * PR;
-        if (pos < static_cast<uint32_t>(a.P)) {
-          const RawVec<T, VEC> r = load_raw<T, VEC>(x + static_cast<size_t>(pos) * a.C);
-#pragma unroll
-          for (int j = 0; j < VEC; ++j) {
-            const float d = elem_fma<T, VEC>(r, j, a.one, -m[j]);
-            q[j] = fmaf(d, d, q[j]);
-          }
-        }
-      }
-      split_channel_sums<TPR, VEC>(q, cvx, fold, tot);
-      if (writer) {
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          part[sp * per + (cvx * VEC + j) * 2] = m[j];
-          part[sp * per + (cvx * VEC + j) * 2 + 1] = q[j];
-        }
+      for (int j = 0; j < (INSTANCE ? VEC : 1); ++j) {
+        const int u = INSTANCE ? static_cast<int>(cvx) * VEC + j : static_cast<int>(gi);
+        part[sp * per + u * 2] = mean[j];
+        part[sp * per + u * 2 + 1] = var[j];
       }
     }
     lds_barrier();

@@ -38,16 +38,19 @@ SplitPlan plan_split(const ClProblem &p, bool aligned, bool backward) {
   s.tiles = static_cast<int>(p.channels / tile_ch);
   // Block shape: positions per block PB = NL * TPR / 8 (128, 256, 512 or 1024);
   // planes beyond 16 blocks of the largest shape are left to the other kernels.
-  // First choice, from a sweep of shapes (cold, forward / backward us):
-  //  groups, forward: 256 x 8, four blocks to a CU (float and planes from 4096
-  //    positions: 512 x 8 - [16,64,64,256] half 15.5 vs 15.7, float 25.0 vs 26.7);
-  //  groups, backward: 512 x 8 where that still gives two blocks per CU
-  //    ([16,64,64,256] 23.5 vs 25.4, [32,56,56,256] 38.7 vs 41.6), else 256 x 8
-  //    ([4,32,32,1024] 11.4 vs 12.4);
-  //  instances exchange 64 channels x 2 words per block and partner, so fewer,
-  //    larger blocks: 512 x 8 up to 2048 positions ([32,28,28,512] 14.6 / 21.6
-  //    against 20.9 / 40.9 with the line-piece kernels), 1024 x 8 beyond
-  //    ([16,64,64,256] 19.0 / 27.4 against 21.6 / 40.4);
+  // First choice, from sweeps of the shapes (cold, forward / backward us):
+  //  forward: several blocks to a CU, so that one block's exchange and stores
+  //    run while the next one's loads arrive - groups 256 x 8 (float and planes
+  //    from 4096 positions: 512 x 8; [16,64,64,256] half 13.7 vs 14.3), instances
+  //    512 x 8 ([16,64,64,256] 15.2 against 17.1 with 1024 x 8), 256 x 8 where
+  //    512 x 8 leaves CUs without a block ([4,32,32,1024] 7.9 vs 8.8);
+  //  backward: 1024 x 8, one block per CU (dy waits in 128 KB of LDS), for
+  //    instances and for groups whose plane one such block holds whole, where
+  //    that gives every CU a block and the plane's last block is not mostly
+  //    empty ([16,64,64,256] instances 22.8 vs 25.0; [32,28,28,512] groups
+  //    17.5 vs 20.2; but [32,56,56,128] instances, 3136 = 3 x 1024 + 64
+  //    positions, 22.1 vs 20.4); else 512 x 8 where that still gives two blocks
+  //    per CU (instances: one), else 256 x 8 ([4,32,32,1024] 11.1 vs 11.6);
   //  any plane that one block of a smaller shape holds whole takes that shape.
   static const int shapes[][2] = {{256, 4}, {256, 8}, {512, 8}, {1024, 8}, {512, 4}, {1024, 4}};
   const int ftpr = tune_int("GN_CL_SPLIT_TPR", 0), fnl = tune_int("GN_CL_SPLIT_NL", 0);
@@ -67,16 +70,26 @@ SplitPlan plan_split(const ClProblem &p, bool aligned, bool backward) {
     for (int i = 0; i < 6 && !s.ok; ++i)
       if (shapes[i][0] == ftpr && shapes[i][1] == fnl) take(i);
   } else {
+    const int64_t cus = device_cus();
+    auto blocks_of = [&](int i) {
+      const int64_t pb = static_cast<int64_t>(shapes[i][0]) * shapes[i][1] / kSplitTV;
+      return p.batch * s.tiles * ((p.spatial + pb - 1) / pb);
+    };
+    auto well_filled = [&](int i) { // the plane's blocks hold at least 90 % of their positions
+      const int64_t pb = static_cast<int64_t>(shapes[i][0]) * shapes[i][1] / kSplitTV;
+      return p.spatial * 10 >= ((p.spatial + pb - 1) / pb) * pb * 9;
+    };
     int first = 1; // 256 x 8
     if (p.spatial <= 128) {
       first = 0;
     } else if (p.spatial <= 256) {
       first = 1;
+    } else if (backward && blocks_of(3) >= cus && well_filled(3) && (s.instance || p.spatial <= 1024)) {
+      first = 3;
     } else if (s.instance) {
-      first = p.spatial <= 2048 ? 2 : 3;
+      first = blocks_of(2) >= cus ? 2 : 1;
     } else if (backward) {
-      const int64_t blocks512 = p.batch * s.tiles * ((p.spatial + 511) / 512);
-      if (blocks512 >= 2 * static_cast<int64_t>(device_cus())) first = 2;
+      if (blocks_of(2) >= 2 * cus) first = 2;
     } else if (p.spatial >= 4096 || (p.dtype == NBLAHIP_F32 && p.spatial >= 2048)) {
       first = 2;
     }

@@ -13,10 +13,14 @@ from _util import assert_close, load_package, to_np
 K = load_package()
 
 # (shape, axis, dtype name): tensors that take the split reduction, i.e. use
-# the scratch array (channel-last with many rows; planes with few channels).
+# the scratch array (channel-last with many rows - 96 channels, which the
+# kernel that holds the tensor on the chip does not take; planes with few
+# channels), and a pair that does not need it (held on the chip, the partials
+# travel through the exchange array): the entry point must agree there too.
 CASES = [
-    [((64, 56, 56, 64), 3, "f16"), ((8, 28, 28, 32), 3, "f16")],
-    [((32, 16, 56, 56), 1, "f32"), ((32, 8, 40, 40), 1, "f32")],
+    ([((64, 56, 56, 96), 3, "f16"), ((8, 28, 28, 32), 3, "f16")], True),
+    ([((32, 16, 56, 56), 1, "f32"), ((32, 8, 40, 40), 1, "f32")], True),
+    ([((64, 56, 56, 64), 3, "f16"), ((56, 56, 56, 64), 3, "f16")], False),
 ]
 
 
@@ -47,8 +51,9 @@ def test_shapes_beyond_the_static_array_are_rejected():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("pair", CASES, ids=["channel_last_f16", "planes_f32"])
-def test_static_scratch_matches_the_workspace_entry_point(pair):
+@pytest.mark.parametrize("pair,partials", CASES,
+                         ids=["channel_last_f16", "planes_f32", "channel_last_on_chip_f16"])
+def test_static_scratch_matches_the_workspace_entry_point(pair, partials):
     import torch
     from oracle import norm_ref as R
     L = K.lib()
@@ -66,7 +71,7 @@ def test_static_scratch_matches_the_workspace_entry_point(pair):
         torch.cuda.synchronize()
         _, fin = K.profile_query("bn_finalize_fwd_kernel")
         K.check(L.nblahip_profile_enable(0))
-        assert fin == 1, "shape does not take the split reduction"
+        assert fin == (1 if partials else 0), "the split reduction was expected / not expected"
         out = (torch.full_like(x, float("nan")), torch.empty_like(m_a), torch.empty_like(v_a))
         # (torch's allocator only sees the wrapper; the library itself never
         # calls an allocating routine)
