@@ -316,7 +316,7 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
           const float xh = norm_elem<T, VEC>(xr, j, mean, istd, nmi);
           px = elem_fma<T, VEC>(d[b], j, xh, px);
         }
-        const bool ok = static_cast<uint32_t>(k) * TB + t < a.nv;
+        const bool ok = static_cast<int>(t) < static_cast<int>(a.nv) - k * TB; // t against a scalar
         sdy += ok ? py : 0.f;
         sdx += ok ? px : 0.f;
       }

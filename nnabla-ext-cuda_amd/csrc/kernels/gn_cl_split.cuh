@@ -317,7 +317,7 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
   __shared__ float fold[NW][UMAX];
   __shared__ float tot[UMAX];
   __shared__ float part[kSplitMax * UMAX * 2];
-  __shared__ float merged[UMAX * 2];
+  __shared__ float merged[UMAX * 2]; // (mean, 1 / std) per unit
   __shared__ int missing[kSplitMax];
   const uint32_t tile = blockIdx.x % a.tiles, ns = blockIdx.x / a.tiles;
   const uint32_t s = ns % a.split, n = ns / a.split;
@@ -394,7 +394,7 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
     float m, v;
     split_merge_stats(a, part, per, u, per_pos, m, v);
     merged[2 * u] = m;
-    merged[2 * u + 1] = v;
+    merged[2 * u + 1] = inv_std(v, a.eps); // once per unit, not once per thread and channel
     if (s == 0) {
       const size_t ug = INSTANCE ? static_cast<size_t>(n) * a.C + tile * TV * VEC + u
                                  : static_cast<size_t>(n) * (a.C / a.cpg) + (tile * TV * VEC) / a.cpg + u;
@@ -407,7 +407,7 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
   for (int j = 0; j < (INSTANCE ? VEC : 1); ++j) {
     const int u = INSTANCE ? static_cast<int>(cvx) * VEC + j : static_cast<int>(gi);
     mean[j] = merged[2 * u];
-    var[j] = merged[2 * u + 1];
+    var[j] = merged[2 * u + 1]; // (1 / std from here on)
   }
 #pragma unroll
   for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
@@ -415,7 +415,7 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
     const int ju = INSTANCE ? j : 0;
-    sc[j] = gam[j] * inv_std(var[ju], a.eps);
+    sc[j] = gam[j] * var[ju];
     mu[j] = mean[ju];
     sh[j] = fmaf(-mean[ju], sc[j], bet[j]);
   }
