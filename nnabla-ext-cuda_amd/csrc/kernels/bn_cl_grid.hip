@@ -116,10 +116,10 @@ __device__ __forceinline__ float grid_channel_sum1(float v, uint32_t cv, uint32_
 
 // (mean, m2) of the rows of block p for channel c, from global memory, in the
 // order block p itself uses (its thread map, slots ascending per thread, the
-// thread's first element as the shift, the same folds): what block p
-// publishes for c, bit for bit.  Only the threads of c's channel vector load
-// (the folds never mix channel vectors) and only c's element is accumulated,
-// so this costs a handful of registers.
+// thread's own mean as the shift, the same folds): what block p publishes for
+// c, bit for bit.  Only the threads of c's channel vector load (the folds
+// never mix channel vectors) and only c's element is accumulated, so this
+// costs a handful of registers.
 template <typename T, int VEC>
 __device__ __forceinline__ void grid_partial_from_memory(const BnClGridArgs &a, uint32_t p,
                                                          uint32_t c, float *fold, float &m,
@@ -129,30 +129,33 @@ __device__ __forceinline__ void grid_partial_from_memory(const BnClGridArgs &a, 
   const uint32_t cvx = t % a.cv, e = c % VEC;
   const uint32_t vbb = grid_block_vectors(a, p);
   const bool mine = cvx == c / VEC;
+  const uint32_t vbp = mine ? vbb : 0u;
   const size_t first = static_cast<size_t>(p) * a.vb;
-  float kk = 0.f, s1 = 0.f, s2 = 0.f, nt = 0.f;
-  if (mine && t < vbb) {
-    const RawVec<T, VEC> r0 = load_raw<T, VEC>(x + (first + t) * VEC);
+  float s = 0.f, s1 = 0.f, s2 = 0.f;
+#pragma unroll 1
+  for (uint32_t v = t; v < vbp; v += kOnchipBlock) {
+    const RawVec<T, VEC> r = load_raw<T, VEC>(x + (first + v) * VEC);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-      const float v0 = elem_fma<T, VEC>(r0, j, a.one, 0.f);
-      kk = static_cast<uint32_t>(j) == e ? v0 : kk;
-    }
-    nt = static_cast<float>((vbb - 1u - t) / kOnchipBlock + 1u);
-#pragma unroll 1
-    for (uint32_t v = t + kOnchipBlock; v < vbb; v += kOnchipBlock) {
-      const RawVec<T, VEC> r = load_raw<T, VEC>(x + (first + v) * VEC);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const float d = elem_fma<T, VEC>(r, j, a.one, -kk);
-        const float n1 = s1 + d;
-        const float n2 = fmaf(d, d, s2);
-        s1 = static_cast<uint32_t>(j) == e ? n1 : s1;
-        s2 = static_cast<uint32_t>(j) == e ? n2 : s2;
-      }
+      const float n = elem_fma<T, VEC>(r, j, a.one, s);
+      s = static_cast<uint32_t>(j) == e ? n : s;
     }
   }
-  m = grid_channel_sum1(fmaf(nt, kk, s1), a.cv, cvx, c, mine, fold, a.C);
+  const float nt = (mine && t < vbb) ? static_cast<float>((vbb - 1u - t) / kOnchipBlock + 1u) : 0.f;
+  const float kk = s * (1.0f / fmaxf(nt, 1.f));
+#pragma unroll 1
+  for (uint32_t v = t; v < vbp; v += kOnchipBlock) {
+    const RawVec<T, VEC> r = load_raw<T, VEC>(x + (first + v) * VEC);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      const float d = elem_fma<T, VEC>(r, j, a.one, -kk);
+      const float n1 = s1 + d;
+      const float n2 = fmaf(d, d, s2);
+      s1 = static_cast<uint32_t>(j) == e ? n1 : s1;
+      s2 = static_cast<uint32_t>(j) == e ? n2 : s2;
+    }
+  }
+  m = grid_channel_sum1(s, a.cv, cvx, c, mine, fold, a.C);
   m *= 1.0f / static_cast<float>(vbb / a.cv);
   const float d = kk - m;
   q = grid_channel_sum1(mine ? fmaf(d, fmaf(nt, d, 2.f * s1), s2) : 0.f, a.cv, cvx, c, mine, fold, a.C);
@@ -332,30 +335,36 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
   // (slot k holds a vector of the block: t against a scalar, no register per slot)
   auto holds = [&](int k) { return static_cast<int>(t) < static_cast<int>(vbb) - k * kOnchipBlock; };
 
-  // ---- this block's partial per channel, in ONE pass over the slots, taken by
-  // every wave as its own loads arrive (the memory system serves a CU's waves
+  // ---- this block's partial per channel, from sums every wave takes over its
+  // OWN registers as its loads arrive (the memory system serves a CU's waves
   // one after the other, 2 to 18 us after the start here: what a wave does
   // before the block's first barrier hides behind the other waves' loads, what
   // comes after it keeps memory idle - a second pass about the block's mean
-  // cost 5.8 us of [256,56,56,64]'s 49).  Per thread and channel, with the
-  // thread's first element as the shift K: s1 = sum (x - K), s2 = sum (x - K)^2
-  // over its n slots.  Then mean = sum_t (n K + s1) / rows, and about it
+  // cost 5.8 us of [256,56,56,64]'s 49).  Per thread and channel: s = sum x,
+  // then about the thread's own mean K = s / n: s1 = sum (x - K) (rounding
+  // residue), s2 = sum (x - K)^2.  Then mean = sum_t s / rows, and about it
   // m2 = sum_t (s2 + 2 e s1 + n e^2), e = K - mean: two block sums of a few
-  // operations per thread.  K is one of the thread's own values, so the three
-  // terms cancel to no less than that element's own share of m2.
+  // operations per thread.  sum_t n e^2 is the variance between the threads'
+  // means, never more than m2 itself: nothing cancels, whatever the data.
   float m[VEC], q[VEC];
   {
     float kk[VEC], s1[VEC], s2[VEC];
-    {
-      const RawVec<T, VEC> r0 = slot(0);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        kk[j] = holds(0) ? elem_fma<T, VEC>(r0, j, a.one, 0.f) : 0.f;
-        s1[j] = s2[j] = 0.f;
+    for (int j = 0; j < VEC; ++j) m[j] = s1[j] = s2[j] = 0.f;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      if (holds(k)) {
+        const RawVec<T, VEC> r = slot(k);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) m[j] = elem_fma<T, VEC>(r, j, a.one, m[j]);
       }
     }
+    const float nt = t < vbb ? static_cast<float>((vbb - 1u - t) / kOnchipBlock + 1u) : 0.f;
+    const float rnt = 1.0f / fmaxf(nt, 1.f);
 #pragma unroll
-    for (int k = 1; k < NL; ++k) {
+    for (int j = 0; j < VEC; ++j) kk[j] = m[j] * rnt;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
       if (holds(k)) {
         const RawVec<T, VEC> r = slot(k);
 #pragma unroll
@@ -366,9 +375,6 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
         }
       }
     }
-    const float nt = t < vbb ? static_cast<float>((vbb - 1u - t) / kOnchipBlock + 1u) : 0.f;
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) m[j] = fmaf(nt, kk[j], s1[j]);
     grid_channel_sums<VEC>(m, a.cv, cvx, fold, tot, a.C);
     const float icnt = 1.0f / static_cast<float>(vbb / a.cv);
 #pragma unroll

@@ -107,18 +107,35 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
     const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t;
     raw[k] = load_raw<T, VEC>(x + onchip_offset(a, c, min(v, a.nv - 1u), VEC));
   }
-  // Statistics in ONE pass, taken by every wave as its own loads arrive (the
-  // memory system serves a CU's waves one after the other: what a wave does
-  // before the block's first barrier hides behind the other waves' loads, a
-  // second pass about the mean would keep memory idle).  Per thread, with its
-  // first element as the shift K: s1 = sum (x - K), s2 = sum (x - K)^2 over its
-  // n elements; mean = sum_t (n K + s1) / N and, about it,
-  // var = sum_t (s2 + 2 e s1 + n e^2) / N with e = K - mean: two block sums of
-  // a few operations per thread.  K is one of the thread's own elements, so
-  // the three terms cancel to no less than that element's own share.
-  // (OVER: the vectors beyond the held ones are read here once, and once more for y.)
+  // Statistics from sums every wave takes over its OWN registers as its loads
+  // arrive (the memory system serves a CU's waves one after the other: what a
+  // wave does before the block's first barrier hides behind the other waves'
+  // loads, a second pass about the block's mean would keep memory idle).  Per
+  // thread: s = sum x, then about the thread's own mean K = s / n:
+  // s1 = sum (x - K) (rounding residue), s2 = sum (x - K)^2; mean = sum_t s / N
+  // and, about it, var = sum_t (s2 + 2 e s1 + n e^2) / N with e = K - mean: two
+  // block sums of a few operations per thread.  sum_t n e^2 is the variance
+  // between the threads' means, never more than the total: nothing cancels,
+  // whatever the data.
+  // (OVER: the vectors beyond the held ones are read here once, shifted by the
+  // K of the thread's held elements, and once more for y.)
   auto held = [&](int k) { return static_cast<int>(t) < static_cast<int>(a.nv) - k * kOnchipBlock; };
-  const float kk = held(0) ? elem_fma<T, VEC>(raw[0], 0, a.one, 0.f) : 0.f;
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < NS; ++k) {
+    const float part = raw_sum<T, VEC>(parked[k], 0.f);
+    s += held(NR + k) ? part : 0.f;
+    spill[k * kOnchipBlock + t] = __builtin_bit_cast(Slot<T, VEC>, parked[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < NR; ++k) {
+    const float part = raw_sum<T, VEC>(raw[k], 0.f);
+    s += held(k) ? part : 0.f;
+  }
+  constexpr uint32_t kHeld = static_cast<uint32_t>(NR + NS) * kOnchipBlock;
+  const uint32_t nvh = OVER ? min(a.nv, kHeld) : a.nv; // held vectors of the channel
+  const float nh = t < nvh ? static_cast<float>(((nvh - 1u - t) / kOnchipBlock + 1u) * VEC) : 0.f;
+  const float kk = s * (1.0f / fmaxf(nh, 1.f));
   float s1 = 0.f, s2 = 0.f;
   auto take = [&](const RawVec<T, VEC> &r) {
 #pragma unroll
@@ -131,13 +148,12 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
 #pragma unroll
   for (int k = 0; k < NS; ++k) {
     if (held(NR + k)) take(parked[k]);
-    spill[k * kOnchipBlock + t] = __builtin_bit_cast(Slot<T, VEC>, parked[k]);
   }
 #pragma unroll
   for (int k = 0; k < NR; ++k) {
     if (held(k)) take(raw[k]);
   }
-  constexpr uint32_t kHeld = static_cast<uint32_t>(NR + NS) * kOnchipBlock;
+  float nt = nh; // elements of the thread, held and streamed
   if constexpr (OVER) {
     constexpr int BO = 4;
 #pragma unroll 1
@@ -151,8 +167,9 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
         if (v0 + b * kOnchipBlock + t < a.nv) take(xo[b]);
       }
     }
+    nt = t < a.nv ? static_cast<float>(((a.nv - 1u - t) / kOnchipBlock + 1u) * VEC) : 0.f;
   }
-  const float nt = t < a.nv ? static_cast<float>(((a.nv - 1u - t) / kOnchipBlock + 1u) * VEC) : 0.f;
+  // (n K + s1 = the thread's sum of x, held and streamed)
   const float mean = onchip_block_sum(fmaf(nt, kk, s1), red) * a.inv_N;
   const float e = kk - mean;
   const float var = onchip_block_sum(fmaf(e, fmaf(nt, e, 2.f * s1), s2), red) * a.inv_N;

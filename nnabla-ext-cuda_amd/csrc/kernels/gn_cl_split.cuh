@@ -223,20 +223,20 @@ __device__ __forceinline__ void split_merge_stats(const ClSplitArgs &a, const fl
   var = m2 * a.inv_R;
 }
 
-// The (mean, m2) part of block sp of a sample for the thread's units, in ONE
-// pass over the block's vectors, which every wave takes as its own loads
-// arrive (the memory system serves a CU's waves one after the other: what a
-// wave does before the block's first barrier hides behind the other waves'
-// loads; a second pass about the block's mean kept memory idle for 2.2 us of
-// an instance's 18).  Per thread and unit, with the thread's first element as
-// the shift K: s1 = sum (x - K), s2 = sum (x - K)^2 over its n elements; then
-// mean = sum_t (n K + s1) / count and, about it, m2 = sum_t (s2 + 2 e s1 + n e^2)
-// with e = K - mean: two block sums of a few operations per thread.  K is one
-// of the thread's own elements, so the three terms cancel to no less than that
-// element's own share of m2.  get(k): the vector at position
-// sp * PB + prow + k * PR (asked for only where that lies inside the plane).
-// ROLLED: a loop (vectors from global memory, few registers) instead of
-// straight-line code; the arithmetic is the same, element by element.
+// The (mean, m2) part of block sp of a sample for the thread's units, from
+// sums every wave takes over its OWN vectors as its loads arrive (the memory
+// system serves a CU's waves one after the other: what a wave does before the
+// block's first barrier hides behind the other waves' loads; a second pass
+// about the block's mean kept memory idle).  Per thread and unit: s = sum x,
+// then about the thread's own mean K = s / n: s1 = sum (x - K) (rounding
+// residue), s2 = sum (x - K)^2; then mean = sum_t s / count and, about it,
+// m2 = sum_t (s2 + 2 e s1 + n e^2) with e = K - mean: two block sums of a few
+// operations per thread.  sum_t n e^2 is the variance between the threads'
+// means, never more than m2 itself: nothing cancels, whatever the data.
+// get(k): the vector at position sp * PB + prow + k * PR (asked for only where
+// that lies inside the plane).  ROLLED: loops (vectors from global memory, few
+// registers) instead of straight-line code; the arithmetic is the same,
+// element by element.
 template <typename T, int VEC, int NL, int TPR, bool INSTANCE, bool ROLLED, class Get>
 __device__ __forceinline__ void split_block_part(const ClSplitArgs &a, int sp, uint32_t prow,
                                                  uint32_t cvx, uint32_t gi, float per_pos, Get get,
@@ -249,20 +249,15 @@ __device__ __forceinline__ void split_block_part(const ClSplitArgs &a, int sp, u
   const int nk = left <= 0 ? 0 : min(NL, (left + PR - 1) / PR); // the thread's vectors
   float kk[SV], s1[SV], s2[SV];
 #pragma unroll
-  for (int j = 0; j < SV; ++j) kk[j] = s1[j] = s2[j] = 0.f;
-  if (nk > 0) {
-    const RawVec<T, VEC> r0 = get(0);
+  for (int j = 0; j < SV; ++j) m[j] = s1[j] = s2[j] = 0.f;
+  auto add = [&](int k) {
+    const RawVec<T, VEC> r = get(k);
 #pragma unroll
-    for (int j = 0; j < SV; ++j) kk[j] = elem_fma<T, VEC>(r0, j, a.one, 0.f);
-    if constexpr (!INSTANCE) {
-#pragma unroll
-      for (int j = 1; j < VEC; ++j) {
-        const float d = elem_fma<T, VEC>(r0, j, a.one, -kk[0]);
-        s1[0] += d;
-        s2[0] = fmaf(d, d, s2[0]);
-      }
+    for (int j = 0; j < VEC; ++j) {
+      const int ju = INSTANCE ? j : 0;
+      m[ju] = elem_fma<T, VEC>(r, j, a.one, m[ju]);
     }
-  }
+  };
   auto take = [&](int k) {
     const RawVec<T, VEC> r = get(k);
 #pragma unroll
@@ -273,20 +268,29 @@ __device__ __forceinline__ void split_block_part(const ClSplitArgs &a, int sp, u
       s2[ju] = fmaf(d, d, s2[ju]);
     }
   };
+  const float nt = static_cast<float>(nk * (INSTANCE ? 1 : VEC));
+  const float rnt = 1.0f / fmaxf(nt, 1.f);
   if constexpr (ROLLED) {
 #pragma unroll 1
-    for (int k = 1; k < nk; ++k) take(k);
+    for (int k = 0; k < nk; ++k) add(k);
+#pragma unroll
+    for (int j = 0; j < SV; ++j) kk[j] = m[j] * rnt;
+#pragma unroll 1
+    for (int k = 0; k < nk; ++k) take(k);
   } else {
 #pragma unroll
-    for (int k = 1; k < NL; ++k) {
+    for (int k = 0; k < NL; ++k) {
+      if (k < nk) add(k);
+    }
+#pragma unroll
+    for (int j = 0; j < SV; ++j) kk[j] = m[j] * rnt;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
       if (k < nk) take(k);
     }
   }
-  const float nt = static_cast<float>(nk * (INSTANCE ? 1 : VEC));
   const float cnt = split_count(a, sp) * per_pos;
   if constexpr (INSTANCE) {
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) m[j] = fmaf(nt, kk[j], s1[j]);
     split_channel_sums<TPR, VEC>(m, cvx, fold, tot);
     const float icnt = 1.0f / cnt;
 #pragma unroll
@@ -297,7 +301,7 @@ __device__ __forceinline__ void split_block_part(const ClSplitArgs &a, int sp, u
     }
     split_channel_sums<TPR, VEC>(q, cvx, fold, tot);
   } else {
-    m[0] = split_group_sum<TPR>(fmaf(nt, kk[0], s1[0]), a.cvg_shift, cvx, gi, fold) / cnt;
+    m[0] = split_group_sum<TPR>(m[0], a.cvg_shift, cvx, gi, fold) / cnt;
     const float e = kk[0] - m[0];
     q[0] = split_group_sum<TPR>(fmaf(e, fmaf(nt, e, 2.f * s1[0]), s2[0]), a.cvg_shift, cvx, gi, fold);
   }

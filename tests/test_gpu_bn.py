@@ -505,6 +505,50 @@ def test_bn_channel_last_backward_held_on_the_chip(m, c, dtype):
     assert torch.equal(params[1], dg) and torch.equal(params[2], db)
 
 
+@pytest.mark.parametrize("kind", ["offset", "outlier_first", "constant"])
+@pytest.mark.parametrize("shape,axis,dtype,kernel", [
+    ((32, 64, 56, 56), 1, torch.float32, "bn_onchip_fwd_kernel"),
+    ((32, 64, 56, 56), 1, torch.float16, "bn_onchip_fwd_kernel"),
+    ((150000, 64), 1, torch.float32, "bn_cl_grid_fwd_kernel"),
+    ((150000, 64), 1, torch.float16, "bn_cl_grid_fwd_kernel"),
+])
+def test_one_pass_statistics_on_hard_data(kind, shape, axis, dtype, kernel):
+    """The statistics shift by each thread's own mean: a mean far
+    from zero, one huge value in the very first element of every channel (1000
+    deviations off everything else its thread holds), and constant data
+    (variance 0 to rounding) must all come out within the statistics' tolerance."""
+    dn = dtype_name(dtype)
+    rng = np.random.default_rng(77)
+    c = shape[axis]
+    if kind == "offset":
+        x = rng.standard_normal(shape) + (300.0 if dtype == torch.float32 else 40.0)
+    elif kind == "outlier_first":
+        x = rng.standard_normal(shape)
+        first = [0] * len(shape)
+        first[axis] = slice(None)
+        x[tuple(first)] = 1000.0
+    else:
+        x = np.full(shape, 3.25)
+    x = rounded(x, dtype)
+    y_r, m_r, v_r, _, _ = R.bn_forward_batch(x, None, None, None, None, axis, 0.9, 1e-5)
+    K.tune_set("BN_CL_GRID_MIN_SLOTS", 1)
+    try:
+        K.check(K.lib().nblahip_profile_enable(8))
+        y, m, v = K.bn_forward_batch(to_dev(x, dtype), None, None, None, None, axis, 0.9, 1e-5)
+        torch.cuda.synchronize()
+        assert K.profile_kernels() == [kernel]
+    finally:
+        K.check(K.lib().nblahip_profile_enable(0))
+        K.tune_reset()
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    if kind == "constant":
+        assert float(v.abs().max()) < 1e-10
+    # (at an offset of 300 a float x is itself only known to 3e-5, and so is x - mean)
+    assert_close(to_np(y), y_r, dn, "y", "y",
+                 scale=10.0 if kind == "offset" and dtype == torch.float32 else 1.0 if kind == "constant" else None)
+
+
 def test_two_chip_filling_forwards_at_once():
     """Two host threads, each on its own stream, run the forward that holds the
     whole tensor on the chip at the same time: each launch wants every CU, so

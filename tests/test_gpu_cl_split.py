@@ -109,6 +109,48 @@ def test_split_kernels_match_the_oracle_with_and_without_the_exchange(n, sp, c, 
         assert torch.equal(a_, b_)
 
 
+@pytest.mark.parametrize("kind", ["offset", "outlier_first", "constant"])
+@pytest.mark.parametrize("groups", [8, 64])
+@pytest.mark.parametrize("dtype", [F32, F16])
+def test_one_pass_statistics_on_hard_data(kind, groups, dtype):
+    """The statistics shift by each thread's own mean: a mean far
+    from zero, one huge value at the first position of every channel (1000
+    deviations off everything else its thread holds) and constant data
+    (variance 0 to rounding) must come out within the statistics' tolerance; groups of 8 channels and
+    instances."""
+    dn = dtype_name(dtype)
+    n, sp, c = 3, (40, 40), 64
+    rng = np.random.default_rng(78)
+    shape = (n,) + sp + (c,)
+    if kind == "offset":
+        x = rng.standard_normal(shape) + (300.0 if dtype == F32 else 40.0)
+    elif kind == "outlier_first":
+        x = rng.standard_normal(shape)
+        x[:, 0, 0, :] = 1000.0
+    else:
+        x = np.full(shape, 3.25)
+    x = rounded(x, dtype)
+    xt = to_cf(x)
+    K.check(K.lib().nblahip_profile_enable(8))
+    if groups == c:
+        y_r, m_r, v_r = R.in_forward(xt, None, None, n, c, 1e-5)
+        y, m, v = K.in_forward(to_dev(x, dtype), None, None, 1e-5, channel_last=True)
+    else:
+        y_r, m_r, v_r = R.gn_forward(xt, None, None, n, c, groups, 1e-5)
+        y, m, v = K.gn_forward(to_dev(x, dtype), None, None, groups, 1e-5, channel_last=True)
+    torch.cuda.synchronize()
+    names = K.profile_kernels()
+    K.check(K.lib().nblahip_profile_enable(0))
+    assert names == ["cl_split_fwd_kernel"], names
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    if kind == "constant":
+        assert float(v.abs().max()) < 1e-10
+    # (at an offset of 300 a float x is itself only known to 3e-5, and so is x - mean)
+    assert_close(to_np(y), to_cl(y_r.reshape(xt.shape)), dn, "y", "y",
+                 scale=10.0 if kind == "offset" and dtype == F32 else 1.0 if kind == "constant" else None)
+
+
 @pytest.mark.parametrize("spin", [64, 0])
 def test_split_flags(spin):
     """no_scale/no_bias, dmean/dvar, accumulation onto dx/dgamma/dbeta, parameter
