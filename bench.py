@@ -455,6 +455,17 @@ def config_table(K, steps, warmup, only=None):
             row[key + "_warm_us"] = round(warm * 1e3, 2)
             row[key + "_GBps"] = round(nbytes / ms / 1e6, 1)
         last = legs[-1][0]
+        # What the memory system gives a plain copy of one tensor of this size
+        # in the same rotated loop (x -> y of every buffer set in turn, 2 S per
+        # call): the practical ceiling beside the 8 TB/s of the data sheet.
+        def plain_copy(i, sets=w.sets):
+            b = sets[i % len(sets)]
+            b["y"].copy_(b["x"], non_blocking=True)
+        x0 = w.sets[0]["x"]
+        cms = time_calls([plain_copy], steps, warmup)
+        row["copy_us"] = round(cms * 1e3, 2)
+        row["copy_GBps"] = round(2 * x0.numel() * x0.element_size() / cms / 1e6, 1)
+        row["pct_of_copy_speed"] = round(row[last + "_GBps"] / row["copy_GBps"] * 100, 1)
         if w.bwd is not None:
             row["pct_of_hbm_peak"] = round(row[last + "_GBps"] / HBM_PEAK_GBS * 100, 1)
             row["pct_of_hbm_peak_warm"] = round(
