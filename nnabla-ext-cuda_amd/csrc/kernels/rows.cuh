@@ -328,7 +328,7 @@ row_bwd_kernel(const RowArgs a) {
   __shared__ uint4 park[PARK ? NL * TPR : 1];
   __shared__ float lds[2 * 16];
   __shared__ float part[GN ? 2 * NW * NL : 1];
-  __shared__ float xfold[(MODE == kRowLN && RPB > 1) ? (RPB / 2) * TPR * VEC : 1];
+  __shared__ float xfold[(MODE == kRowLN && RPB > 1) ? 2 * NL * (RPB / 2) * TPR * VEC : 1];
   const int t = threadIdx.x % TPR;
   const int sub = threadIdx.x / TPR;
   const T *__restrict__ x = static_cast<const T *>(a.x);
@@ -657,32 +657,47 @@ row_bwd_kernel(const RowArgs a) {
 
   if constexpr (MODE == kRowLN) {
     // Fold the RPB row groups of a block into group 0 (a halving tree, fixed
-    // order), then write the block's partial [2][R].
+    // order; every accumulator of a thread goes through a level together: two
+    // barriers per level, not two per level and accumulator), then write the
+    // block's partial [2][R].
     float *wsb = a.ws + static_cast<size_t>(blockIdx.x) * 2 * a.R;
+    if constexpr (RPB > 1) {
+      constexpr int kSlab = (RPB / 2) * TPR * VEC; // one accumulator of every thread of the upper half
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
+      for (int half = RPB / 2; half >= 1; half /= 2) {
+        lds_barrier(); // the previous level has been read
+        if (sub >= half && sub < 2 * half) {
 #pragma unroll
-      for (int k = 0; k < NL; ++k) {
-        float(&acc)[VEC] = (q == 0) ? acc_g[k] : acc_b[k];
-        if constexpr (RPB > 1) {
+          for (int k = 0; k < NL; ++k) {
 #pragma unroll
-          for (int half = RPB / 2; half >= 1; half /= 2) {
-            lds_barrier(); // the previous level has been read
-            if (sub >= half && sub < 2 * half) {
-#pragma unroll
-              for (int j = 0; j < VEC; ++j) xfold[((sub - half) * TPR + t) * VEC + j] = acc[j];
-            }
-            lds_barrier();
-            if (sub < half) {
-#pragma unroll
-              for (int j = 0; j < VEC; ++j) acc[j] += xfold[(sub * TPR + t) * VEC + j];
+            for (int j = 0; j < VEC; ++j) {
+              xfold[(2 * k) * kSlab + ((sub - half) * TPR + t) * VEC + j] = acc_g[k][j];
+              xfold[(2 * k + 1) * kSlab + ((sub - half) * TPR + t) * VEC + j] = acc_b[k][j];
             }
           }
         }
-        const int col = (k * TPR + t) * VEC;
-        if (sub == 0 && col < a.R) {
+        lds_barrier();
+        if (sub < half) {
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) wsb[static_cast<size_t>(q) * a.R + col + j] = acc[j];
+          for (int k = 0; k < NL; ++k) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) {
+              acc_g[k][j] += xfold[(2 * k) * kSlab + (sub * TPR + t) * VEC + j];
+              acc_b[k][j] += xfold[(2 * k + 1) * kSlab + (sub * TPR + t) * VEC + j];
+            }
+          }
+        }
+      }
+    }
+    if (sub == 0) {
+#pragma unroll
+      for (int k = 0; k < NL; ++k) {
+        const int col = (k * TPR + t) * VEC;
+        if (col < a.R) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) wsb[col + j] = acc_g[k][j];
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) wsb[static_cast<size_t>(a.R) + col + j] = acc_b[k][j];
         }
       }
     }
