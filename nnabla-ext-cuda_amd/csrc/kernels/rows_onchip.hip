@@ -14,12 +14,9 @@
 
 namespace nblahip {
 
-// OVER: the row is longer than the NR + NS slots.  The mean of the held part
-// serves as the shift K of the whole row: the held part's second pass and ONE
-// read of the rest accumulate sum (x - K) and sum (x - K)^2, from which
-// mean = K + s1/R and var = q/R - (s1/R)^2 (K is the mean of 10^5 elements of
-// the same row: the subtracted square is tiny against the variance).  The rest
-// is read a second time for y: 2 S + (1 - 25600 / nv) S.
+// OVER: the row is longer than the NR + NS slots.  The rest is read once for
+// the statistics (into the same per-thread sums as the held part) and a second
+// time for y: 2 S + (1 - 25600 / nv) S.
 template <typename T, int VEC, int NR, int NS, bool OVER = false>
 __global__ void __launch_bounds__(kOnchipBlock)
 row_onchip_fwd_kernel(const RowArgs a) {
@@ -47,49 +44,52 @@ row_onchip_fwd_kernel(const RowArgs a) {
     const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t;
     raw[k] = load_raw<T, VEC>(x + min(v, nv - 1u) * VEC);
   }
+  // Statistics from sums every wave takes over its OWN registers as its loads
+  // arrive (the memory system serves a CU's waves one after the other: what a
+  // wave does before the block's first barrier hides behind the other waves'
+  // loads, a second pass about the row's mean would keep memory idle).  Per
+  // thread: s = sum x, then about the thread's own mean K = s / n:
+  // s1 = sum (x - K) (rounding residue), s2 = sum (x - K)^2; mean = sum_t s / R
+  // and, about it, var = sum_t (s2 + 2 e s1 + n e^2) / R with e = K - mean: two
+  // block sums of a few operations per thread.  sum_t n e^2 is the variance
+  // between the threads' means, never more than the total: nothing cancels.
+  // (OVER: the vectors beyond the held ones are read here once, shifted by the
+  // K of the thread's held elements, and once more for y.)
+  auto held = [&](int k) { return static_cast<int>(t) < static_cast<int>(nv) - k * kOnchipBlock; };
   float s = 0.f;
 #pragma unroll
   for (int k = 0; k < NS; ++k) {
     const float part = raw_sum<T, VEC>(parked[k], 0.f);
-    s += (static_cast<uint32_t>(NR + k) * kOnchipBlock + t < nv) ? part : 0.f;
+    s += held(NR + k) ? part : 0.f;
     spill[k * kOnchipBlock + t] = __builtin_bit_cast(uint4, parked[k]);
   }
 #pragma unroll
   for (int k = 0; k < NR; ++k) {
     const float part = raw_sum<T, VEC>(raw[k], 0.f);
-    s += (static_cast<uint32_t>(k) * kOnchipBlock + t < nv) ? part : 0.f;
+    s += held(k) ? part : 0.f;
   }
-  // (OVER: the shift K, over the held elements only)
   constexpr uint32_t kHeld = static_cast<uint32_t>(NR + NS) * kOnchipBlock;
-  float mean = onchip_block_sum(s, red) * (OVER ? 1.0f / (static_cast<float>(kHeld) * VEC) : a.inv_R);
+  const uint32_t nvh = OVER ? min(nv, kHeld) : nv; // held vectors of the row
+  const float nh = t < nvh ? static_cast<float>(((nvh - 1u - t) / kOnchipBlock + 1u) * VEC) : 0.f;
+  const float kk = s * (1.0f / fmaxf(nh, 1.f));
+  float s1 = 0.f, s2 = 0.f;
+  auto take = [&](const RawVec<T, VEC> &r) {
 #pragma unroll
-  for (int k = 0; k < NR; ++k) keep_packed<T, VEC>(raw[k]);
-
-  float q = 0.f;
-  float s1 = 0.f; // OVER: sum (x - K), the held part's rounding residue included
-#pragma unroll
-  for (int k = 0; k < NR; ++k) {
-    if (static_cast<uint32_t>(k) * kOnchipBlock + t < nv) {
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const float d = elem_fma<T, VEC>(raw[k], j, a.one, -mean);
-        q = fmaf(d, d, q);
-        if constexpr (OVER) s1 += d;
-      }
+    for (int j = 0; j < VEC; ++j) {
+      const float d = elem_fma<T, VEC>(r, j, a.one, -kk);
+      s1 += d;
+      s2 = fmaf(d, d, s2);
     }
-  }
+  };
 #pragma unroll
   for (int k = 0; k < NS; ++k) {
-    if (static_cast<uint32_t>(NR + k) * kOnchipBlock + t < nv) {
-      const RawVec<T, VEC> r = __builtin_bit_cast(RawVec<T, VEC>, spill[k * kOnchipBlock + t]);
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) {
-        const float d = elem_fma<T, VEC>(r, j, a.one, -mean);
-        q = fmaf(d, d, q);
-        if constexpr (OVER) s1 += d;
-      }
-    }
+    if (held(NR + k)) take(parked[k]);
   }
+#pragma unroll
+  for (int k = 0; k < NR; ++k) {
+    if (held(k)) take(raw[k]);
+  }
+  float nt = nh; // elements of the thread, held and streamed
   constexpr int BO = 4; // vectors per thread and step of the streamed rest
   if constexpr (OVER) {
 #pragma unroll 1
@@ -100,25 +100,15 @@ row_onchip_fwd_kernel(const RowArgs a) {
         xo[b] = load_raw<T, VEC>(x + min(v0 + b * kOnchipBlock + t, nv - 1u) * VEC);
 #pragma unroll
       for (int b = 0; b < BO; ++b) {
-        float ps = 0.f, pq = 0.f;
-#pragma unroll
-        for (int j = 0; j < VEC; ++j) {
-          const float d = elem_fma<T, VEC>(xo[b], j, a.one, -mean);
-          ps += d;
-          pq = fmaf(d, d, pq);
-        }
-        const bool ok = v0 + b * kOnchipBlock + t < nv;
-        s1 += ok ? ps : 0.f;
-        q += ok ? pq : 0.f;
+        if (v0 + b * kOnchipBlock + t < nv) take(xo[b]);
       }
     }
-    s1 = onchip_block_sum(s1, red) * a.inv_R; // mean - K
+    nt = t < nv ? static_cast<float>(((nv - 1u - t) / kOnchipBlock + 1u) * VEC) : 0.f;
   }
-  float var = onchip_block_sum(q, red) * a.inv_R;
-  if constexpr (OVER) {
-    var = fmaxf(var - s1 * s1, 0.f);
-    mean += s1;
-  }
+  // (n K + s1 = the thread's sum of x, held and streamed)
+  const float mean = onchip_block_sum(fmaf(nt, kk, s1), red) * a.inv_R;
+  const float e = kk - mean;
+  const float var = onchip_block_sum(fmaf(e, fmaf(nt, e, 2.f * s1), s2), red) * a.inv_R;
   const float istd = inv_std(var, a.eps);
   if (t == 0) {
     a.mean[row] = mean;
