@@ -439,6 +439,7 @@ int bn_fwd_train_impl(const BnProblem &p, bool stats_only, hipStream_t st) {
 
 int launch_bn_fwd_train(const BnProblem &p, hipStream_t st) {
   int status = 0;
+  if (bn_pack_fwd_train(p, st, &status)) return status;
   if (bn_rows_fwd_train(p, st, &status)) return status;
   if (bn_onchip_fwd_train(p, st, &status)) return status;
   if (bn_cl_cached_fwd_train(p, st, &status)) return status;
@@ -464,6 +465,7 @@ int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
   if (!p.out && !p.dgamma && !p.dbeta && !p.dz && !p.sums_out) return 0;
   {
     int status = 0;
+    if (bn_pack_bwd(p, st, &status)) return status;
     if (bn_rows_bwd(p, st, &status)) return status;
     if (bn_onchip_bwd(p, st, &status)) return status;
     if (bn_cl_cached_bwd(p, st, &status)) return status;

@@ -144,6 +144,11 @@ bool bn_cl_cached_fwd_train(const BnProblem &p, hipStream_t st, int *status);
 bool bn_cl_grid_fwd_train(const BnProblem &p, hipStream_t st, int *status);
 bool bn_cl_grid_bwd(const BnProblem &p, hipStream_t st, int *status);
 bool bn_cl_cached_bwd(const BnProblem &p, hipStream_t st, int *status);
+// Training forward / backward for planes that are not a whole number of
+// 16-byte vectors (7x7, half 14x14): a pack of 2, 4 or 8 neighbouring channels,
+// whose planes together are, held on one CU (bn_pack.hip).
+bool bn_pack_fwd_train(const BnProblem &p, hipStream_t st, int *status);
+bool bn_pack_bwd(const BnProblem &p, hipStream_t st, int *status);
 int launch_bn_infer(const BnProblem &p, hipStream_t st);
 int launch_bn_fwd_train(const BnProblem &p, hipStream_t st);
 int launch_bn_bwd(const BnProblem &p, hipStream_t st);

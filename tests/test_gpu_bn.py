@@ -34,6 +34,13 @@ SMALL = [
     # scalar loads, channel-last with a handful of channels as strided rows
     ((32, 64, 13, 13), 1), ((40, 5, 13, 15), 1), ((8, 14, 14, 3), 3), ((1, 64, 64, 3), 3),
     ((64, 13, 13, 3), 3), ((90, 7), 1), ((1000, 1), 1), ((2, 31, 33, 8), 3),
+    # planes that are no whole number of 16-byte vectors, a pack of 2 / 4 / 8 neighbouring
+    # channels per block: every slot count, samples that do not fill the last sweep, fewer
+    # samples than a sweep, more samples than the backward holds, 121-vector segments,
+    # pairs of half 14x14 planes (backward only)
+    ((64, 1024, 7, 7), 1), ((256, 256, 7, 7), 1), ((200, 64, 14, 14), 1), ((20, 1024, 3, 3), 1),
+    ((300, 256, 5, 5), 1), ((100, 264, 7, 7), 1), ((440, 256, 7, 7), 1), ((190, 512, 7, 7), 1),
+    ((40, 256, 11, 11), 1),
 ]
 DTYPES = [torch.float32, torch.float16]
 
@@ -90,6 +97,8 @@ def test_bn_training_forward_backward(shape, axis, dtype):
 @pytest.mark.parametrize("shape,axis", [((4, 8, 6, 6), 1), ((37, 24), 1), ((6, 5, 4, 8), 3),
                                         # a channel per block, cached in registers
                                         ((8, 64, 12, 12), 1), ((4, 48, 7, 9), 1), ((3, 300, 2, 2), 1),
+                                        # a pack of channels per block (planes of 49 elements)
+                                        ((90, 256, 7, 7), 1),
                                         # channel-last, a channel vector's column per block
                                         ((8, 7, 7, 256), 3), ((300, 512), 1)])
 def test_bn_flags(shape, axis):

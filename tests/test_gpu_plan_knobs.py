@@ -164,6 +164,10 @@ SWITCHES = [
     ("bn_rows_off", run_bn, ((32, 64, 14, 14), 1, F16), {"BN_ROWS": 0},
      ["bn_stats_planes_kernel", "bn_finalize_fwd_kernel", "bn_apply_planes_kernel",
       "bn_finalize_bwd_kernel"], ["row_fwd_kernel_bn", "row_bwd_kernel_bn"]),
+    ("bn_pack_off", run_bn, ((96, 256, 7, 7), 1, F16), {"BN_PACK": 0},
+     ["bn_stats_planes_kernel", "bn_bwd_reduce_planes_kernel"], ["bn_pack_fwd_kernel", "bn_pack_bwd_kernel"]),
+    ("bn_pack_min_pct_up", run_bn, ((96, 256, 7, 7), 1, F16), {"BN_PACK_MIN_PCT": 50},
+     ["bn_stats_planes_kernel"], ["bn_pack_fwd_kernel", "bn_pack_bwd_kernel"]),
     ("bn_cl_grid_off", run_bn, ((100352, 64), 1, F16), {"BN_CL_GRID": 0},
      ["bn_stats_cl_kernel", "bn_finalize_fwd_kernel", "bn_apply_cl_kernel"], ["bn_cl_grid_fwd_kernel"],
      {"BN_CL_GRID_MIN_SLOTS": 1}),
@@ -268,6 +272,10 @@ GRIDS = [
      ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
     ("bn_onchip_streamed_few_channels", run_bn, ((64, 8, 56, 56), 1, F32),
      [{"BN_ONCHIP_STREAMED_MIN_PCT": 1}], ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
+    ("bn_pack_few_channels", run_bn, ((48, 16, 7, 7), 1, F16), [{"BN_PACK_SHORT_MIN_PCT": 0}],
+     ["bn_pack_fwd_kernel", "bn_pack_bwd_kernel"], []),
+    ("bn_pack_plain_block_order", run_bn, ((96, 256, 7, 7), 1, F16), [{"BN_PACK_XCD_MAP": 0}],
+     ["bn_pack_fwd_kernel", "bn_pack_bwd_kernel"], []),
     ("ln_bwd_blocks_per_cu", run_ln, (4096, 1024, F16), [{"LN_BWD_BLOCKS_PER_CU": v} for v in (1, 2, 4)],
      ["row_bwd_kernel_ln", "ln_param_reduce_kernel"], []),
     ("ln_wave_per_short_row", run_ln, (1000, 32, F32), [{"ROW_SUBWAVE": 0}],
