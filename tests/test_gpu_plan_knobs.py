@@ -274,7 +274,8 @@ GRIDS = [
      [{"BN_ONCHIP_STREAMED_MIN_PCT": 1}], ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
     ("bn_pack_few_channels", run_bn, ((48, 16, 7, 7), 1, F16), [{"BN_PACK_SHORT_MIN_PCT": 0}],
      ["bn_pack_fwd_kernel", "bn_pack_bwd_kernel"], []),
-    ("bn_pack_plain_block_order", run_bn, ((96, 256, 7, 7), 1, F16), [{"BN_PACK_XCD_MAP": 0}],
+    ("bn_pack_plain_block_order", run_bn, ((96, 256, 7, 7), 1, F16),
+     [{"BN_PACK_XCD_MAP": 0}, {"BN_PACK_EDGE_STORES": 0}],
      ["bn_pack_fwd_kernel", "bn_pack_bwd_kernel"], []),
     ("ln_bwd_blocks_per_cu", run_ln, (4096, 1024, F16), [{"LN_BWD_BLOCKS_PER_CU": v} for v in (1, 2, 4)],
      ["row_bwd_kernel_ln", "ln_param_reduce_kernel"], []),
