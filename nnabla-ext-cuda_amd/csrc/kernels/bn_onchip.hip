@@ -60,7 +60,39 @@ struct BnOnchipArgs {
   uint32_t gmod;
   float *pairs; // may be null
   int accum_dx, accum_g, accum_b;
+  // Planes that are no whole number of 128-byte lines share their first and
+  // last line with the neighbouring channels' planes: plane_bytes != 0 then,
+  // and neighbouring channels run on the same XCD (per_xcd channels each).
+  uint32_t plane_bytes;
+  uint32_t per_xcd;
 };
+
+// Channel of block b.  Workgroups go to the 8 XCDs round-robin by index; with
+// planes that share lines, neighbouring channels take the same XCD, whose L2
+// then fetches a shared line once and merges the partial writes to it.
+__device__ __forceinline__ uint32_t onchip_channel(const BnOnchipArgs &a, uint32_t b) {
+  return a.per_xcd ? (b % 8u) * a.per_xcd + b / 8u : b;
+}
+
+// Writes vector v of the channel (at dst).  A vector in a line that the plane
+// shares with a neighbour is written with an ordinary store, which L2 merges
+// with the neighbour's part of the line; non-temporal stores of line pieces
+// go to memory piece by piece.
+template <typename T, int VEC>
+__device__ __forceinline__ void onchip_store(const BnOnchipArgs &a, T *dst, uint32_t v,
+                                             const float (&o)[VEC]) {
+  if (a.plane_bytes) {
+    const uint32_t w = v - a.vpp.div(v) * a.vpp.d;
+    const uintptr_t addr = reinterpret_cast<uintptr_t>(dst);
+    const uintptr_t first = addr - static_cast<uintptr_t>(w) * sizeof(RawVec<T, VEC>);
+    const uintptr_t line = addr >> 7;
+    if (line < ((first + 127u) >> 7) || line >= ((first + a.plane_bytes) >> 7)) {
+      store_vec<T, VEC, false>(dst, o);
+      return;
+    }
+  }
+  store_vec<T, VEC>(dst, o);
+}
 
 // Element offset of vector v of channel c (planes are contiguous, a channel's
 // planes lie C*size2 apart).
@@ -83,7 +115,7 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
   static_assert(sizeof(RawVec<T, VEC>) == sizeof(Slot<T, VEC>), "8- or 16-byte vectors");
   __shared__ float red[kOnchipBlock / kWave];
   __shared__ Slot<T, VEC> spill[NS > 0 ? NS * kOnchipBlock : 1];
-  const uint32_t c = blockIdx.x;
+  const uint32_t c = onchip_channel(a, blockIdx.x);
   const uint32_t t = threadIdx.x;
   const T *__restrict__ x = static_cast<const T *>(a.x);
   T *__restrict__ y = static_cast<T *>(a.y);
@@ -208,7 +240,7 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
 #pragma unroll
       for (int j = 0; j < VEC; ++j) o[j] = fmaxf(0.f, o[j]);
     }
-    store_vec<T, VEC>(y + off, o);
+    onchip_store<T, VEC>(a, y + off, v, o);
   };
   const uint32_t t2 = fresh(t);
 #pragma unroll
@@ -259,7 +291,7 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
   constexpr int NL = NR + NS;
   __shared__ float red[TB / kWave];
   __shared__ Slot<T, VEC> spill[NS > 0 ? NS * TB : 1];
-  const uint32_t c = blockIdx.x;
+  const uint32_t c = onchip_channel(a, blockIdx.x);
   const uint32_t t = threadIdx.x;
   const T *__restrict__ x = static_cast<const T *>(a.x);
   const T *__restrict__ dy = static_cast<const T *>(a.dy);
@@ -416,7 +448,7 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
 #pragma unroll
           for (int j = 0; j < VEC; ++j) o[j] += old[j];
         }
-        store_vec<T, VEC>(dst, o);
+        onchip_store<T, VEC>(a, dst, v, o);
         last = o[0];
       }
     }
@@ -450,7 +482,7 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
 #pragma unroll
             for (int j = 0; j < VEC; ++j) o[j] += old[j];
           }
-          store_vec<T, VEC>(dst, o);
+          onchip_store<T, VEC>(a, dst, v0 + b * TB + t, o);
         }
       }
     }
@@ -504,6 +536,21 @@ int run_onchip_bwd(int64_t nv, const BnOnchipArgs &a, hipStream_t st) {
   return last_launch_status();
 }
 
+// Planes that share lines with their neighbours: edge stores and the XCD map.
+void onchip_edge_plan(BnOnchipArgs &a, int64_t plane_bytes) {
+  a.plane_bytes = 0;
+  a.per_xcd = 0;
+  // Short planes only, where two of a handful of lines are shared: 784-byte
+  // planes ([256,1024,14,14] float) forward 106.3 -> 94.9 us, [256,256,14,14]
+  // 25.4 / 34.4 -> 20.3 / 31.1 us, 392-byte planes ([256,1024,14,14] half)
+  // forward 54.9 -> 43.3 us; with 1568-byte planes ([256,512,28,28] half) the
+  // forward gains 2 % and the backward, which reads dy twice through the same
+  // L2, loses 4 %.
+  if (plane_bytes % 128 == 0 || plane_bytes > tune_int("BN_ONCHIP_EDGE_STORES_MAX_BYTES", 1024)) return;
+  a.plane_bytes = static_cast<uint32_t>(plane_bytes);
+  if (a.C % 8 == 0) a.per_xcd = a.C / 8;
+}
+
 // Shape test shared by both directions; fills the common arguments.
 bool onchip_args(const BnProblem &p, bool backward, BnOnchipArgs &a, int &nl, int max_nl = 25) {
   if (!tune_int("BN_ONCHIP", 1)) return false;
@@ -551,6 +598,7 @@ bool onchip_args(const BnProblem &p, bool backward, BnOnchipArgs &a, int &nl, in
   a.eps = p.eps;
   a.one = 1.0f;
   a.gmod = a.C;
+  onchip_edge_plan(a, p.size2 * (p.dtype == NBLAHIP_F16 ? 2 : 4));
   return true;
 }
 
@@ -621,6 +669,7 @@ bool in_onchip_bwd(const RowProblem &p, hipStream_t st, int *status) {
   a.inv_N = static_cast<float>(1.0 / static_cast<double>(p.R));
   a.eps = p.eps;
   a.one = 1.0f;
+  onchip_edge_plan(a, p.R * (p.dtype == NBLAHIP_F16 ? 2 : 4));
   *status = p.dtype != NBLAHIP_F16 ? run_onchip_bwd<float, 4>(nv, a, st)
                                    : run_onchip_bwd<__half, 8>(nv, a, st);
   return true;

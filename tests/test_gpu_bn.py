@@ -41,6 +41,8 @@ SMALL = [
     ((64, 1024, 7, 7), 1), ((256, 256, 7, 7), 1), ((200, 64, 14, 14), 1), ((20, 1024, 3, 3), 1),
     ((300, 256, 5, 5), 1), ((100, 264, 7, 7), 1), ((440, 256, 7, 7), 1), ((190, 512, 7, 7), 1),
     ((40, 256, 11, 11), 1),
+    # a channel per CU whose planes share cache lines with the neighbouring channels'
+    ((256, 64, 14, 14), 1), ((250, 40, 10, 10), 1),
 ]
 DTYPES = [torch.float32, torch.float16]
 
