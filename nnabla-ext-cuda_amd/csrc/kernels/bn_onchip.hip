@@ -546,7 +546,7 @@ void onchip_edge_plan(BnOnchipArgs &a, int64_t plane_bytes) {
   // forward 54.9 -> 43.3 us; with 1568-byte planes ([256,512,28,28] half) the
   // forward gains 2 % and the backward, which reads dy twice through the same
   // L2, loses 4 %.
-  if (plane_bytes % 128 == 0 || plane_bytes > tune_int("BN_ONCHIP_EDGE_STORES_MAX_BYTES", 1024)) return;
+  if (plane_bytes % 128 == 0 || plane_bytes > tune_int("BN_EDGE_STORES_MAX_BYTES", 1024)) return;
   a.plane_bytes = static_cast<uint32_t>(plane_bytes);
   if (a.C % 8 == 0) a.per_xcd = a.C / 8;
 }

@@ -66,6 +66,12 @@ struct RowArgs {
   // elements between the end of one and the start of the next.
   FastDiv plane;
   uint32_t plane_jump;
+  // ... planes that are no whole number of 128-byte lines share their first and
+  // last line with the neighbouring channels' planes: edge_bytes = the plane's
+  // size then (else 0), and neighbouring blocks run on the same XCD (per_xcd
+  // blocks each; 0: plain order).
+  uint32_t edge_bytes;
+  uint32_t per_xcd;
   float *rmean; // running statistics, may be null
   float *rvar;
   float decay, unbias;
@@ -81,6 +87,37 @@ __device__ __forceinline__ uint32_t row_elem_offset(const RowArgs &a, int col) {
   } else {
     return static_cast<uint32_t>(col);
   }
+}
+
+// BatchNormalization rows: block index with neighbouring channels on the same
+// XCD (workgroups go to the 8 XCDs round-robin), whose L2 then fetches a line
+// two planes share once and merges the partial writes to it.
+template <bool STRIDED> __device__ __forceinline__ uint32_t row_block_index(const RowArgs &a) {
+  if constexpr (STRIDED) {
+    if (a.per_xcd) return (blockIdx.x % 8u) * a.per_xcd + blockIdx.x / 8u;
+  }
+  return blockIdx.x;
+}
+
+// Store of the vector at column col of a row.  BatchNormalization rows whose
+// planes share lines with their neighbours write the vectors inside such a
+// line with an ordinary store (L2 merges the line's parts; non-temporal
+// stores of line pieces go to memory piece by piece).
+template <typename T, int VEC, bool STRIDED>
+__device__ __forceinline__ void row_store(const RowArgs &a, T *dst, int col, const float (&o)[VEC]) {
+  if constexpr (STRIDED) {
+    if (a.edge_bytes) {
+      const uint32_t w = static_cast<uint32_t>(col) - a.plane.div(static_cast<uint32_t>(col)) * a.plane.d;
+      const uintptr_t addr = reinterpret_cast<uintptr_t>(dst);
+      const uintptr_t first = addr - static_cast<uintptr_t>(w) * sizeof(T);
+      const uintptr_t line = addr >> 7;
+      if (line < ((first + 127u) >> 7) || line >= ((first + a.edge_bytes) >> 7)) {
+        store_vec<T, VEC, false>(dst, o);
+        return;
+      }
+    }
+  }
+  store_vec<T, VEC>(dst, o);
 }
 
 // GroupNormalization backward thread map.  A wave-wide load never crosses a
@@ -189,7 +226,7 @@ row_fwd_kernel(const RowArgs a) {
     }
   }
 
-  for (int row = blockIdx.x * RPB + sub; row < a.rows; row += gridDim.x * RPB) {
+  for (int row = row_block_index<STRIDED>(a) * RPB + sub; row < a.rows; row += gridDim.x * RPB) {
     const size_t base = static_cast<size_t>(row) * (STRIDED ? a.plane.d : a.R);
     RawVec<T, VEC> raw[NL];
 #pragma unroll
@@ -284,7 +321,7 @@ row_fwd_kernel(const RowArgs a) {
           for (int j = 0; j < VEC; ++j)
             o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mean), g, bk[k]);
         }
-        store_vec<T, VEC>(y + base + row_elem_offset<STRIDED>(a, col), o);
+        row_store<T, VEC, (STRIDED && TPR * NL < 8192)>(a, y + base + row_elem_offset<STRIDED>(a, col), col, o);
       }
     }
   }
@@ -369,7 +406,7 @@ row_bwd_kernel(const RowArgs a) {
   constexpr bool CH = (MODE == kRowINc);
   const int channels = static_cast<int>(a.pmod);
   const int nunits = CH ? channels : a.rows;
-  const int u0 = CH ? static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x) * RPB + sub;
+  const int u0 = CH ? static_cast<int>(blockIdx.x) : static_cast<int>(row_block_index<BN>(a)) * RPB + sub;
   const int ustride = CH ? static_cast<int>(gridDim.x) : static_cast<int>(gridDim.x) * RPB;
   const int inner_n = CH ? a.rows / channels : 1;
   for (int unit = u0; unit < nunits; unit += ustride) {
@@ -625,7 +662,7 @@ row_bwd_kernel(const RowArgs a) {
 #pragma unroll
             for (int j = 0; j < VEC; ++j) o[j] += old[j];
           }
-          store_vec<T, VEC>(dst, o);
+          row_store<T, VEC, (BN && TPR * NL < 8192)>(a, dst, col, o);
         }
       }
     }

@@ -585,6 +585,14 @@ static bool bn_rows_cfg(const BnProblem &p, bool backward, RowCfg &cfg, RowArgs 
   a.cpg = 1;
   a.plane = FastDiv(static_cast<uint32_t>(p.size2));
   a.plane_jump = static_cast<uint32_t>((p.C - 1) * p.size2);
+  // short planes that share cache lines with their neighbours (bn_onchip.hip
+  // has the measurements behind the limit)
+  const int64_t plane_bytes = p.size2 * (p.dtype == NBLAHIP_F16 ? 2 : 4);
+  if (plane_bytes % 128 != 0 && plane_bytes <= tune_int("BN_EDGE_STORES_MAX_BYTES", 1024)) {
+    a.edge_bytes = static_cast<uint32_t>(plane_bytes);
+    const int64_t blocks = cached_grid(p.C, cfg.tpr);
+    if (blocks % 8 == 0) a.per_xcd = static_cast<uint32_t>(blocks / 8);
+  }
   return true;
 }
 

@@ -272,9 +272,11 @@ GRIDS = [
      ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
     # planes that share cache lines with their neighbours: ordinary stores there, or not
     ("bn_onchip_edge_stores_off", run_bn, ((256, 64, 14, 14), 1, F32),
-     [{"BN_ONCHIP_EDGE_STORES_MAX_BYTES": 0}], ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
+     [{"BN_EDGE_STORES_MAX_BYTES": 0}], ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
+    ("bn_rows_edge_stores_off", run_bn, ((32, 64, 14, 14), 1, F16), [{"BN_EDGE_STORES_MAX_BYTES": 0}],
+     ["row_fwd_kernel_bn", "row_bwd_kernel_bn"], []),
     ("bn_onchip_edge_stores_longer_planes", run_bn, ((128, 64, 28, 28), 1, F16),
-     [{"BN_ONCHIP_EDGE_STORES_MAX_BYTES": 4096}], ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
+     [{"BN_EDGE_STORES_MAX_BYTES": 4096}], ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
     ("bn_onchip_streamed_few_channels", run_bn, ((64, 8, 56, 56), 1, F32),
      [{"BN_ONCHIP_STREAMED_MIN_PCT": 1}], ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
     ("bn_pack_few_channels", run_bn, ((48, 16, 7, 7), 1, F16), [{"BN_PACK_SHORT_MIN_PCT": 0}],
