@@ -389,8 +389,12 @@ size_t bn_workspace_bytes(int64_t size0, int64_t C, int64_t size2, int dtype) {
   const BnPlan a = make_plan(size0, C, size2, dtype, true);
   const BnPlan b = make_plan(size0, C, size2, dtype, false);
   const uint32_t S = std::max(a.S, b.S);
-  return part_bytes(static_cast<uint32_t>(C), S) +
-         align_up(static_cast<size_t>(C) * sizeof(BnParam), 256);
+  const size_t split_reduction = part_bytes(static_cast<uint32_t>(C), S) +
+                                 align_up(static_cast<size_t>(C) * sizeof(BnParam), 256);
+  // channel-last tensors through the split kernels: a (sum dy*xh, sum dy) pair
+  // per channel and block of the rows
+  const size_t split_pairs = size2 == 1 ? static_cast<size_t>(kClSplitMaxBlocks) * C * 2 * sizeof(float) : 0;
+  return std::max(split_reduction, split_pairs);
 }
 
 int launch_bn_infer(const BnProblem &p, hipStream_t st) {
@@ -437,6 +441,66 @@ int bn_fwd_train_impl(const BnProblem &p, bool stats_only, hipStream_t st) {
 }
 } // namespace
 
+// Channel-last BatchNormalization as the InstanceNormalization of ONE sample
+// whose plane is all the rows: the split kernels (gn_cl_split.hip) take planes
+// of up to 65536 positions (64 blocks of 1024), a unit per channel, one pass
+// over x per direction.
+static bool bn_as_cl_problem(const BnProblem &p, ClProblem &q) {
+  if (!tune_int("BN_CL_SPLIT", 1)) return false;
+  if (p.size2 != 1 || p.relu || p.z || p.y || p.dz || p.sums_out || p.sums_in) return false;
+  if (p.size0 < 2) return false;
+  q = ClProblem{};
+  q.dtype = p.dtype;
+  q.x = p.x;
+  q.gamma = p.gamma;
+  q.batch = 1;
+  q.spatial = p.size0;
+  q.channels = p.C;
+  q.groups = static_cast<int>(p.C);
+  q.eps = p.eps;
+  q.ws = p.ws;
+  q.ws_bytes = p.ws_bytes;
+  q.as_batch_norm = 1;
+  return true;
+}
+
+bool bn_cl_split_fwd_train(const BnProblem &p, hipStream_t st, int *status) {
+  ClProblem q;
+  if (!p.out || !bn_as_cl_problem(p, q)) return false;
+  q.out = p.out;
+  q.beta = p.beta;
+  q.mean = p.batch_mean;
+  q.var = p.batch_var;
+  q.rmean = p.rmean;
+  q.rvar = p.rvar;
+  q.decay = p.decay;
+  const double N = static_cast<double>(p.size0);
+  q.unbias = static_cast<float>(N / (N - 1.0));
+  return cl_split_fwd(q, aligned16(p.x) && aligned16(p.out), st, status);
+}
+
+bool bn_cl_split_bwd(const BnProblem &p, hipStream_t st, int *status) {
+  ClProblem q;
+  if (!p.batch_stat || !bn_as_cl_problem(p, q)) return false;
+  q.dy = p.dy;
+  q.out = p.out;
+  q.mean = const_cast<float *>(p.mean);
+  q.var = const_cast<float *>(p.var);
+  q.dmean = p.dmean;
+  q.dvar = p.dvar;
+  q.dgamma = p.dgamma;
+  q.dbeta = p.dbeta;
+  q.accum_dx = p.accum_dx;
+  float *pairs = nullptr;
+  int64_t pair_batches = 0;
+  const bool al = aligned16(p.x) && aligned16(p.dy) && (!p.out || aligned16(p.out));
+  if (!cl_split_bwd(q, al, &pairs, &pair_batches, st, status)) return false;
+  if (*status == 0 && (p.dgamma || p.dbeta))
+    *status = launch_pair_param_reduce("pair_param_reduce_cl_kernel", pairs, pair_batches, p.C, p.dgamma,
+                                       p.dbeta, 1, 1, p.accum_g, p.accum_b, st);
+  return true;
+}
+
 int launch_bn_fwd_train(const BnProblem &p, hipStream_t st) {
   int status = 0;
   if (bn_pack_fwd_train(p, st, &status)) return status;
@@ -444,6 +508,7 @@ int launch_bn_fwd_train(const BnProblem &p, hipStream_t st) {
   if (bn_onchip_fwd_train(p, st, &status)) return status;
   if (bn_cl_cached_fwd_train(p, st, &status)) return status;
   if (bn_cl_grid_fwd_train(p, st, &status)) return status;
+  if (bn_cl_split_fwd_train(p, st, &status)) return status;
   return bn_fwd_train_impl(p, false, st);
 }
 
@@ -470,6 +535,7 @@ int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
     if (bn_onchip_bwd(p, st, &status)) return status;
     if (bn_cl_cached_bwd(p, st, &status)) return status;
     if (bn_cl_grid_bwd(p, st, &status)) return status;
+    if (bn_cl_split_bwd(p, st, &status)) return status;
   }
   const bool al = aligned16(p.x) && aligned16(p.dy) && (!p.out || aligned16(p.out)) &&
                   (!p.y || aligned16(p.y)) && (!p.dz || aligned16(p.dz));
@@ -650,9 +716,12 @@ int cl_bwd_apply_t(const ClProblem &p, const BnPlan &pl, const BnParam *params, 
 size_t cl_workspace_bytes(int64_t batch, int64_t spatial, int64_t channels, int dtype) {
   const BnPlan a = make_cl_plan(batch, spatial, channels, dtype, true);
   const BnPlan b = make_cl_plan(batch, spatial, channels, dtype, false);
-  return cl_part_bytes(batch, channels, std::max(a.S, b.S)) +
-         align_up(static_cast<size_t>(batch) * channels * sizeof(BnParam), 256) +
-         align_up(static_cast<size_t>(batch) * channels * 2 * sizeof(float), 256);
+  const size_t split_reduction = cl_part_bytes(batch, channels, std::max(a.S, b.S)) +
+                                 align_up(static_cast<size_t>(batch) * channels * sizeof(BnParam), 256) +
+                                 align_up(static_cast<size_t>(batch) * channels * 2 * sizeof(float), 256);
+  // the split kernels (gn_cl_split.hip): a pair per channel and block of a plane
+  const size_t split_pairs = static_cast<size_t>(batch) * kClSplitMaxBlocks * channels * 2 * sizeof(float);
+  return std::max(split_reduction, split_pairs);
 }
 
 int launch_cl_fwd(const ClProblem &p, hipStream_t st) {

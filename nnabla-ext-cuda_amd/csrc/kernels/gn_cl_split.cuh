@@ -31,7 +31,7 @@
 namespace nblahip {
 
 constexpr int kSplitTV = 8;    // 16-byte vectors per column tile (one 128-byte line per position)
-constexpr int kSplitMax = 16;  // most blocks per (sample, column tile)
+constexpr int kSplitMax = kClSplitMaxBlocks; // most blocks per (sample, column tile)
 
 struct ClSplitArgs {
   const void *x;
@@ -55,7 +55,32 @@ struct ClSplitArgs {
   int cvg_shift; // log2 of the vectors per unit (groups only)
   float eps, inv_R, one;
   int accum_dx;
+  // Block order: 0: the column tile runs fastest (b = (n * split + s) * tiles +
+  // tile), 1: the blocks of a (sample, tile) are neighbours (b = (n * tiles +
+  // tile) * split + s) - for grids beyond what the chip holds at once, where a
+  // block's partners must not be a whole round of blocks away.
+  int partners_adjacent;
+  // BatchNormalization through these kernels (one sample, a unit per channel):
+  // running statistics to update, may be null.
+  float *rmean, *rvar;
+  float decay, unbias;
 };
+
+// (column tile, block of the plane, sample) of block b.
+__device__ __forceinline__ void split_block_coords(const ClSplitArgs &a, uint32_t b, uint32_t &tile,
+                                                   uint32_t &s, uint32_t &n) {
+  if (a.partners_adjacent) {
+    s = b % a.split;
+    const uint32_t nt = b / a.split;
+    tile = nt % a.tiles;
+    n = nt / a.tiles;
+  } else {
+    tile = b % a.tiles;
+    const uint32_t ns = b / a.tiles;
+    s = ns % a.split;
+    n = ns / a.split;
+  }
+}
 
 // Polls the partners' words into part[] (a thread takes the two words of a
 // unit at a time, the first reads of up to four units in flight together: a
@@ -311,7 +336,9 @@ __device__ __forceinline__ void split_block_part(const ClSplitArgs &a, int sp, u
 // Forward.  Block b = ((n * split + s) * tiles + tile); thread t owns vector
 // t % 8 of the tile at positions s * PB + t / 8 + k * (TPR / 8), k < NL.
 // ---------------------------------------------------------------------------
-template <typename T, int VEC, int NL, int TPR, bool INSTANCE>
+// MANY: more than 16 blocks per (sample, column tile); their partials lie in
+// LDS sized by the launch (BatchNormalization's single plane of all rows).
+template <typename T, int VEC, int NL, int TPR, bool INSTANCE, bool MANY = false>
 __global__ void __launch_bounds__(TPR)
 cl_split_fwd_kernel(const ClSplitArgs a) {
   constexpr int TV = kSplitTV;
@@ -320,11 +347,13 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
   constexpr int UMAX = INSTANCE ? TV * VEC : TV;
   __shared__ float fold[NW][UMAX];
   __shared__ float tot[UMAX];
-  __shared__ float part[kSplitMax * UMAX * 2];
+  __shared__ float part16[MANY ? 1 : 16 * UMAX * 2];
+  extern __shared__ float part_many[]; // [split][2 * units of the tile], sized by the launch
+  float *const part = MANY ? part_many : part16;
   __shared__ float merged[UMAX * 2]; // (mean, 1 / std) per unit
   __shared__ int missing[kSplitMax];
-  const uint32_t tile = blockIdx.x % a.tiles, ns = blockIdx.x / a.tiles;
-  const uint32_t s = ns % a.split, n = ns / a.split;
+  uint32_t tile, s, n;
+  split_block_coords(a, blockIdx.x, tile, s, n);
   const uint32_t cvx = threadIdx.x % TV, prow = threadIdx.x / TV;
   const uint32_t ch = (tile * TV + cvx) * VEC;
   const uint32_t gi = INSTANCE ? 0u : (cvx >> a.cvg_shift);
@@ -338,6 +367,11 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
   const bool writer = prow == 0 && (INSTANCE || (cvx & ((1u << a.cvg_shift) - 1)) == 0);
 
   if (threadIdx.x < kSplitMax) missing[threadIdx.x] = 0;
+  auto unit_index = [&]() -> size_t { // statistics index of unit threadIdx.x of the tile
+    return INSTANCE ? static_cast<size_t>(n) * a.C + tile * TV * VEC + threadIdx.x
+                    : static_cast<size_t>(n) * (a.C / a.cpg) + (tile * TV * VEC) / a.cpg + threadIdx.x;
+  };
+  float unit_mean = 0.f, unit_var = 0.f; // kept for the running statistics
   float gam[VEC], bet[VEC]; // ahead of the tensor's loads: they travel together
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
@@ -400,10 +434,11 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
     merged[2 * u] = m;
     merged[2 * u + 1] = inv_std(v, a.eps); // once per unit, not once per thread and channel
     if (s == 0) {
-      const size_t ug = INSTANCE ? static_cast<size_t>(n) * a.C + tile * TV * VEC + u
-                                 : static_cast<size_t>(n) * (a.C / a.cpg) + (tile * TV * VEC) / a.cpg + u;
+      const size_t ug = unit_index();
       a.mean[ug] = m;
       a.var[ug] = v;
+      unit_mean = m;
+      unit_var = v;
     }
   }
   lds_barrier();
@@ -438,6 +473,15 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
       }
       store_vec<T, VEC>(y + static_cast<size_t>(pos) * a.C, o);
     }
+  }
+  // BatchNormalization: the running statistics, by the unit threads of the
+  // plane's first block.  At the very end: their loads cost this wave a round
+  // trip that nothing else waits for (ahead of the tensor's loads the test for
+  // them cost every Group/InstanceNormalization forward 0.4 us).
+  if (a.rmean && s == 0 && static_cast<int>(threadIdx.x) < U) {
+    const size_t ug = unit_index();
+    a.rmean[ug] = a.decay * a.rmean[ug] + (1.f - a.decay) * unit_mean;
+    a.rvar[ug] = a.decay * a.rvar[ug] + (1.f - a.decay) * unit_var * a.unbias;
   }
 }
 
@@ -486,7 +530,7 @@ __device__ __forceinline__ void split_pairs_from_memory(
 // wrote): both in registers cost more than the 128 a thread may use with two
 // blocks of 512 on a CU.
 // ---------------------------------------------------------------------------
-template <typename T, int VEC, int NL, int TPR, bool INSTANCE>
+template <typename T, int VEC, int NL, int TPR, bool INSTANCE, bool MANY = false>
 __global__ void __launch_bounds__(TPR, 4)
 cl_split_bwd_kernel(const ClSplitArgs a) {
   constexpr int TV = kSplitTV;
@@ -498,12 +542,14 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
   __shared__ RawVec<T, VEC> park[NL * TPR];
   __shared__ float fold[NW][2 * CH];
   __shared__ float chs[2][CH]; // [0]: sum dy*xh, [1]: sum dy per channel of the tile
-  __shared__ float part[kSplitMax * UMAX * 2];
+  __shared__ float part16[MANY ? 1 : 16 * UMAX * 2];
+  extern __shared__ float part_many[]; // [split][2 * units of the tile], sized by the launch
+  float *const part = MANY ? part_many : part16;
   __shared__ float coef[UMAX * 2]; // (cA, cb) per unit
   __shared__ float gch[CH];        // gamma of the tile's channels
   __shared__ int missing[kSplitMax];
-  const uint32_t tile = blockIdx.x % a.tiles, ns = blockIdx.x / a.tiles;
-  const uint32_t s = ns % a.split, n = ns / a.split;
+  uint32_t tile, s, n;
+  split_block_coords(a, blockIdx.x, tile, s, n);
   const uint32_t cvx = threadIdx.x % TV, prow = threadIdx.x / TV;
   const uint32_t ch0 = tile * CH, ch = ch0 + cvx * VEC;
   const uint32_t gi = INSTANCE ? 0u : (cvx >> a.cvg_shift);

@@ -15,13 +15,18 @@ struct SplitPlan {
   int vec = 8, tpr = 512, nl = 8;
   int tiles = 0, split = 0, pb = 0, cpg = 1, cvg_shift = 0, units = 0; // units per tile
   size_t words = 0;
+  bool partners_adjacent = false;
+  int64_t lds_bytes = 0;
 };
 
 SplitPlan plan_split(const ClProblem &p, bool aligned, bool backward) {
   SplitPlan s;
-  if (!aligned || !tune_int("GN_CL_SPLIT", 1)) return s;
+  if (!aligned) return s;
+  if (!p.as_batch_norm) { // (BatchNormalization has its own switch)
+    if (!tune_int("GN_CL_SPLIT", 1)) return s;
+    if (p.groups == p.channels && !tune_int("GN_CL_SPLIT_INSTANCES", 1)) return s;
+  }
   if (!p.bc_gamma || !p.bc_beta) return s;
-  if (p.groups == p.channels && !tune_int("GN_CL_SPLIT_INSTANCES", 1)) return s;
   const int esz = p.dtype == NBLAHIP_F16 ? 2 : 4;
   s.vec = 16 / esz;
   const int64_t tile_ch = static_cast<int64_t>(kSplitTV) * s.vec; // channels of a 128-byte line
@@ -37,7 +42,8 @@ SplitPlan plan_split(const ClProblem &p, bool aligned, bool backward) {
   s.units = s.instance ? static_cast<int>(tile_ch) : kSplitTV >> s.cvg_shift;
   s.tiles = static_cast<int>(p.channels / tile_ch);
   // Block shape: positions per block PB = NL * TPR / 8 (128, 256, 512 or 1024);
-  // planes beyond 16 blocks of the largest shape are left to the other kernels.
+  // planes beyond 16 blocks of the largest shape are left to the other kernels
+  // (BatchNormalization's single plane of all rows: beyond 64 blocks).
   // First choice, from sweeps of the shapes (cold, forward / backward us):
   //  forward: several blocks to a CU, so that one block's exchange and stores
   //    run while the next one's loads arrive - groups 256 x 8 (float and planes
@@ -58,7 +64,22 @@ SplitPlan plan_split(const ClProblem &p, bool aligned, bool backward) {
   auto take = [&](int i) {
     const int64_t pb = static_cast<int64_t>(shapes[i][0]) * shapes[i][1] / kSplitTV;
     const int64_t split = (p.spatial + pb - 1) / pb;
-    if (split > kSplitMax) return false;
+    // (more than 16 blocks per plane only for BatchNormalization's single plane
+    // of all rows, and only in the largest blocks: the partials a block collects
+    // grow with the number of its partners)
+    if (split > (p.as_batch_norm && i == 3 ? kSplitMax : 16)) return false;
+    s.lds_bytes = 16 * 1024; // forward: folds and partials, far from the limit
+    if (backward) {
+      // LDS of cl_split_bwd_kernel: dy parked, the folds, and the blocks'
+      // partials (sized by the launch) - together at most the CU's 160 KB
+      const int64_t ch = tile_ch, umax = s.instance ? ch : kSplitTV;
+      const int64_t fixed = static_cast<int64_t>(shapes[i][0]) * shapes[i][1] * 16 +
+                            (shapes[i][0] / 64) * 2 * ch * 4 + 2 * ch * 4 + umax * 2 * 4 + ch * 4 +
+                            kSplitMax * 4 + 256;
+      const int64_t partials = (split > 16 ? split : 16) * 2 * umax * 4;
+      if (fixed + partials > 160 * 1024) return false;
+      s.lds_bytes = fixed + partials;
+    }
     s.tpr = shapes[i][0];
     s.nl = shapes[i][1];
     s.pb = static_cast<int>(pb);
@@ -97,6 +118,16 @@ SplitPlan plan_split(const ClProblem &p, bool aligned, bool backward) {
   }
   if (!s.ok) return s;
   const int64_t blocks = p.batch * s.tiles * static_cast<int64_t>(s.split);
+  // More blocks than the chip holds at once (a CU takes 1024 threads of these
+  // kernels, and what its LDS allows): a block's partners must be its
+  // neighbours in the grid, or they are not running yet when it polls for
+  // their parts.
+  const int64_t per_cu = std::max<int64_t>(1, std::min<int64_t>(1024 / s.tpr, 160 * 1024 / s.lds_bytes));
+  s.partners_adjacent = blocks > device_cus() * per_cu;
+  // With more than 16 partners a grid of several rounds stalls on the planes
+  // that straddle two rounds ([256,14,14,1024] half forward, 49 blocks per
+  // column tile, 784 in all: 80 us against 62 us of the split reduction).
+  if (s.split > 16 && s.partners_adjacent) s.ok = false;
   s.words = static_cast<size_t>(blocks) * 2 * s.units;
   if (blocks > (1ll << 30) || s.words > xchg_capacity()) s.ok = false;
   if (backward &&
@@ -128,11 +159,18 @@ ClSplitArgs make_args(const ClProblem &p, const SplitPlan &s) {
   a.inv_R = static_cast<float>(1.0 / (static_cast<double>(p.spatial) * (s.instance ? 1 : s.cpg)));
   a.one = 1.0f;
   a.accum_dx = p.accum_dx;
+  a.partners_adjacent = s.partners_adjacent ? 1 : 0;
+  a.rmean = p.rmean;
+  a.rvar = p.rvar;
+  a.decay = p.decay;
+  a.unbias = p.unbias;
   return a;
 }
 
 template <typename T, int VEC, bool INSTANCE>
 int run(bool backward, const SplitPlan &s, const ClSplitArgs &a, unsigned grid, hipStream_t st) {
+  // the blocks' partials of every unit of a tile, in LDS
+  const size_t part_bytes = static_cast<size_t>(s.split) * 2 * s.units * sizeof(float);
 #define SPLIT_CASE(TPR, NL)                                                                      \
   if (s.tpr == (TPR) && s.nl == (NL)) {                                                          \
     if (backward) {                                                                              \
@@ -143,6 +181,19 @@ int run(bool backward, const SplitPlan &s, const ClSplitArgs &a, unsigned grid, 
                      dim3(grid), dim3(TPR), 0, st, a);                                           \
     }                                                                                            \
     return last_launch_status();                                                                 \
+  }
+  if constexpr (INSTANCE) {
+    if (s.split > 16) { // (planned only in the largest block shape)
+      if (s.tpr != 1024 || s.nl != 8) return NBLAHIP_EINVAL;
+      if (backward) {
+        NBLAHIP_LAUNCH("cl_split_bwd_kernel", (cl_split_bwd_kernel<T, VEC, 8, 1024, true, true>),
+                       dim3(grid), dim3(1024), part_bytes, st, a);
+      } else {
+        NBLAHIP_LAUNCH("cl_split_fwd_kernel", (cl_split_fwd_kernel<T, VEC, 8, 1024, true, true>),
+                       dim3(grid), dim3(1024), part_bytes, st, a);
+      }
+      return last_launch_status();
+    }
   }
   SPLIT_CASE(256, 4)
   SPLIT_CASE(256, 8)

@@ -147,6 +147,10 @@ bool bn_cl_cached_bwd(const BnProblem &p, hipStream_t st, int *status);
 // Training forward / backward for planes that are not a whole number of
 // 16-byte vectors (7x7, half 14x14): a pack of 2, 4 or 8 neighbouring channels,
 // whose planes together are, held on one CU (bn_pack.hip).
+// Channel-last training forward / backward of up to 65536 rows through the
+// split kernels of gn_cl_split.hip (all rows as one sample, a unit per channel).
+bool bn_cl_split_fwd_train(const BnProblem &p, hipStream_t st, int *status);
+bool bn_cl_split_bwd(const BnProblem &p, hipStream_t st, int *status);
 bool bn_pack_fwd_train(const BnProblem &p, hipStream_t st, int *status);
 bool bn_pack_bwd(const BnProblem &p, hipStream_t st, int *status);
 int launch_bn_infer(const BnProblem &p, hipStream_t st);
@@ -201,6 +205,12 @@ struct ClProblem {
   float eps = 0.f;
   void *ws = nullptr;
   size_t ws_bytes = 0;
+  // Channel-last BatchNormalization through the split kernels (one "sample" of
+  // all rows, a unit per channel): the running statistics to update, may be null.
+  float *rmean = nullptr;
+  float *rvar = nullptr;
+  float decay = 0.f, unbias = 1.f;
+  int as_batch_norm = 0;
 };
 // Register-cached channel-last GroupNormalization (gn_cl_rows.hip): false when
 // the shape is not theirs, else *status holds the launch result.  The backward
@@ -210,6 +220,7 @@ bool gn_cl_cached_bwd(const ClProblem &p, bool aligned, float *pairs, hipStream_
 // Split channel-last kernels (gn_cl_split.hip): a block owns whole 128-byte
 // lines of a position range, the blocks of a sample exchange partial sums.  The
 // backward leaves per-block pairs in the workspace: *pairs is [*pair_batches][C][2].
+constexpr int kClSplitMaxBlocks = 64; // blocks per (sample, column tile), i.e. pairs per channel
 bool cl_split_fwd(const ClProblem &p, bool aligned, hipStream_t st, int *status);
 bool cl_split_bwd(const ClProblem &p, bool aligned, float **pairs, int64_t *pair_batches,
                   hipStream_t st, int *status);

@@ -41,6 +41,10 @@ SMALL = [
     ((64, 1024, 7, 7), 1), ((256, 256, 7, 7), 1), ((200, 64, 14, 14), 1), ((20, 1024, 3, 3), 1),
     ((300, 256, 5, 5), 1), ((100, 264, 7, 7), 1), ((440, 256, 7, 7), 1), ((190, 512, 7, 7), 1),
     ((40, 256, 11, 11), 1),
+    # channel-last through the split kernels (all rows as one plane, a unit per channel):
+    # 13, 3 and 49 blocks per column tile, rows that do not fill the last block, float
+    ((64, 14, 14, 128), 3), ((3000, 192), 1), ((256, 14, 14, 64), 3), ((20000, 64), 1),
+    ((777, 96), 1),
     # a channel per CU whose planes share cache lines with the neighbouring channels'
     ((256, 64, 14, 14), 1), ((250, 40, 10, 10), 1),
 ]
@@ -101,6 +105,8 @@ def test_bn_training_forward_backward(shape, axis, dtype):
                                         ((8, 64, 12, 12), 1), ((4, 48, 7, 9), 1), ((3, 300, 2, 2), 1),
                                         # a pack of channels per block (planes of 49 elements)
                                         ((90, 256, 7, 7), 1),
+                                        # channel-last through the split kernels
+                                        ((40, 14, 14, 64), 3),
                                         # channel-last, a channel vector's column per block
                                         ((8, 7, 7, 256), 3), ((300, 512), 1)])
 def test_bn_flags(shape, axis):

@@ -178,7 +178,10 @@ SWITCHES = [
      ["bn_cl_grid_bwd_kernel"], {"BN_CL_GRID_MIN_SLOTS": 1}),
     ("bn_cl_cached_off", run_bn, ((32, 7, 7, 256), 3, F16), {"BN_CL_CACHED": 0},
      ["bn_stats_cl_kernel", "bn_apply_cl_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
-     ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"]),
+     ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"], {"BN_CL_SPLIT": 0}),
+    ("bn_cl_split_off", run_bn, ((64, 14, 14, 256), 3, F16), {"BN_CL_SPLIT": 0},
+     ["bn_stats_cl_kernel", "bn_apply_cl_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
+     ["cl_split_fwd_kernel", "cl_split_bwd_kernel"]),
     # rows: LayerNormalization / GroupNormalization / InstanceNormalization
     ("ln_force_stream", run_ln, (64, 1024, F32), {"FORCE_STREAM": 1},
      ["row_stats_stream_kernel", "row_apply_fwd_kernel", "ln_row_sums_stream_kernel",
@@ -263,8 +266,8 @@ GRIDS = [
     ("bn_masked_planes_off", run_bn, ((64, 64, 7, 7), 1, F16), [{"BN_ROWS": 0, "BN_MASKED_PLANES": 0}],
      ["bn_stats_planes_kernel", "bn_apply_planes_kernel"], []),
     ("bn_cl_grids", run_bn, ((64, 28, 28, 64), 3, F16),
-     [{"BN_CL_BLOCKS_PER_CU": a, "BN_CL_FWD_APPLY_BLOCKS_PER_CU": b, "BN_CL_APPLY_BLOCKS_PER_CU": c}
-      for a, b, c in ((1, 1, 1), (2, 4, 2), (8, 3, 7))],
+     [{"BN_CL_BLOCKS_PER_CU": a, "BN_CL_FWD_APPLY_BLOCKS_PER_CU": b, "BN_CL_APPLY_BLOCKS_PER_CU": c,
+       "BN_CL_SPLIT": 0} for a, b, c in ((1, 1, 1), (2, 4, 2), (8, 3, 7))],
      ["bn_stats_cl_kernel", "bn_apply_cl_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
      []),
     ("bn_onchip_few_channels", run_bn, ((32, 4, 56, 56), 1, F16),
