@@ -94,9 +94,9 @@ def n_sets(bytes_per_set):
 # the tensor passes their direction then makes; the split reduction makes 3
 # forward (x for the statistics, x again, y) and 5 backward.
 BN_ONCHIP_FWD = ("bn_onchip_fwd_kernel", "row_fwd_kernel_bn", "in_cl_row_fwd_kernel",
-                 "bn_cl_grid_fwd_kernel", "bn_pack_fwd_kernel")
+                 "bn_cl_grid_fwd_kernel", "bn_pack_fwd_kernel", "bn_chan_split_fwd_kernel")
 BN_ONCHIP_BWD = {"bn_onchip_bwd_kernel": 4, "row_bwd_kernel_bn": 3, "in_cl_row_bwd_kernel": 3,
-                 "bn_pack_bwd_kernel": 3}
+                 "bn_pack_bwd_kernel": 3, "bn_chan_split_bwd_kernel": 3}
 # bn_onchip_bwd_kernel holds x of a channel on its CU and streams dy twice
 # (x, 2 dy, dx = 4 passes); of a channel beyond 20480 16-byte vectors it holds
 # 18432 and reads the rest of x twice as well.

@@ -151,6 +151,11 @@ bool bn_cl_cached_bwd(const BnProblem &p, hipStream_t st, int *status);
 // split kernels of gn_cl_split.hip (all rows as one sample, a unit per channel).
 bool bn_cl_split_fwd_train(const BnProblem &p, hipStream_t st, int *status);
 bool bn_cl_split_bwd(const BnProblem &p, hipStream_t st, int *status);
+// Training forward / backward for fewer channels than CUs: a channel split
+// over 2 - 8 blocks that hold their samples on chip and exchange partial sums
+// (bn_split_channel.hip).
+bool bn_chan_split_fwd_train(const BnProblem &p, hipStream_t st, int *status);
+bool bn_chan_split_bwd(const BnProblem &p, hipStream_t st, int *status);
 bool bn_pack_fwd_train(const BnProblem &p, hipStream_t st, int *status);
 bool bn_pack_bwd(const BnProblem &p, hipStream_t st, int *status);
 int launch_bn_infer(const BnProblem &p, hipStream_t st);

@@ -45,6 +45,10 @@ SMALL = [
     # 13, 3 and 49 blocks per column tile, rows that do not fill the last block, float
     ((64, 14, 14, 128), 3), ((3000, 192), 1), ((256, 14, 14, 64), 3), ((20000, 64), 1),
     ((777, 96), 1),
+    # fewer channels than CUs: a channel split over 2 / 4 / 8 blocks that exchange their sums
+    # (whole and ragged last blocks, both directions in registers, LDS slots)
+    ((32, 64, 56, 56), 1), ((16, 128, 56, 56), 1), ((24, 32, 48, 48), 1), ((21, 64, 40, 40), 1),
+    ((32, 16, 112, 112), 1),
     # a channel per CU whose planes share cache lines with the neighbouring channels'
     ((256, 64, 14, 14), 1), ((250, 40, 10, 10), 1),
 ]
@@ -105,6 +109,8 @@ def test_bn_training_forward_backward(shape, axis, dtype):
                                         ((8, 64, 12, 12), 1), ((4, 48, 7, 9), 1), ((3, 300, 2, 2), 1),
                                         # a pack of channels per block (planes of 49 elements)
                                         ((90, 256, 7, 7), 1),
+                                        # a channel split over 4 blocks
+                                        ((40, 64, 32, 32), 1),
                                         # channel-last through the split kernels
                                         ((40, 14, 14, 64), 3),
                                         # channel-last, a channel vector's column per block
@@ -523,13 +529,18 @@ def test_bn_channel_last_backward_held_on_the_chip(m, c, dtype):
 
 
 @pytest.mark.parametrize("kind", ["offset", "outlier_first", "constant"])
-@pytest.mark.parametrize("shape,axis,dtype,kernel", [
-    ((32, 64, 56, 56), 1, torch.float32, "bn_onchip_fwd_kernel"),
-    ((32, 64, 56, 56), 1, torch.float16, "bn_onchip_fwd_kernel"),
-    ((150000, 64), 1, torch.float32, "bn_cl_grid_fwd_kernel"),
-    ((150000, 64), 1, torch.float16, "bn_cl_grid_fwd_kernel"),
+@pytest.mark.parametrize("shape,axis,dtype,kernel,knobs", [
+    ((32, 64, 56, 56), 1, torch.float32, "bn_onchip_fwd_kernel", {"BN_CHAN_SPLIT": 0}),
+    ((32, 64, 56, 56), 1, torch.float16, "bn_onchip_fwd_kernel", {"BN_CHAN_SPLIT": 0}),
+    ((32, 64, 56, 56), 1, torch.float32, "bn_chan_split_fwd_kernel", {}),
+    ((32, 64, 56, 56), 1, torch.float16, "bn_chan_split_fwd_kernel", {}),
+    ((150000, 64), 1, torch.float32, "bn_cl_grid_fwd_kernel", {"BN_CL_GRID_MIN_SLOTS": 1}),
+    ((150000, 64), 1, torch.float16, "bn_cl_grid_fwd_kernel", {"BN_CL_GRID_MIN_SLOTS": 1}),
+    ((200, 256, 7, 7), 1, torch.float32, "bn_pack_fwd_kernel", {}),
+    ((200, 256, 7, 7), 1, torch.float16, "bn_pack_fwd_kernel", {}),
+    ((12000, 128), 1, torch.float16, "cl_split_fwd_kernel", {}),
 ])
-def test_one_pass_statistics_on_hard_data(kind, shape, axis, dtype, kernel):
+def test_one_pass_statistics_on_hard_data(kind, shape, axis, dtype, kernel, knobs):
     """The statistics shift by each thread's own mean: a mean far
     from zero, one huge value in the very first element of every channel (1000
     deviations off everything else its thread holds), and constant data
@@ -548,7 +559,8 @@ def test_one_pass_statistics_on_hard_data(kind, shape, axis, dtype, kernel):
         x = np.full(shape, 3.25)
     x = rounded(x, dtype)
     y_r, m_r, v_r, _, _ = R.bn_forward_batch(x, None, None, None, None, axis, 0.9, 1e-5)
-    K.tune_set("BN_CL_GRID_MIN_SLOTS", 1)
+    for name, value in knobs.items():
+        K.tune_set(name, value)
     try:
         K.check(K.lib().nblahip_profile_enable(8))
         y, m, v = K.bn_forward_batch(to_dev(x, dtype), None, None, None, None, axis, 0.9, 1e-5)

@@ -125,6 +125,9 @@ def run_in(n, c, sp, dtype, channel_last=False, seed=4):
 # GroupNormalization rows about the channel-last kernels that own whole groups
 # run with the split kernels (which take those shapes by default) switched off.
 NO_SPLIT = {"GN_CL_SPLIT": 0}
+# BatchNormalization rows about the kernels that give a channel one block run
+# with the channel split over several blocks (the default for few channels) off.
+NO_CHAN_SPLIT = {"BN_CHAN_SPLIT": 0}
 
 
 def kernels_of(run, args, knobs):
@@ -152,15 +155,18 @@ SWITCHES = [
     ("bn_onchip_off", run_bn, ((32, 64, 56, 56), 1, F16), {"BN_ONCHIP": 0},
      ["bn_stats_planes_kernel", "bn_apply_planes_kernel", "bn_bwd_reduce_planes_kernel",
       "bn_bwd_apply_planes_kernel"],
-     ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"]),
+     ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], NO_CHAN_SPLIT),
     ("bn_onchip_fwd_max", run_bn, ((32, 32, 56, 56), 1, F32), {"BN_ONCHIP_FWD_MAX": 16},
-     ["bn_stats_planes_kernel"], ["bn_onchip_fwd_kernel"]),
+     ["bn_stats_planes_kernel"], ["bn_onchip_fwd_kernel"], NO_CHAN_SPLIT),
     ("bn_onchip_bwd_max", run_bn, ((32, 64, 56, 56), 1, F16), {"BN_ONCHIP_BWD_MAX": 8},
-     ["bn_onchip_fwd_kernel", "bn_bwd_reduce_planes_kernel"], ["bn_onchip_bwd_kernel"]),
+     ["bn_onchip_fwd_kernel", "bn_bwd_reduce_planes_kernel"], ["bn_onchip_bwd_kernel"], NO_CHAN_SPLIT),
     ("bn_onchip_min_pct_up", run_bn, ((32, 64, 56, 56), 1, F16),
      {"BN_ONCHIP_FWD_MIN_PCT": 100, "BN_ONCHIP_BWD_MIN_PCT": 100},
      ["bn_stats_planes_kernel", "bn_bwd_reduce_planes_kernel"],
-     ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"]),
+     ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], NO_CHAN_SPLIT),
+    ("bn_chan_split_off", run_bn, ((32, 64, 56, 56), 1, F16), {"BN_CHAN_SPLIT": 0},
+     ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"],
+     ["bn_chan_split_fwd_kernel", "bn_chan_split_bwd_kernel"]),
     ("bn_rows_off", run_bn, ((32, 64, 14, 14), 1, F16), {"BN_ROWS": 0},
      ["bn_stats_planes_kernel", "bn_finalize_fwd_kernel", "bn_apply_planes_kernel",
       "bn_finalize_bwd_kernel"], ["row_fwd_kernel_bn", "row_bwd_kernel_bn"]),
@@ -275,13 +281,19 @@ GRIDS = [
      ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
     # planes that share cache lines with their neighbours: ordinary stores there, or not
     ("bn_onchip_edge_stores_off", run_bn, ((256, 64, 14, 14), 1, F32),
-     [{"BN_EDGE_STORES_MAX_BYTES": 0}], ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
+     [{"BN_EDGE_STORES_MAX_BYTES": 0, **NO_CHAN_SPLIT}], ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
     ("bn_rows_edge_stores_off", run_bn, ((32, 64, 14, 14), 1, F16), [{"BN_EDGE_STORES_MAX_BYTES": 0}],
      ["row_fwd_kernel_bn", "row_bwd_kernel_bn"], []),
     ("bn_onchip_edge_stores_longer_planes", run_bn, ((128, 64, 28, 28), 1, F16),
      [{"BN_EDGE_STORES_MAX_BYTES": 4096}], ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
     ("bn_onchip_streamed_few_channels", run_bn, ((64, 8, 56, 56), 1, F32),
      [{"BN_ONCHIP_STREAMED_MIN_PCT": 1}], ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
+    # a channel split over 8 blocks on a quarter of the CUs; every partner's part
+    # recomputed because no poll is allowed
+    ("bn_chan_split_few_blocks", run_bn, ((40, 8, 32, 32), 1, F32), [{"BN_CHAN_SPLIT_MIN_PCT": 1}],
+     ["bn_chan_split_fwd_kernel", "bn_chan_split_bwd_kernel"], []),
+    ("bn_chan_split_no_polls", run_bn, ((32, 64, 56, 56), 1, F16), [{"XCHG_SPIN": 0}],
+     ["bn_chan_split_fwd_kernel", "bn_chan_split_bwd_kernel"], []),
     ("bn_pack_few_channels", run_bn, ((48, 16, 7, 7), 1, F16), [{"BN_PACK_SHORT_MIN_PCT": 0}],
      ["bn_pack_fwd_kernel", "bn_pack_bwd_kernel"], []),
     ("bn_pack_plain_block_order", run_bn, ((96, 256, 7, 7), 1, F16),

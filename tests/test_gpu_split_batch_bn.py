@@ -89,14 +89,15 @@ def test_split_batch_equals_whole_batch(splits, rest, axis, dtype):
 
 
 def test_one_worker_is_bitwise_the_plain_path():
-    """(On a shape whose channels do not fit one block's registers: there the
-    plain path is the same split reduction; smaller channels take the
-    single-pass row kernels, which sum in another order.)"""
+    """(On a shape whose plain path is the same split reduction: channels that
+    do not fit one block's registers, and too few of them for the kernels that
+    hold a channel on one CU or split it over several; those and the
+    single-pass row kernels sum in another order.)"""
     torch.manual_seed(3)
-    x = torch.randn(64, 32, 48, 48, device="cuda")
+    x = torch.randn(64, 8, 48, 48, device="cuda")
     dy = torch.randn_like(x)
-    g = torch.rand(32, device="cuda") + 0.5
-    b = torch.randn(32, device="cuda")
+    g = torch.rand(8, device="cuda") + 0.5
+    b = torch.randn(8, device="cuda")
     y0, m0, v0 = K.bn_forward_batch(x, b, g, None, None, 1, 0.9, 1e-5)
     dx0, dg0, db0 = K.bn_backward(x, dy, g, m0, v0, 1, 1e-5)
     m, v = K.bn_local_stats(x, 1)
