@@ -320,13 +320,17 @@ __device__ __forceinline__ void chan_pair_from_memory(const BnChanSplitArgs &a, 
 //   sdx = sum dy*xh (= dgamma), sdy = sum dy (= dbeta),
 //   dx = dy*g*istd + xh*cA + cb,  cA = -istd*g*sdx/N + 2*dvar*std/N,
 //   cb = -g*sdy*istd/N + dmean/N.
-// NL vectors of x per thread in registers; dy in batches of B, its first ND
-// vectors per thread parked in LDS, the others read again for dx.
-template <typename T, int VEC, int NL, int ND, int B>
+// NL vectors of x per thread: the first NL - NXS in registers, NXS in LDS; dy
+// in batches of B, its first ND vectors per thread parked in LDS (NXS + ND <=
+// 9: 144 KB), the others read again for dx.
+template <typename T, int VEC, int NL, int NXS, int ND, int B>
 __global__ void __launch_bounds__(kOnchipBlock)
 bn_chan_split_bwd_kernel(const BnChanSplitArgs a) {
   static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors");
+  static_assert(NXS + ND <= 9 && NXS < NL, "LDS slots");
+  constexpr int NXR = NL - NXS;
   __shared__ uint4 park[ND > 0 ? ND * kOnchipBlock : 1];
+  __shared__ uint4 xlds[NXS > 0 ? NXS * kOnchipBlock : 1];
   __shared__ float red[32];
   __shared__ float got[2 * kChanSplitMax];
   __shared__ int miss[kChanSplitMax];
@@ -345,12 +349,27 @@ bn_chan_split_bwd_kernel(const BnChanSplitArgs a) {
   const uint32_t nvb = chan_block_samples(a, sp) * a.vpp.d;
   const uint32_t last = nvb - 1u;
 
-  RawVec<T, VEC> xr[NL];
+  RawVec<T, VEC> xr[NXR];
+  {
+    RawVec<T, VEC> xp[NXS > 0 ? NXS : 1];
 #pragma unroll
-  for (int k = 0; k < NL; ++k) {
-    const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t;
-    xr[k] = load_raw<T, VEC>(x + chan_offset(a, c, sp, min(v, last), VEC));
+    for (int k = 0; k < NXS; ++k) {
+      const uint32_t v = static_cast<uint32_t>(NXR + k) * kOnchipBlock + t;
+      xp[k] = load_raw<T, VEC>(x + chan_offset(a, c, sp, min(v, last), VEC));
+    }
+#pragma unroll
+    for (int k = 0; k < NXR; ++k) {
+      const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t;
+      xr[k] = load_raw<T, VEC>(x + chan_offset(a, c, sp, min(v, last), VEC));
+    }
+#pragma unroll
+    for (int k = 0; k < NXS; ++k) xlds[k * kOnchipBlock + t] = __builtin_bit_cast(uint4, xp[k]);
   }
+  // (each thread reads back only what it wrote: no barrier)
+  auto xvec = [&](int k) -> RawVec<T, VEC> {
+    if (k < NXR) return xr[k < NXR ? k : 0];
+    return __builtin_bit_cast(RawVec<T, VEC>, xlds[(k - NXR) * kOnchipBlock + t]);
+  };
   const float istd = 1.0f / sqrtf(vpe);
   const float nmi = -mean * istd;
 
@@ -374,9 +393,10 @@ bn_chan_split_bwd_kernel(const BnChanSplitArgs a) {
       if (k < NL) {
         if (k < ND) park[(k < ND ? k : 0) * kOnchipBlock + t] = __builtin_bit_cast(uint4, d[i]);
         if (static_cast<uint32_t>(k) * kOnchipBlock + t < nvb) {
+          const RawVec<T, VEC> xk = xvec(k);
 #pragma unroll
           for (int j = 0; j < VEC; ++j) {
-            const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+            const float xh = norm_elem<T, VEC>(xk, j, mean, istd, nmi);
             sdx = elem_fma<T, VEC>(d[i], j, xh, sdx);
             sdy = elem_fma<T, VEC>(d[i], j, a.one, sdy);
           }
@@ -417,7 +437,7 @@ bn_chan_split_bwd_kernel(const BnChanSplitArgs a) {
 
   // ---- pass 2: dx = dy*gi + (x - mean)*A2 + cb  (half: x*A2 + B2, one mixed fma)
 #pragma unroll
-  for (int k = 0; k < NL; ++k) forget<T, VEC>(xr[k]);
+  for (int k = 0; k < NXR; ++k) forget<T, VEC>(xr[k]);
   const float cA = -istd * g * fin[0] * a.inv_N + (a.dvar ? 2.f * p_dvar * (vpe * istd) * a.inv_N : 0.f);
   const float cb = -g * fin[1] * istd * a.inv_N + (a.dmean ? p_dmean * a.inv_N : 0.f);
   const float gi = g * istd;
@@ -448,7 +468,7 @@ bn_chan_split_bwd_kernel(const BnChanSplitArgs a) {
 #pragma unroll
   for (int k = 0; k < ND && k < NL; ++k) {
     const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t2;
-    if (v < nvb) emit(xr[k], __builtin_bit_cast(RawVec<T, VEC>, park[k * kOnchipBlock + t]), v);
+    if (v < nvb) emit(xvec(k), __builtin_bit_cast(RawVec<T, VEC>, park[k * kOnchipBlock + t]), v);
   }
   float lastv = B2;
 #pragma unroll
@@ -468,7 +488,7 @@ bn_chan_split_bwd_kernel(const BnChanSplitArgs a) {
       const int k = k0 + i;
       const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t3;
       if (k < NL && v < nvb) {
-        emit(xr[k < NL ? k : 0], d[i], v);
+        emit(xvec(k < NL ? k : 0), d[i], v);
         lastv = __builtin_bit_cast(float, __builtin_bit_cast(uint4, d[i]).x);
       }
     }
@@ -479,7 +499,7 @@ bn_chan_split_bwd_kernel(const BnChanSplitArgs a) {
 namespace {
 
 constexpr int kChanFwdMax = 25; // vectors per thread the forward holds (16 registers + 9 LDS)
-constexpr int kChanBwdMax = 12; // vectors of x per thread the backward holds
+constexpr int kChanBwdMax = 21; // vectors of x per thread the backward holds (12 registers + 9 LDS)
 
 template <typename T, int VEC>
 int run_chan_fwd(int nl, const BnChanSplitArgs &a, unsigned grid, hipStream_t st) {
@@ -504,18 +524,21 @@ int run_chan_fwd(int nl, const BnChanSplitArgs &a, unsigned grid, hipStream_t st
 template <typename T, int VEC>
 int run_chan_bwd(int nl, const BnChanSplitArgs &a, unsigned grid, hipStream_t st) {
   constexpr int kB = sizeof(T) == 2 ? 2 : 4;
-#define CHAN_CASE(NL)                                                                            \
+#define CHAN_CASE(NL, NXS, ND)                                                                   \
   if (nl <= (NL)) {                                                                              \
-    NBLAHIP_LAUNCH("bn_chan_split_bwd_kernel",                                                   \
-                   (bn_chan_split_bwd_kernel<T, VEC, NL, ((NL) < 9 ? (NL) : 9), kB>), dim3(grid), \
-                   dim3(kOnchipBlock), 0, st, a);                                                \
+    NBLAHIP_LAUNCH("bn_chan_split_bwd_kernel", (bn_chan_split_bwd_kernel<T, VEC, NL, NXS, ND, kB>), \
+                   dim3(grid), dim3(kOnchipBlock), 0, st, a);                                    \
     return last_launch_status();                                                                 \
   }
-  CHAN_CASE(2)
-  CHAN_CASE(4)
-  CHAN_CASE(7)
-  CHAN_CASE(9)
-  CHAN_CASE(12)
+  CHAN_CASE(2, 0, 2)
+  CHAN_CASE(4, 0, 4)
+  CHAN_CASE(7, 0, 7)
+  CHAN_CASE(9, 0, 9)
+  CHAN_CASE(12, 0, 9)
+  CHAN_CASE(14, 2, 7)
+  CHAN_CASE(16, 4, 5)
+  CHAN_CASE(18, 6, 3)
+  CHAN_CASE(21, 9, 0)
 #undef CHAN_CASE
   return NBLAHIP_EINVAL;
 }

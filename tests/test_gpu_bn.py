@@ -48,7 +48,7 @@ SMALL = [
     # fewer channels than CUs: a channel split over 2 / 4 / 8 blocks that exchange their sums
     # (whole and ragged last blocks, both directions in registers, LDS slots)
     ((32, 64, 56, 56), 1), ((16, 128, 56, 56), 1), ((24, 32, 48, 48), 1), ((21, 64, 40, 40), 1),
-    ((32, 16, 112, 112), 1),
+    ((32, 16, 112, 112), 1), ((64, 64, 56, 56), 1), ((84, 64, 56, 56), 1),
     # a channel per CU whose planes share cache lines with the neighbouring channels'
     ((256, 64, 14, 14), 1), ((250, 40, 10, 10), 1),
 ]
