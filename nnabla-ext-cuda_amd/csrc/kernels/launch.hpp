@@ -73,6 +73,10 @@ struct RowProblem {
 // InstanceNormalization backward with a plane's x held on one CU (bn_onchip.hip);
 // false: not taken.  Leaves the per-plane (dgamma, dbeta) parts in p.ws.
 bool in_onchip_bwd(const RowProblem &p, hipStream_t st, int *status);
+// GroupNormalization backward with a group of 128 - 336 KB held on one CU
+// (gn_onchip_bwd.hip); false: not taken.  Leaves the per-(sample, channel)
+// (dgamma, dbeta) parts in p.ws.
+bool gn_onchip_bwd(const RowProblem &p, hipStream_t st, int *status);
 
 struct RowCfg {
   bool ok = false;

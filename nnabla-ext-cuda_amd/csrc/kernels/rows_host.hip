@@ -464,6 +464,8 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
       cfg.ok = false;
   }
   if (!cfg.ok && !tune_int("FORCE_STREAM", 0)) {
+    if (int status = 0; gn_onchip_bwd(p, st, &status))
+      return status ? status : launch_pair_reduce(p, static_cast<const float *>(p.ws), st);
     if (int status = 0; in_onchip_bwd(p, st, &status))
       return status ? status : launch_pair_reduce(p, static_cast<const float *>(p.ws), st);
   }

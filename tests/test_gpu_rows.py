@@ -199,7 +199,9 @@ def test_gn_forward_backward(n, c, sp, groups, dtype):
 
 
 @pytest.mark.parametrize("n,c,sp,groups", [(4, 64, (16, 16), 8), (2, 32, (7, 7), 8),
-                                           (2, 160, (64, 64), 16)])
+                                           (2, 160, (64, 64), 16),
+                                           # the group held on one CU in the backward
+                                           (4, 320, (64, 64), 32)])
 def test_gn_flags(n, c, sp, groups):
     dtype = torch.float32
     x, dy, g, b = make_nc(n, c, sp, dtype, 5)
@@ -390,6 +392,10 @@ ONCHIP_ROWS = [
     ("in", torch.float16, 1, 64, (360, 360), 0), ("in", torch.float16, 2, 33, (2, 70004), 0),
     # ... with the first 18432 vectors held and the rest streamed
     ("in", torch.float32, 1, 230, (300, 300), 0), ("in", torch.float16, 1, 240, (2, 150004), 0),
+    # GroupNormalization backward with the group held on its CU: x in registers and LDS,
+    # dy parked in what LDS is left (10, 15, 20 and 12 vectors per thread)
+    ("gn", torch.float16, 3, 960, (64, 64), 32), ("gn", torch.float32, 2, 640, (64, 64), 32),
+    ("gn", torch.float16, 2, 1536, (64, 32), 64), ("gn", torch.float32, 4, 192, (64, 64), 16),
 ]
 
 
