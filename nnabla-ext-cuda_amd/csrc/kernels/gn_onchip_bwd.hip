@@ -1,8 +1,8 @@
-// GroupNormalization backward for groups of 128 KB - 336 KB (channel-first),
+// GroupNormalization backward for groups of 64 KB - 336 KB (channel-first),
 // with the group held on one CU.
 //
 // The row kernels (rows.cuh) keep a group's x and dy in 8 vectors per thread of
-// a 1024-thread block: 128 KB.  Beyond that the backward used to stream: the
+// a 1024-thread block: 128 KB.  Beyond that the backward streams: the
 // per-plane sums in one pass, dx in a second (5 S).  Here one 1024-thread block
 // per group holds up to 21 vectors of x per thread (12 in registers, 9 in LDS)
 // and parks dy in the LDS that x leaves free (9 slots of 16 KB in all; the
@@ -231,6 +231,9 @@ int run_gn_onchip_bwd(int nl, const GnOnchipArgs &a, unsigned grid, hipStream_t 
                    dim3(grid), dim3(kOnchipBlock), 0, st, a);                                    \
     return last_launch_status();                                                                 \
   }
+  GN_CASE(3, 0, 3)
+  GN_CASE(5, 0, 5)
+  GN_CASE(7, 0, 7)
   GN_CASE(9, 0, 9)
   GN_CASE(12, 0, 9)
   GN_CASE(14, 2, 7)
@@ -255,7 +258,12 @@ bool gn_onchip_bwd(const RowProblem &p, hipStream_t st, int *status) {
   if (p.spatial % (64 * vec) != 0 || cpg > kGnOnchipMaxCpg) return false;
   const int64_t nv = p.R / vec;
   const int64_t nl = (nv + kOnchipBlock - 1) / kOnchipBlock;
-  if (nl <= 8 || nl > 21) return false; // (up to 8: the row kernels)
+  // From 5 vectors per thread (groups beyond 64 KB), where it also beats the
+  // row kernels that hold such a group in 8 vectors per thread of smaller
+  // blocks: 80 KB half groups 35.7 -> 26.8 us, 128 KB 26.1 -> 20.4 us, float
+  // 128 KB 40.1 -> 37.2 us; at 64 KB ([16,256,64,64] half, two 512-thread
+  // blocks per CU there) 20.4 against 22.7 us.
+  if (nl < tune_int("GN_ONCHIP_BWD_MIN_NL", 5) || nl > 21) return false;
   // a block is alone on its CU: groups for at least this share of the CUs
   if (p.rows * 100 < static_cast<int64_t>(device_cus()) * tune_int("ROW_ONCHIP_BWD_MIN_PCT", 25))
     return false;

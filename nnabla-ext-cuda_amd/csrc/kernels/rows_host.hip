@@ -463,9 +463,11 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
         !tune_int("GN_FLOAT_1024X8", 1))
       cfg.ok = false;
   }
-  if (!cfg.ok && !tune_int("FORCE_STREAM", 0)) {
+  if (!tune_int("FORCE_STREAM", 0)) {
     if (int status = 0; gn_onchip_bwd(p, st, &status))
       return status ? status : launch_pair_reduce(p, static_cast<const float *>(p.ws), st);
+  }
+  if (!cfg.ok && !tune_int("FORCE_STREAM", 0)) {
     if (int status = 0; in_onchip_bwd(p, st, &status))
       return status ? status : launch_pair_reduce(p, static_cast<const float *>(p.ws), st);
   }
