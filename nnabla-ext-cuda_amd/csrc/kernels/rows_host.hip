@@ -269,6 +269,10 @@ int launch_row_fwd(const RowProblem &p, hipStream_t st) {
   // a row over more threads instead.
   const int max_nl = p.mode == kRowLN ? 4 : 8;
   const RowCfg cfg = pick_row_cfg(vec, p.R, max_nl, max_nl, 4, p.mode == kRowLN);
+  // (rows beyond 64 KB held on one CU also where the row kernels' layouts reach)
+  if (int status = 0; cfg.ok && !tune_int("FORCE_STREAM", 0) && p.R / vec > 4096 &&
+                      row_onchip_fwd(p, a, vec, st, &status))
+    return status;
   if (cfg.ok && !tune_int("FORCE_STREAM", 0)) {
     return run_row_fwd_cached(p.dtype, cfg, a, cached_grid(p.rows, cfg.tpr), st);
   }

@@ -188,7 +188,10 @@ int run_onchip_fwd(int nl, const RowArgs &a, int grid, hipStream_t st) {
 
 } // namespace
 
-// Rows of 8193..25600 full vectors, at least an eighth as many as there are
+// Rows of 4097..25600 full vectors (from 64 KB on it also beats the row kernels
+// that hold such a row in 8 vectors per thread: 80 KB half groups 18.0 -> 14.0
+// us, 120 KB 24.4 -> 19.7 us, float 80 KB 17.3 -> 13.4 us, 128 KB half planes
+// 25.6 -> 21.0 us; 64 KB: 12.2 either way), at least an eighth as many as there are
 // CUs (the block is alone on its CU; with fewer rows the streaming kernels,
 // which split a row over many blocks, use more of the chip: 32 groups of 160 KB
 // 8.3 vs 11.8 us, 16 of 320 KB 12.6 vs 11.7 us); up to 65536 vectors with the
@@ -198,7 +201,7 @@ bool row_onchip_fwd(const RowProblem &p, const RowArgs &a, int vec, hipStream_t 
   if (p.mode == kRowLN || !p.out) return false;
   if (vec != (p.dtype == NBLAHIP_F16 ? 8 : 4)) return false;
   const int64_t nv = p.R / vec;
-  if (nv <= 8192 || nv > 65536) return false;
+  if (nv < tune_int("ROW_ONCHIP_FWD_MIN_VECTORS", 4097) || nv > 65536) return false;
   const int min_pct = nv <= 25 * kOnchipBlock ? tune_int("ROW_ONCHIP_MIN_PCT", 12)
                                               : tune_int("ROW_ONCHIP_STREAMED_MIN_PCT", 88);
   if (p.rows * 100 < static_cast<int64_t>(device_cus()) * min_pct) return false;
