@@ -39,14 +39,17 @@ struct GnOnchipArgs {
   uint32_t G;    // groups per sample (gamma of row r starts at (r % G) * cpg)
   uint32_t cpg;  // channels per group
   uint32_t nv;   // vectors per row
-  FastDiv rpc;   // 64-vector runs per channel
+  FastDiv rpc;   // 64-vector runs per channel (planes of whole runs)
+  FastDiv pv;    // vectors per plane (planes of 8, 16 or 32 vectors: SUB > 0)
   float eps, inv_R, one;
   int accum_dx;
 };
 
 } // namespace
 
-template <typename T, int VEC, int NL, int NXS, int ND, int B>
+// SUB > 0: planes of 64 >> SUB vectors, i.e. 2, 4 or 8 channels side by side
+// in a wave's load; the per-channel sums are sums over the lanes of a channel.
+template <typename T, int VEC, int NL, int NXS, int ND, int B, int SUB = 0>
 __global__ void __launch_bounds__(kOnchipBlock)
 gn_onchip_bwd_kernel(const GnOnchipArgs a) {
   static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors");
@@ -55,7 +58,8 @@ gn_onchip_bwd_kernel(const GnOnchipArgs a) {
   constexpr int NW = kOnchipBlock / kWave;
   __shared__ uint4 park[ND > 0 ? ND * kOnchipBlock : 1];
   __shared__ uint4 xlds[NXS > 0 ? NXS * kOnchipBlock : 1];
-  __shared__ float part[2 * NL * NW]; // (sum dy*xh, sum dy) per run of 64 vectors
+  // (sum dy*xh, sum dy) per run of 64 vectors; SUB > 0: per channel
+  __shared__ float part[SUB > 0 ? 2 * kGnOnchipMaxCpg : 2 * NL * NW];
   __shared__ float gch[kGnOnchipMaxCpg];
   __shared__ float red[32];
   const uint32_t t = threadIdx.x;
@@ -127,11 +131,22 @@ gn_onchip_bwd_kernel(const GnOnchipArgs a) {
             sdy = elem_fma<T, VEC>(d[i], j, a.one, sdy);
           }
         }
-        sdx = wave_sum(sdx);
-        sdy = wave_sum(sdy);
-        if (lane == 0) {
-          part[2 * (k * NW + wave)] = sdx;
-          part[2 * (k * NW + wave) + 1] = sdy;
+        if constexpr (SUB > 0) {
+          constexpr int PV = kWave >> SUB;
+          sdx = group_sum<PV>(sdx);
+          sdy = group_sum<PV>(sdy);
+          const uint32_t v = static_cast<uint32_t>(k) * kOnchipBlock + t;
+          if (lane % PV == 0 && v < a.nv) { // (a channel lies in one wave's load: written once)
+            part[2 * (v / PV)] = sdx;
+            part[2 * (v / PV) + 1] = sdy;
+          }
+        } else {
+          sdx = wave_sum(sdx);
+          sdy = wave_sum(sdy);
+          if (lane == 0) {
+            part[2 * (k * NW + wave)] = sdx;
+            part[2 * (k * NW + wave) + 1] = sdy;
+          }
         }
       }
     }
@@ -143,9 +158,14 @@ gn_onchip_bwd_kernel(const GnOnchipArgs a) {
   float c1 = 0.f, c2 = 0.f;
   if (t < a.cpg) {
     float sdx = 0.f, sdy = 0.f;
-    for (uint32_t e = t * a.rpc.d; e < (t + 1u) * a.rpc.d; ++e) {
-      sdx += part[2 * e];
-      sdy += part[2 * e + 1];
+    if constexpr (SUB > 0) {
+      sdx = part[2 * t];
+      sdy = part[2 * t + 1];
+    } else {
+      for (uint32_t e = t * a.rpc.d; e < (t + 1u) * a.rpc.d; ++e) {
+        sdx += part[2 * e];
+        sdy += part[2 * e + 1];
+      }
     }
     if (a.pairs) {
       const size_t o = 2 * (static_cast<size_t>(row) * a.cpg + t);
@@ -167,7 +187,7 @@ gn_onchip_bwd_kernel(const GnOnchipArgs a) {
   const float A2 = istd * cA;
   const float B2 = sizeof(T) == 2 ? fmaf(nmi, cA, cb) : cb;
   auto emit = [&](const RawVec<T, VEC> &xv, const RawVec<T, VEC> &dv, int k, uint32_t v) {
-    const float gi = gch[a.rpc.div(static_cast<uint32_t>(k) * NW + wave)] * istd;
+    const float gi = (SUB > 0 ? gch[v >> (6 - SUB)] : gch[a.rpc.div(static_cast<uint32_t>(k) * NW + wave)]) * istd;
     float o[VEC];
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
@@ -222,26 +242,39 @@ gn_onchip_bwd_kernel(const GnOnchipArgs a) {
 
 namespace {
 
-template <typename T, int VEC>
+template <typename T, int VEC, int SUB>
 int run_gn_onchip_bwd(int nl, const GnOnchipArgs &a, unsigned grid, hipStream_t st) {
   constexpr int kB = sizeof(T) == 2 ? 2 : 4;
 #define GN_CASE(NL, NXS, ND)                                                                     \
   if (nl <= (NL)) {                                                                              \
-    NBLAHIP_LAUNCH("gn_onchip_bwd_kernel", (gn_onchip_bwd_kernel<T, VEC, NL, NXS, ND, kB>),      \
+    NBLAHIP_LAUNCH("gn_onchip_bwd_kernel", (gn_onchip_bwd_kernel<T, VEC, NL, NXS, ND, kB, SUB>), \
                    dim3(grid), dim3(kOnchipBlock), 0, st, a);                                    \
     return last_launch_status();                                                                 \
   }
+  GN_CASE(2, 0, 2)
   GN_CASE(3, 0, 3)
   GN_CASE(5, 0, 5)
   GN_CASE(7, 0, 7)
   GN_CASE(9, 0, 9)
   GN_CASE(12, 0, 9)
-  GN_CASE(14, 2, 7)
-  GN_CASE(16, 4, 5)
-  GN_CASE(18, 6, 3)
-  GN_CASE(21, 9, 0)
+  if constexpr (SUB == 0) {
+    GN_CASE(14, 2, 7)
+    GN_CASE(16, 4, 5)
+    GN_CASE(18, 6, 3)
+    GN_CASE(21, 9, 0)
+  }
 #undef GN_CASE
   return NBLAHIP_EINVAL;
+}
+
+template <typename T, int VEC>
+int run_gn_onchip_bwd_sub(int sub, int nl, const GnOnchipArgs &a, unsigned grid, hipStream_t st) {
+  switch (sub) {
+  case 0: return run_gn_onchip_bwd<T, VEC, 0>(nl, a, grid, st);
+  case 1: return run_gn_onchip_bwd<T, VEC, 1>(nl, a, grid, st);
+  case 2: return run_gn_onchip_bwd<T, VEC, 2>(nl, a, grid, st);
+  default: return run_gn_onchip_bwd<T, VEC, 3>(nl, a, grid, st);
+  }
 }
 
 } // namespace
@@ -254,16 +287,27 @@ bool gn_onchip_bwd(const RowProblem &p, hipStream_t st, int *status) {
   const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
   if (!aligned16(p.x) || !aligned16(p.dy) || (p.out && !aligned16(p.out))) return false;
   const int64_t cpg = p.channels / p.groups;
-  // a wave's load inside one channel: planes of whole 64-vector runs
-  if (p.spatial % (64 * vec) != 0 || cpg > kGnOnchipMaxCpg) return false;
+  // a wave's load inside one channel (planes of whole 64-vector runs), or 2, 4
+  // or 8 whole channels inside a wave's load (planes of 32, 16 or 8 vectors)
+  if (p.spatial % vec != 0 || cpg > kGnOnchipMaxCpg) return false;
+  const int64_t pv = p.spatial / vec;
+  int sub = 0;
+  if (pv % 64 != 0) {
+    if (pv != 32 && pv != 16 && pv != 8) return false;
+    sub = pv == 32 ? 1 : pv == 16 ? 2 : 3;
+  }
   const int64_t nv = p.R / vec;
   const int64_t nl = (nv + kOnchipBlock - 1) / kOnchipBlock;
+  // Small planes leave half and more of the row kernels' lanes idle (a wave's
+  // load there never crosses a channel): from 2 vectors per thread
+  // ([16,2560,16,16] half 32.0 us with them).
+  if (sub > 0 && (nl < tune_int("GN_ONCHIP_BWD_SMALL_PLANES_MIN_NL", 2) || nl > 12)) return false;
   // From 5 vectors per thread (groups beyond 64 KB), where it also beats the
   // row kernels that hold such a group in 8 vectors per thread of smaller
   // blocks: 80 KB half groups 35.7 -> 26.8 us, 128 KB 26.1 -> 20.4 us, float
   // 128 KB 40.1 -> 37.2 us; at 64 KB ([16,256,64,64] half, two 512-thread
   // blocks per CU there) 20.4 against 22.7 us.
-  if (nl < tune_int("GN_ONCHIP_BWD_MIN_NL", 5) || nl > 21) return false;
+  if (sub == 0 && (nl < tune_int("GN_ONCHIP_BWD_MIN_NL", 5) || nl > 21)) return false;
   // a block is alone on its CU: groups for at least this share of the CUs
   if (p.rows * 100 < static_cast<int64_t>(device_cus()) * tune_int("ROW_ONCHIP_BWD_MIN_PCT", 25))
     return false;
@@ -282,14 +326,15 @@ bool gn_onchip_bwd(const RowProblem &p, hipStream_t st, int *status) {
   a.G = static_cast<uint32_t>(p.groups);
   a.cpg = static_cast<uint32_t>(cpg);
   a.nv = static_cast<uint32_t>(nv);
-  a.rpc = FastDiv(static_cast<uint32_t>(p.spatial / (64 * vec)));
+  a.rpc = FastDiv(static_cast<uint32_t>(std::max<int64_t>(1, pv / 64)));
+  a.pv = FastDiv(static_cast<uint32_t>(pv));
   a.eps = p.eps;
   a.inv_R = static_cast<float>(1.0 / static_cast<double>(p.R));
   a.one = 1.0f;
   a.accum_dx = p.accum_dx;
   const unsigned grid = static_cast<unsigned>(p.rows);
-  *status = p.dtype == NBLAHIP_F16 ? run_gn_onchip_bwd<__half, 8>(static_cast<int>(nl), a, grid, st)
-                                   : run_gn_onchip_bwd<float, 4>(static_cast<int>(nl), a, grid, st);
+  *status = p.dtype == NBLAHIP_F16 ? run_gn_onchip_bwd_sub<__half, 8>(sub, static_cast<int>(nl), a, grid, st)
+                                   : run_gn_onchip_bwd_sub<float, 4>(sub, static_cast<int>(nl), a, grid, st);
   return true;
 }
 

@@ -166,6 +166,10 @@ GN_SHAPES = [(2, 8, (8, 8), 4), (3, 6, (5,), 2), (1, 4, (2, 2), 1), (2, 6, (4,),
              (3, 24, (24, 24), 3), (2, 14, (72,), 2),
              # float groups of 64-128 KB: 1024 threads x 8 loads, dy parked in LDS (fixed map)
              (2, 16, (64, 64), 2),
+             # planes of 8, 16 and 32 vectors with the group held on one CU in the backward:
+             # 2, 4 or 8 channels side by side in a wave's load
+             (4, 2560, (16, 16), 32), (2, 4096, (8, 16), 32), (4, 2048, (16, 8), 16),
+             (4, 2048, (8, 8), 16),
              # one group of 2M elements per sample: split streaming reductions
              (2, 32, (256, 256), 1), (1, 6, (333, 333), 2)]
 
