@@ -732,6 +732,7 @@ int launch_cl_fwd(const ClProblem &p, hipStream_t st) {
     int status = 0;
     if (cl_split_fwd(p, al, st, &status)) return status;
     if (gn_cl_cached_fwd(p, al, st, &status)) return status;
+    if (cl_tile_fwd(p, al, st, &status)) return status;
   }
   const BnPlan pl = make_cl_plan(p.batch, p.spatial, p.channels, p.dtype, al);
   const ClWs w = cl_carve(p, pl);
@@ -781,6 +782,13 @@ int launch_cl_bwd(const ClProblem &p, hipStream_t st) {
         return launch_pair_param_reduce("pair_param_reduce_cl_kernel", w.pairs, p.batch, p.channels,
                                         p.dgamma, p.dbeta, p.bc_gamma, p.bc_beta, p.accum_g,
                                         p.accum_b, st);
+      return 0;
+    }
+    if (cl_tile_bwd(p, al, &pairs, &pair_batches, st, &status)) {
+      if (status) return status;
+      if (p.dgamma || p.dbeta)
+        return launch_pair_param_reduce("pair_param_reduce_cl_kernel", pairs, pair_batches,
+                                        p.channels, p.dgamma, p.dbeta, 1, 1, p.accum_g, p.accum_b, st);
       return 0;
     }
   }

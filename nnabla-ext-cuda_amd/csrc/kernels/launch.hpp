@@ -233,6 +233,13 @@ constexpr int kClSplitMaxBlocks = 64; // blocks per (sample, column tile), i.e. 
 bool cl_split_fwd(const ClProblem &p, bool aligned, hipStream_t st, int *status);
 bool cl_split_bwd(const ClProblem &p, bool aligned, float **pairs, int64_t *pair_batches,
                   hipStream_t st, int *status);
+// Channel-last GroupNormalization with groups that are no whole number of
+// vectors (gn_cl_tile.hip): a block owns whole rows of a position range, the
+// blocks of a sample exchange per-group partial sums.  The backward leaves
+// per-block pairs in the workspace like cl_split_bwd.
+bool cl_tile_fwd(const ClProblem &p, bool aligned, hipStream_t st, int *status);
+bool cl_tile_bwd(const ClProblem &p, bool aligned, float **pairs, int64_t *pair_batches,
+                 hipStream_t st, int *status);
 int launch_cl_fwd(const ClProblem &p, hipStream_t st);
 int launch_cl_bwd(const ClProblem &p, hipStream_t st);
 size_t cl_workspace_bytes(int64_t batch, int64_t spatial, int64_t channels, int dtype);

@@ -54,7 +54,13 @@ GN_CL_SHAPES = [(2, (8, 8), 8, 4), (3, (5,), 6, 2), (1, (2, 2), 4, 1), (2, (4,),
                 (2, (56, 56), 64, 8), (9, (16, 16), 32, 4), (1, (90, 90), 8, 1),
                 # half data, 8 channels per group, a block for every CU left: blocks that
                 # take 2 or 4 neighbouring groups (ragged planes; the 1024 x 8 layout)
-                (4, (32, 32), 1024, 128), (8, (33, 33), 1024, 128), (16, (64, 64), 256, 32)]
+                (4, (32, 32), 1024, 128), (8, (33, 33), 1024, 128), (16, (64, 64), 256, 32),
+                # groups that are no whole number of vectors, a block per range of
+                # positions: 10, 20, 40, 80 and 6 channels per group, one to eleven
+                # vectors per thread, ragged position counts, 64 groups
+                (16, (16, 16), 320, 32), (8, (33, 31), 160, 16), (4, (40, 40), 640, 32),
+                (8, (48, 48), 320, 32), (16, (32, 32), 1280, 32), (16, (16, 16), 2560, 32),
+                (8, (32, 32), 192, 32), (4, (24, 24), 640, 64), (16, (61, 64), 320, 32)]
 
 
 @pytest.mark.parametrize("n,sp,c,groups", GN_CL_SHAPES)
@@ -138,7 +144,7 @@ def test_in_channel_last_per_sample_parameters_and_flags(n, sp, c, bcg, bcb):
     assert_close(to_np(db), db_r, "f32", "pgrad", "dbeta")
 
 
-@pytest.mark.parametrize("n,sp,c,groups", [(4, (16, 16), 64, 8), (2, (7, 7), 24, 8)])
+@pytest.mark.parametrize("n,sp,c,groups", [(4, (16, 16), 64, 8), (2, (7, 7), 24, 8), (8, (32, 32), 160, 16)])
 def test_gn_channel_last_flags(n, sp, c, groups):
     """no_scale/no_bias, 3-output dmean/dvar, accumulation, propagate_down."""
     rng = np.random.default_rng(5)

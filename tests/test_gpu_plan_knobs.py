@@ -229,6 +229,12 @@ SWITCHES = [
      ["in_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], ["cl_split_fwd_kernel", "cl_split_bwd_kernel"]),
     ("in_cl_split_off_float", run_in, (3, 64, (19, 19), F32, True), {"GN_CL_SPLIT_INSTANCES": 0},
      ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"], ["cl_split_fwd_kernel", "cl_split_bwd_kernel"]),
+    ("gn_cl_tile_off", run_gn, (8, 320, (48, 48), 32, F16, True), {"GN_CL_TILE": 0},
+     ["bn_stats_cl_kernel", "bn_bwd_reduce_cl_kernel"], ["gn_cl_tile_fwd_kernel", "gn_cl_tile_bwd_kernel"]),
+    ("gn_cl_tile_off_float", run_gn, (8, 160, (33, 31), 16, F32, True), {"GN_CL_TILE": 0},
+     ["bn_stats_cl_kernel", "bn_bwd_reduce_cl_kernel"], ["gn_cl_tile_fwd_kernel", "gn_cl_tile_bwd_kernel"]),
+    ("gn_cl_tile_min_pct_up", run_gn, (4, 640, (40, 40), 32, F16, True), {"GN_CL_TILE_MIN_PCT": 60},
+     ["bn_stats_cl_kernel", "bn_bwd_reduce_cl_kernel"], ["gn_cl_tile_fwd_kernel", "gn_cl_tile_bwd_kernel"]),
     ("gn_cl_wide_off", run_gn, (4, 1024, (32, 32), 128, F16, True),
      {"GN_CL_WIDE": 0, "GN_CL_WIDE_BWD": 0}, ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"],
      ["gn_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], NO_SPLIT),
@@ -237,7 +243,8 @@ SWITCHES = [
      ["in_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], NO_SPLIT),
     ("gn_cl_cached_off", run_gn, (2, 128, (20, 20), 8, F32, True), {"GN_CL_CACHED": 0},
      ["bn_stats_cl_kernel", "gn_cl_finalize_fwd_kernel", "bn_bwd_reduce_cl_kernel",
-      "gn_cl_finalize_bwd_kernel"], ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"], NO_SPLIT),
+      "gn_cl_finalize_bwd_kernel"], ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"],
+     {**NO_SPLIT, "GN_CL_TILE": 0}),
     ("in_cl_cached_off", run_in, (2, 128, (20, 20), F32, True), {"IN_CL_CACHED": 0},
      ["bn_stats_cl_kernel", "gn_cl_finalize_fwd_kernel", "gn_cl_finalize_bwd_kernel"],
      ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"], NO_SPLIT),
@@ -333,6 +340,12 @@ GRIDS = [
      ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], []),
     ("in_cl_split_no_polls", run_in, (2, 64, (30, 30), F32, True), [{"XCHG_SPIN": 0}],
      ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], []),
+    ("gn_cl_tile_no_polls", run_gn, (8, 320, (48, 48), 32, F16, True), [{"XCHG_SPIN": 0}],
+     ["gn_cl_tile_fwd_kernel", "gn_cl_tile_bwd_kernel"], []),
+    ("gn_cl_tile_no_polls_float", run_gn, (8, 160, (33, 31), 16, F32, True), [{"XCHG_SPIN": 0}],
+     ["gn_cl_tile_fwd_kernel", "gn_cl_tile_bwd_kernel"], []),
+    ("gn_cl_tile_few_blocks", run_gn, (1, 320, (16, 16), 32, F16, True), [{"GN_CL_TILE_MIN_PCT": 1}],
+     ["gn_cl_tile_fwd_kernel", "gn_cl_tile_bwd_kernel"], []),
     ("gn_cl_wide_plain_block_order", run_gn, (4, 1024, (32, 32), 128, F16, True),
      [{"GN_CL_XCD_MAP": 0, **NO_SPLIT}],
      ["gn_cl_wide_fwd_kernel", "cl_wide_bwd_kernel"], []),
