@@ -147,6 +147,14 @@ __device__ __forceinline__ void chan_exchange(const BnChanSplitArgs &a, uint32_t
   lds_barrier();
 }
 
+// The partners whose pair did not arrive, a bit each: every wave reads the
+// flags side by side (one LDS round trip, not one per partner) and gets the
+// same mask.  After chan_exchange's barrier.
+__device__ __forceinline__ uint64_t chan_missing(const BnChanSplitArgs &a, uint32_t sp, const int *miss) {
+  const uint32_t lane = threadIdx.x % kWave;
+  return __ballot(lane < a.SP && lane != sp && miss[lane] != 0);
+}
+
 } // namespace
 
 template <typename T, int VEC, int NR, int NS>
@@ -225,8 +233,9 @@ bn_chan_split_fwd_kernel(const BnChanSplitArgs a) {
 
   // ---- the partners' parts, the merge in block order (Chan), the statistics
   chan_exchange(a, c, sp, m, q, got, miss);
-  for (uint32_t p = 0; p < a.SP; ++p) {
-    if (p == sp || !miss[p]) continue; // same answer in every thread
+  const uint64_t late = chan_missing(a, sp, miss);
+  for (uint64_t todo = late; todo != 0; todo &= todo - 1) {
+    const uint32_t p = static_cast<uint32_t>(__builtin_ctzll(todo));
     float pm, pq;
     chan_part_from_memory<T, VEC>(a, c, p, red, pm, pq);
     if (t == 0) {
@@ -234,19 +243,25 @@ bn_chan_split_fwd_kernel(const BnChanSplitArgs a) {
       got[2 * p + 1] = pq;
     }
   }
-  lds_barrier();
+  if (late != 0) lds_barrier();
   if (t == 0) {
     const float per = static_cast<float>(a.vpp.d * VEC);
-    float mean = got[0], m2 = got[1], n = static_cast<float>(chan_block_samples(a, 0)) * per;
-    for (uint32_t p = 1; p < a.SP; ++p) {
-      const float nb = static_cast<float>(chan_block_samples(a, p)) * per;
+    float mean = 0.f, m2 = 0.f, n = 0.f;
+    for_pairs_in_order(got, 2, static_cast<int>(a.SP), [&](int p, float pm, float pq) {
+      const float nb = static_cast<float>(chan_block_samples(a, static_cast<uint32_t>(p))) * per;
+      if (p == 0) {
+        mean = pm;
+        m2 = pq;
+        n = nb;
+        return;
+      }
       const float tot = n + nb;
-      const float d = got[2 * p] - mean;
+      const float d = pm - mean;
       const float wgt = nb / tot;
       mean = fmaf(d, wgt, mean);
-      m2 = m2 + got[2 * p + 1] + d * d * (n * wgt);
+      m2 = m2 + pq + d * d * (n * wgt);
       n = tot;
-    }
+    });
     const float var = m2 * a.inv_N;
     fin[0] = mean;
     fin[1] = var;
@@ -409,8 +424,9 @@ bn_chan_split_bwd_kernel(const BnChanSplitArgs a) {
 
   // ---- the partners' parts, the totals in block order, dgamma / dbeta
   chan_exchange(a, c, sp, sdx, sdy, got, miss);
-  for (uint32_t p = 0; p < a.SP; ++p) {
-    if (p == sp || !miss[p]) continue; // same answer in every thread
+  const uint64_t late = chan_missing(a, sp, miss);
+  for (uint64_t todo = late; todo != 0; todo &= todo - 1) {
+    const uint32_t p = static_cast<uint32_t>(__builtin_ctzll(todo));
     float px, py;
     chan_pair_from_memory<T, VEC>(a, c, p, mean, istd, nmi, red, px, py);
     if (t == 0) {
@@ -418,13 +434,13 @@ bn_chan_split_bwd_kernel(const BnChanSplitArgs a) {
       got[2 * p + 1] = py;
     }
   }
-  lds_barrier();
+  if (late != 0) lds_barrier();
   if (t == 0) {
     float tx = 0.f, ty = 0.f;
-    for (uint32_t p = 0; p < a.SP; ++p) {
-      tx += got[2 * p];
-      ty += got[2 * p + 1];
-    }
+    for_pairs_in_order(got, 2, static_cast<int>(a.SP), [&](int, float px, float py) {
+      tx += px;
+      ty += py;
+    });
     fin[0] = tx;
     fin[1] = ty;
     if (sp == 0) {

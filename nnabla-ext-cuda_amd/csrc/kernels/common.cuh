@@ -618,4 +618,24 @@ __device__ __forceinline__ float inv_std(float var, float eps) {
   return 1.0f / sqrtf(var + eps);
 }
 
+// Calls f(i, lds[i * stride], lds[i * stride + 1]) for i = 0 .. n - 1 in order,
+// with the LDS reads of eight steps in flight together: a loop that reads as it
+// goes pays an LDS round trip per step (2 us for 16 partners' partial sums).
+template <typename F>
+__device__ __forceinline__ void for_pairs_in_order(const float *lds, int stride, int n, F f) {
+  for (int i0 = 0; i0 < n; i0 += 8) {
+    float v0[8], v1[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int idx = min(i0 + i, n - 1);
+      v0[i] = lds[idx * stride];
+      v1[i] = lds[idx * stride + 1];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (i0 + i < n) f(i0 + i, v0[i], v1[i]);
+    }
+  }
+}
+
 } // namespace nblahip

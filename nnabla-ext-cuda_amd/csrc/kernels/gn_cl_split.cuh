@@ -86,7 +86,8 @@ __device__ __forceinline__ void split_block_coords(const ClSplitArgs &a, uint32_
 // unit at a time, the first reads of up to four units in flight together: a
 // tile of an instance in 16 blocks of 256 threads has 1920 words to collect per
 // block, four round trips one after the other when polled unit by unit); words
-// that do not turn up mark their block in missing[].
+// that do not turn up mark their block in missing[] (and missing[kSplitMax]:
+// "any at all", the one flag a block reads when every word has arrived).
 template <int TPR>
 __device__ __forceinline__ void split_collect(const ClSplitArgs &a, const unsigned long long *base,
                                               uint32_t self, int per, float *part, int *missing) {
@@ -122,6 +123,7 @@ __device__ __forceinline__ void split_collect(const ClSplitArgs &a, const unsign
         part[idx + 1] = v1;
       } else {
         missing[idx / per] = 1;
+        missing[kSplitMax] = 1;
       }
     }
   }
@@ -233,17 +235,22 @@ __device__ __forceinline__ float split_count(const ClSplitArgs &a, int sp) {
 // order; counts follow from the geometry.  Returns mean, var (biased).
 __device__ __forceinline__ void split_merge_stats(const ClSplitArgs &a, const float *part, int per,
                                                   int u, float per_pos, float &mean, float &var) {
-  float m = part[u * 2], m2 = part[u * 2 + 1], n = split_count(a, 0) * per_pos;
-  for (int sp = 1; sp < a.split; ++sp) {
+  float m = 0.f, m2 = 0.f, n = 0.f;
+  for_pairs_in_order(part + u * 2, per, a.split, [&](int sp, float mb, float qb) {
     const float nb = split_count(a, sp) * per_pos;
-    const float mb = part[sp * per + u * 2], qb = part[sp * per + u * 2 + 1];
+    if (sp == 0) {
+      m = mb;
+      m2 = qb;
+      n = nb;
+      return;
+    }
     const float tot = n + nb;
     const float d = mb - m;
     const float wgt = nb / tot;
     m = fmaf(d, wgt, m);
     m2 = m2 + qb + d * d * (n * wgt);
     n = tot;
-  }
+  });
   mean = m;
   var = m2 * a.inv_R;
 }
@@ -351,7 +358,7 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
   extern __shared__ float part_many[]; // [split][2 * units of the tile], sized by the launch
   float *const part = MANY ? part_many : part16;
   __shared__ float merged[UMAX * 2]; // (mean, 1 / std) per unit
-  __shared__ int missing[kSplitMax];
+  __shared__ int missing[kSplitMax + 1];
   uint32_t tile, s, n;
   split_block_coords(a, blockIdx.x, tile, s, n);
   const uint32_t cvx = threadIdx.x % TV, prow = threadIdx.x / TV;
@@ -366,7 +373,7 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
       a.xchg + (static_cast<size_t>(n) * a.tiles + tile) * a.split * per;
   const bool writer = prow == 0 && (INSTANCE || (cvx & ((1u << a.cvg_shift) - 1)) == 0);
 
-  if (threadIdx.x < kSplitMax) missing[threadIdx.x] = 0;
+  if (threadIdx.x <= kSplitMax) missing[threadIdx.x] = 0;
   auto unit_index = [&]() -> size_t { // statistics index of unit threadIdx.x of the tile
     return INSTANCE ? static_cast<size_t>(n) * a.C + tile * TV * VEC + threadIdx.x
                     : static_cast<size_t>(n) * (a.C / a.cpg) + (tile * TV * VEC) / a.cpg + threadIdx.x;
@@ -403,7 +410,8 @@ cl_split_fwd_kernel(const ClSplitArgs a) {
   split_publish_own<TPR>(a, slots, s, per, part);
   split_collect<TPR>(a, slots, s, per, part, missing);
   lds_barrier();
-  for (int sp = 0; sp < a.split; ++sp) {
+  const bool any_missing = missing[kSplitMax] != 0; // (a flag per partner costs an LDS round trip each)
+  for (int sp = 0; any_missing && sp < a.split; ++sp) {
     if (sp == static_cast<int>(s) || !missing[sp]) continue; // same answer in every thread
     // Partner sp has not published: its part from global memory, one vector
     // at a time (the block's own vectors stay in registers).
@@ -547,7 +555,7 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
   float *const part = MANY ? part_many : part16;
   __shared__ float coef[UMAX * 2]; // (cA, cb) per unit
   __shared__ float gch[CH];        // gamma of the tile's channels
-  __shared__ int missing[kSplitMax];
+  __shared__ int missing[kSplitMax + 1];
   uint32_t tile, s, n;
   split_block_coords(a, blockIdx.x, tile, s, n);
   const uint32_t cvx = threadIdx.x % TV, prow = threadIdx.x / TV;
@@ -565,7 +573,7 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
   const size_t stat = INSTANCE ? static_cast<size_t>(n) * a.C + ch
                                : static_cast<size_t>(n) * (a.C / a.cpg) + ch0 / a.cpg + gi;
 
-  if (threadIdx.x < kSplitMax) missing[threadIdx.x] = 0;
+  if (threadIdx.x <= kSplitMax) missing[threadIdx.x] = 0;
   // Small loads first, so that they travel with the tensor's: the thread's
   // statistics, gamma of channel threadIdx.x of the tile, and what the thread
   // of unit threadIdx.x needs for the unit's coefficients.
@@ -655,7 +663,8 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
   // ---- the partners' parts
   split_collect<TPR>(a, slots, s, per, part, missing);
   lds_barrier();
-  for (int sp = 0; sp < a.split; ++sp) {
+  const bool any_missing = missing[kSplitMax] != 0; // (a flag per partner costs an LDS round trip each)
+  for (int sp = 0; any_missing && sp < a.split; ++sp) {
     if (sp == static_cast<int>(s) || !missing[sp]) continue; // same answer in every thread
     // Partner sp has not published: its sums from global memory, a vector at a time.
     split_pairs_from_memory<T, VEC, NL, TPR, INSTANCE, SV>(a, x, dy, sp, prow, cvx, mean, istd, nmi,
@@ -668,10 +677,10 @@ cl_split_bwd_kernel(const ClSplitArgs a) {
   if (unit_thread) {
     const int u = static_cast<int>(threadIdx.x);
     float t2 = 0.f, s1 = 0.f;
-    for (int sp = 0; sp < a.split; ++sp) {
-      t2 += part[sp * per + 2 * u];
-      s1 += part[sp * per + 2 * u + 1];
-    }
+    for_pairs_in_order(part + 2 * u, per, a.split, [&](int, float p0, float p1) {
+      t2 += p0;
+      s1 += p1;
+    });
     if constexpr (INSTANCE) { // the exchanged sums are per channel, without gamma
       t2 *= g_c;
       s1 *= g_c;

@@ -279,17 +279,23 @@ gn_cl_tile_fwd_kernel(const ClTileArgs a) {
   // ---- merge in block order (Chan; a thread per group), the statistics
   if (t < a.G) {
     const float cpg = static_cast<float>(a.cpgd.d);
-    float m = part[t * 2], m2 = part[t * 2 + 1], cnt = static_cast<float>(tile_positions(a, 0)) * cpg;
-    for (uint32_t sp = 1; sp < a.split; ++sp) {
-      const float nbp = static_cast<float>(tile_positions(a, sp)) * cpg;
-      const float mb = part[(sp * a.G + t) * 2], qb = part[(sp * a.G + t) * 2 + 1];
+    float m = 0.f, m2 = 0.f, cnt = 0.f;
+    for_pairs_in_order(part + t * 2, 2 * static_cast<int>(a.G), static_cast<int>(a.split),
+                       [&](int sp, float mb, float qb) {
+      const float nbp = static_cast<float>(tile_positions(a, static_cast<uint32_t>(sp))) * cpg;
+      if (sp == 0) {
+        m = mb;
+        m2 = qb;
+        cnt = nbp;
+        return;
+      }
       const float total = cnt + nbp;
       const float d = mb - m;
       const float wgt = nbp / total;
       m = fmaf(d, wgt, m);
       m2 = m2 + qb + d * d * (cnt * wgt);
       cnt = total;
-    }
+    });
     const float var = m2 * a.inv_R;
     merged[2 * t] = m;
     merged[2 * t + 1] = inv_std(var, a.eps);
@@ -505,10 +511,11 @@ gn_cl_tile_bwd_kernel(const ClTileArgs a) {
   // ---- totals in block order and the group's coefficients (a thread per group)
   if (t < a.G) {
     float t2 = 0.f, s1 = 0.f;
-    for (uint32_t sp = 0; sp < a.split; ++sp) {
-      t2 += part[(sp * a.G + t) * 2];
-      s1 += part[(sp * a.G + t) * 2 + 1];
-    }
+    for_pairs_in_order(part + t * 2, 2 * static_cast<int>(a.G), static_cast<int>(a.split),
+                       [&](int, float q0, float q1) {
+      t2 += q0;
+      s1 += q1;
+    });
     const float vpe = u_var + a.eps;
     const float is = 1.0f / sqrtf(vpe);
     coef[2 * t] = -is * t2 * a.inv_R + (a.dvar ? 2.f * u_dvar * (vpe * is) * a.inv_R : 0.f);
