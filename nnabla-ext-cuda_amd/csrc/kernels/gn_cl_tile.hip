@@ -47,6 +47,7 @@ struct ClTileArgs {
   FastDiv cvd;     // (the same, for t -> (position, vector))
   FastDiv cpgd;    // channels per group, for channel -> group
   FastDiv gd;      // groups, for exchange word -> block
+  FastDiv rpid;    // positions per sweep, for positions -> rows that hold one more
   uint32_t rpi;    // positions per sweep = 1024 / cv
   uint32_t active; // threads that own a vector = rpi * cv
   uint32_t split;  // blocks per sample
@@ -89,19 +90,90 @@ __device__ __forceinline__ float tile_column(const ClTileArgs &a, const float *c
   return (s0 + s1) + (s2 + s3);
 }
 
-// Forward: per-group totals of the threads' per-element values, a wave per
-// group (a lane per column, then across the lanes).  Ends with a barrier.
+// Forward: (mean, m2) per group from the threads' per-element (mean, m2) over
+// their positions, in one trip through LDS.  A thread per column merges the
+// rows of the sweep (row r holds full + (r < rem) positions) into the column's
+// mean and m2 and leaves them in row 0 of its column (nobody else reads that
+// column); a wave per group merges the group's columns - equal counts, so the
+// group's mean is the mean of the columns' means and its m2 the sum of theirs
+// plus npos * sum (mean_c - mean)^2 - across its lanes.  Nothing is squared
+// before its mean is taken off.  tot: [G][2].  Ends with a barrier.
+constexpr int kTileColsPerLane = 2; // columns of a group a lane takes: groups of up to 128 channels
+
 template <int VEC>
-__device__ __forceinline__ void tile_group_sums(const float (&v)[VEC], const ClTileArgs &a,
-                                                bool owner, float *cols, float *tot) {
-  tile_put_cols<VEC>(v, a, owner, cols);
-  const uint32_t wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+__device__ __forceinline__ void tile_group_stats(const float (&mu)[VEC], const float (&m2)[VEC],
+                                                 const ClTileArgs &a, uint32_t npos, float *cmu,
+                                                 float *cm2, float *tot) {
+  const uint32_t t = threadIdx.x;
+  lds_barrier(); // earlier readers of cmu / cm2 / tot are done
+  if (t < a.active) {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      cmu[t * VEC + j] = mu[j]; // (threads without a position: zeros, and their rows count nothing)
+      cm2[t * VEC + j] = m2[j];
+    }
+  }
+  lds_barrier();
+  const uint32_t full = a.rpid.div(npos), rem = npos - full * a.rpi;
+  const float fn = static_cast<float>(npos);
+  const float inv_n = 1.0f / fn;
+  auto rows = [&](uint32_t r) { return static_cast<float>(full + (r < rem ? 1u : 0u)); };
+  for (uint32_t c = t; c < a.C; c += kOnchipBlock) {
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    uint32_t r = 0;
+    for (; r + 4 <= a.rpi; r += 4) {
+      s0 = fmaf(rows(r), cmu[r * a.C + c], s0);
+      s1 = fmaf(rows(r + 1), cmu[(r + 1) * a.C + c], s1);
+      s2 = fmaf(rows(r + 2), cmu[(r + 2) * a.C + c], s2);
+      s3 = fmaf(rows(r + 3), cmu[(r + 3) * a.C + c], s3);
+    }
+    for (; r < a.rpi; ++r) s0 = fmaf(rows(r), cmu[r * a.C + c], s0);
+    const float mc = ((s0 + s1) + (s2 + s3)) * inv_n;
+    float q0 = 0.f, q1 = 0.f, q2 = 0.f, q3 = 0.f;
+    for (r = 0; r + 4 <= a.rpi; r += 4) {
+      const float e0 = cmu[r * a.C + c] - mc, e1 = cmu[(r + 1) * a.C + c] - mc;
+      const float e2 = cmu[(r + 2) * a.C + c] - mc, e3 = cmu[(r + 3) * a.C + c] - mc;
+      q0 = fmaf(rows(r) * e0, e0, q0 + cm2[r * a.C + c]);
+      q1 = fmaf(rows(r + 1) * e1, e1, q1 + cm2[(r + 1) * a.C + c]);
+      q2 = fmaf(rows(r + 2) * e2, e2, q2 + cm2[(r + 2) * a.C + c]);
+      q3 = fmaf(rows(r + 3) * e3, e3, q3 + cm2[(r + 3) * a.C + c]);
+    }
+    for (; r < a.rpi; ++r) {
+      const float e0 = cmu[r * a.C + c] - mc;
+      q0 = fmaf(rows(r) * e0, e0, q0 + cm2[r * a.C + c]);
+    }
+    cmu[c] = mc;
+    cm2[c] = (q0 + q1) + (q2 + q3);
+  }
+  lds_barrier();
+  const uint32_t wave = t / kWave, lane = t % kWave;
   const uint32_t cpg = a.cpgd.d;
+  const float inv_cpg = 1.0f / static_cast<float>(cpg);
   for (uint32_t g = wave; g < a.G; g += kOnchipBlock / kWave) {
-    float s = 0.f;
-    for (uint32_t i = lane; i < cpg; i += kWave) s += tile_column(a, cols, g * cpg + i);
-    s = wave_sum(s);
-    if (lane == 0) tot[g] = s;
+    float cmean[kTileColsPerLane], cq[kTileColsPerLane];
+    float lane_means = 0.f;
+#pragma unroll
+    for (int q = 0; q < kTileColsPerLane; ++q) {
+      const uint32_t i = lane + q * kWave;
+      const bool has = i < cpg;
+      cmean[q] = has ? cmu[g * cpg + i] : 0.f;
+      cq[q] = has ? cm2[g * cpg + i] : 0.f;
+      lane_means += cmean[q];
+    }
+    const float mean_g = wave_sum(lane_means) * inv_cpg;
+    float lane_q = 0.f;
+#pragma unroll
+    for (int q = 0; q < kTileColsPerLane; ++q) {
+      if (lane + q * kWave < cpg) {
+        const float e = cmean[q] - mean_g;
+        lane_q += fmaf(fn * e, e, cq[q]);
+      }
+    }
+    lane_q = wave_sum(lane_q);
+    if (lane == 0) {
+      tot[2 * g] = mean_g;
+      tot[2 * g + 1] = lane_q;
+    }
   }
   lds_barrier();
 }
@@ -146,8 +218,8 @@ gn_cl_tile_fwd_kernel(const ClTileArgs a) {
   static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors");
   constexpr int NL = NR + NS;
   __shared__ uint4 spill[NS > 0 ? NS * kOnchipBlock : 1];
-  __shared__ float cols[kOnchipBlock * VEC];
-  __shared__ float tot[kTileMaxG];
+  __shared__ float cmu[kOnchipBlock * VEC], cm2[kOnchipBlock * VEC];
+  __shared__ float tot[2 * kTileMaxG];
   __shared__ float part[kTileMaxSplit * 2 * kTileMaxG];
   __shared__ float merged[2 * kTileMaxG]; // (mean, 1 / std) per group
   __shared__ float gch[kTileMaxC], bch[kTileMaxC];
@@ -238,20 +310,9 @@ gn_cl_tile_fwd_kernel(const ClTileArgs a) {
 #pragma unroll 1
       for (int k = 0; k < nk; ++k) take(k);
     }
-    const float nt = static_cast<float>(nk);
-    float val[VEC];
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) val[j] = nt * mu_t[j];
-    tile_group_sums<VEC>(val, a, nk > 0, cols, tot);
-    const float icnt = 1.0f / (static_cast<float>(npos) * static_cast<float>(a.cpgd.d));
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      const float e = mu_t[j] - tot[a.cpgd.div(ch + j)] * icnt;
-      val[j] = fmaf(nt * e, e, m2[j]);
-    }
-    pm = t < a.G ? tot[t] * icnt : 0.f;
-    tile_group_sums<VEC>(val, a, nk > 0, cols, tot);
-    pq = t < a.G ? tot[t] : 0.f;
+    tile_group_stats<VEC>(mu_t, m2, a, npos, cmu, cm2, tot);
+    pm = t < a.G ? tot[2 * t] : 0.f;
+    pq = t < a.G ? tot[2 * t + 1] : 0.f;
   };
 
   // ---- this block's part, published; the partners' parts
@@ -583,7 +644,7 @@ TilePlan plan_tile(const ClProblem &p, bool aligned, int max_nl) {
   if (!p.bc_gamma || !p.bc_beta || p.groups == p.channels) return pl;
   const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
   if (p.channels % vec != 0 || p.channels > kTileMaxC || p.groups > kTileMaxG) return pl;
-  if (p.channels % p.groups != 0) return pl;
+  if (p.channels % p.groups != 0 || p.channels / p.groups > kTileColsPerLane * kWave) return pl;
   const int64_t cv = p.channels / vec;
   if (cv > 512) return pl;
   const int64_t rpi = kOnchipBlock / cv;
@@ -630,6 +691,7 @@ ClTileArgs tile_args(const ClProblem &p, const TilePlan &pl) {
   a.cvd = FastDiv(pl.cv);
   a.cpgd = FastDiv(static_cast<uint32_t>(p.channels / p.groups));
   a.gd = FastDiv(static_cast<uint32_t>(p.groups));
+  a.rpid = FastDiv(pl.rpi);
   a.rpi = pl.rpi;
   a.active = pl.rpi * pl.cv;
   a.split = pl.split;
@@ -641,13 +703,14 @@ ClTileArgs tile_args(const ClProblem &p, const TilePlan &pl) {
   return a;
 }
 
-// Vectors per thread the forward holds: 11 (half: the per-element scale and
-// shift take 16 registers more than float's) or 16 in registers, 5 in LDS.
+// Vectors per thread the forward holds: 13 (half: the per-element scale and
+// shift take 16 registers more than float's) or 16 in registers, 3 (half: its
+// per-element statistics take 64 KB of LDS on their way to the groups) or 5 in LDS.
 constexpr int tile_fwd_max(int dtype) { return dtype == NBLAHIP_F16 ? 16 : 21; }
 
 template <typename T, int VEC>
 int run_tile_fwd(int nl, const ClTileArgs &a, unsigned grid, hipStream_t st) {
-  constexpr int kTop = sizeof(T) == 2 ? 11 : 16;
+  constexpr int kTop = sizeof(T) == 2 ? 13 : 16;
 #define TILE_CASE(NR, NS)                                                                        \
   if (nl <= (NR) + (NS)) {                                                                       \
     NBLAHIP_LAUNCH("gn_cl_tile_fwd_kernel", (gn_cl_tile_fwd_kernel<T, VEC, NR, NS>), dim3(grid), \
@@ -659,10 +722,16 @@ int run_tile_fwd(int nl, const ClTileArgs &a, unsigned grid, hipStream_t st) {
   TILE_CASE(9, 0)
   if constexpr (sizeof(T) == 4) {
     TILE_CASE(12, 0)
+  } else {
+    TILE_CASE(11, 0)
   }
   TILE_CASE(kTop, 0)
   TILE_CASE(kTop, 2)
-  TILE_CASE(kTop, 5)
+  if constexpr (sizeof(T) == 2) {
+    TILE_CASE(kTop, 3)
+  } else {
+    TILE_CASE(kTop, 5)
+  }
 #undef TILE_CASE
   return NBLAHIP_EINVAL;
 }
