@@ -36,7 +36,8 @@ namespace nblahip {
 namespace {
 
 constexpr int kGridMaxBlocks = 256; // partials per channel a block merges (one per thread of a wave quad)
-constexpr int kGridMaxC = 128;      // channels (LDS fold of the per-channel sums)
+constexpr int kGridMaxC = 128;      // channels (LDS fold of the per-channel sums) of the layouts that hold most
+constexpr int kGridWideC = 512;     // channels of the layouts with three LDS slots fewer
 
 struct BnClGridArgs {
   const void *x;
@@ -276,19 +277,19 @@ __device__ __forceinline__ void grid_pair_result(const BnClGridArgs &a, uint32_t
 
 } // namespace
 
-template <typename T, int VEC, int NR, int NS>
+template <typename T, int VEC, int NR, int NS, int CMAX>
 __global__ void __launch_bounds__(kOnchipBlock)
 bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
   static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors");
   constexpr int NL = NR + NS;
   __shared__ uint4 spill[NS > 0 ? NS * kOnchipBlock : 1];
-  __shared__ float fold[16 * kGridMaxC];
-  __shared__ float tot[kGridMaxC];
-  __shared__ float fin[2 * kGridMaxC];   // (mean, var) per channel
+  __shared__ float fold[16 * CMAX];
+  __shared__ float tot[CMAX];
+  __shared__ float fin[2 * CMAX];   // (mean, var) per channel
   __shared__ float got[2 * kGridMaxBlocks];
   __shared__ int miss[kGridMaxBlocks + 2]; // [kGridMaxBlocks], [+1]: any partial / any result missing
   __shared__ float wel[3 * 16];
-  __shared__ float gb[2 * kGridMaxC]; // gamma, beta
+  __shared__ float gb[2 * CMAX]; // gamma, beta
   const uint32_t b = blockIdx.x;
   const uint32_t t = threadIdx.x;
   // gamma and beta of channel t, asked for ahead of the tensor (behind the
@@ -322,7 +323,7 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
     }
     if (t < a.C) { // (they arrive first; read behind the barriers of the folds)
       gb[t] = gamma_t;
-      gb[kGridMaxC + t] = beta_t;
+      gb[CMAX + t] = beta_t;
     }
 #pragma unroll
     for (int k = 0; k < NS; ++k) spill[k * kOnchipBlock + t] = __builtin_bit_cast(uint4, parked[k]);
@@ -447,7 +448,7 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
   for (int j = 0; j < VEC; ++j) {
     mu[j] = fin[2 * (ch + j)];
     sc[j] = gb[ch + j] * inv_std(fin[2 * (ch + j) + 1], a.eps);
-    be[j] = gb[kGridMaxC + ch + j];
+    be[j] = gb[CMAX + ch + j];
     sh[j] = fmaf(-mu[j], sc[j], be[j]);
   }
   const uint32_t t2 = fresh(t);
@@ -478,20 +479,20 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
 // beyond that is streamed with dy in both passes), dy is streamed twice in
 // batches of B vectors; the blocks exchange (sdx, sdy) per channel in the
 // forward's two stages, block c writing dgamma[c] / dbeta[c].
-template <typename T, int VEC, int NR, int NS, int B>
+template <typename T, int VEC, int NR, int NS, int B, int CMAX>
 __global__ void __launch_bounds__(kOnchipBlock)
 bn_cl_grid_bwd_kernel(const BnClGridArgs a) {
   static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors");
   constexpr int NL = NR + NS;
   __shared__ uint4 spill[NS > 0 ? NS * kOnchipBlock : 1];
-  __shared__ float fold[16 * kGridMaxC];
-  __shared__ float tot[kGridMaxC];
-  __shared__ float fin[2 * kGridMaxC]; // (sdx, sdy) totals per channel
-  __shared__ int finmiss[kGridMaxC];
+  __shared__ float fold[16 * CMAX];
+  __shared__ float tot[CMAX];
+  __shared__ float fin[2 * CMAX]; // (sdx, sdy) totals per channel
+  __shared__ int finmiss[CMAX];
   __shared__ float got[2 * kGridMaxBlocks];
   __shared__ int miss[kGridMaxBlocks + 2];
   __shared__ float wel[16];
-  __shared__ float par[5 * kGridMaxC]; // mean, var, gamma, dvar, dmean
+  __shared__ float par[5 * CMAX]; // mean, var, gamma, dvar, dmean
   const uint32_t b = blockIdx.x;
   const uint32_t t = threadIdx.x;
   // The parameters of channel t, asked for ahead of the tensor: behind the LDS
@@ -536,17 +537,17 @@ bn_cl_grid_bwd_kernel(const BnClGridArgs a) {
   };
   if (t < a.C) {
     par[t] = p_mean;
-    par[kGridMaxC + t] = p_var;
-    par[2 * kGridMaxC + t] = p_gamma;
-    par[3 * kGridMaxC + t] = p_dvar;
-    par[4 * kGridMaxC + t] = p_dmean;
+    par[CMAX + t] = p_var;
+    par[2 * CMAX + t] = p_gamma;
+    par[3 * CMAX + t] = p_dvar;
+    par[4 * CMAX + t] = p_dmean;
   }
   lds_barrier();
   float mean[VEC], istd[VEC], nmi[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
     mean[j] = par[ch + j];
-    istd[j] = 1.0f / sqrtf(par[kGridMaxC + ch + j] + a.eps);
+    istd[j] = 1.0f / sqrtf(par[CMAX + ch + j] + a.eps);
     nmi[j] = -mean[j] * istd[j];
   }
 
@@ -646,12 +647,12 @@ bn_cl_grid_bwd_kernel(const BnClGridArgs a) {
   float gi[VEC], A2[VEC], B2[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
-    const float g = par[2 * kGridMaxC + ch + j];
-    const float vpe = par[kGridMaxC + ch + j] + a.eps;
+    const float g = par[2 * CMAX + ch + j];
+    const float vpe = par[CMAX + ch + j] + a.eps;
     const float cA = -istd[j] * g * fin[2 * (ch + j)] * a.inv_N +
-                     (a.dvar ? 2.f * par[3 * kGridMaxC + ch + j] * (vpe * istd[j]) * a.inv_N : 0.f);
+                     (a.dvar ? 2.f * par[3 * CMAX + ch + j] * (vpe * istd[j]) * a.inv_N : 0.f);
     const float cb = -g * fin[2 * (ch + j) + 1] * istd[j] * a.inv_N +
-                     (a.dmean ? par[4 * kGridMaxC + ch + j] * a.inv_N : 0.f);
+                     (a.dmean ? par[4 * CMAX + ch + j] * a.inv_N : 0.f);
     gi[j] = g * istd[j];
     A2[j] = istd[j] * cA;
     B2[j] = sizeof(T) == 2 ? fmaf(nmi[j], cA, cb) : cb;
@@ -710,19 +711,28 @@ namespace {
 
 template <typename T, int VEC>
 int run_grid_fwd(int nl, const BnClGridArgs &a, hipStream_t st) {
-#define GRID_CASE(NR, NS)                                                                        \
+#define GRID_CASE(NR, NS, CMAX)                                                                  \
   if (nl <= (NR) + (NS)) {                                                                       \
-    NBLAHIP_LAUNCH("bn_cl_grid_fwd_kernel", (bn_cl_grid_fwd_kernel<T, VEC, NR, NS>),             \
+    NBLAHIP_LAUNCH("bn_cl_grid_fwd_kernel", (bn_cl_grid_fwd_kernel<T, VEC, NR, NS, CMAX>),       \
                    dim3(a.nblocks), dim3(kOnchipBlock), 0, st, a);                               \
     return last_launch_status();                                                                 \
   }
-  GRID_CASE(4, 0)
-  GRID_CASE(8, 0)
-  GRID_CASE(12, 0)
-  GRID_CASE(16, 0)
-  GRID_CASE(16, 3)
-  GRID_CASE(16, 6)
-  GRID_CASE(16, 9)
+  if (a.C <= static_cast<uint32_t>(kGridMaxC)) {
+    GRID_CASE(4, 0, kGridMaxC)
+    GRID_CASE(8, 0, kGridMaxC)
+    GRID_CASE(12, 0, kGridMaxC)
+    GRID_CASE(16, 0, kGridMaxC)
+    GRID_CASE(16, 3, kGridMaxC)
+    GRID_CASE(16, 6, kGridMaxC)
+    GRID_CASE(16, 9, kGridMaxC)
+  } else { // the per-channel arrays take 32 KB more of LDS
+    GRID_CASE(4, 0, kGridWideC)
+    GRID_CASE(8, 0, kGridWideC)
+    GRID_CASE(12, 0, kGridWideC)
+    GRID_CASE(16, 0, kGridWideC)
+    GRID_CASE(16, 3, kGridWideC)
+    GRID_CASE(16, 6, kGridWideC)
+  }
 #undef GRID_CASE
   return NBLAHIP_EINVAL;
 }
@@ -733,23 +743,31 @@ namespace {
 
 template <typename T, int VEC>
 int run_grid_bwd(int nl, const BnClGridArgs &a, hipStream_t st) {
-#define GRID_CASE(NR, NS)                                                                        \
+  constexpr int B = sizeof(T) == 2 ? 2 : 4;
+#define GRID_CASE(NR, NS, CMAX)                                                                  \
   if (nl <= (NR) + (NS)) {                                                                       \
-    NBLAHIP_LAUNCH("bn_cl_grid_bwd_kernel", (bn_cl_grid_bwd_kernel<T, VEC, NR, NS, (sizeof(T) == 2 ? 2 : 4)>),          \
+    constexpr int kNS = (NS) > 9 ? ((CMAX) > kGridMaxC ? 6 : 9) : (NS);                          \
+    NBLAHIP_LAUNCH("bn_cl_grid_bwd_kernel", (bn_cl_grid_bwd_kernel<T, VEC, NR, kNS, B, CMAX>),   \
                    dim3(a.nblocks), dim3(kOnchipBlock), 0, st, a);                               \
     return last_launch_status();                                                                 \
   }
-  GRID_CASE(4, 0)
-  GRID_CASE(8, 0)
-  GRID_CASE(12, 0)
-  GRID_CASE(12, 3)
-  GRID_CASE(12, 6)
-  GRID_CASE(12, 9)
+  if (a.C <= static_cast<uint32_t>(kGridMaxC)) {
+    GRID_CASE(4, 0, kGridMaxC)
+    GRID_CASE(8, 0, kGridMaxC)
+    GRID_CASE(12, 0, kGridMaxC)
+    GRID_CASE(12, 3, kGridMaxC)
+    GRID_CASE(12, 6, kGridMaxC)
+    // (more per thread than the 21 vectors held: the rest is streamed with dy)
+    GRID_CASE(12, 1 << 20, kGridMaxC)
+  } else {
+    GRID_CASE(4, 0, kGridWideC)
+    GRID_CASE(8, 0, kGridWideC)
+    GRID_CASE(12, 0, kGridWideC)
+    GRID_CASE(12, 3, kGridWideC)
+    GRID_CASE(12, 1 << 20, kGridWideC)
+  }
 #undef GRID_CASE
-  // more per thread than the 21 vectors held: the rest is streamed with dy
-  NBLAHIP_LAUNCH("bn_cl_grid_bwd_kernel", (bn_cl_grid_bwd_kernel<T, VEC, 12, 9, (sizeof(T) == 2 ? 2 : 4)>),
-                 dim3(a.nblocks), dim3(kOnchipBlock), 0, st, a);
-  return last_launch_status();
+  return NBLAHIP_EINVAL;
 }
 
 // Shape test and the arguments both directions share; nl = vectors per thread.
@@ -757,7 +775,13 @@ bool grid_args(const BnProblem &p, BnClGridArgs &a, int &nl) {
   if (!tune_int("BN_CL_GRID", 1)) return false;
   if (p.size2 != 1 || p.relu || p.z || p.y || p.dz || p.sums_out || p.sums_in) return false;
   const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
-  if (p.C % vec != 0 || p.C > kGridMaxC || !aligned16(p.x) || (p.out && !aligned16(p.out))) return false;
+  if (p.C % vec != 0 || p.C > kGridWideC || !aligned16(p.x) || (p.out && !aligned16(p.out))) return false;
+  // 129 - 512 channels: from the rows on that the split kernels' backward no
+  // longer holds (36 blocks of 1024 rows); below, those take both directions
+  // ([128,14,14,512] half 17.8 / 20.0 us against 23.6 / 30.5 us here).
+  if (p.C > kGridMaxC &&
+      (!tune_int("BN_CL_GRID_WIDE", 1) || p.size0 < tune_int("BN_CL_GRID_WIDE_MIN_ROWS", 36865)))
+    return false;
   const int64_t cv = p.C / vec;
   if ((cv & (cv - 1)) != 0 || cv > kWave) return false;
   const int64_t M = p.size0;
@@ -804,6 +828,7 @@ bool bn_cl_grid_fwd_train(const BnProblem &p, hipStream_t st, int *status) {
   BnClGridArgs a;
   int nl = 0;
   if (!p.out || !grid_args(p, a, nl)) return false;
+  if (p.C > kGridMaxC && nl > 22) return false; // (the wide layouts hold 16 + 6 vectors)
   a.y = p.out;
   a.beta = p.beta;
   a.mean = p.batch_mean;

@@ -422,7 +422,10 @@ def test_bn_training_forward_in_place(shape, axis, dtype):
 # per-channel partials exchanged between the blocks.
 @pytest.mark.parametrize("m,c,dtype", [(100352, 64, torch.float16), (100353, 64, torch.float16),
                                        (200000, 32, torch.float32), (150000, 128, torch.float16),
-                                       (1000001, 8, torch.float16), (40000, 128, torch.float32)])
+                                       (1000001, 8, torch.float16), (40000, 128, torch.float32),
+                                       # 256 and 512 channels: a block merges one or two channels
+                                       (40000, 256, torch.float16), (50000, 512, torch.float16),
+                                       (40000, 256, torch.float32)])
 def test_bn_channel_last_held_on_the_chip(m, c, dtype):
     """Against the oracle; bit-identical when no poll is allowed (every block
     then computes the partials and channel results it needs itself); close to
@@ -470,7 +473,10 @@ def test_bn_channel_last_held_on_the_chip(m, c, dtype):
                                        (200000, 32, torch.float32), (150000, 128, torch.float16),
                                        (1000001, 8, torch.float16), (40000, 128, torch.float32),
                                        # more of x than a block holds: the rest is read again
-                                       (750000, 64, torch.float16), (380000, 64, torch.float32)])
+                                       (750000, 64, torch.float16), (380000, 64, torch.float32),
+                                       # 256 and 512 channels; more than the 18 vectors held with them
+                                       (40000, 256, torch.float16), (50000, 512, torch.float16),
+                                       (40000, 256, torch.float32), (170000, 256, torch.float16)])
 def test_bn_channel_last_backward_held_on_the_chip(m, c, dtype):
     """Backward with x held on the chip and the (sum dy*xh, sum dy) pairs
     exchanged: against the oracle with the 3-output terms, bit-identical when no

@@ -179,6 +179,10 @@ SWITCHES = [
      {"BN_CL_GRID_MIN_SLOTS": 1}),
     ("bn_cl_grid_from_fewer_vectors", run_bn, ((100352, 64), 1, F16), {"BN_CL_GRID_MIN_SLOTS": 1},
      ["bn_cl_grid_fwd_kernel"], ["bn_stats_cl_kernel"]),
+    ("bn_cl_grid_wide_off", run_bn, ((256, 14, 14, 256), 3, F16), {"BN_CL_GRID_WIDE": 0},
+     ["cl_split_fwd_kernel", "bn_bwd_reduce_cl_kernel"], ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"]),
+    ("bn_cl_grid_wide_from_more_rows", run_bn, ((256, 14, 14, 256), 3, F32), {"BN_CL_GRID_WIDE_MIN_ROWS": 60000},
+     ["bn_stats_cl_kernel", "bn_bwd_reduce_cl_kernel"], ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"]),
     ("bn_cl_grid_bwd_off", run_bn, ((100352, 64), 1, F16), {"BN_CL_GRID_BWD": 0},
      ["bn_cl_grid_fwd_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
      ["bn_cl_grid_bwd_kernel"], {"BN_CL_GRID_MIN_SLOTS": 1}),
@@ -291,6 +295,8 @@ GRIDS = [
        "BN_CL_SPLIT": 0} for a, b, c in ((1, 1, 1), (2, 4, 2), (8, 3, 7))],
      ["bn_stats_cl_kernel", "bn_apply_cl_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
      []),
+    ("bn_cl_grid_wide_fewer_rows", run_bn, ((128, 14, 14, 512), 3, F16), [{"BN_CL_GRID_WIDE_MIN_ROWS": 1}],
+     ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"], []),
     ("bn_onchip_few_channels", run_bn, ((32, 4, 56, 56), 1, F16),
      [{"BN_ONCHIP_FWD_MIN_PCT": 1, "BN_ONCHIP_BWD_MIN_PCT": 1}],
      ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
