@@ -659,7 +659,7 @@ TilePlan plan_tile(const ClProblem &p, bool aligned, int max_nl) {
   if (split > kTileMaxSplit || nl_of(split) > max_nl) return pl;
   const int64_t pb = (p.spatial + split - 1) / split;
   split = (p.spatial + pb - 1) / pb; // every block holds a position
-  if (p.batch * split * 100 < cus * tune_int("GN_CL_TILE_MIN_PCT", 10)) return pl;
+  if (p.batch * split * 100 < cus * tune_int("GN_CL_TILE_MIN_PCT", 1)) return pl;
   // Partners wait for each other: a block per CU at most, all there at once.
   if (p.batch * split > cus) return pl;
   if (static_cast<size_t>(p.batch) * split * 2 * p.groups > xchg_capacity()) return pl;

@@ -350,7 +350,7 @@ GRIDS = [
      ["gn_cl_tile_fwd_kernel", "gn_cl_tile_bwd_kernel"], []),
     ("gn_cl_tile_no_polls_float", run_gn, (8, 160, (33, 31), 16, F32, True), [{"XCHG_SPIN": 0}],
      ["gn_cl_tile_fwd_kernel", "gn_cl_tile_bwd_kernel"], []),
-    ("gn_cl_tile_few_blocks", run_gn, (1, 320, (16, 16), 32, F16, True), [{"GN_CL_TILE_MIN_PCT": 1}],
+    ("gn_cl_tile_few_blocks", run_gn, (1, 320, (6, 6), 32, F16, True), [{"GN_CL_TILE_MIN_PCT": 0}],
      ["gn_cl_tile_fwd_kernel", "gn_cl_tile_bwd_kernel"], []),
     ("gn_cl_wide_plain_block_order", run_gn, (4, 1024, (32, 32), 128, F16, True),
      [{"GN_CL_XCD_MAP": 0, **NO_SPLIT}],
