@@ -13,6 +13,10 @@ int run_row_fwd_cached(int dtype, const RowCfg &cfg, const RowArgs &args, int gr
 // A row of up to 400 KB held on one CU (registers + LDS), GroupNormalization and
 // InstanceNormalization forward; false: not taken.
 bool row_onchip_fwd(const RowProblem &p, const RowArgs &args, int vec, hipStream_t st, int *status);
+// InstanceNormalization planes that are no whole number of 16-byte vectors, with
+// 16-byte loads over the tensor's aligned vectors; false: not taken.
+bool row_masked_fwd(const RowProblem &p, hipStream_t st, int *status);
+bool row_masked_bwd(const RowProblem &p, hipStream_t st, int *status); // the pairs to p.ws
 int run_row_bwd_cached_ln(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
                           hipStream_t st);
 // Resident blocks per CU of the LayerNormalization backward kernel for cfg

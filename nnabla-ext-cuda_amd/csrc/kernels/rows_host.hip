@@ -262,6 +262,7 @@ static int stream_fwd_t(const RowProblem &p, const RowArgs &a, hipStream_t st) {
 }
 
 int launch_row_fwd(const RowProblem &p, hipStream_t st) {
+  if (int status = 0; !tune_int("FORCE_STREAM", 0) && row_masked_fwd(p, st, &status)) return status;
   const int vec = row_vec(p, false);
   const RowArgs a = make_args(p);
   // LayerNormalization keeps gamma/beta of its columns in registers too: with
@@ -426,6 +427,8 @@ static int launch_pair_reduce(const RowProblem &p, const float *pairs, hipStream
 
 int launch_row_bwd(const RowProblem &p, hipStream_t st) {
   if (!p.out && !p.dgamma && !p.dbeta) return 0;
+  if (int status = 0; !tune_int("FORCE_STREAM", 0) && row_masked_bwd(p, st, &status))
+    return status ? status : launch_pair_reduce(p, static_cast<const float *>(p.ws), st);
   const int vec = row_vec(p, true);
   RowArgs a = make_args(p);
   // LayerNormalization also keeps per-column accumulators, gamma and the

@@ -238,7 +238,11 @@ IN_SHAPES = [(2, 3, (4, 4)), (3, 5, (7,)), (1, 2, (3, 2)), (4, 16, (16, 16)), (2
              (4, 8, (14, 14)), (2, 3, (6, 6)), (2, 300, (14, 14)), (3, 2, (90, 90)),
              (8, 64, (8, 8)), (5, 33, (7, 7)), (3, 300, (4, 4)), (2, 129, (3, 5)), (7, 11, (6,)),
              # a few very long rows: split streaming reductions
-             (2, 4, (64, 64, 64)), (1, 2, (999, 1001))]
+             (2, 4, (64, 64, 64)), (1, 2, (999, 1001)),
+             # planes that are no whole number of vectors, taken with the tensor's aligned
+             # vectors: one wave to 1024 threads per row, a tensor that ends inside a vector
+             (3, 5, (7, 7)), (2, 3, (5, 5)), (6, 10, (9, 7)), (16, 64, (63, 63)), (4, 8, (65, 65)),
+             (2, 4, (129, 129)), (1, 3, (255, 255)), (3, 2, (181, 90))]
 
 
 @pytest.mark.parametrize("n,c,sp", IN_SHAPES)
@@ -262,7 +266,8 @@ def test_in_forward_backward(n, c, sp, dtype):
     assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
 
 
-@pytest.mark.parametrize("n,c,sp", [(3, 4, (6, 6)), (2, 3, (300, 300)), (2, 32, (190, 190))])
+@pytest.mark.parametrize("n,c,sp", [(3, 4, (6, 6)), (2, 3, (300, 300)), (2, 32, (190, 190)),
+                                    (2, 6, (33, 31))])
 @pytest.mark.parametrize("bcg,bcb", [(False, False), (True, False), (False, True)])
 def test_in_per_sample_parameters_and_flags(n, c, sp, bcg, bcb):
     """gamma/beta of batch*channels elements (no broadcast over the batch),
@@ -449,7 +454,7 @@ def test_in_backward_held_on_chip_accumulate_and_parameter_gradients_only(dtype)
 
 
 @pytest.mark.parametrize("n,c,sp", [(2, 8, (16, 16)), (1, 3, (300, 300)), (4, 64, (7, 7)),
-                                    (1, 64, (400, 400)), (1, 226, (2, 104008))])
+                                    (1, 64, (400, 400)), (1, 226, (2, 104008)), (2, 8, (63, 63))])
 def test_in_forward_in_place(n, c, sp):
     x, _, g, b = make_nc(n, c, sp, torch.float16, 32)
     y_r, m_r, v_r = R.in_forward(x, b, g, n, c, 1e-5)
