@@ -13,6 +13,12 @@
 //
 // The tensor may end inside the last vector of its last row: that one vector is
 // loaded element by element.
+//
+// GroupNormalization whose planes are no whole number of vectors takes the same
+// route (gn_masked_*): a row is a group's planes, a vector may hold the end of
+// one channel and the start of the next, so gamma / beta are picked per element
+// (one boundary per vector at most: planes of VEC elements and more) and the
+// backward's per-channel sums are split at that boundary.
 #include <algorithm>
 
 #include "common.cuh"
@@ -38,6 +44,10 @@ struct MaskedRowArgs {
   uint32_t pmod, pmod_b; // parameter index = row % pmod (beta: pmod_b)
   float eps, inv_R, one;
   int accum_dx;
+  // GroupNormalization: elements per plane, channels per group (pmod = groups;
+  // parameter index = (row % pmod) * cpg + element / plane)
+  FastDiv plane;
+  uint32_t cpg;
 };
 
 // The part of the row that vector v of the row's threads holds.
@@ -262,6 +272,247 @@ in_masked_bwd_kernel(const MaskedRowArgs a) {
   }
 }
 
+// GroupNormalization: the channels (within the group) of the first and the last
+// element of a piece, and the element of the vector where the second begins
+// (VEC when the piece lies inside one channel).
+struct PieceChannels {
+  uint32_t c0, c1;
+  int jb;
+};
+
+template <int VEC>
+__device__ __forceinline__ PieceChannels piece_channels(const MaskedRowArgs &a, const RowPiece &p) {
+  PieceChannels pc;
+  const int first = p.col + p.lo, last = p.col + p.hi - 1;
+  pc.c0 = p.ok ? a.plane.div(static_cast<uint32_t>(first)) : 0u;
+  pc.c1 = p.ok ? a.plane.div(static_cast<uint32_t>(last)) : 0u;
+  pc.jb = pc.c1 != pc.c0 ? static_cast<int>((pc.c0 + 1u) * a.plane.d) - p.col : VEC;
+  return pc;
+}
+
+template <typename T, int VEC, int NL, int TPR>
+__global__ void __launch_bounds__(TPR)
+gn_masked_fwd_kernel(const MaskedRowArgs a) {
+  static_assert(TPR >= 256, "a block per row");
+  __shared__ float lds[2 * 16];
+  const int t = threadIdx.x;
+  const T *__restrict__ x = static_cast<const T *>(a.x);
+  T *__restrict__ y = static_cast<T *>(a.out);
+  for (int row = static_cast<int>(blockIdx.x); row < a.rows; row += gridDim.x) {
+    const size_t base = static_cast<size_t>(row) * a.R;
+    const int head = static_cast<int>(base % VEC);
+    const uint32_t pb = (static_cast<uint32_t>(row) % a.pmod) * a.cpg;
+    RawVec<T, VEC> raw[NL];
+#pragma unroll
+    for (int k = 0; k < NL; ++k)
+      raw[k] = load_piece<T, VEC>(x + base, head, row_piece<VEC>(a, base, head, k * TPR + t));
+    // gamma and beta of the piece's one or two channels, behind the row's loads
+    float g0[NL], g1[NL], b0[NL], b1[NL];
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const PieceChannels pc = piece_channels<VEC>(a, row_piece<VEC>(a, base, head, k * TPR + t));
+      g0[k] = a.gamma ? a.gamma[pb + pc.c0] : 1.f;
+      g1[k] = a.gamma ? a.gamma[pb + pc.c1] : 1.f;
+      b0[k] = a.beta ? a.beta[pb + pc.c0] : 0.f;
+      b1[k] = a.beta ? a.beta[pb + pc.c1] : 0.f;
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) s = raw_sum<T, VEC>(raw[k], s);
+    const float mean = row_sum<TPR>(s, lds) * a.inv_R;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+    float q = 0.f;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const RowPiece p = row_piece<VEC>(a, base, head, k * TPR + t);
+      if (p.ok) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float d = elem_fma<T, VEC>(raw[k], j, a.one, -mean);
+          q = (j >= p.lo && j < p.hi) ? fmaf(d, d, q) : q;
+        }
+      }
+    }
+    const float var = row_sum<TPR>(q, lds) * a.inv_R;
+    const float istd = inv_std(var, a.eps);
+    if (t == 0) {
+      a.mean[row] = mean;
+      a.var[row] = var;
+    }
+#pragma unroll
+    for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const RowPiece p = row_piece<VEC>(a, base, head, k * TPR + t);
+      if (p.ok) {
+        const PieceChannels pc = piece_channels<VEC>(a, p);
+        const float gs0 = g0[k] * istd, gs1 = g1[k] * istd;
+        const float sh0 = fmaf(-mean, gs0, b0[k]), sh1 = fmaf(-mean, gs1, b1[k]);
+        float o[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const bool second = j >= pc.jb;
+          if constexpr (sizeof(T) == 2) {
+            o[j] = elem_fma<T, VEC>(raw[k], j, second ? gs1 : gs0, second ? sh1 : sh0);
+          } else {
+            o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mean), second ? gs1 : gs0, second ? b1[k] : b0[k]);
+          }
+        }
+        store_piece<T, VEC>(y + base, p, o, 0);
+      }
+    }
+  }
+}
+
+// GroupNormalization backward.  The 64 vectors a wave holds in one slot meet two
+// channels at most (planes of 64 * VEC elements and more): per slot the wave
+// adds its lanes' (sum dy*xh, sum dy) for the first of them and for the next,
+// a thread per channel then adds the runs that belong to it in slot and wave
+// order - the pair per (row, channel) that dgamma / dbeta are summed from - and
+// the row's s1 = sum g*sdy, t2 = sum g*sdx follow from those.
+template <typename T, int VEC, int NL, int TPR>
+__global__ void __launch_bounds__(TPR)
+gn_masked_bwd_kernel(const MaskedRowArgs a) {
+  static_assert(TPR >= 256, "a block per row");
+  constexpr int NW = TPR / kWave;
+  __shared__ float lds[2 * 16];
+  __shared__ float runs[NL * NW * 4]; // per (slot, wave): sdx, sdy of the wave's first channel, of the next
+  const int t = threadIdx.x;
+  const int wave = t / kWave, lane = t % kWave;
+  const T *__restrict__ x = static_cast<const T *>(a.x);
+  const T *__restrict__ dy = static_cast<const T *>(a.dy);
+  T *dx = static_cast<T *>(a.out);
+  for (int row = static_cast<int>(blockIdx.x); row < a.rows; row += gridDim.x) {
+    const size_t base = static_cast<size_t>(row) * a.R;
+    const int head = static_cast<int>(base % VEC);
+    const uint32_t pb = (static_cast<uint32_t>(row) % a.pmod) * a.cpg;
+    const float mean = a.mean[row];
+    const float vpe = a.var[row] + a.eps;
+    const float u_dvar = a.dvar ? a.dvar[row] : 0.f;
+    const float u_dmean = a.dmean ? a.dmean[row] : 0.f;
+    const float g_t = (a.gamma && static_cast<uint32_t>(t) < a.cpg) ? a.gamma[pb + t] : 1.f;
+    RawVec<T, VEC> xr[NL], dr[NL];
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const RowPiece p = row_piece<VEC>(a, base, head, k * TPR + t);
+      xr[k] = load_piece<T, VEC>(x + base, head, p);
+      dr[k] = load_piece<T, VEC>(dy + base, head, p);
+    }
+    const float istd = 1.0f / sqrtf(vpe);
+    const float nmi = -mean * istd;
+    // the first channel of the wave's run in slot k (the same in every lane)
+    auto run_channel = [&](int k) {
+      const int first = max((k * TPR + wave * kWave) * VEC - head, 0);
+      return a.plane.div(static_cast<uint32_t>(min(first, a.R - 1)));
+    };
+    lds_barrier(); // runs[] of the previous row has been consumed
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const RowPiece p = row_piece<VEC>(a, base, head, k * TPR + t);
+      const PieceChannels pc = piece_channels<VEC>(a, p);
+      // the whole piece, then - in the one lane of some hundred whose vector holds
+      // a channel boundary - what lies behind the boundary
+      float sx0 = 0.f, sy0 = 0.f, sx1 = 0.f, sy1 = 0.f;
+      sy0 = raw_sum<T, VEC>(dr[k], 0.f);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+        sx0 = elem_fma<T, VEC>(dr[k], j, xh, sx0);
+      }
+      if (pc.jb < VEC) {
+#pragma unroll
+        for (int j = 1; j < VEC; ++j) {
+          if (j >= pc.jb) {
+            const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+            const float d = elem_fma<T, VEC>(dr[k], j, a.one, 0.f);
+            sx1 = fmaf(d, xh, sx1);
+            sy1 += d;
+          }
+        }
+        sx0 -= sx1;
+        sy0 -= sy1;
+      }
+      const uint32_t cw = run_channel(k);
+      // the channel of the run's last element: the same for most runs, and then
+      // nothing belongs to the next channel
+      const int run_last = min((k * TPR + wave * kWave + kWave) * VEC - head, a.R) - 1;
+      const bool two = run_last >= 0 && a.plane.div(static_cast<uint32_t>(run_last)) != cw;
+      // (a piece outside the row holds zeros: whichever channel takes them)
+      const bool first0 = pc.c0 == cw, first1 = pc.c1 == cw;
+      float ax = (first0 ? sx0 : 0.f) + ((first1 && pc.jb < VEC) ? sx1 : 0.f);
+      float ay = (first0 ? sy0 : 0.f) + ((first1 && pc.jb < VEC) ? sy1 : 0.f);
+      float bx = 0.f, by = 0.f;
+      ax = wave_sum(ax);
+      ay = wave_sum(ay);
+      if (two) { // (the same answer in every lane)
+        bx = (first0 ? 0.f : sx0) + ((first1 || pc.jb >= VEC) ? 0.f : sx1);
+        by = (first0 ? 0.f : sy0) + ((first1 || pc.jb >= VEC) ? 0.f : sy1);
+        bx = wave_sum(bx);
+        by = wave_sum(by);
+      }
+      if (lane == 0) {
+        float *r = runs + (k * NW + wave) * 4;
+        r[0] = ax;
+        r[1] = ay;
+        r[2] = bx;
+        r[3] = by;
+      }
+    }
+    lds_barrier();
+    float c1 = 0.f, c2 = 0.f;
+    if (static_cast<uint32_t>(t) < a.cpg) {
+      // The runs (slot, wave) follow the row's vectors in order: channel t meets
+      // the runs of its first to its last vector.
+      float sdx = 0.f, sdy = 0.f;
+      const int run_lo = (t * static_cast<int>(a.plane.d) + head) / (VEC * kWave);
+      const int run_hi = ((t + 1) * static_cast<int>(a.plane.d) - 1 + head) / (VEC * kWave);
+      for (int run = run_lo; run <= run_hi; ++run) {
+        const int first = max(run * kWave * VEC - head, 0);
+        const uint32_t cw = a.plane.div(static_cast<uint32_t>(min(first, a.R - 1)));
+        const float *r = runs + run * 4;
+        if (cw == static_cast<uint32_t>(t)) {
+          sdx += r[0];
+          sdy += r[1];
+        } else if (cw + 1u == static_cast<uint32_t>(t)) {
+          sdx += r[2];
+          sdy += r[3];
+        }
+      }
+      const size_t o = 2 * (static_cast<size_t>(row) * a.cpg + t);
+      a.ws[o] = sdx;
+      a.ws[o + 1] = sdy;
+      c1 = g_t * sdy;
+      c2 = g_t * sdx;
+    }
+    row_sum2<TPR>(c1, c2, lds);
+    if (dx == nullptr) continue;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      keep_packed<T, VEC>(xr[k]);
+      keep_packed<T, VEC>(dr[k]);
+    }
+    const float cA = -istd * c2 * a.inv_R + (a.dvar ? 2.f * u_dvar * (vpe * istd) * a.inv_R : 0.f);
+    const float cb = -c1 * istd * a.inv_R + (a.dmean ? u_dmean * a.inv_R : 0.f);
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const RowPiece p = row_piece<VEC>(a, base, head, k * TPR + t);
+      if (p.ok) {
+        const PieceChannels pc = piece_channels<VEC>(a, p);
+        const float gi0 = (a.gamma ? a.gamma[pb + pc.c0] : 1.f) * istd;
+        const float gi1 = (a.gamma ? a.gamma[pb + pc.c1] : 1.f) * istd;
+        float o[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+          o[j] = elem_fma<T, VEC>(dr[k], j, j >= pc.jb ? gi1 : gi0, fmaf(xh, cA, cb));
+        }
+        store_piece<T, VEC>(dx + base, p, o, a.accum_dx);
+      }
+    }
+  }
+}
+
 namespace {
 
 MaskedRowArgs masked_args(const RowProblem &p) {
@@ -281,6 +532,13 @@ MaskedRowArgs masked_args(const RowProblem &p) {
   a.total = static_cast<long long>(p.rows) * p.R;
   a.pmod = static_cast<uint32_t>(p.bc_gamma ? p.channels : p.rows);
   a.pmod_b = static_cast<uint32_t>(p.bc_beta ? p.channels : p.rows);
+  a.plane = FastDiv(static_cast<uint32_t>(p.R));
+  a.cpg = 1;
+  if (p.mode == kRowGN) {
+    a.pmod = a.pmod_b = static_cast<uint32_t>(p.groups);
+    a.cpg = static_cast<uint32_t>(p.channels / p.groups);
+    a.plane = FastDiv(static_cast<uint32_t>(p.spatial));
+  }
   a.eps = p.eps;
   a.inv_R = static_cast<float>(1.0 / static_cast<double>(p.R));
   a.one = 1.0f;
@@ -297,10 +555,11 @@ struct MaskedCfg {
 
 // The layout with the fewest idle slots (a slot beyond the row still issues
 // its load); among equals the fewest threads.
-MaskedCfg pick_masked(int64_t nv) {
+MaskedCfg pick_masked(int64_t nv, int min_tpr = 64) {
   MaskedCfg c;
   int64_t best = 0;
   for (int tpr : {64, 256, 512, 1024}) {
+    if (tpr < min_tpr) continue;
     for (int nl : {1, 2, 3, 4, 5, 6, 8}) {
       const int64_t cap = static_cast<int64_t>(tpr) * nl;
       if (cap >= nv && (!c.ok || cap < best)) {
@@ -315,13 +574,47 @@ MaskedCfg pick_masked(int64_t nv) {
 }
 
 bool masked_plan(const RowProblem &p, bool backward, MaskedCfg &cfg) {
-  if (p.mode != kRowIN || !tune_int("ROW_MASKED", 1)) return false;
+  if ((p.mode != kRowIN && p.mode != kRowGN) || !tune_int("ROW_MASKED", 1)) return false;
   const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
-  if (p.R % vec == 0 || p.R < 2 * vec) return false; // whole vectors: the plain kernels
+  if (p.R < 2 * vec) return false;
   if (!aligned16(p.x) || (p.out && !aligned16(p.out)) || (backward && !aligned16(p.dy))) return false;
   if (p.rows >= (int64_t{1} << 31) / std::max<int64_t>(1, p.R)) return false;
-  cfg = pick_masked((p.R + 2 * vec - 2) / vec);
+  if (p.mode == kRowIN) {
+    if (p.R % vec == 0) return false; // whole vectors: the plain kernels
+    cfg = pick_masked((p.R + 2 * vec - 2) / vec);
+    return cfg.ok;
+  }
+  // groups: planes that are no whole number of vectors, long enough for one
+  // channel boundary per vector (backward: two channels per wave-wide run), a
+  // thread per channel of the group
+  if (p.spatial % vec == 0 || !tune_int("ROW_MASKED_GROUPS", 1)) return false;
+  if (p.spatial < (backward ? 64 * vec : vec) || p.channels / p.groups > 256) return false;
+  cfg = pick_masked((p.R + 2 * vec - 2) / vec, 256);
   return cfg.ok;
+}
+
+template <typename T, int VEC, bool BWD>
+int run_masked_groups(const MaskedCfg &c, const MaskedRowArgs &a, int grid, hipStream_t st) {
+#define MASKED_CASE(NL, TPR)                                                                       \
+  if (c.nl == (NL) && c.tpr == (TPR)) {                                                            \
+    if constexpr (BWD) {                                                                           \
+      NBLAHIP_LAUNCH("gn_masked_bwd_kernel", (gn_masked_bwd_kernel<T, VEC, NL, TPR>), dim3(grid),  \
+                     dim3(TPR), 0, st, a);                                                         \
+    } else {                                                                                       \
+      NBLAHIP_LAUNCH("gn_masked_fwd_kernel", (gn_masked_fwd_kernel<T, VEC, NL, TPR>), dim3(grid),  \
+                     dim3(TPR), 0, st, a);                                                         \
+    }                                                                                              \
+    return last_launch_status();                                                                   \
+  }
+#define MASKED_TPR(TPR)                                                                 \
+  MASKED_CASE(1, TPR) MASKED_CASE(2, TPR) MASKED_CASE(3, TPR) MASKED_CASE(4, TPR)       \
+  MASKED_CASE(5, TPR) MASKED_CASE(6, TPR) MASKED_CASE(8, TPR)
+  MASKED_TPR(256)
+  MASKED_TPR(512)
+  MASKED_TPR(1024)
+#undef MASKED_TPR
+#undef MASKED_CASE
+  return NBLAHIP_EINVAL;
 }
 
 template <typename T, int VEC, bool BWD>
@@ -360,6 +653,12 @@ bool row_masked_fwd(const RowProblem &p, hipStream_t st, int *status) {
   MaskedCfg c;
   if (!masked_plan(p, false, c)) return false;
   const MaskedRowArgs a = masked_args(p);
+  if (p.mode == kRowGN) {
+    const int grid = static_cast<int>(std::min<int64_t>(p.rows, 1 << 20));
+    *status = p.dtype == NBLAHIP_F16 ? run_masked_groups<__half, 8, false>(c, a, grid, st)
+                                     : run_masked_groups<float, 4, false>(c, a, grid, st);
+    return true;
+  }
   const int grid = masked_grid(p.rows, c.tpr);
   *status = p.dtype == NBLAHIP_F16 ? run_masked<__half, 8, false>(c, a, grid, st)
                                    : run_masked<float, 4, false>(c, a, grid, st);
@@ -369,8 +668,15 @@ bool row_masked_fwd(const RowProblem &p, hipStream_t st, int *status) {
 bool row_masked_bwd(const RowProblem &p, hipStream_t st, int *status) {
   MaskedCfg c;
   if (!masked_plan(p, true, c)) return false;
-  if (static_cast<size_t>(p.rows) * 2 * sizeof(float) > p.ws_bytes) return false;
+  const int64_t cpg = p.mode == kRowGN ? p.channels / p.groups : 1;
+  if (static_cast<size_t>(p.rows) * cpg * 2 * sizeof(float) > p.ws_bytes) return false;
   const MaskedRowArgs a = masked_args(p);
+  if (p.mode == kRowGN) {
+    const int grid = static_cast<int>(std::min<int64_t>(p.rows, 1 << 20));
+    *status = p.dtype == NBLAHIP_F16 ? run_masked_groups<__half, 8, true>(c, a, grid, st)
+                                     : run_masked_groups<float, 4, true>(c, a, grid, st);
+    return true;
+  }
   const int grid = masked_grid(p.rows, c.tpr);
   *status = p.dtype == NBLAHIP_F16 ? run_masked<__half, 8, true>(c, a, grid, st)
                                    : run_masked<float, 4, true>(c, a, grid, st);

@@ -171,7 +171,11 @@ GN_SHAPES = [(2, 8, (8, 8), 4), (3, 6, (5,), 2), (1, 4, (2, 2), 1), (2, 6, (4,),
              (4, 2560, (16, 16), 32), (2, 4096, (8, 16), 32), (4, 2048, (16, 8), 16),
              (4, 2048, (8, 8), 16),
              # one group of 2M elements per sample: split streaming reductions
-             (2, 32, (256, 256), 1), (1, 6, (333, 333), 2)]
+             (2, 32, (256, 256), 1), (1, 6, (333, 333), 2),
+             # planes that are no whole number of vectors, taken with the tensor's aligned
+             # vectors (a channel boundary inside a vector); short planes: the forward only
+             (2, 16, (63, 63), 4), (4, 32, (33, 33), 8), (2, 8, (17, 17), 2), (3, 6, (5, 7), 3),
+             (2, 256, (63, 63), 32), (1, 24, (65, 65), 3), (3, 9, (31, 33), 3), (2, 12, (127, 9), 2)]
 
 
 def make_nc(n, c, sp, dtype, seed):
@@ -205,7 +209,9 @@ def test_gn_forward_backward(n, c, sp, groups, dtype):
 @pytest.mark.parametrize("n,c,sp,groups", [(4, 64, (16, 16), 8), (2, 32, (7, 7), 8),
                                            (2, 160, (64, 64), 16),
                                            # the group held on one CU in the backward
-                                           (4, 320, (64, 64), 32)])
+                                           (4, 320, (64, 64), 32),
+                                           # planes that are no whole number of vectors
+                                           (2, 16, (33, 31), 4)])
 def test_gn_flags(n, c, sp, groups):
     dtype = torch.float32
     x, dy, g, b = make_nc(n, c, sp, dtype, 5)
