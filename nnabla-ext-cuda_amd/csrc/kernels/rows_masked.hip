@@ -513,6 +513,207 @@ gn_masked_bwd_kernel(const MaskedRowArgs a) {
   }
 }
 
+// GroupNormalization, a group's planes side by side in one block: TPP threads
+// per plane (one wave or more), so a thread's pieces lie inside its plane - no
+// channel boundary inside a vector, gamma / beta one scalar per thread - and the
+// planes meet only in the sums: per wave through LDS, added in wave order.
+// For groups of up to 16 channels whose plane TPP * NL vectors hold.
+struct GroupPlanesArgs {
+  MaskedRowArgs r;
+  int tpp_shift; // threads per plane = 1 << tpp_shift (64 ... 1024)
+  int len;       // elements per plane
+};
+
+template <int VEC>
+__device__ __forceinline__ RowPiece plane_piece(const GroupPlanesArgs &g, size_t base, int head, int v) {
+  RowPiece p;
+  p.col = v * VEC - head;
+  p.ok = p.col < g.len;
+  p.lo = p.col < 0 ? -p.col : 0;
+  p.hi = min(VEC, g.len - p.col);
+  p.tail = static_cast<long long>(base) + p.col + VEC > g.r.total;
+  return p;
+}
+
+template <typename T, int VEC, int NL>
+__global__ void __launch_bounds__(1024)
+gn_planes_masked_fwd_kernel(const GroupPlanesArgs g) {
+  const MaskedRowArgs &a = g.r;
+  __shared__ float wsum[2][16];
+  const int t = threadIdx.x;
+  const int nw = blockDim.x / kWave, wave = t / kWave, lane = t % kWave;
+  const int pl = t >> g.tpp_shift, tp = t & ((1 << g.tpp_shift) - 1);
+  const int tpp = 1 << g.tpp_shift;
+  const T *__restrict__ x = static_cast<const T *>(a.x);
+  T *__restrict__ y = static_cast<T *>(a.out);
+  for (int row = static_cast<int>(blockIdx.x); row < a.rows; row += gridDim.x) {
+    const size_t base = static_cast<size_t>(row) * a.R + static_cast<size_t>(pl) * g.len;
+    const int head = static_cast<int>(base % VEC);
+    const uint32_t pc = (static_cast<uint32_t>(row) % a.pmod) * a.cpg + pl;
+    const float gam = a.gamma ? a.gamma[pc] : 1.f;
+    const float bet = a.beta ? a.beta[pc] : 0.f;
+    RawVec<T, VEC> raw[NL];
+#pragma unroll
+    for (int k = 0; k < NL; ++k)
+      raw[k] = load_piece<T, VEC>(x + base, head, plane_piece<VEC>(g, base, head, k * tpp + tp));
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) s = raw_sum<T, VEC>(raw[k], s);
+    s = wave_sum(s);
+    lds_barrier(); // the previous row's sums have been read
+    if (lane == 0) wsum[0][wave] = s;
+    lds_barrier();
+    float tot = 0.f;
+    for (int w = 0; w < nw; ++w) tot += wsum[0][w];
+    const float mean = tot * a.inv_R;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+    float q = 0.f;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const RowPiece p = plane_piece<VEC>(g, base, head, k * tpp + tp);
+      if (p.ok) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float d = elem_fma<T, VEC>(raw[k], j, a.one, -mean);
+          q = (j >= p.lo && j < p.hi) ? fmaf(d, d, q) : q;
+        }
+      }
+    }
+    q = wave_sum(q);
+    if (lane == 0) wsum[1][wave] = q;
+    lds_barrier();
+    float qt = 0.f;
+    for (int w = 0; w < nw; ++w) qt += wsum[1][w];
+    const float var = qt * a.inv_R;
+    const float istd = inv_std(var, a.eps);
+    if (t == 0) {
+      a.mean[row] = mean;
+      a.var[row] = var;
+    }
+#pragma unroll
+    for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+    const float gs = gam * istd;
+    const float sh = fmaf(-mean, gs, bet);
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const RowPiece p = plane_piece<VEC>(g, base, head, k * tpp + tp);
+      if (p.ok) {
+        float o[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          if constexpr (sizeof(T) == 2) {
+            o[j] = elem_fma<T, VEC>(raw[k], j, gs, sh);
+          } else {
+            o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mean), gs, bet);
+          }
+        }
+        store_piece<T, VEC>(y + base, p, o, 0);
+      }
+    }
+  }
+}
+
+template <typename T, int VEC, int NL>
+__global__ void __launch_bounds__(1024)
+gn_planes_masked_bwd_kernel(const GroupPlanesArgs g) {
+  const MaskedRowArgs &a = g.r;
+  __shared__ float wsum[16][2]; // per wave: sum dy*xh, sum dy
+  __shared__ float gch[16];     // gamma of the group's channels
+  const int t = threadIdx.x;
+  const int nw = blockDim.x / kWave, wave = t / kWave, lane = t % kWave;
+  const int pl = t >> g.tpp_shift, tp = t & ((1 << g.tpp_shift) - 1);
+  const int tpp = 1 << g.tpp_shift;
+  const int wpp = tpp / kWave; // waves per plane
+  const T *__restrict__ x = static_cast<const T *>(a.x);
+  const T *__restrict__ dy = static_cast<const T *>(a.dy);
+  T *dx = static_cast<T *>(a.out);
+  for (int row = static_cast<int>(blockIdx.x); row < a.rows; row += gridDim.x) {
+    const size_t base = static_cast<size_t>(row) * a.R + static_cast<size_t>(pl) * g.len;
+    const int head = static_cast<int>(base % VEC);
+    const uint32_t pb = (static_cast<uint32_t>(row) % a.pmod) * a.cpg;
+    const float gam = a.gamma ? a.gamma[pb + pl] : 1.f;
+    const float g_t = (a.gamma && static_cast<uint32_t>(t) < a.cpg) ? a.gamma[pb + t] : 1.f;
+    const float mean = a.mean[row];
+    const float vpe = a.var[row] + a.eps;
+    const float u_dvar = a.dvar ? a.dvar[row] : 0.f;
+    const float u_dmean = a.dmean ? a.dmean[row] : 0.f;
+    RawVec<T, VEC> xr[NL], dr[NL];
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const RowPiece p = plane_piece<VEC>(g, base, head, k * tpp + tp);
+      xr[k] = load_piece<T, VEC>(x + base, head, p);
+      dr[k] = load_piece<T, VEC>(dy + base, head, p);
+    }
+    const float istd = 1.0f / sqrtf(vpe);
+    const float nmi = -mean * istd;
+    float sdy = 0.f, sdx = 0.f;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      sdy = raw_sum<T, VEC>(dr[k], sdy);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+        sdx = elem_fma<T, VEC>(dr[k], j, xh, sdx);
+      }
+    }
+    sdx = wave_sum(sdx);
+    sdy = wave_sum(sdy);
+    lds_barrier(); // the previous row's sums have been read
+    if (lane == 0) {
+      wsum[wave][0] = sdx;
+      wsum[wave][1] = sdy;
+    }
+    if (static_cast<uint32_t>(t) < a.cpg) gch[t] = g_t;
+    lds_barrier();
+    // the planes' pairs (the row's share of dgamma / dbeta), a thread per plane
+    if (static_cast<uint32_t>(t) < a.cpg) {
+      float px = 0.f, py = 0.f;
+      for (int w = t * wpp; w < (t + 1) * wpp; ++w) {
+        px += wsum[w][0];
+        py += wsum[w][1];
+      }
+      const size_t o = 2 * (static_cast<size_t>(row) * a.cpg + t);
+      a.ws[o] = px;
+      a.ws[o + 1] = py;
+    }
+    if (dx == nullptr) continue;
+    // the group's s1 = sum g*sdy, t2 = sum g*sdx: planes in order, each plane's waves in order
+    float s1 = 0.f, t2 = 0.f;
+    for (uint32_t c = 0; c < a.cpg; ++c) {
+      float px = 0.f, py = 0.f;
+      for (int w = static_cast<int>(c) * wpp; w < static_cast<int>(c + 1) * wpp; ++w) {
+        px += wsum[w][0];
+        py += wsum[w][1];
+      }
+      s1 = fmaf(gch[c], py, s1);
+      t2 = fmaf(gch[c], px, t2);
+    }
+    (void)nw;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      keep_packed<T, VEC>(xr[k]);
+      keep_packed<T, VEC>(dr[k]);
+    }
+    const float cA = -istd * t2 * a.inv_R + (a.dvar ? 2.f * u_dvar * (vpe * istd) * a.inv_R : 0.f);
+    const float cb = -s1 * istd * a.inv_R + (a.dmean ? u_dmean * a.inv_R : 0.f);
+    const float gi = gam * istd;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const RowPiece p = plane_piece<VEC>(g, base, head, k * tpp + tp);
+      if (p.ok) {
+        float o[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+          o[j] = elem_fma<T, VEC>(dr[k], j, gi, fmaf(xh, cA, cb));
+        }
+        store_piece<T, VEC>(dx + base, p, o, a.accum_dx);
+      }
+    }
+  }
+}
+
 namespace {
 
 MaskedRowArgs masked_args(const RowProblem &p) {
@@ -573,6 +774,36 @@ MaskedCfg pick_masked(int64_t nv, int min_tpr = 64) {
   return c;
 }
 
+// The planes-side-by-side layout for a group: threads per plane (a power of two
+// from 64) and vectors per thread, fewest idle slots; ok = false when the
+// group's channels times the threads of a plane exceed a block.
+struct PlanesCfg {
+  bool ok = false;
+  int tpp_shift = 6, nl = 1;
+};
+
+PlanesCfg pick_planes(const RowProblem &p, int vec, bool backward) {
+  PlanesCfg c;
+  const int64_t cpg = p.channels / p.groups;
+  if (cpg > 16 || !tune_int("ROW_MASKED_PLANES", 1)) return c;
+  const int64_t nv = (p.spatial + 2 * vec - 2) / vec;
+  int64_t best = 0;
+  for (int sh = 6; sh <= 10; ++sh) {
+    if ((cpg << sh) > 1024) break;
+    for (int nl : {1, 2, 3, 4, 5, 6, 8}) {
+      if (backward && nl > 6) continue; // (x and dy of 8 vectors: past 128 registers)
+      const int64_t cap = static_cast<int64_t>(nl) << sh;
+      if (cap >= nv && (!c.ok || cap < best)) {
+        c.ok = true;
+        c.tpp_shift = sh;
+        c.nl = nl;
+        best = cap;
+      }
+    }
+  }
+  return c;
+}
+
 bool masked_plan(const RowProblem &p, bool backward, MaskedCfg &cfg) {
   if ((p.mode != kRowIN && p.mode != kRowGN) || !tune_int("ROW_MASKED", 1)) return false;
   const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
@@ -588,9 +819,43 @@ bool masked_plan(const RowProblem &p, bool backward, MaskedCfg &cfg) {
   // channel boundary per vector (backward: two channels per wave-wide run), a
   // thread per channel of the group
   if (p.spatial % vec == 0 || !tune_int("ROW_MASKED_GROUPS", 1)) return false;
+  if (p.spatial >= 2 * vec && pick_planes(p, vec, backward).ok) return true; // the planes side by side
   if (p.spatial < (backward ? 64 * vec : vec) || p.channels / p.groups > 256) return false;
   cfg = pick_masked((p.R + 2 * vec - 2) / vec, 256);
   return cfg.ok;
+}
+
+template <typename T, int VEC, bool BWD>
+int run_group_planes(const PlanesCfg &c, const GroupPlanesArgs &g, int grid, int block, hipStream_t st) {
+#define PLANES_CASE(NL)                                                                            \
+  if (c.nl == (NL)) {                                                                              \
+    if constexpr (BWD) {                                                                           \
+      NBLAHIP_LAUNCH("gn_planes_masked_bwd_kernel", (gn_planes_masked_bwd_kernel<T, VEC, NL>),     \
+                     dim3(grid), dim3(block), 0, st, g);                                           \
+    } else {                                                                                       \
+      NBLAHIP_LAUNCH("gn_planes_masked_fwd_kernel", (gn_planes_masked_fwd_kernel<T, VEC, NL>),     \
+                     dim3(grid), dim3(block), 0, st, g);                                           \
+    }                                                                                              \
+    return last_launch_status();                                                                   \
+  }
+  PLANES_CASE(1) PLANES_CASE(2) PLANES_CASE(3) PLANES_CASE(4) PLANES_CASE(5) PLANES_CASE(6)
+  if constexpr (!BWD) {
+    PLANES_CASE(8)
+  }
+#undef PLANES_CASE
+  return NBLAHIP_EINVAL;
+}
+
+template <bool BWD>
+int launch_group_planes(const RowProblem &p, const PlanesCfg &c, const MaskedRowArgs &a, hipStream_t st) {
+  GroupPlanesArgs g{};
+  g.r = a;
+  g.tpp_shift = c.tpp_shift;
+  g.len = static_cast<int>(p.spatial);
+  const int block = static_cast<int>((p.channels / p.groups) << c.tpp_shift);
+  const int grid = static_cast<int>(std::min<int64_t>(p.rows, 1 << 20));
+  return p.dtype == NBLAHIP_F16 ? run_group_planes<__half, 8, BWD>(c, g, grid, block, st)
+                                : run_group_planes<float, 4, BWD>(c, g, grid, block, st);
 }
 
 template <typename T, int VEC, bool BWD>
@@ -654,6 +919,11 @@ bool row_masked_fwd(const RowProblem &p, hipStream_t st, int *status) {
   if (!masked_plan(p, false, c)) return false;
   const MaskedRowArgs a = masked_args(p);
   if (p.mode == kRowGN) {
+    const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
+    if (const PlanesCfg pc = pick_planes(p, vec, false); pc.ok && p.spatial >= 2 * vec) {
+      *status = launch_group_planes<false>(p, pc, a, st);
+      return true;
+    }
     const int grid = static_cast<int>(std::min<int64_t>(p.rows, 1 << 20));
     *status = p.dtype == NBLAHIP_F16 ? run_masked_groups<__half, 8, false>(c, a, grid, st)
                                      : run_masked_groups<float, 4, false>(c, a, grid, st);
@@ -672,6 +942,11 @@ bool row_masked_bwd(const RowProblem &p, hipStream_t st, int *status) {
   if (static_cast<size_t>(p.rows) * cpg * 2 * sizeof(float) > p.ws_bytes) return false;
   const MaskedRowArgs a = masked_args(p);
   if (p.mode == kRowGN) {
+    const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
+    if (const PlanesCfg pc = pick_planes(p, vec, true); pc.ok && p.spatial >= 2 * vec) {
+      *status = launch_group_planes<true>(p, pc, a, st);
+      return true;
+    }
     const int grid = static_cast<int>(std::min<int64_t>(p.rows, 1 << 20));
     *status = p.dtype == NBLAHIP_F16 ? run_masked_groups<__half, 8, true>(c, a, grid, st)
                                      : run_masked_groups<float, 4, true>(c, a, grid, st);

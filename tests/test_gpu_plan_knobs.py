@@ -219,9 +219,15 @@ SWITCHES = [
     ("gn_onchip_bwd_small_planes_off", run_gn, (4, 2560, (16, 16), 32, F16),
      {"GN_ONCHIP_BWD_SMALL_PLANES_MIN_NL": 99}, ["row_bwd_kernel_gn"], ["gn_onchip_bwd_kernel"]),
     ("rows_masked_groups_off", run_gn, (2, 64, (63, 63), 8, F16), {"ROW_MASKED_GROUPS": 0},
-     ["row_stats_stream_kernel"], ["gn_masked_fwd_kernel", "gn_masked_bwd_kernel"]),
+     ["row_stats_stream_kernel"], ["gn_planes_masked_fwd_kernel", "gn_planes_masked_bwd_kernel"]),
     ("rows_masked_groups_off_float", run_gn, (3, 12, (33, 33), 4, F32), {"ROW_MASKED": 0},
-     [], ["gn_masked_fwd_kernel", "gn_masked_bwd_kernel"]),
+     [], ["gn_planes_masked_fwd_kernel", "gn_planes_masked_bwd_kernel"]),
+    ("rows_masked_planes_off", run_gn, (2, 64, (63, 63), 8, F16), {"ROW_MASKED_PLANES": 0},
+     ["gn_masked_fwd_kernel", "gn_masked_bwd_kernel"],
+     ["gn_planes_masked_fwd_kernel", "gn_planes_masked_bwd_kernel"]),
+    ("rows_masked_planes_off_float", run_gn, (2, 8, (65, 65), 2, F32), {"ROW_MASKED_PLANES": 0},
+     ["gn_masked_fwd_kernel", "gn_masked_bwd_kernel"],
+     ["gn_planes_masked_fwd_kernel", "gn_planes_masked_bwd_kernel"]),
     ("rows_masked_off", run_in, (4, 32, (63, 63), F16), {"ROW_MASKED": 0},
      ["row_fwd_kernel"], ["in_masked_fwd_kernel", "in_masked_bwd_kernel"]),
     ("rows_masked_off_float", run_in, (3, 10, (9, 7), F32), {"ROW_MASKED": 0},
