@@ -756,9 +756,23 @@ struct MaskedCfg {
 
 // The layout with the fewest idle slots (a slot beyond the row still issues
 // its load); among equals the fewest threads.
-MaskedCfg pick_masked(int64_t nv, int min_tpr = 64) {
+MaskedCfg pick_masked(int64_t nv, int min_tpr = 8) {
   MaskedCfg c;
   int64_t best = 0;
+  // (planes of a few vectors: several rows per wave, at most 4 vectors a thread)
+  for (int tpr : {8, 16, 32}) {
+    if (tpr < min_tpr) continue;
+    for (int nl : {1, 2, 4}) {
+      const int64_t cap = static_cast<int64_t>(tpr) * nl;
+      if (cap >= nv && (!c.ok || cap < best)) {
+        c.ok = true;
+        c.tpr = tpr;
+        c.nl = nl;
+        best = cap;
+      }
+    }
+  }
+  if (c.ok) return c;
   for (int tpr : {64, 256, 512, 1024}) {
     if (tpr < min_tpr) continue;
     for (int nl : {1, 2, 3, 4, 5, 6, 8}) {
@@ -898,6 +912,9 @@ int run_masked(const MaskedCfg &c, const MaskedRowArgs &a, int grid, hipStream_t
 #define MASKED_TPR(TPR)                                                                 \
   MASKED_CASE(1, TPR) MASKED_CASE(2, TPR) MASKED_CASE(3, TPR) MASKED_CASE(4, TPR)       \
   MASKED_CASE(5, TPR) MASKED_CASE(6, TPR) MASKED_CASE(8, TPR)
+  MASKED_CASE(1, 8) MASKED_CASE(2, 8) MASKED_CASE(4, 8)
+  MASKED_CASE(1, 16) MASKED_CASE(2, 16) MASKED_CASE(4, 16)
+  MASKED_CASE(1, 32) MASKED_CASE(2, 32) MASKED_CASE(4, 32)
   MASKED_TPR(64)
   MASKED_TPR(256)
   MASKED_TPR(512)
