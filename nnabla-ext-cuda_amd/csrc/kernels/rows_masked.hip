@@ -517,7 +517,8 @@ gn_masked_bwd_kernel(const MaskedRowArgs a) {
 // per plane (one wave or more), so a thread's pieces lie inside its plane - no
 // channel boundary inside a vector, gamma / beta one scalar per thread - and the
 // planes meet only in the sums: per wave through LDS, added in wave order.
-// For groups of up to 16 channels whose plane TPP * NL vectors hold.
+// For groups of up to 64 channels whose plane TPP * NL vectors hold
+// (channels * TPP threads: a block of 1024 at most).
 struct GroupPlanesArgs {
   MaskedRowArgs r;
   int tpp_shift; // threads per plane = 1 << tpp_shift (64 ... 1024)
@@ -535,15 +536,28 @@ __device__ __forceinline__ RowPiece plane_piece(const GroupPlanesArgs &g, size_t
   return p;
 }
 
-template <typename T, int VEC, int NL>
+// SUB: 8, 16 or 32 threads per plane (several planes per wave; the sums per
+// plane then), 0: whole waves per plane.
+template <typename T, int VEC, int NL, int SUB>
 __global__ void __launch_bounds__(1024)
 gn_planes_masked_fwd_kernel(const GroupPlanesArgs g) {
   const MaskedRowArgs &a = g.r;
-  __shared__ float wsum[2][16];
+  __shared__ float wsum[2][64];
   const int t = threadIdx.x;
-  const int nw = blockDim.x / kWave, wave = t / kWave, lane = t % kWave;
+  const int wave = t / kWave, lane = t % kWave;
   const int pl = t >> g.tpp_shift, tp = t & ((1 << g.tpp_shift) - 1);
   const int tpp = 1 << g.tpp_shift;
+  // the block's partial sums: one per wave, or one per plane
+  const int nparts = SUB > 0 ? static_cast<int>(a.cpg) : static_cast<int>(blockDim.x) / kWave;
+  const int part = SUB > 0 ? pl : wave;
+  const bool writer = SUB > 0 ? tp == 0 : lane == 0;
+  auto part_sum = [&](float v) {
+    if constexpr (SUB > 0) {
+      return group_sum<(SUB > 0 ? SUB : 8)>(v);
+    } else {
+      return wave_sum(v);
+    }
+  };
   const T *__restrict__ x = static_cast<const T *>(a.x);
   T *__restrict__ y = static_cast<T *>(a.out);
   for (int row = static_cast<int>(blockIdx.x); row < a.rows; row += gridDim.x) {
@@ -559,12 +573,12 @@ gn_planes_masked_fwd_kernel(const GroupPlanesArgs g) {
     float s = 0.f;
 #pragma unroll
     for (int k = 0; k < NL; ++k) s = raw_sum<T, VEC>(raw[k], s);
-    s = wave_sum(s);
+    s = part_sum(s);
     lds_barrier(); // the previous row's sums have been read
-    if (lane == 0) wsum[0][wave] = s;
+    if (writer) wsum[0][part] = s;
     lds_barrier();
     float tot = 0.f;
-    for (int w = 0; w < nw; ++w) tot += wsum[0][w];
+    for (int w = 0; w < nparts; ++w) tot += wsum[0][w];
     const float mean = tot * a.inv_R;
 #pragma unroll
     for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
@@ -580,11 +594,11 @@ gn_planes_masked_fwd_kernel(const GroupPlanesArgs g) {
         }
       }
     }
-    q = wave_sum(q);
-    if (lane == 0) wsum[1][wave] = q;
+    q = part_sum(q);
+    if (writer) wsum[1][part] = q;
     lds_barrier();
     float qt = 0.f;
-    for (int w = 0; w < nw; ++w) qt += wsum[1][w];
+    for (int w = 0; w < nparts; ++w) qt += wsum[1][w];
     const float var = qt * a.inv_R;
     const float istd = inv_std(var, a.eps);
     if (t == 0) {
@@ -614,17 +628,26 @@ gn_planes_masked_fwd_kernel(const GroupPlanesArgs g) {
   }
 }
 
-template <typename T, int VEC, int NL>
+template <typename T, int VEC, int NL, int SUB>
 __global__ void __launch_bounds__(1024)
 gn_planes_masked_bwd_kernel(const GroupPlanesArgs g) {
   const MaskedRowArgs &a = g.r;
-  __shared__ float wsum[16][2]; // per wave: sum dy*xh, sum dy
-  __shared__ float gch[16];     // gamma of the group's channels
+  __shared__ float wsum[64][2]; // per wave (SUB: per plane): sum dy*xh, sum dy
+  __shared__ float gch[64];     // gamma of the group's channels
   const int t = threadIdx.x;
-  const int nw = blockDim.x / kWave, wave = t / kWave, lane = t % kWave;
+  const int wave = t / kWave, lane = t % kWave;
   const int pl = t >> g.tpp_shift, tp = t & ((1 << g.tpp_shift) - 1);
   const int tpp = 1 << g.tpp_shift;
-  const int wpp = tpp / kWave; // waves per plane
+  const int wpp = SUB > 0 ? 1 : tpp / kWave; // partial sums per plane
+  const int part = SUB > 0 ? pl : wave;
+  const bool writer = SUB > 0 ? tp == 0 : lane == 0;
+  auto part_sum = [&](float v) {
+    if constexpr (SUB > 0) {
+      return group_sum<(SUB > 0 ? SUB : 8)>(v);
+    } else {
+      return wave_sum(v);
+    }
+  };
   const T *__restrict__ x = static_cast<const T *>(a.x);
   const T *__restrict__ dy = static_cast<const T *>(a.dy);
   T *dx = static_cast<T *>(a.out);
@@ -657,12 +680,12 @@ gn_planes_masked_bwd_kernel(const GroupPlanesArgs g) {
         sdx = elem_fma<T, VEC>(dr[k], j, xh, sdx);
       }
     }
-    sdx = wave_sum(sdx);
-    sdy = wave_sum(sdy);
+    sdx = part_sum(sdx);
+    sdy = part_sum(sdy);
     lds_barrier(); // the previous row's sums have been read
-    if (lane == 0) {
-      wsum[wave][0] = sdx;
-      wsum[wave][1] = sdy;
+    if (writer) {
+      wsum[part][0] = sdx;
+      wsum[part][1] = sdy;
     }
     if (static_cast<uint32_t>(t) < a.cpg) gch[t] = g_t;
     lds_barrier();
@@ -689,7 +712,6 @@ gn_planes_masked_bwd_kernel(const GroupPlanesArgs g) {
       s1 = fmaf(gch[c], py, s1);
       t2 = fmaf(gch[c], px, t2);
     }
-    (void)nw;
 #pragma unroll
     for (int k = 0; k < NL; ++k) {
       keep_packed<T, VEC>(xr[k]);
@@ -793,18 +815,19 @@ MaskedCfg pick_masked(int64_t nv, int min_tpr = 8) {
 // group's channels times the threads of a plane exceed a block.
 struct PlanesCfg {
   bool ok = false;
-  int tpp_shift = 6, nl = 1;
+  int tpp_shift = 6, nl = 1; // (shift 3 - 5: several planes per wave)
 };
 
 PlanesCfg pick_planes(const RowProblem &p, int vec, bool backward) {
   PlanesCfg c;
   const int64_t cpg = p.channels / p.groups;
-  if (cpg > 16 || !tune_int("ROW_MASKED_PLANES", 1)) return c;
+  if (cpg > 64 || !tune_int("ROW_MASKED_PLANES", 1)) return c;
   const int64_t nv = (p.spatial + 2 * vec - 2) / vec;
   int64_t best = 0;
-  for (int sh = 6; sh <= 10; ++sh) {
+  for (int sh = 3; sh <= 10; ++sh) {
     if ((cpg << sh) > 1024) break;
     for (int nl : {1, 2, 3, 4, 5, 6, 8}) {
+      if (sh < 6 && nl != 1 && nl != 2 && nl != 4) continue; // (the sub-wave layouts' cases)
       if (backward && nl > 6) continue; // (x and dy of 8 vectors: past 128 registers)
       const int64_t cap = static_cast<int64_t>(nl) << sh;
       if (cap >= nv && (!c.ok || cap < best)) {
@@ -841,21 +864,26 @@ bool masked_plan(const RowProblem &p, bool backward, MaskedCfg &cfg) {
 
 template <typename T, int VEC, bool BWD>
 int run_group_planes(const PlanesCfg &c, const GroupPlanesArgs &g, int grid, int block, hipStream_t st) {
-#define PLANES_CASE(NL)                                                                            \
-  if (c.nl == (NL)) {                                                                              \
+  const int sub = c.tpp_shift < 6 ? 1 << c.tpp_shift : 0;
+#define PLANES_CASE(NL, SUB)                                                                       \
+  if (c.nl == (NL) && sub == (SUB)) {                                                              \
     if constexpr (BWD) {                                                                           \
-      NBLAHIP_LAUNCH("gn_planes_masked_bwd_kernel", (gn_planes_masked_bwd_kernel<T, VEC, NL>),     \
+      NBLAHIP_LAUNCH("gn_planes_masked_bwd_kernel", (gn_planes_masked_bwd_kernel<T, VEC, NL, SUB>),\
                      dim3(grid), dim3(block), 0, st, g);                                           \
     } else {                                                                                       \
-      NBLAHIP_LAUNCH("gn_planes_masked_fwd_kernel", (gn_planes_masked_fwd_kernel<T, VEC, NL>),     \
+      NBLAHIP_LAUNCH("gn_planes_masked_fwd_kernel", (gn_planes_masked_fwd_kernel<T, VEC, NL, SUB>),\
                      dim3(grid), dim3(block), 0, st, g);                                           \
     }                                                                                              \
     return last_launch_status();                                                                   \
   }
-  PLANES_CASE(1) PLANES_CASE(2) PLANES_CASE(3) PLANES_CASE(4) PLANES_CASE(5) PLANES_CASE(6)
+  PLANES_CASE(1, 0) PLANES_CASE(2, 0) PLANES_CASE(3, 0) PLANES_CASE(4, 0) PLANES_CASE(5, 0)
+  PLANES_CASE(6, 0)
   if constexpr (!BWD) {
-    PLANES_CASE(8)
+    PLANES_CASE(8, 0)
   }
+  PLANES_CASE(1, 8) PLANES_CASE(2, 8) PLANES_CASE(4, 8)
+  PLANES_CASE(1, 16) PLANES_CASE(2, 16) PLANES_CASE(4, 16)
+  PLANES_CASE(1, 32) PLANES_CASE(2, 32) PLANES_CASE(4, 32)
 #undef PLANES_CASE
   return NBLAHIP_EINVAL;
 }
