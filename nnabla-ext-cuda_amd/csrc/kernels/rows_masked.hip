@@ -823,20 +823,28 @@ PlanesCfg pick_planes(const RowProblem &p, int vec, bool backward) {
   const int64_t cpg = p.channels / p.groups;
   if (cpg > 64 || !tune_int("ROW_MASKED_PLANES", 1)) return c;
   const int64_t nv = (p.spatial + 2 * vec - 2) / vec;
-  int64_t best = 0;
-  for (int sh = 3; sh <= 10; ++sh) {
-    if ((cpg << sh) > 1024) break;
-    for (int nl : {1, 2, 3, 4, 5, 6, 8}) {
-      if (sh < 6 && nl != 1 && nl != 2 && nl != 4) continue; // (the sub-wave layouts' cases)
-      if (backward && nl > 6) continue; // (x and dy of 8 vectors: past 128 registers)
-      const int64_t cap = static_cast<int64_t>(nl) << sh;
-      if (cap >= nv && (!c.ok || cap < best)) {
-        c.ok = true;
-        c.tpp_shift = sh;
-        c.nl = nl;
-        best = cap;
+  // The backward holds x and dy: 8 vectors of each are past 128 registers (52 -
+  // 64 bytes of spills).  Taken for half data where nothing smaller fits
+  // ([8,128,127,127] G=32: 27.6 against 32.1 us through the boundary-splitting
+  // kernel; float [16,256,63,63]: 55.8 against 51.8 us, so not there).
+  for (int most : {6, 8}) {
+    if (most == 8 && backward && p.dtype != NBLAHIP_F16) break;
+    int64_t best = 0;
+    for (int sh = 3; sh <= 10; ++sh) {
+      if ((cpg << sh) > 1024) break;
+      for (int nl : {1, 2, 3, 4, 5, 6, 8}) {
+        if (sh < 6 && nl != 1 && nl != 2 && nl != 4) continue; // (the sub-wave layouts' cases)
+        if (backward && nl > most) continue;
+        const int64_t cap = static_cast<int64_t>(nl) << sh;
+        if (cap >= nv && (!c.ok || cap < best)) {
+          c.ok = true;
+          c.tpp_shift = sh;
+          c.nl = nl;
+          best = cap;
+        }
       }
     }
+    if (c.ok || !backward) break;
   }
   return c;
 }
@@ -878,9 +886,7 @@ int run_group_planes(const PlanesCfg &c, const GroupPlanesArgs &g, int grid, int
   }
   PLANES_CASE(1, 0) PLANES_CASE(2, 0) PLANES_CASE(3, 0) PLANES_CASE(4, 0) PLANES_CASE(5, 0)
   PLANES_CASE(6, 0)
-  if constexpr (!BWD) {
-    PLANES_CASE(8, 0)
-  }
+  PLANES_CASE(8, 0)
   PLANES_CASE(1, 8) PLANES_CASE(2, 8) PLANES_CASE(4, 8)
   PLANES_CASE(1, 16) PLANES_CASE(2, 16) PLANES_CASE(4, 16)
   PLANES_CASE(1, 32) PLANES_CASE(2, 32) PLANES_CASE(4, 32)

@@ -178,7 +178,7 @@ GN_SHAPES = [(2, 8, (8, 8), 4), (3, 6, (5,), 2), (1, 4, (2, 2), 1), (2, 6, (4,),
              (2, 256, (63, 63), 32), (1, 24, (65, 65), 3), (3, 9, (31, 33), 3), (2, 12, (127, 9), 2),
              # ... several planes per wave (8, 16, 32 threads per plane), up to 64 channels per group
              (4, 1280, (15, 15), 32), (8, 512, (7, 7), 32), (4, 60, (9, 9), 6), (3, 48, (5, 5), 3),
-             (2, 128, (11, 13), 2), (2, 40, (17, 19), 1)]
+             (2, 128, (11, 13), 2), (2, 40, (17, 19), 1), (2, 8, (127, 127), 2)]
 
 
 def make_nc(n, c, sp, dtype, seed):
