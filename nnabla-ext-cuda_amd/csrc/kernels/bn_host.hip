@@ -507,6 +507,7 @@ int launch_bn_fwd_train(const BnProblem &p, hipStream_t st) {
   if (bn_rows_fwd_train(p, st, &status)) return status;
   if (bn_chan_split_fwd_train(p, st, &status)) return status;
   if (bn_onchip_fwd_train(p, st, &status)) return status;
+  if (bn_masked_fwd_train(p, st, &status)) return status;
   if (bn_cl_cached_fwd_train(p, st, &status)) return status;
   if (bn_cl_grid_fwd_train(p, st, &status)) return status;
   if (bn_cl_split_fwd_train(p, st, &status)) return status;
@@ -535,6 +536,7 @@ int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
     if (bn_rows_bwd(p, st, &status)) return status;
     if (bn_chan_split_bwd(p, st, &status)) return status;
     if (bn_onchip_bwd(p, st, &status)) return status;
+    if (bn_masked_bwd(p, st, &status)) return status;
     if (bn_cl_cached_bwd(p, st, &status)) return status;
     if (bn_cl_grid_bwd(p, st, &status)) return status;
     if (bn_cl_split_bwd(p, st, &status)) return status;

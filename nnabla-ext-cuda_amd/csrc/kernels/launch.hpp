@@ -160,6 +160,10 @@ bool bn_cl_split_bwd(const BnProblem &p, hipStream_t st, int *status);
 // (bn_split_channel.hip).
 bool bn_chan_split_fwd_train(const BnProblem &p, hipStream_t st, int *status);
 bool bn_chan_split_bwd(const BnProblem &p, hipStream_t st, int *status);
+// Planes that are no whole number of vectors, a channel held by one block
+// (rows_masked.hip); false: not taken.
+bool bn_masked_fwd_train(const BnProblem &p, hipStream_t st, int *status);
+bool bn_masked_bwd(const BnProblem &p, hipStream_t st, int *status);
 bool bn_pack_fwd_train(const BnProblem &p, hipStream_t st, int *status);
 bool bn_pack_bwd(const BnProblem &p, hipStream_t st, int *status);
 int launch_bn_infer(const BnProblem &p, hipStream_t st);

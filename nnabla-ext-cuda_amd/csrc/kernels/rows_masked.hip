@@ -23,6 +23,7 @@
 
 #include "common.cuh"
 #include "launch.hpp"
+#include "onchip.cuh"
 #include "rows.cuh"
 #include "rows_dispatch.hpp"
 
@@ -736,6 +737,194 @@ gn_planes_masked_bwd_kernel(const GroupPlanesArgs g) {
   }
 }
 
+// BatchNormalization (planes layout) over planes that are no whole number of
+// vectors (17 x 17, 35 x 35): a block holds its channel - the N planes (n, c),
+// each taken through the tensor's aligned vectors with masked edges as above -
+// in registers between the statistics and the normalization: 2 S forward and
+// 3 S backward in one launch each, the channel's dgamma / dbeta written by the
+// block itself.  The split reduction these shapes took otherwise reads x twice
+// through three launches per direction.
+struct BnMaskedArgs {
+  const void *x;
+  const void *dy;
+  void *out;
+  const float *gamma, *beta;
+  float *bmean, *bvar;       // forward: the batch statistics, written
+  float *rmean, *rvar;       // forward: running statistics, may be null
+  const float *mean, *var;   // backward: read
+  const float *dmean, *dvar; // may be null
+  float *dgamma, *dbeta;     // may be null
+  uint32_t N, C, HW;
+  uint32_t nvp; // vectors a plane can meet = (HW + 2 * VEC - 2) / VEC
+  FastDiv nvpd;
+  long long total;
+  float inv_cnt, unbias, decay, eps, one;
+  int accum_dx, accum_g, accum_b;
+};
+
+// Piece i of channel c: vector i % nvp of plane i / nvp.
+template <int VEC>
+__device__ __forceinline__ RowPiece bn_piece(const BnMaskedArgs &a, uint32_t c, uint32_t i, size_t &base,
+                                             int &head) {
+  const uint32_t n = a.nvpd.div(i);
+  const uint32_t v = i - n * a.nvp;
+  const bool plane = n < a.N;
+  base = (static_cast<size_t>(plane ? n : 0u) * a.C + c) * a.HW;
+  head = static_cast<int>(base % VEC);
+  RowPiece p;
+  p.col = static_cast<int>(v) * VEC - head;
+  p.ok = plane && p.col < static_cast<int>(a.HW);
+  p.lo = p.col < 0 ? -p.col : 0;
+  p.hi = min(VEC, static_cast<int>(a.HW) - p.col);
+  p.tail = static_cast<long long>(base) + p.col + VEC > a.total;
+  return p;
+}
+
+// TB threads per block: 1024, or 256 for channels of few vectors (several
+// blocks to a CU then, one's sums under another's loads).
+template <typename T, int VEC, int NL, int TB>
+__global__ void __launch_bounds__(TB)
+bn_masked_fwd_kernel(const BnMaskedArgs a) {
+  __shared__ float red[TB / kWave];
+  const uint32_t t = threadIdx.x;
+  const T *__restrict__ x = static_cast<const T *>(a.x);
+  T *__restrict__ y = static_cast<T *>(a.out);
+  for (uint32_t c = blockIdx.x; c < a.C; c += gridDim.x) {
+    const float gam = a.gamma ? a.gamma[c] : 1.f;
+    const float bet = a.beta ? a.beta[c] : 0.f;
+    const float rm = a.rmean ? a.rmean[c] : 0.f;
+    const float rv = a.rvar ? a.rvar[c] : 0.f;
+    RawVec<T, VEC> raw[NL];
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      size_t base;
+      int head;
+      const RowPiece p = bn_piece<VEC>(a, c, k * TB + t, base, head);
+      raw[k] = load_piece<T, VEC>(x + base, head, p);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) s = raw_sum<T, VEC>(raw[k], s);
+    const float mean = onchip_block_sum<TB>(s, red) * a.inv_cnt;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+    float q = 0.f;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      size_t base;
+      int head;
+      const RowPiece p = bn_piece<VEC>(a, c, k * TB + t, base, head);
+      if (p.ok) {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float d = elem_fma<T, VEC>(raw[k], j, a.one, -mean);
+          q = (j >= p.lo && j < p.hi) ? fmaf(d, d, q) : q;
+        }
+      }
+    }
+    const float var = onchip_block_sum<TB>(q, red) * a.inv_cnt;
+    const float istd = inv_std(var, a.eps);
+    if (t == 0) {
+      a.bmean[c] = mean;
+      a.bvar[c] = var;
+      if (a.rmean) a.rmean[c] = a.decay * rm + (1.f - a.decay) * mean;
+      if (a.rvar) a.rvar[c] = a.decay * rv + (1.f - a.decay) * var * a.unbias;
+    }
+#pragma unroll
+    for (int k = 0; k < NL; ++k) keep_packed<T, VEC>(raw[k]);
+    const float gs = gam * istd;
+    const float sh = fmaf(-mean, gs, bet);
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      size_t base;
+      int head;
+      const RowPiece p = bn_piece<VEC>(a, c, k * TB + t, base, head);
+      if (p.ok) {
+        float o[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          if constexpr (sizeof(T) == 2) {
+            o[j] = elem_fma<T, VEC>(raw[k], j, gs, sh);
+          } else {
+            o[j] = fmaf(elem_fma<T, VEC>(raw[k], j, a.one, -mean), gs, bet);
+          }
+        }
+        store_piece<T, VEC>(y + base, p, o, 0);
+      }
+    }
+  }
+}
+
+template <typename T, int VEC, int NL, int TB>
+__global__ void __launch_bounds__(TB)
+bn_masked_bwd_kernel(const BnMaskedArgs a) {
+  __shared__ float red[TB / kWave];
+  const uint32_t t = threadIdx.x;
+  const T *__restrict__ x = static_cast<const T *>(a.x);
+  const T *__restrict__ dy = static_cast<const T *>(a.dy);
+  T *dx = static_cast<T *>(a.out);
+  for (uint32_t c = blockIdx.x; c < a.C; c += gridDim.x) {
+    const float gam = a.gamma ? a.gamma[c] : 1.f;
+    const float mean = a.mean[c];
+    const float vpe = a.var[c] + a.eps;
+    const float u_dvar = a.dvar ? a.dvar[c] : 0.f;
+    const float u_dmean = a.dmean ? a.dmean[c] : 0.f;
+    const float old_g = (a.dgamma && a.accum_g) ? a.dgamma[c] : 0.f;
+    const float old_b = (a.dbeta && a.accum_b) ? a.dbeta[c] : 0.f;
+    RawVec<T, VEC> xr[NL], dr[NL];
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      size_t base;
+      int head;
+      const RowPiece p = bn_piece<VEC>(a, c, k * TB + t, base, head);
+      xr[k] = load_piece<T, VEC>(x + base, head, p);
+      dr[k] = load_piece<T, VEC>(dy + base, head, p);
+    }
+    const float istd = 1.0f / sqrtf(vpe);
+    const float nmi = -mean * istd;
+    float sdy = 0.f, sdx = 0.f;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      sdy = raw_sum<T, VEC>(dr[k], sdy);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+        sdx = elem_fma<T, VEC>(dr[k], j, xh, sdx);
+      }
+    }
+    sdx = onchip_block_sum<TB>(sdx, red);
+    sdy = onchip_block_sum<TB>(sdy, red);
+    if (t == 0) {
+      if (a.dgamma) a.dgamma[c] = sdx + old_g;
+      if (a.dbeta) a.dbeta[c] = sdy + old_b;
+    }
+    if (dx == nullptr) continue;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      keep_packed<T, VEC>(xr[k]);
+      keep_packed<T, VEC>(dr[k]);
+    }
+    const float cA = -istd * gam * sdx * a.inv_cnt + (a.dvar ? 2.f * u_dvar * (vpe * istd) * a.inv_cnt : 0.f);
+    const float cb = -gam * sdy * istd * a.inv_cnt + (a.dmean ? u_dmean * a.inv_cnt : 0.f);
+    const float gi = gam * istd;
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      size_t base;
+      int head;
+      const RowPiece p = bn_piece<VEC>(a, c, k * TB + t, base, head);
+      if (p.ok) {
+        float o[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float xh = norm_elem<T, VEC>(xr[k], j, mean, istd, nmi);
+          o[j] = elem_fma<T, VEC>(dr[k], j, gi, fmaf(xh, cA, cb));
+        }
+        store_piece<T, VEC>(dx + base, p, o, a.accum_dx);
+      }
+    }
+  }
+}
+
 namespace {
 
 MaskedRowArgs masked_args(const RowProblem &p) {
@@ -1006,6 +1195,113 @@ bool row_masked_bwd(const RowProblem &p, hipStream_t st, int *status) {
   const int grid = masked_grid(p.rows, c.tpr);
   *status = p.dtype == NBLAHIP_F16 ? run_masked<__half, 8, true>(c, a, grid, st)
                                    : run_masked<float, 4, true>(c, a, grid, st);
+  return true;
+}
+
+namespace {
+
+// Eligibility and arguments of the masked BatchNormalization kernels; nl =
+// vectors per thread, tb = threads per block.
+bool bn_masked_args(const BnProblem &p, bool backward, BnMaskedArgs &a, int &nl, int &tb) {
+  if (!tune_int("BN_MASKED_ONCHIP", 1)) return false;
+  if (p.relu || p.z || p.y || p.dz || p.sums_out || p.sums_in) return false;
+  const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
+  if (p.size2 % vec == 0 || p.size2 < 2 * vec || p.size0 < 1) return false;
+  if (!aligned16(p.x) || (p.out && !aligned16(p.out)) || (backward && !aligned16(p.dy))) return false;
+  const int64_t total = p.size0 * p.C * p.size2;
+  if (total >= (int64_t{1} << 31)) return false;
+  const int64_t nvp = (p.size2 + 2 * vec - 2) / vec;
+  const int64_t pieces = p.size0 * nvp;
+  // (beyond: x, or x and dy, no longer fit the registers of a 1024-thread block)
+  const int most = backward ? 5 : (p.dtype == NBLAHIP_F16 ? 8 : 6);
+  tb = (pieces + 255) / 256 <= most ? 256 : kOnchipBlock;
+  nl = static_cast<int>((pieces + tb - 1) / tb);
+  if (nl > most) return false;
+  // (fewer channels than this share of the CUs: most of the chip would idle)
+  if (p.C * 100 < static_cast<int64_t>(device_cus()) * tune_int("BN_MASKED_ONCHIP_MIN_PCT", 25)) return false;
+  a = BnMaskedArgs{};
+  a.x = p.x;
+  a.dy = p.dy;
+  a.out = p.out;
+  a.gamma = p.gamma;
+  a.beta = p.beta;
+  a.bmean = p.batch_mean;
+  a.bvar = p.batch_var;
+  a.rmean = p.rmean;
+  a.rvar = p.rvar;
+  a.mean = p.mean;
+  a.var = p.var;
+  a.dmean = p.dmean;
+  a.dvar = p.dvar;
+  a.dgamma = p.dgamma;
+  a.dbeta = p.dbeta;
+  a.N = static_cast<uint32_t>(p.size0);
+  a.C = static_cast<uint32_t>(p.C);
+  a.HW = static_cast<uint32_t>(p.size2);
+  a.nvp = static_cast<uint32_t>(nvp);
+  a.nvpd = FastDiv(a.nvp);
+  a.total = total;
+  const double cnt = static_cast<double>(p.size0) * static_cast<double>(p.size2);
+  a.inv_cnt = static_cast<float>(1.0 / cnt);
+  a.unbias = static_cast<float>(cnt / std::max(cnt - 1.0, 1.0));
+  a.decay = p.decay;
+  a.eps = p.eps;
+  a.one = 1.0f;
+  a.accum_dx = p.accum_dx;
+  a.accum_g = p.accum_g;
+  a.accum_b = p.accum_b;
+  return true;
+}
+
+template <typename T, int VEC, bool BWD, int TB>
+int run_bn_masked(int nl, const BnMaskedArgs &a, unsigned grid, hipStream_t st) {
+#define BN_MASKED_CASE(NL)                                                                         \
+  if (nl <= (NL)) {                                                                                \
+    if constexpr (BWD) {                                                                           \
+      NBLAHIP_LAUNCH("bn_masked_bwd_kernel", (bn_masked_bwd_kernel<T, VEC, NL, TB>), dim3(grid),   \
+                     dim3(TB), 0, st, a);                                                          \
+    } else {                                                                                       \
+      NBLAHIP_LAUNCH("bn_masked_fwd_kernel", (bn_masked_fwd_kernel<T, VEC, NL, TB>), dim3(grid),   \
+                     dim3(TB), 0, st, a);                                                          \
+    }                                                                                              \
+    return last_launch_status();                                                                   \
+  }
+  BN_MASKED_CASE(1) BN_MASKED_CASE(2) BN_MASKED_CASE(3) BN_MASKED_CASE(4) BN_MASKED_CASE(5)
+  if constexpr (!BWD) {
+    BN_MASKED_CASE(6)
+    if constexpr (sizeof(T) == 2) {
+      BN_MASKED_CASE(8)
+    }
+  }
+#undef BN_MASKED_CASE
+  return NBLAHIP_EINVAL;
+}
+
+template <bool BWD>
+int launch_bn_masked(const BnProblem &p, int nl, int tb, const BnMaskedArgs &a, hipStream_t st) {
+  const unsigned grid = static_cast<unsigned>(std::min<int64_t>(p.C, 1 << 20));
+  if (p.dtype == NBLAHIP_F16)
+    return tb == 256 ? run_bn_masked<__half, 8, BWD, 256>(nl, a, grid, st)
+                     : run_bn_masked<__half, 8, BWD, kOnchipBlock>(nl, a, grid, st);
+  return tb == 256 ? run_bn_masked<float, 4, BWD, 256>(nl, a, grid, st)
+                   : run_bn_masked<float, 4, BWD, kOnchipBlock>(nl, a, grid, st);
+}
+
+} // namespace
+
+bool bn_masked_fwd_train(const BnProblem &p, hipStream_t st, int *status) {
+  BnMaskedArgs a;
+  int nl = 0, tb = 0;
+  if (!p.out || !p.batch_mean || !p.batch_var || !bn_masked_args(p, false, a, nl, tb)) return false;
+  *status = launch_bn_masked<false>(p, nl, tb, a, st);
+  return true;
+}
+
+bool bn_masked_bwd(const BnProblem &p, hipStream_t st, int *status) {
+  BnMaskedArgs a;
+  int nl = 0, tb = 0;
+  if (!p.batch_stat || !p.mean || !p.var || !bn_masked_args(p, true, a, nl, tb)) return false;
+  *status = launch_bn_masked<true>(p, nl, tb, a, st);
   return true;
 }
 

@@ -51,6 +51,11 @@ SMALL = [
     ((32, 16, 112, 112), 1), ((64, 64, 56, 56), 1), ((84, 64, 56, 56), 1),
     # a channel per CU whose planes share cache lines with the neighbouring channels'
     ((256, 64, 14, 14), 1), ((250, 40, 10, 10), 1),
+    # planes that are no whole number of vectors, a channel held by one block through the
+    # tensor's aligned vectors with masked edges: one to eight vectors per thread, a
+    # tensor that ends inside a vector
+    ((32, 288, 35, 35), 1), ((32, 768, 17, 17), 1), ((7, 96, 17, 17), 1), ((3, 70, 9, 11), 1),
+    ((64, 160, 17, 17), 1), ((5, 65, 3, 7), 1), ((40, 64, 35, 35), 1),
 ]
 DTYPES = [torch.float32, torch.float16]
 
@@ -109,6 +114,8 @@ def test_bn_training_forward_backward(shape, axis, dtype):
                                         ((8, 64, 12, 12), 1), ((4, 48, 7, 9), 1), ((3, 300, 2, 2), 1),
                                         # a pack of channels per block (planes of 49 elements)
                                         ((90, 256, 7, 7), 1),
+                                        # odd planes, a channel held by one block
+                                        ((6, 80, 17, 17), 1),
                                         # a channel split over 4 blocks
                                         ((40, 64, 32, 32), 1),
                                         # channel-last through the split kernels
@@ -389,6 +396,7 @@ def check_channel_on_chip(shape, dtype):
 @pytest.mark.parametrize("shape,axis,dtype", [
     ((8, 12, 14, 14), 1, torch.float32),      # split reduction
     ((8, 64, 12, 12), 1, torch.float32),      # channel in one block's registers
+    ((9, 72, 17, 17), 1, torch.float16),      # odd planes, a channel held by one block
     ((37, 64, 32, 32), 1, torch.float32),     # channel held on one CU
     ((131, 232, 16, 32), 1, torch.float16),   # ... with a streamed remainder
     ((8, 7, 7, 256), 3, torch.float16),       # channel-last, column in registers

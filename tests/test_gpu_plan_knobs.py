@@ -167,18 +167,22 @@ SWITCHES = [
     ("bn_chan_split_off", run_bn, ((32, 64, 56, 56), 1, F16), {"BN_CHAN_SPLIT": 0},
      ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"],
      ["bn_chan_split_fwd_kernel", "bn_chan_split_bwd_kernel"]),
-    ("bn_rows_off", run_bn, ((32, 64, 14, 14), 1, F16), {"BN_ROWS": 0},
+    ("bn_rows_off", run_bn, ((32, 64, 14, 14), 1, F16), {"BN_ROWS": 0, "BN_MASKED_ONCHIP": 0},
      ["bn_stats_planes_kernel", "bn_finalize_fwd_kernel", "bn_apply_planes_kernel",
       "bn_finalize_bwd_kernel"], ["row_fwd_kernel_bn", "row_bwd_kernel_bn"]),
-    ("bn_pack_off", run_bn, ((96, 256, 7, 7), 1, F16), {"BN_PACK": 0},
+    ("bn_pack_off", run_bn, ((96, 256, 7, 7), 1, F16), {"BN_PACK": 0, "BN_MASKED_ONCHIP": 0},
      ["bn_stats_planes_kernel", "bn_bwd_reduce_planes_kernel"], ["bn_pack_fwd_kernel", "bn_pack_bwd_kernel"]),
-    ("bn_pack_min_pct_up", run_bn, ((96, 256, 7, 7), 1, F16), {"BN_PACK_MIN_PCT": 50},
+    ("bn_pack_min_pct_up", run_bn, ((96, 256, 7, 7), 1, F16), {"BN_PACK_MIN_PCT": 50, "BN_MASKED_ONCHIP": 0},
      ["bn_stats_planes_kernel"], ["bn_pack_fwd_kernel", "bn_pack_bwd_kernel"]),
     ("bn_cl_grid_off", run_bn, ((100352, 64), 1, F16), {"BN_CL_GRID": 0},
      ["bn_stats_cl_kernel", "bn_finalize_fwd_kernel", "bn_apply_cl_kernel"], ["bn_cl_grid_fwd_kernel"],
      {"BN_CL_GRID_MIN_SLOTS": 1}),
     ("bn_cl_grid_from_fewer_vectors", run_bn, ((100352, 64), 1, F16), {"BN_CL_GRID_MIN_SLOTS": 1},
      ["bn_cl_grid_fwd_kernel"], ["bn_stats_cl_kernel"]),
+    ("bn_masked_onchip_off", run_bn, ((64, 160, 17, 17), 1, F16), {"BN_MASKED_ONCHIP": 0},
+     ["bn_apply_planes_kernel"], ["bn_masked_fwd_kernel", "bn_masked_bwd_kernel"]),
+    ("bn_masked_onchip_min_pct_up", run_bn, ((64, 160, 17, 17), 1, F32), {"BN_MASKED_ONCHIP_MIN_PCT": 80},
+     ["bn_apply_planes_kernel"], ["bn_masked_fwd_kernel", "bn_masked_bwd_kernel"]),
     ("bn_cl_grid_wide_off", run_bn, ((256, 14, 14, 256), 3, F16), {"BN_CL_GRID_WIDE": 0},
      ["cl_split_fwd_kernel", "bn_bwd_reduce_cl_kernel"], ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"]),
     ("bn_cl_grid_wide_from_more_rows", run_bn, ((256, 14, 14, 256), 3, F32), {"BN_CL_GRID_WIDE_MIN_ROWS": 60000},
@@ -302,7 +306,8 @@ GRIDS = [
     ("bn_apply_persistent", run_bn, ((16, 48, 28, 28), 1, F32),
      [{"BN_ROWS": 0, "BN_APPLY_BLOCKS_PER_CU": v} for v in (1, 3)],
      ["bn_apply_planes_kernel", "bn_bwd_apply_planes_kernel"], []),
-    ("bn_masked_planes_off", run_bn, ((64, 64, 7, 7), 1, F16), [{"BN_ROWS": 0, "BN_MASKED_PLANES": 0}],
+    ("bn_masked_planes_off", run_bn, ((64, 64, 7, 7), 1, F16),
+     [{"BN_ROWS": 0, "BN_MASKED_PLANES": 0, "BN_MASKED_ONCHIP": 0}],
      ["bn_stats_planes_kernel", "bn_apply_planes_kernel"], []),
     ("bn_cl_grids", run_bn, ((64, 28, 28, 64), 3, F16),
      [{"BN_CL_BLOCKS_PER_CU": a, "BN_CL_FWD_APPLY_BLOCKS_PER_CU": b, "BN_CL_APPLY_BLOCKS_PER_CU": c,
