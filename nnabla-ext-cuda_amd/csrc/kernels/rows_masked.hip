@@ -18,7 +18,12 @@
 // route (gn_masked_*): a row is a group's planes, a vector may hold the end of
 // one channel and the start of the next, so gamma / beta are picked per element
 // (one boundary per vector at most: planes of VEC elements and more) and the
-// backward's per-channel sums are split at that boundary.
+// backward's per-channel sums are split at that boundary.  Where a group's
+// planes fit a block side by side (gn_planes_masked_*), every plane has threads
+// of its own and the planes meet only in the sums.
+//
+// BatchNormalization in the planes layout (bn_masked_*): a block holds its
+// channel, the N planes (n, c), through the same pieces.
 #include <algorithm>
 
 #include "common.cuh"
