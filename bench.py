@@ -44,7 +44,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 # One lap over a workload's buffer sets must exceed L2 (8 x 4 MB) plus the
-# Infinity Cache (256 MB), with room to spare.
+# Infinity Cache (256 MB), with room to spare; --lap-mb sets another lap (the
+# sensitivity of the cold figures to the lap is what shows whether a cyclic
+# walk of this size really misses the memory-side cache).
 LAP_BYTES = 352 << 20
 
 
@@ -442,7 +444,9 @@ def config_table(K, steps, warmup, only=None):
         if only and only not in name:
             continue
         w = make(name)
-        row = {"config": name, "buffer_sets": w.nsets}
+        row = {"config": name, "buffer_sets": w.nsets,
+               "lap_bytes": sum(t.numel() * t.element_size() for s_ in w.sets
+                                for t in s_.values() if t is not None)}
         legs = [("fwd", [w.fwd], w.fwd_bytes)]
         if w.bwd is not None:
             legs += [("bwd", [w.bwd], w.bwd_bytes), ("fwd_bwd", [w.fwd, w.bwd], w.fwd_bytes + w.bwd_bytes)]
@@ -649,6 +653,8 @@ def main():
     ap.add_argument("--only", default=None, help="table rows whose name contains this text")
     ap.add_argument("--torch-native", action="store_true",
                     help="also time torch's own normalization kernels on the same shapes")
+    ap.add_argument("--lap-mb", type=int, default=LAP_BYTES >> 20,
+                    help="bytes (MiB) one lap over a workload's rotated buffer sets must exceed")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a float32->float16 convert of the workload's x (a plain "
                          "streaming kernel of known traffic: 4 B read, 2 B written per element) "
@@ -659,6 +665,9 @@ def main():
               "batch; the exchange between shards belongs to the caller's communicator)",
               file=sys.stderr)
         sys.exit(2)
+
+    global LAP_BYTES
+    LAP_BYTES = max(1, args.lap_mb) << 20
 
     import torch
     K = load_package()
@@ -734,6 +743,7 @@ def main():
                                              "between statistics and apply"},
                    "buffer_sets": w.nsets,
                    "lap_bytes": w.nsets * 4 * S,
+                   "lap_floor_bytes": LAP_BYTES,
                    "median_us": round(med_us, 2), "min_us": round(min_us, 2),
                    "warm_ms_per_step": round(warm_ms, 5),
                    "warm_GBps": round((fb + bb) / warm_ms / 1e6, 1),

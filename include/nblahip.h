@@ -59,6 +59,14 @@ NBLAHIP_EXPORT int nblahip_abi_version(void);
  * BatchNormalization.  x is viewed as [size0, size1, size2] with size1 = C the
  * normalised axis (src/nbla/cuda/function/generic/batch_normalization.cu:34-35,
  * 53-55); size2 == 1 is the channel-last layout.  N = size0*size2.
+ *
+ * Aliasing: y may be x itself (in place), dx may be x or dy itself; an output
+ * that overlaps an input tensor only in part is rejected with NBLAHIP_EALIAS
+ * before anything is launched.  In-place calls never take the kernels whose
+ * blocks exchange partial sums (a block that gives up waiting for a partner
+ * reads the partner's part of the inputs again, which the partner would
+ * already be overwriting): they run on the plans without an exchange, with
+ * the same results within the summation order.
  * ---------------------------------------------------------------------- */
 
 /* Replaces forward_impl_global + forward_global_kernel
@@ -336,6 +344,9 @@ NBLAHIP_EXPORT int nblahip_in_bwd(const void *x, const void *dy,
  * and write the channel-last tensor in place of those transposes.  Results
  * equal the channel-first entry points applied to the transposed tensor.
  * Both directions need a workspace of *_cl_workspace_bytes; batch <= 65535.
+ * Aliasing as for BatchNormalization: y == x, dx == x and dx == dy are in-place
+ * calls and run on the kernels without an exchange between blocks; a partial
+ * overlap is rejected with NBLAHIP_EALIAS.
  * ---------------------------------------------------------------------- */
 NBLAHIP_EXPORT size_t nblahip_gn_cl_workspace_bytes(int64_t batch,
                                                     int64_t spatial,

@@ -225,13 +225,15 @@ def bn_forward_global(x, beta, gamma, rmean, rvar, axis=1, eps=1e-5):
     return y
 
 
-def bn_forward_batch(x, beta, gamma, rmean, rvar, axis=1, decay_rate=0.9, eps=1e-5, ws=None):
-    """Returns y, batch_mean, batch_var; rmean/rvar are updated in place."""
+def bn_forward_batch(x, beta, gamma, rmean, rvar, axis=1, decay_rate=0.9, eps=1e-5, ws=None,
+                     y=None):
+    """Returns y, batch_mean, batch_var; rmean/rvar are updated in place.
+    y: the output tensor (x itself for an in-place call); allocated when None."""
     import torch
     assert x.is_contiguous()
     s0, c, s2 = _bn_sizes(x.shape, axis)
     dt = _dtype_code(x)
-    y = torch.empty_like(x)
+    y = torch.empty_like(x) if y is None else y
     mean = torch.empty(c, dtype=torch.float32, device=x.device)
     var = torch.empty(c, dtype=torch.float32, device=x.device)
     need = lib().nblahip_bn_workspace_bytes(s0, c, s2, dt)
@@ -453,11 +455,11 @@ def _ncs(x, channel_last=False):
     return n, c, sp
 
 
-def gn_forward(x, beta, gamma, num_groups, eps=1e-5, channel_last=False, ws=None):
+def gn_forward(x, beta, gamma, num_groups, eps=1e-5, channel_last=False, ws=None, y=None):
     import torch
     assert x.is_contiguous()
     n, c, sp = _ncs(x, channel_last)
-    y = torch.empty_like(x)
+    y = torch.empty_like(x) if y is None else y
     mean = torch.empty(n * num_groups, dtype=torch.float32, device=x.device)
     var = torch.empty(n * num_groups, dtype=torch.float32, device=x.device)
     if channel_last:
@@ -508,11 +510,11 @@ def gn_backward(x, dy, gamma, mean, var, num_groups, eps=1e-5, dmean=None, dvar=
 
 
 def in_forward(x, beta, gamma, eps=1e-5, bc_gamma=True, bc_beta=True, channel_last=False,
-               ws=None):
+               ws=None, y=None):
     import torch
     assert x.is_contiguous()
     n, c, sp = _ncs(x, channel_last)
-    y = torch.empty_like(x)
+    y = torch.empty_like(x) if y is None else y
     mean = torch.empty(n * c, dtype=torch.float32, device=x.device)
     var = torch.empty(n * c, dtype=torch.float32, device=x.device)
     if channel_last:

@@ -52,6 +52,13 @@ int check_fwd_alias(const void *x, void *y, size_t tensor_bytes, const float *ga
 
 size_t elem_bytes(int dtype) { return dtype == NBLAHIP_F16 ? 2 : 4; }
 
+// An output tensor may be one of the call's input tensors itself (in place:
+// every kernel reads an element before the same thread writes it), but must
+// not overlap one in part.
+int check_in_place(const void *out, const void *in, size_t tensor_bytes) {
+  return out != in && ranges_overlap(out, tensor_bytes, in, tensor_bytes) ? NBLAHIP_EALIAS : 0;
+}
+
 // Scratch of nblahip_bn_fwd_train_static, the entry point for callers that
 // cannot allocate: one array per GPU in the code object's own data segment,
 // held until the process ends.  `scratch` below is only the host-side handle
@@ -95,6 +102,10 @@ int bn_fwd_infer_impl(const void *x, const void *z, int relu, const float *rmean
   const int d = check_dims3(size0, size1, size2);
   if (d) return d < 0 ? d : 0;
   if (!x || !y || !rmean || !rvar) return NBLAHIP_EINVAL;
+  {
+    const size_t tb = static_cast<size_t>(size0) * size1 * size2 * elem_bytes(dtype);
+    if (check_in_place(y, x, tb) || check_in_place(y, z, tb)) return NBLAHIP_EALIAS;
+  }
   BnProblem p;
   p.dtype = dtype;
   p.x = x;
@@ -121,6 +132,10 @@ int bn_fwd_train_impl(const void *x, const void *z, int relu, const float *gamma
   const int d = check_dims3(size0, size1, size2);
   if (d) return d < 0 ? d : 0;
   if (!x || !y || !batch_mean || !batch_var) return NBLAHIP_EINVAL;
+  {
+    const size_t tb = static_cast<size_t>(size0) * size1 * size2 * elem_bytes(dtype);
+    if (check_in_place(y, x, tb) || check_in_place(y, z, tb)) return NBLAHIP_EALIAS;
+  }
   if (int e = check_ws(workspace, workspace_bytes, bn_workspace_bytes(size0, size1, size2, dtype)))
     return e;
   BnProblem p;
@@ -156,6 +171,12 @@ int bn_bwd_impl(int fused, const void *x, const void *y_out, const void *dy, con
   if (d) return d < 0 ? d : 0;
   if (!x || !dy || !mean || !var) return NBLAHIP_EINVAL;
   if (fused ? !y_out : (y_out || dz)) return NBLAHIP_EINVAL;
+  {
+    const size_t tb = static_cast<size_t>(size0) * size1 * size2 * elem_bytes(dtype);
+    if (check_in_place(dx, x, tb) || check_in_place(dx, dy, tb) || check_in_place(dz, dy, tb) ||
+        ranges_overlap(dz, tb, x, tb))
+      return NBLAHIP_EALIAS;
+  }
   if (int e = check_ws(workspace, workspace_bytes, bn_workspace_bytes(size0, size1, size2, dtype)))
     return e;
   BnProblem p;
@@ -623,6 +644,8 @@ int cl_fwd(ClProblem &p, const void *x, const float *gamma, const float *beta, v
            float *mean, float *var, float eps, void *workspace, size_t workspace_bytes,
            void *stream) {
   if (!x || !y || !mean || !var) return NBLAHIP_EINVAL;
+  if (check_in_place(y, x, static_cast<size_t>(p.batch) * p.spatial * p.channels * elem_bytes(p.dtype)))
+    return NBLAHIP_EALIAS;
   if (int e = check_ws(workspace, workspace_bytes,
                        cl_workspace_bytes(p.batch, p.spatial, p.channels, p.dtype)))
     return e;
@@ -643,6 +666,10 @@ int cl_bwd(ClProblem &p, const void *x, const void *dy, const float *gamma, cons
            float *dbeta, int accum_dx, int accum_dgamma, int accum_dbeta, float eps,
            void *workspace, size_t workspace_bytes, void *stream) {
   if (!x || !dy || !mean || !var) return NBLAHIP_EINVAL;
+  {
+    const size_t tb = static_cast<size_t>(p.batch) * p.spatial * p.channels * elem_bytes(p.dtype);
+    if (check_in_place(dx, x, tb) || check_in_place(dx, dy, tb)) return NBLAHIP_EALIAS;
+  }
   if (int e = check_ws(workspace, workspace_bytes,
                        cl_workspace_bytes(p.batch, p.spatial, p.channels, p.dtype)))
     return e;

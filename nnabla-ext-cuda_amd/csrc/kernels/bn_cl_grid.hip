@@ -784,6 +784,10 @@ bool grid_args(const BnProblem &p, BnClGridArgs &a, int &nl) {
     return false;
   const int64_t cv = p.C / vec;
   if ((cv & (cv - 1)) != 0 || cv > kWave) return false;
+  // A block whose partner's word does not arrive reads the partner's rows of x
+  // (and dy) again, which the partner may already be overwriting in place.
+  const uint64_t tensor_bytes = static_cast<uint64_t>(p.size0 * p.C) * (p.dtype == NBLAHIP_F16 ? 2 : 4);
+  if (ranges_overlap(p.out, p.x, tensor_bytes) || ranges_overlap(p.out, p.dy, tensor_bytes)) return false;
   const int64_t M = p.size0;
   const int blocks = std::min(device_cus(), kGridMaxBlocks);
   // whole rows per block, the same for every block but the last

@@ -567,6 +567,11 @@ bool chan_split_args(const BnProblem &p, bool backward, BnChanSplitArgs &a, int 
   if (p.size2 % vec != 0 || !aligned16(p.x) || (p.out && !aligned16(p.out))) return false;
   if (backward && !aligned16(p.dy)) return false;
   if (p.size0 * p.C * p.size2 >= (int64_t{1} << 31)) return false;
+  // A block whose partner's word does not arrive reads the partner's part of x
+  // (and dy) again, which the partner may already be overwriting in place.
+  const uint64_t tensor_bytes = static_cast<uint64_t>(p.size0 * p.C * p.size2) * (p.dtype == NBLAHIP_F16 ? 2 : 4);
+  if (ranges_overlap(p.out, p.x, tensor_bytes) || (backward && ranges_overlap(p.out, p.dy, tensor_bytes)))
+    return false;
   // Short planes that share cache lines with the neighbouring channels' stay
   // with the kernels that put neighbouring channels on one XCD and store the
   // shared lines accordingly (bn_onchip.hip, the row kernels).

@@ -28,6 +28,11 @@ SplitPlan plan_split(const ClProblem &p, bool aligned, bool backward) {
   }
   if (!p.bc_gamma || !p.bc_beta) return s;
   const int esz = p.dtype == NBLAHIP_F16 ? 2 : 4;
+  // A block whose partner's word does not arrive reads the partner's part of x
+  // (and dy) again, which the partner may already be overwriting in place.
+  const uint64_t tensor_bytes = static_cast<uint64_t>(p.batch * p.spatial * p.channels) * esz;
+  if (ranges_overlap(p.out, p.x, tensor_bytes) || (backward && ranges_overlap(p.out, p.dy, tensor_bytes)))
+    return s;
   s.vec = 16 / esz;
   const int64_t tile_ch = static_cast<int64_t>(kSplitTV) * s.vec; // channels of a 128-byte line
   if (p.channels % tile_ch != 0) return s;

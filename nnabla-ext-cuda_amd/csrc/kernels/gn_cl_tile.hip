@@ -644,6 +644,10 @@ TilePlan plan_tile(const ClProblem &p, bool aligned, int max_nl) {
   if (!p.bc_gamma || !p.bc_beta || p.groups == p.channels) return pl;
   const int vec = p.dtype == NBLAHIP_F16 ? 8 : 4;
   if (p.channels % vec != 0 || p.channels > kTileMaxC || p.groups > kTileMaxG) return pl;
+  // A block whose partner's word does not arrive reads the partner's positions
+  // of x (and dy) again, which the partner may already be overwriting in place.
+  const uint64_t tensor_bytes = static_cast<uint64_t>(p.batch * p.spatial * p.channels) * (16 / vec);
+  if (ranges_overlap(p.out, p.x, tensor_bytes) || ranges_overlap(p.out, p.dy, tensor_bytes)) return pl;
   if (p.channels % p.groups != 0 || p.channels / p.groups > kTileColsPerLane * kWave) return pl;
   const int64_t cv = p.channels / vec;
   if (cv > 512) return pl;

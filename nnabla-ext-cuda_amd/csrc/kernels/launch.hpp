@@ -33,6 +33,16 @@ enum RowMode {
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+// True when the byte ranges [a, a + bytes) and [b, b + bytes) share a byte
+// (null pointers overlap nothing).  The kernels whose blocks may recompute a
+// partner's partial sums from global memory read tensors that the partner is
+// already overwriting when the output shares memory with an input, so their
+// plans turn such calls down and the kernels without an exchange take them.
+inline bool ranges_overlap(const void *a, const void *b, uint64_t bytes) {
+  if (!a || !b || bytes == 0) return false;
+  const uintptr_t pa = reinterpret_cast<uintptr_t>(a), pb = reinterpret_cast<uintptr_t>(b);
+  return pa < pb ? pb - pa < bytes : pa - pb < bytes;
+}
 
 // Number of compute units of the current device (cached per device).
 int device_cus();
