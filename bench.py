@@ -12,7 +12,7 @@ loop over one set of buffers serves part of every call from cache - which a
 training step, whose activations were written a whole network ago, never
 sees.  Every workload here therefore owns several distinct sets of buffers
 (real sizes, no flush kernel) and the timed loop walks them in turn, one lap
-being larger than L2 + Infinity Cache; these "rotated" times are the ones
+being four times L2 + Infinity Cache (1 GiB; --lap-mb); these "rotated" times are the ones
 `value`, `roofline` and `pct_of_hbm_peak` are based on.  The same loop over
 set 0 alone is reported beside them as `warm`.
 
@@ -44,10 +44,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 # One lap over a workload's buffer sets must exceed L2 (8 x 4 MB) plus the
-# Infinity Cache (256 MB), with room to spare; --lap-mb sets another lap (the
-# sensitivity of the cold figures to the lap is what shows whether a cyclic
-# walk of this size really misses the memory-side cache).
-LAP_BYTES = 352 << 20
+# Infinity Cache (256 MB) several times over: a cyclic walk of 1.2-1.4 times the
+# cache still hits in it (measured: the 33 MB configurations and their plain
+# copy run 10-35 % faster over a 352 MiB lap than over 1 GiB, and 2 GiB changes
+# nothing further), so the default lap is 1 GiB.  --lap-mb sets another one.
+LAP_BYTES = 1024 << 20
 
 
 def log(*a):
@@ -644,6 +645,7 @@ def load_traffic(kernel):
 
 
 def main():
+    global LAP_BYTES
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
@@ -651,6 +653,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-table", action="store_true", help="skip the per-config table")
     ap.add_argument("--only", default=None, help="table rows whose name contains this text")
+    ap.add_argument("--table-only", action="store_true",
+                    help="only the per-configuration table (with --only: a few rows), printed as "
+                         "one JSON line {\"configs\": [...]}; no headline workload, no CPU "
+                         "baseline - the short command for per-kernel counter runs")
     ap.add_argument("--torch-native", action="store_true",
                     help="also time torch's own normalization kernels on the same shapes")
     ap.add_argument("--lap-mb", type=int, default=LAP_BYTES >> 20,
@@ -666,7 +672,6 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
-    global LAP_BYTES
     LAP_BYTES = max(1, args.lap_mb) << 20
 
     import torch
@@ -674,6 +679,12 @@ def main():
     L = K.lib()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
+
+    if args.table_only:
+        print(json.dumps({"lap_floor_bytes": LAP_BYTES, "steps": args.steps,
+                          "configs": config_table(K, args.steps, args.warmup, args.only)}),
+              flush=True)
+        return
 
     name = ("BatchNormalization training fwd+bwd fp32 NCHW x[32,256,56,56] "
             "(benchmark configuration 2), decay_rate 0.9, eps 1e-5")

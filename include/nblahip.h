@@ -518,6 +518,14 @@ NBLAHIP_EXPORT int nblahip_tune_set(const char *name, int value);
 NBLAHIP_EXPORT int nblahip_tune_get(const char *name, int fallback);
 NBLAHIP_EXPORT int nblahip_tune_reset(void);
 
+/* Testing aid, no counterpart in the reference.  The kernels whose blocks
+ * exchange partial sums tag every exchanged word with a per-launch epoch, a
+ * 32-bit counter per GPU; when it wraps (after 2^32 such launches) the library
+ * waits for the device, clears its exchange array and starts over at 1.  This
+ * sets the counter of the current device so that a test can walk it across
+ * the wrap. */
+NBLAHIP_EXPORT int nblahip_xchg_set_epoch(unsigned int epoch);
+
 #ifdef __cplusplus
 }
 #endif

@@ -106,6 +106,7 @@ SIGNATURES = {
     "nblahip_tune_set": (_int, [ctypes.c_char_p, _int]),
     "nblahip_tune_get": (_int, [ctypes.c_char_p, _int]),
     "nblahip_tune_reset": (_int, []),
+    "nblahip_xchg_set_epoch": (_int, [ctypes.c_uint]),
 }
 
 _lib = None

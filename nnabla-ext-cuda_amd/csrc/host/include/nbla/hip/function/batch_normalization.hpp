@@ -37,6 +37,21 @@ protected:
   virtual void forward_impl_batch(const Variables &inputs, const Variables &outputs,
                                   const bool update_inputs);
   virtual void forward_impl_global(const Variables &inputs, const Variables &outputs);
+  // backward_impl dispatches on batch_stat to one of these two, as the
+  // reference does (batch_normalization.cu:200-212); a subclass may override
+  // either (the reference's cudnn class overrides backward_impl_batch,
+  // include/nbla/cuda/cudnn/function/batch_normalization.hpp:90).  The
+  // reference leaves the inference-mode backward to the core's
+  // backward_impl_global on the CPU; here it runs on the device.
+  virtual void backward_impl_batch(const Variables &inputs, const Variables &outputs,
+                                   const vector<bool> &propagate_down, const vector<bool> &accum);
+  virtual void backward_impl_global(const Variables &inputs, const Variables &outputs,
+                                    const vector<bool> &propagate_down, const vector<bool> &accum);
   virtual void recompute_impl(const Variables &inputs, const Variables &outputs);
+
+private:
+  void backward_launch(const Variables &inputs, const Variables &outputs,
+                       const vector<bool> &propagate_down, const vector<bool> &accum,
+                       bool batch_stat);
 };
 } // namespace nbla

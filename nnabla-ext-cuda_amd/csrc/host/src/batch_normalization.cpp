@@ -89,6 +89,33 @@ void BatchNormalizationHip<T>::backward_impl(const Variables &inputs, const Vari
                                              const vector<bool> &propagate_down,
                                              const vector<bool> &accum) {
   hip_set_device(this->device_);
+  if (this->batch_stat_) { // Training mode.
+    backward_impl_batch(inputs, outputs, propagate_down, accum);
+  } else { // Testing mode.
+    backward_impl_global(inputs, outputs, propagate_down, accum);
+  }
+}
+
+template <typename T>
+void BatchNormalizationHip<T>::backward_impl_batch(const Variables &inputs,
+                                                   const Variables &outputs,
+                                                   const vector<bool> &propagate_down,
+                                                   const vector<bool> &accum) {
+  backward_launch(inputs, outputs, propagate_down, accum, true);
+}
+
+template <typename T>
+void BatchNormalizationHip<T>::backward_impl_global(const Variables &inputs,
+                                                    const Variables &outputs,
+                                                    const vector<bool> &propagate_down,
+                                                    const vector<bool> &accum) {
+  backward_launch(inputs, outputs, propagate_down, accum, false);
+}
+
+template <typename T>
+void BatchNormalizationHip<T>::backward_launch(const Variables &inputs, const Variables &outputs,
+                                               const vector<bool> &propagate_down,
+                                               const vector<bool> &accum, bool batch_stat) {
   const bool pd_x = propagate_down[0];
   const bool pd_beta = !this->no_bias_ && propagate_down[this->b_idx_];
   const bool pd_gamma = !this->no_scale_ && propagate_down[this->g_idx_];
@@ -102,7 +129,7 @@ void BatchNormalizationHip<T>::backward_impl(const Variables &inputs, const Vari
   // Statistics the forward normalised with, and the gradients that reach the
   // mean/var outputs in the three-output form.
   const float *mean, *var, *dmean = nullptr, *dvar = nullptr;
-  if (this->batch_stat_) {
+  if (batch_stat) {
     Variable *batch_mean = &this->mean_;
     Variable *batch_var = &this->var_;
     if (outputs.size() == 3) {
@@ -129,7 +156,7 @@ void BatchNormalizationHip<T>::backward_impl(const Variables &inputs, const Vari
   NBLA_HIP_CHECK(nblahip_bn_bwd(
       x, dy, gamma, mean, var, dmean, dvar, dx, dgamma, dbeta, pd_x && accum[0],
       pd_gamma && accum[this->g_idx_], pd_beta && accum[this->b_idx_], this->size0_, this->size1_,
-      this->size2_, this->eps_, this->batch_stat_ ? 1 : 0, HipDtype<T>::code, ws, workspace_bytes_,
+      this->size2_, this->eps_, batch_stat ? 1 : 0, HipDtype<T>::code, ws, workspace_bytes_,
       nullptr));
 }
 

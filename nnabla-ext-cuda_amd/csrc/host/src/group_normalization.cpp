@@ -18,8 +18,14 @@ void GroupNormalizationHip<T>::setup_impl(const Variables &inputs, const Variabl
   channel_size_ = layout_.channels;
   batch_size_ = layout_.batch;
   spatial_size_ = layout_.spatial;
-  NBLA_CHECK(x->size() < (Size_t(1) << 31), error_code::value,
-             "GroupNormalizationHip indexes with 32 bits: fewer than 2^31 elements required.");
+  // Tensors of 2^31 elements and more run as several launches over ranges of
+  // samples (the kernel layer indexes one launch with 32 bits); one sample, and
+  // a tensor that has to be permuted first, must stay below that.
+  NBLA_CHECK(channel_size_ * spatial_size_ < (Size_t(1) << 31) &&
+                 (!layout_.data.needed() || x->size() < (Size_t(1) << 31)),
+             error_code::value,
+             "GroupNormalizationHip indexes with 32 bits: fewer than 2^31 elements per sample "
+             "required (per tensor where the layout needs a permutation).");
   mean_.reshape(Shape_t{batch_size_ * this->num_groups_}, true);
   var_.reshape(Shape_t{batch_size_ * this->num_groups_}, true);
   hip_set_device(this->device_); // argument errors above are reported without a device

@@ -51,21 +51,29 @@ void init_hip() {
   ArrayCreator::add_creator("HipCachedHostArray", [](Size_t s, dtypes d, const Context &c) -> Array * {
     return new HipCachedHostArray(s, d, c);
   });
-  // The pinned host array is a host array: plain copies to and from CpuArray.
-  ArraySynchronizer::add_synchronizer("HipCachedHostArray", "CpuArray",
-                                      [](Array *src, Array *dst, const int) { dst->copy_from(src); });
-  ArraySynchronizer::add_synchronizer("CpuArray", "HipCachedHostArray",
-                                      [](Array *src, Array *dst, const int) { dst->copy_from(src); });
-  ArraySynchronizer::add_synchronizer("HipCachedHostArray", "HipCachedHostArray",
-                                      [](Array *src, Array *dst, const int) { dst->copy_from(src); });
+  // The pinned host array is a host array: plain copies to and from CpuArray -
+  // once the source's pending transfer (an ASYNC device-to-host copy leaves a
+  // HipEvent on the pinned array) has landed, as the reference's synchronizers
+  // wait first (src/nbla/cuda/array/cuda_array.cpp:88,125,164).
+  auto host_copy = [](Array *src, Array *dst, const int async_flags) {
+    src->wait_event(dst->context(), async_flags & ~(AsyncFlag::ASYNC | AsyncFlag::UNSAFE));
+    dst->copy_from(src);
+  };
+  ArraySynchronizer::add_synchronizer("HipCachedHostArray", "CpuArray", host_copy);
+  ArraySynchronizer::add_synchronizer("CpuArray", "HipCachedHostArray", host_copy);
+  ArraySynchronizer::add_synchronizer("HipCachedHostArray", "HipCachedHostArray", host_copy);
   const char *device_classes[] = {"HipArray", "HipCachedArray"};
   for (const char *dc : device_classes) {
     ArraySynchronizer::add_synchronizer(dc, "CpuArray", synchronizer_hip_array_cpu_array);
     ArraySynchronizer::add_synchronizer("CpuArray", dc, synchronizer_cpu_array_hip_array);
     ArraySynchronizer::add_synchronizer(dc, "HipCachedHostArray", synchronizer_hip_array_cpu_array);
     ArraySynchronizer::add_synchronizer("HipCachedHostArray", dc, synchronizer_cpu_array_hip_array);
+    // device to device on the function stream, behind the source's pending upload
     for (const char *dc2 : device_classes)
-      ArraySynchronizer::add_synchronizer(dc, dc2, [](Array *src, Array *dst, const int) { dst->copy_from(src); });
+      ArraySynchronizer::add_synchronizer(dc, dc2, [](Array *src, Array *dst, const int async_flags) {
+        src->wait_event(dst->context(), async_flags);
+        dst->copy_from(src);
+      });
   }
 
   // Functions: same names as the reference registers, new backend key.

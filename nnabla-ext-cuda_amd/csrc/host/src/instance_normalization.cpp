@@ -19,8 +19,12 @@ void InstanceNormalizationHip<T>::setup_impl(const Variables &inputs, const Vari
   channel_size_ = layout_.channels;
   batch_size_ = layout_.batch;
   spatial_size_ = layout_.spatial;
-  NBLA_CHECK(x->size() < (Size_t(1) << 31), error_code::value,
-             "InstanceNormalizationHip indexes with 32 bits: fewer than 2^31 elements required.");
+  // (as GroupNormalizationHip: ranges of samples per launch beyond 2^31 elements)
+  NBLA_CHECK(channel_size_ * spatial_size_ < (Size_t(1) << 31) &&
+                 (!layout_.data.needed() || x->size() < (Size_t(1) << 31)),
+             error_code::value,
+             "InstanceNormalizationHip indexes with 32 bits: fewer than 2^31 elements per sample "
+             "required (per tensor where the layout needs a permutation).");
   mean_.reshape(Shape_t{batch_size_ * channel_size_}, true);
   var_.reshape(Shape_t{batch_size_ * channel_size_}, true);
   hip_set_device(this->device_); // argument errors above are reported without a device

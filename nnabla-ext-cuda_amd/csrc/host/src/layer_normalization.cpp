@@ -21,8 +21,14 @@ void LayerNormalizationHip<T>::setup_impl(const Variables &inputs, const Variabl
   batch_size_ = 1;
   for (const auto b : ba) batch_size_ *= x_shape[b];
   reduce_size_ = inputs[0]->size() / std::max<Size_t>(batch_size_, 1);
-  NBLA_CHECK(inputs[0]->size() < (Size_t(1) << 31), error_code::value,
-             "LayerNormalizationHip indexes with 32 bits: fewer than 2^31 elements required.");
+  // Tensors of 2^31 elements and more run as several launches over ranges of
+  // rows (the kernel layer indexes one launch with 32 bits); one row, and a
+  // tensor that has to be permuted first, must stay below that.
+  NBLA_CHECK(reduce_size_ < (Size_t(1) << 31) &&
+                 (!adaptor_.needed() || inputs[0]->size() < (Size_t(1) << 31)),
+             error_code::value,
+             "LayerNormalizationHip indexes with 32 bits: fewer than 2^31 elements per row "
+             "required (per tensor where the batch axes are not the leading ones).");
   mean_.reshape(Shape_t{batch_size_}, true);
   var_.reshape(Shape_t{batch_size_}, true);
   hip_set_device(this->device_); // argument errors above are reported without a device

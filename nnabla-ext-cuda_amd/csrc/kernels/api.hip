@@ -1,6 +1,7 @@
 // C-ABI entry points of the normalization kernels: argument validation and
 // translation into launch-layer problems.  Nothing here allocates, throws or
 // waits for the device.
+#include <algorithm>
 #include <atomic>
 
 #include "launch.hpp"
@@ -26,6 +27,81 @@ int check_dims3(int64_t a, int64_t b, int64_t c) {
   if (a > kMaxElems || b > kMaxElems || c > kMaxElems) return NBLAHIP_ERANGE;
   const __int128 total = static_cast<__int128>(a) * b * c;
   if (total > kMaxElems) return NBLAHIP_ERANGE;
+  return 0;
+}
+
+// The kernels index a tensor with 32 bits.  The reduction units of the row
+// normalizations are independent of each other - LayerNormalization rows, the
+// samples of Group / InstanceNormalization - so a tensor of 2^31 elements and
+// more (the reference indexes these with Size_t: layer_normalization.cu:99,
+// group_normalization.cu:57-62) runs as several launches over ranges of units,
+// each below 2^31 elements; the parameter gradients of the later ranges
+// accumulate onto the first range's.  One unit alone must stay below 2^31
+// elements.  0: proceed; 1: empty tensor; <0: error.
+int check_dims_units(int64_t units, int64_t b, int64_t c) {
+  if (units < 0 || b < 0 || c < 0) return NBLAHIP_EINVAL;
+  if (units == 0 || b == 0 || c == 0) return 1;
+  if (units > kMaxElems || b > kMaxElems || c > kMaxElems) return NBLAHIP_ERANGE;
+  if (static_cast<__int128>(b) * c > kMaxElems) return NBLAHIP_ERANGE;
+  return 0;
+}
+
+// Units per launch: as many as stay below 2^31 elements (and below `cap`).
+int64_t units_per_launch(int64_t units, int64_t unit_elems, int64_t cap = kMaxElems) {
+  return std::max<int64_t>(1, std::min(units, std::min(cap, kMaxElems / std::max<int64_t>(1, unit_elems))));
+}
+
+// Workspace of a call that runs in ranges of `per` units: the larger of what
+// a full range and the last, shorter one need.
+template <class F> size_t chunked_workspace(int64_t units, int64_t per, F bytes_of) {
+  const int64_t tail = units % per;
+  return std::max(bytes_of(std::min(units, per)), tail ? bytes_of(tail) : size_t{0});
+}
+
+// The range [u0, u0 + n) of the units of a row problem.  unit_rows: statistics
+// rows per unit (LayerNormalization: 1; GN: groups; IN: channels).
+RowProblem row_range(const RowProblem &p, int64_t u0, int64_t n, int64_t unit_rows, bool is_ln) {
+  RowProblem q = p;
+  const size_t esz = p.dtype == NBLAHIP_F16 ? 2 : 4;
+  const size_t unit_elems = static_cast<size_t>(unit_rows) * static_cast<size_t>(p.R);
+  const size_t off = static_cast<size_t>(u0) * unit_elems * esz;
+  q.x = static_cast<const char *>(p.x) + off;
+  if (p.dy) q.dy = static_cast<const char *>(p.dy) + off;
+  if (p.out) q.out = static_cast<char *>(p.out) + off;
+  const int64_t r0 = u0 * unit_rows;
+  if (p.mean) q.mean = p.mean + r0;
+  if (p.var) q.var = p.var + r0;
+  if (p.dmean) q.dmean = p.dmean + r0;
+  if (p.dvar) q.dvar = p.dvar + r0;
+  q.rows = n * unit_rows;
+  if (!is_ln) {
+    q.batch = n;
+    // per-sample InstanceNormalization parameters move with the samples; shared
+    // ones accumulate over the ranges
+    if (!p.bc_gamma) {
+      if (p.gamma) q.gamma = p.gamma + u0 * p.channels;
+      if (p.dgamma) q.dgamma = p.dgamma + u0 * p.channels;
+    }
+    if (!p.bc_beta) {
+      if (p.beta) q.beta = p.beta + u0 * p.channels;
+      if (p.dbeta) q.dbeta = p.dbeta + u0 * p.channels;
+    }
+  }
+  if (u0 > 0) {
+    if (is_ln || p.bc_gamma) q.accum_g = 1;
+    if (is_ln || p.bc_beta) q.accum_b = 1;
+  }
+  return q;
+}
+
+int run_rows(const RowProblem &p, int64_t units, int64_t unit_rows, bool is_ln, bool forward,
+             hipStream_t st) {
+  const int64_t per = units_per_launch(units, unit_rows * p.R);
+  if (per >= units) return forward ? launch_row_fwd(p, st) : launch_row_bwd(p, st);
+  for (int64_t u0 = 0; u0 < units; u0 += per) {
+    const RowProblem q = row_range(p, u0, std::min(per, units - u0), unit_rows, is_ln);
+    if (const int e = forward ? launch_row_fwd(q, st) : launch_row_bwd(q, st)) return e;
+  }
   return 0;
 }
 
@@ -398,7 +474,7 @@ int nblahip_ln_fwd(const void *x, const float *gamma, const float *beta, void *y
                    float *var, int64_t outer, int64_t reduce, float eps, int dtype,
                    void *stream) {
   if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
-  const int d = check_dims3(outer, reduce, 1);
+  const int d = check_dims_units(outer, reduce, 1);
   if (d) return d < 0 ? d : 0;
   if (!x || !y || !mean || !var) return NBLAHIP_EINVAL;
   if (int e = check_fwd_alias(x, y, static_cast<size_t>(outer) * reduce * elem_bytes(dtype), gamma,
@@ -417,12 +493,17 @@ int nblahip_ln_fwd(const void *x, const float *gamma, const float *beta, void *y
   p.rows = outer;
   p.R = reduce;
   p.eps = eps;
-  return launch_row_fwd(p, as_stream(stream));
+  return run_rows(p, outer, 1, true, true, as_stream(stream));
+}
+
+static size_t ln_bwd_workspace(int64_t outer, int64_t reduce) {
+  return chunked_workspace(outer, units_per_launch(outer, reduce),
+                           [&](int64_t n) { return row_bwd_workspace_bytes(kRowLN, n, reduce, 0); });
 }
 
 size_t nblahip_ln_bwd_workspace_bytes(int64_t outer, int64_t reduce, int dtype) {
-  if (!dtype_ok(dtype) || check_dims3(outer, reduce, 1) != 0) return 0;
-  return row_bwd_workspace_bytes(kRowLN, outer, reduce, 0);
+  if (!dtype_ok(dtype) || check_dims_units(outer, reduce, 1) != 0) return 0;
+  return ln_bwd_workspace(outer, reduce);
 }
 
 int nblahip_ln_bwd(const void *x, const void *dy, const float *gamma, const float *mean,
@@ -431,11 +512,10 @@ int nblahip_ln_bwd(const void *x, const void *dy, const float *gamma, const floa
                    int64_t outer, int64_t reduce, float eps, int dtype, void *workspace,
                    size_t workspace_bytes, void *stream) {
   if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
-  const int d = check_dims3(outer, reduce, 1);
+  const int d = check_dims_units(outer, reduce, 1);
   if (d) return d < 0 ? d : 0;
   if (!x || !dy || !mean || !var) return NBLAHIP_EINVAL;
-  if (int e = check_ws(workspace, workspace_bytes, row_bwd_workspace_bytes(kRowLN, outer, reduce, 0)))
-    return e;
+  if (int e = check_ws(workspace, workspace_bytes, ln_bwd_workspace(outer, reduce))) return e;
   RowProblem p;
   p.dtype = dtype;
   p.mode = kRowLN;
@@ -457,7 +537,7 @@ int nblahip_ln_bwd(const void *x, const void *dy, const float *gamma, const floa
   p.eps = eps;
   p.ws = workspace;
   p.ws_bytes = workspace_bytes;
-  return launch_row_bwd(p, as_stream(stream));
+  return run_rows(p, outer, 1, true, false, as_stream(stream));
 }
 
 // ----------------------------------------------------------------------------
@@ -466,7 +546,7 @@ int nblahip_ln_bwd(const void *x, const void *dy, const float *gamma, const floa
 static int gn_problem(RowProblem &p, int64_t batch, int64_t channels, int64_t spatial, int groups,
                       int dtype) {
   if (!dtype_ok(dtype) || groups <= 0) return NBLAHIP_EINVAL;
-  const int d = check_dims3(batch, channels, spatial);
+  const int d = check_dims_units(batch, channels, spatial);
   if (d) return d;
   if (channels % groups != 0) return NBLAHIP_EINVAL;
   p.dtype = dtype;
@@ -498,14 +578,21 @@ int nblahip_gn_fwd(const void *x, const float *gamma, const float *beta, void *y
   p.mean = mean;
   p.var = var;
   p.eps = eps;
-  return launch_row_fwd(p, as_stream(stream));
+  return run_rows(p, batch, groups, false, true, as_stream(stream));
+}
+
+// (mode kRowGN or kRowIN; unit_rows = statistics rows per sample)
+static size_t planes_bwd_workspace(int mode, const RowProblem &p, int64_t unit_rows) {
+  return chunked_workspace(p.batch, units_per_launch(p.batch, p.channels * p.spatial), [&](int64_t n) {
+    return row_bwd_workspace_bytes(mode, n * unit_rows, p.R, n * p.channels);
+  });
 }
 
 size_t nblahip_gn_bwd_workspace_bytes(int64_t batch, int64_t channels, int64_t spatial,
                                       int groups, int dtype) {
   RowProblem p;
   if (gn_problem(p, batch, channels, spatial, groups, dtype) != 0) return 0;
-  return row_bwd_workspace_bytes(kRowGN, p.rows, p.R, batch * channels);
+  return planes_bwd_workspace(kRowGN, p, groups);
 }
 
 int nblahip_gn_bwd(const void *x, const void *dy, const float *gamma, const float *mean,
@@ -517,9 +604,7 @@ int nblahip_gn_bwd(const void *x, const void *dy, const float *gamma, const floa
   const int d = gn_problem(p, batch, channels, spatial, groups, dtype);
   if (d) return d < 0 ? d : 0;
   if (!x || !dy || !mean || !var) return NBLAHIP_EINVAL;
-  if (int e = check_ws(workspace, workspace_bytes,
-                       row_bwd_workspace_bytes(kRowGN, p.rows, p.R, batch * channels)))
-    return e;
+  if (int e = check_ws(workspace, workspace_bytes, planes_bwd_workspace(kRowGN, p, groups))) return e;
   p.x = x;
   p.dy = dy;
   p.out = dx;
@@ -536,7 +621,7 @@ int nblahip_gn_bwd(const void *x, const void *dy, const float *gamma, const floa
   p.eps = eps;
   p.ws = workspace;
   p.ws_bytes = workspace_bytes;
-  return launch_row_bwd(p, as_stream(stream));
+  return run_rows(p, batch, groups, false, false, as_stream(stream));
 }
 
 // ----------------------------------------------------------------------------
@@ -545,7 +630,7 @@ int nblahip_gn_bwd(const void *x, const void *dy, const float *gamma, const floa
 static int in_problem(RowProblem &p, int64_t batch, int64_t channels, int64_t spatial,
                       int bc_gamma, int bc_beta, int dtype) {
   if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
-  const int d = check_dims3(batch, channels, spatial);
+  const int d = check_dims_units(batch, channels, spatial);
   if (d) return d;
   p.dtype = dtype;
   p.mode = kRowIN;
@@ -579,14 +664,14 @@ int nblahip_in_fwd(const void *x, const float *gamma, const float *beta, void *y
   p.mean = mean;
   p.var = var;
   p.eps = eps;
-  return launch_row_fwd(p, as_stream(stream));
+  return run_rows(p, batch, channels, false, true, as_stream(stream));
 }
 
 size_t nblahip_in_bwd_workspace_bytes(int64_t batch, int64_t channels, int64_t spatial,
                                       int dtype) {
   RowProblem p;
   if (in_problem(p, batch, channels, spatial, 1, 1, dtype) != 0) return 0;
-  return row_bwd_workspace_bytes(kRowIN, p.rows, p.R, batch * channels);
+  return planes_bwd_workspace(kRowIN, p, channels);
 }
 
 int nblahip_in_bwd(const void *x, const void *dy, const float *gamma, const float *mean,
@@ -598,9 +683,7 @@ int nblahip_in_bwd(const void *x, const void *dy, const float *gamma, const floa
   const int d = in_problem(p, batch, channels, spatial, bc_gamma, bc_beta, dtype);
   if (d) return d < 0 ? d : 0;
   if (!x || !dy || !mean || !var) return NBLAHIP_EINVAL;
-  if (int e = check_ws(workspace, workspace_bytes,
-                       row_bwd_workspace_bytes(kRowIN, p.rows, p.R, batch * channels)))
-    return e;
+  if (int e = check_ws(workspace, workspace_bytes, planes_bwd_workspace(kRowIN, p, channels))) return e;
   p.x = x;
   p.dy = dy;
   p.out = dx;
@@ -617,7 +700,7 @@ int nblahip_in_bwd(const void *x, const void *dy, const float *gamma, const floa
   p.eps = eps;
   p.ws = workspace;
   p.ws_bytes = workspace_bytes;
-  return launch_row_bwd(p, as_stream(stream));
+  return run_rows(p, batch, channels, false, false, as_stream(stream));
 }
 
 // ---------------------------------------------------------------------------
@@ -628,15 +711,59 @@ namespace {
 int cl_problem(ClProblem &p, int64_t batch, int64_t spatial, int64_t channels, int groups,
                int dtype) {
   if (!dtype_ok(dtype) || groups <= 0) return NBLAHIP_EINVAL;
-  const int d = check_dims3(batch, spatial, channels);
+  const int d = check_dims_units(batch, spatial, channels);
   if (d) return d;
   if (channels % groups != 0) return NBLAHIP_EINVAL;
-  if (batch > 65535) return NBLAHIP_ERANGE; // one slab per grid y/z index
   p.dtype = dtype;
   p.batch = batch;
   p.spatial = spatial;
   p.channels = channels;
   p.groups = groups;
+  return 0;
+}
+
+// Samples per launch: the kernels put the sample on a grid axis (65535 at
+// most) and index a launch's tensor with 32 bits; larger batches and tensors
+// run as several launches over ranges of samples (see check_dims_units).
+constexpr int64_t kClMaxBatch = 65535;
+int64_t cl_per_launch(const ClProblem &p) {
+  return units_per_launch(p.batch, p.spatial * p.channels, kClMaxBatch);
+}
+size_t cl_workspace(const ClProblem &p) {
+  return chunked_workspace(p.batch, cl_per_launch(p), [&](int64_t n) {
+    return cl_workspace_bytes(n, p.spatial, p.channels, p.dtype);
+  });
+}
+int run_cl(const ClProblem &p, bool forward, hipStream_t st) {
+  const int64_t per = cl_per_launch(p);
+  if (per >= p.batch) return forward ? launch_cl_fwd(p, st) : launch_cl_bwd(p, st);
+  const size_t esz = elem_bytes(p.dtype);
+  for (int64_t u0 = 0; u0 < p.batch; u0 += per) {
+    ClProblem q = p;
+    q.batch = std::min(per, p.batch - u0);
+    const size_t off = static_cast<size_t>(u0) * p.spatial * p.channels * esz;
+    q.x = static_cast<const char *>(p.x) + off;
+    if (p.dy) q.dy = static_cast<const char *>(p.dy) + off;
+    if (p.out) q.out = static_cast<char *>(p.out) + off;
+    const int64_t r0 = u0 * p.groups;
+    q.mean = p.mean + r0;
+    q.var = p.var + r0;
+    if (p.dmean) q.dmean = p.dmean + r0;
+    if (p.dvar) q.dvar = p.dvar + r0;
+    if (!p.bc_gamma) {
+      if (p.gamma) q.gamma = p.gamma + u0 * p.channels;
+      if (p.dgamma) q.dgamma = p.dgamma + u0 * p.channels;
+    } else if (u0 > 0) {
+      q.accum_g = 1;
+    }
+    if (!p.bc_beta) {
+      if (p.beta) q.beta = p.beta + u0 * p.channels;
+      if (p.dbeta) q.dbeta = p.dbeta + u0 * p.channels;
+    } else if (u0 > 0) {
+      q.accum_b = 1;
+    }
+    if (const int e = forward ? launch_cl_fwd(q, st) : launch_cl_bwd(q, st)) return e;
+  }
   return 0;
 }
 
@@ -646,9 +773,7 @@ int cl_fwd(ClProblem &p, const void *x, const float *gamma, const float *beta, v
   if (!x || !y || !mean || !var) return NBLAHIP_EINVAL;
   if (check_in_place(y, x, static_cast<size_t>(p.batch) * p.spatial * p.channels * elem_bytes(p.dtype)))
     return NBLAHIP_EALIAS;
-  if (int e = check_ws(workspace, workspace_bytes,
-                       cl_workspace_bytes(p.batch, p.spatial, p.channels, p.dtype)))
-    return e;
+  if (int e = check_ws(workspace, workspace_bytes, cl_workspace(p))) return e;
   p.x = x;
   p.out = y;
   p.gamma = gamma;
@@ -658,7 +783,7 @@ int cl_fwd(ClProblem &p, const void *x, const float *gamma, const float *beta, v
   p.eps = eps;
   p.ws = workspace;
   p.ws_bytes = workspace_bytes;
-  return launch_cl_fwd(p, as_stream(stream));
+  return run_cl(p, true, as_stream(stream));
 }
 
 int cl_bwd(ClProblem &p, const void *x, const void *dy, const float *gamma, const float *mean,
@@ -670,9 +795,7 @@ int cl_bwd(ClProblem &p, const void *x, const void *dy, const float *gamma, cons
     const size_t tb = static_cast<size_t>(p.batch) * p.spatial * p.channels * elem_bytes(p.dtype);
     if (check_in_place(dx, x, tb) || check_in_place(dx, dy, tb)) return NBLAHIP_EALIAS;
   }
-  if (int e = check_ws(workspace, workspace_bytes,
-                       cl_workspace_bytes(p.batch, p.spatial, p.channels, p.dtype)))
-    return e;
+  if (int e = check_ws(workspace, workspace_bytes, cl_workspace(p))) return e;
   p.x = x;
   p.dy = dy;
   p.out = dx;
@@ -689,7 +812,7 @@ int cl_bwd(ClProblem &p, const void *x, const void *dy, const float *gamma, cons
   p.eps = eps;
   p.ws = workspace;
   p.ws_bytes = workspace_bytes;
-  return launch_cl_bwd(p, as_stream(stream));
+  return run_cl(p, false, as_stream(stream));
 }
 } // namespace
 
@@ -697,7 +820,7 @@ size_t nblahip_gn_cl_workspace_bytes(int64_t batch, int64_t spatial, int64_t cha
                                      int dtype) {
   ClProblem p;
   if (cl_problem(p, batch, spatial, channels, groups, dtype) != 0) return 0;
-  return cl_workspace_bytes(batch, spatial, channels, dtype);
+  return cl_workspace(p);
 }
 
 int nblahip_gn_cl_fwd(const void *x, const float *gamma, const float *beta, void *y, float *mean,
@@ -729,7 +852,7 @@ size_t nblahip_in_cl_workspace_bytes(int64_t batch, int64_t spatial, int64_t cha
   if (cl_problem(p, batch, spatial, channels, static_cast<int>(std::max<int64_t>(channels, 1)),
                  dtype) != 0)
     return 0;
-  return cl_workspace_bytes(batch, spatial, channels, dtype);
+  return cl_workspace(p);
 }
 
 int nblahip_in_cl_fwd(const void *x, const float *gamma, const float *beta, void *y, float *mean,

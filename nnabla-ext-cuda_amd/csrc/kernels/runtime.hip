@@ -10,6 +10,7 @@
 
 #include "common.cuh"
 #include "launch.hpp"
+#include "xchg.cuh"
 
 namespace nblahip {
 
@@ -396,6 +397,13 @@ int nblahip_fill(void *dst, int dtype, float value, int64_t n, void *stream) {
     return NBLAHIP_EINVAL;
   }
   return last_launch_status();
+}
+
+int nblahip_xchg_set_epoch(unsigned int epoch) {
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return hip_status(e);
+  xchg_debug_set_epoch(dev, epoch);
+  return 0;
 }
 
 } // extern "C"

@@ -63,5 +63,7 @@ bool xchg_acquire(size_t words, hipStream_t stream, unsigned long long **region,
                   int *status);
 // Most words one launch may ask for.
 size_t xchg_capacity();
+// Testing aid: the epoch the next launch on device `dev` continues from.
+void xchg_debug_set_epoch(int dev, uint32_t epoch);
 
 } // namespace nblahip

@@ -106,3 +106,24 @@ def test_device_arrays_store_every_dtype(dtype):
     v.cast_raw("HipArray", dtype)
     v.zero_data()
     np.testing.assert_array_equal(v.get_raw(dtype), np.zeros(5000, dtype))
+
+
+def test_host_reader_of_a_pinned_array_waits_for_its_pending_download():
+    """An ASYNC device-to-pinned-host cast leaves the transfer's event on the
+    pinned array; a following host read through another host class (a plain
+    copy between two host arrays) must wait for it before it copies."""
+    n = 32 << 20
+    x = np.arange(n, dtype=np.float32)
+    vx = B.Variable((n,))
+    vx.set_data(x)
+    vx.cast("HipCachedArray")
+    for k in range(3):
+        vx.cast("HipCachedHostArray", device_id="", async_flags=B.ASYNC)   # enqueued, not waited for
+        got = vx.d                                                          # CpuArray <- pinned array
+        np.testing.assert_array_equal(got, x)
+        vx.cast("HipCachedArray")                                           # head back on the device
+        x = x + 1
+        vx.set_data(x)
+        vx.cast("HipCachedArray")
+    B.device_synchronize()
+    assert B.pending_transfers() == 0

@@ -343,3 +343,43 @@ def test_instance_flags_through_the_split_kernels():
     assert_close(to_np(dbet), db_r, "f32", "pgrad", "dbeta only")
     torch.cuda.synchronize()
     assert ran(K.profile_kernels())
+
+
+def test_epoch_wrap_and_ring_end():
+    """The per-launch epoch is a 32-bit counter: walked across its wrap (the
+    library then clears the exchange array and starts over) and, with launches
+    of many exchange words, several times round the ring, results stay
+    bit-identical to the first call and the exchanging kernels keep running."""
+    n, sp, c, groups = 16, (64, 64), 256, 32       # 16 x 4 x 16 blocks' words per launch
+    x, dy, g, b = make(n, sp, c, F16, 77)
+    xd, dyd, gd, bd = to_dev(x, F16), to_dev(dy, F16), to_dev(g), to_dev(b)
+
+    def run():
+        y, m, v = K.gn_forward(xd, bd, gd, groups, 1e-5, channel_last=True)
+        dx, dgam, dbet = K.gn_backward(xd, dyd, gd, m, v, groups, 1e-5, channel_last=True)
+        return [y, m, v, dx, dgam, dbet]
+
+    first = run()
+    K.check(K.lib().nblahip_xchg_set_epoch(0xFFFFFFFF - 5))
+    K.check(K.lib().nblahip_profile_enable(256))
+    for _ in range(12):                              # 24 launches: across the wrap
+        out = run()
+        for a_, b_ in zip(first, out):
+            assert torch.equal(a_, b_)
+    torch.cuda.synchronize()
+    names = K.profile_kernels()
+    K.check(K.lib().nblahip_profile_enable(0))
+    assert ran(names), names
+    # many launches with large regions: round the ring more than once
+    big = make(64, (32, 32), 512, F16, 78)
+    bx, bdy, bg, bb = to_dev(big[0], F16), to_dev(big[1], F16), to_dev(big[2]), to_dev(big[3])
+    ref = None
+    for _ in range(40):
+        y, m, v = K.in_forward(bx, bb, bg, 1e-5, channel_last=True)
+        if ref is None:
+            ref = (y.clone(), m.clone(), v.clone())
+        else:
+            assert torch.equal(y, ref[0]) and torch.equal(m, ref[1]) and torch.equal(v, ref[2])
+    out = run()
+    for a_, b_ in zip(first, out):
+        assert torch.equal(a_, b_)

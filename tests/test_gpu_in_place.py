@@ -58,7 +58,7 @@ BN_CASES = [
     ((32, 64, 56, 56), 1, F16, "bn_chan_split"),
     ((37, 64, 32, 32), 1, F32, "bn_chan_split"),
     # channel-last, the whole tensor held on the chip
-    ((100352, 64), 1, F16, "bn_cl_grid"),
+    ((200704, 64), 1, F16, "bn_cl_grid"),
     ((40000, 256), 1, F32, "bn_cl_grid"),
     # channel-last through the split kernels (all rows as one plane)
     ((64, 14, 14, 1024), 3, F16, "cl_split"),

@@ -129,11 +129,151 @@ def test_group_and_instance_normalization_just_below_2_31_elements(kind):
 
 
 def test_one_more_element_is_refused():
+    """BatchNormalization reduces over the whole tensor and indexes it with 32
+    bits, as the reference's kernels do (kernel/batch_normalization.cuh:246-254):
+    2^31 elements are refused.  The row normalizations take larger tensors in
+    ranges of rows / samples, but one row or sample must stay below 2^31."""
     L = K.lib()
     s = torch.cuda.current_stream().cuda_stream
     t = torch.empty(16, device="cuda")
     p = t.data_ptr()
     assert L.nblahip_bn_fwd_infer(p, p, p, None, None, p, 1 << 11, 1 << 10, 1 << 10, 1e-5, 1,
                                   s) == -3                 # 2^31 elements
-    assert L.nblahip_in_fwd(p, None, None, p, p, p, 1 << 11, 1 << 10, 1 << 10, 1, 1, 1e-5, 1,
-                            s) == -3
+    assert L.nblahip_in_fwd(p, None, None, p, p, p, 2, 1 << 16, 1 << 15, 1, 1, 1e-5, 1,
+                            s) == -3                       # 2^31 elements per sample
+    assert L.nblahip_ln_fwd(p, None, None, p, p, p, 2, 1 << 31, 1e-5, 1, s) == -3
+    assert L.nblahip_gn_cl_fwd(p, None, None, p, p, p, 2, 1 << 16, 1 << 15, 1, 1e-5, 1, p, 0,
+                               s) == -3
+
+
+# ---------------------------------------------------------------------------
+# 2^31 elements and more (the reference indexes the row normalizations with
+# Size_t: layer_normalization.cu:99, group_normalization.cu:57-62): the C-ABI
+# runs ranges of rows / samples below 2^31 elements each, the parameter
+# gradients of the later ranges accumulating onto the first.  The input is a
+# small block tiled along the batch; first, middle and last tile are held to
+# the float64 oracle of the block (the last range is shorter and may take
+# another thread layout, so tiles are compared to the oracle, not bit for bit
+# to each other), statistics likewise, dgamma / dbeta to tiles x the block's.
+def _tiles_close(t, n_tiles, ref, dn, kind, what):
+    for k in (0, n_tiles // 2, n_tiles - 2, n_tiles - 1):
+        assert_close(to_np(t[k]), ref, dn, kind, f"{what}, tile {k}")
+
+
+@pytest.mark.parametrize("accum", [False, True])
+def test_layer_normalization_above_2_31_elements(accum):
+    _need(30)
+    Rr, blk = 8192, 64
+    tiles = (1 << 31) // (Rr * blk) + 5                # 4101 tiles -> 2 150 105 088 elements
+    rows = tiles * blk
+    assert rows * Rr > (1 << 31)
+    rng = np.random.default_rng(71)
+    xb = (rng.standard_normal((blk, Rr)) + rng.uniform(-3, 3, (blk, 1))).astype(np.float16)
+    dyb = rng.standard_normal((blk, Rr)).astype(np.float16)
+    g = (rng.standard_normal(Rr) * 0.1 + 1).astype(np.float32)
+    b = (rng.standard_normal(Rr) * 0.1).astype(np.float32)
+    x = torch.from_numpy(xb).cuda().repeat(tiles, 1)
+    dy = torch.from_numpy(dyb).cuda().repeat(tiles, 1)
+    gd, bd = to_dev(g), to_dev(b)
+    y, m, v = K.ln_forward(x, bd, gd, rows, 1e-5)
+    y_r, m_r, v_r = R.ln_forward(xb, b, g, blk, 1e-5)
+    _tiles_close(y.view(tiles, blk, Rr), tiles, y_r, "f16", "y", "y")
+    _tiles_close(m.view(tiles, blk), tiles, m_r, "f16", "stat", "mean")
+    _tiles_close(v.view(tiles, blk), tiles, v_r, "f16", "stat", "var")
+    del y
+    pre_g = torch.full((Rr,), 3.0, device="cuda")
+    pre_b = torch.full((Rr,), -2.0, device="cuda")
+    dx, dg, db = K.ln_backward(x, dy, gd, m, v, rows, 1e-5,
+                               dgamma=pre_g.clone() if accum else None,
+                               dbeta=pre_b.clone() if accum else None,
+                               accum=(False, accum, accum))
+    dx_r, dg_r, db_r = R.ln_backward(xb, dyb, g, m_r, v_r, blk, 1e-5)
+    _tiles_close(dx.view(tiles, blk, Rr), tiles, dx_r, "f16", "grad", "dx")
+    off_g, off_b = (3.0, -2.0) if accum else (0.0, 0.0)
+    assert_close((to_np(dg) - off_g) / tiles, dg_r, "f16", "pgrad", "dgamma / tiles")
+    assert_close((to_np(db) - off_b) / tiles, db_r, "f16", "pgrad", "dbeta / tiles")
+
+
+@pytest.mark.parametrize("kind", ["gn", "in", "in_per_sample", "gn_cl", "in_cl"])
+def test_group_and_instance_normalization_above_2_31_elements(kind):
+    _need(30)
+    c, sp, groups = 256, 4096, 32
+    n = (1 << 31) // (c * sp) + 3                      # 2051 samples
+    cl = kind.endswith("_cl")
+    per_sample = kind == "in_per_sample"
+    rng = np.random.default_rng(73)
+    shape_b = (1, sp, c) if cl else (1, c, sp)
+    xb = (rng.standard_normal(shape_b) * 1.5).astype(np.float16)
+    dyb = rng.standard_normal(shape_b).astype(np.float16)
+    g = rng.uniform(0.5, 1.5, c).astype(np.float32)
+    b = (rng.standard_normal(c) * 0.1).astype(np.float32)
+    x = torch.from_numpy(xb).cuda().repeat(n, 1, 1)
+    dy = torch.from_numpy(dyb).cuda().repeat(n, 1, 1)
+    assert x.numel() > (1 << 31)
+    gd, bd = to_dev(g), to_dev(b)
+    if per_sample:                                      # gamma / beta of shape [N, C]
+        gd, bd = gd.repeat(n).contiguous(), bd.repeat(n).contiguous()
+    xt = np.moveaxis(xb, -1, 1) if cl else xb
+    dyt = np.moveaxis(dyb, -1, 1) if cl else dyb
+    back = (lambda a: np.moveaxis(np.asarray(a).reshape(xt.shape), 1, -1)) if cl else \
+        (lambda a: np.asarray(a).reshape(xt.shape))
+    bc = not per_sample
+    if kind.startswith("gn"):
+        y, m, v = K.gn_forward(x, bd, gd, groups, 1e-5, channel_last=cl)
+        y_r, m_r, v_r = R.gn_forward(xt, b, g, 1, c, groups, 1e-5)
+        dx_r, dg_r, db_r = R.gn_backward(xt, dyt, g, m_r, v_r, 1, c, groups, 1e-5)
+    else:
+        y, m, v = K.in_forward(x, bd, gd, 1e-5, bc_gamma=bc, bc_beta=bc, channel_last=cl)
+        y_r, m_r, v_r = R.in_forward(xt, b, g, 1, c, 1e-5)
+        dx_r, dg_r, db_r = R.in_backward(xt, dyt, g, m_r, v_r, 1, c, 1e-5)
+    per = m.numel() // n
+    _tiles_close(m.view(n, per), n, np.asarray(m_r).ravel(), "f16", "stat", "mean")
+    _tiles_close(v.view(n, per), n, np.asarray(v_r).ravel(), "f16", "stat", "var")
+    _tiles_close(y, n, back(y_r)[0], "f16", "y", "y")
+    del y
+    if kind.startswith("gn"):
+        dx, dg, db = K.gn_backward(x, dy, gd, m, v, groups, 1e-5, channel_last=cl)
+    else:
+        dx, dg, db = K.in_backward(x, dy, gd, m, v, 1e-5, bc_gamma=bc, bc_beta=bc, channel_last=cl)
+    _tiles_close(dx, n, back(dx_r)[0], "f16", "grad", "dx")
+    if per_sample:
+        _tiles_close(dg.view(n, c), n, dg_r, "f16", "pgrad", "dgamma per sample")
+        _tiles_close(db.view(n, c), n, db_r, "f16", "pgrad", "dbeta per sample")
+    else:
+        assert_close(to_np(dg) / n, dg_r, "f16", "pgrad", "dgamma / n")
+        assert_close(to_np(db) / n, db_r, "f16", "pgrad", "dbeta / n")
+
+
+@pytest.mark.parametrize("kind", ["gn_cl", "in_cl"])
+def test_channel_last_batch_beyond_65535(kind):
+    """70 000 samples: the channel-last kernels put the sample on a grid axis
+    (65535 at most); the C-ABI runs them in two ranges.  The reference has no
+    such limit (group_normalization.cu:57-62)."""
+    n, blk, sp, c, groups = 70000, 8, (4, 4), 64, 8
+    tiles = n // blk
+    rng = np.random.default_rng(74)
+    xb = (rng.standard_normal((blk,) + sp + (c,)) * 1.5 + rng.uniform(-1, 1, (blk, 1, 1, c))).astype(np.float16)
+    dyb = rng.standard_normal((blk,) + sp + (c,)).astype(np.float16)
+    g = rng.uniform(0.5, 1.5, c).astype(np.float32)
+    b = (rng.standard_normal(c) * 0.1).astype(np.float32)
+    x = torch.from_numpy(xb).cuda().repeat(tiles, 1, 1, 1)
+    dy = torch.from_numpy(dyb).cuda().repeat(tiles, 1, 1, 1)
+    gd, bd = to_dev(g), to_dev(b)
+    xt, dyt = np.moveaxis(xb, -1, 1), np.moveaxis(dyb, -1, 1)
+    back = lambda a: np.moveaxis(np.asarray(a).reshape(xt.shape), 1, -1)
+    if kind == "gn_cl":
+        y, m, v = K.gn_forward(x, bd, gd, groups, 1e-5, channel_last=True)
+        dx, dg, db = K.gn_backward(x, dy, gd, m, v, groups, 1e-5, channel_last=True)
+        y_r, m_r, v_r = R.gn_forward(xt, b, g, blk, c, groups, 1e-5)
+        dx_r, dg_r, db_r = R.gn_backward(xt, dyt, g, m_r, v_r, blk, c, groups, 1e-5)
+    else:
+        y, m, v = K.in_forward(x, bd, gd, 1e-5, channel_last=True)
+        dx, dg, db = K.in_backward(x, dy, gd, m, v, 1e-5, channel_last=True)
+        y_r, m_r, v_r = R.in_forward(xt, b, g, blk, c, 1e-5)
+        dx_r, dg_r, db_r = R.in_backward(xt, dyt, g, m_r, v_r, blk, c, 1e-5)
+    per = m.numel() // tiles
+    _tiles_close(m.view(tiles, per), tiles, np.asarray(m_r).ravel(), "f16", "stat", "mean")
+    _tiles_close(y.view((tiles, blk) + sp + (c,)), tiles, back(y_r), "f16", "y", "y")
+    _tiles_close(dx.view((tiles, blk) + sp + (c,)), tiles, back(dx_r), "f16", "grad", "dx")
+    assert_close(to_np(dg) / tiles, dg_r, "f16", "pgrad", "dgamma / tiles")
+    assert_close(to_np(db) / tiles, db_r, "f16", "pgrad", "dbeta / tiles")
