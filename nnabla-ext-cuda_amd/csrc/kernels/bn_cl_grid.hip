@@ -12,8 +12,9 @@
 // The blocks then exchange their per-channel partials as {value, epoch} words
 // (xchg.cuh) in two stages: block c merges the partials of channel c from all
 // blocks (fixed order), writes mean / var / running statistics and publishes
-// the result once per block (were all blocks to poll the same C words, the one
-// memory channel that holds them would queue the polls of 16 000 threads); every
+// the result in eight copies (block b reads copy b % 8: all blocks polling the
+// same C words queue up on the memory channel that holds them, a copy per block
+// is 256 scattered stores per channel); every
 // block reads its copy of the C results and normalizes what it holds: x
 // crosses the memory system once (2 S).
 //
@@ -33,11 +34,30 @@
 
 namespace nblahip {
 
+#ifdef NBLAHIP_GRID_DBG
+// Phase clocks of a debug build (never compiled into the library that ships).
+__device__ unsigned long long grid_dbg_clk[256 * 16];
+#define GRID_CLK(i)                                                                    \
+  do {                                                                                 \
+    if (threadIdx.x == 0) grid_dbg_clk[blockIdx.x * 16 + (i)] = wall_clock64();        \
+  } while (0)
+#else
+#define GRID_CLK(i) \
+  do {              \
+  } while (0)
+#endif
+
 namespace {
 
 constexpr int kGridMaxBlocks = 256; // partials per channel a block merges (one per thread of a wave quad)
 constexpr int kGridMaxC = 128;      // channels (LDS fold of the per-channel sums) of the layouts that hold most
 constexpr int kGridWideC = 512;     // channels of the layouts with three LDS slots fewer
+// Copies of the per-channel results of stage 2; block b reads copy b % 8.  A
+// copy per block (256 scattered 8-byte stores per channel) made the second hop
+// three times as slow as the first, one copy for all makes every block poll the
+// same eight cache lines ([256,56,56,64] half forward / backward: 49.1 / 76.0 us
+// with 256 copies, 46.9 / 75.0 with 8, 48.4 / 76.0 with one).
+constexpr uint32_t kGridCopies = 8;
 
 struct BnClGridArgs {
   const void *x;
@@ -58,9 +78,10 @@ struct BnClGridArgs {
   int accum_dx, accum_g, accum_b;
   unsigned long long *x1; // stage 1: [nblocks][C][2] = (mean, m2) of the block's rows
                           //          (backward: (sum dy*xh, sum dy))
-  unsigned long long *x2; // stage 2: [nblocks][C][2] = (mean, var), a copy for every block
+  unsigned long long *x2; // stage 2: [copies][C][2] = (mean, var)
   uint32_t epoch;
   int spin;
+  uint32_t copies; // copies of the stage-2 results; block b reads copy b % copies
 };
 
 // Vectors of block b.
@@ -80,24 +101,25 @@ template <int VEC>
 __device__ __forceinline__ void grid_channel_sums(float (&v)[VEC], uint32_t cv, uint32_t cvx,
                                                   float *fold, float *tot, uint32_t C) {
   constexpr int NW = kOnchipBlock / kWave;
-#pragma unroll
-  for (int j = 0; j < VEC; ++j) {
-    for (uint32_t off = cv; off < kWave; off <<= 1) v[j] += __shfl_xor(v[j], off);
-  }
+  lanes_sum_from<VEC>(v, cv); // (a step at a time for all values, off the LDS crossbar: xor_add)
+  GRID_CLK(10);
   if ((threadIdx.x & (kWave - 1)) < cv) {
 #pragma unroll
     for (int j = 0; j < VEC; ++j) fold[(threadIdx.x / kWave) * C + cvx * VEC + j] = v[j];
   }
   lds_barrier();
+  GRID_CLK(11);
   if (threadIdx.x < C) {
     float t = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) t += fold[w * C + threadIdx.x];
     tot[threadIdx.x] = t;
   }
+  GRID_CLK(12);
   lds_barrier();
 #pragma unroll
   for (int j = 0; j < VEC; ++j) v[j] = tot[cvx * VEC + j];
+  GRID_CLK(13);
 }
 
 // The same fold for ONE channel (element e of the vectors of channel vector
@@ -105,7 +127,7 @@ __device__ __forceinline__ void grid_channel_sums(float (&v)[VEC], uint32_t cv, 
 __device__ __forceinline__ float grid_channel_sum1(float v, uint32_t cv, uint32_t cvx, uint32_t c,
                                                    bool mine, float *fold, uint32_t C) {
   constexpr int NW = kOnchipBlock / kWave;
-  for (uint32_t off = cv; off < kWave; off <<= 1) v += __shfl_xor(v, off);
+  v = lanes_sum_from(v, cv);
   lds_barrier(); // earlier readers of fold are done
   if ((threadIdx.x & (kWave - 1)) < cv && mine) fold[(threadIdx.x / kWave) * C + c] = v;
   lds_barrier();
@@ -184,6 +206,7 @@ __device__ __forceinline__ void grid_channel_result(const BnClGridArgs &a, uint3
     if (!ok) miss[kGridMaxBlocks] = 1;
   }
   lds_barrier();
+  GRID_CLK(9);
   for (uint32_t p = 0; miss[kGridMaxBlocks] && p < a.nblocks; ++p) {
     if (!miss[p]) continue; // same answer in every thread
     float m, q;
@@ -292,6 +315,7 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
   __shared__ float gb[2 * CMAX]; // gamma, beta
   const uint32_t b = blockIdx.x;
   const uint32_t t = threadIdx.x;
+  GRID_CLK(0);
   // gamma and beta of channel t, asked for ahead of the tensor (behind the
   // exchange they would cost a memory round trip of their own)
   float gamma_t = 1.f, beta_t = 0.f;
@@ -376,7 +400,9 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
         }
       }
     }
+    GRID_CLK(1);
     grid_channel_sums<VEC>(m, a.cv, cvx, fold, tot, a.C);
+    GRID_CLK(2);
     const float icnt = 1.0f / static_cast<float>(vbb / a.cv);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
@@ -385,6 +411,7 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
       q[j] = fmaf(e, fmaf(nt, e, 2.f * s1[j]), s2[j]);
     }
     grid_channel_sums<VEC>(q, a.cv, cvx, fold, tot, a.C);
+    GRID_CLK(3);
   }
   // publish (mean, m2) of every channel: a word per thread (through fin, which
   // is free until the results arrive)
@@ -398,31 +425,34 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
   lds_barrier();
   for (uint32_t e = t; e < 2 * a.C; e += kOnchipBlock)
     xchg_publish(a.x1 + static_cast<size_t>(b) * a.C * 2 + e, fin[e], a.epoch);
+  GRID_CLK(4);
 
   // ---- stage 2: block c merges channel c, writes its statistics, publishes
   for (uint32_t c = b; c < a.C; c += a.nblocks) {
     float mean, var;
     grid_channel_result<T, VEC>(a, c, miss, got, wel, fold, mean, var);
+    GRID_CLK(5);
     if (t == 0) {
       a.mean[c] = mean;
       a.var[c] = var;
       if (a.rmean) a.rmean[c] = a.decay * a.rmean[c] + (1.f - a.decay) * mean;
       if (a.rvar) a.rvar[c] = a.decay * a.rvar[c] + (1.f - a.decay) * var * a.unbias;
     }
-    if (t < a.nblocks) { // a copy for block t
+    if (t < a.copies) { // copy t
       unsigned long long *w = a.x2 + (static_cast<size_t>(t) * a.C + c) * 2;
       xchg_publish(w, mean, a.epoch);
       xchg_publish(w + 1, var, a.epoch);
     }
   }
 
+  GRID_CLK(6);
   // ---- every block: the C results (merged here where one does not arrive)
   lds_barrier();
   if (t == 0) miss[kGridMaxBlocks + 1] = 0;
   lds_barrier();
   for (uint32_t c = t; c < a.C; c += kOnchipBlock) {
     float v0 = 0.f, v1 = 0.f;
-    const bool ok = xchg_poll2(a.x2 + (static_cast<size_t>(b) * a.C + c) * 2, a.epoch, a.spin, &v0, &v1);
+    const bool ok = xchg_poll2(a.x2 + (static_cast<size_t>(b % a.copies) * a.C + c) * 2, a.epoch, a.spin, &v0, &v1);
     fin[2 * c] = v0;
     fin[2 * c + 1] = ok ? v1 : -1.f; // a variance is never negative: marks "missing"
     if (!ok) miss[kGridMaxBlocks + 1] = 1;
@@ -440,6 +470,7 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
     lds_barrier();
   }
 
+  GRID_CLK(7);
   // ---- normalize what the block holds
 #pragma unroll
   for (int k = 0; k < NR; ++k) forget<T, VEC>(raw[k]);
@@ -469,6 +500,7 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
       store_vec<T, VEC>(y + static_cast<size_t>(v) * VEC, o);
     }
   }
+  GRID_CLK(8);
 }
 
 // Backward (batch statistics).  With xh = (x-mean)*istd per channel:
@@ -608,7 +640,7 @@ bn_cl_grid_bwd_kernel(const BnClGridArgs a) {
       if (a.dgamma) a.dgamma[c] = tx + (a.accum_g ? a.dgamma[c] : 0.f);
       if (a.dbeta) a.dbeta[c] = ty + (a.accum_b ? a.dbeta[c] : 0.f);
     }
-    if (t < a.nblocks) { // a copy for block t
+    if (t < a.copies) { // copy t
       unsigned long long *w = a.x2 + (static_cast<size_t>(t) * a.C + c) * 2;
       xchg_publish(w, tx, a.epoch);
       xchg_publish(w + 1, ty, a.epoch);
@@ -622,7 +654,7 @@ bn_cl_grid_bwd_kernel(const BnClGridArgs a) {
   lds_barrier();
   for (uint32_t c = t; c < a.C; c += kOnchipBlock) {
     float v0 = 0.f, v1 = 0.f;
-    const bool ok = xchg_poll2(a.x2 + (static_cast<size_t>(b) * a.C + c) * 2, a.epoch, a.spin, &v0, &v1);
+    const bool ok = xchg_poll2(a.x2 + (static_cast<size_t>(b % a.copies) * a.C + c) * 2, a.epoch, a.spin, &v0, &v1);
     fin[2 * c] = v0;
     fin[2 * c + 1] = v1;
     finmiss[c] = ok ? 0 : 1;
@@ -815,12 +847,13 @@ bool grid_args(const BnProblem &p, BnClGridArgs &a, int &nl) {
   a.eps = p.eps;
   a.one = 1.0f;
   a.spin = tune_int("XCHG_SPIN", 64) * 16; // a whole-chip exchange: wait longer before recomputing
+  a.copies = std::min<uint32_t>(kGridCopies, a.nblocks);
   return true;
 }
 
 // Exchange words of both stages.
 bool grid_exchange(const BnProblem &p, BnClGridArgs &a, hipStream_t st, int *status) {
-  const size_t words = static_cast<size_t>(a.nblocks) * p.C * 4;
+  const size_t words = static_cast<size_t>(a.nblocks + a.copies) * p.C * 2;
   if (!xchg_acquire(words, st, &a.x1, &a.epoch, status)) return false;
   a.x2 = a.x1 + static_cast<size_t>(a.nblocks) * p.C * 2;
   return true;
@@ -866,3 +899,10 @@ bool bn_cl_grid_bwd(const BnProblem &p, hipStream_t st, int *status) {
 }
 
 } // namespace nblahip
+
+#ifdef NBLAHIP_GRID_DBG
+extern "C" __attribute__((visibility("default"))) int nblahip_debug_grid_clocks(unsigned long long *host) {
+  return static_cast<int>(hipMemcpyFromSymbol(host, HIP_SYMBOL(nblahip::grid_dbg_clk),
+                                              sizeof(unsigned long long) * 256 * 16));
+}
+#endif

@@ -420,6 +420,89 @@ __device__ __forceinline__ float wave_sum(float v) {
   return (read_lane(v, 0) + read_lane(v, 16)) + (read_lane(v, 32) + read_lane(v, 48));
 }
 
+// v + (v of lane ^ OFF), OFF a power of two below 64, without the LDS crossbar
+// where the vector unit has a path of its own: quad_perm for 1 and 2, a row
+// rotation for 8 (lane (i + 8) % 16 of the 16-lane row is lane i ^ 8), and
+// gfx950's row and half-wave swaps for 16 and 32 (with both operands the same
+// register, v_permlane16_swap leaves rows (r0, r0, r2, r2) and (r1, r1, r3, r3),
+// v_permlane32_swap halves (lo, lo) and (hi, hi): their sum is the butterfly
+// step, in every lane the same two addends).  ds_bpermute for 4.  Sixteen waves
+// folding 8 values over 3 steps through ds_bpermute kept a CU's LDS busy for
+// 1.4 us; on these paths the same fold is 60 vector instructions per wave.
+// (Written as inline assembly: the builtins of ROCm 7.2's compiler,
+// __builtin_amdgcn_permlane16_swap / 32_swap, return the first register for
+// both halves of their result pair.  The swap works in place on two registers;
+// the idle cycles around it keep it clear of the vector results before it and
+// of its readers, which the compiler's hazard pass cannot see inside asm.)
+__device__ __forceinline__ float swap_add16(float v) {
+  float a = v, b = v;
+  asm volatile("s_nop 3\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return a + b;
+}
+__device__ __forceinline__ float swap_add32(float v) {
+  float a = v, b = v;
+  asm volatile("s_nop 3\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return a + b;
+}
+template <int OFF> __device__ __forceinline__ float xor_add(float v) {
+  static_assert(OFF == 1 || OFF == 2 || OFF == 4 || OFF == 8 || OFF == 16 || OFF == 32, "lane bit");
+  if constexpr (OFF == 1) {
+    return v + dpp_move<0xB1>(v);
+  } else if constexpr (OFF == 2) {
+    return v + dpp_move<0x4E>(v);
+  } else if constexpr (OFF == 8) {
+    return v + dpp_move<0x128>(v); // row_ror:8
+  } else if constexpr (OFF == 16) {
+    return swap_add16(v);
+  } else if constexpr (OFF == 32) {
+    return swap_add32(v);
+  } else {
+    return v + __shfl_xor(v, OFF);
+  }
+}
+
+// Butterfly sums of N values at once over the lane bits lo, 2 lo, ... 32
+// (lanes_sum_from: every lane ends with the sum over the lanes that differ
+// from it in those bits only) or 1, 2, ... hi / 2 (lanes_sum_below); lo and hi
+// are powers of two known at run time, uniform over the wave.  A step at a time
+// for all values, so that the cross-lane operations of a step overlap.
+template <int N> __device__ __forceinline__ void lanes_sum_from(float (&v)[N], uint32_t lo) {
+#define NBLAHIP_STEP(OFF)                                  \
+  if (lo <= (OFF)) {                                       \
+    _Pragma("unroll") for (int j = 0; j < N; ++j) v[j] = xor_add<OFF>(v[j]); \
+  }
+  NBLAHIP_STEP(1)
+  NBLAHIP_STEP(2)
+  NBLAHIP_STEP(4)
+  NBLAHIP_STEP(8)
+  NBLAHIP_STEP(16)
+  NBLAHIP_STEP(32)
+#undef NBLAHIP_STEP
+}
+template <int N> __device__ __forceinline__ void lanes_sum_below(float (&v)[N], uint32_t hi) {
+#define NBLAHIP_STEP(OFF)                                  \
+  if (hi > (OFF)) {                                        \
+    _Pragma("unroll") for (int j = 0; j < N; ++j) v[j] = xor_add<OFF>(v[j]); \
+  }
+  NBLAHIP_STEP(1)
+  NBLAHIP_STEP(2)
+  NBLAHIP_STEP(4)
+  NBLAHIP_STEP(8)
+  NBLAHIP_STEP(16)
+  NBLAHIP_STEP(32)
+#undef NBLAHIP_STEP
+}
+__device__ __forceinline__ float lanes_sum_from(float x, uint32_t lo) {
+  float v[1] = {x};
+  lanes_sum_from<1>(v, lo);
+  return v[0];
+}
+__device__ __forceinline__ float lanes_sum_below(float x, uint32_t hi) {
+  float v[1] = {x};
+  lanes_sum_below<1>(v, hi);
+  return v[0];
+}
+
 // Sum over aligned groups of G = 4, 8, 16 or 32 adjacent lanes (every lane of
 // a group returns the group's sum): the first steps of wave_sum, and one lane
 // exchange between the two 16-lane rows for G = 32.  Lanes of a group must be
@@ -430,7 +513,7 @@ template <int G> __device__ __forceinline__ float group_sum(float v) {
   v += dpp_move<0x4E>(v);
   if constexpr (G >= 8) v += dpp_move<0x141>(v);
   if constexpr (G >= 16) v += dpp_move<0x140>(v);
-  if constexpr (G == 32) v += __shfl_xor(v, 16);
+  if constexpr (G == 32) v = xor_add<16>(v);
   return v;
 }
 

@@ -228,6 +228,8 @@ gn_cl_row_bwd_kernel(const GnClArgs a) {
   // butterfly over the lane bits above log2(cvg), then one LDS row per wave.
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
+  // (through the LDS crossbar: on the vector unit's swap paths, xor_add, these
+  // two kernels need a few registers more than their 128 and spill)
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
     for (int off = static_cast<int>(a.cvg.d); off < kWave; off <<= 1) {
@@ -597,11 +599,7 @@ in_cl_wide_fwd_kernel(const GnClArgs a) {
   // sums over the threads with the same channel vector (lane % CVB == cvx)
   auto block_sums = [&](float (&v)[VEC]) {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-#pragma unroll
-      for (int off = CVB; off < kWave; off <<= 1) v[j] += __shfl_xor(v[j], off);
-    }
+    lanes_sum_from<VEC>(v, static_cast<uint32_t>(CVB));
     lds_barrier(); // previous readers of lds are done
     if (lane < CVB) {
 #pragma unroll
@@ -720,8 +718,8 @@ gn_cl_wide_fwd_kernel(const GnClArgs a) {
   }
   auto group_block_sum = [&](float v) -> float {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    for (int off = static_cast<int>(a.chunk.d); off < kWave; off <<= 1) v += __shfl_xor(v, off);
-    for (int off = 1; off < static_cast<int>(a.cvg.d); off <<= 1) v += __shfl_xor(v, off);
+    v = lanes_sum_from(v, a.chunk.d);
+    v = lanes_sum_below(v, a.cvg.d);
     lds_barrier(); // previous readers of lds are done
     if (lane < static_cast<int>(a.chunk.d) && cvx == sg * a.cvg.d) lds[wave][sg] = v;
     lds_barrier();
@@ -851,6 +849,7 @@ cl_wide_bwd_kernel(const GnClArgs a) {
     }
   }
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  // (as above: the swap paths cost this kernel registers it does not have)
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
 #pragma unroll

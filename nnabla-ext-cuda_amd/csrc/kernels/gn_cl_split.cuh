@@ -145,10 +145,8 @@ template <int TPR>
 __device__ __forceinline__ float split_group_sum(float v, int cvg_shift, uint32_t cvx, uint32_t gi,
                                                  float (*fold)[kSplitTV]) {
   constexpr int NW = TPR / kWave;
-  for (int off = 1; off < (1 << cvg_shift); off <<= 1) v += __shfl_xor(v, off);
-  v += __shfl_xor(v, 8);
-  v += __shfl_xor(v, 16);
-  v += __shfl_xor(v, 32);
+  v = lanes_sum_below(v, 1u << cvg_shift);
+  v = lanes_sum_from(v, 8u);
   lds_barrier(); // earlier readers of fold are done
   if ((threadIdx.x & (kWave - 1)) < kSplitTV && (cvx & ((1u << cvg_shift) - 1)) == 0)
     fold[threadIdx.x / kWave][gi] = v;
@@ -168,11 +166,7 @@ __device__ __forceinline__ void split_channel_sums(float (&v)[VEC], uint32_t cvx
                                                    float (*fold)[kSplitTV * VEC], float *tot) {
   constexpr int NW = TPR / kWave;
 #pragma unroll
-  for (int j = 0; j < VEC; ++j) {
-    v[j] += __shfl_xor(v[j], 8);
-    v[j] += __shfl_xor(v[j], 16);
-    v[j] += __shfl_xor(v[j], 32);
-  }
+  for (int j = 0; j < VEC; ++j) v[j] = xor_add<32>(xor_add<16>(xor_add<8>(v[j])));
   lds_barrier(); // earlier readers of fold / tot are done
   if ((threadIdx.x & (kWave - 1)) < kSplitTV) {
 #pragma unroll
@@ -201,12 +195,8 @@ __device__ __forceinline__ void split_pair_sums(float (&sdx)[VEC], float (&sdy)[
   constexpr int CH = kSplitTV * VEC;
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
-    sdx[j] += __shfl_xor(sdx[j], 8);
-    sdy[j] += __shfl_xor(sdy[j], 8);
-    sdx[j] += __shfl_xor(sdx[j], 16);
-    sdy[j] += __shfl_xor(sdy[j], 16);
-    sdx[j] += __shfl_xor(sdx[j], 32);
-    sdy[j] += __shfl_xor(sdy[j], 32);
+    sdx[j] = xor_add<32>(xor_add<16>(xor_add<8>(sdx[j])));
+    sdy[j] = xor_add<32>(xor_add<16>(xor_add<8>(sdy[j])));
   }
   lds_barrier(); // earlier readers of fold / chs are done
   if ((threadIdx.x & (kWave - 1)) < kSplitTV) {

@@ -394,8 +394,7 @@ ln_param_reduce_kernel(const float *__restrict__ ws, int nparts, int R,
 #pragma unroll
     for (int u = 0; u < 8; ++u) s += v[u];
   }
-  s += __shfl_xor(s, 16);
-  s += __shfl_xor(s, 32);
+  s = xor_add<32>(xor_add<16>(s));
   if ((threadIdx.x & 63) < 16) red[wave][cx] = s;
   lds_barrier();
   if (threadIdx.x < 16 && live) {

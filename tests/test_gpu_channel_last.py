@@ -279,9 +279,15 @@ def test_channel_last_argument_errors():
                                2, 16, 8, 4, 1e-5, 0, ws.data_ptr(), 16, s) == -2  # too small
     assert L.nblahip_gn_cl_fwd(x.data_ptr(), None, None, y.data_ptr(), m.data_ptr(), m.data_ptr(),
                                0, 16, 8, 4, 1e-5, 0, None, 0, s) == 0           # empty: no-op
-    assert L.nblahip_in_cl_fwd(x.data_ptr(), None, None, y.data_ptr(), m.data_ptr(), m.data_ptr(),
+    # (a batch beyond 65535 runs in ranges of samples; it needs its own workspace)
+    assert L.nblahip_in_cl_workspace_bytes(70000, 1, 8, 0) > ws.numel()
+    # (y = x: with these sizes the two small buffers would overlap in part)
+    assert L.nblahip_in_cl_fwd(x.data_ptr(), None, None, x.data_ptr(), m.data_ptr(), m.data_ptr(),
                                70000, 1, 8, 1, 1, 1e-5, 0, ws.data_ptr(), ws.numel(),
-                               s) == -3                                         # batch > 65535
+                               s) == -2
+    assert L.nblahip_in_cl_fwd(x.data_ptr(), None, None, x.data_ptr(), m.data_ptr(), m.data_ptr(),
+                               2, 1 << 16, 1 << 15, 1, 1, 1e-5, 0, ws.data_ptr(), ws.numel(),
+                               s) == -3                                         # 2^31 elements per sample
     assert L.nblahip_in_cl_bwd(x.data_ptr(), None, None, m.data_ptr(), m.data_ptr(), None, None,
                                y.data_ptr(), None, None, 0, 0, 0, 2, 16, 8, 1, 1, 1e-5, 0,
                                ws.data_ptr(), ws.numel(), s) == -1              # dy missing

@@ -368,7 +368,7 @@ def test_row_argument_errors():
                             None, y.data_ptr(), None, None, 0, 0, 0, 8, 64, 1e-5, 0, None, 0,
                             s) == -2                               # workspace missing
     assert L.nblahip_ln_fwd(x.data_ptr(), None, None, y.data_ptr(), m.data_ptr(), m.data_ptr(),
-                            1 << 20, 1 << 20, 1e-5, 0, s) == -3    # >= 2^31 elements
+                            2, 1 << 31, 1e-5, 0, s) == -3          # >= 2^31 elements per row
 
 
 @pytest.mark.parametrize("outer,Rr", [(64, 1024), (300, 48), (2, 131072), (3, 40004)])
