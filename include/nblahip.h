@@ -461,6 +461,20 @@ NBLAHIP_EXPORT int nblahip_convert(void *dst, int dst_dtype, const void *src,
 NBLAHIP_EXPORT int nblahip_fill(void *dst, int dtype, float value, int64_t n,
                                 void *stream);
 
+/* Up to 16 small arrays converted between float16 and float32 in one launch:
+ * dst[k][i] = (dst_dtype) src[k][i] for i < n[k] (arrays with n[k] == 0 are
+ * skipped).  The normalization entry points take gamma, beta, statistics and
+ * their gradients in float32; a "hip:half" graph that stores them in half
+ * precision, as the reference's plain cuda:half type config does (Tc = half:
+ * layer_normalization.cu:91-93, batch_normalization.cu:124-143), has its
+ * Function classes stage them through this call - one launch before the
+ * kernels for everything they read, one after for everything they wrote - so
+ * the stored arrays keep their type. */
+NBLAHIP_EXPORT int nblahip_stage_params(int count, const void *const *src,
+                                        int src_dtype, void *const *dst,
+                                        int dst_dtype, const int64_t *n,
+                                        void *stream);
+
 /* Axis permutation of a contiguous tensor (float32 or float16):
  *   dst[i_perm[0], ..., i_perm[ndim-1]] = src[i_0, ..., i_{ndim-1}]
  * i.e. axis k of dst is axis perm[k] of src, whose extents are shape[0..ndim-1]

@@ -72,6 +72,11 @@ NNABLA_HIP_EXPORT int nnabla_hip_variable_get_raw(nnabla_hip_variable *v, int wh
 NNABLA_HIP_EXPORT int nnabla_hip_pending_transfers(uint64_t *count);
 NNABLA_HIP_EXPORT int nnabla_hip_variable_zero(nnabla_hip_variable *v, int which);
 NNABLA_HIP_EXPORT int nnabla_hip_variable_fill(nnabla_hip_variable *v, int which, float value);
+/* dtype the variable's up-to-date array is stored in (codes as above: 0 float,
+ * 1 half, 0x100 + n otherwise), -1 when it holds nothing yet (never written,
+ * or zeroed / filled lazily). */
+NNABLA_HIP_EXPORT int nnabla_hip_variable_stored_dtype(nnabla_hip_variable *v, int which,
+                                                       int *dtype);
 
 /* Function creation through the registry.  `backends` is the context's backend
  * preference list, comma separated (e.g. "hip:half,hip:float"). */

@@ -107,6 +107,8 @@ SIGNATURES = {
     "nblahip_tune_get": (_int, [ctypes.c_char_p, _int]),
     "nblahip_tune_reset": (_int, []),
     "nblahip_xchg_set_epoch": (_int, [ctypes.c_uint]),
+    "nblahip_stage_params": (_int, [_int, ctypes.POINTER(_c_void_p), _int, ctypes.POINTER(_c_void_p),
+                                    _int, ctypes.POINTER(_i64), _c_void_p]),
 }
 
 _lib = None

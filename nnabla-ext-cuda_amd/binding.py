@@ -41,6 +41,7 @@ SIGNATURES = {
     "nnabla_hip_pending_transfers": (_I, [ctypes.POINTER(ctypes.c_uint64)]),
     "nnabla_hip_variable_zero": (_I, [_P, _I]),
     "nnabla_hip_variable_fill": (_I, [_P, _I, _F]),
+    "nnabla_hip_variable_stored_dtype": (_I, [_P, _I, ctypes.POINTER(_I)]),
     "nnabla_hip_create_batch_normalization": (_P, [_S, _S, _S, _IP, _I, _F, _F, _I, _I, _I]),
     "nnabla_hip_create_fused_batch_normalization": (_P, [_S, _S, _S, _IP, _I, _F, _F, _I, _S]),
     "nnabla_hip_create_layer_normalization": (_P, [_S, _S, _S, _IP, _I, _F, _I, _I]),
@@ -244,6 +245,12 @@ class Variable:
 
     def zero_grad(self):
         _check(lib().nnabla_hip_variable_zero(self._h, 1))
+
+    def stored_dtype(self, which=0):
+        """"float", "half", "other" or None (nothing stored yet) of data (0) / grad (1)."""
+        d = _I(0)
+        _check(lib().nnabla_hip_variable_stored_dtype(self._h, which, ctypes.byref(d)))
+        return {0: "float", 1: "half", -1: None}.get(d.value, "other")
 
     def fill_grad(self, v):
         _check(lib().nnabla_hip_variable_fill(self._h, 1, float(v)))

@@ -482,6 +482,13 @@ public:
     zeroing_ = filling_ = false;
   }
   bool zeroing() const { return zeroing_; }
+  // dtype of the up-to-date materialisation (the core's SyncedArray::dtype()
+  // likewise raises for an array that holds nothing yet).
+  dtypes dtype() const {
+    NBLA_CHECK(has_head_ && !zeroing_ && !filling_ && !head_.first.empty(), error_code::unclassified,
+               "Array is not initialized.");
+    return static_cast<dtypes>(head_.second);
+  }
 };
 typedef shared_ptr<SyncedArray> SyncedArrayPtr;
 

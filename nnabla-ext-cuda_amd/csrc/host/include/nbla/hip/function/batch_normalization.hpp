@@ -1,14 +1,19 @@
 // BatchNormalizationHip<T>: the "hip" implementation of BatchNormalization,
 // same constructor, name()/allowed_array_classes() and *_impl overrides as
 // BatchNormalizationCuda<T> (include/nbla/cuda/function/batch_normalization.hpp:31-85).
-// Statistics, gamma/beta and their gradients are float32 for every T, as in
-// the reference's cudnn context
+// The kernels take statistics, gamma/beta and their gradients as float32 for
+// every T, as the reference's cudnn context does
 // (src/nbla/cuda/cudnn/function/generic/batch_normalization.cu:94-99,193-227).
+// Arrays that a "hip:half" graph stores in half - the plain cuda:half config's
+// Tc (batch_normalization.cu:124-143) - are read and written where they lie
+// and keep their type (nbla/hip/utils/param_stage.hpp); the batch statistics
+// the function keeps for its own backward stay float32.
 #pragma once
 
 #include <nbla/function/batch_normalization.hpp>
 #include <nbla/hip/common.hpp>
 #include <nbla/hip/hip.hpp>
+#include <nbla/hip/utils/param_stage.hpp>
 
 namespace nbla {
 
@@ -17,6 +22,7 @@ protected:
   int device_;
   Variable workspace_; // split-reduction partials + per-channel parameters
   size_t workspace_bytes_ = 0;
+  Variable stage_; // float32 staging of parameters / statistics stored in half (ParamStage)
 
 public:
   BatchNormalizationHip(const Context &ctx, const vector<int> axes, float decay_rate, float eps,

@@ -6,6 +6,7 @@
 #include <nbla/function/instance_normalization.hpp>
 #include <nbla/hip/common.hpp>
 #include <nbla/hip/hip.hpp>
+#include <nbla/hip/utils/param_stage.hpp>
 #include <nbla/hip/utils/channel_layout.hpp>
 
 namespace nbla {
@@ -17,6 +18,7 @@ protected:
   bool channel_last_ = false; // x is [batch..., spatial..., channel]
   Variable mean_, var_;   // float32 per-(n, c) statistics kept for backward
   Variable workspace_;
+  Variable stage_; // float32 staging of parameters / statistics stored in half (ParamStage)
   size_t workspace_bytes_ = 0;
   // Layouts that are neither channel-first nor channel-last: permuted copies
   // of x / dy / y / dx, of the statistics and of per-sample parameters, alive

@@ -7,6 +7,7 @@
 #include <nbla/hip/common.hpp>
 #include <nbla/hip/hip.hpp>
 #include <nbla/hip/utils/axis_adaptor.hpp>
+#include <nbla/hip/utils/param_stage.hpp>
 
 namespace nbla {
 
@@ -17,6 +18,7 @@ protected:
   Variable mean_, var_;   // float32 row statistics kept for backward
   Variable workspace_;
   size_t workspace_bytes_ = 0;
+  Variable stage_; // float32 staging of parameters / statistics stored in half (ParamStage)
   // Batch axes that are not the leading ones: permuted copies of x / dy / y /
   // dx, alive only inside a call.
   AxisAdaptor adaptor_;

@@ -4,6 +4,8 @@
 #include <nbla/hip/function/batch_normalization.hpp>
 #include <nbla/variable.hpp>
 
+#include <type_traits>
+
 namespace nbla {
 
 template <typename T>
@@ -15,6 +17,10 @@ void BatchNormalizationHip<T>::setup_impl(const Variables &inputs, const Variabl
   workspace_bytes_ = nblahip_bn_workspace_bytes(this->size0_, this->size1_, this->size2_,
                                                 HipDtype<T>::code);
   workspace_.reshape(Shape_t{static_cast<Size_t>((workspace_bytes_ + 3) / 4)}, true);
+  if (std::is_same<T, Half>::value) {
+    const Size_t c = this->size1_;
+    stage_.reshape(Shape_t{ParamStage::capacity_for({c, c, c, c, c, c, c, c})}, true);
+  }
 }
 
 template <typename T>
@@ -49,36 +55,41 @@ void BatchNormalizationHip<T>::forward_impl_batch(const Variables &inputs, const
     batch_var = outputs[2];
   }
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
-  const float *beta =
-      this->no_bias_ ? nullptr : inputs[this->b_idx_]->template get_data_pointer<float>(this->ctx_);
-  const float *gamma =
-      this->no_scale_ ? nullptr : inputs[this->g_idx_]->template get_data_pointer<float>(this->ctx_);
-  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
-  float *m = batch_mean->cast_data_and_get_pointer<float>(this->ctx_, true);
-  float *v = batch_var->cast_data_and_get_pointer<float>(this->ctx_, true);
+  // (parameters and statistics a half graph stores in half are read and
+  // written where they lie: ParamStage)
+  ParamStage st;
+  st.begin(this->ctx_, std::is_same<T, Half>::value, &stage_);
+  const float *beta = this->no_bias_ ? nullptr : st.in(inputs[this->b_idx_]);
+  const float *gamma = this->no_scale_ ? nullptr : st.in(inputs[this->g_idx_]);
   // Running statistics are read-modify-write inputs; recompute leaves them.
-  float *rm = !update_inputs
-                  ? nullptr
-                  : inputs[this->m_idx_]->template cast_data_and_get_pointer<float>(this->ctx_);
-  float *rv = !update_inputs
-                  ? nullptr
-                  : inputs[this->v_idx_]->template cast_data_and_get_pointer<float>(this->ctx_);
+  float *rm = !update_inputs ? nullptr : st.out(inputs[this->m_idx_], true);
+  float *rv = !update_inputs ? nullptr : st.out(inputs[this->v_idx_], true);
+  T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
+  // (statistics kept inside the function stay float32; exposed ones follow the parameters)
+  const bool exposed = outputs.size() == 3;
+  float *m = exposed ? st.out(batch_mean, false)
+                     : batch_mean->cast_data_and_get_pointer<float>(this->ctx_, true);
+  float *v = exposed ? st.out(batch_var, false)
+                     : batch_var->cast_data_and_get_pointer<float>(this->ctx_, true);
+  st.load();
   float *ws = workspace_.cast_data_and_get_pointer<float>(this->ctx_, true);
   NBLA_HIP_CHECK(nblahip_bn_fwd_train(x, gamma, beta, y, m, v, rm, rv, this->size0_, this->size1_,
                                       this->size2_, this->decay_rate_, this->eps_,
                                       HipDtype<T>::code, ws, workspace_bytes_, nullptr));
+  st.store();
 }
 
 template <typename T>
 void BatchNormalizationHip<T>::forward_impl_global(const Variables &inputs,
                                                    const Variables &outputs) {
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
-  const float *beta =
-      this->no_bias_ ? nullptr : inputs[this->b_idx_]->template get_data_pointer<float>(this->ctx_);
-  const float *gamma =
-      this->no_scale_ ? nullptr : inputs[this->g_idx_]->template get_data_pointer<float>(this->ctx_);
-  const float *rm = inputs[this->m_idx_]->template get_data_pointer<float>(this->ctx_);
-  const float *rv = inputs[this->v_idx_]->template get_data_pointer<float>(this->ctx_);
+  ParamStage st;
+  st.begin(this->ctx_, std::is_same<T, Half>::value, &stage_);
+  const float *beta = this->no_bias_ ? nullptr : st.in(inputs[this->b_idx_]);
+  const float *gamma = this->no_scale_ ? nullptr : st.in(inputs[this->g_idx_]);
+  const float *rm = st.in(inputs[this->m_idx_]);
+  const float *rv = st.in(inputs[this->v_idx_]);
+  st.load();
   T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
   NBLA_HIP_CHECK(nblahip_bn_fwd_infer(x, rm, rv, gamma, beta, y, this->size0_, this->size1_,
                                       this->size2_, this->eps_, HipDtype<T>::code, nullptr));
@@ -123,8 +134,9 @@ void BatchNormalizationHip<T>::backward_launch(const Variables &inputs, const Va
 
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
   const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
-  const float *gamma =
-      this->no_scale_ ? nullptr : inputs[this->g_idx_]->template get_data_pointer<float>(this->ctx_);
+  ParamStage st;
+  st.begin(this->ctx_, std::is_same<T, Half>::value, &stage_);
+  const float *gamma = this->no_scale_ ? nullptr : st.in(inputs[this->g_idx_]);
 
   // Statistics the forward normalised with, and the gradients that reach the
   // mean/var outputs in the three-output form.
@@ -135,29 +147,27 @@ void BatchNormalizationHip<T>::backward_launch(const Variables &inputs, const Va
     if (outputs.size() == 3) {
       batch_mean = outputs[1];
       batch_var = outputs[2];
-      dmean = batch_mean->get_grad_pointer<float>(this->ctx_);
-      dvar = batch_var->get_grad_pointer<float>(this->ctx_);
+      dmean = st.in(batch_mean, true);
+      dvar = st.in(batch_var, true);
     }
-    mean = batch_mean->get_data_pointer<float>(this->ctx_);
-    var = batch_var->get_data_pointer<float>(this->ctx_);
+    mean = st.in(batch_mean);
+    var = st.in(batch_var);
   } else {
-    mean = inputs[this->m_idx_]->template get_data_pointer<float>(this->ctx_);
-    var = inputs[this->v_idx_]->template get_data_pointer<float>(this->ctx_);
+    mean = st.in(inputs[this->m_idx_]);
+    var = st.in(inputs[this->v_idx_]);
   }
 
   T *dx = !pd_x ? nullptr : inputs[0]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[0]);
-  float *dbeta = !pd_beta ? nullptr
-                          : inputs[this->b_idx_]->template cast_grad_and_get_pointer<float>(
-                                this->ctx_, !accum[this->b_idx_]);
-  float *dgamma = !pd_gamma ? nullptr
-                            : inputs[this->g_idx_]->template cast_grad_and_get_pointer<float>(
-                                  this->ctx_, !accum[this->g_idx_]);
+  float *dbeta = !pd_beta ? nullptr : st.out(inputs[this->b_idx_], accum[this->b_idx_], true);
+  float *dgamma = !pd_gamma ? nullptr : st.out(inputs[this->g_idx_], accum[this->g_idx_], true);
+  st.load();
   float *ws = workspace_.cast_data_and_get_pointer<float>(this->ctx_, true);
   NBLA_HIP_CHECK(nblahip_bn_bwd(
       x, dy, gamma, mean, var, dmean, dvar, dx, dgamma, dbeta, pd_x && accum[0],
       pd_gamma && accum[this->g_idx_], pd_beta && accum[this->b_idx_], this->size0_, this->size1_,
       this->size2_, this->eps_, batch_stat ? 1 : 0, HipDtype<T>::code, ws, workspace_bytes_,
       nullptr));
+  st.store();
 }
 
 template class BatchNormalizationHip<float>;

@@ -260,6 +260,19 @@ int nnabla_hip_variable_fill(nnabla_hip_variable *v, int which, float value) {
   return guarded([&] { pick(v, which)->fill(value); });
 }
 
+int nnabla_hip_variable_stored_dtype(nnabla_hip_variable *v, int which, int *dtype) {
+  return guarded([&] {
+    NBLA_CHECK(dtype, error_code::value, "dtype is null");
+    NdArrayPtr a = pick(v, which);
+    try {
+      const dtypes d = a->array()->dtype();
+      *dtype = d == dtypes::FLOAT ? 0 : d == dtypes::HALF ? 1 : 0x100 + static_cast<int>(d);
+    } catch (...) {
+      *dtype = -1;
+    }
+  });
+}
+
 nnabla_hip_function *nnabla_hip_create_batch_normalization(const char *backends,
                                                            const char *array_class,
                                                            const char *device_id, const int *axes,

@@ -3,6 +3,8 @@
 #include <nbla/hip/function/group_normalization.hpp>
 #include <nbla/variable.hpp>
 
+#include <type_traits>
+
 namespace nbla {
 
 template <typename T>
@@ -35,6 +37,10 @@ void GroupNormalizationHip<T>::setup_impl(const Variables &inputs, const Variabl
                     : nblahip_gn_bwd_workspace_bytes(batch_size_, channel_size_, spatial_size_,
                                                      this->num_groups_, HipDtype<T>::code);
   workspace_.reshape(Shape_t{static_cast<Size_t>((workspace_bytes_ + 3) / 4)}, true);
+  if (std::is_same<T, Half>::value) {
+    const Size_t np = channel_size_, ns = batch_size_ * this->num_groups_;
+    stage_.reshape(Shape_t{ParamStage::capacity_for({np, np, np, np, ns, ns, ns, ns})}, true);
+  }
 }
 
 template <typename T>
@@ -49,18 +55,24 @@ void GroupNormalizationHip<T>::forward_impl(const Variables &inputs, const Varia
   const int beta_idx = 1;
   const int gamma_idx = this->no_bias_ ? 1 : 2;
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
-  const float *beta =
-      this->no_bias_ ? nullptr : inputs[beta_idx]->template get_data_pointer<float>(this->ctx_);
-  const float *gamma =
-      this->no_scale_ ? nullptr : inputs[gamma_idx]->template get_data_pointer<float>(this->ctx_);
+  // (parameters and statistics a half graph stores in half are read and
+  // written where they lie: ParamStage; statistics kept inside the function
+  // stay float32)
+  ParamStage st;
+  st.begin(this->ctx_, std::is_same<T, Half>::value, &stage_);
+  const float *beta = this->no_bias_ ? nullptr : st.in(inputs[beta_idx]);
+  const float *gamma = this->no_scale_ ? nullptr : st.in(inputs[gamma_idx]);
   T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
-  float *mean = v_mean->cast_data_and_get_pointer<float>(this->ctx_, true);
-  float *var = v_var->cast_data_and_get_pointer<float>(this->ctx_, true);
+  const bool exposed = outputs.size() == 3;
+  float *mean = exposed ? st.out(v_mean, false) : v_mean->cast_data_and_get_pointer<float>(this->ctx_, true);
+  float *var = exposed ? st.out(v_var, false) : v_var->cast_data_and_get_pointer<float>(this->ctx_, true);
+  st.load();
   if (channel_last_) {
     float *ws = workspace_.cast_data_and_get_pointer<float>(this->ctx_, true);
     NBLA_HIP_CHECK(nblahip_gn_cl_fwd(x, gamma, beta, y, mean, var, batch_size_, spatial_size_,
                                      channel_size_, this->num_groups_, this->eps_,
                                      HipDtype<T>::code, ws, workspace_bytes_, nullptr));
+    st.store();
     workspace_.data()->array()->clear();
     return;
   }
@@ -93,6 +105,7 @@ void GroupNormalizationHip<T>::forward_impl(const Variables &inputs, const Varia
     adaptor_release(stat_a_);
     adaptor_release(stat_b_);
   }
+  st.store();
 }
 
 template <typename T>
@@ -113,22 +126,22 @@ void GroupNormalizationHip<T>::backward_impl(const Variables &inputs, const Vari
   if (outputs.size() == 3) {
     v_mean = outputs[1];
     v_var = outputs[2];
-    dmean = v_mean->get_grad_pointer<float>(this->ctx_);
-    dvar = v_var->get_grad_pointer<float>(this->ctx_);
   }
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
   const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
-  const float *gamma =
-      this->no_scale_ ? nullptr : inputs[gamma_idx]->template get_data_pointer<float>(this->ctx_);
-  const float *mean = v_mean->get_data_pointer<float>(this->ctx_);
-  const float *var = v_var->get_data_pointer<float>(this->ctx_);
+  ParamStage st;
+  st.begin(this->ctx_, std::is_same<T, Half>::value, &stage_);
+  const float *gamma = this->no_scale_ ? nullptr : st.in(inputs[gamma_idx]);
+  if (outputs.size() == 3) {
+    dmean = st.in(v_mean, true);
+    dvar = st.in(v_var, true);
+  }
+  const float *mean = st.in(v_mean);
+  const float *var = st.in(v_var);
   T *dx = !pd_x ? nullptr : inputs[0]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[0]);
-  float *dbeta = !pd_beta ? nullptr
-                          : inputs[beta_idx]->template cast_grad_and_get_pointer<float>(
-                                this->ctx_, !accum[beta_idx]);
-  float *dgamma = !pd_gamma ? nullptr
-                            : inputs[gamma_idx]->template cast_grad_and_get_pointer<float>(
-                                  this->ctx_, !accum[gamma_idx]);
+  float *dbeta = !pd_beta ? nullptr : st.out(inputs[beta_idx], accum[beta_idx], true);
+  float *dgamma = !pd_gamma ? nullptr : st.out(inputs[gamma_idx], accum[gamma_idx], true);
+  st.load();
   float *ws = workspace_.cast_data_and_get_pointer<float>(this->ctx_, true);
   if (channel_last_) {
     NBLA_HIP_CHECK(nblahip_gn_cl_bwd(x, dy, gamma, mean, var, dmean, dvar, dx, dgamma, dbeta,
@@ -136,6 +149,7 @@ void GroupNormalizationHip<T>::backward_impl(const Variables &inputs, const Vari
                                      pd_beta && accum[beta_idx], batch_size_, spatial_size_,
                                      channel_size_, this->num_groups_, this->eps_,
                                      HipDtype<T>::code, ws, workspace_bytes_, nullptr));
+    st.store();
     workspace_.data()->array()->clear();
     return;
   }
@@ -182,6 +196,7 @@ void GroupNormalizationHip<T>::backward_impl(const Variables &inputs, const Vari
   if (adapt_stats) {
     for (Variable *v : {&stat_a_, &stat_b_, &stat_c_, &stat_d_}) adaptor_release(*v);
   }
+  st.store();
   workspace_.data()->array()->clear();
 }
 

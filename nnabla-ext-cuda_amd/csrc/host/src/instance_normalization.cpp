@@ -4,6 +4,8 @@
 #include <nbla/hip/function/instance_normalization.hpp>
 #include <nbla/variable.hpp>
 
+#include <type_traits>
+
 namespace nbla {
 
 template <typename T>
@@ -34,6 +36,10 @@ void InstanceNormalizationHip<T>::setup_impl(const Variables &inputs, const Vari
                     : nblahip_in_bwd_workspace_bytes(batch_size_, channel_size_, spatial_size_,
                                                      HipDtype<T>::code);
   workspace_.reshape(Shape_t{static_cast<Size_t>((workspace_bytes_ + 3) / 4)}, true);
+  if (std::is_same<T, Half>::value) {
+    const Size_t np = batch_size_ * channel_size_, ns = batch_size_ * channel_size_;
+    stage_.reshape(Shape_t{ParamStage::capacity_for({np, np, np, np, ns, ns, ns, ns})}, true);
+  }
 }
 
 template <typename T>
@@ -46,19 +52,25 @@ void InstanceNormalizationHip<T>::forward_impl(const Variables &inputs, const Va
     v_var = outputs[2];
   }
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
-  const float *beta = this->no_bias_ ? nullptr
-                                     : inputs[this->beta_idx_]->template get_data_pointer<float>(this->ctx_);
-  const float *gamma = this->no_scale_ ? nullptr
-                                       : inputs[this->gamma_idx_]->template get_data_pointer<float>(this->ctx_);
+  // (parameters and statistics a half graph stores in half are read and
+  // written where they lie: ParamStage; statistics kept inside the function
+  // stay float32)
+  ParamStage st;
+  st.begin(this->ctx_, std::is_same<T, Half>::value, &stage_);
+  const float *beta = this->no_bias_ ? nullptr : st.in(inputs[this->beta_idx_]);
+  const float *gamma = this->no_scale_ ? nullptr : st.in(inputs[this->gamma_idx_]);
   T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
-  float *mean = v_mean->cast_data_and_get_pointer<float>(this->ctx_, true);
-  float *var = v_var->cast_data_and_get_pointer<float>(this->ctx_, true);
+  const bool exposed = outputs.size() == 3;
+  float *mean = exposed ? st.out(v_mean, false) : v_mean->cast_data_and_get_pointer<float>(this->ctx_, true);
+  float *var = exposed ? st.out(v_var, false) : v_var->cast_data_and_get_pointer<float>(this->ctx_, true);
+  st.load();
   const int bc_gamma = this->need_gamma_broadcast_ ? 1 : 0, bc_beta = this->need_beta_broadcast_ ? 1 : 0;
   if (channel_last_) {
     float *ws = workspace_.cast_data_and_get_pointer<float>(this->ctx_, true);
     NBLA_HIP_CHECK(nblahip_in_cl_fwd(x, gamma, beta, y, mean, var, batch_size_, spatial_size_,
                                      channel_size_, bc_gamma, bc_beta, this->eps_,
                                      HipDtype<T>::code, ws, workspace_bytes_, nullptr));
+    st.store();
     workspace_.data()->array()->clear();
     return;
   }
@@ -101,6 +113,7 @@ void InstanceNormalizationHip<T>::forward_impl(const Variables &inputs, const Va
     layout_.stats.to_caller(vk, var, false, NBLAHIP_F32);
     for (Variable *v : {&stat_a_, &stat_b_, &stat_c_, &stat_d_}) adaptor_release(*v);
   }
+  st.store();
 }
 
 template <typename T>
@@ -121,22 +134,22 @@ void InstanceNormalizationHip<T>::backward_impl(const Variables &inputs, const V
   if (outputs.size() == 3) {
     v_mean = outputs[1];
     v_var = outputs[2];
-    dmean = v_mean->get_grad_pointer<float>(this->ctx_);
-    dvar = v_var->get_grad_pointer<float>(this->ctx_);
   }
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
   const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
-  const float *gamma =
-      this->no_scale_ ? nullptr : inputs[gamma_idx]->template get_data_pointer<float>(this->ctx_);
-  const float *mean = v_mean->get_data_pointer<float>(this->ctx_);
-  const float *var = v_var->get_data_pointer<float>(this->ctx_);
+  ParamStage st;
+  st.begin(this->ctx_, std::is_same<T, Half>::value, &stage_);
+  const float *gamma = this->no_scale_ ? nullptr : st.in(inputs[gamma_idx]);
+  if (outputs.size() == 3) {
+    dmean = st.in(v_mean, true);
+    dvar = st.in(v_var, true);
+  }
+  const float *mean = st.in(v_mean);
+  const float *var = st.in(v_var);
   T *dx = !pd_x ? nullptr : inputs[0]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[0]);
-  float *dbeta = !pd_beta ? nullptr
-                          : inputs[beta_idx]->template cast_grad_and_get_pointer<float>(
-                                this->ctx_, !accum[beta_idx]);
-  float *dgamma = !pd_gamma ? nullptr
-                            : inputs[gamma_idx]->template cast_grad_and_get_pointer<float>(
-                                  this->ctx_, !accum[gamma_idx]);
+  float *dbeta = !pd_beta ? nullptr : st.out(inputs[beta_idx], accum[beta_idx], true);
+  float *dgamma = !pd_gamma ? nullptr : st.out(inputs[gamma_idx], accum[gamma_idx], true);
+  st.load();
   float *ws = workspace_.cast_data_and_get_pointer<float>(this->ctx_, true);
   const int bc_gamma = this->need_gamma_broadcast_ ? 1 : 0, bc_beta = this->need_beta_broadcast_ ? 1 : 0;
   if (channel_last_) {
@@ -145,6 +158,7 @@ void InstanceNormalizationHip<T>::backward_impl(const Variables &inputs, const V
                                      pd_beta && accum[beta_idx], batch_size_, spatial_size_,
                                      channel_size_, bc_gamma, bc_beta, this->eps_,
                                      HipDtype<T>::code, ws, workspace_bytes_, nullptr));
+    st.store();
     workspace_.data()->array()->clear();
     return;
   }
@@ -206,6 +220,7 @@ void InstanceNormalizationHip<T>::backward_impl(const Variables &inputs, const V
     for (Variable *v : {&stat_a_, &stat_b_, &stat_c_, &stat_d_, &stat_e_, &stat_f_, &stat_g_})
       adaptor_release(*v);
   }
+  st.store();
   workspace_.data()->array()->clear();
 }
 

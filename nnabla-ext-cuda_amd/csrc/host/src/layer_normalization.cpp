@@ -3,6 +3,8 @@
 #include <nbla/hip/function/layer_normalization.hpp>
 #include <nbla/variable.hpp>
 
+#include <type_traits>
+
 namespace nbla {
 
 template <typename T>
@@ -34,6 +36,12 @@ void LayerNormalizationHip<T>::setup_impl(const Variables &inputs, const Variabl
   hip_set_device(this->device_); // argument errors above are reported without a device
   workspace_bytes_ = nblahip_ln_bwd_workspace_bytes(batch_size_, reduce_size_, HipDtype<T>::code);
   workspace_.reshape(Shape_t{static_cast<Size_t>((workspace_bytes_ + 3) / 4)}, true);
+  if (std::is_same<T, Half>::value) {
+    stage_.reshape(Shape_t{ParamStage::capacity_for({reduce_size_, reduce_size_, reduce_size_,
+                                                     reduce_size_, batch_size_, batch_size_,
+                                                     batch_size_, batch_size_})},
+                   true);
+  }
 }
 
 template <typename T>
@@ -48,13 +56,16 @@ void LayerNormalizationHip<T>::forward_impl(const Variables &inputs, const Varia
   const int beta_idx = 1;
   const int gamma_idx = this->no_bias_ ? 1 : 2;
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
-  const float *beta =
-      this->no_bias_ ? nullptr : inputs[beta_idx]->template get_data_pointer<float>(this->ctx_);
-  const float *gamma =
-      this->no_scale_ ? nullptr : inputs[gamma_idx]->template get_data_pointer<float>(this->ctx_);
+  ParamStage st;
+  st.begin(this->ctx_, std::is_same<T, Half>::value, &stage_);
+  const float *beta = this->no_bias_ ? nullptr : st.in(inputs[beta_idx]);
+  const float *gamma = this->no_scale_ ? nullptr : st.in(inputs[gamma_idx]);
   T *y = outputs[0]->cast_data_and_get_pointer<T>(this->ctx_, true);
-  float *mean = v_mean->cast_data_and_get_pointer<float>(this->ctx_, true);
-  float *var = v_var->cast_data_and_get_pointer<float>(this->ctx_, true);
+  // (statistics kept inside the function stay float32; exposed ones follow the parameters)
+  const bool exposed = outputs.size() == 3;
+  float *mean = exposed ? st.out(v_mean, false) : v_mean->cast_data_and_get_pointer<float>(this->ctx_, true);
+  float *var = exposed ? st.out(v_var, false) : v_var->cast_data_and_get_pointer<float>(this->ctx_, true);
+  st.load();
   const T *xk = x;
   T *yk = y;
   if (adaptor_.needed()) {
@@ -66,6 +77,7 @@ void LayerNormalizationHip<T>::forward_impl(const Variables &inputs, const Varia
   }
   NBLA_HIP_CHECK(nblahip_ln_fwd(xk, gamma, beta, yk, mean, var, batch_size_, reduce_size_,
                                 this->eps_, HipDtype<T>::code, nullptr));
+  st.store();
   if (adaptor_.needed()) {
     adaptor_.to_caller(yk, y, false, HipDtype<T>::code);
     adaptor_release(adapt_a_);
@@ -87,26 +99,24 @@ void LayerNormalizationHip<T>::backward_impl(const Variables &inputs, const Vari
 
   Variable *v_mean = &mean_;
   Variable *v_var = &var_;
+  ParamStage st;
+  st.begin(this->ctx_, std::is_same<T, Half>::value, &stage_);
+  const float *gamma = this->no_scale_ ? nullptr : st.in(inputs[gamma_idx]);
   const float *dmean = nullptr, *dvar = nullptr;
   if (outputs.size() == 3) {
     v_mean = outputs[1];
     v_var = outputs[2];
-    dmean = v_mean->get_grad_pointer<float>(this->ctx_);
-    dvar = v_var->get_grad_pointer<float>(this->ctx_);
+    dmean = st.in(v_mean, true);
+    dvar = st.in(v_var, true);
   }
   const T *x = inputs[0]->get_data_pointer<T>(this->ctx_);
   const T *dy = outputs[0]->get_grad_pointer<T>(this->ctx_);
-  const float *gamma =
-      this->no_scale_ ? nullptr : inputs[gamma_idx]->template get_data_pointer<float>(this->ctx_);
-  const float *mean = v_mean->get_data_pointer<float>(this->ctx_);
-  const float *var = v_var->get_data_pointer<float>(this->ctx_);
+  const float *mean = st.in(v_mean);
+  const float *var = st.in(v_var);
   T *dx = !pd_x ? nullptr : inputs[0]->cast_grad_and_get_pointer<T>(this->ctx_, !accum[0]);
-  float *dbeta = !pd_beta ? nullptr
-                          : inputs[beta_idx]->template cast_grad_and_get_pointer<float>(
-                                this->ctx_, !accum[beta_idx]);
-  float *dgamma = !pd_gamma ? nullptr
-                            : inputs[gamma_idx]->template cast_grad_and_get_pointer<float>(
-                                  this->ctx_, !accum[gamma_idx]);
+  float *dbeta = !pd_beta ? nullptr : st.out(inputs[beta_idx], accum[beta_idx], true);
+  float *dgamma = !pd_gamma ? nullptr : st.out(inputs[gamma_idx], accum[gamma_idx], true);
+  st.load();
   float *ws = workspace_.cast_data_and_get_pointer<float>(this->ctx_, true);
   const bool adapt = adaptor_.needed();
   T *dxk = dx;
@@ -124,6 +134,7 @@ void LayerNormalizationHip<T>::backward_impl(const Variables &inputs, const Vari
                                 !adapt && pd_x && accum[0], pd_gamma && accum[gamma_idx],
                                 pd_beta && accum[beta_idx], batch_size_, reduce_size_, this->eps_,
                                 HipDtype<T>::code, ws, workspace_bytes_, nullptr));
+  st.store();
   if (adapt) {
     if (pd_x) adaptor_.to_caller(dxk, dx, accum[0], HipDtype<T>::code);
     adaptor_release(adapt_a_);

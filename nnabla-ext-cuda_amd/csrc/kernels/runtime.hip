@@ -1,5 +1,6 @@
 // Runtime shims of the C-ABI (device management, memory, dtype conversion)
 // and the small host utilities shared by the launch code.
+#include <algorithm>
 #include <atomic>
 #include <cstdlib>
 #include <cstring>
@@ -114,6 +115,23 @@ template <typename D>
 __global__ void __launch_bounds__(256) fill_kernel(D *__restrict__ dst, float v, int64_t n) {
   const D d = from_f32<D>(v);
   for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < n; i += gridDim.x * 256ll) dst[i] = d;
+}
+
+// Several small arrays converted in one launch (blockIdx.y: the array).
+constexpr int kStageMax = 16;
+struct StageArgs {
+  const void *src[kStageMax];
+  void *dst[kStageMax];
+  int64_t n[kStageMax];
+};
+template <typename D, typename S>
+__global__ void __launch_bounds__(256) stage_params_kernel(const StageArgs a) {
+  const int k = blockIdx.y;
+  const S *__restrict__ src = static_cast<const S *>(a.src[k]);
+  D *__restrict__ dst = static_cast<D *>(a.dst[k]);
+  const int64_t n = a.n[k];
+  for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < n; i += gridDim.x * 256ll)
+    dst[i] = from_f32<D>(to_f32<S>(src[i]));
 }
 
 static unsigned flat_grid(int64_t n) {
@@ -395,6 +413,37 @@ int nblahip_fill(void *dst, int dtype, float value, int64_t n, void *stream) {
     NBLAHIP_LAUNCH("fill_kernel", (fill_kernel<__half>), g, b, 0, st, static_cast<__half *>(dst), value, n);
   } else {
     return NBLAHIP_EINVAL;
+  }
+  return last_launch_status();
+}
+
+int nblahip_stage_params(int count, const void *const *src, int src_dtype, void *const *dst,
+                         int dst_dtype, const int64_t *n, void *stream) {
+  if (count == 0) return 0;
+  if (count < 0 || count > kStageMax || !src || !dst || !n) return NBLAHIP_EINVAL;
+  const bool up = src_dtype == NBLAHIP_F16 && dst_dtype == NBLAHIP_F32;
+  const bool down = src_dtype == NBLAHIP_F32 && dst_dtype == NBLAHIP_F16;
+  if (!up && !down) return NBLAHIP_EINVAL;
+  StageArgs a{};
+  int64_t longest = 0;
+  int used = 0;
+  for (int k = 0; k < count; ++k) {
+    if (n[k] < 0) return NBLAHIP_EINVAL;
+    if (n[k] == 0) continue;
+    if (!src[k] || !dst[k]) return NBLAHIP_EINVAL;
+    a.src[used] = src[k];
+    a.dst[used] = dst[k];
+    a.n[used] = n[k];
+    longest = std::max(longest, n[k]);
+    ++used;
+  }
+  if (used == 0) return 0;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 g(std::min(flat_grid(longest), 1024u), used), b(256);
+  if (up) {
+    NBLAHIP_LAUNCH("stage_params_kernel", (stage_params_kernel<float, __half>), g, b, 0, st, a);
+  } else {
+    NBLAHIP_LAUNCH("stage_params_kernel", (stage_params_kernel<__half, float>), g, b, 0, st, a);
   }
   return last_launch_status();
 }
