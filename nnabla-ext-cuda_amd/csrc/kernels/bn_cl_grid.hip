@@ -34,19 +34,6 @@
 
 namespace nblahip {
 
-#ifdef NBLAHIP_GRID_DBG
-// Phase clocks of a debug build (never compiled into the library that ships).
-__device__ unsigned long long grid_dbg_clk[256 * 16];
-#define GRID_CLK(i)                                                                    \
-  do {                                                                                 \
-    if (threadIdx.x == 0) grid_dbg_clk[blockIdx.x * 16 + (i)] = wall_clock64();        \
-  } while (0)
-#else
-#define GRID_CLK(i) \
-  do {              \
-  } while (0)
-#endif
-
 namespace {
 
 constexpr int kGridMaxBlocks = 256; // partials per channel a block merges (one per thread of a wave quad)
@@ -102,24 +89,20 @@ __device__ __forceinline__ void grid_channel_sums(float (&v)[VEC], uint32_t cv, 
                                                   float *fold, float *tot, uint32_t C) {
   constexpr int NW = kOnchipBlock / kWave;
   lanes_sum_from<VEC>(v, cv); // (a step at a time for all values, off the LDS crossbar: xor_add)
-  GRID_CLK(10);
   if ((threadIdx.x & (kWave - 1)) < cv) {
 #pragma unroll
     for (int j = 0; j < VEC; ++j) fold[(threadIdx.x / kWave) * C + cvx * VEC + j] = v[j];
   }
   lds_barrier();
-  GRID_CLK(11);
   if (threadIdx.x < C) {
     float t = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) t += fold[w * C + threadIdx.x];
     tot[threadIdx.x] = t;
   }
-  GRID_CLK(12);
   lds_barrier();
 #pragma unroll
   for (int j = 0; j < VEC; ++j) v[j] = tot[cvx * VEC + j];
-  GRID_CLK(13);
 }
 
 // The same fold for ONE channel (element e of the vectors of channel vector
@@ -206,7 +189,6 @@ __device__ __forceinline__ void grid_channel_result(const BnClGridArgs &a, uint3
     if (!ok) miss[kGridMaxBlocks] = 1;
   }
   lds_barrier();
-  GRID_CLK(9);
   for (uint32_t p = 0; miss[kGridMaxBlocks] && p < a.nblocks; ++p) {
     if (!miss[p]) continue; // same answer in every thread
     float m, q;
@@ -315,7 +297,6 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
   __shared__ float gb[2 * CMAX]; // gamma, beta
   const uint32_t b = blockIdx.x;
   const uint32_t t = threadIdx.x;
-  GRID_CLK(0);
   // gamma and beta of channel t, asked for ahead of the tensor (behind the
   // exchange they would cost a memory round trip of their own)
   float gamma_t = 1.f, beta_t = 0.f;
@@ -400,9 +381,7 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
         }
       }
     }
-    GRID_CLK(1);
     grid_channel_sums<VEC>(m, a.cv, cvx, fold, tot, a.C);
-    GRID_CLK(2);
     const float icnt = 1.0f / static_cast<float>(vbb / a.cv);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
@@ -411,7 +390,6 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
       q[j] = fmaf(e, fmaf(nt, e, 2.f * s1[j]), s2[j]);
     }
     grid_channel_sums<VEC>(q, a.cv, cvx, fold, tot, a.C);
-    GRID_CLK(3);
   }
   // publish (mean, m2) of every channel: a word per thread (through fin, which
   // is free until the results arrive)
@@ -425,13 +403,11 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
   lds_barrier();
   for (uint32_t e = t; e < 2 * a.C; e += kOnchipBlock)
     xchg_publish(a.x1 + static_cast<size_t>(b) * a.C * 2 + e, fin[e], a.epoch);
-  GRID_CLK(4);
 
   // ---- stage 2: block c merges channel c, writes its statistics, publishes
   for (uint32_t c = b; c < a.C; c += a.nblocks) {
     float mean, var;
     grid_channel_result<T, VEC>(a, c, miss, got, wel, fold, mean, var);
-    GRID_CLK(5);
     if (t == 0) {
       a.mean[c] = mean;
       a.var[c] = var;
@@ -445,7 +421,6 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
     }
   }
 
-  GRID_CLK(6);
   // ---- every block: the C results (merged here where one does not arrive)
   lds_barrier();
   if (t == 0) miss[kGridMaxBlocks + 1] = 0;
@@ -470,7 +445,6 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
     lds_barrier();
   }
 
-  GRID_CLK(7);
   // ---- normalize what the block holds
 #pragma unroll
   for (int k = 0; k < NR; ++k) forget<T, VEC>(raw[k]);
@@ -500,7 +474,6 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
       store_vec<T, VEC>(y + static_cast<size_t>(v) * VEC, o);
     }
   }
-  GRID_CLK(8);
 }
 
 // Backward (batch statistics).  With xh = (x-mean)*istd per channel:
@@ -827,11 +800,15 @@ bool grid_args(const BnProblem &p, BnClGridArgs &a, int &nl) {
   const int64_t vb = rows_pb * cv;
   nl = static_cast<int>((vb + kOnchipBlock - 1) / kOnchipBlock);
   const int64_t nblocks = (M + rows_pb - 1) / rows_pb;
-  // Up to what the chip holds, and from 6 vectors per thread: the exchange and
-  // the folds cost about 9 us whatever the size, one read of x saves 0.16 us
-  // per MB ([256,56,56,64] half 57.8 -> 49.4 us, [128,56,56,64] 35.0 -> 30.9 us,
-  // [64,56,56,64] 24.1 -> 22.0 us, [32,56,56,64] 18.4 -> 19.5 us).
-  if (nl < tune_int("BN_CL_GRID_MIN_SLOTS", 6) || nl > 25 || nblocks < blocks / 2) return false;
+  // Up to what the chip holds, and from 8192 rows: below, the split kernels
+  // (a block per 1024 rows) are as fast or faster.  Kernel time of forward +
+  // backward, this against the split kernels / the split reduction, half
+  // [M, 64]: 22.8 vs 21.9 us at M = 6272, 23.1 vs 29.1 at 12544, 24.8 vs 32.9 at
+  // 50176, 29.5 vs 45.5 at 100352, 33.6 vs 55.0 at 150528; float 19.5 vs 18.6,
+  // 20.0 vs 22.2, 24.2 vs 31.5; [M, 128] half 24.1 vs 22.5 at 6272, 25.1 vs 29.4
+  // at 12544.
+  if (nl < tune_int("BN_CL_GRID_MIN_SLOTS", 1) || nl > 25 || nblocks < blocks / 2) return false;
+  if (M < tune_int("BN_CL_GRID_MIN_ROWS", 8192)) return false;
   a = BnClGridArgs{};
   a.x = p.x;
   a.gamma = p.gamma;
@@ -899,10 +876,3 @@ bool bn_cl_grid_bwd(const BnProblem &p, hipStream_t st, int *status) {
 }
 
 } // namespace nblahip
-
-#ifdef NBLAHIP_GRID_DBG
-extern "C" __attribute__((visibility("default"))) int nblahip_debug_grid_clocks(unsigned long long *host) {
-  return static_cast<int>(hipMemcpyFromSymbol(host, HIP_SYMBOL(nblahip::grid_dbg_clk),
-                                              sizeof(unsigned long long) * 256 * 16));
-}
-#endif

@@ -572,16 +572,19 @@ bool onchip_args(const BnProblem &p, bool backward, BnOnchipArgs &a, int &nl, in
   if (vec == 4 && p.dtype == NBLAHIP_F16 && nl > 16) return false;
   // A block is alone on its CU, so fewer channels than CUs leave CUs idle -
   // but a CU alone pulls far more than its 1/256 share of the bandwidth, and
-  // the split reduction pays a finalize launch: the forward wins down to an
-  // eighth of the CUs ([32,32,56,56] float 15.3 -> 10.4 us), the backward down
-  // to a quarter ([32,64,56,56] 25.6 -> 22.8 us; with 32 channels 16 -> 19 us).
-  // With a streamed remainder (channels beyond what the layouts hold) only
-  // with a channel for nearly every CU: [32,64,112,112] half (50176 vectors)
-  // 33.6 / 43.1 vs 35.7 / 52.0 us.
+  // the split reduction pays two launches more per direction: with whole
+  // channels held, both directions win at every channel count (kernel time of
+  // forward + backward, [16,C,56,56] float: 18.1 vs 26.7 us at C = 8, 19.4 vs
+  // 21.1 at 32, 24.2 vs 25.9 at 60; [32,C,56,56] half: 22.5 vs 26.7 at C = 4,
+  // 23.4 vs 28.3 at 28).  With a streamed remainder (channels beyond what the
+  // layouts hold) from channels for half the CUs: [32,C,56,56] float forward +
+  // backward 39.3 vs 31.8 us at C = 32, 44.4 vs 41.3 at 64, 55.1 vs 63.5 at
+  // 128, 88.4 vs 99.3 at 224; [32,C,112,112] half 97.0 vs 78.1 at 64, 119.5 vs
+  // 140.1 at 128.
   const bool whole = nv <= (backward ? 20480 : 25600);
-  const int min_pct = !whole     ? tune_int("BN_ONCHIP_STREAMED_MIN_PCT", 88)
-                      : backward ? tune_int("BN_ONCHIP_BWD_MIN_PCT", 25)
-                                 : tune_int("BN_ONCHIP_FWD_MIN_PCT", 12);
+  const int min_pct = !whole     ? tune_int("BN_ONCHIP_STREAMED_MIN_PCT", 50)
+                      : backward ? tune_int("BN_ONCHIP_BWD_MIN_PCT", 1)
+                                 : tune_int("BN_ONCHIP_FWD_MIN_PCT", 1);
   if (p.C * 100 < static_cast<int64_t>(device_cus()) * min_pct) return false;
   a = BnOnchipArgs{};
   a.x = p.x;
@@ -644,9 +647,12 @@ bool in_onchip_bwd(const RowProblem &p, hipStream_t st, int *status) {
     return false;
   const int64_t nv = p.R / vec;
   if (nv <= 8192 || nv > 65536) return false;
-  // (longer planes keep 18432 vectors and stream the rest, which pays with a
-  // plane for nearly every CU, as for BatchNormalization)
-  const int min_pct = nv <= 20480 ? tune_int("ROW_ONCHIP_BWD_MIN_PCT", 25)
+  // (whole planes: from any number of them - [1,C,256,256] float forward +
+  // backward 30.8 vs 36.6 us of kernel time at C = 32, 35.0 vs 42.6 at 56;
+  // longer planes keep 18432 vectors and stream the rest, which pays only with
+  // a plane for nearly every CU: [1,C,512,512] float 123 vs 67 us at C = 32,
+  // 135 vs 99 at 56)
+  const int min_pct = nv <= 20480 ? tune_int("ROW_ONCHIP_BWD_MIN_PCT", 1)
                                   : tune_int("ROW_ONCHIP_STREAMED_MIN_PCT", 88);
   if (p.rows * 100 < static_cast<int64_t>(device_cus()) * min_pct) return false;
   BnOnchipArgs a{};

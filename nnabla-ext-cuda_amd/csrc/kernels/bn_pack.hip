@@ -506,14 +506,15 @@ bool pack_args(const BnProblem &p, bool backward, BnPackArgs &a, int &nl) {
   // ([256,1024,14,14] half backward 87.8 -> 69.1 us; forward 55.4 / 55.0;
   // [64,1024,14,14] 16.7 / 19.2 -> 19.4 / 20.9 us).
   if (G == 2 && !(backward && p.size0 * (p.size2 / 4) > 8 * kOnchipBlock)) return false;
-  // A block is alone on its CU: with packs for fewer than an eighth of the CUs
-  // the chip is left idle ([256,512,7,7] half, 64 packs: 19.8 / 22.5 -> 16.2 /
-  // 17.3 us).  Channels of up to 4096 elements, which the row kernels take
-  // element by element in one launch, want a pack for half the CUs
-  // ([64,512,7,7] half, 64 packs: 7.7 / 7.7 -> 8.5 / 9.2 us; [64,2048,7,7]:
-  // 17.6 / 20.8 -> 10.8 / 11.5 us).
+  // A block is alone on its CU, and still a few packs beat the three launches
+  // of the masked split reduction ([96,240,7,7] half, 30 packs: 18.4 vs 27.0 us
+  // of kernel time forward + backward).  Channels of up to 4096 elements, which
+  // the row kernels take element by element in one launch, want a pack for
+  // every CU ([64,512,7,7] half, 64 packs: 7.7 / 7.7 -> 8.5 / 9.2 us;
+  // [32,256,7,7]: rows 8.2 us, packs 12.7; [32,1024,7,7], 128 packs: rows 10.8,
+  // packs 13.5; [64,2048,7,7], 256 packs: 17.6 / 20.8 -> 10.8 / 11.5 us).
   const bool short_channels = p.size0 * p.size2 <= 4096;
-  const int min_pct = short_channels ? tune_int("BN_PACK_SHORT_MIN_PCT", 50) : tune_int("BN_PACK_MIN_PCT", 12);
+  const int min_pct = short_channels ? tune_int("BN_PACK_SHORT_MIN_PCT", 100) : tune_int("BN_PACK_MIN_PCT", 1);
   if ((p.C / G) * 100 < static_cast<int64_t>(device_cus()) * min_pct) return false;
   a = BnPackArgs{};
   a.x = p.x;

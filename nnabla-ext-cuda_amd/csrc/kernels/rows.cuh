@@ -179,12 +179,7 @@ template <int TPR, int MODE> struct RowBwdBlock {
 template <typename T, int VEC, int NL, int TPR, int MODE> struct RowBwdOccupancy {
   static constexpr bool kGn512 =
       (MODE == kRowGN || MODE == kRowGNm) && TPR == 512 && NL == 8 && sizeof(T) == 2;
-#ifdef NBLAHIP_EXP_LN_CAP_F32
-  static constexpr bool kLnF32 = MODE == kRowLN && TPR == 64 && NL == 4 && sizeof(T) == 4;
-  static constexpr int kMinWaves = (kGn512 || kLnF32) ? 4 : 1;
-#else
   static constexpr int kMinWaves = kGn512 ? 4 : 1;
-#endif
 };
 
 // ---------------------------------------------------------------------------
@@ -358,11 +353,7 @@ row_bwd_kernel(const RowArgs a) {
   constexpr int NW = TPR / kWave;
   // LayerNormalization keeps xh and dg of a row in registers between the
   // reduction and the dx step when they are few; otherwise they are recomputed.
-#ifdef NBLAHIP_EXP_LN_NOKEEP_F32
-  constexpr bool KEEP = (MODE == kRowLN) && (NL * VEC <= 16) && sizeof(T) == 2;
-#else
   constexpr bool KEEP = (MODE == kRowLN) && (NL * VEC <= 16);
-#endif
   constexpr bool GN = MODE == kRowGN || MODE == kRowGNm;
   constexpr bool BN = MODE == kRowBN; // strided rows, dgamma/dbeta written here
   constexpr bool GNM = MODE == kRowGNm; // run-time thread map (GnSlot)

@@ -1223,7 +1223,7 @@ bool bn_masked_args(const BnProblem &p, bool backward, BnMaskedArgs &a, int &nl,
   nl = static_cast<int>((pieces + tb - 1) / tb);
   if (nl > most) return false;
   // (fewer channels than this share of the CUs: most of the chip would idle)
-  if (p.C * 100 < static_cast<int64_t>(device_cus()) * tune_int("BN_MASKED_ONCHIP_MIN_PCT", 12)) return false;
+  if (p.C * 100 < static_cast<int64_t>(device_cus()) * tune_int("BN_MASKED_ONCHIP_MIN_PCT", 1)) return false;
   a = BnMaskedArgs{};
   a.x = p.x;
   a.dy = p.dy;

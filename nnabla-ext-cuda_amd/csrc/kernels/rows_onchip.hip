@@ -202,8 +202,14 @@ bool row_onchip_fwd(const RowProblem &p, const RowArgs &a, int vec, hipStream_t 
   if (vec != (p.dtype == NBLAHIP_F16 ? 8 : 4)) return false;
   const int64_t nv = p.R / vec;
   if (nv < tune_int("ROW_ONCHIP_FWD_MIN_VECTORS", 4097) || nv > 65536) return false;
-  const int min_pct = nv <= 25 * kOnchipBlock ? tune_int("ROW_ONCHIP_MIN_PCT", 12)
-                                              : tune_int("ROW_ONCHIP_STREAMED_MIN_PCT", 88);
+  // Rows that one block's registers hold as well (up to 8192 vectors) want
+  // rows for an eighth of the CUs (fewer: [1,C,256,256] half 21.8 vs 20.5 us at
+  // C = 24); longer ones, which otherwise stream, win from the first row
+  // ([1,C,512,256] half forward + backward 34.8 vs 42.7 us at C = 4, 33.9 vs
+  // 43.1 at 24; [1,C,256,256] float 28.6 vs 37.7 at 4, 27.8 vs 38.0 at 24).
+  const int min_pct = nv <= 25 * kOnchipBlock
+                          ? tune_int("ROW_ONCHIP_MIN_PCT", nv <= 8 * kOnchipBlock ? 12 : 1)
+                          : tune_int("ROW_ONCHIP_STREAMED_MIN_PCT", 88);
   if (p.rows * 100 < static_cast<int64_t>(device_cus()) * min_pct) return false;
   const int nl = static_cast<int>((nv + kOnchipBlock - 1) / kOnchipBlock);
   const int grid = static_cast<int>(p.rows);

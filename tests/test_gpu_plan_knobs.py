@@ -177,8 +177,10 @@ SWITCHES = [
     ("bn_cl_grid_off", run_bn, ((100352, 64), 1, F16), {"BN_CL_GRID": 0},
      ["bn_stats_cl_kernel", "bn_finalize_fwd_kernel", "bn_apply_cl_kernel"], ["bn_cl_grid_fwd_kernel"],
      {"BN_CL_GRID_MIN_SLOTS": 1}),
-    ("bn_cl_grid_from_fewer_vectors", run_bn, ((100352, 64), 1, F16), {"BN_CL_GRID_MIN_SLOTS": 1},
-     ["bn_cl_grid_fwd_kernel"], ["bn_stats_cl_kernel"]),
+    ("bn_cl_grid_from_more_vectors", run_bn, ((100352, 64), 1, F16), {"BN_CL_GRID_MIN_SLOTS": 9},
+     ["bn_stats_cl_kernel"], ["bn_cl_grid_fwd_kernel"]),
+    ("bn_cl_grid_from_fewer_rows", run_bn, ((6272, 64), 1, F16), {"BN_CL_GRID_MIN_ROWS": 1},
+     ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"], ["cl_split_fwd_kernel"]),
     ("bn_masked_onchip_off", run_bn, ((64, 160, 17, 17), 1, F16), {"BN_MASKED_ONCHIP": 0},
      ["bn_apply_planes_kernel"], ["bn_masked_fwd_kernel", "bn_masked_bwd_kernel"]),
     ("bn_masked_onchip_min_pct_up", run_bn, ((64, 160, 17, 17), 1, F32), {"BN_MASKED_ONCHIP_MIN_PCT": 80},
@@ -311,13 +313,13 @@ GRIDS = [
      ["bn_stats_planes_kernel", "bn_apply_planes_kernel"], []),
     ("bn_cl_grids", run_bn, ((64, 28, 28, 64), 3, F16),
      [{"BN_CL_BLOCKS_PER_CU": a, "BN_CL_FWD_APPLY_BLOCKS_PER_CU": b, "BN_CL_APPLY_BLOCKS_PER_CU": c,
-       "BN_CL_SPLIT": 0} for a, b, c in ((1, 1, 1), (2, 4, 2), (8, 3, 7))],
+       "BN_CL_SPLIT": 0, "BN_CL_GRID": 0} for a, b, c in ((1, 1, 1), (2, 4, 2), (8, 3, 7))],
      ["bn_stats_cl_kernel", "bn_apply_cl_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
      []),
     ("bn_cl_grid_wide_fewer_rows", run_bn, ((128, 14, 14, 512), 3, F16), [{"BN_CL_GRID_WIDE_MIN_ROWS": 1}],
      ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"], []),
     ("bn_onchip_few_channels", run_bn, ((32, 4, 56, 56), 1, F16),
-     [{"BN_ONCHIP_FWD_MIN_PCT": 1, "BN_ONCHIP_BWD_MIN_PCT": 1}],
+     [{"BN_ONCHIP_FWD_MIN_PCT": 1, "BN_ONCHIP_BWD_MIN_PCT": 1, **NO_CHAN_SPLIT}],
      ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
     # planes that share cache lines with their neighbours: ordinary stores there, or not
     ("bn_onchip_edge_stores_off", run_bn, ((256, 64, 14, 14), 1, F32),
@@ -327,7 +329,7 @@ GRIDS = [
     ("bn_onchip_edge_stores_longer_planes", run_bn, ((128, 64, 28, 28), 1, F16),
      [{"BN_EDGE_STORES_MAX_BYTES": 4096}], ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
     ("bn_onchip_streamed_few_channels", run_bn, ((64, 8, 56, 56), 1, F32),
-     [{"BN_ONCHIP_STREAMED_MIN_PCT": 1}], ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
+     [{"BN_ONCHIP_STREAMED_MIN_PCT": 1, **NO_CHAN_SPLIT}], ["bn_onchip_fwd_kernel", "bn_onchip_bwd_kernel"], []),
     # a channel split over 8 blocks on a quarter of the CUs; every partner's part
     # recomputed because no poll is allowed
     ("bn_chan_split_few_blocks", run_bn, ((40, 8, 32, 32), 1, F32), [{"BN_CHAN_SPLIT_MIN_PCT": 1}],

@@ -89,21 +89,27 @@ def test_split_batch_equals_whole_batch(splits, rest, axis, dtype):
 
 
 def test_one_worker_is_bitwise_the_plain_path():
-    """(On a shape whose plain path is the same split reduction: channels that
-    do not fit one block's registers, and too few of them for the kernels that
-    hold a channel on one CU or split it over several; those and the
-    single-pass row kernels sum in another order.)"""
+    """(With the plain path on the same split reduction: the kernels that hold
+    a channel on one CU or split it over several blocks, which take this shape
+    by default, and the single-pass row kernels sum in another order and are
+    switched off for the comparison.)"""
     torch.manual_seed(3)
     x = torch.randn(64, 8, 48, 48, device="cuda")
     dy = torch.randn_like(x)
     g = torch.rand(8, device="cuda") + 0.5
     b = torch.randn(8, device="cuda")
-    y0, m0, v0 = K.bn_forward_batch(x, b, g, None, None, 1, 0.9, 1e-5)
-    dx0, dg0, db0 = K.bn_backward(x, dy, g, m0, v0, 1, 1e-5)
-    m, v = K.bn_local_stats(x, 1)
+    K.tune_reset()
+    K.tune_set("BN_CHAN_SPLIT", 0)
+    K.tune_set("BN_ONCHIP", 0)
+    try:
+        y0, m0, v0 = K.bn_forward_batch(x, b, g, None, None, 1, 0.9, 1e-5)
+        dx0, dg0, db0 = K.bn_backward(x, dy, g, m0, v0, 1, 1e-5)
+        m, v = K.bn_local_stats(x, 1)
+        sums, dg, db = K.bn_backward_local_sums(x, dy, m, v, 1, 1e-5)
+        dx = K.bn_backward_apply_sums(x, dy, g, m, v, sums, 64 * 48 * 48, 1, 1e-5)
+    finally:
+        K.tune_reset()
     assert torch.equal(m, m0) and torch.equal(v, v0)
-    sums, dg, db = K.bn_backward_local_sums(x, dy, m, v, 1, 1e-5)
-    dx = K.bn_backward_apply_sums(x, dy, g, m, v, sums, 64 * 48 * 48, 1, 1e-5)
     assert torch.equal(dg, dg0) and torch.equal(db, db0)
     assert torch.equal(dx, dx0)
 

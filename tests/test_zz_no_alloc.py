@@ -15,12 +15,15 @@ K = load_package()
 # (shape, axis, dtype name): tensors that take the split reduction, i.e. use
 # the scratch array (channel-last with many rows - 96 channels, which the
 # kernel that holds the tensor on the chip does not take; planes with few
-# channels), and a pair that does not need it (held on the chip, the partials
-# travel through the exchange array): the entry point must agree there too.
+# channels, with the plans that hold a channel on one CU or split it over
+# several blocks switched off), and a pair that does not need it (held on the
+# chip, the partials travel through the exchange array): the entry point must
+# agree there too.
 CASES = [
-    ([((64, 56, 56, 96), 3, "f16"), ((8, 28, 28, 32), 3, "f16")], True),
-    ([((32, 8, 56, 56), 1, "f32"), ((32, 8, 40, 40), 1, "f32")], True),
-    ([((64, 56, 56, 64), 3, "f16"), ((56, 56, 56, 64), 3, "f16")], False),
+    ([((64, 56, 56, 96), 3, "f16"), ((8, 28, 28, 32), 3, "f16")], True, {}),
+    ([((32, 8, 56, 56), 1, "f32"), ((32, 8, 40, 40), 1, "f32")], True,
+     {"BN_CHAN_SPLIT": 0, "BN_ONCHIP": 0}),
+    ([((64, 56, 56, 64), 3, "f16"), ((56, 56, 56, 64), 3, "f16")], False, {}),
 ]
 
 
@@ -51,9 +54,19 @@ def test_shapes_beyond_the_static_array_are_rejected():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("pair,partials", CASES,
+@pytest.mark.parametrize("pair,partials,knobs", CASES,
                          ids=["channel_last_f16", "planes_f32", "channel_last_on_chip_f16"])
-def test_static_scratch_matches_the_workspace_entry_point(pair, partials):
+def test_static_scratch_matches_the_workspace_entry_point(pair, partials, knobs):
+    K.tune_reset()
+    for name, value in knobs.items():
+        K.tune_set(name, value)
+    try:
+        _static_against_workspace(pair, partials)
+    finally:
+        K.tune_reset()
+
+
+def _static_against_workspace(pair, partials):
     import torch
     from oracle import norm_ref as R
     L = K.lib()
