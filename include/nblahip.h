@@ -46,7 +46,8 @@ enum nblahip_status {
   NBLAHIP_OK = 0,
   NBLAHIP_EINVAL = -1,    /* NULL required pointer, non-positive size, bad enum */
   NBLAHIP_EWORKSPACE = -2,/* workspace NULL, misaligned or too small */
-  NBLAHIP_ERANGE = -3,    /* tensor has 2^31 or more elements */
+  NBLAHIP_ERANGE = -3,    /* 2^31 or more elements in a BatchNormalization tensor or in
+                             one row / sample / group of the other functions */
   NBLAHIP_EALIAS = -4     /* output overlaps an input it must not overlap */
 };
 
@@ -343,7 +344,9 @@ NBLAHIP_EXPORT int nblahip_in_bwd(const void *x, const void *dy,
  * instance_normalization.cu:40-51, :81-94, :187-207); these entry points read
  * and write the channel-last tensor in place of those transposes.  Results
  * equal the channel-first entry points applied to the transposed tensor.
- * Both directions need a workspace of *_cl_workspace_bytes; batch <= 65535.
+ * Both directions need a workspace of *_cl_workspace_bytes.  Batches beyond
+ * 65535 and tensors of 2^31 elements and more run as several launches over
+ * ranges of samples (one sample must stay below 2^31 elements).
  * Aliasing as for BatchNormalization: y == x, dx == x and dx == dy are in-place
  * calls and run on the kernels without an exchange between blocks; a partial
  * overlap is rejected with NBLAHIP_EALIAS.
