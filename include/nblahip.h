@@ -463,6 +463,14 @@ NBLAHIP_EXPORT int nblahip_convert(void *dst, int dst_dtype, const void *src,
 /* dst[i] = value for n elements of dtype. */
 NBLAHIP_EXPORT int nblahip_fill(void *dst, int dtype, float value, int64_t n,
                                 void *stream);
+/* dst[i] = the low elem_bytes (1, 2, 4 or 8) bytes of pattern, for n elements:
+ * the value fill of the array layer for the dtypes the functions here do not
+ * compute in (CudaArray::fill covers every dtype through cuda_fill<T>,
+ * include/nbla/cuda/array/cuda_array.cuh:44-55,99; the caller converts the
+ * value to the element type). */
+NBLAHIP_EXPORT int nblahip_fill_bytes(void *dst, int elem_bytes,
+                                      unsigned long long pattern, int64_t n,
+                                      void *stream);
 
 /* Up to 16 small arrays converted between float16 and float32 in one launch:
  * dst[k][i] = (dst_dtype) src[k][i] for i < n[k] (arrays with n[k] == 0 are

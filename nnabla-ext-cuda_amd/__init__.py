@@ -96,6 +96,7 @@ SIGNATURES = {
     "nblahip_memset": (_int, [_c_void_p, _int, _sz, _c_void_p]),
     "nblahip_convert": (_int, [_c_void_p, _int, _c_void_p, _int, _i64, _c_void_p]),
     "nblahip_fill": (_int, [_c_void_p, _int, _f, _i64, _c_void_p]),
+    "nblahip_fill_bytes": (_int, [_c_void_p, _int, ctypes.c_ulonglong, _i64, _c_void_p]),
     "nblahip_permute": (_int, [_c_void_p, _c_void_p, _int, ctypes.POINTER(_i64),
                                ctypes.POINTER(_int), _int, _int, _c_void_p]),
     "nblahip_profile_enable": (_int, [_int]),

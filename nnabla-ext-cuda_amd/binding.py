@@ -255,6 +255,9 @@ class Variable:
     def fill_grad(self, v):
         _check(lib().nnabla_hip_variable_fill(self._h, 1, float(v)))
 
+    def fill_data(self, v):
+        _check(lib().nnabla_hip_variable_fill(self._h, 0, float(v)))
+
 
 def _handles(vs):
     arr = (ctypes.c_void_p * max(len(vs), 1))(*[v._h for v in vs])

@@ -2,6 +2,8 @@
 #include <nbla/hip/array/hip_array.hpp>
 #include <nbla/hip/hip.hpp>
 
+#include <cstring>
+
 namespace nbla {
 
 HipArray::HipArray(Size_t size, dtypes dtype, const Context &ctx, bool cached)
@@ -27,9 +29,9 @@ namespace {
 bool is_float_dtype(dtypes d) { return d == dtypes::FLOAT || d == dtypes::HALF; }
 } // namespace
 
-// Any dtype is stored and moved (the reference's CudaArray holds every dtype,
-// src/nbla/cuda/array/cuda_array.cpp:211-279); value fills and conversions
-// exist for the two float types the normalization functions compute in.
+// Any dtype is stored, moved and filled (the reference's CudaArray holds every
+// dtype, src/nbla/cuda/array/cuda_array.cpp:211-279); conversions exist for
+// the two float types the normalization functions compute in.
 void HipArray::zero() {
   hip_set_device(device_);
   if (is_float_dtype(dtype_)) {
@@ -39,10 +41,40 @@ void HipArray::zero() {
   }
 }
 
+namespace {
+// `value` converted to the element type as a C++ cast does, as raw bytes.
+template <typename D> unsigned long long element_bits(float value) {
+  const D d = static_cast<D>(value);
+  unsigned long long bits = 0;
+  std::memcpy(&bits, &d, sizeof(D));
+  return bits;
+}
+unsigned long long fill_pattern(dtypes dtype, float value) {
+  switch (dtype) {
+  case dtypes::BOOL: return value != 0.f ? 1u : 0u;
+  case dtypes::BYTE: return element_bits<int8_t>(value);
+  case dtypes::UBYTE: return element_bits<uint8_t>(value);
+  case dtypes::SHORT: return element_bits<int16_t>(value);
+  case dtypes::USHORT: return element_bits<uint16_t>(value);
+  case dtypes::INT: return element_bits<int32_t>(value);
+  case dtypes::UINT: return element_bits<uint32_t>(value);
+  case dtypes::LONG: return element_bits<int64_t>(value);
+  case dtypes::ULONG: return element_bits<uint64_t>(value);
+  case dtypes::DOUBLE: return element_bits<double>(value);
+  default: NBLA_ERROR(error_code::type, "HipArray::fill: unknown dtype");
+  }
+}
+} // namespace
+
 void HipArray::fill(float value) {
   if (value == 0.f) return zero();
   hip_set_device(device_);
-  NBLA_HIP_CHECK(nblahip_fill(ptr_, hip_dtype_code(dtype_), value, size_, nullptr));
+  if (is_float_dtype(dtype_)) {
+    NBLA_HIP_CHECK(nblahip_fill(ptr_, hip_dtype_code(dtype_), value, size_, nullptr));
+  } else {
+    NBLA_HIP_CHECK(nblahip_fill_bytes(ptr_, static_cast<int>(sizeof_dtype(dtype_)),
+                                      fill_pattern(dtype_, value), size_, nullptr));
+  }
 }
 
 void HipArray::copy_from(const Array *src) {

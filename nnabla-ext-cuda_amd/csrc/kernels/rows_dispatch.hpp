@@ -19,6 +19,13 @@ bool row_masked_fwd(const RowProblem &p, hipStream_t st, int *status);
 bool row_masked_bwd(const RowProblem &p, hipStream_t st, int *status); // the pairs to p.ws
 int run_row_bwd_cached_ln(int dtype, const RowCfg &cfg, const RowArgs &args, int grid,
                           hipStream_t st);
+// LayerNormalization backward over rows that are no whole number of 16-byte
+// vectors or start off a 16-byte boundary, with 16-byte accesses at element
+// alignment (rows_ln_loose.hip).  wanted: the problem is one of these (vec: the
+// width the aligned layouts would use); cfg: a wave-per-row layout of full
+// vectors for the row length rounded up to whole vectors.
+bool ln_loose_bwd_wanted(const RowProblem &p, int vec);
+int ln_loose_bwd(const RowProblem &p, const RowArgs &a, const RowCfg &cfg, int grid, hipStream_t st);
 // Resident blocks per CU of the LayerNormalization backward kernel for cfg
 // (0 when the runtime cannot tell).
 int row_bwd_ln_resident_blocks(int dtype, const RowCfg &cfg);

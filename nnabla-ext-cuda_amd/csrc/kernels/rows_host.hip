@@ -434,6 +434,21 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
   // LayerNormalization also keeps per-column accumulators, gamma and the
   // normalised row in registers.
   const bool ln = p.mode == kRowLN;
+  if (!tune_int("FORCE_STREAM", 0) && ln_loose_bwd_wanted(p, vec)) {
+    const int full = p.dtype == NBLAHIP_F16 ? 8 : 4;
+    const RowCfg loose = pick_ln_bwd_cfg(p.dtype, (p.R + full - 1) / full * full, full);
+    if (loose.ok && loose.tpr == 64) {
+      const int grid = ln_bwd_grid(p.rows, loose.tpr);
+      if (int e = ln_loose_bwd(p, a, loose, grid, st)) return e;
+      if (p.dgamma || p.dbeta) {
+        NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 15) / 16), dim3(1024), 0, st,
+                           static_cast<const float *>(p.ws), grid, a.R, p.dgamma, p.dbeta,
+                           p.accum_g, p.accum_b);
+        if (int e = last_launch_status()) return e;
+      }
+      return 0;
+    }
+  }
   const int nl_small = ln ? 4 : 8;
   const int nl_1024 = ln ? (p.dtype == NBLAHIP_F16 ? 1 : 2) : 8;
   RowCfg cfg = ln ? pick_ln_bwd_cfg(p.dtype, p.R, vec)

@@ -117,6 +117,11 @@ __global__ void __launch_bounds__(256) fill_kernel(D *__restrict__ dst, float v,
   for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < n; i += gridDim.x * 256ll) dst[i] = d;
 }
 
+template <typename W>
+__global__ void __launch_bounds__(256) fill_words_kernel(W *__restrict__ dst, W v, int64_t n) {
+  for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < n; i += gridDim.x * 256ll) dst[i] = v;
+}
+
 // Several small arrays converted in one launch (blockIdx.y: the array).
 constexpr int kStageMax = 16;
 struct StageArgs {
@@ -412,6 +417,37 @@ int nblahip_fill(void *dst, int dtype, float value, int64_t n, void *stream) {
   } else if (dtype == NBLAHIP_F16) {
     NBLAHIP_LAUNCH("fill_kernel", (fill_kernel<__half>), g, b, 0, st, static_cast<__half *>(dst), value, n);
   } else {
+    return NBLAHIP_EINVAL;
+  }
+  return last_launch_status();
+}
+
+int nblahip_fill_bytes(void *dst, int elem_bytes, unsigned long long pattern, int64_t n,
+                       void *stream) {
+  if (n == 0) return 0;
+  if (!dst || n < 0) return NBLAHIP_EINVAL;
+  if (reinterpret_cast<uintptr_t>(dst) % static_cast<uintptr_t>(elem_bytes > 0 ? elem_bytes : 1))
+    return NBLAHIP_EINVAL;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 g(flat_grid(n)), b(256);
+  switch (elem_bytes) {
+  case 1:
+    NBLAHIP_LAUNCH("fill_kernel", (fill_words_kernel<uint8_t>), g, b, 0, st, static_cast<uint8_t *>(dst),
+                   static_cast<uint8_t>(pattern), n);
+    break;
+  case 2:
+    NBLAHIP_LAUNCH("fill_kernel", (fill_words_kernel<uint16_t>), g, b, 0, st, static_cast<uint16_t *>(dst),
+                   static_cast<uint16_t>(pattern), n);
+    break;
+  case 4:
+    NBLAHIP_LAUNCH("fill_kernel", (fill_words_kernel<uint32_t>), g, b, 0, st, static_cast<uint32_t *>(dst),
+                   static_cast<uint32_t>(pattern), n);
+    break;
+  case 8:
+    NBLAHIP_LAUNCH("fill_kernel", (fill_words_kernel<unsigned long long>), g, b, 0, st,
+                   static_cast<unsigned long long *>(dst), pattern, n);
+    break;
+  default:
     return NBLAHIP_EINVAL;
   }
   return last_launch_status();

@@ -108,6 +108,38 @@ def test_device_arrays_store_every_dtype(dtype):
     np.testing.assert_array_equal(v.get_raw(dtype), np.zeros(5000, dtype))
 
 
+@pytest.mark.parametrize("dtype,value", [("int8", -5), ("uint8", 200), ("int16", -1234), ("uint16", 60000),
+                                         ("int32", 70000), ("uint32", 3000000000), ("int64", -7),
+                                         ("uint64", 9), ("bool", 1), ("float64", 2.5),
+                                         ("float32", 1.25), ("float16", -0.5)])
+def test_device_arrays_fill_every_dtype(dtype, value):
+    """fill() with a value other than zero on a device array of any dtype (the
+    value converted to the element type), first materialised on the device."""
+    v = B.Variable((4099,))
+    v.fill_data(value)
+    v.cast_raw("HipArray", dtype)
+    np.testing.assert_array_equal(v.get_raw(dtype), np.full(4099, value, dtype))
+
+
+def test_fill_bytes_entry_point():
+    """The C-ABI fill of 1-, 2-, 4- and 8-byte elements; an odd element size and
+    a misaligned destination are argument errors."""
+    import torch
+    from _util import load_package
+    K = load_package()
+    L = K.lib()
+    for dt, nbytes, pattern in [(torch.uint8, 1, 0xAB), (torch.int16, 2, 0x1234),
+                                (torch.int32, 4, 0x7EADBEEF), (torch.int64, 8, 0x0123456789ABCDEF)]:
+        t = torch.zeros(100003, dtype=dt, device="cuda")
+        K.check(L.nblahip_fill_bytes(t.data_ptr(), nbytes, pattern, t.numel() - 3, None))
+        torch.cuda.synchronize()
+        assert (t[:-3] == pattern).all() and (t[-3:] == 0).all()
+    t = torch.zeros(64, dtype=torch.int32, device="cuda")
+    assert L.nblahip_fill_bytes(t.data_ptr(), 3, 1, 4, None) == -1
+    assert L.nblahip_fill_bytes(t.data_ptr() + 2, 4, 1, 4, None) == -1
+    assert L.nblahip_fill_bytes(t.data_ptr(), 4, 1, 0, None) == 0
+
+
 def test_host_reader_of_a_pinned_array_waits_for_its_pending_download():
     """An ASYNC device-to-pinned-host cast leaves the transfer's event on the
     pinned array; a following host read through another host class (a plain

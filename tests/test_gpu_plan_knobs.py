@@ -209,6 +209,8 @@ SWITCHES = [
      ["row_stats_stream_kernel", "plane_sums_stream_kernel"], ["row_fwd_kernel", "row_bwd_kernel_in"]),
     ("ln_long_rows_all_streaming", run_ln, (24, 18432, F16), {"LN_LONG_ROWS_CACHED": 0},
      ["ln_row_sums_stream_kernel", "row_bwd_dx_kernel"], ["row_bwd_kernel_lnx"]),
+    ("ln_odd_rows_scalar", run_ln, (40, 1023, F16), {"LN_LOOSE": 0},
+     ["row_bwd_kernel_ln"], ["ln_loose_bwd_kernel"]),
     ("in_rows_instead_of_channel_blocks", run_in, (4, 256, (32, 32), F16), {"IN_NO_CHANNEL_BLOCKS": 1},
      ["row_bwd_kernel_in", "pair_param_reduce_kernel"], ["row_bwd_kernel_inc"]),
     ("gn_float_groups_streamed", run_gn, (4, 64, (64, 64), 8, F32), {"GN_FLOAT_1024X8": 0},
