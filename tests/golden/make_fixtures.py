@@ -155,6 +155,18 @@ def main():
     gn_case("gn_f32_stat_grads", 2, 12, (5, 7), 3, "f32", 33, stat_grads=True)
     gn_case("in_f32_stat_grads", 2, 12, (5, 7), 12, "f32", 34, stat_grads=True)
     gn_case("gn_f32_one_group", 2, 6, (9,), 1, "f32", 35)
+    # shapes of the plans that came later: planes that are no whole number of
+    # 16-byte vectors (7x7: channel packs / rows; 17x17: masked vectors), an odd
+    # hidden size, odd planes for Instance / GroupNormalization, and a tensor
+    # wide enough for the channel-last kernels (tests run it channel-last too)
+    bn_case("bn_nchw_f16_7x7_planes", (8, 24, 7, 7), 1, "f16", 41)
+    bn_case("bn_nchw_f32_17x17_planes", (5, 4, 17, 17), 1, "f32", 42, mean=1.0, std=2.0)
+    ln_case("ln_f16_odd_hidden", 5, 1023, "f16", 43)
+    ln_case("ln_f32_odd_hidden_stat_grads", 4, 515, "f32", 44, stat_grads=True)
+    gn_case("in_f16_odd_planes", 2, 6, (15, 15), 6, "f16", 45)
+    gn_case("gn_f16_odd_planes", 2, 8, (9, 7), 2, "f16", 46)
+    gn_case("gn_f16_wide", 2, 64, (8, 8), 8, "f16", 47)
+    gn_case("in_f16_wide", 2, 64, (8, 8), 64, "f16", 48)
 
 
 if __name__ == "__main__":

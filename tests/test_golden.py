@@ -31,7 +31,7 @@ def load(name):
 
 def test_fixture_inventory():
     kinds = {load(n)["kind"] for n in NAMES}
-    assert kinds == {"bn", "ln", "gn"} and len(NAMES) >= 14
+    assert kinds == {"bn", "ln", "gn"} and len(NAMES) >= 22
 
 
 def close64(got, ref, name):
@@ -184,3 +184,83 @@ def test_hip_path_reproduces_golden(name):
         assert_close(got.detach().float().cpu().numpy(), ref, dn, kind, f"{name} {what}")
 
     run(d, HipOps(dn), check)
+
+
+class HipChannelLastOps(HipOps):
+    """Group / InstanceNormalization fixtures (stored channel-first) run through
+    the channel-last entry points on the transposed tensors; outputs come back
+    transposed."""
+
+    @staticmethod
+    def cl(a):
+        return np.ascontiguousarray(np.moveaxis(np.asarray(a), 1, -1))
+
+    def back(self, t):
+        return self.torch.movedim(t, -1, 1).contiguous()
+
+    def gn_forward(self, x, b, g, groups, eps):
+        xd = self.dev(self.cl(x), True)
+        if groups == x.shape[1]:
+            y, m, v = self.K.in_forward(xd, self.dev(b), self.dev(g), eps, channel_last=True)
+        else:
+            y, m, v = self.K.gn_forward(xd, self.dev(b), self.dev(g), groups, eps, channel_last=True)
+        return self.back(y), m, v
+
+    def gn_backward(self, x, dy, g, m, v, groups, eps, dm, dv):
+        kw = dict(dmean=None if dm is None else self.dev(dm), dvar=None if dv is None else self.dev(dv),
+                  channel_last=True)
+        xd, dyd = self.dev(self.cl(x), True), self.dev(self.cl(dy), True)
+        if groups == x.shape[1]:
+            dx, dg, db = self.K.in_backward(xd, dyd, self.dev(g), m, v, eps, **kw)
+        else:
+            dx, dg, db = self.K.gn_backward(xd, dyd, self.dev(g), m, v, groups, eps, **kw)
+        return self.back(dx), dg, db
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", [n for n in NAMES if n.startswith(("gn_", "in_"))])
+def test_hip_channel_last_reproduces_golden(name):
+    d = load(name)
+    dn = d["dtype"]
+
+    def check(what, got, ref, kind):
+        assert_close(got.detach().float().cpu().numpy(), ref, dn, kind, f"{name} channel-last {what}")
+
+    run(d, HipChannelLastOps(dn), check)
+
+
+# Fixtures again with the default plan of their shape switched off, so that the
+# plans behind it are held to the same vectors: (fixture, knobs).
+PLAN_VARIANTS = [
+    ("bn_nchw_f16_7x7_planes", {"BN_ROWS": 0}),                       # channel packs / masked split reduction
+    ("bn_nchw_f16_7x7_planes", {"BN_ROWS": 0, "BN_PACK": 0}),
+    ("bn_nchw_f32_17x17_planes", {"BN_ROWS": 0}),                     # a channel per block, masked vectors
+    ("bn_nchw_f32_17x17_planes", {"BN_ROWS": 0, "BN_MASKED_ONCHIP": 0}),
+    ("bn_nchw_f32_17x17_planes", {"BN_ROWS": 0, "BN_MASKED_ONCHIP": 0, "BN_MASKED_PLANES": 0}),
+    ("bn_nhwc_f16_outliers", {"BN_CL_CACHED": 0}),
+    ("bn_nhwc_f16_outliers", {"BN_CL_CACHED": 0, "BN_CL_SPLIT": 0}),
+    ("ln_f16_odd_hidden", {"LN_LOOSE": 0}),
+    ("ln_f16_odd_hidden", {"FORCE_STREAM": 1}),
+    ("in_f16_odd_planes", {"ROW_MASKED": 0}),
+    ("gn_f16_odd_planes", {"ROW_MASKED": 0}),
+    ("gn_f16_wide", {"FORCE_STREAM": 1}),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,knobs", PLAN_VARIANTS)
+def test_hip_plan_variants_reproduce_golden(name, knobs):
+    d = load(name)
+    dn = d["dtype"]
+    K = load_package()
+
+    def check(what, got, ref, kind):
+        assert_close(got.detach().float().cpu().numpy(), ref, dn, kind, f"{name} {knobs} {what}")
+
+    K.tune_reset()
+    for k, v in knobs.items():
+        K.tune_set(k, v)
+    try:
+        run(d, HipOps(dn), check)
+    finally:
+        K.tune_reset()
