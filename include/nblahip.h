@@ -46,8 +46,9 @@ enum nblahip_status {
   NBLAHIP_OK = 0,
   NBLAHIP_EINVAL = -1,    /* NULL required pointer, non-positive size, bad enum */
   NBLAHIP_EWORKSPACE = -2,/* workspace NULL, misaligned or too small */
-  NBLAHIP_ERANGE = -3,    /* 2^31 or more elements in a BatchNormalization tensor or in
-                             one row / sample / group of the other functions */
+  NBLAHIP_ERANGE = -3,    /* 2^31 or more elements in one row / sample / slice ahead of
+                             the channel axis, or in a tensor given to an entry point
+                             that does not run in ranges */
   NBLAHIP_EALIAS = -4     /* output overlaps an input it must not overlap */
 };
 
@@ -68,6 +69,15 @@ NBLAHIP_EXPORT int nblahip_abi_version(void);
  * reads the partner's part of the inputs again, which the partner would
  * already be overwriting): they run on the plans without an exchange, with
  * the same results within the summation order.
+ *
+ * Sizes: a tensor of fewer than 2^31 elements is one sequence of launches.
+ * Larger ones run in ranges along size0 - a channel runs through the whole
+ * tensor, so the ranges are the steps of a split batch (further down): local
+ * statistics per range, nblahip_bn_merge_stats, the normalization per range;
+ * backward: the local sums per range, their sum, dx per range.  size1*size2
+ * must stay below 2^31; the fused backward has no ranged form.  The reference
+ * indexes with int (kernel/batch_normalization.cuh:246-254) and has no such
+ * path.
  * ---------------------------------------------------------------------- */
 
 /* Replaces forward_impl_global + forward_global_kernel

@@ -12,8 +12,12 @@ template <typename T>
 void BatchNormalizationHip<T>::setup_impl(const Variables &inputs, const Variables &outputs) {
   BatchNormalization<T>::setup_impl(inputs, outputs);
   hip_set_device(this->device_);
-  NBLA_CHECK(inputs[0]->size() < (Size_t(1) << 31), error_code::value,
-             "BatchNormalizationHip indexes with 32 bits: fewer than 2^31 elements required.");
+  // Tensors of 2^31 elements and more run in ranges along the outermost axes
+  // (local statistics, merge, normalization per range inside the kernel
+  // layer); one slice of those axes must stay below that.
+  NBLA_CHECK(this->size1_ * this->size2_ < (Size_t(1) << 31), error_code::value,
+             "BatchNormalizationHip indexes with 32 bits: fewer than 2^31 elements per slice of the "
+             "axes ahead of the channel axis required.");
   workspace_bytes_ = nblahip_bn_workspace_bytes(this->size0_, this->size1_, this->size2_,
                                                 HipDtype<T>::code);
   workspace_.reshape(Shape_t{static_cast<Size_t>((workspace_bytes_ + 3) / 4)}, true);

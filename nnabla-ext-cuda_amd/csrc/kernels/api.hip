@@ -135,6 +135,61 @@ int check_in_place(const void *out, const void *in, size_t tensor_bytes) {
   return out != in && ranges_overlap(out, tensor_bytes, in, tensor_bytes) ? NBLAHIP_EALIAS : 0;
 }
 
+// BatchNormalization tensors of 2^31 elements and more.  A channel runs
+// through the whole tensor, so ranges of samples are not independent of each
+// other as the rows of the other functions are: they run as the steps of a
+// batch that is split over workers - local statistics per range, their merge,
+// the normalization per range; backward: the local sums per range, their sum,
+// dx per range - with the ranges' statistics and sums behind the launches' own
+// workspace.  (The reference indexes these tensors with int and has no such
+// path.)  One sample must stay below 2^31 elements.
+struct BnRanges {
+  int64_t per = 0; // samples (size0 slices) per range
+  int count = 0;   // ranges; 0: the tensor fits one launch
+};
+
+// 0: proceed (r.count == 0: one launch); 1: empty tensor; <0: error.
+int bn_ranges(int64_t size0, int64_t C, int64_t size2, BnRanges &r) {
+  const int d = check_dims_units(size0, C, size2);
+  if (d) return d;
+  r.per = units_per_launch(size0, C * size2);
+  r.count = r.per >= size0 ? 0 : static_cast<int>((size0 + r.per - 1) / r.per);
+  return 0;
+}
+
+size_t bn_stats_floats(int64_t C) { return 2 * static_cast<size_t>(C) + 1; }
+
+// Workspace of a ranged call: [a launch's workspace][statistics count x (2C+1)]
+// [pair sums count x 2C][their total 2C], each part 256-byte aligned.
+struct BnRangedWs {
+  size_t launch = 0, stats = 0, sums = 0, total = 0;
+  size_t bytes() const { return launch + stats + sums + total; }
+};
+
+BnRangedWs bn_ranged_ws(int64_t size0, int64_t C, int64_t size2, int dtype, const BnRanges &r) {
+  auto up = [](size_t b) { return (b + 255) / 256 * 256; };
+  BnRangedWs w;
+  w.launch = up(chunked_workspace(size0, r.per, [&](int64_t n) { return bn_workspace_bytes(n, C, size2, dtype); }));
+  w.stats = up(static_cast<size_t>(r.count) * bn_stats_floats(C) * sizeof(float));
+  w.sums = up(static_cast<size_t>(r.count) * 2 * static_cast<size_t>(C) * sizeof(float));
+  w.total = up(2 * static_cast<size_t>(C) * sizeof(float));
+  return w;
+}
+
+size_t bn_any_workspace_bytes(int64_t size0, int64_t C, int64_t size2, int dtype) {
+  BnRanges r;
+  if (bn_ranges(size0, C, size2, r) != 0) return 0;
+  if (r.count == 0) return bn_workspace_bytes(size0, C, size2, dtype);
+  return bn_ranged_ws(size0, C, size2, dtype, r).bytes();
+}
+
+const void *advance(const void *p, int64_t elems, int dtype) {
+  return p ? static_cast<const char *>(p) + static_cast<size_t>(elems) * (dtype == NBLAHIP_F16 ? 2 : 4) : nullptr;
+}
+void *advance(void *p, int64_t elems, int dtype) {
+  return p ? static_cast<char *>(p) + static_cast<size_t>(elems) * (dtype == NBLAHIP_F16 ? 2 : 4) : nullptr;
+}
+
 // Scratch of nblahip_bn_fwd_train_static, the entry point for callers that
 // cannot allocate: one array per GPU in the code object's own data segment,
 // held until the process ends.  `scratch` below is only the host-side handle
@@ -175,7 +230,8 @@ int bn_fwd_infer_impl(const void *x, const void *z, int relu, const float *rmean
                       int64_t size0, int64_t size1, int64_t size2, float eps, int dtype,
                       void *stream) {
   if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
-  const int d = check_dims3(size0, size1, size2);
+  BnRanges ranges;
+  const int d = bn_ranges(size0, size1, size2, ranges);
   if (d) return d < 0 ? d : 0;
   if (!x || !y || !rmean || !rvar) return NBLAHIP_EINVAL;
   {
@@ -196,7 +252,18 @@ int bn_fwd_infer_impl(const void *x, const void *z, int relu, const float *rmean
   p.eps = eps;
   p.relu = relu;
   p.z = z;
-  return launch_bn_infer(p, as_stream(stream));
+  if (ranges.count == 0) return launch_bn_infer(p, as_stream(stream));
+  // (elementwise: the ranges need nothing from each other)
+  for (int64_t s0 = 0; s0 < size0; s0 += ranges.per) {
+    BnProblem q = p;
+    const int64_t at = s0 * size1 * size2;
+    q.size0 = std::min(ranges.per, size0 - s0);
+    q.x = advance(x, at, dtype);
+    q.z = advance(z, at, dtype);
+    q.out = advance(y, at, dtype);
+    if (int e = launch_bn_infer(q, as_stream(stream))) return e;
+  }
+  return 0;
 }
 
 int bn_fwd_train_impl(const void *x, const void *z, int relu, const float *gamma,
@@ -205,15 +272,62 @@ int bn_fwd_train_impl(const void *x, const void *z, int relu, const float *gamma
                       float decay_rate, float eps, int dtype, void *workspace,
                       size_t workspace_bytes, void *stream) {
   if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
-  const int d = check_dims3(size0, size1, size2);
+  BnRanges ranges;
+  const int d = bn_ranges(size0, size1, size2, ranges);
   if (d) return d < 0 ? d : 0;
   if (!x || !y || !batch_mean || !batch_var) return NBLAHIP_EINVAL;
   {
     const size_t tb = static_cast<size_t>(size0) * size1 * size2 * elem_bytes(dtype);
     if (check_in_place(y, x, tb) || check_in_place(y, z, tb)) return NBLAHIP_EALIAS;
   }
-  if (int e = check_ws(workspace, workspace_bytes, bn_workspace_bytes(size0, size1, size2, dtype)))
+  if (int e = check_ws(workspace, workspace_bytes, bn_any_workspace_bytes(size0, size1, size2, dtype)))
     return e;
+  if (ranges.count > 0) {
+    hipStream_t st = as_stream(stream);
+    const BnRangedWs w = bn_ranged_ws(size0, size1, size2, dtype, ranges);
+    float *stats = reinterpret_cast<float *>(static_cast<char *>(workspace) + w.launch);
+    const size_t stride = bn_stats_floats(size1);
+    int i = 0;
+    for (int64_t s0 = 0; s0 < size0; s0 += ranges.per, ++i) {
+      BnProblem q;
+      q.dtype = dtype;
+      q.x = advance(x, s0 * size1 * size2, dtype);
+      q.batch_mean = stats + i * stride;
+      q.batch_var = stats + i * stride + size1;
+      q.size0 = std::min(ranges.per, size0 - s0);
+      q.C = size1;
+      q.size2 = size2;
+      q.ws = workspace;
+      q.ws_bytes = w.launch;
+      if (int e = launch_bn_local_stats(q, st)) return e;
+      // (the range's count: its elements per channel, as the merge's weight)
+      if (int e = nblahip_fill(stats + i * stride + 2 * size1, NBLAHIP_F32,
+                               static_cast<float>(static_cast<double>(q.size0) * static_cast<double>(size2)), 1, st))
+        return e;
+    }
+    if (int e = launch_bn_merge_stats(stats, ranges.count, size1, batch_mean, batch_var, rmean, rvar,
+                                      decay_rate, st))
+      return e;
+    for (int64_t s0 = 0; s0 < size0; s0 += ranges.per) {
+      BnProblem q;
+      const int64_t at = s0 * size1 * size2;
+      q.dtype = dtype;
+      q.x = advance(x, at, dtype);
+      q.z = advance(z, at, dtype);
+      q.out = advance(y, at, dtype);
+      q.mean = batch_mean;
+      q.var = batch_var;
+      q.gamma = gamma;
+      q.beta = beta;
+      q.size0 = std::min(ranges.per, size0 - s0);
+      q.C = size1;
+      q.size2 = size2;
+      q.eps = eps;
+      q.relu = relu;
+      if (int e = launch_bn_infer(q, st)) return e;
+    }
+    return 0;
+  }
   BnProblem p;
   p.dtype = dtype;
   p.x = x;
@@ -243,8 +357,11 @@ int bn_bwd_impl(int fused, const void *x, const void *y_out, const void *dy, con
                 float eps, int batch_stat, int dtype, void *workspace, size_t workspace_bytes,
                 void *stream) {
   if (!dtype_ok(dtype)) return NBLAHIP_EINVAL;
-  const int d = check_dims3(size0, size1, size2);
+  BnRanges ranges;
+  const int d = bn_ranges(size0, size1, size2, ranges);
   if (d) return d < 0 ? d : 0;
+  // (the fused backward, which gates dy by the stored output on the way, has no ranged form)
+  if (ranges.count > 0 && fused) return NBLAHIP_ERANGE;
   if (!x || !dy || !mean || !var) return NBLAHIP_EINVAL;
   if (fused ? !y_out : (y_out || dz)) return NBLAHIP_EINVAL;
   {
@@ -253,8 +370,61 @@ int bn_bwd_impl(int fused, const void *x, const void *y_out, const void *dy, con
         ranges_overlap(dz, tb, x, tb))
       return NBLAHIP_EALIAS;
   }
-  if (int e = check_ws(workspace, workspace_bytes, bn_workspace_bytes(size0, size1, size2, dtype)))
+  if (int e = check_ws(workspace, workspace_bytes, bn_any_workspace_bytes(size0, size1, size2, dtype)))
     return e;
+  if (ranges.count > 0) {
+    hipStream_t st = as_stream(stream);
+    const BnRangedWs w = bn_ranged_ws(size0, size1, size2, dtype, ranges);
+    float *sums = reinterpret_cast<float *>(static_cast<char *>(workspace) + w.launch + w.stats);
+    float *total = reinterpret_cast<float *>(static_cast<char *>(workspace) + w.launch + w.stats + w.sums);
+    BnProblem base;
+    base.dtype = dtype;
+    base.gamma = gamma;
+    base.mean = mean;
+    base.var = var;
+    base.C = size1;
+    base.size2 = size2;
+    base.eps = eps;
+    base.ws = workspace;
+    base.ws_bytes = w.launch;
+    int i = 0;
+    for (int64_t s0 = 0; s0 < size0; s0 += ranges.per, ++i) {
+      BnProblem q = base;
+      const int64_t at = s0 * size1 * size2;
+      q.x = advance(x, at, dtype);
+      q.dy = advance(dy, at, dtype);
+      q.size0 = std::min(ranges.per, size0 - s0);
+      q.dgamma = dgamma;
+      q.dbeta = dbeta;
+      q.accum_g = i == 0 ? accum_dgamma : 1;
+      q.accum_b = i == 0 ? accum_dbeta : 1;
+      q.batch_stat = batch_stat;
+      if (batch_stat) {
+        q.sums_out = sums + static_cast<size_t>(i) * 2 * size1; // this range's (sum dy*(x-mean), sum dy)
+      } else {
+        q.out = advance(dx, at, dtype); // fixed statistics: dx is elementwise
+        q.accum_dx = accum_dx;
+      }
+      if (int e = launch_bn_bwd(q, st)) return e;
+    }
+    if (!batch_stat || !dx) return 0;
+    if (int e = launch_sum_rows(sums, ranges.count, 2 * size1, total, st)) return e;
+    for (int64_t s0 = 0; s0 < size0; s0 += ranges.per) {
+      BnProblem q = base;
+      const int64_t at = s0 * size1 * size2;
+      q.x = advance(x, at, dtype);
+      q.dy = advance(dy, at, dtype);
+      q.out = advance(dx, at, dtype);
+      q.size0 = std::min(ranges.per, size0 - s0);
+      q.dmean = dmean;
+      q.dvar = dvar;
+      q.sums_in = total;
+      q.total_count = static_cast<double>(size0) * static_cast<double>(size2);
+      q.accum_dx = accum_dx;
+      if (int e = launch_bn_bwd_from_sums(q, st)) return e;
+    }
+    return 0;
+  }
   BnProblem p;
   p.dtype = dtype;
   p.x = x;
@@ -294,8 +464,8 @@ int nblahip_bn_fwd_infer(const void *x, const float *rmean, const float *rvar,
 }
 
 size_t nblahip_bn_workspace_bytes(int64_t size0, int64_t size1, int64_t size2, int dtype) {
-  if (!dtype_ok(dtype) || check_dims3(size0, size1, size2) != 0) return 0;
-  return bn_workspace_bytes(size0, size1, size2, dtype);
+  if (!dtype_ok(dtype)) return 0;
+  return bn_any_workspace_bytes(size0, size1, size2, dtype);
 }
 
 int nblahip_bn_fwd_train(const void *x, const float *gamma, const float *beta, void *y,

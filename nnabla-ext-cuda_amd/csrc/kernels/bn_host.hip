@@ -587,6 +587,23 @@ int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
   return 0;
 }
 
+namespace {
+__global__ void __launch_bounds__(256)
+sum_rows_kernel(const float *__restrict__ in, int rows, uint32_t n, float *__restrict__ out) {
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  if (i >= n) return;
+  float s = 0.f;
+  for (int r = 0; r < rows; ++r) s += in[static_cast<size_t>(r) * n + i];
+  out[i] = s;
+}
+} // namespace
+
+int launch_sum_rows(const float *in, int rows, int64_t n, float *out, hipStream_t st) {
+  NBLAHIP_LAUNCH("sum_rows_kernel", sum_rows_kernel, dim3(static_cast<uint32_t>((n + 255) / 256)),
+                 dim3(256), 0, st, in, rows, static_cast<uint32_t>(n), out);
+  return last_launch_status();
+}
+
 int launch_bn_bwd_from_sums(const BnProblem &p, hipStream_t st) {
   if (!p.out) return 0;
   const bool al = aligned16(p.x) && aligned16(p.dy) && aligned16(p.out);

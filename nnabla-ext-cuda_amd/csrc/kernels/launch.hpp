@@ -186,6 +186,8 @@ int launch_bn_merge_stats(const float *stats, int workers, int64_t C, float *bat
                           float *batch_var, float *rmean, float *rvar, float decay,
                           hipStream_t st);
 int launch_bn_bwd_from_sums(const BnProblem &p, hipStream_t st);
+// out[i] = in[0][i] + in[1][i] + ... + in[rows-1][i], i < n (rows in order).
+int launch_sum_rows(const float *in, int rows, int64_t n, float *out, hipStream_t st);
 size_t bn_workspace_bytes(int64_t size0, int64_t C, int64_t size2, int dtype);
 
 // Optional per-kernel timing.  When enabled, a launch goes through

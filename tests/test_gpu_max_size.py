@@ -1,5 +1,6 @@
-"""Tensors just below the 2^31-element limit of the C-ABI (fp16, 4.3 GB each):
-the 32-bit index arithmetic of the kernels must not wrap.  The input is a small
+"""Tensors just below 2^31 elements (fp16, 4.3 GB each), the most one launch
+indexes, and just above, where the C-ABI runs ranges: the 32-bit index
+arithmetic of the kernels must not wrap.  The input is a small
 block tiled along the batch, so every tile must reproduce the result of the
 block alone, which the float64 oracle checks; parameter gradients scale with
 the number of tiles."""
@@ -128,17 +129,21 @@ def test_group_and_instance_normalization_just_below_2_31_elements(kind):
     assert_close(to_np(db) / n, db_r, "f16", "pgrad", "dbeta / n")
 
 
-def test_one_more_element_is_refused():
-    """BatchNormalization reduces over the whole tensor and indexes it with 32
-    bits, as the reference's kernels do (kernel/batch_normalization.cuh:246-254):
-    2^31 elements are refused.  The row normalizations take larger tensors in
-    ranges of rows / samples, but one row or sample must stay below 2^31."""
+def test_one_unit_of_2_31_elements_is_refused():
+    """Tensors of 2^31 elements and more run in ranges of rows / samples, but
+    one row, one sample (for BatchNormalization: one slice of the axes ahead of
+    the channel axis) must stay below 2^31 elements; the fused backward has no
+    ranged form.  Refused before anything is launched (the buffers here hold
+    16 elements)."""
     L = K.lib()
     s = torch.cuda.current_stream().cuda_stream
     t = torch.empty(16, device="cuda")
     p = t.data_ptr()
-    assert L.nblahip_bn_fwd_infer(p, p, p, None, None, p, 1 << 11, 1 << 10, 1 << 10, 1e-5, 1,
-                                  s) == -3                 # 2^31 elements
+    assert L.nblahip_bn_fwd_infer(p, p, p, None, None, p, 2, 1 << 16, 1 << 15, 1e-5, 1,
+                                  s) == -3                 # 2^31 elements per slice
+    assert L.nblahip_bn_workspace_bytes(2, 1 << 16, 1 << 15, 1) == 0
+    assert L.nblahip_fused_bn_bwd(p, p, p, None, p, p, None, None, p, None, None, None, 0, 0, 0, 0,
+                                  1 << 11, 1 << 10, 1 << 10, 1e-5, 1, 1, p, 0, s) == -3
     assert L.nblahip_in_fwd(p, None, None, p, p, p, 2, 1 << 16, 1 << 15, 1, 1, 1e-5, 1,
                             s) == -3                       # 2^31 elements per sample
     assert L.nblahip_ln_fwd(p, None, None, p, p, p, 2, 1 << 31, 1e-5, 1, s) == -3
@@ -277,3 +282,71 @@ def test_channel_last_batch_beyond_65535(kind):
     _tiles_close(dx.view((tiles, blk) + sp + (c,)), tiles, back(dx_r), "f16", "grad", "dx")
     assert_close(to_np(dg) / tiles, dg_r, "f16", "pgrad", "dgamma / tiles")
     assert_close(to_np(db) / tiles, db_r, "f16", "pgrad", "dbeta / tiles")
+
+
+@pytest.mark.parametrize("layout", ["planes", "channel_last"])
+def test_batch_normalization_above_2_31_elements(layout):
+    """A channel runs through the whole tensor, so the ranges are not
+    independent: local statistics per range, their merge, normalization per
+    range; backward: local sums per range, their sum, dx per range.  The batch
+    is n1 copies of one sample followed by n2 copies of another, so that the
+    two ranges (2047 + 4 samples) have different statistics and the merge must
+    weight them; expected values from the two samples in float64."""
+    _need(30)
+    c, sp = 256, 4096
+    n = (1 << 31) // (c * sp) + 3                      # 2051 samples, two ranges
+    n2 = 100
+    n1 = n - n2
+    rng = np.random.default_rng(75)
+    cl = layout == "channel_last"
+    shape_b = (1, sp, c) if cl else (1, c, sp)
+    axis = 2 if cl else 1
+    xa = (rng.standard_normal(shape_b) * 2 + 1).astype(np.float16)
+    xb = (rng.standard_normal(shape_b) * 0.5 - 2).astype(np.float16)
+    dya = rng.standard_normal(shape_b).astype(np.float16)
+    dyb = (rng.standard_normal(shape_b) * 2).astype(np.float16)
+    g = rng.uniform(0.5, 1.5, c).astype(np.float32)
+    b = (rng.standard_normal(c) * 0.1).astype(np.float32)
+    x = torch.cat([torch.from_numpy(xa).cuda().repeat(n1, 1, 1), torch.from_numpy(xb).cuda().repeat(n2, 1, 1)])
+    dy = torch.cat([torch.from_numpy(dya).cuda().repeat(n1, 1, 1), torch.from_numpy(dyb).cuda().repeat(n2, 1, 1)])
+    assert x.numel() > (1 << 31) and x.is_contiguous()
+    gd, bd = to_dev(g), to_dev(b)
+    rm, rv = torch.zeros(c, device="cuda"), torch.ones(c, device="cuda")
+
+    # float64 expectations per channel
+    red = (0, 1) if cl else (0, 2)
+    X = [xa.astype(np.float64), xb.astype(np.float64)]
+    D = [dya.astype(np.float64), dyb.astype(np.float64)]
+    W = [n1, n2]
+    N = float(n) * sp
+    mean = sum(w * a.sum(axis=red) for w, a in zip(W, X)) / N
+    bshape = (1, 1, c) if cl else (1, c, 1)
+    var = sum(w * ((a - mean.reshape(bshape)) ** 2).sum(axis=red) for w, a in zip(W, X)) / N
+    istd = 1.0 / np.sqrt(var + 1e-5)
+    G, Bt = g.astype(np.float64).reshape(bshape), b.astype(np.float64).reshape(bshape)
+    XH = [(a - mean.reshape(bshape)) * istd.reshape(bshape) for a in X]
+    Y = [xh * G + Bt for xh in XH]
+    sdy = sum(w * d.sum(axis=red) for w, d in zip(W, D))
+    sdx = sum(w * (d * xh).sum(axis=red) for w, d, xh in zip(W, D, XH))
+    DX = [G * istd.reshape(bshape) * (d - sdy.reshape(bshape) / N - xh * sdx.reshape(bshape) / N)
+          for d, xh in zip(D, XH)]
+
+    y, m, v = K.bn_forward_batch(x, bd, gd, rm, rv, axis, 0.9, 1e-5)
+    assert_close(to_np(m), mean, "f16", "stat", "mean")
+    assert_close(to_np(v), var, "f16", "stat", "var")
+    assert_close(to_np(rm), 0.1 * mean, "f16", "stat", "running mean")
+    assert_close(to_np(rv), 0.9 + 0.1 * var * N / (N - 1), "f16", "stat", "running var")
+    for k, which in ((0, 0), (n1 - 1, 0), (n1, 1), (n - 5, 1), (n - 1, 1)):
+        assert_close(to_np(y[k:k + 1]), Y[which], "f16", "y", f"y of sample {k}")
+    del y
+    yi = K.bn_forward_global(x, bd, gd, m, v, axis, 1e-5)   # fixed statistics: elementwise ranges
+    for k, which in ((0, 0), (n1, 1), (n - 1, 1)):
+        assert_close(to_np(yi[k:k + 1]), Y[which], "f16", "y", f"inference y of sample {k}")
+    del yi
+    pre = torch.full((c,), 2.0, device="cuda")
+    dx, dg, db = K.bn_backward(x, dy, gd, m, v, axis, 1e-5, dgamma=pre.clone(), dbeta=pre.clone(),
+                               accum=(False, True, True))
+    for k, which in ((0, 0), (n1 - 1, 0), (n1, 1), (n - 5, 1), (n - 1, 1)):
+        assert_close(to_np(dx[k:k + 1]), DX[which], "f16", "grad", f"dx of sample {k}")
+    assert_close((to_np(dg) - 2.0) / n, sdx / n, "f16", "pgrad", "dgamma / n")
+    assert_close((to_np(db) - 2.0) / n, sdy / n, "f16", "pgrad", "dbeta / n")
