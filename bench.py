@@ -102,8 +102,9 @@ BN_ONCHIP_BWD = {"bn_onchip_bwd_kernel": 4, "row_bwd_kernel_bn": 3, "in_cl_row_b
                  "bn_pack_bwd_kernel": 3, "bn_chan_split_bwd_kernel": 3}
 # bn_onchip_bwd_kernel holds x of a channel on its CU and streams dy twice
 # (x, 2 dy, dx = 4 passes); of a channel beyond 20480 16-byte vectors it holds
-# 18432 and reads the rest of x twice as well.
-BN_ONCHIP_BWD_HELD, BN_ONCHIP_BWD_WHOLE = 18432, 20480
+# 18432 from the start plus 3072 parked in LDS on their way through the first
+# pass, and reads the rest of x twice as well.
+BN_ONCHIP_BWD_HELD, BN_ONCHIP_BWD_WHOLE = 18432 + 3072, 20480
 # bn_onchip_fwd_kernel holds up to 25600 vectors of a channel; the rest of a
 # longer channel is read twice.
 BN_ONCHIP_FWD_HELD = 25600

@@ -15,7 +15,9 @@
 // (sums, then dx): x once, dy twice, dx once = 4 S where the split reduction
 // moves 5 S; dgamma/dbeta are written by the channel's block, no finalize.
 // Beside x a thread needs a batch of dy, so it holds fewer vectors: 18432 per
-// channel with 1024 threads, 20480 with 512; the rest of x is streamed with dy.
+// channel with 1024 threads, 20480 with 512; the rest of x is streamed with dy
+// (its first 3072 vectors parked in the LDS that is left, so that the second
+// pass does not read them again).
 //
 // The block is alone on its CU, so fewer channels than CUs leave CUs idle; the
 // path still wins down to an eighth (forward) or a quarter (backward) of the
@@ -282,15 +284,21 @@ bn_onchip_fwd_kernel(const BnOnchipArgs a) {
 // threads (and 320 bytes of LDS per thread instead of 160).
 // OVER: the channel is longer than the NR + NS slots held on chip; the
 // vectors beyond them are streamed like dy (x and dy read in both passes, a
-// rolled loop of small batches), so only the held part saves its second read:
-// (18432 / nv) S of the 5 S.
+// rolled loop of small batches), so only the held part - and what the first
+// pass parks in LDS - saves its second read: (21504 / nv) S of the 5 S.
 template <typename T, int VEC, int NR, int NS, int B, int TB, bool OVER = false>
 __global__ void __launch_bounds__(TB)
 bn_onchip_bwd_kernel(const BnOnchipArgs a) {
   static_assert(sizeof(RawVec<T, VEC>) == sizeof(Slot<T, VEC>), "8- or 16-byte vectors");
   constexpr int NL = NR + NS;
+  // OVER: the LDS the held slots leave free parks the first NX slots of x
+  // beyond them on their way through the first pass (each thread reads back
+  // only what it wrote), so the second pass reads those from LDS, not again
+  // from memory: (5 - (NL + NX) * TB / nv) S.
+  constexpr int NX = (OVER && TB == 1024) ? (9 - NS > 0 ? 9 - NS : 0) : 0;
   __shared__ float red[TB / kWave];
   __shared__ Slot<T, VEC> spill[NS > 0 ? NS * TB : 1];
+  __shared__ Slot<T, VEC> extra[NX > 0 ? NX * TB : 1];
   const uint32_t c = onchip_channel(a, blockIdx.x);
   const uint32_t t = threadIdx.x;
   const T *__restrict__ x = static_cast<const T *>(a.x);
@@ -387,6 +395,11 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
       }
 #pragma unroll
       for (int b = 0; b < BO; ++b) {
+        if constexpr (NX > 0) {
+          // (the slot index is the same for the whole block: a scalar branch)
+          const uint32_t slot = (v0 - static_cast<uint32_t>(NL) * TB) / TB + b;
+          if (slot < static_cast<uint32_t>(NX)) extra[slot * TB + t] = __builtin_bit_cast(Slot<T, VEC>, xo[b]);
+        }
         float py = raw_sum<T, VEC>(d[b], 0.f), px = 0.f;
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
@@ -463,7 +476,13 @@ bn_onchip_bwd_kernel(const BnOnchipArgs a) {
 #pragma unroll
       for (int b = 0; b < BO; ++b) {
         off[b] = onchip_offset(a, c, min(v0 + b * TB + t, a.nv - 1u), VEC);
-        xo[b] = load_raw<T, VEC>(x + off[b]);
+        bool parked = false;
+        if constexpr (NX > 0) {
+          const uint32_t slot = (v0 - static_cast<uint32_t>(NL) * TB) / TB + b;
+          parked = slot < static_cast<uint32_t>(NX);
+          if (parked) xo[b] = __builtin_bit_cast(RawVec<T, VEC>, extra[slot * TB + t]);
+        }
+        if (!parked) xo[b] = load_raw<T, VEC>(x + off[b]);
         d[b] = load_raw<T, VEC>(dy + off[b]);
       }
 #pragma unroll

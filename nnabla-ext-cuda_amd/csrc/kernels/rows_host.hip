@@ -438,7 +438,8 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
     const int full = p.dtype == NBLAHIP_F16 ? 8 : 4;
     const RowCfg loose = pick_ln_bwd_cfg(p.dtype, (p.R + full - 1) / full * full, full);
     if (loose.ok && loose.tpr == 64) {
-      const int grid = ln_bwd_grid(p.rows, loose.tpr);
+      // (four vectors per lane: 139 - 218 registers, one 512-thread block per CU)
+      const int grid = ln_bwd_grid(p.rows, loose.tpr, loose.nl >= 4 ? 1 : 2);
       if (int e = ln_loose_bwd(p, a, loose, grid, st)) return e;
       if (p.dgamma || p.dbeta) {
         NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 15) / 16), dim3(1024), 0, st,

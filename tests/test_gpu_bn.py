@@ -332,15 +332,18 @@ def test_bn_argument_errors():
 # every CU and 8193 to 25600 vectors per channel.  N picks the vectors per
 # thread (9 to 25), hence the register/LDS layout; odd N leaves the last slot
 # partly filled.  Backward layouts that hold the whole channel end at 20480
-# vectors (the last one with 512 threads per block); beyond, 18432 are held
-# and the rest is streamed.
+# vectors (the last one with 512 threads per block); beyond, 18432 are held,
+# the next 3072 parked in LDS by the first pass, and the rest is streamed.
 ONCHIP_CASES = [(torch.float32, 33), (torch.float32, 47), (torch.float32, 55), (torch.float32, 63),
                 (torch.float32, 71), (torch.float32, 77), (torch.float32, 85), (torch.float32, 99),
                 (torch.float16, 67), (torch.float16, 111), (torch.float16, 141),
                 (torch.float16, 155), (torch.float16, 197),
                 # longer than the chip holds: 25600 (forward) / 18432 (backward) vectors
                 # stay, the rest is streamed
-                (torch.float32, 131), (torch.float16, 301)]
+                (torch.float32, 131), (torch.float16, 301),
+                # ... with a remainder short enough for the LDS the held slots leave
+                # free (3072 vectors, parked during the backward's first pass)
+                (torch.float32, 83), (torch.float16, 165), (torch.float32, 84)]
 
 
 @pytest.mark.parametrize("dtype,n", ONCHIP_CASES)
