@@ -126,6 +126,10 @@ unsigned grid_of(const GnClArgs &a) {
   GN_CL_CASES_TPR(CASE, T, VEC, 256) GN_CL_CASES_TPR(CASE, T, VEC, 512) GN_CL_CASES_TPR(CASE, T, VEC, 1024)
 // ... and one wave per unit (small planes or groups).
 #define IN_CL_CASES(CASE, T, VEC) GN_CL_CASES_TPR(CASE, T, VEC, 64) GN_CL_CASES(CASE, T, VEC)
+// The backwards take groups / planes of up to 2048 vectors (pick_cfg,
+// pick_in_cfg), which the wave and the 256-thread layouts hold: the larger
+// blocks are never picked.
+#define CL_CASES_BWD(CASE, T, VEC) GN_CL_CASES_TPR(CASE, T, VEC, 64) GN_CL_CASES_TPR(CASE, T, VEC, 256)
 
 #define FWD_CASE(T, VEC, NL, TPR)                                                              \
   if (c.nl == (NL) && c.tpr == (TPR)) {                                                        \
@@ -164,9 +168,9 @@ int run_in_fwd(int dtype, const GnClCfg &c, const GnClArgs &a, hipStream_t st) {
 
 int run_in_bwd(int dtype, const GnClCfg &c, const GnClArgs &a, hipStream_t st) {
   if (dtype == NBLAHIP_F16) {
-    IN_CL_CASES(IN_BWD_CASE, __half, 8)
+    CL_CASES_BWD(IN_BWD_CASE, __half, 8)
   } else {
-    IN_CL_CASES(IN_BWD_CASE, float, 4)
+    CL_CASES_BWD(IN_BWD_CASE, float, 4)
   }
   return NBLAHIP_EINVAL;
 }
@@ -182,9 +186,9 @@ int run_fwd(int dtype, const GnClCfg &c, const GnClArgs &a, hipStream_t st) {
 
 int run_bwd(int dtype, const GnClCfg &c, const GnClArgs &a, hipStream_t st) {
   if (dtype == NBLAHIP_F16) {
-    IN_CL_CASES(BWD_CASE, __half, 8)
+    CL_CASES_BWD(BWD_CASE, __half, 8)
   } else {
-    IN_CL_CASES(BWD_CASE, float, 4)
+    CL_CASES_BWD(BWD_CASE, float, 4)
   }
   return NBLAHIP_EINVAL;
 }

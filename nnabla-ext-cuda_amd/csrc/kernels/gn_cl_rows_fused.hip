@@ -10,6 +10,10 @@ namespace nblahip {
   FUSED_CASES_TPR(CASE, T, VEC, 64) FUSED_CASES_TPR(CASE, T, VEC, 256)   \
   FUSED_CASES_TPR(CASE, T, VEC, 512) FUSED_CASES_TPR(CASE, T, VEC, 1024)
 
+// The backward takes planes of up to 2048 positions (pick_in_cfg), which the
+// wave and the 256-thread layouts hold: the larger blocks are never picked.
+#define FUSED_CASES_BWD(CASE, T, VEC) FUSED_CASES_TPR(CASE, T, VEC, 64) FUSED_CASES_TPR(CASE, T, VEC, 256)
+
 #define FWD_CASE(T, VEC, NL, TPR)                                                                \
   if (nl == (NL) && tpr == (TPR)) {                                                              \
     if (fuse == 2) {                                                                             \
@@ -40,9 +44,9 @@ int run_in_fwd_fused(int dtype, int tpr, int nl, const GnClArgs &a, unsigned gri
 
 int run_in_bwd_fused(int dtype, int tpr, int nl, const GnClArgs &a, unsigned grid, hipStream_t st) {
   if (dtype == NBLAHIP_F16) {
-    FUSED_CASES(BWD_CASE, __half, 8)
+    FUSED_CASES_BWD(BWD_CASE, __half, 8)
   } else {
-    FUSED_CASES(BWD_CASE, float, 4)
+    FUSED_CASES_BWD(BWD_CASE, float, 4)
   }
   return NBLAHIP_EINVAL;
 }

@@ -8,6 +8,26 @@
 
 namespace nblahip {
 
+// The layouts pick_ln_bwd_cfg hands out (rows_host.hip), and no others: up to
+// four vectors per thread (the per-column accumulators make every load cost
+// about 27 registers: eight of them spill 600 - 1200 bytes per lane), one per
+// thread at 1024 threads - two for float.
+#define LN_CASES_TPR(CASE, T, VEC, TPR) CASE(T, VEC, 1, TPR) CASE(T, VEC, 2, TPR) CASE(T, VEC, 4, TPR)
+#define LN_CASES_VEC(CASE, T, VEC)                                                     \
+  NBLAHIP_ROW_CASES_SUBWAVE(CASE, T, VEC)                                              \
+  LN_CASES_TPR(CASE, T, VEC, 64)                                                       \
+  LN_CASES_TPR(CASE, T, VEC, 256)                                                      \
+  LN_CASES_TPR(CASE, T, VEC, 512)                                                      \
+  CASE(T, VEC, 1, 1024)
+#define LN_CASES(CASE, T)                                                              \
+  LN_CASES_VEC(CASE, T, FullVec<T>::value)                                             \
+  LN_CASES_VEC(CASE, T, MidVec<T>::value)                                              \
+  LN_CASES_VEC(CASE, T, 1)                                                             \
+  if constexpr (sizeof(T) == 4) {                                                      \
+    CASE(T, FullVec<T>::value, 2, 1024)                                                \
+    CASE(T, 1, 2, 1024)                                                                \
+  }
+
 #define BWD_CASE(T, VEC, NL, TPR)                                                      \
   if (cfg.vec == (VEC) && cfg.nl == (NL) && cfg.tpr == (TPR)) {                        \
     NBLAHIP_LAUNCH("row_bwd_kernel_ln", (row_bwd_kernel<T, VEC, NL, TPR, kRowLN>), dim3(grid),           \
@@ -17,7 +37,7 @@ namespace nblahip {
 
 template <typename T>
 static int run_bwd_t(const RowCfg &cfg, const RowArgs &args, int grid, hipStream_t st) {
-  NBLAHIP_ROW_CASES(BWD_CASE, T)
+  LN_CASES(BWD_CASE, T)
   return NBLAHIP_EINVAL;
 }
 
@@ -35,7 +55,7 @@ static int run_bwd_t(const RowCfg &cfg, const RowArgs &args, int grid, hipStream
   }
 
 template <typename T> static int occupancy_t(const RowCfg &cfg) {
-  NBLAHIP_ROW_CASES(OCC_CASE, T)
+  LN_CASES(OCC_CASE, T)
   return 0;
 }
 

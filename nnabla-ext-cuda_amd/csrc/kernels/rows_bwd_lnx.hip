@@ -11,9 +11,19 @@ namespace nblahip {
     return last_launch_status();                                                       \
   }
 
+// This mode takes the rows beyond the layouts of the plain LayerNormalization
+// backward (more than 2048 vectors), for which pick_row_cfg (rows_host.hip:
+// eight vectors per thread below 1024 threads, four - scalar rows: eight - at
+// 1024) has these layouts left.
 template <typename T>
 static int run_bwd_t(const RowCfg &cfg, const RowArgs &args, int grid, hipStream_t st) {
-  NBLAHIP_ROW_CASES_BLOCK(BWD_CASE, T)
+  BWD_CASE(T, FullVec<T>::value, 8, 512)
+  BWD_CASE(T, MidVec<T>::value, 8, 512)
+  BWD_CASE(T, 1, 8, 512)
+  BWD_CASE(T, FullVec<T>::value, 4, 1024)
+  BWD_CASE(T, MidVec<T>::value, 4, 1024)
+  BWD_CASE(T, 1, 4, 1024)
+  BWD_CASE(T, 1, 8, 1024)
   return NBLAHIP_EINVAL;
 }
 
