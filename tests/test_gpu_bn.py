@@ -434,9 +434,13 @@ def test_bn_training_forward_in_place(shape, axis, dtype):
 @pytest.mark.parametrize("m,c,dtype", [(100352, 64, torch.float16), (100353, 64, torch.float16),
                                        (200000, 32, torch.float32), (150000, 128, torch.float16),
                                        (1000001, 8, torch.float16), (40000, 128, torch.float32),
-                                       # 256 and 512 channels: a block merges one or two channels
+                                       # more than 128 channels: column strips, a block merges several channels
                                        (40000, 256, torch.float16), (50000, 512, torch.float16),
-                                       (40000, 256, torch.float32)])
+                                       (40000, 256, torch.float32),
+                                       # 8 and 16 strips; 3 strips of 64 channels (255 blocks); strips of 32 channels
+                                       (20001, 1024, torch.float16), (9000, 2048, torch.float32),
+                                       (40000, 192, torch.float16), (37000, 96, torch.float32),
+                                       (12345, 4096, torch.float16)])
 def test_bn_channel_last_held_on_the_chip(m, c, dtype):
     """Against the oracle; bit-identical when no poll is allowed (every block
     then computes the partials and channel results it needs itself); close to
@@ -485,9 +489,14 @@ def test_bn_channel_last_held_on_the_chip(m, c, dtype):
                                        (1000001, 8, torch.float16), (40000, 128, torch.float32),
                                        # more of x than a block holds: the rest is read again
                                        (750000, 64, torch.float16), (380000, 64, torch.float32),
-                                       # 256 and 512 channels; more than the 18 vectors held with them
+                                       # 256 and 512 channels (column strips); more than the 21 vectors held
                                        (40000, 256, torch.float16), (50000, 512, torch.float16),
-                                       (40000, 256, torch.float32), (170000, 256, torch.float16)])
+                                       (40000, 256, torch.float32), (170000, 256, torch.float16),
+                                       # column strips: 8 and 16 of them; 3 of 64 channels; of 32 channels;
+                                       # 32 of them; more of x than the blocks of a strip hold
+                                       (20001, 1024, torch.float16), (9000, 2048, torch.float32),
+                                       (40000, 192, torch.float16), (37000, 96, torch.float32),
+                                       (12345, 4096, torch.float16), (46000, 1024, torch.float16)])
 def test_bn_channel_last_backward_held_on_the_chip(m, c, dtype):
     """Backward with x held on the chip and the (sum dy*xh, sum dy) pairs
     exchanged: against the oracle with the 3-output terms, bit-identical when no

@@ -187,8 +187,16 @@ SWITCHES = [
      ["bn_apply_planes_kernel"], ["bn_masked_fwd_kernel", "bn_masked_bwd_kernel"]),
     ("bn_cl_grid_wide_off", run_bn, ((256, 14, 14, 256), 3, F16), {"BN_CL_GRID_WIDE": 0},
      ["cl_split_fwd_kernel", "bn_bwd_reduce_cl_kernel"], ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"]),
-    ("bn_cl_grid_wide_from_more_rows", run_bn, ((256, 14, 14, 256), 3, F32), {"BN_CL_GRID_WIDE_MIN_ROWS": 60000},
+    ("bn_cl_grid_wide_from_more_rows", run_bn, ((256, 14, 14, 256), 3, F32), {"BN_CL_GRID_WIDE_MIN_ROWS": 60000, "BN_CL_GRID_WIDE_MIN_KB": 1000000},
      ["bn_stats_cl_kernel", "bn_bwd_reduce_cl_kernel"], ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"]),
+    ("bn_cl_grid_strips_off", run_bn, ((128, 14, 14, 1024), 3, F16), {"BN_CL_GRID_STRIPS": 0},
+     ["bn_stats_cl_kernel", "bn_bwd_reduce_cl_kernel"], ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"]),
+    ("bn_cl_grid_strips_of_8_vectors", run_bn, ((256, 14, 14, 768), 3, F16), {"BN_CL_GRID_STRIP_VECS": 8},
+     ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"], []),
+    ("bn_cl_grid_strips_no_narrower_than", run_bn, ((256, 28, 28, 192), 3, F16), {"BN_CL_GRID_STRIP_MIN_VECS": 16},
+     ["bn_stats_cl_kernel", "bn_bwd_reduce_cl_kernel"], ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"]),
+    ("bn_cl_grid_wide_from_more_bytes", run_bn, ((64, 14, 14, 1024), 3, F32), {"BN_CL_GRID_WIDE_MIN_KB": 1000000},
+     ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"]),
     ("bn_cl_grid_bwd_off", run_bn, ((100352, 64), 1, F16), {"BN_CL_GRID_BWD": 0},
      ["bn_cl_grid_fwd_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
      ["bn_cl_grid_bwd_kernel"], {"BN_CL_GRID_MIN_SLOTS": 1}),

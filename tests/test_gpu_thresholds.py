@@ -130,10 +130,15 @@ CASES = [
      [("below", ((6272, 64), 1, F16), {"BN_CL_GRID_MIN_ROWS": 1}, "cl_split_fwd_kernel", "bn_cl_grid_fwd_kernel"),
       ("above", ((12544, 64), 1, F16), {"BN_CL_GRID_MIN_ROWS": 999999}, "bn_cl_grid_fwd_kernel", "cl_split_fwd_kernel"),
       ("above_f32", ((12544, 128), 1, F32), {"BN_CL_GRID_MIN_ROWS": 999999}, "bn_cl_grid_fwd_kernel", "cl_split_fwd_kernel")]),
-    # ... with 129 - 512 channels: from 36865 rows
+    # ... with more than 128 channels: from 36865 rows
     ("bn_cl_grid_wide_min_rows", P.run_bn, {},
      [("below", ((128, 16, 16, 256), 3, F16), {"BN_CL_GRID_WIDE_MIN_ROWS": 1}, None, "bn_cl_grid_fwd_kernel"),
       ("above", ((256, 14, 14, 256), 3, F16), {"BN_CL_GRID_WIDE_MIN_ROWS": 999999}, "bn_cl_grid_fwd_kernel", None)]),
+    # ... or from 32 MiB
+    ("bn_cl_grid_wide_min_kb", P.run_bn, {},
+     [("below", ((128, 7, 7, 2048), 3, F16), {"BN_CL_GRID_WIDE_MIN_KB": 1}, "cl_split_fwd_kernel", "bn_cl_grid_fwd_kernel"),
+      ("above", ((64, 14, 14, 1024), 3, F32), {"BN_CL_GRID_WIDE_MIN_KB": 1000000}, "bn_cl_grid_fwd_kernel",
+       "cl_split_fwd_kernel")]),
     # short planes that share cache lines: ordinary stores inside the shared lines up to 1 KB
     ("bn_edge_stores_max_bytes", P.run_bn, NCS,
      [("below", ((256, 256, 14, 14), 1, F16), {"BN_EDGE_STORES_MAX_BYTES": 0}, "bn_onchip_fwd_kernel", "bn_onchip_fwd_kernel"),
