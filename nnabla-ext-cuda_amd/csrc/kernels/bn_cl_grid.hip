@@ -76,6 +76,7 @@ struct BnClGridArgs {
   uint32_t kstep;   // vectors between a thread's consecutive slots = (1024 / cv) * ld
   uint32_t lp;      // stage 2: 2^lp threads per channel, one per block of the strip (2^lp >= ranges)
   uint32_t gu;      // stage 2: channels per block (gu << lp <= 1024)
+  uint32_t hv;      // forward: vectors of a block that its threads hold (the rest is streamed), a multiple of 1024
   float inv_N, unbias, decay, eps, one;
   // backward
   const void *dy;
@@ -185,10 +186,11 @@ __device__ __forceinline__ void grid_partial_from_memory(const BnClGridArgs &a, 
   const uint32_t vbb = grid_range_rows(a, r) << a.cvsh;
   const bool mine = cvx == cl / VEC;
   const uint32_t vbp = mine ? vbb : 0u;
+  const uint32_t vbh = min(vbb, a.hv); // the vectors that block holds: its threads' shifts are their means
   const uint32_t tb = grid_offset(a, t);
   float sx = 0.f, s1 = 0.f, s2 = 0.f;
 #pragma unroll 1
-  for (uint32_t v = t, off = tb; v < vbp; v += kOnchipBlock, off += a.kstep) {
+  for (uint32_t v = t, off = tb; v < min(vbp, vbh); v += kOnchipBlock, off += a.kstep) {
     const RawVec<T, VEC> rr = load_raw<T, VEC>(x + static_cast<size_t>(off) * VEC);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
@@ -196,8 +198,9 @@ __device__ __forceinline__ void grid_partial_from_memory(const BnClGridArgs &a, 
       sx = static_cast<uint32_t>(j) == e ? n : sx;
     }
   }
+  const float nh = (mine && t < vbh) ? static_cast<float>((vbh - 1u - t) / kOnchipBlock + 1u) : 0.f;
   const float nt = (mine && t < vbb) ? static_cast<float>((vbb - 1u - t) / kOnchipBlock + 1u) : 0.f;
-  const float kk = sx * (1.0f / fmaxf(nt, 1.f));
+  const float kk = sx * (1.0f / fmaxf(nh, 1.f));
 #pragma unroll 1
   for (uint32_t v = t, off = tb; v < vbp; v += kOnchipBlock, off += a.kstep) {
     const RawVec<T, VEC> rr = load_raw<T, VEC>(x + static_cast<size_t>(off) * VEC);
@@ -210,7 +213,7 @@ __device__ __forceinline__ void grid_partial_from_memory(const BnClGridArgs &a, 
       s2 = static_cast<uint32_t>(j) == e ? n2 : s2;
     }
   }
-  m = grid_channel_sum1(sx, a.cv, cl, mine, fold, a.cs);
+  m = grid_channel_sum1(fmaf(nt, kk, s1), a.cv, cl, mine, fold, a.cs);
   m *= 1.0f / static_cast<float>(vbb >> a.cvsh);
   const float d = kk - m;
   q = grid_channel_sum1(mine ? fmaf(d, fmaf(nt, d, 2.f * s1), s2) : 0.f, a.cv, cl, mine, fold, a.cs);
@@ -332,7 +335,9 @@ __device__ __forceinline__ void grid_pair_result(const BnClGridArgs &a, uint32_t
 
 } // namespace
 
-template <typename T, int VEC, int NR, int NS>
+// OVER: the block has more vectors than the NR + NS its threads hold; the rest
+// is read for the statistics and again for the normalization.
+template <typename T, int VEC, int NR, int NS, bool OVER>
 __global__ void __launch_bounds__(kOnchipBlock)
 bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
   static_assert(sizeof(RawVec<T, VEC>) == 16, "16-byte vectors");
@@ -409,6 +414,9 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
   // m2 = sum_t (s2 + 2 e s1 + n e^2), e = K - mean: two block sums of a few
   // operations per thread.  sum_t n e^2 is the variance between the threads'
   // means, never more than m2 itself: nothing cancels, whatever the data.
+  // (The thread's sum enters the mean as n K + s1.  What a block streams, OVER,
+  // is taken about the K of the vectors held: K is then not the thread's mean
+  // but close to it, s1 no longer a residue, and the same formulas hold.)
   float m[VEC], q[VEC];
   {
     float kk[VEC], s1[VEC], s2[VEC];
@@ -422,8 +430,10 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
         for (int j = 0; j < VEC; ++j) m[j] = elem_fma<T, VEC>(r, j, a.one, m[j]);
       }
     }
+    const uint32_t vbh = OVER ? min(vbb, static_cast<uint32_t>(NL) * kOnchipBlock) : vbb;
+    const float nh = t < vbh ? static_cast<float>((vbh - 1u - t) / kOnchipBlock + 1u) : 0.f;
     const float nt = t < vbb ? static_cast<float>((vbb - 1u - t) / kOnchipBlock + 1u) : 0.f;
-    const float rnt = 1.0f / fmaxf(nt, 1.f);
+    const float rnt = 1.0f / fmaxf(nh, 1.f);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) kk[j] = m[j] * rnt;
 #pragma unroll
@@ -438,6 +448,30 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
         }
       }
     }
+    if constexpr (OVER) { // two vectors in flight
+#pragma unroll 1
+      for (uint32_t o = tb + static_cast<uint32_t>(NL) * a.kstep; o <= last; o += 2 * a.kstep) {
+        const uint32_t o1 = o + a.kstep;
+        const RawVec<T, VEC> r0 = load_raw<T, VEC>(x + static_cast<size_t>(o) * VEC);
+        const RawVec<T, VEC> r1 = load_raw<T, VEC>(x + static_cast<size_t>(min(o1, last)) * VEC);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+          const float d = elem_fma<T, VEC>(r0, j, a.one, -kk[j]);
+          s1[j] += d;
+          s2[j] = fmaf(d, d, s2[j]);
+        }
+        if (o1 <= last) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) {
+            const float d = elem_fma<T, VEC>(r1, j, a.one, -kk[j]);
+            s1[j] += d;
+            s2[j] = fmaf(d, d, s2[j]);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) m[j] = fmaf(nt, kk[j], s1[j]);
     grid_channel_sums<VEC>(m, a.cv, cvx, fold, tot, a.cs);
     const float icnt = 1.0f / static_cast<float>(vbb >> a.cvsh);
 #pragma unroll
@@ -535,6 +569,28 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
         }
       }
       store_vec<T, VEC>(y + static_cast<size_t>(o) * VEC, ov);
+    }
+  }
+  if constexpr (OVER) {
+    auto emit = [&](const RawVec<T, VEC> &r, uint32_t o) {
+      float ov[VEC];
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        if constexpr (sizeof(T) == 2) {
+          ov[j] = elem_fma<T, VEC>(r, j, sc[j], sh[j]);
+        } else {
+          ov[j] = fmaf(elem_fma<T, VEC>(r, j, a.one, -mu[j]), sc[j], be[j]);
+        }
+      }
+      store_vec<T, VEC>(y + static_cast<size_t>(o) * VEC, ov);
+    };
+#pragma unroll 1
+    for (uint32_t o = tb2 + static_cast<uint32_t>(NL) * a.kstep; o <= last; o += 2 * a.kstep) {
+      const uint32_t o1 = o + a.kstep;
+      const RawVec<T, VEC> r0 = load_raw<T, VEC>(x + static_cast<size_t>(o) * VEC);
+      const RawVec<T, VEC> r1 = load_raw<T, VEC>(x + static_cast<size_t>(min(o1, last)) * VEC);
+      emit(r0, o);
+      if (o1 <= last) emit(r1, o1);
     }
   }
 }
@@ -650,16 +706,28 @@ bn_cl_grid_bwd_kernel(const BnClGridArgs a) {
     }
     __builtin_amdgcn_sched_barrier(0); // the next batch's loads stay below: hoisted, the batches add up
   }
+  // (what the block does not hold: x and dy streamed, two vectors of each in flight)
 #pragma unroll 1
   for (uint32_t o = grid_offset(a, fresh_after(t, sdx[0])) + static_cast<uint32_t>(NL) * a.kstep; o <= last;
-       o += a.kstep) {
-    const RawVec<T, VEC> xr = load_raw<T, VEC>(x + static_cast<size_t>(o) * VEC);
-    const RawVec<T, VEC> dr = load_raw<T, VEC>(dy + static_cast<size_t>(o) * VEC);
+       o += 2 * a.kstep) {
+    const uint32_t o1 = o + a.kstep;
+    const RawVec<T, VEC> xr0 = load_raw<T, VEC>(x + static_cast<size_t>(o) * VEC);
+    const RawVec<T, VEC> dr0 = load_raw<T, VEC>(dy + static_cast<size_t>(o) * VEC);
+    const RawVec<T, VEC> xr1 = load_raw<T, VEC>(x + static_cast<size_t>(min(o1, last)) * VEC);
+    const RawVec<T, VEC> dr1 = load_raw<T, VEC>(dy + static_cast<size_t>(min(o1, last)) * VEC);
 #pragma unroll
     for (int j = 0; j < VEC; ++j) {
-      const float xh = norm_elem<T, VEC>(xr, j, mean[j], istd[j], nmi[j]);
-      sdx[j] = elem_fma<T, VEC>(dr, j, xh, sdx[j]);
-      sdy[j] = elem_fma<T, VEC>(dr, j, a.one, sdy[j]);
+      const float xh = norm_elem<T, VEC>(xr0, j, mean[j], istd[j], nmi[j]);
+      sdx[j] = elem_fma<T, VEC>(dr0, j, xh, sdx[j]);
+      sdy[j] = elem_fma<T, VEC>(dr0, j, a.one, sdy[j]);
+    }
+    if (o1 <= last) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float xh = norm_elem<T, VEC>(xr1, j, mean[j], istd[j], nmi[j]);
+        sdx[j] = elem_fma<T, VEC>(dr1, j, xh, sdx[j]);
+        sdy[j] = elem_fma<T, VEC>(dr1, j, a.one, sdy[j]);
+      }
     }
   }
   grid_channel_sums<VEC>(sdx, a.cv, cvx, fold, tot, a.cs);
@@ -784,10 +852,14 @@ bn_cl_grid_bwd_kernel(const BnClGridArgs a) {
   }
 #pragma unroll 1
   for (uint32_t o = grid_offset(a, fresh_after(t, lastv)) + static_cast<uint32_t>(NL) * a.kstep; o <= last;
-       o += a.kstep) {
-    const RawVec<T, VEC> xr = load_raw<T, VEC>(x + static_cast<size_t>(o) * VEC);
-    const RawVec<T, VEC> dr = load_raw<T, VEC>(dy + static_cast<size_t>(o) * VEC);
-    emit(xr, dr, o);
+       o += 2 * a.kstep) {
+    const uint32_t o1 = o + a.kstep;
+    const RawVec<T, VEC> xr0 = load_raw<T, VEC>(x + static_cast<size_t>(o) * VEC);
+    const RawVec<T, VEC> dr0 = load_raw<T, VEC>(dy + static_cast<size_t>(o) * VEC);
+    const RawVec<T, VEC> xr1 = load_raw<T, VEC>(x + static_cast<size_t>(min(o1, last)) * VEC);
+    const RawVec<T, VEC> dr1 = load_raw<T, VEC>(dy + static_cast<size_t>(min(o1, last)) * VEC);
+    emit(xr0, dr0, o);
+    if (o1 <= last) emit(xr1, dr1, o1);
   }
 }
 
@@ -797,7 +869,7 @@ template <typename T, int VEC>
 int run_grid_fwd(int nl, const BnClGridArgs &a, hipStream_t st) {
 #define GRID_CASE(NR, NS)                                                                        \
   if (nl <= (NR) + (NS)) {                                                                       \
-    NBLAHIP_LAUNCH("bn_cl_grid_fwd_kernel", (bn_cl_grid_fwd_kernel<T, VEC, NR, NS>),             \
+    NBLAHIP_LAUNCH("bn_cl_grid_fwd_kernel", (bn_cl_grid_fwd_kernel<T, VEC, NR, NS, false>),      \
                    dim3(a.nblocks), dim3(kOnchipBlock), 0, st, a);                               \
     return last_launch_status();                                                                 \
   }
@@ -809,7 +881,10 @@ int run_grid_fwd(int nl, const BnClGridArgs &a, hipStream_t st) {
   GRID_CASE(16, 6)
   GRID_CASE(16, 9)
 #undef GRID_CASE
-  return NBLAHIP_EINVAL;
+  // (more per thread than the 25 vectors held: the rest is read twice)
+  NBLAHIP_LAUNCH("bn_cl_grid_fwd_kernel", (bn_cl_grid_fwd_kernel<T, VEC, 16, 9, true>), dim3(a.nblocks),
+                 dim3(kOnchipBlock), 0, st, a);
+  return last_launch_status();
 }
 
 template <typename T, int VEC>
@@ -857,7 +932,8 @@ bool grid_args(const BnProblem &p, BnClGridArgs &a, int &nl) {
 
   // Column strips: the widest power of two of vectors that divides a row, up
   // to 128 channels.  One strip: the block's rows are contiguous memory.
-  const int blocks = std::min(device_cus(), kGridMaxBlocks);
+  // (fewer blocks than CUs: for tests of the streamed remainder on small tensors)
+  const int blocks = std::max(8, std::min({device_cus(), kGridMaxBlocks, tune_int("BN_CL_GRID_BLOCKS", kGridMaxBlocks)}));
   int64_t cv = std::min<int64_t>(ld & -ld, kGridMaxC / vec);
   for (const int64_t cap = tune_int("BN_CL_GRID_STRIP_VECS", kWave); cv > cap && cv > 1;) cv >>= 1;
   const int64_t strips = ld / cv;
@@ -893,7 +969,7 @@ bool grid_args(const BnProblem &p, BnClGridArgs &a, int &nl) {
       return false;
   }
   const int64_t nblocks = ranges * strips;
-  if (nl < tune_int("BN_CL_GRID_MIN_SLOTS", 1) || nl > kGridMaxSlots || nblocks < blocks / 2) return false;
+  if (nl < tune_int("BN_CL_GRID_MIN_SLOTS", 1) || nblocks < blocks / 2) return false;
   const int lp = log2_of(static_cast<uint32_t>(ranges));
   const int64_t gu = (p.C + nblocks - 1) / nblocks;
   if ((gu << lp) > kOnchipBlock) return false;
@@ -940,6 +1016,12 @@ bool bn_cl_grid_fwd_train(const BnProblem &p, hipStream_t st, int *status) {
   BnClGridArgs a;
   int nl = 0;
   if (!p.out || !grid_args(p, a, nl)) return false;
+  // More than the 25 vectors per thread held: the rest is read twice, 2 S for
+  // what is held and 3 S for the rest in one launch against 3 S in three
+  // ([256,28,28,384] half, 154 MB, 37 vectors: 92.4 -> 67.9 us; 205 MB: 113.7 ->
+  // 93.6; 308 MB, 74 vectors: 166.2 -> 150.3; 411 MB, 98 vectors: 223.4 -> 220.9).
+  if (nl > tune_int("BN_CL_GRID_FWD_MAX_SLOTS", 80)) return false;
+  a.hv = nl > kGridMaxSlots ? static_cast<uint32_t>(kGridMaxSlots) * kOnchipBlock : ~0u;
   a.y = p.out;
   a.beta = p.beta;
   a.mean = p.batch_mean;
@@ -955,7 +1037,11 @@ bool bn_cl_grid_bwd(const BnProblem &p, hipStream_t st, int *status) {
   BnClGridArgs a;
   int nl = 0;
   if (!p.batch_stat || !tune_int("BN_CL_GRID_BWD", 1) || !grid_args(p, a, nl)) return false;
-  if (!aligned16(p.dy)) return false;
+  // Beyond the 21 vectors per thread a block holds, x is read twice like dy: 4 S
+  // for what is held and 5 S for the rest in one launch against 5 S in three
+  // ([256,28,28,384] half, 154 MB: 138.7 -> 116.9 us; 205 MB half 182.5 ->
+  // 179.6, float 189.7 -> 166.4; 257 MB, 62 vectors: 220.4 -> 227.6).
+  if (!aligned16(p.dy) || nl > tune_int("BN_CL_GRID_BWD_MAX_SLOTS", 50)) return false;
   a.dy = p.dy;
   a.dx = p.out;
   a.mean = const_cast<float *>(p.mean);

@@ -445,6 +445,20 @@ def test_bn_channel_last_held_on_the_chip(m, c, dtype):
     """Against the oracle; bit-identical when no poll is allowed (every block
     then computes the partials and channel results it needs itself); close to
     the split reduction; running statistics updated once."""
+    _held_forward(m, c, dtype, {})
+
+
+# Fewer blocks than CUs, so that a small tensor is more than the blocks hold:
+# 47 and 59 vectors per thread (25 held), with one strip, with three, in float.
+@pytest.mark.parametrize("m,c,dtype,blocks", [(48000, 128, torch.float16, 16), (24001, 384, torch.float16, 24),
+                                              (40000, 64, torch.float32, 16), (60000, 128, torch.float16, 16)])
+def test_bn_channel_last_more_than_the_chip_holds(m, c, dtype, blocks):
+    """What the blocks do not hold is read for the statistics and again for
+    the normalization; same checks as with everything held."""
+    _held_forward(m, c, dtype, {"BN_CL_GRID_BLOCKS": blocks, "BN_CL_GRID_WIDE_MIN_KB": 1})
+
+
+def _held_forward(m, c, dtype, extra):
     dn = dtype_name(dtype)
     x, _, g, b, rm, rv = make_bn((m, c), 1, dtype, 5, mean=1.0, std=2.0)
     y_r, m_r, v_r, rm_r, rv_r = R.bn_forward_batch(x, b, g, rm, rv, 1, 0.9, 1e-5)
@@ -464,9 +478,9 @@ def test_bn_channel_last_held_on_the_chip(m, c, dtype):
         return [y, mean, var, rmd, rvd], names
 
     try:
-        held, names = run({"BN_CL_GRID_MIN_SLOTS": 1})
+        held, names = run({**extra, "BN_CL_GRID_MIN_SLOTS": 1})
         assert names == ["bn_cl_grid_fwd_kernel"], names
-        alone, names = run({"BN_CL_GRID_MIN_SLOTS": 1, "XCHG_SPIN": 0})
+        alone, names = run({**extra, "BN_CL_GRID_MIN_SLOTS": 1, "XCHG_SPIN": 0})
         assert names == ["bn_cl_grid_fwd_kernel"], names
         split, names = run({"BN_CL_GRID": 0})
         assert "bn_cl_grid_fwd_kernel" not in names
@@ -502,6 +516,17 @@ def test_bn_channel_last_backward_held_on_the_chip(m, c, dtype):
     exchanged: against the oracle with the 3-output terms, bit-identical when no
     poll is allowed, close to the split reduction; accumulation and the
     parameters-only call."""
+    _held_backward(m, c, dtype, {})
+
+
+@pytest.mark.parametrize("m,c,dtype,blocks", [(48000, 128, torch.float16, 16), (24001, 384, torch.float16, 24),
+                                              (40000, 64, torch.float32, 16)])
+def test_bn_channel_last_backward_more_than_the_chip_holds(m, c, dtype, blocks):
+    """40 and 47 vectors per thread, 21 of x held: the rest streamed two at a time."""
+    _held_backward(m, c, dtype, {"BN_CL_GRID_BLOCKS": blocks, "BN_CL_GRID_WIDE_MIN_KB": 1})
+
+
+def _held_backward(m, c, dtype, extra):
     dn = dtype_name(dtype)
     x, dy, g, b, _, _ = make_bn((m, c), 1, dtype, 6, mean=1.0, std=2.0)
     rng = np.random.default_rng(7)
@@ -526,16 +551,16 @@ def test_bn_channel_last_backward_held_on_the_chip(m, c, dtype):
         return out, names
 
     try:
-        held, names = run({"BN_CL_GRID_MIN_SLOTS": 1})
+        held, names = run({**extra, "BN_CL_GRID_MIN_SLOTS": 1})
         assert names == ["bn_cl_grid_bwd_kernel"], names
-        alone, names = run({"BN_CL_GRID_MIN_SLOTS": 1, "XCHG_SPIN": 0})
+        alone, names = run({**extra, "BN_CL_GRID_MIN_SLOTS": 1, "XCHG_SPIN": 0})
         assert names == ["bn_cl_grid_bwd_kernel"], names
         split, names = run({"BN_CL_GRID_BWD": 0, "BN_CL_GRID_MIN_SLOTS": 1})
         assert "bn_cl_grid_bwd_kernel" not in names
-        acc, names = run({"BN_CL_GRID_MIN_SLOTS": 1}, dx=to_dev(pre_dx, dtype), dgamma=to_dev(pre_g),
+        acc, names = run({**extra, "BN_CL_GRID_MIN_SLOTS": 1}, dx=to_dev(pre_dx, dtype), dgamma=to_dev(pre_g),
                          dbeta=to_dev(pre_b), accum=(True, True, True))
         assert names == ["bn_cl_grid_bwd_kernel"], names
-        params, names = run({"BN_CL_GRID_MIN_SLOTS": 1}, need=(False, True, True))
+        params, names = run({**extra, "BN_CL_GRID_MIN_SLOTS": 1}, need=(False, True, True))
         assert names == ["bn_cl_grid_bwd_kernel"], names
     finally:
         K.tune_reset()
@@ -562,6 +587,9 @@ def test_bn_channel_last_backward_held_on_the_chip(m, c, dtype):
     ((32, 64, 56, 56), 1, torch.float16, "bn_chan_split_fwd_kernel", {}),
     ((150000, 64), 1, torch.float32, "bn_cl_grid_fwd_kernel", {"BN_CL_GRID_MIN_SLOTS": 1}),
     ((150000, 64), 1, torch.float16, "bn_cl_grid_fwd_kernel", {"BN_CL_GRID_MIN_SLOTS": 1}),
+    # (more than the blocks hold: the streamed part is taken about the mean of the part held)
+    ((48000, 128), 1, torch.float16, "bn_cl_grid_fwd_kernel", {"BN_CL_GRID_MIN_SLOTS": 1, "BN_CL_GRID_BLOCKS": 16}),
+    ((40000, 64), 1, torch.float32, "bn_cl_grid_fwd_kernel", {"BN_CL_GRID_MIN_SLOTS": 1, "BN_CL_GRID_BLOCKS": 16}),
     ((200, 256, 7, 7), 1, torch.float32, "bn_pack_fwd_kernel", {}),
     ((200, 256, 7, 7), 1, torch.float16, "bn_pack_fwd_kernel", {}),
     ((12000, 128), 1, torch.float16, "cl_split_fwd_kernel", {"BN_CL_GRID": 0}),

@@ -197,6 +197,13 @@ SWITCHES = [
      ["bn_stats_cl_kernel", "bn_bwd_reduce_cl_kernel"], ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"]),
     ("bn_cl_grid_wide_from_more_bytes", run_bn, ((64, 14, 14, 1024), 3, F32), {"BN_CL_GRID_WIDE_MIN_KB": 1000000},
      ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"]),
+    # (16 blocks instead of one per CU: 47 vectors per thread, the remainder streamed)
+    ("bn_cl_grid_fewer_blocks", run_bn, ((48000, 128), 1, F16), {"BN_CL_GRID_BLOCKS": 16},
+     ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"], []),
+    ("bn_cl_grid_fwd_max_slots", run_bn, ((48000, 128), 1, F16), {"BN_CL_GRID_FWD_MAX_SLOTS": 25},
+     ["bn_cl_grid_bwd_kernel"], ["bn_cl_grid_fwd_kernel"], {"BN_CL_GRID_BLOCKS": 16}),
+    ("bn_cl_grid_bwd_max_slots", run_bn, ((48000, 128), 1, F16), {"BN_CL_GRID_BWD_MAX_SLOTS": 25},
+     ["bn_cl_grid_fwd_kernel"], ["bn_cl_grid_bwd_kernel"], {"BN_CL_GRID_BLOCKS": 16}),
     ("bn_cl_grid_bwd_off", run_bn, ((100352, 64), 1, F16), {"BN_CL_GRID_BWD": 0},
      ["bn_cl_grid_fwd_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
      ["bn_cl_grid_bwd_kernel"], {"BN_CL_GRID_MIN_SLOTS": 1}),

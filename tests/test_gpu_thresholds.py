@@ -139,6 +139,12 @@ CASES = [
      [("below", ((128, 7, 7, 2048), 3, F16), {"BN_CL_GRID_WIDE_MIN_KB": 1}, "cl_split_fwd_kernel", "bn_cl_grid_fwd_kernel"),
       ("above", ((64, 14, 14, 1024), 3, F32), {"BN_CL_GRID_WIDE_MIN_KB": 1000000}, "bn_cl_grid_fwd_kernel",
        "cl_split_fwd_kernel")]),
+    # ... and up to 80 / 50 vectors per thread (25 / 21 held): beyond, three launches are as fast
+    ("bn_cl_grid_max_slots", P.run_bn, {},
+     [("below", ((256, 28, 28, 512), 3, F16), {"BN_CL_GRID_FWD_MAX_SLOTS": 25, "BN_CL_GRID_BWD_MAX_SLOTS": 25},
+       "bn_cl_grid_fwd_kernel", "bn_stats_cl_kernel"),
+      ("above", ((256, 56, 56, 256), 3, F16), {"BN_CL_GRID_FWD_MAX_SLOTS": 120, "BN_CL_GRID_BWD_MAX_SLOTS": 120},
+       "bn_stats_cl_kernel", "bn_cl_grid_fwd_kernel")]),
     # short planes that share cache lines: ordinary stores inside the shared lines up to 1 KB
     ("bn_edge_stores_max_bytes", P.run_bn, NCS,
      [("below", ((256, 256, 14, 14), 1, F16), {"BN_EDGE_STORES_MAX_BYTES": 0}, "bn_onchip_fwd_kernel", "bn_onchip_fwd_kernel"),
