@@ -545,13 +545,22 @@ bn_cl_grid_fwd_kernel(const BnClGridArgs a) {
   // ---- normalize what the block holds
 #pragma unroll
   for (int k = 0; k < NR; ++k) forget<T, VEC>(raw[k]);
+  // (scale and shift of a channel by one thread, through fold, which is free
+  // now: 1 / sqrt once per channel instead of VEC times in every thread,
+  // behind the exchange where every instruction is on the critical path)
+  if (t < a.cs) {
+    const float scale = gb[t] * inv_std(fin[2 * t + 1], a.eps);
+    fold[t] = scale;
+    fold[CMAX + t] = fmaf(-fin[2 * t], scale, gb[CMAX + t]);
+  }
+  lds_barrier();
   float sc[VEC], sh[VEC], mu[VEC], be[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
     mu[j] = fin[2 * (ch + j)];
-    sc[j] = gb[ch + j] * inv_std(fin[2 * (ch + j) + 1], a.eps);
+    sc[j] = fold[ch + j];
     be[j] = gb[CMAX + ch + j];
-    sh[j] = fmaf(-mu[j], sc[j], be[j]);
+    sh[j] = fold[CMAX + ch + j];
   }
   const uint32_t tb2 = grid_offset(a, fresh(t));
 #pragma unroll
@@ -616,7 +625,7 @@ bn_cl_grid_bwd_kernel(const BnClGridArgs a) {
   __shared__ int finmiss[CMAX];
   __shared__ uint32_t flags[kGridFlagWords];
   __shared__ float wsum[16];
-  __shared__ float par[5 * CMAX]; // mean, var, gamma, dvar, dmean
+  __shared__ float par[6 * CMAX]; // mean, var, gamma, dvar, dmean, istd
   const uint32_t b = blockIdx.x;
   const uint32_t t = threadIdx.x;
   const uint32_t strip = b % a.strips, range = b / a.strips;
@@ -668,13 +677,14 @@ bn_cl_grid_bwd_kernel(const BnClGridArgs a) {
     par[2 * CMAX + t] = p_gamma;
     par[3 * CMAX + t] = p_dvar;
     par[4 * CMAX + t] = p_dmean;
+    par[5 * CMAX + t] = 1.0f / sqrtf(p_var + a.eps);
   }
   lds_barrier();
   float mean[VEC], istd[VEC], nmi[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
     mean[j] = par[ch + j];
-    istd[j] = 1.0f / sqrtf(par[CMAX + ch + j] + a.eps);
+    istd[j] = par[5 * CMAX + ch + j];
     nmi[j] = -mean[j] * istd[j];
   }
 
@@ -791,22 +801,29 @@ bn_cl_grid_bwd_kernel(const BnClGridArgs a) {
   // ---- pass 2: dx = dy*gi + (x - mean)*A2 + cb  (half: x*A2 + B2, one mixed fma)
 #pragma unroll
   for (int k = 0; k < NR; ++k) forget<T, VEC>(raw[k]);
-  // (mean and istd from LDS again: kept in registers across the exchange,
-  // they and the vectors of x are more than a thread has)
+  // The coefficients of a channel by one thread, through fold, which is free
+  // now (behind the exchange every instruction is on the critical path); the
+  // means from LDS again: kept in registers across the exchange, they and the
+  // vectors of x are more than a thread has.
+  if (t < a.cs) {
+    const float g = par[2 * CMAX + t];
+    const float vpe = par[CMAX + t] + a.eps;
+    const float is = par[5 * CMAX + t];
+    const float cA = -is * g * fin[2 * t] * a.inv_N +
+                     (a.dvar ? 2.f * par[3 * CMAX + t] * (vpe * is) * a.inv_N : 0.f);
+    const float cb = -g * fin[2 * t + 1] * is * a.inv_N + (a.dmean ? par[4 * CMAX + t] * a.inv_N : 0.f);
+    fold[t] = g * is;
+    fold[CMAX + t] = is * cA;
+    fold[2 * CMAX + t] = sizeof(T) == 2 ? fmaf(-par[t] * is, cA, cb) : cb;
+  }
+  lds_barrier();
   float gi[VEC], A2[VEC], B2[VEC], mean2[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
-    const float g = par[2 * CMAX + ch + j];
-    const float vpe = par[CMAX + ch + j] + a.eps;
-    const float is = 1.0f / sqrtf(vpe);
     mean2[j] = par[ch + j];
-    const float cA = -is * g * fin[2 * (ch + j)] * a.inv_N +
-                     (a.dvar ? 2.f * par[3 * CMAX + ch + j] * (vpe * is) * a.inv_N : 0.f);
-    const float cb = -g * fin[2 * (ch + j) + 1] * is * a.inv_N +
-                     (a.dmean ? par[4 * CMAX + ch + j] * a.inv_N : 0.f);
-    gi[j] = g * is;
-    A2[j] = is * cA;
-    B2[j] = sizeof(T) == 2 ? fmaf(-mean2[j] * is, cA, cb) : cb;
+    gi[j] = fold[ch + j];
+    A2[j] = fold[CMAX + ch + j];
+    B2[j] = fold[2 * CMAX + ch + j];
   }
   auto emit = [&](const RawVec<T, VEC> &xr, const RawVec<T, VEC> &dr, uint32_t o) {
     float ov[VEC];

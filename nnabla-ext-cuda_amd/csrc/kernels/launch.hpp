@@ -97,7 +97,8 @@ struct RowCfg {
 // caller).  max_nl / max_nl_1024 bound the loads per thread below / at 1024
 // threads; min_tpr is 256 for the GroupNormalization backward and 4 where
 // several rows may share a wave; percol: LayerNormalization parameter layout.
-RowCfg pick_row_cfg(int vec, int64_t R, int max_nl, int max_nl_1024, int min_tpr, bool percol);
+RowCfg pick_row_cfg(int vec, int64_t R, int max_nl, int max_nl_1024, int min_tpr, bool percol,
+                    bool three = false);
 
 int launch_row_fwd(const RowProblem &p, hipStream_t st);
 int launch_row_bwd(const RowProblem &p, hipStream_t st);

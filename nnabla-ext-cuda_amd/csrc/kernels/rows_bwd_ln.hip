@@ -21,6 +21,9 @@ namespace nblahip {
   CASE(T, VEC, 1, 1024)
 #define LN_CASES(CASE, T)                                                              \
   LN_CASES_VEC(CASE, T, FullVec<T>::value)                                             \
+  CASE(T, FullVec<T>::value, 3, 64)                                                    \
+  CASE(T, FullVec<T>::value, 3, 256)                                                   \
+  CASE(T, FullVec<T>::value, 3, 512)                                                   \
   LN_CASES_VEC(CASE, T, MidVec<T>::value)                                              \
   LN_CASES_VEC(CASE, T, 1)                                                             \
   if constexpr (sizeof(T) == 4) {                                                      \

@@ -50,6 +50,12 @@ int run_row_bwd_cached_gnm(int dtype, const RowCfg &cfg, const RowArgs &args, in
 #define NBLAHIP_ROW_CASES_TPR(CASE, T, VEC, TPR) \
   CASE(T, VEC, 1, TPR) CASE(T, VEC, 2, TPR) CASE(T, VEC, 4, TPR) CASE(T, VEC, 8, TPR)
 
+// Three loads per thread with the widest vector: rows of 3 x 2^k vectors (hidden
+// sizes 768, 1536, 3072, 6144, 12288) exactly, 5 x 2^k (2560, 5120) at 83 %.
+#define NBLAHIP_ROW_CASES_THREE(CASE, T)                                          \
+  CASE(T, FullVec<T>::value, 3, 64) CASE(T, FullVec<T>::value, 3, 256)            \
+  CASE(T, FullVec<T>::value, 3, 512) CASE(T, FullVec<T>::value, 3, 1024)
+
 // Rows of a few hundred bytes: several rows per wave, at most 4 loads each.
 #define NBLAHIP_ROW_CASES_SUBWAVE(CASE, T, VEC)                                   \
   CASE(T, VEC, 1, 4) CASE(T, VEC, 2, 4) CASE(T, VEC, 4, 4)                        \

@@ -18,6 +18,7 @@ namespace nblahip {
 template <typename T>
 static int run_fwd_t(const RowCfg &cfg, const RowArgs &args, int grid, hipStream_t st) {
   NBLAHIP_ROW_CASES(FWD_CASE, T)
+  NBLAHIP_ROW_CASES_THREE(FWD_CASE, T)
   return NBLAHIP_EINVAL;
 }
 

@@ -38,18 +38,20 @@ static bool pick_subwave(RowCfg &c, int64_t nv, bool percol) {
   return percol ? take(32, 2) : take(16, 4);
 }
 
-RowCfg pick_row_cfg(int vec, int64_t R, int max_nl, int max_nl_1024, int min_tpr, bool percol) {
+RowCfg pick_row_cfg(int vec, int64_t R, int max_nl, int max_nl_1024, int min_tpr, bool percol,
+                    bool three) {
   RowCfg c;
   c.vec = vec;
   const int64_t nv = R / c.vec;
   if (min_tpr < 64 && pick_subwave(c, nv, percol)) return c;
   static const int tprs[4] = {64, 256, 512, 1024};
-  static const int nls[4] = {1, 2, 4, 8};
+  static const int nls[5] = {1, 2, 3, 4, 8};
   for (int tpr : tprs) {
     if (tpr < min_tpr) continue;
     const int cap = tpr == 1024 ? max_nl_1024 : max_nl;
     for (int nl : nls) {
       if (nl > cap) break;
+      if (nl == 3 && !three) continue;
       if (static_cast<int64_t>(tpr) * nl >= nv) {
         c.ok = true;
         c.tpr = tpr;
@@ -77,11 +79,12 @@ static RowCfg pick_ln_bwd_cfg(int dtype, int64_t R, int vec) {
     return c;
   };
   if (pick_subwave(c, nv, true)) return c;
-  for (int nl : {1, 2, 4})
-    if (64 * nl >= nv) return take(64, nl);
-  for (int nl : {1, 2, 4})
+  const bool three = vec == (dtype == NBLAHIP_F16 ? 8 : 4) && tune_int("ROW_NL3", 1);
+  for (int nl : {1, 2, 3, 4})
+    if ((nl != 3 || three) && 64 * nl >= nv) return take(64, nl);
+  for (int nl : {1, 2, 3, 4})
     for (int tpr : {256, 512})
-      if (static_cast<int64_t>(tpr) * nl >= nv) return take(tpr, nl);
+      if ((nl != 3 || three) && static_cast<int64_t>(tpr) * nl >= nv) return take(tpr, nl);
   const int cap_1024 = dtype == NBLAHIP_F16 ? 1 : 2; // beyond: spills
   for (int nl : {1, 2})
     if (nl <= cap_1024 && 1024 * nl >= nv) return take(1024, nl);
@@ -269,7 +272,8 @@ int launch_row_fwd(const RowProblem &p, hipStream_t st) {
   // 8 loads per thread it needs 140-210 VGPRs (8 waves per CU), so it spreads
   // a row over more threads instead.
   const int max_nl = p.mode == kRowLN ? 4 : 8;
-  const RowCfg cfg = pick_row_cfg(vec, p.R, max_nl, max_nl, 4, p.mode == kRowLN);
+  const bool three = vec == (p.dtype == NBLAHIP_F16 ? 8 : 4) && tune_int("ROW_NL3", 1);
+  const RowCfg cfg = pick_row_cfg(vec, p.R, max_nl, max_nl, 4, p.mode == kRowLN, three);
   // (rows beyond 64 KB held on one CU also where the row kernels' layouts reach)
   if (int status = 0; cfg.ok && !tune_int("FORCE_STREAM", 0) && p.R / vec > 4096 &&
                       row_onchip_fwd(p, a, vec, st, &status))
