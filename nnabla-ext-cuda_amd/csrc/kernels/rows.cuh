@@ -39,6 +39,7 @@ struct RowArgs {
   // (beta uses pmod_b in place of pmod: InstanceNormalization may broadcast
   // gamma and beta differently.)
   int percol;
+  int ahead; // forward, LayerNormalization: the persistent launch whose blocks ask for their next row ahead
   uint32_t pmod;
   uint32_t pmod_b;
   uint32_t pmul;
@@ -190,10 +191,14 @@ template <typename T, int VEC, int NL, int TPR, int MODE> struct RowBwdOccupancy
 // ---------------------------------------------------------------------------
 // STRIDED: BatchNormalization rows (see RowArgs::plane); also updates the
 // running statistics.
-template <typename T, int VEC, int NL, int TPR, bool PERCOL, bool STRIDED = false>
+// AHEAD: for a persistent launch (a few blocks per CU, each walking many
+// rows): the next row's loads are issued before the current row's sums, so a
+// block always has a row in flight.
+template <typename T, int VEC, int NL, int TPR, bool PERCOL, bool STRIDED = false, bool AHEAD = false>
 __global__ void __launch_bounds__(RowBlock<TPR>::kBlock,
                                   ((PERCOL && TPR == 1024 && NL <= 4) ? 8 : 1))
 row_fwd_kernel(const RowArgs a) {
+  static_assert(!AHEAD || (PERCOL && !STRIDED), "rows ahead: LayerNormalization only");
   constexpr int RPB = RowBlock<TPR>::kRowsPerBlock;
   __shared__ float lds[2 * 16];
   const int t = threadIdx.x % TPR;
@@ -226,17 +231,37 @@ row_fwd_kernel(const RowArgs a) {
     }
   }
 
+  RawVec<T, VEC> ahead[AHEAD ? NL : 1];
+  if constexpr (AHEAD) {
+    const int row0 = min(static_cast<int>(row_block_index<STRIDED>(a) * RPB + sub), static_cast<int>(a.rows) - 1);
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const int col = (k * TPR + t) * VEC;
+      ahead[k] = load_raw<T, VEC>(x + static_cast<size_t>(row0) * a.R + (col < a.R ? col : 0));
+    }
+  }
   for (int row = row_block_index<STRIDED>(a) * RPB + sub; row < a.rows; row += gridDim.x * RPB) {
     const size_t base = static_cast<size_t>(row) * (STRIDED ? a.plane.d : a.R);
     RawVec<T, VEC> raw[NL];
+    if constexpr (AHEAD) {
+      // (behind the last row: that row again - a load nobody waits for)
+      const int nrow = min(row + static_cast<int>(gridDim.x) * RPB, static_cast<int>(a.rows) - 1);
 #pragma unroll
-    for (int k = 0; k < NL; ++k) {
-      // Out-of-row lanes load column 0 (always valid) and are zeroed after:
-      // no branch, so the NL loads are in flight together.
-      const int col = (k * TPR + t) * VEC;
-      const bool ok = col < a.R;
-      raw[k] = raw_or_zero<T, VEC>(
-          ok, load_raw<T, VEC>(x + base + row_elem_offset<STRIDED>(a, ok ? col : 0)));
+      for (int k = 0; k < NL; ++k) {
+        const int col = (k * TPR + t) * VEC;
+        raw[k] = raw_or_zero<T, VEC>(col < a.R, ahead[k]);
+        ahead[k] = load_raw<T, VEC>(x + static_cast<size_t>(nrow) * a.R + (col < a.R ? col : 0));
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < NL; ++k) {
+        // Out-of-row lanes load column 0 (always valid) and are zeroed after:
+        // no branch, so the NL loads are in flight together.
+        const int col = (k * TPR + t) * VEC;
+        const bool ok = col < a.R;
+        raw[k] = raw_or_zero<T, VEC>(
+            ok, load_raw<T, VEC>(x + base + row_elem_offset<STRIDED>(a, ok ? col : 0)));
+      }
     }
     float gk[PERCOL ? 1 : NL], bk[PERCOL ? 1 : NL];
     if constexpr (!PERCOL) {

@@ -68,7 +68,7 @@ RowCfg pick_row_cfg(int vec, int64_t R, int max_nl, int max_nl_1024, int min_tpr
 // 256 or 512 threads with the fewest loads per thread (the per-column
 // accumulators make every load cost about 27 VGPRs), and the 1024-thread
 // layout, the slowest, only for rows nothing else holds.
-static RowCfg pick_ln_bwd_cfg(int dtype, int64_t R, int vec) {
+static RowCfg pick_ln_bwd_cfg(int dtype, int64_t R, int vec, bool allow_three = true) {
   RowCfg c;
   c.vec = vec;
   const int64_t nv = R / c.vec;
@@ -79,7 +79,7 @@ static RowCfg pick_ln_bwd_cfg(int dtype, int64_t R, int vec) {
     return c;
   };
   if (pick_subwave(c, nv, true)) return c;
-  const bool three = vec == (dtype == NBLAHIP_F16 ? 8 : 4) && tune_int("ROW_NL3", 1);
+  const bool three = allow_three && vec == (dtype == NBLAHIP_F16 ? 8 : 4) && tune_int("ROW_NL3", 1);
   for (int nl : {1, 2, 3, 4})
     if ((nl != 3 || three) && 64 * nl >= nv) return take(64, nl);
   for (int nl : {1, 2, 3, 4})
@@ -279,7 +279,31 @@ int launch_row_fwd(const RowProblem &p, hipStream_t st) {
                       row_onchip_fwd(p, a, vec, st, &status))
     return status;
   if (cfg.ok && !tune_int("FORCE_STREAM", 0)) {
-    return run_row_fwd_cached(p.dtype, cfg, a, cached_grid(p.rows, cfg.tpr), st);
+    int grid = cached_grid(p.rows, cfg.tpr);
+    // LayerNormalization: a block per row (or per four rows) launches waves
+    // faster than they can be started once a row is a few KB - [8192,4096]
+    // half: 8192 blocks, 33 us from HBM, 4.0 TB/s.  A few blocks per CU that
+    // walk the rows and ask for their next row before they sum the current one:
+    // 25 us.  Blocks per CU by measurement (us, block per row -> this):
+    // half [12288,4096] 49.0 -> 35.9 with 2, [8192,5120] 42.1 -> 30.8,
+    // [16384,3072] 48.9 -> 35.9 with 3 (41.9 with 2), [4096,8192] 29.5 -> 25.7,
+    // a wave per row [65536,768] 41.7 -> 36.5 with 3, [16384,1024] 14.8 -> 14.3;
+    // float [8192,4096] 49.5 -> 47.3 with 2, [32768,2048] 95.3 -> 89.5 (118.6
+    // with 1); not for float rows of a wave or less ([65536,768] 66.6 -> 71.9).
+    const bool full = vec == (p.dtype == NBLAHIP_F16 ? 8 : 4);
+    if (p.mode == kRowLN && full && cfg.tpr >= 64 && cfg.tpr <= 512 && cfg.nl <= 4 && tune_int("LN_FWD_AHEAD", 1)) {
+      const int64_t row_bytes = p.R * (p.dtype == NBLAHIP_F16 ? 2 : 4);
+      int per_cu = 0;
+      if (cfg.tpr >= 256) per_cu = (p.dtype == NBLAHIP_F16 && row_bytes < 8192) ? 3 : 2;
+      else if (p.dtype == NBLAHIP_F16 && cfg.nl >= 2) per_cu = 3;
+      per_cu = tune_int("LN_FWD_BLOCKS_PER_CU", per_cu);
+      if (per_cu > 0 && grid > 2 * per_cu * device_cus()) {
+        RowArgs b = a;
+        b.ahead = 1;
+        return run_row_fwd_cached(p.dtype, cfg, b, per_cu * device_cus(), st);
+      }
+    }
+    return run_row_fwd_cached(p.dtype, cfg, a, grid, st);
   }
   if (int status = 0; !tune_int("FORCE_STREAM", 0) && row_onchip_fwd(p, a, vec, st, &status))
     return status;
@@ -440,7 +464,8 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
   const bool ln = p.mode == kRowLN;
   if (!tune_int("FORCE_STREAM", 0) && ln_loose_bwd_wanted(p, vec)) {
     const int full = p.dtype == NBLAHIP_F16 ? 8 : 4;
-    const RowCfg loose = pick_ln_bwd_cfg(p.dtype, (p.R + full - 1) / full * full, full);
+    // (the kernel for rows at element alignment exists with 1, 2 and 4 vectors per lane)
+    const RowCfg loose = pick_ln_bwd_cfg(p.dtype, (p.R + full - 1) / full * full, full, false);
     if (loose.ok && loose.tpr == 64) {
       // (four vectors per lane: 139 - 218 registers, one 512-thread block per CU)
       const int grid = ln_bwd_grid(p.rows, loose.tpr, loose.nl >= 4 ? 1 : 2);

@@ -224,6 +224,10 @@ SWITCHES = [
      ["row_stats_stream_kernel", "plane_sums_stream_kernel"], ["row_fwd_kernel", "row_bwd_kernel_in"]),
     ("ln_long_rows_all_streaming", run_ln, (24, 18432, F16), {"LN_LONG_ROWS_CACHED": 0},
      ["ln_row_sums_stream_kernel", "row_bwd_dx_kernel"], ["row_bwd_kernel_lnx"]),
+    # (the forward kernel has one name for every launch shape: these pin the results only)
+    ("ln_fwd_block_per_row", run_ln, (1501, 4096, F16), {"LN_FWD_AHEAD": 0}, ["row_fwd_kernel"], []),
+    ("ln_fwd_one_block_per_cu", run_ln, (1501, 4096, F16), {"LN_FWD_BLOCKS_PER_CU": 1}, ["row_fwd_kernel"], []),
+    ("ln_no_three_vector_layouts", run_ln, (300, 6144, F16), {"ROW_NL3": 0}, ["row_fwd_kernel"], []),
     ("ln_odd_rows_scalar", run_ln, (40, 1023, F16), {"LN_LOOSE": 0},
      ["row_bwd_kernel_ln"], ["ln_loose_bwd_kernel"]),
     ("in_rows_instead_of_channel_blocks", run_in, (4, 256, (32, 32), F16), {"IN_NO_CHANNEL_BLOCKS": 1},

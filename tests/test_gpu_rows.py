@@ -389,6 +389,43 @@ def test_ln_forward_in_place(outer, Rr):
     assert_close(to_np(var), v_r, "f32", "stat", "var")
 
 
+# Many rows of a few KB: a few blocks per CU walk the rows and ask for their next
+# row ahead.  Two and three blocks per CU, a block and a wave per row, 1 to 4
+# vectors per thread, a last round that not every block takes part in.
+@pytest.mark.parametrize("outer,Rr,dtype", [(1501, 4096, torch.float16), (2100, 3072, torch.float16),
+                                            (1203, 6144, torch.float16), (1101, 8192, torch.float16),
+                                            (7003, 768, torch.float16), (9001, 1024, torch.float16),
+                                            (1333, 4096, torch.float32), (1100, 3072, torch.float32),
+                                            (1250, 2560, torch.float32), (1037, 16384, torch.float16)])
+def test_ln_forward_rows_ahead(outer, Rr, dtype):
+    """Against the oracle; bit for bit what the block-per-row launch gives
+    (same arithmetic per row); in place as well."""
+    dn = dtype_name(dtype)
+    x, _, g, b = make_ln(outer, Rr, dtype, 41)
+    y_r, m_r, v_r = R.ln_forward(x, b, g, outer, 1e-5)
+    xd, gd, bd = to_dev(x, dtype), to_dev(g), to_dev(b)
+    try:
+        K.tune_reset()
+        y, m, v = K.ln_forward(xd, bd, gd, outer, 1e-5)
+        K.tune_set("LN_FWD_AHEAD", 0)
+        y0, m0, v0 = K.ln_forward(xd, bd, gd, outer, 1e-5)
+        K.tune_reset()
+        L = K.lib()
+        xin = xd.clone()
+        mi, vi = torch.empty(outer, device="cuda"), torch.empty(outer, device="cuda")
+        K.check(L.nblahip_ln_fwd(xin.data_ptr(), gd.data_ptr(), bd.data_ptr(), xin.data_ptr(),
+                                 mi.data_ptr(), vi.data_ptr(), outer, Rr, 1e-5, K._dtype_code(xin),
+                                 torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+    finally:
+        K.tune_reset()
+    assert_close(to_np(m), m_r, dn, "stat", "mean")
+    assert_close(to_np(v), v_r, dn, "stat", "var")
+    assert_close(to_np(y), y_r, dn, "y", "y")
+    assert torch.equal(y, y0) and torch.equal(m, m0) and torch.equal(v, v0)
+    assert torch.equal(xin, y) and torch.equal(mi, m) and torch.equal(vi, v)
+
+
 # Rows of 128-400 KB on at least a quarter as many rows as CUs: the forward holds
 # a row on one CU (registers + LDS).  One shape per layout (10 to 25 vectors per
 # thread), a row that ends inside a wave's load, several channels per row.
