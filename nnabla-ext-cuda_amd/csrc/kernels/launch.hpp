@@ -91,6 +91,7 @@ bool gn_onchip_bwd(const RowProblem &p, hipStream_t st, int *status);
 struct RowCfg {
   bool ok = false;
   int vec = 1, tpr = 64, nl = 1;
+  bool ahead = false; // LayerNormalization backward: the kernel that asks for its next row ahead
 };
 
 // vec: elements per load (alignment and divisibility already checked by the

@@ -370,15 +370,19 @@ row_fwd_kernel(const RowArgs a) {
 // Padded lanes hold x = dy = 0 in registers; dy == 0 keeps them out of every
 // sum.
 // ---------------------------------------------------------------------------
-template <typename T, int VEC, int NL, int TPR, int MODE>
+// BAHEAD (LayerNormalization): the block asks for its next row's x, dy and
+// statistics before it works on the current row.
+template <typename T, int VEC, int NL, int TPR, int MODE, bool BAHEAD = false>
 __global__ void __launch_bounds__((RowBwdBlock<TPR, MODE>::kBlock),
                                    (RowBwdOccupancy<T, VEC, NL, TPR, MODE>::kMinWaves))
 row_bwd_kernel(const RowArgs a) {
+  static_assert(!BAHEAD || MODE == kRowLN, "rows ahead: LayerNormalization only");
   constexpr int RPB = RowBwdBlock<TPR, MODE>::kRowsPerBlock;
   constexpr int NW = TPR / kWave;
   // LayerNormalization keeps xh and dg of a row in registers between the
   // reduction and the dx step when they are few; otherwise they are recomputed.
-  constexpr bool KEEP = (MODE == kRowLN) && (NL * VEC <= 16);
+  // (not with the next row's vectors in registers as well)
+  constexpr bool KEEP = (MODE == kRowLN) && (NL * VEC <= 16) && !BAHEAD;
   constexpr bool GN = MODE == kRowGN || MODE == kRowGNm;
   constexpr bool BN = MODE == kRowBN; // strided rows, dgamma/dbeta written here
   constexpr bool GNM = MODE == kRowGNm; // run-time thread map (GnSlot)
@@ -434,6 +438,20 @@ row_bwd_kernel(const RowArgs a) {
   const int u0 = CH ? static_cast<int>(blockIdx.x) : static_cast<int>(row_block_index<BN>(a)) * RPB + sub;
   const int ustride = CH ? static_cast<int>(gridDim.x) : static_cast<int>(gridDim.x) * RPB;
   const int inner_n = CH ? a.rows / channels : 1;
+  RawVec<T, VEC> xa[BAHEAD ? NL : 1], da[BAHEAD ? NL : 1];
+  float mean_a = 0.f, var_a = 0.f;
+  if constexpr (BAHEAD) {
+    const int r0 = min(u0, nunits - 1);
+#pragma unroll
+    for (int k = 0; k < NL; ++k) {
+      const int col = (k * TPR + t) * VEC;
+      const size_t o = static_cast<size_t>(r0) * a.R + (col < a.R ? col : 0);
+      xa[k] = load_raw<T, VEC>(x + o);
+      da[k] = load_raw<T, VEC>(dy + o);
+    }
+    mean_a = a.mean[r0];
+    var_a = a.var[r0];
+  }
   for (int unit = u0; unit < nunits; unit += ustride) {
   float ch_sdx = 0.f, ch_sdy = 0.f; // kRowINc: this wave's share of the channel sums
   for (int rr = CH ? sub : 0; rr < inner_n; rr += CH ? RPB : 1) {
@@ -471,6 +489,25 @@ row_bwd_kernel(const RowArgs a) {
       var_early = a.var[row];
     }
     RawVec<T, VEC> xr[NL], dr[NL];
+    float mean_now = 0.f, var_now = 0.f;
+    if constexpr (BAHEAD) {
+      // (behind the block's last row: the tensor's last row again - loads nobody waits for)
+      const int nrow = min(unit + ustride, nunits - 1);
+      mean_now = mean_a;
+      var_now = var_a;
+#pragma unroll
+      for (int k = 0; k < NL; ++k) {
+        const int col = (k * TPR + t) * VEC;
+        const bool ok = col < a.R;
+        xr[k] = raw_or_zero<T, VEC>(ok, xa[k]);
+        dr[k] = raw_or_zero<T, VEC>(ok, da[k]);
+        const size_t o = static_cast<size_t>(nrow) * a.R + (ok ? col : 0);
+        xa[k] = load_raw<T, VEC>(x + o);
+        da[k] = load_raw<T, VEC>(dy + o);
+      }
+      mean_a = a.mean[nrow];
+      var_a = a.var[nrow];
+    } else
 #pragma unroll
     for (int k = 0; k < NL; ++k) {
       int col = (k * TPR + t) * VEC;
@@ -497,8 +534,8 @@ row_bwd_kernel(const RowArgs a) {
         return dr[k];
       }
     };
-    const float mean = PARK ? mean_early : a.mean[row];
-    const float vpe = (PARK ? var_early : a.var[row]) + a.eps;
+    const float mean = BAHEAD ? mean_now : PARK ? mean_early : a.mean[row];
+    const float vpe = (BAHEAD ? var_now : PARK ? var_early : a.var[row]) + a.eps;
     const float istd = 1.0f / sqrtf(vpe);
     const float nmi = -mean * istd;
 

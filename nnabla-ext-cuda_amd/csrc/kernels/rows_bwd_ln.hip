@@ -31,8 +31,23 @@ namespace nblahip {
     CASE(T, 1, 2, 1024)                                                                \
   }
 
+// Layouts that exist with the next row asked for ahead: a block per row, two
+// or three of the widest vectors per thread in half, three at 512 threads in
+// float (ln_bwd_rows_ahead in rows_host.hip has the measurements).
+template <typename T, int VEC, int NL, int TPR>
+constexpr bool kBwdAhead = VEC == FullVec<T>::value &&
+                           (sizeof(T) == 2 ? (NL == 2 || NL == 3) && (TPR == 256 || TPR == 512)
+                                           : NL == 3 && TPR == 512);
+
 #define BWD_CASE(T, VEC, NL, TPR)                                                      \
   if (cfg.vec == (VEC) && cfg.nl == (NL) && cfg.tpr == (TPR)) {                        \
+    if constexpr (kBwdAhead<T, VEC, NL, TPR>) {                                        \
+      if (cfg.ahead) {                                                                 \
+        NBLAHIP_LAUNCH("row_bwd_kernel_ln", (row_bwd_kernel<T, VEC, NL, TPR, kRowLN, true>),             \
+                       dim3(grid), dim3(RowBwdBlock<TPR, kRowLN>::kBlock), 0, st, args);                \
+        return last_launch_status();                                                   \
+      }                                                                                \
+    }                                                                                  \
     NBLAHIP_LAUNCH("row_bwd_kernel_ln", (row_bwd_kernel<T, VEC, NL, TPR, kRowLN>), dim3(grid),           \
                        dim3(RowBwdBlock<TPR, kRowLN>::kBlock), 0, st, args);                      \
     return last_launch_status();                                                       \
@@ -50,6 +65,15 @@ static int run_bwd_t(const RowCfg &cfg, const RowArgs &args, int grid, hipStream
 #define OCC_CASE(T, VEC, NL, TPR)                                                      \
   if (cfg.vec == (VEC) && cfg.nl == (NL) && cfg.tpr == (TPR)) {                        \
     int n = 0;                                                                         \
+    if constexpr (kBwdAhead<T, VEC, NL, TPR>) {                                        \
+      if (cfg.ahead) {                                                                 \
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(                              \
+                &n, row_bwd_kernel<T, VEC, NL, TPR, kRowLN, true>,                     \
+                RowBwdBlock<TPR, kRowLN>::kBlock, 0) != hipSuccess)                    \
+          n = 0;                                                                       \
+        return n;                                                                      \
+      }                                                                                \
+    }                                                                                  \
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(                                  \
             &n, row_bwd_kernel<T, VEC, NL, TPR, kRowLN>,                               \
             RowBwdBlock<TPR, kRowLN>::kBlock, 0) != hipSuccess)                        \
@@ -64,8 +88,8 @@ template <typename T> static int occupancy_t(const RowCfg &cfg) {
 
 int row_bwd_ln_resident_blocks(int dtype, const RowCfg &cfg) {
   static std::mutex mu;
-  static std::map<std::tuple<int, int, int, int>, int> cache;
-  const auto key = std::make_tuple(dtype, cfg.vec, cfg.nl, cfg.tpr);
+  static std::map<std::tuple<int, int, int, int, bool>, int> cache;
+  const auto key = std::make_tuple(dtype, cfg.vec, cfg.nl, cfg.tpr, cfg.ahead);
   std::lock_guard<std::mutex> lock(mu);
   auto it = cache.find(key);
   if (it == cache.end()) {

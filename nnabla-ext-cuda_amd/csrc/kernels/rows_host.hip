@@ -91,6 +91,11 @@ static RowCfg pick_ln_bwd_cfg(int dtype, int64_t R, int vec, bool allow_three = 
   return c;
 }
 
+static bool ln_bwd_rows_ahead(int dtype, const RowCfg &c, int vec) {
+  if (dtype == NBLAHIP_F16) return vec == 8 && (c.nl == 2 || c.nl == 3) && (c.tpr == 256 || c.tpr == 512);
+  return vec == 4 && c.nl == 3 && c.tpr == 512;
+}
+
 // GroupNormalization backward: vector width, block size, loads per thread and
 // the thread map of GnSlot (written into a).  Candidates are the widest vector
 // and scalar loads, and the block sizes whose map fits 8 loads per thread; the
@@ -525,8 +530,28 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
   }
   if (cfg.ok && !tune_int("FORCE_STREAM", 0)) {
     if (p.mode == kRowLN) {
-      const int resident = row_bwd_ln_resident_blocks(p.dtype, cfg);
-      const int grid = ln_bwd_grid(p.rows, cfg.tpr, resident > 0 ? resident : 2);
+      // A block per row with two or three vectors per thread: the blocks ask
+      // for their next row before they work on the current one (cold, us,
+      // backward alone / forward + backward in turn: half [8192,5120] 73.7 ->
+      // 54.5 / 102.1 -> 95.8, [4096,8192] 55.0 -> 47.0 / 77.2 -> 75.4; float
+      // [8192,5120] 102.8 -> 93.8 / 153.1 -> 150.8).  Not with one vector per
+      // thread ([16384,3072] half 73.5 -> 76.7) or four (nothing either way), not
+      // the other float layouts ([16384,3072] 178.7 -> 183.3 in turn), and not a
+      // wave per row: with the next row's vectors the half kernel has one
+      // 512-thread block per CU instead of two, which gains 5 % from HBM and
+      // loses as much where a step's backward finds x in the Infinity Cache
+      // ([65536,768] half 62.5 -> 59.1 alone, 97.6 -> 106.6 in turn; held to 128
+      // registers it spills and loses both).  Only where a block has several
+      // rows to walk.
+      cfg.ahead = ln_bwd_rows_ahead(p.dtype, cfg, vec) && tune_int("LN_BWD_AHEAD", 1);
+      int resident = row_bwd_ln_resident_blocks(p.dtype, cfg);
+      int grid = ln_bwd_grid(p.rows, cfg.tpr, resident > 0 ? resident : 2);
+      const int64_t row_blocks = cfg.tpr <= 64 ? (p.rows + 512 / cfg.tpr - 1) / (512 / cfg.tpr) : p.rows;
+      if (cfg.ahead && row_blocks < 2 * static_cast<int64_t>(grid)) {
+        cfg.ahead = false;
+        resident = row_bwd_ln_resident_blocks(p.dtype, cfg);
+        grid = ln_bwd_grid(p.rows, cfg.tpr, resident > 0 ? resident : 2);
+      }
       if (int e = run_row_bwd_cached_ln(p.dtype, cfg, a, grid, st)) return e;
       if (p.dgamma || p.dbeta) {
         NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 15) / 16), dim3(1024), 0, st,

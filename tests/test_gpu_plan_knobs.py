@@ -228,6 +228,7 @@ SWITCHES = [
     ("ln_fwd_block_per_row", run_ln, (1501, 4096, F16), {"LN_FWD_AHEAD": 0}, ["row_fwd_kernel"], []),
     ("ln_fwd_one_block_per_cu", run_ln, (1501, 4096, F16), {"LN_FWD_BLOCKS_PER_CU": 1}, ["row_fwd_kernel"], []),
     ("ln_no_three_vector_layouts", run_ln, (300, 6144, F16), {"ROW_NL3": 0}, ["row_fwd_kernel"], []),
+    ("ln_bwd_no_rows_ahead", run_ln, (4100, 1024, F16), {"LN_BWD_AHEAD": 0}, ["row_bwd_kernel_ln"], []),
     ("ln_odd_rows_scalar", run_ln, (40, 1023, F16), {"LN_LOOSE": 0},
      ["row_bwd_kernel_ln"], ["ln_loose_bwd_kernel"]),
     ("in_rows_instead_of_channel_blocks", run_in, (4, 256, (32, 32), F16), {"IN_NO_CHANNEL_BLOCKS": 1},

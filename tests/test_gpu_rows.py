@@ -426,6 +426,46 @@ def test_ln_forward_rows_ahead(outer, Rr, dtype):
     assert torch.equal(xin, y) and torch.equal(mi, m) and torch.equal(vi, v)
 
 
+# ... and the backward with two or three vectors per thread: a wave and a block
+# per row, a last round that not every block takes part in.
+@pytest.mark.parametrize("outer,Rr,dtype", [(9001, 1024, torch.float16), (5003, 768, torch.float32),
+                                            (1301, 8192, torch.float16), (1203, 5120, torch.float16),
+                                            (1100, 5120, torch.float32), (1501, 4096, torch.float32),
+                                            (2100, 6144, torch.float16)])
+def test_ln_backward_rows_ahead(outer, Rr, dtype):
+    """Against the oracle, with the statistics' gradients; close to what the
+    kernel without the rows ahead gives (that one keeps dy*gamma of a short row
+    in registers, this one multiplies gamma*istd first: other roundings); dx
+    does not depend on the grid."""
+    dn = dtype_name(dtype)
+    x, dy, g, b = make_ln(outer, Rr, dtype, 43)
+    rng = np.random.default_rng(44)
+    dm, dv = rng.standard_normal(outer), rng.standard_normal(outer)
+    _, m_r, v_r = R.ln_forward(x, b, g, outer, 1e-5)
+    dx_r, dg_r, db_r = R.ln_backward(x, dy, g, m_r, v_r, outer, 1e-5, dm, dv)
+    xd, dyd, gd = to_dev(x, dtype), to_dev(dy, dtype), to_dev(g)
+    md, vd, dmd, dvd = to_dev(m_r), to_dev(v_r), to_dev(dm), to_dev(dv)
+    try:
+        K.tune_reset()
+        K.tune_set("LN_BWD_BLOCKS_PER_CU", 1)
+        dx, dg, db = K.ln_backward(xd, dyd, gd, md, vd, outer, 1e-5, dmean=dmd, dvar=dvd)
+        K.tune_set("LN_BWD_AHEAD", 0)
+        dx0, dg0, db0 = K.ln_backward(xd, dyd, gd, md, vd, outer, 1e-5, dmean=dmd, dvar=dvd)
+        K.tune_reset()
+        dx2, dg2, db2 = K.ln_backward(xd, dyd, gd, md, vd, outer, 1e-5, dmean=dmd, dvar=dvd)
+    finally:
+        K.tune_reset()
+    assert_close(to_np(dx), dx_r, dn, "grad", "dx")
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
+    assert_close(to_np(dx0), to_np(dx).astype(np.float64), dn, "grad", "dx against the kernel without rows ahead")
+    assert_close(to_np(dg0), to_np(dg).astype(np.float64), dn, "pgrad", "dgamma against it")
+    assert_close(to_np(db0), to_np(db).astype(np.float64), dn, "pgrad", "dbeta against it")
+    assert torch.equal(dx2, dx)
+    assert_close(to_np(dg2), dg_r, dn, "pgrad", "dgamma, default grid")
+    assert_close(to_np(db2), db_r, dn, "pgrad", "dbeta, default grid")
+
+
 # Rows of 128-400 KB on at least a quarter as many rows as CUs: the forward holds
 # a row on one CU (registers + LDS).  One shape per layout (10 to 25 vectors per
 # thread), a row that ends inside a wave's load, several channels per row.
