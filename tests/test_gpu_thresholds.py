@@ -7,14 +7,14 @@ the knob decides about the shape, and the default plan must not be more than
 from the crossover shows up here instead of staying silent.  Times are sums of
 the library's per-kernel event timing over forward + backward, averaged over
 repetitions that walk rotated buffer sets.  The measured pairs are written to
-gpurun_out/thresholds.json when that directory exists."""
+thresholds.json in the directory that NBLAHIP_RESULTS_DIR names, if it is set."""
 import json
 import os
 
 import pytest
 import torch
 
-from _util import ROOT, load_package
+from _util import load_package
 import test_gpu_plan_knobs as P
 
 pytestmark = pytest.mark.gpu
@@ -34,8 +34,8 @@ def _default_knobs():
 @pytest.fixture(scope="module", autouse=True)
 def _dump():
     yield
-    out = os.path.join(ROOT, "gpurun_out")
-    if os.path.isdir(out) and RESULTS:
+    out = os.environ.get("NBLAHIP_RESULTS_DIR", "")
+    if out and os.path.isdir(out) and RESULTS:
         with open(os.path.join(out, "thresholds.json"), "w") as f:
             json.dump(RESULTS, f, indent=1)
 
