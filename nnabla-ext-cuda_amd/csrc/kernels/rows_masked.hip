@@ -1049,6 +1049,22 @@ bool masked_plan(const RowProblem &p, bool backward, MaskedCfg &cfg) {
   if (p.R < 2 * vec) return false;
   if (!aligned16(p.x) || (p.out && !aligned16(p.out)) || (backward && !aligned16(p.dy))) return false;
   if (p.rows >= (int64_t{1} << 31) / std::max<int64_t>(1, p.R)) return false;
+  // Half planes of up to 1024 elements that are a whole number of 8-byte
+  // vectors (6 x 6, 10 x 10, 14 x 14 ... 30 x 30): the plain row kernels with
+  // those vectors win over the masked 16-byte pieces - InstanceNormalization in
+  // both directions (forward + backward us, masked -> plain: [128,512,14,14]
+  // 42.3 -> 38.1, [128,2048,6,6] 40.6 -> 31.7, [64,256,26,26] 31.1 -> 26.3,
+  // [16,256,30,30] 17.7 -> 12.5), GroupNormalization in the forward
+  // ([128,512,14,14] 18.2 -> 13.2, [128,2048,6,6] 25.3 -> 11.6, [16,256,30,30]
+  // 8.6 -> 7.1) and, from 129 elements on, in the backward ([128,512,14,14] 32.0
+  // -> 21.9, [64,256,26,26] 22.5 -> 20.8; but [128,2048,6,6] 37.4 -> 49.9).
+  // Larger planes stay here: [16,256,46,46] InstanceNormalization 23.2 against
+  // 38.8 through the row kernels (a block per channel walks the batch), the
+  // forwards 3-13 % ahead as well.
+  if (p.dtype == NBLAHIP_F16 && p.spatial % 4 == 0 && p.spatial <= 1024 && p.R / 4 <= 8192 &&
+      !tune_int("ROW_MASKED_MID", 0)) {
+    if (p.mode == kRowIN || !backward || p.spatial > 128) return false;
+  }
   if (p.mode == kRowIN) {
     if (p.R % vec == 0) return false; // whole vectors: the plain kernels
     cfg = pick_masked((p.R + 2 * vec - 2) / vec);

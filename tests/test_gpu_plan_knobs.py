@@ -256,6 +256,11 @@ SWITCHES = [
     ("rows_masked_planes_off_float", run_gn, (2, 8, (65, 65), 2, F32), {"ROW_MASKED_PLANES": 0},
      ["gn_masked_fwd_kernel", "gn_masked_bwd_kernel"],
      ["gn_planes_masked_fwd_kernel", "gn_planes_masked_bwd_kernel"]),
+    # (half planes of whole 8-byte vectors go to the plain row kernels: the knob brings the masked ones back)
+    ("rows_masked_for_quad_planes", run_in, (6, 40, (14, 14), F16), {"ROW_MASKED_MID": 1},
+     ["in_masked_fwd_kernel", "in_masked_bwd_kernel"], ["row_fwd_kernel"]),
+    ("rows_masked_for_quad_planes_groups", run_gn, (6, 64, (14, 14), 8, F16), {"ROW_MASKED_MID": 1},
+     ["gn_planes_masked_fwd_kernel", "gn_planes_masked_bwd_kernel"], ["row_fwd_kernel"]),
     ("rows_masked_off", run_in, (4, 32, (63, 63), F16), {"ROW_MASKED": 0},
      ["row_fwd_kernel"], ["in_masked_fwd_kernel", "in_masked_bwd_kernel"]),
     ("rows_masked_off_float", run_in, (3, 10, (9, 7), F32), {"ROW_MASKED": 0},
