@@ -965,24 +965,23 @@ bool grid_args(const BnProblem &p, BnClGridArgs &a, int &nl) {
   nl = static_cast<int>((rows_pb * cv + kOnchipBlock - 1) / kOnchipBlock);
   ranges = (M + rows_pb - 1) / rows_pb;
   // From the rows on below which the split kernels (a block per 1024 rows) are
-  // as fast or faster.  Kernel time of forward + backward, this against the
-  // split kernels / the split reduction, half [M, 64]: 22.8 vs 21.9 us at
-  // M = 6272, 23.1 vs 29.1 at 12544, 24.8 vs 32.9 at 50176, 29.5 vs 45.5 at
-  // 100352, 33.6 vs 55.0 at 150528; float 19.5 vs 18.6, 20.0 vs 22.2, 24.2 vs
-  // 31.5; [M, 128] half 24.1 vs 22.5 at 6272, 25.1 vs 29.4 at 12544.  More than
-  // 128 channels: from the rows on that the split kernels' backward no longer
-  // holds (36 blocks of 1024 rows), or from 32 MiB; below, those take both
-  // directions and are as fast or faster (forward / backward us, this against
-  // them: [128,14,14,512] half 23.6 / 30.5 vs 17.8 / 20.0, [64,14,14,768] half
-  // 17.0 / 21.7 vs 16.7 / 19.3, [128,7,7,2048] half 17.6 / 23.2 vs 17.1 / 22.9,
-  // but [64,14,14,768] float 20.0 / 30.2 vs 24.2 / 34.4, [64,14,14,1024] float
-  // 23.6 / 38.1 vs 31.3 / 44.7, [256,7,7,2048] half 25.7 / 41.7 vs 35.6 / 49.4).
+  // as fast or faster.  Forward + backward us from HBM, this against the split
+  // kernels (or, beyond what those take, the split reduction).  Up to 128
+  // channels, half [M, 64]: 22.8 vs 21.9 at M = 6272, 23.1 vs 29.1 at 12544,
+  // 24.8 vs 32.9 at 50176, 33.6 vs 55.0 at 150528; float 19.5 vs 18.6, 20.0 vs
+  // 22.2, 24.2 vs 31.5.  More channels (column strips), half: [6272,256] 22.5 vs
+  // 24.3, [12544,256] 24.7 vs 31.7, [12544,512] 28.6 vs 34.6, [6272,1024] 27.9 vs
+  // 28.9, [12544,1024] 38.3 vs 40.8, [25088,1024] 65.1 vs 97.0, [6272,2048] 37.2
+  // vs 41.7, [3136,4096] 36.8 vs 40.2; float [12544,256] 27.1 vs 30.9,
+  // [6272,1024] 35.4 vs 37.5, [12544,1024] 62.0 vs 77.6, [3136,2048] 34.5 vs
+  // 36.5; but [3136,256] half 22.2 vs 21.5, [3136,512] float 21.6 vs 20.4: from
+  // 8192 rows or 24 MiB.
   if (p.C <= kGridMaxC) {
     if (M < tune_int("BN_CL_GRID_MIN_ROWS", 8192)) return false;
   } else {
     if (!tune_int("BN_CL_GRID_WIDE", 1)) return false;
-    if (M < tune_int("BN_CL_GRID_WIDE_MIN_ROWS", 36865) &&
-        tensor_bytes < static_cast<uint64_t>(tune_int("BN_CL_GRID_WIDE_MIN_KB", 32768)) * 1024u)
+    if (M < tune_int("BN_CL_GRID_WIDE_MIN_ROWS", 8192) &&
+        tensor_bytes < static_cast<uint64_t>(tune_int("BN_CL_GRID_WIDE_MIN_KB", 24576)) * 1024u)
       return false;
   }
   const int64_t nblocks = ranges * strips;

@@ -414,17 +414,28 @@ static bool bn_cl_cfg(const BnProblem &p, bool backward, GnClCfg &c, GnClArgs &a
   q.groups = static_cast<int>(p.C);
   q.eps = p.eps;
   q.accum_dx = p.accum_dx;
-  // Up to 2048 rows the single pass wins in both directions ([32,7,7,2048]
-  // half: 17 / 17 -> 9 / 10 us); the forward still does up to 4096 rows when
-  // there are at least 64 blocks (14 vs 23 us), the backward does not (24 vs 24 us
-  // at 3136 rows, 49 vs 25 us at 6272).
+  // The single pass wins up to 1024 rows and 4 MiB, and on anything up to
+  // 1 MiB; beyond, the split kernels (forward + backward us from HBM, this
+  // against them: half [1024,1024] 15.9 vs 17.9, [1024,4096] 26.5 vs 22.6,
+  // [1568,2048] 24.6 vs 20.7, [4096,1024] 31.8 vs 24.3; float [1568,4096] 66.1 vs
+  // 35.7, [2048,2048] 44.5 vs 27.8; a block per channel vector walks the rows
+  // alone).
   c = pick_in_cfg(q, al, backward, a, 2); // also the few rows of a fully connected layer's batch
   if (!c.ok) return false;
   // a handful of blocks: the split reduction fills the chip (tensors of up to
   // 2 MB excepted: there its three launches cost more than idle CUs)
   const int64_t bytes = p.size0 * p.C * (p.dtype == NBLAHIP_F16 ? 2 : 4);
   if (a.units < 32 && bytes > (2 << 20)) return false;
-  if (p.size0 > 2048 && (p.size0 > 4096 || a.units < 64)) return false;
+  // (FusedBatchNormalization has no split kernels to fall to: up to 2048 rows,
+  // the forward up to 4096 with at least 64 blocks, against its three-kernel path)
+  if (p.z || p.relu || p.y || p.dz) return !(p.size0 > 2048 && (p.size0 > 4096 || a.units < 64));
+  if (bytes > (1 << 20)) {
+    if (p.size0 > tune_int("BN_CL_CACHED_MAX_ROWS", 1024) ||
+        bytes >= static_cast<int64_t>(tune_int("BN_CL_CACHED_MAX_KB", 4096)) * 1024)
+      return false;
+  } else if (p.size0 > 2048) {
+    return false;
+  }
   return true;
 }
 

@@ -61,7 +61,7 @@ BN_CASES = [
     ((200704, 64), 1, F16, "bn_cl_grid"),
     ((40000, 256), 1, F32, "bn_cl_grid"),
     # channel-last through the split kernels (all rows as one plane)
-    ((64, 14, 14, 1024), 3, F16, "cl_split"),
+    ((32, 14, 14, 1024), 3, F16, "cl_split"),
 ]
 
 

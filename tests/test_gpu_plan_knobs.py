@@ -195,7 +195,8 @@ SWITCHES = [
      ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"], []),
     ("bn_cl_grid_strips_no_narrower_than", run_bn, ((256, 28, 28, 192), 3, F16), {"BN_CL_GRID_STRIP_MIN_VECS": 16},
      ["bn_stats_cl_kernel", "bn_bwd_reduce_cl_kernel"], ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"]),
-    ("bn_cl_grid_wide_from_more_bytes", run_bn, ((64, 14, 14, 1024), 3, F32), {"BN_CL_GRID_WIDE_MIN_KB": 1000000},
+    ("bn_cl_grid_wide_from_more_bytes", run_bn, ((64, 14, 14, 1024), 3, F32),
+     {"BN_CL_GRID_WIDE_MIN_KB": 1000000, "BN_CL_GRID_WIDE_MIN_ROWS": 999999},
      ["cl_split_fwd_kernel", "cl_split_bwd_kernel"], ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"]),
     # (16 blocks instead of one per CU: 47 vectors per thread, the remainder streamed)
     ("bn_cl_grid_fewer_blocks", run_bn, ((48000, 128), 1, F16), {"BN_CL_GRID_BLOCKS": 16},
@@ -207,10 +208,14 @@ SWITCHES = [
     ("bn_cl_grid_bwd_off", run_bn, ((100352, 64), 1, F16), {"BN_CL_GRID_BWD": 0},
      ["bn_cl_grid_fwd_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
      ["bn_cl_grid_bwd_kernel"], {"BN_CL_GRID_MIN_SLOTS": 1}),
+    ("bn_cl_cached_more_rows", run_bn, ((1568, 512), 1, F16), {"BN_CL_CACHED_MAX_ROWS": 2048},
+     ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"], ["cl_split_fwd_kernel"]),
+    ("bn_cl_cached_more_bytes", run_bn, ((1024, 4096), 1, F16), {"BN_CL_CACHED_MAX_KB": 16384},
+     ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"], ["cl_split_fwd_kernel"]),
     ("bn_cl_cached_off", run_bn, ((32, 7, 7, 256), 3, F16), {"BN_CL_CACHED": 0},
      ["bn_stats_cl_kernel", "bn_apply_cl_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
      ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"], {"BN_CL_SPLIT": 0}),
-    ("bn_cl_split_off", run_bn, ((64, 14, 14, 256), 3, F16), {"BN_CL_SPLIT": 0},
+    ("bn_cl_split_off", run_bn, ((32, 14, 14, 256), 3, F16), {"BN_CL_SPLIT": 0},
      ["bn_stats_cl_kernel", "bn_apply_cl_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
      ["cl_split_fwd_kernel", "cl_split_bwd_kernel"]),
     # rows: LayerNormalization / GroupNormalization / InstanceNormalization

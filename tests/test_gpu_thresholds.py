@@ -130,15 +130,24 @@ CASES = [
      [("below", ((6272, 64), 1, F16), {"BN_CL_GRID_MIN_ROWS": 1}, "cl_split_fwd_kernel", "bn_cl_grid_fwd_kernel"),
       ("above", ((12544, 64), 1, F16), {"BN_CL_GRID_MIN_ROWS": 999999}, "bn_cl_grid_fwd_kernel", "cl_split_fwd_kernel"),
       ("above_f32", ((12544, 128), 1, F32), {"BN_CL_GRID_MIN_ROWS": 999999}, "bn_cl_grid_fwd_kernel", "cl_split_fwd_kernel")]),
-    # ... with more than 128 channels: from 36865 rows
+    # ... with more than 128 channels: from 8192 rows as well
     ("bn_cl_grid_wide_min_rows", P.run_bn, {},
-     [("below", ((128, 16, 16, 256), 3, F16), {"BN_CL_GRID_WIDE_MIN_ROWS": 1}, None, "bn_cl_grid_fwd_kernel"),
-      ("above", ((256, 14, 14, 256), 3, F16), {"BN_CL_GRID_WIDE_MIN_ROWS": 999999}, "bn_cl_grid_fwd_kernel", None)]),
-    # ... or from 32 MiB
+     [("below", ((32, 14, 14, 256), 3, F16), {"BN_CL_GRID_WIDE_MIN_ROWS": 1}, "cl_split_fwd_kernel",
+       "bn_cl_grid_fwd_kernel"),
+      ("above", ((64, 14, 14, 256), 3, F16), {"BN_CL_GRID_WIDE_MIN_ROWS": 999999, "BN_CL_GRID_WIDE_MIN_KB": 1000000},
+       "bn_cl_grid_fwd_kernel", "cl_split_fwd_kernel")]),
+    # ... or from 24 MiB
     ("bn_cl_grid_wide_min_kb", P.run_bn, {},
-     [("below", ((128, 7, 7, 2048), 3, F16), {"BN_CL_GRID_WIDE_MIN_KB": 1}, "cl_split_fwd_kernel", "bn_cl_grid_fwd_kernel"),
-      ("above", ((64, 14, 14, 1024), 3, F32), {"BN_CL_GRID_WIDE_MIN_KB": 1000000}, "bn_cl_grid_fwd_kernel",
+     [("below", ((32, 14, 14, 1024), 3, F16), {"BN_CL_GRID_WIDE_MIN_KB": 1}, "cl_split_fwd_kernel", "bn_cl_grid_fwd_kernel"),
+      ("above", ((128, 7, 7, 2048), 3, F16), {"BN_CL_GRID_WIDE_MIN_KB": 1000000}, "bn_cl_grid_fwd_kernel",
        "cl_split_fwd_kernel")]),
+    # few rows, a block per channel vector: up to 1024 rows and 4 MiB
+    ("bn_cl_cached_max", P.run_bn, {},
+     [("below", ((1024, 1024), 1, F16), {"BN_CL_CACHED": 0}, "in_cl_row_fwd_kernel", "cl_split_fwd_kernel"),
+      ("above_rows", ((1568, 2048), 1, F16), {"BN_CL_CACHED_MAX_ROWS": 4096, "BN_CL_CACHED_MAX_KB": 1000000},
+       "cl_split_fwd_kernel", "in_cl_row_fwd_kernel"),
+      ("above_bytes", ((1024, 4096), 1, F16), {"BN_CL_CACHED_MAX_KB": 1000000}, "cl_split_fwd_kernel",
+       "in_cl_row_fwd_kernel")]),
     # ... and up to 80 / 50 vectors per thread (25 / 21 held): beyond, three launches are as fast
     ("bn_cl_grid_max_slots", P.run_bn, {},
      [("below", ((256, 28, 28, 512), 3, F16), {"BN_CL_GRID_FWD_MAX_SLOTS": 25, "BN_CL_GRID_BWD_MAX_SLOTS": 25},
