@@ -568,9 +568,16 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
     // float 126 vs 75 us) nor for float planes of 512 vectors and more in
     // batches of 8 and more (10-18 % slower than a row per block plus the
     // batch sum; smaller batches save more on the second launch).
+    // Half planes of 512 vectors and more: only with a block for every CU and
+    // no second round (us, a block per channel against a row per block plus
+    // the batch sum: [16,256,64,64] 20.2 vs 23.2, [32,256,64,64] 37.5 vs 40.6, but
+    // [16,320,64,64] 28.5 vs 26.8, [8,1024,64,64] 43.2 vs 40.6), and not beyond
+    // 1024 vectors ([16,256,128,128] 84.7 vs 73.5).
     const bool big_float = p.dtype == NBLAHIP_F32 && cfg.tpr * cfg.nl >= 512 && p.batch >= 8;
+    const bool big_half = p.dtype == NBLAHIP_F16 && cfg.tpr * cfg.nl >= 512 &&
+                          (p.channels > device_cus() || cfg.tpr * cfg.nl > 1024);
     if (p.mode == kRowIN && p.bc_gamma && p.bc_beta && p.batch > 1 &&
-        p.channels >= device_cus() && !big_float && !(cfg.tpr == 1024 && cfg.nl == 8) &&
+        p.channels >= device_cus() && !big_float && !big_half && !(cfg.tpr == 1024 && cfg.nl == 8) &&
         cfg.tpr >= 64 && !tune_int("IN_NO_CHANNEL_BLOCKS", 0)) {
       const int grid = static_cast<int>(std::min<int64_t>(p.channels, 1 << 20));
       return run_row_bwd_cached_inc(p.dtype, cfg, a, grid, st);
