@@ -975,12 +975,13 @@ bool grid_args(const BnProblem &p, BnClGridArgs &a, int &nl) {
   // vs 41.7, [3136,4096] 36.8 vs 40.2; float [12544,256] 27.1 vs 30.9,
   // [6272,1024] 35.4 vs 37.5, [12544,1024] 62.0 vs 77.6, [3136,2048] 34.5 vs
   // 36.5; but [3136,256] half 22.2 vs 21.5, [3136,512] float 21.6 vs 20.4: from
-  // 8192 rows or 24 MiB.
+  // 10240 rows ([8192,128] float 20.6 vs 17.5) or, with more than 128 channels,
+  // 24 MiB.
   if (p.C <= kGridMaxC) {
-    if (M < tune_int("BN_CL_GRID_MIN_ROWS", 8192)) return false;
+    if (M < tune_int("BN_CL_GRID_MIN_ROWS", 10240)) return false;
   } else {
     if (!tune_int("BN_CL_GRID_WIDE", 1)) return false;
-    if (M < tune_int("BN_CL_GRID_WIDE_MIN_ROWS", 8192) &&
+    if (M < tune_int("BN_CL_GRID_WIDE_MIN_ROWS", 10240) &&
         tensor_bytes < static_cast<uint64_t>(tune_int("BN_CL_GRID_WIDE_MIN_KB", 24576)) * 1024u)
       return false;
   }

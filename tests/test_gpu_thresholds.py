@@ -125,12 +125,12 @@ CASES = [
     ("bn_masked_onchip_min_pct", P.run_bn, {},
      [("few", ((64, 8, 17, 17), 1, F16), {"BN_MASKED_ONCHIP_MIN_PCT": 100}, "bn_masked_fwd_kernel", None),
       ("more", ((64, 32, 17, 17), 1, F32), {"BN_MASKED_ONCHIP_MIN_PCT": 100}, "bn_masked_fwd_kernel", None)]),
-    # channel-last, the tensor held on the chip: from 8192 rows
+    # channel-last, the tensor held on the chip: from 10240 rows
     ("bn_cl_grid_min_rows", P.run_bn, {},
      [("below", ((6272, 64), 1, F16), {"BN_CL_GRID_MIN_ROWS": 1}, "cl_split_fwd_kernel", "bn_cl_grid_fwd_kernel"),
       ("above", ((12544, 64), 1, F16), {"BN_CL_GRID_MIN_ROWS": 999999}, "bn_cl_grid_fwd_kernel", "cl_split_fwd_kernel"),
       ("above_f32", ((12544, 128), 1, F32), {"BN_CL_GRID_MIN_ROWS": 999999}, "bn_cl_grid_fwd_kernel", "cl_split_fwd_kernel")]),
-    # ... with more than 128 channels: from 8192 rows as well
+    # ... with more than 128 channels: from 10240 rows as well
     ("bn_cl_grid_wide_min_rows", P.run_bn, {},
      [("below", ((32, 14, 14, 256), 3, F16), {"BN_CL_GRID_WIDE_MIN_ROWS": 1}, "cl_split_fwd_kernel",
        "bn_cl_grid_fwd_kernel"),
