@@ -419,13 +419,21 @@ struct BnParamSrc {
 // STRADDLE: planes of nvp.d ELEMENTS (>= VEC, no multiple of VEC); a vector
 // then holds the end of one plane and the start of the next at most, and each
 // element picks the parameters of its own channel.
+// The parameters of the planes a block step meets (one per vector at most, and
+// the plane after a straddling vector's) go through LDS, each computed by one
+// thread: taken per vector they cost the inference path four loads and a
+// division by a square root each time, more than the vector's own traffic.
+constexpr uint32_t kApplyStep = 256u * kBnUnroll;
+constexpr uint32_t kApplyTab = kApplyStep + 4;
+
 template <typename T, int VEC, int FUSE = 0, bool STRADDLE = false>
 __global__ void __launch_bounds__(256)
 bn_apply_planes_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
                        FastDiv nvp, FastDiv cdiv, uint32_t total_vec,
                        const T *__restrict__ z) {
-  for (uint32_t i0 = blockIdx.x * (256u * kBnUnroll) + threadIdx.x; i0 < total_vec;
-       i0 += gridDim.x * (256u * kBnUnroll)) {
+  __shared__ float tab[3 * kApplyTab];
+  for (uint32_t vb = blockIdx.x * kApplyStep; vb < total_vec; vb += gridDim.x * kApplyStep) {
+    const uint32_t i0 = vb + threadIdx.x;
     float v[kBnUnroll][VEC];
     float zv[FUSE == 2 ? kBnUnroll : 1][VEC];
 #pragma unroll
@@ -436,32 +444,44 @@ bn_apply_planes_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc sr
         if constexpr (FUSE == 2) load_vec<T, VEC>(z + static_cast<size_t>(i) * VEC, zv[u]);
       }
     }
+    const uint32_t ve = min(vb + kApplyStep, total_vec) - 1;
+    const uint32_t p0 = nvp.div(STRADDLE ? vb * VEC : vb);
+    const uint32_t p1 = STRADDLE ? nvp.div(ve * VEC + (VEC - 1)) + 1 : nvp.div(ve);
+    __syncthreads(); // the step before has read its table
+    for (uint32_t k = threadIdx.x; k <= p1 - p0; k += 256u) {
+      const uint32_t plane = p0 + k;
+      const BnParam q = src.get(plane - cdiv.div(plane) * cdiv.d);
+      tab[k] = q.mean;
+      tab[kApplyTab + k] = q.a;
+      tab[2 * kApplyTab + k] = q.b;
+    }
+    __syncthreads();
 #pragma unroll
     for (int u = 0; u < kBnUnroll; ++u) {
       const uint32_t i = i0 + u * 256u;
       if (i < total_vec) {
         const uint32_t plane = nvp.div(STRADDLE ? i * VEC : i);
-        const uint32_t c = plane - cdiv.div(plane) * cdiv.d;
-        const BnParam q = src.get(c);
+        const uint32_t k = plane - p0;
+        const float qm = tab[k], qa = tab[kApplyTab + k], qb = tab[2 * kApplyTab + k];
         float o[VEC];
         if constexpr (STRADDLE) {
           // elements j >= cross belong to the next plane
           const int cross = static_cast<int>(nvp.d - (i * VEC - plane * nvp.d));
-          const BnParam q1 = src.get(c + 1 == cdiv.d ? 0u : c + 1);
+          const float nm = tab[k + 1], na = tab[kApplyTab + k + 1], nb = tab[2 * kApplyTab + k + 1];
 #pragma unroll
           for (int j = 0; j < VEC; ++j) {
             const bool nx = j >= cross;
-            o[j] = (v[u][j] - (nx ? q1.mean : q.mean)) * (nx ? q1.a : q.a) + (nx ? q1.b : q.b);
+            o[j] = (v[u][j] - (nx ? nm : qm)) * (nx ? na : qa) + (nx ? nb : qb);
           }
         } else if constexpr (sizeof(T) == 2) {
           // Half output: one mixed-precision fma per element; the folded shift
           // loses nothing a 10-bit mantissa can hold.
-          const float shift = fmaf(-q.mean, q.a, q.b);
+          const float shift = fmaf(-qm, qa, qb);
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) o[j] = fmaf(v[u][j], q.a, shift);
+          for (int j = 0; j < VEC; ++j) o[j] = fmaf(v[u][j], qa, shift);
         } else {
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) o[j] = (v[u][j] - q.mean) * q.a + q.b;
+          for (int j = 0; j < VEC; ++j) o[j] = (v[u][j] - qm) * qa + qb;
         }
         if constexpr (FUSE == 2) {
 #pragma unroll
@@ -484,10 +504,12 @@ bn_apply_planes_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc sr
 // R = 256 / cols rows per step (threads past R*cols idle; for ncv dividing 256
 // there are none and the block walks the slab as one contiguous run).  Wider
 // rows are cut into ntiles = ceil(ncv / 256) column tiles;
-// gridDim.x = ntiles * row blocks.
+// gridDim.x = ntiles * row blocks.  (The forward kernel can take narrower
+// tiles, tile_cols a power of two: fewer channels per block to prepare.)
 // ---------------------------------------------------------------------------
 struct ClApplyMap {
   uint32_t cv;       // channel vector of this thread
+  uint32_t col;      // ... counted from the tile's first
   uint32_t row0;     // first row
   uint32_t R;        // rows between the U loads of one step
   uint32_t row_step; // rows between steps
@@ -495,14 +517,16 @@ struct ClApplyMap {
 };
 
 template <int U>
-__device__ __forceinline__ ClApplyMap cl_apply_map(uint32_t ncv, uint32_t ntiles) {
+__device__ __forceinline__ ClApplyMap cl_apply_map(uint32_t ncv, uint32_t ntiles,
+                                                   uint32_t tile_cols = 256u) {
   ClApplyMap m;
-  const uint32_t cols = min(ncv, 256u);
+  const uint32_t cols = min(ncv, tile_cols);
   m.R = 256u / cols;
   const uint32_t tr = threadIdx.x / cols;
   const uint32_t tile = blockIdx.x % ntiles;
   const uint32_t rb = blockIdx.x / ntiles;
-  m.cv = tile * 256u + (threadIdx.x - tr * cols);
+  m.col = threadIdx.x - tr * cols;
+  m.cv = tile * tile_cols + m.col;
   m.active = tr < m.R && m.cv < ncv;
   m.row0 = rb * m.R * U + tr;
   m.row_step = (gridDim.x / ntiles) * m.R * U;
@@ -516,14 +540,30 @@ template <typename T, int VEC, int FUSE = 0>
 __global__ void __launch_bounds__(256)
 bn_apply_cl_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
                    uint32_t ncv, uint32_t ntiles, uint32_t M, const T *__restrict__ z,
-                   float one) {
+                   float one, uint32_t tile_cols) {
   // blockIdx.y: slab (sample) index; each slab has its own ncv*VEC parameters.
   const size_t slab = static_cast<size_t>(blockIdx.y) * M * ncv * VEC;
   x += slab;
   y += slab;
   if constexpr (FUSE == 2) z += slab;
   if (src.params) src.params += static_cast<size_t>(blockIdx.y) * ncv * VEC;
-  const ClApplyMap map = cl_apply_map<kBnUnroll>(ncv, ntiles);
+  const ClApplyMap map = cl_apply_map<kBnUnroll>(ncv, ntiles, tile_cols);
+  // The parameters of the block's channels go through LDS, each computed by
+  // one thread from coalesced loads: every thread taking its own VEC channels
+  // costs the inference path 4*VEC strided loads and VEC divisions by a square
+  // root per thread, which the texture path serializes over the block.
+  __shared__ float tab[3 * 256 * VEC];
+  {
+    const uint32_t c0 = (blockIdx.x % ntiles) * tile_cols * VEC;
+    const uint32_t nch = min(tile_cols * VEC, ncv * VEC - c0);
+    for (uint32_t k = threadIdx.x; k < nch; k += 256u) {
+      const BnParam q = src.get(c0 + k);
+      tab[k] = q.mean;
+      tab[256 * VEC + k] = q.a;
+      tab[2 * 256 * VEC + k] = (sizeof(T) == 2) ? fmaf(-q.mean, q.a, q.b) : q.b;
+    }
+    __syncthreads();
+  }
   if (!map.active) return;
   const uint32_t cv = map.cv;
   // y = x*pa + ps with ps = pb - mean*pa for half output (one mixed fma per
@@ -531,10 +571,10 @@ bn_apply_cl_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc src,
   float pm[VEC], pa[VEC], pb[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
-    const BnParam q = src.get(cv * VEC + j);
-    pm[j] = q.mean;
-    pa[j] = q.a;
-    pb[j] = (sizeof(T) == 2) ? fmaf(-q.mean, q.a, q.b) : q.b;
+    const uint32_t k = map.col * VEC + j;
+    pm[j] = tab[k];
+    pa[j] = tab[256 * VEC + k];
+    pb[j] = tab[2 * 256 * VEC + k];
   }
   for (uint32_t r0 = map.row0; r0 < M; r0 += map.row_step) {
     RawVec<T, VEC> raw[kBnUnroll];

@@ -84,6 +84,37 @@ def test_bn_inference(shape, axis, dtype, affine):
     assert_close(to_np(y), ref, dtype_name(dtype), "y", "y")
 
 
+# The apply kernels keep the parameters of the channels a block meets in a
+# table: planes of one vector and of 9 to 49 elements (up to a thousand planes
+# per block step, vectors that straddle two planes, the wrap from the last
+# channel to the first), channel-last rows of 1 to 260 vectors (column tiles
+# that are not full, rows narrower than a tile).
+TABLES = [
+    ((70, 300, 2, 4), 1), ((33, 300, 3, 3), 1), ((16, 130, 7, 7), 1), ((40, 17, 5, 5), 1),
+    ((9, 1000, 1, 8), 1), ((128, 3, 3, 5), 1), ((2, 5, 333, 8), 1),
+    ((1200, 8), 1), ((700, 200), 1), ((300, 520), 1), ((150, 1000), 1), ((90, 2080), 1),
+    ((64, 7, 7, 2048), 3), ((400, 133), 1),
+]
+
+
+@pytest.mark.parametrize("shape,axis", TABLES)
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tile", [None, 16, 256])
+def test_bn_inference_parameter_tables(shape, axis, dtype, tile):
+    if tile is not None and shape[axis] != shape[-1]:
+        pytest.skip("tile width: channel-last only")
+    x, _, g, b, rm, rv = make_bn(shape, axis, dtype, 3)
+    ref = R.bn_forward_global(x, b, g, rm, rv, axis, 1e-5)
+    if tile is not None:
+        K.tune_set("BN_CL_FWD_APPLY_TILE", tile)
+    try:
+        y = K.bn_forward_global(to_dev(x, dtype), to_dev(b), to_dev(g), to_dev(rm), to_dev(rv), axis,
+                                1e-5)
+    finally:
+        K.tune_reset()
+    assert_close(to_np(y), ref, dtype_name(dtype), "y", "y")
+
+
 @pytest.mark.parametrize("shape,axis", SMALL)
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_bn_training_forward_backward(shape, axis, dtype):

@@ -337,15 +337,25 @@ GRIDS = [
      ["bn_finalize_fwd_kernel", "bn_finalize_bwd_kernel"]),
     ("bn_direct_never", run_bn, ((8, 256, 28, 28), 1, F16), [{"BN_ROWS": 0, "BN_DIRECT": 0}],
      ["bn_stats_planes_kernel", "bn_finalize_fwd_kernel", "bn_finalize_bwd_kernel"], []),
-    ("bn_apply_persistent", run_bn, ((16, 48, 28, 28), 1, F32),
-     [{"BN_ROWS": 0, "BN_APPLY_BLOCKS_PER_CU": v} for v in (1, 3)],
+    # (588 block steps of 1024 vectors: with one block per CU each block takes two or three)
+    ("bn_apply_persistent", run_bn, ((64, 48, 28, 28), 1, F32),
+     [{"BN_ROWS": 0, "BN_CHAN_SPLIT": 0, "BN_ONCHIP": 0, "BN_APPLY_BLOCKS_PER_CU": v} for v in (1, 3)],
      ["bn_apply_planes_kernel", "bn_bwd_apply_planes_kernel"], []),
+    # (planes of 49 halves: vectors that straddle two planes, a table per block step)
+    ("bn_apply_persistent_straddle", run_bn, ((256, 256, 7, 7), 1, F16),
+     [{"BN_ROWS": 0, "BN_CHAN_SPLIT": 0, "BN_ONCHIP": 0, "BN_MASKED_ONCHIP": 0, "BN_PACK": 0,
+       "BN_APPLY_BLOCKS_PER_CU": 1}],
+     ["bn_stats_planes_kernel", "bn_apply_planes_kernel"], []),
     ("bn_masked_planes_off", run_bn, ((64, 64, 7, 7), 1, F16),
      [{"BN_ROWS": 0, "BN_MASKED_PLANES": 0, "BN_MASKED_ONCHIP": 0}],
      ["bn_stats_planes_kernel", "bn_apply_planes_kernel"], []),
     ("bn_cl_grids", run_bn, ((64, 28, 28, 64), 3, F16),
      [{"BN_CL_BLOCKS_PER_CU": a, "BN_CL_FWD_APPLY_BLOCKS_PER_CU": b, "BN_CL_APPLY_BLOCKS_PER_CU": c,
        "BN_CL_SPLIT": 0, "BN_CL_GRID": 0} for a, b, c in ((1, 1, 1), (2, 4, 2), (8, 3, 7))],
+     ["bn_stats_cl_kernel", "bn_apply_cl_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
+     []),
+    ("bn_cl_apply_tile", run_bn, ((16, 14, 14, 1000), 3, F16),
+     [{"BN_CL_FWD_APPLY_TILE": t, "BN_CL_SPLIT": 0, "BN_CL_GRID": 0} for t in (16, 128, 256)],
      ["bn_stats_cl_kernel", "bn_apply_cl_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
      []),
     ("bn_cl_grid_wide_fewer_rows", run_bn, ((128, 14, 14, 512), 3, F16), [{"BN_CL_GRID_WIDE_MIN_ROWS": 1}],
