@@ -504,8 +504,8 @@ bn_apply_planes_kernel(const T *__restrict__ x, T *__restrict__ y, BnParamSrc sr
 // R = 256 / cols rows per step (threads past R*cols idle; for ncv dividing 256
 // there are none and the block walks the slab as one contiguous run).  Wider
 // rows are cut into ntiles = ceil(ncv / 256) column tiles;
-// gridDim.x = ntiles * row blocks.  (The forward kernel can take narrower
-// tiles, tile_cols a power of two: fewer channels per block to prepare.)
+// gridDim.x = ntiles * row blocks.  (Narrower tiles, tile_cols a power of two:
+// fewer channels per block to prepare.)
 // ---------------------------------------------------------------------------
 struct ClApplyMap {
   uint32_t cv;       // channel vector of this thread
@@ -922,7 +922,8 @@ __global__ void __launch_bounds__(256)
 bn_bwd_apply_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
                        T *__restrict__ dx, const BnParam *__restrict__ params,
                        uint32_t ncv, uint32_t ntiles, uint32_t M, int accum,
-                       const T *__restrict__ y, T *__restrict__ dz, int accum_dz) {
+                       const T *__restrict__ y, T *__restrict__ dz, int accum_dz,
+                       uint32_t tile_cols) {
   constexpr int U = 2;
   const size_t slab = static_cast<size_t>(blockIdx.y) * M * ncv * VEC;
   x += slab;
@@ -933,19 +934,34 @@ bn_bwd_apply_cl_kernel(const T *__restrict__ x, const T *__restrict__ dy,
     if (dz) dz += slab;
   }
   params += static_cast<size_t>(blockIdx.y) * ncv * VEC;
-  const ClApplyMap map = cl_apply_map<U>(ncv, ntiles);
-  if (!map.active) return;
-  const uint32_t cv = map.cv;
+  const ClApplyMap map = cl_apply_map<U>(ncv, ntiles, tile_cols);
   // dx = pa*dy + pb*(x - mean) + pc = pa*dy + (pb*x + ps), ps = pc - pb*mean:
   // pb*(x-mean) is the small curvature term, so folding the mean costs nothing
   // measurable in float either (|pb*mean| <= |dvar|*2|mean|/N).
+  // The coefficients of the block's channels through LDS, a channel per thread
+  // (as in the forward kernel: a thread fetching its own VEC parameter structs
+  // touches a cache line per lane and load).
+  __shared__ float tab[3 * 256 * VEC];
+  {
+    const uint32_t c0 = (blockIdx.x % ntiles) * tile_cols * VEC;
+    const uint32_t nch = min(tile_cols * VEC, ncv * VEC - c0);
+    for (uint32_t k = threadIdx.x; k < nch; k += 256u) {
+      const BnParam q = params[c0 + k];
+      tab[k] = q.a;
+      tab[256 * VEC + k] = q.b;
+      tab[2 * 256 * VEC + k] = fmaf(-q.b, q.mean, q.c);
+    }
+    __syncthreads();
+  }
+  if (!map.active) return;
+  const uint32_t cv = map.cv;
   float pa[VEC], pb[VEC], ps[VEC];
 #pragma unroll
   for (int j = 0; j < VEC; ++j) {
-    const BnParam q = params[cv * VEC + j];
-    pa[j] = q.a;
-    pb[j] = q.b;
-    ps[j] = fmaf(-q.b, q.mean, q.c);
+    const uint32_t k = map.col * VEC + j;
+    pa[j] = tab[k];
+    pb[j] = tab[256 * VEC + k];
+    ps[j] = tab[2 * 256 * VEC + k];
   }
   for (uint32_t r0 = map.row0; r0 < M; r0 += map.row_step) {
     RawVec<T, VEC> xr[U], dr[U];

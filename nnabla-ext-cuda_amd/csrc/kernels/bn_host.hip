@@ -88,8 +88,7 @@ ClApplyGrid cl_apply_grid(uint64_t M, uint32_t ncv, int unroll, int per_cu, uint
 // of its tile's channels before its first load: with 64 vectors (a wave per
 // row segment of 1 KiB) [256,7,7,2048] half takes 21 us in inference, with 256
 // vectors 26 us (a plain copy 21.5 us).
-uint32_t cl_apply_tile_cols() {
-  const int t = tune_int("BN_CL_FWD_APPLY_TILE", 64);
+uint32_t cl_apply_tile_cols(int t) {
   uint32_t c = 16;
   while (c < 256u && static_cast<int>(c) < t) c <<= 1;
   return c;
@@ -191,7 +190,7 @@ int fwd_apply_fuse_t(const BnProblem &p, const BnPlan &pl, const BnParamSrc &src
   const uint64_t total = static_cast<uint64_t>(p.size0) * p.C * p.size2;
   const uint32_t total_vec = static_cast<uint32_t>(total / VEC);
   if (pl.channel_last) {
-    const uint32_t tile_cols = cl_apply_tile_cols();
+    const uint32_t tile_cols = cl_apply_tile_cols(tune_int("BN_CL_FWD_APPLY_TILE", 64));
     const ClApplyGrid g = cl_apply_grid(static_cast<uint64_t>(p.size0), pl.ncv, kBnUnroll,
                                         tune_int("BN_CL_FWD_APPLY_BLOCKS_PER_CU", 4), 1, tile_cols);
     NBLAHIP_LAUNCH(FUSE ? "bn_apply_cl_kernel_fused" : "bn_apply_cl_kernel",
@@ -330,12 +329,13 @@ int bwd_apply_fuse_t(const BnProblem &p, const BnPlan &pl, const BnParam *params
   const uint64_t total = static_cast<uint64_t>(p.size0) * p.C * p.size2;
   const uint32_t total_vec = static_cast<uint32_t>(total / VEC);
   if (pl.channel_last) {
+    const uint32_t tile_cols = cl_apply_tile_cols(tune_int("BN_CL_APPLY_TILE", 64));
     const ClApplyGrid g = cl_apply_grid(static_cast<uint64_t>(p.size0), pl.ncv, 2,
-                                        tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 4), 1);
+                                        tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 3), 1, tile_cols);
     NBLAHIP_LAUNCH(FUSED ? "bn_bwd_apply_cl_kernel_fused" : "bn_bwd_apply_cl_kernel",
                    (bn_bwd_apply_cl_kernel<T, VEC, FUSED>), dim3(g.x), dim3(256), 0, st, x, dy, dx,
                    params, pl.ncv, g.ntiles, static_cast<uint32_t>(p.size0), p.accum_dx, y, dz,
-                   p.accum_dz);
+                   p.accum_dz, tile_cols);
   } else {
     if constexpr (kFullVec<T, VEC>) {
       if (pl.masked) {
@@ -712,7 +712,7 @@ int cl_stats_t(const ClProblem &p, const BnPlan &pl, float *part, hipStream_t st
 template <typename T, int VEC>
 int cl_apply_t(const ClProblem &p, const BnPlan &pl, const BnParam *params, hipStream_t st) {
   const ClApplyGrid g = cl_apply_grid(static_cast<uint64_t>(p.spatial), pl.ncv, kBnUnroll,
-                                      tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 4),
+                                      tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 3),
                                       static_cast<uint64_t>(p.batch));
   NBLAHIP_LAUNCH("bn_apply_cl_kernel", (bn_apply_cl_kernel<T, VEC>),
                  dim3(g.x, static_cast<uint32_t>(p.batch)), dim3(256), 0, st,
@@ -736,14 +736,15 @@ int cl_bwd_reduce_t(const ClProblem &p, const BnPlan &pl, float *part2, hipStrea
 
 template <typename T, int VEC>
 int cl_bwd_apply_t(const ClProblem &p, const BnPlan &pl, const BnParam *params, hipStream_t st) {
+  const uint32_t tile_cols = cl_apply_tile_cols(tune_int("BN_CL_APPLY_TILE", 64));
   const ClApplyGrid g = cl_apply_grid(static_cast<uint64_t>(p.spatial), pl.ncv, 2,
-                                      tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 4),
-                                      static_cast<uint64_t>(p.batch));
+                                      tune_int("BN_CL_APPLY_BLOCKS_PER_CU", 3),
+                                      static_cast<uint64_t>(p.batch), tile_cols);
   NBLAHIP_LAUNCH("bn_bwd_apply_cl_kernel", (bn_bwd_apply_cl_kernel<T, VEC>),
                  dim3(g.x, static_cast<uint32_t>(p.batch)), dim3(256), 0, st,
                  static_cast<const T *>(p.x), static_cast<const T *>(p.dy), static_cast<T *>(p.out),
                  params, pl.ncv, g.ntiles, static_cast<uint32_t>(p.spatial), p.accum_dx,
-                 static_cast<const T *>(nullptr), static_cast<T *>(nullptr), 0);
+                 static_cast<const T *>(nullptr), static_cast<T *>(nullptr), 0, tile_cols);
   return last_launch_status();
 }
 
@@ -760,11 +761,41 @@ size_t cl_workspace_bytes(int64_t batch, int64_t spatial, int64_t channels, int 
   return std::max(split_reduction, split_pairs);
 }
 
+// Groups whose channel count keeps them from the split kernels: whether the
+// tile kernels (blocks of whole rows, a block per CU) are tried before the
+// cached ones (a block per group, 16-byte pieces of the rows).  The cached
+// kernels win on small groups and on tensors of a few MB (one short launch
+// without an exchange); vectors per group from which the tile kernels are ahead,
+// on 8-60 MB tensors from HBM: half forward 2048 ([16,36,36,400] G=25 15.9 against
+// 14.8 us, [16,48,48,200] 18.2 / 14.3, [16,64,64,200] 28.0 / 17.6; below,
+// [16,32,32,400] 13.4 / 13.7, [16,28,28,200] 8.8 / 12.6), half backward 768
+// ([16,28,28,200] 17.6 / 16.7, [16,32,32,200] 20.0 / 16.9, [16,40,40,200] 25.0 / 18.3;
+// below, [16,24,24,200] 15.7 / 16.5), float forward 768 ([32,28,28,100] G=25
+// 12.7 / 11.4, [32,40,40,100] 22.4 / 14.2; below, [32,20,20,100] 8.2 / 10.1), float
+// backward 512 ([32,24,24,100] 18.0 / 15.2, [32,32,32,72] G=9 18.9 / 16.1; below,
+// [32,16,16,72] 10.2 / 12.3).
+static bool cl_tile_first(const ClProblem &p, bool backward) {
+  if (p.groups == p.channels) return false;
+  const bool half = p.dtype == NBLAHIP_F16;
+  const int64_t vec = half ? 8 : 4;
+  const int64_t cpg = p.channels / p.groups;
+  if (cpg % vec != 0) return false;
+  if (p.channels % (8 * vec) == 0) return false; // whole 128-byte lines: not measured here
+  if (p.batch * p.spatial * p.channels * (half ? 2 : 4) <= (4 << 20)) return false;
+  const int64_t nv = p.spatial * (cpg / vec);
+  const int64_t from = half ? (backward ? tune_int("GN_CL_TILE_FIRST_BWD", 768)
+                                        : tune_int("GN_CL_TILE_FIRST_FWD", 2048))
+                            : (backward ? tune_int("GN_CL_TILE_FIRST_BWD_F32", 512)
+                                        : tune_int("GN_CL_TILE_FIRST_FWD_F32", 768));
+  return nv > from;
+}
+
 int launch_cl_fwd(const ClProblem &p, hipStream_t st) {
   const bool al = aligned16(p.x) && aligned16(p.out);
   {
     int status = 0;
     if (cl_split_fwd(p, al, st, &status)) return status;
+    if (cl_tile_first(p, false) && cl_tile_fwd(p, al, st, &status)) return status;
     if (gn_cl_cached_fwd(p, al, st, &status)) return status;
     if (cl_tile_fwd(p, al, st, &status)) return status;
   }
@@ -810,6 +841,15 @@ int launch_cl_bwd(const ClProblem &p, hipStream_t st) {
                                         p.channels, p.dgamma, p.dbeta, 1, 1, p.accum_g, p.accum_b, st);
       return 0;
     }
+    auto after_tile = [&]() -> int {
+      if (status) return status;
+      if (p.dgamma || p.dbeta)
+        return launch_pair_param_reduce("pair_param_reduce_cl_kernel", pairs, pair_batches,
+                                        p.channels, p.dgamma, p.dbeta, 1, 1, p.accum_g, p.accum_b, st);
+      return 0;
+    };
+    if (cl_tile_first(p, true) && cl_tile_bwd(p, al, &pairs, &pair_batches, st, &status))
+      return after_tile();
     if (gn_cl_cached_bwd(p, al, w.pairs, st, &status)) {
       if (status) return status;
       if (p.dgamma || p.dbeta)
@@ -818,13 +858,7 @@ int launch_cl_bwd(const ClProblem &p, hipStream_t st) {
                                         p.accum_b, st);
       return 0;
     }
-    if (cl_tile_bwd(p, al, &pairs, &pair_batches, st, &status)) {
-      if (status) return status;
-      if (p.dgamma || p.dbeta)
-        return launch_pair_param_reduce("pair_param_reduce_cl_kernel", pairs, pair_batches,
-                                        p.channels, p.dgamma, p.dbeta, 1, 1, p.accum_g, p.accum_b, st);
-      return 0;
-    }
+    if (cl_tile_bwd(p, al, &pairs, &pair_batches, st, &status)) return after_tile();
   }
   const uint32_t cpg = static_cast<uint32_t>(p.channels / p.groups);
 #define CALL(T, V) cl_bwd_reduce_t<T, V>(p, pl, w.part, st)

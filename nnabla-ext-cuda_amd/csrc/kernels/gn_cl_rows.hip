@@ -18,6 +18,16 @@ struct GnClCfg {
   int vec = 1, tpr = 256, nl = 1;
 };
 
+// Whether the blocks of gpl neighbouring units go to one XCD (GN_CL_XCD_MAP:
+// 0 never, 2 only where gpl divides the units of a sample).  Where it does not
+// divide them the sets of gpl units lie askew to the cache lines, and a line
+// still has two XCDs fetching it instead of up to eight: [15,64,64,200] half
+// instances forward 47.8 us without the map.
+bool xcd_map_for(int64_t units_per_sample, int64_t gpl) {
+  const int mode = tune_int("GN_CL_XCD_MAP", 1);
+  return mode == 1 || (mode == 2 && units_per_sample % gpl == 0);
+}
+
 // The cached kernels apply when a group is at least one vector of channels
 // wide (cpg = VEC * cvg, cvg in {1, 2, 4, 8}), fits 8 loads per thread of a
 // block, and is big enough to be worth a block; parameters shared by the batch.
@@ -62,7 +72,7 @@ GnClCfg pick_cfg(const ClProblem &p, bool aligned, bool backward, GnClArgs &a) {
   a.cvg = FastDiv(static_cast<uint32_t>(cvg));
   const int64_t line = 128 / (p.dtype == NBLAHIP_F16 ? 2 : 4); // elements per 128-byte line
   const int64_t gpl = line / cpg;
-  a.gpl = (gpl >= 2 && p.groups % gpl == 0 && tune_int("GN_CL_XCD_MAP", 1)) ? static_cast<int>(gpl) : 1;
+  a.gpl = (gpl >= 2 && xcd_map_for(p.groups, gpl)) ? static_cast<int>(gpl) : 1;
   a.eps = p.eps;
   a.inv_R = static_cast<float>(1.0 / (static_cast<double>(p.spatial) * cpg));
   a.one = 1.0f;
@@ -83,8 +93,22 @@ GnClCfg pick_in_cfg(const ClProblem &p, bool aligned, bool backward, GnClArgs &a
   if (nv < (min_positions >= 0 ? min_positions : tune_int("IN_CL_MIN", 32))) return c;
   // Beyond 2048 positions the three-kernel path is as fast or faster in float
   // and in the backward pass (64x64 planes, half: backward 49 vs 44 us; 56x56
-  // float: 62 / 130 vs 57 / 92 us); below, the single pass wins by 1.3-2x.
+  // float: 62 / 130 vs 57 / 92 us).
   if ((backward || p.dtype == NBLAHIP_F32) && nv > 2048) return c;
+  // InstanceNormalization proper, tensors beyond a few MB (below, the single
+  // launch wins), planes from which the three-kernel path is ahead from HBM,
+  // this against it: half forward 2048 positions ([28,48,48,200] 28.8 vs 25.7 us,
+  // [15,64,64,200] 29.2 vs 24.4; below, [40,40,40,200] 26.2 vs 28.0), float forward
+  // 1024 ([32,36,36,100] 20.6 vs 18.4, [32,40,40,100] 24.1 vs 20.1; below,
+  // [32,32,32,100] 16.4 vs 16.8), float backward 640 ([32,28,28,100] 19.9 vs 18.7,
+  // [32,32,32,72] 19.6 vs 18.5; below, [32,24,24,100] 16.4 vs 17.6).
+  if (min_positions < 0 &&
+      p.batch * p.spatial * p.channels * (p.dtype == NBLAHIP_F16 ? 2 : 4) > (4 << 20)) {
+    const int64_t most = p.dtype == NBLAHIP_F16 ? tune_int("IN_CL_MAX", 2048)
+                         : backward             ? tune_int("IN_CL_MAX_F32_BWD", 640)
+                                                : tune_int("IN_CL_MAX_F32_FWD", 1024);
+    if (nv > most) return c;
+  }
   for (int tpr : {64, 256, 512, 1024}) {
     for (int nl : {1, 2, 4, 8}) {
       if (static_cast<int64_t>(tpr) * nl < nv) continue;
@@ -106,7 +130,7 @@ GnClCfg pick_in_cfg(const ClProblem &p, bool aligned, bool backward, GnClArgs &a
   a.units = static_cast<int>(p.batch * a.G);
   a.cvg = FastDiv(1);
   const int gpl = 128 / (vec * (p.dtype == NBLAHIP_F16 ? 2 : 4)); // vectors per 128-byte line
-  a.gpl = (a.G % gpl == 0 && tune_int("GN_CL_XCD_MAP", 1)) ? gpl : 1;
+  a.gpl = xcd_map_for(a.G, gpl) ? gpl : 1;
   a.eps = p.eps;
   a.inv_R = static_cast<float>(1.0 / static_cast<double>(p.spatial));
   a.one = 1.0f;
@@ -116,7 +140,7 @@ GnClCfg pick_in_cfg(const ClProblem &p, bool aligned, bool backward, GnClArgs &a
 
 unsigned grid_of(const GnClArgs &a) {
   if (a.gpl <= 1) return static_cast<unsigned>(a.units);
-  const unsigned sets = static_cast<unsigned>(a.units / a.gpl);
+  const unsigned sets = static_cast<unsigned>((a.units + a.gpl - 1) / a.gpl);
   return (sets + kXcds - 1) / kXcds * kXcds * static_cast<unsigned>(a.gpl);
 }
 
@@ -273,7 +297,7 @@ bool wide_fwd(const ClProblem &p, bool aligned, hipStream_t st, int *status) {
         a.cvg = FastDiv(static_cast<uint32_t>(cvg));
         a.chunk = FastDiv(static_cast<uint32_t>(cvg * w));
         const int64_t gpl = 128 / (cpg * w * 2); // blocks sharing a 128-byte line
-        a.gpl = (gpl >= 2 && a.G % gpl == 0 && tune_int("GN_CL_XCD_MAP", 1)) ? static_cast<int>(gpl) : 1;
+        a.gpl = (gpl >= 2 && xcd_map_for(a.G, gpl)) ? static_cast<int>(gpl) : 1;
         a.eps = p.eps;
         a.inv_R = static_cast<float>(1.0 / (static_cast<double>(p.spatial) * (instance ? 1 : cpg)));
         a.one = 1.0f;
@@ -360,7 +384,7 @@ bool wide_bwd(const ClProblem &p, bool aligned, float *pairs, hipStream_t st, in
         a.cpg = vec;
         a.units = static_cast<int>(blocks);
         const int64_t gpl = 128 / (vec * w * 2); // blocks sharing a 128-byte line
-        a.gpl = (gpl >= 2 && a.G % gpl == 0 && tune_int("GN_CL_XCD_MAP", 1)) ? static_cast<int>(gpl) : 1;
+        a.gpl = (gpl >= 2 && xcd_map_for(a.G, gpl)) ? static_cast<int>(gpl) : 1;
         a.eps = p.eps;
         a.inv_R = static_cast<float>(1.0 / (static_cast<double>(p.spatial) * (instance ? 1 : vec)));
         a.one = 1.0f;

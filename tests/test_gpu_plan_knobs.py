@@ -355,7 +355,8 @@ GRIDS = [
      ["bn_stats_cl_kernel", "bn_apply_cl_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
      []),
     ("bn_cl_apply_tile", run_bn, ((16, 14, 14, 1000), 3, F16),
-     [{"BN_CL_FWD_APPLY_TILE": t, "BN_CL_SPLIT": 0, "BN_CL_GRID": 0} for t in (16, 128, 256)],
+     [{"BN_CL_FWD_APPLY_TILE": t, "BN_CL_APPLY_TILE": u, "BN_CL_SPLIT": 0, "BN_CL_GRID": 0}
+      for t, u in ((16, 256), (128, 16), (256, 128))],
      ["bn_stats_cl_kernel", "bn_apply_cl_kernel", "bn_bwd_reduce_cl_kernel", "bn_bwd_apply_cl_kernel"],
      []),
     ("bn_cl_grid_wide_fewer_rows", run_bn, ((128, 14, 14, 512), 3, F16), [{"BN_CL_GRID_WIDE_MIN_ROWS": 1}],
@@ -433,6 +434,32 @@ GRIDS = [
      ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"], []),
     ("in_cl_fewer_positions", run_in, (4, 64, (4, 4), F16, True), [{"IN_CL_MIN": 8, **NO_SPLIT}],
      ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"], []),
+    # block order by line-sharing sets only where the sets divide a sample's units
+    ("gn_cl_rows_block_order_whole_sets", run_gn, (2, 120, (20, 20), 15, F32, True),
+     [{"GN_CL_XCD_MAP": m, **NO_SPLIT} for m in (1, 2)],
+     ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"], []),
+    # groups no split kernel takes, tensors beyond 4 MiB: the tile kernels ahead
+    # of the cached ones from a number of vectors per group, either way round
+    ("gn_cl_tile_first_half", run_gn, (16, 200, (28, 28), 25, F16, True),
+     [{"GN_CL_TILE_FIRST_FWD": 0, "GN_CL_TILE_FIRST_BWD": 0}],
+     ["gn_cl_tile_fwd_kernel", "gn_cl_tile_bwd_kernel"], []),
+    ("gn_cl_tile_later_half", run_gn, (16, 200, (28, 28), 25, F16, True),
+     [{"GN_CL_TILE_FIRST_FWD": 100000, "GN_CL_TILE_FIRST_BWD": 100000}],
+     ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"], []),
+    ("gn_cl_tile_first_float", run_gn, (32, 100, (24, 24), 25, F32, True),
+     [{"GN_CL_TILE_FIRST_FWD_F32": 0, "GN_CL_TILE_FIRST_BWD_F32": 0}],
+     ["gn_cl_tile_fwd_kernel", "gn_cl_tile_bwd_kernel"], []),
+    ("gn_cl_tile_later_float", run_gn, (32, 100, (24, 24), 25, F32, True),
+     [{"GN_CL_TILE_FIRST_FWD_F32": 100000, "GN_CL_TILE_FIRST_BWD_F32": 100000}],
+     ["gn_cl_row_fwd_kernel", "gn_cl_row_bwd_kernel"], []),
+    # InstanceNormalization proper beyond 4 MiB: most positions the cached kernels take
+    ("in_cl_cached_more_positions", run_in, (8, 200, (48, 48), F16, True), [{"IN_CL_MAX": 4096}],
+     ["in_cl_row_fwd_kernel"], []),
+    ("in_cl_cached_fewer_positions", run_in, (16, 200, (40, 40), F16, True), [{"IN_CL_MAX": 1024}],
+     ["bn_stats_cl_kernel", "bn_bwd_reduce_cl_kernel"], ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"]),
+    ("in_cl_cached_positions_float", run_in, (32, 100, (28, 28), F32, True),
+     [{"IN_CL_MAX_F32_FWD": 512, "IN_CL_MAX_F32_BWD": 1024}],
+     ["bn_stats_cl_kernel", "in_cl_row_bwd_kernel"], ["in_cl_row_fwd_kernel", "bn_bwd_reduce_cl_kernel"]),
 ]
 
 
