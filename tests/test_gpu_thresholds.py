@@ -181,6 +181,26 @@ CASES = [
     # channel-last groups that are no whole number of vectors: from 1 % of the CUs (3 blocks)
     ("gn_cl_tile_min_pct", P.run_gn, {},
      [("above", (4, 320, (8, 8), 32, F16, True), {"GN_CL_TILE_MIN_PCT": 100}, "gn_cl_tile_fwd_kernel", None)]),
+    # channel-last groups of whole vectors off the 128-byte grid, beyond 4 MiB: the
+    # position tiles ahead of the cached kernels from 2048 / 768 vectors per group
+    ("gn_cl_tile_first", P.run_gn, {},
+     [("below", (32, 200, (24, 24), 25, F16, True), {"GN_CL_TILE_FIRST_FWD": 0, "GN_CL_TILE_FIRST_BWD": 0},
+       "gn_cl_row_fwd_kernel", "gn_cl_tile_fwd_kernel"),
+      ("above", (16, 200, (48, 48), 25, F16, True), {"GN_CL_TILE_FIRST_FWD": 100000, "GN_CL_TILE_FIRST_BWD": 100000},
+       "gn_cl_tile_fwd_kernel", "gn_cl_row_fwd_kernel"),
+      ("below_f32", (64, 72, (16, 16), 9, F32, True), {"GN_CL_TILE_FIRST_FWD_F32": 0, "GN_CL_TILE_FIRST_BWD_F32": 0},
+       "gn_cl_row_fwd_kernel", "gn_cl_tile_fwd_kernel"),
+      ("above_f32", (32, 100, (40, 40), 25, F32, True),
+       {"GN_CL_TILE_FIRST_FWD_F32": 100000, "GN_CL_TILE_FIRST_BWD_F32": 100000},
+       "gn_cl_tile_fwd_kernel", "gn_cl_row_fwd_kernel")]),
+    # channel-last InstanceNormalization beyond 4 MiB: cached instances up to 2048 positions
+    ("in_cl_max", P.run_in, {},
+     [("below", (40, 200, (40, 40), F16, True), {"IN_CL_MAX": 1024}, "in_cl_row_fwd_kernel", "bn_stats_cl_kernel"),
+      ("above", (15, 200, (64, 64), F16, True), {"IN_CL_MAX": 8192}, "bn_stats_cl_kernel", "in_cl_row_fwd_kernel"),
+      ("below_f32", (32, 100, (24, 24), F32, True), {"IN_CL_MAX_F32_FWD": 256, "IN_CL_MAX_F32_BWD": 256},
+       "in_cl_row_fwd_kernel", "bn_stats_cl_kernel"),
+      ("above_f32", (32, 100, (40, 40), F32, True), {"IN_CL_MAX_F32_FWD": 4096, "IN_CL_MAX_F32_BWD": 4096},
+       "bn_stats_cl_kernel", "in_cl_row_fwd_kernel")]),
 ]
 FLAT = [(cid, run, base, side) for cid, run, base, sides in CASES for side in sides]
 
