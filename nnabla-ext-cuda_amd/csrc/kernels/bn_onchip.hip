@@ -596,12 +596,14 @@ bool onchip_args(const BnProblem &p, bool backward, BnOnchipArgs &a, int &nl, in
   // forward + backward, [16,C,56,56] float: 18.1 vs 26.7 us at C = 8, 19.4 vs
   // 21.1 at 32, 24.2 vs 25.9 at 60; [32,C,56,56] half: 22.5 vs 26.7 at C = 4,
   // 23.4 vs 28.3 at 28).  With a streamed remainder (channels beyond what the
-  // layouts hold) from channels for half the CUs: [32,C,56,56] float forward +
-  // backward 39.3 vs 31.8 us at C = 32, 44.4 vs 41.3 at 64, 55.1 vs 63.5 at
-  // 128, 88.4 vs 99.3 at 224; [32,C,112,112] half 97.0 vs 78.1 at 64, 119.5 vs
-  // 140.1 at 128.
+  // layouts hold) from channels for 37 % of the CUs: [32,C,56,56] float forward +
+  // backward 39.3 vs 31.8 us at C = 32, 42.0 vs 38.7 at 64, 43.8 vs 44.6 at 80,
+  // 46.7 vs 50.6 at 96, 55.1 vs 63.5 at 128, 88.4 vs 99.3 at 224; [32,C,112,112]
+  // half 105.6 vs 75.9 at 64, 113.9 vs 112.5 at 96, 124.3 vs 126.9 at 112, 119.5
+  // vs 140.1 at 128.  (Only where no channel split over several blocks applies:
+  // that takes these shapes first, 24 - 42 us on the float ones.)
   const bool whole = nv <= (backward ? 20480 : 25600);
-  const int min_pct = !whole     ? tune_int("BN_ONCHIP_STREAMED_MIN_PCT", 50)
+  const int min_pct = !whole     ? tune_int("BN_ONCHIP_STREAMED_MIN_PCT", 37)
                       : backward ? tune_int("BN_ONCHIP_BWD_MIN_PCT", 1)
                                  : tune_int("BN_ONCHIP_FWD_MIN_PCT", 1);
   if (p.C * 100 < static_cast<int64_t>(device_cus()) * min_pct) return false;

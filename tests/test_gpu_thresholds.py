@@ -102,10 +102,10 @@ TIMERS = {P.run_bn: time_bn, P.run_gn: time_gn, P.run_in: time_in}
 # plan, kernel that the default plan runs, kernel that the forced plan runs)])
 NCS = P.NO_CHAN_SPLIT
 CASES = [
-    # a channel with a streamed remainder held on one CU: from channels for half the CUs
+    # a channel with a streamed remainder held on one CU: from channels for 37 % of the CUs
     ("bn_onchip_streamed_min_pct", P.run_bn, NCS,
-     [("below", ((32, 96, 56, 56), 1, F32), {"BN_ONCHIP_STREAMED_MIN_PCT": 1}, "bn_bwd_reduce_planes_kernel", "bn_onchip_bwd_kernel"),
-      ("above", ((32, 128, 56, 56), 1, F32), {"BN_ONCHIP_STREAMED_MIN_PCT": 100}, "bn_onchip_bwd_kernel", "bn_bwd_reduce_planes_kernel")]),
+     [("below", ((32, 64, 56, 56), 1, F32), {"BN_ONCHIP_STREAMED_MIN_PCT": 1}, "bn_bwd_reduce_planes_kernel", "bn_onchip_bwd_kernel"),
+      ("above", ((32, 112, 56, 56), 1, F32), {"BN_ONCHIP_STREAMED_MIN_PCT": 100}, "bn_onchip_bwd_kernel", "bn_bwd_reduce_planes_kernel")]),
     # whole channels held on one CU: from the first channel (the old thresholds, an
     # eighth and a quarter of the CUs, left 20 - 45 % on the table below them)
     ("bn_onchip_whole_channels", P.run_bn, NCS,
@@ -184,7 +184,7 @@ CASES = [
     # channel-last groups of whole vectors off the 128-byte grid, beyond 4 MiB: the
     # position tiles ahead of the cached kernels from 2048 / 768 vectors per group
     ("gn_cl_tile_first", P.run_gn, {},
-     [("below", (32, 200, (24, 24), 25, F16, True), {"GN_CL_TILE_FIRST_FWD": 0, "GN_CL_TILE_FIRST_BWD": 0},
+     [("below", (16, 200, (32, 32), 25, F16, True), {"GN_CL_TILE_FIRST_FWD": 0, "GN_CL_TILE_FIRST_BWD": 0},
        "gn_cl_row_fwd_kernel", "gn_cl_tile_fwd_kernel"),
       ("above", (16, 200, (48, 48), 25, F16, True), {"GN_CL_TILE_FIRST_FWD": 100000, "GN_CL_TILE_FIRST_BWD": 100000},
        "gn_cl_tile_fwd_kernel", "gn_cl_row_fwd_kernel"),
