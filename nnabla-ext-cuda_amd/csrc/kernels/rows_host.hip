@@ -358,6 +358,24 @@ size_t row_bwd_workspace_bytes(int mode, int64_t rows, int64_t R, int64_t planes
          align_up(static_cast<size_t>(rows) * 2 * sizeof(float), 256) + align_up(split, 256);
 }
 
+// Fold of the LayerNormalization column partials ws[nparts][2][R].  From
+// partials of 8 MB on (and rows of whole 16-byte pieces) the kernel that reads
+// 256-byte runs; below, the one with 2R/16 blocks, which spreads a small fold
+// over more of the chip.
+static int launch_ln_param_reduce(const float *ws, int nparts, int R, float *dgamma, float *dbeta,
+                                  int accum_g, int accum_b, hipStream_t st) {
+  const int64_t bytes = static_cast<int64_t>(nparts) * 2 * R * 4;
+  if (R % 4 == 0 && aligned16(ws) &&
+      bytes >= static_cast<int64_t>(tune_int("LN_REDUCE_WIDE_MIN_KB", 8192)) * 1024) {
+    NBLAHIP_LAUNCH("ln_param_reduce_wide_kernel", ln_param_reduce_wide_kernel, dim3((2 * R + 63) / 64),
+                   dim3(1024), 0, st, ws, nparts, R, dgamma, dbeta, accum_g, accum_b);
+  } else {
+    NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * R + 15) / 16),
+                   dim3(1024), 0, st, ws, nparts, R, dgamma, dbeta, accum_g, accum_b);
+  }
+  return last_launch_status();
+}
+
 // LayerNormalization dgamma/dbeta by the streaming kernel: column partials over
 // row chunks (kept after the row sums in the workspace), then their fold.
 template <typename T, int VEC>
@@ -371,9 +389,7 @@ static int stream_ln_colgrad_t(const RowProblem &p, const RowArgs &a, hipStream_
                  static_cast<const T *>(p.x), static_cast<const T *>(p.dy), p.mean, p.var, a.rows,
                  a.R, rpc, p.eps, part);
   if (int e = last_launch_status()) return e;
-  NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 15) / 16),
-                 dim3(1024), 0, st, part, Y, a.R, p.dgamma, p.dbeta, p.accum_g, p.accum_b);
-  return last_launch_status();
+  return launch_ln_param_reduce(part, Y, a.R, p.dgamma, p.dbeta, p.accum_g, p.accum_b, st);
 }
 
 // vec: the row kernels' vector width for this problem (x and dy aligned, R a
@@ -476,10 +492,9 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
       const int grid = ln_bwd_grid(p.rows, loose.tpr, loose.nl >= 4 ? 1 : 2);
       if (int e = ln_loose_bwd(p, a, loose, grid, st)) return e;
       if (p.dgamma || p.dbeta) {
-        NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 15) / 16), dim3(1024), 0, st,
-                           static_cast<const float *>(p.ws), grid, a.R, p.dgamma, p.dbeta,
-                           p.accum_g, p.accum_b);
-        if (int e = last_launch_status()) return e;
+        if (int e = launch_ln_param_reduce(static_cast<const float *>(p.ws), grid, a.R, p.dgamma,
+                                           p.dbeta, p.accum_g, p.accum_b, st))
+          return e;
       }
       return 0;
     }
@@ -554,10 +569,9 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
       }
       if (int e = run_row_bwd_cached_ln(p.dtype, cfg, a, grid, st)) return e;
       if (p.dgamma || p.dbeta) {
-        NBLAHIP_LAUNCH("ln_param_reduce_kernel", ln_param_reduce_kernel, dim3((2 * a.R + 15) / 16), dim3(1024), 0, st,
-                           static_cast<const float *>(p.ws), grid, a.R, p.dgamma, p.dbeta,
-                           p.accum_g, p.accum_b);
-        if (int e = last_launch_status()) return e;
+        if (int e = launch_ln_param_reduce(static_cast<const float *>(p.ws), grid, a.R, p.dgamma,
+                                           p.dbeta, p.accum_g, p.accum_b, st))
+          return e;
       }
       return 0;
     }

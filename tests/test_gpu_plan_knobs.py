@@ -434,6 +434,13 @@ GRIDS = [
      ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"], []),
     ("in_cl_fewer_positions", run_in, (4, 64, (4, 4), F16, True), [{"IN_CL_MIN": 8, **NO_SPLIT}],
      ["in_cl_row_fwd_kernel", "in_cl_row_bwd_kernel"], []),
+    # the fold of the LayerNormalization column partials in 256-byte runs, from any size / never
+    ("ln_param_reduce_wide", run_ln, (300, 2048, F16), [{"LN_REDUCE_WIDE_MIN_KB": 0}],
+     ["row_bwd_kernel_ln", "ln_param_reduce_wide_kernel"], ["ln_param_reduce_kernel"]),
+    ("ln_param_reduce_wide_float", run_ln, (77, 5124, F32), [{"LN_REDUCE_WIDE_MIN_KB": 0}],
+     ["ln_param_reduce_wide_kernel"], ["ln_param_reduce_kernel"]),
+    ("ln_param_reduce_narrow", run_ln, (2048, 8192, F16), [{"LN_REDUCE_WIDE_MIN_KB": 1000000}],
+     ["row_bwd_kernel_ln", "ln_param_reduce_kernel"], ["ln_param_reduce_wide_kernel"]),
     # block order by line-sharing sets only where the sets divide a sample's units
     ("gn_cl_rows_block_order_whole_sets", run_gn, (2, 120, (20, 20), 15, F32, True),
      [{"GN_CL_XCD_MAP": m, **NO_SPLIT} for m in (1, 2)],
