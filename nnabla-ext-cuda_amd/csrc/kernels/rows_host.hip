@@ -68,7 +68,9 @@ RowCfg pick_row_cfg(int vec, int64_t R, int max_nl, int max_nl_1024, int min_tpr
 // 256 or 512 threads with the fewest loads per thread (the per-column
 // accumulators make every load cost about 27 VGPRs), and the 1024-thread
 // layout, the slowest, only for rows nothing else holds.
-static RowCfg pick_ln_bwd_cfg(int dtype, int64_t R, int vec, bool allow_three = true) {
+// rows: how many there are (0: unknown); the layouts that ask for the next row
+// ahead want several rows per block.
+static RowCfg pick_ln_bwd_cfg(int dtype, int64_t R, int vec, bool allow_three = true, int64_t rows = 0) {
   RowCfg c;
   c.vec = vec;
   const int64_t nv = R / c.vec;
@@ -80,8 +82,21 @@ static RowCfg pick_ln_bwd_cfg(int dtype, int64_t R, int vec, bool allow_three = 
   };
   if (pick_subwave(c, nv, true)) return c;
   const bool three = allow_three && vec == (dtype == NBLAHIP_F16 ? 8 : 4) && tune_int("ROW_NL3", 1);
+  // (for sweeps: a layout of 64, 256 or 512 threads forced where it holds the row)
+  if (const int ftpr = tune_int("LN_BWD_TPR", 0), fnl = tune_int("LN_BWD_NL", 0);
+      (ftpr == 64 || ftpr == 256 || ftpr == 512) && (fnl == 1 || fnl == 2 || fnl == 4 || (fnl == 3 && three)) &&
+      static_cast<int64_t>(ftpr) * fnl >= nv)
+    return take(ftpr, fnl);
   for (int nl : {1, 2, 3, 4})
     if ((nl != 3 || three) && 64 * nl >= nv) return take(64, nl);
+  // Half rows of 257 - 512 vectors: 256 threads with two vectors each and the
+  // next row asked for ahead, not 512 threads with one (backward cold, us:
+  // [13056,2560] 55.3 -> 47.4, [10752,3072] 49.6 -> 42.4, [8192,4096] 46.9 -> 43.8;
+  // without the rows ahead it loses, 59.5 / 53.2 / 50.6; float: 1280 - 2048
+  // elements 46.4 / 43.2 / 42.0 with 512 x 1 against 55.0 / 49.6 / 45.9).
+  if (dtype == NBLAHIP_F16 && vec == 8 && nv > 256 && nv <= 512 && rows >= 2048 &&
+      tune_int("LN_BWD_AHEAD", 1) && tune_int("LN_BWD_256X2", 1))
+    return take(256, 2);
   for (int nl : {1, 2, 3, 4})
     for (int tpr : {256, 512})
       if ((nl != 3 || three) && static_cast<int64_t>(tpr) * nl >= nv) return take(tpr, nl);
@@ -501,7 +516,7 @@ int launch_row_bwd(const RowProblem &p, hipStream_t st) {
   }
   const int nl_small = ln ? 4 : 8;
   const int nl_1024 = ln ? (p.dtype == NBLAHIP_F16 ? 1 : 2) : 8;
-  RowCfg cfg = ln ? pick_ln_bwd_cfg(p.dtype, p.R, vec)
+  RowCfg cfg = ln ? pick_ln_bwd_cfg(p.dtype, p.R, vec, true, p.rows)
                   : pick_row_cfg(vec, p.R, nl_small, nl_1024, p.mode == kRowGN ? 256 : 4, false);
   bool gn_map = false;
   if (p.mode == kRowGN) {

@@ -441,6 +441,16 @@ GRIDS = [
      ["ln_param_reduce_wide_kernel"], ["ln_param_reduce_kernel"]),
     ("ln_param_reduce_narrow", run_ln, (2048, 8192, F16), [{"LN_REDUCE_WIDE_MIN_KB": 1000000}],
      ["row_bwd_kernel_ln", "ln_param_reduce_kernel"], ["ln_param_reduce_wide_kernel"]),
+    # half rows of 257 - 512 vectors: 256 threads x 2 vectors with the next row ahead (default),
+    # 512 x 1, and the layouts a sweep can force
+    ("ln_bwd_256x2_off", run_ln, (2304, 3072, F16), [{"LN_BWD_256X2": 0}, {"LN_BWD_AHEAD": 0}],
+     ["row_bwd_kernel_ln"], []),
+    ("ln_bwd_forced_layouts", run_ln, (2100, 2560, F16),
+     [{"LN_BWD_TPR": t, "LN_BWD_NL": n} for t, n in ((512, 1), (256, 2), (256, 3), (512, 2), (256, 4), (512, 4))],
+     ["row_bwd_kernel_ln"], []),
+    ("ln_bwd_forced_layouts_float", run_ln, (2100, 1000, F32),
+     [{"LN_BWD_TPR": t, "LN_BWD_NL": n} for t, n in ((64, 4), (256, 1), (256, 2), (512, 1), (512, 3))],
+     ["row_bwd_kernel_ln"], []),
     # block order by line-sharing sets only where the sets divide a sample's units
     ("gn_cl_rows_block_order_whole_sets", run_gn, (2, 120, (20, 20), 15, F32, True),
      [{"GN_CL_XCD_MAP": m, **NO_SPLIT} for m in (1, 2)],
