@@ -46,6 +46,18 @@ RowCfg pick_row_cfg(int vec, int64_t R, int max_nl, int max_nl_1024, int min_tpr
   if (min_tpr < 64 && pick_subwave(c, nv, percol)) return c;
   static const int tprs[4] = {64, 256, 512, 1024};
   static const int nls[5] = {1, 2, 3, 4, 8};
+  // (for sweeps: a layout of whole waves forced where it holds the row)
+  if (const int ftpr = tune_int("ROW_TPR", 0), fnl = tune_int("ROW_NL", 0);
+      ftpr >= 64 && ftpr >= min_tpr && fnl > 0 && static_cast<int64_t>(ftpr) * fnl >= nv) {
+    for (int tpr : tprs)
+      for (int nl : nls)
+        if (tpr == ftpr && nl == fnl && nl <= (tpr == 1024 ? max_nl_1024 : max_nl) && (nl != 3 || three)) {
+          c.ok = true;
+          c.tpr = tpr;
+          c.nl = nl;
+          return c;
+        }
+  }
   for (int tpr : tprs) {
     if (tpr < min_tpr) continue;
     const int cap = tpr == 1024 ? max_nl_1024 : max_nl;

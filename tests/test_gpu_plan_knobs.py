@@ -451,6 +451,9 @@ GRIDS = [
     ("ln_bwd_forced_layouts_float", run_ln, (2100, 1000, F32),
      [{"LN_BWD_TPR": t, "LN_BWD_NL": n} for t, n in ((64, 4), (256, 1), (256, 2), (512, 1), (512, 3))],
      ["row_bwd_kernel_ln"], []),
+    ("in_forced_wave_layouts", run_in, (6, 40, (32, 32), F16),
+     [{"ROW_TPR": t, "ROW_NL": n} for t, n in ((64, 2), (64, 4), (256, 1), (256, 2), (512, 1), (1024, 1))],
+     ["row_fwd_kernel"], []),
     # block order by line-sharing sets only where the sets divide a sample's units
     ("gn_cl_rows_block_order_whole_sets", run_gn, (2, 120, (20, 20), 15, F32, True),
      [{"GN_CL_XCD_MAP": m, **NO_SPLIT} for m in (1, 2)],
