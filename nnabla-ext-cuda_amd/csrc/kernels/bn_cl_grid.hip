@@ -926,6 +926,7 @@ int run_grid_bwd(int nl, const BnClGridArgs &a, hipStream_t st) {
 }
 
 constexpr int kGridMaxSlots = 25; // vectors per thread the forward layouts hold
+constexpr int kGridBwdHeld = 21;  // ... and the backward layouts (12 in registers, 9 in LDS)
 
 int log2_of(uint32_t v) {
   int s = 0;
@@ -955,8 +956,9 @@ bool grid_args(const BnProblem &p, BnClGridArgs &a, int &nl) {
   for (const int64_t cap = tune_int("BN_CL_GRID_STRIP_VECS", kWave); cv > cap && cv > 1;) cv >>= 1;
   const int64_t strips = ld / cv;
   if (strips > 1) {
-    // (a strip's row segment is at least a cache line)
-    if (!tune_int("BN_CL_GRID_STRIPS", 1) || cv < tune_int("BN_CL_GRID_STRIP_MIN_VECS", 8)) return false;
+    // (a strip's row segment is at least half a cache line; the callers take
+    // the halves only for tensors the chip holds whole)
+    if (!tune_int("BN_CL_GRID_STRIPS", 1) || cv < tune_int("BN_CL_GRID_STRIP_MIN_VECS", 4)) return false;
     if (strips > blocks / 8) return false;
   }
   int64_t ranges = std::max<int64_t>(blocks / strips, 1);
@@ -1038,6 +1040,14 @@ bool bn_cl_grid_fwd_train(const BnProblem &p, hipStream_t st, int *status) {
   // ([256,28,28,384] half, 154 MB, 37 vectors: 92.4 -> 67.9 us; 205 MB: 113.7 ->
   // 93.6; 308 MB, 74 vectors: 166.2 -> 150.3; 411 MB, 98 vectors: 223.4 -> 220.9).
   if (nl > tune_int("BN_CL_GRID_FWD_MAX_SLOTS", 80)) return false;
+  // Strips of 64 bytes (rows that are no whole number of 128-byte segments: 96,
+  // 160, 480, 672 half channels) share their cache lines with the neighbouring
+  // strip's blocks: ahead of the three launches where every vector is held
+  // (half forward / backward us, [128,14,14,672] 33.5 / 57.4 -> 24.3 / 40.1,
+  // [64,56,56,96] 32.1 / 54.5 -> 28.4 / 46.7, [128,28,28,480] forward 64.3 -> 59.6),
+  // behind them where a remainder is streamed ([256,28,28,288] backward 104.7 ->
+  // 133.6, [128,28,28,480] backward 90.7 -> 102.3).
+  if (a.cv < 8 && nl > kGridMaxSlots) return false;
   a.hv = nl > kGridMaxSlots ? static_cast<uint32_t>(kGridMaxSlots) * kOnchipBlock : ~0u;
   a.y = p.out;
   a.beta = p.beta;
@@ -1059,6 +1069,17 @@ bool bn_cl_grid_bwd(const BnProblem &p, hipStream_t st, int *status) {
   // ([256,28,28,384] half, 154 MB: 138.7 -> 116.9 us; 205 MB half 182.5 ->
   // 179.6, float 189.7 -> 166.4; 257 MB, 62 vectors: 220.4 -> 227.6).
   if (!aligned16(p.dy) || nl > tune_int("BN_CL_GRID_BWD_MAX_SLOTS", 50)) return false;
+  // (64-byte strips, see the forward: backward only up to 56 MiB in half, 16 MiB
+  // in float - us, this against the three launches, [N,28,28,C]: half C = 96
+  // 24 MiB 33.2 / 37.8, 48 MiB 57.4 / 68.1, 64 MiB 73.3 / 68.7; C = 288 48 MiB
+  // 55.0 / 79.4, 80 MiB 85.7 / 85.2; float C = 80 12 MiB 17.2 / 18.2, 24 MiB
+  // 31.0 / 27.8, 48 MiB 55.0 / 47.1)
+  if (a.cv < 8) {
+    const uint64_t bytes = static_cast<uint64_t>(p.size0) * p.C * (p.dtype == NBLAHIP_F16 ? 2 : 4);
+    const int most_kb = p.dtype == NBLAHIP_F16 ? tune_int("BN_CL_GRID_NARROW_BWD_MAX_KB", 57344)
+                                               : tune_int("BN_CL_GRID_NARROW_BWD_MAX_KB_F32", 16384);
+    if (nl > kGridBwdHeld || bytes > static_cast<uint64_t>(most_kb) * 1024u) return false;
+  }
   a.dy = p.dy;
   a.dx = p.out;
   a.mean = const_cast<float *>(p.mean);

@@ -451,6 +451,20 @@ GRIDS = [
     ("ln_bwd_forced_layouts_float", run_ln, (2100, 1000, F32),
      [{"LN_BWD_TPR": t, "LN_BWD_NL": n} for t, n in ((64, 4), (256, 1), (256, 2), (512, 1), (512, 3))],
      ["row_bwd_kernel_ln"], []),
+    # channel-last rows that are no whole number of 128-byte segments: column strips of 64 bytes
+    # on the grid-resident kernels (default where the chip holds the tensor), or the three launches
+    ("bn_cl_grid_narrow_strips_off", run_bn, ((16, 28, 28, 96), 3, F16), [{"BN_CL_GRID_STRIP_MIN_VECS": 8}],
+     ["bn_stats_cl_kernel", "bn_bwd_reduce_cl_kernel"], ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"]),
+    ("bn_cl_grid_narrow_strips", run_bn, ((16, 28, 28, 96), 3, F16), [{}],
+     ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"], []),
+    ("bn_cl_grid_narrow_strips_float", run_bn, ((16, 28, 28, 80), 3, F32), [{}],
+     ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"], []),
+    ("bn_cl_grid_narrow_backward_limit", run_bn, ((16, 28, 28, 160), 3, F16),
+     [{"BN_CL_GRID_NARROW_BWD_MAX_KB": 1024}], ["bn_cl_grid_fwd_kernel", "bn_bwd_reduce_cl_kernel"],
+     ["bn_cl_grid_bwd_kernel"]),
+    ("bn_cl_grid_narrow_backward_limit_float", run_bn, ((16, 28, 28, 80), 3, F32),
+     [{"BN_CL_GRID_NARROW_BWD_MAX_KB_F32": 1024}], ["bn_cl_grid_fwd_kernel", "bn_bwd_reduce_cl_kernel"],
+     ["bn_cl_grid_bwd_kernel"]),
     ("in_forced_wave_layouts", run_in, (6, 40, (32, 32), F16),
      [{"ROW_TPR": t, "ROW_NL": n} for t, n in ((64, 2), (64, 4), (256, 1), (256, 2), (512, 1), (1024, 1))],
      ["row_fwd_kernel"], []),

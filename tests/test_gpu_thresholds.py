@@ -154,6 +154,12 @@ CASES = [
        "bn_cl_grid_fwd_kernel", "bn_stats_cl_kernel"),
       ("above", ((256, 56, 56, 256), 3, F16), {"BN_CL_GRID_FWD_MAX_SLOTS": 120, "BN_CL_GRID_BWD_MAX_SLOTS": 120},
        "bn_stats_cl_kernel", "bn_cl_grid_fwd_kernel")]),
+    # ... rows of 64-byte strips: backward up to 56 MiB in half, 16 MiB in float
+    ("bn_cl_grid_narrow_bwd_max_kb", P.run_bn, {},
+     [("below", ((320, 28, 28, 96), 3, F16), {"BN_CL_GRID_NARROW_BWD_MAX_KB": 1024}, "bn_cl_grid_bwd_kernel", "bn_bwd_reduce_cl_kernel"),
+      ("above", ((560, 28, 28, 96), 3, F16), {"BN_CL_GRID_NARROW_BWD_MAX_KB": 1000000}, "bn_bwd_reduce_cl_kernel", "bn_cl_grid_bwd_kernel"),
+      ("below_f32", ((48, 28, 28, 80), 3, F32), {"BN_CL_GRID_NARROW_BWD_MAX_KB_F32": 1024}, "bn_cl_grid_bwd_kernel", "bn_bwd_reduce_cl_kernel"),
+      ("above_f32", ((200, 28, 28, 80), 3, F32), {"BN_CL_GRID_NARROW_BWD_MAX_KB_F32": 1000000}, "bn_bwd_reduce_cl_kernel", "bn_cl_grid_bwd_kernel")]),
     # short planes that share cache lines: ordinary stores inside the shared lines up to 1 KB
     ("bn_edge_stores_max_bytes", P.run_bn, NCS,
      [("below", ((256, 256, 14, 14), 1, F16), {"BN_EDGE_STORES_MAX_BYTES": 0}, "bn_onchip_fwd_kernel", "bn_onchip_fwd_kernel"),
