@@ -979,7 +979,15 @@ bool grid_args(const BnProblem &p, BnClGridArgs &a, int &nl) {
   // 36.5; but [3136,256] half 22.2 vs 21.5, [3136,512] float 21.6 vs 20.4: from
   // 10240 rows ([8192,128] float 20.6 vs 17.5) or, with more than 128 channels,
   // 24 MiB.
-  if (p.C <= kGridMaxC) {
+  // (Rows that are no whole number of 128-byte segments: no split kernel takes
+  // them, the other plan is three launches, and these kernels are ahead from the
+  // first tensor they accept - forward / backward us, [N,14,14,C] half: 1568 rows
+  // of 480 channels 13.7 / 13.0 -> 10.0 / 10.7, 3136 of 96 13.0 / 13.2 -> 10.4 /
+  // 11.2, 6272 of 672 19.2 / 21.3 -> 12.9 / 14.8; float 3136 of 80 12.7 / 13.2 ->
+  // 8.9 / 9.2.)
+  if (p.C % (8 * vec) != 0) {
+    if (M < tune_int("BN_CL_GRID_NARROW_MIN_ROWS", 1)) return false;
+  } else if (p.C <= kGridMaxC) {
     if (M < tune_int("BN_CL_GRID_MIN_ROWS", 10240)) return false;
   } else {
     if (!tune_int("BN_CL_GRID_WIDE", 1)) return false;

@@ -459,6 +459,10 @@ GRIDS = [
      ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"], []),
     ("bn_cl_grid_narrow_strips_float", run_bn, ((16, 28, 28, 80), 3, F32), [{}],
      ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"], []),
+    ("bn_cl_grid_narrow_few_rows", run_bn, ((16, 14, 14, 96), 3, F16), [{}],
+     ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"], []),
+    ("bn_cl_grid_narrow_from_more_rows", run_bn, ((16, 14, 14, 96), 3, F16), [{"BN_CL_GRID_NARROW_MIN_ROWS": 10240}],
+     ["bn_stats_cl_kernel", "bn_bwd_reduce_cl_kernel"], ["bn_cl_grid_fwd_kernel"]),
     ("bn_cl_grid_narrow_backward_limit", run_bn, ((16, 28, 28, 160), 3, F16),
      [{"BN_CL_GRID_NARROW_BWD_MAX_KB": 1024}], ["bn_cl_grid_fwd_kernel", "bn_bwd_reduce_cl_kernel"],
      ["bn_cl_grid_bwd_kernel"]),

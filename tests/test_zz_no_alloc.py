@@ -15,13 +15,15 @@ K = load_package()
 # (shape, axis, dtype name): tensors that take the split reduction, i.e. use
 # the scratch array (channel-last with many rows - 96 channels, which the
 # kernel that holds the tensor on the chip takes only in 64-byte column
-# strips, switched off here; planes with few
+# strips, switched off here, and 32 channels in fewer rows than it is given;
+# planes with few
 # channels, with the plans that hold a channel on one CU or split it over
 # several blocks switched off), and a pair that does not need it (held on the
 # chip, the partials travel through the exchange array): the entry point must
 # agree there too.
 CASES = [
-    ([((64, 56, 56, 96), 3, "f16"), ((8, 28, 28, 32), 3, "f16")], True, {"BN_CL_GRID_STRIP_MIN_VECS": 8}),
+    ([((64, 56, 56, 96), 3, "f16"), ((8, 28, 28, 32), 3, "f16")], True,
+     {"BN_CL_GRID_STRIP_MIN_VECS": 8, "BN_CL_GRID_NARROW_MIN_ROWS": 10240}),
     ([((32, 8, 56, 56), 1, "f32"), ((32, 8, 40, 40), 1, "f32")], True,
      {"BN_CHAN_SPLIT": 0, "BN_ONCHIP": 0}),
     ([((64, 56, 56, 64), 3, "f16"), ((56, 56, 56, 64), 3, "f16")], False, {}),
