@@ -516,6 +516,17 @@ bool pack_args(const BnProblem &p, bool backward, BnPackArgs &a, int &nl) {
   const bool short_channels = p.size0 * p.size2 <= 4096;
   const int min_pct = short_channels ? tune_int("BN_PACK_SHORT_MIN_PCT", 100) : tune_int("BN_PACK_MIN_PCT", 1);
   if ((p.C / G) * 100 < static_cast<int64_t>(device_cus()) * min_pct) return false;
+  // Few packs of long channels, where a block per channel can hold the channel:
+  // that many more blocks win (forward / backward us, packs against the masked
+  // block per channel or, shorter channels, the row kernels: [256,256,7,7] half,
+  // 32 packs, 18.6 / 20.4 vs 15.6 / 13.4; [128,160,7,7] half, 20 packs, 11.1 / 11.7
+  // vs 6.6 / 6.4; [256,320,7,7] half, 40 packs, 19.1 / 20.5 vs 17.3 / 18.7;
+  // [128,160,7,7] float, 40 packs, 11.0 / 11.1 vs 7.5 / 8.7; from 64 packs on the
+  // packs are ahead, [256,512,7,7] half 19.1 / 21.0 vs 19.6 / 23.2).
+  if (!short_channels &&
+      (p.C / G) * 100 < static_cast<int64_t>(device_cus()) * tune_int("BN_PACK_MIN_PCT_MASKED", 16) &&
+      bn_masked_takes(p, backward))
+    return false;
   a = BnPackArgs{};
   a.x = p.x;
   a.gamma = p.gamma;

@@ -175,6 +175,8 @@ bool bn_chan_split_bwd(const BnProblem &p, hipStream_t st, int *status);
 // Planes that are no whole number of vectors, a channel held by one block
 // (rows_masked.hip); false: not taken.
 bool bn_masked_fwd_train(const BnProblem &p, hipStream_t st, int *status);
+// Whether the masked kernels (a block per channel) would take this problem.
+bool bn_masked_takes(const BnProblem &p, bool backward);
 bool bn_masked_bwd(const BnProblem &p, hipStream_t st, int *status);
 bool bn_pack_fwd_train(const BnProblem &p, hipStream_t st, int *status);
 bool bn_pack_bwd(const BnProblem &p, hipStream_t st, int *status);

@@ -1310,6 +1310,12 @@ int launch_bn_masked(const BnProblem &p, int nl, int tb, const BnMaskedArgs &a, 
 
 } // namespace
 
+bool bn_masked_takes(const BnProblem &p, bool backward) {
+  BnMaskedArgs a;
+  int nl = 0, tb = 0;
+  return bn_masked_args(p, backward, a, nl, tb);
+}
+
 bool bn_masked_fwd_train(const BnProblem &p, hipStream_t st, int *status) {
   BnMaskedArgs a;
   int nl = 0, tb = 0;

@@ -622,7 +622,7 @@ def _held_backward(m, c, dtype, extra):
     ((48000, 128), 1, torch.float16, "bn_cl_grid_fwd_kernel", {"BN_CL_GRID_MIN_SLOTS": 1, "BN_CL_GRID_BLOCKS": 16}),
     ((40000, 64), 1, torch.float32, "bn_cl_grid_fwd_kernel", {"BN_CL_GRID_MIN_SLOTS": 1, "BN_CL_GRID_BLOCKS": 16}),
     ((200, 256, 7, 7), 1, torch.float32, "bn_pack_fwd_kernel", {}),
-    ((200, 256, 7, 7), 1, torch.float16, "bn_pack_fwd_kernel", {}),
+    ((200, 384, 7, 7), 1, torch.float16, "bn_pack_fwd_kernel", {}),
     ((12000, 128), 1, torch.float16, "cl_split_fwd_kernel", {"BN_CL_GRID": 0}),
 ])
 def test_one_pass_statistics_on_hard_data(kind, shape, axis, dtype, kernel, knobs):

@@ -170,9 +170,9 @@ SWITCHES = [
     ("bn_rows_off", run_bn, ((32, 64, 14, 14), 1, F16), {"BN_ROWS": 0, "BN_MASKED_ONCHIP": 0},
      ["bn_stats_planes_kernel", "bn_finalize_fwd_kernel", "bn_apply_planes_kernel",
       "bn_finalize_bwd_kernel"], ["row_fwd_kernel_bn", "row_bwd_kernel_bn"]),
-    ("bn_pack_off", run_bn, ((96, 256, 7, 7), 1, F16), {"BN_PACK": 0, "BN_MASKED_ONCHIP": 0},
+    ("bn_pack_off", run_bn, ((96, 384, 7, 7), 1, F16), {"BN_PACK": 0, "BN_MASKED_ONCHIP": 0},
      ["bn_stats_planes_kernel", "bn_bwd_reduce_planes_kernel"], ["bn_pack_fwd_kernel", "bn_pack_bwd_kernel"]),
-    ("bn_pack_min_pct_up", run_bn, ((96, 256, 7, 7), 1, F16), {"BN_PACK_MIN_PCT": 50, "BN_MASKED_ONCHIP": 0},
+    ("bn_pack_min_pct_up", run_bn, ((96, 384, 7, 7), 1, F16), {"BN_PACK_MIN_PCT": 50, "BN_MASKED_ONCHIP": 0},
      ["bn_stats_planes_kernel"], ["bn_pack_fwd_kernel", "bn_pack_bwd_kernel"]),
     ("bn_cl_grid_off", run_bn, ((100352, 64), 1, F16), {"BN_CL_GRID": 0},
      ["bn_stats_cl_kernel", "bn_finalize_fwd_kernel", "bn_apply_cl_kernel"], ["bn_cl_grid_fwd_kernel"],
@@ -381,7 +381,7 @@ GRIDS = [
      ["bn_chan_split_fwd_kernel", "bn_chan_split_bwd_kernel"], []),
     ("bn_pack_few_channels", run_bn, ((48, 16, 7, 7), 1, F16), [{"BN_PACK_SHORT_MIN_PCT": 0}],
      ["bn_pack_fwd_kernel", "bn_pack_bwd_kernel"], []),
-    ("bn_pack_plain_block_order", run_bn, ((96, 256, 7, 7), 1, F16),
+    ("bn_pack_plain_block_order", run_bn, ((96, 384, 7, 7), 1, F16),
      [{"BN_PACK_XCD_MAP": 0}, {"BN_PACK_EDGE_STORES": 0}],
      ["bn_pack_fwd_kernel", "bn_pack_bwd_kernel"], []),
     ("ln_bwd_blocks_per_cu", run_ln, (4096, 1024, F16), [{"LN_BWD_BLOCKS_PER_CU": v} for v in (1, 2, 4)],
@@ -459,6 +459,11 @@ GRIDS = [
      ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"], []),
     ("bn_cl_grid_narrow_strips_float", run_bn, ((16, 28, 28, 80), 3, F32), [{}],
      ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"], []),
+    # few channel packs where a block per channel holds the channel: the masked kernels (default) / packs
+    ("bn_pack_few_packs_to_masked", run_bn, ((256, 96, 7, 7), 1, F16), [{}],
+     ["bn_masked_fwd_kernel", "bn_masked_bwd_kernel"], ["bn_pack_fwd_kernel"]),
+    ("bn_pack_few_packs", run_bn, ((256, 96, 7, 7), 1, F16), [{"BN_PACK_MIN_PCT_MASKED": 1}],
+     ["bn_pack_fwd_kernel", "bn_pack_bwd_kernel"], ["bn_masked_fwd_kernel"]),
     ("bn_cl_grid_narrow_few_rows", run_bn, ((16, 14, 14, 96), 3, F16), [{}],
      ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"], []),
     ("bn_cl_grid_narrow_from_more_rows", run_bn, ((16, 14, 14, 96), 3, F16), [{"BN_CL_GRID_NARROW_MIN_ROWS": 10240}],

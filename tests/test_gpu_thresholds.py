@@ -121,6 +121,11 @@ CASES = [
       ("short_below", ((32, 256, 7, 7), 1, F16), {"BN_PACK_SHORT_MIN_PCT": 1}, "row_fwd_kernel_bn", "bn_pack_fwd_kernel"),
       ("short_below_more", ((32, 1024, 7, 7), 1, F16), {"BN_PACK_SHORT_MIN_PCT": 1}, "row_fwd_kernel_bn", "bn_pack_fwd_kernel"),
       ("short_above", ((64, 2048, 7, 7), 1, F16), {"BN_PACK_SHORT_MIN_PCT": 101}, "bn_pack_fwd_kernel", "row_fwd_kernel_bn")]),
+    # ... long channels in few packs, where a block per channel holds the channel: packs from 16 % of the CUs
+    ("bn_pack_min_pct_masked", P.run_bn, {},
+     [("below", ((256, 256, 7, 7), 1, F16), {"BN_PACK_MIN_PCT_MASKED": 1}, "bn_masked_fwd_kernel", "bn_pack_fwd_kernel"),
+      ("above", ((256, 512, 7, 7), 1, F16), {"BN_PACK_MIN_PCT_MASKED": 100}, "bn_pack_fwd_kernel", "bn_masked_fwd_kernel"),
+      ("below_f32", ((128, 160, 7, 7), 1, F32), {"BN_PACK_MIN_PCT_MASKED": 1}, "bn_masked_fwd_kernel", "bn_pack_fwd_kernel")]),
     # odd planes with a channel held by one block: from the first channel
     ("bn_masked_onchip_min_pct", P.run_bn, {},
      [("few", ((64, 8, 17, 17), 1, F16), {"BN_MASKED_ONCHIP_MIN_PCT": 100}, "bn_masked_fwd_kernel", None),
