@@ -403,7 +403,7 @@ struct BnParamSrc {
   __device__ __forceinline__ BnParam get(uint32_t c) const {
     if (params) return params[c];
     BnParam q;
-    q.mean = rmean[c];
+    q.mean = rmean ? rmean[c] : 0.f; // (no mean: the inference-mode backward, dx = dy * a)
     q.a = (gamma ? gamma[c] : 1.f) * inv_std(rvar[c], eps);
     q.b = beta ? beta[c] : 0.f;
     q.c = 0.f;

@@ -581,6 +581,31 @@ int launch_bn_bwd(const BnProblem &p, hipStream_t st) {
   if (need_sums) {
     if (int e = do_bwd_reduce(p, pl, part2, fin, st)) return e;
   }
+  // Inference mode, plain BatchNormalization: dx = dy * gamma / std needs neither
+  // x nor the sums, so it is the forward's inference apply over dy - 2 S instead
+  // of the backward apply's 3 S, and no finalize launch where no parameter
+  // gradient is wanted ([32,256,56,56] float, dx alone 57.2 -> 40 us, with
+  // dgamma / dbeta 79.5 -> 66).
+  const bool infer_dx = !p.batch_stat && p.out && !p.accum_dx && !p.y && !p.dz && !p.z && !p.relu &&
+                        tune_int("BN_INFER_BWD_AS_APPLY", 1);
+  if (infer_dx) {
+    if (need_sums && !pl.direct_bwd) {
+      NBLAHIP_LAUNCH("bn_finalize_bwd_kernel", bn_finalize_bwd_kernel,
+                     dim3(static_cast<uint32_t>(p.C)), dim3(kBnBlock), 0, st, part2, pl.S, fin);
+      if (int e = last_launch_status()) return e;
+    }
+    BnProblem q = p;
+    q.x = p.dy;
+    q.dy = nullptr;
+    BnParamSrc src{};
+    src.params = nullptr;
+    src.rmean = nullptr;
+    src.rvar = p.var;
+    src.gamma = p.gamma;
+    src.beta = nullptr;
+    src.eps = p.eps;
+    return do_fwd_apply(q, pl, src, st);
+  }
   if ((p.out || need_sums) && (!need_sums || !pl.direct_bwd)) {
     // Without the reduction (inference-mode dx only) S = 0 leaves the sums at zero.
     NBLAHIP_LAUNCH("bn_finalize_bwd_kernel", bn_finalize_bwd_kernel,

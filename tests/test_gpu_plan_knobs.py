@@ -59,6 +59,25 @@ def run_bn(shape, axis, dtype, seed=1):
     assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
 
 
+def run_bn_infer_bwd(shape, axis, dtype, seed=5):
+    """Inference-mode backward (running statistics): dx alone, then dx, dgamma, dbeta."""
+    dn = dtype_name(dtype)
+    rng = np.random.default_rng(seed)
+    c = shape[axis]
+    x = rounded(rng.standard_normal(shape) * 2 + 1, dtype)
+    dy = rounded(rng.standard_normal(shape), dtype)
+    g = f32(rng.uniform(0.5, 1.5, c))
+    rm, rv = f32(rng.standard_normal(c) * 0.1), f32(rng.uniform(0.5, 2.0, c))
+    dx_r, dg_r, db_r = R.bn_backward_global(x, dy, g, rm, rv, axis, 1e-5)
+    xd, dyd, gd, rmd, rvd = to_dev(x, dtype), to_dev(dy, dtype), to_dev(g), to_dev(rm), to_dev(rv)
+    dx, _, _ = K.bn_backward(xd, dyd, gd, rmd, rvd, axis, 1e-5, batch_stat=False, need=(True, False, False))
+    assert_close(to_np(dx), dx_r, dn, "grad", "dx alone")
+    dx, dg, db = K.bn_backward(xd, dyd, gd, rmd, rvd, axis, 1e-5, batch_stat=False)
+    assert_close(to_np(dx), dx_r, dn, "grad", "dx")
+    assert_close(to_np(dg), dg_r, dn, "pgrad", "dgamma")
+    assert_close(to_np(db), db_r, dn, "pgrad", "dbeta")
+
+
 def run_ln(outer, Rr, dtype, seed=2):
     dn = dtype_name(dtype)
     rng = np.random.default_rng(seed)
@@ -459,6 +478,15 @@ GRIDS = [
      ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"], []),
     ("bn_cl_grid_narrow_strips_float", run_bn, ((16, 28, 28, 80), 3, F32), [{}],
      ["bn_cl_grid_fwd_kernel", "bn_cl_grid_bwd_kernel"], []),
+    # inference-mode backward: dx through the forward's inference apply over dy (default) / the backward apply
+    ("bn_infer_bwd_as_apply", run_bn_infer_bwd, ((16, 48, 28, 28), 1, F16), [{}],
+     ["bn_apply_planes_kernel", "bn_bwd_reduce_planes_kernel"], ["bn_bwd_apply_planes_kernel"]),
+    ("bn_infer_bwd_as_apply_channel_last", run_bn_infer_bwd, ((16, 28, 28, 48), 3, F32), [{}],
+     ["bn_apply_cl_kernel", "bn_bwd_reduce_cl_kernel"], ["bn_bwd_apply_cl_kernel"]),
+    ("bn_infer_bwd_as_apply_odd_planes", run_bn_infer_bwd, ((16, 48, 13, 13), 1, F16), [{}],
+     ["bn_apply_planes_kernel"], ["bn_bwd_apply_planes_kernel"]),
+    ("bn_infer_bwd_through_backward_apply", run_bn_infer_bwd, ((16, 48, 28, 28), 1, F16),
+     [{"BN_INFER_BWD_AS_APPLY": 0}], ["bn_bwd_apply_planes_kernel"], ["bn_apply_planes_kernel"]),
     # few channel packs where a block per channel holds the channel: the masked kernels (default) / packs
     ("bn_pack_few_packs_to_masked", run_bn, ((256, 96, 7, 7), 1, F16), [{}],
      ["bn_masked_fwd_kernel", "bn_masked_bwd_kernel"], ["bn_pack_fwd_kernel"]),
